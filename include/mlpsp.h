@@ -1,0 +1,114 @@
+/* libmlpsp_hip: MI355X (gfx950) tile-based forward renderer for MLP Splatting -- C ABI.
+ *
+ * Every pointer named *_dev or documented as "device" is HIP device memory owned by the caller;
+ * the library never allocates, frees or keeps device memory and never synchronises, except where
+ * a function says it blocks.  All kernels are enqueued on `stream` (a hipStream_t passed as
+ * void*; NULL = the default stream).  Functions return 0 (MLPSP_OK) or a bit mask of the MLPSP_E_*
+ * values below; mlpsp_strerror() gives the message the reference raises for that condition.
+ *
+ * Tensor layouts are those of the reference extension (row-major, contiguous, f32 unless noted):
+ *   rays_o, rays_d [B,3] (rays_d unit length), B = width*height, pixel = y*width + x
+ *   positions, log_scales [N,3]; quats [N,4] unit (w,x,y,z)
+ *   tile list: tile_offsets [T+1] int32, candidates [P] int32, tile = ty*ceil(width/tile_w) + tx
+ *   freq, att [F]; W1 [N,H,12F] b1 [N,H] W2 [N,H,H] b2 [N,H] W3 [N,4,H] b3 [N,4]
+ *   feat_attr [N,C] (slots = 1) or [N,slots,C] with slots in {4,5}, C <= 512
+ *   outputs rgb [B,3], alpha [B,1], t [B,1], feat [B,C]
+ *
+ * Reference interface replaced: the pybind11 module of scannet/cuda/np_tile_kernels.cu:7224-7252
+ * (forward entry points) and the PyTorch culling of scannet/cumodel.py:994-1070.
+ */
+#ifndef MLPSP_H
+#define MLPSP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MLPSP_OK 0
+#define MLPSP_E_OFFSETS 1        /* tile_offsets not monotone / not covering the list (np_tile_kernels.cu:4499-4503) */
+#define MLPSP_E_CAPACITY 2       /* a tile holds more candidates than the capacity (np_tile_kernels.cu:4506-4509) */
+#define MLPSP_E_IDS 4            /* a candidate id is outside [0, N) (np_tile_kernels.cu:4513-4519) */
+#define MLPSP_E_PIXEL_OVERFLOW 8 /* a pixel met a 257th hit in per-pixel order (np_tile_kernels.cu:798-809) */
+#define MLPSP_E_NONFINITE 16     /* non-finite operand or activation in the bf16 MFMA path (rgb_wmma.cuh:260) */
+#define MLPSP_E_ARGUMENT 32      /* a size or pointer argument is unusable */
+#define MLPSP_E_RUNTIME 64       /* a HIP call failed */
+#define MLPSP_E_SCRATCH 128      /* the scratch buffer is too small for this input: retry with a larger one */
+
+#define MLPSP_TILE_CAPACITY_MAX 2048 /* largest per-tile list the in-LDS sort accepts */
+#define MLPSP_PIXEL_HIT_CAPACITY 256 /* per-pixel-order hit buffer (np_tile_kernels.cu:760) */
+#define MLPSP_PRIM_RECORD_BYTES 64   /* bytes per primitive of the prepared geometry buffer */
+
+#define MLPSP_KEY_LIST_ORDER 0 /* consume the list as given (presorted kernel, np_tile_kernels.cu:4242-4478) */
+#define MLPSP_KEY_TSTAR 1      /* Mahalanobis t* of the tile-centre ray (np_tile_kernels.cu:483-518) */
+#define MLPSP_KEY_DEPTH 2      /* plain centre-ray depth (np_tile_kernels.cu:5538-5542) */
+
+typedef void* mlpsp_stream_t;
+
+/* Library version (major*10000 + minor*100 + patch). */
+int mlpsp_version(void);
+
+/* Message for one MLPSP_E_* bit, worded as the reference's TORCH_CHECK for that condition
+ * (np_tile_kernels.cu:4578-4598). */
+const char* mlpsp_strerror(int code);
+
+/* Per-primitive geometry in kernel-ready form: centre, exp(-2 log_s), unit quaternion, log_s.
+ * Replaces the per-candidate gathers + __expf of np_tile_kernels.cu:1947-1956, 676-678.
+ * prim_records_dev: N * MLPSP_PRIM_RECORD_BYTES bytes, 64-byte aligned. */
+int mlpsp_prepare_primitives(const float* positions_dev, const float* log_scales_dev, const float* quats_dev,
+                             int num_primitives, void* prim_records_dev, mlpsp_stream_t stream);
+
+/* Tile-list validation = validate_tile_candidate_capacity (np_tile_kernels.cu:4485-4589).
+ * capacity 0 = no cap (per-pixel and presorted entry points).  status_dev: 2 int32 of device
+ * scratch.  BLOCKS: one 8-byte device-to-host copy, then returns the status mask;
+ * status_host[0] = mask, status_host[1] = largest over-capacity tile length. */
+int mlpsp_validate_tile_lists(const int32_t* tile_offsets_dev, const int32_t* candidates_dev, int num_tiles,
+                              int num_candidates, int capacity, int num_primitives, int32_t* status_dev,
+                              int32_t status_host[2], mlpsp_stream_t stream);
+
+/* Legacy screen-space culling, sparse: replaces the dense [tiles x primitives] overlap matrix of
+ * scannet/cumodel.py:994-1070 (one camera) and :838-949 (tile_view_ids_dev != NULL: K views, tile
+ * t uses view tile_view_ids_dev[t]).  view_matrices: K row-major 4x4 on the HOST, proj: 4x4 on
+ * the host.  Within a tile, candidate ids ascend.
+ * Step 1 (count): writes exclusive offsets to tile_offsets_dev[T+1]; BLOCKS to return the total
+ *   in *num_pairs_out.  scratch_dev: at least mlpsp_bin_scratch_bytes() bytes, 256-byte aligned,
+ *   reused by step 2; MLPSP_E_SCRATCH asks for a larger one (primitives spanning very many tiles).
+ * Step 2 (fill): writes candidates_dev[num_pairs]. */
+size_t mlpsp_bin_scratch_bytes(int num_primitives, int num_views, int width, int height, int tile);
+int mlpsp_bin_legacy_count(const float* positions_dev, const float* log_scales_dev, int num_primitives,
+                           const float* view_matrices_host, int num_views, const int32_t* tile_view_ids_dev,
+                           const float* proj_host, int width, int height, int tile, float threshold,
+                           void* scratch_dev, size_t scratch_bytes, int32_t* tile_offsets_dev,
+                           int64_t* num_pairs_out, mlpsp_stream_t stream);
+int mlpsp_bin_legacy_fill(int num_primitives, int num_views, const int32_t* tile_view_ids_dev, int width,
+                          int height, int tile, const void* scratch_dev, size_t scratch_bytes,
+                          const int32_t* tile_offsets_dev, int32_t* candidates_dev, mlpsp_stream_t stream);
+
+/* Per-tile depth-key sort = the in-kernel cub::BlockRadixSort of np_tile_kernels.cu:1929-1990,
+ * materialised: sorted_ids_dev[P] holds, tile by tile, the candidates in ascending key order, ties
+ * in list order; entries past min(len, capacity) keep list order.  sorted_keys_dev may be NULL.
+ * capacity <= MLPSP_TILE_CAPACITY_MAX (0 = that maximum). */
+int mlpsp_sort_tiles(const float* rays_o_dev, const float* rays_d_dev, const void* prim_records_dev,
+                     const int32_t* candidates_dev, const int32_t* tile_offsets_dev, int width, int height,
+                     int tile_w, int tile_h, int key_family, int capacity, int32_t* sorted_ids_dev,
+                     float* sorted_keys_dev, mlpsp_stream_t stream);
+
+/* Tile-centre-order forward, scalar f32 (render_tiles_kernel_tilecenter_order,
+ * np_tile_kernels.cu:1837-2137; with out_t_dev != NULL also the expected depth of :5432-5719).
+ * order_dev: the tile lists in processing order (mlpsp_sort_tiles output, or the candidates
+ * themselves for MLPSP_KEY_LIST_ORDER).  counters_dev: NULL or 4 int64 {unused, tile-primitives
+ * processed, tile-primitives with a hit, hits}, accumulated (zero them first). */
+int mlpsp_render_tilecenter_f32(const float* rays_o_dev, const float* rays_d_dev, const void* prim_records_dev,
+                                const int32_t* order_dev, const int32_t* tile_offsets_dev, const float* freq_dev,
+                                const float* att_dev, int num_frequencies, const float* W1, const float* b1,
+                                const float* W2, const float* b2, const float* W3, const float* b3,
+                                int num_primitives, int hidden, int width, int height, int tile_w, int tile_h,
+                                float threshold, float* out_rgb_dev, float* out_alpha_dev, float* out_t_dev,
+                                int64_t* counters_dev, mlpsp_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MLPSP_H */

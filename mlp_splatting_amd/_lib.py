@@ -1,0 +1,71 @@
+"""ctypes binding of ``libmlpsp_hip.so`` (the C ABI declared in ``include/mlpsp.h``).
+
+The library is built in-tree by ``mlp_splatting_amd/csrc/Makefile``.  There is no fallback: if the
+shared object is missing or does not export a declared symbol, loading raises.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+import subprocess
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libmlpsp_hip.so")
+CSRC_DIR = os.path.join(_HERE, "csrc")
+
+E_OFFSETS, E_CAPACITY, E_IDS, E_PIXEL_OVERFLOW, E_NONFINITE, E_ARGUMENT, E_RUNTIME, E_SCRATCH = 1, 2, 4, 8, 16, 32, 64, 128
+KEY_LIST_ORDER, KEY_TSTAR, KEY_DEPTH = 0, 1, 2
+TILE_CAPACITY_MAX = 2048
+PIXEL_HIT_CAPACITY = 256
+PRIM_RECORD_BYTES = 64
+
+_vp, _i, _f, _i64, _sz = C.c_void_p, C.c_int, C.c_float, C.c_int64, C.c_size_t
+
+# name -> (restype, argtypes); one entry per function declared in include/mlpsp.h
+SIGNATURES = {
+    "mlpsp_version": (_i, []),
+    "mlpsp_strerror": (C.c_char_p, [_i]),
+    "mlpsp_prepare_primitives": (_i, [_vp, _vp, _vp, _i, _vp, _vp]),
+    "mlpsp_validate_tile_lists": (_i, [_vp, _vp, _i, _i, _i, _i, _vp, C.POINTER(C.c_int32), _vp]),
+    "mlpsp_bin_scratch_bytes": (_sz, [_i, _i, _i, _i, _i]),
+    "mlpsp_bin_legacy_count": (_i, [_vp, _vp, _i, C.POINTER(_f), _i, _vp, C.POINTER(_f), _i, _i, _i, _f, _vp, _sz, _vp,
+                                    C.POINTER(_i64), _vp]),
+    "mlpsp_bin_legacy_fill": (_i, [_i, _i, _vp, _i, _i, _i, _vp, _sz, _vp, _vp, _vp]),
+    "mlpsp_sort_tiles": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp]),
+    "mlpsp_render_tilecenter_f32": (_i, [_vp] * 7 + [_i] + [_vp] * 6 + [_i, _i, _i, _i, _i, _i, _f, _vp, _vp, _vp,
+                                                                       _vp, _vp]),
+}
+
+_lib = None
+
+
+def build(verbose: bool = False) -> str:
+    """Compile every HIP source for gfx950 into ``libmlpsp_hip.so`` (hipcc cross-compiles; no GPU needed)."""
+    out = None if verbose else subprocess.DEVNULL
+    subprocess.check_call(["make", "-C", CSRC_DIR, "-j8"], stdout=out, stderr=out)
+    return LIB_PATH
+
+
+def load():
+    """Return the loaded library with argument types set; raise if it is absent or incomplete."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(
+            f"libmlpsp_hip.so not found at {LIB_PATH}; build it with `make -C {CSRC_DIR}` "
+            "(there is no CPU or PyTorch fallback for the renderer)")
+    lib = C.CDLL(LIB_PATH)
+    for name, (restype, argtypes) in SIGNATURES.items():
+        try:
+            fn = getattr(lib, name)
+        except AttributeError as exc:
+            raise RuntimeError(f"libmlpsp_hip.so does not export {name}; rebuild the library") from exc
+        fn.restype = restype
+        fn.argtypes = argtypes
+    _lib = lib
+    return lib
+
+
+def strerror(code: int) -> str:
+    return load().mlpsp_strerror(int(code)).decode()

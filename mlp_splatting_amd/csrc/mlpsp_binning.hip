@@ -1,0 +1,307 @@
+// libmlpsp_hip: projection of primitive supports and tile binning (the "legacy" screen-space rule).
+//
+// The reference evaluates a dense [tiles x primitives] boolean matrix (scannet/cumodel.py:1028-1070).
+// Here the same predicate is evaluated sparsely and deterministically, without atomics and without
+// a sort, in two levels:
+//   level 1: the frame is cut into super-tiles of 8x8 tiles.  Workgroup (chunk c, super-tile s)
+//            tests 2048 consecutive primitives against the super-tile rectangle (a superset of the
+//            union of its tiles' tests), counts, and after a scan writes the survivors in ascending
+//            id order -> one ascending candidate list per super-tile.
+//   level 2: one wavefront per tile walks its super-tile's list 64 ids at a time, applies the exact
+//            per-tile test, counts with a ballot, and after a scan writes the tile's candidates at
+//            ballot-prefix positions -> tile-major lists, ascending id inside a tile, which is the
+//            order `nonzero()` on the dense matrix yields.
+// All kernels are HBM/L2-bound integer and compare work; nothing here wants MFMA.
+#include "mlpsp_device.hpp"
+#include "mlpsp_host.hpp"
+
+#include <math.h>
+
+namespace mlpsp {
+
+constexpr int kSuper = 8;       // tiles per super-tile side
+constexpr int kChunk = 2048;    // primitives per level-1 workgroup
+constexpr int kBinThreads = 256;
+
+struct BinScratch {
+  float* mats;        // K view matrices (16 floats each) then the projection (16 floats)
+  float4* bounds;     // [K][N] (minx, maxx, miny, maxy); all NaN when behind the near plane
+  int32_t* l1_counts; // [S*NC + 1] counts, then exclusive offsets after the scan
+  long long* totals;  // [0] level-1 entries, [1] tile-list entries
+  int32_t* l1_list;   // [l1_capacity]
+  long long l1_capacity;
+};
+
+__host__ __device__ inline size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
+
+inline BinScratch carve(void* base, size_t bytes, int N, int K, int S, int NC) {
+  BinScratch b;
+  char* p = static_cast<char*>(base);
+  size_t off = 0;
+  b.mats = reinterpret_cast<float*>(p + off);
+  off += align256((size_t)(K + 1) * 16 * sizeof(float));
+  b.bounds = reinterpret_cast<float4*>(p + off);
+  off += align256((size_t)K * N * sizeof(float4));
+  b.l1_counts = reinterpret_cast<int32_t*>(p + off);
+  off += align256(((size_t)S * NC + 1) * sizeof(int32_t));
+  b.totals = reinterpret_cast<long long*>(p + off);
+  off += 256;
+  b.l1_list = reinterpret_cast<int32_t*>(p + off);
+  b.l1_capacity = bytes > off ? (long long)((bytes - off) / sizeof(int32_t)) : 0;
+  return b;
+}
+
+struct BinGeom {
+  int W, H, ts, ntx, nty, nsx, nsy, N, K, NC;
+};
+
+// Screen-space bounds of primitive i under view k (scannet/cumodel.py:1001-1041).  The 4-term dot
+// products are fma chains from the last term inwards.
+__global__ __launch_bounds__(kBinThreads) void bin_bounds_kernel(const float* __restrict__ pos,
+                                                                 const float* __restrict__ logs,
+                                                                 const float* __restrict__ mats, BinGeom g, float rm,
+                                                                 float focal, float4* __restrict__ bounds) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  const int k = blockIdx.y;
+  if (i >= g.N) return;
+  const float* V = mats + k * 16;
+  const float* Pm = mats + g.K * 16;
+  const float x = pos[i * 3 + 0], y = pos[i * 3 + 1], z = pos[i * 3 + 2];
+  float pv[4], clip[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) pv[r] = fmaf(V[r * 4 + 0], x, fmaf(V[r * 4 + 1], y, fmaf(V[r * 4 + 2], z, V[r * 4 + 3])));
+  const float depth = pv[2];
+  const float s = fmaxf(fmaxf(det_exp(logs[i * 3 + 0]), det_exp(logs[i * 3 + 1])), det_exp(logs[i * 3 + 2]));
+  const float world_radius = s * rm;
+  const float pr = (world_radius / (depth + 1e-8f)) * focal;
+#pragma unroll
+  for (int r = 0; r < 4; ++r)
+    clip[r] = fmaf(Pm[r * 4 + 0], pv[0], fmaf(Pm[r * 4 + 1], pv[1], fmaf(Pm[r * 4 + 2], pv[2], Pm[r * 4 + 3] * pv[3])));
+  float w = clip[3];
+  w = (w == 0.f) ? w + 1e-6f : w;
+  const float sx = (((clip[0] / w) + 1.f) * 0.5f) * (float)g.W;
+  const float sy = (((clip[1] / w) + 1.f) * 0.5f) * (float)g.H;
+  const float nan = __builtin_nanf("");
+  const bool front = depth > 0.001f;
+  bounds[(size_t)k * g.N + i] = front ? make_float4(sx - pr, sx + pr, sy - pr, sy + pr) : make_float4(nan, nan, nan, nan);
+}
+
+// strict inequalities of scannet/cumodel.py:1043-1044 on an axis-aligned pixel rectangle
+__device__ __forceinline__ bool rect_overlap(const float4 b, float x0, float x1, float y0, float y1) {
+  return (b.x < x1) && (b.y > x0) && (b.z < y1) && (b.w > y0);
+}
+
+__device__ __forceinline__ bool super_overlap(const float4* __restrict__ bounds, const BinGeom& g, int i, float x0,
+                                              float x1, float y0, float y1) {
+  bool any = false;
+  for (int k = 0; k < g.K; ++k) any |= rect_overlap(bounds[(size_t)k * g.N + i], x0, x1, y0, y1);
+  return any;
+}
+
+__device__ __forceinline__ void super_rect(const BinGeom& g, int s, float& x0, float& x1, float& y0, float& y1) {
+  const int sx = s % g.nsx, sy = s / g.nsx;
+  x0 = (float)(sx * kSuper * g.ts);
+  y0 = (float)(sy * kSuper * g.ts);
+  x1 = (float)(min((sx + 1) * kSuper, g.ntx) * g.ts);
+  y1 = (float)(min((sy + 1) * kSuper, g.nty) * g.ts);
+}
+
+__device__ __forceinline__ unsigned lanes_below(unsigned long long mask) {
+  return __builtin_amdgcn_mbcnt_hi((unsigned)(mask >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)mask, 0u));
+}
+
+// level 1.  grid = (NC, S).  FILL = false: l1_counts[s*NC + c] = survivors; FILL = true: write them.
+template <bool FILL>
+__global__ __launch_bounds__(kBinThreads) void bin_level1_kernel(const float4* __restrict__ bounds, BinGeom g,
+                                                                 int32_t* __restrict__ l1_counts,
+                                                                 int32_t* __restrict__ l1_list, long long l1_capacity) {
+  __shared__ int s_wave[kBinThreads / 64];
+  const int c = blockIdx.x, s = blockIdx.y;
+  const int wave = threadIdx.x >> 6;
+  float x0, x1, y0, y1;
+  super_rect(g, s, x0, x1, y0, y1);
+  int running = FILL ? l1_counts[s * g.NC + c] : 0;
+  for (int r = 0; r < kChunk / kBinThreads; ++r) {
+    const int i = c * kChunk + r * kBinThreads + threadIdx.x;
+    const bool keep = (i < g.N) && super_overlap(bounds, g, i, x0, x1, y0, y1);
+    const unsigned long long m = __ballot(keep);
+    if ((threadIdx.x & 63) == 0) s_wave[wave] = __popcll(m);
+    __syncthreads();
+    int before = 0, total = 0;
+#pragma unroll
+    for (int w = 0; w < kBinThreads / 64; ++w) {
+      const int cw = s_wave[w];
+      before += (w < wave) ? cw : 0;
+      total += cw;
+    }
+    if (FILL && keep) {
+      const long long dst = (long long)running + before + lanes_below(m);
+      if (dst < l1_capacity) l1_list[dst] = i;
+    }
+    running += total;
+    __syncthreads();
+  }
+  if (!FILL && threadIdx.x == 0) l1_counts[s * g.NC + c] = running;
+}
+
+// In-place exclusive scan of data[0..n) by one workgroup; data[n] and *total receive the sum.
+__global__ __launch_bounds__(1024) void exclusive_scan_kernel(int32_t* __restrict__ data, int n,
+                                                              long long* __restrict__ total) {
+  __shared__ long long s_part[1024];
+  const int t = threadIdx.x;
+  const int per = (n + 1023) / 1024;
+  const int lo = min(t * per, n), hi = min(lo + per, n);
+  long long sum = 0;
+  for (int i = lo; i < hi; ++i) sum += data[i];
+  s_part[t] = sum;
+  __syncthreads();
+  for (int d = 1; d < 1024; d <<= 1) {
+    const long long v = (t >= d) ? s_part[t - d] : 0;
+    __syncthreads();
+    s_part[t] += v;
+    __syncthreads();
+  }
+  long long run = s_part[t] - sum;
+  for (int i = lo; i < hi; ++i) {
+    const int v = data[i];
+    data[i] = (int32_t)run;
+    run += v;
+  }
+  if (t == 1023) {
+    data[n] = (int32_t)s_part[1023];
+    *total = s_part[1023];
+  }
+}
+
+// level 2.  One wavefront per tile, 4 tiles per workgroup.
+template <bool FILL>
+__global__ __launch_bounds__(kBinThreads) void bin_level2_kernel(const float4* __restrict__ bounds, BinGeom g,
+                                                                 const int32_t* __restrict__ tile_view_ids,
+                                                                 const int32_t* __restrict__ l1_offsets,
+                                                                 const int32_t* __restrict__ l1_list,
+                                                                 long long l1_capacity,
+                                                                 int32_t* __restrict__ tile_offsets,
+                                                                 int32_t* __restrict__ cand) {
+  const int tile = blockIdx.x * (kBinThreads / 64) + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  if (tile >= g.ntx * g.nty) return;
+  const int tx = tile % g.ntx, ty = tile / g.ntx;
+  const int s = (ty / kSuper) * g.nsx + (tx / kSuper);
+  const int view = tile_view_ids ? tile_view_ids[tile] : 0;
+  const float4* __restrict__ vb = bounds + (size_t)view * g.N;
+  const float x0 = (float)(tx * g.ts), x1 = (float)((tx + 1) * g.ts);
+  const float y0 = (float)(ty * g.ts), y1 = (float)((ty + 1) * g.ts);
+  // clamped so that an overflowed level-1 list (reported to the host) is never read past its end
+  const int lo = (int)min((long long)l1_offsets[s * g.NC], l1_capacity);
+  const int hi = (int)min((long long)l1_offsets[(s + 1) * g.NC], l1_capacity);
+  int running = FILL ? tile_offsets[tile] : 0;
+  for (int base = lo; base < hi; base += 64) {
+    const int j = base + lane;
+    int id = -1;
+    bool keep = false;
+    if (j < hi) {
+      id = l1_list[j];
+      keep = rect_overlap(vb[id], x0, x1, y0, y1);
+    }
+    const unsigned long long m = __ballot(keep);
+    if (FILL && keep) cand[running + lanes_below(m)] = id;
+    running += __popcll(m);
+  }
+  if (!FILL && lane == 0) tile_offsets[tile] = running;
+}
+
+inline BinGeom make_geom(int N, int K, int W, int H, int ts) {
+  BinGeom g;
+  g.W = W; g.H = H; g.ts = ts;
+  g.ntx = ceil_div(W, ts); g.nty = ceil_div(H, ts);
+  g.nsx = ceil_div(g.ntx, kSuper); g.nsy = ceil_div(g.nty, kSuper);
+  g.N = N; g.K = K; g.NC = ceil_div(N > 0 ? N : 1, kChunk);
+  return g;
+}
+
+}  // namespace mlpsp
+
+using namespace mlpsp;
+
+MLPSP_API size_t mlpsp_bin_scratch_bytes(int num_primitives, int num_views, int width, int height, int tile) {
+  if (num_primitives < 0 || num_views <= 0 || checked_num_tiles(width, height, tile, tile) <= 0) return 0;
+  const BinGeom g = make_geom(num_primitives, num_views, width, height, tile);
+  const size_t S = (size_t)g.nsx * g.nsy;
+  size_t bytes = align256((size_t)(num_views + 1) * 16 * sizeof(float)) +
+                 align256((size_t)num_views * num_primitives * sizeof(float4)) +
+                 align256((S * g.NC + 1) * sizeof(int32_t)) + 256;
+  // room for every primitive to touch 8 super-tiles per view, plus slack for tiny scenes
+  bytes += align256(((size_t)8 * num_views * num_primitives + 65536) * sizeof(int32_t));
+  return bytes;
+}
+
+MLPSP_API int mlpsp_bin_legacy_count(const float* positions_dev, const float* log_scales_dev, int num_primitives,
+                                     const float* view_matrices_host, int num_views,
+                                     const int32_t* tile_view_ids_dev, const float* proj_host, int width, int height,
+                                     int tile, float threshold, void* scratch_dev, size_t scratch_bytes,
+                                     int32_t* tile_offsets_dev, int64_t* num_pairs_out, mlpsp_stream_t stream) {
+  const int64_t T = checked_num_tiles(width, height, tile, tile);
+  if (T <= 0 || num_primitives < 0 || num_views <= 0 || !view_matrices_host || !proj_host || !scratch_dev ||
+      !tile_offsets_dev || !num_pairs_out)
+    return MLPSP_E_ARGUMENT;
+  if (!(threshold > 0.f && threshold < 1.f)) return MLPSP_E_ARGUMENT;
+  if (scratch_bytes < mlpsp_bin_scratch_bytes(num_primitives, num_views, width, height, tile)) return MLPSP_E_SCRATCH;
+  hipStream_t s = (hipStream_t)stream;
+  const BinGeom g = make_geom(num_primitives, num_views, width, height, tile);
+  const int S = g.nsx * g.nsy;
+  const BinScratch b = carve(scratch_dev, scratch_bytes, num_primitives, num_views, S, g.NC);
+  *num_pairs_out = 0;
+  if (num_primitives == 0) {
+    MLPSP_HIP_TRY(hipMemsetAsync(tile_offsets_dev, 0, (size_t)(T + 1) * sizeof(int32_t), s));
+    MLPSP_HIP_TRY(hipMemsetAsync(b.totals, 0, 2 * sizeof(long long), s));
+    return MLPSP_OK;
+  }
+  // scalar constants in f32, in the order the reference's tensor expressions evaluate them
+  const float rm = sqrtf(-2.0f * logf(threshold));
+  const float fx = (proj_host[0] * (float)width) / 2.0f, fy = (proj_host[5] * (float)height) / 2.0f;
+  const float focal = (fx + fy) * 0.5f;
+  MLPSP_HIP_TRY(hipMemcpyAsync(b.mats, view_matrices_host, (size_t)num_views * 16 * sizeof(float),
+                               hipMemcpyHostToDevice, s));
+  MLPSP_HIP_TRY(hipMemcpyAsync(b.mats + (size_t)num_views * 16, proj_host, 16 * sizeof(float), hipMemcpyHostToDevice, s));
+  hipLaunchKernelGGL(bin_bounds_kernel, dim3(ceil_div(num_primitives, kBinThreads), num_views), dim3(kBinThreads), 0, s,
+                     positions_dev, log_scales_dev, b.mats, g, rm, focal, b.bounds);
+  MLPSP_LAUNCH_CHECK();
+  hipLaunchKernelGGL((bin_level1_kernel<false>), dim3(g.NC, S), dim3(kBinThreads), 0, s, b.bounds, g, b.l1_counts,
+                     b.l1_list, b.l1_capacity);
+  MLPSP_LAUNCH_CHECK();
+  hipLaunchKernelGGL(exclusive_scan_kernel, dim3(1), dim3(1024), 0, s, b.l1_counts, S * g.NC, b.totals);
+  MLPSP_LAUNCH_CHECK();
+  hipLaunchKernelGGL((bin_level1_kernel<true>), dim3(g.NC, S), dim3(kBinThreads), 0, s, b.bounds, g, b.l1_counts,
+                     b.l1_list, b.l1_capacity);
+  MLPSP_LAUNCH_CHECK();
+  hipLaunchKernelGGL((bin_level2_kernel<false>), dim3(ceil_div((int)T, kBinThreads / 64)), dim3(kBinThreads), 0, s,
+                     b.bounds, g, tile_view_ids_dev, b.l1_counts, b.l1_list, b.l1_capacity, tile_offsets_dev,
+                     (int32_t*)nullptr);
+  MLPSP_LAUNCH_CHECK();
+  hipLaunchKernelGGL(exclusive_scan_kernel, dim3(1), dim3(1024), 0, s, tile_offsets_dev, (int)T, b.totals + 1);
+  MLPSP_LAUNCH_CHECK();
+  // one blocking readback: level-1 entry count (overflow check) and the number of pairs
+  long long totals[2] = {0, 0};
+  MLPSP_HIP_TRY(hipMemcpyAsync(totals, b.totals, 2 * sizeof(long long), hipMemcpyDeviceToHost, s));
+  MLPSP_HIP_TRY(hipStreamSynchronize(s));
+  if (totals[0] > b.l1_capacity) return MLPSP_E_SCRATCH;
+  if (totals[1] > 2147483647LL) return MLPSP_E_ARGUMENT;
+  *num_pairs_out = totals[1];
+  return MLPSP_OK;
+}
+
+MLPSP_API int mlpsp_bin_legacy_fill(int num_primitives, int num_views, const int32_t* tile_view_ids_dev, int width,
+                                    int height, int tile, const void* scratch_dev, size_t scratch_bytes,
+                                    const int32_t* tile_offsets_dev, int32_t* candidates_dev, mlpsp_stream_t stream) {
+  const int64_t T = checked_num_tiles(width, height, tile, tile);
+  if (T <= 0 || num_primitives < 0 || num_views <= 0 || !scratch_dev || !tile_offsets_dev) return MLPSP_E_ARGUMENT;
+  if (num_primitives == 0) return MLPSP_OK;
+  if (!candidates_dev) return MLPSP_E_ARGUMENT;
+  const BinGeom g = make_geom(num_primitives, num_views, width, height, tile);
+  const BinScratch b = carve(const_cast<void*>(scratch_dev), scratch_bytes, num_primitives, num_views, g.nsx * g.nsy, g.NC);
+  hipLaunchKernelGGL((bin_level2_kernel<true>), dim3(ceil_div((int)T, kBinThreads / 64)), dim3(kBinThreads), 0,
+                     (hipStream_t)stream, b.bounds, g, tile_view_ids_dev, b.l1_counts, b.l1_list, b.l1_capacity,
+                     const_cast<int32_t*>(tile_offsets_dev), candidates_dev);
+  MLPSP_LAUNCH_CHECK();
+  return MLPSP_OK;
+}

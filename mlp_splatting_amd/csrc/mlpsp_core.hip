@@ -1,0 +1,216 @@
+// libmlpsp_hip: primitive preparation, tile-list validation and the per-tile depth-key sort.
+#include "mlpsp_device.hpp"
+#include "mlpsp_host.hpp"
+
+namespace mlpsp {
+
+// ---------------------------------------------------------------------------------------------
+// prepare: [N,3]+[N,3]+[N,4] -> one 64-byte record per primitive (HBM-bound: 40 B in, 64 B out)
+// ---------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void prepare_primitives_kernel(const float* __restrict__ pos,
+                                                                 const float* __restrict__ logs,
+                                                                 const float* __restrict__ quats, int N,
+                                                                 PrimRecord* __restrict__ out) {
+  const int p = blockIdx.x * blockDim.x + threadIdx.x;
+  if (p >= N) return;
+  PrimRecord r;
+  r.cx = pos[p * 3 + 0];
+  r.cy = pos[p * 3 + 1];
+  r.cz = pos[p * 3 + 2];
+  r.lgx = logs[p * 3 + 0];
+  r.lgy = logs[p * 3 + 1];
+  r.lgz = logs[p * 3 + 2];
+  r.qw = quats[p * 4 + 0];
+  r.qx = quats[p * 4 + 1];
+  r.qy = quats[p * 4 + 2];
+  r.qz = quats[p * 4 + 3];
+  r.mx = det_exp(-2.f * r.lgx);
+  r.my = det_exp(-2.f * r.lgy);
+  r.mz = det_exp(-2.f * r.lgz);
+  r.pad0 = r.pad1 = r.pad2 = 0.f;
+  float4* dst = reinterpret_cast<float4*>(out + p);
+  dst[0] = make_float4(r.cx, r.cy, r.cz, r.mx);
+  dst[1] = make_float4(r.my, r.mz, r.qw, r.qx);
+  dst[2] = make_float4(r.qy, r.qz, r.lgx, r.lgy);
+  dst[3] = make_float4(r.lgz, 0.f, 0.f, 0.f);
+}
+
+// ---------------------------------------------------------------------------------------------
+// validate (np_tile_kernels.cu:4485-4520): grid-stride over tiles, then over candidates
+// ---------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void validate_tile_lists_kernel(const int32_t* __restrict__ offsets,
+                                                                  const int32_t* __restrict__ cand, int num_tiles,
+                                                                  int num_cand, int capacity, int num_prims,
+                                                                  int32_t* __restrict__ status) {
+  const int64_t stride = (int64_t)blockDim.x * gridDim.x;
+  const int64_t first = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  for (int64_t tile = first; tile < num_tiles; tile += stride) {
+    const int start = offsets[tile];
+    const int end = offsets[tile + 1];
+    if (start < 0 || end < start || end > num_cand || (tile == 0 && start != 0) ||
+        (tile == num_tiles - 1 && end != num_cand)) {
+      atomicOr(status, 1);
+      continue;
+    }
+    const int count = end - start;
+    if (capacity > 0 && count > capacity) {
+      atomicOr(status, 2);
+      atomicMax(status + 1, count);
+    }
+  }
+  bool invalid = false;
+  for (int64_t i = first; i < num_cand; i += stride) {
+    const int p = cand[i];
+    invalid |= (p < 0) || (p >= num_prims);
+  }
+  if (invalid) atomicOr(status, 4);
+}
+
+// ---------------------------------------------------------------------------------------------
+// per-tile key + stable sort.  One 256-thread workgroup per tile.  Each candidate becomes the
+// 64-bit word (key bits << 32 | list index): keys are positive floats, whose bit patterns order
+// like their values, and the list index in the low word makes equal keys keep list order, which
+// is what a stable radix sort on the key alone yields.  Bitonic network in LDS on the next power
+// of two, padded with all-ones words.
+// ---------------------------------------------------------------------------------------------
+constexpr int kSortThreads = 256;
+constexpr int kSortMax = MLPSP_TILE_CAPACITY_MAX;
+
+__global__ __launch_bounds__(kSortThreads) void sort_tiles_kernel(
+    const float* __restrict__ rays_o, const float* __restrict__ rays_d, const PrimRecord* __restrict__ prims,
+    const int32_t* __restrict__ cand, const int32_t* __restrict__ offsets, TileGeom g, int family, int capacity,
+    int32_t* __restrict__ sorted_ids, float* __restrict__ sorted_keys) {
+  __shared__ unsigned long long s_key[kSortMax];
+  __shared__ int32_t s_id[kSortMax];
+  const int tile = blockIdx.x;
+  const int tid = threadIdx.x;
+  const int start = offsets[tile];
+  const int len = offsets[tile + 1] - start;
+  if (len <= 0) return;
+  const int n = len < capacity ? len : capacity;
+
+  const int pc = centre_pixel(g, tile);
+  const float ox = rays_o[pc * 3 + 0], oy = rays_o[pc * 3 + 1], oz = rays_o[pc * 3 + 2];
+  const float dx = rays_d[pc * 3 + 0], dy = rays_d[pc * 3 + 1], dz = rays_d[pc * 3 + 2];
+
+  int npad = 2;
+  while (npad < n) npad <<= 1;
+
+  for (int i = tid; i < npad; i += kSortThreads) {
+    unsigned long long w = ~0ull;
+    if (i < n) {
+      const int p = cand[start + i];
+      s_id[i] = p;
+      const PrimRecord P = prims[p];
+      const float key = (family == MLPSP_KEY_DEPTH) ? key_depth(ox, oy, oz, dx, dy, dz, P)
+                                                    : key_tstar(ox, oy, oz, dx, dy, dz, P);
+      w = ((unsigned long long)float_to_bits(key) << 32) | (unsigned)i;
+    }
+    s_key[i] = w;
+  }
+  __syncthreads();
+
+  for (int k = 2; k <= npad; k <<= 1) {
+    for (int j = k >> 1; j > 0; j >>= 1) {
+      for (int t = tid; t < (npad >> 1); t += kSortThreads) {
+        const int lo = ((t & ~(j - 1)) << 1) | (t & (j - 1));
+        const int hi = lo | j;
+        const unsigned long long a = s_key[lo], b = s_key[hi];
+        const bool ascending = (lo & k) == 0;
+        if ((a > b) == ascending) {
+          s_key[lo] = b;
+          s_key[hi] = a;
+        }
+      }
+      __syncthreads();
+    }
+  }
+
+  for (int i = tid; i < len; i += kSortThreads) {
+    if (i < n) {
+      const unsigned long long w = s_key[i];
+      sorted_ids[start + i] = s_id[(int)(w & 0xffffffffu)];
+      if (sorted_keys) sorted_keys[start + i] = bits_to_float((uint32_t)(w >> 32));
+    } else {
+      sorted_ids[start + i] = cand[start + i];
+      if (sorted_keys) sorted_keys[start + i] = kInvalidKey;
+    }
+  }
+}
+
+}  // namespace mlpsp
+
+using namespace mlpsp;
+
+MLPSP_API int mlpsp_version(void) { return 100; }
+
+MLPSP_API const char* mlpsp_strerror(int code) {
+  switch (code) {
+    case MLPSP_OK: return "ok";
+    case MLPSP_E_OFFSETS:
+      return "tile_offsets must start at zero, end at the candidate-list length, and be monotonic/in bounds";
+    case MLPSP_E_CAPACITY:
+      return "tile candidate capacity exceeded; refusing to truncate or use an inconsistent forward/backward order";
+    case MLPSP_E_IDS: return "candidate primitive IDs must be in [0, num_primitives)";
+    case MLPSP_E_PIXEL_OVERFLOW:
+      return "per-pixel intersection capacity 256 exceeded; refusing to return a silently truncated result";
+    case MLPSP_E_NONFINITE: return "non-finite operand or activation in the reduced-precision MLP";
+    case MLPSP_E_ARGUMENT: return "invalid argument";
+    case MLPSP_E_RUNTIME: return "HIP runtime error";
+    case MLPSP_E_SCRATCH: return "scratch buffer too small for this input";
+    default: return "unknown mlpsp status";
+  }
+}
+
+MLPSP_API int mlpsp_prepare_primitives(const float* positions_dev, const float* log_scales_dev,
+                                       const float* quats_dev, int num_primitives, void* prim_records_dev,
+                                       mlpsp_stream_t stream) {
+  if (num_primitives < 0) return MLPSP_E_ARGUMENT;
+  if (num_primitives == 0) return MLPSP_OK;
+  if (!positions_dev || !log_scales_dev || !quats_dev || !prim_records_dev) return MLPSP_E_ARGUMENT;
+  if (reinterpret_cast<uintptr_t>(prim_records_dev) % 64 != 0) return MLPSP_E_ARGUMENT;
+  hipLaunchKernelGGL(prepare_primitives_kernel, dim3(ceil_div(num_primitives, 256)), dim3(256), 0,
+                     (hipStream_t)stream, positions_dev, log_scales_dev, quats_dev, num_primitives,
+                     (PrimRecord*)prim_records_dev);
+  MLPSP_LAUNCH_CHECK();
+  return MLPSP_OK;
+}
+
+MLPSP_API int mlpsp_validate_tile_lists(const int32_t* tile_offsets_dev, const int32_t* candidates_dev,
+                                        int num_tiles, int num_candidates, int capacity, int num_primitives,
+                                        int32_t* status_dev, int32_t status_host[2], mlpsp_stream_t stream) {
+  if (num_tiles <= 0 || num_candidates < 0 || num_primitives < 0 || !tile_offsets_dev || !status_dev || !status_host)
+    return MLPSP_E_ARGUMENT;
+  if (num_candidates > 0 && !candidates_dev) return MLPSP_E_ARGUMENT;
+  hipStream_t s = (hipStream_t)stream;
+  MLPSP_HIP_TRY(hipMemsetAsync(status_dev, 0, 2 * sizeof(int32_t), s));
+  const int64_t work = num_tiles > num_candidates ? num_tiles : num_candidates;
+  int64_t blocks = (work + 255) / 256;
+  if (blocks > 4096) blocks = 4096;
+  hipLaunchKernelGGL(validate_tile_lists_kernel, dim3((unsigned)blocks), dim3(256), 0, s, tile_offsets_dev,
+                     candidates_dev, num_tiles, num_candidates, capacity, num_primitives, status_dev);
+  MLPSP_LAUNCH_CHECK();
+  MLPSP_HIP_TRY(hipMemcpyAsync(status_host, status_dev, 2 * sizeof(int32_t), hipMemcpyDeviceToHost, s));
+  MLPSP_HIP_TRY(hipStreamSynchronize(s));
+  int mask = status_host[0] & (MLPSP_E_OFFSETS | MLPSP_E_CAPACITY | MLPSP_E_IDS);
+  if (capacity <= 0) mask &= ~MLPSP_E_CAPACITY;
+  return mask;
+}
+
+MLPSP_API int mlpsp_sort_tiles(const float* rays_o_dev, const float* rays_d_dev, const void* prim_records_dev,
+                               const int32_t* candidates_dev, const int32_t* tile_offsets_dev, int width,
+                               int height, int tile_w, int tile_h, int key_family, int capacity,
+                               int32_t* sorted_ids_dev, float* sorted_keys_dev, mlpsp_stream_t stream) {
+  const int64_t T = checked_num_tiles(width, height, tile_w, tile_h);
+  if (T <= 0 || T > 2147483647LL) return MLPSP_E_ARGUMENT;
+  if (key_family != MLPSP_KEY_TSTAR && key_family != MLPSP_KEY_DEPTH) return MLPSP_E_ARGUMENT;
+  if (capacity < 0 || capacity > MLPSP_TILE_CAPACITY_MAX) return MLPSP_E_ARGUMENT;
+  if (capacity == 0) capacity = MLPSP_TILE_CAPACITY_MAX;
+  if (!rays_o_dev || !rays_d_dev || !tile_offsets_dev) return MLPSP_E_ARGUMENT;
+  TileGeom g{width, height, tile_w, tile_h, ceil_div(width, tile_w), ceil_div(height, tile_h)};
+  hipLaunchKernelGGL(sort_tiles_kernel, dim3((unsigned)T), dim3(kSortThreads), 0, (hipStream_t)stream, rays_o_dev,
+                     rays_d_dev, (const PrimRecord*)prim_records_dev, candidates_dev, tile_offsets_dev, g, key_family,
+                     capacity, sorted_ids_dev, sorted_keys_dev);
+  MLPSP_LAUNCH_CHECK();
+  return MLPSP_OK;
+}

@@ -1,0 +1,148 @@
+"""Torch-level wrappers of the C ABI: tensors in, tensors out, kernels on the current stream.
+
+PyTorch is used for device memory and the stream only.  Every function here ends in a call into
+``libmlpsp_hip.so``; none has a PyTorch or CPU fallback.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import math
+
+import torch
+
+from . import _lib
+
+TILE_CAPACITY_DEFAULT = 1536  # scannet/cumodel.py:102
+
+
+def _check(code: int, what: str) -> None:
+    if code != 0:
+        msgs = [_lib.strerror(bit) for bit in (1, 2, 4, 8, 16, 32, 64, 128) if code & bit]
+        raise RuntimeError(f"{what}: " + "; ".join(msgs))
+
+
+def _ptr(t):
+    return None if t is None else C.c_void_p(t.data_ptr())
+
+
+def _stream(device):
+    return C.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+
+
+def _f32c(t, name):
+    if not (t.is_cuda and t.dtype == torch.float32):
+        raise RuntimeError(f"{name} must be a float32 tensor on the GPU")
+    return t if t.is_contiguous() else t.contiguous()
+
+
+def num_tiles(W: int, H: int, TW: int, TH: int) -> int:
+    return ((W + TW - 1) // TW) * ((H + TH - 1) // TH)
+
+
+def prepare_primitives(positions, log_scales, quats):
+    """[N,3],[N,3],[N,4] -> opaque per-primitive geometry records (uint8 [N*64])."""
+    positions, log_scales, quats = _f32c(positions, "positions"), _f32c(log_scales, "log_scales"), _f32c(quats, "quats")
+    n = positions.shape[0]
+    rec = torch.empty(max(n, 1) * _lib.PRIM_RECORD_BYTES, dtype=torch.uint8, device=positions.device)
+    code = _lib.load().mlpsp_prepare_primitives(_ptr(positions), _ptr(log_scales), _ptr(quats), n, _ptr(rec),
+                                                _stream(positions.device))
+    _check(code, "mlpsp_prepare_primitives")
+    return rec
+
+
+def validate_tile_lists(candidates, tile_offsets, n_tiles: int, capacity: int, num_primitives: int, path_name: str):
+    """Raise the reference's RuntimeError texts (np_tile_kernels.cu:4578-4588) for a bad tile list."""
+    for t, nm in ((candidates, "culled_prim_indices"), (tile_offsets, "tile_offsets")):
+        if not (t.is_cuda and t.dtype == torch.int32 and t.dim() == 1 and t.is_contiguous()):
+            raise RuntimeError(f"{path_name}: {nm} must be a contiguous CUDA int32 vector")
+    if tile_offsets.numel() != n_tiles + 1:
+        raise RuntimeError(f"{path_name}: tile_offsets length mismatch (got {tile_offsets.numel()}, "
+                           f"expected {n_tiles + 1})")
+    status_dev = torch.empty(2, dtype=torch.int32, device=candidates.device)
+    status = (C.c_int32 * 2)()
+    code = _lib.load().mlpsp_validate_tile_lists(_ptr(tile_offsets), _ptr(candidates), n_tiles, candidates.numel(),
+                                                 int(capacity), int(num_primitives), _ptr(status_dev), status,
+                                                 _stream(candidates.device))
+    if code & _lib.E_OFFSETS:
+        raise RuntimeError(f"{path_name}: tile_offsets must start at zero, end at the candidate-list length, "
+                           "and be monotonic/in bounds")
+    if code & _lib.E_CAPACITY:
+        raise RuntimeError(f"{path_name}: tile candidate capacity {capacity} exceeded (maximum observed tile length "
+                           f"{status[1]}); refusing to truncate or use an inconsistent forward/backward order")
+    if code & _lib.E_IDS:
+        raise RuntimeError(f"{path_name}: candidate primitive IDs must be in [0, num_primitives)")
+    _check(code, path_name)
+
+
+def bin_legacy(positions, log_scales, view_matrices, proj_matrix, W: int, H: int, tile: int, threshold: float,
+               tile_view_ids=None):
+    """Sparse form of the reference's screen-space culling (scannet/cumodel.py:994-1070, 838-949).
+
+    view_matrices [K,4,4] / proj_matrix [4,4] may live on any device (they are read on the host).
+    Returns (culled_prim_indices int32 [P], tile_offsets int32 [T+1]); ids ascend inside a tile.
+    """
+    positions, log_scales = _f32c(positions, "positions"), _f32c(log_scales, "log_scales")
+    dev = positions.device
+    vm = view_matrices.detach().to("cpu", torch.float32).reshape(-1, 4, 4).contiguous()
+    pm = proj_matrix.detach().to("cpu", torch.float32).reshape(4, 4).contiguous()
+    K, n = vm.shape[0], positions.shape[0]
+    T = num_tiles(W, H, tile, tile)
+    tv = None
+    if tile_view_ids is not None:
+        tv = tile_view_ids.to(device=dev, dtype=torch.int32).contiguous()
+        if tv.numel() != T:
+            raise ValueError(f"tile_view_ids length mismatch: got {tv.numel()}, expected {T}")
+    lib = _lib.load()
+    offsets = torch.empty(T + 1, dtype=torch.int32, device=dev)
+    fp = C.POINTER(C.c_float)
+    nbytes = lib.mlpsp_bin_scratch_bytes(n, K, W, H, tile)
+    total = C.c_int64(0)
+    for _ in range(6):
+        scratch = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+        code = lib.mlpsp_bin_legacy_count(_ptr(positions), _ptr(log_scales), n, C.cast(vm.data_ptr(), fp), K, _ptr(tv),
+                                          C.cast(pm.data_ptr(), fp), W, H, tile, float(threshold), _ptr(scratch),
+                                          nbytes, _ptr(offsets), C.byref(total), _stream(dev))
+        if code != _lib.E_SCRATCH:
+            break
+        nbytes *= 4
+    _check(code, "mlpsp_bin_legacy_count")
+    cand = torch.empty(int(total.value), dtype=torch.int32, device=dev)
+    if total.value > 0:
+        code = lib.mlpsp_bin_legacy_fill(n, K, _ptr(tv), W, H, tile, _ptr(scratch), nbytes, _ptr(offsets), _ptr(cand),
+                                         _stream(dev))
+        _check(code, "mlpsp_bin_legacy_fill")
+    return cand, offsets
+
+
+def sort_tiles(rays_o, rays_d, records, candidates, tile_offsets, W, H, TW, TH, family=_lib.KEY_TSTAR,
+               capacity=TILE_CAPACITY_DEFAULT, want_keys=False):
+    """Materialised per-tile depth order: (sorted_ids [P], sorted_keys [P] | None)."""
+    dev = rays_o.device
+    sorted_ids = torch.empty_like(candidates)
+    keys = torch.empty(candidates.numel(), dtype=torch.float32, device=dev) if want_keys else None
+    code = _lib.load().mlpsp_sort_tiles(_ptr(rays_o), _ptr(rays_d), _ptr(records), _ptr(candidates), _ptr(tile_offsets),
+                                        W, H, TW, TH, int(family), int(capacity), _ptr(sorted_ids), _ptr(keys),
+                                        _stream(dev))
+    _check(code, "mlpsp_sort_tiles")
+    return sorted_ids, keys
+
+
+def render_tilecenter_f32(rays_o, rays_d, records, order, tile_offsets, freq, att, W1, b1, W2, b2, W3, b3, W, H, TW,
+                          TH, threshold, with_t=False, counters=None):
+    """Scalar-f32 tile-centre forward over materialised per-tile orders -> (rgb, alpha, t|None)."""
+    dev = rays_o.device
+    B = W * H
+    rgb = torch.empty(B, 3, dtype=torch.float32, device=dev)
+    alpha = torch.empty(B, 1, dtype=torch.float32, device=dev)
+    t = torch.empty(B, 1, dtype=torch.float32, device=dev) if with_t else None
+    n, hidden, F = W1.shape[0], W2.shape[1], freq.shape[0]
+    code = _lib.load().mlpsp_render_tilecenter_f32(
+        _ptr(rays_o), _ptr(rays_d), _ptr(records), _ptr(order), _ptr(tile_offsets), _ptr(freq), _ptr(att), F,
+        _ptr(W1), _ptr(b1), _ptr(W2), _ptr(b2), _ptr(W3), _ptr(b3), n, hidden, W, H, TW, TH, float(threshold),
+        _ptr(rgb), _ptr(alpha), _ptr(t), _ptr(counters), _stream(dev))
+    _check(code, "mlpsp_render_tilecenter_f32")
+    return rgb, alpha, t
+
+
+def radius_multiplier(threshold: float) -> float:
+    return math.sqrt(-2.0 * math.log(threshold))
