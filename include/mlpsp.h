@@ -36,6 +36,8 @@ extern "C" {
 #define MLPSP_E_ARGUMENT 32      /* a size or pointer argument is unusable */
 #define MLPSP_E_RUNTIME 64       /* a HIP call failed */
 #define MLPSP_E_SCRATCH 128      /* the scratch buffer is too small for this input: retry with a larger one */
+#define MLPSP_E_MIXED_ORIGINS 256 /* ray-cone binning: a tile's rays do not share one origin (camera.py:121-122) */
+#define MLPSP_E_WIDE_CONE 512    /* ray-cone binning: a tile's ray cone spans >= 90 degrees (camera.py:126) */
 
 #define MLPSP_TILE_CAPACITY_MAX 2048 /* largest per-tile list the in-LDS sort accepts */
 #define MLPSP_PIXEL_HIT_CAPACITY 256 /* per-pixel-order hit buffer (np_tile_kernels.cu:760) */
@@ -86,6 +88,18 @@ int mlpsp_bin_legacy_fill(int num_primitives, int num_views, const int32_t* tile
                           int height, int tile, const void* scratch_dev, size_t scratch_bytes,
                           const int32_t* tile_offsets_dev, int32_t* candidates_dev, mlpsp_stream_t stream);
 
+/* Ray-cone culling from the actual rays = ray_cone_candidates (scannet/camera.py:102-146), for
+ * cameras that are not a centred pinhole.  Same two steps and blocking behaviour as the legacy
+ * binning; tile <= 16.  Within a tile, candidate ids ascend. */
+size_t mlpsp_bin_raycone_scratch_bytes(int num_primitives, int width, int height, int tile);
+int mlpsp_bin_raycone_count(const float* rays_o_dev, const float* rays_d_dev, const float* positions_dev,
+                            const float* log_scales_dev, int num_primitives, int width, int height, int tile,
+                            float threshold, void* scratch_dev, size_t scratch_bytes, int32_t* tile_offsets_dev,
+                            int64_t* num_pairs_out, mlpsp_stream_t stream);
+int mlpsp_bin_raycone_fill(int num_primitives, int width, int height, int tile, const void* scratch_dev,
+                           size_t scratch_bytes, const int32_t* tile_offsets_dev, int32_t* candidates_dev,
+                           mlpsp_stream_t stream);
+
 /* Per-tile depth-key sort = the in-kernel cub::BlockRadixSort of np_tile_kernels.cu:1929-1990,
  * materialised: sorted_ids_dev[P] holds, tile by tile, the candidates in ascending key order, ties
  * in list order; entries past min(len, capacity) keep list order.  sorted_keys_dev may be NULL.
@@ -107,6 +121,35 @@ int mlpsp_render_tilecenter_f32(const float* rays_o_dev, const float* rays_d_dev
                                 int num_primitives, int hidden, int width, int height, int tile_w, int tile_h,
                                 float threshold, float* out_rgb_dev, float* out_alpha_dev, float* out_t_dev,
                                 int64_t* counters_dev, mlpsp_stream_t stream);
+
+/* Tile-centre-order forward with the gated feature channel, scalar f32
+ * (render_tiles_kernel_tilecenter_order_with_feat, np_tile_kernels.cu:5794-6112).
+ * feat_slots: 1 (feat_attr [N,C]), 4 or 5 ([N,slots,C]); feat_channels <= 512.
+ * out_feat_dev [B,C] is fully written (no pre-zeroing needed). */
+int mlpsp_render_tilecenter_feat_f32(const float* rays_o_dev, const float* rays_d_dev, const void* prim_records_dev,
+                                     const int32_t* order_dev, const int32_t* tile_offsets_dev,
+                                     const float* freq_dev, const float* att_dev, int num_frequencies,
+                                     const float* W1, const float* b1, const float* W2, const float* b2,
+                                     const float* W3, const float* b3, int num_primitives, int hidden,
+                                     const float* feat_attr_dev, int feat_slots, int feat_channels,
+                                     float gating_beta, float gating_temp, int width, int height, int tile_w,
+                                     int tile_h, float threshold, float* out_rgb_dev, float* out_alpha_dev,
+                                     float* out_feat_dev, mlpsp_stream_t stream);
+
+/* Per-pixel-order forward (render_tiles_kernel_with_sort[_and_feat], np_tile_kernels.cu:715-1208):
+ * every pixel blends its own hits in order of its own t.  candidates_dev is the unsorted tile list.
+ * out_feat_dev == NULL renders RGB only.  workspace_dev: mlpsp_per_pixel_workspace_bytes() bytes,
+ * 256-byte aligned.  BLOCKS (one 4-byte readback): returns MLPSP_E_PIXEL_OVERFLOW if some pixel
+ * met a 257th hit, in which case the outputs must be discarded. */
+size_t mlpsp_per_pixel_workspace_bytes(int width, int height, int tile_w, int tile_h);
+int mlpsp_render_per_pixel_f32(const float* rays_o_dev, const float* rays_d_dev, const void* prim_records_dev,
+                               const int32_t* candidates_dev, const int32_t* tile_offsets_dev, const float* freq_dev,
+                               const float* att_dev, int num_frequencies, const float* W1, const float* b1,
+                               const float* W2, const float* b2, const float* W3, const float* b3,
+                               int num_primitives, int hidden, const float* feat_attr_dev, int feat_slots,
+                               int feat_channels, float gating_beta, float gating_temp, int width, int height,
+                               int tile_w, int tile_h, float threshold, void* workspace_dev, size_t workspace_bytes,
+                               float* out_rgb_dev, float* out_alpha_dev, float* out_feat_dev, mlpsp_stream_t stream);
 
 #ifdef __cplusplus
 }

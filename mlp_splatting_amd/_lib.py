@@ -14,6 +14,7 @@ LIB_PATH = os.path.join(_HERE, "libmlpsp_hip.so")
 CSRC_DIR = os.path.join(_HERE, "csrc")
 
 E_OFFSETS, E_CAPACITY, E_IDS, E_PIXEL_OVERFLOW, E_NONFINITE, E_ARGUMENT, E_RUNTIME, E_SCRATCH = 1, 2, 4, 8, 16, 32, 64, 128
+E_MIXED_ORIGINS, E_WIDE_CONE = 256, 512
 KEY_LIST_ORDER, KEY_TSTAR, KEY_DEPTH = 0, 1, 2
 TILE_CAPACITY_MAX = 2048
 PIXEL_HIT_CAPACITY = 256
@@ -31,9 +32,17 @@ SIGNATURES = {
     "mlpsp_bin_legacy_count": (_i, [_vp, _vp, _i, C.POINTER(_f), _i, _vp, C.POINTER(_f), _i, _i, _i, _f, _vp, _sz, _vp,
                                     C.POINTER(_i64), _vp]),
     "mlpsp_bin_legacy_fill": (_i, [_i, _i, _vp, _i, _i, _i, _vp, _sz, _vp, _vp, _vp]),
+    "mlpsp_bin_raycone_scratch_bytes": (_sz, [_i, _i, _i, _i]),
+    "mlpsp_bin_raycone_count": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _f, _vp, _sz, _vp, C.POINTER(_i64), _vp]),
+    "mlpsp_bin_raycone_fill": (_i, [_i, _i, _i, _i, _vp, _sz, _vp, _vp, _vp]),
     "mlpsp_sort_tiles": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp]),
     "mlpsp_render_tilecenter_f32": (_i, [_vp] * 7 + [_i] + [_vp] * 6 + [_i, _i, _i, _i, _i, _i, _f, _vp, _vp, _vp,
                                                                        _vp, _vp]),
+    "mlpsp_render_tilecenter_feat_f32": (_i, [_vp] * 7 + [_i] + [_vp] * 6 + [_i, _i, _vp, _i, _i, _f, _f, _i, _i, _i, _i,
+                                                                            _f, _vp, _vp, _vp, _vp]),
+    "mlpsp_per_pixel_workspace_bytes": (_sz, [_i, _i, _i, _i]),
+    "mlpsp_render_per_pixel_f32": (_i, [_vp] * 7 + [_i] + [_vp] * 6 + [_i, _i, _vp, _i, _i, _f, _f, _i, _i, _i, _i, _f,
+                                                                      _vp, _sz, _vp, _vp, _vp, _vp]),
 }
 
 _lib = None

@@ -158,6 +158,8 @@ MLPSP_API const char* mlpsp_strerror(int code) {
     case MLPSP_E_ARGUMENT: return "invalid argument";
     case MLPSP_E_RUNTIME: return "HIP runtime error";
     case MLPSP_E_SCRATCH: return "scratch buffer too small for this input";
+    case MLPSP_E_MIXED_ORIGINS: return "Each tile must use a single camera origin";
+    case MLPSP_E_WIDE_CONE: return "Tile ray cone spans >=90 degrees";
     default: return "unknown mlpsp status";
   }
 }

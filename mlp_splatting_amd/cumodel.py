@@ -1,0 +1,464 @@
+"""Scene module with the Python-facing API of the reference's ``scannet/cumodel.py``, forward only.
+
+Same module-level names (``_tile_ext``, ``_tile_ext_key``, ``_tile_ext_build_config``, the two
+encodings, ``_encode_x6``, ``_mlp_forward_indexed``) and the same class
+``NeuralPrimitiveSceneTileCUDA`` (constructor arguments, parameter names and shapes, methods,
+error behaviour), so that code written against the reference module -- an evaluator, a benchmark
+harness, a test that monkeypatches ``_tile_ext`` -- runs against this one.  What differs is below
+the API: culling is the sparse HIP binning instead of a dense [tiles x primitives] tensor
+expression, and the extension object is ``tile_ext.TileExt`` on ``libmlpsp_hip.so``.
+
+Training (autograd backward, record emission) is outside this build: ``forward`` returns tensors
+without a graph.
+"""
+from __future__ import annotations
+
+import os
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from . import ops
+from .camera import ray_cone_candidates
+
+# Extension object, created on first use; tests may install their own (scannet/cumodel.py:78-80).
+_tile_ext = None
+_tile_error = None
+_tile_ext_key = None
+
+
+def _tile_ext_build_config(tile_size=None):
+    """(key, name, flags) naming the extension build selected by the environment
+    (scannet/cumodel.py:96-130).  The capacities the reference bakes in at compile time are run-time
+    arguments of this library, but names, accepted values and errors are kept."""
+    rreg = os.environ.get("MLPSP_NVCC_MAXRREGCOUNT", "").strip()
+    flags = []
+    suffix = "default"
+    capacity = int(os.environ.get("MLPSP_TILE_CANDIDATE_CAPACITY", "1536"))
+    if capacity not in {768, 1536}:
+        raise ValueError("MLPSP_TILE_CANDIDATE_CAPACITY must be 768 or 1536")
+    if os.environ.get("MLPSP_TRAINING_BACKEND", "legacy") == "csr":
+        hits = int(os.environ.get("MLPSP_CSR_MAX_HITS", "128"))
+        if hits not in {128, 256, 512}:
+            raise ValueError("MLPSP_CSR_MAX_HITS must be 128, 256 or 512; overflow is an error")
+        flags += ["-DMLPSP_TILECENTER_BLOCK_THREADS=64", "-DMLPSP_BACKWARD_RECOMPUTE_GEOMETRY=1",
+                  f"-DMLPSP_TILECENTER_MAX_HITS={hits}", "-DMLPSP_BACKWARD_MIN_BLOCKS_PER_SM=8"]
+        suffix = f"csr_h{hits}"
+    if capacity != 768:
+        flags.append(f"-DMLPSP_MAX_TILE_PRIMS={capacity}")
+        suffix += f"_c{capacity}"
+    if rreg:
+        try:
+            value = int(rreg)
+        except ValueError:
+            value = 0
+        if value > 0:
+            flags.append(f"-maxrregcount={value}")
+            suffix += f"_rreg{value}"
+    name = f"np_tile_kernels_{suffix}"
+    return (name, tuple(flags)), name, flags
+
+
+def _tile_capacity_from_env() -> int:
+    return int(os.environ.get("MLPSP_TILE_CANDIDATE_CAPACITY", "1536"))
+
+
+class IntegratedPositionalEncoding(nn.Module):
+    """freq_k = 2^k pi; the attenuation exp(-freq^2 sigma^2 / 2) scales the phase
+    (scannet/cumodel.py:132-155)."""
+
+    def __init__(self, in_dim=6, num_frequencies=10, sigma=0.01):
+        super().__init__()
+        self.in_dim = in_dim
+        self.num_frequencies = num_frequencies
+        self.sigma2 = sigma ** 2
+        self.register_buffer("freq_bands", 2.0 ** torch.linspace(0.0, num_frequencies - 1, num_frequencies) * torch.pi)
+        self.register_buffer("runtime_frequency_weights", torch.ones(num_frequencies), persistent=False)
+
+    def set_runtime_frequency_weights(self, weights: torch.Tensor):
+        with torch.no_grad():
+            self.runtime_frequency_weights.copy_(
+                weights.to(device=self.runtime_frequency_weights.device, dtype=self.runtime_frequency_weights.dtype))
+
+    def forward(self, x):
+        att = torch.exp(-0.5 * (self.freq_bands ** 2) * self.sigma2) * self.runtime_frequency_weights
+        phase = (x[..., None] * self.freq_bands * att).view(*x.shape[:-1], -1)
+        return torch.cat([torch.sin(phase), torch.cos(phase)], dim=-1)
+
+    @property
+    def out_dim(self):
+        return self.in_dim * self.num_frequencies * 2
+
+
+class FourierFeatureEncoding(nn.Module):
+    """freq_k = 2^k, amplitude weights (scannet/cumodel.py:158-180)."""
+
+    def __init__(self, in_dim=6, num_frequencies=10):
+        super().__init__()
+        self.in_dim = in_dim
+        self.num_frequencies = num_frequencies
+        self.register_buffer("freq_bands", 2.0 ** torch.linspace(0.0, num_frequencies - 1, num_frequencies))
+        self.register_buffer("runtime_frequency_weights", torch.ones(num_frequencies), persistent=False)
+
+    def set_runtime_frequency_weights(self, weights: torch.Tensor):
+        with torch.no_grad():
+            self.runtime_frequency_weights.copy_(
+                weights.to(device=self.runtime_frequency_weights.device, dtype=self.runtime_frequency_weights.dtype))
+
+    def forward(self, x):
+        phase = x[..., None] * self.freq_bands
+        w = self.runtime_frequency_weights.view(*([1] * (phase.ndim - 1)), self.num_frequencies)
+        s = (torch.sin(phase) * w).view(*x.shape[:-1], -1)
+        c = (torch.cos(phase) * w).view(*x.shape[:-1], -1)
+        return torch.cat([s, c], dim=-1)
+
+    @property
+    def out_dim(self):
+        return self.in_dim * self.num_frequencies * 2
+
+
+def _encode_x6(x6: torch.Tensor, freq: torch.Tensor, att: torch.Tensor) -> torch.Tensor:
+    """[M,6] -> [M,12F]: all sines (index c*F+f) then all cosines (scannet/cumodel.py:183-190)."""
+    phase = x6[:, :, None] * freq[None, None, :] * att[None, None, :]
+    m = x6.shape[0]
+    return torch.cat([torch.sin(phase).reshape(m, -1), torch.cos(phase).reshape(m, -1)], dim=-1)
+
+
+def _mlp_forward_indexed(x_enc, prim_ids, W1, b1, W2, b2, W3, b3):
+    """Per-record MLP with gathered weights -> (rgb [M,3], sigma_raw [M,1]) (scannet/cumodel.py:193-216)."""
+    hcap = min(int(W1.shape[1]), 64)
+    w1 = W1.index_select(0, prim_ids)[:, :hcap, :]
+    c1 = b1.index_select(0, prim_ids)[:, :hcap]
+    w2 = W2.index_select(0, prim_ids)[:, :hcap, :hcap]
+    c2 = b2.index_select(0, prim_ids)[:, :hcap]
+    w3 = W3.index_select(0, prim_ids)[:, :, :hcap]
+    c3 = b3.index_select(0, prim_ids)
+    h = F.relu(torch.einsum("mhi,mi->mh", w1, x_enc) + c1)
+    h = F.relu(torch.einsum("moh,mh->mo", w2, h) + c2)
+    o = torch.einsum("moh,mh->mo", w3, h) + c3
+    return torch.sigmoid(o[:, :3]), F.softplus(o[:, 3:4])
+
+
+def _add_background(rgb, alpha, bg):
+    """rgb + clamp(1 - alpha, 0, 1) * bg (scannet/cumodel.py:252-256)."""
+    if bg is None:
+        return rgb
+    if bg.numel() == 1:
+        bg = bg.repeat(3)
+    return rgb + (1.0 - alpha).clamp(0.0, 1.0) * bg.view(1, 3)
+
+
+class NeuralPrimitiveSceneTileCUDA(nn.Module):
+    """Tile-based single-pass MLP-splatting renderer: full-frame rays in, image out.
+
+    Call ``set_image_size`` first; ``forward`` needs ``B == W*H`` rays.
+    """
+
+    requires_full_image = True
+
+    def __init__(self, num_primitives=1024, hidden_dim=32, pe_frequencies=6, initial_positions=None,
+                 use_integrated_pe=True, pe_sigma: float = 0.01, min_points: int = 10, tile_size: int = 8,
+                 feature_dim_low: int = 0, feature_slots: int = 4, feature_gating_beta: float = 1.5,
+                 feature_gating_temp: float = 2.0):
+        super().__init__()
+        if int(hidden_dim) > 32:
+            raise ValueError("NeuralPrimitiveSceneTileCUDA currently supports hidden_dim <= 32 "
+                             "(kernel scratch-cap tuning in backward/full path).")
+        self.num_primitives = num_primitives
+        self.hidden_dim = hidden_dim
+        self.pe_frequencies = pe_frequencies
+        self.use_integrated_pe = bool(use_integrated_pe)
+        self.pe_sigma = float(pe_sigma)
+        if self.pe_sigma <= 0.0:
+            raise ValueError("pe_sigma must be > 0.")
+        self.image_size = None
+        self.tile_size = int(tile_size)
+        if self.tile_size <= 0:
+            raise ValueError("tile_size must be a positive integer.")
+        if self.tile_size not in (8, 16):
+            raise ValueError("NeuralPrimitiveSceneTileCUDA supports tile_size in {8, 16}.")
+        self.tile_order_mode_override = None
+        self.feature_dim_low = int(max(0, feature_dim_low))
+        self.feature_slots = int(max(1, feature_slots))
+        self.feature_gating_beta = float(feature_gating_beta)
+        self.feature_gating_temp = float(feature_gating_temp)
+        if self.feature_dim_low > 0 and self.feature_slots not in (4, 5):
+            raise ValueError("feature_slots must be 4 (canonical) or 5 (legacy) when features are enabled.")
+        if self.feature_gating_beta <= 0.0:
+            raise ValueError("feature_gating_beta must be > 0.")
+        if self.feature_gating_temp <= 0.0:
+            raise ValueError("feature_gating_temp must be > 0.")
+
+        if initial_positions is not None:
+            raise NotImplementedError("octree initialisation from a point cloud belongs to the training side; "
+                                      "construct with num_primitives and load a state dict instead")
+        n = int(num_primitives)
+        self.positions = nn.Parameter(torch.rand(n, 3) * 2.0 - 1.0)
+        self.log_scales = nn.Parameter(torch.log(torch.ones(n) * 0.1).unsqueeze(-1).repeat(1, 3))
+        self.quats = nn.Parameter(torch.tensor([1.0, 0.0, 0.0, 0.0]).view(1, 4).repeat(n, 1))
+        if self.use_integrated_pe:
+            self.encoder = IntegratedPositionalEncoding(in_dim=6, num_frequencies=pe_frequencies, sigma=self.pe_sigma)
+        else:
+            self.encoder = FourierFeatureEncoding(in_dim=6, num_frequencies=pe_frequencies)
+        enc, h = self.encoder.out_dim, hidden_dim
+        self.W1 = nn.Parameter(torch.randn(n, h, enc) * 0.01)
+        self.b1 = nn.Parameter(torch.zeros(n, h))
+        self.W2 = nn.Parameter(torch.randn(n, h, h) * 0.01)
+        self.b2 = nn.Parameter(torch.zeros(n, h))
+        self.W3 = nn.Parameter(torch.randn(n, 4, h) * 0.01)
+        self.b3 = nn.Parameter(torch.zeros(n, 4))
+        if self.feature_dim_low > 0:
+            if self.feature_slots == 5:
+                feat = torch.zeros(n, 5, self.feature_dim_low)
+                feat[:, 0, :].normal_(mean=0.0, std=0.01)
+            else:
+                feat = torch.randn(n, self.feature_slots, self.feature_dim_low) * 0.01
+            self.feat_attr = nn.Parameter(feat)
+        else:
+            self.feat_attr = None
+        self.register_buffer("stat_sum_w", torch.zeros(n, dtype=torch.float32))
+        self.register_buffer("stat_max_w", torch.zeros(n, dtype=torch.float32))
+        self.register_buffer("stat_hits", torch.zeros(n, dtype=torch.int32))
+        self.register_buffer("stat_contrib_count", torch.zeros(n, dtype=torch.int32))
+        self.register_buffer("stat_sum_werr", torch.zeros(n, dtype=torch.float32))
+        self.register_buffer("alpha_accum", torch.zeros(n, dtype=torch.float32))
+
+    # ------------------------------------------------------------------------------------------
+    @torch.no_grad()
+    def reset_w_stats(self):
+        n, dev = self.positions.shape[0], self.positions.device
+        self.stat_sum_w = torch.zeros(n, device=dev, dtype=torch.float32)
+        self.stat_hits = torch.zeros(n, device=dev, dtype=torch.int32)
+        self.stat_max_w = torch.zeros(n, device=dev, dtype=torch.float32)
+        self.stat_sum_werr = torch.zeros(n, device=dev, dtype=torch.float32)
+        self.stat_contrib_count = torch.zeros(n, device=dev, dtype=torch.int32)
+
+    def set_image_size(self, W: int, H: int):
+        self.image_size = (int(W), int(H))
+
+    def _activate_cuda_device(self) -> torch.device:
+        device = self.positions.device
+        if device.type != "cuda":
+            raise RuntimeError("NeuralPrimitiveSceneTileCUDA must be moved to a CUDA device before rendering.")
+        if device.index is None:
+            device = torch.device("cuda", torch.cuda.current_device())
+        torch.cuda.set_device(device.index)
+        return device
+
+    def _resolve_tile_order_mode(self) -> str:
+        mode = self.tile_order_mode_override
+        if mode is None or str(mode).strip() == "":
+            mode = os.environ.get("MLPSP_TILE_ORDER", "tilecenter")
+        mode = str(mode).strip().lower()
+        mode = {"tile_center": "tilecenter", "tile-center": "tilecenter"}.get(mode, mode)
+        if mode not in {"tilecenter", "per_pixel"}:
+            raise ValueError(f"Unsupported tile order {mode!r}; use 'tilecenter' or 'per_pixel'.")
+        return mode
+
+    def _ensure_tile_ext(self):
+        return self._ensure_tile_ext_static()
+
+    @staticmethod
+    def _ensure_tile_ext_static(tile_size=None):
+        """The extension object for the build the environment selects; cached in the module globals
+        ``_tile_ext`` / ``_tile_ext_key`` exactly where the reference caches its JIT module."""
+        global _tile_ext, _tile_ext_key
+        key, _name, _flags = _tile_ext_build_config()
+        if _tile_ext is None or _tile_ext_key != key:
+            from .tile_ext import TileExt
+            _tile_ext = TileExt(max_tile_prims=_tile_capacity_from_env())
+            _tile_ext_key = key
+        return _tile_ext
+
+    # ------------------------------------------------------------------------------------------
+    def _frequency_tables(self, device):
+        """freq and att as the kernels take them (scannet/cumodel.py:1078-1086)."""
+        freq = self.encoder.freq_bands.to(device=device, dtype=torch.float32)
+        if isinstance(self.encoder, IntegratedPositionalEncoding):
+            att = torch.exp(-0.5 * (freq * freq) * float(self.encoder.sigma2))
+        else:
+            att = torch.ones_like(freq)
+        if hasattr(self.encoder, "runtime_frequency_weights"):
+            att = att * self.encoder.runtime_frequency_weights.to(device=device, dtype=torch.float32)
+        return freq.contiguous(), att.contiguous()
+
+    def _legacy_culling(self, view_matrices, proj_matrix, score_threshold, tile_size, tile_view_ids=None):
+        """Screen-space tile lists: same rule as scannet/cumodel.py:994-1070, evaluated sparsely on the GPU."""
+        W, H = self.image_size
+        return ops.bin_legacy(self.positions.detach(), self.log_scales.detach(), view_matrices, proj_matrix, W, H,
+                              int(tile_size), float(score_threshold), tile_view_ids)
+
+    @torch.no_grad()
+    def build_tilecenter_culling_from_tile_views(self, tile_view_ids, view_matrices, proj_matrix,
+                                                 score_threshold: float = 1e-3, tile_size: int | None = None):
+        """Tile lists when every tile takes its rays from one of K views (scannet/cumodel.py:838-949)."""
+        if getattr(self, "camera_mode", "legacy-centered") == "colmap-native":
+            return None, None
+        if self.image_size is None:
+            raise ValueError("image_size must be set before building tile culling.")
+        W, H = self.image_size
+        device = self._activate_cuda_device()
+        tile_size = int(self.tile_size if tile_size is None else tile_size)
+        if tile_size <= 0:
+            raise ValueError("tile_size must be a positive integer.")
+        num_tiles = ops.num_tiles(W, H, tile_size, tile_size)
+        tile_view_ids = tile_view_ids.to(device=device, dtype=torch.long).reshape(-1)
+        if tile_view_ids.numel() != num_tiles:
+            raise ValueError(f"tile_view_ids length mismatch: got {tile_view_ids.numel()}, expected {num_tiles}")
+        if view_matrices.ndim != 3 or view_matrices.shape[1:] != (4, 4):
+            raise ValueError("view_matrices must have shape (K,4,4)")
+        if int(view_matrices.shape[0]) <= 0:
+            raise ValueError("view_matrices must contain at least one view")
+        if int(tile_view_ids.min().item()) < 0 or int(tile_view_ids.max().item()) >= int(view_matrices.shape[0]):
+            raise ValueError("tile_view_ids contains out-of-range view indices")
+        return self._legacy_culling(view_matrices, proj_matrix, score_threshold, tile_size, tile_view_ids)
+
+    def _tile_lists(self, ray_o, ray_d, score_threshold, view_matrix, proj_matrix, culled_prim_indices, tile_offsets,
+                    device, allow_native=True):
+        W, H = self.image_size
+        tile_size = int(self.tile_size)
+        num_tiles = ops.num_tiles(W, H, tile_size, tile_size)
+        external = (culled_prim_indices is not None) or (tile_offsets is not None)
+        if allow_native and getattr(self, "camera_mode", "legacy-centered") == "colmap-native":
+            if external:
+                raise ValueError("Native camera culling must be derived from the actual rays")
+            culled_prim_indices, tile_offsets = ray_cone_candidates(
+                ray_o, ray_d, self.positions, self.log_scales, W, H, tile_size, score_threshold)
+            external = True
+        if external:
+            if culled_prim_indices is None or tile_offsets is None:
+                raise ValueError("Both culled_prim_indices and tile_offsets must be provided together.")
+            culled_prim_indices = culled_prim_indices.to(device=device, dtype=torch.int32)
+            tile_offsets = tile_offsets.to(device=device, dtype=torch.int32)
+            if tile_offsets.numel() != num_tiles + 1:
+                raise ValueError(f"tile_offsets length mismatch: got {tile_offsets.numel()}, expected {num_tiles + 1}")
+            return culled_prim_indices, tile_offsets
+        if view_matrix is None or proj_matrix is None:
+            raise ValueError("Tile renderer requires view_matrix/proj_matrix unless external culling is provided.")
+        return self._legacy_culling(view_matrix.reshape(1, 4, 4), proj_matrix, score_threshold, tile_size)
+
+    def _base_args(self, ray_o, ray_d, culled_prim_indices, tile_offsets, device):
+        freq, att = self._frequency_tables(device)
+        return (ray_o.contiguous(), F.normalize(ray_d, dim=-1).contiguous(), self.positions.detach().contiguous(),
+                self.log_scales.detach().contiguous(), F.normalize(self.quats.detach(), dim=-1).contiguous(),
+                culled_prim_indices, tile_offsets.to(torch.int32), freq, att,
+                self.W1.detach().contiguous(), self.b1.detach().contiguous(), self.W2.detach().contiguous(),
+                self.b2.detach().contiguous(), self.W3.detach().contiguous(), self.b3.detach().contiguous())
+
+    @staticmethod
+    def _background(bg_color, ray_o):
+        if bg_color is None:
+            return None
+        if not torch.is_tensor(bg_color):
+            return torch.tensor(bg_color, dtype=ray_o.dtype, device=ray_o.device)
+        return bg_color.to(ray_o.device, dtype=ray_o.dtype)
+
+    # ------------------------------------------------------------------------------------------
+    def forward(self, ray_o, ray_d, score_threshold=1e-3, bg_color=None, view_matrix=None, proj_matrix=None,
+                culled_prim_indices=None, tile_offsets=None, return_feature: bool = False, feature_target=None):
+        """rgb [B,3], or (rgb, feat [B,C]) with ``return_feature`` (scannet/cumodel.py:951-1160)."""
+        if self.image_size is None:
+            raise ValueError("image_size must be set on NeuralPrimitiveSceneTileCUDA before calling forward.")
+        W, H = self.image_size
+        assert ray_o.shape[0] == W * H, "Tile renderer requires full-frame rays (B == W*H)"
+        device = self._activate_cuda_device()
+        ts = int(self.tile_size)
+        with torch.no_grad():
+            culled_prim_indices, tile_offsets = self._tile_lists(
+                ray_o, ray_d, score_threshold, view_matrix, proj_matrix, culled_prim_indices, tile_offsets, device)
+            use_tilecenter = self._resolve_tile_order_mode() == "tilecenter"
+            ext = self._ensure_tile_ext()
+            if feature_target is not None:
+                if not return_feature or self.feat_attr is None or not use_tilecenter or ts != 8:
+                    raise ValueError("CSR feature training requires tilecenter8 and direct feature attributes")
+                raise NotImplementedError("record-based feature training is not part of the forward renderer")
+            base = self._base_args(ray_o, ray_d, culled_prim_indices, tile_offsets, device)
+            bg = self._background(bg_color, ray_o)
+            dims = (int(W), int(H), ts, ts, float(score_threshold))
+            if (not return_feature) or (self.feat_attr is None):
+                if use_tilecenter:
+                    rgb, alpha = ext.render_tiles_forward_tilecenter(*base, *dims)
+                else:
+                    rgb, alpha = ext.render_tiles_forward(*base, *dims)
+                rgb = _add_background(rgb, alpha, bg)
+                if return_feature and self.feat_attr is None:
+                    raise RuntimeError("return_feature=True requested but feat_attr is not initialized.")
+                return rgb
+            feat_args = (self.feat_attr.detach().contiguous(), float(self.feature_gating_beta),
+                         float(self.feature_gating_temp))
+            if use_tilecenter:
+                rgb, alpha, feat = ext.render_tiles_forward_tilecenter_with_feat(*base, *feat_args, *dims)
+            else:
+                rgb, alpha, feat = ext.render_tiles_forward_per_pixel_with_feat(*base, *feat_args, *dims)
+            return _add_background(rgb, alpha, bg), feat
+
+    def render_feature_map(self, ray_o, ray_d, score_threshold: float = 1e-3, view_matrix=None, proj_matrix=None,
+                           culled_prim_indices=None, tile_offsets=None):
+        """The feature image alone, through ``forward`` (scannet/cumodel.py:1162-1193)."""
+        if self.feat_attr is None:
+            raise RuntimeError("Feature rendering requested but feature_dim_low == 0.")
+        if self.image_size is None:
+            raise ValueError("image_size must be set before calling render_feature_map.")
+        W, H = self.image_size
+        if ray_o.shape[0] != W * H:
+            raise ValueError("render_feature_map requires full-frame rays (B == W*H).")
+        _rgb, feat = self.forward(ray_o=ray_o, ray_d=ray_d, score_threshold=score_threshold, bg_color=None,
+                                  view_matrix=view_matrix, proj_matrix=proj_matrix,
+                                  culled_prim_indices=culled_prim_indices, tile_offsets=tile_offsets,
+                                  return_feature=True)
+        return feat
+
+    @torch.no_grad()
+    def render_rgb_alpha_no_grad(self, ray_o, ray_d, score_threshold: float = 1e-3, bg_color=None, view_matrix=None,
+                                 proj_matrix=None, collect_w_stats: bool = False, gt_rgb=None):
+        """(rgb, alpha) under the tile-centre pipeline (scannet/cumodel.py:1196-1383)."""
+        if getattr(self, "camera_mode", "legacy-centered") == "colmap-native":
+            raise NotImplementedError("Native camera statistics rendering is not implemented; use forward for RGB/features")
+        if self.image_size is None:
+            raise ValueError("image_size must be set on NeuralPrimitiveSceneTileCUDA before calling render_rgb_alpha_no_grad.")
+        if view_matrix is None or proj_matrix is None:
+            raise ValueError("Tile renderer requires view_matrix and proj_matrix for culling.")
+        W, H = self.image_size
+        B = ray_o.shape[0]
+        assert B == W * H, "Tile renderer requires full-frame rays (B == W*H)"
+        device = self._activate_cuda_device()
+        ts = int(self.tile_size)
+        cand, offsets = self._legacy_culling(view_matrix.reshape(1, 4, 4), proj_matrix, score_threshold, ts)
+        ext = self._ensure_tile_ext()
+        base = self._base_args(ray_o, ray_d, cand, offsets, device)
+        dims = (int(W), int(H), ts, ts, float(score_threshold))
+        if collect_w_stats:
+            if gt_rgb is None:
+                raise ValueError("collect_w_stats=True requires gt_rgb (shape=(B,3), B=W*H) to compute pixel_error "
+                                 "inside the CUDA kernel.")
+            if gt_rgb.dim() != 2 or gt_rgb.shape[0] != B or gt_rgb.shape[1] != 3:
+                raise ValueError(f"gt_rgb must have shape (B,3) with B=W*H={B}, got {tuple(gt_rgb.shape)}")
+            gt_rgb = gt_rgb.to(device=device, dtype=torch.float32).contiguous()
+            rgb, alpha = ext.render_tiles_forward_tilecenter_stats(
+                *base[:9], int(base[7].numel()), *base[9:], int(self.W1.shape[0]), int(self.W1.shape[1]),
+                int(self.W1.shape[2]), *dims, gt_rgb, self.stat_sum_w.contiguous(), self.stat_max_w.contiguous(),
+                self.stat_hits.contiguous(), self.stat_sum_werr.contiguous(), self.stat_contrib_count.contiguous())
+        else:
+            rgb, alpha = ext.render_tiles_forward_tilecenter(*base, *dims)
+        return _add_background(rgb, alpha, self._background(bg_color, ray_o)), alpha
+
+    @torch.no_grad()
+    def render_rgb_t_no_grad(self, ray_o, ray_d, score_threshold: float = 1e-3, bg_color=None, view_matrix=None,
+                             proj_matrix=None):
+        """(rgb, t, alpha) with t the expected depth (scannet/cumodel.py:1385-1525)."""
+        if getattr(self, "camera_mode", "legacy-centered") == "colmap-native":
+            raise NotImplementedError("Native camera depth rendering is not implemented; use forward for RGB/features")
+        if self.image_size is None:
+            raise ValueError("image_size must be set on NeuralPrimitiveSceneTileCUDA before calling render_rgb_t_no_grad.")
+        if view_matrix is None or proj_matrix is None:
+            raise ValueError("Tile renderer requires view_matrix and proj_matrix for culling.")
+        W, H = self.image_size
+        assert ray_o.shape[0] == W * H, "Tile renderer requires full-frame rays (B == W*H)"
+        device = self._activate_cuda_device()
+        ts = int(self.tile_size)
+        cand, offsets = self._legacy_culling(view_matrix.reshape(1, 4, 4), proj_matrix, score_threshold, ts)
+        ext = self._ensure_tile_ext()
+        base = self._base_args(ray_o, ray_d, cand, offsets, device)
+        rgb, alpha, t = ext.render_tiles_forward_tilecenter_with_t(*base, int(W), int(H), ts, ts, float(score_threshold))
+        return _add_background(rgb, alpha, self._background(bg_color, ray_o)), t, alpha

@@ -146,3 +146,63 @@ def render_tilecenter_f32(rays_o, rays_d, records, order, tile_offsets, freq, at
 
 def radius_multiplier(threshold: float) -> float:
     return math.sqrt(-2.0 * math.log(threshold))
+
+
+def _feat_shape(feat_attr):
+    """(slots, channels) with the reference's checks (np_tile_kernels.cu:6158-6169)."""
+    if not (feat_attr.is_cuda and feat_attr.dtype == torch.float32 and feat_attr.dim() in (2, 3)):
+        raise RuntimeError("feat_attr must be a float32 CUDA tensor of 2 or 3 dimensions")
+    if feat_attr.dim() == 2:
+        slots, ch = 1, feat_attr.shape[1]
+    else:
+        slots, ch = feat_attr.shape[1], feat_attr.shape[2]
+        if slots not in (4, 5):
+            raise RuntimeError("3D feat_attr expects slots in {4,5}")
+    if ch <= 0:
+        raise RuntimeError("feat_attr feature dimension must be positive")
+    if ch > 512:
+        raise RuntimeError("feat_attr feature dimension must be <= 512")
+    return int(slots), int(ch)
+
+
+def render_tilecenter_feat_f32(rays_o, rays_d, records, order, tile_offsets, freq, att, W1, b1, W2, b2, W3, b3,
+                               feat_attr, beta, temp, W, H, TW, TH, threshold):
+    """Scalar-f32 tile-centre forward with the gated feature channel -> (rgb, alpha, feat [B,C])."""
+    dev = rays_o.device
+    slots, ch = _feat_shape(feat_attr)
+    B = W * H
+    rgb = torch.empty(B, 3, dtype=torch.float32, device=dev)
+    alpha = torch.empty(B, 1, dtype=torch.float32, device=dev)
+    feat = torch.empty(B, ch, dtype=torch.float32, device=dev)
+    n, hidden, F = W1.shape[0], W2.shape[1], freq.shape[0]
+    code = _lib.load().mlpsp_render_tilecenter_feat_f32(
+        _ptr(rays_o), _ptr(rays_d), _ptr(records), _ptr(order), _ptr(tile_offsets), _ptr(freq), _ptr(att), F,
+        _ptr(W1), _ptr(b1), _ptr(W2), _ptr(b2), _ptr(W3), _ptr(b3), n, hidden, _ptr(feat_attr), slots, ch,
+        float(beta), float(temp), W, H, TW, TH, float(threshold), _ptr(rgb), _ptr(alpha), _ptr(feat), _stream(dev))
+    _check(code, "mlpsp_render_tilecenter_feat_f32")
+    return rgb, alpha, feat
+
+
+def render_per_pixel_f32(rays_o, rays_d, records, candidates, tile_offsets, freq, att, W1, b1, W2, b2, W3, b3, W, H,
+                         TW, TH, threshold, path_name, feat_attr=None, beta=1.5, temp=2.0):
+    """Per-pixel-order forward -> (rgb, alpha, feat|None); raises the reference's overflow error."""
+    dev = rays_o.device
+    lib = _lib.load()
+    B = W * H
+    slots, ch = _feat_shape(feat_attr) if feat_attr is not None else (0, 0)
+    rgb = torch.empty(B, 3, dtype=torch.float32, device=dev)
+    alpha = torch.empty(B, 1, dtype=torch.float32, device=dev)
+    feat = torch.empty(B, ch, dtype=torch.float32, device=dev) if feat_attr is not None else None
+    nbytes = lib.mlpsp_per_pixel_workspace_bytes(W, H, TW, TH)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    n, hidden, F = W1.shape[0], W2.shape[1], freq.shape[0]
+    code = lib.mlpsp_render_per_pixel_f32(
+        _ptr(rays_o), _ptr(rays_d), _ptr(records), _ptr(candidates), _ptr(tile_offsets), _ptr(freq), _ptr(att), F,
+        _ptr(W1), _ptr(b1), _ptr(W2), _ptr(b2), _ptr(W3), _ptr(b3), n, hidden, _ptr(feat_attr), slots, ch,
+        float(beta), float(temp), W, H, TW, TH, float(threshold), _ptr(ws), nbytes, _ptr(rgb), _ptr(alpha),
+        _ptr(feat), _stream(dev))
+    if code & _lib.E_PIXEL_OVERFLOW:
+        raise RuntimeError(f"{path_name}: per-pixel intersection capacity {_lib.PIXEL_HIT_CAPACITY} exceeded; "
+                           "refusing to return a silently truncated result")
+    _check(code, path_name)
+    return rgb, alpha, feat

@@ -1,0 +1,269 @@
+"""The renderer extension object: same entry-point names, positional signatures, return values and
+error texts as the reference's pybind11 module (scannet/cuda/np_tile_kernels.cu:7224-7252,
+forward entry points), implemented on the C ABI of ``libmlpsp_hip.so``.
+
+``TileExt()`` is what ``cumodel._ensure_tile_ext_static()`` returns and what a test installs with
+``monkeypatch.setattr(cumodel, "_tile_ext", ...)``.  Entry points that belong to the reference's
+training/backward side are not provided; calling one raises ``NotImplementedError`` naming it.
+"""
+from __future__ import annotations
+
+import threading
+import warnings
+
+import torch
+
+from . import _lib, ops
+
+MAX_TILE_PRIMS = 1536          # MLPSP_MAX_TILE_PRIMS as built by scannet/cumodel.py:102-118
+MAX_H_TILECENTER = 32          # MLPSP_MAX_H (np_tile_kernels.cu:36-38)
+
+_BACKWARD_ONLY = (
+    "render_tiles_backward_count_per_pixel", "render_tiles_backward_count_tilecenter",
+    "render_tiles_backward_emit_per_pixel", "render_tiles_backward_emit_tilecenter",
+    "render_tiles_backward_featattr_per_pixel", "render_tiles_backward_featattr_tilecenter",
+    "render_tiles_backward_tilecenter_full", "render_tiles_backward_tilecenter_full_with_feat",
+    "render_tiles_mlp_records", "render_tiles_training_records", "render_tiles_training_records_wmma",
+    "primitive_records_reverse", "render_tiles_backward_tilecenter_traversal",
+    "render_tiles_backward_tilecenter_backprop_noatomic", "training_wmma_safety_stats",
+)
+
+
+def _chk(cond, msg="Expected condition to be true"):
+    if not cond:
+        raise RuntimeError(msg)
+
+
+def _is_f32_2d(t, cols):
+    return t.is_cuda and t.dtype == torch.float32 and t.dim() == 2 and t.shape[1] == cols
+
+
+class TileExt:
+    """Forward entry points of the tile renderer on one MI355X."""
+
+    def __init__(self, max_tile_prims: int = MAX_TILE_PRIMS):
+        _lib.load()  # fail now, loudly, if the HIP library is absent
+        self.max_tile_prims = int(max_tile_prims)
+        self._lock = threading.Lock()
+        self._mfma_calls = 0
+        self._mfma_fallbacks = 0
+
+    def __getattr__(self, name):
+        if name in _BACKWARD_ONLY:
+            def _missing(*_a, **_k):
+                raise NotImplementedError(f"{name} belongs to the training/backward path, which this build does not provide")
+            return _missing
+        raise AttributeError(name)
+
+    # ------------------------------------------------------------------------------------------
+    # shared argument checks (np_tile_kernels.cu:5242-5275)
+    # ------------------------------------------------------------------------------------------
+    @staticmethod
+    def _check_base(rays_o, rays_d, positions, log_scales, quats, cand, offsets, freq, att):
+        _chk(_is_f32_2d(rays_o, 3), "rays_o must be a CUDA float32 [B,3] tensor")
+        _chk(_is_f32_2d(rays_d, 3), "rays_d must be a CUDA float32 [B,3] tensor")
+        _chk(_is_f32_2d(positions, 3), "positions must be a CUDA float32 [N,3] tensor")
+        _chk(_is_f32_2d(log_scales, 3), "log_scales must be a CUDA float32 [N,3] tensor")
+        _chk(_is_f32_2d(quats, 4), "quats must be a CUDA float32 [N,4] tensor")
+        _chk(cand.is_cuda and cand.dtype == torch.int32 and cand.dim() == 1, "culled_prim_indices must be CUDA int32 1-D")
+        _chk(offsets.is_cuda and offsets.dtype == torch.int32 and offsets.dim() == 1, "tile_offsets must be CUDA int32 1-D")
+        _chk(freq.is_cuda and freq.dtype == torch.float32 and freq.dim() == 1, "freq_bands must be CUDA float32 1-D")
+        _chk(att.is_cuda and att.dtype == torch.float32 and att.dim() == 1, "attenuation must be CUDA float32 1-D")
+
+    @staticmethod
+    def _weights_f32(ws, allow_low_precision):
+        W1 = ws[0]
+        _chk(all(w.is_cuda for w in ws), "MLP tensors must be CUDA tensors")
+        _chk(all(w.dtype == W1.dtype for w in ws), "W/b tensors must share the same dtype")
+        ok = (torch.float32, torch.float16, torch.bfloat16) if allow_low_precision else (torch.float32,)
+        _chk(W1.dtype in ok, "W/b tensors must be float32, float16, or bfloat16" if allow_low_precision
+             else "W/b tensors must be float32")
+        # Stored half/bfloat16 weights are widened exactly, as the reference's cast_copy does when
+        # it stages them (np_tile_kernels.cu:2016-2021).
+        return [w.float().contiguous() for w in ws]
+
+    def _prepare(self, args, name, capacity, tile_limit, low_precision=False, hidden_limit=64):
+        (rays_o, rays_d, positions, log_scales, quats, cand, offsets, freq, att, W1, b1, W2, b2, W3, b3,
+         Wimg, Himg, TW, TH, thr) = args
+        Wimg, Himg, TW, TH = int(Wimg), int(Himg), int(TW), int(TH)
+        if tile_limit is not None:
+            _chk(0 < TW * TH <= tile_limit[0], tile_limit[1])
+        self._check_base(rays_o, rays_d, positions, log_scales, quats, cand, offsets, freq, att)
+        ws = self._weights_f32([W1, b1, W2, b2, W3, b3], low_precision)
+        _chk(rays_o.shape[0] == Wimg * Himg, "B must equal W*H for tile renderer")
+        _chk(Wimg > 0 and Himg > 0 and TW > 0 and TH > 0, f"{name}: image and tile dimensions must be positive")
+        n_tiles = ops.num_tiles(Wimg, Himg, TW, TH)
+        cand = cand.contiguous()
+        offsets = offsets.contiguous()
+        with torch.cuda.device(rays_o.device):
+            ops.validate_tile_lists(cand, offsets, n_tiles, capacity, positions.shape[0], name)
+        F = freq.shape[0]
+        _chk(W1.shape[2] == 6 * F * 2, "Encoded dim must be 6*F*2")
+        _chk(W2.shape[1] <= hidden_limit, f"{name} currently supports hidden_dim <= {hidden_limit}")
+        geo = (rays_o.contiguous(), rays_d.contiguous(), positions.contiguous(), log_scales.contiguous(),
+               quats.contiguous())
+        return geo, cand, offsets, freq.contiguous(), att.contiguous(), ws, (Wimg, Himg, TW, TH, float(thr))
+
+    # ------------------------------------------------------------------------------------------
+    # tile-centre order
+    # ------------------------------------------------------------------------------------------
+    def _tilecenter(self, args, name, family, capacity, with_t=False, low_precision=False, hidden_limit=MAX_H_TILECENTER):
+        geo, cand, offsets, freq, att, ws, (W, H, TW, TH, thr) = self._prepare(
+            args, name, capacity,
+            (256, "Tile-center order kernel requires 0 < TW*TH <= MLPSP_TILECENTER_BLOCK_THREADS"),
+            low_precision, hidden_limit)
+        rays_o, rays_d, positions, log_scales, quats = geo
+        with torch.cuda.device(rays_o.device):
+            rec = ops.prepare_primitives(positions, log_scales, quats)
+            if family == _lib.KEY_LIST_ORDER or cand.numel() == 0:
+                order = cand
+            else:
+                order, _ = ops.sort_tiles(rays_o, rays_d, rec, cand, offsets, W, H, TW, TH, family, capacity)
+            return ops.render_tilecenter_f32(rays_o, rays_d, rec, order, offsets, freq, att, *ws, W, H, TW, TH, thr,
+                                             with_t=with_t)
+
+    def render_tiles_forward_tilecenter(self, *args):
+        """(rgb [B,3], alpha [B,1]); np_tile_kernels.cu:5225-5347."""
+        rgb, alpha, _ = self._tilecenter(args, "render_tiles_forward_tilecenter", _lib.KEY_TSTAR,
+                                         self.max_tile_prims, low_precision=True)
+        return rgb, alpha
+
+    def render_tiles_autograd_tilecenter(self, *args):
+        """Forward-only alias (np_tile_kernels.cu:4780-4860, 5040-5061)."""
+        rgb, alpha, _ = self._tilecenter(args, "render_tiles_autograd_tilecenter", _lib.KEY_TSTAR, self.max_tile_prims)
+        return rgb, alpha
+
+    def render_tiles_autograd_tilecenter_presorted(self, *args):
+        """Consumes host-sorted lists of any length (np_tile_kernels.cu:4880-4948, kernel :4242-4478)."""
+        rgb, alpha, _ = self._tilecenter(args, "render_tiles_autograd_tilecenter_presorted", _lib.KEY_LIST_ORDER, 0)
+        return rgb, alpha
+
+    def render_tiles_forward_tilecenter_with_t(self, *args):
+        """(rgb, alpha, t [B,1]); plain centre-depth order (np_tile_kernels.cu:5432-5792)."""
+        return self._tilecenter(args, "render_tiles_forward_tilecenter_with_t", _lib.KEY_DEPTH, self.max_tile_prims,
+                                with_t=True, hidden_limit=64)
+
+    def render_tiles_forward_tilecenter_with_feat(self, *args):
+        """(rgb, alpha, feat [B,C]); np_tile_kernels.cu:6114-6204."""
+        base, (feat_attr, beta, temp), dims = args[:15], args[15:18], args[18:]
+        name = "render_tiles_forward_tilecenter_with_feat"
+        _chk(feat_attr.is_cuda and feat_attr.dtype == torch.float32 and feat_attr.dim() in (2, 3),
+             "feat_attr must be a CUDA float32 tensor with 2 or 3 dimensions")
+        geo, cand, offsets, freq, att, ws, (W, H, TW, TH, thr) = self._prepare(
+            (*base, *dims), name, self.max_tile_prims,
+            (256, "Tile-center feature kernel requires 0 < TW*TH <= MLPSP_TILECENTER_BLOCK_THREADS"))
+        rays_o, rays_d, positions, log_scales, quats = geo
+        _chk(feat_attr.shape[0] == positions.shape[0], "feat_attr first dimension must match primitive count")
+        ops._feat_shape(feat_attr)
+        with torch.cuda.device(rays_o.device):
+            rec = ops.prepare_primitives(positions, log_scales, quats)
+            order = cand
+            if cand.numel() > 0:
+                order, _ = ops.sort_tiles(rays_o, rays_d, rec, cand, offsets, W, H, TW, TH, _lib.KEY_TSTAR,
+                                          self.max_tile_prims)
+            return ops.render_tilecenter_feat_f32(rays_o, rays_d, rec, order, offsets, freq, att, *ws,
+                                                  feat_attr.contiguous(), beta, temp, W, H, TW, TH, thr)
+
+    # ------------------------------------------------------------------------------------------
+    # per-pixel order
+    # ------------------------------------------------------------------------------------------
+    def _per_pixel(self, args, name, feat=None):
+        geo, cand, offsets, freq, att, ws, (W, H, TW, TH, thr) = self._prepare(args, name, 0, None, False, MAX_H_TILECENTER)
+        _chk(0 < TW * TH <= 256, "Tile size too large")
+        rays_o, rays_d, positions, log_scales, quats = geo
+        with torch.cuda.device(rays_o.device):
+            rec = ops.prepare_primitives(positions, log_scales, quats)
+            if feat is None:
+                return ops.render_per_pixel_f32(rays_o, rays_d, rec, cand, offsets, freq, att, *ws, W, H, TW, TH, thr, name)
+            feat_attr, beta, temp = feat
+            return ops.render_per_pixel_f32(rays_o, rays_d, rec, cand, offsets, freq, att, *ws, W, H, TW, TH, thr, name,
+                                            feat_attr=feat_attr.contiguous(), beta=beta, temp=temp)
+
+    def render_tiles_forward(self, *args):
+        """(rgb, alpha), per-pixel order; np_tile_kernels.cu:5064-5132."""
+        rgb, alpha, _ = self._per_pixel(args, "render_tiles_forward")
+        return rgb, alpha
+
+    def render_tiles_autograd(self, *args):
+        """Forward-only alias of the per-pixel renderer (np_tile_kernels.cu:4989-5038)."""
+        rgb, alpha, _ = self._per_pixel(args, "render_tiles_autograd")
+        return rgb, alpha
+
+    def render_tiles_forward_per_pixel_with_feat(self, *args):
+        """(rgb, alpha, feat); np_tile_kernels.cu:5134-5222."""
+        base, (feat_attr, beta, temp), dims = args[:15], args[15:18], args[18:]
+        _chk(feat_attr.is_cuda and feat_attr.dtype == torch.float32 and feat_attr.dim() in (2, 3),
+             "feat_attr must be a CUDA float32 tensor with 2 or 3 dimensions")
+        _chk(feat_attr.shape[0] == base[2].shape[0], "feat_attr first dimension must match primitive count")
+        ops._feat_shape(feat_attr)
+        return self._per_pixel((*base, *dims), "render_tiles_forward_per_pixel_with_feat", (feat_attr, beta, temp))
+
+    # ------------------------------------------------------------------------------------------
+    # statistics forward (pruning statistics are not rebuilt; the render itself is)
+    # ------------------------------------------------------------------------------------------
+    def render_tiles_forward_tilecenter_stats(self, rays_o, rays_d, positions, log_scales, quats, cand, offsets,
+                                              freq, att, F, W1, b1, W2, b2, W3, b3, N, H, IN, Wimg, Himg, TW, TH, thr,
+                                              gt_rgb, stat_sum_w, stat_max_w, stat_hits, stat_sum_werr,
+                                              stat_contrib_count):
+        """Validates and renders like np_tile_kernels.cu:5349-5428 (centre-depth order) and returns
+        (rgb, alpha); the five per-primitive statistic buffers are left untouched."""
+        _chk(0 < int(TW) * int(TH) <= 256, "Tile-center order kernel currently supports 0 < TW*TH <= 256")
+        for t in (stat_sum_w, stat_max_w, stat_sum_werr):
+            _chk(t.is_cuda and t.dtype == torch.float32 and t.numel() == N)
+        for t in (stat_hits, stat_contrib_count):
+            _chk(t.is_cuda and t.dtype == torch.int32 and t.numel() == N)
+        _chk(gt_rgb.is_cuda and gt_rgb.dtype == torch.float32 and tuple(gt_rgb.shape) == (int(Himg) * int(Wimg), 3))
+        args = (rays_o, rays_d, positions, log_scales, quats, cand, offsets, freq, att, W1, b1, W2, b2, W3, b3,
+                Wimg, Himg, TW, TH, thr)
+        rgb, alpha, _ = self._tilecenter(args, "render_tiles_forward_tilecenter_stats", _lib.KEY_DEPTH,
+                                         self.max_tile_prims, hidden_limit=64)
+        return rgb, alpha
+
+    # ------------------------------------------------------------------------------------------
+    # reduced-precision matrix-core path (rgb_wmma.cuh:225-274)
+    # ------------------------------------------------------------------------------------------
+    def rgb_wmma_safety_stats(self):
+        return [self._mfma_calls, self._mfma_fallbacks]
+
+    def render_tiles_rgb_wmma(self, x, width, height, threshold, bf16):
+        """[rgb, alpha] with the 72->32->32->4 MLP on the matrix cores, f32 everywhere else."""
+        _chk(len(x) == 15, "WMMA requires the 15 scene tensors")
+        width, height, threshold = int(width), int(height), float(threshold)
+        _chk(width > 0 and height > 0 and 0.0 < threshold < 1.0)
+        _chk(width <= 2147483647 and height <= 2147483647 and width <= 2147483647 // height,
+             "WMMA image dimensions exceed int32 pixel indexing")
+        for i, t in enumerate(x):
+            _chk(t.is_cuda and t.is_contiguous() and t.device == x[0].device)
+            _chk(t.dtype == (torch.int32 if i in (5, 6) else torch.float32))
+        pixels, n = width * height, x[2].shape[0]
+        _chk(tuple(x[0].shape) == (pixels, 3) and x[1].shape == x[0].shape)
+        _chk(x[2].dim() == 2 and x[2].shape[1] == 3 and x[3].shape == x[2].shape)
+        _chk(tuple(x[4].shape) == (n, 4))
+        _chk(x[7].dim() == 1 and x[7].numel() == 6 and x[8].shape == x[7].shape)
+        _chk(tuple(x[9].shape) == (n, 32, 72) and tuple(x[10].shape) == (n, 32))
+        _chk(tuple(x[11].shape) == (n, 32, 32) and x[12].shape == x[10].shape)
+        _chk(tuple(x[13].shape) == (n, 4, 32) and tuple(x[14].shape) == (n, 4))
+        name = "render_tiles_rgb_wmma"
+        with torch.cuda.device(x[0].device):
+            ops.validate_tile_lists(x[5], x[6], ops.num_tiles(width, height, 8, 8), self.max_tile_prims, n, name)
+            with self._lock:
+                self._mfma_calls += 1
+            rec = ops.prepare_primitives(x[2], x[3], x[4])
+            order = x[5]
+            if x[5].numel() > 0:
+                order, _ = ops.sort_tiles(x[0], x[1], rec, x[5], x[6], width, height, 8, 8, _lib.KEY_TSTAR,
+                                          self.max_tile_prims)
+            rgb, alpha, nonfinite = ops.render_tilecenter_mfma(x[0], x[1], rec, order, x[6], x[7], x[8], *x[9:15],
+                                                               width, height, threshold, bf16=bool(bf16))
+            if nonfinite:
+                for i, t in enumerate(x):
+                    if i not in (5, 6):
+                        _chk(bool(torch.isfinite(t).all()), "WMMA input is nonfinite; refusing fallback")
+                warnings.warn("WMMA operand/activation overflow: rendering this frame with scalar FP32 instead")
+                with self._lock:
+                    self._mfma_fallbacks += 1
+                rgb, alpha, _ = ops.render_tilecenter_f32(x[0], x[1], rec, order, x[6], x[7], x[8], *x[9:15], width,
+                                                          height, 8, 8, threshold)
+                _chk(bool(torch.isfinite(rgb).all()) and bool(torch.isfinite(alpha).all()),
+                     "Scalar FP32 fallback output is nonfinite")
+        return [rgb, alpha]

@@ -1,0 +1,245 @@
+"""The extension object's contract, case for case as the reference's renderer tests state it
+(tests/test_cuda_renderer.py:250-388, tests/test_candidate_capacity.py, tests/test_training_wmma.py:370-386):
+capacity and id errors are raised before any render kernel runs, with the reference's wording, and
+the device stays usable afterwards."""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def tile_ext(device):
+    from mlp_splatting_amd.tile_ext import TileExt
+    return TileExt()
+
+
+def _renderer_inputs(n, device):
+    hidden, frequencies = 1, 1
+    encoded = 12 * frequencies
+    positions = torch.zeros((n, 3), device=device)
+    positions[:, 2] = 1.0
+    quats = torch.zeros((n, 4), device=device)
+    quats[:, 0] = 1.0
+    return {
+        "rays_o": torch.zeros((1, 3), device=device), "rays_d": torch.tensor([[0.0, 0.0, 1.0]], device=device),
+        "positions": positions, "log_scales": torch.zeros((n, 3), device=device), "quats": quats,
+        "candidates": torch.arange(n, device=device, dtype=torch.int32),
+        "offsets": torch.tensor([0, n], device=device, dtype=torch.int32),
+        "freq": torch.ones(frequencies, device=device), "attenuation": torch.ones(frequencies, device=device),
+        "W1": torch.zeros((n, hidden, encoded), device=device), "b1": torch.zeros((n, hidden), device=device),
+        "W2": torch.zeros((n, hidden, hidden), device=device), "b2": torch.zeros((n, hidden), device=device),
+        "W3": torch.zeros((n, 4, hidden), device=device), "b3": torch.zeros((n, 4), device=device),
+        "feat_attr": torch.zeros((n, 4, 2), device=device),
+    }
+
+
+def _base(d):
+    return tuple(d[k] for k in ("rays_o", "rays_d", "positions", "log_scales", "quats", "candidates", "offsets", "freq",
+                                "attenuation", "W1", "b1", "W2", "b2", "W3", "b3"))
+
+
+DIMS = (1, 1, 1, 1, 1.0e-3)
+PLAIN = {"render_tiles_forward", "render_tiles_autograd", "render_tiles_autograd_tilecenter",
+         "render_tiles_autograd_tilecenter_presorted", "render_tiles_forward_tilecenter",
+         "render_tiles_forward_tilecenter_with_t"}
+ALL_FORWARD = sorted(PLAIN | {"render_tiles_forward_per_pixel_with_feat", "render_tiles_forward_tilecenter_with_feat",
+                              "render_tiles_forward_tilecenter_stats"})
+
+
+def _invoke(ext, name, d):
+    base = _base(d)
+    if name in PLAIN:
+        return getattr(ext, name)(*base, *DIMS)
+    if name in ("render_tiles_forward_per_pixel_with_feat", "render_tiles_forward_tilecenter_with_feat"):
+        return getattr(ext, name)(*base, d["feat_attr"], 1.0, 1.0, *DIMS)
+    if name == "render_tiles_forward_tilecenter_stats":
+        n = d["positions"].shape[0]
+        dev = d["positions"].device
+        stats = [torch.zeros(n, device=dev, dtype=dt) for dt in (torch.float32, torch.float32, torch.int32, torch.float32, torch.int32)]
+        return ext.render_tiles_forward_tilecenter_stats(*base[:9], d["freq"].numel(), *base[9:], n, d["W2"].shape[1],
+                                                         d["W1"].shape[2], *DIMS, torch.ones((1, 3), device=dev), *stats)
+    raise AssertionError(name)
+
+
+@pytest.mark.parametrize("name,capacity,error", [
+    ("render_tiles_autograd", 256, "per-pixel intersection capacity 256 exceeded"),
+    ("render_tiles_forward", 256, "per-pixel intersection capacity 256 exceeded"),
+    ("render_tiles_forward_per_pixel_with_feat", 256, "per-pixel intersection capacity 256 exceeded"),
+    ("render_tiles_forward_tilecenter", 1536, "tile candidate capacity 1536 exceeded"),
+    ("render_tiles_forward_tilecenter_with_feat", 1536, "tile candidate capacity 1536 exceeded"),
+    ("render_tiles_forward_tilecenter_with_t", 1536, "tile candidate capacity 1536 exceeded"),
+    ("render_tiles_autograd_tilecenter", 1536, "tile candidate capacity 1536 exceeded"),
+])
+def test_entry_points_fail_explicitly_on_capacity_overflow(tile_ext, device, name, capacity, error):
+    with pytest.raises(RuntimeError, match=error):
+        _invoke(tile_ext, name, _renderer_inputs(capacity + 1, device))
+    torch.cuda.synchronize()
+
+
+def test_capacity_error_reports_the_observed_length(tile_ext, device):
+    with pytest.raises(RuntimeError, match=r"maximum observed tile length 1600\); refusing to truncate"):
+        _invoke(tile_ext, "render_tiles_forward_tilecenter", _renderer_inputs(1600, device))
+
+
+@pytest.mark.parametrize("name,capacity", [("render_tiles_forward", 256), ("render_tiles_forward_tilecenter", 512),
+                                           ("render_tiles_forward_tilecenter", 1536)])
+def test_capacity_boundary_is_accepted(tile_ext, device, name, capacity):
+    outputs = _invoke(tile_ext, name, _renderer_inputs(capacity, device))
+    assert all(torch.isfinite(o).all() for o in outputs)
+
+
+@pytest.mark.parametrize("name", ["render_tiles_autograd", "render_tiles_forward", "render_tiles_forward_per_pixel_with_feat"])
+def test_per_pixel_allows_large_tile_candidate_lists_when_hits_fit(tile_ext, device, name):
+    d = _renderer_inputs(386, device)
+    d["positions"][256:, 0] = 100.0
+    outputs = _invoke(tile_ext, name, d)
+    assert all(torch.isfinite(o).all() for o in outputs)
+
+
+@pytest.mark.parametrize("name", ["render_tiles_forward_per_pixel_with_feat", "render_tiles_forward_tilecenter_with_feat"])
+def test_removed_eight_slot_cube_gating_is_rejected(tile_ext, device, name):
+    d = _renderer_inputs(1, device)
+    d["feat_attr"] = torch.zeros((1, 8, 2), device=device)
+    with pytest.raises(RuntimeError, match=r"slots in \{4,5\}"):
+        _invoke(tile_ext, name, d)
+
+
+def test_feature_dimension_limit(tile_ext, device):
+    d = _renderer_inputs(1, device)
+    d["feat_attr"] = torch.zeros((1, 4, 513), device=device)
+    with pytest.raises(RuntimeError, match="must be <= 512"):
+        _invoke(tile_ext, "render_tiles_forward_tilecenter_with_feat", d)
+
+
+def test_tile_offsets_must_cover_the_candidate_list(tile_ext, device):
+    d = _renderer_inputs(2, device)
+    d["offsets"] = torch.tensor([1, 2], device=device, dtype=torch.int32)
+    with pytest.raises(RuntimeError, match="tile_offsets must start at zero"):
+        _invoke(tile_ext, "render_tiles_forward", d)
+    d["offsets"] = torch.tensor([0, 1, 2], device=device, dtype=torch.int32)
+    with pytest.raises(RuntimeError, match="tile_offsets length mismatch"):
+        _invoke(tile_ext, "render_tiles_forward_tilecenter", d)
+
+
+@pytest.mark.parametrize("name", ALL_FORWARD)
+@pytest.mark.parametrize("invalid_id", [-1, 2])
+def test_entry_points_reject_invalid_primitive_ids_before_rendering(tile_ext, device, name, invalid_id):
+    d = _renderer_inputs(2, device)
+    d["candidates"][0] = invalid_id
+    with pytest.raises(RuntimeError, match="candidate primitive IDs must be in"):
+        _invoke(tile_ext, name, d)
+    torch.cuda.synchronize()   # an illegal access would surface here
+
+
+@pytest.mark.parametrize("name", ["render_tiles_forward", "render_tiles_forward_tilecenter"])
+@pytest.mark.parametrize("n", [0, 2])
+def test_primitive_id_boundaries_and_empty_scene_are_accepted(tile_ext, device, name, n):
+    outputs = _invoke(tile_ext, name, _renderer_inputs(n, device))
+    assert all(torch.isfinite(o).all() for o in outputs)
+    if n == 0:
+        assert all(not o.any() for o in outputs)
+
+
+def test_presorted_streams_and_validates_candidates_beyond_shared_capacity(tile_ext, device):
+    d = _renderer_inputs(1537, device)
+    d["positions"][:-1, 0] = 100.0
+    d["b3"][:, 3] = 1.0
+    one = _renderer_inputs(1, device)
+    one["b3"][:, 3] = 1.0
+    name = "render_tiles_autograd_tilecenter_presorted"
+    expected = _invoke(tile_ext, name, one)
+    actual = _invoke(tile_ext, name, d)
+    assert expected[1].item() > 0
+    for value, reference in zip(actual, expected):
+        torch.testing.assert_close(value, reference, rtol=0, atol=0)
+    for invalid_id in (-1, 1537):
+        d["candidates"][-1] = invalid_id
+        with pytest.raises(RuntimeError, match="candidate primitive IDs must be in"):
+            _invoke(tile_ext, name, d)
+        torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("n", [768, 769, 1024, 1536])
+def test_only_the_last_candidate_hits_is_not_truncated(tile_ext, device, n):
+    d = _renderer_inputs(n, device)
+    d["positions"][:-1, 0] = 100.0
+    d["b3"][:] = torch.tensor([0.5, 0.5, 0.5, 2.0], device=device)
+    one = _renderer_inputs(1, device)
+    one["b3"][:] = torch.tensor([0.5, 0.5, 0.5, 2.0], device=device)
+    got = _invoke(tile_ext, "render_tiles_forward_tilecenter", d)
+    want = _invoke(tile_ext, "render_tiles_forward_tilecenter", one)
+    assert want[1].item() > 0
+    for a, b in zip(got, want):
+        torch.testing.assert_close(a, b, rtol=0, atol=0)
+
+
+def test_stable_depth_ties_follow_list_order(tile_ext, device):
+    n = 12
+    d = _renderer_inputs(n, device)
+    d["b3"][:, 3] = 8.0
+    d["b3"][:, 0] = torch.linspace(-3, 3, n, device=device)
+    d["candidates"] = torch.arange(n - 1, -1, -1, device=device, dtype=torch.int32)
+    rgb, alpha = _invoke(tile_ext, "render_tiles_forward_tilecenter", d)
+    assert abs(float(rgb[0, 0] / alpha[0, 0]) - float(torch.sigmoid(d["b3"][11, 0]))) < 1e-5
+
+
+def test_closed_form_geometric_series(tile_ext, device):
+    import math
+    d = _renderer_inputs(40, device)
+    b3 = [0.3, -0.4, 1.1, 0.2]
+    d["b3"][:] = torch.tensor(b3, device=device)
+    rgb, alpha = _invoke(tile_ext, "render_tiles_forward_tilecenter", d)
+    a = 1 - math.exp(-math.log1p(math.exp(b3[3])))
+    k = next(i for i in range(1, 100) if (1 - a) ** i < 1e-3)
+    colour = 1 / (1 + np.exp(-np.array(b3[:3])))
+    np.testing.assert_allclose(rgb.cpu().numpy()[0], colour * (1 - (1 - a) ** k), atol=2e-6)
+    assert abs(alpha.item() - (1 - (1 - a) ** k)) < 2e-6
+
+
+def test_stored_half_precision_weights_are_widened_exactly(tile_ext, device):
+    d = _renderer_inputs(3, device)
+    d["b3"][:] = torch.tensor([0.25, -0.5, 1.0, 0.75], device=device)      # exactly representable in bf16 and fp16
+    want = _invoke(tile_ext, "render_tiles_forward_tilecenter", d)
+    for dt in (torch.float16, torch.bfloat16):
+        dd = dict(d)
+        for k in ("W1", "b1", "W2", "b2", "W3", "b3"):
+            dd[k] = d[k].to(dt)
+        got = _invoke(tile_ext, "render_tiles_forward_tilecenter", dd)
+        for a, b in zip(got, want):
+            torch.testing.assert_close(a, b, rtol=0, atol=0)
+    dd = dict(d)
+    dd["W1"] = d["W1"].half()
+    with pytest.raises(RuntimeError, match="share the same dtype"):
+        _invoke(tile_ext, "render_tiles_forward_tilecenter", dd)
+
+
+def test_kernels_run_on_the_current_stream(tile_ext, device):
+    # tests/test_training_wmma.py:370-386: work is enqueued on the caller's current stream
+    d = _renderer_inputs(4, device)
+    d["b3"][:, 3] = 0.5
+    want = _invoke(tile_ext, "render_tiles_forward_tilecenter", d)
+    side = torch.cuda.Stream(device=device)
+    side.wait_stream(torch.cuda.current_stream(device))
+    with torch.cuda.stream(side):
+        got = _invoke(tile_ext, "render_tiles_forward_tilecenter", d)
+    side.synchronize()
+    for a, b in zip(got, want):
+        torch.testing.assert_close(a, b, rtol=0, atol=0)
+
+
+def test_inputs_are_not_mutated(tile_ext, device):
+    d = _renderer_inputs(5, device)
+    before = {k: v.clone() for k, v in d.items()}
+    _invoke(tile_ext, "render_tiles_forward_tilecenter_with_feat", d)
+    _invoke(tile_ext, "render_tiles_forward", d)
+    for k, v in d.items():
+        assert torch.equal(v, before[k]), k
+
+
+def test_backward_entry_points_say_they_are_not_built(tile_ext):
+    with pytest.raises(NotImplementedError, match="training/backward"):
+        tile_ext.render_tiles_backward_tilecenter_full()
+    with pytest.raises(AttributeError):
+        tile_ext.no_such_entry_point

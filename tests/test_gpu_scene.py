@@ -1,0 +1,146 @@
+"""The scene module on the GPU: the call an evaluator makes (scannet/eval_rgb_psnr.py:443-493,
+tools/benchmark_inference.py:121-149) against the oracle, plus the no-grad helpers."""
+import numpy as np
+import pytest
+import torch
+
+from conftest import to_dev
+from helpers import Frame, bits
+
+pytestmark = pytest.mark.gpu
+
+
+def _scene_from(fr, device, feature=False, tile=8):
+    from mlp_splatting_amd.cumodel import NeuralPrimitiveSceneTileCUDA
+    sc = fr.scene
+    C = sc.feat_attr.shape[2] if (feature and sc.feat_attr is not None) else 0
+    scene = NeuralPrimitiveSceneTileCUDA(num_primitives=sc.n, hidden_dim=sc.hidden, tile_size=tile, feature_dim_low=C)
+    state = {"positions": sc.positions, "log_scales": sc.log_scales, "quats": sc.quats, "W1": sc.W1, "b1": sc.b1,
+             "W2": sc.W2, "b2": sc.b2, "W3": sc.W3, "b3": sc.b3}
+    if C:
+        state["feat_attr"] = sc.feat_attr
+    missing, unexpected = scene.load_state_dict({k: torch.from_numpy(v) for k, v in state.items()}, strict=False)
+    assert not unexpected and set(missing) <= {"stat_sum_w", "stat_max_w", "stat_hits", "stat_contrib_count",
+                                               "stat_sum_werr", "alpha_accum", "encoder.freq_bands"}
+    scene = scene.to(device).eval()
+    scene.set_image_size(fr.W, fr.H)
+    return scene
+
+
+def _call(scene, fr, device, **kw):
+    with torch.inference_mode():
+        return scene(to_dev(fr.rays_o, device), to_dev(fr.rays_d, device), score_threshold=fr.thr,
+                     view_matrix=to_dev(fr.view, device), proj_matrix=to_dev(fr.proj, device), **kw)
+
+
+def test_forward_matches_oracle_end_to_end(device, oracle_mod):
+    fr = Frame("cfg1_5k_160x120")
+    scene = _scene_from(fr, device)
+    rgb = _call(scene, fr, device)
+    cand, off = fr.oracle_lists(oracle_mod)
+    sc = fr.scene
+    # The module normalises quaternions and ray directions itself, with torch on the device
+    # (scannet/cumodel.py:1088, 1114); the oracle is fed the very same normalised values.
+    q = torch.nn.functional.normalize(to_dev(sc.quats, device), dim=-1).cpu().numpy()
+    rd = torch.nn.functional.normalize(to_dev(fr.rays_d, device), dim=-1).cpu().numpy()
+    # ... and the module's own frequency tables (torch's exp on the device, scannet/cumodel.py:1078-1086)
+    freq, att = (t.cpu().numpy() for t in scene._frequency_tables(device))
+    np.testing.assert_allclose(freq, sc.freq, rtol=1e-6)
+    np.testing.assert_allclose(att, sc.att, rtol=1e-6)
+    want = oracle_mod.render_tilecenter(fr.rays_o, rd, sc.positions, sc.log_scales, q, cand, off, freq, att,
+                                        *sc.mlp(), *fr.dims)
+    assert rgb.shape == (fr.W * fr.H, 3) and not rgb.requires_grad
+    assert np.array_equal(bits(rgb.cpu().numpy()), bits(want["rgb"]))
+    img = rgb.view(fr.H, fr.W, 3).clamp(0.0, 1.0)
+    assert float(img.mean()) > 0.1
+
+
+def test_background_and_external_lists(device, oracle_mod):
+    fr = Frame("cfg1_5k_160x120", n=800, width=40, height=24)
+    scene = _scene_from(fr, device)
+    cand, off = fr.oracle_lists(oracle_mod)
+    plain = _call(scene, fr, device)
+    ext_lists = _call(scene, fr, device, culled_prim_indices=to_dev(cand, device).long(), tile_offsets=to_dev(off, device).long())
+    assert torch.equal(plain, ext_lists)       # int64 lists are accepted and cast (scannet/cumodel.py:986-987)
+    rgb_a = scene.render_rgb_alpha_no_grad(to_dev(fr.rays_o, device), to_dev(fr.rays_d, device), fr.thr,
+                                           view_matrix=to_dev(fr.view, device), proj_matrix=to_dev(fr.proj, device))
+    bg = _call(scene, fr, device, bg_color=[0.2, 0.4, 0.6])
+    want = rgb_a[0] + (1 - rgb_a[1]).clamp(0, 1) * torch.tensor([0.2, 0.4, 0.6], device=device)
+    torch.testing.assert_close(bg, want, rtol=0, atol=1e-7)
+    with pytest.raises(ValueError, match="provided together"):
+        _call(scene, fr, device, culled_prim_indices=to_dev(cand, device))
+    with pytest.raises(ValueError, match="tile_offsets length mismatch"):
+        _call(scene, fr, device, culled_prim_indices=to_dev(cand, device), tile_offsets=to_dev(off[:-1], device))
+    with pytest.raises(RuntimeError, match="feat_attr is not initialized"):
+        _call(scene, fr, device, return_feature=True)
+
+
+def test_feature_path_returns_the_same_rgb_as_the_rgb_only_path(device, oracle_mod):
+    # the benchmark's parity block (tools/benchmark_inference.py:287-311)
+    fr = Frame("cfg1_5k_160x120", n=800, width=40, height=24, feature_dim=64)
+    scene = _scene_from(fr, device, feature=True)
+    rgb = _call(scene, fr, device)
+    rgb_f, feat = _call(scene, fr, device, return_feature=True)
+    assert torch.equal(rgb, rgb_f) and feat.shape == (fr.W * fr.H, 64)
+    cand, off = fr.oracle_lists(oracle_mod)
+    sc = fr.scene
+    want = oracle_mod.render_tilecenter(*fr.base_numpy(cand, off), *fr.dims, feat_attr=sc.feat_attr)
+    np.testing.assert_allclose(feat.cpu().numpy(), want["feat"], atol=1e-6)
+    torch.testing.assert_close(scene.render_feature_map(to_dev(fr.rays_o, device), to_dev(fr.rays_d, device), fr.thr,
+                                                        view_matrix=to_dev(fr.view, device),
+                                                        proj_matrix=to_dev(fr.proj, device)), feat, rtol=0, atol=0)
+
+
+def test_per_pixel_mode_and_tile16(device, oracle_mod):
+    fr = Frame("cfg1_5k_160x120", n=800, width=48, height=32)
+    scene = _scene_from(fr, device)
+    scene.tile_order_mode_override = "per_pixel"
+    rgb_pp = _call(scene, fr, device)
+    cand, off = fr.oracle_lists(oracle_mod)
+    want = oracle_mod.render_per_pixel(*fr.base_numpy(cand, off), *fr.dims)
+    np.testing.assert_allclose(rgb_pp.cpu().numpy(), want["rgb"], atol=1e-6)
+    fr16 = Frame("cfg1_5k_160x120", n=800, width=48, height=32, tile=16)
+    scene16 = _scene_from(fr16, device, tile=16)
+    rgb16 = _call(scene16, fr16, device)
+    c16, o16 = fr16.oracle_lists(oracle_mod)
+    want16 = oracle_mod.render_tilecenter(*fr16.base_numpy(c16, o16), *fr16.dims)
+    np.testing.assert_allclose(rgb16.cpu().numpy(), want16["rgb"], atol=1e-6)
+
+
+def test_public_no_grad_helpers_return_finite_detached_outputs(device):
+    # tests/test_cuda_renderer.py:48-89
+    from mlp_splatting_amd.cumodel import NeuralPrimitiveSceneTileCUDA
+    scene = NeuralPrimitiveSceneTileCUDA(num_primitives=1).to(device)
+    scene.set_image_size(1, 1)
+    scene.tile_order_mode_override = "tilecenter"
+    with torch.no_grad():
+        scene.positions.zero_()
+        scene.positions[:, 2] = 1.0
+        scene.log_scales.fill_(-2.0)
+    rays_o = torch.zeros((1, 3), device=device)
+    rays_d = torch.tensor([[0.0, 0.0, 1.0]], device=device)
+    view, projection = torch.eye(4, device=device), torch.eye(4, device=device)
+    rgb, alpha = scene.render_rgb_alpha_no_grad(rays_o, rays_d, view_matrix=view, proj_matrix=projection)
+    rgb_d, depth, alpha_d = scene.render_rgb_t_no_grad(rays_o, rays_d, view_matrix=view, proj_matrix=projection)
+    for out in (rgb, alpha, rgb_d, depth, alpha_d):
+        assert out.device == device and torch.isfinite(out).all() and not out.requires_grad
+    assert abs(float(depth) - 1.0) < 1e-6 and float(alpha) > 0
+    out = scene(rays_o, rays_d, view_matrix=view, proj_matrix=projection)
+    assert out.shape == (1, 3)
+
+
+def test_native_camera_mode_uses_ray_cone_lists(device, oracle_mod):
+    # tests/test_camera_cuda.py:34-41: conservative culling leaves the image unchanged
+    fr = Frame("cfg1_5k_160x120", n=600, width=40, height=24)
+    scene = _scene_from(fr, device)
+    scene.camera_mode = "colmap-native"
+    rgb_native = _call(scene, fr, device)
+    T = (fr.W // 8) * (fr.H // 8)
+    every = torch.arange(600, dtype=torch.int32, device=device).repeat(T)
+    offs = torch.arange(T + 1, dtype=torch.int32, device=device) * 600
+    scene.camera_mode = "legacy-centered"
+    rgb_all = _call(scene, fr, device, culled_prim_indices=every, tile_offsets=offs)
+    torch.testing.assert_close(rgb_native, rgb_all, rtol=0, atol=1e-6)
+    scene.camera_mode = "colmap-native"
+    with pytest.raises(ValueError, match="derived from the actual rays"):
+        _call(scene, fr, device, culled_prim_indices=every, tile_offsets=offs)
