@@ -1,0 +1,166 @@
+"""Forward-render throughput of the tile renderer on one MI355X.
+
+A step is one full forward render of one camera pose through the scene module's public call
+(`scene(rays_o, rays_d, score_threshold=, view_matrix=, proj_matrix=)`): sparse tile binning, tile-list
+validation, per-tile depth sort and the render kernel.  The workload is the 200k-primitive, 1200x680
+synthetic scene (seed 0) seen from 32 seeded poses; scene and rays are resident in HBM before the clock
+starts.  Prints ONE JSON line.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK = {"f32": 157.3, "bf16": 2500.0}          # MI355X dense peaks, TFLOP/s
+HBM_PEAK_GBS = 8000.0
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=96)
+    ap.add_argument("--warmup", type=int, default=32)
+    ap.add_argument("--workload", default="cfg3_200k_1200x680")
+    ap.add_argument("--precision", choices=["f32", "bf16"], default=None,
+                    help="MLP arithmetic of the render kernel (default: bf16 matrix cores when built, else f32)")
+    ap.add_argument("--poses", type=int, default=32)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (each GPU box has one GPU); "
+              "run with --gpus 1", file=sys.stderr)
+        return 2
+
+    import numpy as np
+    import torch
+
+    from mlp_splatting_amd import _lib, ops, synthetic as syn
+    from mlp_splatting_amd.cumodel import NeuralPrimitiveSceneTileCUDA
+
+    _lib.load()
+    dev = torch.device("cuda", int(os.environ.get("LOCAL_RANK", "0")))
+    torch.cuda.set_device(dev)
+    precision = args.precision or ("bf16" if hasattr(ops, "render_tilecenter_mfma") else "f32")
+
+    sc, cfg = syn.scene_for_config(args.workload)
+    W, H, f, thr = cfg["width"], cfg["height"], cfg["focal"], cfg["threshold"]
+
+    def t(a):
+        return torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+
+    scene = NeuralPrimitiveSceneTileCUDA(num_primitives=sc.n, hidden_dim=sc.hidden, feature_dim_low=0)
+    scene.load_state_dict({"positions": torch.from_numpy(sc.positions), "log_scales": torch.from_numpy(sc.log_scales),
+                           "quats": torch.from_numpy(sc.quats), "W1": torch.from_numpy(sc.W1),
+                           "b1": torch.from_numpy(sc.b1), "W2": torch.from_numpy(sc.W2), "b2": torch.from_numpy(sc.b2),
+                           "W3": torch.from_numpy(sc.W3), "b3": torch.from_numpy(sc.b3)}, strict=False)
+    scene = scene.to(dev).eval()
+    scene.set_image_size(W, H)
+    scene.render_precision = precision
+    proj = t(syn.projection_matrix(f, W, H))
+    poses = syn.random_poses(args.poses, 0)
+    frames = []
+    for c2w in poses:
+        ro, rd = syn.pinhole_rays(W, H, f, c2w)
+        frames.append((t(ro), t(rd), t(syn.view_matrix(c2w))))
+
+    def render(i):
+        ro, rd, view = frames[i % len(frames)]
+        with torch.inference_mode():
+            return scene(ro, rd, score_threshold=thr, view_matrix=view, proj_matrix=proj)
+
+    for i in range(args.warmup):
+        render(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        render(i)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    fps = args.steps / elapsed
+
+    # ---- the render kernel alone: HIP events on the stream it is launched on, and its work counters
+    freq, att = scene._frequency_tables(dev)
+    quats = torch.nn.functional.normalize(scene.quats.detach(), dim=-1).contiguous()
+    weights = [p.detach().contiguous() for p in (scene.W1, scene.b1, scene.W2, scene.b2, scene.W3, scene.b3)]
+    kernel_ms, hits, proc, cand_total, sort_ms, bin_ms = 0.0, 0, 0, 0, 0.0, 0.0
+    packed = ops.pack_mfma_weights(*weights, bf16=True) if precision == "bf16" else None
+    n_probe = min(len(frames), 8)
+    for i in range(n_probe):
+        ro, rd_raw, view = frames[i]
+        rd = torch.nn.functional.normalize(rd_raw, dim=-1).contiguous()
+        e = [torch.cuda.Event(enable_timing=True) for _ in range(4)]
+        rec = ops.prepare_primitives(scene.positions.detach(), scene.log_scales.detach(), quats)
+        e[0].record()
+        cand, off = ops.bin_legacy(scene.positions.detach(), scene.log_scales.detach(), view[None], proj, W, H, 8, thr)
+        e[1].record()
+        order, _ = ops.sort_tiles(ro, rd, rec, cand, off, W, H, 8, 8)
+        counters = torch.zeros(4, dtype=torch.int64, device=dev)
+        e[2].record()
+        if precision == "bf16":
+            ops.render_tilecenter_mfma(ro, rd, rec, order, off, freq, att, *weights, W, H, thr, bf16=True,
+                                       counters=counters, packed=packed)
+        else:
+            ops.render_tilecenter_f32(ro, rd, rec, order, off, freq, att, *weights, W, H, 8, 8, thr, counters=counters)
+        e[3].record()
+        torch.cuda.synchronize()
+        bin_ms += e[0].elapsed_time(e[1])
+        sort_ms += e[1].elapsed_time(e[2])
+        kernel_ms += e[2].elapsed_time(e[3])
+        c = counters.cpu().numpy()
+        hits += int(c[3])
+        proc += int(c[1])
+        cand_total += int(cand.numel())
+    flops_per_hit = 2 * (72 * sc.hidden + sc.hidden * sc.hidden + 4 * sc.hidden)
+    achieved_tflops = flops_per_hit * hits / (kernel_ms * 1e-3) / 1e12
+    # sort kernel: 48 algorithmic bytes per candidate (4 id + 40 geometry in, 4 id out)
+    sort_gbs = 48.0 * cand_total / (sort_ms * 1e-3) / 1e9
+
+    out = {
+        "metric": "forward_render_frames_per_sec_1200x680_200k_primitives",
+        "value": round(fps, 3), "unit": "frames/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(1000.0 * elapsed / args.steps, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": precision, "data": "synthetic",
+        "config": {"workload": args.workload, "primitives": sc.n, "width": W, "height": H, "tile": 8,
+                   "threshold": thr, "poses": len(frames), "log_scale_mean": cfg["log_scale_mean"],
+                   "mlp": f"72-{sc.hidden}-{sc.hidden}-4", "entry": "NeuralPrimitiveSceneTileCUDA.forward"},
+        "mpix_per_sec": round(fps * W * H / 1e6, 2),
+        "roofline": {"bound": "mfma", "kernel": "render_tilecenter_" + ("mfma" if precision == "bf16" else "f32"),
+                     "achieved": round(achieved_tflops, 3), "peak": PEAK[precision], "unit": "TFLOP/s",
+                     "frac": round(achieved_tflops / PEAK[precision], 5), "traffic": None,
+                     "ms_per_launch": round(kernel_ms / n_probe, 4), "hits_per_launch": hits // n_probe,
+                     "tile_primitives_per_launch": proc // n_probe, "flops_per_hit": flops_per_hit},
+        "stages": {"bin_ms": round(bin_ms / n_probe, 4), "sort_ms": round(sort_ms / n_probe, 4),
+                   "render_ms": round(kernel_ms / n_probe, 4),
+                   "sort_hbm": {"bound": "hbm", "achieved": round(sort_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                                "frac": round(sort_gbs / HBM_PEAK_GBS, 5)},
+                   "candidates_per_launch": cand_total // n_probe},
+    }
+
+    if not args.no_cpu_baseline:
+        # the CPU restatement of the same algorithm, on this host's cores: ONE full frame (pose 0)
+        import oracle
+        ro, rd_raw, view = frames[0]
+        rd = torch.nn.functional.normalize(rd_raw, dim=-1).cpu().numpy()
+        ro_np, view_np = ro.cpu().numpy(), view.cpu().numpy()
+        tc = time.perf_counter()
+        cand, off = oracle.bin_legacy(sc.positions, sc.log_scales, view_np[None], proj.cpu().numpy(), W, H, 8, thr)
+        res = oracle.render_tilecenter(ro_np, rd, sc.positions, sc.log_scales, quats.cpu().numpy(), cand, off,
+                                       freq.cpu().numpy(), att.cpu().numpy(), *sc.mlp(), W, H, 8, 8, thr)
+        cpu_s = time.perf_counter() - tc
+        gpu_rgb = render(0).cpu().numpy()
+        out["cpu_baseline"] = {"value": round(1.0 / cpu_s, 4), "unit": "frames/s", "cores": oracle.num_threads(),
+                               "kind": "port", "sample": "1 full frame (pose 0) of the same workload: binning + "
+                               "per-tile sort + f32 render, OpenMP over tiles",
+                               "ms_per_frame": round(cpu_s * 1e3, 1),
+                               "gpu_vs_cpu_image_max_abs": float(np.abs(gpu_rgb - res["rgb"]).max())}
+    print(json.dumps(out))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

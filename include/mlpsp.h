@@ -42,6 +42,7 @@ extern "C" {
 #define MLPSP_TILE_CAPACITY_MAX 2048 /* largest per-tile list the in-LDS sort accepts */
 #define MLPSP_PIXEL_HIT_CAPACITY 256 /* per-pixel-order hit buffer (np_tile_kernels.cu:760) */
 #define MLPSP_PRIM_RECORD_BYTES 64   /* bytes per primitive of the prepared geometry buffer */
+#define MLPSP_MFMA_PACK_BYTES 7808   /* bytes per primitive of the packed matrix-core weight buffer */
 
 #define MLPSP_KEY_LIST_ORDER 0 /* consume the list as given (presorted kernel, np_tile_kernels.cu:4242-4478) */
 #define MLPSP_KEY_TSTAR 1      /* Mahalanobis t* of the tile-centre ray (np_tile_kernels.cu:483-518) */
@@ -150,6 +151,25 @@ int mlpsp_render_per_pixel_f32(const float* rays_o_dev, const float* rays_d_dev,
                                int feat_channels, float gating_beta, float gating_temp, int width, int height,
                                int tile_w, int tile_h, float threshold, void* workspace_dev, size_t workspace_bytes,
                                float* out_rgb_dev, float* out_alpha_dev, float* out_feat_dev, mlpsp_stream_t stream);
+
+/* Matrix-core path for the released 72->32->32->4 MLP (F = 6, H = 32), 8x8 tiles; the counterpart of
+ * render_tiles_rgb_wmma (scannet/cuda/rgb_wmma.cuh:75-274).
+ * mlpsp_pack_mfma_weights: rounds W1, W2, W3 to bf16 (use_bf16 != 0) or fp16 and stores them, with the
+ *   f32 biases, in MFMA operand order: mlpsp_mfma_pack_bytes(N) bytes, 128-byte aligned.  Done once per
+ *   set of weights (the reference re-casts them for every tile and primitive, rgb_wmma.cuh:162-174).
+ * mlpsp_render_tilecenter_mfma: geometry, activations and compositing in f32; encoded inputs, weights
+ *   and hidden activations in bf16/fp16 with f32 accumulation.  *nonfinite_dev (int32, zeroed by the
+ *   call) becomes 1 if a non-finite operand, pre-activation or logit was met on an active ray, in
+ *   which case the caller re-renders the frame with mlpsp_render_tilecenter_f32 (rgb_wmma.cuh:260-272). */
+size_t mlpsp_mfma_pack_bytes(int num_primitives);
+int mlpsp_pack_mfma_weights(const float* W1, const float* b1, const float* W2, const float* b2, const float* W3,
+                            const float* b3, int num_primitives, int use_bf16, void* packed_dev,
+                            mlpsp_stream_t stream);
+int mlpsp_render_tilecenter_mfma(const float* rays_o_dev, const float* rays_d_dev, const void* prim_records_dev,
+                                 const int32_t* order_dev, const int32_t* tile_offsets_dev, const float* freq_dev,
+                                 const float* att_dev, const void* packed_dev, int num_primitives, int use_bf16,
+                                 int width, int height, float threshold, float* out_rgb_dev, float* out_alpha_dev,
+                                 int32_t* nonfinite_dev, int64_t* counters_dev, mlpsp_stream_t stream);
 
 #ifdef __cplusplus
 }

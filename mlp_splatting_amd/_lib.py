@@ -19,6 +19,7 @@ KEY_LIST_ORDER, KEY_TSTAR, KEY_DEPTH = 0, 1, 2
 TILE_CAPACITY_MAX = 2048
 PIXEL_HIT_CAPACITY = 256
 PRIM_RECORD_BYTES = 64
+MFMA_PACK_BYTES = 7808
 
 _vp, _i, _f, _i64, _sz = C.c_void_p, C.c_int, C.c_float, C.c_int64, C.c_size_t
 
@@ -43,6 +44,9 @@ SIGNATURES = {
     "mlpsp_per_pixel_workspace_bytes": (_sz, [_i, _i, _i, _i]),
     "mlpsp_render_per_pixel_f32": (_i, [_vp] * 7 + [_i] + [_vp] * 6 + [_i, _i, _vp, _i, _i, _f, _f, _i, _i, _i, _i, _f,
                                                                       _vp, _sz, _vp, _vp, _vp, _vp]),
+    "mlpsp_mfma_pack_bytes": (_sz, [_i]),
+    "mlpsp_pack_mfma_weights": (_i, [_vp] * 6 + [_i, _i, _vp, _vp]),
+    "mlpsp_render_tilecenter_mfma": (_i, [_vp] * 8 + [_i, _i, _i, _i, _f, _vp, _vp, _vp, _vp, _vp]),
 }
 
 _lib = None

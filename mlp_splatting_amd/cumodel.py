@@ -179,6 +179,9 @@ class NeuralPrimitiveSceneTileCUDA(nn.Module):
         if self.tile_size not in (8, 16):
             raise ValueError("NeuralPrimitiveSceneTileCUDA supports tile_size in {8, 16}.")
         self.tile_order_mode_override = None
+        # MLP arithmetic of the RGB tile-centre render: "f32" (scalar, the reference's default kernel) or
+        # "bf16"/"fp16" (matrix cores; needs the 72->32->32->4 MLP and 8x8 tiles, else f32 is used).
+        self.render_precision = os.environ.get("MLPSP_RENDER_PRECISION", "f32")
         self.feature_dim_low = int(max(0, feature_dim_low))
         self.feature_slots = int(max(1, feature_slots))
         self.feature_gating_beta = float(feature_gating_beta)
@@ -377,7 +380,15 @@ class NeuralPrimitiveSceneTileCUDA(nn.Module):
             bg = self._background(bg_color, ray_o)
             dims = (int(W), int(H), ts, ts, float(score_threshold))
             if (not return_feature) or (self.feat_attr is None):
-                if use_tilecenter:
+                precision = str(getattr(self, "render_precision", "f32")).lower()
+                if precision not in {"f32", "bf16", "fp16"}:
+                    raise ValueError(f"Unsupported render_precision {precision!r}; use 'f32', 'bf16' or 'fp16'.")
+                matrix_cores = (use_tilecenter and precision != "f32" and ts == 8 and int(self.hidden_dim) == 32
+                                and int(self.pe_frequencies) == 6)
+                if matrix_cores:
+                    rgb, alpha = ext.render_tiles_rgb_wmma(list(base), int(W), int(H), float(score_threshold),
+                                                           precision == "bf16")
+                elif use_tilecenter:
                     rgb, alpha = ext.render_tiles_forward_tilecenter(*base, *dims)
                 else:
                     rgb, alpha = ext.render_tiles_forward(*base, *dims)

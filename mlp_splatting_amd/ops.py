@@ -206,3 +206,39 @@ def render_per_pixel_f32(rays_o, rays_d, records, candidates, tile_offsets, freq
                            "refusing to return a silently truncated result")
     _check(code, path_name)
     return rgb, alpha, feat
+
+
+def pack_mfma_weights(W1, b1, W2, b2, W3, b3, bf16=True):
+    """Weights of the 72->32->32->4 MLP in matrix-core operand order (uint8 [N*7808]); once per scene."""
+    n = W1.shape[0]
+    if tuple(W1.shape[1:]) != (32, 72) or tuple(W2.shape[1:]) != (32, 32) or tuple(W3.shape[1:]) != (4, 32):
+        raise RuntimeError("the matrix-core path supports the 72->32->32->4 MLP only")
+    ws = [_f32c(w, "weights") for w in (W1, b1, W2, b2, W3, b3)]
+    lib = _lib.load()
+    packed = torch.empty(lib.mlpsp_mfma_pack_bytes(n), dtype=torch.uint8, device=W1.device)
+    code = lib.mlpsp_pack_mfma_weights(*[_ptr(w) for w in ws], n, int(bool(bf16)), _ptr(packed), _stream(W1.device))
+    _check(code, "mlpsp_pack_mfma_weights")
+    return packed
+
+
+def render_tilecenter_mfma(rays_o, rays_d, records, order, tile_offsets, freq, att, W1, b1, W2, b2, W3, b3, W, H,
+                           threshold, bf16=True, counters=None, packed=None, check=True):
+    """Matrix-core tile-centre forward (8x8 tiles) -> (rgb, alpha, nonfinite).
+
+    ``nonfinite`` is a bool when ``check`` (one 4-byte readback) or the int32 device flag otherwise.
+    """
+    dev = rays_o.device
+    if freq.numel() != 6:
+        raise RuntimeError("the matrix-core path supports 6 frequencies only")
+    if packed is None:
+        packed = pack_mfma_weights(W1, b1, W2, b2, W3, b3, bf16)
+    B = W * H
+    rgb = torch.empty(B, 3, dtype=torch.float32, device=dev)
+    alpha = torch.empty(B, 1, dtype=torch.float32, device=dev)
+    flag = torch.empty(1, dtype=torch.int32, device=dev)
+    code = _lib.load().mlpsp_render_tilecenter_mfma(
+        _ptr(rays_o), _ptr(rays_d), _ptr(records), _ptr(order), _ptr(tile_offsets), _ptr(freq), _ptr(att), _ptr(packed),
+        W1.shape[0], int(bool(bf16)), W, H, float(threshold), _ptr(rgb), _ptr(alpha), _ptr(flag), _ptr(counters),
+        _stream(dev))
+    _check(code, "mlpsp_render_tilecenter_mfma")
+    return rgb, alpha, (bool(flag.item()) if check else flag)

@@ -47,6 +47,8 @@ class TileExt:
         self._lock = threading.Lock()
         self._mfma_calls = 0
         self._mfma_fallbacks = 0
+        self._pack_key = None
+        self._pack = None
 
     def __getattr__(self, name):
         if name in _BACKWARD_ONLY:
@@ -225,6 +227,16 @@ class TileExt:
     def rgb_wmma_safety_stats(self):
         return [self._mfma_calls, self._mfma_fallbacks]
 
+    def _packed_weights(self, ws, bf16):
+        """Matrix-core operand copy of the six weight tensors, rebuilt only when one of them changed
+        (identity, shape or in-place version) -- the scene's weights are constant during inference."""
+        key = (bool(bf16),) + tuple((w.data_ptr(), w._version, tuple(w.shape), str(w.device)) for w in ws)
+        with self._lock:
+            if self._pack_key != key:
+                self._pack = ops.pack_mfma_weights(*ws, bf16=bf16)
+                self._pack_key = key
+            return self._pack
+
     def render_tiles_rgb_wmma(self, x, width, height, threshold, bf16):
         """[rgb, alpha] with the 72->32->32->4 MLP on the matrix cores, f32 everywhere else."""
         _chk(len(x) == 15, "WMMA requires the 15 scene tensors")
@@ -253,8 +265,9 @@ class TileExt:
             if x[5].numel() > 0:
                 order, _ = ops.sort_tiles(x[0], x[1], rec, x[5], x[6], width, height, 8, 8, _lib.KEY_TSTAR,
                                           self.max_tile_prims)
+            packed = self._packed_weights(list(x[9:15]), bool(bf16))
             rgb, alpha, nonfinite = ops.render_tilecenter_mfma(x[0], x[1], rec, order, x[6], x[7], x[8], *x[9:15],
-                                                               width, height, threshold, bf16=bool(bf16))
+                                                               width, height, threshold, bf16=bool(bf16), packed=packed)
             if nonfinite:
                 for i, t in enumerate(x):
                     if i not in (5, 6):

@@ -1,0 +1,125 @@
+"""The matrix-core render path (bf16 / fp16 MFMA, f32 accumulate) against the oracle.
+
+Tolerances, on the final image (absolute): 5e-3 with bf16 operands, 5e-4 with fp16 operands, against
+BOTH the oracle's emulation of the reference's rounding points (rgb_wmma.cuh:144-213) and the plain f32
+oracle.  The hit geometry is the f32 path's, so the work counters must agree exactly with the f32 oracle
+except where a pixel's transmittance lands on the 1e-3 floor.
+"""
+import numpy as np
+import pytest
+import torch
+
+from conftest import to_dev
+from helpers import Frame
+
+pytestmark = pytest.mark.gpu
+
+TOL = {True: 5e-3, False: 5e-4}
+
+
+def _mfma(fr, device, cand, off, bf16, counters=None):
+    from mlp_splatting_amd import ops
+    sc = fr.scene
+    t = lambda a: to_dev(a, device)
+    rec = ops.prepare_primitives(t(sc.positions), t(sc.log_scales), t(sc.quats))
+    ro, rd, c, o = t(fr.rays_o), t(fr.rays_d), t(cand), t(off)
+    order, _ = ops.sort_tiles(ro, rd, rec, c, o, fr.W, fr.H, 8, 8)
+    return ops.render_tilecenter_mfma(ro, rd, rec, order, o, t(sc.freq), t(sc.att), *[t(w) for w in sc.mlp()], fr.W,
+                                      fr.H, fr.thr, bf16=bf16, counters=counters)
+
+
+@pytest.mark.parametrize("bf16", [True, False])
+@pytest.mark.parametrize("width,height", [(160, 120), (52, 44)])
+def test_matrix_core_render_against_oracle(device, oracle_mod, bf16, width, height):
+    fr = Frame("cfg1_5k_160x120", hidden=32, width=width, height=height)
+    cand, off = fr.oracle_lists(oracle_mod)
+    emu = oracle_mod.render_tilecenter(*fr.base_numpy(cand, off), *fr.dims, precision=1 if bf16 else 2)
+    f32 = oracle_mod.render_tilecenter(*fr.base_numpy(cand, off), *fr.dims)
+    counters = torch.zeros(4, dtype=torch.int64, device=device)
+    rgb, alpha, nonfinite = _mfma(fr, device, cand, off, bf16, counters)
+    assert not nonfinite and f32["alpha"].mean() > 0.5
+    got, got_a = rgb.cpu().numpy(), alpha.cpu().numpy()
+    tol = TOL[bf16]
+    print(f"bf16={bf16}: max|gpu-emu|={np.abs(got - emu['rgb']).max():.2e} max|gpu-f32|={np.abs(got - f32['rgb']).max():.2e}")
+    assert np.abs(got - emu["rgb"]).max() <= tol and np.abs(got_a - emu["alpha"]).max() <= tol
+    assert np.abs(got - f32["rgb"]).max() <= tol and np.abs(got_a - f32["alpha"]).max() <= tol
+    assert np.abs(got - f32["rgb"]).max() > 0            # it is not the f32 kernel in disguise
+    c = counters.cpu().numpy()
+    assert abs(int(c[3]) - int(emu["stats"][3])) <= 0.002 * emu["stats"][3]
+    assert c[1] >= c[2] > 0
+
+
+def test_matrix_core_matches_rounded_closed_form(device):
+    # zero weights: colour = sigmoid(b3), independent of the operand rounding -> must equal the f32 kernel
+    from mlp_splatting_amd.tile_ext import TileExt
+    ext = TileExt()
+    n = 6
+    pos = torch.zeros(n, 3, device=device); pos[:, 2] = torch.arange(1, n + 1, device=device)
+    quats = torch.zeros(n, 4, device=device); quats[:, 0] = 1
+    b3 = torch.tensor([[0.3, -0.4, 1.1, 0.2]], device=device).repeat(n, 1)
+    W, H = 8, 8
+    ro = torch.zeros(W * H, 3, device=device)
+    rd = torch.nn.functional.normalize(torch.tensor([[0.0, 0.0, 1.0]], device=device).repeat(W * H, 1) +
+                                       0.01 * torch.randn(W * H, 3, device=device), dim=-1).contiguous()
+    x = [ro, rd, pos, torch.full((n, 3), -1.0, device=device), quats, torch.arange(n, dtype=torch.int32, device=device),
+         torch.tensor([0, n], dtype=torch.int32, device=device), torch.ones(6, device=device), torch.ones(6, device=device),
+         torch.zeros(n, 32, 72, device=device), torch.zeros(n, 32, device=device), torch.zeros(n, 32, 32, device=device),
+         torch.zeros(n, 32, device=device), torch.zeros(n, 4, 32, device=device), b3]
+    rgb, alpha = ext.render_tiles_rgb_wmma(x, W, H, 1e-3, True)
+    want = ext.render_tiles_forward_tilecenter(*x, W, H, 8, 8, 1e-3)
+    torch.testing.assert_close(rgb, want[0], rtol=0, atol=1e-6)
+    torch.testing.assert_close(alpha, want[1], rtol=0, atol=1e-6)
+    assert float(alpha.mean()) > 0.5
+
+
+def test_overflow_falls_back_to_f32_for_the_whole_frame(device, oracle_mod):
+    # rgb_wmma.cuh:260-272 / tests/test_training_wmma.py:308-339: a weight beyond the fp16 range makes
+    # the rounded operand infinite -> flag -> the frame is rendered by the scalar f32 kernel instead
+    from mlp_splatting_amd.tile_ext import TileExt
+    fr = Frame("cfg1_5k_160x120", n=400, hidden=32, width=32, height=24)
+    cand, off = fr.oracle_lists(oracle_mod)
+    sc = fr.scene
+    sc.W2[cand[0], 3, 5] = 1.0e5           # finite in f32 and bf16, infinite in fp16
+    ext = TileExt()
+    x = [to_dev(a, device) for a in fr.base_numpy(cand, off)]
+    calls0, fb0 = ext.rgb_wmma_safety_stats()
+    with pytest.warns(UserWarning, match="scalar FP32 instead"):
+        rgb, alpha = ext.render_tiles_rgb_wmma(x, fr.W, fr.H, fr.thr, False)
+    want = ext.render_tiles_forward_tilecenter(*x, fr.W, fr.H, 8, 8, fr.thr)
+    assert torch.equal(rgb, want[0]) and torch.equal(alpha, want[1])
+    assert ext.rgb_wmma_safety_stats() == [calls0 + 1, fb0 + 1]
+    rgb_b, _ = ext.render_tiles_rgb_wmma(x, fr.W, fr.H, fr.thr, True)       # bf16 holds 1e5: no fallback
+    assert ext.rgb_wmma_safety_stats() == [calls0 + 2, fb0 + 1]
+    # non-finite INPUT is an error, not a fallback
+    x[9] = x[9].clone()
+    x[9][int(cand[0]), 0, 0] = float("nan")
+    with pytest.raises(RuntimeError, match="input is nonfinite"):
+        ext.render_tiles_rgb_wmma(x, fr.W, fr.H, fr.thr, True)
+
+
+def test_packed_weights_are_cached_until_a_tensor_changes(device, oracle_mod):
+    from mlp_splatting_amd.tile_ext import TileExt
+    fr = Frame("cfg1_5k_160x120", n=300, hidden=32, width=24, height=16)
+    cand, off = fr.oracle_lists(oracle_mod)
+    ext = TileExt()
+    x = [to_dev(a, device) for a in fr.base_numpy(cand, off)]
+    a, _ = ext.render_tiles_rgb_wmma(x, fr.W, fr.H, fr.thr, True)
+    pack1 = ext._pack
+    b, _ = ext.render_tiles_rgb_wmma(x, fr.W, fr.H, fr.thr, True)
+    assert ext._pack is pack1 and torch.equal(a, b)
+    x[14].add_(0.5)                                          # in-place edit bumps the tensor version
+    c, _ = ext.render_tiles_rgb_wmma(x, fr.W, fr.H, fr.thr, True)
+    assert ext._pack is not pack1 and not torch.equal(a, c)
+
+
+def test_scene_module_precision_switch(device, oracle_mod):
+    from test_gpu_scene import _call, _scene_from
+    fr = Frame("cfg1_5k_160x120", n=1500, hidden=32, width=64, height=48)
+    scene = _scene_from(fr, device)
+    ref = _call(scene, fr, device)
+    scene.render_precision = "bf16"
+    fast = _call(scene, fr, device)
+    assert 0 < float((fast - ref).abs().max()) <= 5e-3
+    scene.render_precision = "int8"
+    with pytest.raises(ValueError, match="render_precision"):
+        _call(scene, fr, device)
