@@ -158,9 +158,10 @@ int mlpsp_render_per_pixel_f32(const float* rays_o_dev, const float* rays_d_dev,
  *   f32 biases, in MFMA operand order: mlpsp_mfma_pack_bytes(N) bytes, 128-byte aligned.  Done once per
  *   set of weights (the reference re-casts them for every tile and primitive, rgb_wmma.cuh:162-174).
  * mlpsp_render_tilecenter_mfma: geometry, activations and compositing in f32; encoded inputs, weights
- *   and hidden activations in bf16/fp16 with f32 accumulation.  *nonfinite_dev (int32, zeroed by the
- *   call) becomes 1 if a non-finite operand, pre-activation or logit was met on an active ray, in
- *   which case the caller re-renders the frame with mlpsp_render_tilecenter_f32 (rgb_wmma.cuh:260-272). */
+ *   and hidden activations in bf16/fp16 with f32 accumulation.  status_dev: 16 int32 of device
+ *   scratch, zeroed by the call; status_dev[0] becomes 1 if a non-finite operand, pre-activation or
+ *   logit was met on an active ray, in which case the caller re-renders the frame with
+ *   mlpsp_render_tilecenter_f32 (rgb_wmma.cuh:260-272); the other words are reserved. */
 size_t mlpsp_mfma_pack_bytes(int num_primitives);
 int mlpsp_pack_mfma_weights(const float* W1, const float* b1, const float* W2, const float* b2, const float* W3,
                             const float* b3, int num_primitives, int use_bf16, void* packed_dev,
@@ -169,7 +170,7 @@ int mlpsp_render_tilecenter_mfma(const float* rays_o_dev, const float* rays_d_de
                                  const int32_t* order_dev, const int32_t* tile_offsets_dev, const float* freq_dev,
                                  const float* att_dev, const void* packed_dev, int num_primitives, int use_bf16,
                                  int width, int height, float threshold, float* out_rgb_dev, float* out_alpha_dev,
-                                 int32_t* nonfinite_dev, int64_t* counters_dev, mlpsp_stream_t stream);
+                                 int32_t* status_dev, int64_t* counters_dev, mlpsp_stream_t stream);
 
 #ifdef __cplusplus
 }

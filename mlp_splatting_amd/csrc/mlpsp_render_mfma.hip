@@ -19,7 +19,9 @@
 // Layer-1 k-slots: lane group g = l/32 owns frequencies 3g..3g+2 of every input component, so both
 // groups evaluate 18 (sin, cos) pairs per pixel block and each pair lands in one 32-bit operand word.
 // sin/cos use the native v_sin_f32/v_cos_f32 (argument in revolutions); their error (~1e-6) is far
-// below the bf16 rounding applied next.
+// below the bf16 rounding applied next.  (Measured alternatives that did not pay on gfx950: a 4096-entry
+// LDS sin/cos table -- same kernel time, 2x the image error; persistent wavefronts with a tile work
+// queue -- 6 % slower than one wavefront per tile.)
 #include "mlpsp_device.hpp"
 #include "mlpsp_host.hpp"
 
@@ -138,24 +140,71 @@ __global__ __launch_bounds__(64) void pack_mfma_weights_kernel(const float* __re
 // render
 // ---------------------------------------------------------------------------------------------
 
+// True if some pre-activation is +-inf or exceeds the operand type's range.  A NaN cannot appear here
+// on its own: the operands are finite (weights are checked when packed, phases when encoded), so a
+// non-finite accumulator is an overflow, which shows as +-inf -- and the max chain sees infinities.
+// One-instruction forms.  fmaxf() in C costs two (the compiler first quiets a possible signalling NaN
+// with v_max x,x,x), which would double the 64 ReLUs per (tile, primitive).
+__device__ __forceinline__ float relu(float x) {
+  float y;
+  asm("v_max_f32_e32 %0, 0, %1" : "=v"(y) : "v"(x));
+  return y;
+}
+__device__ __forceinline__ float max3_abs(float a, float b, float c) {
+  float y;
+  asm("v_max3_f32 %0, |%1|, |%2|, |%3|" : "=v"(y) : "v"(a), "v"(b), "v"(c));
+  return y;
+}
 template <typename T>
-__device__ __forceinline__ bool not_finite_in(const f32x16& v) {
-  bool bad = false;
+__device__ __forceinline__ bool out_of_range_in(const f32x16& v) {
+  float m = max3_abs(v[0], v[1], v[2]);
 #pragma unroll
-  for (int r = 0; r < 16; ++r) bad |= !(__builtin_fabsf(v[r]) <= Ops<T>::kMax);
-  return bad;
+  for (int r = 3; r < 15; r += 2) m = max3_abs(m, v[r], v[r + 1]);
+  m = max3_abs(m, v[15], v[15]);
+  return !(m <= Ops<T>::kMax);
+}
+
+// f32 activations with the native exp2/log2/rcp instructions (relative error ~1e-6, far below the
+// operand rounding of this path).  Same formulas as np_tile_kernels.cu:75-83, 2092-2103.
+__device__ __forceinline__ float fast_exp(float x) { return __builtin_amdgcn_exp2f(x * 1.44269504f); }
+__device__ __forceinline__ float fast_sigmoid(float x) { return __builtin_amdgcn_rcpf(1.0f + fast_exp(-x)); }
+__device__ __forceinline__ float fast_softplus(float x) {
+  const float e = fast_exp(x);
+  const float mid = __builtin_amdgcn_logf(1.0f + e) * 0.693147181f;
+  float y = (x < -20.f) ? e : mid;
+  y = (x > 20.f) ? x : y;
+  return y;
+}
+__device__ __forceinline__ void fast_blend_step(PixelAcc& a, float o0, float o1, float o2, float o3, float decay) {
+  const float sigma = fast_softplus(o3) * decay;
+  const float alpha = 1.f - fast_exp(-sigma);
+  const float w = a.trans * alpha;
+  a.cr = fmaf(w, fast_sigmoid(o0), a.cr);
+  a.cg = fmaf(w, fast_sigmoid(o1), a.cg);
+  a.cb = fmaf(w, fast_sigmoid(o2), a.cb);
+  a.trans = a.trans * (1.f - alpha);
 }
 
 template <typename T>
 __global__ __launch_bounds__(64) void render_tilecenter_mfma_kernel(
     const float* __restrict__ rays_o, const float* __restrict__ rays_d, const PrimRecord* __restrict__ prims,
     const int32_t* __restrict__ order, const int32_t* __restrict__ offsets, const float* __restrict__ freq,
-    const float* __restrict__ att, const unsigned char* __restrict__ packed, int N, int W, int H, int ntx, int per_xcd, int num_tiles, float thr,
-    float* __restrict__ out_rgb, float* __restrict__ out_alpha, int32_t* __restrict__ nonfinite,
-    unsigned long long* __restrict__ counters) {
+    const float* __restrict__ att, const unsigned char* __restrict__ packed, int N, int W, int H, int ntx,
+    int per_xcd, int num_tiles, float thr, float* __restrict__ out_rgb, float* __restrict__ out_alpha,
+    int32_t* __restrict__ status, unsigned long long* __restrict__ counters) {
+  // XCD-aware work assignment: XCD k (blockIdx.x % 8) walks tiles [k*per_xcd, (k+1)*per_xcd) in
+  // row-major order, so neighbouring tiles -- which share most primitives -- run together on one L2.
   const int tile = (blockIdx.x % kNumXcd) * per_xcd + blockIdx.x / kNumXcd;
   if (tile >= num_tiles) return;
   const int l = threadIdx.x, g = l >> 5;
+  // per-lane phase scales, freq_f * att_f / (2 pi) revolutions per unit input: lane group g evaluates
+  // frequencies 3g, 3g+1, 3g+2
+  constexpr float kInvTwoPi = 0.159154943f;
+  const float kf0 = (freq[3 * g + 0] * att[3 * g + 0]) * kInvTwoPi;
+  const float kf1 = (freq[3 * g + 1] * att[3 * g + 1]) * kInvTwoPi;
+  const float kf2 = (freq[3 * g + 2] * att[3 * g + 2]) * kInvTwoPi;
+  unsigned n_proc = 0, n_proc_hit = 0, n_hits = 0;
+  bool bad = false;
   const int tx = tile % ntx, ty = tile / ntx;
   const int x = tx * 8 + (l & 7), y = ty * 8 + (l >> 3);
   const bool valid = (x < W) && (y < H);
@@ -166,17 +215,9 @@ __global__ __launch_bounds__(64) void render_tilecenter_mfma_kernel(
               rdz = valid ? rays_d[pix * 3 + 2] : 0.f;
   // the pixel this lane shares an MFMA column with: lane l and lane l^32 both hold column l%32
   const float prdx = __shfl_xor(rdx, 32), prdy = __shfl_xor(rdy, 32), prdz = __shfl_xor(rdz, 32);
-  // per-lane phase scales in revolutions per unit input, freq_f * att_f / (2 pi): group g evaluates
-  // frequencies 3g, 3g+1, 3g+2
-  constexpr float kInvTwoPi = 0.159154943f;
-  const float kf0 = (freq[3 * g + 0] * att[3 * g + 0]) * kInvTwoPi;
-  const float kf1 = (freq[3 * g + 1] * att[3 * g + 1]) * kInvTwoPi;
-  const float kf2 = (freq[3 * g + 2] * att[3 * g + 2]) * kInvTwoPi;
 
   const int start = offsets[tile], end = offsets[tile + 1];
   PixelAcc acc = {0.f, 0.f, 0.f, 1.f, 0.f, 0.f};
-  unsigned n_proc = 0, n_proc_hit = 0, n_hits = 0;
-  bool bad = false;
 
   for (int i = start; i < end; ++i) {
     const int p = __builtin_amdgcn_readfirstlane(order[i]);
@@ -202,17 +243,6 @@ __global__ __launch_bounds__(64) void render_tilecenter_mfma_kernel(
         a3[s] = u32x4{0u, 0u, 0u, 0u};
         if ((l & 31) < 4) a3[s] = *reinterpret_cast<const u32x4*>(blk + kOffW3 + ((s * 2 + g) * 4 + (l & 3)) * 16);
       }
-      f32x16 bias1, bias2;
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const f32x4 v1 = *reinterpret_cast<const f32x4*>(blk + kOffB1 + g * 64 + q * 16);
-        const f32x4 v2 = *reinterpret_cast<const f32x4*>(blk + kOffB2 + g * 64 + q * 16);
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          bias1[4 * q + e] = v1[e];
-          bias2[4 * q + e] = v2[e];
-        }
-      }
       const f32x4 b3v = *reinterpret_cast<const f32x4*>(blk + kOffB3);
       const int wflag = *reinterpret_cast<const int32_t*>(blk + kOffFlag);
       bad |= (wflag != 0);
@@ -223,16 +253,26 @@ __global__ __launch_bounds__(64) void render_tilecenter_mfma_kernel(
       float o_blk[2][4];
 #pragma unroll
       for (int b = 0; b < 2; ++b) {
-#pragma unroll
-        for (int k = 0; k < 4; ++k) o_blk[b][k] = 0.f;
         const unsigned half_mask = (unsigned)(mask >> (32 * b));
         if (half_mask != 0u) {   // wave-uniform: skip a 32-pixel block nobody hits
           const bool own = (b == g);
           const float xin[6] = {own ? rdx : prdx, own ? rdy : prdy, own ? rdz : prdz,
                                 own ? h.dx : pdx, own ? h.dy : pdy, own ? h.dz : pdz};
           const bool col_active = (half_mask >> (l & 31)) & 1u;
+          // biases are the C operand of each layer's first MFMA; an MFMA overwrites its C registers,
+          // so each column block fetches its own copy (L1-resident) instead of copying 32 registers
+          f32x16 d1, d2;
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const f32x4 v1 = *reinterpret_cast<const f32x4*>(blk + kOffB1 + g * 64 + q * 16);
+            const f32x4 v2 = *reinterpret_cast<const f32x4*>(blk + kOffB2 + g * 64 + q * 16);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              d1[4 * q + e] = v1[e];
+              d2[4 * q + e] = v2[e];
+            }
+          }
           // layer 1: 18 (sin, cos) words per lane, 5 K-steps
-          f32x16 d1 = bias1;
 #pragma unroll
           for (int s = 0; s < 5; ++s) {
             u32x4 bw;
@@ -249,38 +289,32 @@ __global__ __launch_bounds__(64) void render_tilecenter_mfma_kernel(
             }
             d1 = Ops<T>::mfma(a1[s], bw, d1);
           }
-          bad |= col_active && not_finite_in<T>(d1);
+          bad |= col_active && out_of_range_in<T>(d1);
           // layer 2: the D registers, rectified and rounded, are the next B operand
-          f32x16 d2 = bias2;
 #pragma unroll
           for (int s = 0; s < 2; ++s) {
             u32x4 bw;
 #pragma unroll
             for (int d = 0; d < 4; ++d)
-              bw[d] = Ops<T>::pack2(fmaxf(d1[8 * s + 2 * d], 0.f), fmaxf(d1[8 * s + 2 * d + 1], 0.f));
+              bw[d] = Ops<T>::pack2(relu(d1[8 * s + 2 * d]), relu(d1[8 * s + 2 * d + 1]));
             d2 = Ops<T>::mfma(a2[s], bw, d2);
           }
-          bad |= col_active && not_finite_in<T>(d2);
+          bad |= col_active && out_of_range_in<T>(d2);
           // layer 3: rows 0..3 of a 32-row product; row k lands in register k of lane group 0
-          f32x16 d3;
-#pragma unroll
-          for (int r = 0; r < 16; ++r) d3[r] = 0.f;
-          if (g == 0) {
-            d3[0] = b3v[0];
-            d3[1] = b3v[1];
-            d3[2] = b3v[2];
-            d3[3] = b3v[3];
-          }
+          f32x16 d3 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
           for (int s = 0; s < 2; ++s) {
             u32x4 bw;
 #pragma unroll
             for (int d = 0; d < 4; ++d)
-              bw[d] = Ops<T>::pack2(fmaxf(d2[8 * s + 2 * d], 0.f), fmaxf(d2[8 * s + 2 * d + 1], 0.f));
+              bw[d] = Ops<T>::pack2(relu(d2[8 * s + 2 * d]), relu(d2[8 * s + 2 * d + 1]));
             d3 = Ops<T>::mfma(a3[s], bw, d3);
           }
 #pragma unroll
           for (int k = 0; k < 4; ++k) o_blk[b][k] = d3[k];
+        } else {
+#pragma unroll
+          for (int k = 0; k < 4; ++k) o_blk[b][k] = 0.f;
         }
       }
       // pixel l < 32 reads block 0 from its own lane; pixel l >= 32 reads block 1 from lane l-32
@@ -288,12 +322,12 @@ __global__ __launch_bounds__(64) void render_tilecenter_mfma_kernel(
 #pragma unroll
       for (int k = 0; k < 4; ++k) {
         const float from_partner = __shfl_xor(o_blk[1][k], 32);
-        o[k] = g ? from_partner : o_blk[0][k];
+        o[k] = (g ? from_partner : o_blk[0][k]) + b3v[k];
       }
       if (hit) {
         bad |= !(__builtin_fabsf(o[0]) <= 3.4028235e38f) || !(__builtin_fabsf(o[1]) <= 3.4028235e38f) ||
                !(__builtin_fabsf(o[2]) <= 3.4028235e38f) || !(__builtin_fabsf(o[3]) <= 3.4028235e38f);
-        blend_step(acc, o[0], o[1], o[2], o[3], h.decay, h.t);
+        fast_blend_step(acc, o[0], o[1], o[2], o[3], h.decay);
       }
     }
     if (__ballot(valid && (acc.trans >= kTransmittanceFloor)) == 0ull) break;
@@ -305,7 +339,7 @@ __global__ __launch_bounds__(64) void render_tilecenter_mfma_kernel(
     out_rgb[pix * 3 + 2] = acc.cb;
     out_alpha[pix] = 1.f - acc.trans;
   }
-  if (__ballot(bad) != 0ull && l == 0) atomicExch(nonfinite, 1);
+  if (__ballot(bad) != 0ull && l == 0) atomicExch(status, 1);
   if (counters && l == 0) {
     atomicAdd(counters + 1, (unsigned long long)n_proc);
     atomicAdd(counters + 2, (unsigned long long)n_proc_hit);
@@ -344,15 +378,15 @@ MLPSP_API int mlpsp_render_tilecenter_mfma(const float* rays_o_dev, const float*
                                            const int32_t* tile_offsets_dev, const float* freq_dev,
                                            const float* att_dev, const void* packed_dev, int num_primitives,
                                            int use_bf16, int width, int height, float threshold, float* out_rgb_dev,
-                                           float* out_alpha_dev, int32_t* nonfinite_dev, int64_t* counters_dev,
+                                           float* out_alpha_dev, int32_t* status_dev, int64_t* counters_dev,
                                            mlpsp_stream_t stream) {
   const int64_t T = checked_num_tiles(width, height, 8, 8);
   if (T <= 0 || T > 2147483647LL - 8 || num_primitives < 0) return MLPSP_E_ARGUMENT;
   if (!rays_o_dev || !rays_d_dev || !tile_offsets_dev || !freq_dev || !att_dev || !out_rgb_dev || !out_alpha_dev ||
-      !nonfinite_dev)
+      !status_dev)
     return MLPSP_E_ARGUMENT;
   if (num_primitives > 0 && !packed_dev) return MLPSP_E_ARGUMENT;
-  MLPSP_HIP_TRY(hipMemsetAsync(nonfinite_dev, 0, sizeof(int32_t), (hipStream_t)stream));
+  MLPSP_HIP_TRY(hipMemsetAsync(status_dev, 0, 16 * sizeof(int32_t), (hipStream_t)stream));
   const int per_xcd = (int)((T + kNumXcd - 1) / kNumXcd);
   const dim3 grid((unsigned)(per_xcd * kNumXcd)), block(64);
   hipStream_t s = (hipStream_t)stream;
@@ -362,12 +396,12 @@ MLPSP_API int mlpsp_render_tilecenter_mfma(const float* rays_o_dev, const float*
     hipLaunchKernelGGL(render_tilecenter_mfma_kernel<__bf16>, grid, block, 0, s, rays_o_dev, rays_d_dev,
                        (const PrimRecord*)prim_records_dev, order_dev, tile_offsets_dev, freq_dev, att_dev,
                        (const unsigned char*)packed_dev, num_primitives, width, height, ntx, per_xcd, (int)T, threshold,
-                       out_rgb_dev, out_alpha_dev, nonfinite_dev, ctr);
+                       out_rgb_dev, out_alpha_dev, status_dev, ctr);
   else
     hipLaunchKernelGGL(render_tilecenter_mfma_kernel<_Float16>, grid, block, 0, s, rays_o_dev, rays_d_dev,
                        (const PrimRecord*)prim_records_dev, order_dev, tile_offsets_dev, freq_dev, att_dev,
                        (const unsigned char*)packed_dev, num_primitives, width, height, ntx, per_xcd, (int)T, threshold,
-                       out_rgb_dev, out_alpha_dev, nonfinite_dev, ctr);
+                       out_rgb_dev, out_alpha_dev, status_dev, ctr);
   MLPSP_LAUNCH_CHECK();
   return MLPSP_OK;
 }

@@ -235,10 +235,10 @@ def render_tilecenter_mfma(rays_o, rays_d, records, order, tile_offsets, freq, a
     B = W * H
     rgb = torch.empty(B, 3, dtype=torch.float32, device=dev)
     alpha = torch.empty(B, 1, dtype=torch.float32, device=dev)
-    flag = torch.empty(1, dtype=torch.int32, device=dev)
+    flag = torch.empty(16, dtype=torch.int32, device=dev)
     code = _lib.load().mlpsp_render_tilecenter_mfma(
         _ptr(rays_o), _ptr(rays_d), _ptr(records), _ptr(order), _ptr(tile_offsets), _ptr(freq), _ptr(att), _ptr(packed),
         W1.shape[0], int(bool(bf16)), W, H, float(threshold), _ptr(rgb), _ptr(alpha), _ptr(flag), _ptr(counters),
         _stream(dev))
     _check(code, "mlpsp_render_tilecenter_mfma")
-    return rgb, alpha, (bool(flag.item()) if check else flag)
+    return rgb, alpha, (bool(flag[0].item()) if check else flag)
