@@ -98,7 +98,7 @@ def main() -> int:
         e[0].record()
         cand, off = ops.bin_legacy(scene.positions.detach(), scene.log_scales.detach(), view[None], proj, W, H, 8, thr)
         e[1].record()
-        order, _ = ops.sort_tiles(ro, rd, rec, cand, off, W, H, 8, 8)
+        order, _ = ops.sort_tiles(ro, rd, rec, cand, off, W, H, 8, 8, cull_threshold=thr)
         counters = torch.zeros(4, dtype=torch.int64, device=dev)
         e[2].record()
         if precision == "bf16":

@@ -104,11 +104,15 @@ int mlpsp_bin_raycone_fill(int num_primitives, int width, int height, int tile, 
 /* Per-tile depth-key sort = the in-kernel cub::BlockRadixSort of np_tile_kernels.cu:1929-1990,
  * materialised: sorted_ids_dev[P] holds, tile by tile, the candidates in ascending key order, ties
  * in list order; entries past min(len, capacity) keep list order.  sorted_keys_dev may be NULL.
- * capacity <= MLPSP_TILE_CAPACITY_MAX (0 = that maximum). */
+ * capacity <= MLPSP_TILE_CAPACITY_MAX (0 = that maximum).
+ * cull_threshold: 0 = off.  In (0,1) (the render's score threshold): a candidate that provably hits
+ * no ray of its tile at that threshold is written as ~id (negative).  The render entry points skip
+ * negative ids, so images are unchanged; ~ recovers the plain sorted list.  Has no counterpart in the
+ * reference, whose kernels run the full ray test on every candidate. */
 int mlpsp_sort_tiles(const float* rays_o_dev, const float* rays_d_dev, const void* prim_records_dev,
                      const int32_t* candidates_dev, const int32_t* tile_offsets_dev, int width, int height,
-                     int tile_w, int tile_h, int key_family, int capacity, int32_t* sorted_ids_dev,
-                     float* sorted_keys_dev, mlpsp_stream_t stream);
+                     int tile_w, int tile_h, int key_family, int capacity, float cull_threshold,
+                     int32_t* sorted_ids_dev, float* sorted_keys_dev, mlpsp_stream_t stream);
 
 /* Tile-centre-order forward, scalar f32 (render_tiles_kernel_tilecenter_order,
  * np_tile_kernels.cu:1837-2137; with out_t_dev != NULL also the expected depth of :5432-5719).

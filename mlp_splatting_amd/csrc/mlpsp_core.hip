@@ -2,6 +2,8 @@
 #include "mlpsp_device.hpp"
 #include "mlpsp_host.hpp"
 
+#include <math.h>
+
 namespace mlpsp {
 
 // ---------------------------------------------------------------------------------------------
@@ -27,12 +29,14 @@ __global__ __launch_bounds__(256) void prepare_primitives_kernel(const float* __
   r.mx = det_exp(-2.f * r.lgx);
   r.my = det_exp(-2.f * r.lgy);
   r.mz = det_exp(-2.f * r.lgz);
-  r.pad0 = r.pad1 = r.pad2 = 0.f;
+  r.s2x = det_exp(2.f * r.lgx);
+  r.s2y = det_exp(2.f * r.lgy);
+  r.s2z = det_exp(2.f * r.lgz);
   float4* dst = reinterpret_cast<float4*>(out + p);
   dst[0] = make_float4(r.cx, r.cy, r.cz, r.mx);
   dst[1] = make_float4(r.my, r.mz, r.qw, r.qx);
   dst[2] = make_float4(r.qy, r.qz, r.lgx, r.lgy);
-  dst[3] = make_float4(r.lgz, 0.f, 0.f, 0.f);
+  dst[3] = make_float4(r.lgz, r.s2x, r.s2y, r.s2z);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -72,16 +76,36 @@ __global__ __launch_bounds__(256) void validate_tile_lists_kernel(const int32_t*
 // like their values, and the list index in the low word makes equal keys keep list order, which
 // is what a stable radix sort on the key alone yields.  Bitonic network in LDS on the next power
 // of two, padded with all-ones words.
+//
+// Optional conservative culling (cull_threshold in (0,1)): a candidate list comes from a bounding
+// circle on screen, and more than half of its entries hit no pixel of the tile -- yet the render
+// kernels spend a full 64-lane ray/ellipsoid test on each.  Here, where one LANE handles one
+// candidate, the tile's rays are enclosed in the pyramid of its four corner rays (verified against
+// every ray of the tile), and a candidate whose threshold ellipsoid {x : (x-c)^T A (x-c) < -2 ln thr}
+// lies entirely beyond one of the pyramid's four faces can be hit by no ray of the tile.  For a face
+// with inward normal n through the common origin o that is  n.(c-o) < 0  and
+// (n.(c-o))^2 >= -2 ln thr * sum_k s_k^2 (R^T n)_k^2, tested with a 2 % margin on the radius, far
+// above f32 rounding.  Such an entry is written as ~id (negative): the render kernels skip negative
+// ids, so the image is unchanged bit for bit, and ~ recovers the exact sorted list.
 // ---------------------------------------------------------------------------------------------
 constexpr int kSortThreads = 256;
 constexpr int kSortMax = MLPSP_TILE_CAPACITY_MAX;
 
+struct TilePyramid {
+  float ox, oy, oz;
+  float n[4][3];
+  int enabled;   // bit j: face j usable
+};
+
 __global__ __launch_bounds__(kSortThreads) void sort_tiles_kernel(
     const float* __restrict__ rays_o, const float* __restrict__ rays_d, const PrimRecord* __restrict__ prims,
     const int32_t* __restrict__ cand, const int32_t* __restrict__ offsets, TileGeom g, int family, int capacity,
-    int32_t* __restrict__ sorted_ids, float* __restrict__ sorted_keys) {
+    float cull_r2, int32_t* __restrict__ sorted_ids, float* __restrict__ sorted_keys) {
   __shared__ unsigned long long s_key[kSortMax];
   __shared__ int32_t s_id[kSortMax];
+  __shared__ TilePyramid s_pyr;
+  __shared__ int s_face_ok[4];
+  __shared__ int s_origin_ok;
   const int tile = blockIdx.x;
   const int tid = threadIdx.x;
   const int start = offsets[tile];
@@ -96,12 +120,78 @@ __global__ __launch_bounds__(kSortThreads) void sort_tiles_kernel(
   int npad = 2;
   while (npad < n) npad <<= 1;
 
+  // ---- the tile's ray pyramid (only when culling is requested)
+  const bool culling = cull_r2 > 0.f;
+  if (culling) {
+    const int tx = tile % g.ntx, ty = tile / g.ntx;
+    const int x0 = tx * g.TW, y0 = ty * g.TH;
+    const int x1 = min(x0 + g.TW, g.W) - 1, y1 = min(y0 + g.TH, g.H) - 1;
+    if (tid == 0) {
+      const int corner[4] = {y0 * g.W + x0, y0 * g.W + x1, y1 * g.W + x1, y1 * g.W + x0};
+      float d[4][3];
+      for (int k = 0; k < 4; ++k)
+        for (int e = 0; e < 3; ++e) d[k][e] = rays_d[corner[k] * 3 + e];
+      s_pyr.ox = rays_o[corner[0] * 3 + 0];
+      s_pyr.oy = rays_o[corner[0] * 3 + 1];
+      s_pyr.oz = rays_o[corner[0] * 3 + 2];
+      for (int j = 0; j < 4; ++j) {
+        const float* a = d[j];
+        const float* b = d[(j + 1) & 3];
+        float nx = a[1] * b[2] - a[2] * b[1], ny = a[2] * b[0] - a[0] * b[2], nz = a[0] * b[1] - a[1] * b[0];
+        // orient towards the tile-centre ray; a face the centre ray (nearly) lies in is not used
+        const float side = nx * dx + ny * dy + nz * dz;
+        const float len = sqrtf(nx * nx + ny * ny + nz * nz);
+        const float sgn = side < 0.f ? -1.f : 1.f;
+        s_pyr.n[j][0] = sgn * nx;
+        s_pyr.n[j][1] = sgn * ny;
+        s_pyr.n[j][2] = sgn * nz;
+        s_face_ok[j] = (len > 0.f && fabsf(side) > 1e-4f * len) ? 1 : 0;
+      }
+      s_origin_ok = 1;
+    }
+    __syncthreads();
+    // every ray of the tile must start at the common origin and lie inside every face used
+    for (int k = tid; k < g.TW * g.TH; k += kSortThreads) {
+      const int x = x0 + k % g.TW, y = y0 + k / g.TW;
+      if (x < g.W && y < g.H) {
+        const int pix = y * g.W + x;
+        if (rays_o[pix * 3] != s_pyr.ox || rays_o[pix * 3 + 1] != s_pyr.oy || rays_o[pix * 3 + 2] != s_pyr.oz)
+          s_origin_ok = 0;
+        const float rx = rays_d[pix * 3], ry = rays_d[pix * 3 + 1], rz = rays_d[pix * 3 + 2];
+        for (int j = 0; j < 4; ++j) {
+          const float inside = s_pyr.n[j][0] * rx + s_pyr.n[j][1] * ry + s_pyr.n[j][2] * rz;
+          const float len = sqrtf(s_pyr.n[j][0] * s_pyr.n[j][0] + s_pyr.n[j][1] * s_pyr.n[j][1] +
+                                  s_pyr.n[j][2] * s_pyr.n[j][2]);
+          if (!(inside >= -1e-6f * len)) s_face_ok[j] = 0;
+        }
+      }
+    }
+    __syncthreads();
+    if (tid == 0)
+      s_pyr.enabled = s_origin_ok ? (s_face_ok[0] | (s_face_ok[1] << 1) | (s_face_ok[2] << 2) | (s_face_ok[3] << 3)) : 0;
+    __syncthreads();
+  }
+  const int faces = culling ? s_pyr.enabled : 0;
+
   for (int i = tid; i < npad; i += kSortThreads) {
     unsigned long long w = ~0ull;
     if (i < n) {
-      const int p = cand[start + i];
-      s_id[i] = p;
+      int p = cand[start + i];
       const PrimRecord P = prims[p];
+      if (faces) {
+        const float ex = P.cx - s_pyr.ox, ey = P.cy - s_pyr.oy, ez = P.cz - s_pyr.oz;
+        bool outside = false;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const float nx = s_pyr.n[j][0], ny = s_pyr.n[j][1], nz = s_pyr.n[j][2];
+          const float dist = nx * ex + ny * ey + nz * ez;
+          const Vec3 nl = quat_rotate_conj(P.qw, P.qx, P.qy, P.qz, Vec3{nx, ny, nz});
+          const float h2 = P.s2x * (nl.x * nl.x) + P.s2y * (nl.y * nl.y) + P.s2z * (nl.z * nl.z);
+          outside |= ((faces >> j) & 1) && (dist < 0.f) && (dist * dist >= cull_r2 * h2);
+        }
+        if (outside) p = ~p;
+      }
+      s_id[i] = p;
       const float key = (family == MLPSP_KEY_DEPTH) ? key_depth(ox, oy, oz, dx, dy, dz, P)
                                                     : key_tstar(ox, oy, oz, dx, dy, dz, P);
       w = ((unsigned long long)float_to_bits(key) << 32) | (unsigned)i;
@@ -132,7 +222,7 @@ __global__ __launch_bounds__(kSortThreads) void sort_tiles_kernel(
       sorted_ids[start + i] = s_id[(int)(w & 0xffffffffu)];
       if (sorted_keys) sorted_keys[start + i] = bits_to_float((uint32_t)(w >> 32));
     } else {
-      sorted_ids[start + i] = cand[start + i];
+      sorted_ids[start + i] = cand[start + i];   // beyond the sort capacity: list order, never culled
       if (sorted_keys) sorted_keys[start + i] = kInvalidKey;
     }
   }
@@ -202,7 +292,8 @@ MLPSP_API int mlpsp_validate_tile_lists(const int32_t* tile_offsets_dev, const i
 MLPSP_API int mlpsp_sort_tiles(const float* rays_o_dev, const float* rays_d_dev, const void* prim_records_dev,
                                const int32_t* candidates_dev, const int32_t* tile_offsets_dev, int width,
                                int height, int tile_w, int tile_h, int key_family, int capacity,
-                               int32_t* sorted_ids_dev, float* sorted_keys_dev, mlpsp_stream_t stream) {
+                               float cull_threshold, int32_t* sorted_ids_dev, float* sorted_keys_dev,
+                               mlpsp_stream_t stream) {
   const int64_t T = checked_num_tiles(width, height, tile_w, tile_h);
   if (T <= 0 || T > 2147483647LL) return MLPSP_E_ARGUMENT;
   if (key_family != MLPSP_KEY_TSTAR && key_family != MLPSP_KEY_DEPTH) return MLPSP_E_ARGUMENT;
@@ -210,9 +301,12 @@ MLPSP_API int mlpsp_sort_tiles(const float* rays_o_dev, const float* rays_d_dev,
   if (capacity == 0) capacity = MLPSP_TILE_CAPACITY_MAX;
   if (!rays_o_dev || !rays_d_dev || !tile_offsets_dev) return MLPSP_E_ARGUMENT;
   TileGeom g{width, height, tile_w, tile_h, ceil_div(width, tile_w), ceil_div(height, tile_h)};
+  // squared radius of the threshold ellipsoid in units of the scales, with a 2 % margin on the radius
+  float cull_r2 = 0.f;
+  if (cull_threshold > 0.f && cull_threshold < 1.f) cull_r2 = -2.0f * logf(cull_threshold) * 1.0404f + 1e-6f;
   hipLaunchKernelGGL(sort_tiles_kernel, dim3((unsigned)T), dim3(kSortThreads), 0, (hipStream_t)stream, rays_o_dev,
                      rays_d_dev, (const PrimRecord*)prim_records_dev, candidates_dev, tile_offsets_dev, g, key_family,
-                     capacity, sorted_ids_dev, sorted_keys_dev);
+                     capacity, cull_r2, sorted_ids_dev, sorted_keys_dev);
   MLPSP_LAUNCH_CHECK();
   return MLPSP_OK;
 }

@@ -127,12 +127,13 @@ __device__ __forceinline__ Vec3 quat_rotate_conj(float qw, float qx, float qy, f
 }
 
 // One primitive's geometry as the kernels consume it: 16 floats, 64-byte aligned, written by
-// the prepare kernel.  m = exp(-2 log_s) is the diagonal of the precision matrix.
+// the prepare kernel.  m = exp(-2 log_s) is the diagonal of the precision matrix, s2 = exp(2 log_s)
+// the squared semi-axes (used only by the conservative tile culling of the sort kernel).
 struct __attribute__((aligned(64))) PrimRecord {
   float cx, cy, cz, mx;
   float my, mz, qw, qx;
   float qy, qz, lgx, lgy;
-  float lgz, pad0, pad1, pad2;
+  float lgz, s2x, s2y, s2z;
 };
 
 struct HitInfo {

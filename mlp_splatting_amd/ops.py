@@ -115,14 +115,17 @@ def bin_legacy(positions, log_scales, view_matrices, proj_matrix, W: int, H: int
 
 
 def sort_tiles(rays_o, rays_d, records, candidates, tile_offsets, W, H, TW, TH, family=_lib.KEY_TSTAR,
-               capacity=TILE_CAPACITY_DEFAULT, want_keys=False):
-    """Materialised per-tile depth order: (sorted_ids [P], sorted_keys [P] | None)."""
+               capacity=TILE_CAPACITY_DEFAULT, want_keys=False, cull_threshold=0.0):
+    """Materialised per-tile depth order: (sorted_ids [P], sorted_keys [P] | None).
+
+    With ``cull_threshold`` (the render's score threshold) candidates that provably hit no ray of their
+    tile come back as ``~id``; the render kernels skip them, the image is unchanged."""
     dev = rays_o.device
     sorted_ids = torch.empty_like(candidates)
     keys = torch.empty(candidates.numel(), dtype=torch.float32, device=dev) if want_keys else None
     code = _lib.load().mlpsp_sort_tiles(_ptr(rays_o), _ptr(rays_d), _ptr(records), _ptr(candidates), _ptr(tile_offsets),
-                                        W, H, TW, TH, int(family), int(capacity), _ptr(sorted_ids), _ptr(keys),
-                                        _stream(dev))
+                                        W, H, TW, TH, int(family), int(capacity), float(cull_threshold),
+                                        _ptr(sorted_ids), _ptr(keys), _stream(dev))
     _check(code, "mlpsp_sort_tiles")
     return sorted_ids, keys
 

@@ -120,7 +120,8 @@ class TileExt:
             if family == _lib.KEY_LIST_ORDER or cand.numel() == 0:
                 order = cand
             else:
-                order, _ = ops.sort_tiles(rays_o, rays_d, rec, cand, offsets, W, H, TW, TH, family, capacity)
+                order, _ = ops.sort_tiles(rays_o, rays_d, rec, cand, offsets, W, H, TW, TH, family, capacity,
+                                          cull_threshold=thr)
             return ops.render_tilecenter_f32(rays_o, rays_d, rec, order, offsets, freq, att, *ws, W, H, TW, TH, thr,
                                              with_t=with_t)
 
@@ -162,7 +163,7 @@ class TileExt:
             order = cand
             if cand.numel() > 0:
                 order, _ = ops.sort_tiles(rays_o, rays_d, rec, cand, offsets, W, H, TW, TH, _lib.KEY_TSTAR,
-                                          self.max_tile_prims)
+                                          self.max_tile_prims, cull_threshold=thr)
             return ops.render_tilecenter_feat_f32(rays_o, rays_d, rec, order, offsets, freq, att, *ws,
                                                   feat_attr.contiguous(), beta, temp, W, H, TW, TH, thr)
 
@@ -264,7 +265,7 @@ class TileExt:
             order = x[5]
             if x[5].numel() > 0:
                 order, _ = ops.sort_tiles(x[0], x[1], rec, x[5], x[6], width, height, 8, 8, _lib.KEY_TSTAR,
-                                          self.max_tile_prims)
+                                          self.max_tile_prims, cull_threshold=threshold)
             packed = self._packed_weights(list(x[9:15]), bool(bf16))
             rgb, alpha, nonfinite = ops.render_tilecenter_mfma(x[0], x[1], rec, order, x[6], x[7], x[8], *x[9:15],
                                                                width, height, threshold, bf16=bool(bf16), packed=packed)

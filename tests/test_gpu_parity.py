@@ -111,6 +111,62 @@ def test_sorted_tile_lists_match_oracle_keys_and_order(device, oracle_mod, frame
     _assert_bits(keys, want_keys, "sort keys")
 
 
+@pytest.mark.parametrize("name,n,width,height,tile,eye", [
+    ("cfg1_5k_160x120", None, 160, 120, 8, (0.3, -0.2, -0.5)), ("cfg1_5k_160x120", 4000, 100, 76, 16, (1.0, 0.8, -1.2)),
+    ("cfg2_50k_640x480", 20000, 200, 136, 8, (-0.7, 0.4, 0.9)), ("cfg1_5k_160x120", 1500, 21, 13, 8, (0.1, 0.1, -0.2))])
+def test_conservative_tile_culling_never_drops_a_hit(device, oracle_mod, name, n, width, height, tile, eye):
+    # entries marked ~id must (1) leave the sorted order intact once un-marked, (2) be a real saving, and
+    # (3) change no bit of the image: the oracle, which tests every candidate, is the witness
+    from mlp_splatting_amd import ops
+    fr = Frame(name, n=n, width=width, height=height, tile=tile, eye=eye, target=(0, 0, 0.1))
+    sc = fr.scene
+    cand, off = fr.oracle_lists(oracle_mod)
+    rec = ops.prepare_primitives(_t(sc.positions, device), _t(sc.log_scales, device), _t(sc.quats, device))
+    ro, rd, c, o = _t(fr.rays_o, device), _t(fr.rays_d, device), _t(cand, device), _t(off, device)
+    plain, _ = ops.sort_tiles(ro, rd, rec, c, o, fr.W, fr.H, tile, tile)
+    culled, _ = ops.sort_tiles(ro, rd, rec, c, o, fr.W, fr.H, tile, tile, cull_threshold=fr.thr)
+    plain, culled = plain.cpu().numpy(), culled.cpu().numpy()
+    np.testing.assert_array_equal(np.where(culled < 0, ~culled, culled), plain)
+    frac = (culled < 0).mean()
+    assert frac > 0.15, frac
+    want = oracle_mod.render_tilecenter(*fr.base_numpy(cand, off), *fr.dims)
+    rgb, alpha, _ = ops.render_tilecenter_f32(ro, rd, rec, _t(culled, device), o, _t(sc.freq, device), _t(sc.att, device),
+                                              *[_t(w, device) for w in sc.mlp()], fr.W, fr.H, tile, tile, fr.thr)
+    _assert_bits(rgb, want["rgb"], "rgb with culled lists")
+    _assert_bits(alpha, want["alpha"], "alpha with culled lists")
+    # the witness again, entry by entry: no culled (tile, primitive) has a hitting pixel
+    ntx = (fr.W + tile - 1) // tile
+    bad = 0
+    rng = np.random.default_rng(0)
+    for t in rng.choice(off.size - 1, size=min(40, off.size - 1), replace=False):
+        tx, ty = t % ntx, t // ntx
+        pix = [y * fr.W + x for y in range(ty * tile, min((ty + 1) * tile, fr.H)) for x in range(tx * tile, min((tx + 1) * tile, fr.W))]
+        for p in ~culled[off[t]:off[t + 1]][culled[off[t]:off[t + 1]] < 0][:25]:
+            for q in pix:
+                hit, _ = oracle_mod.hit(fr.rays_o[q], fr.rays_d[q], sc.positions[p], sc.log_scales[p], sc.quats[p], fr.thr)
+                bad += int(hit)
+    assert bad == 0
+
+
+def test_culling_is_off_for_tiles_with_mixed_origins_or_degenerate_pyramids(device, oracle_mod):
+    from mlp_splatting_amd import ops
+    fr = Frame("cfg1_5k_160x120", n=1500, width=32, height=24)
+    sc = fr.scene
+    cand, off = fr.oracle_lists(oracle_mod)
+    rec = ops.prepare_primitives(_t(sc.positions, device), _t(sc.log_scales, device), _t(sc.quats, device))
+    ro = fr.rays_o.copy()
+    ro[::7, 0] += 1e-3                                    # per-pixel origins: no common apex
+    c, o = _t(cand, device), _t(off, device)
+    ids, _ = ops.sort_tiles(_t(ro, device), _t(fr.rays_d, device), rec, c, o, fr.W, fr.H, 8, 8, cull_threshold=fr.thr)
+    assert int((ids < 0).sum()) == 0
+    fr1 = Frame("cfg1_5k_160x120", n=300, width=12, height=6, tile=1)           # 1x1 tiles: no pyramid
+    c1, o1 = fr1.oracle_lists(oracle_mod)
+    rec1 = ops.prepare_primitives(_t(fr1.scene.positions, device), _t(fr1.scene.log_scales, device), _t(fr1.scene.quats, device))
+    ids1, _ = ops.sort_tiles(_t(fr1.rays_o, device), _t(fr1.rays_d, device), rec1, _t(c1, device), _t(o1, device), 12, 6, 1, 1,
+                             cull_threshold=fr1.thr)
+    assert int((ids1 < 0).sum()) == 0
+
+
 def _render_gpu(fr, device, cand, off, family=1, with_t=False):
     from mlp_splatting_amd import ops
     sc = fr.scene
