@@ -176,6 +176,31 @@ int mlpsp_render_tilecenter_mfma(const float* rays_o_dev, const float* rays_d_de
                                  int width, int height, float threshold, float* out_rgb_dev, float* out_alpha_dev,
                                  int32_t* status_dev, int64_t* counters_dev, mlpsp_stream_t stream);
 
+/* Matrix-core render with the gated feature channel (feat_slots 1, 4 or 5; channels <= 512).  No
+ * counterpart in the reference, whose tensor-core kernel is RGB only; the feature semantics are those of
+ * np_tile_kernels.cu:6036-6075 (feat += w * (base + sum_s g_s attr_s)) with this kernel's weights w.
+ * The render kernel emits, per tile, the primitives that hit and their per-pixel coefficients w*g_s
+ * rounded to fp16 into the workspace; a grouped fp16 GEMM (f32 accumulate) on the matrix cores then
+ * forms the image from the fp16 attribute copy, whatever use_bf16 selects for the MLP.  out_feat_dev [B,C] is fully written.
+ *
+ * mlpsp_pack_mfma_feat: feat_attr f32 [N,S,C] ([N,C] for S = 1) -> operand copy (once per scene);
+ * status_dev[0] = 1 if a value is not finite in fp16 (then use the f32 feature kernel).
+ * num_pairs = length of order_dev = tile_offsets[num_tiles].  feat_slots = 0 renders RGB only and
+ * ignores the feature and workspace arguments.  MLPSP_E_SCRATCH if the workspace is too small or not
+ * 256-byte aligned. */
+size_t mlpsp_mfma_feat_pack_bytes(int num_primitives, int feat_slots, int feat_channels);
+int mlpsp_pack_mfma_feat(const float* feat_attr_dev, int num_primitives, int feat_slots, int feat_channels,
+                         void* packed_feat_dev, int32_t* status_dev, mlpsp_stream_t stream);
+size_t mlpsp_mfma_feat_workspace_bytes(int64_t num_pairs, int width, int height, int feat_slots);
+int mlpsp_render_tilecenter_mfma_feat(const float* rays_o_dev, const float* rays_d_dev, const void* prim_records_dev,
+                                      const int32_t* order_dev, const int32_t* tile_offsets_dev, int64_t num_pairs,
+                                      const float* freq_dev, const float* att_dev, const void* packed_dev,
+                                      int num_primitives, int use_bf16, const void* packed_feat_dev, int feat_slots,
+                                      int feat_channels, float gating_beta, float gating_temp, int width, int height,
+                                      float threshold, void* workspace_dev, size_t workspace_bytes,
+                                      float* out_rgb_dev, float* out_alpha_dev, float* out_feat_dev,
+                                      int32_t* status_dev, int64_t* counters_dev, mlpsp_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -175,7 +175,7 @@ __device__ __forceinline__ float fast_softplus(float x) {
   y = (x > 20.f) ? x : y;
   return y;
 }
-__device__ __forceinline__ void fast_blend_step(PixelAcc& a, float o0, float o1, float o2, float o3, float decay) {
+__device__ __forceinline__ float fast_blend_step(PixelAcc& a, float o0, float o1, float o2, float o3, float decay) {
   const float sigma = fast_softplus(o3) * decay;
   const float alpha = 1.f - fast_exp(-sigma);
   const float w = a.trans * alpha;
@@ -183,15 +183,40 @@ __device__ __forceinline__ void fast_blend_step(PixelAcc& a, float o0, float o1,
   a.cg = fmaf(w, fast_sigmoid(o1), a.cg);
   a.cb = fmaf(w, fast_sigmoid(o2), a.cb);
   a.trans = a.trans * (1.f - alpha);
+  return w;
+}
+// tetrahedral gates (np_tile_kernels.cu:97-124) with the native exp/rcp
+__device__ __forceinline__ void fast_tetra_gates(float qlx, float qly, float qlz, float lgx, float lgy, float lgz,
+                                                 float beta, float temp, float g[4]) {
+  const float ux = fminf(1.f, fmaxf(-1.f, qlx * __builtin_amdgcn_rcpf(beta * fast_exp(lgx) + 1e-6f)));
+  const float uy = fminf(1.f, fmaxf(-1.f, qly * __builtin_amdgcn_rcpf(beta * fast_exp(lgy) + 1e-6f)));
+  const float uz = fminf(1.f, fmaxf(-1.f, qlz * __builtin_amdgcn_rcpf(beta * fast_exp(lgz) + 1e-6f)));
+  const float l0 = temp * ((ux + uy) + uz), l1 = temp * ((ux - uy) - uz);
+  const float l2 = temp * ((-ux + uy) - uz), l3 = temp * ((-ux - uy) + uz);
+  const float lm = fmaxf(fmaxf(l0, l1), fmaxf(l2, l3));
+  const float e0 = fast_exp(l0 - lm), e1 = fast_exp(l1 - lm), e2 = fast_exp(l2 - lm), e3 = fast_exp(l3 - lm);
+  const float inv = __builtin_amdgcn_rcpf(fmaxf(((e0 + e1) + e2) + e3, 1e-8f));
+  g[0] = e0 * inv;
+  g[1] = e1 * inv;
+  g[2] = e2 * inv;
+  g[3] = e3 * inv;
 }
 
-template <typename T>
+// SP = 0: RGB only.  SP = 4 or 8: the kernel also emits, per tile, the compact list of primitives that
+// hit at least one pixel (hit_ids[start + m]) and per (such primitive, pixel) the SP compositing
+// coefficients of the gated feature channel, rounded to fp16 (they lie in [0, 1]; fp16 keeps 11
+// significant bits there, bf16 only 8): (w g0, w g1, w g2, w g3) for 4 slots,
+// (w, 0, 0, 0) for one slot, (w, w g0, .., w g3, 0, 0, 0) for 5 slots (np_tile_kernels.cu:6036-6075:
+// feat += w * (base + sum_s g_s attr_s)).  The feature image is then one grouped GEMM over those lists
+// (feat_gemm_kernel below).
+template <typename T, int SP>
 __global__ __launch_bounds__(64) void render_tilecenter_mfma_kernel(
     const float* __restrict__ rays_o, const float* __restrict__ rays_d, const PrimRecord* __restrict__ prims,
     const int32_t* __restrict__ order, const int32_t* __restrict__ offsets, const float* __restrict__ freq,
     const float* __restrict__ att, const unsigned char* __restrict__ packed, int N, int W, int H, int ntx,
     int per_xcd, int num_tiles, float thr, float* __restrict__ out_rgb, float* __restrict__ out_alpha,
-    int32_t* __restrict__ status, unsigned long long* __restrict__ counters) {
+    int32_t* __restrict__ status, unsigned long long* __restrict__ counters, int slots, float beta, float temp,
+    int32_t* __restrict__ hit_ids, int32_t* __restrict__ tile_hits, unsigned* __restrict__ coef) {
   // XCD-aware work assignment: XCD k (blockIdx.x % 8) walks tiles [k*per_xcd, (k+1)*per_xcd) in
   // row-major order, so neighbouring tiles -- which share most primitives -- run together on one L2.
   const int tile = (blockIdx.x % kNumXcd) * per_xcd + blockIdx.x / kNumXcd;
@@ -218,6 +243,7 @@ __global__ __launch_bounds__(64) void render_tilecenter_mfma_kernel(
 
   const int start = offsets[tile], end = offsets[tile + 1];
   PixelAcc acc = {0.f, 0.f, 0.f, 1.f, 0.f, 0.f};
+  int n_emit = 0;
 
   for (int i = start; i < end; ++i) {
     const int p = __builtin_amdgcn_readfirstlane(order[i]);
@@ -324,10 +350,26 @@ __global__ __launch_bounds__(64) void render_tilecenter_mfma_kernel(
         const float from_partner = __shfl_xor(o_blk[1][k], 32);
         o[k] = (g ? from_partner : o_blk[0][k]) + b3v[k];
       }
+      float w = 0.f;
       if (hit) {
         bad |= !(__builtin_fabsf(o[0]) <= 3.4028235e38f) || !(__builtin_fabsf(o[1]) <= 3.4028235e38f) ||
                !(__builtin_fabsf(o[2]) <= 3.4028235e38f) || !(__builtin_fabsf(o[3]) <= 3.4028235e38f);
-        fast_blend_step(acc, o[0], o[1], o[2], o[3], h.decay);
+        w = fast_blend_step(acc, o[0], o[1], o[2], o[3], h.decay);
+      }
+      if constexpr (SP > 0) {
+        float gt[4] = {0.f, 0.f, 0.f, 0.f};
+        if (hit && slots > 1) fast_tetra_gates(h.qlx, h.qly, h.qlz, P.lgx, P.lgy, P.lgz, beta, temp, gt);
+        const size_t row = (size_t)(start + n_emit) * 64 + l;
+        if constexpr (SP == 4) {
+          const unsigned c01 = (slots > 1) ? Ops<_Float16>::pack2(w * gt[0], w * gt[1]) : Ops<_Float16>::pack2(w, 0.f);
+          const unsigned c23 = Ops<_Float16>::pack2(w * gt[2], w * gt[3]);
+          *reinterpret_cast<uint2*>(coef + row * 2) = make_uint2(c01, c23);
+        } else {
+          const u32x4 c = {Ops<_Float16>::pack2(w, w * gt[0]), Ops<_Float16>::pack2(w * gt[1], w * gt[2]), Ops<_Float16>::pack2(w * gt[3], 0.f), 0u};
+          *reinterpret_cast<u32x4*>(coef + row * 4) = c;
+        }
+        if (l == 0) hit_ids[start + n_emit] = p;
+        ++n_emit;
       }
     }
     if (__ballot(valid && (acc.trans >= kTransmittanceFloor)) == 0ull) break;
@@ -339,11 +381,137 @@ __global__ __launch_bounds__(64) void render_tilecenter_mfma_kernel(
     out_rgb[pix * 3 + 2] = acc.cb;
     out_alpha[pix] = 1.f - acc.trans;
   }
+  if constexpr (SP > 0) {
+    if (l == 0) tile_hits[tile] = n_emit;
+  }
   if (__ballot(bad) != 0ull && l == 0) atomicExch(status, 1);
   if (counters && l == 0) {
     atomicAdd(counters + 1, (unsigned long long)n_proc);
     atomicAdd(counters + 2, (unsigned long long)n_proc_hit);
     atomicAdd(counters + 3, (unsigned long long)n_hits);
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// feature channel: pack + grouped GEMM
+// ---------------------------------------------------------------------------------------------
+
+// feat_attr f32 [N, S, C] (S = 1: [N, C])  ->  fp16 [N, C, SP] (the reference's inference export stores
+// these attributes as fp16 too, scannet/cumodel.py:317-381), the SP slot values of one (primitive, channel)
+// contiguous (slot order as the coefficient records above, zero padded).  flag[0] = 1 if a rounded value
+// is not finite.
+template <int SP>
+__global__ __launch_bounds__(256) void pack_feat_kernel(const float* __restrict__ attr, int N, int S, int C,
+                                                        unsigned* __restrict__ out, int32_t* __restrict__ flag) {
+  const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= (size_t)N * C) return;
+  const size_t p = idx / C;
+  const int c = (int)(idx % C);
+  float v[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  bool bad = false;
+  for (int s = 0; s < S; ++s) {
+    v[s] = attr[(p * S + s) * C + c];
+    bad |= !(__builtin_fabsf(Ops<_Float16>::round_trip(v[s])) <= Ops<_Float16>::kMax);
+  }
+#pragma unroll
+  for (int d = 0; d < SP / 2; ++d) out[idx * (SP / 2) + d] = Ops<_Float16>::pack2(v[2 * d], v[2 * d + 1]);
+  if (bad) atomicExch(flag, 1);
+}
+
+// out_feat[pixel, c] = sum over the tile's hit records e and slots s of coef[e, pixel, s] * attr[id_e, c, s]:
+// per tile a [64 pixels] x [K = SP * hits] x [C] product on v_mfma_f32_32x32x16.  One 256-thread block per
+// tile; wavefront v owns channels [128 v, 128 v + 128) as 2 pixel blocks x 4 channel blocks of f32
+// accumulators.  Pixels are the M operand and channels the N operand, so that an accumulator register
+// holds 32 consecutive channels of one pixel across lanes: every store is a full 128-byte line.
+// K-slot j of lane group g is (record 16/SP * step + g * 8/SP + j / SP, slot j % SP): both operands are
+// plain 8- or 16-byte loads, coalesced over 32 pixels / 32 channels.
+template <int SP>
+__global__ __launch_bounds__(256) void feat_gemm_kernel(const unsigned* __restrict__ attr, const int32_t* __restrict__ hit_ids,
+                                                        const unsigned* __restrict__ coef,
+                                                        const int32_t* __restrict__ offsets,
+                                                        const int32_t* __restrict__ tile_hits, int C, int W, int H,
+                                                        int ntx, int per_xcd, int num_tiles,
+                                                        float* __restrict__ out_feat) {
+  const int tile = (blockIdx.x % kNumXcd) * per_xcd + blockIdx.x / kNumXcd;
+  if (tile >= num_tiles) return;
+  const int wave = threadIdx.x >> 6, l = threadIdx.x & 63, g = l >> 5, m = l & 31;
+  const int c0 = ((int)blockIdx.y * 4 + wave) * 128;
+  if (c0 >= C) return;
+  const int ncb = min(4, (C - c0 + 31) / 32);
+  constexpr int EPL = 8 / SP;         // records per lane group and K-step
+  constexpr int DW = SP / 2;          // dwords per (record, pixel) and per (primitive, channel)
+  const int start = offsets[tile], hits = tile_hits[tile];
+  f32x16 acc[2][4];
+#pragma unroll
+  for (int pb = 0; pb < 2; ++pb)
+#pragma unroll
+    for (int cb = 0; cb < 4; ++cb)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[pb][cb][r] = 0.f;
+  int ch[4];
+#pragma unroll
+  for (int cb = 0; cb < 4; ++cb) ch[cb] = min(c0 + 32 * cb + m, C - 1);
+
+  for (int e = 0; e < hits; e += 2 * EPL) {
+    u32x4 apix[2] = {{0u, 0u, 0u, 0u}, {0u, 0u, 0u, 0u}}, bch[4];
+#pragma unroll
+    for (int cb = 0; cb < 4; ++cb) bch[cb] = u32x4{0u, 0u, 0u, 0u};
+#pragma unroll
+    for (int u = 0; u < EPL; ++u) {
+      const int ent = e + g * EPL + u;
+      if (ent < hits) {
+        const size_t prim = (size_t)hit_ids[start + ent];
+        const unsigned* __restrict__ crow = coef + ((size_t)(start + ent) * 64 + m) * DW;
+        const unsigned* __restrict__ arow = attr + prim * C * DW;
+        if constexpr (SP == 4) {
+#pragma unroll
+          for (int pb = 0; pb < 2; ++pb) {
+            const uint2 v = *reinterpret_cast<const uint2*>(crow + pb * 32 * DW);
+            apix[pb][2 * u] = v.x;
+            apix[pb][2 * u + 1] = v.y;
+          }
+#pragma unroll
+          for (int cb = 0; cb < 4; ++cb) {
+            if (cb < ncb) {
+              const uint2 v = *reinterpret_cast<const uint2*>(arow + (size_t)ch[cb] * DW);
+              bch[cb][2 * u] = v.x;
+              bch[cb][2 * u + 1] = v.y;
+            }
+          }
+        } else {
+#pragma unroll
+          for (int pb = 0; pb < 2; ++pb) apix[pb] = *reinterpret_cast<const u32x4*>(crow + pb * 32 * DW);
+#pragma unroll
+          for (int cb = 0; cb < 4; ++cb)
+            if (cb < ncb) bch[cb] = *reinterpret_cast<const u32x4*>(arow + (size_t)ch[cb] * DW);
+        }
+      }
+    }
+#pragma unroll
+    for (int cb = 0; cb < 4; ++cb) {
+      if (cb < ncb) {
+#pragma unroll
+        for (int pb = 0; pb < 2; ++pb) acc[pb][cb] = Ops<_Float16>::mfma(apix[pb], bch[cb], acc[pb][cb]);
+      }
+    }
+  }
+
+  const int tx = tile % ntx, ty = tile / ntx;
+#pragma unroll
+  for (int pb = 0; pb < 2; ++pb) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int q = 32 * pb + d_row(r, g);
+      const int x = tx * 8 + (q & 7), y = ty * 8 + (q >> 3);
+      if (x < W && y < H) {
+        float* __restrict__ dst = out_feat + (size_t)(y * W + x) * C;
+#pragma unroll
+        for (int cb = 0; cb < 4; ++cb) {
+          const int c = c0 + 32 * cb + m;
+          if (cb < ncb && c < C) dst[c] = acc[pb][cb][r];
+        }
+      }
+    }
   }
 }
 
@@ -373,6 +541,125 @@ MLPSP_API int mlpsp_pack_mfma_weights(const float* W1, const float* b1, const fl
   return MLPSP_OK;
 }
 
+namespace {
+constexpr size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
+inline int feat_pad(int slots) { return slots == 5 ? 8 : 4; }
+
+template <typename E, int SP>
+void launch_mfma(dim3 grid, hipStream_t s, const float* rays_o, const float* rays_d, const void* prims, const int32_t* order,
+                 const int32_t* offsets, const float* freq, const float* att, const void* packed, int N, int W, int H,
+                 int ntx, int per_xcd, int T, float thr, float* rgb, float* alpha, int32_t* status,
+                 unsigned long long* ctr, int slots, float beta, float temp, int32_t* hit_ids, int32_t* tile_hits,
+                 unsigned* coef) {
+  hipLaunchKernelGGL((render_tilecenter_mfma_kernel<E, SP>), grid, dim3(64), 0, s, rays_o, rays_d,
+                     (const PrimRecord*)prims, order, offsets, freq, att, (const unsigned char*)packed, N, W, H, ntx,
+                     per_xcd, T, thr, rgb, alpha, status, ctr, slots, beta, temp, hit_ids, tile_hits, coef);
+}
+}  // namespace
+
+MLPSP_API size_t mlpsp_mfma_feat_pack_bytes(int num_primitives, int feat_slots, int feat_channels) {
+  if (num_primitives < 0 || feat_channels <= 0 || !(feat_slots == 1 || feat_slots == 4 || feat_slots == 5)) return 0;
+  return align256((size_t)(num_primitives > 0 ? num_primitives : 1) * feat_channels * feat_pad(feat_slots) * 2);
+}
+
+MLPSP_API int mlpsp_pack_mfma_feat(const float* feat_attr_dev, int num_primitives, int feat_slots, int feat_channels,
+                                   void* packed_feat_dev, int32_t* status_dev, mlpsp_stream_t stream) {
+  if (num_primitives < 0 || feat_channels <= 0 || feat_channels > 512 ||
+      !(feat_slots == 1 || feat_slots == 4 || feat_slots == 5) || !status_dev)
+    return MLPSP_E_ARGUMENT;
+  hipStream_t s = (hipStream_t)stream;
+  MLPSP_HIP_TRY(hipMemsetAsync(status_dev, 0, sizeof(int32_t), s));
+  if (num_primitives == 0) return MLPSP_OK;
+  if (!feat_attr_dev || !packed_feat_dev || reinterpret_cast<uintptr_t>(packed_feat_dev) % 16 != 0) return MLPSP_E_ARGUMENT;
+  const size_t total = (size_t)num_primitives * feat_channels;
+  const dim3 grid((unsigned)((total + 255) / 256)), block(256);
+  unsigned* out = (unsigned*)packed_feat_dev;
+#define MLPSP_PACK_FEAT(SP) \
+  hipLaunchKernelGGL((pack_feat_kernel<SP>), grid, block, 0, s, feat_attr_dev, num_primitives, feat_slots, feat_channels, out, status_dev)
+  if (feat_pad(feat_slots) == 4) MLPSP_PACK_FEAT(4);
+  else MLPSP_PACK_FEAT(8);
+#undef MLPSP_PACK_FEAT
+  MLPSP_LAUNCH_CHECK();
+  return MLPSP_OK;
+}
+
+MLPSP_API size_t mlpsp_mfma_feat_workspace_bytes(int64_t num_pairs, int width, int height, int feat_slots) {
+  const int64_t T = checked_num_tiles(width, height, 8, 8);
+  if (T <= 0 || num_pairs < 0 || !(feat_slots == 1 || feat_slots == 4 || feat_slots == 5)) return 0;
+  return align256((size_t)num_pairs * 4) + align256((size_t)T * 4) +
+         align256((size_t)num_pairs * 64 * feat_pad(feat_slots) * 2) + 256;
+}
+
+MLPSP_API int mlpsp_render_tilecenter_mfma_feat(const float* rays_o_dev, const float* rays_d_dev,
+                                                const void* prim_records_dev, const int32_t* order_dev,
+                                                const int32_t* tile_offsets_dev, int64_t num_pairs,
+                                                const float* freq_dev, const float* att_dev, const void* packed_dev,
+                                                int num_primitives, int use_bf16, const void* packed_feat_dev,
+                                                int feat_slots, int feat_channels, float gating_beta,
+                                                float gating_temp, int width, int height, float threshold,
+                                                void* workspace_dev, size_t workspace_bytes, float* out_rgb_dev,
+                                                float* out_alpha_dev, float* out_feat_dev, int32_t* status_dev,
+                                                int64_t* counters_dev, mlpsp_stream_t stream) {
+  const int64_t T = checked_num_tiles(width, height, 8, 8);
+  if (T <= 0 || T > 2147483647LL - 8 || num_primitives < 0 || num_pairs < 0 || num_pairs > 2147483647LL)
+    return MLPSP_E_ARGUMENT;
+  if (!rays_o_dev || !rays_d_dev || !tile_offsets_dev || !freq_dev || !att_dev || !out_rgb_dev || !out_alpha_dev ||
+      !status_dev)
+    return MLPSP_E_ARGUMENT;
+  if (num_primitives > 0 && !packed_dev) return MLPSP_E_ARGUMENT;
+  int32_t *hit_ids = nullptr, *tile_hits = nullptr;
+  unsigned* coef = nullptr;
+  if (feat_slots != 0) {
+    if (!(feat_slots == 1 || feat_slots == 4 || feat_slots == 5) || feat_channels <= 0 || feat_channels > 512 ||
+        !out_feat_dev || (num_primitives > 0 && !packed_feat_dev))
+      return MLPSP_E_ARGUMENT;
+    if (!workspace_dev || reinterpret_cast<uintptr_t>(workspace_dev) % 256 != 0 ||
+        workspace_bytes < mlpsp_mfma_feat_workspace_bytes(num_pairs, width, height, feat_slots))
+      return MLPSP_E_SCRATCH;
+    unsigned char* ws = (unsigned char*)workspace_dev;
+    hit_ids = (int32_t*)ws;
+    ws += align256((size_t)num_pairs * 4);
+    tile_hits = (int32_t*)ws;
+    ws += align256((size_t)T * 4);
+    coef = (unsigned*)ws;
+  }
+  MLPSP_HIP_TRY(hipMemsetAsync(status_dev, 0, 16 * sizeof(int32_t), (hipStream_t)stream));
+  const int per_xcd = (int)((T + kNumXcd - 1) / kNumXcd);
+  const dim3 grid((unsigned)(per_xcd * kNumXcd));
+  hipStream_t s = (hipStream_t)stream;
+  auto* ctr = reinterpret_cast<unsigned long long*>(counters_dev);
+  const int ntx = ceil_div(width, 8);
+  const int sp = feat_slots ? feat_pad(feat_slots) : 0;
+#define MLPSP_MFMA_GO(TT, SP)                                                                                     \
+  launch_mfma<TT, SP>(grid, s, rays_o_dev, rays_d_dev, prim_records_dev, order_dev, tile_offsets_dev, freq_dev,   \
+                      att_dev, packed_dev, num_primitives, width, height, ntx, per_xcd, (int)T, threshold,        \
+                      out_rgb_dev, out_alpha_dev, status_dev, ctr, feat_slots, gating_beta, gating_temp, hit_ids, \
+                      tile_hits, coef)
+#define MLPSP_MFMA_SP(TT)                 \
+  do {                                    \
+    if (sp == 0) MLPSP_MFMA_GO(TT, 0);    \
+    else if (sp == 4) MLPSP_MFMA_GO(TT, 4); \
+    else MLPSP_MFMA_GO(TT, 8);            \
+  } while (0)
+  if (use_bf16) MLPSP_MFMA_SP(__bf16);
+  else MLPSP_MFMA_SP(_Float16);
+#undef MLPSP_MFMA_SP
+#undef MLPSP_MFMA_GO
+  MLPSP_LAUNCH_CHECK();
+  if (sp != 0) {
+    const dim3 ggrid((unsigned)(per_xcd * kNumXcd), (unsigned)ceil_div(feat_channels, 512)), gblock(256);
+#define MLPSP_FEAT_GEMM(SP)                                                                                  \
+  hipLaunchKernelGGL((feat_gemm_kernel<SP>), ggrid, gblock, 0, s, (const unsigned*)packed_feat_dev, hit_ids, \
+                     coef, tile_offsets_dev, tile_hits, feat_channels, width, height, ntx, per_xcd, (int)T,  \
+                     out_feat_dev)
+    if (sp == 4) MLPSP_FEAT_GEMM(4);
+    else MLPSP_FEAT_GEMM(8);
+#undef MLPSP_FEAT_GEMM
+    MLPSP_LAUNCH_CHECK();
+  }
+  return MLPSP_OK;
+}
+
 MLPSP_API int mlpsp_render_tilecenter_mfma(const float* rays_o_dev, const float* rays_d_dev,
                                            const void* prim_records_dev, const int32_t* order_dev,
                                            const int32_t* tile_offsets_dev, const float* freq_dev,
@@ -380,28 +667,8 @@ MLPSP_API int mlpsp_render_tilecenter_mfma(const float* rays_o_dev, const float*
                                            int use_bf16, int width, int height, float threshold, float* out_rgb_dev,
                                            float* out_alpha_dev, int32_t* status_dev, int64_t* counters_dev,
                                            mlpsp_stream_t stream) {
-  const int64_t T = checked_num_tiles(width, height, 8, 8);
-  if (T <= 0 || T > 2147483647LL - 8 || num_primitives < 0) return MLPSP_E_ARGUMENT;
-  if (!rays_o_dev || !rays_d_dev || !tile_offsets_dev || !freq_dev || !att_dev || !out_rgb_dev || !out_alpha_dev ||
-      !status_dev)
-    return MLPSP_E_ARGUMENT;
-  if (num_primitives > 0 && !packed_dev) return MLPSP_E_ARGUMENT;
-  MLPSP_HIP_TRY(hipMemsetAsync(status_dev, 0, 16 * sizeof(int32_t), (hipStream_t)stream));
-  const int per_xcd = (int)((T + kNumXcd - 1) / kNumXcd);
-  const dim3 grid((unsigned)(per_xcd * kNumXcd)), block(64);
-  hipStream_t s = (hipStream_t)stream;
-  auto* ctr = reinterpret_cast<unsigned long long*>(counters_dev);
-  const int ntx = ceil_div(width, 8);
-  if (use_bf16)
-    hipLaunchKernelGGL(render_tilecenter_mfma_kernel<__bf16>, grid, block, 0, s, rays_o_dev, rays_d_dev,
-                       (const PrimRecord*)prim_records_dev, order_dev, tile_offsets_dev, freq_dev, att_dev,
-                       (const unsigned char*)packed_dev, num_primitives, width, height, ntx, per_xcd, (int)T, threshold,
-                       out_rgb_dev, out_alpha_dev, status_dev, ctr);
-  else
-    hipLaunchKernelGGL(render_tilecenter_mfma_kernel<_Float16>, grid, block, 0, s, rays_o_dev, rays_d_dev,
-                       (const PrimRecord*)prim_records_dev, order_dev, tile_offsets_dev, freq_dev, att_dev,
-                       (const unsigned char*)packed_dev, num_primitives, width, height, ntx, per_xcd, (int)T, threshold,
-                       out_rgb_dev, out_alpha_dev, status_dev, ctr);
-  MLPSP_LAUNCH_CHECK();
-  return MLPSP_OK;
+  return mlpsp_render_tilecenter_mfma_feat(rays_o_dev, rays_d_dev, prim_records_dev, order_dev, tile_offsets_dev, 0,
+                                           freq_dev, att_dev, packed_dev, num_primitives, use_bf16, nullptr, 0, 0, 0.f,
+                                           0.f, width, height, threshold, nullptr, 0, out_rgb_dev, out_alpha_dev,
+                                           nullptr, status_dev, counters_dev, stream);
 }

@@ -379,12 +379,12 @@ class NeuralPrimitiveSceneTileCUDA(nn.Module):
             base = self._base_args(ray_o, ray_d, culled_prim_indices, tile_offsets, device)
             bg = self._background(bg_color, ray_o)
             dims = (int(W), int(H), ts, ts, float(score_threshold))
+            precision = str(getattr(self, "render_precision", "f32")).lower()
+            if precision not in {"f32", "bf16", "fp16"}:
+                raise ValueError(f"Unsupported render_precision {precision!r}; use 'f32', 'bf16' or 'fp16'.")
+            matrix_cores = (use_tilecenter and precision != "f32" and ts == 8 and int(self.hidden_dim) == 32
+                            and int(self.pe_frequencies) == 6)
             if (not return_feature) or (self.feat_attr is None):
-                precision = str(getattr(self, "render_precision", "f32")).lower()
-                if precision not in {"f32", "bf16", "fp16"}:
-                    raise ValueError(f"Unsupported render_precision {precision!r}; use 'f32', 'bf16' or 'fp16'.")
-                matrix_cores = (use_tilecenter and precision != "f32" and ts == 8 and int(self.hidden_dim) == 32
-                                and int(self.pe_frequencies) == 6)
                 if matrix_cores:
                     rgb, alpha = ext.render_tiles_rgb_wmma(list(base), int(W), int(H), float(score_threshold),
                                                            precision == "bf16")
@@ -398,7 +398,10 @@ class NeuralPrimitiveSceneTileCUDA(nn.Module):
                 return rgb
             feat_args = (self.feat_attr.detach().contiguous(), float(self.feature_gating_beta),
                          float(self.feature_gating_temp))
-            if use_tilecenter:
+            if matrix_cores:
+                rgb, alpha, feat = ext.render_tiles_rgb_wmma_with_feat(list(base), *feat_args, int(W), int(H),
+                                                                       float(score_threshold), precision == "bf16")
+            elif use_tilecenter:
                 rgb, alpha, feat = ext.render_tiles_forward_tilecenter_with_feat(*base, *feat_args, *dims)
             else:
                 rgb, alpha, feat = ext.render_tiles_forward_per_pixel_with_feat(*base, *feat_args, *dims)

@@ -245,3 +245,50 @@ def render_tilecenter_mfma(rays_o, rays_d, records, order, tile_offsets, freq, a
         _stream(dev))
     _check(code, "mlpsp_render_tilecenter_mfma")
     return rgb, alpha, (bool(flag[0].item()) if check else flag)
+
+
+def pack_mfma_feat(feat_attr):
+    """fp16 matrix-core operand copy of the feature attributes -> (packed uint8 tensor, nonfinite flag)."""
+    dev = feat_attr.device
+    slots, ch = _feat_shape(feat_attr)
+    lib = _lib.load()
+    n = feat_attr.shape[0]
+    packed = torch.empty(lib.mlpsp_mfma_feat_pack_bytes(n, slots, ch), dtype=torch.uint8, device=dev)
+    flag = torch.empty(1, dtype=torch.int32, device=dev)
+    _check(lib.mlpsp_pack_mfma_feat(_ptr(feat_attr), n, slots, ch, _ptr(packed), _ptr(flag),
+                                    _stream(dev)), "mlpsp_pack_mfma_feat")
+    return packed, bool(flag.item())
+
+
+def render_tilecenter_mfma_feat(rays_o, rays_d, records, order, tile_offsets, freq, att, W1, b1, W2, b2, W3, b3,
+                                feat_attr, beta, temp, W, H, threshold, bf16=True, packed=None, packed_feat=None,
+                                check=True):
+    """Matrix-core tile-centre forward with the gated feature channel -> (rgb, alpha, feat, nonfinite).
+    ``packed_feat`` is the result of :func:`pack_mfma_feat` for ``feat_attr`` (built here when omitted;
+    non-finite rounded attributes raise)."""
+    dev = rays_o.device
+    if freq.numel() != 6:
+        raise RuntimeError("the matrix-core path supports 6 frequencies only")
+    slots, ch = _feat_shape(feat_attr)
+    if packed is None:
+        packed = pack_mfma_weights(W1, b1, W2, b2, W3, b3, bf16)
+    if packed_feat is None:
+        packed_feat, bad = pack_mfma_feat(feat_attr)
+        if bad:
+            raise RuntimeError("feature attributes are not finite in fp16")
+    lib = _lib.load()
+    B = W * H
+    pairs = int(order.numel())
+    ws_bytes = lib.mlpsp_mfma_feat_workspace_bytes(pairs, W, H, slots)
+    workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    rgb = torch.empty(B, 3, dtype=torch.float32, device=dev)
+    alpha = torch.empty(B, 1, dtype=torch.float32, device=dev)
+    feat = torch.empty(B, ch, dtype=torch.float32, device=dev)
+    flag = torch.empty(16, dtype=torch.int32, device=dev)
+    code = lib.mlpsp_render_tilecenter_mfma_feat(
+        _ptr(rays_o), _ptr(rays_d), _ptr(records), _ptr(order), _ptr(tile_offsets), pairs, _ptr(freq), _ptr(att),
+        _ptr(packed), W1.shape[0], int(bool(bf16)), _ptr(packed_feat), slots, ch, float(beta), float(temp), W, H,
+        float(threshold), _ptr(workspace), ws_bytes, _ptr(rgb), _ptr(alpha), _ptr(feat), _ptr(flag), None,
+        _stream(dev))
+    _check(code, "mlpsp_render_tilecenter_mfma_feat")
+    return rgb, alpha, feat, (bool(flag[0].item()) if check else flag)

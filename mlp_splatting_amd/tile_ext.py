@@ -49,6 +49,8 @@ class TileExt:
         self._mfma_fallbacks = 0
         self._pack_key = None
         self._pack = None
+        self._feat_pack_key = None
+        self._feat_pack = None
 
     def __getattr__(self, name):
         if name in _BACKWARD_ONLY:
@@ -238,8 +240,31 @@ class TileExt:
                 self._pack_key = key
             return self._pack
 
+    def _packed_feat(self, feat_attr):
+        """fp16 operand copy of the feature attributes, cached like the weights -> (packed, nonfinite)."""
+        key = (feat_attr.data_ptr(), feat_attr._version, tuple(feat_attr.shape), str(feat_attr.device))
+        with self._lock:
+            if self._feat_pack_key != key:
+                self._feat_pack = ops.pack_mfma_feat(feat_attr)
+                self._feat_pack_key = key
+            return self._feat_pack
+
     def render_tiles_rgb_wmma(self, x, width, height, threshold, bf16):
         """[rgb, alpha] with the 72->32->32->4 MLP on the matrix cores, f32 everywhere else."""
+        return self._rgb_wmma(x, None, width, height, threshold, bf16, "render_tiles_rgb_wmma")
+
+    def render_tiles_rgb_wmma_with_feat(self, x, feat_attr, beta, temp, width, height, threshold, bf16):
+        """[rgb, alpha, feat]: the matrix-core render with the gated feature channel composited by the
+        same weights (feature semantics of np_tile_kernels.cu:6036-6075; the reference's tensor-core
+        kernel itself is RGB only)."""
+        _chk(feat_attr.is_cuda and feat_attr.dtype == torch.float32 and feat_attr.dim() in (2, 3),
+             "feat_attr must be a CUDA float32 tensor with 2 or 3 dimensions")
+        _chk(feat_attr.shape[0] == x[2].shape[0], "feat_attr first dimension must match primitive count")
+        ops._feat_shape(feat_attr)
+        return self._rgb_wmma(x, (feat_attr.contiguous(), float(beta), float(temp)), width, height, threshold, bf16,
+                              "render_tiles_rgb_wmma_with_feat")
+
+    def _rgb_wmma(self, x, feat, width, height, threshold, bf16, name):
         _chk(len(x) == 15, "WMMA requires the 15 scene tensors")
         width, height, threshold = int(width), int(height), float(threshold)
         _chk(width > 0 and height > 0 and 0.0 < threshold < 1.0)
@@ -256,7 +281,6 @@ class TileExt:
         _chk(tuple(x[9].shape) == (n, 32, 72) and tuple(x[10].shape) == (n, 32))
         _chk(tuple(x[11].shape) == (n, 32, 32) and x[12].shape == x[10].shape)
         _chk(tuple(x[13].shape) == (n, 4, 32) and tuple(x[14].shape) == (n, 4))
-        name = "render_tiles_rgb_wmma"
         with torch.cuda.device(x[0].device):
             ops.validate_tile_lists(x[5], x[6], ops.num_tiles(width, height, 8, 8), self.max_tile_prims, n, name)
             with self._lock:
@@ -267,8 +291,26 @@ class TileExt:
                 order, _ = ops.sort_tiles(x[0], x[1], rec, x[5], x[6], width, height, 8, 8, _lib.KEY_TSTAR,
                                           self.max_tile_prims, cull_threshold=threshold)
             packed = self._packed_weights(list(x[9:15]), bool(bf16))
-            rgb, alpha, nonfinite = ops.render_tilecenter_mfma(x[0], x[1], rec, order, x[6], x[7], x[8], *x[9:15],
-                                                               width, height, threshold, bf16=bool(bf16), packed=packed)
+            packed_feat = None
+            if feat is not None:
+                packed_feat, bad_attr = self._packed_feat(feat[0])
+                if bad_attr:                      # e.g. |attr| beyond the fp16 range: exact path instead
+                    warnings.warn("feature attributes overflow fp16: "
+                                  "rendering this frame with scalar FP32 instead")
+                    with self._lock:
+                        self._mfma_fallbacks += 1
+                    return list(ops.render_tilecenter_feat_f32(x[0], x[1], rec, order, x[6], x[7], x[8], *x[9:15],
+                                                               feat[0], feat[1], feat[2], width, height, 8, 8, threshold))
+            if feat is None:
+                rgb, alpha, nonfinite = ops.render_tilecenter_mfma(x[0], x[1], rec, order, x[6], x[7], x[8], *x[9:15],
+                                                                   width, height, threshold, bf16=bool(bf16),
+                                                                   packed=packed)
+                out = [rgb, alpha]
+            else:
+                rgb, alpha, fmap, nonfinite = ops.render_tilecenter_mfma_feat(
+                    x[0], x[1], rec, order, x[6], x[7], x[8], *x[9:15], feat[0], feat[1], feat[2], width, height,
+                    threshold, bf16=bool(bf16), packed=packed, packed_feat=packed_feat)
+                out = [rgb, alpha, fmap]
             if nonfinite:
                 for i, t in enumerate(x):
                     if i not in (5, 6):
@@ -276,8 +318,11 @@ class TileExt:
                 warnings.warn("WMMA operand/activation overflow: rendering this frame with scalar FP32 instead")
                 with self._lock:
                     self._mfma_fallbacks += 1
-                rgb, alpha, _ = ops.render_tilecenter_f32(x[0], x[1], rec, order, x[6], x[7], x[8], *x[9:15], width,
-                                                          height, 8, 8, threshold)
-                _chk(bool(torch.isfinite(rgb).all()) and bool(torch.isfinite(alpha).all()),
-                     "Scalar FP32 fallback output is nonfinite")
-        return [rgb, alpha]
+                if feat is None:
+                    out = list(ops.render_tilecenter_f32(x[0], x[1], rec, order, x[6], x[7], x[8], *x[9:15], width,
+                                                         height, 8, 8, threshold))[:2]
+                else:
+                    out = list(ops.render_tilecenter_feat_f32(x[0], x[1], rec, order, x[6], x[7], x[8], *x[9:15],
+                                                              feat[0], feat[1], feat[2], width, height, 8, 8, threshold))
+                _chk(all(bool(torch.isfinite(t).all()) for t in out), "Scalar FP32 fallback output is nonfinite")
+        return out

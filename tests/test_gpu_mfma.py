@@ -123,3 +123,64 @@ def test_scene_module_precision_switch(device, oracle_mod):
     scene.render_precision = "int8"
     with pytest.raises(ValueError, match="render_precision"):
         _call(scene, fr, device)
+
+
+@pytest.mark.parametrize("slots,channels", [(4, 200), (5, 512), (1, 36)])
+@pytest.mark.parametrize("bf16", [True, False])
+def test_matrix_core_feature_render_against_oracle(device, oracle_mod, bf16, slots, channels):
+    # the feature image shares the weights w of the RGB image, so it inherits the same tolerance scaled
+    # by the attribute magnitude (|feat_attr| <= ~4 in this scene -> measured against max|feat|)
+    from mlp_splatting_amd import ops
+    fr = Frame("cfg1_5k_160x120", n=1200, hidden=32, width=56, height=40, feature_dim=channels,
+               feature_slots=slots if slots > 1 else 4)
+    sc = fr.scene
+    fa = sc.feat_attr if slots > 1 else np.ascontiguousarray(sc.feat_attr[:, 0])
+    cand, off = fr.oracle_lists(oracle_mod)
+    want = oracle_mod.render_tilecenter(*fr.base_numpy(cand, off), *fr.dims, feat_attr=fa, beta=1.3, temp=2.2)
+    t = lambda a: to_dev(a, device)
+    rec = ops.prepare_primitives(t(sc.positions), t(sc.log_scales), t(sc.quats))
+    ro, rd, c, o = t(fr.rays_o), t(fr.rays_d), t(cand), t(off)
+    order, _ = ops.sort_tiles(ro, rd, rec, c, o, fr.W, fr.H, 8, 8, cull_threshold=fr.thr)
+    ws = [t(w) for w in sc.mlp()]
+    rgb, alpha, feat, nonfinite = ops.render_tilecenter_mfma_feat(ro, rd, rec, order, o, t(sc.freq), t(sc.att), *ws,
+                                                                  t(fa), 1.3, 2.2, fr.W, fr.H, fr.thr, bf16=bf16)
+    rgb0, alpha0, _ = ops.render_tilecenter_mfma(ro, rd, rec, order, o, t(sc.freq), t(sc.att), *ws, fr.W, fr.H, fr.thr,
+                                                 bf16=bf16)
+    assert not nonfinite
+    assert torch.equal(rgb, rgb0) and torch.equal(alpha, alpha0)         # every channel chunk walks the same hits
+    scale = float(np.abs(want["feat"]).max())
+    err = float(np.abs(feat.cpu().numpy() - want["feat"]).max())
+    print(f"bf16={bf16} slots={slots} C={channels}: max|feat err|={err:.2e} of max|feat|={scale:.2e}")
+    assert scale > 1e-2 and 0 < err <= TOL[bf16] * max(1.0, scale)
+    assert np.abs(rgb.cpu().numpy() - want["rgb"]).max() <= TOL[bf16]
+
+
+def test_scene_module_feature_precision_switch(device, oracle_mod):
+    from test_gpu_scene import _call, _scene_from
+    fr = Frame("cfg1_5k_160x120", n=800, width=40, height=24, hidden=32, feature_dim=64)
+    scene = _scene_from(fr, device, feature=True)
+    rgb, feat = _call(scene, fr, device, return_feature=True)
+    scene.render_precision = "bf16"
+    rgb_b, feat_b = _call(scene, fr, device, return_feature=True)
+    assert torch.equal(rgb_b, _call(scene, fr, device))
+    assert 0 < float((rgb_b - rgb).abs().max()) <= 5e-3
+    assert 0 < float((feat_b - feat).abs().max()) <= 5e-3 * max(1.0, float(feat.abs().max()))
+
+
+def test_feature_attributes_beyond_fp16_fall_back_to_the_exact_kernel(device, oracle_mod):
+    from mlp_splatting_amd.tile_ext import TileExt
+    fr = Frame("cfg1_5k_160x120", n=400, hidden=32, width=32, height=24, feature_dim=40)
+    cand, off = fr.oracle_lists(oracle_mod)
+    x = [to_dev(a, device) for a in fr.base_numpy(cand, off)]
+    fa = to_dev(fr.scene.feat_attr, device).clone()
+    ext = TileExt()
+    rgb, alpha, feat = ext.render_tiles_rgb_wmma_with_feat(x, fa, 1.0, 4.0, fr.W, fr.H, fr.thr, True)
+    exact = ext.render_tiles_forward_tilecenter_with_feat(*x, fa, 1.0, 4.0, fr.W, fr.H, 8, 8, fr.thr)
+    assert 0 < float((feat - exact[2]).abs().max()) <= 5e-3 * max(1.0, float(exact[2].abs().max()))
+    fa[int(cand[0]), 2, 7] = 1.0e5                      # finite in f32, infinite in fp16
+    calls0, fb0 = ext.rgb_wmma_safety_stats()
+    with pytest.warns(UserWarning, match="overflow fp16"):
+        out = ext.render_tiles_rgb_wmma_with_feat(x, fa, 1.0, 4.0, fr.W, fr.H, fr.thr, True)
+    exact = ext.render_tiles_forward_tilecenter_with_feat(*x, fa, 1.0, 4.0, fr.W, fr.H, 8, 8, fr.thr)
+    assert all(torch.equal(a, b) for a, b in zip(out, exact))
+    assert ext.rgb_wmma_safety_stats() == [calls0 + 1, fb0 + 1]
