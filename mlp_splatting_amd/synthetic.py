@@ -37,7 +37,7 @@ CONFIGS = {
 
 # Mean of the natural-log scales used for the 200k-primitive scenes (sigma stays 0.5).
 LOG_SCALE_MEAN_200K = -3.85
-LOG_SCALE_MEAN_200K_CLUSTERED = -4.3
+LOG_SCALE_MEAN_200K_CLUSTERED = -6.0
 
 
 @dataclass

@@ -1,0 +1,207 @@
+"""Parity at the full sizes of the benchmark configurations (50k / 200k primitives, up to 2400x1360).
+
+Where the oracle finishes a frame in seconds on the box's host cores it is the checker, bit for bit; beyond
+that the tests use properties that hold at any size: sortedness and idempotence of the per-tile order, the
+image being independent of the conservative culling, alpha in [0, 1], linearity of the feature image in the
+attributes and its closed form for constant attributes (gates sum to one, so feat = alpha * v).
+"""
+import numpy as np
+import pytest
+import torch
+
+from conftest import to_dev
+
+pytestmark = pytest.mark.gpu
+
+
+class _Big:
+    """A 200k-primitive scene resident on the device, with its frames."""
+
+    def __init__(self, name, device):
+        from mlp_splatting_amd import ops, synthetic as syn
+        self.sc, self.cfg = syn.scene_for_config(name)
+        cfg, sc = self.cfg, self.sc
+        self.W, self.H, self.f, self.thr = cfg["width"], cfg["height"], cfg["focal"], cfg["threshold"]
+        self.device = device
+        self.pos, self.logs, self.quats = (to_dev(a, device) for a in (sc.positions, sc.log_scales, sc.quats))
+        self.ws = [to_dev(a, device) for a in sc.mlp()]
+        self.freq, self.att = to_dev(sc.freq, device), to_dev(sc.att, device)
+        self.rec = ops.prepare_primitives(self.pos, self.logs, self.quats)
+        self.poses = syn.random_poses(32, 0)
+
+    def single_view(self, pose_index):
+        from mlp_splatting_amd import ops, synthetic as syn
+        c2w = self.poses[pose_index]
+        ro, rd = syn.pinhole_rays(self.W, self.H, self.f, c2w)
+        rd = syn.normalize_rays(rd)
+        view = syn.view_matrix(c2w)[None]
+        proj = syn.projection_matrix(self.f, self.W, self.H)
+        cand, off = ops.bin_legacy(self.pos, self.logs, torch.from_numpy(view), torch.from_numpy(proj), self.W, self.H,
+                                   8, self.thr)
+        return dict(ro=ro, rd=rd, view=view, proj=proj, W=self.W, H=self.H, tv=None, cand=cand, off=off,
+                    ro_t=to_dev(ro, self.device), rd_t=to_dev(rd, self.device))
+
+    def oracle_base(self, fr, cand, off):
+        sc = self.sc
+        return (fr["ro"], fr["rd"], sc.positions, sc.log_scales, sc.quats, cand, off, sc.freq, sc.att, *sc.mlp())
+
+
+@pytest.fixture(scope="module")
+def cfg3(device):
+    return _Big("cfg3_200k_1200x680", device)
+
+
+def _bits_equal(t, want):
+    return np.array_equal(t.cpu().numpy().view(np.uint32), np.ascontiguousarray(want, np.float32).view(np.uint32))
+
+
+def test_cfg2_lists_order_and_image_are_bit_exact(device, oracle_mod):
+    # 50k primitives at 640x480: tile lists (counts and order), sorted order and keys, f32 image
+    from helpers import Frame
+    from mlp_splatting_amd import ops
+    fr = Frame("cfg2_50k_640x480", eye=(0.2, -0.1, 0.1), target=(0.1, 0.0, 2.0))
+    sc = fr.scene
+    cand_o, off_o = fr.oracle_lists(oracle_mod)
+    t = lambda a: to_dev(a, device)
+    pos, logs, quats = t(sc.positions), t(sc.log_scales), t(sc.quats)
+    cand, off = ops.bin_legacy(pos, logs, torch.from_numpy(fr.view[None]), torch.from_numpy(fr.proj), fr.W, fr.H, 8, fr.thr)
+    counts = np.diff(off_o)
+    print(f"cfg2: P={cand_o.size} max/tile={counts.max()}")
+    assert counts.max() <= 1536 and cand_o.size > 1_000_000
+    assert np.array_equal(off.cpu().numpy(), off_o) and np.array_equal(cand.cpu().numpy(), cand_o)
+    ids_o, keys_o = oracle_mod.sort_tiles(fr.rays_o, fr.rays_d, sc.positions, sc.log_scales, sc.quats, cand_o, off_o,
+                                          fr.W, fr.H, 8, 8)
+    rec = ops.prepare_primitives(pos, logs, quats)
+    ro, rd = t(fr.rays_o), t(fr.rays_d)
+    ids, keys = ops.sort_tiles(ro, rd, rec, cand, off, fr.W, fr.H, 8, 8, want_keys=True)
+    assert np.array_equal(ids.cpu().numpy(), ids_o) and _bits_equal(keys, keys_o)
+    want = oracle_mod.render_tilecenter(*fr.base_numpy(cand_o, off_o), *fr.dims)
+    ids_c, _ = ops.sort_tiles(ro, rd, rec, cand, off, fr.W, fr.H, 8, 8, cull_threshold=fr.thr)
+    rgb, alpha, _ = ops.render_tilecenter_f32(ro, rd, rec, ids_c, off, t(sc.freq), t(sc.att), *[t(w) for w in sc.mlp()],
+                                              fr.W, fr.H, 8, 8, fr.thr)
+    assert _bits_equal(rgb, want["rgb"]) and _bits_equal(alpha, want["alpha"])
+    assert want["alpha"].mean() > 0.5
+
+
+def test_cfg3_f32_frame_is_bit_exact_and_bf16_within_tolerance(cfg3, oracle_mod):
+    from mlp_splatting_amd import ops
+    b = cfg3
+    fr = b.single_view(0)
+    cand, off = fr["cand"].cpu().numpy(), fr["off"].cpu().numpy()
+    cand_o, off_o = oracle_mod.bin_legacy(b.sc.positions, b.sc.log_scales, fr["view"], fr["proj"], b.W, b.H, 8, b.thr)
+    assert np.array_equal(off, off_o) and np.array_equal(cand, cand_o)
+    assert np.diff(off_o).max() <= 1536
+    want = oracle_mod.render_tilecenter(*b.oracle_base(fr, cand_o, off_o), b.W, b.H, 8, 8, b.thr)
+    ids, _ = ops.sort_tiles(fr["ro_t"], fr["rd_t"], b.rec, fr["cand"], fr["off"], b.W, b.H, 8, 8, cull_threshold=b.thr)
+    counters = torch.zeros(4, dtype=torch.int64, device=b.device)
+    rgb, alpha, _ = ops.render_tilecenter_f32(fr["ro_t"], fr["rd_t"], b.rec, ids, fr["off"], b.freq, b.att, *b.ws,
+                                              b.W, b.H, 8, 8, b.thr, counters=counters)
+    assert _bits_equal(rgb, want["rgb"]) and _bits_equal(alpha, want["alpha"])
+    assert int(counters[3]) == int(want["stats"][3]) > 10_000_000          # same hits, pixel for pixel
+    fast, fast_a, nonfinite = ops.render_tilecenter_mfma(fr["ro_t"], fr["rd_t"], b.rec, ids, fr["off"], b.freq, b.att,
+                                                         *b.ws, b.W, b.H, b.thr, bf16=True)
+    err = float((fast - rgb).abs().max())
+    print(f"cfg3 pose 0: hits={int(counters[3])} bf16 max|err|={err:.2e}")
+    assert not nonfinite and 0 < err <= 5e-3 and float((fast_a - alpha).abs().max()) <= 5e-3
+
+
+def test_cfg3_order_properties_over_poses(cfg3):
+    from mlp_splatting_amd import ops
+    b = cfg3
+    for pose in (1, 7, 19):
+        fr = b.single_view(pose)
+        off = fr["off"]
+        counts = (off[1:] - off[:-1])
+        assert int(counts.max()) <= 1536
+        ids, keys = ops.sort_tiles(fr["ro_t"], fr["rd_t"], b.rec, fr["cand"], off, b.W, b.H, 8, 8, want_keys=True)
+        # keys ascend inside every tile
+        tile_of = torch.repeat_interleave(torch.arange(counts.numel(), device=b.device), counts.long())
+        same_tile = tile_of[1:] == tile_of[:-1]
+        assert bool((keys[1:][same_tile] >= keys[:-1][same_tile]).all())
+        # a permutation of each tile's list: sorting ids inside tiles gives back the ascending input
+        composite = tile_of.long() * (b.sc.n + 1) + ids.long()
+        assert torch.equal(torch.sort(composite).values, tile_of.long() * (b.sc.n + 1) + fr["cand"].long())
+        # idempotent: sorting the sorted list changes nothing
+        ids2, keys2 = ops.sort_tiles(fr["ro_t"], fr["rd_t"], b.rec, ids, off, b.W, b.H, 8, 8, want_keys=True)
+        assert torch.equal(keys2, keys) and torch.equal(ids2, ids)
+        # culling never changes the image, and alpha stays in [0, 1]
+        ids_c, _ = ops.sort_tiles(fr["ro_t"], fr["rd_t"], b.rec, fr["cand"], off, b.W, b.H, 8, 8, cull_threshold=b.thr)
+        assert 0.2 < float((ids_c < 0).float().mean()) < 0.7
+        assert torch.equal(torch.where(ids_c < 0, ~ids_c, ids_c), ids)
+        a = ops.render_tilecenter_mfma(fr["ro_t"], fr["rd_t"], b.rec, ids, off, b.freq, b.att, *b.ws, b.W, b.H, b.thr)
+        c = ops.render_tilecenter_mfma(fr["ro_t"], fr["rd_t"], b.rec, ids_c, off, b.freq, b.att, *b.ws, b.W, b.H, b.thr)
+        assert torch.equal(a[0], c[0]) and torch.equal(a[1], c[1])
+        assert float(a[1].min()) >= 0.0 and float(a[1].max()) <= 1.0 and bool(torch.isfinite(a[0]).all())
+
+
+def test_cfg3_every_pose_fits_the_tile_capacity(cfg3):
+    b = cfg3
+    worst = max(int((fr["off"][1:] - fr["off"][:-1]).max()) for fr in (b.single_view(i) for i in range(32)))
+    print(f"cfg3: worst tile over 32 poses = {worst}")
+    assert 1400 < worst <= 1536
+
+
+def test_cfg5_feature_image_properties_at_512_channels(cfg3):
+    # config 5 = the config-3 scene + feat_attr [N, 4, 512]
+    from mlp_splatting_amd import ops
+    b = cfg3
+    fr = b.single_view(3)
+    ids, _ = ops.sort_tiles(fr["ro_t"], fr["rd_t"], b.rec, fr["cand"], fr["off"], b.W, b.H, 8, 8, cull_threshold=b.thr)
+    g = torch.Generator(device=b.device)
+    g.manual_seed(11)
+    C = 512
+    fa = torch.randn(b.sc.n, 4, C, device=b.device, generator=g) * 0.05
+    fb = torch.randn(b.sc.n, 4, C, device=b.device, generator=g) * 0.05
+    args = (fr["ro_t"], fr["rd_t"], b.rec, ids, fr["off"], b.freq, b.att, *b.ws)
+    tail = (1.0, 4.0, b.W, b.H, b.thr)
+    rgb, alpha, feat_a, bad = ops.render_tilecenter_mfma_feat(*args, fa, *tail)
+    rgb0, alpha0, _ = ops.render_tilecenter_mfma(*args, b.W, b.H, b.thr)
+    assert not bad and torch.equal(rgb, rgb0) and torch.equal(alpha, alpha0)
+    scale = float(feat_a.abs().max())
+    assert scale > 0.02
+    # exact kernel on the same frame (the 136 ms path): same image within the reduced-precision tolerance
+    exact = ops.render_tilecenter_feat_f32(*args, fa, 1.0, 4.0, b.W, b.H, 8, 8, b.thr)
+    err = float((feat_a - exact[2]).abs().max())
+    print(f"cfg5: max|feat| = {scale:.3f}, matrix-core vs exact = {err:.2e}")
+    assert 0 < err <= 5e-3
+    # linear in the attributes
+    feat_b = ops.render_tilecenter_mfma_feat(*args, fb, *tail)[2]
+    feat_ab = ops.render_tilecenter_mfma_feat(*args, fa + fb, *tail)[2]
+    assert float((feat_ab - (feat_a + feat_b)).abs().max()) <= 1e-3
+    del feat_b, feat_ab, fb
+    # constant rows: the gates sum to one, so the feature image is alpha * v
+    v = torch.linspace(-1.0, 1.0, C, device=b.device)
+    fc = v[None, None, :].expand(b.sc.n, 4, C).contiguous()
+    for out in (ops.render_tilecenter_mfma_feat(*args, fc, *tail), ops.render_tilecenter_feat_f32(*args, fc, 1.0, 4.0, b.W, b.H, 8, 8, b.thr)):
+        tol = 5e-3 if len(out) == 4 else 2e-5
+        assert float((out[2] - out[1] * v[None, :]).abs().max()) <= tol
+
+
+def test_cfg4_mosaic_lists_and_image_match_the_oracle(device, oracle_mod):
+    # four 1200x680 views per call, 30 % of the primitives inside a 0.5 m box: several tiles come
+    # close to the 1,536 capacity and none exceeds it
+    from mlp_splatting_amd import ops, synthetic as syn
+    b = _Big("cfg4_200k_mosaic4", device)
+    W, H = b.W, b.H                              # the whole 2400 x 1360 frame
+    ro, rd, tv, views = syn.mosaic_frame(W // 2, H // 2, b.f, b.poses[:4])
+    rd = syn.normalize_rays(rd)
+    proj = syn.projection_matrix(b.f, W, H)
+    cand, off = ops.bin_legacy(b.pos, b.logs, torch.from_numpy(views), torch.from_numpy(proj), W, H, 8, b.thr,
+                               tile_view_ids=torch.from_numpy(tv))
+    cand_o, off_o = oracle_mod.bin_legacy(b.sc.positions, b.sc.log_scales, views, proj, W, H, 8, b.thr, tile_view_ids=tv)
+    counts = np.diff(off_o)
+    print(f"cfg4: P={cand_o.size} max/tile={counts.max()} tiles over 1200: {(counts > 1200).sum()}")
+    assert np.array_equal(off.cpu().numpy(), off_o) and np.array_equal(cand.cpu().numpy(), cand_o)
+    assert 1400 < counts.max() <= 1536 and (counts > 1200).sum() >= 3
+    ro_t, rd_t = to_dev(ro, device), to_dev(rd, device)
+    ids, _ = ops.sort_tiles(ro_t, rd_t, b.rec, cand, off, W, H, 8, 8, cull_threshold=b.thr)
+    rgb, alpha, _ = ops.render_tilecenter_f32(ro_t, rd_t, b.rec, ids, off, b.freq, b.att, *b.ws, W, H, 8, 8, b.thr)
+    fr = dict(ro=ro, rd=rd)
+    want = oracle_mod.render_tilecenter(*b.oracle_base(fr, cand_o, off_o), W, H, 8, 8, b.thr)
+    assert _bits_equal(rgb, want["rgb"]) and _bits_equal(alpha, want["alpha"])
+    fast = ops.render_tilecenter_mfma(ro_t, rd_t, b.rec, ids, off, b.freq, b.att, *b.ws, W, H, b.thr)
+    assert not fast[2] and float((fast[0] - rgb).abs().max()) <= 5e-3
+    # one more tile entry than the capacity is refused, as the reference does
+    ops.validate_tile_lists(cand, off, ops.num_tiles(W, H, 8, 8), 1536, b.sc.n, "mosaic")
+    with pytest.raises(RuntimeError, match=f"capacity {int(counts.max()) - 1} exceeded"):
+        ops.validate_tile_lists(cand, off, ops.num_tiles(W, H, 8, 8), int(counts.max()) - 1, b.sc.n, "mosaic")
