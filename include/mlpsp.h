@@ -127,10 +127,24 @@ int mlpsp_render_tilecenter_f32(const float* rays_o_dev, const float* rays_d_dev
                                 float threshold, float* out_rgb_dev, float* out_alpha_dev, float* out_t_dev,
                                 int64_t* counters_dev, mlpsp_stream_t stream);
 
+/* Workspace of the feature renders below.  The render kernel hands the feature kernel one "hit record"
+ * per (64-pixel wavefront of a tile, primitive that hits one of its pixels); how many there will be is
+ * only known after the frame (early termination), so records come from a pool of pool_records records.
+ * pool_records < 0 asks for the worst case (one per candidate and wavefront + 15 per wavefront), which can
+ * never run out; a smaller pool that runs out sets the call's overflow status and the caller repeats the
+ * frame with a larger one.  fp16_records: 0 for mlpsp_render_tilecenter_feat_f32, 1 for
+ * mlpsp_render_tilecenter_mfma_feat (tile_w = tile_h = 8).  0 on bad arguments. */
+size_t mlpsp_feat_workspace_bytes(int64_t num_pairs, int width, int height, int tile_w, int tile_h, int feat_slots,
+                                  int fp16_records, int64_t pool_records);
+
 /* Tile-centre-order forward with the gated feature channel, scalar f32
  * (render_tiles_kernel_tilecenter_order_with_feat, np_tile_kernels.cu:5794-6112).
  * feat_slots: 1 (feat_attr [N,C]), 4 or 5 ([N,slots,C]); feat_channels <= 512.
- * out_feat_dev [B,C] is fully written (no pre-zeroing needed). */
+ * out_feat_dev [B,C] is fully written (no pre-zeroing needed).  num_pairs = length of order_dev.
+ * workspace_dev: 256-byte aligned, at least mlpsp_feat_workspace_bytes(.., pool_records = 0) bytes
+ * (MLPSP_E_SCRATCH otherwise); whatever it holds beyond that is the record pool.
+ * status_dev[0] (device int32) = 1 if the pool ran out: out_feat_dev is then incomplete (RGB and alpha
+ * are complete either way). */
 int mlpsp_render_tilecenter_feat_f32(const float* rays_o_dev, const float* rays_d_dev, const void* prim_records_dev,
                                      const int32_t* order_dev, const int32_t* tile_offsets_dev,
                                      const float* freq_dev, const float* att_dev, int num_frequencies,
@@ -138,8 +152,9 @@ int mlpsp_render_tilecenter_feat_f32(const float* rays_o_dev, const float* rays_
                                      const float* W3, const float* b3, int num_primitives, int hidden,
                                      const float* feat_attr_dev, int feat_slots, int feat_channels,
                                      float gating_beta, float gating_temp, int width, int height, int tile_w,
-                                     int tile_h, float threshold, float* out_rgb_dev, float* out_alpha_dev,
-                                     float* out_feat_dev, mlpsp_stream_t stream);
+                                     int tile_h, float threshold, int64_t num_pairs, void* workspace_dev,
+                                     size_t workspace_bytes, float* out_rgb_dev, float* out_alpha_dev,
+                                     float* out_feat_dev, int32_t* status_dev, mlpsp_stream_t stream);
 
 /* Per-pixel-order forward (render_tiles_kernel_with_sort[_and_feat], np_tile_kernels.cu:715-1208):
  * every pixel blends its own hits in order of its own t.  candidates_dev is the unsorted tile list.
@@ -186,12 +201,12 @@ int mlpsp_render_tilecenter_mfma(const float* rays_o_dev, const float* rays_d_de
  * mlpsp_pack_mfma_feat: feat_attr f32 [N,S,C] ([N,C] for S = 1) -> operand copy (once per scene);
  * status_dev[0] = 1 if a value is not finite in fp16 (then use the f32 feature kernel).
  * num_pairs = length of order_dev = tile_offsets[num_tiles].  feat_slots = 0 renders RGB only and
- * ignores the feature and workspace arguments.  MLPSP_E_SCRATCH if the workspace is too small or not
+ * ignores the feature and workspace arguments.  Workspace: mlpsp_feat_workspace_bytes(.., fp16_records = 1, ..);
+ * status_dev[1] = 1 if its record pool ran out.  MLPSP_E_SCRATCH if the workspace is too small or not
  * 256-byte aligned. */
 size_t mlpsp_mfma_feat_pack_bytes(int num_primitives, int feat_slots, int feat_channels);
 int mlpsp_pack_mfma_feat(const float* feat_attr_dev, int num_primitives, int feat_slots, int feat_channels,
                          void* packed_feat_dev, int32_t* status_dev, mlpsp_stream_t stream);
-size_t mlpsp_mfma_feat_workspace_bytes(int64_t num_pairs, int width, int height, int feat_slots);
 int mlpsp_render_tilecenter_mfma_feat(const float* rays_o_dev, const float* rays_d_dev, const void* prim_records_dev,
                                       const int32_t* order_dev, const int32_t* tile_offsets_dev, int64_t num_pairs,
                                       const float* freq_dev, const float* att_dev, const void* packed_dev,

@@ -1,0 +1,110 @@
+// The scalar-f32 tile-centre render kernel (shared by the RGB entry point and the feature entry point,
+// which asks it to emit hit records).
+#pragma once
+#include "mlpsp_device.hpp"
+#include "mlpsp_hitrec.hpp"
+#include "mlpsp_host.hpp"
+#include "mlpsp_mlp.hpp"
+
+namespace mlpsp {
+
+// EMIT = 0: image only.  EMIT = 1 / 2: also emit one hit record per primitive that hits a pixel of this
+// wavefront, float[K][64] with K = 1 (the compositing weight w) / K = 5 (w and the four tetrahedral
+// gates); w = -1 marks a pixel the primitive did not hit (weights are never negative).
+template <int HT, int FT, int EMIT>
+__global__ __launch_bounds__(64) void render_tilecenter_f32_kernel(
+    const float* __restrict__ rays_o, const float* __restrict__ rays_d, const PrimRecord* __restrict__ prims,
+    const int32_t* __restrict__ order, const int32_t* __restrict__ offsets, const float* __restrict__ freq,
+    const float* __restrict__ att, int F, const float* __restrict__ W1, const float* __restrict__ b1,
+    const float* __restrict__ W2, const float* __restrict__ b2, const float* __restrict__ W3,
+    const float* __restrict__ b3, int N, int H, TileGeom g, int waves_per_tile, int per_xcd,
+    int num_items, float thr, float* __restrict__ out_rgb, float* __restrict__ out_alpha, float* __restrict__ out_t,
+    unsigned long long* __restrict__ counters, float beta, float temp, HitPool hp) {
+  // The weight pointers are separate __restrict__ parameters (not a struct): only then does the compiler
+  // know that the record stores below cannot alias them and keeps fetching weights with scalar loads.
+  const MlpPtrs mlp{W1, b1, W2, b2, W3, b3};
+  // XCD-aware work assignment: XCD k (blockIdx.x % 8) walks items [k*per_xcd, (k+1)*per_xcd).
+  const int item = (blockIdx.x % kNumXcd) * per_xcd + blockIdx.x / kNumXcd;
+  if (item >= num_items) return;
+  const int tile = item / waves_per_tile, wslot = item % waves_per_tile;
+  const int slot = wslot * 64 + threadIdx.x;
+  const int tx = tile % g.ntx, ty = tile / g.ntx;
+  const int lx = slot % g.TW, ly = slot / g.TW;
+  const int x = tx * g.TW + lx, y = ty * g.TH + ly;
+  const bool valid = (slot < g.TW * g.TH) && (x < g.W) && (y < g.H);
+  const int pix = valid ? (y * g.W + x) : 0;
+
+  const float rox = valid ? rays_o[pix * 3 + 0] : 0.f;
+  const float roy = valid ? rays_o[pix * 3 + 1] : 0.f;
+  const float roz = valid ? rays_o[pix * 3 + 2] : 0.f;
+  const float rdx = valid ? rays_d[pix * 3 + 0] : 0.f;
+  const float rdy = valid ? rays_d[pix * 3 + 1] : 0.f;
+  const float rdz = valid ? rays_d[pix * 3 + 2] : 0.f;
+
+  const int start = offsets[tile];
+  const int end = offsets[tile + 1];
+
+  PixelAcc acc = {0.f, 0.f, 0.f, 1.f, 0.f, 0.f};
+  unsigned n_proc = 0, n_proc_hit = 0, n_hits = 0;
+  HitEmitter em = hit_emitter_begin(hp, wslot, start, tile);
+
+  for (int i = start; i < end; ++i) {
+    const int p = __builtin_amdgcn_readfirstlane(order[i]);
+    if (p < 0 || p >= N) continue;
+    const PrimRecord P = prims[p];
+    HitInfo h;
+    const bool live = valid && (acc.trans >= kTransmittanceFloor);
+    const bool hit = live && hit_rot(rox, roy, roz, rdx, rdy, rdz, P, thr, h);
+    const unsigned long long hit_mask = __ballot(hit);
+    ++n_proc;
+    if (hit_mask != 0ull) {
+      ++n_proc_hit;
+      n_hits += __popcll(hit_mask);
+      int rs = -1;
+      if constexpr (EMIT > 0) rs = hit_emitter_next(hp, em, (int)threadIdx.x);
+      float* __restrict__ rec = reinterpret_cast<float*>(hp.records + (size_t)(rs < 0 ? 0 : rs) * hp.record_bytes);
+      if (hit) {
+        const float x6[6] = {rdx, rdy, rdz, h.dx, h.dy, h.dz};
+        float o[4];
+        mlp_eval<HT, FT>(x6, freq, att, F, H, mlp, p, o);
+        const float w = blend_step(acc, o[0], o[1], o[2], o[3], h.decay, h.t);
+        if constexpr (EMIT > 0) {
+          if (rs >= 0) {
+            rec[threadIdx.x] = w;
+            if constexpr (EMIT > 1) {
+              float gt[4];
+              tetra_gates(h.qlx, h.qly, h.qlz, P.lgx, P.lgy, P.lgz, beta, temp, gt);
+#pragma unroll
+              for (int k = 0; k < 4; ++k) rec[(k + 1) * 64 + threadIdx.x] = gt[k];
+            }
+          }
+        }
+      } else if constexpr (EMIT > 0) {
+        if (rs >= 0) rec[threadIdx.x] = -1.f;       // the gates of a missed pixel are never read
+      }
+      if constexpr (EMIT > 0) {
+        if (rs >= 0 && threadIdx.x == 0) hp.hit_ids[rs] = p;
+      }
+    }
+    if (__ballot(valid && (acc.trans >= kTransmittanceFloor)) == 0ull) break;
+  }
+
+  if (valid) {
+    out_rgb[pix * 3 + 0] = acc.cr;
+    out_rgb[pix * 3 + 1] = acc.cg;
+    out_rgb[pix * 3 + 2] = acc.cb;
+    out_alpha[pix] = 1.f - acc.trans;
+    if (out_t) out_t[pix] = acc.t_acc / (acc.w_acc > 1e-8f ? acc.w_acc : 1.f);
+  }
+  if constexpr (EMIT > 0) {
+    if (threadIdx.x == 0) hp.item_hits[item] = em.count;
+  }
+  if (counters && threadIdx.x == 0) {
+    atomicAdd(counters + 1, (unsigned long long)n_proc);
+    atomicAdd(counters + 2, (unsigned long long)n_proc_hit);
+    atomicAdd(counters + 3, (unsigned long long)n_hits);
+  }
+}
+
+}  // namespace mlpsp
+

@@ -23,6 +23,7 @@
 // LDS sin/cos table -- same kernel time, 2x the image error; persistent wavefronts with a tile work
 // queue -- 6 % slower than one wavefront per tile.)
 #include "mlpsp_device.hpp"
+#include "mlpsp_hitrec.hpp"
 #include "mlpsp_host.hpp"
 
 namespace mlpsp {
@@ -203,7 +204,7 @@ __device__ __forceinline__ void fast_tetra_gates(float qlx, float qly, float qlz
 }
 
 // SP = 0: RGB only.  SP = 4 or 8: the kernel also emits, per tile, the compact list of primitives that
-// hit at least one pixel (hit_ids[start + m]) and per (such primitive, pixel) the SP compositing
+// hit at least one pixel (hit records, mlpsp_hitrec.hpp) and per (such primitive, pixel) the SP compositing
 // coefficients of the gated feature channel, rounded to fp16 (they lie in [0, 1]; fp16 keeps 11
 // significant bits there, bf16 only 8): (w g0, w g1, w g2, w g3) for 4 slots,
 // (w, 0, 0, 0) for one slot, (w, w g0, .., w g3, 0, 0, 0) for 5 slots (np_tile_kernels.cu:6036-6075:
@@ -216,7 +217,7 @@ __global__ __launch_bounds__(64) void render_tilecenter_mfma_kernel(
     const float* __restrict__ att, const unsigned char* __restrict__ packed, int N, int W, int H, int ntx,
     int per_xcd, int num_tiles, float thr, float* __restrict__ out_rgb, float* __restrict__ out_alpha,
     int32_t* __restrict__ status, unsigned long long* __restrict__ counters, int slots, float beta, float temp,
-    int32_t* __restrict__ hit_ids, int32_t* __restrict__ tile_hits, unsigned* __restrict__ coef) {
+    HitPool hp) {
   // XCD-aware work assignment: XCD k (blockIdx.x % 8) walks tiles [k*per_xcd, (k+1)*per_xcd) in
   // row-major order, so neighbouring tiles -- which share most primitives -- run together on one L2.
   const int tile = (blockIdx.x % kNumXcd) * per_xcd + blockIdx.x / kNumXcd;
@@ -243,7 +244,7 @@ __global__ __launch_bounds__(64) void render_tilecenter_mfma_kernel(
 
   const int start = offsets[tile], end = offsets[tile + 1];
   PixelAcc acc = {0.f, 0.f, 0.f, 1.f, 0.f, 0.f};
-  int n_emit = 0;
+  HitEmitter em = hit_emitter_begin(hp, 0, start, tile);
 
   for (int i = start; i < end; ++i) {
     const int p = __builtin_amdgcn_readfirstlane(order[i]);
@@ -359,17 +360,20 @@ __global__ __launch_bounds__(64) void render_tilecenter_mfma_kernel(
       if constexpr (SP > 0) {
         float gt[4] = {0.f, 0.f, 0.f, 0.f};
         if (hit && slots > 1) fast_tetra_gates(h.qlx, h.qly, h.qlz, P.lgx, P.lgy, P.lgz, beta, temp, gt);
-        const size_t row = (size_t)(start + n_emit) * 64 + l;
-        if constexpr (SP == 4) {
-          const unsigned c01 = (slots > 1) ? Ops<_Float16>::pack2(w * gt[0], w * gt[1]) : Ops<_Float16>::pack2(w, 0.f);
-          const unsigned c23 = Ops<_Float16>::pack2(w * gt[2], w * gt[3]);
-          *reinterpret_cast<uint2*>(coef + row * 2) = make_uint2(c01, c23);
-        } else {
-          const u32x4 c = {Ops<_Float16>::pack2(w, w * gt[0]), Ops<_Float16>::pack2(w * gt[1], w * gt[2]), Ops<_Float16>::pack2(w * gt[3], 0.f), 0u};
-          *reinterpret_cast<u32x4*>(coef + row * 4) = c;
+        const int rs = hit_emitter_next(hp, em, l);
+        if (rs >= 0) {
+          unsigned* __restrict__ coef = reinterpret_cast<unsigned*>(hp.records + (size_t)rs * hp.record_bytes);
+          if constexpr (SP == 4) {
+            const unsigned c01 = (slots > 1) ? Ops<_Float16>::pack2(w * gt[0], w * gt[1]) : Ops<_Float16>::pack2(w, 0.f);
+            const unsigned c23 = Ops<_Float16>::pack2(w * gt[2], w * gt[3]);
+            *reinterpret_cast<uint2*>(coef + l * 2) = make_uint2(c01, c23);
+          } else {
+            const u32x4 c = {Ops<_Float16>::pack2(w, w * gt[0]), Ops<_Float16>::pack2(w * gt[1], w * gt[2]),
+                             Ops<_Float16>::pack2(w * gt[3], 0.f), 0u};
+            *reinterpret_cast<u32x4*>(coef + l * 4) = c;
+          }
+          if (l == 0) hp.hit_ids[rs] = p;
         }
-        if (l == 0) hit_ids[start + n_emit] = p;
-        ++n_emit;
       }
     }
     if (__ballot(valid && (acc.trans >= kTransmittanceFloor)) == 0ull) break;
@@ -382,7 +386,7 @@ __global__ __launch_bounds__(64) void render_tilecenter_mfma_kernel(
     out_alpha[pix] = 1.f - acc.trans;
   }
   if constexpr (SP > 0) {
-    if (l == 0) tile_hits[tile] = n_emit;
+    if (l == 0) hp.item_hits[tile] = em.count;
   }
   if (__ballot(bad) != 0ull && l == 0) atomicExch(status, 1);
   if (counters && l == 0) {
@@ -426,10 +430,8 @@ __global__ __launch_bounds__(256) void pack_feat_kernel(const float* __restrict_
 // K-slot j of lane group g is (record 16/SP * step + g * 8/SP + j / SP, slot j % SP): both operands are
 // plain 8- or 16-byte loads, coalesced over 32 pixels / 32 channels.
 template <int SP>
-__global__ __launch_bounds__(256) void feat_gemm_kernel(const unsigned* __restrict__ attr, const int32_t* __restrict__ hit_ids,
-                                                        const unsigned* __restrict__ coef,
-                                                        const int32_t* __restrict__ offsets,
-                                                        const int32_t* __restrict__ tile_hits, int C, int W, int H,
+__global__ __launch_bounds__(256) void feat_gemm_kernel(const unsigned* __restrict__ attr, HitPool hp,
+                                                        const int32_t* __restrict__ offsets, int C, int W, int H,
                                                         int ntx, int per_xcd, int num_tiles,
                                                         float* __restrict__ out_feat) {
   const int tile = (blockIdx.x % kNumXcd) * per_xcd + blockIdx.x / kNumXcd;
@@ -440,7 +442,8 @@ __global__ __launch_bounds__(256) void feat_gemm_kernel(const unsigned* __restri
   const int ncb = min(4, (C - c0 + 31) / 32);
   constexpr int EPL = 8 / SP;         // records per lane group and K-step
   constexpr int DW = SP / 2;          // dwords per (record, pixel) and per (primitive, channel)
-  const int start = offsets[tile], hits = tile_hits[tile];
+  const int hits = hp.item_hits[tile];
+  const int table_base = (offsets[tile] >> 4) + tile;
   f32x16 acc[2][4];
 #pragma unroll
   for (int pb = 0; pb < 2; ++pb)
@@ -460,8 +463,9 @@ __global__ __launch_bounds__(256) void feat_gemm_kernel(const unsigned* __restri
     for (int u = 0; u < EPL; ++u) {
       const int ent = e + g * EPL + u;
       if (ent < hits) {
-        const size_t prim = (size_t)hit_ids[start + ent];
-        const unsigned* __restrict__ crow = coef + ((size_t)(start + ent) * 64 + m) * DW;
+        const int rs = hit_slot(hp, table_base, ent);
+        const size_t prim = (size_t)hp.hit_ids[rs];
+        const unsigned* __restrict__ crow = reinterpret_cast<const unsigned*>(hp.records + (size_t)rs * hp.record_bytes) + m * DW;
         const unsigned* __restrict__ arow = attr + prim * C * DW;
         if constexpr (SP == 4) {
 #pragma unroll
@@ -549,11 +553,10 @@ template <typename E, int SP>
 void launch_mfma(dim3 grid, hipStream_t s, const float* rays_o, const float* rays_d, const void* prims, const int32_t* order,
                  const int32_t* offsets, const float* freq, const float* att, const void* packed, int N, int W, int H,
                  int ntx, int per_xcd, int T, float thr, float* rgb, float* alpha, int32_t* status,
-                 unsigned long long* ctr, int slots, float beta, float temp, int32_t* hit_ids, int32_t* tile_hits,
-                 unsigned* coef) {
+                 unsigned long long* ctr, int slots, float beta, float temp, const HitPool& hp) {
   hipLaunchKernelGGL((render_tilecenter_mfma_kernel<E, SP>), grid, dim3(64), 0, s, rays_o, rays_d,
                      (const PrimRecord*)prims, order, offsets, freq, att, (const unsigned char*)packed, N, W, H, ntx,
-                     per_xcd, T, thr, rgb, alpha, status, ctr, slots, beta, temp, hit_ids, tile_hits, coef);
+                     per_xcd, T, thr, rgb, alpha, status, ctr, slots, beta, temp, hp);
 }
 }  // namespace
 
@@ -583,13 +586,6 @@ MLPSP_API int mlpsp_pack_mfma_feat(const float* feat_attr_dev, int num_primitive
   return MLPSP_OK;
 }
 
-MLPSP_API size_t mlpsp_mfma_feat_workspace_bytes(int64_t num_pairs, int width, int height, int feat_slots) {
-  const int64_t T = checked_num_tiles(width, height, 8, 8);
-  if (T <= 0 || num_pairs < 0 || !(feat_slots == 1 || feat_slots == 4 || feat_slots == 5)) return 0;
-  return align256((size_t)num_pairs * 4) + align256((size_t)T * 4) +
-         align256((size_t)num_pairs * 64 * feat_pad(feat_slots) * 2) + 256;
-}
-
 MLPSP_API int mlpsp_render_tilecenter_mfma_feat(const float* rays_o_dev, const float* rays_d_dev,
                                                 const void* prim_records_dev, const int32_t* order_dev,
                                                 const int32_t* tile_offsets_dev, int64_t num_pairs,
@@ -607,34 +603,28 @@ MLPSP_API int mlpsp_render_tilecenter_mfma_feat(const float* rays_o_dev, const f
       !status_dev)
     return MLPSP_E_ARGUMENT;
   if (num_primitives > 0 && !packed_dev) return MLPSP_E_ARGUMENT;
-  int32_t *hit_ids = nullptr, *tile_hits = nullptr;
-  unsigned* coef = nullptr;
+  hipStream_t s = (hipStream_t)stream;
+  HitPool hp{};
   if (feat_slots != 0) {
     if (!(feat_slots == 1 || feat_slots == 4 || feat_slots == 5) || feat_channels <= 0 || feat_channels > 512 ||
         !out_feat_dev || (num_primitives > 0 && !packed_feat_dev))
       return MLPSP_E_ARGUMENT;
     if (!workspace_dev || reinterpret_cast<uintptr_t>(workspace_dev) % 256 != 0 ||
-        workspace_bytes < mlpsp_mfma_feat_workspace_bytes(num_pairs, width, height, feat_slots))
+        workspace_bytes < hitpool_min_bytes(num_pairs, T, 1))
       return MLPSP_E_SCRATCH;
-    unsigned char* ws = (unsigned char*)workspace_dev;
-    hit_ids = (int32_t*)ws;
-    ws += align256((size_t)num_pairs * 4);
-    tile_hits = (int32_t*)ws;
-    ws += align256((size_t)T * 4);
-    coef = (unsigned*)ws;
+    hp = hitpool_carve(workspace_dev, workspace_bytes, num_pairs, T, 1, 64 * 2 * feat_pad(feat_slots));
+    MLPSP_HIP_TRY(hipMemsetAsync(hp.counters, 0, 64 * sizeof(int32_t), s));
   }
-  MLPSP_HIP_TRY(hipMemsetAsync(status_dev, 0, 16 * sizeof(int32_t), (hipStream_t)stream));
+  MLPSP_HIP_TRY(hipMemsetAsync(status_dev, 0, 16 * sizeof(int32_t), s));
   const int per_xcd = (int)((T + kNumXcd - 1) / kNumXcd);
   const dim3 grid((unsigned)(per_xcd * kNumXcd));
-  hipStream_t s = (hipStream_t)stream;
   auto* ctr = reinterpret_cast<unsigned long long*>(counters_dev);
   const int ntx = ceil_div(width, 8);
   const int sp = feat_slots ? feat_pad(feat_slots) : 0;
 #define MLPSP_MFMA_GO(TT, SP)                                                                                     \
   launch_mfma<TT, SP>(grid, s, rays_o_dev, rays_d_dev, prim_records_dev, order_dev, tile_offsets_dev, freq_dev,   \
                       att_dev, packed_dev, num_primitives, width, height, ntx, per_xcd, (int)T, threshold,        \
-                      out_rgb_dev, out_alpha_dev, status_dev, ctr, feat_slots, gating_beta, gating_temp, hit_ids, \
-                      tile_hits, coef)
+                      out_rgb_dev, out_alpha_dev, status_dev, ctr, feat_slots, gating_beta, gating_temp, hp)
 #define MLPSP_MFMA_SP(TT)                 \
   do {                                    \
     if (sp == 0) MLPSP_MFMA_GO(TT, 0);    \
@@ -648,14 +638,15 @@ MLPSP_API int mlpsp_render_tilecenter_mfma_feat(const float* rays_o_dev, const f
   MLPSP_LAUNCH_CHECK();
   if (sp != 0) {
     const dim3 ggrid((unsigned)(per_xcd * kNumXcd), (unsigned)ceil_div(feat_channels, 512)), gblock(256);
-#define MLPSP_FEAT_GEMM(SP)                                                                                  \
-  hipLaunchKernelGGL((feat_gemm_kernel<SP>), ggrid, gblock, 0, s, (const unsigned*)packed_feat_dev, hit_ids, \
-                     coef, tile_offsets_dev, tile_hits, feat_channels, width, height, ntx, per_xcd, (int)T,  \
-                     out_feat_dev)
+#define MLPSP_FEAT_GEMM(SP)                                                                                       \
+  hipLaunchKernelGGL((feat_gemm_kernel<SP>), ggrid, gblock, 0, s, (const unsigned*)packed_feat_dev, hp,           \
+                     tile_offsets_dev, feat_channels, width, height, ntx, per_xcd, (int)T, out_feat_dev)
     if (sp == 4) MLPSP_FEAT_GEMM(4);
     else MLPSP_FEAT_GEMM(8);
 #undef MLPSP_FEAT_GEMM
     MLPSP_LAUNCH_CHECK();
+    // status_dev[1] = 1 if the record pool was too small (the feature image is then incomplete)
+    MLPSP_HIP_TRY(hipMemcpyAsync(status_dev + 1, hp.counters + 1, sizeof(int32_t), hipMemcpyDeviceToDevice, s));
   }
   return MLPSP_OK;
 }

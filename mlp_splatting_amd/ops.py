@@ -168,21 +168,39 @@ def _feat_shape(feat_attr):
     return int(slots), int(ch)
 
 
+def _feat_pool_sizes(pairs: int):
+    """Record-pool sizes to try in turn: a quarter of the candidates (at the 200k-primitive benchmark scene
+    8 % of them hit before their tile saturates), then the worst case, which cannot run out."""
+    first = max(pairs // 4, 1 << 16)
+    return (first, -1) if first < pairs else (-1,)
+
+
 def render_tilecenter_feat_f32(rays_o, rays_d, records, order, tile_offsets, freq, att, W1, b1, W2, b2, W3, b3,
                                feat_attr, beta, temp, W, H, TW, TH, threshold):
     """Scalar-f32 tile-centre forward with the gated feature channel -> (rgb, alpha, feat [B,C])."""
     dev = rays_o.device
     slots, ch = _feat_shape(feat_attr)
     B = W * H
+    lib = _lib.load()
     rgb = torch.empty(B, 3, dtype=torch.float32, device=dev)
     alpha = torch.empty(B, 1, dtype=torch.float32, device=dev)
     feat = torch.empty(B, ch, dtype=torch.float32, device=dev)
+    status = torch.empty(1, dtype=torch.int32, device=dev)
     n, hidden, F = W1.shape[0], W2.shape[1], freq.shape[0]
-    code = _lib.load().mlpsp_render_tilecenter_feat_f32(
-        _ptr(rays_o), _ptr(rays_d), _ptr(records), _ptr(order), _ptr(tile_offsets), _ptr(freq), _ptr(att), F,
-        _ptr(W1), _ptr(b1), _ptr(W2), _ptr(b2), _ptr(W3), _ptr(b3), n, hidden, _ptr(feat_attr), slots, ch,
-        float(beta), float(temp), W, H, TW, TH, float(threshold), _ptr(rgb), _ptr(alpha), _ptr(feat), _stream(dev))
-    _check(code, "mlpsp_render_tilecenter_feat_f32")
+    pairs = int(order.numel())
+    for pool in _feat_pool_sizes(pairs):
+        nbytes = lib.mlpsp_feat_workspace_bytes(pairs, W, H, TW, TH, slots, 0, pool)
+        if nbytes == 0:
+            raise RuntimeError("mlpsp_feat_workspace_bytes: bad arguments")
+        workspace = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+        code = lib.mlpsp_render_tilecenter_feat_f32(
+            _ptr(rays_o), _ptr(rays_d), _ptr(records), _ptr(order), _ptr(tile_offsets), _ptr(freq), _ptr(att), F,
+            _ptr(W1), _ptr(b1), _ptr(W2), _ptr(b2), _ptr(W3), _ptr(b3), n, hidden, _ptr(feat_attr), slots, ch,
+            float(beta), float(temp), W, H, TW, TH, float(threshold), pairs, _ptr(workspace), nbytes, _ptr(rgb),
+            _ptr(alpha), _ptr(feat), _ptr(status), _stream(dev))
+        _check(code, "mlpsp_render_tilecenter_feat_f32")
+        if pool < 0 or int(status.item()) == 0:
+            break
     return rgb, alpha, feat
 
 
@@ -279,16 +297,23 @@ def render_tilecenter_mfma_feat(rays_o, rays_d, records, order, tile_offsets, fr
     lib = _lib.load()
     B = W * H
     pairs = int(order.numel())
-    ws_bytes = lib.mlpsp_mfma_feat_workspace_bytes(pairs, W, H, slots)
-    workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
     rgb = torch.empty(B, 3, dtype=torch.float32, device=dev)
     alpha = torch.empty(B, 1, dtype=torch.float32, device=dev)
     feat = torch.empty(B, ch, dtype=torch.float32, device=dev)
     flag = torch.empty(16, dtype=torch.int32, device=dev)
-    code = lib.mlpsp_render_tilecenter_mfma_feat(
-        _ptr(rays_o), _ptr(rays_d), _ptr(records), _ptr(order), _ptr(tile_offsets), pairs, _ptr(freq), _ptr(att),
-        _ptr(packed), W1.shape[0], int(bool(bf16)), _ptr(packed_feat), slots, ch, float(beta), float(temp), W, H,
-        float(threshold), _ptr(workspace), ws_bytes, _ptr(rgb), _ptr(alpha), _ptr(feat), _ptr(flag), None,
-        _stream(dev))
+    for pool in _feat_pool_sizes(pairs):
+        ws_bytes = lib.mlpsp_feat_workspace_bytes(pairs, W, H, 8, 8, slots, 1, pool)
+        workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+        code = lib.mlpsp_render_tilecenter_mfma_feat(
+            _ptr(rays_o), _ptr(rays_d), _ptr(records), _ptr(order), _ptr(tile_offsets), pairs, _ptr(freq), _ptr(att),
+            _ptr(packed), W1.shape[0], int(bool(bf16)), _ptr(packed_feat), slots, ch, float(beta), float(temp), W, H,
+            float(threshold), _ptr(workspace), ws_bytes, _ptr(rgb), _ptr(alpha), _ptr(feat), _ptr(flag), None,
+            _stream(dev))
+        _check(code, "mlpsp_render_tilecenter_mfma_feat")
+        if pool < 0:
+            break
+        host_flag = flag[:2].tolist()               # one read-back: [non-finite, pool ran out]
+        if host_flag[1] == 0:
+            return rgb, alpha, feat, (bool(host_flag[0]) if check else flag)
     _check(code, "mlpsp_render_tilecenter_mfma_feat")
     return rgb, alpha, feat, (bool(flag[0].item()) if check else flag)
