@@ -151,6 +151,14 @@ __device__ __forceinline__ float relu(float x) {
   asm("v_max_f32_e32 %0, 0, %1" : "=v"(y) : "v"(x));
   return y;
 }
+// ReLU of two packed 16-bit floats in one instruction: as signed 16-bit integers every negative float
+// (and -0) is below zero and every non-negative one keeps its bits, for bf16 and fp16 alike; rounding
+// commutes with ReLU, so rounding first gives the same operand.
+__device__ __forceinline__ unsigned relu_packed(unsigned x) {
+  unsigned y;
+  asm("v_pk_max_i16 %0, %1, 0" : "=v"(y) : "v"(x));
+  return y;
+}
 __device__ __forceinline__ float max3_abs(float a, float b, float c) {
   float y;
   asm("v_max3_f32 %0, |%1|, |%2|, |%3|" : "=v"(y) : "v"(a), "v"(b), "v"(c));
@@ -323,7 +331,7 @@ __global__ __launch_bounds__(64) void render_tilecenter_mfma_kernel(
             u32x4 bw;
 #pragma unroll
             for (int d = 0; d < 4; ++d)
-              bw[d] = Ops<T>::pack2(relu(d1[8 * s + 2 * d]), relu(d1[8 * s + 2 * d + 1]));
+              bw[d] = relu_packed(Ops<T>::pack2(d1[8 * s + 2 * d], d1[8 * s + 2 * d + 1]));
             d2 = Ops<T>::mfma(a2[s], bw, d2);
           }
           bad |= col_active && out_of_range_in<T>(d2);
@@ -334,7 +342,7 @@ __global__ __launch_bounds__(64) void render_tilecenter_mfma_kernel(
             u32x4 bw;
 #pragma unroll
             for (int d = 0; d < 4; ++d)
-              bw[d] = Ops<T>::pack2(relu(d2[8 * s + 2 * d]), relu(d2[8 * s + 2 * d + 1]));
+              bw[d] = relu_packed(Ops<T>::pack2(d2[8 * s + 2 * d], d2[8 * s + 2 * d + 1]));
             d3 = Ops<T>::mfma(a3[s], bw, d3);
           }
 #pragma unroll
