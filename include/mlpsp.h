@@ -76,7 +76,8 @@ int mlpsp_validate_tile_lists(const int32_t* tile_offsets_dev, const int32_t* ca
  * t uses view tile_view_ids_dev[t]).  view_matrices: K row-major 4x4 on the HOST, proj: 4x4 on
  * the host.  Within a tile, candidate ids ascend.
  * Step 1 (count): writes exclusive offsets to tile_offsets_dev[T+1]; BLOCKS to return the total
- *   in *num_pairs_out.  scratch_dev: at least mlpsp_bin_scratch_bytes() bytes, 256-byte aligned,
+ *   in counts_out[0] and the length of the longest tile list in counts_out[1] (what the capacity
+ *   check of the render entry points compares with MLPSP_MAX_TILE_PRIMS).  scratch_dev: at least mlpsp_bin_scratch_bytes() bytes, 256-byte aligned,
  *   reused by step 2; MLPSP_E_SCRATCH asks for a larger one (primitives spanning very many tiles).
  * Step 2 (fill): writes candidates_dev[num_pairs]. */
 size_t mlpsp_bin_scratch_bytes(int num_primitives, int num_views, int width, int height, int tile);
@@ -84,7 +85,7 @@ int mlpsp_bin_legacy_count(const float* positions_dev, const float* log_scales_d
                            const float* view_matrices_host, int num_views, const int32_t* tile_view_ids_dev,
                            const float* proj_host, int width, int height, int tile, float threshold,
                            void* scratch_dev, size_t scratch_bytes, int32_t* tile_offsets_dev,
-                           int64_t* num_pairs_out, mlpsp_stream_t stream);
+                           int64_t counts_out[2], mlpsp_stream_t stream);
 int mlpsp_bin_legacy_fill(int num_primitives, int num_views, const int32_t* tile_view_ids_dev, int width,
                           int height, int tile, const void* scratch_dev, size_t scratch_bytes,
                           const int32_t* tile_offsets_dev, int32_t* candidates_dev, mlpsp_stream_t stream);

@@ -27,7 +27,7 @@ struct BinScratch {
   float* mats;        // K view matrices (16 floats each) then the projection (16 floats)
   float4* bounds;     // [K][N] (minx, maxx, miny, maxy); all NaN when behind the near plane
   int32_t* l1_counts; // [S*NC + 1] counts, then exclusive offsets after the scan
-  long long* totals;  // [0] level-1 entries, [1] tile-list entries
+  long long* totals;  // [0] level-1 entries, [1] tile-list entries, [2] longest tile list
   int32_t* l1_list;   // [l1_capacity]
   long long l1_capacity;
 };
@@ -144,15 +144,25 @@ __global__ __launch_bounds__(kBinThreads) void bin_level1_kernel(const float4* _
   if (!FILL && threadIdx.x == 0) l1_counts[s * g.NC + c] = running;
 }
 
-// In-place exclusive scan of data[0..n) by one workgroup; data[n] and *total receive the sum.
+// In-place exclusive scan of data[0..n) by one workgroup; data[n] and *total receive the sum, *largest
+// (if not null) the largest element.
 __global__ __launch_bounds__(1024) void exclusive_scan_kernel(int32_t* __restrict__ data, int n,
-                                                              long long* __restrict__ total) {
+                                                              long long* __restrict__ total,
+                                                              long long* __restrict__ largest) {
   __shared__ long long s_part[1024];
+  __shared__ int s_max;
   const int t = threadIdx.x;
+  if (t == 0) s_max = 0;
+  __syncthreads();
   const int per = (n + 1023) / 1024;
   const int lo = min(t * per, n), hi = min(lo + per, n);
   long long sum = 0;
-  for (int i = lo; i < hi; ++i) sum += data[i];
+  int mx = 0;
+  for (int i = lo; i < hi; ++i) {
+    sum += data[i];
+    mx = max(mx, data[i]);
+  }
+  if (largest && mx > 0) atomicMax(&s_max, mx);
   s_part[t] = sum;
   __syncthreads();
   for (int d = 1; d < 1024; d <<= 1) {
@@ -170,6 +180,7 @@ __global__ __launch_bounds__(1024) void exclusive_scan_kernel(int32_t* __restric
   if (t == 1023) {
     data[n] = (int32_t)s_part[1023];
     *total = s_part[1023];
+    if (largest) *largest = s_max;
   }
 }
 
@@ -239,10 +250,10 @@ MLPSP_API int mlpsp_bin_legacy_count(const float* positions_dev, const float* lo
                                      const float* view_matrices_host, int num_views,
                                      const int32_t* tile_view_ids_dev, const float* proj_host, int width, int height,
                                      int tile, float threshold, void* scratch_dev, size_t scratch_bytes,
-                                     int32_t* tile_offsets_dev, int64_t* num_pairs_out, mlpsp_stream_t stream) {
+                                     int32_t* tile_offsets_dev, int64_t counts_out[2], mlpsp_stream_t stream) {
   const int64_t T = checked_num_tiles(width, height, tile, tile);
   if (T <= 0 || num_primitives < 0 || num_views <= 0 || !view_matrices_host || !proj_host || !scratch_dev ||
-      !tile_offsets_dev || !num_pairs_out)
+      !tile_offsets_dev || !counts_out)
     return MLPSP_E_ARGUMENT;
   if (!(threshold > 0.f && threshold < 1.f)) return MLPSP_E_ARGUMENT;
   if (scratch_bytes < mlpsp_bin_scratch_bytes(num_primitives, num_views, width, height, tile)) return MLPSP_E_SCRATCH;
@@ -250,10 +261,10 @@ MLPSP_API int mlpsp_bin_legacy_count(const float* positions_dev, const float* lo
   const BinGeom g = make_geom(num_primitives, num_views, width, height, tile);
   const int S = g.nsx * g.nsy;
   const BinScratch b = carve(scratch_dev, scratch_bytes, num_primitives, num_views, S, g.NC);
-  *num_pairs_out = 0;
+  counts_out[0] = counts_out[1] = 0;
   if (num_primitives == 0) {
     MLPSP_HIP_TRY(hipMemsetAsync(tile_offsets_dev, 0, (size_t)(T + 1) * sizeof(int32_t), s));
-    MLPSP_HIP_TRY(hipMemsetAsync(b.totals, 0, 2 * sizeof(long long), s));
+    MLPSP_HIP_TRY(hipMemsetAsync(b.totals, 0, 3 * sizeof(long long), s));
     return MLPSP_OK;
   }
   // scalar constants in f32, in the order the reference's tensor expressions evaluate them
@@ -269,7 +280,8 @@ MLPSP_API int mlpsp_bin_legacy_count(const float* positions_dev, const float* lo
   hipLaunchKernelGGL((bin_level1_kernel<false>), dim3(g.NC, S), dim3(kBinThreads), 0, s, b.bounds, g, b.l1_counts,
                      b.l1_list, b.l1_capacity);
   MLPSP_LAUNCH_CHECK();
-  hipLaunchKernelGGL(exclusive_scan_kernel, dim3(1), dim3(1024), 0, s, b.l1_counts, S * g.NC, b.totals);
+  hipLaunchKernelGGL(exclusive_scan_kernel, dim3(1), dim3(1024), 0, s, b.l1_counts, S * g.NC, b.totals,
+                     (long long*)nullptr);
   MLPSP_LAUNCH_CHECK();
   hipLaunchKernelGGL((bin_level1_kernel<true>), dim3(g.NC, S), dim3(kBinThreads), 0, s, b.bounds, g, b.l1_counts,
                      b.l1_list, b.l1_capacity);
@@ -278,15 +290,17 @@ MLPSP_API int mlpsp_bin_legacy_count(const float* positions_dev, const float* lo
                      b.bounds, g, tile_view_ids_dev, b.l1_counts, b.l1_list, b.l1_capacity, tile_offsets_dev,
                      (int32_t*)nullptr);
   MLPSP_LAUNCH_CHECK();
-  hipLaunchKernelGGL(exclusive_scan_kernel, dim3(1), dim3(1024), 0, s, tile_offsets_dev, (int)T, b.totals + 1);
+  hipLaunchKernelGGL(exclusive_scan_kernel, dim3(1), dim3(1024), 0, s, tile_offsets_dev, (int)T, b.totals + 1,
+                     b.totals + 2);
   MLPSP_LAUNCH_CHECK();
   // one blocking readback: level-1 entry count (overflow check) and the number of pairs
-  long long totals[2] = {0, 0};
-  MLPSP_HIP_TRY(hipMemcpyAsync(totals, b.totals, 2 * sizeof(long long), hipMemcpyDeviceToHost, s));
+  long long totals[3] = {0, 0, 0};
+  MLPSP_HIP_TRY(hipMemcpyAsync(totals, b.totals, 3 * sizeof(long long), hipMemcpyDeviceToHost, s));
   MLPSP_HIP_TRY(hipStreamSynchronize(s));
   if (totals[0] > b.l1_capacity) return MLPSP_E_SCRATCH;
   if (totals[1] > 2147483647LL) return MLPSP_E_ARGUMENT;
-  *num_pairs_out = totals[1];
+  counts_out[0] = totals[1];
+  counts_out[1] = totals[2];
   return MLPSP_OK;
 }
 

@@ -289,8 +289,14 @@ class NeuralPrimitiveSceneTileCUDA(nn.Module):
     def _legacy_culling(self, view_matrices, proj_matrix, score_threshold, tile_size, tile_view_ids=None):
         """Screen-space tile lists: same rule as scannet/cumodel.py:994-1070, evaluated sparsely on the GPU."""
         W, H = self.image_size
-        return ops.bin_legacy(self.positions.detach(), self.log_scales.detach(), view_matrices, proj_matrix, W, H,
-                              int(tile_size), float(score_threshold), tile_view_ids)
+        cand, offsets, longest = ops.bin_legacy(self.positions.detach(), self.log_scales.detach(), view_matrices,
+                                                proj_matrix, W, H, int(tile_size), float(score_threshold),
+                                                tile_view_ids, with_longest=True)
+        # lists fresh from the binning kernels need no second validation pass on the device
+        note = getattr(self._ensure_tile_ext(), "note_binned_lists", None)
+        if note is not None:
+            note(cand, offsets, longest, self.positions.shape[0])
+        return cand, offsets
 
     @torch.no_grad()
     def build_tilecenter_culling_from_tile_views(self, tile_view_ids, view_matrices, proj_matrix,

@@ -75,11 +75,12 @@ def validate_tile_lists(candidates, tile_offsets, n_tiles: int, capacity: int, n
 
 
 def bin_legacy(positions, log_scales, view_matrices, proj_matrix, W: int, H: int, tile: int, threshold: float,
-               tile_view_ids=None):
+               tile_view_ids=None, with_longest=False):
     """Sparse form of the reference's screen-space culling (scannet/cumodel.py:994-1070, 838-949).
 
     view_matrices [K,4,4] / proj_matrix [4,4] may live on any device (they are read on the host).
     Returns (culled_prim_indices int32 [P], tile_offsets int32 [T+1]); ids ascend inside a tile.
+    ``with_longest`` appends the length of the longest tile list (known from the same read-back).
     """
     positions, log_scales = _f32c(positions, "positions"), _f32c(log_scales, "log_scales")
     dev = positions.device
@@ -93,24 +94,30 @@ def bin_legacy(positions, log_scales, view_matrices, proj_matrix, W: int, H: int
         if tv.numel() != T:
             raise ValueError(f"tile_view_ids length mismatch: got {tv.numel()}, expected {T}")
     lib = _lib.load()
-    offsets = torch.empty(T + 1, dtype=torch.int32, device=dev)
+    # ordinary (version-counted) tensors even under torch.inference_mode(): a later in-place edit of the
+    # lists must be detectable by whoever skips re-validating them
+    with torch.inference_mode(False):
+        offsets = torch.empty(T + 1, dtype=torch.int32, device=dev)
     fp = C.POINTER(C.c_float)
     nbytes = lib.mlpsp_bin_scratch_bytes(n, K, W, H, tile)
-    total = C.c_int64(0)
+    counts = (C.c_int64 * 2)()
     for _ in range(6):
         scratch = torch.empty(nbytes, dtype=torch.uint8, device=dev)
         code = lib.mlpsp_bin_legacy_count(_ptr(positions), _ptr(log_scales), n, C.cast(vm.data_ptr(), fp), K, _ptr(tv),
                                           C.cast(pm.data_ptr(), fp), W, H, tile, float(threshold), _ptr(scratch),
-                                          nbytes, _ptr(offsets), C.byref(total), _stream(dev))
+                                          nbytes, _ptr(offsets), counts, _stream(dev))
         if code != _lib.E_SCRATCH:
             break
         nbytes *= 4
     _check(code, "mlpsp_bin_legacy_count")
-    cand = torch.empty(int(total.value), dtype=torch.int32, device=dev)
-    if total.value > 0:
+    with torch.inference_mode(False):
+        cand = torch.empty(int(counts[0]), dtype=torch.int32, device=dev)
+    if counts[0] > 0:
         code = lib.mlpsp_bin_legacy_fill(n, K, _ptr(tv), W, H, tile, _ptr(scratch), nbytes, _ptr(offsets), _ptr(cand),
                                          _stream(dev))
         _check(code, "mlpsp_bin_legacy_fill")
+    if with_longest:
+        return cand, offsets, int(counts[1])
     return cand, offsets
 
 

@@ -50,6 +50,7 @@ class TileExt:
         self._pack_key = None
         self._pack = None
         self._feat_pack_key = None
+        self._binned = None
         self._feat_pack = None
 
     def __getattr__(self, name):
@@ -62,6 +63,40 @@ class TileExt:
     # ------------------------------------------------------------------------------------------
     # shared argument checks (np_tile_kernels.cu:5242-5275)
     # ------------------------------------------------------------------------------------------
+    # ------------------------------------------------------------------------------------------
+    # tile-list validation
+    # ------------------------------------------------------------------------------------------
+    @staticmethod
+    def _list_key(cand, offsets, n):
+        try:
+            versions = (cand._version, offsets._version)
+        except RuntimeError:          # inference tensors carry no version counter: an edit could not be seen
+            return None
+        return (cand.data_ptr(), cand.numel(), offsets.data_ptr(), offsets.numel(), versions, str(cand.device), int(n))
+
+    def note_binned_lists(self, cand, offsets, longest, num_primitives):
+        """Tile lists that this library's own binning kernels have just written are well-formed by
+        construction (offsets monotonic and covering the list, ids in range); ``longest`` is the length
+        of their longest tile list, which the binning read back together with the pair count.  The next
+        render call that receives these very tensors, unmodified, checks the capacity against
+        ``longest`` on the host instead of running the device validation pass with its blocking
+        read-back (np_tile_kernels.cu:4553-4588).  Anything else is validated on the device."""
+        key = self._list_key(cand, offsets, num_primitives)
+        with self._lock:
+            self._binned = None if key is None else (key, int(longest))
+
+    def _validate(self, cand, offsets, n_tiles, capacity, n, name):
+        with self._lock:
+            binned = self._binned
+        if (binned is not None and cand.is_cuda and offsets.is_cuda and cand.dtype == torch.int32
+                and offsets.dtype == torch.int32 and offsets.numel() == n_tiles + 1
+                and binned[0] == self._list_key(cand, offsets, n)):   # (a None key never matches)
+            if capacity > 0 and binned[1] > capacity:
+                raise RuntimeError(f"{name}: tile candidate capacity {capacity} exceeded (maximum observed tile length "
+                                   f"{binned[1]}); refusing to truncate or use an inconsistent forward/backward order")
+            return
+        ops.validate_tile_lists(cand, offsets, n_tiles, capacity, n, name)
+
     @staticmethod
     def _check_base(rays_o, rays_d, positions, log_scales, quats, cand, offsets, freq, att):
         _chk(_is_f32_2d(rays_o, 3), "rays_o must be a CUDA float32 [B,3] tensor")
@@ -100,7 +135,7 @@ class TileExt:
         cand = cand.contiguous()
         offsets = offsets.contiguous()
         with torch.cuda.device(rays_o.device):
-            ops.validate_tile_lists(cand, offsets, n_tiles, capacity, positions.shape[0], name)
+            self._validate(cand, offsets, n_tiles, capacity, positions.shape[0], name)
         F = freq.shape[0]
         _chk(W1.shape[2] == 6 * F * 2, "Encoded dim must be 6*F*2")
         _chk(W2.shape[1] <= hidden_limit, f"{name} currently supports hidden_dim <= {hidden_limit}")
@@ -282,7 +317,7 @@ class TileExt:
         _chk(tuple(x[11].shape) == (n, 32, 32) and x[12].shape == x[10].shape)
         _chk(tuple(x[13].shape) == (n, 4, 32) and tuple(x[14].shape) == (n, 4))
         with torch.cuda.device(x[0].device):
-            ops.validate_tile_lists(x[5], x[6], ops.num_tiles(width, height, 8, 8), self.max_tile_prims, n, name)
+            self._validate(x[5], x[6], ops.num_tiles(width, height, 8, 8), self.max_tile_prims, n, name)
             with self._lock:
                 self._mfma_calls += 1
             rec = ops.prepare_primitives(x[2], x[3], x[4])

@@ -144,3 +144,40 @@ def test_native_camera_mode_uses_ray_cone_lists(device, oracle_mod):
     scene.camera_mode = "colmap-native"
     with pytest.raises(ValueError, match="derived from the actual rays"):
         _call(scene, fr, device, culled_prim_indices=every, tile_offsets=offs)
+
+
+def test_lists_from_the_own_binning_skip_device_validation_but_keep_the_capacity_check(device, oracle_mod, monkeypatch):
+    from mlp_splatting_amd import cumodel, ops
+    from mlp_splatting_amd.tile_ext import TileExt
+    fr = Frame("cfg1_5k_160x120", n=1500, hidden=32, width=64, height=48)
+    scene = _scene_from(fr, device)
+    ref = _call(scene, fr, device)
+    calls = []
+    real = ops.validate_tile_lists
+    monkeypatch.setattr(ops, "validate_tile_lists", lambda *a, **k: (calls.append(a[-1]), real(*a, **k))[1])
+    for precision in ("f32", "bf16"):
+        scene.render_precision = precision
+        out = _call(scene, fr, device)
+        assert precision == "bf16" or torch.equal(out, ref)
+    assert calls == []                                   # no device pass for lists the binning just wrote
+    scene.render_precision = "f32"
+    # the same lists handed in by the caller are validated on the device, as the reference does
+    cand, off = fr.oracle_lists(oracle_mod)
+    ext_lists = dict(culled_prim_indices=to_dev(cand, device), tile_offsets=to_dev(off, device))
+    assert torch.equal(_call(scene, fr, device, **ext_lists), ref) and len(calls) == 1
+    # ... and a list edited after the binning noted it is validated again (and rejected)
+    ext = cumodel.NeuralPrimitiveSceneTileCUDA._ensure_tile_ext_static()
+    c, o, longest = ops.bin_legacy(to_dev(fr.scene.positions, device), to_dev(fr.scene.log_scales, device),
+                                   torch.from_numpy(fr.view[None]), torch.from_numpy(fr.proj), fr.W, fr.H, 8, fr.thr,
+                                   with_longest=True)
+    assert longest == int(np.diff(off).max())
+    ext.note_binned_lists(c, o, longest, fr.scene.n)
+    c[0] = fr.scene.n + 5
+    with pytest.raises(RuntimeError, match="candidate primitive IDs must be in"):
+        _call(scene, fr, device, culled_prim_indices=c, tile_offsets=o)
+    # the capacity check needs no device pass: it uses the longest list the binning reported
+    monkeypatch.setattr(cumodel, "_tile_ext", TileExt(max_tile_prims=longest - 1))
+    with pytest.raises(RuntimeError, match=f"capacity {longest - 1} exceeded \\(maximum observed tile length {longest}\\)"):
+        _call(scene, fr, device)
+    monkeypatch.setattr(cumodel, "_tile_ext", TileExt(max_tile_prims=longest))
+    assert torch.equal(_call(scene, fr, device), ref)
