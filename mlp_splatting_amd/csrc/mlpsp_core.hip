@@ -85,8 +85,9 @@ __global__ __launch_bounds__(256) void validate_tile_lists_kernel(const int32_t*
 // lies entirely beyond one of the pyramid's four faces can be hit by no ray of the tile.  For a face
 // with inward normal n through the common origin o that is  n.(c-o) < 0  and
 // (n.(c-o))^2 >= -2 ln thr * sum_k s_k^2 (R^T n)_k^2, tested with a 2 % margin on the radius, far
-// above f32 rounding.  Such an entry is written as ~id (negative): the render kernels skip negative
-// ids, so the image is unchanged bit for bit, and ~ recovers the exact sorted list.
+// above f32 rounding.  Such an entry is written as ~id (negative) AFTER the tile's sorted survivors, in
+// list order: the render kernels skip negative ids, so the image is unchanged bit for bit, and only the
+// survivors go through the sorting network.
 // ---------------------------------------------------------------------------------------------
 constexpr int kSortThreads = 256;
 constexpr int kSortMax = MLPSP_TILE_CAPACITY_MAX;
@@ -103,6 +104,8 @@ __global__ __launch_bounds__(kSortThreads) void sort_tiles_kernel(
     float cull_r2, int32_t* __restrict__ sorted_ids, float* __restrict__ sorted_keys) {
   __shared__ unsigned long long s_key[kSortMax];
   __shared__ int32_t s_id[kSortMax];
+  __shared__ int32_t s_cull[kSortMax];
+  __shared__ int s_wave_cnt[kSortThreads / 64];
   __shared__ TilePyramid s_pyr;
   __shared__ int s_face_ok[4];
   __shared__ int s_origin_ok;
@@ -116,9 +119,6 @@ __global__ __launch_bounds__(kSortThreads) void sort_tiles_kernel(
   const int pc = centre_pixel(g, tile);
   const float ox = rays_o[pc * 3 + 0], oy = rays_o[pc * 3 + 1], oz = rays_o[pc * 3 + 2];
   const float dx = rays_d[pc * 3 + 0], dy = rays_d[pc * 3 + 1], dz = rays_d[pc * 3 + 2];
-
-  int npad = 2;
-  while (npad < n) npad <<= 1;
 
   // ---- the tile's ray pyramid (only when culling is requested)
   const bool culling = cull_r2 > 0.f;
@@ -173,14 +173,20 @@ __global__ __launch_bounds__(kSortThreads) void sort_tiles_kernel(
   }
   const int faces = culling ? s_pyr.enabled : 0;
 
-  for (int i = tid; i < npad; i += kSortThreads) {
-    unsigned long long w = ~0ull;
+  // ---- keys; survivors are compacted to the front of s_key (the network then sorts only them),
+  //      culled entries go to s_cull in list order and are appended after the sorted survivors
+  const int wave = tid >> 6, lane = tid & 63;
+  int ns = 0;                                            // survivors so far (block-uniform)
+  for (int i0 = 0; i0 < n; i0 += kSortThreads) {
+    const int i = i0 + tid;
+    bool keep = false, outside = false;
+    int p = 0;
+    float key = 0.f;
     if (i < n) {
-      int p = cand[start + i];
+      p = cand[start + i];
       const PrimRecord P = prims[p];
       if (faces) {
         const float ex = P.cx - s_pyr.ox, ey = P.cy - s_pyr.oy, ez = P.cz - s_pyr.oz;
-        bool outside = false;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           const float nx = s_pyr.n[j][0], ny = s_pyr.n[j][1], nz = s_pyr.n[j][2];
@@ -189,15 +195,31 @@ __global__ __launch_bounds__(kSortThreads) void sort_tiles_kernel(
           const float h2 = P.s2x * (nl.x * nl.x) + P.s2y * (nl.y * nl.y) + P.s2z * (nl.z * nl.z);
           outside |= ((faces >> j) & 1) && (dist < 0.f) && (dist * dist >= cull_r2 * h2);
         }
-        if (outside) p = ~p;
       }
+      keep = !outside;
       s_id[i] = p;
-      const float key = (family == MLPSP_KEY_DEPTH) ? key_depth(ox, oy, oz, dx, dy, dz, P)
-                                                    : key_tstar(ox, oy, oz, dx, dy, dz, P);
-      w = ((unsigned long long)float_to_bits(key) << 32) | (unsigned)i;
+      if (keep)
+        key = (family == MLPSP_KEY_DEPTH) ? key_depth(ox, oy, oz, dx, dy, dz, P) : key_tstar(ox, oy, oz, dx, dy, dz, P);
     }
-    s_key[i] = w;
+    const unsigned long long m = __ballot(keep);
+    if (lane == 0) s_wave_cnt[wave] = __popcll(m);
+    __syncthreads();
+    int before = 0, total = 0;
+#pragma unroll
+    for (int v = 0; v < kSortThreads / 64; ++v) {
+      const int c = s_wave_cnt[v];
+      before += (v < wave) ? c : 0;
+      total += c;
+    }
+    const int kept_before = ns + before + __popcll(m & ((1ull << lane) - 1ull));
+    if (keep) s_key[kept_before] = ((unsigned long long)float_to_bits(key) << 32) | (unsigned)i;
+    else if (i < n) s_cull[i - kept_before] = ~p;
+    ns += total;
+    __syncthreads();
   }
+  int npad = 2;
+  while (npad < ns) npad <<= 1;
+  for (int i = ns + tid; i < npad; i += kSortThreads) s_key[i] = ~0ull;
   __syncthreads();
 
   for (int k = 2; k <= npad; k <<= 1) {
@@ -217,12 +239,15 @@ __global__ __launch_bounds__(kSortThreads) void sort_tiles_kernel(
   }
 
   for (int i = tid; i < len; i += kSortThreads) {
-    if (i < n) {
+    if (i < ns) {
       const unsigned long long w = s_key[i];
       sorted_ids[start + i] = s_id[(int)(w & 0xffffffffu)];
       if (sorted_keys) sorted_keys[start + i] = bits_to_float((uint32_t)(w >> 32));
+    } else if (i < n) {
+      sorted_ids[start + i] = s_cull[i - ns];      // culled: ~id, list order, after every survivor
+      if (sorted_keys) sorted_keys[start + i] = kInvalidKey;
     } else {
-      sorted_ids[start + i] = cand[start + i];   // beyond the sort capacity: list order, never culled
+      sorted_ids[start + i] = cand[start + i];     // beyond the sort capacity: list order, never culled
       if (sorted_keys) sorted_keys[start + i] = kInvalidKey;
     }
   }

@@ -127,7 +127,11 @@ def test_cfg3_order_properties_over_poses(cfg3):
         # culling never changes the image, and alpha stays in [0, 1]
         ids_c, _ = ops.sort_tiles(fr["ro_t"], fr["rd_t"], b.rec, fr["cand"], off, b.W, b.H, 8, 8, cull_threshold=b.thr)
         assert 0.2 < float((ids_c < 0).float().mean()) < 0.7
-        assert torch.equal(torch.where(ids_c < 0, ~ids_c, ids_c), ids)
+        # survivors keep their sorted order; the culled ids follow them
+        comp_c = tile_of.long() * (b.sc.n + 1) + torch.where(ids_c < 0, ~ids_c, ids_c).long()
+        assert torch.equal(torch.sort(comp_c).values, torch.sort(composite).values)
+        kept = ~torch.isin(composite, comp_c[ids_c < 0])
+        assert torch.equal(composite[kept], comp_c[ids_c >= 0])
         a = ops.render_tilecenter_mfma(fr["ro_t"], fr["rd_t"], b.rec, ids, off, b.freq, b.att, *b.ws, b.W, b.H, b.thr)
         c = ops.render_tilecenter_mfma(fr["ro_t"], fr["rd_t"], b.rec, ids_c, off, b.freq, b.att, *b.ws, b.W, b.H, b.thr)
         assert torch.equal(a[0], c[0]) and torch.equal(a[1], c[1])
