@@ -86,7 +86,7 @@ __global__ __launch_bounds__(256) void validate_tile_lists_kernel(const int32_t*
 // with inward normal n through the common origin o that is  n.(c-o) < 0  and
 // (n.(c-o))^2 >= -2 ln thr * sum_k s_k^2 (R^T n)_k^2, tested with a 2 % margin on the radius, far
 // above f32 rounding.  Such an entry is written as ~id (negative) AFTER the tile's sorted survivors, in
-// list order: the render kernels skip negative ids, so the image is unchanged bit for bit, and only the
+// reverse list order: the render kernels skip negative ids, so the image is unchanged bit for bit, and only the
 // survivors go through the sorting network.
 // ---------------------------------------------------------------------------------------------
 constexpr int kSortThreads = 256;
@@ -103,9 +103,7 @@ __global__ __launch_bounds__(kSortThreads) void sort_tiles_kernel(
     const int32_t* __restrict__ cand, const int32_t* __restrict__ offsets, TileGeom g, int family, int capacity,
     float cull_r2, int32_t* __restrict__ sorted_ids, float* __restrict__ sorted_keys) {
   __shared__ unsigned long long s_key[kSortMax];
-  __shared__ int32_t s_id[kSortMax];
-  __shared__ int32_t s_cull[kSortMax];
-  __shared__ int s_wave_cnt[kSortThreads / 64];
+  __shared__ int s_wave_cnt[2][kSortThreads / 64];
   __shared__ TilePyramid s_pyr;
   __shared__ int s_face_ok[4];
   __shared__ int s_origin_ok;
@@ -174,10 +172,11 @@ __global__ __launch_bounds__(kSortThreads) void sort_tiles_kernel(
   const int faces = culling ? s_pyr.enabled : 0;
 
   // ---- keys; survivors are compacted to the front of s_key (the network then sorts only them),
-  //      culled entries go to s_cull in list order and are appended after the sorted survivors
+  //      culled entries are written straight to the end of the tile's output, last one first
   const int wave = tid >> 6, lane = tid & 63;
   int ns = 0;                                            // survivors so far (block-uniform)
-  for (int i0 = 0; i0 < n; i0 += kSortThreads) {
+  int round = 0;
+  for (int i0 = 0; i0 < n; i0 += kSortThreads, round ^= 1) {
     const int i = i0 + tid;
     bool keep = false, outside = false;
     int p = 0;
@@ -197,33 +196,48 @@ __global__ __launch_bounds__(kSortThreads) void sort_tiles_kernel(
         }
       }
       keep = !outside;
-      s_id[i] = p;
       if (keep)
         key = (family == MLPSP_KEY_DEPTH) ? key_depth(ox, oy, oz, dx, dy, dz, P) : key_tstar(ox, oy, oz, dx, dy, dz, P);
     }
     const unsigned long long m = __ballot(keep);
-    if (lane == 0) s_wave_cnt[wave] = __popcll(m);
-    __syncthreads();
+    if (lane == 0) s_wave_cnt[round][wave] = __popcll(m);
+    __syncthreads();                                     // (the two count buffers alternate: one barrier per round)
     int before = 0, total = 0;
 #pragma unroll
     for (int v = 0; v < kSortThreads / 64; ++v) {
-      const int c = s_wave_cnt[v];
+      const int c = s_wave_cnt[round][v];
       before += (v < wave) ? c : 0;
       total += c;
     }
     const int kept_before = ns + before + __popcll(m & ((1ull << lane) - 1ull));
-    if (keep) s_key[kept_before] = ((unsigned long long)float_to_bits(key) << 32) | (unsigned)i;
-    else if (i < n) s_cull[i - kept_before] = ~p;
+    if (keep) {
+      s_key[kept_before] = ((unsigned long long)float_to_bits(key) << 32) | (unsigned)i;
+    } else if (i < n) {
+      const int pos = start + n - 1 - (i - kept_before);
+      sorted_ids[pos] = ~p;
+      if (sorted_keys) sorted_keys[pos] = kInvalidKey;
+    }
     ns += total;
-    __syncthreads();
   }
   int npad = 2;
   while (npad < ns) npad <<= 1;
   for (int i = ns + tid; i < npad; i += kSortThreads) s_key[i] = ~0ull;
   __syncthreads();
 
+  // ---- bitonic network.  Thread t of a step handles the pair (lo, lo | j) with lo built from t, so for
+  //      j < 64 the 64 lanes of a wavefront touch only their own 128 consecutive entries: those steps
+  //      need no workgroup barrier, only program order inside the wavefront (LDS operations of one
+  //      wavefront complete in order).  A workgroup barrier separates any step with j >= 64 from its
+  //      neighbours.
+  int prev_j = 64;
   for (int k = 2; k <= npad; k <<= 1) {
     for (int j = k >> 1; j > 0; j >>= 1) {
+      if (j >= 64 || prev_j >= 64) __syncthreads();
+      else {
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+      }
+      prev_j = j;
       for (int t = tid; t < (npad >> 1); t += kSortThreads) {
         const int lo = ((t & ~(j - 1)) << 1) | (t & (j - 1));
         const int hi = lo | j;
@@ -234,19 +248,16 @@ __global__ __launch_bounds__(kSortThreads) void sort_tiles_kernel(
           s_key[hi] = a;
         }
       }
-      __syncthreads();
     }
   }
+  __syncthreads();
 
   for (int i = tid; i < len; i += kSortThreads) {
     if (i < ns) {
       const unsigned long long w = s_key[i];
-      sorted_ids[start + i] = s_id[(int)(w & 0xffffffffu)];
+      sorted_ids[start + i] = cand[start + (int)(w & 0xffffffffu)];
       if (sorted_keys) sorted_keys[start + i] = bits_to_float((uint32_t)(w >> 32));
-    } else if (i < n) {
-      sorted_ids[start + i] = s_cull[i - ns];      // culled: ~id, list order, after every survivor
-      if (sorted_keys) sorted_keys[start + i] = kInvalidKey;
-    } else {
+    } else if (i >= n) {
       sorted_ids[start + i] = cand[start + i];     // beyond the sort capacity: list order, never culled
       if (sorted_keys) sorted_keys[start + i] = kInvalidKey;
     }
@@ -325,6 +336,7 @@ MLPSP_API int mlpsp_sort_tiles(const float* rays_o_dev, const float* rays_d_dev,
   if (capacity < 0 || capacity > MLPSP_TILE_CAPACITY_MAX) return MLPSP_E_ARGUMENT;
   if (capacity == 0) capacity = MLPSP_TILE_CAPACITY_MAX;
   if (!rays_o_dev || !rays_d_dev || !tile_offsets_dev) return MLPSP_E_ARGUMENT;
+  if (sorted_ids_dev && sorted_ids_dev == candidates_dev) return MLPSP_E_ARGUMENT;   // not an in-place sort
   TileGeom g{width, height, tile_w, tile_h, ceil_div(width, tile_w), ceil_div(height, tile_h)};
   // squared radius of the threshold ellipsoid in units of the scales, with a 2 % margin on the radius
   float cull_r2 = 0.f;
