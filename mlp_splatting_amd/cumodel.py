@@ -275,8 +275,31 @@ class NeuralPrimitiveSceneTileCUDA(nn.Module):
         return _tile_ext
 
     # ------------------------------------------------------------------------------------------
+    def _cached(self, name, sources, extra, build):
+        """``build()`` once per state of the ``sources`` tensors (identity, shape, in-place version): the
+        scene is constant while rendering, and every small torch op skipped is a kernel launch less per
+        frame.  The value is built outside inference mode so that it carries a version counter itself."""
+        try:
+            key = tuple((t.data_ptr(), t._version, tuple(t.shape), str(t.device)) for t in sources) + tuple(extra)
+        except RuntimeError:                      # inference tensors have no version counter: do not cache
+            return build()
+        cache = self.__dict__.setdefault("_mlpsp_cache", {})
+        hit = cache.get(name)
+        if hit is None or hit[0] != key:
+            with torch.inference_mode(False), torch.no_grad():
+                hit = (key, build())
+            cache[name] = hit
+        return hit[1]
+
     def _frequency_tables(self, device):
         """freq and att as the kernels take them (scannet/cumodel.py:1078-1086)."""
+        sources = [self.encoder.freq_bands]
+        if hasattr(self.encoder, "runtime_frequency_weights"):
+            sources.append(self.encoder.runtime_frequency_weights)
+        extra = (str(device), float(getattr(self.encoder, "sigma2", 0.0)))
+        return self._cached("frequency_tables", sources, extra, lambda: self._build_frequency_tables(device))
+
+    def _build_frequency_tables(self, device):
         freq = self.encoder.freq_bands.to(device=device, dtype=torch.float32)
         if isinstance(self.encoder, IntegratedPositionalEncoding):
             att = torch.exp(-0.5 * (freq * freq) * float(self.encoder.sigma2))
@@ -347,10 +370,16 @@ class NeuralPrimitiveSceneTileCUDA(nn.Module):
             raise ValueError("Tile renderer requires view_matrix/proj_matrix unless external culling is provided.")
         return self._legacy_culling(view_matrix.reshape(1, 4, 4), proj_matrix, score_threshold, tile_size)
 
-    def _base_args(self, ray_o, ray_d, culled_prim_indices, tile_offsets, device):
+    def _unit_quats(self):
+        return self._cached("unit_quats", [self.quats], (),
+                            lambda: F.normalize(self.quats.detach(), dim=-1).contiguous())
+
+    def _base_args(self, ray_o, ray_d, culled_prim_indices, tile_offsets, device, unit_dirs=None):
         freq, att = self._frequency_tables(device)
-        return (ray_o.contiguous(), F.normalize(ray_d, dim=-1).contiguous(), self.positions.detach().contiguous(),
-                self.log_scales.detach().contiguous(), F.normalize(self.quats.detach(), dim=-1).contiguous(),
+        if unit_dirs is None:
+            unit_dirs = F.normalize(ray_d, dim=-1).contiguous()
+        return (ray_o.contiguous(), unit_dirs, self.positions.detach().contiguous(),
+                self.log_scales.detach().contiguous(), self._unit_quats(),
                 culled_prim_indices, tile_offsets.to(torch.int32), freq, att,
                 self.W1.detach().contiguous(), self.b1.detach().contiguous(), self.W2.detach().contiguous(),
                 self.b2.detach().contiguous(), self.W3.detach().contiguous(), self.b3.detach().contiguous())
@@ -374,6 +403,9 @@ class NeuralPrimitiveSceneTileCUDA(nn.Module):
         device = self._activate_cuda_device()
         ts = int(self.tile_size)
         with torch.no_grad():
+            # queued before the binning, whose pair count is a blocking read-back: the device then has
+            # this work to do while the host waits, instead of idling while the host issues it afterwards
+            unit_dirs = F.normalize(ray_d, dim=-1).contiguous()
             culled_prim_indices, tile_offsets = self._tile_lists(
                 ray_o, ray_d, score_threshold, view_matrix, proj_matrix, culled_prim_indices, tile_offsets, device)
             use_tilecenter = self._resolve_tile_order_mode() == "tilecenter"
@@ -382,7 +414,7 @@ class NeuralPrimitiveSceneTileCUDA(nn.Module):
                 if not return_feature or self.feat_attr is None or not use_tilecenter or ts != 8:
                     raise ValueError("CSR feature training requires tilecenter8 and direct feature attributes")
                 raise NotImplementedError("record-based feature training is not part of the forward renderer")
-            base = self._base_args(ray_o, ray_d, culled_prim_indices, tile_offsets, device)
+            base = self._base_args(ray_o, ray_d, culled_prim_indices, tile_offsets, device, unit_dirs)
             bg = self._background(bg_color, ray_o)
             dims = (int(W), int(H), ts, ts, float(score_threshold))
             precision = str(getattr(self, "render_precision", "f32")).lower()

@@ -51,6 +51,8 @@ class TileExt:
         self._pack = None
         self._feat_pack_key = None
         self._binned = None
+        self._rec_key = None
+        self._rec = None
         self._feat_pack = None
 
     def __getattr__(self, name):
@@ -153,7 +155,7 @@ class TileExt:
             low_precision, hidden_limit)
         rays_o, rays_d, positions, log_scales, quats = geo
         with torch.cuda.device(rays_o.device):
-            rec = ops.prepare_primitives(positions, log_scales, quats)
+            rec = self._records(positions, log_scales, quats)
             if family == _lib.KEY_LIST_ORDER or cand.numel() == 0:
                 order = cand
             else:
@@ -196,7 +198,7 @@ class TileExt:
         _chk(feat_attr.shape[0] == positions.shape[0], "feat_attr first dimension must match primitive count")
         ops._feat_shape(feat_attr)
         with torch.cuda.device(rays_o.device):
-            rec = ops.prepare_primitives(positions, log_scales, quats)
+            rec = self._records(positions, log_scales, quats)
             order = cand
             if cand.numel() > 0:
                 order, _ = ops.sort_tiles(rays_o, rays_d, rec, cand, offsets, W, H, TW, TH, _lib.KEY_TSTAR,
@@ -212,7 +214,7 @@ class TileExt:
         _chk(0 < TW * TH <= 256, "Tile size too large")
         rays_o, rays_d, positions, log_scales, quats = geo
         with torch.cuda.device(rays_o.device):
-            rec = ops.prepare_primitives(positions, log_scales, quats)
+            rec = self._records(positions, log_scales, quats)
             if feat is None:
                 return ops.render_per_pixel_f32(rays_o, rays_d, rec, cand, offsets, freq, att, *ws, W, H, TW, TH, thr, name)
             feat_attr, beta, temp = feat
@@ -264,6 +266,18 @@ class TileExt:
     # ------------------------------------------------------------------------------------------
     def rgb_wmma_safety_stats(self):
         return [self._mfma_calls, self._mfma_fallbacks]
+
+    def _records(self, positions, log_scales, quats):
+        """Per-primitive geometry records, rebuilt only when one of the three tensors changed."""
+        try:
+            key = tuple((t.data_ptr(), t._version, tuple(t.shape), str(t.device)) for t in (positions, log_scales, quats))
+        except RuntimeError:                      # inference tensors have no version counter: no caching
+            return ops.prepare_primitives(positions, log_scales, quats)
+        with self._lock:
+            if self._rec_key != key:
+                self._rec = ops.prepare_primitives(positions, log_scales, quats)
+                self._rec_key = key
+            return self._rec
 
     def _packed_weights(self, ws, bf16):
         """Matrix-core operand copy of the six weight tensors, rebuilt only when one of them changed
@@ -320,7 +334,7 @@ class TileExt:
             self._validate(x[5], x[6], ops.num_tiles(width, height, 8, 8), self.max_tile_prims, n, name)
             with self._lock:
                 self._mfma_calls += 1
-            rec = ops.prepare_primitives(x[2], x[3], x[4])
+            rec = self._records(x[2], x[3], x[4])
             order = x[5]
             if x[5].numel() > 0:
                 order, _ = ops.sort_tiles(x[0], x[1], rec, x[5], x[6], width, height, 8, 8, _lib.KEY_TSTAR,

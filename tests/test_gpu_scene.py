@@ -181,3 +181,26 @@ def test_lists_from_the_own_binning_skip_device_validation_but_keep_the_capacity
         _call(scene, fr, device)
     monkeypatch.setattr(cumodel, "_tile_ext", TileExt(max_tile_prims=longest))
     assert torch.equal(_call(scene, fr, device), ref)
+
+
+def test_cached_scene_derivatives_follow_in_place_parameter_updates(device, oracle_mod):
+    # unit quaternions, frequency tables, geometry records and packed weights are cached per tensor
+    # version: an optimiser-style in-place update must show in the very next frame
+    fr = Frame("cfg1_5k_160x120", n=1200, hidden=32, width=48, height=32)
+    for precision in ("f32", "bf16"):
+        scene = _scene_from(fr, device)
+        scene.render_precision = precision
+        a = _call(scene, fr, device)
+        assert torch.equal(_call(scene, fr, device), a)
+        with torch.no_grad():
+            scene.log_scales.add_(0.2)
+            scene.quats.mul_(torch.tensor([1.0, -1.0, 1.0, 1.0], device=device))
+            scene.b3.add_(0.3)
+        b = _call(scene, fr, device)
+        fresh = _scene_from(fr, device)
+        fresh.render_precision = precision
+        fresh.load_state_dict(scene.state_dict())
+        assert not torch.equal(a, b) and torch.equal(_call(fresh, fr, device), b)
+        scene.encoder.set_runtime_frequency_weights(torch.tensor([1.0, 0.9, 0.8, 0.7, 0.6, 0.5]))
+        c = _call(scene, fr, device)
+        assert not torch.equal(c, b)
