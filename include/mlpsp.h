@@ -75,7 +75,7 @@ int mlpsp_validate_tile_lists(const int32_t* tile_offsets_dev, const int32_t* ca
  * scannet/cumodel.py:994-1070 (one camera) and :838-949 (tile_view_ids_dev != NULL: K views, tile
  * t uses view tile_view_ids_dev[t]).  view_matrices: K row-major 4x4 on the HOST, proj: 4x4 on
  * the host.  Within a tile, candidate ids ascend.
- * Step 1 (count): writes exclusive offsets to tile_offsets_dev[T+1]; BLOCKS to return the total
+ * Step 1 (count): writes exclusive offsets to tile_offsets_dev[T+1] (16-byte aligned); BLOCKS to return the total
  *   in counts_out[0] and the length of the longest tile list in counts_out[1] (what the capacity
  *   check of the render entry points compares with MLPSP_MAX_TILE_PRIMS).  scratch_dev: at least mlpsp_bin_scratch_bytes() bytes, 256-byte aligned,
  *   reused by step 2; MLPSP_E_SCRATCH asks for a larger one (primitives spanning very many tiles).

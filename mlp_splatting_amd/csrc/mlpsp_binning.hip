@@ -3,7 +3,7 @@
 // The reference evaluates a dense [tiles x primitives] boolean matrix (scannet/cumodel.py:1028-1070).
 // Here the same predicate is evaluated sparsely and deterministically, without atomics and without
 // a sort, in two levels:
-//   level 1: the frame is cut into super-tiles of 8x8 tiles.  Workgroup (chunk c, super-tile s)
+//   level 1: the frame is cut into super-tiles of 8x8 tiles.  Wavefront (chunk c, super-tile s)
 //            tests 2048 consecutive primitives against the super-tile rectangle (a superset of the
 //            union of its tiles' tests), counts, and after a scan writes the survivors in ascending
 //            id order -> one ascending candidate list per super-tile.
@@ -29,6 +29,7 @@ struct BinScratch {
   int32_t* l1_counts; // [S*NC + 1] counts, then exclusive offsets after the scan
   long long* totals;  // [0] level-1 entries, [1] tile-list entries, [2] longest tile list
   int32_t* l1_list;   // [l1_capacity]
+  float4* l1_bounds;  // [l1_capacity] bounds of the listed primitives, one view only (else null)
   long long l1_capacity;
 };
 
@@ -46,8 +47,13 @@ inline BinScratch carve(void* base, size_t bytes, int N, int K, int S, int NC) {
   off += align256(((size_t)S * NC + 1) * sizeof(int32_t));
   b.totals = reinterpret_cast<long long*>(p + off);
   off += 256;
+  // one view: the level-1 lists carry the bounds next to the ids (20 bytes per entry), so that level 2
+  // streams them instead of gathering 16 bytes per lane from all over the bounds array
+  const size_t entry = sizeof(int32_t) + (K == 1 ? sizeof(float4) : 0);
+  b.l1_capacity = bytes > off + 512 ? (long long)((bytes - off - 512) / entry) : 0;
   b.l1_list = reinterpret_cast<int32_t*>(p + off);
-  b.l1_capacity = bytes > off ? (long long)((bytes - off) / sizeof(int32_t)) : 0;
+  off += align256((size_t)b.l1_capacity * sizeof(int32_t));
+  b.l1_bounds = (K == 1) ? reinterpret_cast<float4*>(p + off) : nullptr;
   return b;
 }
 
@@ -110,77 +116,117 @@ __device__ __forceinline__ unsigned lanes_below(unsigned long long mask) {
   return __builtin_amdgcn_mbcnt_hi((unsigned)(mask >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)mask, 0u));
 }
 
-// level 1.  grid = (NC, S).  FILL = false: l1_counts[s*NC + c] = survivors; FILL = true: write them.
+// level 1.  grid = (NC, ceil(S / 4)); wavefront w of a workgroup owns super-tile 4 * blockIdx.y + w and walks the
+// chunk's 2048 primitives 64 at a time (no workgroup barrier: counts and positions come from ballots).
+// FILL = false: l1_counts[s*NC + c] = survivors; FILL = true: write them.
 template <bool FILL>
 __global__ __launch_bounds__(kBinThreads) void bin_level1_kernel(const float4* __restrict__ bounds, BinGeom g,
                                                                  int32_t* __restrict__ l1_counts,
-                                                                 int32_t* __restrict__ l1_list, long long l1_capacity) {
-  __shared__ int s_wave[kBinThreads / 64];
-  const int c = blockIdx.x, s = blockIdx.y;
-  const int wave = threadIdx.x >> 6;
+                                                                 int32_t* __restrict__ l1_list,
+                                                                 float4* __restrict__ l1_bounds, long long l1_capacity) {
+  const int c = blockIdx.x, s = blockIdx.y * (kBinThreads / 64) + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  if (s >= g.nsx * g.nsy) return;
   float x0, x1, y0, y1;
   super_rect(g, s, x0, x1, y0, y1);
-  int running = FILL ? l1_counts[s * g.NC + c] : 0;
-  for (int r = 0; r < kChunk / kBinThreads; ++r) {
-    const int i = c * kChunk + r * kBinThreads + threadIdx.x;
+  long long running = FILL ? l1_counts[s * g.NC + c] : 0;
+  const int first = c * kChunk;
+#pragma unroll 4
+  for (int r = 0; r < kChunk / 64; ++r) {
+    const int i = first + r * 64 + lane;
     const bool keep = (i < g.N) && super_overlap(bounds, g, i, x0, x1, y0, y1);
     const unsigned long long m = __ballot(keep);
-    if ((threadIdx.x & 63) == 0) s_wave[wave] = __popcll(m);
-    __syncthreads();
-    int before = 0, total = 0;
-#pragma unroll
-    for (int w = 0; w < kBinThreads / 64; ++w) {
-      const int cw = s_wave[w];
-      before += (w < wave) ? cw : 0;
-      total += cw;
-    }
     if (FILL && keep) {
-      const long long dst = (long long)running + before + lanes_below(m);
-      if (dst < l1_capacity) l1_list[dst] = i;
+      const long long dst = running + lanes_below(m);
+      if (dst < l1_capacity) {
+        l1_list[dst] = i;
+        if (l1_bounds) l1_bounds[dst] = bounds[i];
+      }
     }
-    running += total;
-    __syncthreads();
+    running += __popcll(m);
   }
-  if (!FILL && threadIdx.x == 0) l1_counts[s * g.NC + c] = running;
+  if (!FILL && lane == 0) l1_counts[s * g.NC + c] = (int32_t)running;
 }
 
 // In-place exclusive scan of data[0..n) by one workgroup; data[n] and *total receive the sum, *largest
-// (if not null) the largest element.
+// (if not null) the largest element.  data must be 16-byte aligned.  A pass covers 8 slabs of 4096
+// elements: thread t owns elements 4t..4t+3 of every slab, so all loads and stores are coalesced 16-byte
+// accesses and the 8 loads of a pass are independent (one memory latency per pass, and one pass covers
+// 32768 elements).  Thread sums are scanned with wavefront shuffles, wavefront totals through LDS.
+constexpr int kScanSlabs = 8;
 __global__ __launch_bounds__(1024) void exclusive_scan_kernel(int32_t* __restrict__ data, int n,
                                                               long long* __restrict__ total,
                                                               long long* __restrict__ largest) {
-  __shared__ long long s_part[1024];
-  __shared__ int s_max;
-  const int t = threadIdx.x;
-  if (t == 0) s_max = 0;
-  __syncthreads();
-  const int per = (n + 1023) / 1024;
-  const int lo = min(t * per, n), hi = min(lo + per, n);
-  long long sum = 0;
+  __shared__ long long s_wave[kScanSlabs][16];
+  __shared__ int s_wmax[16];
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+  long long carry = 0;
   int mx = 0;
-  for (int i = lo; i < hi; ++i) {
-    sum += data[i];
-    mx = max(mx, data[i]);
+  for (int pass0 = 0; pass0 < n; pass0 += kScanSlabs * 4096) {
+    int4 v[kScanSlabs];
+#pragma unroll
+    for (int u = 0; u < kScanSlabs; ++u) {
+      const int idx = pass0 + u * 4096 + t * 4;
+      if (idx + 3 < n) {
+        v[u] = *reinterpret_cast<const int4*>(data + idx);
+      } else {
+        v[u].x = (idx < n) ? data[idx] : 0;
+        v[u].y = (idx + 1 < n) ? data[idx + 1] : 0;
+        v[u].z = (idx + 2 < n) ? data[idx + 2] : 0;
+        v[u].w = 0;
+      }
+    }
+    long long incl[kScanSlabs];
+#pragma unroll
+    for (int u = 0; u < kScanSlabs; ++u) {
+      mx = max(max(mx, max(v[u].x, v[u].y)), max(v[u].z, v[u].w));
+      long long x = (long long)v[u].x + v[u].y + v[u].z + v[u].w;
+#pragma unroll
+      for (int d = 1; d < 64; d <<= 1) {
+        const long long up = __shfl_up(x, d);
+        if (lane >= d) x += up;
+      }
+      incl[u] = x;
+      if (lane == 63) s_wave[u][wave] = x;
+    }
+    __syncthreads();
+    long long base = carry;
+#pragma unroll
+    for (int u = 0; u < kScanSlabs; ++u) {
+      long long before = 0, slab = 0;
+#pragma unroll
+      for (int w = 0; w < 16; ++w) {
+        const long long c = s_wave[u][w];
+        before += (w < wave) ? c : 0;
+        slab += c;
+      }
+      const long long own = (long long)v[u].x + v[u].y + v[u].z + v[u].w;
+      const long long e0 = base + before + incl[u] - own;
+      const int idx = pass0 + u * 4096 + t * 4;
+      const int4 o = make_int4((int)e0, (int)(e0 + v[u].x), (int)(e0 + v[u].x + v[u].y),
+                               (int)(e0 + v[u].x + v[u].y + v[u].z));
+      if (idx + 3 < n) {
+        *reinterpret_cast<int4*>(data + idx) = o;
+      } else {
+        if (idx < n) data[idx] = o.x;
+        if (idx + 1 < n) data[idx + 1] = o.y;
+        if (idx + 2 < n) data[idx + 2] = o.z;
+      }
+      base += slab;
+    }
+    carry = base;
+    __syncthreads();
   }
-  if (largest && mx > 0) atomicMax(&s_max, mx);
-  s_part[t] = sum;
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) mx = max(mx, __shfl_xor(mx, d));
+  if (lane == 0) s_wmax[wave] = mx;
   __syncthreads();
-  for (int d = 1; d < 1024; d <<= 1) {
-    const long long v = (t >= d) ? s_part[t - d] : 0;
-    __syncthreads();
-    s_part[t] += v;
-    __syncthreads();
-  }
-  long long run = s_part[t] - sum;
-  for (int i = lo; i < hi; ++i) {
-    const int v = data[i];
-    data[i] = (int32_t)run;
-    run += v;
-  }
-  if (t == 1023) {
-    data[n] = (int32_t)s_part[1023];
-    *total = s_part[1023];
-    if (largest) *largest = s_max;
+  if (t == 0) {
+    int all_max = 0;
+    for (int w = 0; w < 16; ++w) all_max = max(all_max, s_wmax[w]);
+    data[n] = (int32_t)carry;
+    *total = carry;
+    if (largest) *largest = all_max;
   }
 }
 
@@ -190,6 +236,7 @@ __global__ __launch_bounds__(kBinThreads) void bin_level2_kernel(const float4* _
                                                                  const int32_t* __restrict__ tile_view_ids,
                                                                  const int32_t* __restrict__ l1_offsets,
                                                                  const int32_t* __restrict__ l1_list,
+                                                                 const float4* __restrict__ l1_bounds,
                                                                  long long l1_capacity,
                                                                  int32_t* __restrict__ tile_offsets,
                                                                  int32_t* __restrict__ cand) {
@@ -212,7 +259,7 @@ __global__ __launch_bounds__(kBinThreads) void bin_level2_kernel(const float4* _
     bool keep = false;
     if (j < hi) {
       id = l1_list[j];
-      keep = rect_overlap(vb[id], x0, x1, y0, y1);
+      keep = rect_overlap(l1_bounds ? l1_bounds[j] : vb[id], x0, x1, y0, y1);
     }
     const unsigned long long m = __ballot(keep);
     if (FILL && keep) cand[running + lanes_below(m)] = id;
@@ -242,7 +289,8 @@ MLPSP_API size_t mlpsp_bin_scratch_bytes(int num_primitives, int num_views, int 
                  align256((size_t)num_views * num_primitives * sizeof(float4)) +
                  align256((S * g.NC + 1) * sizeof(int32_t)) + 256;
   // room for every primitive to touch 8 super-tiles per view, plus slack for tiny scenes
-  bytes += align256(((size_t)8 * num_views * num_primitives + 65536) * sizeof(int32_t));
+  const size_t entry = sizeof(int32_t) + (num_views == 1 ? sizeof(float4) : 0);
+  bytes += align256(((size_t)8 * num_views * num_primitives + 65536) * entry) + 512;
   return bytes;
 }
 
@@ -256,6 +304,8 @@ MLPSP_API int mlpsp_bin_legacy_count(const float* positions_dev, const float* lo
       !tile_offsets_dev || !counts_out)
     return MLPSP_E_ARGUMENT;
   if (!(threshold > 0.f && threshold < 1.f)) return MLPSP_E_ARGUMENT;
+  if (reinterpret_cast<uintptr_t>(tile_offsets_dev) % 16 != 0 || reinterpret_cast<uintptr_t>(scratch_dev) % 256 != 0)
+    return MLPSP_E_ARGUMENT;
   if (scratch_bytes < mlpsp_bin_scratch_bytes(num_primitives, num_views, width, height, tile)) return MLPSP_E_SCRATCH;
   hipStream_t s = (hipStream_t)stream;
   const BinGeom g = make_geom(num_primitives, num_views, width, height, tile);
@@ -277,17 +327,17 @@ MLPSP_API int mlpsp_bin_legacy_count(const float* positions_dev, const float* lo
   hipLaunchKernelGGL(bin_bounds_kernel, dim3(ceil_div(num_primitives, kBinThreads), num_views), dim3(kBinThreads), 0, s,
                      positions_dev, log_scales_dev, b.mats, g, rm, focal, b.bounds);
   MLPSP_LAUNCH_CHECK();
-  hipLaunchKernelGGL((bin_level1_kernel<false>), dim3(g.NC, S), dim3(kBinThreads), 0, s, b.bounds, g, b.l1_counts,
-                     b.l1_list, b.l1_capacity);
+  hipLaunchKernelGGL((bin_level1_kernel<false>), dim3(g.NC, ceil_div(S, kBinThreads / 64)), dim3(kBinThreads), 0, s, b.bounds, g, b.l1_counts,
+                     b.l1_list, b.l1_bounds, b.l1_capacity);
   MLPSP_LAUNCH_CHECK();
   hipLaunchKernelGGL(exclusive_scan_kernel, dim3(1), dim3(1024), 0, s, b.l1_counts, S * g.NC, b.totals,
                      (long long*)nullptr);
   MLPSP_LAUNCH_CHECK();
-  hipLaunchKernelGGL((bin_level1_kernel<true>), dim3(g.NC, S), dim3(kBinThreads), 0, s, b.bounds, g, b.l1_counts,
-                     b.l1_list, b.l1_capacity);
+  hipLaunchKernelGGL((bin_level1_kernel<true>), dim3(g.NC, ceil_div(S, kBinThreads / 64)), dim3(kBinThreads), 0, s, b.bounds, g, b.l1_counts,
+                     b.l1_list, b.l1_bounds, b.l1_capacity);
   MLPSP_LAUNCH_CHECK();
   hipLaunchKernelGGL((bin_level2_kernel<false>), dim3(ceil_div((int)T, kBinThreads / 64)), dim3(kBinThreads), 0, s,
-                     b.bounds, g, tile_view_ids_dev, b.l1_counts, b.l1_list, b.l1_capacity, tile_offsets_dev,
+                     b.bounds, g, tile_view_ids_dev, b.l1_counts, b.l1_list, b.l1_bounds, b.l1_capacity, tile_offsets_dev,
                      (int32_t*)nullptr);
   MLPSP_LAUNCH_CHECK();
   hipLaunchKernelGGL(exclusive_scan_kernel, dim3(1), dim3(1024), 0, s, tile_offsets_dev, (int)T, b.totals + 1,
@@ -314,7 +364,7 @@ MLPSP_API int mlpsp_bin_legacy_fill(int num_primitives, int num_views, const int
   const BinGeom g = make_geom(num_primitives, num_views, width, height, tile);
   const BinScratch b = carve(const_cast<void*>(scratch_dev), scratch_bytes, num_primitives, num_views, g.nsx * g.nsy, g.NC);
   hipLaunchKernelGGL((bin_level2_kernel<true>), dim3(ceil_div((int)T, kBinThreads / 64)), dim3(kBinThreads), 0,
-                     (hipStream_t)stream, b.bounds, g, tile_view_ids_dev, b.l1_counts, b.l1_list, b.l1_capacity,
+                     (hipStream_t)stream, b.bounds, g, tile_view_ids_dev, b.l1_counts, b.l1_list, b.l1_bounds, b.l1_capacity,
                      const_cast<int32_t*>(tile_offsets_dev), candidates_dev);
   MLPSP_LAUNCH_CHECK();
   return MLPSP_OK;
