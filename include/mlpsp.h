@@ -128,6 +128,23 @@ int mlpsp_render_tilecenter_f32(const float* rays_o_dev, const float* rays_d_dev
                                 float threshold, float* out_rgb_dev, float* out_alpha_dev, float* out_t_dev,
                                 int64_t* counters_dev, mlpsp_stream_t stream);
 
+/* Pruning-statistics forward (render_tiles_kernel_tilecenter_order_stats, np_tile_kernels.cu:2139-2519,
+ * wrapper :5349-5428): renders like mlpsp_render_tilecenter_f32 and, per processed primitive p, adds to
+ * stat_sum_w[p] the sum over the tile's pixels of the compositing weight w, raises stat_max_w[p] to the
+ * largest w, adds to stat_hits[p] the number of pixels with w > 1e-8, to stat_sum_werr[p] the sum of
+ * w * err over pixels with w > 0.1 (err = L1 distance of the pixel's colour after this step from
+ * gt_rgb_dev [B,3]) and to stat_contrib[p] their number.  The five buffers [N] are updated in place with
+ * atomics (the last two may be NULL); the reference sorts this kernel's tiles with MLPSP_KEY_DEPTH. */
+int mlpsp_render_tilecenter_stats_f32(const float* rays_o_dev, const float* rays_d_dev, const void* prim_records_dev,
+                                      const int32_t* order_dev, const int32_t* tile_offsets_dev,
+                                      const float* freq_dev, const float* att_dev, int num_frequencies,
+                                      const float* W1, const float* b1, const float* W2, const float* b2,
+                                      const float* W3, const float* b3, int num_primitives, int hidden, int width,
+                                      int height, int tile_w, int tile_h, float threshold, const float* gt_rgb_dev,
+                                      float* out_rgb_dev, float* out_alpha_dev, float* stat_sum_w_dev,
+                                      float* stat_max_w_dev, int32_t* stat_hits_dev, float* stat_sum_werr_dev,
+                                      int32_t* stat_contrib_dev, mlpsp_stream_t stream);
+
 /* Workspace of the feature renders below.  The render kernel hands the feature kernel one "hit record"
  * per (64-pixel wavefront of a tile, primitive that hits one of its pixels); how many there will be is
  * only known after the frame (early termination), so records come from a pool of pool_records records.

@@ -54,3 +54,45 @@ MLPSP_API int mlpsp_render_tilecenter_f32(const float* rays_o_dev, const float* 
   MLPSP_LAUNCH_CHECK();
   return MLPSP_OK;
 }
+
+MLPSP_API int mlpsp_render_tilecenter_stats_f32(const float* rays_o_dev, const float* rays_d_dev,
+                                                const void* prim_records_dev, const int32_t* order_dev,
+                                                const int32_t* tile_offsets_dev, const float* freq_dev,
+                                                const float* att_dev, int num_frequencies, const float* W1,
+                                                const float* b1, const float* W2, const float* b2, const float* W3,
+                                                const float* b3, int num_primitives, int hidden, int width,
+                                                int height, int tile_w, int tile_h, float threshold,
+                                                const float* gt_rgb_dev, float* out_rgb_dev, float* out_alpha_dev,
+                                                float* stat_sum_w_dev, float* stat_max_w_dev, int32_t* stat_hits_dev,
+                                                float* stat_sum_werr_dev, int32_t* stat_contrib_dev,
+                                                mlpsp_stream_t stream) {
+  const int64_t T = checked_num_tiles(width, height, tile_w, tile_h);
+  if (T <= 0) return MLPSP_E_ARGUMENT;
+  const int64_t tile_px = (int64_t)tile_w * tile_h;
+  if (tile_px <= 0 || tile_px > 256) return MLPSP_E_ARGUMENT;
+  if (num_frequencies <= 0 || num_frequencies > 16 || hidden <= 0 || hidden > 64 || num_primitives < 0)
+    return MLPSP_E_ARGUMENT;
+  if (!rays_o_dev || !rays_d_dev || !tile_offsets_dev || !out_rgb_dev || !out_alpha_dev || !gt_rgb_dev)
+    return MLPSP_E_ARGUMENT;
+  if (num_primitives > 0 && (!stat_sum_w_dev || !stat_max_w_dev || !stat_hits_dev)) return MLPSP_E_ARGUMENT;
+  const int wpt = (int)((tile_px + 63) / 64);
+  const int64_t items = T * wpt;
+  if (items > 2147483647LL - 8) return MLPSP_E_ARGUMENT;
+  const int per_xcd = (int)((items + kNumXcd - 1) / kNumXcd);
+  TileGeom g{width, height, tile_w, tile_h, ceil_div(width, tile_w), ceil_div(height, tile_h)};
+  const dim3 grid((unsigned)(per_xcd * kNumXcd)), block(64);
+  hipStream_t s = (hipStream_t)stream;
+#define MLPSP_STATS_LAUNCH(HT, FT)                                                                               \
+  hipLaunchKernelGGL((render_tilecenter_f32_kernel<HT, FT, 0, true>), grid, block, 0, s, rays_o_dev, rays_d_dev, \
+                     (const PrimRecord*)prim_records_dev, order_dev, tile_offsets_dev, freq_dev, att_dev,        \
+                     num_frequencies, W1, b1, W2, b2, W3, b3, num_primitives, hidden, g, wpt, per_xcd,           \
+                     (int)items, threshold, out_rgb_dev, out_alpha_dev, (float*)nullptr,                         \
+                     (unsigned long long*)nullptr, 0.f, 0.f, HitPool{}, gt_rgb_dev, stat_sum_w_dev,              \
+                     stat_max_w_dev, stat_hits_dev, stat_sum_werr_dev, stat_contrib_dev)
+  if (hidden == 32 && num_frequencies == 6) MLPSP_STATS_LAUNCH(32, 6);
+  else if (hidden == 16 && num_frequencies == 6) MLPSP_STATS_LAUNCH(16, 6);
+  else MLPSP_STATS_LAUNCH(0, 0);
+#undef MLPSP_STATS_LAUNCH
+  MLPSP_LAUNCH_CHECK();
+  return MLPSP_OK;
+}

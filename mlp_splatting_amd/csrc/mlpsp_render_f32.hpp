@@ -11,7 +11,23 @@ namespace mlpsp {
 // EMIT = 0: image only.  EMIT = 1 / 2: also emit one hit record per primitive that hits a pixel of this
 // wavefront, float[K][64] with K = 1 (the compositing weight w) / K = 5 (w and the four tetrahedral
 // gates); w = -1 marks a pixel the primitive did not hit (weights are never negative).
-template <int HT, int FT, int EMIT>
+//
+// STATS: also accumulate the pruning statistics of np_tile_kernels.cu:2139-2519: per processed primitive
+// the wavefront reduces over its pixels  w,  max w,  [w > 1e-8],  [w > 0.1] * w * err  and  [w > 0.1]
+// (err = L1 colour error of the pixel after this blend step against gt_rgb) and adds them to the five
+// per-primitive buffers with atomics, as the reference does per block (:2435-2456).
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) v += __shfl_xor(v, d);
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) v = fmaxf(v, __shfl_xor(v, d));
+  return v;
+}
+
+template <int HT, int FT, int EMIT, bool STATS = false>
 __global__ __launch_bounds__(64) void render_tilecenter_f32_kernel(
     const float* __restrict__ rays_o, const float* __restrict__ rays_d, const PrimRecord* __restrict__ prims,
     const int32_t* __restrict__ order, const int32_t* __restrict__ offsets, const float* __restrict__ freq,
@@ -19,7 +35,10 @@ __global__ __launch_bounds__(64) void render_tilecenter_f32_kernel(
     const float* __restrict__ W2, const float* __restrict__ b2, const float* __restrict__ W3,
     const float* __restrict__ b3, int N, int H, TileGeom g, int waves_per_tile, int per_xcd,
     int num_items, float thr, float* __restrict__ out_rgb, float* __restrict__ out_alpha, float* __restrict__ out_t,
-    unsigned long long* __restrict__ counters, float beta, float temp, HitPool hp) {
+    unsigned long long* __restrict__ counters, float beta, float temp, HitPool hp,
+    const float* __restrict__ gt_rgb = nullptr, float* __restrict__ stat_sum_w = nullptr,
+    float* __restrict__ stat_max_w = nullptr, int32_t* __restrict__ stat_hits = nullptr,
+    float* __restrict__ stat_sum_werr = nullptr, int32_t* __restrict__ stat_contrib = nullptr) {
   // The weight pointers are separate __restrict__ parameters (not a struct): only then does the compiler
   // know that the record stores below cannot alias them and keeps fetching weights with scalar loads.
   const MlpPtrs mlp{W1, b1, W2, b2, W3, b3};
@@ -46,6 +65,14 @@ __global__ __launch_bounds__(64) void render_tilecenter_f32_kernel(
 
   PixelAcc acc = {0.f, 0.f, 0.f, 1.f, 0.f, 0.f};
   unsigned n_proc = 0, n_proc_hit = 0, n_hits = 0;
+  float gtr = 0.f, gtg = 0.f, gtb = 0.f;
+  if constexpr (STATS) {
+    if (valid) {
+      gtr = gt_rgb[pix * 3 + 0];
+      gtg = gt_rgb[pix * 3 + 1];
+      gtb = gt_rgb[pix * 3 + 2];
+    }
+  }
   HitEmitter em = hit_emitter_begin(hp, wslot, start, tile);
 
   for (int i = start; i < end; ++i) {
@@ -61,6 +88,7 @@ __global__ __launch_bounds__(64) void render_tilecenter_f32_kernel(
       ++n_proc_hit;
       n_hits += __popcll(hit_mask);
       int rs = -1;
+      float w_stat = 0.f;
       if constexpr (EMIT > 0) rs = hit_emitter_next(hp, em, (int)threadIdx.x);
       float* __restrict__ rec = reinterpret_cast<float*>(hp.records + (size_t)(rs < 0 ? 0 : rs) * hp.record_bytes);
       if (hit) {
@@ -68,6 +96,7 @@ __global__ __launch_bounds__(64) void render_tilecenter_f32_kernel(
         float o[4];
         mlp_eval<HT, FT>(x6, freq, att, F, H, mlp, p, o);
         const float w = blend_step(acc, o[0], o[1], o[2], o[3], h.decay, h.t);
+        w_stat = w;
         if constexpr (EMIT > 0) {
           if (rs >= 0) {
             rec[threadIdx.x] = w;
@@ -84,6 +113,21 @@ __global__ __launch_bounds__(64) void render_tilecenter_f32_kernel(
       }
       if constexpr (EMIT > 0) {
         if (rs >= 0 && threadIdx.x == 0) hp.hit_ids[rs] = p;
+      }
+      if constexpr (STATS) {
+        const float lw = hit ? w_stat : 0.f;
+        const bool contrib = hit && (lw > 1e-1f);
+        float lerr = 0.f;
+        if (contrib) lerr = lw * ((fabsf(acc.cr - gtr) + fabsf(acc.cg - gtg)) + fabsf(acc.cb - gtb));
+        const float s_w = wave_sum(lw), m_w = wave_max(lw), s_err = wave_sum(lerr);
+        const int n_hit = __popcll(__ballot(hit && (lw > 1e-8f))), n_con = __popcll(__ballot(contrib));
+        if (threadIdx.x == 0) {
+          atomicAdd(stat_sum_w + p, s_w);
+          atomicMax(reinterpret_cast<int*>(stat_max_w + p), __float_as_int(m_w));   // weights are >= 0
+          atomicAdd(stat_hits + p, n_hit);
+          if (stat_sum_werr) atomicAdd(stat_sum_werr + p, s_err);
+          if (stat_contrib) atomicAdd(stat_contrib + p, n_con);
+        }
       }
     }
     if (__ballot(valid && (acc.trans >= kTransmittanceFloor)) == 0ull) break;

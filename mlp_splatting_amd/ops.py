@@ -158,6 +158,24 @@ def radius_multiplier(threshold: float) -> float:
     return math.sqrt(-2.0 * math.log(threshold))
 
 
+def render_tilecenter_stats_f32(rays_o, rays_d, records, order, tile_offsets, freq, att, W1, b1, W2, b2, W3, b3, W, H,
+                                TW, TH, threshold, gt_rgb, stat_sum_w, stat_max_w, stat_hits, stat_sum_werr=None,
+                                stat_contrib=None):
+    """Scalar-f32 tile-centre forward that also accumulates the five pruning statistics in place -> (rgb, alpha)."""
+    dev = rays_o.device
+    B = W * H
+    rgb = torch.empty(B, 3, dtype=torch.float32, device=dev)
+    alpha = torch.empty(B, 1, dtype=torch.float32, device=dev)
+    n, hidden, F = W1.shape[0], W2.shape[1], freq.shape[0]
+    code = _lib.load().mlpsp_render_tilecenter_stats_f32(
+        _ptr(rays_o), _ptr(rays_d), _ptr(records), _ptr(order), _ptr(tile_offsets), _ptr(freq), _ptr(att), F,
+        _ptr(W1), _ptr(b1), _ptr(W2), _ptr(b2), _ptr(W3), _ptr(b3), n, hidden, W, H, TW, TH, float(threshold),
+        _ptr(gt_rgb), _ptr(rgb), _ptr(alpha), _ptr(stat_sum_w), _ptr(stat_max_w), _ptr(stat_hits),
+        _ptr(stat_sum_werr), _ptr(stat_contrib), _stream(dev))
+    _check(code, "mlpsp_render_tilecenter_stats_f32")
+    return rgb, alpha
+
+
 def _feat_shape(feat_attr):
     """(slots, channels) with the reference's checks (np_tile_kernels.cu:6158-6169)."""
     if not (feat_attr.is_cuda and feat_attr.dtype == torch.float32 and feat_attr.dim() in (2, 3)):

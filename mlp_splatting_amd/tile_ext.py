@@ -148,7 +148,8 @@ class TileExt:
     # ------------------------------------------------------------------------------------------
     # tile-centre order
     # ------------------------------------------------------------------------------------------
-    def _tilecenter(self, args, name, family, capacity, with_t=False, low_precision=False, hidden_limit=MAX_H_TILECENTER):
+    def _tilecenter(self, args, name, family, capacity, with_t=False, low_precision=False, hidden_limit=MAX_H_TILECENTER,
+                    stats=None):
         geo, cand, offsets, freq, att, ws, (W, H, TW, TH, thr) = self._prepare(
             args, name, capacity,
             (256, "Tile-center order kernel requires 0 < TW*TH <= MLPSP_TILECENTER_BLOCK_THREADS"),
@@ -161,6 +162,10 @@ class TileExt:
             else:
                 order, _ = ops.sort_tiles(rays_o, rays_d, rec, cand, offsets, W, H, TW, TH, family, capacity,
                                           cull_threshold=thr)
+            if stats is not None:
+                rgb, alpha = ops.render_tilecenter_stats_f32(rays_o, rays_d, rec, order, offsets, freq, att, *ws, W, H,
+                                                             TW, TH, thr, *stats)
+                return rgb, alpha, None
             return ops.render_tilecenter_f32(rays_o, rays_d, rec, order, offsets, freq, att, *ws, W, H, TW, TH, thr,
                                              with_t=with_t)
 
@@ -247,18 +252,21 @@ class TileExt:
                                               freq, att, F, W1, b1, W2, b2, W3, b3, N, H, IN, Wimg, Himg, TW, TH, thr,
                                               gt_rgb, stat_sum_w, stat_max_w, stat_hits, stat_sum_werr,
                                               stat_contrib_count):
-        """Validates and renders like np_tile_kernels.cu:5349-5428 (centre-depth order) and returns
-        (rgb, alpha); the five per-primitive statistic buffers are left untouched."""
+        """(rgb, alpha) in centre-depth order; the five per-primitive statistic buffers are updated in
+        place (np_tile_kernels.cu:2139-2519, wrapper :5349-5428)."""
         _chk(0 < int(TW) * int(TH) <= 256, "Tile-center order kernel currently supports 0 < TW*TH <= 256")
         for t in (stat_sum_w, stat_max_w, stat_sum_werr):
-            _chk(t.is_cuda and t.dtype == torch.float32 and t.numel() == N)
+            _chk(t.is_cuda and t.dtype == torch.float32 and t.numel() == N and t.is_contiguous())
         for t in (stat_hits, stat_contrib_count):
-            _chk(t.is_cuda and t.dtype == torch.int32 and t.numel() == N)
+            _chk(t.is_cuda and t.dtype == torch.int32 and t.numel() == N and t.is_contiguous())
+        _chk(int(N) == positions.shape[0], "N must be the primitive count")
         _chk(gt_rgb.is_cuda and gt_rgb.dtype == torch.float32 and tuple(gt_rgb.shape) == (int(Himg) * int(Wimg), 3))
         args = (rays_o, rays_d, positions, log_scales, quats, cand, offsets, freq, att, W1, b1, W2, b2, W3, b3,
                 Wimg, Himg, TW, TH, thr)
         rgb, alpha, _ = self._tilecenter(args, "render_tiles_forward_tilecenter_stats", _lib.KEY_DEPTH,
-                                         self.max_tile_prims, hidden_limit=64)
+                                         self.max_tile_prims, hidden_limit=64,
+                                         stats=(gt_rgb.contiguous(), stat_sum_w, stat_max_w, stat_hits, stat_sum_werr,
+                                                stat_contrib_count))
         return rgb, alpha
 
     # ------------------------------------------------------------------------------------------

@@ -207,6 +207,26 @@ def render_tilecenter(rays_o, rays_d, pos, log_s, quats, cand, offsets, freq, at
     return {"rgb": rgb, "alpha": alpha, "t": t, "feat": feat, "stats": stats}
 
 
+def render_stats(rays_o, rays_d, pos, log_s, quats, cand, offsets, freq, att, W1, b1, W2, b2, W3, b3,
+                 W, H, TW, TH, thr, gt_rgb, *, capacity=1536, nthreads=0):
+    """Pruning-statistics forward -> dict(rgb, alpha, sum_w, max_w, hits, sum_werr, contrib), the five
+    statistics as the increments one call adds to zeroed per-primitive buffers (float64 / int64)."""
+    args, keep = _scene_args(rays_o, rays_d, pos, log_s, quats, cand, offsets, freq, att, W1, b1, W2, b2, W3, b3)
+    gt = _fa(gt_rgb)
+    B, n = W * H, int(np.asarray(pos).shape[0])
+    rgb = np.zeros((B, 3), np.float32)
+    alpha = np.zeros((B, 1), np.float32)
+    sum_w, max_w, sum_werr = (np.zeros(n, np.float64) for _ in range(3))
+    hits, contrib = np.zeros(n, np.int64), np.zeros(n, np.int64)
+    _d = C.POINTER(C.c_double)
+    lib().mlpsp_oracle_render_stats(*args, int(W), int(H), int(TW), int(TH), C.c_float(thr), int(capacity), _p(gt, _f),
+                                    _p(rgb, _f), _p(alpha, _f), _p(sum_w, _d), _p(max_w, _d), _p(hits, _l),
+                                    _p(sum_werr, _d), _p(contrib, _l), int(nthreads))
+    del keep
+    return {"rgb": rgb, "alpha": alpha, "sum_w": sum_w, "max_w": max_w, "hits": hits, "sum_werr": sum_werr,
+            "contrib": contrib}
+
+
 def render_per_pixel(rays_o, rays_d, pos, log_s, quats, cand, offsets, freq, att, W1, b1, W2, b2, W3, b3,
                      W, H, TW, TH, thr, *, feat_attr=None, beta=1.5, temp=2.0, nthreads=0):
     """Returns dict(rgb, alpha, feat|None, overflow: bool)."""

@@ -25,6 +25,8 @@
 //   legacy + tile-view binning ........................... pinned by brute force over the dense predicate
 //   ray-cone binning ..................................... pinned by the reference's own brute-force test
 //   gates / feature ...................................... pinned by softmax closed form + framebuffer sum
+//   pruning statistics ................................... pinned by the geometric-series weights of
+//       stacked identical primitives and by sum_p sum_w[p] = sum_pixels alpha
 //   bf16/fp16 mixed-precision MLP ........................ pinned against a numpy emulation of the
 //       rounding points; the reference entry point itself (render_tiles_rgb_wmma) has no test in
 //       the reference: "parity unpinned" beyond the stated tolerances.
@@ -796,6 +798,100 @@ ORACLE_API void mlpsp_oracle_render_tilecenter(
     }
   }
   if (stats) { stats[0] = s_cand; stats[1] = s_proc; stats[2] = s_proc_hit; stats[3] = s_hits; }
+}
+
+// ------------------------------------------------------------------------------------------
+// Pruning statistics forward: scannet/cuda/np_tile_kernels.cu:2139-2519 (kernel), :5349-5428 (wrapper).
+// Plain centre-depth order (:2243-2249), f32.  Per (tile, processed primitive) the block reduces over
+// its pixels  w,  max w,  [w > 1e-8],  [w > 0.1] * w * err,  [w > 0.1]  with err the L1 colour error of
+// the pixel AFTER this blend step against gt_rgb (:2394-2412), and adds them to five per-primitive
+// buffers (:2449-2456).  The reference's reduction and atomic order is unspecified; the sums are kept
+// in double here and compared with a tolerance.
+// ------------------------------------------------------------------------------------------
+ORACLE_API void mlpsp_oracle_render_stats(
+    const float* rays_o, const float* rays_d, const float* pos, const float* logs, const float* quats,
+    const int32_t* cand, const int32_t* offsets, const float* freq, const float* att, int F,
+    const float* W1, const float* b1, const float* W2, const float* b2, const float* W3, const float* b3,
+    int N, int H, int Wimg, int Himg, int TW, int TH, float thr, int capacity, const float* gt_rgb,
+    float* out_rgb, float* out_alpha, double* sum_w, double* max_w, int64_t* hits, double* sum_werr,
+    int64_t* contrib, int nthreads) {
+  Scene S{};
+  S.rays_o = rays_o; S.rays_d = rays_d; S.pos = pos; S.logs = logs; S.quats = quats;
+  S.cand = cand; S.offsets = offsets; S.freq = freq; S.att = att; S.F = F;
+  S.W1 = W1; S.b1 = b1; S.W2 = W2; S.b2 = b2; S.W3 = W3; S.b3 = b3; S.N = N; S.H = H;
+  S.Wimg = Wimg; S.Himg = Himg; S.TW = TW; S.TH = TH; S.thr = thr;
+  const int ntx = (Wimg + TW - 1) / TW, nty = (Himg + TH - 1) / TH, T = ntx * nty, npx = TW * TH;
+  constexpr float kWEps = 1e-1f;
+  if (nthreads <= 0) nthreads = omp_get_max_threads();
+#pragma omp parallel num_threads(nthreads)
+  {
+    std::vector<KeyId> buf;
+    std::vector<PixelState> st(npx);
+    std::vector<int> pixidx(npx);
+#pragma omp for schedule(dynamic, 4)
+    for (int tile = 0; tile < T; ++tile) {
+      const int tx = tile % ntx, ty = tile / ntx;
+      for (int k = 0; k < npx; ++k) {
+        const int x = tx * TW + k % TW, y = ty * TH + k / TW;
+        pixidx[k] = (x < Wimg && y < Himg) ? (y * Wimg + x) : -1;
+        st[k] = PixelState();
+      }
+      sort_tile(S, tile, 2, capacity, buf);
+      for (size_t i = 0; i < buf.size(); ++i) {
+        const int p = buf[i].id;
+        if (p < 0 || p >= N) continue;
+        const Prim P = load_prim(pos, logs, quats, p);
+        const MlpView M = mlp_of(S, p);
+        double t_sum = 0.0, t_werr = 0.0;
+        float t_max = 0.f;
+        int64_t t_hits = 0, t_contrib = 0;
+        int nactive = 0;
+        for (int k = 0; k < npx; ++k) {
+          const int pix = pixidx[k];
+          if (pix < 0) continue;
+          PixelState& ps = st[k];
+          if (ps.trans >= 1e-3f) {
+            Hit h;
+            const float* ro = rays_o + (size_t)pix * 3;
+            const float* rd = rays_d + (size_t)pix * 3;
+            if (hit_rot(ro[0], ro[1], ro[2], rd[0], rd[1], rd[2], P, thr, h)) {
+              const float x6[6] = {rd[0], rd[1], rd[2], h.dx, h.dy, h.dz};
+              float o[4];
+              mlp_f32(x6, freq, att, M, o);
+              const float w = blend(ps, o, h.decay, h.t);
+              const float* gt = gt_rgb + (size_t)pix * 3;
+              const float err = (std::fabs(ps.Cx - gt[0]) + std::fabs(ps.Cy - gt[1])) + std::fabs(ps.Cz - gt[2]);
+              t_sum += (double)w;
+              t_max = w > t_max ? w : t_max;
+              t_hits += (w > 1e-8f) ? 1 : 0;
+              if (w > kWEps) {
+                t_werr += (double)(w * err);
+                ++t_contrib;
+              }
+            }
+          }
+          if (ps.trans >= 1e-3f) ++nactive;
+        }
+#pragma omp atomic
+        sum_w[p] += t_sum;
+#pragma omp atomic
+        sum_werr[p] += t_werr;
+#pragma omp atomic
+        hits[p] += t_hits;
+#pragma omp atomic
+        contrib[p] += t_contrib;
+#pragma omp critical(mlpsp_stat_max)
+        { if ((double)t_max > max_w[p]) max_w[p] = (double)t_max; }
+        if (nactive == 0) break;
+      }
+      for (int k = 0; k < npx; ++k) {
+        const int pix = pixidx[k];
+        if (pix < 0) continue;
+        out_rgb[pix * 3 + 0] = st[k].Cx; out_rgb[pix * 3 + 1] = st[k].Cy; out_rgb[pix * 3 + 2] = st[k].Cz;
+        out_alpha[pix] = 1.f - st[k].trans;
+      }
+    }
+  }
 }
 
 // ------------------------------------------------------------------------------------------

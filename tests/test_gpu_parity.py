@@ -288,3 +288,39 @@ def test_per_pixel_render_is_bit_exact(device, oracle_mod, with_feat):
     # per-pixel and tile-centre orders differ on real scenes: the two oracles must not coincide here
     tc = oracle_mod.render_tilecenter(*fr.base_numpy(cand, off), *fr.dims)
     assert np.abs(tc["rgb"] - want["rgb"]).max() > 1e-4
+
+
+@pytest.mark.parametrize("tile,hidden", [(8, 32), (16, 16), (8, 8)])
+def test_statistics_forward_against_oracle(device, oracle_mod, tile, hidden):
+    # np_tile_kernels.cu:2139-2519.  Image bit-exact; integer statistics and the maximum exact; the two
+    # float sums are reductions in an unspecified order (wavefront shuffles + atomics here, block
+    # reduce + atomics in the reference): relative 1e-5 against the oracle's double-precision sums.
+    from mlp_splatting_amd import ops
+    fr = Frame("cfg1_5k_160x120", n=2500, hidden=hidden, width=72, height=48, tile=tile)
+    sc = fr.scene
+    cand, off = fr.oracle_lists(oracle_mod)
+    gt = np.random.default_rng(5).random((fr.W * fr.H, 3), dtype=np.float32)
+    want = oracle_mod.render_stats(*fr.base_numpy(cand, off), *fr.dims, gt)
+    rec = ops.prepare_primitives(_t(sc.positions, device), _t(sc.log_scales, device), _t(sc.quats, device))
+    ro, rd, c, o = _t(fr.rays_o, device), _t(fr.rays_d, device), _t(cand, device), _t(off, device)
+    order, _ = ops.sort_tiles(ro, rd, rec, c, o, fr.W, fr.H, tile, tile, family=2, cull_threshold=fr.thr)
+    n = sc.n
+    st = [torch.zeros(n, device=device, dtype=dt) for dt in (torch.float32, torch.float32, torch.int32, torch.float32, torch.int32)]
+    args = (ro, rd, rec, order, o, _t(sc.freq, device), _t(sc.att, device), *[_t(w, device) for w in sc.mlp()],
+            fr.W, fr.H, tile, tile, fr.thr, _t(gt, device))
+    rgb, alpha = ops.render_tilecenter_stats_f32(*args, *st)
+    _assert_bits(rgb, want["rgb"], "rgb")
+    _assert_bits(alpha, want["alpha"], "alpha")
+    sum_w, max_w, hits, sum_werr, contrib = (t.cpu().numpy() for t in st)
+    assert np.array_equal(hits, want["hits"]) and np.array_equal(contrib, want["contrib"])
+    assert np.array_equal(max_w, want["max_w"].astype(np.float32)) and want["contrib"].sum() > 50
+    np.testing.assert_allclose(sum_w, want["sum_w"], rtol=1e-5, atol=1e-7)
+    np.testing.assert_allclose(sum_werr, want["sum_werr"], rtol=1e-5, atol=1e-7)
+    # a second frame accumulates: sums and counts double, the maximum stays
+    ops.render_tilecenter_stats_f32(*args, *st)
+    assert np.array_equal(st[2].cpu().numpy(), 2 * want["hits"]) and np.array_equal(st[1].cpu().numpy(), max_w)
+    np.testing.assert_allclose(st[0].cpu().numpy(), 2 * want["sum_w"], rtol=1e-5, atol=1e-7)
+    # the two optional buffers may be absent
+    st2 = [torch.zeros(n, device=device, dtype=dt) for dt in (torch.float32, torch.float32, torch.int32)]
+    ops.render_tilecenter_stats_f32(*args, *st2)
+    assert np.array_equal(st2[2].cpu().numpy(), want["hits"])

@@ -204,3 +204,35 @@ def test_cached_scene_derivatives_follow_in_place_parameter_updates(device, orac
         scene.encoder.set_runtime_frequency_weights(torch.tensor([1.0, 0.9, 0.8, 0.7, 0.6, 0.5]))
         c = _call(scene, fr, device)
         assert not torch.equal(c, b)
+
+
+def test_statistics_collection_through_the_scene_module(device, oracle_mod):
+    # scannet/cumodel.py:1196-1383: render_rgb_alpha_no_grad(collect_w_stats=True, gt_rgb=...) accumulates
+    # into the module's five statistic buffers; reset_w_stats() clears them
+    fr = Frame("cfg1_5k_160x120", n=1500, hidden=32, width=64, height=48)
+    scene = _scene_from(fr, device)
+    gt = np.random.default_rng(9).random((fr.W * fr.H, 3), dtype=np.float32)
+    kw = dict(view_matrix=to_dev(fr.view, device), proj_matrix=to_dev(fr.proj, device))
+    ro, rd = to_dev(fr.rays_o, device), to_dev(fr.rays_d, device)
+    rgb0, alpha0 = scene.render_rgb_alpha_no_grad(ro, rd, fr.thr, **kw)
+    assert float(scene.stat_sum_w.sum()) == 0.0
+    with pytest.raises(ValueError, match="requires gt_rgb"):
+        scene.render_rgb_alpha_no_grad(ro, rd, fr.thr, collect_w_stats=True, **kw)
+    rgb, alpha = scene.render_rgb_alpha_no_grad(ro, rd, fr.thr, collect_w_stats=True, gt_rgb=to_dev(gt, device), **kw)
+    cand, off = fr.oracle_lists(oracle_mod)
+    q = torch.nn.functional.normalize(to_dev(fr.scene.quats, device), dim=-1).cpu().numpy()
+    rdn = torch.nn.functional.normalize(rd, dim=-1).cpu().numpy()
+    freq, att = (t.cpu().numpy() for t in scene._frequency_tables(device))
+    sc = fr.scene
+    want = oracle_mod.render_stats(fr.rays_o, rdn, sc.positions, sc.log_scales, q, cand, off, freq, att, *sc.mlp(),
+                                   *fr.dims, gt)
+    assert np.array_equal(bits(rgb.cpu().numpy()), bits(want["rgb"]))
+    assert np.array_equal(scene.stat_hits.cpu().numpy(), want["hits"])
+    assert np.array_equal(scene.stat_contrib_count.cpu().numpy(), want["contrib"])
+    np.testing.assert_allclose(scene.stat_sum_w.cpu().numpy(), want["sum_w"], rtol=1e-5, atol=1e-7)
+    np.testing.assert_allclose(scene.stat_sum_werr.cpu().numpy(), want["sum_werr"], rtol=1e-5, atol=1e-7)
+    assert np.array_equal(scene.stat_max_w.cpu().numpy(), want["max_w"].astype(np.float32))
+    # the depth-ordered image differs from the t*-ordered one only where the two orders differ
+    assert float((rgb - rgb0).abs().max()) < 0.5
+    scene.reset_w_stats()
+    assert int(scene.stat_hits.sum()) == 0 and float(scene.stat_sum_werr.sum()) == 0.0

@@ -333,3 +333,44 @@ def test_two_dimensional_feature_attribute_is_ungated(oracle_mod):
     a = 1 - math.exp(-math.log(2.0))
     w = np.array([a * (1 - a) ** i for i in range(3)])
     np.testing.assert_allclose(out["feat"][0], (w[:, None] * fa).sum(0), atol=1e-6)
+
+
+# ---------------------------------------------------------------------------------------------
+# pruning statistics (np_tile_kernels.cu:2139-2519)
+# ---------------------------------------------------------------------------------------------
+def test_statistics_of_a_zero_weight_stack_follow_the_geometric_series(oracle_mod):
+    # n identical primitives on one pixel: w_i = a (1-a)^i, colour after step i = c (1 - (1-a)^(i+1))
+    n = 12
+    b3 = [0.4, -0.3, 0.9, 0.5]
+    s = stack_scene(n, b3=b3)
+    gt = np.array([[0.2, 0.6, 0.1]], np.float32)
+    out = oracle_mod.render_stats(*base(s), *DIMS1, gt)
+    plain = oracle_mod.render_tilecenter(*base(s), *DIMS1, family=2)
+    assert np.array_equal(out["rgb"], plain["rgb"]) and np.array_equal(out["alpha"], plain["alpha"])
+    a = 1.0 - np.exp(-np.log1p(np.exp(b3[3])))             # decay = 1 on the centre ray
+    c = 1.0 / (1.0 + np.exp(-np.array(b3[:3])))
+    w = a * (1.0 - a) ** np.arange(n)
+    live = np.concatenate([[True], (1.0 - a) ** np.arange(1, n) >= 1e-3])   # transmittance before step i
+    w = np.where(live, w, 0.0)
+    np.testing.assert_allclose(out["sum_w"], w, rtol=2e-6, atol=1e-9)
+    np.testing.assert_allclose(out["max_w"], w, rtol=2e-6, atol=1e-9)          # one pixel: max = sum
+    assert np.array_equal(out["hits"], (w > 1e-8).astype(np.int64))
+    assert np.array_equal(out["contrib"], (w > 0.1).astype(np.int64)) and 0 < out["contrib"].sum() < live.sum()
+    colour = c[None, :] * (1.0 - (1.0 - a) ** (np.arange(n) + 1))[:, None]
+    err = np.abs(colour - gt.astype(np.float64)).sum(axis=1)
+    np.testing.assert_allclose(out["sum_werr"], np.where(w > 0.1, w * err, 0.0), rtol=5e-6, atol=1e-9)
+
+
+def test_statistics_sum_to_the_image_alpha_and_order_by_plain_depth(oracle_mod):
+    from helpers import Frame
+    fr = Frame("cfg1_5k_160x120", n=600, width=40, height=24)
+    cand, off = fr.oracle_lists(oracle_mod)
+    gt = np.random.default_rng(3).random((fr.W * fr.H, 3), dtype=np.float32)
+    out = oracle_mod.render_stats(*fr.base_numpy(cand, off), *fr.dims, gt)
+    plain = oracle_mod.render_tilecenter(*fr.base_numpy(cand, off), *fr.dims, family=2)
+    assert np.array_equal(out["rgb"], plain["rgb"]) and np.array_equal(out["alpha"], plain["alpha"])
+    # every pixel's weights sum to its alpha = 1 - T
+    np.testing.assert_allclose(out["sum_w"].sum(), plain["alpha"].astype(np.float64).sum(), rtol=1e-5)
+    assert 0 < out["hits"].sum() <= plain["stats"][3]      # hits with w > 1e-8 among all evaluated hits
+    assert (out["max_w"] <= out["sum_w"] + 1e-12).all() and (out["contrib"] <= out["hits"]).all()
+    assert (out["sum_werr"] <= 3.0 * out["sum_w"] + 1e-9).all() and out["contrib"].sum() > 0
