@@ -93,6 +93,19 @@ def main() -> int:
     elapsed = time.perf_counter() - t0
     fps = args.steps / elapsed
 
+    # per-frame latency distribution, the way tools/benchmark_inference.py:121-149 times a frame: a
+    # synchronise on both sides of every call (so nothing overlaps between frames, unlike the loop above)
+    lat = []
+    for i in range(min(args.steps, 3 * len(frames))):
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        render(i)
+        torch.cuda.synchronize()
+        lat.append((time.perf_counter() - t1) * 1e3)
+    lat = np.sort(np.asarray(lat))
+    latency = {"mean_ms": round(float(lat.mean()), 4), "median_ms": round(float(np.median(lat)), 4),
+               "p95_ms": round(float(lat[min(len(lat) - 1, int(0.95 * len(lat)))]), 4), "frames": int(len(lat))}
+
     # ---- the render kernel alone: HIP events on the stream it is launched on, and its work counters
     freq, att = scene._frequency_tables(dev)
     quats = torch.nn.functional.normalize(scene.quats.detach(), dim=-1).contiguous()
@@ -129,11 +142,27 @@ def main() -> int:
         hits += int(c[3])
         proc += int(c[1])
         cand_total += int(cand.numel())
+    # what the matrix cores sustain on this box with nothing else in the way
+    mfma_probe = None
+    if precision == "bf16":
+        sink = torch.zeros(1, device=dev)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        lib = _lib.load()
+        stream = torch.cuda.current_stream(dev).cuda_stream
+        lib.mlpsp_probe_mfma_bf16(200, sink.data_ptr(), stream)
+        e0.record()
+        probe_flops = lib.mlpsp_probe_mfma_bf16(4000, sink.data_ptr(), stream)
+        e1.record()
+        torch.cuda.synchronize()
+        mfma_probe = round(probe_flops / (e0.elapsed_time(e1) * 1e-3) / 1e12, 1)
     flops_per_hit = 2 * (72 * sc.hidden + sc.hidden * sc.hidden + 4 * sc.hidden)
     achieved_tflops = flops_per_hit * hits / (kernel_ms * 1e-3) / 1e12
     # sort kernel: 8 compulsory bytes per candidate (4 id in, 4 id out) + the 64-byte record of every primitive
     # once (the per-candidate geometry gathers are served by L2)
     sort_gbs = (8.0 * cand_total + 64.0 * sc.n * n_probe) / (sort_ms * 1e-3) / 1e9
+    # binning: 24 bytes per primitive in, 4 per candidate and per tile out
+    T_tiles = ((W + 7) // 8) * ((H + 7) // 8)
+    bin_gbs = (24.0 * sc.n * n_probe + 4.0 * cand_total + 4.0 * (T_tiles + 1) * n_probe) / (bin_ms * 1e-3) / 1e9
 
     out = {
         "metric": "forward_render_frames_per_sec_1200x680_200k_primitives",
@@ -143,17 +172,20 @@ def main() -> int:
         "config": {"workload": args.workload, "primitives": sc.n, "width": W, "height": H, "tile": 8,
                    "threshold": thr, "poses": len(frames), "log_scale_mean": cfg["log_scale_mean"],
                    "mlp": f"72-{sc.hidden}-{sc.hidden}-4", "entry": "NeuralPrimitiveSceneTileCUDA.forward"},
-        "mpix_per_sec": round(fps * W * H / 1e6, 2),
+        "mpix_per_sec": round(fps * W * H / 1e6, 2), "latency": latency,
         "roofline": {"bound": "mfma", "kernel": "render_tilecenter_" + ("mfma" if precision == "bf16" else "f32"),
                      "achieved": round(achieved_tflops, 3), "peak": PEAK[precision], "unit": "TFLOP/s",
                      "frac": round(achieved_tflops / PEAK[precision], 5),
                      "traffic": MEASURED_TRAFFIC_BYTES.get((args.workload, precision)),
                      "ms_per_launch": round(kernel_ms / n_probe, 4), "hits_per_launch": hits // n_probe,
-                     "tile_primitives_per_launch": proc // n_probe, "flops_per_hit": flops_per_hit},
+                     "tile_primitives_per_launch": proc // n_probe, "flops_per_hit": flops_per_hit,
+                     "measured_mfma_peak": mfma_probe},
         "stages": {"bin_ms": round(bin_ms / n_probe, 4), "sort_ms": round(sort_ms / n_probe, 4),
                    "render_ms": round(kernel_ms / n_probe, 4),
                    "sort_hbm": {"bound": "hbm", "achieved": round(sort_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                                 "frac": round(sort_gbs / HBM_PEAK_GBS, 5)},
+                   "bin_hbm": {"bound": "hbm", "achieved": round(bin_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                               "frac": round(bin_gbs / HBM_PEAK_GBS, 5)},
                    "candidates_per_launch": cand_total // n_probe},
     }
 

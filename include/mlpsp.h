@@ -234,6 +234,12 @@ int mlpsp_render_tilecenter_mfma_feat(const float* rays_o_dev, const float* rays
                                       float* out_rgb_dev, float* out_alpha_dev, float* out_feat_dev,
                                       int32_t* status_dev, int64_t* counters_dev, mlpsp_stream_t stream);
 
+/* Measurement aid, no counterpart in the reference: launches a kernel that does nothing but
+ * v_mfma_f32_32x32x16_bf16 on register operands (2,048 workgroups x 4 wavefronts x iterations x 8
+ * instructions) and returns the FLOPs it issues (-1 on error); time it on the stream to see what the
+ * chip sustains next to the data-sheet peak.  sink_dev: one float, left untouched in practice. */
+int64_t mlpsp_probe_mfma_bf16(int iterations, float* sink_dev, mlpsp_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -529,6 +529,25 @@ __global__ __launch_bounds__(256) void feat_gemm_kernel(const unsigned* __restri
   }
 }
 
+// Measurement aid: what the chip sustains on v_mfma_f32_32x32x16_bf16 when nothing else is in the way.
+// Every wavefront runs `iterations` rounds of 8 independent accumulations on register operands.
+__global__ __launch_bounds__(256) void probe_mfma_bf16_kernel(int iterations, float* __restrict__ sink) {
+  u32x4 a = {0x3f803f80u + threadIdx.x, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u}, b = a;
+  f32x16 acc[8];
+#pragma unroll
+  for (int k = 0; k < 8; ++k)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[k][r] = 0.f;
+  for (int it = 0; it < iterations; ++it) {
+#pragma unroll
+    for (int k = 0; k < 8; ++k) acc[k] = Ops<__bf16>::mfma(a, b, acc[k]);
+  }
+  float v = 0.f;
+#pragma unroll
+  for (int k = 0; k < 8; ++k) v += acc[k][0];
+  if (v == 12345.678f) sink[0] = v;      // keeps the accumulations alive; practically never true
+}
+
 }  // namespace mlpsp
 
 using namespace mlpsp;
@@ -672,4 +691,12 @@ MLPSP_API int mlpsp_render_tilecenter_mfma(const float* rays_o_dev, const float*
                                            freq_dev, att_dev, packed_dev, num_primitives, use_bf16, nullptr, 0, 0, 0.f,
                                            0.f, width, height, threshold, nullptr, 0, out_rgb_dev, out_alpha_dev,
                                            nullptr, status_dev, counters_dev, stream);
+}
+
+MLPSP_API int64_t mlpsp_probe_mfma_bf16(int iterations, float* sink_dev, mlpsp_stream_t stream) {
+  if (iterations <= 0 || !sink_dev) return -1;
+  const int blocks = 256 * 8;      // 8 workgroups of 4 wavefronts per CU: two wavefronts per SIMD
+  hipLaunchKernelGGL(probe_mfma_bf16_kernel, dim3(blocks), dim3(256), 0, (hipStream_t)stream, iterations, sink_dev);
+  if (hipGetLastError() != hipSuccess) return -1;
+  return (int64_t)blocks * 4 * iterations * 8 * (2LL * 32 * 32 * 16);   // FLOPs issued
 }
