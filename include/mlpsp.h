@@ -145,6 +145,30 @@ int mlpsp_render_tilecenter_stats_f32(const float* rays_o_dev, const float* rays
                                       float* stat_max_w_dev, int32_t* stat_hits_dev, float* stat_sum_werr_dev,
                                       int32_t* stat_contrib_dev, mlpsp_stream_t stream);
 
+/* Training-records forward (render_tiles_training_records, np_tile_kernels.cu:6897-6998; kernel :2925-3206
+ * in record modes 1 and 3).  t* order, f32, hidden <= 32.  Per pixel, one record per hit taken while the
+ * pixel is live (T >= 1e-3) and holds fewer than max_hits records: ids [R], x6 [R,6] (ray direction, world
+ * offset), masks [R,2] (ReLU bit masks of the two hidden layers), raw [R,8] (R, G, B, sigma_raw, T before the
+ * hit, alpha, decay, sigma logit), gates [R,4]; rgb/alpha are the composite of the records.
+ * Step 1 (count): counts_dev [B] int32.  The caller scans them into record_offsets_dev [B+1] int64
+ * (exclusive) and allocates R = record_offsets[B] records.  Step 2 (emit) writes them.
+ * overflow_dev (int32, zeroed by the count step): 1 if a live pixel reached max_hits -- the reference
+ * raises "hit capacity" then (:4601-4609); nothing is truncated silently. */
+int mlpsp_records_count(const float* rays_o_dev, const float* rays_d_dev, const void* prim_records_dev,
+                        const int32_t* order_dev, const int32_t* tile_offsets_dev, const float* freq_dev,
+                        const float* att_dev, int num_frequencies, const float* W1, const float* b1, const float* W2,
+                        const float* b2, const float* W3, const float* b3, int num_primitives, int hidden, int width,
+                        int height, int tile_w, int tile_h, float threshold, int max_hits, int32_t* counts_dev,
+                        int32_t* overflow_dev, mlpsp_stream_t stream);
+int mlpsp_records_emit(const float* rays_o_dev, const float* rays_d_dev, const void* prim_records_dev,
+                       const int32_t* order_dev, const int32_t* tile_offsets_dev, const float* freq_dev,
+                       const float* att_dev, int num_frequencies, const float* W1, const float* b1, const float* W2,
+                       const float* b2, const float* W3, const float* b3, int num_primitives, int hidden, int width,
+                       int height, int tile_w, int tile_h, float threshold, int max_hits, float gating_beta,
+                       float gating_temp, const int64_t* record_offsets_dev, int32_t* ids_dev, float* x6_dev,
+                       int32_t* masks_dev, float* raw_dev, float* gates_dev, float* out_rgb_dev, float* out_alpha_dev,
+                       int32_t* overflow_dev, mlpsp_stream_t stream);
+
 /* Workspace of the feature renders below.  The render kernel hands the feature kernel one "hit record"
  * per (64-pixel wavefront of a tile, primitive that hits one of its pixels); how many there will be is
  * only known after the frame (early termination), so records come from a pool of pool_records records.

@@ -11,9 +11,14 @@ struct MlpPtrs {
 // Fixed-shape MLP, fully unrolled: activations live in VGPRs, weights arrive as scalar operands.
 // Accumulation order per hidden unit is that of np_tile_kernels.cu:2050-2089: start from the bias,
 // then for j = c*F+f ascending add W1[h][j]*sin_j and W1[h][j+6F]*cos_j.
-template <int H, int F>
+//
+// REC selects the arithmetic of the record kernels (mlp_eval_rgb_sigma, np_tile_kernels.cu:313-381): layer 2 is
+// bias + (fma chain started at zero) there, which rounds differently from the chain started at the bias,
+// and masks[l] receives bit h iff hidden unit h of layer l+1 is positive (:371-379).
+template <int H, int F, bool REC = false>
 __device__ __forceinline__ void mlp_fixed(const float x6[6], const float* __restrict__ freq,
-                                          const float* __restrict__ att, const MlpPtrs& m, int p, float out[4]) {
+                                          const float* __restrict__ att, const MlpPtrs& m, int p, float out[4],
+                                          uint32_t* masks = nullptr) {
   constexpr int IN = 12 * F, HALF = 6 * F;
   float sn[HALF], cs[HALF];
 #pragma unroll
@@ -43,9 +48,10 @@ __device__ __forceinline__ void mlp_fixed(const float x6[6], const float* __rest
   }
 #pragma unroll
   for (int o = 0; o < H; ++o) {
-    float acc = bb2[o];
+    float acc = REC ? 0.f : bb2[o];
 #pragma unroll
     for (int h = 0; h < H; ++h) acc = fmaf(w2[o * H + h], h1[h], acc);
+    if constexpr (REC) acc = bb2[o] + acc;
     h2[o] = acc > 0.f ? acc : 0.f;
   }
 #pragma unroll
@@ -55,13 +61,24 @@ __device__ __forceinline__ void mlp_fixed(const float x6[6], const float* __rest
     for (int h = 0; h < H; ++h) acc = fmaf(w3[k * H + h], h2[h], acc);
     out[k] = acc;
   }
+  if constexpr (REC) {
+    uint32_t m1 = 0u, m2 = 0u;
+#pragma unroll
+    for (int h = 0; h < H && h < 32; ++h) {
+      m1 |= (h1[h] > 0.f) ? (1u << h) : 0u;
+      m2 |= (h2[h] > 0.f) ? (1u << h) : 0u;
+    }
+    masks[0] = m1;
+    masks[1] = m2;
+  }
 }
 
 // Any H <= 64, F <= 16: same order, run-time loops (activations spill to scratch; used for the
 // odd shapes only).
+template <bool REC = false>
 static __device__ __noinline__ void mlp_generic(const float x6[6], const float* __restrict__ freq,
                                          const float* __restrict__ att, int F, int H, const MlpPtrs& m, int p,
-                                         float out[4]) {
+                                         float out[4], uint32_t* masks = nullptr) {
   const int IN = 12 * F, HALF = 6 * F;
   float h1[64], h2[64];
   const float* w1 = m.W1 + (size_t)p * H * IN;
@@ -84,8 +101,9 @@ static __device__ __noinline__ void mlp_generic(const float x6[6], const float* 
   }
   for (int h = 0; h < H; ++h) h1[h] = h1[h] > 0.f ? h1[h] : 0.f;
   for (int o = 0; o < H; ++o) {
-    float acc = bb2[o];
+    float acc = REC ? 0.f : bb2[o];
     for (int h = 0; h < H; ++h) acc = fmaf(w2[o * H + h], h1[h], acc);
+    if constexpr (REC) acc = bb2[o] + acc;
     h2[o] = acc > 0.f ? acc : 0.f;
   }
   for (int k = 0; k < 4; ++k) {
@@ -93,15 +111,24 @@ static __device__ __noinline__ void mlp_generic(const float x6[6], const float* 
     for (int h = 0; h < H; ++h) acc = fmaf(w3[k * H + h], h2[h], acc);
     out[k] = acc;
   }
+  if constexpr (REC) {
+    uint32_t m1 = 0u, m2 = 0u;
+    for (int h = 0; h < H && h < 32; ++h) {
+      m1 |= (h1[h] > 0.f) ? (1u << h) : 0u;
+      m2 |= (h2[h] > 0.f) ? (1u << h) : 0u;
+    }
+    masks[0] = m1;
+    masks[1] = m2;
+  }
 }
 
 // HT > 0: fixed shape (fully unrolled); HT == 0: run-time H and F.
-template <int HT, int FT>
+template <int HT, int FT, bool REC = false>
 __device__ __forceinline__ void mlp_eval(const float x6[6], const float* __restrict__ freq,
                                          const float* __restrict__ att, int F, int H, const MlpPtrs& m, int p,
-                                         float out[4]) {
-  if constexpr (HT > 0) mlp_fixed<HT, FT>(x6, freq, att, m, p, out);
-  else mlp_generic(x6, freq, att, F, H, m, p, out);
+                                         float out[4], uint32_t* masks = nullptr) {
+  if constexpr (HT > 0) mlp_fixed<HT, FT, REC>(x6, freq, att, m, p, out, masks);
+  else mlp_generic<REC>(x6, freq, att, F, H, m, p, out, masks);
 }
 
 }  // namespace mlpsp

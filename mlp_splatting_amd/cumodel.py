@@ -64,6 +64,14 @@ def _tile_capacity_from_env() -> int:
     return int(os.environ.get("MLPSP_TILE_CANDIDATE_CAPACITY", "1536"))
 
 
+def _max_hits_from_env() -> int:
+    """MLPSP_TILECENTER_MAX_HITS of the selected build: MLPSP_CSR_MAX_HITS in the csr backend
+    (scannet/cumodel.py:106-113), else the kernel's default 512 (np_tile_kernels.cu:48-50)."""
+    if os.environ.get("MLPSP_TRAINING_BACKEND", "legacy") == "csr":
+        return int(os.environ.get("MLPSP_CSR_MAX_HITS", "128"))
+    return 512
+
+
 class IntegratedPositionalEncoding(nn.Module):
     """freq_k = 2^k pi; the attenuation exp(-freq^2 sigma^2 / 2) scales the phase
     (scannet/cumodel.py:132-155)."""
@@ -270,7 +278,7 @@ class NeuralPrimitiveSceneTileCUDA(nn.Module):
         key, _name, _flags = _tile_ext_build_config()
         if _tile_ext is None or _tile_ext_key != key:
             from .tile_ext import TileExt
-            _tile_ext = TileExt(max_tile_prims=_tile_capacity_from_env())
+            _tile_ext = TileExt(max_tile_prims=_tile_capacity_from_env(), max_hits=_max_hits_from_env())
             _tile_ext_key = key
         return _tile_ext
 

@@ -176,6 +176,44 @@ def render_tilecenter_stats_f32(rays_o, rays_d, records, order, tile_offsets, fr
     return rgb, alpha
 
 
+def training_records(rays_o, rays_d, records, order, tile_offsets, freq, att, W1, b1, W2, b2, W3, b3, W, H, TW, TH,
+                     threshold, beta, temp, max_hits, path_name="render_tiles_training_records"):
+    """Training-records forward -> (rgb, alpha, ids, x6, raw, masks, gates, offsets int64 [B+1]);
+    raises the reference's hit-capacity error (np_tile_kernels.cu:4601-4609)."""
+    dev = rays_o.device
+    lib = _lib.load()
+    B = W * H
+    n, hidden, F = W1.shape[0], W2.shape[1], freq.shape[0]
+    counts = torch.zeros(B, dtype=torch.int32, device=dev)
+    overflow = torch.empty(1, dtype=torch.int32, device=dev)
+    head = (_ptr(rays_o), _ptr(rays_d), _ptr(records), _ptr(order), _ptr(tile_offsets), _ptr(freq), _ptr(att), F,
+            _ptr(W1), _ptr(b1), _ptr(W2), _ptr(b2), _ptr(W3), _ptr(b3), n, hidden, W, H, TW, TH, float(threshold),
+            int(max_hits))
+
+    def refuse():
+        raise RuntimeError(f"{path_name}: tile-center backward hit capacity {int(max_hits)} reached before "
+                           "transmittance termination; refusing to return truncated gradients")
+
+    _check(lib.mlpsp_records_count(*head, _ptr(counts), _ptr(overflow), _stream(dev)), "mlpsp_records_count")
+    offsets = torch.zeros(B + 1, dtype=torch.int64, device=dev)
+    torch.cumsum(counts, 0, out=offsets[1:])
+    total, over = int(offsets[-1].item()), int(overflow.item())
+    if over:
+        refuse()
+    ids = torch.empty(total, dtype=torch.int32, device=dev)
+    x6 = torch.empty(total, 6, dtype=torch.float32, device=dev)
+    masks = torch.empty(total, 2, dtype=torch.int32, device=dev)
+    raw = torch.empty(total, 8, dtype=torch.float32, device=dev)
+    gates = torch.empty(total, 4, dtype=torch.float32, device=dev)
+    rgb = torch.zeros(B, 3, dtype=torch.float32, device=dev)
+    alpha = torch.zeros(B, 1, dtype=torch.float32, device=dev)
+    if total:
+        _check(lib.mlpsp_records_emit(*head, float(beta), float(temp), _ptr(offsets), _ptr(ids), _ptr(x6), _ptr(masks),
+                                      _ptr(raw), _ptr(gates), _ptr(rgb), _ptr(alpha), _ptr(overflow), _stream(dev)),
+               "mlpsp_records_emit")
+    return rgb, alpha, ids, x6, raw, masks, gates, offsets
+
+
 def _feat_shape(feat_attr):
     """(slots, channels) with the reference's checks (np_tile_kernels.cu:6158-6169)."""
     if not (feat_attr.is_cuda and feat_attr.dtype == torch.float32 and feat_attr.dim() in (2, 3)):

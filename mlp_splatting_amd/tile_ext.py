@@ -23,7 +23,7 @@ _BACKWARD_ONLY = (
     "render_tiles_backward_emit_per_pixel", "render_tiles_backward_emit_tilecenter",
     "render_tiles_backward_featattr_per_pixel", "render_tiles_backward_featattr_tilecenter",
     "render_tiles_backward_tilecenter_full", "render_tiles_backward_tilecenter_full_with_feat",
-    "render_tiles_mlp_records", "render_tiles_training_records", "render_tiles_training_records_wmma",
+    "render_tiles_mlp_records", "render_tiles_training_records_wmma",
     "primitive_records_reverse", "render_tiles_backward_tilecenter_traversal",
     "render_tiles_backward_tilecenter_backprop_noatomic", "training_wmma_safety_stats",
 )
@@ -41,9 +41,10 @@ def _is_f32_2d(t, cols):
 class TileExt:
     """Forward entry points of the tile renderer on one MI355X."""
 
-    def __init__(self, max_tile_prims: int = MAX_TILE_PRIMS):
+    def __init__(self, max_tile_prims: int = MAX_TILE_PRIMS, max_hits: int = 512):
         _lib.load()  # fail now, loudly, if the HIP library is absent
         self.max_tile_prims = int(max_tile_prims)
+        self.max_hits = int(max_hits)          # MLPSP_TILECENTER_MAX_HITS (np_tile_kernels.cu:48-50, 67-69)
         self._lock = threading.Lock()
         self._mfma_calls = 0
         self._mfma_fallbacks = 0
@@ -244,6 +245,41 @@ class TileExt:
         _chk(feat_attr.shape[0] == base[2].shape[0], "feat_attr first dimension must match primitive count")
         ops._feat_shape(feat_attr)
         return self._per_pixel((*base, *dims), "render_tiles_forward_per_pixel_with_feat", (feat_attr, beta, temp))
+
+    # ------------------------------------------------------------------------------------------
+    # training-records forward (np_tile_kernels.cu:6897-6998, forward_only = true)
+    # ------------------------------------------------------------------------------------------
+    def render_tiles_training_records(self, x, width, height, tile, threshold, beta, temp):
+        """[rgb, alpha, ids, x6, raw, masks, gates, offsets]: one record per hit and pixel, in each
+        pixel's compositing order.  ``x`` = the 15 scene tensors + two adjoint placeholders that the
+        forward-only mode never reads (scannet/csr_training.py:37-39)."""
+        name = "render_tiles_mlp_records"
+        _chk(len(x) == 17, "Expected 15 scene inputs and RGB/T adjoints")
+        width, height, tile = int(width), int(height), int(tile)
+        _chk(width > 0 and height > 0 and tile in (8, 16))
+        for i, t in enumerate(x):
+            _chk(t.is_cuda and t.is_contiguous(), "Inputs must be contiguous CUDA tensors")
+            _chk(t.device == x[0].device, "Inputs must share a device")
+            _chk(t.dtype == (torch.int32 if i in (5, 6) else torch.float32),
+                 "Records path requires FP32 inputs and int32 tile lists")
+        pixels, n = width * height, x[2].shape[0]
+        _chk(tuple(x[0].shape) == (pixels, 3) and x[1].shape == x[0].shape)
+        _chk(x[2].dim() == 2 and x[2].shape[1] == 3 and x[3].shape == x[2].shape and tuple(x[4].shape) == (n, 4))
+        _chk(x[7].dim() == 1 and x[8].shape == x[7].shape and x[9].dim() == 3 and x[9].shape[0] == n)
+        h, inp, f = x[9].shape[1], x[9].shape[2], x[7].numel()
+        _chk(0 < h <= 32 and f > 0 and inp == 12 * f)
+        _chk(tuple(x[10].shape) == (n, h) and tuple(x[11].shape) == (n, h, h) and x[12].shape == x[10].shape)
+        _chk(tuple(x[13].shape) == (n, 4, h) and tuple(x[14].shape) == (n, 4))
+        _chk(x[15].shape == x[0].shape and x[16].dim() == 1 and x[16].numel() == pixels)
+        with torch.cuda.device(x[0].device):
+            self._validate(x[5], x[6], ops.num_tiles(width, height, tile, tile), self.max_tile_prims, n, name)
+            rec = self._records(x[2], x[3], x[4])
+            order = x[5]
+            if x[5].numel() > 0:
+                order, _ = ops.sort_tiles(x[0], x[1], rec, x[5], x[6], width, height, tile, tile, _lib.KEY_TSTAR,
+                                          self.max_tile_prims, cull_threshold=float(threshold))
+            return list(ops.training_records(x[0], x[1], rec, order, x[6], x[7], x[8], *x[9:15], width, height, tile,
+                                             tile, float(threshold), float(beta), float(temp), self.max_hits, name))
 
     # ------------------------------------------------------------------------------------------
     # statistics forward (pruning statistics are not rebuilt; the render itself is)

@@ -25,6 +25,8 @@
 //   legacy + tile-view binning ........................... pinned by brute force over the dense predicate
 //   ray-cone binning ..................................... pinned by the reference's own brute-force test
 //   gates / feature ...................................... pinned by softmax closed form + framebuffer sum
+//   training records ..................................... pinned by recomposition (sum T a c = rgb,
+//       T' = T (1 - a)), the forward image within 2e-6, masks against an einsum restatement
 //   pruning statistics ................................... pinned by the geometric-series weights of
 //       stacked identical primitives and by sum_p sum_w[p] = sum_pixels alpha
 //   bf16/fp16 mixed-precision MLP ........................ pinned against a numpy emulation of the
@@ -292,6 +294,53 @@ inline void mlp_f32(const float x6[6], const float* freq, const float* att, cons
     o3 = fmaf(M.W3[3 * H + h], hi, o3);
   }
   out[0] = o0; out[1] = o1; out[2] = o2; out[3] = o3;
+}
+
+// The MLP as the record kernels evaluate it (mlp_eval_rgb_sigma, scannet/cuda/np_tile_kernels.cu:313-381):
+// layer 1 and 3 as above, layer 2 as bias + (fma chain started at zero) (:349-353, row_dot_vec :208-212),
+// which rounds differently from the forward kernels' chain started at the bias; masks[l] has bit h set
+// iff hidden unit h of layer l+1 is positive after ReLU (:371-379).
+inline void mlp_f32_records(const float x6[6], const float* freq, const float* att, const MlpView& M, float out[4],
+                            uint32_t masks[2]) {
+  float h1[MAXH], h2[MAXH];
+  const int H = M.H, IN = M.IN, F = M.F, cos_off = IN / 2;
+  for (int h = 0; h < H; ++h) h1[h] = M.b1[h];
+  for (int c = 0; c < 6; ++c) {
+    for (int f = 0; f < F; ++f) {
+      const float xproj = (x6[c] * freq[f]) * att[f];
+      const int j = c * F + f;
+      float s, co;
+      det_sincos(xproj, &s, &co);
+      for (int h = 0; h < H; ++h) {
+        const float* Wi = M.W1 + (size_t)h * IN;
+        h1[h] = fmaf(Wi[j], s, h1[h]);
+        h1[h] = fmaf(Wi[j + cos_off], co, h1[h]);
+      }
+    }
+  }
+  for (int h = 0; h < H; ++h) h1[h] = h1[h] > 0.f ? h1[h] : 0.f;
+  for (int o = 0; o < H; ++o) {
+    const float* row = M.W2 + (size_t)o * H;
+    float dot = 0.f;
+    for (int h = 0; h < H; ++h) dot = fmaf(row[h], h1[h], dot);
+    const float acc = M.b2[o] + dot;
+    h2[o] = acc > 0.f ? acc : 0.f;
+  }
+  float o0 = M.b3[0], o1 = M.b3[1], o2 = M.b3[2], o3 = M.b3[3];
+  for (int h = 0; h < H; ++h) {
+    const float hi = h2[h];
+    o0 = fmaf(M.W3[0 * H + h], hi, o0);
+    o1 = fmaf(M.W3[1 * H + h], hi, o1);
+    o2 = fmaf(M.W3[2 * H + h], hi, o2);
+    o3 = fmaf(M.W3[3 * H + h], hi, o3);
+  }
+  out[0] = o0; out[1] = o1; out[2] = o2; out[3] = o3;
+  uint32_t m1 = 0, m2 = 0;
+  for (int h = 0; h < H && h < 32; ++h) {
+    if (h1[h] > 0.f) m1 |= (1u << h);
+    if (h2[h] > 0.f) m2 |= (1u << h);
+  }
+  masks[0] = m1; masks[1] = m2;
 }
 
 // Mixed-precision MLP, rounding points of scannet/cuda/rgb_wmma.cuh:144-213: encoded inputs and
@@ -892,6 +941,106 @@ ORACLE_API void mlpsp_oracle_render_stats(
       }
     }
   }
+}
+
+// ------------------------------------------------------------------------------------------
+// Training-records forward: scannet/cuda/np_tile_kernels.cu:2925-3206 (modes 1 and 3), wrapper
+// :6897-6998.  t* order, f32, hidden <= 32.  Per pixel, for every hit taken while the pixel is live
+// (T >= 1e-3) and has fewer than max_hits records: id, x6 = (ray direction, world offset), ReLU masks,
+// raw = (R, G, B, sigma_raw, T before the hit, alpha, decay, sigma logit), gates; rgb and alpha are the
+// composite of those records.  A live pixel that already holds max_hits records sets *overflow (the
+// reference then raises "hit capacity", :3166-3168, 4601-4609).
+// Two-phase: ids == nullptr -> counts[B] only; else records are written at offsets[pix] + k.
+// ------------------------------------------------------------------------------------------
+ORACLE_API void mlpsp_oracle_records(
+    const float* rays_o, const float* rays_d, const float* pos, const float* logs, const float* quats,
+    const int32_t* cand, const int32_t* offsets, const float* freq, const float* att, int F,
+    const float* W1, const float* b1, const float* W2, const float* b2, const float* W3, const float* b3,
+    int N, int H, int Wimg, int Himg, int TW, int TH, float thr, int capacity, int max_hits, float beta, float temp,
+    int32_t* counts, int32_t* overflow, const int64_t* rec_offsets, int32_t* ids, float* x6_out, int32_t* masks_out,
+    float* raw_out, float* gates_out, float* out_rgb, float* out_alpha, int nthreads) {
+  Scene S{};
+  S.rays_o = rays_o; S.rays_d = rays_d; S.pos = pos; S.logs = logs; S.quats = quats;
+  S.cand = cand; S.offsets = offsets; S.freq = freq; S.att = att; S.F = F;
+  S.W1 = W1; S.b1 = b1; S.W2 = W2; S.b2 = b2; S.W3 = W3; S.b3 = b3; S.N = N; S.H = H;
+  S.Wimg = Wimg; S.Himg = Himg; S.TW = TW; S.TH = TH; S.thr = thr;
+  const int ntx = (Wimg + TW - 1) / TW, nty = (Himg + TH - 1) / TH, T = ntx * nty, npx = TW * TH;
+  int ovf = 0;
+  if (nthreads <= 0) nthreads = omp_get_max_threads();
+#pragma omp parallel num_threads(nthreads) reduction(| : ovf)
+  {
+    std::vector<KeyId> buf;
+    std::vector<float> trans(npx), cr(npx), cg(npx), cb(npx);
+    std::vector<int> used(npx), pixidx(npx);
+#pragma omp for schedule(dynamic, 4)
+    for (int tile = 0; tile < T; ++tile) {
+      const int tx = tile % ntx, ty = tile / ntx;
+      for (int k = 0; k < npx; ++k) {
+        const int x = tx * TW + k % TW, y = ty * TH + k / TW;
+        pixidx[k] = (x < Wimg && y < Himg) ? (y * Wimg + x) : -1;
+        trans[k] = 1.f; cr[k] = cg[k] = cb[k] = 0.f; used[k] = 0;
+      }
+      sort_tile(S, tile, 1, capacity, buf);
+      for (size_t i = 0; i < buf.size(); ++i) {
+        const int p = buf[i].id;
+        int nactive = 0;
+        if (p >= 0 && p < N) {
+          const Prim P = load_prim(pos, logs, quats, p);
+          const MlpView M = mlp_of(S, p);
+          for (int k = 0; k < npx; ++k) {
+            const int pix = pixidx[k];
+            if (pix < 0 || trans[k] < 1e-3f || used[k] >= max_hits) continue;
+            Hit h;
+            const float* ro = rays_o + (size_t)pix * 3;
+            const float* rd = rays_d + (size_t)pix * 3;
+            if (!hit_rot(ro[0], ro[1], ro[2], rd[0], rd[1], rd[2], P, thr, h)) continue;
+            const float v6[6] = {rd[0], rd[1], rd[2], h.dx, h.dy, h.dz};
+            float o[4];
+            uint32_t mk[2];
+            mlp_f32_records(v6, freq, att, M, o, mk);
+            const float R = o_sigmoid(o[0]), G = o_sigmoid(o[1]), Bc = o_sigmoid(o[2]);
+            const float sigma_raw = o_softplus(o[3]);
+            const float sigma = sigma_raw * h.decay;
+            const float alpha = 1.f - det_exp(-sigma);
+            if (ids) {
+              const int64_t r = rec_offsets[pix] + used[k];
+              ids[r] = p;
+              for (int c = 0; c < 6; ++c) x6_out[r * 6 + c] = v6[c];
+              masks_out[r * 2] = (int32_t)mk[0];
+              masks_out[r * 2 + 1] = (int32_t)mk[1];
+              float* raw = raw_out + r * 8;
+              raw[0] = R; raw[1] = G; raw[2] = Bc; raw[3] = sigma_raw;
+              raw[4] = trans[k]; raw[5] = alpha; raw[6] = h.decay; raw[7] = o[3];
+              tetra_gates(h.qlx, h.qly, h.qlz, P.lgx, P.lgy, P.lgz, beta, temp, gates_out + r * 4);
+              const float weight = trans[k] * alpha;
+              cr[k] = fmaf(weight, R, cr[k]);
+              cg[k] = fmaf(weight, G, cg[k]);
+              cb[k] = fmaf(weight, Bc, cb[k]);
+            }
+            trans[k] *= (1.f - alpha);
+            ++used[k];
+          }
+        }
+        for (int k = 0; k < npx; ++k) {
+          if (pixidx[k] < 0 || trans[k] < 1e-3f) continue;
+          ++nactive;
+          if (used[k] >= max_hits) ovf |= 1;
+        }
+        if (nactive == 0) break;
+      }
+      for (int k = 0; k < npx; ++k) {
+        const int pix = pixidx[k];
+        if (pix < 0) continue;
+        if (!ids) {
+          counts[pix] = used[k];
+        } else {
+          out_rgb[pix * 3 + 0] = cr[k]; out_rgb[pix * 3 + 1] = cg[k]; out_rgb[pix * 3 + 2] = cb[k];
+          out_alpha[pix] = 1.f - trans[k];
+        }
+      }
+    }
+  }
+  if (overflow) *overflow = ovf;
 }
 
 // ------------------------------------------------------------------------------------------

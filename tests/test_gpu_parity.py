@@ -324,3 +324,47 @@ def test_statistics_forward_against_oracle(device, oracle_mod, tile, hidden):
     st2 = [torch.zeros(n, device=device, dtype=dt) for dt in (torch.float32, torch.float32, torch.int32)]
     ops.render_tilecenter_stats_f32(*args, *st2)
     assert np.array_equal(st2[2].cpu().numpy(), want["hits"])
+
+
+@pytest.mark.parametrize("tile,hidden,n", [(8, 32, 1500), (16, 16, 2500), (8, 8, 900)])
+def test_training_records_are_bit_exact(device, oracle_mod, tile, hidden, n):
+    # np_tile_kernels.cu:2925-3206 (record modes 1/3): counts, order, every record field, rgb, alpha
+    from mlp_splatting_amd.tile_ext import TileExt
+    fr = Frame("cfg1_5k_160x120", n=n, hidden=hidden, width=72, height=48, tile=tile)
+    cand, off = fr.oracle_lists(oracle_mod)
+    want = oracle_mod.records(*fr.base_numpy(cand, off), *fr.dims, max_hits=512, beta=1.3, temp=2.2)
+    x = [_t(a, device) for a in fr.base_numpy(cand, off)]
+    x += [torch.zeros_like(x[0]), torch.zeros(fr.W * fr.H, device=device)]
+    ext = TileExt()
+    rgb, alpha, ids, x6, raw, masks, gates, offsets = ext.render_tiles_training_records(x, fr.W, fr.H, tile, fr.thr, 1.3, 2.2)
+    assert offsets.dtype == torch.int64 and np.array_equal(offsets.cpu().numpy(), want["offsets"])
+    assert want["offsets"][-1] > 5000 and np.array_equal(ids.cpu().numpy(), want["ids"])
+    assert np.array_equal(masks.cpu().numpy(), want["masks"])
+    for got, key in ((rgb, "rgb"), (alpha, "alpha"), (x6, "x6"), (raw, "raw"), (gates, "gates")):
+        _assert_bits(got, want[key], key)
+    # primitive-major grouping of those records (scannet/primitive_csr.py:14-29)
+    from mlp_splatting_amd.primitive_csr import group_records
+    csr = group_records(ids, x6, raw[:, :4].contiguous(), fr.scene.n, masks)
+    counts = np.bincount(want["ids"], minlength=fr.scene.n)
+    assert np.array_equal(np.diff(csr.offsets.cpu().numpy()), counts)
+    order = csr.record_indices.cpu().numpy()
+    assert np.array_equal(want["ids"][order], np.sort(want["ids"], kind="stable"))
+    assert np.array_equal(order, np.argsort(want["ids"], kind="stable"))
+
+
+def test_training_records_hit_capacity_is_an_error(device, oracle_mod):
+    from mlp_splatting_amd.tile_ext import TileExt
+    fr = Frame("cfg1_5k_160x120", n=1500, hidden=32, width=32, height=24)
+    cand, off = fr.oracle_lists(oracle_mod)
+    want = oracle_mod.records(*fr.base_numpy(cand, off), *fr.dims, max_hits=512)
+    deepest = int(np.diff(want["offsets"]).max())
+    assert deepest > 8
+    x = [_t(a, device) for a in fr.base_numpy(cand, off)]
+    x += [torch.zeros_like(x[0]), torch.zeros(fr.W * fr.H, device=device)]
+    assert oracle_mod.records(*fr.base_numpy(cand, off), *fr.dims, max_hits=deepest - 1)["overflow"]
+    with pytest.raises(RuntimeError, match=f"hit capacity {deepest - 1} reached before transmittance termination"):
+        TileExt(max_hits=deepest - 1).render_tiles_training_records(x, fr.W, fr.H, 8, fr.thr, 1.5, 2.0)
+    # empty lists: empty records, zero image
+    x[5], x[6] = torch.zeros(0, dtype=torch.int32, device=device), torch.zeros_like(x[6])
+    out = TileExt().render_tiles_training_records(x, fr.W, fr.H, 8, fr.thr, 1.5, 2.0)
+    assert out[2].numel() == 0 and int(out[7][-1]) == 0 and float(out[0].abs().max()) == 0.0

@@ -374,3 +374,71 @@ def test_statistics_sum_to_the_image_alpha_and_order_by_plain_depth(oracle_mod):
     assert 0 < out["hits"].sum() <= plain["stats"][3]      # hits with w > 1e-8 among all evaluated hits
     assert (out["max_w"] <= out["sum_w"] + 1e-12).all() and (out["contrib"] <= out["hits"]).all()
     assert (out["sum_werr"] <= 3.0 * out["sum_w"] + 1e-9).all() and out["contrib"].sum() > 0
+
+
+# ---------------------------------------------------------------------------------------------
+# training records (np_tile_kernels.cu:2925-3206 modes 1/3, wrapper :6897-6998)
+# ---------------------------------------------------------------------------------------------
+def test_records_of_a_zero_weight_stack(oracle_mod):
+    # tests/test_training_wmma.py:103-139 style: n coincident primitives on one pixel
+    n, b3 = 9, [0.4, -0.3, 0.9, 0.5]
+    s = stack_scene(n, b3=b3)
+    out = oracle_mod.records(*base(s), *DIMS1)
+    a = 1.0 - np.exp(-np.log1p(np.exp(b3[3])))
+    k = next(i for i in range(1, 100) if (1 - a) ** i < 1e-3)
+    m = min(n, k)
+    assert not out["overflow"] and out["offsets"].tolist() == [0, m] and out["ids"].tolist() == list(range(m))
+    raw = out["raw"]
+    np.testing.assert_allclose(raw[:, :3], np.tile(1 / (1 + np.exp(-np.array(b3[:3]))), (m, 1)), rtol=2e-6)
+    np.testing.assert_allclose(raw[:, 3], np.log1p(np.exp(b3[3])), rtol=2e-6)       # softplus
+    np.testing.assert_allclose(raw[:, 4], (1 - a) ** np.arange(m), rtol=1e-5)        # T before each hit
+    np.testing.assert_allclose(raw[:, 5], a, rtol=2e-6)
+    assert np.all(raw[:, 6] == 1.0) and np.all(raw[:, 7] == np.float32(b3[3]))       # decay on the centre ray, logit
+    assert np.array_equal(out["x6"], np.tile(np.array([[0, 0, 1, 0, 0, 0]], np.float32), (m, 1)))
+    assert np.all(out["masks"] == 0)                                                  # zero weights, zero biases
+    np.testing.assert_allclose(out["gates"], 0.25)                                    # q = 0: uniform gates
+    # hit capacity (np_tile_kernels.cu:3166-3168): a pixel that is still live with max_hits records overflows,
+    # even at the end of its list; one that saturated in time does not
+    assert oracle_mod.records(*base(s), *DIMS1, max_hits=3)["overflow"]
+    assert oracle_mod.records(*base(stack_scene(3, b3=b3)), *DIMS1, max_hits=3)["overflow"]
+    opaque = oracle_mod.records(*base(stack_scene(5, b3=[0, 0, 0, 20.0])), *DIMS1, max_hits=1)
+    assert not opaque["overflow"] and opaque["offsets"].tolist() == [0, 1]
+
+
+def test_records_recompose_the_image_and_match_the_forward_render(oracle_mod):
+    from helpers import Frame
+    fr = Frame("cfg1_5k_160x120", n=700, hidden=16, width=40, height=24)
+    sc = fr.scene
+    cand, off = fr.oracle_lists(oracle_mod)
+    out = oracle_mod.records(*fr.base_numpy(cand, off), *fr.dims, max_hits=512, beta=1.3, temp=2.2)
+    fwd = oracle_mod.render_tilecenter(*fr.base_numpy(cand, off), *fr.dims)
+    assert not out["overflow"] and out["offsets"][-1] == fwd["stats"][3] > 5000      # one record per evaluated hit
+    # tests/test_primitive_csr.py:49-53: records-forward image == tile-centre forward within 2e-6
+    np.testing.assert_allclose(out["rgb"], fwd["rgb"], atol=2e-6)
+    np.testing.assert_allclose(out["alpha"], fwd["alpha"], atol=2e-6)
+    offs, raw, ids = out["offsets"], out["raw"].astype(np.float64), out["ids"]
+    pix_of = np.repeat(np.arange(fr.W * fr.H), np.diff(offs))
+    first = np.zeros(len(ids), bool)
+    first[offs[:-1][np.diff(offs) > 0]] = True
+    assert np.all(raw[first, 4] == 1.0)                                               # T starts at one
+    nxt = ~first[1:]                                                                  # record i+1 continues pixel of i
+    np.testing.assert_allclose(raw[1:, 4][nxt], (raw[:-1, 4] * (1 - raw[:-1, 5]))[nxt], rtol=3e-7)
+    np.testing.assert_allclose(raw[:, 5], 1 - np.exp(-raw[:, 3] * raw[:, 6]), atol=2e-7)
+    np.testing.assert_allclose(raw[:, 3], np.log1p(np.exp(raw[:, 7])), rtol=3e-6)
+    rgb = np.zeros((fr.W * fr.H, 3))
+    np.add.at(rgb, pix_of, (raw[:, 4] * raw[:, 5])[:, None] * raw[:, :3])
+    np.testing.assert_allclose(rgb, out["rgb"], atol=2e-6)
+    assert np.array_equal(out["x6"][:, :3], fr.rays_d[pix_of])                        # tests/test_training_wmma.py:123-125
+    np.testing.assert_allclose(out["gates"].sum(1), 1.0, atol=1e-6)
+    assert (raw[:, 6] > fr.thr).all() and (raw[:, 4] >= 1e-3).all()
+    # ReLU masks against an independent float64 evaluation (units whose pre-activation is not near zero)
+    enc = np.concatenate([np.sin(out["x6"][:, :, None] * (sc.freq * sc.att)[None, None, :]).reshape(len(ids), -1),
+                          np.cos(out["x6"][:, :, None] * (sc.freq * sc.att)[None, None, :]).reshape(len(ids), -1)], 1)
+    pre1 = np.einsum("rhi,ri->rh", sc.W1[ids].astype(np.float64), enc.astype(np.float64)) + sc.b1[ids]
+    pre2 = np.einsum("roh,rh->ro", sc.W2[ids].astype(np.float64), np.maximum(pre1, 0)) + sc.b2[ids]
+    for layer, pre in enumerate((pre1, pre2)):
+        bitsm = (out["masks"][:, layer].astype(np.int64)[:, None] >> np.arange(sc.hidden)[None, :]) & 1
+        sure = np.abs(pre) > 1e-5
+        assert np.array_equal(bitsm[sure], (pre > 0)[sure].astype(np.int64)) and sure.mean() > 0.99
+    o3 = np.einsum("rh,rh->r", sc.W3[ids, 3].astype(np.float64), np.maximum(pre2, 0)) + sc.b3[ids, 3]
+    np.testing.assert_allclose(raw[:, 7], o3, atol=2e-5)
