@@ -57,31 +57,50 @@ def main() -> int:
     torch.cuda.set_device(dev)
     precision = args.precision or ("bf16" if hasattr(ops, "render_tilecenter_mfma") else "f32")
 
-    sc, cfg = syn.scene_for_config(args.workload)
+    feature_dim = int(syn.CONFIGS[args.workload]["feature_dim"])
+    sc, cfg = syn.scene_for_config(args.workload, with_features=False)
     W, H, f, thr = cfg["width"], cfg["height"], cfg["focal"], cfg["threshold"]
+    mosaic = args.workload.startswith("cfg4")
 
     def t(a):
         return torch.from_numpy(np.ascontiguousarray(a)).to(dev)
 
-    scene = NeuralPrimitiveSceneTileCUDA(num_primitives=sc.n, hidden_dim=sc.hidden, feature_dim_low=0)
+    scene = NeuralPrimitiveSceneTileCUDA(num_primitives=sc.n, hidden_dim=sc.hidden, feature_dim_low=feature_dim)
     scene.load_state_dict({"positions": torch.from_numpy(sc.positions), "log_scales": torch.from_numpy(sc.log_scales),
                            "quats": torch.from_numpy(sc.quats), "W1": torch.from_numpy(sc.W1),
                            "b1": torch.from_numpy(sc.b1), "W2": torch.from_numpy(sc.W2), "b2": torch.from_numpy(sc.b2),
                            "W3": torch.from_numpy(sc.W3), "b3": torch.from_numpy(sc.b3)}, strict=False)
     scene = scene.to(dev).eval()
+    if feature_dim:
+        # feat_attr [N,4,C] ~ N(0, 0.05), drawn on the device (1.6 GB at 200k x 4 x 512)
+        gen = torch.Generator(device=dev)
+        gen.manual_seed(0)
+        with torch.no_grad():
+            scene.feat_attr.copy_(torch.randn(scene.feat_attr.shape, device=dev, generator=gen) * 0.05)
     scene.set_image_size(W, H)
     scene.render_precision = precision
     proj = t(syn.projection_matrix(f, W, H))
     poses = syn.random_poses(args.poses, 0)
     frames = []
-    for c2w in poses:
-        ro, rd = syn.pinhole_rays(W, H, f, c2w)
-        frames.append((t(ro), t(rd), t(syn.view_matrix(c2w))))
+    if mosaic:
+        # four views of (W/2) x (H/2) per call; tile t renders view tile_view_ids[t]
+        for g0 in range(0, len(poses) - 3, 4):
+            ro, rd, tv, views = syn.mosaic_frame(W // 2, H // 2, f, poses[g0:g0 + 4])
+            frames.append((t(ro), t(rd), t(views), t(tv)))
+    else:
+        for c2w in poses:
+            ro, rd = syn.pinhole_rays(W, H, f, c2w)
+            frames.append((t(ro), t(rd), t(syn.view_matrix(c2w))[None], None))
 
     def render(i):
-        ro, rd, view = frames[i % len(frames)]
+        ro, rd, views, tv = frames[i % len(frames)]
         with torch.inference_mode():
-            return scene(ro, rd, score_threshold=thr, view_matrix=view, proj_matrix=proj)
+            if tv is not None:
+                cand, off = scene.build_tilecenter_culling_from_tile_views(tv, views, proj, thr)
+                return scene(ro, rd, score_threshold=thr, culled_prim_indices=cand, tile_offsets=off)
+            out = scene(ro, rd, score_threshold=thr, view_matrix=views[0], proj_matrix=proj,
+                        return_feature=bool(feature_dim))
+            return out[0] if feature_dim else out
 
     for i in range(args.warmup):
         render(i)
@@ -118,12 +137,13 @@ def main() -> int:
     for i in list(range(n_probe)) * 2:
         if i == 0:
             kernel_ms, hits, proc, cand_total, sort_ms, bin_ms = 0.0, 0, 0, 0, 0.0, 0.0
-        ro, rd_raw, view = frames[i]
+        ro, rd_raw, views, tv = frames[i]
         rd = torch.nn.functional.normalize(rd_raw, dim=-1).contiguous()
         e = [torch.cuda.Event(enable_timing=True) for _ in range(4)]
         rec = ops.prepare_primitives(scene.positions.detach(), scene.log_scales.detach(), quats)
         e[0].record()
-        cand, off = ops.bin_legacy(scene.positions.detach(), scene.log_scales.detach(), view[None], proj, W, H, 8, thr)
+        cand, off = ops.bin_legacy(scene.positions.detach(), scene.log_scales.detach(), views, proj, W, H, 8, thr,
+                                   tile_view_ids=tv)
         e[1].record()
         order, _ = ops.sort_tiles(ro, rd, rec, cand, off, W, H, 8, 8, cull_threshold=thr)
         counters = torch.zeros(4, dtype=torch.int64, device=dev)
@@ -165,13 +185,15 @@ def main() -> int:
     bin_gbs = (24.0 * sc.n * n_probe + 4.0 * cand_total + 4.0 * (T_tiles + 1) * n_probe) / (bin_ms * 1e-3) / 1e9
 
     out = {
-        "metric": "forward_render_frames_per_sec_1200x680_200k_primitives",
+        "metric": ("forward_render_frames_per_sec_1200x680_200k_primitives" if args.workload.startswith("cfg3")
+                   else f"forward_render_frames_per_sec_{args.workload}"),
         "value": round(fps, 3), "unit": "frames/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(1000.0 * elapsed / args.steps, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": precision, "data": "synthetic",
         "config": {"workload": args.workload, "primitives": sc.n, "width": W, "height": H, "tile": 8,
                    "threshold": thr, "poses": len(frames), "log_scale_mean": cfg["log_scale_mean"],
-                   "mlp": f"72-{sc.hidden}-{sc.hidden}-4", "entry": "NeuralPrimitiveSceneTileCUDA.forward"},
+                   "mlp": f"72-{sc.hidden}-{sc.hidden}-4", "feature_channels": feature_dim,
+                   "views_per_call": 4 if mosaic else 1, "entry": "NeuralPrimitiveSceneTileCUDA.forward"},
         "mpix_per_sec": round(fps * W * H / 1e6, 2), "latency": latency,
         "roofline": {"bound": "mfma", "kernel": "render_tilecenter_" + ("mfma" if precision == "bf16" else "f32"),
                      "achieved": round(achieved_tflops, 3), "peak": PEAK[precision], "unit": "TFLOP/s",
@@ -200,18 +222,27 @@ def main() -> int:
     if not args.no_cpu_baseline:
         # the CPU restatement of the same algorithm, on this host's cores: ONE full frame (pose 0)
         import oracle
-        ro, rd_raw, view = frames[0]
+        ro, rd_raw, views, tv = frames[0]
         rd = torch.nn.functional.normalize(rd_raw, dim=-1).cpu().numpy()
-        ro_np, view_np = ro.cpu().numpy(), view.cpu().numpy()
+        ro_np = ro.cpu().numpy()
         tc = time.perf_counter()
-        cand, off = oracle.bin_legacy(sc.positions, sc.log_scales, view_np[None], proj.cpu().numpy(), W, H, 8, thr)
+        cand, off = oracle.bin_legacy(sc.positions, sc.log_scales, views.cpu().numpy(), proj.cpu().numpy(), W, H, 8, thr,
+                                      tile_view_ids=None if tv is None else tv.cpu().numpy())
+        fkw = {}
+        if feature_dim:
+            fkw = dict(feat_attr=scene.feat_attr.detach().cpu().numpy(), beta=float(scene.feature_gating_beta),
+                       temp=float(scene.feature_gating_temp))
+            tc = time.perf_counter()          # the 1.6 GB attribute download is not part of the CPU figure
+            cand, off = oracle.bin_legacy(sc.positions, sc.log_scales, views.cpu().numpy(), proj.cpu().numpy(), W, H, 8,
+                                          thr)
         res = oracle.render_tilecenter(ro_np, rd, sc.positions, sc.log_scales, quats.cpu().numpy(), cand, off,
-                                       freq.cpu().numpy(), att.cpu().numpy(), *sc.mlp(), W, H, 8, 8, thr)
+                                       freq.cpu().numpy(), att.cpu().numpy(), *sc.mlp(), W, H, 8, 8, thr, **fkw)
         cpu_s = time.perf_counter() - tc
         gpu_rgb = render(0).cpu().numpy()
         out["cpu_baseline"] = {"value": round(1.0 / cpu_s, 4), "unit": "frames/s", "cores": oracle.num_threads(),
                                "kind": "port", "sample": "1 full frame (pose 0) of the same workload: binning + "
-                               "per-tile sort + f32 render, OpenMP over tiles",
+                               "per-tile sort + f32 render" + (" with the feature channel" if feature_dim else "") +
+                               ", OpenMP over tiles",
                                "ms_per_frame": round(cpu_s * 1e3, 1),
                                "gpu_vs_cpu_image_max_abs": float(np.abs(gpu_rgb - res["rgb"]).max())}
     print(json.dumps(out))

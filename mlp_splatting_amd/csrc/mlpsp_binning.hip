@@ -121,6 +121,7 @@ __device__ __forceinline__ unsigned lanes_below(unsigned long long mask) {
 // FILL = false: l1_counts[s*NC + c] = survivors; FILL = true: write them.
 template <bool FILL>
 __global__ __launch_bounds__(kBinThreads) void bin_level1_kernel(const float4* __restrict__ bounds, BinGeom g,
+                                                                 const int32_t* __restrict__ tile_view_ids,
                                                                  int32_t* __restrict__ l1_counts,
                                                                  int32_t* __restrict__ l1_list,
                                                                  float4* __restrict__ l1_bounds, long long l1_capacity) {
@@ -129,12 +130,42 @@ __global__ __launch_bounds__(kBinThreads) void bin_level1_kernel(const float4* _
   if (s >= g.nsx * g.nsy) return;
   float x0, x1, y0, y1;
   super_rect(g, s, x0, x1, y0, y1);
+  // Several views: only the views that tiles of this super-tile actually use can contribute (lane l looks
+  // at tile l of the 8 x 8 block); up to four distinct ones are kept, more fall back to testing all K.
+  int nviews = g.K, v0 = 0, v1 = 0, v2 = 0, v3 = 0;
+  if (g.K > 1 && tile_view_ids) {
+    const int tx = (s % g.nsx) * kSuper + (lane & 7), ty = (s / g.nsx) * kSuper + (lane >> 3);
+    const bool has = tx < g.ntx && ty < g.nty;
+    const int view = has ? tile_view_ids[ty * g.ntx + tx] : -1;
+    unsigned long long pending = __ballot(has);
+    int found = 0;
+    while (pending != 0ull && found <= 4) {
+      const int v = __builtin_amdgcn_readlane(view, (int)__builtin_ctzll(pending));
+      pending &= ~__ballot(has && view == v);
+      if (found == 0) v0 = v;
+      else if (found == 1) v1 = v;
+      else if (found == 2) v2 = v;
+      else if (found == 3) v3 = v;
+      ++found;
+    }
+    if (found <= 4) nviews = -found;       // negative: use the explicit list
+  }
   long long running = FILL ? l1_counts[s * g.NC + c] : 0;
   const int first = c * kChunk;
 #pragma unroll 4
   for (int r = 0; r < kChunk / 64; ++r) {
     const int i = first + r * 64 + lane;
-    const bool keep = (i < g.N) && super_overlap(bounds, g, i, x0, x1, y0, y1);
+    bool keep = false;
+    if (i < g.N) {
+      if (nviews >= 0) {
+        keep = super_overlap(bounds, g, i, x0, x1, y0, y1);
+      } else {
+        keep = rect_overlap(bounds[(size_t)v0 * g.N + i], x0, x1, y0, y1);
+        if (nviews <= -2) keep |= rect_overlap(bounds[(size_t)v1 * g.N + i], x0, x1, y0, y1);
+        if (nviews <= -3) keep |= rect_overlap(bounds[(size_t)v2 * g.N + i], x0, x1, y0, y1);
+        if (nviews <= -4) keep |= rect_overlap(bounds[(size_t)v3 * g.N + i], x0, x1, y0, y1);
+      }
+    }
     const unsigned long long m = __ballot(keep);
     if (FILL && keep) {
       const long long dst = running + lanes_below(m);
@@ -327,14 +358,14 @@ MLPSP_API int mlpsp_bin_legacy_count(const float* positions_dev, const float* lo
   hipLaunchKernelGGL(bin_bounds_kernel, dim3(ceil_div(num_primitives, kBinThreads), num_views), dim3(kBinThreads), 0, s,
                      positions_dev, log_scales_dev, b.mats, g, rm, focal, b.bounds);
   MLPSP_LAUNCH_CHECK();
-  hipLaunchKernelGGL((bin_level1_kernel<false>), dim3(g.NC, ceil_div(S, kBinThreads / 64)), dim3(kBinThreads), 0, s, b.bounds, g, b.l1_counts,
-                     b.l1_list, b.l1_bounds, b.l1_capacity);
+  hipLaunchKernelGGL((bin_level1_kernel<false>), dim3(g.NC, ceil_div(S, kBinThreads / 64)), dim3(kBinThreads), 0, s, b.bounds, g,
+                     tile_view_ids_dev, b.l1_counts, b.l1_list, b.l1_bounds, b.l1_capacity);
   MLPSP_LAUNCH_CHECK();
   hipLaunchKernelGGL(exclusive_scan_kernel, dim3(1), dim3(1024), 0, s, b.l1_counts, S * g.NC, b.totals,
                      (long long*)nullptr);
   MLPSP_LAUNCH_CHECK();
-  hipLaunchKernelGGL((bin_level1_kernel<true>), dim3(g.NC, ceil_div(S, kBinThreads / 64)), dim3(kBinThreads), 0, s, b.bounds, g, b.l1_counts,
-                     b.l1_list, b.l1_bounds, b.l1_capacity);
+  hipLaunchKernelGGL((bin_level1_kernel<true>), dim3(g.NC, ceil_div(S, kBinThreads / 64)), dim3(kBinThreads), 0, s, b.bounds, g,
+                     tile_view_ids_dev, b.l1_counts, b.l1_list, b.l1_bounds, b.l1_capacity);
   MLPSP_LAUNCH_CHECK();
   hipLaunchKernelGGL((bin_level2_kernel<false>), dim3(ceil_div((int)T, kBinThreads / 64)), dim3(kBinThreads), 0, s,
                      b.bounds, g, tile_view_ids_dev, b.l1_counts, b.l1_list, b.l1_bounds, b.l1_capacity, tile_offsets_dev,

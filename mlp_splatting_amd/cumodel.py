@@ -350,7 +350,8 @@ class NeuralPrimitiveSceneTileCUDA(nn.Module):
             raise ValueError("view_matrices must have shape (K,4,4)")
         if int(view_matrices.shape[0]) <= 0:
             raise ValueError("view_matrices must contain at least one view")
-        if int(tile_view_ids.min().item()) < 0 or int(tile_view_ids.max().item()) >= int(view_matrices.shape[0]):
+        lo, hi = torch.stack(torch.aminmax(tile_view_ids)).tolist()          # one read-back for both bounds
+        if lo < 0 or hi >= int(view_matrices.shape[0]):
             raise ValueError("tile_view_ids contains out-of-range view indices")
         return self._legacy_culling(view_matrices, proj_matrix, score_threshold, tile_size, tile_view_ids)
 

@@ -107,12 +107,14 @@ def make_scene(n: int, hidden: int = 32, seed: int = 0, log_scale_mean: float = 
     return Scene(positions, log_scales, quats, W1, b1, W2, b2, W3, b3, feat, freq, att)
 
 
-def scene_for_config(name: str, seed: int = 0, n_override: int | None = None) -> tuple[Scene, dict]:
+def scene_for_config(name: str, seed: int = 0, n_override: int | None = None,
+                     with_features: bool = True) -> tuple[Scene, dict]:
     cfg = dict(CONFIGS[name])
     if cfg["log_scale_mean"] is None:
         cfg["log_scale_mean"] = LOG_SCALE_MEAN_200K_CLUSTERED if cfg["cluster_frac"] > 0 else LOG_SCALE_MEAN_200K
     n = cfg["n"] if n_override is None else int(n_override)
-    scene = make_scene(n, cfg["hidden"], seed, cfg["log_scale_mean"], cfg["feature_dim"], 4, cfg["cluster_frac"])
+    scene = make_scene(n, cfg["hidden"], seed, cfg["log_scale_mean"], cfg["feature_dim"] if with_features else 0, 4,
+                       cfg["cluster_frac"])
     return scene, cfg
 
 
