@@ -21,10 +21,11 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the render kernel, from hardware counters: two profiled runs of
 #   rocprofv3 --pmc FETCH_SIZE -- python3 bench.py --steps 16 --warmup 8 --no-cpu-baseline --copy-calibration
 #   rocprofv3 --pmc WRITE_SIZE -- (same)
-# averaged over the run's 40 launches, each counter scaled by what it reads for the 1 GiB device copies of
-# --copy-calibration (FETCH_SIZE reads 524,300 KiB for 1,048,576 KiB copied: factor 2.0; WRITE_SIZE reads
-# 1,048,576 KiB: factor 1.0).  Render kernel: 51,624 KiB x 2.0 fetched + 16,327 KiB written.
-MEASURED_TRAFFIC_BYTES = {("cfg3_200k_1200x680", "bf16"): int((51623.6 * 2.0 + 16327.1) * 1024)}
+# averaged over the run's 56 launches, each counter scaled by what it reads for the 1 GiB device copies of
+# --copy-calibration (FETCH_SIZE reads 524,307 KiB for 1,048,576 KiB copied: factor 2.0; WRITE_SIZE reads
+# 1,048,576 KiB: factor 1.0).  Render kernel: 121,921 KiB x 2.0 fetched + 54,889 KiB written (this includes the
+# scratch traffic of the values the kernel's 128-register budget spills).
+MEASURED_TRAFFIC_BYTES = {("cfg3_200k_1200x680", "bf16"): int((121920.7 * 2.0 + 54889.0) * 1024)}
 
 
 def main() -> int:
