@@ -26,6 +26,12 @@
 #include "mlpsp_hitrec.hpp"
 #include "mlpsp_host.hpp"
 
+// 32-channel accumulator tiles per wavefront of the feature GEMM (2 and 4 measure the same: the kernel moves
+// ~4 GB per frame through L2 and the fabric and is bound there, not by occupancy)
+#ifndef MLPSP_GEMM_NCB
+#define MLPSP_GEMM_NCB 4
+#endif
+
 namespace mlpsp {
 
 typedef float f32x16 __attribute__((ext_vector_type(16)));
@@ -435,11 +441,12 @@ __global__ __launch_bounds__(256) void pack_feat_kernel(const float* __restrict_
 // out_feat[pixel, c] = sum over the tile's hit records e and slots s of coef[e, pixel, s] * attr[id_e, c, s]:
 // per tile a [64 pixels] x [K = SP * hits] x [C] product on v_mfma_f32_32x32x16.  One 256-thread block per
 // tile; wavefront v owns channels [128 v, 128 v + 128) as 2 pixel blocks x 4 channel blocks of f32
-// accumulators.  Pixels are the M operand and channels the N operand, so that an accumulator register
+// accumulators (NCB = 4).  The records' pool slots and primitive ids are staged in LDS once per block, and
+// the operands of one K-step are loaded while the previous one multiplies.  Pixels are the M operand and channels the N operand, so that an accumulator register
 // holds 32 consecutive channels of one pixel across lanes: every store is a full 128-byte line.
 // K-slot j of lane group g is (record 16/SP * step + g * 8/SP + j / SP, slot j % SP): both operands are
 // plain 8- or 16-byte loads, coalesced over 32 pixels / 32 channels.
-template <int SP>
+template <int SP, int NCB>
 __global__ __launch_bounds__(256) void feat_gemm_kernel(const unsigned* __restrict__ attr, HitPool hp,
                                                         const int32_t* __restrict__ offsets, int C, int W, int H,
                                                         int ntx, int per_xcd, int num_tiles,
@@ -447,34 +454,40 @@ __global__ __launch_bounds__(256) void feat_gemm_kernel(const unsigned* __restri
   const int tile = (blockIdx.x % kNumXcd) * per_xcd + blockIdx.x / kNumXcd;
   if (tile >= num_tiles) return;
   const int wave = threadIdx.x >> 6, l = threadIdx.x & 63, g = l >> 5, m = l & 31;
-  const int c0 = ((int)blockIdx.y * 4 + wave) * 128;
-  if (c0 >= C) return;
-  const int ncb = min(4, (C - c0 + 31) / 32);
+  const int c0 = ((int)blockIdx.y * 4 + wave) * (32 * NCB);
+  const bool active = c0 < C;              // a wavefront without channels still helps staging and meets the barriers
+  const int ncb = active ? min(NCB, (C - c0 + 31) / 32) : 0;
   constexpr int EPL = 8 / SP;         // records per lane group and K-step
+  constexpr int STEP = 2 * EPL;       // records per K-step (one MFMA per accumulator tile)
   constexpr int DW = SP / 2;          // dwords per (record, pixel) and per (primitive, channel)
+  constexpr int kStage = 1024;        // records whose pool slot and primitive id are staged in LDS at a time
+  __shared__ int s_slot[kStage];
+  __shared__ int s_prim[kStage];
   const int hits = hp.item_hits[tile];
   const int table_base = (offsets[tile] >> 4) + tile;
-  f32x16 acc[2][4];
+  f32x16 acc[2][NCB];
 #pragma unroll
   for (int pb = 0; pb < 2; ++pb)
 #pragma unroll
-    for (int cb = 0; cb < 4; ++cb)
+    for (int cb = 0; cb < NCB; ++cb)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[pb][cb][r] = 0.f;
-  int ch[4];
+  int ch[NCB];
 #pragma unroll
-  for (int cb = 0; cb < 4; ++cb) ch[cb] = min(c0 + 32 * cb + m, C - 1);
+  for (int cb = 0; cb < NCB; ++cb) ch[cb] = min(c0 + 32 * cb + m, C - 1);
 
-  for (int e = 0; e < hits; e += 2 * EPL) {
-    u32x4 apix[2] = {{0u, 0u, 0u, 0u}, {0u, 0u, 0u, 0u}}, bch[4];
+  // operands of the K-step that starts at staged record e (zero where the list has ended)
+  auto load = [&](int e, int n, u32x4 (&apix)[2], u32x4 (&bch)[NCB]) {
 #pragma unroll
-    for (int cb = 0; cb < 4; ++cb) bch[cb] = u32x4{0u, 0u, 0u, 0u};
+    for (int pb = 0; pb < 2; ++pb) apix[pb] = u32x4{0u, 0u, 0u, 0u};
+#pragma unroll
+    for (int cb = 0; cb < NCB; ++cb) bch[cb] = u32x4{0u, 0u, 0u, 0u};
 #pragma unroll
     for (int u = 0; u < EPL; ++u) {
       const int ent = e + g * EPL + u;
-      if (ent < hits) {
-        const int rs = hit_slot(hp, table_base, ent);
-        const size_t prim = (size_t)hp.hit_ids[rs];
+      if (ent < n) {
+        const int rs = s_slot[ent];
+        const size_t prim = (size_t)s_prim[ent];
         const unsigned* __restrict__ crow = reinterpret_cast<const unsigned*>(hp.records + (size_t)rs * hp.record_bytes) + m * DW;
         const unsigned* __restrict__ arow = attr + prim * C * DW;
         if constexpr (SP == 4) {
@@ -485,7 +498,7 @@ __global__ __launch_bounds__(256) void feat_gemm_kernel(const unsigned* __restri
             apix[pb][2 * u + 1] = v.y;
           }
 #pragma unroll
-          for (int cb = 0; cb < 4; ++cb) {
+          for (int cb = 0; cb < NCB; ++cb) {
             if (cb < ncb) {
               const uint2 v = *reinterpret_cast<const uint2*>(arow + (size_t)ch[cb] * DW);
               bch[cb][2 * u] = v.x;
@@ -496,19 +509,47 @@ __global__ __launch_bounds__(256) void feat_gemm_kernel(const unsigned* __restri
 #pragma unroll
           for (int pb = 0; pb < 2; ++pb) apix[pb] = *reinterpret_cast<const u32x4*>(crow + pb * 32 * DW);
 #pragma unroll
-          for (int cb = 0; cb < 4; ++cb)
+          for (int cb = 0; cb < NCB; ++cb)
             if (cb < ncb) bch[cb] = *reinterpret_cast<const u32x4*>(arow + (size_t)ch[cb] * DW);
         }
       }
     }
+  };
+  auto multiply = [&](const u32x4 (&apix)[2], const u32x4 (&bch)[NCB]) {
 #pragma unroll
-    for (int cb = 0; cb < 4; ++cb) {
+    for (int cb = 0; cb < NCB; ++cb) {
       if (cb < ncb) {
 #pragma unroll
         for (int pb = 0; pb < 2; ++pb) acc[pb][cb] = Ops<_Float16>::mfma(apix[pb], bch[cb], acc[pb][cb]);
       }
     }
+  };
+
+  for (int base = 0; base < hits; base += kStage) {
+    const int n = min(kStage, hits - base);
+    // record -> (pool slot, primitive id) once per block, so that the K loop below has a single level of
+    // global loads to wait for
+    for (int k = threadIdx.x; k < n; k += 256) {
+      const int rs = hit_slot(hp, table_base, base + k);
+      s_slot[k] = rs;
+      s_prim[k] = hp.hit_ids[rs];
+    }
+    __syncthreads();
+    if (active) {
+      // two operand sets: the loads of one K-step are in flight while the other multiplies
+      u32x4 apA[2], bcA[NCB], apB[2], bcB[NCB];
+      load(0, n, apA, bcA);
+      for (int e = 0; e < n; e += 2 * STEP) {
+        if (e + STEP < n) load(e + STEP, n, apB, bcB);
+        multiply(apA, bcA);
+        if (e + STEP >= n) break;
+        if (e + 2 * STEP < n) load(e + 2 * STEP, n, apA, bcA);
+        multiply(apB, bcB);
+      }
+    }
+    __syncthreads();
   }
+  if (!active) return;
 
   const int tx = tile % ntx, ty = tile / ntx;
 #pragma unroll
@@ -520,7 +561,7 @@ __global__ __launch_bounds__(256) void feat_gemm_kernel(const unsigned* __restri
       if (x < W && y < H) {
         float* __restrict__ dst = out_feat + (size_t)(y * W + x) * C;
 #pragma unroll
-        for (int cb = 0; cb < 4; ++cb) {
+        for (int cb = 0; cb < NCB; ++cb) {
           const int c = c0 + 32 * cb + m;
           if (cb < ncb && c < C) dst[c] = acc[pb][cb][r];
         }
@@ -575,6 +616,7 @@ MLPSP_API int mlpsp_pack_mfma_weights(const float* W1, const float* b1, const fl
 }
 
 namespace {
+constexpr int kGemmNcb = MLPSP_GEMM_NCB;   // 32-channel accumulator tiles per wavefront of the feature GEMM
 constexpr size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 inline int feat_pad(int slots) { return slots == 5 ? 8 : 4; }
 
@@ -666,9 +708,9 @@ MLPSP_API int mlpsp_render_tilecenter_mfma_feat(const float* rays_o_dev, const f
 #undef MLPSP_MFMA_GO
   MLPSP_LAUNCH_CHECK();
   if (sp != 0) {
-    const dim3 ggrid((unsigned)(per_xcd * kNumXcd), (unsigned)ceil_div(feat_channels, 512)), gblock(256);
+    const dim3 ggrid((unsigned)(per_xcd * kNumXcd), (unsigned)ceil_div(feat_channels, 128 * kGemmNcb)), gblock(256);
 #define MLPSP_FEAT_GEMM(SP)                                                                                       \
-  hipLaunchKernelGGL((feat_gemm_kernel<SP>), ggrid, gblock, 0, s, (const unsigned*)packed_feat_dev, hp,           \
+  hipLaunchKernelGGL((feat_gemm_kernel<SP, kGemmNcb>), ggrid, gblock, 0, s, (const unsigned*)packed_feat_dev, hp, \
                      tile_offsets_dev, feat_channels, width, height, ntx, per_xcd, (int)T, out_feat_dev)
     if (sp == 4) MLPSP_FEAT_GEMM(4);
     else MLPSP_FEAT_GEMM(8);
