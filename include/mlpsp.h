@@ -86,6 +86,19 @@ int mlpsp_bin_legacy_count(const float* positions_dev, const float* log_scales_d
                            const float* proj_host, int width, int height, int tile, float threshold,
                            void* scratch_dev, size_t scratch_bytes, int32_t* tile_offsets_dev,
                            int64_t counts_out[2], mlpsp_stream_t stream);
+/* The same lists without any host synchronisation, for callers that queue a whole frame: candidates_dev
+ * holds cand_capacity entries chosen by the caller (e.g. last frame's count plus a margin).
+ * counts_dev (device int64[4]) receives {pairs, longest tile list, level-1 scratch entries, guard}.  If the
+ * pairs exceed cand_capacity or the level-1 lists overflow the scratch, guard = 1 and EVERY tile list is left
+ * empty (offsets all zero, nothing written to candidates_dev), so that kernels already queued behind this
+ * call touch nothing; the caller reads counts_dev when it next synchronises, enlarges what was too small
+ * and repeats the frame.  No counterpart in the reference (its culling is synchronous PyTorch). */
+int mlpsp_bin_legacy_async(const float* positions_dev, const float* log_scales_dev, int num_primitives,
+                           const float* view_matrices_host, int num_views, const int32_t* tile_view_ids_dev,
+                           const float* proj_host, int width, int height, int tile, float threshold,
+                           void* scratch_dev, size_t scratch_bytes, int32_t* tile_offsets_dev,
+                           int32_t* candidates_dev, int64_t cand_capacity, int64_t* counts_dev,
+                           mlpsp_stream_t stream);
 int mlpsp_bin_legacy_fill(int num_primitives, int num_views, const int32_t* tile_view_ids_dev, int width,
                           int height, int tile, const void* scratch_dev, size_t scratch_bytes,
                           const int32_t* tile_offsets_dev, int32_t* candidates_dev, mlpsp_stream_t stream);

@@ -27,7 +27,7 @@ struct BinScratch {
   float* mats;        // K view matrices (16 floats each) then the projection (16 floats)
   float4* bounds;     // [K][N] (minx, maxx, miny, maxy); all NaN when behind the near plane
   int32_t* l1_counts; // [S*NC + 1] counts, then exclusive offsets after the scan
-  long long* totals;  // [0] level-1 entries, [1] tile-list entries, [2] longest tile list
+  long long* totals;  // [0] level-1 entries, [1] tile-list entries, [2] longest tile list, [3] guard status
   int32_t* l1_list;   // [l1_capacity]
   float4* l1_bounds;  // [l1_capacity] bounds of the listed primitives, one view only (else null)
   long long l1_capacity;
@@ -63,15 +63,21 @@ struct BinGeom {
 
 // Screen-space bounds of primitive i under view k (scannet/cumodel.py:1001-1041).  The 4-term dot
 // products are fma chains from the last term inwards.
+// One view: the two matrices travel as kernel arguments (no host-to-device copy in front of the frame).
+struct BinMats {
+  float v[16], p[16];
+};
+
+template <bool ARGS>
 __global__ __launch_bounds__(kBinThreads) void bin_bounds_kernel(const float* __restrict__ pos,
                                                                  const float* __restrict__ logs,
-                                                                 const float* __restrict__ mats, BinGeom g, float rm,
-                                                                 float focal, float4* __restrict__ bounds) {
+                                                                 const float* __restrict__ mats, BinMats one, BinGeom g,
+                                                                 float rm, float focal, float4* __restrict__ bounds) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   const int k = blockIdx.y;
   if (i >= g.N) return;
-  const float* V = mats + k * 16;
-  const float* Pm = mats + g.K * 16;
+  const float* V = ARGS ? one.v : mats + k * 16;
+  const float* Pm = ARGS ? one.p : mats + g.K * 16;
   const float x = pos[i * 3 + 0], y = pos[i * 3 + 1], z = pos[i * 3 + 2];
   float pv[4], clip[4];
 #pragma unroll
@@ -270,10 +276,12 @@ __global__ __launch_bounds__(kBinThreads) void bin_level2_kernel(const float4* _
                                                                  const float4* __restrict__ l1_bounds,
                                                                  long long l1_capacity,
                                                                  int32_t* __restrict__ tile_offsets,
-                                                                 int32_t* __restrict__ cand) {
+                                                                 int32_t* __restrict__ cand,
+                                                                 const long long* __restrict__ skip_flag = nullptr) {
   const int tile = blockIdx.x * (kBinThreads / 64) + (threadIdx.x >> 6);
   const int lane = threadIdx.x & 63;
   if (tile >= g.ntx * g.nty) return;
+  if (FILL && skip_flag && *skip_flag != 0) return;       // the guard emptied the lists: nothing may be written
   const int tx = tile % g.ntx, ty = tile / g.ntx;
   const int s = (ty / kSuper) * g.nsx + (tx / kSuper);
   const int view = tile_view_ids ? tile_view_ids[tile] : 0;
@@ -325,38 +333,34 @@ MLPSP_API size_t mlpsp_bin_scratch_bytes(int num_primitives, int num_views, int 
   return bytes;
 }
 
-MLPSP_API int mlpsp_bin_legacy_count(const float* positions_dev, const float* log_scales_dev, int num_primitives,
-                                     const float* view_matrices_host, int num_views,
-                                     const int32_t* tile_view_ids_dev, const float* proj_host, int width, int height,
-                                     int tile, float threshold, void* scratch_dev, size_t scratch_bytes,
-                                     int32_t* tile_offsets_dev, int64_t counts_out[2], mlpsp_stream_t stream) {
-  const int64_t T = checked_num_tiles(width, height, tile, tile);
-  if (T <= 0 || num_primitives < 0 || num_views <= 0 || !view_matrices_host || !proj_host || !scratch_dev ||
-      !tile_offsets_dev || !counts_out)
-    return MLPSP_E_ARGUMENT;
-  if (!(threshold > 0.f && threshold < 1.f)) return MLPSP_E_ARGUMENT;
-  if (reinterpret_cast<uintptr_t>(tile_offsets_dev) % 16 != 0 || reinterpret_cast<uintptr_t>(scratch_dev) % 256 != 0)
-    return MLPSP_E_ARGUMENT;
-  if (scratch_bytes < mlpsp_bin_scratch_bytes(num_primitives, num_views, width, height, tile)) return MLPSP_E_SCRATCH;
-  hipStream_t s = (hipStream_t)stream;
-  const BinGeom g = make_geom(num_primitives, num_views, width, height, tile);
+namespace {
+// Enqueues bounds -> level 1 (count, scan, fill) -> level 2 count -> scan.  Leaves the exclusive tile offsets in
+// tile_offsets_dev and (level-1 entries, pairs, longest tile list) in b.totals[0..2]; no host synchronisation.
+int enqueue_bin_count(const float* positions_dev, const float* log_scales_dev, int num_primitives,
+                      const float* view_matrices_host, int num_views, const int32_t* tile_view_ids_dev,
+                      const float* proj_host, int width, int height, int tile, float threshold, const BinGeom& g,
+                      const BinScratch& b, int64_t T, int32_t* tile_offsets_dev, hipStream_t s) {
   const int S = g.nsx * g.nsy;
-  const BinScratch b = carve(scratch_dev, scratch_bytes, num_primitives, num_views, S, g.NC);
-  counts_out[0] = counts_out[1] = 0;
-  if (num_primitives == 0) {
-    MLPSP_HIP_TRY(hipMemsetAsync(tile_offsets_dev, 0, (size_t)(T + 1) * sizeof(int32_t), s));
-    MLPSP_HIP_TRY(hipMemsetAsync(b.totals, 0, 3 * sizeof(long long), s));
-    return MLPSP_OK;
-  }
   // scalar constants in f32, in the order the reference's tensor expressions evaluate them
   const float rm = sqrtf(-2.0f * logf(threshold));
   const float fx = (proj_host[0] * (float)width) / 2.0f, fy = (proj_host[5] * (float)height) / 2.0f;
   const float focal = (fx + fy) * 0.5f;
-  MLPSP_HIP_TRY(hipMemcpyAsync(b.mats, view_matrices_host, (size_t)num_views * 16 * sizeof(float),
-                               hipMemcpyHostToDevice, s));
-  MLPSP_HIP_TRY(hipMemcpyAsync(b.mats + (size_t)num_views * 16, proj_host, 16 * sizeof(float), hipMemcpyHostToDevice, s));
-  hipLaunchKernelGGL(bin_bounds_kernel, dim3(ceil_div(num_primitives, kBinThreads), num_views), dim3(kBinThreads), 0, s,
-                     positions_dev, log_scales_dev, b.mats, g, rm, focal, b.bounds);
+  BinMats one{};
+  if (num_views == 1) {
+    for (int e = 0; e < 16; ++e) {
+      one.v[e] = view_matrices_host[e];
+      one.p[e] = proj_host[e];
+    }
+    hipLaunchKernelGGL(bin_bounds_kernel<true>, dim3(ceil_div(num_primitives, kBinThreads), 1), dim3(kBinThreads), 0, s,
+                       positions_dev, log_scales_dev, (const float*)nullptr, one, g, rm, focal, b.bounds);
+  } else {
+    MLPSP_HIP_TRY(hipMemcpyAsync(b.mats, view_matrices_host, (size_t)num_views * 16 * sizeof(float),
+                                 hipMemcpyHostToDevice, s));
+    MLPSP_HIP_TRY(hipMemcpyAsync(b.mats + (size_t)num_views * 16, proj_host, 16 * sizeof(float), hipMemcpyHostToDevice,
+                                 s));
+    hipLaunchKernelGGL(bin_bounds_kernel<false>, dim3(ceil_div(num_primitives, kBinThreads), num_views),
+                       dim3(kBinThreads), 0, s, positions_dev, log_scales_dev, b.mats, one, g, rm, focal, b.bounds);
+  }
   MLPSP_LAUNCH_CHECK();
   hipLaunchKernelGGL((bin_level1_kernel<false>), dim3(g.NC, ceil_div(S, kBinThreads / 64)), dim3(kBinThreads), 0, s, b.bounds, g,
                      tile_view_ids_dev, b.l1_counts, b.l1_list, b.l1_bounds, b.l1_capacity);
@@ -374,6 +378,66 @@ MLPSP_API int mlpsp_bin_legacy_count(const float* positions_dev, const float* lo
   hipLaunchKernelGGL(exclusive_scan_kernel, dim3(1), dim3(1024), 0, s, tile_offsets_dev, (int)T, b.totals + 1,
                      b.totals + 2);
   MLPSP_LAUNCH_CHECK();
+  return MLPSP_OK;
+}
+
+int check_bin_args(int64_t T, const float* view_matrices_host, const float* proj_host, void* scratch_dev,
+                   size_t scratch_bytes, int32_t* tile_offsets_dev, int num_primitives, int num_views, int width,
+                   int height, int tile, float threshold) {
+  if (T <= 0 || num_primitives < 0 || num_views <= 0 || !view_matrices_host || !proj_host || !scratch_dev ||
+      !tile_offsets_dev)
+    return MLPSP_E_ARGUMENT;
+  if (!(threshold > 0.f && threshold < 1.f)) return MLPSP_E_ARGUMENT;
+  if (reinterpret_cast<uintptr_t>(tile_offsets_dev) % 16 != 0 || reinterpret_cast<uintptr_t>(scratch_dev) % 256 != 0)
+    return MLPSP_E_ARGUMENT;
+  if (scratch_bytes < mlpsp_bin_scratch_bytes(num_primitives, num_views, width, height, tile)) return MLPSP_E_SCRATCH;
+  return MLPSP_OK;
+}
+}  // namespace
+
+namespace mlpsp {
+// After the counting pass of the asynchronous binning: if the level-1 lists overflowed their scratch or the
+// pairs do not fit the caller's candidate buffer, empty every tile list (offsets := 0) and raise the guard
+// word, so that the fill, sort and render kernels queued behind find nothing to read or write.
+__global__ __launch_bounds__(256) void bin_guard_kernel(long long* __restrict__ totals, long long l1_capacity,
+                                                        long long cand_capacity, int32_t* __restrict__ tile_offsets,
+                                                        int num_offsets, long long* __restrict__ counts_out) {
+  const bool bad = totals[0] > l1_capacity || totals[1] > cand_capacity;
+  if (bad)
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < num_offsets; i += gridDim.x * blockDim.x) tile_offsets[i] = 0;
+  if (blockIdx.x == 0 && threadIdx.x == 0) {
+    totals[3] = bad ? 1 : 0;
+    counts_out[0] = totals[1];
+    counts_out[1] = totals[2];
+    counts_out[2] = totals[0];
+    counts_out[3] = bad ? 1 : 0;
+  }
+}
+}  // namespace mlpsp
+
+MLPSP_API int mlpsp_bin_legacy_count(const float* positions_dev, const float* log_scales_dev, int num_primitives,
+                                     const float* view_matrices_host, int num_views,
+                                     const int32_t* tile_view_ids_dev, const float* proj_host, int width, int height,
+                                     int tile, float threshold, void* scratch_dev, size_t scratch_bytes,
+                                     int32_t* tile_offsets_dev, int64_t counts_out[2], mlpsp_stream_t stream) {
+  const int64_t T = checked_num_tiles(width, height, tile, tile);
+  if (!counts_out) return MLPSP_E_ARGUMENT;
+  const int rc = check_bin_args(T, view_matrices_host, proj_host, scratch_dev, scratch_bytes, tile_offsets_dev,
+                                num_primitives, num_views, width, height, tile, threshold);
+  if (rc != MLPSP_OK) return rc;
+  hipStream_t s = (hipStream_t)stream;
+  const BinGeom g = make_geom(num_primitives, num_views, width, height, tile);
+  const BinScratch b = carve(scratch_dev, scratch_bytes, num_primitives, num_views, g.nsx * g.nsy, g.NC);
+  counts_out[0] = counts_out[1] = 0;
+  if (num_primitives == 0) {
+    MLPSP_HIP_TRY(hipMemsetAsync(tile_offsets_dev, 0, (size_t)(T + 1) * sizeof(int32_t), s));
+    MLPSP_HIP_TRY(hipMemsetAsync(b.totals, 0, 4 * sizeof(long long), s));
+    return MLPSP_OK;
+  }
+  const int erc = enqueue_bin_count(positions_dev, log_scales_dev, num_primitives, view_matrices_host, num_views,
+                                    tile_view_ids_dev, proj_host, width, height, tile, threshold, g, b, T,
+                                    tile_offsets_dev, s);
+  if (erc != MLPSP_OK) return erc;
   // one blocking readback: level-1 entry count (overflow check) and the number of pairs
   long long totals[3] = {0, 0, 0};
   MLPSP_HIP_TRY(hipMemcpyAsync(totals, b.totals, 3 * sizeof(long long), hipMemcpyDeviceToHost, s));
@@ -382,6 +446,40 @@ MLPSP_API int mlpsp_bin_legacy_count(const float* positions_dev, const float* lo
   if (totals[1] > 2147483647LL) return MLPSP_E_ARGUMENT;
   counts_out[0] = totals[1];
   counts_out[1] = totals[2];
+  return MLPSP_OK;
+}
+
+MLPSP_API int mlpsp_bin_legacy_async(const float* positions_dev, const float* log_scales_dev, int num_primitives,
+                                     const float* view_matrices_host, int num_views,
+                                     const int32_t* tile_view_ids_dev, const float* proj_host, int width, int height,
+                                     int tile, float threshold, void* scratch_dev, size_t scratch_bytes,
+                                     int32_t* tile_offsets_dev, int32_t* candidates_dev, int64_t cand_capacity,
+                                     int64_t* counts_dev, mlpsp_stream_t stream) {
+  const int64_t T = checked_num_tiles(width, height, tile, tile);
+  if (!counts_dev || cand_capacity < 0 || cand_capacity > 2147483647LL || (cand_capacity > 0 && !candidates_dev))
+    return MLPSP_E_ARGUMENT;
+  const int rc = check_bin_args(T, view_matrices_host, proj_host, scratch_dev, scratch_bytes, tile_offsets_dev,
+                                num_primitives, num_views, width, height, tile, threshold);
+  if (rc != MLPSP_OK) return rc;
+  hipStream_t s = (hipStream_t)stream;
+  const BinGeom g = make_geom(num_primitives, num_views, width, height, tile);
+  const BinScratch b = carve(scratch_dev, scratch_bytes, num_primitives, num_views, g.nsx * g.nsy, g.NC);
+  if (num_primitives == 0) {
+    MLPSP_HIP_TRY(hipMemsetAsync(tile_offsets_dev, 0, (size_t)(T + 1) * sizeof(int32_t), s));
+    MLPSP_HIP_TRY(hipMemsetAsync(counts_dev, 0, 4 * sizeof(int64_t), s));
+    return MLPSP_OK;
+  }
+  const int erc = enqueue_bin_count(positions_dev, log_scales_dev, num_primitives, view_matrices_host, num_views,
+                                    tile_view_ids_dev, proj_host, width, height, tile, threshold, g, b, T,
+                                    tile_offsets_dev, s);
+  if (erc != MLPSP_OK) return erc;
+  hipLaunchKernelGGL(bin_guard_kernel, dim3(64), dim3(256), 0, s, b.totals, b.l1_capacity, (long long)cand_capacity,
+                     tile_offsets_dev, (int)(T + 1), (long long*)counts_dev);
+  MLPSP_LAUNCH_CHECK();
+  hipLaunchKernelGGL((bin_level2_kernel<true>), dim3(ceil_div((int)T, kBinThreads / 64)), dim3(kBinThreads), 0, s,
+                     b.bounds, g, tile_view_ids_dev, b.l1_counts, b.l1_list, b.l1_bounds, b.l1_capacity, tile_offsets_dev,
+                     candidates_dev, (const long long*)(b.totals + 3));
+  MLPSP_LAUNCH_CHECK();
   return MLPSP_OK;
 }
 

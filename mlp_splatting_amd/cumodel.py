@@ -14,6 +14,7 @@ without a graph.
 from __future__ import annotations
 
 import os
+import weakref
 
 import torch
 import torch.nn as nn
@@ -58,6 +59,34 @@ def _tile_ext_build_config(tile_size=None):
             suffix += f"_rreg{value}"
     name = f"np_tile_kernels_{suffix}"
     return (name, tuple(flags)), name, flags
+
+
+_host_copies = {}
+
+
+def _host_matrix(t):
+    """A float32 host copy of a small device tensor (view / projection matrices), remembered for as long
+    as that very tensor object is alive and unmodified: the binning reads its matrices on the host, and a
+    device-to-host copy per frame is a synchronisation per frame.  The entry is keyed by the object and
+    checked through a weak reference and the in-place version, so a new tensor at a recycled address
+    never hits."""
+    if not torch.is_tensor(t) or not t.is_cuda:
+        return t
+    try:
+        version = t._version
+    except RuntimeError:                              # inference tensors carry no version counter
+        return t.detach().to("cpu", torch.float32)
+    hit = _host_copies.get(id(t))
+    if hit is not None and hit[0]() is t and hit[1] == version:
+        return hit[2]
+    if len(_host_copies) > 512:
+        _host_copies.clear()
+    host = t.detach().to("cpu", torch.float32)
+    try:
+        _host_copies[id(t)] = (weakref.ref(t), version, host)
+    except TypeError:
+        pass
+    return host
 
 
 def _tile_capacity_from_env() -> int:
@@ -320,8 +349,9 @@ class NeuralPrimitiveSceneTileCUDA(nn.Module):
     def _legacy_culling(self, view_matrices, proj_matrix, score_threshold, tile_size, tile_view_ids=None):
         """Screen-space tile lists: same rule as scannet/cumodel.py:994-1070, evaluated sparsely on the GPU."""
         W, H = self.image_size
-        cand, offsets, longest = ops.bin_legacy(self.positions.detach(), self.log_scales.detach(), view_matrices,
-                                                proj_matrix, W, H, int(tile_size), float(score_threshold),
+        cand, offsets, longest = ops.bin_legacy(self.positions.detach(), self.log_scales.detach(),
+                                                _host_matrix(view_matrices), _host_matrix(proj_matrix), W, H,
+                                                int(tile_size), float(score_threshold),
                                                 tile_view_ids, with_longest=True)
         # lists fresh from the binning kernels need no second validation pass on the device
         note = getattr(self._ensure_tile_ext(), "note_binned_lists", None)
@@ -377,7 +407,8 @@ class NeuralPrimitiveSceneTileCUDA(nn.Module):
             return culled_prim_indices, tile_offsets
         if view_matrix is None or proj_matrix is None:
             raise ValueError("Tile renderer requires view_matrix/proj_matrix unless external culling is provided.")
-        return self._legacy_culling(view_matrix.reshape(1, 4, 4), proj_matrix, score_threshold, tile_size)
+        return self._legacy_culling(_host_matrix(view_matrix).reshape(1, 4, 4), _host_matrix(proj_matrix),
+                                    score_threshold, tile_size)
 
     def _unit_quats(self):
         return self._cached("unit_quats", [self.quats], (),
@@ -415,10 +446,21 @@ class NeuralPrimitiveSceneTileCUDA(nn.Module):
             # queued before the binning, whose pair count is a blocking read-back: the device then has
             # this work to do while the host waits, instead of idling while the host issues it afterwards
             unit_dirs = F.normalize(ray_d, dim=-1).contiguous()
-            culled_prim_indices, tile_offsets = self._tile_lists(
-                ray_o, ray_d, score_threshold, view_matrix, proj_matrix, culled_prim_indices, tile_offsets, device)
             use_tilecenter = self._resolve_tile_order_mode() == "tilecenter"
             ext = self._ensure_tile_ext()
+            own_lists = (culled_prim_indices is None and tile_offsets is None and view_matrix is not None
+                         and proj_matrix is not None
+                         and getattr(self, "camera_mode", "legacy-centered") != "colmap-native")
+            if (own_lists and use_tilecenter and ts == 8 and not return_feature and feature_target is None
+                    and getattr(self, "queued_frames", True) and hasattr(ext, "render_frame_queued")):
+                done = self._forward_queued(ext, ray_o, unit_dirs, score_threshold, view_matrix, proj_matrix, bg_color,
+                                            device)
+                if done is not None:
+                    return done
+            culled_prim_indices, tile_offsets = self._tile_lists(
+                ray_o, ray_d, score_threshold, view_matrix, proj_matrix, culled_prim_indices, tile_offsets, device)
+            if own_lists and hasattr(ext, "note_frame_pairs"):
+                ext.note_frame_pairs(int(culled_prim_indices.numel()))
             if feature_target is not None:
                 if not return_feature or self.feat_attr is None or not use_tilecenter or ts != 8:
                     raise ValueError("CSR feature training requires tilecenter8 and direct feature attributes")
@@ -454,6 +496,28 @@ class NeuralPrimitiveSceneTileCUDA(nn.Module):
                 rgb, alpha, feat = ext.render_tiles_forward_per_pixel_with_feat(*base, *feat_args, *dims)
             return _add_background(rgb, alpha, bg), feat
 
+    def _forward_queued(self, ext, ray_o, unit_dirs, score_threshold, view_matrix, proj_matrix, bg_color, device):
+        """The RGB frame with binning, sort and render queued back to back and one read-back at the end
+        (``TileExt.render_frame_queued``); None when that path does not apply or has to be repeated the
+        synchronous way.  Same images and errors as the step-by-step path."""
+        precision = str(getattr(self, "render_precision", "f32")).lower()
+        if precision not in {"f32", "bf16", "fp16"}:
+            raise ValueError(f"Unsupported render_precision {precision!r}; use 'f32', 'bf16' or 'fp16'.")
+        if precision != "f32" and not (int(self.hidden_dim) == 32 and int(self.pe_frequencies) == 6):
+            precision = "f32"
+        W, H = self.image_size
+        freq, att = self._frequency_tables(device)
+        ws = [p.detach().contiguous() for p in (self.W1, self.b1, self.W2, self.b2, self.W3, self.b3)]
+        if any(w.dtype != torch.float32 for w in ws):
+            return None                       # stored half-precision weights take the step-by-step path
+        out = ext.render_frame_queued(ray_o.contiguous(), unit_dirs, self.positions.detach().contiguous(),
+                                      self.log_scales.detach().contiguous(), self._unit_quats(), freq, att, ws,
+                                      _host_matrix(view_matrix).reshape(1, 4, 4), _host_matrix(proj_matrix), int(W),
+                                      int(H), float(score_threshold), precision)
+        if out is None:
+            return None
+        return _add_background(out[0], out[1], self._background(bg_color, ray_o))
+
     def render_feature_map(self, ray_o, ray_d, score_threshold: float = 1e-3, view_matrix=None, proj_matrix=None,
                            culled_prim_indices=None, tile_offsets=None):
         """The feature image alone, through ``forward`` (scannet/cumodel.py:1162-1193)."""
@@ -485,7 +549,8 @@ class NeuralPrimitiveSceneTileCUDA(nn.Module):
         assert B == W * H, "Tile renderer requires full-frame rays (B == W*H)"
         device = self._activate_cuda_device()
         ts = int(self.tile_size)
-        cand, offsets = self._legacy_culling(view_matrix.reshape(1, 4, 4), proj_matrix, score_threshold, ts)
+        cand, offsets = self._legacy_culling(_host_matrix(view_matrix).reshape(1, 4, 4), _host_matrix(proj_matrix),
+                                             score_threshold, ts)
         ext = self._ensure_tile_ext()
         base = self._base_args(ray_o, ray_d, cand, offsets, device)
         dims = (int(W), int(H), ts, ts, float(score_threshold))
@@ -518,7 +583,8 @@ class NeuralPrimitiveSceneTileCUDA(nn.Module):
         assert ray_o.shape[0] == W * H, "Tile renderer requires full-frame rays (B == W*H)"
         device = self._activate_cuda_device()
         ts = int(self.tile_size)
-        cand, offsets = self._legacy_culling(view_matrix.reshape(1, 4, 4), proj_matrix, score_threshold, ts)
+        cand, offsets = self._legacy_culling(_host_matrix(view_matrix).reshape(1, 4, 4), _host_matrix(proj_matrix),
+                                             score_threshold, ts)
         ext = self._ensure_tile_ext()
         base = self._base_args(ray_o, ray_d, cand, offsets, device)
         rgb, alpha, t = ext.render_tiles_forward_tilecenter_with_t(*base, int(W), int(H), ts, ts, float(score_threshold))

@@ -121,6 +121,38 @@ def bin_legacy(positions, log_scales, view_matrices, proj_matrix, W: int, H: int
     return cand, offsets
 
 
+def bin_legacy_async(positions, log_scales, view_matrices, proj_matrix, W: int, H: int, tile: int, threshold: float,
+                     cand_capacity: int, tile_view_ids=None, scratch_scale: int = 1):
+    """:func:`bin_legacy` without any host synchronisation -> (candidates [cand_capacity], tile_offsets [T+1],
+    counts int64 [4] on the device = pairs, longest tile list, level-1 entries, guard).  If guard is set the
+    lists are empty: read ``counts`` at the next synchronisation, enlarge ``cand_capacity`` (pairs) or
+    ``scratch_scale`` (level-1 entries) and repeat."""
+    positions, log_scales = _f32c(positions, "positions"), _f32c(log_scales, "log_scales")
+    dev = positions.device
+    vm = view_matrices.detach().to("cpu", torch.float32).reshape(-1, 4, 4).contiguous()
+    pm = proj_matrix.detach().to("cpu", torch.float32).reshape(4, 4).contiguous()
+    K, n = vm.shape[0], positions.shape[0]
+    T = num_tiles(W, H, tile, tile)
+    tv = None
+    if tile_view_ids is not None:
+        tv = tile_view_ids.to(device=dev, dtype=torch.int32).contiguous()
+        if tv.numel() != T:
+            raise ValueError(f"tile_view_ids length mismatch: got {tv.numel()}, expected {T}")
+    lib = _lib.load()
+    fp = C.POINTER(C.c_float)
+    nbytes = lib.mlpsp_bin_scratch_bytes(n, K, W, H, tile) * int(scratch_scale)
+    with torch.inference_mode(False):
+        offsets = torch.empty(T + 1, dtype=torch.int32, device=dev)
+        cand = torch.empty(int(cand_capacity), dtype=torch.int32, device=dev)
+    scratch = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    counts = torch.empty(4, dtype=torch.int64, device=dev)
+    code = lib.mlpsp_bin_legacy_async(_ptr(positions), _ptr(log_scales), n, C.cast(vm.data_ptr(), fp), K, _ptr(tv),
+                                      C.cast(pm.data_ptr(), fp), W, H, tile, float(threshold), _ptr(scratch), nbytes,
+                                      _ptr(offsets), _ptr(cand), int(cand_capacity), _ptr(counts), _stream(dev))
+    _check(code, "mlpsp_bin_legacy_async")
+    return cand, offsets, counts
+
+
 def sort_tiles(rays_o, rays_d, records, candidates, tile_offsets, W, H, TW, TH, family=_lib.KEY_TSTAR,
                capacity=TILE_CAPACITY_DEFAULT, want_keys=False, cull_threshold=0.0):
     """Materialised per-tile depth order: (sorted_ids [P], sorted_keys [P] | None).

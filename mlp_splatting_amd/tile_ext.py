@@ -54,6 +54,8 @@ class TileExt:
         self._binned = None
         self._rec_key = None
         self._rec = None
+        self._queue_capacity = 0          # candidate-buffer estimate of render_frame_queued (0: not seeded yet)
+        self._queue_scratch_scale = 1
         self._feat_pack = None
 
     def __getattr__(self, name):
@@ -245,6 +247,75 @@ class TileExt:
         _chk(feat_attr.shape[0] == base[2].shape[0], "feat_attr first dimension must match primitive count")
         ops._feat_shape(feat_attr)
         return self._per_pixel((*base, *dims), "render_tiles_forward_per_pixel_with_feat", (feat_attr, beta, temp))
+
+    # ------------------------------------------------------------------------------------------
+    # a whole frame queued without a host synchronisation in its middle (no counterpart in the reference)
+    # ------------------------------------------------------------------------------------------
+    def render_frame_queued(self, rays_o, unit_dirs, positions, log_scales, unit_quats, freq, att, ws, view_matrices,
+                            proj_matrix, width, height, threshold, precision):
+        """(rgb, alpha) of one 8x8-tile, tile-centre-order RGB frame: binning, sort and render are queued
+        back to back and ONE read-back at the end brings the pair count, the longest tile list and the
+        non-finite flag.  The candidate buffer is sized from the previous frame's count; if this frame
+        needs more (or the level-1 scratch overflows) every list was left empty on the device: the
+        estimate is enlarged and None is returned, and the caller renders the frame the synchronous way.
+        Errors are those of the entry points it stands for (capacity text of np_tile_kernels.cu:4578-4588,
+        fallback policy of rgb_wmma.cuh:260-272)."""
+        name = "render_tiles_rgb_wmma" if precision != "f32" else "render_tiles_forward_tilecenter"
+        width, height, threshold = int(width), int(height), float(threshold)
+        with self._lock:
+            cap, scale = self._queue_capacity, self._queue_scratch_scale
+        if cap <= 0:
+            return None
+        n = positions.shape[0]
+        with torch.cuda.device(rays_o.device):
+            rec = self._records(positions, log_scales, unit_quats)
+            cand, offsets, counts = ops.bin_legacy_async(positions, log_scales, view_matrices, proj_matrix, width,
+                                                         height, 8, threshold, cap, scratch_scale=scale)
+            order, _ = ops.sort_tiles(rays_o, unit_dirs, rec, cand, offsets, width, height, 8, 8, _lib.KEY_TSTAR,
+                                      self.max_tile_prims, cull_threshold=threshold)
+            if precision != "f32":
+                packed = self._packed_weights(list(ws), precision == "bf16")
+                rgb, alpha, flag = ops.render_tilecenter_mfma(rays_o, unit_dirs, rec, order, offsets, freq, att, *ws,
+                                                              width, height, threshold, bf16=(precision == "bf16"),
+                                                              packed=packed, check=False)
+                pairs, longest, l1_entries, guard, nonfinite = torch.cat([counts, flag[:1].to(torch.int64)]).tolist()
+            else:
+                rgb, alpha, _ = ops.render_tilecenter_f32(rays_o, unit_dirs, rec, order, offsets, freq, att, *ws, width,
+                                                          height, 8, 8, threshold)
+                pairs, longest, l1_entries, guard = counts.tolist()
+                nonfinite = 0
+            with self._lock:
+                if guard:
+                    if pairs > cap:
+                        self._queue_capacity = int(pairs * 1.3) + 65536
+                    else:
+                        self._queue_scratch_scale = scale * 4
+                    return None
+                if pairs > 0.9 * cap:                       # stay ahead of a slowly growing scene
+                    self._queue_capacity = int(pairs * 1.3) + 65536
+                if precision != "f32":
+                    self._mfma_calls += 1
+            if longest > self.max_tile_prims:
+                raise RuntimeError(f"{name}: tile candidate capacity {self.max_tile_prims} exceeded (maximum observed "
+                                   f"tile length {longest}); refusing to truncate or use an inconsistent "
+                                   "forward/backward order")
+            if nonfinite:
+                for t in (rays_o, unit_dirs, positions, log_scales, unit_quats, freq, att, *ws):
+                    _chk(bool(torch.isfinite(t).all()), "WMMA input is nonfinite; refusing fallback")
+                warnings.warn("WMMA operand/activation overflow: rendering this frame with scalar FP32 instead")
+                with self._lock:
+                    self._mfma_fallbacks += 1
+                rgb, alpha, _ = ops.render_tilecenter_f32(rays_o, unit_dirs, rec, order, offsets, freq, att, *ws, width,
+                                                          height, 8, 8, threshold)
+                _chk(bool(torch.isfinite(rgb).all()) and bool(torch.isfinite(alpha).all()),
+                     "Scalar FP32 fallback output is nonfinite")
+        return rgb, alpha
+
+    def note_frame_pairs(self, pairs: int):
+        """Seed the candidate-buffer estimate of :meth:`render_frame_queued` from a synchronous frame."""
+        with self._lock:
+            if pairs * 1.1 > self._queue_capacity:
+                self._queue_capacity = int(pairs * 1.3) + 65536
 
     # ------------------------------------------------------------------------------------------
     # training-records forward (np_tile_kernels.cu:6897-6998, forward_only = true)

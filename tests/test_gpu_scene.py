@@ -236,3 +236,48 @@ def test_statistics_collection_through_the_scene_module(device, oracle_mod):
     assert float((rgb - rgb0).abs().max()) < 0.5
     scene.reset_w_stats()
     assert int(scene.stat_hits.sum()) == 0 and float(scene.stat_sum_werr.sum()) == 0.0
+
+
+def test_queued_frames_equal_step_by_step_frames(device, oracle_mod, monkeypatch):
+    # the frame queued without a mid-frame read-back (TileExt.render_frame_queued) is the same frame
+    from mlp_splatting_amd import cumodel
+    from mlp_splatting_amd.tile_ext import TileExt
+    fr = Frame("cfg1_5k_160x120", n=1500, hidden=32, width=64, height=48)
+    for precision in ("f32", "bf16"):
+        monkeypatch.setattr(cumodel, "_tile_ext", TileExt())
+        scene = _scene_from(fr, device)
+        scene.render_precision = precision
+        scene.queued_frames = False
+        ref = _call(scene, fr, device)
+        scene.queued_frames = True
+        ext = cumodel._tile_ext
+        ext._queue_capacity = 0
+        first = _call(scene, fr, device)                 # seeds the candidate-buffer estimate, step by step
+        assert ext._queue_capacity > 0 and torch.equal(first, ref)
+        calls = []
+        real = ext.render_frame_queued
+        monkeypatch.setattr(ext, "render_frame_queued", lambda *a, **k: (calls.append(1), real(*a, **k))[1])
+        assert torch.equal(_call(scene, fr, device), ref) and calls == [1]
+        # an estimate that is too small: the lists were left empty on the device, the frame is repeated
+        # step by step and the estimate grows
+        ext._queue_capacity = 16
+        assert torch.equal(_call(scene, fr, device), ref) and ext._queue_capacity > 1000
+        assert torch.equal(_call(scene, fr, device), ref)
+        # a view matrix edited in place is a new view (the host copy is keyed by the tensor's version)
+        view = to_dev(fr.view, device)
+        kw = dict(score_threshold=fr.thr, proj_matrix=to_dev(fr.proj, device))
+        ro, rd = to_dev(fr.rays_o, device), to_dev(fr.rays_d, device)
+        a = scene(ro, rd, view_matrix=view, **kw)
+        view[0, 3] += 0.5
+        b = scene(ro, rd, view_matrix=view, **kw)
+        scene.queued_frames = False
+        assert torch.equal(a, ref) and torch.equal(scene(ro, rd, view_matrix=view, **kw), b) and not torch.equal(a, b)
+    # the capacity error comes out of the queued path too
+    monkeypatch.setattr(cumodel, "_tile_ext", TileExt())
+    scene = _scene_from(fr, device)
+    _call(scene, fr, device)
+    cand, off = fr.oracle_lists(oracle_mod)
+    longest = int(np.diff(off).max())
+    cumodel._tile_ext.max_tile_prims = longest - 1
+    with pytest.raises(RuntimeError, match=f"capacity {longest - 1} exceeded \\(maximum observed tile length {longest}\\)"):
+        _call(scene, fr, device)
