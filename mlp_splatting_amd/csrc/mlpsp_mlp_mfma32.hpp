@@ -1,0 +1,185 @@
+// Wave-level f32 evaluation of one primitive's 72->32->32->4 MLP for the 64 pixels of a wavefront on the
+// matrix cores, bit-identical to the scalar chain of mlp_fixed<32, 6>.
+//
+// v_mfma_f32_32x32x2_f32 computes, per output element, fma(a1, b1, fma(a0, b0, c)) with both steps
+// rounded as IEEE f32 fused multiply-adds (no flush of denormals): one instruction is two consecutive links
+// of the reference's accumulation chain (np_tile_kernels.cu:2050-2089), so 36 of them walk layer 1 in the
+// order sin_j, cos_j and 16 walk layer 2 in the order h = 2i, 2i+1.
+//
+// Operand layout.  The wavefront's pixels form two column blocks (pixels 0..31 and 32..63), one accumulator
+// tile each.  Lane (n = lane % 32, g = lane / 32) of a 32x32 f32 accumulator tile holds column n and rows
+// 8q + 4g + r in register 4q + r.  The weight rows are fed in permuted order -- row 8q + 4g + r of the
+// A operand is hidden unit 2(4q + r) + g -- so register i of lane (n, g) holds hidden unit 2i + g: exactly
+// the B operand (k = g) of the next layer's i-th instruction.  Layer outputs therefore feed the next layer
+// from registers, with a ReLU in between and no shuffles.  Layer-1 inputs are computed per lane = pixel and
+// moved into operand position by one half-wave swap per sin/cos pair; the same swap brings the 32 layer-2
+// outputs of a pixel onto its own lane for the 4-wide output layer, which runs on the vector ALU with
+// scalar weight operands.
+#pragma once
+#include "mlpsp_device.hpp"
+
+namespace mlpsp {
+
+typedef float mf32x16 __attribute__((ext_vector_type(16)));
+typedef float mf32x4 __attribute__((ext_vector_type(4)));
+
+// Exchanges lanes 32..63 of a with lanes 0..31 of b.
+__device__ __forceinline__ void half_swap(float& a, float& b) {
+  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(a), __float_as_uint(b), false, false);
+  a = __uint_as_float(r[0]);
+  b = __uint_as_float(r[1]);
+}
+__device__ __forceinline__ void half_swap(uint32_t& a, uint32_t& b) {
+  const auto r = __builtin_amdgcn_permlane32_swap(a, b, false, false);
+  a = r[0];
+  b = r[1];
+}
+
+// 16 consecutive floats at src + 16 g  ->  element i = src[2i + g]  (g = lane / 32): eight swaps pair the
+// even entries of the two half-waves.
+__device__ __forceinline__ void load_interleaved16(const float* __restrict__ src, int g, float v[16]) {
+  const mf32x4* __restrict__ s4 = reinterpret_cast<const mf32x4*>(src + 16 * g);
+  float c[16];
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const mf32x4 t = s4[q];
+    c[4 * q + 0] = t[0];
+    c[4 * q + 1] = t[1];
+    c[4 * q + 2] = t[2];
+    c[4 * q + 3] = t[3];
+  }
+#pragma unroll
+  for (int t = 0; t < 8; ++t) {
+    half_swap(c[2 * t], c[2 * t + 1]);   // c[2t] = (src[2t], src[2t+1]), c[2t+1] = (src[16+2t], src[17+2t])
+    v[t] = c[2 * t];
+    v[8 + t] = c[2 * t + 1];
+  }
+}
+
+// max(x, +0): v_max_f32 yields the same bits as x > 0 ? x : 0 for every x (NaN -> 0, -0 -> +0).  Written
+// as a builtin, not as inline assembly: the compiler must see the instruction to keep the wait states
+// between a matrix-core result and its first reader.
+__device__ __forceinline__ float relu_f32(float x) { return __builtin_fmaxf(x, 0.f); }
+
+// The encoding of the ray direction (input components 0..2) does not depend on the primitive: its 18
+// sin/cos pairs are computed once per pixel and kept in B-operand position (after the half-wave swap).
+struct DirOperands {
+  float b0[18], b1[18];
+};
+__device__ __forceinline__ void encode_direction(float rdx, float rdy, float rdz, const float* __restrict__ freq,
+                                                 const float* __restrict__ att, DirOperands& d) {
+  const float x3[3] = {rdx, rdy, rdz};
+#pragma unroll
+  for (int c = 0; c < 3; ++c) {
+#pragma unroll
+    for (int f = 0; f < 6; ++f) {
+      float s, co;
+      det_sincos((x3[c] * freq[f]) * att[f], s, co);
+      half_swap(s, co);
+      d.b0[c * 6 + f] = s;
+      d.b1[c * 6 + f] = co;
+    }
+  }
+}
+
+// All 64 lanes must be active.  x6 is the lane's own pixel's input (components 0..2 enter through dir,
+// which encode_direction() made from them); out is the lane's own pixel's output.
+// REC selects the record kernels' layer-2 rounding (bias added after a chain started at zero) and fills
+// masks[0..1] with the ReLU masks of the lane's pixel.
+template <bool REC = false>
+__device__ __forceinline__ void mlp_wave_mfma32(const float x6[6], const float* __restrict__ freq,
+                                                const float* __restrict__ att, const float* __restrict__ W1,
+                                                const float* __restrict__ b1, const float* __restrict__ W2,
+                                                const float* __restrict__ b2, const float* __restrict__ W3,
+                                                const float* __restrict__ b3, int p, const DirOperands& dir,
+                                                float out[4], uint32_t* masks = nullptr) {
+  constexpr int H = 32, IN = 72, HALF = 36;
+  const int lane = threadIdx.x & 63, m = lane & 31, g = lane >> 5;
+  const int hid = 8 * (m >> 3) + 2 * (m & 3) + ((m >> 2) & 1);
+
+  // A operands: lane (m, g) supplies row hid, k = g of every instruction.
+  float a1[HALF];
+  {
+    const mf32x4* __restrict__ s4 = reinterpret_cast<const mf32x4*>(W1 + (size_t)p * (H * IN) + hid * IN + HALF * g);
+#pragma unroll
+    for (int q = 0; q < HALF / 4; ++q) {
+      const mf32x4 t = s4[q];
+      a1[4 * q + 0] = t[0];
+      a1[4 * q + 1] = t[1];
+      a1[4 * q + 2] = t[2];
+      a1[4 * q + 3] = t[3];
+    }
+  }
+  float a2[16], bias1[16], bias2[16];
+  load_interleaved16(W2 + (size_t)p * (H * H) + hid * H, g, a2);
+  load_interleaved16(b1 + (size_t)p * H, g, bias1);
+  load_interleaved16(b2 + (size_t)p * H, g, bias2);
+
+  mf32x16 d0, d1;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) d0[i] = d1[i] = bias1[i];
+#pragma unroll
+  for (int j = 0; j < 18; ++j) {
+    d0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a1[j], dir.b0[j], d0, 0, 0, 0);
+    d1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a1[j], dir.b1[j], d1, 0, 0, 0);
+  }
+#pragma unroll
+  for (int c = 3; c < 6; ++c) {
+#pragma unroll
+    for (int f = 0; f < 6; ++f) {
+      float s, co;
+      det_sincos((x6[c] * freq[f]) * att[f], s, co);
+      half_swap(s, co);   // s: (sin, cos) of pixels 0..31, co: (sin, cos) of pixels 32..63
+      d0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a1[c * 6 + f], s, d0, 0, 0, 0);
+      d1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a1[c * 6 + f], co, d1, 0, 0, 0);
+    }
+  }
+
+  mf32x16 e0, e1;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) e0[i] = e1[i] = REC ? 0.f : bias2[i];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    e0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a2[i], relu_f32(d0[i]), e0, 0, 0, 0);
+    e1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a2[i], relu_f32(d1[i]), e1, 0, 0, 0);
+  }
+  if constexpr (REC) {
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      e0[i] = bias2[i] + e0[i];
+      e1[i] = bias2[i] + e1[i];
+    }
+  }
+
+  // Output layer on the lane's own pixel: register i of the two blocks, swapped, is (h2[2i], h2[2i+1]).
+  const float* __restrict__ w3 = W3 + (size_t)p * (4 * H);
+  const float* __restrict__ bb3 = b3 + (size_t)p * 4;
+  float acc[4] = {bb3[0], bb3[1], bb3[2], bb3[3]};
+  uint32_t m2 = 0u;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    float even = relu_f32(e0[i]), odd = relu_f32(e1[i]);
+    half_swap(even, odd);
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      acc[k] = fmaf(w3[k * H + 2 * i], even, acc[k]);
+      acc[k] = fmaf(w3[k * H + 2 * i + 1], odd, acc[k]);
+    }
+    if constexpr (REC) m2 |= (even > 0.f ? (1u << (2 * i)) : 0u) | (odd > 0.f ? (2u << (2 * i)) : 0u);
+  }
+#pragma unroll
+  for (int k = 0; k < 4; ++k) out[k] = acc[k];
+  if constexpr (REC) {
+    uint32_t lo = 0u, hi = 0u;   // bits 2i + g of blocks 0 and 1, as held by this lane
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      lo |= d0[i] > 0.f ? (1u << (2 * i + g)) : 0u;
+      hi |= d1[i] > 0.f ? (1u << (2 * i + g)) : 0u;
+    }
+    half_swap(lo, hi);
+    masks[0] = lo | hi;
+    masks[1] = m2;
+  }
+}
+
+}  // namespace mlpsp

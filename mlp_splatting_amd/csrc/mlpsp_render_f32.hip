@@ -42,12 +42,13 @@ MLPSP_API int mlpsp_render_tilecenter_f32(const float* rays_o_dev, const float* 
   const dim3 grid((unsigned)(per_xcd * kNumXcd)), block(64);
   hipStream_t s = (hipStream_t)stream;
   auto* ctr = reinterpret_cast<unsigned long long*>(counters_dev);
-#define MLPSP_F32_LAUNCH(HT, FT)                                                                                  \
-  hipLaunchKernelGGL((render_tilecenter_f32_kernel<HT, FT, 0>), grid, block, 0, s, rays_o_dev, rays_d_dev,        \
+#define MLPSP_F32_LAUNCH(HT, FT, ...)                                                                             \
+  hipLaunchKernelGGL((render_tilecenter_f32_kernel<HT, FT, 0, ##__VA_ARGS__>), grid, block, 0, s, rays_o_dev, rays_d_dev,        \
                      (const PrimRecord*)prim_records_dev, order_dev, tile_offsets_dev, freq_dev, att_dev,         \
                      num_frequencies, W1, b1, W2, b2, W3, b3, num_primitives, hidden, g, wpt, per_xcd, (int)items, threshold,           \
                      out_rgb_dev, out_alpha_dev, out_t_dev, ctr, 0.f, 0.f, HitPool{})
-  if (hidden == 32 && num_frequencies == 6) MLPSP_F32_LAUNCH(32, 6);
+  if (use_mfma32(hidden, num_frequencies, W1, b1, W2, b2)) MLPSP_F32_LAUNCH(32, 6, false, true);
+  else if (hidden == 32 && num_frequencies == 6) MLPSP_F32_LAUNCH(32, 6);
   else if (hidden == 16 && num_frequencies == 6) MLPSP_F32_LAUNCH(16, 6);
   else MLPSP_F32_LAUNCH(0, 0);
 #undef MLPSP_F32_LAUNCH
@@ -82,14 +83,15 @@ MLPSP_API int mlpsp_render_tilecenter_stats_f32(const float* rays_o_dev, const f
   TileGeom g{width, height, tile_w, tile_h, ceil_div(width, tile_w), ceil_div(height, tile_h)};
   const dim3 grid((unsigned)(per_xcd * kNumXcd)), block(64);
   hipStream_t s = (hipStream_t)stream;
-#define MLPSP_STATS_LAUNCH(HT, FT)                                                                               \
-  hipLaunchKernelGGL((render_tilecenter_f32_kernel<HT, FT, 0, true>), grid, block, 0, s, rays_o_dev, rays_d_dev, \
+#define MLPSP_STATS_LAUNCH(HT, FT, ...)                                                                          \
+  hipLaunchKernelGGL((render_tilecenter_f32_kernel<HT, FT, 0, true, ##__VA_ARGS__>), grid, block, 0, s, rays_o_dev, rays_d_dev, \
                      (const PrimRecord*)prim_records_dev, order_dev, tile_offsets_dev, freq_dev, att_dev,        \
                      num_frequencies, W1, b1, W2, b2, W3, b3, num_primitives, hidden, g, wpt, per_xcd,           \
                      (int)items, threshold, out_rgb_dev, out_alpha_dev, (float*)nullptr,                         \
                      (unsigned long long*)nullptr, 0.f, 0.f, HitPool{}, gt_rgb_dev, stat_sum_w_dev,              \
                      stat_max_w_dev, stat_hits_dev, stat_sum_werr_dev, stat_contrib_dev)
-  if (hidden == 32 && num_frequencies == 6) MLPSP_STATS_LAUNCH(32, 6);
+  if (use_mfma32(hidden, num_frequencies, W1, b1, W2, b2)) MLPSP_STATS_LAUNCH(32, 6, true);
+  else if (hidden == 32 && num_frequencies == 6) MLPSP_STATS_LAUNCH(32, 6);
   else if (hidden == 16 && num_frequencies == 6) MLPSP_STATS_LAUNCH(16, 6);
   else MLPSP_STATS_LAUNCH(0, 0);
 #undef MLPSP_STATS_LAUNCH

@@ -1,10 +1,12 @@
 // The scalar-f32 tile-centre render kernel (shared by the RGB entry point and the feature entry point,
 // which asks it to emit hit records).
 #pragma once
+#include <cstdlib>
 #include "mlpsp_device.hpp"
 #include "mlpsp_hitrec.hpp"
 #include "mlpsp_host.hpp"
 #include "mlpsp_mlp.hpp"
+#include "mlpsp_mlp_mfma32.hpp"
 
 namespace mlpsp {
 
@@ -27,7 +29,9 @@ __device__ __forceinline__ float wave_max(float v) {
   return v;
 }
 
-template <int HT, int FT, int EMIT, bool STATS = false>
+// MF: the 72->32->32->4 MLP runs on the matrix cores for all 64 pixels at once (mlp_wave_mfma32, same bits);
+// requires HT == 32, FT == 6 and 16-byte aligned weight arrays.
+template <int HT, int FT, int EMIT, bool STATS = false, bool MF = false>
 __global__ __launch_bounds__(64) void render_tilecenter_f32_kernel(
     const float* __restrict__ rays_o, const float* __restrict__ rays_d, const PrimRecord* __restrict__ prims,
     const int32_t* __restrict__ order, const int32_t* __restrict__ offsets, const float* __restrict__ freq,
@@ -74,6 +78,8 @@ __global__ __launch_bounds__(64) void render_tilecenter_f32_kernel(
     }
   }
   HitEmitter em = hit_emitter_begin(hp, wslot, start, tile);
+  DirOperands dir;
+  if constexpr (MF) encode_direction(rdx, rdy, rdz, freq, att, dir);
 
   for (int i = start; i < end; ++i) {
     const int p = __builtin_amdgcn_readfirstlane(order[i]);
@@ -91,10 +97,12 @@ __global__ __launch_bounds__(64) void render_tilecenter_f32_kernel(
       float w_stat = 0.f;
       if constexpr (EMIT > 0) rs = hit_emitter_next(hp, em, (int)threadIdx.x);
       float* __restrict__ rec = reinterpret_cast<float*>(hp.records + (size_t)(rs < 0 ? 0 : rs) * hp.record_bytes);
+      // (lanes that did not hit carry no hit point; the matrix-core evaluation runs on all 64 lanes)
+      const float x6[6] = {rdx, rdy, rdz, hit ? h.dx : 0.f, hit ? h.dy : 0.f, hit ? h.dz : 0.f};
+      float o[4];
+      if constexpr (MF) mlp_wave_mfma32<false>(x6, freq, att, W1, b1, W2, b2, W3, b3, p, dir, o);
       if (hit) {
-        const float x6[6] = {rdx, rdy, rdz, h.dx, h.dy, h.dz};
-        float o[4];
-        mlp_eval<HT, FT>(x6, freq, att, F, H, mlp, p, o);
+        if constexpr (!MF) mlp_eval<HT, FT>(x6, freq, att, F, H, mlp, p, o);
         const float w = blend_step(acc, o[0], o[1], o[2], o[3], h.decay, h.t);
         w_stat = w;
         if constexpr (EMIT > 0) {
@@ -148,6 +156,17 @@ __global__ __launch_bounds__(64) void render_tilecenter_f32_kernel(
     atomicAdd(counters + 2, (unsigned long long)n_proc_hit);
     atomicAdd(counters + 3, (unsigned long long)n_hits);
   }
+}
+
+// Whether the matrix-core f32 evaluation applies: the fixed 72->32->32->4 shape, weight arrays that can be
+// read 16 bytes at a time, and no request for the scalar kernel (environment MLPSP_F32_SCALAR=1, which
+// exists for comparison runs).
+inline bool use_mfma32(int hidden, int num_frequencies, const float* W1, const float* b1, const float* W2,
+                       const float* b2) {
+  if (hidden != 32 || num_frequencies != 6) return false;
+  if (((uintptr_t)W1 | (uintptr_t)b1 | (uintptr_t)W2 | (uintptr_t)b2) & 15u) return false;
+  const char* e = getenv("MLPSP_F32_SCALAR");
+  return !(e && e[0] == '1');
 }
 
 }  // namespace mlpsp

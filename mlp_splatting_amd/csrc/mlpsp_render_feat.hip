@@ -168,14 +168,17 @@ MLPSP_API int mlpsp_render_tilecenter_feat_f32(
   const int per_xcd = (int)((items + kNumXcd - 1) / kNumXcd);
   TileGeom g{width, height, tile_w, tile_h, ceil_div(width, tile_w), ceil_div(height, tile_h)};
   const dim3 grid((unsigned)(per_xcd * kNumXcd)), block(64);
-#define MLPSP_EMIT_LAUNCH(HT, FT, EM)                                                                             \
-  hipLaunchKernelGGL((render_tilecenter_f32_kernel<HT, FT, EM>), grid, block, 0, s, rays_o_dev, rays_d_dev,       \
+#define MLPSP_EMIT_LAUNCH(HT, FT, EM, ...)                                                                        \
+  hipLaunchKernelGGL((render_tilecenter_f32_kernel<HT, FT, EM, ##__VA_ARGS__>), grid, block, 0, s, rays_o_dev, rays_d_dev,       \
                      (const PrimRecord*)prim_records_dev, order_dev, tile_offsets_dev, freq_dev, att_dev,         \
                      num_frequencies, W1, b1, W2, b2, W3, b3, num_primitives, hidden, g, wpt, per_xcd, (int)items, threshold,          \
                      out_rgb_dev, out_alpha_dev, (float*)nullptr, (unsigned long long*)nullptr, gating_beta,      \
                      gating_temp, hp)
   const bool gated = feat_slots > 1;
-  if (hidden == 32 && num_frequencies == 6) {
+  if (use_mfma32(hidden, num_frequencies, W1, b1, W2, b2)) {
+    if (gated) MLPSP_EMIT_LAUNCH(32, 6, 2, false, true);
+    else MLPSP_EMIT_LAUNCH(32, 6, 1, false, true);
+  } else if (hidden == 32 && num_frequencies == 6) {
     if (gated) MLPSP_EMIT_LAUNCH(32, 6, 2);
     else MLPSP_EMIT_LAUNCH(32, 6, 1);
   } else {
