@@ -7,6 +7,8 @@
 #include "mlpsp_device.hpp"
 #include "mlpsp_host.hpp"
 #include "mlpsp_mlp.hpp"
+#include "mlpsp_mlp_mfma32.hpp"
+#include "mlpsp_render_f32.hpp"
 
 namespace mlpsp {
 
@@ -21,7 +23,8 @@ struct RecordOut {
   float* alpha;               // [B,1]
 };
 
-template <int HT, int FT, bool EMIT>
+// MF: the MLP of a hit runs on the matrix cores for the whole wavefront (mlp_wave_mfma32, same bits).
+template <int HT, int FT, bool EMIT, bool MF = false>
 __global__ __launch_bounds__(64) void records_kernel(
     const float* __restrict__ rays_o, const float* __restrict__ rays_d, const PrimRecord* __restrict__ prims,
     const int32_t* __restrict__ order, const int32_t* __restrict__ offsets, const float* __restrict__ freq,
@@ -49,6 +52,8 @@ __global__ __launch_bounds__(64) void records_kernel(
   float trans = 1.f, cr = 0.f, cg = 0.f, cb = 0.f;
   int used = 0;
   bool over = false;
+  DirOperands dir;
+  if constexpr (MF) encode_direction(rdx, rdy, rdz, freq, att, dir);
   for (int i = start; i < end; ++i) {
     const int p = __builtin_amdgcn_readfirstlane(order[i]);
     if (p < 0 || p >= N) continue;
@@ -57,11 +62,12 @@ __global__ __launch_bounds__(64) void records_kernel(
     const bool can = valid && (trans >= kTransmittanceFloor) && (used < max_hits);
     const bool hit = can && hit_rot(rox, roy, roz, rdx, rdy, rdz, P, thr, h);
     if (__ballot(hit) != 0ull) {
+      const float x6[6] = {rdx, rdy, rdz, hit ? h.dx : 0.f, hit ? h.dy : 0.f, hit ? h.dz : 0.f};
+      float o[4];
+      uint32_t mk[2];
+      if constexpr (MF) mlp_wave_mfma32<true>(x6, freq, att, W1, b1, W2, b2, W3, b3, p, dir, o, mk);
       if (hit) {
-        const float x6[6] = {rdx, rdy, rdz, h.dx, h.dy, h.dz};
-        float o[4];
-        uint32_t mk[2];
-        mlp_eval<HT, FT, true>(x6, freq, att, F, H, mlp, p, o, mk);
+        if constexpr (!MF) mlp_eval<HT, FT, true>(x6, freq, att, F, H, mlp, p, o, mk);
         const float R = sigmoid(o[0]), G = sigmoid(o[1]), Bc = sigmoid(o[2]);
         const float sigma_raw = softplus(o[3]);
         const float sigma = sigma_raw * h.decay;
@@ -134,13 +140,14 @@ int records_launch(bool emit, const float* rays_o, const float* rays_d, const vo
   const int per_xcd = (int)((items + kNumXcd - 1) / kNumXcd);
   TileGeom g{width, height, tile_w, tile_h, ceil_div(width, tile_w), ceil_div(height, tile_h)};
   const dim3 grid((unsigned)(per_xcd * kNumXcd)), block(64);
-#define MLPSP_REC_LAUNCH(HT, FT, EM)                                                                              \
-  hipLaunchKernelGGL((records_kernel<HT, FT, EM>), grid, block, 0, s, rays_o, rays_d, (const PrimRecord*)prims,   \
+#define MLPSP_REC_LAUNCH(HT, FT, ...)                                                                             \
+  hipLaunchKernelGGL((records_kernel<HT, FT, ##__VA_ARGS__>), grid, block, 0, s, rays_o, rays_d, (const PrimRecord*)prims,   \
                      order, offsets, freq, att, F, W1, b1, W2, b2, W3, b3, N, hidden, g, wpt, per_xcd, (int)items, \
                      thr, max_hits, beta, temp, counts, overflow, out)
 #define MLPSP_REC_SHAPES(EM)                                          \
   do {                                                                \
-    if (hidden == 32 && F == 6) MLPSP_REC_LAUNCH(32, 6, EM);          \
+    if (use_mfma32(hidden, F, W1, b1, W2, b2)) MLPSP_REC_LAUNCH(32, 6, EM, true); \
+    else if (hidden == 32 && F == 6) MLPSP_REC_LAUNCH(32, 6, EM);     \
     else if (hidden == 16 && F == 6) MLPSP_REC_LAUNCH(16, 6, EM);     \
     else MLPSP_REC_LAUNCH(0, 0, EM);                                  \
   } while (0)

@@ -199,6 +199,74 @@ def test_tilecentre_render_is_bit_exact_config1(device, oracle_mod, frame1):
     np.testing.assert_array_equal(counters[1:], want["stats"][1:])   # processed, with-hit, hits
 
 
+def test_scalar_and_matrix_core_f32_evaluations_agree_bit_for_bit(device, oracle_mod, frame1, monkeypatch):
+    """The 72-32-32-4 shape runs on the matrix cores; MLPSP_F32_SCALAR=1 and weight arrays that are not
+    16-byte aligned select the scalar kernel.  All three must produce the oracle's bits."""
+    from mlp_splatting_amd import ops
+    fr = frame1
+    cand, off = fr.lists
+    want = oracle_mod.render_tilecenter(*fr.base_numpy(cand, off), *fr.dims)
+    monkeypatch.setenv("MLPSP_F32_SCALAR", "1")
+    rgb, alpha, _, _ = _render_gpu(fr, device, cand, off)
+    monkeypatch.delenv("MLPSP_F32_SCALAR")
+    _assert_bits(rgb, want["rgb"], "rgb (scalar kernel)")
+    _assert_bits(alpha, want["alpha"], "alpha (scalar kernel)")
+    sc = fr.scene
+    rec = ops.prepare_primitives(_t(sc.positions, device), _t(sc.log_scales, device), _t(sc.quats, device))
+    ro, rd, c, o = _t(fr.rays_o, device), _t(fr.rays_d, device), _t(cand, device), _t(off, device)
+    order, _ = ops.sort_tiles(ro, rd, rec, c, o, fr.W, fr.H, fr.tile, fr.tile)
+    weights = []
+    for w in sc.mlp():                      # every array starts 4 bytes past a 16-byte boundary
+        flat = torch.empty(w.size + 1, dtype=torch.float32, device=device)
+        flat[1:] = _t(w, device).reshape(-1)
+        weights.append(flat[1:].view(*w.shape))
+        assert weights[-1].data_ptr() % 16 == 4 and weights[-1].is_contiguous()
+    rgb2, alpha2, _ = ops.render_tilecenter_f32(ro, rd, rec, order, o, _t(sc.freq, device), _t(sc.att, device),
+                                                *weights, fr.W, fr.H, fr.tile, fr.tile, fr.thr)
+    _assert_bits(rgb2, want["rgb"], "rgb (unaligned weights)")
+    _assert_bits(alpha2, want["alpha"], "alpha (unaligned weights)")
+
+
+def test_non_finite_activations_take_the_same_path_in_both_f32_evaluations(device, oracle_mod, monkeypatch):
+    """Huge and non-finite weights of a few primitives (inf - inf, NaN through a ReLU, overflow to inf) must
+    give the oracle's image -- NaN positions included -- from the matrix-core and the scalar kernel."""
+    fr = Frame("cfg1_5k_160x120", n=1200, width=64, height=48)
+    sc = fr.scene
+    cand, off = fr.oracle_lists(oracle_mod)
+    t = int(np.argmax(np.diff(off)))
+    ids = [int(v) for v in dict.fromkeys(cand[off[t]:off[t + 1]].tolist())][:6]     # primitives of the fullest tile
+    W1, b1, W2, b2, W3, b3 = [w.copy() for w in sc.mlp()]
+    W1[ids[0], 5, :] = 3e38
+    W1[ids[0], 6, :] = -3e38
+    b1[ids[1], 0] = np.nan
+    W2[ids[2], 2, 3] = np.inf
+    W2[ids[3], :, :] = 1e30
+    W3[ids[4], 3, :] = -np.inf
+    W3[ids[5], 0, 7] = np.nan
+    sc.W1, sc.b1, sc.W2, sc.b2, sc.W3, sc.b3 = W1, b1, W2, b2, W3, b3
+    weights = sc.mlp()
+    want = oracle_mod.render_tilecenter(*fr.base_numpy(cand, off), *fr.dims)
+    from mlp_splatting_amd import ops
+    rec = ops.prepare_primitives(_t(sc.positions, device), _t(sc.log_scales, device), _t(sc.quats, device))
+    ro, rd, c, o = _t(fr.rays_o, device), _t(fr.rays_d, device), _t(cand, device), _t(off, device)
+    order, _ = ops.sort_tiles(ro, rd, rec, c, o, fr.W, fr.H, fr.tile, fr.tile)
+    outs = []
+    for scalar in (False, True):
+        if scalar:
+            monkeypatch.setenv("MLPSP_F32_SCALAR", "1")
+        rgb, alpha, _ = ops.render_tilecenter_f32(ro, rd, rec, order, o, _t(sc.freq, device), _t(sc.att, device),
+                                                  *[_t(w, device) for w in weights], fr.W, fr.H, fr.tile, fr.tile, fr.thr)
+        outs.append((rgb.cpu().numpy(), alpha.cpu().numpy()))
+    monkeypatch.delenv("MLPSP_F32_SCALAR")
+    nan_a, nan_b = np.isnan(outs[0][0]), np.isnan(outs[1][0])
+    np.testing.assert_array_equal(nan_a, nan_b)
+    assert np.array_equal(bits(outs[0][0])[~nan_a], bits(outs[1][0])[~nan_b])
+    assert np.array_equal(bits(outs[0][1])[~np.isnan(outs[0][1])], bits(outs[1][1])[~np.isnan(outs[1][1])])
+    assert (~nan_a).mean() > 0.5 and nan_a.any()
+    np.testing.assert_array_equal(np.isnan(want["rgb"]), nan_a)
+    assert np.array_equal(bits(want["rgb"])[~nan_a], bits(outs[0][0])[~nan_a])
+
+
 def test_expected_depth_render_is_bit_exact(device, oracle_mod, frame1):
     fr = frame1
     cand, off = fr.lists
