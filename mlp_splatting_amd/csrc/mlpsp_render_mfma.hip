@@ -65,6 +65,11 @@ template <> struct Ops<__bf16> {
   }
   static __device__ __forceinline__ float round_trip(float a) { return (float)(__bf16)a; }
   static constexpr float kMax = 3.38953139e38f;
+  // bf16 has the exponent range of f32: a hidden pre-activation is out of range only if it is (within one
+  // rounding step of) +-inf.  Rounded to +inf it survives the ReLU and turns the next layer's sums into
+  // +-inf or NaN, down to the outputs, whose finiteness every hit checks; rounded to -inf the ReLU removes
+  // it, as it does in exact arithmetic.  The per-layer range check is therefore not needed for this type.
+  static constexpr bool kCheckHidden = false;
 };
 template <> struct Ops<_Float16> {
   using vec8 = f16x8;
@@ -77,6 +82,7 @@ template <> struct Ops<_Float16> {
   }
   static __device__ __forceinline__ float round_trip(float a) { return (float)(_Float16)a; }
   static constexpr float kMax = 65504.0f;
+  static constexpr bool kCheckHidden = true;   // a finite f32 pre-activation above 65504 must be reported
 };
 
 // hidden-unit index held by D register r of lane group g
@@ -150,13 +156,6 @@ __global__ __launch_bounds__(64) void pack_mfma_weights_kernel(const float* __re
 // True if some pre-activation is +-inf or exceeds the operand type's range.  A NaN cannot appear here
 // on its own: the operands are finite (weights are checked when packed, phases when encoded), so a
 // non-finite accumulator is an overflow, which shows as +-inf -- and the max chain sees infinities.
-// One-instruction forms.  fmaxf() in C costs two (the compiler first quiets a possible signalling NaN
-// with v_max x,x,x), which would double the 64 ReLUs per (tile, primitive).
-__device__ __forceinline__ float relu(float x) {
-  float y;
-  asm("v_max_f32_e32 %0, 0, %1" : "=v"(y) : "v"(x));
-  return y;
-}
 // ReLU of two packed 16-bit floats in one instruction: as signed 16-bit integers every negative float
 // (and -0) is below zero and every non-negative one keeps its bits, for bf16 and fp16 alike; rounding
 // commutes with ReLU, so rounding first gives the same operand.
@@ -170,9 +169,13 @@ __device__ __forceinline__ float max3_abs(float a, float b, float c) {
   asm("v_max3_f32 %0, |%1|, |%2|, |%3|" : "=v"(y) : "v"(a), "v"(b), "v"(c));
   return y;
 }
+// The first read of the accumulator tile is a plain C++ operation, not inline assembly: the compiler
+// inserts the wait states a matrix-core result needs before its first reader only for instructions it
+// can see, and everything below depends on that first read.
 template <typename T>
 __device__ __forceinline__ bool out_of_range_in(const f32x16& v) {
-  float m = max3_abs(v[0], v[1], v[2]);
+  float m = __builtin_fabsf(v[0]);
+  m = max3_abs(m, v[1], v[2]);
 #pragma unroll
   for (int r = 3; r < 15; r += 2) m = max3_abs(m, v[r], v[r + 1]);
   m = max3_abs(m, v[15], v[15]);
@@ -258,6 +261,27 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 4))) void
   // the pixel this lane shares an MFMA column with: lane l and lane l^32 both hold column l%32
   const float prdx = __shfl_xor(rdx, 32), prdy = __shfl_xor(rdy, 32), prdz = __shfl_xor(rdz, 32);
 
+  // The encoding of the ray direction (input components 0..2, operand words 0..8 of both column blocks) does
+  // not depend on the primitive: it is computed once per pixel and parked in LDS in operand form -- 18 more
+  // live registers would cost the fourth wavefront per SIMD.  One wavefront per workgroup: no barrier.
+  __shared__ u32x4 s_dirq[2][2][64];
+  __shared__ unsigned s_dir8[2][64];
+#pragma unroll
+  for (int b = 0; b < 2; ++b) {
+    const bool own = (b == g);
+    const float xd[3] = {own ? rdx : prdx, own ? rdy : prdy, own ? rdz : prdz};
+    unsigned wd[9];
+#pragma unroll
+    for (int t = 0; t < 9; ++t) {
+      const float kf = (t % 3 == 0) ? kf0 : ((t % 3 == 1) ? kf1 : kf2);
+      const float rev = xd[t / 3] * kf;
+      wd[t] = Ops<T>::pack2(__builtin_amdgcn_sinf(rev), __builtin_amdgcn_cosf(rev));
+    }
+    s_dirq[b][0][l] = u32x4{wd[0], wd[1], wd[2], wd[3]};
+    s_dirq[b][1][l] = u32x4{wd[4], wd[5], wd[6], wd[7]};
+    s_dir8[b][l] = wd[8];
+  }
+
   const int start = offsets[tile], end = offsets[tile + 1];
   PixelAcc acc = {0.f, 0.f, 0.f, 1.f, 0.f, 0.f};
   HitEmitter em = hit_emitter_begin(hp, 0, start, tile);
@@ -299,8 +323,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 4))) void
         const unsigned half_mask = (unsigned)(mask >> (32 * b));
         if (half_mask != 0u) {   // wave-uniform: skip a 32-pixel block nobody hits
           const bool own = (b == g);
-          const float xin[6] = {own ? rdx : prdx, own ? rdy : prdy, own ? rdz : prdz,
-                                own ? h.dx : pdx, own ? h.dy : pdy, own ? h.dz : pdz};
+          const float xin[3] = {own ? h.dx : pdx, own ? h.dy : pdy, own ? h.dz : pdz};
           const bool col_active = (half_mask >> (l & 31)) & 1u;
           // biases are the C operand of each layer's first MFMA; an MFMA overwrites its C registers,
           // so each column block fetches its own copy (L1-resident) instead of copying 32 registers
@@ -315,16 +338,28 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 4))) void
               d2[4 * q + e] = v2[e];
             }
           }
-          // layer 1: 18 (sin, cos) words per lane, 5 K-steps
+          // layer 1: 18 (sin, cos) words per lane, 5 K-steps; words 0..8 come from LDS.  (The lane index is
+          // made opaque so that the loads stay here and are not hoisted out of the primitive loop into
+          // registers.)
+          int ll = l;
+          asm volatile("" : "+v"(ll));
+          const u32x4 dq0 = s_dirq[b][0][ll], dq1 = s_dirq[b][1][ll];
+          const unsigned d8 = s_dir8[b][ll];
 #pragma unroll
           for (int s = 0; s < 5; ++s) {
             u32x4 bw;
 #pragma unroll
             for (int d = 0; d < 4; ++d) {
               const int t = 4 * s + d;
-              if (t < 18) {
+              if (t < 4) {
+                bw[d] = dq0[d];
+              } else if (t < 8) {
+                bw[d] = dq1[d];
+              } else if (t == 8) {
+                bw[d] = d8;
+              } else if (t < 18) {
                 const float kf = (t % 3 == 0) ? kf0 : ((t % 3 == 1) ? kf1 : kf2);
-                const float rev = xin[t / 3] * kf;
+                const float rev = xin[t / 3 - 3] * kf;
                 bw[d] = Ops<T>::pack2(__builtin_amdgcn_sinf(rev), __builtin_amdgcn_cosf(rev));
               } else {
                 bw[d] = 0u;
@@ -332,7 +367,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 4))) void
             }
             d1 = Ops<T>::mfma(a1[s], bw, d1);
           }
-          bad |= col_active && out_of_range_in<T>(d1);
+          if constexpr (Ops<T>::kCheckHidden) bad |= col_active && out_of_range_in<T>(d1);
           // layer 2: the D registers, rectified and rounded, are the next B operand
 #pragma unroll
           for (int s = 0; s < 2; ++s) {
@@ -342,7 +377,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 4))) void
               bw[d] = relu_packed(Ops<T>::pack2(d1[8 * s + 2 * d], d1[8 * s + 2 * d + 1]));
             d2 = Ops<T>::mfma(a2[s], bw, d2);
           }
-          bad |= col_active && out_of_range_in<T>(d2);
+          if constexpr (Ops<T>::kCheckHidden) bad |= col_active && out_of_range_in<T>(d2);
           // layer 3: rows 0..3 of a 32-row product; row k lands in register k of lane group 0
           f32x16 d3 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
