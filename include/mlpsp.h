@@ -41,7 +41,7 @@ extern "C" {
 
 #define MLPSP_TILE_CAPACITY_MAX 2048 /* largest per-tile list the in-LDS sort accepts */
 #define MLPSP_PIXEL_HIT_CAPACITY 256 /* per-pixel-order hit buffer (np_tile_kernels.cu:760) */
-#define MLPSP_PRIM_RECORD_BYTES 64   /* bytes per primitive of the prepared geometry buffer */
+#define MLPSP_PRIM_RECORD_BYTES 128  /* bytes per primitive of the prepared geometry buffer */
 #define MLPSP_MFMA_PACK_BYTES 7808   /* bytes per primitive of the packed matrix-core weight buffer */
 
 #define MLPSP_KEY_LIST_ORDER 0 /* consume the list as given (presorted kernel, np_tile_kernels.cu:4242-4478) */
@@ -57,9 +57,10 @@ int mlpsp_version(void);
  * (np_tile_kernels.cu:4578-4598). */
 const char* mlpsp_strerror(int code);
 
-/* Per-primitive geometry in kernel-ready form: centre, exp(-2 log_s), unit quaternion, log_s.
+/* Per-primitive geometry in kernel-ready form: centre, exp(-2 log_s), unit quaternion, log_s, exp(2 log_s)
+ * and the quaternion's rotation matrix (quats_dev must hold unit quaternions).
  * Replaces the per-candidate gathers + __expf of np_tile_kernels.cu:1947-1956, 676-678.
- * prim_records_dev: N * MLPSP_PRIM_RECORD_BYTES bytes, 64-byte aligned. */
+ * prim_records_dev: N * MLPSP_PRIM_RECORD_BYTES bytes, 128-byte aligned. */
 int mlpsp_prepare_primitives(const float* positions_dev, const float* log_scales_dev, const float* quats_dev,
                              int num_primitives, void* prim_records_dev, mlpsp_stream_t stream);
 

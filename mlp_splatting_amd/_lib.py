@@ -18,7 +18,7 @@ E_MIXED_ORIGINS, E_WIDE_CONE = 256, 512
 KEY_LIST_ORDER, KEY_TSTAR, KEY_DEPTH = 0, 1, 2
 TILE_CAPACITY_MAX = 2048
 PIXEL_HIT_CAPACITY = 256
-PRIM_RECORD_BYTES = 64
+PRIM_RECORD_BYTES = 128
 MFMA_PACK_BYTES = 7808
 
 _vp, _i, _f, _i64, _sz = C.c_void_p, C.c_int, C.c_float, C.c_int64, C.c_size_t

@@ -7,7 +7,7 @@
 namespace mlpsp {
 
 // ---------------------------------------------------------------------------------------------
-// prepare: [N,3]+[N,3]+[N,4] -> one 64-byte record per primitive (HBM-bound: 40 B in, 64 B out)
+// prepare: [N,3]+[N,3]+[N,4] -> one 128-byte record per primitive (HBM-bound: 40 B in, 128 B out)
 // ---------------------------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void prepare_primitives_kernel(const float* __restrict__ pos,
                                                                  const float* __restrict__ logs,
@@ -37,6 +37,14 @@ __global__ __launch_bounds__(256) void prepare_primitives_kernel(const float* __
   dst[1] = make_float4(r.my, r.mz, r.qw, r.qx);
   dst[2] = make_float4(r.qy, r.qz, r.lgx, r.lgy);
   dst[3] = make_float4(r.lgz, r.s2x, r.s2y, r.s2z);
+  // R(q)^T of the unit quaternion, row by row
+  const float w = r.qw, x = r.qx, y = r.qy, z = r.qz;
+  dst[4] = make_float4(1.f - 2.f * (y * y + z * z), 2.f * (x * y + w * z), 2.f * (x * z - w * y),
+                       2.f * (x * y - w * z));
+  dst[5] = make_float4(1.f - 2.f * (x * x + z * z), 2.f * (y * z + w * x), 2.f * (x * z + w * y),
+                       2.f * (y * z - w * x));
+  dst[6] = make_float4(1.f - 2.f * (x * x + y * y), 0.f, 0.f, 0.f);
+  dst[7] = make_float4(0.f, 0.f, 0.f, 0.f);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -296,7 +304,7 @@ MLPSP_API int mlpsp_prepare_primitives(const float* positions_dev, const float* 
   if (num_primitives < 0) return MLPSP_E_ARGUMENT;
   if (num_primitives == 0) return MLPSP_OK;
   if (!positions_dev || !log_scales_dev || !quats_dev || !prim_records_dev) return MLPSP_E_ARGUMENT;
-  if (reinterpret_cast<uintptr_t>(prim_records_dev) % 64 != 0) return MLPSP_E_ARGUMENT;
+  if (reinterpret_cast<uintptr_t>(prim_records_dev) % 128 != 0) return MLPSP_E_ARGUMENT;
   hipLaunchKernelGGL(prepare_primitives_kernel, dim3(ceil_div(num_primitives, 256)), dim3(256), 0,
                      (hipStream_t)stream, positions_dev, log_scales_dev, quats_dev, num_primitives,
                      (PrimRecord*)prim_records_dev);

@@ -126,15 +126,20 @@ __device__ __forceinline__ Vec3 quat_rotate_conj(float qw, float qx, float qy, f
   return quat_rotate(qw, -qx, -qy, -qz, v);
 }
 
-// One primitive's geometry as the kernels consume it: 16 floats, 64-byte aligned, written by
-// the prepare kernel.  m = exp(-2 log_s) is the diagonal of the precision matrix, s2 = exp(2 log_s)
-// the squared semi-axes (used only by the conservative tile culling of the sort kernel).
-struct __attribute__((aligned(64))) PrimRecord {
+// One primitive's geometry as the kernels consume it: 128 bytes, written by the prepare kernel.
+// m = exp(-2 log_s) is the diagonal of the precision matrix, s2 = exp(2 log_s) the squared semi-axes (used
+// only by the conservative tile culling of the sort kernel).  rt is the world -> local rotation as a matrix,
+// rt[k] = row k of R(q)^T; only the reduced-precision render path uses it (three dot products per vector
+// instead of the quaternion form, which the exact paths must keep to reproduce the reference's roundings).
+struct __attribute__((aligned(128))) PrimRecord {
   float cx, cy, cz, mx;
   float my, mz, qw, qx;
   float qy, qz, lgx, lgy;
   float lgz, s2x, s2y, s2z;
+  float rt[3][3];
+  float pad[7];
 };
+static_assert(sizeof(PrimRecord) == 128, "record size is part of the C ABI");
 
 struct HitInfo {
   float t, dx, dy, dz, qlx, qly, qlz, decay;

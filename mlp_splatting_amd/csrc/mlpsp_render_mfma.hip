@@ -220,6 +220,43 @@ __device__ __forceinline__ void fast_tetra_gates(float qlx, float qly, float qlz
   g[3] = e3 * inv;
 }
 
+// Ray against rotated ellipsoid for this path: same quantities as hit_rot() (np_tile_kernels.cu:659-711), with
+// the world -> local rotation applied as a matrix, the local hit offset taken as vl - t dl (equal to the
+// rotated world offset up to rounding), and the native reciprocal and exp2.  About a third of the
+// instructions of the exactly-rounded form; the differences are of the order of f32 rounding (about 1e-5
+// relative in decay, through the cancellation in vl - t dl).
+//
+// The hit decision itself is a hard threshold, and a primitive that barely hits still contributes up to a
+// few 1e-3 to a pixel, so a decision that differs from the exact path's would show as isolated pixel
+// errors well above the rounding noise of this path.  unsure = the fast quantities are too close to one of
+// the three decision boundaries (decay within 0.4 % of thr, t or denom near zero) to be trusted; the
+// caller then takes the decision -- only the decision -- from hit_rot().
+__device__ __forceinline__ bool hit_rot_fast(float rox, float roy, float roz, float rdx, float rdy, float rdz,
+                                             const PrimRecord& P, float thr, HitInfo& h, bool& unsure) {
+  const float vx = P.cx - rox, vy = P.cy - roy, vz = P.cz - roz;
+  const float dlx = fmaf(P.rt[0][0], rdx, fmaf(P.rt[0][1], rdy, P.rt[0][2] * rdz));
+  const float dly = fmaf(P.rt[1][0], rdx, fmaf(P.rt[1][1], rdy, P.rt[1][2] * rdz));
+  const float dlz = fmaf(P.rt[2][0], rdx, fmaf(P.rt[2][1], rdy, P.rt[2][2] * rdz));
+  const float vlx = fmaf(P.rt[0][0], vx, fmaf(P.rt[0][1], vy, P.rt[0][2] * vz));
+  const float vly = fmaf(P.rt[1][0], vx, fmaf(P.rt[1][1], vy, P.rt[1][2] * vz));
+  const float vlz = fmaf(P.rt[2][0], vx, fmaf(P.rt[2][1], vy, P.rt[2][2] * vz));
+  const float ax = P.mx * dlx, ay = P.my * dly, az = P.mz * dlz;
+  const float denom = fmaf(ax, dlx, fmaf(ay, dly, az * dlz));
+  const float numer = fmaf(ax, vlx, fmaf(ay, vly, az * vlz));
+  const float t = numer * __builtin_amdgcn_rcpf(denom);
+  h.t = t;
+  h.dx = fmaf(-t, rdx, vx);
+  h.dy = fmaf(-t, rdy, vy);
+  h.dz = fmaf(-t, rdz, vz);
+  h.qlx = fmaf(-t, dlx, vlx);
+  h.qly = fmaf(-t, dly, vly);
+  h.qlz = fmaf(-t, dlz, vlz);
+  const float r2 = fmaf(P.mx * h.qlx, h.qlx, fmaf(P.my * h.qly, h.qly, (P.mz * h.qlz) * h.qlz));
+  h.decay = __builtin_amdgcn_exp2f(fmaxf(r2, 0.f) * -0.72134752f);
+  unsure = (__builtin_fabsf(h.decay - thr) <= 4e-3f * thr) || !(__builtin_fabsf(t) >= 1e-4f) || !(denom >= 1e-18f);
+  return !(denom <= 1e-20f) && !(t <= 0.f) && (h.decay > thr);
+}
+
 // SP = 0: RGB only.  SP = 4 or 8: the kernel also emits, per tile, the compact list of primitives that
 // hit at least one pixel (hit records, mlpsp_hitrec.hpp) and per (such primitive, pixel) the SP compositing
 // coefficients of the gated feature channel, rounded to fp16 (they lie in [0, 1]; fp16 keeps 11
@@ -292,7 +329,14 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 4))) void
     const PrimRecord P = prims[p];
     HitInfo h;
     const bool live = valid && (acc.trans >= kTransmittanceFloor);
-    const bool hit = live && hit_rot(rox, roy, roz, rdx, rdy, rdz, P, thr, h);
+    bool unsure;
+    bool hit = hit_rot_fast(rox, roy, roz, rdx, rdy, rdz, P, thr, h, unsure) && live;
+    if (__ballot(unsure && live) != 0ull) {   // rare (about one wavefront step in twenty)
+      if (unsure && live) {
+        HitInfo exact;
+        hit = hit_rot(rox, roy, roz, rdx, rdy, rdz, P, thr, exact);
+      }
+    }
     const unsigned long long mask = __ballot(hit);
     ++n_proc;
     if (mask != 0ull) {
