@@ -351,8 +351,11 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 4))) void
       for (int s = 0; s < 2; ++s) a2[s] = *reinterpret_cast<const u32x4*>(blk + kOffW2 + s * 1024 + l * 16);
 #pragma unroll
       for (int s = 0; s < 2; ++s) {
-        a3[s] = u32x4{0u, 0u, 0u, 0u};
-        if ((l & 31) < 4) a3[s] = *reinterpret_cast<const u32x4*>(blk + kOffW3 + ((s * 2 + g) * 4 + (l & 3)) * 16);
+        // every lane loads one of the four stored rows (no divergent branch, no wait in the middle of the
+        // staging); rows 4..31 of the operand are zero
+        const u32x4 row = *reinterpret_cast<const u32x4*>(blk + kOffW3 + ((s * 2 + g) * 4 + (l & 3)) * 16);
+        const bool stored = (l & 31) < 4;
+        a3[s] = u32x4{stored ? row[0] : 0u, stored ? row[1] : 0u, stored ? row[2] : 0u, stored ? row[3] : 0u};
       }
       const f32x4 b3v = *reinterpret_cast<const f32x4*>(blk + kOffB3);
       const int wflag = *reinterpret_cast<const int32_t*>(blk + kOffFlag);
