@@ -130,14 +130,14 @@ def main() -> int:
     freq, att = scene._frequency_tables(dev)
     quats = torch.nn.functional.normalize(scene.quats.detach(), dim=-1).contiguous()
     weights = [p.detach().contiguous() for p in (scene.W1, scene.b1, scene.W2, scene.b2, scene.W3, scene.b3)]
-    kernel_ms, hits, proc, cand_total, sort_ms, bin_ms = 0.0, 0, 0, 0, 0.0, 0.0
+    kernel_ms, hits, proc, cand_total, sort_ms, bin_ms, hit_waves = 0.0, 0, 0, 0, 0.0, 0.0, 0
     packed = ops.pack_mfma_weights(*weights, bf16=True) if precision == "bf16" else None
     n_probe = min(len(frames), 8)
     # two passes over the same poses: the first only warms the allocator (a first-time tensor size inside
     # the event brackets would be timed as kernel time), the second is measured
     for i in list(range(n_probe)) * 2:
         if i == 0:
-            kernel_ms, hits, proc, cand_total, sort_ms, bin_ms = 0.0, 0, 0, 0, 0.0, 0.0
+            kernel_ms, hits, proc, cand_total, sort_ms, bin_ms, hit_waves = 0.0, 0, 0, 0, 0.0, 0.0, 0
         ro, rd_raw, views, tv = frames[i]
         rd = torch.nn.functional.normalize(rd_raw, dim=-1).contiguous()
         e = [torch.cuda.Event(enable_timing=True) for _ in range(4)]
@@ -162,6 +162,7 @@ def main() -> int:
         c = counters.cpu().numpy()
         hits += int(c[3])
         proc += int(c[1])
+        hit_waves += int(c[2])
         cand_total += int(cand.numel())
     # what the matrix cores sustain on this box with nothing else in the way
     mfma_probe = None
@@ -176,6 +177,24 @@ def main() -> int:
         e1.record()
         torch.cuda.synchronize()
         mfma_probe = round(probe_flops / (e0.elapsed_time(e1) * 1e-3) / 1e12, 1)
+    # do the matrix pipe and the vector ALU of one SIMD overlap?  (mlpsp_probe_issue: modes 0..3)
+    lib = _lib.load()
+    stream = torch.cuda.current_stream(dev).cuda_stream
+    sink = torch.zeros(1, device=dev)
+    probe_ms = []
+    for mode in range(4):
+        lib.mlpsp_probe_issue(mode, 500, sink.data_ptr(), stream)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        lib.mlpsp_probe_issue(mode, 20000, sink.data_ptr(), stream)
+        e1.record()
+        torch.cuda.synchronize()
+        probe_ms.append(e0.elapsed_time(e1))
+    serial, ideal = 0.5 * (probe_ms[0] + probe_ms[1]), 0.5 * max(probe_ms[0], probe_ms[1])
+    issue_probe = {"mfma_ms": round(probe_ms[0], 4), "valu_ms": round(probe_ms[1], 4), "mixed_ms": round(probe_ms[2], 4),
+                   "mixed_if_serial_ms": round(serial, 4), "mixed_if_overlapped_ms": round(ideal, 4),
+                   "overlap": round((serial - probe_ms[2]) / max(serial - ideal, 1e-9), 3),
+                   "sin_issue_vs_fma": round((probe_ms[3] / 2.0) / (probe_ms[1] / 8.0), 2)}
     flops_per_hit = 2 * (72 * sc.hidden + sc.hidden * sc.hidden + 4 * sc.hidden)
     achieved_tflops = flops_per_hit * hits / (kernel_ms * 1e-3) / 1e12
     # sort kernel: 8 compulsory bytes per candidate (4 id in, 4 id out) + the 64-byte record of every primitive
@@ -201,8 +220,9 @@ def main() -> int:
                      "frac": round(achieved_tflops / PEAK[precision], 5),
                      "traffic": MEASURED_TRAFFIC_BYTES.get((args.workload, precision)),
                      "ms_per_launch": round(kernel_ms / n_probe, 4), "hits_per_launch": hits // n_probe,
-                     "tile_primitives_per_launch": proc // n_probe, "flops_per_hit": flops_per_hit,
-                     "measured_mfma_peak": mfma_probe},
+                     "tile_primitives_per_launch": proc // n_probe,
+                     "hit_wavefronts_per_launch": hit_waves // n_probe, "flops_per_hit": flops_per_hit,
+                     "measured_mfma_peak": mfma_probe, "issue_probe": issue_probe},
         "stages": {"bin_ms": round(bin_ms / n_probe, 4), "sort_ms": round(sort_ms / n_probe, 4),
                    "render_ms": round(kernel_ms / n_probe, 4),
                    "sort_hbm": {"bound": "hbm", "achieved": round(sort_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",

@@ -58,6 +58,7 @@ SIGNATURES = {
     "mlpsp_render_tilecenter_mfma_feat": (_i, [_vp] * 5 + [_i64, _vp, _vp, _vp, _i, _i, _vp, _i, _i, _f, _f, _i, _i, _f,
                                                _vp, _sz, _vp, _vp, _vp, _vp, _vp, _vp]),
     "mlpsp_probe_mfma_bf16": (_i64, [_i, _vp, _vp]),
+    "mlpsp_probe_issue": (_i, [_i, _i, _vp, _vp]),
 }
 
 _lib = None

@@ -671,6 +671,42 @@ __global__ __launch_bounds__(256) void probe_mfma_bf16_kernel(int iterations, fl
   if (v == 12345.678f) sink[0] = v;      // keeps the accumulations alive; practically never true
 }
 
+// Measurement aid: do matrix-core and vector-ALU instructions of different wavefronts of one SIMD run
+// concurrently?  Workgroups of 8 wavefronts, one per CU, so every SIMD holds two.  mode 0: all wavefronts
+// issue one 32x32x16 bf16 MFMA per iteration (32 cycles of the matrix pipe); mode 1: all issue 8 independent
+// f32 FMAs per iteration (32 cycles of the vector ALU); mode 2: on every SIMD one wavefront does the
+// former and one the latter; mode 3: all issue 2 v_sin_f32 per iteration.  If the two pipes overlapped,
+// mode 2 would take as long as the slower of modes 0 and 1 run with one wavefront per SIMD, i.e. half of
+// their two-wavefront times; it takes about the sum.
+__global__ __launch_bounds__(512) void probe_issue_kernel(int mode, int iterations, float* __restrict__ sink) {
+  const int wave = threadIdx.x >> 6;
+  const bool do_mfma = mode == 0 || (mode == 2 && wave < 4);
+  const bool do_valu = mode == 1 || (mode == 2 && wave >= 4);
+  u32x4 a = {0x3f803f80u + threadIdx.x, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u}, b = a;
+  f32x16 acc = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  float v[8];
+#pragma unroll
+  for (int k = 0; k < 8; ++k) v[k] = 1e-3f * (float)(threadIdx.x + k);
+  const float m = 1.0001f, c = 1e-3f * (float)threadIdx.x;
+  if (do_mfma) {
+    for (int it = 0; it < iterations; ++it) acc = Ops<__bf16>::mfma(a, b, acc);
+  } else if (do_valu) {
+    for (int it = 0; it < iterations; ++it) {
+#pragma unroll
+      for (int k = 0; k < 8; ++k) v[k] = fmaf(v[k], m, c);
+    }
+  } else if (mode == 3) {
+    for (int it = 0; it < iterations; ++it) {
+      v[0] = __builtin_amdgcn_sinf(v[0]);
+      v[1] = __builtin_amdgcn_sinf(v[1]);
+    }
+  }
+  float r = acc[0];
+#pragma unroll
+  for (int k = 0; k < 8; ++k) r += v[k];
+  if (r == 12345.678f) sink[0] = r;
+}
+
 }  // namespace mlpsp
 
 using namespace mlpsp;
@@ -823,4 +859,11 @@ MLPSP_API int64_t mlpsp_probe_mfma_bf16(int iterations, float* sink_dev, mlpsp_s
   hipLaunchKernelGGL(probe_mfma_bf16_kernel, dim3(blocks), dim3(256), 0, (hipStream_t)stream, iterations, sink_dev);
   if (hipGetLastError() != hipSuccess) return -1;
   return (int64_t)blocks * 4 * iterations * 8 * (2LL * 32 * 32 * 16);   // FLOPs issued
+}
+
+MLPSP_API int mlpsp_probe_issue(int mode, int iterations, float* sink_dev, mlpsp_stream_t stream) {
+  if (mode < 0 || mode > 3 || iterations <= 0 || !sink_dev) return MLPSP_E_ARGUMENT;
+  hipLaunchKernelGGL(probe_issue_kernel, dim3(256), dim3(512), 0, (hipStream_t)stream, mode, iterations, sink_dev);
+  MLPSP_LAUNCH_CHECK();
+  return MLPSP_OK;
 }
