@@ -23,8 +23,7 @@ HBM_PEAK_GBS = 8000.0
 #   rocprofv3 --pmc WRITE_SIZE -- (same)
 # averaged over the run's 56 launches, each counter scaled by what it reads for the 1 GiB device copies of
 # --copy-calibration (FETCH_SIZE reads 524,307 KiB for 1,048,576 KiB copied: factor 2.0; WRITE_SIZE reads
-# 1,048,576 KiB: factor 1.0).  Render kernel: 121,921 KiB x 2.0 fetched + 54,889 KiB written (this includes the
-# scratch traffic of the values the kernel's 128-register budget spills).
+# 1,048,576 KiB: factor 1.0).  Render kernel: 50,777 KiB x 2.0 fetched + 16,813 KiB written.
 MEASURED_TRAFFIC_BYTES = {("cfg3_200k_1200x680", "bf16"): int((121920.7 * 2.0 + 54889.0) * 1024)}
 
 
