@@ -272,6 +272,28 @@ int mlpsp_render_tilecenter_mfma_feat(const float* rays_o_dev, const float* rays
                                       float* out_rgb_dev, float* out_alpha_dev, float* out_feat_dev,
                                       int32_t* status_dev, int64_t* counters_dev, mlpsp_stream_t stream);
 
+/* Weight and bias gradients of the per-primitive 72->32->32->4 MLP over a primitive-major CSR of hit records
+ * = the Triton kernel _grouped_vjp (scannet/primitive_gemm.py:101-166, launched at :214-230).  Segment g covers
+ * records [group_starts[g], min(group_starts[g] + segment, csr_offsets[group_primitives[g] + 1])) of primitive
+ * group_primitives[g]; x6 [R,6] are the saved MLP inputs, grad4 [R,4] the adjoints of the four pre-activation
+ * outputs, relu_masks [R,2] the saved activation masks (NULL: recompute them from the forward pass).
+ * precision 0: IEEE f32 products and sums (fp32 MFMA), 1: fp16 operands, 2: bf16 operands, always with f32
+ * accumulation over the segment; grad4 is multiplied by scale before rounding and the result divided by it.
+ * partial_dev [num_groups, 3524] receives W1 (2304) | b1 (32) | W2 (1024) | b2 (32) | W3 (128) | b3 (4) per
+ * segment.  segment must be a positive multiple of 32. */
+int mlpsp_grouped_vjp(const float* x6_dev, const float* grad4_dev, const int32_t* relu_masks_dev,
+                      const int64_t* csr_offsets_dev, const int64_t* group_primitives_dev,
+                      const int64_t* group_starts_dev, int64_t num_groups, const float* freq_dev,
+                      const float* att_dev, const float* W1, const float* b1, const float* W2, const float* b2,
+                      const float* W3, int precision, float scale, int segment, float* partial_dev,
+                      mlpsp_stream_t stream);
+
+/* Sum of every primitive's segments = _reduce_partials (scannet/primitive_gemm.py:169-183): out_dev
+ * [num_primitives, 3524] = sum over g in [group_offsets[p], group_offsets[p+1]) of partial_dev[g];
+ * nonfinite_dev[0] is cleared and then set to 1 if any sum is NaN or infinite. */
+int mlpsp_reduce_partials(const float* partial_dev, const int64_t* group_offsets_dev, int num_primitives,
+                          float* out_dev, int32_t* nonfinite_dev, mlpsp_stream_t stream);
+
 /* Measurement aid, no counterpart in the reference: launches a kernel that does nothing but
  * v_mfma_f32_32x32x16_bf16 on register operands (2,048 workgroups x 4 wavefronts x iterations x 8
  * instructions) and returns the FLOPs it issues (-1 on error); time it on the stream to see what the

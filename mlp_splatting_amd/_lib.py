@@ -59,6 +59,9 @@ SIGNATURES = {
                                                _vp, _sz, _vp, _vp, _vp, _vp, _vp, _vp]),
     "mlpsp_probe_mfma_bf16": (_i64, [_i, _vp, _vp]),
     "mlpsp_probe_issue": (_i, [_i, _i, _vp, _vp]),
+    "mlpsp_grouped_vjp": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _f, _i, _vp,
+                               _vp]),
+    "mlpsp_reduce_partials": (_i, [_vp, _vp, _i, _vp, _vp, _vp]),
 }
 
 _lib = None

@@ -2,9 +2,9 @@
 ``scannet/primitive_gemm.py``: segment layout of a primitive-major CSR, its identity/version guards, the
 non-finite retry policy and its counters, and argument validation of ``grouped_weight_gradients``.
 
-The device kernels behind ``_launch_grouped_vjp`` belong to training (the reference writes them in Triton,
-scannet/primitive_gemm.py:101-183); they are not part of the forward renderer and are not built here, so
-``_launch_grouped_vjp`` raises.  Everything above it is real and tested on the CPU.
+The device kernels behind ``_launch_grouped_vjp`` (Triton in the reference, scannet/primitive_gemm.py:101-183)
+are the HIP kernels ``mlpsp_grouped_vjp`` / ``mlpsp_reduce_partials`` of libmlpsp_hip: one wavefront per segment,
+32x32 MFMA tiles, f32 accumulation over the segment.
 """
 from __future__ import annotations
 
@@ -120,10 +120,37 @@ def resolve_groups(csr, segment_size=512, groups=None):
     return groups.validate(csr, segment_size)
 
 
+_PRECISION_CODE = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
+
+
 def _launch_grouped_vjp(csr, freq, attenuation, weights, groups, dtype, block_size, scale):
-    """(result [n,3524], nonfinite flag).  The segment VJP kernels are training-side and not built."""
-    raise NotImplementedError("the grouped MLP VJP kernels belong to training and are not part of this forward-render "
-                              "build; primitive_csr.reference_weight_gradients is the per-primitive f32 reference")
+    """(result [n,3524] f32, nonfinite flag [1] int32): per-segment partial gradients, then their sum per
+    primitive (scannet/primitive_gemm.py:214-230).  ``block_size`` only chose the Triton tile height; the
+    HIP kernel always walks a segment in blocks of 32 records."""
+    from . import _lib
+    lib = _lib.load()
+    group_primitives, group_starts, group_offsets = groups
+    device = weights[0].device
+    n = len(weights[0])
+    num_groups = int(group_primitives.numel())
+    partial = torch.empty((max(num_groups, 1), sum(PACKED_GRADIENT_SIZES)), dtype=torch.float32, device=device)
+    result = torch.empty((n, sum(PACKED_GRADIENT_SIZES)), dtype=torch.float32, device=device)
+    flag = torch.zeros(1, dtype=torch.int32, device=device)
+    stream = torch.cuda.current_stream(device).cuda_stream
+    masks = csr.relu_masks
+    with torch.cuda.device(device):
+        rc = lib.mlpsp_grouped_vjp(csr.x6.data_ptr(), csr.grad4.data_ptr(), masks.data_ptr() if masks is not None else None,
+                                   csr.offsets.data_ptr(), group_primitives.data_ptr(), group_starts.data_ptr(),
+                                   num_groups, freq.data_ptr(), attenuation.data_ptr(), *[w.data_ptr() for w in weights[:5]],
+                                   _PRECISION_CODE[dtype], float(scale), int(groups.segment_size), partial.data_ptr(),
+                                   stream)
+        if rc != 0:
+            raise RuntimeError(f"mlpsp_grouped_vjp: {_lib.strerror(rc)}")
+        rc = lib.mlpsp_reduce_partials(partial.data_ptr(), group_offsets.data_ptr(), n, result.data_ptr(),
+                                       flag.data_ptr(), stream)
+        if rc != 0:
+            raise RuntimeError(f"mlpsp_reduce_partials: {_lib.strerror(rc)}")
+    return result, flag
 
 
 @torch.no_grad()
