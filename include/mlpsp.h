@@ -294,6 +294,19 @@ int mlpsp_grouped_vjp(const float* x6_dev, const float* grad4_dev, const int32_t
 int mlpsp_reduce_partials(const float* partial_dev, const int64_t* group_offsets_dev, int num_primitives,
                           float* out_dev, int32_t* nonfinite_dev, mlpsp_stream_t stream);
 
+/* Reverse compositing over saved forward records = primitive_records_reverse_kernel
+ * (scannet/cuda/primitive_records.cuh:3-46; argument checks of its wrapper :48-74 are the caller's).
+ * ids [R], pixel_offsets [num_pixels+1] (int64), x6 [R,6], raw [R,8] as written by mlpsp_records_emit;
+ * grad_rgb [num_pixels,3], grad_t [num_pixels] = adjoint of the final transmittance.  Writes d4 [R,4], the
+ * adjoint of the four pre-activation MLP outputs of every record, and ACCUMULATES (after clearing) the
+ * gradients of positions [N,3], log-scales [N,3] and quaternions [N,4] that flow through the Gaussian
+ * falloff, with f32 atomics (summation order not fixed).  raw, d4 and quats must be 16-byte aligned. */
+int mlpsp_records_reverse(const int32_t* ids_dev, const int64_t* pixel_offsets_dev, const float* x6_dev,
+                          const float* raw_dev, const float* log_scales_dev, const float* quats_dev,
+                          const float* grad_rgb_dev, const float* grad_t_dev, int64_t num_pixels, int num_primitives,
+                          float* d4_dev, float* grad_positions_dev, float* grad_log_scales_dev, float* grad_quats_dev,
+                          mlpsp_stream_t stream);
+
 /* Measurement aid, no counterpart in the reference: launches a kernel that does nothing but
  * v_mfma_f32_32x32x16_bf16 on register operands (2,048 workgroups x 4 wavefronts x iterations x 8
  * instructions) and returns the FLOPs it issues (-1 on error); time it on the stream to see what the

@@ -412,3 +412,17 @@ def render_tilecenter_mfma_feat(rays_o, rays_d, records, order, tile_offsets, fr
             return rgb, alpha, feat, (bool(host_flag[0]) if check else flag)
     _check(code, "mlpsp_render_tilecenter_mfma_feat")
     return rgb, alpha, feat, (bool(flag[0].item()) if check else flag)
+
+
+def records_reverse(ids, offsets, x6, raw, log_scales, quats, grad_rgb, grad_t):
+    """Reverse compositing over saved records -> (d4 [R,4], grad_positions, grad_log_scales, grad_quats)."""
+    dev = ids.device
+    total, pixels, n = ids.numel(), grad_rgb.shape[0], log_scales.shape[0]
+    d4 = torch.empty((total, 4), dtype=torch.float32, device=dev)
+    gp, gs = torch.empty_like(log_scales), torch.empty_like(log_scales)
+    gq = torch.empty_like(quats)
+    with torch.cuda.device(dev):
+        _check(_lib.load().mlpsp_records_reverse(_ptr(ids), _ptr(offsets), _ptr(x6), _ptr(raw), _ptr(log_scales),
+                                                 _ptr(quats), _ptr(grad_rgb), _ptr(grad_t), pixels, n, _ptr(d4), _ptr(gp),
+                                                 _ptr(gs), _ptr(gq), _stream(dev)), "mlpsp_records_reverse")
+    return d4, gp, gs, gq

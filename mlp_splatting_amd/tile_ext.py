@@ -24,7 +24,7 @@ _BACKWARD_ONLY = (
     "render_tiles_backward_featattr_per_pixel", "render_tiles_backward_featattr_tilecenter",
     "render_tiles_backward_tilecenter_full", "render_tiles_backward_tilecenter_full_with_feat",
     "render_tiles_mlp_records", "render_tiles_training_records_wmma",
-    "primitive_records_reverse", "render_tiles_backward_tilecenter_traversal",
+    "render_tiles_backward_tilecenter_traversal",
     "render_tiles_backward_tilecenter_backprop_noatomic", "training_wmma_safety_stats",
 )
 
@@ -351,6 +351,29 @@ class TileExt:
                                           self.max_tile_prims, cull_threshold=float(threshold))
             return list(ops.training_records(x[0], x[1], rec, order, x[6], x[7], x[8], *x[9:15], width, height, tile,
                                              tile, float(threshold), float(beta), float(temp), self.max_hits, name))
+
+    def primitive_records_reverse(self, ids, offsets, x6, raw, logs, quats, grgb, gt):
+        """[d4, grad_positions, grad_log_scales, grad_quats] from saved forward records
+        (scannet/cuda/primitive_records.cuh:48-74: same argument checks, then one reverse walk per pixel)."""
+        tensors = (ids, offsets, x6, raw, logs, quats, grgb, gt)
+        for t in tensors:
+            _chk(t.is_cuda and t.is_contiguous() and t.device == ids.device)
+        _chk(ids.dtype == torch.int32 and offsets.dtype == torch.int64)
+        for t in (x6, raw, logs, quats, grgb, gt):
+            _chk(t.dtype == torch.float32)
+        total, pixels, n = ids.numel(), grgb.shape[0], logs.shape[0]
+        _chk(ids.dim() == 1 and offsets.dim() == 1 and offsets.numel() == pixels + 1)
+        _chk(x6.dim() == 2 and tuple(x6.shape) == (total, 6))
+        _chk(raw.dim() == 2 and tuple(raw.shape) == (total, 8))
+        _chk(logs.dim() == 2 and logs.shape[1] == 3)
+        _chk(quats.dim() == 2 and tuple(quats.shape) == (n, 4))
+        _chk(grgb.dim() == 2 and grgb.shape[1] == 3 and gt.dim() == 1 and gt.numel() == pixels)
+        _chk(int(offsets[0]) == 0 and int(offsets[-1]) == total)
+        _chk(bool((offsets[1:] >= offsets[:-1]).all()))
+        if total:
+            lo, hi = torch.aminmax(ids)
+            _chk(int(lo) >= 0 and int(hi) < n)
+        return list(ops.records_reverse(ids, offsets, x6, raw, logs, quats, grgb, gt))
 
     # ------------------------------------------------------------------------------------------
     # statistics forward (pruning statistics are not rebuilt; the render itself is)

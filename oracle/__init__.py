@@ -271,5 +271,21 @@ def render_per_pixel(rays_o, rays_d, pos, log_s, quats, cand, offsets, freq, att
     return {"rgb": rgb, "alpha": alpha, "feat": feat, "overflow": bool(ov)}
 
 
+def records_reverse(ids, offsets, x6, raw, log_s, quats, grad_rgb, grad_t):
+    """Reverse compositing over saved records -> (d4[R,4], grad_positions[N,3], grad_log_scales[N,3],
+    grad_quats[N,4]), f32, summed sequentially."""
+    ids = np.ascontiguousarray(ids, np.int32)
+    offsets = np.ascontiguousarray(offsets, np.int64)
+    x6, raw = np.ascontiguousarray(x6, np.float32), np.ascontiguousarray(raw, np.float32)
+    log_s, quats = np.ascontiguousarray(log_s, np.float32), np.ascontiguousarray(quats, np.float32)
+    grad_rgb, grad_t = np.ascontiguousarray(grad_rgb, np.float32), np.ascontiguousarray(grad_t, np.float32)
+    d4 = np.zeros((ids.size, 4), np.float32)
+    gp, gs, gq = np.zeros_like(log_s), np.zeros_like(log_s), np.zeros_like(quats)
+    lib().mlpsp_oracle_records_reverse(_p(ids, _i), _p(offsets, _l), _p(x6, _f), _p(raw, _f), _p(log_s, _f),
+                                       _p(quats, _f), _p(grad_rgb, _f), _p(grad_t, _f), C.c_int64(grad_t.size),
+                                       _p(d4, _f), _p(gp, _f), _p(gs, _f), _p(gq, _f))
+    return d4, gp, gs, gq
+
+
 def num_threads() -> int:
     return int(lib().mlpsp_oracle_num_threads())

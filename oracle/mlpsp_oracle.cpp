@@ -27,6 +27,8 @@
 //   gates / feature ...................................... pinned by softmax closed form + framebuffer sum
 //   training records ..................................... pinned by recomposition (sum T a c = rgb,
 //       T' = T (1 - a)), the forward image within 2e-6, masks against an einsum restatement
+//   reverse compositing over records ..................... pinned against float64 autograd through a
+//       differentiable restatement of the compositing (tests/test_oracle_render.py)
 //   pruning statistics ................................... pinned by the geometric-series weights of
 //       stacked identical primitives and by sum_p sum_w[p] = sum_pixels alpha
 //   bf16/fp16 mixed-precision MLP ........................ pinned against a numpy emulation of the
@@ -1106,6 +1108,63 @@ ORACLE_API int mlpsp_oracle_render_per_pixel(
     out_alpha[pix] = 1.f - ps.trans;
   }
   return overflow;
+}
+
+// ------------------------------------------------------------------------------------------
+// Reverse compositing over saved forward records (scannet/cuda/primitive_records.cuh:3-46): per pixel, last
+// record first, the adjoint d4 of the four pre-activation MLP outputs of every record and the geometry
+// gradients that flow through the Gaussian falloff `decay` (the hit offset x6[3:6] is treated as given):
+// grad of positions, log-scales and quaternions, accumulated per primitive.  Here sequential (pixels
+// ascending), so the sums have one fixed order; the device kernels add with atomics in any order.
+// quaternion gradient: chain rule through the rotation matrix, np_tile_kernels.cu:439-479.
+// ------------------------------------------------------------------------------------------
+ORACLE_API void mlpsp_oracle_records_reverse(const int32_t* ids, const int64_t* offsets, const float* x6,
+                                             const float* raw, const float* logs, const float* quats,
+                                             const float* grgb, const float* gt, int64_t pixels, float* d4,
+                                             float* gp, float* gs, float* gq) {
+  for (int64_t pix = 0; pix < pixels; ++pix) {
+    float next = gt[pix];
+    const float g0 = grgb[pix * 3], g1 = grgb[pix * 3 + 1], g2 = grgb[pix * 3 + 2];
+    for (int64_t r = offsets[pix + 1] - 1; r >= offsets[pix]; --r) {
+      const int p = ids[r];
+      const float* v = raw + r * 8;
+      const float R = v[0], G = v[1], B = v[2], sigma_raw = v[3], trans = v[4], alpha = v[5], decay = v[6];
+      const float dotg = (g0 * R + g1 * G) + g2 * B;
+      const float grad_alpha = trans * (dotg - next);
+      next = next * (1.f - alpha) + dotg * alpha;
+      const float grad_sigma = grad_alpha * det_exp(-sigma_raw * decay);
+      const float grad_decay = grad_sigma * sigma_raw;
+      d4[r * 4 + 0] = g0 * (trans * alpha) * R * (1.f - R);
+      d4[r * 4 + 1] = g1 * (trans * alpha) * G * (1.f - G);
+      d4[r * 4 + 2] = g2 * (trans * alpha) * B * (1.f - B);
+      d4[r * 4 + 3] = grad_sigma * decay * o_sigmoid(v[7]);
+      const float dx = x6[r * 6 + 3], dy = x6[r * 6 + 4], dz = x6[r * 6 + 5];
+      const float qw = quats[p * 4], qx = quats[p * 4 + 1], qy = quats[p * 4 + 2], qz = quats[p * 4 + 3];
+      const V3 q = quat_rotate_conj(qw, qx, qy, qz, V3{dx, dy, dz});
+      const float mx = det_exp(-2.f * logs[p * 3]), my = det_exp(-2.f * logs[p * 3 + 1]),
+                  mz = det_exp(-2.f * logs[p * 3 + 2]);
+      const float gx = -grad_decay * decay * mx * q.x;
+      const float gy = -grad_decay * decay * my * q.y;
+      const float gz = -grad_decay * decay * mz * q.z;
+      const V3 gd = quat_rotate(qw, qx, qy, qz, V3{gx, gy, gz});
+      gp[p * 3] += gd.x;
+      gp[p * 3 + 1] += gd.y;
+      gp[p * 3 + 2] += gd.z;
+      gs[p * 3] += grad_decay * decay * mx * q.x * q.x;
+      gs[p * 3 + 1] += grad_decay * decay * my * q.y * q.y;
+      gs[p * 3 + 2] += grad_decay * decay * mz * q.z * q.z;
+      const float r00 = dx * gx, r01 = dx * gy, r02 = dx * gz, r10 = dy * gx, r11 = dy * gy, r12 = dy * gz,
+                  r20 = dz * gx, r21 = dz * gy, r22 = dz * gz;
+      gq[p * 4] += r01 * (-2.f * qz) + r02 * (2.f * qy) + r10 * (2.f * qz) + r12 * (-2.f * qx) + r20 * (-2.f * qy) +
+                   r21 * (2.f * qx);
+      gq[p * 4 + 1] += r01 * (2.f * qy) + r02 * (2.f * qz) + r10 * (2.f * qy) + r11 * (-4.f * qx) + r12 * (-2.f * qw) +
+                       r20 * (2.f * qz) + r21 * (2.f * qw) + r22 * (-4.f * qx);
+      gq[p * 4 + 2] += r00 * (-4.f * qy) + r01 * (2.f * qx) + r02 * (2.f * qw) + r10 * (2.f * qx) + r12 * (2.f * qz) +
+                       r20 * (-2.f * qw) + r21 * (2.f * qz) + r22 * (-4.f * qy);
+      gq[p * 4 + 3] += r00 * (-4.f * qz) + r01 * (-2.f * qw) + r02 * (2.f * qx) + r10 * (2.f * qw) + r11 * (-4.f * qz) +
+                       r12 * (2.f * qy) + r20 * (2.f * qx) + r21 * (2.f * qy);
+    }
+  }
 }
 
 ORACLE_API int mlpsp_oracle_num_threads(void) { return omp_get_max_threads(); }

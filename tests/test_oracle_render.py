@@ -442,3 +442,71 @@ def test_records_recompose_the_image_and_match_the_forward_render(oracle_mod):
         assert np.array_equal(bitsm[sure], (pre > 0)[sure].astype(np.int64)) and sure.mean() > 0.99
     o3 = np.einsum("rh,rh->r", sc.W3[ids, 3].astype(np.float64), np.maximum(pre2, 0)) + sc.b3[ids, 3]
     np.testing.assert_allclose(raw[:, 7], o3, atol=2e-5)
+
+
+def _synthetic_records(seed, pixels=40, n=12, max_per_pixel=9):
+    """Random per-pixel record lists with every raw field computed in float64 from leaves, plus the float64
+    autograd gradients of  sum_pix (grad_rgb . rgb + grad_t * T_final)."""
+    g = torch.Generator().manual_seed(seed)
+    counts = torch.randint(0, max_per_pixel + 1, (pixels,), generator=g)
+    counts[0], counts[1] = 0, max_per_pixel
+    offsets = torch.zeros(pixels + 1, dtype=torch.int64)
+    offsets[1:] = counts.cumsum(0)
+    R = int(offsets[-1])
+    ids = torch.randint(0, n, (R,), generator=g)
+    d = (torch.randn(R, 3, generator=g) * 0.08).double()
+    o = torch.randn(R, 4, generator=g).double().requires_grad_(True)
+    dpos = torch.zeros(n, 3, dtype=torch.float64, requires_grad=True)
+    log_s = (torch.randn(n, 3, generator=g) * 0.3 - 2.3).double().requires_grad_(True)
+    q0 = torch.randn(n, 4, generator=g).double()
+    quats = (q0 / q0.norm(dim=1, keepdim=True)).requires_grad_(True)
+    grad_rgb = torch.randn(pixels, 3, generator=g).double()
+    grad_t = torch.randn(pixels, generator=g).double()
+
+    w, x, y, z = quats[ids].unbind(1)
+    rot = torch.stack([torch.stack([1 - 2 * (y * y + z * z), 2 * (x * y - w * z), 2 * (x * z + w * y)], 1),
+                       torch.stack([2 * (x * y + w * z), 1 - 2 * (x * x + z * z), 2 * (y * z - w * x)], 1),
+                       torch.stack([2 * (x * z - w * y), 2 * (y * z + w * x), 1 - 2 * (x * x + y * y)], 1)], 1)
+    local = torch.einsum("rji,rj->ri", rot, d + dpos[ids])                 # R(q)^T (offset)
+    decay = torch.exp(-0.5 * (torch.exp(-2 * log_s[ids]) * local * local).sum(1))
+    colour = torch.sigmoid(o[:, :3])
+    sigma_raw = torch.nn.functional.softplus(o[:, 3])
+    alpha = 1 - torch.exp(-sigma_raw * decay)
+    trans = torch.ones(R, dtype=torch.float64)
+    loss = torch.zeros((), dtype=torch.float64)
+    trans_rows = []
+    for pix in range(pixels):
+        t = torch.ones((), dtype=torch.float64)
+        for r in range(int(offsets[pix]), int(offsets[pix + 1])):
+            trans_rows.append(t)
+            loss = loss + (grad_rgb[pix] * colour[r]).sum() * t * alpha[r]
+            t = t * (1 - alpha[r])
+        loss = loss + grad_t[pix] * t
+    loss.backward()
+    trans = torch.stack(trans_rows) if trans_rows else trans
+    raw = torch.cat([colour, sigma_raw[:, None], trans[:, None], alpha[:, None], decay[:, None], o[:, 3:4]], 1).detach()
+    x6 = torch.cat([torch.zeros(R, 3, dtype=torch.float64), d], 1)
+    want = (o.grad, dpos.grad, log_s.grad, quats.grad)
+    inputs = (ids.int().numpy(), offsets.numpy(), x6.float().numpy(), raw.float().numpy(), log_s.detach().float().numpy(),
+              quats.detach().float().numpy(), grad_rgb.float().numpy(), grad_t.float().numpy())
+    return inputs, [w.numpy() for w in want]
+
+
+@pytest.mark.parametrize("seed", [0, 1, 2])
+def test_reverse_compositing_matches_float64_autograd(oracle_mod, seed):
+    # primitive_records.cuh:3-46: d4 = dL/d(pre-activation outputs); geometry gradients through the falloff
+    # only (the hit offset is an input), which is exactly what differentiating the restatement above gives
+    inputs, want = _synthetic_records(seed)
+    got = oracle_mod.records_reverse(*inputs)
+    for name, a, b in zip(("d4", "grad_positions", "grad_log_scales", "grad_quats"), got, want):
+        scale = max(1.0, float(np.abs(b).max()))
+        assert np.abs(a - b).max() <= 2e-5 * scale, (name, float(np.abs(a - b).max()), scale)
+        assert np.abs(b).max() > 1e-3, name      # a gradient that is identically zero would pin nothing
+
+
+def test_reverse_compositing_of_empty_pixels_is_zero(oracle_mod):
+    z = np.zeros
+    d4, gp, gs, gq = oracle_mod.records_reverse(z(0, np.int32), z(5, np.int64), z((0, 6), np.float32), z((0, 8), np.float32),
+                                                z((3, 3), np.float32), np.tile(np.float32([1, 0, 0, 0]), (3, 1)),
+                                                np.ones((4, 3), np.float32), np.ones(4, np.float32))
+    assert d4.shape == (0, 4) and not gp.any() and not gs.any() and not gq.any()
