@@ -186,6 +186,49 @@ def _add_background(rgb, alpha, bg):
     return rgb + (1.0 - alpha).clamp(0.0, 1.0) * bg.view(1, 3)
 
 
+class _TileRenderAutogradFn(torch.autograd.Function):
+    """RGB render with gradients for geometry and MLP weights (scannet/cumodel.py:219-378).  The forward is the
+    ordinary f32 render; the backward re-traverses the frame (``render_tiles_backward_tilecenter_full``)."""
+
+    @staticmethod
+    def forward(ctx, rays_o, rays_d, positions, log_scales, quats, culled_prim_indices, tile_offsets, freq, att,
+                W1, b1, W2, b2, W3, b3, Wimg, Himg, TW, TH, threshold, mode, bg_color):
+        ext = NeuralPrimitiveSceneTileCUDA._ensure_tile_ext_static()
+        args = (rays_o, rays_d, positions, log_scales, quats, culled_prim_indices, tile_offsets, freq, att,
+                W1, b1, W2, b2, W3, b3)
+        dims = (int(Wimg), int(Himg), int(TW), int(TH), float(threshold))
+        if mode == 0:
+            rgb, alpha = ext.render_tiles_forward(*args, *dims)
+        elif mode == 1:
+            rgb, alpha = ext.render_tiles_forward_tilecenter(*args, *dims)
+        else:
+            raise ValueError("Unsupported tile mode for backward")
+        rgb = _add_background(rgb, alpha, bg_color)
+        ctx.save_for_backward(*args)
+        ctx.dims, ctx.mode, ctx.bg_color = dims, int(mode), bg_color
+        return rgb
+
+    @staticmethod
+    def backward(ctx, grad_out_rgb):
+        args = ctx.saved_tensors
+        grad_out_rgb = grad_out_rgb.contiguous()
+        if ctx.bg_color is None:
+            grad_t_end = torch.zeros(args[0].shape[0], device=grad_out_rgb.device, dtype=grad_out_rgb.dtype)
+        else:
+            bg = ctx.bg_color.to(device=grad_out_rgb.device, dtype=grad_out_rgb.dtype)
+            if bg.numel() == 1:
+                bg = bg.repeat(3)
+            grad_t_end = (grad_out_rgb * bg.view(1, 3)).sum(dim=-1)
+        if ctx.mode != 1:
+            raise NotImplementedError("the backward of the per-pixel order render is not built; train with the "
+                                      "tile-centre order (MLPSP_TILE_ORDER_MODE=tilecenter, the default)")
+        ext = NeuralPrimitiveSceneTileCUDA._ensure_tile_ext_static()
+        gW1, gb1, gW2, gb2, gW3, gb3, gp, gs, gq = ext.render_tiles_backward_tilecenter_full(
+            *args, grad_out_rgb, grad_t_end, *ctx.dims)
+        return (None, None, gp, gs, gq, None, None, None, None, gW1, gb1, gW2, gb2, gW3, gb3,
+                None, None, None, None, None, None, None)
+
+
 class NeuralPrimitiveSceneTileCUDA(nn.Module):
     """Tile-based single-pass MLP-splatting renderer: full-frame rays in, image out.
 
@@ -442,6 +485,11 @@ class NeuralPrimitiveSceneTileCUDA(nn.Module):
         assert ray_o.shape[0] == W * H, "Tile renderer requires full-frame rays (B == W*H)"
         device = self._activate_cuda_device()
         ts = int(self.tile_size)
+        if (torch.is_grad_enabled() and feature_target is None and not (return_feature and self.feat_attr is not None)
+                and any(t.requires_grad for t in (self.positions, self.log_scales, self.quats, self.W1, self.b1,
+                                                  self.W2, self.b2, self.W3, self.b3))):
+            return self._forward_differentiable(ray_o, ray_d, score_threshold, bg_color, view_matrix, proj_matrix,
+                                                culled_prim_indices, tile_offsets, return_feature, device)
         with torch.no_grad():
             # queued before the binning, whose pair count is a blocking read-back: the device then has
             # this work to do while the host waits, instead of idling while the host issues it afterwards
@@ -495,6 +543,28 @@ class NeuralPrimitiveSceneTileCUDA(nn.Module):
             else:
                 rgb, alpha, feat = ext.render_tiles_forward_per_pixel_with_feat(*base, *feat_args, *dims)
             return _add_background(rgb, alpha, bg), feat
+
+    def _forward_differentiable(self, ray_o, ray_d, score_threshold, bg_color, view_matrix, proj_matrix,
+                                culled_prim_indices, tile_offsets, return_feature, device):
+        """RGB with autograd (scannet/cumodel.py:1110-1131): tile lists and encodings are constants, positions,
+        log-scales, normalised quaternions and MLP weights carry gradients."""
+        W, H = self.image_size
+        ts = int(self.tile_size)
+        with torch.no_grad():
+            unit_dirs = F.normalize(ray_d, dim=-1).contiguous()
+            culled_prim_indices, tile_offsets = self._tile_lists(
+                ray_o, ray_d, score_threshold, view_matrix, proj_matrix, culled_prim_indices, tile_offsets, device)
+            freq, att = self._frequency_tables(device)
+        mode = 1 if self._resolve_tile_order_mode() == "tilecenter" else 0
+        rgb = _TileRenderAutogradFn.apply(
+            ray_o.contiguous(), unit_dirs, self.positions.contiguous(), self.log_scales.contiguous(),
+            F.normalize(self.quats, dim=-1).contiguous(), culled_prim_indices, tile_offsets.to(torch.int32), freq, att,
+            self.W1.contiguous(), self.b1.contiguous(), self.W2.contiguous(), self.b2.contiguous(),
+            self.W3.contiguous(), self.b3.contiguous(), int(W), int(H), ts, ts, float(score_threshold), mode,
+            self._background(bg_color, ray_o))
+        if return_feature and self.feat_attr is None:
+            raise RuntimeError("return_feature=True requested but feat_attr is not initialized.")
+        return rgb
 
     def _forward_queued(self, ext, ray_o, unit_dirs, score_threshold, view_matrix, proj_matrix, bg_color, device):
         """The RGB frame with binning, sort and render queued back to back and one read-back at the end

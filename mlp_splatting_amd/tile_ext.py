@@ -22,7 +22,7 @@ _BACKWARD_ONLY = (
     "render_tiles_backward_count_per_pixel", "render_tiles_backward_count_tilecenter",
     "render_tiles_backward_emit_per_pixel", "render_tiles_backward_emit_tilecenter",
     "render_tiles_backward_featattr_per_pixel", "render_tiles_backward_featattr_tilecenter",
-    "render_tiles_backward_tilecenter_full", "render_tiles_backward_tilecenter_full_with_feat",
+    "render_tiles_backward_tilecenter_full_with_feat",
     "render_tiles_mlp_records", "render_tiles_training_records_wmma",
     "render_tiles_backward_tilecenter_traversal",
     "render_tiles_backward_tilecenter_backprop_noatomic", "training_wmma_safety_stats",
@@ -374,6 +374,30 @@ class TileExt:
             lo, hi = torch.aminmax(ids)
             _chk(int(lo) >= 0 and int(hi) < n)
         return list(ops.records_reverse(ids, offsets, x6, raw, logs, quats, grgb, gt))
+
+    def render_tiles_backward_tilecenter_full(self, rays_o, rays_d, positions, log_scales, quats, cand, offsets,
+                                              freq, att, W1, b1, W2, b2, W3, b3, grad_rgb, grad_t, Wimg, Himg, TW, TH,
+                                              thr):
+        """[gW1, gb1, gW2, gb2, gW3, gb3, grad_positions, grad_log_scales, grad_quats] of the tile-centre-order
+        render for the image adjoint ``grad_rgb`` [B,3] and the adjoint ``grad_t`` [B] of the final transmittance
+        (np_tile_kernels.cu:2928-3530, wrapper :6765-6895).  The reference fuses everything into one kernel;
+        here the same quantities come from the record pipeline it is tested against (tests/test_primitive_csr.py:
+        44-50: equal within 5e-4): records forward -> reverse compositing -> grouped weight gradients in IEEE f32."""
+        from .primitive_csr import group_records, reference_weight_gradients
+        from . import primitive_gemm
+        _chk(int(TW) == int(TH), "square tiles only")
+        x = [rays_o, rays_d, positions, log_scales, quats, cand, offsets, freq, att, W1, b1, W2, b2, W3, b3,
+             grad_rgb.contiguous(), grad_t.contiguous()]
+        rgb, alpha, ids, x6, raw, masks, gates, pixel_offsets = self.render_tiles_training_records(
+            x, Wimg, Himg, TW, thr, 1.5, 2.0)
+        d4, gp, gs, gq = self.primitive_records_reverse(ids, pixel_offsets, x6, raw, log_scales, quats, x[15], x[16])
+        weights = [W1, b1, W2, b2, W3, b3]
+        csr = group_records(ids, x6, d4, positions.shape[0], masks)
+        if tuple(W1.shape[1:]) == (32, 72) and freq.numel() == 6:
+            grads = primitive_gemm.grouped_weight_gradients(csr, freq, att, weights, dtype=torch.float32)
+        else:   # other MLP shapes: the dense chain per primitive (small scenes and tests only)
+            grads = reference_weight_gradients(csr, freq, att, weights)
+        return [*grads, gp, gs, gq]
 
     # ------------------------------------------------------------------------------------------
     # statistics forward (pruning statistics are not rebuilt; the render itself is)

@@ -238,8 +238,9 @@ def test_inputs_are_not_mutated(tile_ext, device):
         assert torch.equal(v, before[k]), k
 
 
-def test_backward_entry_points_say_they_are_not_built(tile_ext):
+def test_backward_entry_points_that_are_not_built_say_so(tile_ext):
     with pytest.raises(NotImplementedError, match="training/backward"):
-        tile_ext.render_tiles_backward_tilecenter_full()
+        tile_ext.render_tiles_backward_tilecenter_full_with_feat()
+    assert callable(tile_ext.render_tiles_backward_tilecenter_full) and callable(tile_ext.primitive_records_reverse)
     with pytest.raises(AttributeError):
         tile_ext.no_such_entry_point

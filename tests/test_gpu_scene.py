@@ -267,11 +267,12 @@ def test_queued_frames_equal_step_by_step_frames(device, oracle_mod, monkeypatch
         view = to_dev(fr.view, device)
         kw = dict(score_threshold=fr.thr, proj_matrix=to_dev(fr.proj, device))
         ro, rd = to_dev(fr.rays_o, device), to_dev(fr.rays_d, device)
-        a = scene(ro, rd, view_matrix=view, **kw)
-        view[0, 3] += 0.5
-        b = scene(ro, rd, view_matrix=view, **kw)
-        scene.queued_frames = False
-        assert torch.equal(a, ref) and torch.equal(scene(ro, rd, view_matrix=view, **kw), b) and not torch.equal(a, b)
+        with torch.no_grad():      # (in grad mode a scene whose parameters require grad renders differentiably, in f32)
+            a = scene(ro, rd, view_matrix=view, **kw)
+            view[0, 3] += 0.5
+            b = scene(ro, rd, view_matrix=view, **kw)
+            scene.queued_frames = False
+            assert torch.equal(a, ref) and torch.equal(scene(ro, rd, view_matrix=view, **kw), b) and not torch.equal(a, b)
     # the capacity error comes out of the queued path too
     monkeypatch.setattr(cumodel, "_tile_ext", TileExt())
     scene = _scene_from(fr, device)

@@ -1,0 +1,120 @@
+"""The differentiable RGB render: scene(...) under autograd, backward through the record pipeline (records
+forward -> reverse compositing -> grouped weight gradients).
+
+What pins it: the record structure (which primitive hits which pixel, in which order, and the hit offsets) is
+taken from the forward records, everything else -- MLP from the weights, falloff from positions, log-scales and
+normalised quaternions, compositing, background -- is recomputed in float64 with torch autograd.  The
+gradients the reference defines flow through the MLP outputs and through the Gaussian falloff at a fixed hit
+offset (scannet/cuda/primitive_records.cuh:3-46); the restatement detaches exactly those inputs."""
+import numpy as np
+import pytest
+import torch
+
+from conftest import to_dev
+from helpers import Frame
+from test_gpu_scene import _scene_from
+
+pytestmark = pytest.mark.gpu
+
+PARAMS = ("positions", "log_scales", "quats", "W1", "b1", "W2", "b2", "W3", "b3")
+
+
+def _float64_gradients(scene, fr, device, weight_img, bg):
+    """d/dparams of  sum(weight_img * rgb)  with rgb recomposed from the frame's records in float64."""
+    ext = scene._ensure_tile_ext()
+    with torch.no_grad():
+        rd = torch.nn.functional.normalize(to_dev(fr.rays_d, device), dim=-1).contiguous()
+        cand, off = scene._tile_lists(to_dev(fr.rays_o, device), rd, fr.thr, to_dev(fr.view, device),
+                                      to_dev(fr.proj, device), None, None, device)
+        freq, att = scene._frequency_tables(device)
+        x = [to_dev(fr.rays_o, device), rd, scene.positions.detach().contiguous(), scene.log_scales.detach().contiguous(),
+             torch.nn.functional.normalize(scene.quats.detach(), dim=-1).contiguous(), cand, off.to(torch.int32), freq, att,
+             *[getattr(scene, k).detach().contiguous() for k in PARAMS[3:]]]
+        x += [torch.zeros_like(x[0]), torch.zeros(fr.W * fr.H, device=device)]
+        rgb, alpha, ids, x6, raw, masks, gates, offsets = ext.render_tiles_training_records(x, fr.W, fr.H, 8, fr.thr, 1.5, 2.0)
+    ids, x6, offsets = ids.cpu().long(), x6.cpu().double(), offsets.cpu()
+    leaves = {k: getattr(scene, k).detach().cpu().double().requires_grad_(True) for k in PARAMS}
+    freq, att = freq.cpu().double(), att.cpu().double()
+    phase = (x6[:, :, None] * freq * att).reshape(len(ids), 36)
+    enc = torch.cat([torch.sin(phase), torch.cos(phase)], 1)
+    h1 = torch.relu(torch.einsum("rhk,rk->rh", leaves["W1"][ids], enc) + leaves["b1"][ids])
+    h2 = torch.relu(torch.einsum("roh,rh->ro", leaves["W2"][ids], h1) + leaves["b2"][ids])
+    out = torch.einsum("roh,rh->ro", leaves["W3"][ids], h2) + leaves["b3"][ids]
+    colour, sigma_raw = torch.sigmoid(out[:, :3]), torch.nn.functional.softplus(out[:, 3])
+    q = torch.nn.functional.normalize(leaves["quats"], dim=-1)[ids]
+    w, qx, qy, qz = q.unbind(1)
+    rot = torch.stack([torch.stack([1 - 2 * (qy * qy + qz * qz), 2 * (qx * qy - w * qz), 2 * (qx * qz + w * qy)], 1),
+                       torch.stack([2 * (qx * qy + w * qz), 1 - 2 * (qx * qx + qz * qz), 2 * (qy * qz - w * qx)], 1),
+                       torch.stack([2 * (qx * qz - w * qy), 2 * (qy * qz + w * qx), 1 - 2 * (qx * qx + qy * qy)], 1)], 1)
+    pos = leaves["positions"][ids]
+    local = torch.einsum("rji,rj->ri", rot, x6[:, 3:6] + (pos - pos.detach()))
+    decay = torch.exp(-0.5 * (torch.exp(-2 * leaves["log_scales"][ids]) * local * local).sum(1))
+    a = 1 - torch.exp(-sigma_raw * decay)
+    wimg = weight_img.cpu().double()
+    loss = torch.zeros((), dtype=torch.float64)
+    for pix in range(fr.W * fr.H):
+        t = torch.ones((), dtype=torch.float64)
+        for r in range(int(offsets[pix]), int(offsets[pix + 1])):
+            loss = loss + (wimg[pix] * colour[r]).sum() * t * a[r]
+            t = t * (1 - a[r])
+        if bg is not None:
+            loss = loss + (wimg[pix] * bg.cpu().double()).sum() * t
+    loss.backward()
+    return {k: v.grad for k, v in leaves.items()}, int(len(ids)), rgb
+
+
+@pytest.mark.parametrize("with_bg", [False, True])
+def test_scene_gradients_match_float64_autograd_over_the_same_records(device, oracle_mod, with_bg):
+    fr = Frame("cfg1_5k_160x120", n=600, hidden=32, width=32, height=24)
+    scene = _scene_from(fr, device).train()
+    torch.manual_seed(0)
+    weight_img = torch.randn(fr.W * fr.H, 3, device=device)
+    bg = torch.tensor([0.2, 0.5, 0.9], device=device) if with_bg else None
+    rgb = scene(to_dev(fr.rays_o, device), to_dev(fr.rays_d, device), score_threshold=fr.thr, bg_color=bg,
+                view_matrix=to_dev(fr.view, device), proj_matrix=to_dev(fr.proj, device))
+    assert rgb.requires_grad
+    (rgb * weight_img).sum().backward()
+    want, num_records, rgb_records = _float64_gradients(scene, fr, device, weight_img, bg)
+    assert num_records > 1500
+    for k in PARAMS:
+        got = getattr(scene, k).grad
+        assert got is not None and got.shape == getattr(scene, k).shape, k
+        g, w = got.cpu().double(), want[k]
+        scale = float(w.abs().max())
+        assert scale > 1e-4, k
+        assert float((g - w).abs().max()) <= 2e-3 * scale, (k, float((g - w).abs().max()), scale)
+        assert float((g - w).norm() / w.norm()) < 1e-3, k
+
+
+def test_inference_calls_are_untouched_by_the_training_path(device, oracle_mod):
+    fr = Frame("cfg1_5k_160x120", n=300, hidden=32, width=32, height=24)
+    scene = _scene_from(fr, device)
+    args = (to_dev(fr.rays_o, device), to_dev(fr.rays_d, device))
+    kw = dict(score_threshold=fr.thr, view_matrix=to_dev(fr.view, device), proj_matrix=to_dev(fr.proj, device))
+    with torch.no_grad():
+        a = scene(*args, **kw)
+    b = scene(*args, **kw)                       # grad mode, parameters require grad: autograd path
+    assert not a.requires_grad and b.requires_grad and torch.equal(a, b.detach())
+    for p in scene.parameters():
+        p.requires_grad_(False)
+    c = scene(*args, **kw)
+    assert not c.requires_grad and torch.equal(a, c)
+
+
+def test_a_few_optimiser_steps_reduce_an_image_loss(device, oracle_mod):
+    fr = Frame("cfg1_5k_160x120", n=400, hidden=32, width=48, height=32)
+    scene = _scene_from(fr, device).train()
+    args = (to_dev(fr.rays_o, device), to_dev(fr.rays_d, device))
+    kw = dict(score_threshold=fr.thr, view_matrix=to_dev(fr.view, device), proj_matrix=to_dev(fr.proj, device))
+    with torch.no_grad():
+        target = (scene(*args, **kw) * 0.5 + 0.2).clamp(0, 1)
+    opt = torch.optim.Adam([{"params": [scene.W1, scene.b1, scene.W2, scene.b2, scene.W3, scene.b3], "lr": 5e-3},
+                            {"params": [scene.positions, scene.log_scales, scene.quats], "lr": 1e-3}])
+    losses = []
+    for _ in range(12):
+        opt.zero_grad(set_to_none=True)
+        loss = (scene(*args, **kw) - target).abs().mean()
+        loss.backward()
+        opt.step()
+        losses.append(float(loss.detach()))
+    assert all(np.isfinite(losses)) and losses[-1] < 0.7 * losses[0], losses
