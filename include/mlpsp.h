@@ -307,6 +307,23 @@ int mlpsp_records_reverse(const int32_t* ids_dev, const int64_t* pixel_offsets_d
                           float* d4_dev, float* grad_positions_dev, float* grad_log_scales_dev, float* grad_quats_dev,
                           mlpsp_stream_t stream);
 
+/* The same reverse walk without atomics, for callers that go on to a primitive-major ordering of the records
+ * anyway (the grouped weight gradients need one): writes d4 [R,4] as above and falloff_adjoint [R] =
+ * dL/d(decay) * decay per record; mlpsp_geometry_gradients then forms the geometry gradients.  No counterpart
+ * as a separate kernel in the reference (it is the first half of primitive_records_reverse_kernel). */
+int mlpsp_records_reverse_adjoints(const int32_t* ids_dev, const int64_t* pixel_offsets_dev, const float* raw_dev,
+                                   const float* grad_rgb_dev, const float* grad_t_dev, int64_t num_pixels,
+                                   float* d4_dev, float* falloff_adjoint_dev, mlpsp_stream_t stream);
+
+/* Second half of primitive_records_reverse_kernel (primitive_records.cuh:23-45) over records in primitive-major
+ * order: primitive p owns rows [csr_offsets[p], csr_offsets[p+1]) of x6_sorted [R,6]; record_indices [R] (int64)
+ * maps a row to its record, whose falloff_adjoint is read.  Writes (not accumulates) grad_positions [N,3],
+ * grad_log_scales [N,3], grad_quats [N,4]; one wavefront per primitive, no atomics, fixed summation order. */
+int mlpsp_geometry_gradients(const int64_t* csr_offsets_dev, const int64_t* record_indices_dev,
+                             const float* x6_sorted_dev, const float* falloff_adjoint_dev, const float* log_scales_dev,
+                             const float* quats_dev, int num_primitives, float* grad_positions_dev,
+                             float* grad_log_scales_dev, float* grad_quats_dev, mlpsp_stream_t stream);
+
 /* Measurement aid, no counterpart in the reference: launches a kernel that does nothing but
  * v_mfma_f32_32x32x16_bf16 on register operands (2,048 workgroups x 4 wavefronts x iterations x 8
  * instructions) and returns the FLOPs it issues (-1 on error); time it on the stream to see what the

@@ -13,11 +13,14 @@
 
 namespace mlpsp {
 
+// ATOMIC = false: no geometry sums; instead falloff_adjoint[r] = dL/d(decay) * decay is written per record and
+// geometry_gradients_kernel below forms the per-primitive sums from a primitive-major ordering of the records.
+template <bool ATOMIC>
 __global__ __launch_bounds__(128) void records_reverse_kernel(
     const int32_t* __restrict__ ids, const long long* __restrict__ offsets, const float* __restrict__ x6,
     const float* __restrict__ raw, const float* __restrict__ logs, const float* __restrict__ quats,
     const float* __restrict__ grgb, const float* __restrict__ gt, long long pixels, float* __restrict__ d4,
-    float* __restrict__ gp, float* __restrict__ gs, float* __restrict__ gq) {
+    float* __restrict__ gp, float* __restrict__ gs, float* __restrict__ gq, float* __restrict__ falloff_adjoint) {
   const long long pix = (long long)blockIdx.x * blockDim.x + threadIdx.x;
   if (pix >= pixels) return;
   float next = gt[pix];
@@ -39,6 +42,10 @@ __global__ __launch_bounds__(128) void records_reverse_kernel(
     d.z = g2 * (trans * alpha) * B * (1.f - B);
     d.w = grad_sigma * decay * sigmoid(vb.w);
     *reinterpret_cast<float4*>(d4 + r * 4) = d;
+    if constexpr (!ATOMIC) {
+      falloff_adjoint[r] = grad_decay * decay;
+      continue;
+    }
     const float dx = x6[r * 6 + 3], dy = x6[r * 6 + 4], dz = x6[r * 6 + 5];
     const float4 qv = *reinterpret_cast<const float4*>(quats + (size_t)p * 4);
     const float qw = qv.x, qx = qv.y, qy = qv.z, qz = qv.w;
@@ -68,6 +75,69 @@ __global__ __launch_bounds__(128) void records_reverse_kernel(
   }
 }
 
+// Geometry gradients from records in primitive-major order: one wavefront per primitive sums, over the
+// primitive's records i in [csr_offsets[p], csr_offsets[p+1]) (hit offset d_i = x6_sorted[i][3:6], falloff
+// adjoint a_i = falloff_adjoint[record_indices[i]]), the local-frame quantities
+//     g_i = -a_i m .* q_i,   q_i = R(q)^T d_i:      sum g,   sum a m q^2,   sum d (x) g
+// and applies the per-primitive linear maps once: grad_position = R sum g, grad_log_scale = sum a m q^2,
+// grad_quat = rotation-matrix chain rule of sum d (x) g (np_tile_kernels.cu:439-479).  Same terms as the atomic
+// variant adds record by record; no atomics, fixed summation order.
+__global__ __launch_bounds__(256) void geometry_gradients_kernel(
+    const long long* __restrict__ csr_offsets, const long long* __restrict__ record_indices,
+    const float* __restrict__ x6_sorted, const float* __restrict__ falloff_adjoint, const float* __restrict__ logs,
+    const float* __restrict__ quats, int N, float* __restrict__ gp, float* __restrict__ gs, float* __restrict__ gq) {
+  const int p = blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  if (p >= N) return;
+  const long long begin = csr_offsets[p], end = csr_offsets[p + 1];
+  const float qw = quats[p * 4], qx = quats[p * 4 + 1], qy = quats[p * 4 + 2], qz = quats[p * 4 + 3];
+  const float mx = det_exp(-2.f * logs[p * 3]), my = det_exp(-2.f * logs[p * 3 + 1]), mz = det_exp(-2.f * logs[p * 3 + 2]);
+  float sg[3] = {0.f, 0.f, 0.f}, ss[3] = {0.f, 0.f, 0.f}, so[9] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  for (long long i = begin + lane; i < end; i += 64) {
+    const float a = falloff_adjoint[record_indices[i]];
+    const float dx = x6_sorted[i * 6 + 3], dy = x6_sorted[i * 6 + 4], dz = x6_sorted[i * 6 + 5];
+    const Vec3 q = quat_rotate_conj(qw, qx, qy, qz, Vec3{dx, dy, dz});
+    const float gx = -a * mx * q.x, gy = -a * my * q.y, gz = -a * mz * q.z;
+    sg[0] += gx;
+    sg[1] += gy;
+    sg[2] += gz;
+    ss[0] += a * mx * q.x * q.x;
+    ss[1] += a * my * q.y * q.y;
+    ss[2] += a * mz * q.z * q.z;
+    so[0] += dx * gx; so[1] += dx * gy; so[2] += dx * gz;
+    so[3] += dy * gx; so[4] += dy * gy; so[5] += dy * gz;
+    so[6] += dz * gx; so[7] += dz * gy; so[8] += dz * gz;
+  }
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+#pragma unroll
+    for (int k = 0; k < 3; ++k) {
+      sg[k] += __shfl_xor(sg[k], d);
+      ss[k] += __shfl_xor(ss[k], d);
+    }
+#pragma unroll
+    for (int k = 0; k < 9; ++k) so[k] += __shfl_xor(so[k], d);
+  }
+  if (lane != 0) return;
+  const Vec3 gd = quat_rotate(qw, qx, qy, qz, Vec3{sg[0], sg[1], sg[2]});
+  gp[p * 3] = gd.x;
+  gp[p * 3 + 1] = gd.y;
+  gp[p * 3 + 2] = gd.z;
+  gs[p * 3] = ss[0];
+  gs[p * 3 + 1] = ss[1];
+  gs[p * 3 + 2] = ss[2];
+  const float r00 = so[0], r01 = so[1], r02 = so[2], r10 = so[3], r11 = so[4], r12 = so[5], r20 = so[6], r21 = so[7],
+              r22 = so[8];
+  gq[p * 4] = r01 * (-2.f * qz) + r02 * (2.f * qy) + r10 * (2.f * qz) + r12 * (-2.f * qx) + r20 * (-2.f * qy) +
+              r21 * (2.f * qx);
+  gq[p * 4 + 1] = r01 * (2.f * qy) + r02 * (2.f * qz) + r10 * (2.f * qy) + r11 * (-4.f * qx) + r12 * (-2.f * qw) +
+                  r20 * (2.f * qz) + r21 * (2.f * qw) + r22 * (-4.f * qx);
+  gq[p * 4 + 2] = r00 * (-4.f * qy) + r01 * (2.f * qx) + r02 * (2.f * qw) + r10 * (2.f * qx) + r12 * (2.f * qz) +
+                  r20 * (-2.f * qw) + r21 * (2.f * qz) + r22 * (-4.f * qy);
+  gq[p * 4 + 3] = r00 * (-4.f * qz) + r01 * (-2.f * qw) + r02 * (2.f * qx) + r10 * (2.f * qw) + r11 * (-4.f * qz) +
+                  r12 * (2.f * qy) + r20 * (2.f * qx) + r21 * (2.f * qy);
+}
+
 }  // namespace mlpsp
 
 using namespace mlpsp;
@@ -90,9 +160,44 @@ MLPSP_API int mlpsp_records_reverse(const int32_t* ids_dev, const int64_t* pixel
   // record arrays may be null only if there are no records (the offsets then end at zero)
   if (((uintptr_t)raw_dev | (uintptr_t)d4_dev | (uintptr_t)quats_dev) & 15u) return MLPSP_E_ARGUMENT;
   const dim3 grid((unsigned)((num_pixels + 127) / 128)), block(128);
-  hipLaunchKernelGGL(records_reverse_kernel, grid, block, 0, s, ids_dev, (const long long*)pixel_offsets_dev, x6_dev,
-                     raw_dev, log_scales_dev, quats_dev, grad_rgb_dev, grad_t_dev, (long long)num_pixels, d4_dev,
-                     grad_positions_dev, grad_log_scales_dev, grad_quats_dev);
+  hipLaunchKernelGGL(records_reverse_kernel<true>, grid, block, 0, s, ids_dev, (const long long*)pixel_offsets_dev,
+                     x6_dev, raw_dev, log_scales_dev, quats_dev, grad_rgb_dev, grad_t_dev, (long long)num_pixels, d4_dev,
+                     grad_positions_dev, grad_log_scales_dev, grad_quats_dev, (float*)nullptr);
+  MLPSP_LAUNCH_CHECK();
+  return MLPSP_OK;
+}
+
+MLPSP_API int mlpsp_records_reverse_adjoints(const int32_t* ids_dev, const int64_t* pixel_offsets_dev,
+                                             const float* raw_dev, const float* grad_rgb_dev, const float* grad_t_dev,
+                                             int64_t num_pixels, float* d4_dev, float* falloff_adjoint_dev,
+                                             mlpsp_stream_t stream) {
+  if (num_pixels < 0 || num_pixels > 2147483647LL * 128) return MLPSP_E_ARGUMENT;
+  if (num_pixels == 0) return MLPSP_OK;
+  if (!pixel_offsets_dev || !grad_rgb_dev || !grad_t_dev) return MLPSP_E_ARGUMENT;
+  if (((uintptr_t)raw_dev | (uintptr_t)d4_dev) & 15u) return MLPSP_E_ARGUMENT;
+  const dim3 grid((unsigned)((num_pixels + 127) / 128)), block(128);
+  hipLaunchKernelGGL(records_reverse_kernel<false>, grid, block, 0, (hipStream_t)stream, ids_dev,
+                     (const long long*)pixel_offsets_dev, (const float*)nullptr, raw_dev, (const float*)nullptr,
+                     (const float*)nullptr, grad_rgb_dev, grad_t_dev, (long long)num_pixels, d4_dev, (float*)nullptr,
+                     (float*)nullptr, (float*)nullptr, falloff_adjoint_dev);
+  MLPSP_LAUNCH_CHECK();
+  return MLPSP_OK;
+}
+
+MLPSP_API int mlpsp_geometry_gradients(const int64_t* csr_offsets_dev, const int64_t* record_indices_dev,
+                                       const float* x6_sorted_dev, const float* falloff_adjoint_dev,
+                                       const float* log_scales_dev, const float* quats_dev, int num_primitives,
+                                       float* grad_positions_dev, float* grad_log_scales_dev, float* grad_quats_dev,
+                                       mlpsp_stream_t stream) {
+  if (num_primitives < 0) return MLPSP_E_ARGUMENT;
+  if (num_primitives == 0) return MLPSP_OK;
+  if (!csr_offsets_dev || !log_scales_dev || !quats_dev || !grad_positions_dev || !grad_log_scales_dev ||
+      !grad_quats_dev)
+    return MLPSP_E_ARGUMENT;
+  hipLaunchKernelGGL(geometry_gradients_kernel, dim3((unsigned)((num_primitives + 3) / 4)), dim3(256), 0,
+                     (hipStream_t)stream, (const long long*)csr_offsets_dev, (const long long*)record_indices_dev,
+                     x6_sorted_dev, falloff_adjoint_dev, log_scales_dev, quats_dev, num_primitives, grad_positions_dev,
+                     grad_log_scales_dev, grad_quats_dev);
   MLPSP_LAUNCH_CHECK();
   return MLPSP_OK;
 }

@@ -426,3 +426,27 @@ def records_reverse(ids, offsets, x6, raw, log_scales, quats, grad_rgb, grad_t):
                                                  _ptr(quats), _ptr(grad_rgb), _ptr(grad_t), pixels, n, _ptr(d4), _ptr(gp),
                                                  _ptr(gs), _ptr(gq), _stream(dev)), "mlpsp_records_reverse")
     return d4, gp, gs, gq
+
+
+def records_reverse_adjoints(ids, offsets, raw, grad_rgb, grad_t):
+    """(d4 [R,4], falloff_adjoint [R]) of the reverse walk, without the atomic geometry sums."""
+    dev = ids.device
+    d4 = torch.empty((ids.numel(), 4), dtype=torch.float32, device=dev)
+    adj = torch.empty(ids.numel(), dtype=torch.float32, device=dev)
+    with torch.cuda.device(dev):
+        _check(_lib.load().mlpsp_records_reverse_adjoints(_ptr(ids), _ptr(offsets), _ptr(raw), _ptr(grad_rgb), _ptr(grad_t),
+                                                          grad_rgb.shape[0], _ptr(d4), _ptr(adj), _stream(dev)),
+               "mlpsp_records_reverse_adjoints")
+    return d4, adj
+
+
+def geometry_gradients(csr_offsets, record_indices, x6_sorted, falloff_adjoint, log_scales, quats):
+    """(grad_positions, grad_log_scales, grad_quats) from records in primitive-major order."""
+    dev = log_scales.device
+    gp, gs, gq = torch.zeros_like(log_scales), torch.zeros_like(log_scales), torch.zeros_like(quats)
+    with torch.cuda.device(dev):
+        _check(_lib.load().mlpsp_geometry_gradients(_ptr(csr_offsets), _ptr(record_indices), _ptr(x6_sorted),
+                                                    _ptr(falloff_adjoint), _ptr(log_scales), _ptr(quats),
+                                                    log_scales.shape[0], _ptr(gp), _ptr(gs), _ptr(gq), _stream(dev)),
+               "mlpsp_geometry_gradients")
+    return gp, gs, gq

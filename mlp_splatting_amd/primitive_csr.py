@@ -24,6 +24,15 @@ class PrimitiveCSR:
     relu_masks: Optional[torch.Tensor] = None
 
 
+def _gather_rows(t, perm):
+    """t[perm] for a 2-D tensor.  Rows of four float32 are gathered as one 16-byte element each: torch's row
+    gather takes 8 ms for 39 M such rows on an MI355X, the same bytes as single elements 0.9 ms."""
+    if t.dim() == 2 and t.shape[1] == 4 and t.dtype == torch.float32 and t.is_contiguous() and t.is_cuda and t.shape[0] > 0:
+        as_elements = torch.view_as_complex(t.view(torch.float64).view(t.shape[0], 1, 2)).reshape(t.shape[0])
+        return torch.view_as_real(as_elements[perm]).view(torch.float32).view(t.shape[0], 4)
+    return t[perm]
+
+
 def group_records(primitive_ids, x6, grad4, num_primitives: int, relu_masks=None) -> PrimitiveCSR:
     """Stable grouping by primitive id: inside a group the records keep their original (pixel) order
     (scannet/primitive_csr.py:23-29)."""
@@ -33,7 +42,8 @@ def group_records(primitive_ids, x6, grad4, num_primitives: int, relu_masks=None
     offsets = torch.zeros(per_primitive.numel() + 1, dtype=per_primitive.dtype, device=per_primitive.device)
     offsets[1:] = torch.cumsum(per_primitive, 0)
     masks = relu_masks[perm] if relu_masks is not None else None
-    return PrimitiveCSR(offsets=offsets, record_indices=perm, x6=x6[perm], grad4=grad4[perm], relu_masks=masks)
+    return PrimitiveCSR(offsets=offsets, record_indices=perm, x6=x6[perm], grad4=_gather_rows(grad4, perm),
+                        relu_masks=masks)
 
 
 @torch.no_grad()

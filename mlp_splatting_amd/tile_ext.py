@@ -390,9 +390,14 @@ class TileExt:
              grad_rgb.contiguous(), grad_t.contiguous()]
         rgb, alpha, ids, x6, raw, masks, gates, pixel_offsets = self.render_tiles_training_records(
             x, Wimg, Himg, TW, thr, 1.5, 2.0)
-        d4, gp, gs, gq = self.primitive_records_reverse(ids, pixel_offsets, x6, raw, log_scales, quats, x[15], x[16])
-        weights = [W1, b1, W2, b2, W3, b3]
-        csr = group_records(ids, x6, d4, positions.shape[0], masks)
+        # reverse walk without atomics; the geometry sums are formed from the primitive-major order that the
+        # weight gradients need anyway
+        with torch.cuda.device(ids.device):
+            d4, falloff_adjoint = ops.records_reverse_adjoints(ids, pixel_offsets, raw, x[15], x[16])
+            weights = [W1, b1, W2, b2, W3, b3]
+            csr = group_records(ids, x6, d4, positions.shape[0], masks)
+            gp, gs, gq = ops.geometry_gradients(csr.offsets, csr.record_indices, csr.x6, falloff_adjoint, log_scales,
+                                                quats)
         if tuple(W1.shape[1:]) == (32, 72) and freq.numel() == 6:
             grads = primitive_gemm.grouped_weight_gradients(csr, freq, att, weights, dtype=torch.float32)
         else:   # other MLP shapes: the dense chain per primitive (small scenes and tests only)

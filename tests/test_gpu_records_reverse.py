@@ -49,6 +49,15 @@ def test_reverse_on_records_of_a_rendered_frame(device, oracle_mod):
         _close(a, b, name)
     # d4 is written record by record, without atomics: same bits
     assert np.array_equal(got[0].cpu().numpy().view(np.uint32), want[0].view(np.uint32))
+    # the atomic-free split (adjoints per record, then one wavefront per primitive) gives the same gradients
+    from mlp_splatting_amd import ops
+    from mlp_splatting_amd.primitive_csr import group_records as _group
+    d4b, adjoint = ops.records_reverse_adjoints(ids, offsets, raw, grgb, gt)
+    assert torch.equal(d4b, got[0])
+    csr_b = _group(ids, x6, d4b, fr.scene.n, masks)
+    split = ops.geometry_gradients(csr_b.offsets, csr_b.record_indices, csr_b.x6, adjoint, x[3], x[4])
+    for name, a, b in zip(("grad_positions", "grad_log_scales", "grad_quats"), split, want[1:]):
+        _close(a, b, name + " (split)")
     # and it feeds the grouped weight gradients
     from mlp_splatting_amd import primitive_gemm as gemm
     from mlp_splatting_amd.primitive_csr import group_records
