@@ -324,6 +324,33 @@ int mlpsp_geometry_gradients(const int64_t* csr_offsets_dev, const int64_t* reco
                              const float* quats_dev, int num_primitives, float* grad_positions_dev,
                              float* grad_log_scales_dev, float* grad_quats_dev, mlpsp_stream_t stream);
 
+/* Streamed feature L1 loss over saved records = _stream_l1 (scannet/record_feature_loss.py:34-63, launched at
+ * :66-89): for every pixel of the low-resolution target [target_height, target_width, channels] (f32, or fp16 if
+ * target_is_half) the feature of its four bilinear source pixels is blended from their record lists
+ * (ids [R], pixel_offsets [width*height+1] int64, raw [R,8], gates [R,4], attributes [N, slots, channels] with
+ * slots 1, 4 or 5), combined with the weights of bilinear down-sampling (align_corners = false) and compared:
+ * signs [target pixels, channels] int8 = sign(prediction - target), loss_partials [target pixels,
+ * ceil(channels/128)] = per-block sums of |prediction - target| / (target pixels * channels), whose total is the
+ * L1 loss.  prediction_dev (same shape as the target, f32) may be NULL. */
+int mlpsp_stream_feature_l1(const int32_t* ids_dev, const int64_t* pixel_offsets_dev, const float* raw_dev,
+                            const float* gates_dev, const float* attributes_dev, const void* target_dev,
+                            int target_is_half, int width, int height, int target_width, int target_height,
+                            int channels, int slots, int8_t* signs_dev, float* loss_partials_dev,
+                            float* prediction_dev, mlpsp_stream_t stream);
+
+/* Gradient of that loss with respect to the attributes = _feature_vjp + _feature_reduce
+ * (scannet/record_feature_loss.py:114-185).  Records in primitive-major order: record_indices [R] (int64) maps a
+ * row of the CSR (csr_offsets [N+1]) to its record, record_pixels [R] (int32) gives a record's pixel; segments as
+ * for mlpsp_grouped_vjp.  mixed != 0 rounds both factors of every product to fp16 (f32 accumulation).
+ * partial_dev [num_groups, slots, channels] is scratch, out_dev [N, slots, channels] the result. */
+int mlpsp_feature_attribute_gradients(const int8_t* signs_dev, const int64_t* record_indices_dev,
+                                      const int32_t* record_pixels_dev, const float* raw_dev, const float* gates_dev,
+                                      const int64_t* csr_offsets_dev, const int64_t* group_primitives_dev,
+                                      const int64_t* group_starts_dev, const int64_t* group_offsets_dev,
+                                      int64_t num_groups, int num_primitives, int width, int height, int target_width,
+                                      int target_height, int channels, int slots, int segment, int mixed,
+                                      float* partial_dev, float* out_dev, mlpsp_stream_t stream);
+
 /* Measurement aid, no counterpart in the reference: launches a kernel that does nothing but
  * v_mfma_f32_32x32x16_bf16 on register operands (2,048 workgroups x 4 wavefronts x iterations x 8
  * instructions) and returns the FLOPs it issues (-1 on error); time it on the stream to see what the

@@ -1,0 +1,243 @@
+// libmlpsp_hip: streamed feature L1 loss over saved records and its gradient with respect to the feature
+// attributes (counterpart of the reference's Triton kernels _stream_l1, _feature_vjp and _feature_reduce,
+// scannet/record_feature_loss.py:12-162).  The high-resolution feature image is never materialised: every
+// low-resolution target pixel blends its (up to) four bilinear source pixels from their record lists, and only
+// the int8 sign of the residual and a scalar loss partial are kept.  Geometry, alpha and the MLP are constants
+// of this loss (:5).
+#include "mlpsp_device.hpp"
+#include "mlpsp_host.hpp"
+
+namespace mlpsp {
+
+// Feature of one high-resolution pixel and channel from its records: sum_r w_r * mix_r, w = T * alpha,
+// mix = base + sum_s gate_s * attr_s (1 slot: attr; 4 slots: gates only; 5 slots: slot 0 is the base)
+// (_blend_pixel, record_feature_loss.py:12-31; same fma chain).
+template <int SLOTS>
+__device__ __forceinline__ float blend_pixel(const int32_t* __restrict__ ids, const long long* __restrict__ offsets,
+                                             const float* __restrict__ raw, const float* __restrict__ gates,
+                                             const float* __restrict__ attr, long long pixel, int c, int C) {
+  float acc = 0.f;
+  const long long begin = offsets[pixel], end = offsets[pixel + 1];
+  for (long long r = begin; r < end; ++r) {
+    const long long p = ids[r];
+    const float w = raw[r * 8 + 4] * raw[r * 8 + 5];
+    float mix = (SLOTS == 1 || SLOTS == 5) ? attr[p * SLOTS * C + c] : 0.f;
+    if constexpr (SLOTS != 1) {
+#pragma unroll
+      for (int s = 0; s < 4; ++s)
+        mix = fmaf(gates[r * 4 + s], attr[(p * SLOTS + s + (SLOTS == 5 ? 1 : 0)) * C + c], mix);
+    }
+    acc = fmaf(w, mix, acc);
+  }
+  return acc;
+}
+
+// One workgroup = one target pixel x 128 channels (_stream_l1, :34-63).  T = float or _Float16 target.
+template <int SLOTS, typename T>
+__global__ __launch_bounds__(128) void stream_l1_kernel(const int32_t* __restrict__ ids,
+                                                        const long long* __restrict__ offsets,
+                                                        const float* __restrict__ raw, const float* __restrict__ gates,
+                                                        const float* __restrict__ attr, const T* __restrict__ target,
+                                                        int8_t* __restrict__ signs, float* __restrict__ loss,
+                                                        float* __restrict__ prediction, int W, int H, int WF, int HF,
+                                                        int C) {
+  __shared__ float s_part[2];
+  const int pix = blockIdx.x, chunk = blockIdx.y;
+  const int c = chunk * 128 + threadIdx.x;
+  const bool valid = c < C;
+  const int cc = valid ? c : 0;
+  const float sx = (float)W / (float)WF, sy = (float)H / (float)HF;
+  float xf = ((float)(pix % WF) + .5f) * sx - .5f;
+  float yf = ((float)(pix / WF) + .5f) * sy - .5f;
+  xf = fmaxf(xf, 0.f);
+  yf = fmaxf(yf, 0.f);
+  const int x0 = (int)xf, y0 = (int)yf;
+  const int x1 = min(x0 + 1, W - 1), y1 = min(y0 + 1, H - 1);
+  const float wx = xf - (float)x0, wy = yf - (float)y0;
+  const float a = blend_pixel<SLOTS>(ids, offsets, raw, gates, attr, (long long)y0 * W + x0, cc, C);
+  const float b = blend_pixel<SLOTS>(ids, offsets, raw, gates, attr, (long long)y0 * W + x1, cc, C);
+  const float cq = blend_pixel<SLOTS>(ids, offsets, raw, gates, attr, (long long)y1 * W + x0, cc, C);
+  const float d = blend_pixel<SLOTS>(ids, offsets, raw, gates, attr, (long long)y1 * W + x1, cc, C);
+  const float value = (1.f - wy) * ((1.f - wx) * a + wx * b) + wy * ((1.f - wx) * cq + wx * d);
+  const float gt = valid ? (float)target[(long long)pix * C + cc] : 0.f;
+  const float delta = value - gt;
+  if (valid) {
+    signs[(long long)pix * C + c] = (int8_t)((delta > 0.f) - (delta < 0.f));
+    if (prediction) prediction[(long long)pix * C + c] = value;
+  }
+  float part = valid ? __builtin_fabsf(delta) : 0.f;
+#pragma unroll
+  for (int sft = 1; sft < 64; sft <<= 1) part += __shfl_xor(part, sft);
+  if ((threadIdx.x & 63) == 0) s_part[threadIdx.x >> 6] = part;
+  __syncthreads();
+  if (threadIdx.x == 0)
+    loss[(long long)pix * gridDim.y + chunk] = (s_part[0] + s_part[1]) / (float)((long long)HF * WF * C);
+}
+
+// Adjoint of the bilinear down-sampling for one high-resolution pixel and channel: the (at most) 2 x 2 target
+// pixels whose footprint contains it, each weighted as in the forward pass (_resample_adjoint, :92-111).
+__device__ __forceinline__ float resample_adjoint(const int8_t* __restrict__ signs, int pix, int c, int W, int H, int WF,
+                                                  int HF, int C) {
+  const int xx = pix % W, yy = pix / W;
+  const float fx = (float)WF / (float)W, fy = (float)HF / (float)H, bx = (float)W / (float)WF, by = (float)H / (float)HF;
+  const int tx = (int)__builtin_floorf(((float)xx + .5f) * fx - .5f);
+  const int ty = (int)__builtin_floorf(((float)yy + .5f) * fy - .5f);
+  float grad = 0.f;
+#pragma unroll
+  for (int dy = 0; dy < 2; ++dy) {
+#pragma unroll
+    for (int dx = 0; dx < 2; ++dx) {
+      const int ix = tx + dx, iy = ty + dy;
+      const float srcx = fmaxf(((float)ix + .5f) * bx - .5f, 0.f);
+      const float srcy = fmaxf(((float)iy + .5f) * by - .5f, 0.f);
+      const float weight = fmaxf(0.f, 1.f - __builtin_fabsf(srcx - (float)xx)) *
+                           fmaxf(0.f, 1.f - __builtin_fabsf(srcy - (float)yy));
+      const bool inside = ix >= 0 && ix < WF && iy >= 0 && iy < HF;
+      const float s = inside ? (float)signs[((long long)iy * WF + ix) * C + c] : 0.f;
+      grad += weight * s;
+    }
+  }
+  return grad;
+}
+
+// One workgroup = one segment of a primitive's records x 64 channels; lane = channel.  accum[slot] +=
+// (T alpha gate_slot)[record] * adjoint[record's pixel, channel]; MIXED rounds both factors to fp16 first, as
+// the reference's mixed GEMM does, and keeps the f32 accumulation (_feature_vjp, :114-149).
+template <int SLOTS, bool MIXED>
+__global__ __launch_bounds__(64) void feature_vjp_kernel(const int8_t* __restrict__ signs,
+                                                         const long long* __restrict__ order,
+                                                         const int32_t* __restrict__ record_pixels,
+                                                         const float* __restrict__ raw, const float* __restrict__ gates,
+                                                         const long long* __restrict__ offsets,
+                                                         const long long* __restrict__ group_prim,
+                                                         const long long* __restrict__ group_start,
+                                                         float* __restrict__ partial, int W, int H, int WF, int HF, int C,
+                                                         int segment) {
+  const long long group = blockIdx.x;
+  const int c = blockIdx.y * 64 + threadIdx.x;
+  const bool valid = c < C;
+  const int cc = valid ? c : 0;
+  const long long p = group_prim[group];
+  const long long begin = group_start[group];
+  const long long seg_end = begin + segment, list_end = offsets[p + 1];
+  const long long end = seg_end < list_end ? seg_end : list_end;
+  float accum[SLOTS];
+#pragma unroll
+  for (int s = 0; s < SLOTS; ++s) accum[s] = 0.f;
+  for (long long row = begin; row < end; ++row) {
+    const long long r = order[row];
+    const int pix = record_pixels[r];
+    const float w = raw[r * 8 + 4] * raw[r * 8 + 5];
+    float bq = resample_adjoint(signs, pix, cc, W, H, WF, HF, C);
+    if constexpr (MIXED) bq = (float)(_Float16)bq;
+#pragma unroll
+    for (int s = 0; s < SLOTS; ++s) {
+      float g = 1.f;
+      if constexpr (SLOTS == 4) g = gates[r * 4 + s];
+      if constexpr (SLOTS == 5) g = (s == 0) ? 1.f : gates[r * 4 + s - 1];
+      float a = w * g;
+      if constexpr (MIXED) a = (float)(_Float16)a;
+      accum[s] += a * bq;
+    }
+  }
+  if (valid) {
+    const float norm = (float)((long long)WF * HF * C);
+#pragma unroll
+    for (int s = 0; s < SLOTS; ++s) partial[(group * SLOTS + s) * C + c] = accum[s] / norm;
+  }
+}
+
+// out[p][k] = sum over the primitive's segments (_feature_reduce, :152-161)
+__global__ __launch_bounds__(256) void feature_reduce_kernel(const float* __restrict__ partial,
+                                                             const long long* __restrict__ group_offsets,
+                                                             float* __restrict__ out, long long params) {
+  const long long p = blockIdx.x;
+  const long long k = (long long)blockIdx.y * 256 + threadIdx.x;
+  if (k >= params) return;
+  float acc = 0.f;
+  for (long long g = group_offsets[p]; g < group_offsets[p + 1]; ++g) acc += partial[g * params + k];
+  out[p * params + k] = acc;
+}
+
+}  // namespace mlpsp
+
+using namespace mlpsp;
+
+MLPSP_API int mlpsp_stream_feature_l1(const int32_t* ids_dev, const int64_t* pixel_offsets_dev, const float* raw_dev,
+                                      const float* gates_dev, const float* attributes_dev, const void* target_dev,
+                                      int target_is_half, int width, int height, int target_width, int target_height,
+                                      int channels, int slots, int8_t* signs_dev, float* loss_partials_dev,
+                                      float* prediction_dev, mlpsp_stream_t stream) {
+  if (width <= 0 || height <= 0 || target_width <= 0 || target_height <= 0 || channels <= 0) return MLPSP_E_ARGUMENT;
+  if (target_width > width || target_height > height) return MLPSP_E_ARGUMENT;
+  if (slots != 1 && slots != 4 && slots != 5) return MLPSP_E_ARGUMENT;
+  if ((int64_t)target_width * target_height > 2147483647LL) return MLPSP_E_ARGUMENT;
+  if (!pixel_offsets_dev || !attributes_dev || !target_dev || !signs_dev || !loss_partials_dev) return MLPSP_E_ARGUMENT;
+  const dim3 grid((unsigned)(target_width * target_height), (unsigned)((channels + 127) / 128)), block(128);
+  hipStream_t s = (hipStream_t)stream;
+#define MLPSP_L1_LAUNCH(SL, T)                                                                                     \
+  hipLaunchKernelGGL((stream_l1_kernel<SL, T>), grid, block, 0, s, ids_dev, (const long long*)pixel_offsets_dev,   \
+                     raw_dev, gates_dev, attributes_dev, (const T*)target_dev, signs_dev, loss_partials_dev,       \
+                     prediction_dev, width, height, target_width, target_height, channels)
+#define MLPSP_L1_SLOTS(T)                         \
+  do {                                            \
+    if (slots == 1) MLPSP_L1_LAUNCH(1, T);        \
+    else if (slots == 4) MLPSP_L1_LAUNCH(4, T);   \
+    else MLPSP_L1_LAUNCH(5, T);                   \
+  } while (0)
+  if (target_is_half) MLPSP_L1_SLOTS(_Float16);
+  else MLPSP_L1_SLOTS(float);
+#undef MLPSP_L1_SLOTS
+#undef MLPSP_L1_LAUNCH
+  MLPSP_LAUNCH_CHECK();
+  return MLPSP_OK;
+}
+
+MLPSP_API int mlpsp_feature_attribute_gradients(const int8_t* signs_dev, const int64_t* record_indices_dev,
+                                                const int32_t* record_pixels_dev, const float* raw_dev,
+                                                const float* gates_dev, const int64_t* csr_offsets_dev,
+                                                const int64_t* group_primitives_dev, const int64_t* group_starts_dev,
+                                                const int64_t* group_offsets_dev, int64_t num_groups,
+                                                int num_primitives, int width, int height, int target_width,
+                                                int target_height, int channels, int slots, int segment, int mixed,
+                                                float* partial_dev, float* out_dev, mlpsp_stream_t stream) {
+  if (width <= 0 || height <= 0 || target_width <= 0 || target_height <= 0 || channels <= 0 || segment <= 0)
+    return MLPSP_E_ARGUMENT;
+  if (target_width > width || target_height > height || num_groups < 0 || num_groups > 2147483647LL ||
+      num_primitives < 0)
+    return MLPSP_E_ARGUMENT;
+  if (slots != 1 && slots != 4 && slots != 5) return MLPSP_E_ARGUMENT;
+  hipStream_t s = (hipStream_t)stream;
+  if (num_groups > 0) {
+    if (!signs_dev || !record_indices_dev || !record_pixels_dev || !raw_dev || !csr_offsets_dev ||
+        !group_primitives_dev || !group_starts_dev || !partial_dev)
+      return MLPSP_E_ARGUMENT;
+    const dim3 grid((unsigned)num_groups, (unsigned)((channels + 63) / 64)), block(64);
+#define MLPSP_FV_LAUNCH(SL, MX)                                                                                    \
+  hipLaunchKernelGGL((feature_vjp_kernel<SL, MX>), grid, block, 0, s, signs_dev,                                   \
+                     (const long long*)record_indices_dev, record_pixels_dev, raw_dev, gates_dev,                  \
+                     (const long long*)csr_offsets_dev, (const long long*)group_primitives_dev,                    \
+                     (const long long*)group_starts_dev, partial_dev, width, height, target_width, target_height,  \
+                     channels, segment)
+#define MLPSP_FV_SLOTS(MX)                         \
+  do {                                             \
+    if (slots == 1) MLPSP_FV_LAUNCH(1, MX);        \
+    else if (slots == 4) MLPSP_FV_LAUNCH(4, MX);   \
+    else MLPSP_FV_LAUNCH(5, MX);                   \
+  } while (0)
+    if (mixed) MLPSP_FV_SLOTS(true);
+    else MLPSP_FV_SLOTS(false);
+#undef MLPSP_FV_SLOTS
+#undef MLPSP_FV_LAUNCH
+    MLPSP_LAUNCH_CHECK();
+  }
+  if (num_primitives > 0) {
+    if (!group_offsets_dev || !out_dev) return MLPSP_E_ARGUMENT;
+    const long long params = (long long)slots * channels;
+    const dim3 grid((unsigned)num_primitives, (unsigned)((params + 255) / 256)), block(256);
+    hipLaunchKernelGGL(feature_reduce_kernel, grid, block, 0, s, partial_dev, (const long long*)group_offsets_dev,
+                       out_dev, params);
+    MLPSP_LAUNCH_CHECK();
+  }
+  return MLPSP_OK;
+}

@@ -485,6 +485,9 @@ class NeuralPrimitiveSceneTileCUDA(nn.Module):
         assert ray_o.shape[0] == W * H, "Tile renderer requires full-frame rays (B == W*H)"
         device = self._activate_cuda_device()
         ts = int(self.tile_size)
+        if feature_target is not None:
+            return self._forward_csr_training(ray_o, ray_d, score_threshold, bg_color, view_matrix, proj_matrix,
+                                              culled_prim_indices, tile_offsets, return_feature, feature_target, device)
         if (torch.is_grad_enabled() and feature_target is None and not (return_feature and self.feat_attr is not None)
                 and any(t.requires_grad for t in (self.positions, self.log_scales, self.quats, self.W1, self.b1,
                                                   self.W2, self.b2, self.W3, self.b3))):
@@ -509,10 +512,6 @@ class NeuralPrimitiveSceneTileCUDA(nn.Module):
                 ray_o, ray_d, score_threshold, view_matrix, proj_matrix, culled_prim_indices, tile_offsets, device)
             if own_lists and hasattr(ext, "note_frame_pairs"):
                 ext.note_frame_pairs(int(culled_prim_indices.numel()))
-            if feature_target is not None:
-                if not return_feature or self.feat_attr is None or not use_tilecenter or ts != 8:
-                    raise ValueError("CSR feature training requires tilecenter8 and direct feature attributes")
-                raise NotImplementedError("record-based feature training is not part of the forward renderer")
             base = self._base_args(ray_o, ray_d, culled_prim_indices, tile_offsets, device, unit_dirs)
             bg = self._background(bg_color, ray_o)
             dims = (int(W), int(H), ts, ts, float(score_threshold))
@@ -543,6 +542,29 @@ class NeuralPrimitiveSceneTileCUDA(nn.Module):
             else:
                 rgb, alpha, feat = ext.render_tiles_forward_per_pixel_with_feat(*base, *feat_args, *dims)
             return _add_background(rgb, alpha, bg), feat
+
+    def _forward_csr_training(self, ray_o, ray_d, score_threshold, bg_color, view_matrix, proj_matrix,
+                              culled_prim_indices, tile_offsets, return_feature, feature_target, device):
+        """(rgb, streamed feature L1 loss) through the record-based training function
+        (scannet/cumodel.py:1098-1108)."""
+        W, H = self.image_size
+        ts = int(self.tile_size)
+        use_tilecenter = self._resolve_tile_order_mode() == "tilecenter"
+        if not return_feature or self.feat_attr is None or not use_tilecenter or ts != 8:
+            raise ValueError("CSR feature training requires tilecenter8 and direct feature attributes")
+        from .csr_training import render_training_csr
+        with torch.no_grad():
+            unit_dirs = F.normalize(ray_d, dim=-1).contiguous()
+            culled_prim_indices, tile_offsets = self._tile_lists(
+                ray_o, ray_d, score_threshold, view_matrix, proj_matrix, culled_prim_indices, tile_offsets, device)
+            freq, att = self._frequency_tables(device)
+        base = [ray_o.contiguous(), unit_dirs, self.positions.contiguous(), self.log_scales.contiguous(),
+                F.normalize(self.quats, dim=-1).contiguous(), culled_prim_indices, tile_offsets.to(torch.int32), freq, att,
+                self.W1.contiguous(), self.b1.contiguous(), self.W2.contiguous(), self.b2.contiguous(),
+                self.W3.contiguous(), self.b3.contiguous()]
+        return render_training_csr(base, self.feat_attr.contiguous(), feature_target, int(W), int(H),
+                                   float(score_threshold), float(self.feature_gating_beta),
+                                   float(self.feature_gating_temp), self._background(bg_color, ray_o))
 
     def _forward_differentiable(self, ray_o, ray_d, score_threshold, bg_color, view_matrix, proj_matrix,
                                 culled_prim_indices, tile_offsets, return_feature, device):

@@ -1,0 +1,78 @@
+"""Streamed feature L1 loss from saved splat records, with the API of the reference's
+``scannet/record_feature_loss.py`` (``streaming_feature_l1``, ``feature_weight_gradients``).
+
+The exact high-resolution feature blend is sampled with the bilinear down-sampling operator
+(``F.interpolate(..., mode="bilinear", align_corners=False)``) without ever materialising the 512-D image; only
+int8 signs of the residual and scalar loss partials are kept.  Geometry, alpha and the MLP are constants of this
+loss (scannet/record_feature_loss.py:1-6).  The kernels are libmlpsp_hip's ``mlpsp_stream_feature_l1`` and
+``mlpsp_feature_attribute_gradients``.
+"""
+from __future__ import annotations
+
+import torch
+
+from . import _lib
+
+
+def _ptr(t):
+    return None if t is None else t.data_ptr()
+
+
+def streaming_feature_l1(records, attributes, target, width, height, *, debug=False):
+    """(loss, signs int8 [hf, wf, C], prediction or None) -- scannet/record_feature_loss.py:66-89."""
+    _, _, ids, x6, raw, masks, gates, offsets = records
+    if target.ndim != 3 or min(target.shape) <= 0:
+        raise ValueError("feature target must have nonempty HWC dimensions")
+    if attributes.dtype != torch.float32 or not attributes.is_contiguous():
+        raise ValueError("feature master attributes must be contiguous FP32")
+    if target.dtype not in (torch.float16, torch.float32):
+        raise ValueError("feature target must be FP16 or FP32")
+    if any(not t.is_cuda or t.device != attributes.device for t in (ids, offsets, raw, gates, attributes, target)):
+        raise ValueError("feature tensors and records must share a CUDA device")
+    hf, wf, channels = target.shape
+    slots = 1 if attributes.ndim == 2 else attributes.shape[1]
+    if slots not in (1, 4, 5) or attributes.shape[-1] != channels:
+        raise ValueError("feature shape does not match the 1/4/5-slot renderer")
+    if hf > height or wf > width:
+        raise ValueError("streamed feature loss supports downsampling only")
+    target = target.contiguous()
+    device = target.device
+    signs = torch.empty(target.shape, device=device, dtype=torch.int8)
+    partial = torch.empty((hf * wf, (channels + 127) // 128), device=device, dtype=torch.float32)
+    pred = torch.empty(target.shape, device=device, dtype=torch.float32) if debug else None
+    with torch.cuda.device(device):
+        rc = _lib.load().mlpsp_stream_feature_l1(
+            _ptr(ids), _ptr(offsets), _ptr(raw), _ptr(gates), _ptr(attributes), _ptr(target),
+            int(target.dtype == torch.float16), int(width), int(height), int(wf), int(hf), int(channels), int(slots),
+            _ptr(signs), _ptr(partial), _ptr(pred), torch.cuda.current_stream(device).cuda_stream)
+    if rc != 0:
+        raise RuntimeError(f"mlpsp_stream_feature_l1: {_lib.strerror(rc)}")
+    return partial.sum(), signs, pred
+
+
+def feature_weight_gradients(records, csr, signs, attributes, width, height, *, mixed=True, segment_size=512,
+                             groups=None):
+    """d loss / d attributes, shaped like ``attributes`` -- scannet/record_feature_loss.py:164-185."""
+    from .primitive_gemm import resolve_groups
+    _, _, ids, x6, raw, masks, gates, pixel_offsets = records
+    hf, wf, channels = signs.shape
+    if signs.dtype != torch.int8 or not signs.is_contiguous():
+        raise ValueError("feature loss signs must be contiguous int8")
+    slots = 1 if attributes.ndim == 2 else attributes.shape[1]
+    if hf > height or wf > width:
+        raise ValueError("streamed feature loss supports downsampling only")
+    primitives, starts, group_offsets = resolve_groups(csr, segment_size, groups)
+    device = ids.device
+    pixels = torch.repeat_interleave(torch.arange(width * height, device=device, dtype=torch.int32),
+                                     pixel_offsets.diff(), output_size=len(ids))
+    partial = torch.empty((max(len(primitives), 1), slots, channels), device=device, dtype=torch.float32)
+    result = torch.empty_like(attributes)
+    with torch.cuda.device(device):
+        rc = _lib.load().mlpsp_feature_attribute_gradients(
+            _ptr(signs), _ptr(csr.record_indices), _ptr(pixels), _ptr(raw), _ptr(gates), _ptr(csr.offsets),
+            _ptr(primitives), _ptr(starts), _ptr(group_offsets), int(len(primitives)), int(len(attributes)), int(width),
+            int(height), int(wf), int(hf), int(channels), int(slots), int(segment_size), int(bool(mixed)),
+            _ptr(partial), _ptr(result), torch.cuda.current_stream(device).cuda_stream)
+    if rc != 0:
+        raise RuntimeError(f"mlpsp_feature_attribute_gradients: {_lib.strerror(rc)}")
+    return result
