@@ -27,6 +27,48 @@ HBM_PEAK_GBS = 8000.0
 MEASURED_TRAFFIC_BYTES = {("cfg3_200k_1200x680", "bf16"): int((121920.7 * 2.0 + 54889.0) * 1024)}
 
 
+def train_steps(args, scene, frames, proj, thr, W, H, sc, dev):
+    """One training step = scene(...) under autograd -> L1 loss against a fixed image -> backward (records
+    forward, reverse compositing, grouped weight gradients in IEEE f32) -> Adam step on every parameter."""
+    import torch
+    scene.train()
+    scene.render_precision = "f32"
+    params = [scene.positions, scene.log_scales, scene.quats, scene.W1, scene.b1, scene.W2, scene.b2, scene.W3, scene.b3]
+    opt = torch.optim.Adam(params, lr=1e-4, fused=True)
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(1)
+    target = torch.rand(W * H, 3, device=dev, generator=gen)
+
+    def step(i):
+        ro, rd, views, _ = frames[i % len(frames)]
+        opt.zero_grad(set_to_none=True)
+        rgb = scene(ro, rd, score_threshold=thr, view_matrix=views[0], proj_matrix=proj)
+        loss = (rgb - target).abs().mean()
+        loss.backward()
+        opt.step()
+        return loss
+
+    steps, warmup = min(args.steps, 24), min(args.warmup, 4)
+    for i in range(warmup):
+        step(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        loss = step(i)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    print(json.dumps({
+        "metric": "training_steps_per_sec_1200x680_200k_primitives", "value": round(steps / elapsed, 3),
+        "unit": "steps/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
+        "ms_per_step": round(1000.0 * elapsed / steps, 3), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": args.workload, "primitives": sc.n, "width": W, "height": H, "tile": 8, "threshold": thr,
+                   "poses": len(frames), "loss": "L1 against a fixed random image", "optimizer": "Adam (fused), all 9 tensors",
+                   "entry": "NeuralPrimitiveSceneTileCUDA.forward + backward"},
+        "final_loss": round(float(loss.detach()), 6)}))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -36,6 +78,9 @@ def main() -> int:
     ap.add_argument("--precision", choices=["f32", "bf16"], default=None,
                     help="MLP arithmetic of the render kernel (default: bf16 matrix cores when built, else f32)")
     ap.add_argument("--poses", type=int, default=32)
+    ap.add_argument("--train", action="store_true",
+                    help="time full training steps instead (f32 render with autograd, L1 image loss, backward through "
+                         "the record pipeline, Adam on all nine parameter tensors); prints its own JSON line")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run 4 plain device copies of 1 GiB, the known-size kernel that hardware counter "
@@ -91,6 +136,9 @@ def main() -> int:
         for c2w in poses:
             ro, rd = syn.pinhole_rays(W, H, f, c2w)
             frames.append((t(ro), t(rd), t(syn.view_matrix(c2w))[None], None))
+
+    if args.train:
+        return train_steps(args, scene, frames, proj, thr, W, H, sc, dev)
 
     def render(i):
         ro, rd, views, tv = frames[i % len(frames)]

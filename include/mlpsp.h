@@ -317,11 +317,15 @@ int mlpsp_records_reverse_adjoints(const int32_t* ids_dev, const int64_t* pixel_
 
 /* Second half of primitive_records_reverse_kernel (primitive_records.cuh:23-45) over records in primitive-major
  * order: primitive p owns rows [csr_offsets[p], csr_offsets[p+1]) of x6_sorted [R,6]; record_indices [R] (int64)
- * maps a row to its record, whose falloff_adjoint is read.  Writes (not accumulates) grad_positions [N,3],
- * grad_log_scales [N,3], grad_quats [N,4]; one wavefront per primitive, no atomics, fixed summation order. */
+ * maps a row to its record, whose falloff_adjoint is read.  The rows are walked in the segments of
+ * mlpsp_grouped_vjp (group_primitives / group_starts [num_groups], group_offsets [N+1], segment), one wavefront
+ * per segment into partial_dev [num_groups, 16] (scratch), then summed per primitive.  Writes (not accumulates)
+ * grad_positions [N,3], grad_log_scales [N,3], grad_quats [N,4]; no atomics, fixed summation order. */
 int mlpsp_geometry_gradients(const int64_t* csr_offsets_dev, const int64_t* record_indices_dev,
                              const float* x6_sorted_dev, const float* falloff_adjoint_dev, const float* log_scales_dev,
-                             const float* quats_dev, int num_primitives, float* grad_positions_dev,
+                             const float* quats_dev, const int64_t* group_primitives_dev,
+                             const int64_t* group_starts_dev, const int64_t* group_offsets_dev, int64_t num_groups,
+                             int segment, int num_primitives, float* partial_dev, float* grad_positions_dev,
                              float* grad_log_scales_dev, float* grad_quats_dev, mlpsp_stream_t stream);
 
 /* Streamed feature L1 loss over saved records = _stream_l1 (scannet/record_feature_loss.py:34-63, launched at

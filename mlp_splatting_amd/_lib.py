@@ -66,7 +66,8 @@ SIGNATURES = {
     "mlpsp_feature_attribute_gradients": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i, _i, _i, _i, _i, _i,
                                                _i, _i, _i, _vp, _vp, _vp]),
     "mlpsp_records_reverse_adjoints": (_i, [_vp, _vp, _vp, _vp, _vp, _i64, _vp, _vp, _vp]),
-    "mlpsp_geometry_gradients": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _vp, _vp]),
+    "mlpsp_geometry_gradients": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i, _i, _vp, _vp, _vp, _vp,
+                                      _vp]),
     "mlpsp_records_reverse": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i, _vp, _vp, _vp, _vp, _vp]),
 }
 

@@ -75,59 +75,84 @@ __global__ __launch_bounds__(128) void records_reverse_kernel(
   }
 }
 
-// Geometry gradients from records in primitive-major order: one wavefront per primitive sums, over the
-// primitive's records i in [csr_offsets[p], csr_offsets[p+1]) (hit offset d_i = x6_sorted[i][3:6], falloff
-// adjoint a_i = falloff_adjoint[record_indices[i]]), the local-frame quantities
-//     g_i = -a_i m .* q_i,   q_i = R(q)^T d_i:      sum g,   sum a m q^2,   sum d (x) g
-// and applies the per-primitive linear maps once: grad_position = R sum g, grad_log_scale = sum a m q^2,
-// grad_quat = rotation-matrix chain rule of sum d (x) g (np_tile_kernels.cu:439-479).  Same terms as the atomic
-// variant adds record by record; no atomics, fixed summation order.
-__global__ __launch_bounds__(256) void geometry_gradients_kernel(
+// Geometry gradients from records in primitive-major order, in two steps.  Step 1, one wavefront per segment
+// (at most `segment` consecutive records of one primitive, the segments of the grouped weight gradients): over
+// the segment's rows i (hit offset d_i = x6_sorted[i][3:6], falloff adjoint a_i = falloff_adjoint[record_indices[i]])
+// the local-frame sums
+//     sum g,   sum a m q^2,   sum d (x) g        with  q_i = R(q)^T d_i,  g_i = -a_i m .* q_i
+// go to partial[segment][15].  Step 2, one thread per primitive, adds its segments and applies the per-primitive
+// linear maps once: grad_position = R sum g, grad_log_scale = sum a m q^2, grad_quat = rotation-matrix chain rule
+// of sum d (x) g (np_tile_kernels.cu:439-479).  Same terms as the atomic variant adds record by record; no
+// atomics, fixed summation order, and a primitive with very many records is spread over many wavefronts.
+__global__ __launch_bounds__(256) void geometry_partials_kernel(
     const long long* __restrict__ csr_offsets, const long long* __restrict__ record_indices,
     const float* __restrict__ x6_sorted, const float* __restrict__ falloff_adjoint, const float* __restrict__ logs,
-    const float* __restrict__ quats, int N, float* __restrict__ gp, float* __restrict__ gs, float* __restrict__ gq) {
-  const int p = blockIdx.x * 4 + (threadIdx.x >> 6);
+    const float* __restrict__ quats, const long long* __restrict__ group_prim,
+    const long long* __restrict__ group_start, long long num_groups, int segment, float* __restrict__ partial) {
+  const long long group = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
   const int lane = threadIdx.x & 63;
-  if (p >= N) return;
-  const long long begin = csr_offsets[p], end = csr_offsets[p + 1];
+  if (group >= num_groups) return;
+  const long long p = group_prim[group];
+  const long long begin = group_start[group];
+  const long long seg_end = begin + segment, list_end = csr_offsets[p + 1];
+  const long long end = seg_end < list_end ? seg_end : list_end;
   const float qw = quats[p * 4], qx = quats[p * 4 + 1], qy = quats[p * 4 + 2], qz = quats[p * 4 + 3];
   const float mx = det_exp(-2.f * logs[p * 3]), my = det_exp(-2.f * logs[p * 3 + 1]), mz = det_exp(-2.f * logs[p * 3 + 2]);
-  float sg[3] = {0.f, 0.f, 0.f}, ss[3] = {0.f, 0.f, 0.f}, so[9] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  float v[15];
+#pragma unroll
+  for (int k = 0; k < 15; ++k) v[k] = 0.f;
   for (long long i = begin + lane; i < end; i += 64) {
     const float a = falloff_adjoint[record_indices[i]];
     const float dx = x6_sorted[i * 6 + 3], dy = x6_sorted[i * 6 + 4], dz = x6_sorted[i * 6 + 5];
     const Vec3 q = quat_rotate_conj(qw, qx, qy, qz, Vec3{dx, dy, dz});
     const float gx = -a * mx * q.x, gy = -a * my * q.y, gz = -a * mz * q.z;
-    sg[0] += gx;
-    sg[1] += gy;
-    sg[2] += gz;
-    ss[0] += a * mx * q.x * q.x;
-    ss[1] += a * my * q.y * q.y;
-    ss[2] += a * mz * q.z * q.z;
-    so[0] += dx * gx; so[1] += dx * gy; so[2] += dx * gz;
-    so[3] += dy * gx; so[4] += dy * gy; so[5] += dy * gz;
-    so[6] += dz * gx; so[7] += dz * gy; so[8] += dz * gz;
+    v[0] += gx;
+    v[1] += gy;
+    v[2] += gz;
+    v[3] += a * mx * q.x * q.x;
+    v[4] += a * my * q.y * q.y;
+    v[5] += a * mz * q.z * q.z;
+    v[6] += dx * gx; v[7] += dx * gy; v[8] += dx * gz;
+    v[9] += dy * gx; v[10] += dy * gy; v[11] += dy * gz;
+    v[12] += dz * gx; v[13] += dz * gy; v[14] += dz * gz;
   }
 #pragma unroll
   for (int d = 1; d < 64; d <<= 1) {
 #pragma unroll
-    for (int k = 0; k < 3; ++k) {
-      sg[k] += __shfl_xor(sg[k], d);
-      ss[k] += __shfl_xor(ss[k], d);
-    }
-#pragma unroll
-    for (int k = 0; k < 9; ++k) so[k] += __shfl_xor(so[k], d);
+    for (int k = 0; k < 15; ++k) v[k] += __shfl_xor(v[k], d);
   }
-  if (lane != 0) return;
-  const Vec3 gd = quat_rotate(qw, qx, qy, qz, Vec3{sg[0], sg[1], sg[2]});
+  if (lane < 15) {
+    float mine = v[0];
+#pragma unroll
+    for (int k = 1; k < 15; ++k) mine = (lane == k) ? v[k] : mine;
+    partial[group * 16 + lane] = mine;
+  }
+}
+
+__global__ __launch_bounds__(256) void geometry_finish_kernel(const float* __restrict__ partial,
+                                                              const long long* __restrict__ group_offsets,
+                                                              const float* __restrict__ quats, int N,
+                                                              float* __restrict__ gp, float* __restrict__ gs,
+                                                              float* __restrict__ gq) {
+  const int p = blockIdx.x * blockDim.x + threadIdx.x;
+  if (p >= N) return;
+  float v[15];
+#pragma unroll
+  for (int k = 0; k < 15; ++k) v[k] = 0.f;
+  for (long long g = group_offsets[p]; g < group_offsets[p + 1]; ++g) {
+#pragma unroll
+    for (int k = 0; k < 15; ++k) v[k] += partial[g * 16 + k];
+  }
+  const float qw = quats[p * 4], qx = quats[p * 4 + 1], qy = quats[p * 4 + 2], qz = quats[p * 4 + 3];
+  const Vec3 gd = quat_rotate(qw, qx, qy, qz, Vec3{v[0], v[1], v[2]});
   gp[p * 3] = gd.x;
   gp[p * 3 + 1] = gd.y;
   gp[p * 3 + 2] = gd.z;
-  gs[p * 3] = ss[0];
-  gs[p * 3 + 1] = ss[1];
-  gs[p * 3 + 2] = ss[2];
-  const float r00 = so[0], r01 = so[1], r02 = so[2], r10 = so[3], r11 = so[4], r12 = so[5], r20 = so[6], r21 = so[7],
-              r22 = so[8];
+  gs[p * 3] = v[3];
+  gs[p * 3 + 1] = v[4];
+  gs[p * 3 + 2] = v[5];
+  const float r00 = v[6], r01 = v[7], r02 = v[8], r10 = v[9], r11 = v[10], r12 = v[11], r20 = v[12], r21 = v[13],
+              r22 = v[14];
   gq[p * 4] = r01 * (-2.f * qz) + r02 * (2.f * qy) + r10 * (2.f * qz) + r12 * (-2.f * qx) + r20 * (-2.f * qy) +
               r21 * (2.f * qx);
   gq[p * 4 + 1] = r01 * (2.f * qy) + r02 * (2.f * qz) + r10 * (2.f * qy) + r11 * (-4.f * qx) + r12 * (-2.f * qw) +
@@ -186,17 +211,29 @@ MLPSP_API int mlpsp_records_reverse_adjoints(const int32_t* ids_dev, const int64
 
 MLPSP_API int mlpsp_geometry_gradients(const int64_t* csr_offsets_dev, const int64_t* record_indices_dev,
                                        const float* x6_sorted_dev, const float* falloff_adjoint_dev,
-                                       const float* log_scales_dev, const float* quats_dev, int num_primitives,
-                                       float* grad_positions_dev, float* grad_log_scales_dev, float* grad_quats_dev,
-                                       mlpsp_stream_t stream) {
-  if (num_primitives < 0) return MLPSP_E_ARGUMENT;
+                                       const float* log_scales_dev, const float* quats_dev,
+                                       const int64_t* group_primitives_dev, const int64_t* group_starts_dev,
+                                       const int64_t* group_offsets_dev, int64_t num_groups, int segment,
+                                       int num_primitives, float* partial_dev, float* grad_positions_dev,
+                                       float* grad_log_scales_dev, float* grad_quats_dev, mlpsp_stream_t stream) {
+  if (num_primitives < 0 || num_groups < 0 || num_groups > 2147483647LL * 4 || segment <= 0) return MLPSP_E_ARGUMENT;
   if (num_primitives == 0) return MLPSP_OK;
-  if (!csr_offsets_dev || !log_scales_dev || !quats_dev || !grad_positions_dev || !grad_log_scales_dev ||
-      !grad_quats_dev)
+  if (!csr_offsets_dev || !log_scales_dev || !quats_dev || !group_offsets_dev || !grad_positions_dev ||
+      !grad_log_scales_dev || !grad_quats_dev)
     return MLPSP_E_ARGUMENT;
-  hipLaunchKernelGGL(geometry_gradients_kernel, dim3((unsigned)((num_primitives + 3) / 4)), dim3(256), 0,
-                     (hipStream_t)stream, (const long long*)csr_offsets_dev, (const long long*)record_indices_dev,
-                     x6_sorted_dev, falloff_adjoint_dev, log_scales_dev, quats_dev, num_primitives, grad_positions_dev,
+  hipStream_t s = (hipStream_t)stream;
+  if (num_groups > 0) {
+    if (!record_indices_dev || !x6_sorted_dev || !falloff_adjoint_dev || !group_primitives_dev || !group_starts_dev ||
+        !partial_dev)
+      return MLPSP_E_ARGUMENT;
+    hipLaunchKernelGGL(geometry_partials_kernel, dim3((unsigned)((num_groups + 3) / 4)), dim3(256), 0, s,
+                       (const long long*)csr_offsets_dev, (const long long*)record_indices_dev, x6_sorted_dev,
+                       falloff_adjoint_dev, log_scales_dev, quats_dev, (const long long*)group_primitives_dev,
+                       (const long long*)group_starts_dev, (long long)num_groups, segment, partial_dev);
+    MLPSP_LAUNCH_CHECK();
+  }
+  hipLaunchKernelGGL(geometry_finish_kernel, dim3((unsigned)((num_primitives + 255) / 256)), dim3(256), 0, s,
+                     partial_dev, (const long long*)group_offsets_dev, quats_dev, num_primitives, grad_positions_dev,
                      grad_log_scales_dev, grad_quats_dev);
   MLPSP_LAUNCH_CHECK();
   return MLPSP_OK;

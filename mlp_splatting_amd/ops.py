@@ -440,13 +440,19 @@ def records_reverse_adjoints(ids, offsets, raw, grad_rgb, grad_t):
     return d4, adj
 
 
-def geometry_gradients(csr_offsets, record_indices, x6_sorted, falloff_adjoint, log_scales, quats):
-    """(grad_positions, grad_log_scales, grad_quats) from records in primitive-major order."""
+def geometry_gradients(csr_offsets, record_indices, x6_sorted, falloff_adjoint, log_scales, quats, groups):
+    """(grad_positions, grad_log_scales, grad_quats) from records in primitive-major order; ``groups`` is the
+    segment layout of primitive_gemm.prepare_groups for the same CSR."""
     dev = log_scales.device
-    gp, gs, gq = torch.zeros_like(log_scales), torch.zeros_like(log_scales), torch.zeros_like(quats)
+    gp, gs, gq = torch.empty_like(log_scales), torch.empty_like(log_scales), torch.empty_like(quats)
+    primitives, starts, group_offsets = groups
+    num_groups = int(primitives.numel())
+    partial = torch.empty((max(num_groups, 1), 16), dtype=torch.float32, device=dev)
     with torch.cuda.device(dev):
         _check(_lib.load().mlpsp_geometry_gradients(_ptr(csr_offsets), _ptr(record_indices), _ptr(x6_sorted),
                                                     _ptr(falloff_adjoint), _ptr(log_scales), _ptr(quats),
-                                                    log_scales.shape[0], _ptr(gp), _ptr(gs), _ptr(gq), _stream(dev)),
+                                                    _ptr(primitives), _ptr(starts), _ptr(group_offsets), num_groups,
+                                                    int(groups.segment_size), log_scales.shape[0], _ptr(partial),
+                                                    _ptr(gp), _ptr(gs), _ptr(gq), _stream(dev)),
                "mlpsp_geometry_gradients")
     return gp, gs, gq

@@ -36,11 +36,11 @@ def _gather_rows(t, perm):
 def group_records(primitive_ids, x6, grad4, num_primitives: int, relu_masks=None) -> PrimitiveCSR:
     """Stable grouping by primitive id: inside a group the records keep their original (pixel) order
     (scannet/primitive_csr.py:23-29)."""
-    ids64 = primitive_ids.to(torch.int64)
-    perm = torch.argsort(primitive_ids, stable=True)
-    per_primitive = torch.bincount(ids64, minlength=num_primitives)
-    offsets = torch.zeros(per_primitive.numel() + 1, dtype=per_primitive.dtype, device=per_primitive.device)
-    offsets[1:] = torch.cumsum(per_primitive, 0)
+    # stable sort once; the per-primitive offsets are then 200k binary searches in the sorted ids (a histogram
+    # of 39 M ids takes 10 ms on an MI355X, the sort 1.7 ms)
+    sorted_ids, perm = torch.sort(primitive_ids, stable=True)
+    bounds = torch.arange(num_primitives + 1, device=primitive_ids.device, dtype=primitive_ids.dtype)
+    offsets = torch.searchsorted(sorted_ids, bounds, right=False).to(torch.int64)
     masks = relu_masks[perm] if relu_masks is not None else None
     return PrimitiveCSR(offsets=offsets, record_indices=perm, x6=x6[perm], grad4=_gather_rows(grad4, perm),
                         relu_masks=masks)

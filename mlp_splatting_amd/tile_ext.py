@@ -396,10 +396,11 @@ class TileExt:
             d4, falloff_adjoint = ops.records_reverse_adjoints(ids, pixel_offsets, raw, x[15], x[16])
             weights = [W1, b1, W2, b2, W3, b3]
             csr = group_records(ids, x6, d4, positions.shape[0], masks)
+            groups = primitive_gemm.prepare_groups(csr)
             gp, gs, gq = ops.geometry_gradients(csr.offsets, csr.record_indices, csr.x6, falloff_adjoint, log_scales,
-                                                quats)
+                                                quats, groups)
         if tuple(W1.shape[1:]) == (32, 72) and freq.numel() == 6:
-            grads = primitive_gemm.grouped_weight_gradients(csr, freq, att, weights, dtype=torch.float32)
+            grads = primitive_gemm.grouped_weight_gradients(csr, freq, att, weights, dtype=torch.float32, groups=groups)
         else:   # other MLP shapes: the dense chain per primitive (small scenes and tests only)
             grads = reference_weight_gradients(csr, freq, att, weights)
         return [*grads, gp, gs, gq]

@@ -55,7 +55,12 @@ def test_reverse_on_records_of_a_rendered_frame(device, oracle_mod):
     d4b, adjoint = ops.records_reverse_adjoints(ids, offsets, raw, grgb, gt)
     assert torch.equal(d4b, got[0])
     csr_b = _group(ids, x6, d4b, fr.scene.n, masks)
-    split = ops.geometry_gradients(csr_b.offsets, csr_b.record_indices, csr_b.x6, adjoint, x[3], x[4])
+    from mlp_splatting_amd import primitive_gemm
+    for segment in (32, 512):
+        split = ops.geometry_gradients(csr_b.offsets, csr_b.record_indices, csr_b.x6, adjoint, x[3], x[4],
+                                       primitive_gemm.prepare_groups(csr_b, segment))
+        for name, a, b in zip(("grad_positions", "grad_log_scales", "grad_quats"), split, want[1:]):
+            _close(a, b, name + f" (split, segment {segment})")
     for name, a, b in zip(("grad_positions", "grad_log_scales", "grad_quats"), split, want[1:]):
         _close(a, b, name + " (split)")
     # and it feeds the grouped weight gradients
