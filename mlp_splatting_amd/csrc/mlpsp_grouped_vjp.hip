@@ -255,6 +255,189 @@ __global__ __launch_bounds__(64) void grouped_vjp_kernel(
   if (lane < 4) out[3520 + lane] = gb3 * inv;
 }
 
+// ---------------------------------------------------------------------------------------------
+// The f32 path.  v_mfma_f32_32x32x2_f32 takes ONE element per lane and operand, so an operand can be read from
+// LDS in either orientation and no transposed copies are needed; and the contraction over the block's records
+// may run in any order, so the weight-gradient products take their A operand -- an adjoint tile, transposed --
+// straight from the accumulator registers that hold it: register i of lane (column c, group g) is row
+// rec(i, g) = 8 (i / 4) + 4 g + i % 4, which is used as "record 2 i + g" of the contraction, the B operand
+// reading the same record's row.  Tiles in LDS: encoding, both hidden activations, d2 and d3 (row-major,
+// [record][column]) and the weights in their own layout: 37 KB per wavefront, four wavefronts per CU.
+// ---------------------------------------------------------------------------------------------
+struct VjpTilesF32 {
+  static constexpr int LD1 = 73, LD32 = 33, LD3 = 5;
+  float w1[32 * LD1];    // [hid][k]
+  float w2[32 * LD32];   // [hid2][hid]
+  float w3[4 * LD32];    // [out][hid2]
+  float enc[32 * LD1];   // [rec][k]
+  float h1[32 * LD32];   // [rec][hid]
+  float h2[32 * LD32];   // [rec][hid2]
+  float d2[32 * LD32];   // [rec][hid2]
+  float d3[32 * LD3];    // [rec][out]
+  int32_t mask[2][32];
+};
+
+__device__ __forceinline__ vf32x16 mfma32(float a, float b, vf32x16 c) {
+  return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
+}
+
+// acc += A B over STEPS MFMAs; element k of the operands at a[k * a_stride], b[k * b_stride] (the caller folds
+// the lane's row/column and k-group into the pointers).  Operands are fetched CHUNK steps ahead of the MFMAs
+// that use them: written as "load, wait, MFMA" per step the LDS latency is paid once per instruction.
+template <int STEPS, int CHUNK>
+__device__ __forceinline__ vf32x16 mma_f32(const float* a, int a_stride, const float* b, int b_stride, vf32x16 acc) {
+  static_assert(STEPS % CHUNK == 0, "whole chunks");
+#pragma unroll
+  for (int c0 = 0; c0 < STEPS; c0 += CHUNK) {
+    float av[CHUNK], bv[CHUNK];
+#pragma unroll
+    for (int s = 0; s < CHUNK; ++s) {
+      av[s] = a[(c0 + s) * a_stride];
+      bv[s] = b[(c0 + s) * b_stride];
+    }
+#pragma unroll
+    for (int s = 0; s < CHUNK; ++s) acc = mfma32(av[s], bv[s], acc);
+  }
+  return acc;
+}
+
+__global__ __launch_bounds__(64) void grouped_vjp_f32_kernel(
+    const float* __restrict__ x6, const float* __restrict__ grad4, const int32_t* __restrict__ masks,
+    const long long* __restrict__ offsets, const long long* __restrict__ group_prim,
+    const long long* __restrict__ group_start, const float* __restrict__ freq, const float* __restrict__ att,
+    const float* __restrict__ W1, const float* __restrict__ b1, const float* __restrict__ W2,
+    const float* __restrict__ b2, const float* __restrict__ W3, float scale, int segment,
+    float* __restrict__ partial) {
+  using TL = VjpTilesF32;
+  __shared__ TL t;
+  const int lane = threadIdx.x, n = lane & 31, g = lane >> 5;
+  const long long group = blockIdx.x;
+  const long long p = group_prim[group];
+  const long long begin = group_start[group];
+  const long long seg_end = begin + segment, list_end = offsets[p + 1];
+  const long long end = seg_end < list_end ? seg_end : list_end;
+  for (int i = lane; i < 32 * 72; i += 64) t.w1[(i / 72) * TL::LD1 + i % 72] = W1[p * 2304 + i];
+  for (int i = lane; i < 32 * 32; i += 64) t.w2[(i >> 5) * TL::LD32 + (i & 31)] = W2[p * 1024 + i];
+  for (int i = lane; i < 4 * 32; i += 64) t.w3[(i >> 5) * TL::LD32 + (i & 31)] = W3[p * 128 + i];
+  const float bias1 = b1[p * 32 + n], bias2 = b2[p * 32 + n];
+  __syncthreads();
+
+  vf32x16 gw1[3], gw2, gw3;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) gw1[0][i] = gw1[1][i] = gw1[2][i] = gw2[i] = gw3[i] = 0.f;
+  float gb1 = 0.f, gb2 = 0.f, gb3 = 0.f;
+  const vf32x16 zero = gw2;
+  const int n2 = n < 8 ? n : 0;    // column of the third 32-wide block of the 72 encoding columns (64 + n2)
+
+  for (long long base = begin; base < end; base += 32) {
+    const long long rec = base + n;
+    const bool live = rec < end;
+#pragma unroll
+    for (int c = 0; c < 3; ++c) {
+      const float x = live ? x6[rec * 6 + 3 * g + c] : 0.f;
+#pragma unroll
+      for (int f = 0; f < 6; ++f) {
+        const int j = (3 * g + c) * 6 + f;
+        float s, co;
+        det_sincos((x * freq[f]) * att[f], s, co);
+        t.enc[n * TL::LD1 + j] = live ? s : 0.f;
+        t.enc[n * TL::LD1 + 36 + j] = live ? co : 0.f;
+      }
+    }
+    if (g == 0) {
+#pragma unroll
+      for (int o = 0; o < 4; ++o) t.d3[n * TL::LD3 + o] = live ? grad4[rec * 4 + o] * scale : 0.f;
+    } else if (masks) {
+      t.mask[0][n] = live ? masks[rec * 2] : 0;
+      t.mask[1][n] = live ? masks[rec * 2 + 1] : 0;
+    }
+    __syncthreads();
+
+    // forward (accumulator column = hidden unit n, register i = record 8 (i/4) + 4 g + i%4)
+    vf32x16 a1 = mma_f32<36, 18>(t.enc + n * TL::LD1 + g, 2, t.w1 + n * TL::LD1 + g, 2, zero);
+    unsigned act1 = 0u, act2 = 0u;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int row = 8 * (i >> 2) + 4 * g + (i & 3);
+      const float h = fmaxf(a1[i] + bias1, 0.f);
+      t.h1[row * TL::LD32 + n] = h;
+      act1 |= (masks ? ((unsigned)t.mask[0][row] >> n) & 1u : (h > 0.f ? 1u : 0u)) << i;
+    }
+    __syncthreads();
+    vf32x16 a2 = mma_f32<16, 16>(t.h1 + n * TL::LD32 + g, 2, t.w2 + n * TL::LD32 + g, 2, zero);
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int row = 8 * (i >> 2) + 4 * g + (i & 3);
+      const float h = fmaxf(a2[i] + bias2, 0.f);
+      t.h2[row * TL::LD32 + n] = h;
+      act2 |= (masks ? ((unsigned)t.mask[1][row] >> n) & 1u : (h > 0.f ? 1u : 0u)) << i;
+    }
+    // backward
+    vf32x16 dd2 = mma_f32<2, 2>(t.d3 + n * TL::LD3 + g, 2, t.w3 + g * TL::LD32 + n, 2 * TL::LD32, zero);
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int row = 8 * (i >> 2) + 4 * g + (i & 3);
+      dd2[i] = ((act2 >> i) & 1u) ? dd2[i] : 0.f;
+      gb2 += dd2[i];
+      t.d2[row * TL::LD32 + n] = dd2[i];
+    }
+    if (lane < 4) {
+      for (int r = 0; r < 32; ++r) gb3 += t.d3[r * TL::LD3 + lane];
+    }
+    __syncthreads();
+    vf32x16 dd1 = mma_f32<16, 16>(t.d2 + n * TL::LD32 + g, 2, t.w2 + g * TL::LD32 + n, 2 * TL::LD32, zero);
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      dd1[i] = ((act1 >> i) & 1u) ? dd1[i] : 0.f;
+      gb1 += dd1[i];
+    }
+    // weight gradients: A = the adjoint tile from registers, B = the activation row of the same record
+#pragma unroll
+    for (int i0 = 0; i0 < 16; i0 += 4) {      // operands of four records ahead of their twenty MFMAs
+      float e0[4], e1[4], e2[4], v1[4], v2[4], v3[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int i = i0 + u, row = 8 * (i >> 2) + 4 * g + (i & 3);
+        e0[u] = t.enc[row * TL::LD1 + n];
+        e1[u] = t.enc[row * TL::LD1 + 32 + n];
+        e2[u] = t.enc[row * TL::LD1 + 64 + n2];
+        v1[u] = t.h1[row * TL::LD32 + n];
+        v2[u] = t.h2[row * TL::LD32 + n];
+        v3[u] = t.d3[row * TL::LD3 + (n < 4 ? n : 0)];
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int i = i0 + u;
+        gw1[0] = mfma32(dd1[i], e0[u], gw1[0]);
+        gw1[1] = mfma32(dd1[i], e1[u], gw1[1]);
+        gw1[2] = mfma32(dd1[i], e2[u], gw1[2]);
+        gw2 = mfma32(dd2[i], v1[u], gw2);
+        gw3 = mfma32(n < 4 ? v3[u] : 0.f, v2[u], gw3);
+      }
+    }
+    __syncthreads();
+  }
+
+  float* __restrict__ out = partial + group * kGradFloats;
+  const float inv = 1.f / scale;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const int row = 8 * (i >> 2) + 4 * g + (i & 3);
+    out[row * 72 + n] = gw1[0][i] * inv;
+    out[row * 72 + 32 + n] = gw1[1][i] * inv;
+    if (n < 8) out[row * 72 + 64 + n] = gw1[2][i] * inv;
+    out[2336 + row * 32 + n] = gw2[i] * inv;
+    if (row < 4) out[3392 + row * 32 + n] = gw3[i] * inv;
+  }
+  gb1 += __shfl_xor(gb1, 32);
+  gb2 += __shfl_xor(gb2, 32);
+  if (g == 0) {
+    out[2304 + n] = gb1 * inv;
+    out[3360 + n] = gb2 * inv;
+  }
+  if (lane < 4) out[3520 + lane] = gb3 * inv;
+}
+
 // One thread per (primitive, gradient element): sum over the primitive's segments; flag non-finite sums.
 __global__ __launch_bounds__(256) void reduce_partials_kernel(const float* __restrict__ partial,
                                                               const long long* __restrict__ group_offsets,
@@ -300,7 +483,11 @@ MLPSP_API int mlpsp_grouped_vjp(const float* x6_dev, const float* grad4_dev, con
                        (const long long*)group_starts_dev, freq_dev, att_dev, W1, b1, W2, b2, W3, scale, segment,  \
                        partial_dev);                                                                               \
   } while (0)
-  if (precision == 0) MLPSP_VJP_LAUNCH(float);
+  if (precision == 0)
+    hipLaunchKernelGGL(grouped_vjp_f32_kernel, grid, block, 0, s, x6_dev, grad4_dev, relu_masks_dev,
+                       (const long long*)csr_offsets_dev, (const long long*)group_primitives_dev,
+                       (const long long*)group_starts_dev, freq_dev, att_dev, W1, b1, W2, b2, W3, scale, segment,
+                       partial_dev);
   else if (precision == 1) MLPSP_VJP_LAUNCH(_Float16);
   else MLPSP_VJP_LAUNCH(__bf16);
 #undef MLPSP_VJP_LAUNCH
