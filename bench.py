@@ -39,11 +39,24 @@ def train_steps(args, scene, frames, proj, thr, W, H, sc, dev):
     gen.manual_seed(1)
     target = torch.rand(W * H, 3, device=dev, generator=gen)
 
+    feature_dim = 0 if scene.feat_attr is None else int(scene.feat_attr.shape[-1])
+    feature_target = None
+    if feature_dim:
+        # record-based step with the streamed feature loss against a quarter-resolution target
+        params.append(scene.feat_attr)
+        opt = torch.optim.Adam(params, lr=1e-4, fused=True)
+        feature_target = (torch.randn(H // 4, W // 4, feature_dim, device=dev, generator=gen) * 0.05).half()
+
     def step(i):
         ro, rd, views, _ = frames[i % len(frames)]
         opt.zero_grad(set_to_none=True)
-        rgb = scene(ro, rd, score_threshold=thr, view_matrix=views[0], proj_matrix=proj)
-        loss = (rgb - target).abs().mean()
+        if feature_target is None:
+            rgb = scene(ro, rd, score_threshold=thr, view_matrix=views[0], proj_matrix=proj)
+            loss = (rgb - target).abs().mean()
+        else:
+            rgb, feature_loss = scene(ro, rd, score_threshold=thr, view_matrix=views[0], proj_matrix=proj,
+                                      return_feature=True, feature_target=feature_target)
+            loss = (rgb - target).abs().mean() + 0.5 * feature_loss
         loss.backward()
         opt.step()
         return loss
@@ -58,12 +71,17 @@ def train_steps(args, scene, frames, proj, thr, W, H, sc, dev):
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     print(json.dumps({
-        "metric": "training_steps_per_sec_1200x680_200k_primitives", "value": round(steps / elapsed, 3),
+        "metric": ("training_steps_per_sec_1200x680_200k_primitives" if not feature_dim else
+                   f"feature_training_steps_per_sec_{args.workload}"), "value": round(steps / elapsed, 3),
         "unit": "steps/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
         "ms_per_step": round(1000.0 * elapsed / steps, 3), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": args.workload, "primitives": sc.n, "width": W, "height": H, "tile": 8, "threshold": thr,
-                   "poses": len(frames), "loss": "L1 against a fixed random image", "optimizer": "Adam (fused), all 9 tensors",
+                   "poses": len(frames), "loss": ("L1 against a fixed random image" if not feature_dim else
+                            "L1 image loss + streamed feature L1 against a quarter-resolution fp16 target"),
+                   "feature_channels": feature_dim, "mlp_gradient_precision": ("f32" if not feature_dim else
+                                                                               os.environ.get("MLPSP_CSR_MLP_PRECISION", "float16")),
+                   "optimizer": "Adam (fused), all parameter tensors",
                    "entry": "NeuralPrimitiveSceneTileCUDA.forward + backward"},
         "final_loss": round(float(loss.detach()), 6)}))
     return 0

@@ -74,15 +74,21 @@ __global__ __launch_bounds__(128) void stream_l1_kernel(const int32_t* __restric
     loss[(long long)pix * gridDim.y + chunk] = (s_part[0] + s_part[1]) / (float)((long long)HF * WF * C);
 }
 
-// Adjoint of the bilinear down-sampling for one high-resolution pixel and channel: the (at most) 2 x 2 target
-// pixels whose footprint contains it, each weighted as in the forward pass (_resample_adjoint, :92-111).
-__device__ __forceinline__ float resample_adjoint(const int8_t* __restrict__ signs, int pix, int c, int W, int H, int WF,
-                                                  int HF, int C) {
+// What a record contributes does not depend on the channel except through the signs it samples: its four
+// bilinear taps (offset of the target pixel's sign row, weight) and its slot factors T alpha gate_s.  Per batch
+// of 64 records these are computed once, lane = record, and parked in LDS; then lane = 4 consecutive channels and
+// every record costs four 4-byte sign loads and the multiply-adds.
+struct RecordTaps {
+  int off[4];      // (iy * WF + ix) * C of the tap's target pixel, or -1 outside the target
+  float weight[4];
+  float a[8];      // slot factors (SLOTS of them), rounded to fp16 in mixed mode
+};
+
+__device__ __forceinline__ void record_taps(int pix, int W, int H, int WF, int HF, int C, RecordTaps& t) {
   const int xx = pix % W, yy = pix / W;
   const float fx = (float)WF / (float)W, fy = (float)HF / (float)H, bx = (float)W / (float)WF, by = (float)H / (float)HF;
   const int tx = (int)__builtin_floorf(((float)xx + .5f) * fx - .5f);
   const int ty = (int)__builtin_floorf(((float)yy + .5f) * fy - .5f);
-  float grad = 0.f;
 #pragma unroll
   for (int dy = 0; dy < 2; ++dy) {
 #pragma unroll
@@ -90,19 +96,18 @@ __device__ __forceinline__ float resample_adjoint(const int8_t* __restrict__ sig
       const int ix = tx + dx, iy = ty + dy;
       const float srcx = fmaxf(((float)ix + .5f) * bx - .5f, 0.f);
       const float srcy = fmaxf(((float)iy + .5f) * by - .5f, 0.f);
-      const float weight = fmaxf(0.f, 1.f - __builtin_fabsf(srcx - (float)xx)) *
-                           fmaxf(0.f, 1.f - __builtin_fabsf(srcy - (float)yy));
+      t.weight[dy * 2 + dx] = fmaxf(0.f, 1.f - __builtin_fabsf(srcx - (float)xx)) *
+                              fmaxf(0.f, 1.f - __builtin_fabsf(srcy - (float)yy));
       const bool inside = ix >= 0 && ix < WF && iy >= 0 && iy < HF;
-      const float s = inside ? (float)signs[((long long)iy * WF + ix) * C + c] : 0.f;
-      grad += weight * s;
+      t.off[dy * 2 + dx] = inside ? (iy * WF + ix) * C : -1;
     }
   }
-  return grad;
 }
 
-// One workgroup = one segment of a primitive's records x 64 channels; lane = channel.  accum[slot] +=
-// (T alpha gate_slot)[record] * adjoint[record's pixel, channel]; MIXED rounds both factors to fp16 first, as
-// the reference's mixed GEMM does, and keeps the f32 accumulation (_feature_vjp, :114-149).
+// One wavefront = one segment of a primitive's records x 256 channels (_feature_vjp, :114-149):
+// accum[slot][channel] += (T alpha gate_slot)[record] * adjoint[record's pixel, channel], the adjoint being the
+// bilinear transpose of the signs (_resample_adjoint, :92-111: taps added in the order (0,0), (0,1), (1,0),
+// (1,1)).  MIXED rounds both factors to fp16 first, as the reference's mixed GEMM does; accumulation is f32.
 template <int SLOTS, bool MIXED>
 __global__ __launch_bounds__(64) void feature_vjp_kernel(const int8_t* __restrict__ signs,
                                                          const long long* __restrict__ order,
@@ -113,38 +118,76 @@ __global__ __launch_bounds__(64) void feature_vjp_kernel(const int8_t* __restric
                                                          const long long* __restrict__ group_start,
                                                          float* __restrict__ partial, int W, int H, int WF, int HF, int C,
                                                          int segment) {
+  __shared__ RecordTaps s_rec[64];
   const long long group = blockIdx.x;
-  const int c = blockIdx.y * 64 + threadIdx.x;
-  const bool valid = c < C;
-  const int cc = valid ? c : 0;
+  const int lane = threadIdx.x;
+  const int c0 = blockIdx.y * 256 + lane * 4;
   const long long p = group_prim[group];
   const long long begin = group_start[group];
   const long long seg_end = begin + segment, list_end = offsets[p + 1];
   const long long end = seg_end < list_end ? seg_end : list_end;
-  float accum[SLOTS];
+  const bool vec = (C % 4 == 0) && (c0 + 3 < C);     // the lane's four channels are one aligned 4-byte load
+  float accum[SLOTS][4];
 #pragma unroll
-  for (int s = 0; s < SLOTS; ++s) accum[s] = 0.f;
-  for (long long row = begin; row < end; ++row) {
-    const long long r = order[row];
-    const int pix = record_pixels[r];
-    const float w = raw[r * 8 + 4] * raw[r * 8 + 5];
-    float bq = resample_adjoint(signs, pix, cc, W, H, WF, HF, C);
-    if constexpr (MIXED) bq = (float)(_Float16)bq;
+  for (int s = 0; s < SLOTS; ++s)
 #pragma unroll
-    for (int s = 0; s < SLOTS; ++s) {
-      float g = 1.f;
-      if constexpr (SLOTS == 4) g = gates[r * 4 + s];
-      if constexpr (SLOTS == 5) g = (s == 0) ? 1.f : gates[r * 4 + s - 1];
-      float a = w * g;
-      if constexpr (MIXED) a = (float)(_Float16)a;
-      accum[s] += a * bq;
+    for (int k = 0; k < 4; ++k) accum[s][k] = 0.f;
+  for (long long base = begin; base < end; base += 64) {
+    const long long row = base + lane;
+    if (row < end) {
+      const long long r = order[row];
+      RecordTaps t;
+      record_taps(record_pixels[r], W, H, WF, HF, C, t);
+      const float w = raw[r * 8 + 4] * raw[r * 8 + 5];
+#pragma unroll
+      for (int s = 0; s < SLOTS; ++s) {
+        float g = 1.f;
+        if constexpr (SLOTS == 4) g = gates[r * 4 + s];
+        if constexpr (SLOTS == 5) g = (s == 0) ? 1.f : gates[r * 4 + s - 1];
+        float a = w * g;
+        if constexpr (MIXED) a = (float)(_Float16)a;
+        t.a[s] = a;
+      }
+      s_rec[lane] = t;
     }
-  }
-  if (valid) {
-    const float norm = (float)((long long)WF * HF * C);
+    __syncthreads();
+    const int count = (int)((end - base) < 64 ? (end - base) : 64);
+    for (int rr = 0; rr < count; ++rr) {
+      const RecordTaps& t = s_rec[rr];
+      float b[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int s = 0; s < SLOTS; ++s) partial[(group * SLOTS + s) * C + c] = accum[s] / norm;
+      for (int tap = 0; tap < 4; ++tap) {
+        const int off = t.off[tap];
+        const float wt = t.weight[tap];
+        float sv[4] = {0.f, 0.f, 0.f, 0.f};
+        if (off >= 0) {
+          if (vec) {
+            const int packed = *reinterpret_cast<const int*>(signs + (long long)off + c0);
+#pragma unroll
+            for (int k = 0; k < 4; ++k) sv[k] = (float)(int8_t)(packed >> (8 * k));
+          } else {
+#pragma unroll
+            for (int k = 0; k < 4; ++k) sv[k] = (c0 + k < C) ? (float)signs[(long long)off + c0 + k] : 0.f;
+          }
+        }
+#pragma unroll
+        for (int k = 0; k < 4; ++k) b[k] += wt * sv[k];
+      }
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        if constexpr (MIXED) b[k] = (float)(_Float16)b[k];
+#pragma unroll
+        for (int s = 0; s < SLOTS; ++s) accum[s][k] += t.a[s] * b[k];
+      }
+    }
+    __syncthreads();
   }
+  const float norm = (float)((long long)WF * HF * C);
+#pragma unroll
+  for (int s = 0; s < SLOTS; ++s)
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+      if (c0 + k < C) partial[(group * SLOTS + s) * C + c0 + k] = accum[s][k] / norm;
 }
 
 // out[p][k] = sum over the primitive's segments (_feature_reduce, :152-161)
@@ -212,7 +255,7 @@ MLPSP_API int mlpsp_feature_attribute_gradients(const int8_t* signs_dev, const i
     if (!signs_dev || !record_indices_dev || !record_pixels_dev || !raw_dev || !csr_offsets_dev ||
         !group_primitives_dev || !group_starts_dev || !partial_dev)
       return MLPSP_E_ARGUMENT;
-    const dim3 grid((unsigned)num_groups, (unsigned)((channels + 63) / 64)), block(64);
+    const dim3 grid((unsigned)num_groups, (unsigned)((channels + 255) / 256)), block(64);
 #define MLPSP_FV_LAUNCH(SL, MX)                                                                                    \
   hipLaunchKernelGGL((feature_vjp_kernel<SL, MX>), grid, block, 0, s, signs_dev,                                   \
                      (const long long*)record_indices_dev, record_pixels_dev, raw_dev, gates_dev,                  \

@@ -375,6 +375,24 @@ class TileExt:
             _chk(int(lo) >= 0 and int(hi) < n)
         return list(ops.records_reverse(ids, offsets, x6, raw, logs, quats, grgb, gt))
 
+    def primitive_records_reverse_adjoints(self, ids, offsets, raw, grgb, gt):
+        """(d4 [R,4], falloff adjoint [R]): the reverse walk of ``primitive_records_reverse`` without its atomic
+        geometry sums (no counterpart in the reference; ``primitive_geometry_gradients`` completes it)."""
+        for t in (ids, offsets, raw, grgb, gt):
+            _chk(t.is_cuda and t.is_contiguous() and t.device == ids.device)
+        _chk(ids.dtype == torch.int32 and offsets.dtype == torch.int64 and raw.dtype == torch.float32)
+        _chk(raw.dim() == 2 and tuple(raw.shape) == (ids.numel(), 8) and offsets.numel() == grgb.shape[0] + 1)
+        _chk(grgb.dim() == 2 and grgb.shape[1] == 3 and gt.numel() == grgb.shape[0])
+        with torch.cuda.device(ids.device):
+            return ops.records_reverse_adjoints(ids, offsets, raw, grgb, gt)
+
+    def primitive_geometry_gradients(self, csr, falloff_adjoint, log_scales, quats, groups):
+        """(grad_positions, grad_log_scales, grad_quats) from a primitive-major CSR of the records and the
+        per-record falloff adjoints, one wavefront per segment of ``groups`` (no atomics)."""
+        with torch.cuda.device(log_scales.device):
+            return ops.geometry_gradients(csr.offsets, csr.record_indices, csr.x6, falloff_adjoint, log_scales, quats,
+                                          groups)
+
     def render_tiles_backward_tilecenter_full(self, rays_o, rays_d, positions, log_scales, quats, cand, offsets,
                                               freq, att, W1, b1, W2, b2, W3, b3, grad_rgb, grad_t, Wimg, Himg, TW, TH,
                                               thr):
