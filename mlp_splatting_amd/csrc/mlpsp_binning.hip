@@ -31,6 +31,11 @@ struct BinScratch {
   int32_t* l1_list;   // [l1_capacity]
   float4* l1_bounds;  // [l1_capacity] bounds of the listed primitives, one view only (else null)
   long long l1_capacity;
+  // survivor masks of the counting passes (one ballot per 64 tested entries), so that the fill passes neither
+  // re-read the bounds nor repeat the tests:
+  unsigned long long* l1_masks;   // [S*NC][kChunk/64]
+  unsigned long long* l2_masks;   // [64 tiles of a super-tile][l1_capacity/64 + S + 1]
+  long long l2_mask_stride;
 };
 
 __host__ __device__ inline size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
@@ -49,11 +54,19 @@ inline BinScratch carve(void* base, size_t bytes, int N, int K, int S, int NC) {
   off += 256;
   // one view: the level-1 lists carry the bounds next to the ids (20 bytes per entry), so that level 2
   // streams them instead of gathering 16 bytes per lane from all over the bounds array
-  const size_t entry = sizeof(int32_t) + (K == 1 ? sizeof(float4) : 0);
-  b.l1_capacity = bytes > off + 512 ? (long long)((bytes - off - 512) / entry) : 0;
+  b.l1_masks = reinterpret_cast<unsigned long long*>(p + off);
+  off += align256((size_t)S * NC * (kChunk / 64) * sizeof(unsigned long long));
+  // per level-1 entry: 4 bytes id (+ 16 bytes bounds with one view) + 64 mask bits for the 64 tiles = 8 bytes
+  const size_t entry = sizeof(int32_t) + (K == 1 ? sizeof(float4) : 0) + 8;
+  const size_t fixed = off + 1024 + align256((size_t)(S + 1) * 64 * sizeof(unsigned long long));
+  b.l1_capacity = bytes > fixed ? (long long)((bytes - fixed) / entry) : 0;
+  b.l1_capacity &= ~63LL;
   b.l1_list = reinterpret_cast<int32_t*>(p + off);
   off += align256((size_t)b.l1_capacity * sizeof(int32_t));
   b.l1_bounds = (K == 1) ? reinterpret_cast<float4*>(p + off) : nullptr;
+  if (K == 1) off += align256((size_t)b.l1_capacity * sizeof(float4));
+  b.l2_mask_stride = b.l1_capacity / 64 + S + 1;
+  b.l2_masks = reinterpret_cast<unsigned long long*>(p + off);
   return b;
 }
 
@@ -118,6 +131,13 @@ __device__ __forceinline__ void super_rect(const BinGeom& g, int s, float& x0, f
   y1 = (float)(min((sy + 1) * kSuper, g.nty) * g.ts);
 }
 
+// mask `which` (wave-uniform) of the 64-bit values held one per lane
+__device__ __forceinline__ unsigned long long lane_value(unsigned long long v, int which) {
+  const unsigned lo = __builtin_amdgcn_readlane((unsigned)v, which);
+  const unsigned hi = __builtin_amdgcn_readlane((unsigned)(v >> 32), which);
+  return ((unsigned long long)hi << 32) | lo;
+}
+
 __device__ __forceinline__ unsigned lanes_below(unsigned long long mask) {
   return __builtin_amdgcn_mbcnt_hi((unsigned)(mask >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)mask, 0u));
 }
@@ -130,7 +150,8 @@ __global__ __launch_bounds__(kBinThreads) void bin_level1_kernel(const float4* _
                                                                  const int32_t* __restrict__ tile_view_ids,
                                                                  int32_t* __restrict__ l1_counts,
                                                                  int32_t* __restrict__ l1_list,
-                                                                 float4* __restrict__ l1_bounds, long long l1_capacity) {
+                                                                 float4* __restrict__ l1_bounds, long long l1_capacity,
+                                                                 unsigned long long* __restrict__ l1_masks) {
   const int c = blockIdx.x, s = blockIdx.y * (kBinThreads / 64) + (threadIdx.x >> 6);
   const int lane = threadIdx.x & 63;
   if (s >= g.nsx * g.nsy) return;
@@ -158,6 +179,49 @@ __global__ __launch_bounds__(kBinThreads) void bin_level1_kernel(const float4* _
   }
   long long running = FILL ? l1_counts[s * g.NC + c] : 0;
   const int first = c * kChunk;
+  unsigned long long* __restrict__ masks = l1_masks + ((size_t)s * g.NC + c) * (kChunk / 64);
+  static_assert(kChunk / 64 <= 64, "one ballot per lane");
+  if constexpr (FILL) {
+    // the counting pass left one ballot per 64 primitives: no bounds are read again except the survivors'.
+    // Lane r fetches ballot r (one coalesced load instead of a chain of dependent ones).
+    const unsigned long long mine = lane < kChunk / 64 ? masks[lane] : 0ull;
+    for (int r = 0; r < kChunk / 64; ++r) {
+      const unsigned long long m = lane_value(mine, r);
+      if (m == 0ull) continue;
+      if ((m >> lane) & 1ull) {
+        const int i = first + r * 64 + lane;
+        const long long dst = running + lanes_below(m);
+        if (dst < l1_capacity) {
+          l1_list[dst] = i;
+          if (l1_bounds) l1_bounds[dst] = bounds[i];
+        }
+      }
+      running += __popcll(m);
+    }
+    return;
+  }
+  unsigned long long mine = 0ull;
+  if (g.K == 1) {
+    // one view: eight independent 16-byte loads in flight per step (NaN bounds fail every comparison)
+    const float nanv = __builtin_nanf("");
+    for (int r0 = 0; r0 < kChunk / 64; r0 += 8) {
+      float4 bb[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int i = first + (r0 + u) * 64 + lane;
+        bb[u] = (i < g.N) ? bounds[i] : make_float4(nanv, nanv, nanv, nanv);
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const unsigned long long m = __ballot(rect_overlap(bb[u], x0, x1, y0, y1));
+        mine = (lane == r0 + u) ? m : mine;
+        running += __popcll(m);
+      }
+    }
+    if (lane < kChunk / 64) masks[lane] = mine;
+    if (lane == 0) l1_counts[s * g.NC + c] = (int32_t)running;
+    return;
+  }
 #pragma unroll 4
   for (int r = 0; r < kChunk / 64; ++r) {
     const int i = first + r * 64 + lane;
@@ -173,16 +237,11 @@ __global__ __launch_bounds__(kBinThreads) void bin_level1_kernel(const float4* _
       }
     }
     const unsigned long long m = __ballot(keep);
-    if (FILL && keep) {
-      const long long dst = running + lanes_below(m);
-      if (dst < l1_capacity) {
-        l1_list[dst] = i;
-        if (l1_bounds) l1_bounds[dst] = bounds[i];
-      }
-    }
+    mine = (lane == r) ? m : mine;
     running += __popcll(m);
   }
-  if (!FILL && lane == 0) l1_counts[s * g.NC + c] = (int32_t)running;
+  if (lane < kChunk / 64) masks[lane] = mine;
+  if (lane == 0) l1_counts[s * g.NC + c] = (int32_t)running;
 }
 
 // In-place exclusive scan of data[0..n) by one workgroup; data[n] and *total receive the sum, *largest
@@ -277,6 +336,8 @@ __global__ __launch_bounds__(kBinThreads) void bin_level2_kernel(const float4* _
                                                                  long long l1_capacity,
                                                                  int32_t* __restrict__ tile_offsets,
                                                                  int32_t* __restrict__ cand,
+                                                                 unsigned long long* __restrict__ l2_masks,
+                                                                 long long l2_mask_stride,
                                                                  const long long* __restrict__ skip_flag = nullptr) {
   const int tile = blockIdx.x * (kBinThreads / 64) + (threadIdx.x >> 6);
   const int lane = threadIdx.x & 63;
@@ -292,7 +353,57 @@ __global__ __launch_bounds__(kBinThreads) void bin_level2_kernel(const float4* _
   const int lo = (int)min((long long)l1_offsets[s * g.NC], l1_capacity);
   const int hi = (int)min((long long)l1_offsets[(s + 1) * g.NC], l1_capacity);
   int running = FILL ? tile_offsets[tile] : 0;
-  for (int base = lo; base < hi; base += 64) {
+  // ballot b of this tile lives at [tile within its super-tile][lo / 64 + s + b]: super-tile lists are
+  // consecutive in the level-1 array, so adding s keeps the slots of neighbouring lists apart
+  unsigned long long* __restrict__ masks =
+      l2_masks + (size_t)((ty % kSuper) * kSuper + (tx % kSuper)) * l2_mask_stride + (lo >> 6) + s;
+  const int nb = (hi - lo + 63) >> 6;
+  if constexpr (FILL) {
+    for (int b0 = 0; b0 < nb; b0 += 64) {       // 64 ballots per coalesced load, lane b holds ballot b0 + b
+      const unsigned long long mine = (b0 + lane < nb) ? masks[b0 + lane] : 0ull;
+      const int nhere = min(64, nb - b0);
+      for (int b = 0; b < nhere; b += 8) {      // eight ballots at a time: their id loads are in flight together
+        unsigned long long m[8];
+        int id[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) m[u] = (b + u < nhere) ? lane_value(mine, (b + u) & 63) : 0ull;
+#pragma unroll
+        for (int u = 0; u < 8; ++u) id[u] = ((m[u] >> lane) & 1ull) ? l1_list[lo + ((b0 + b + u) << 6) + lane] : 0;
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          if ((m[u] >> lane) & 1ull) cand[running + lanes_below(m[u])] = id[u];
+          running += __popcll(m[u]);
+        }
+      }
+    }
+    return;
+  }
+  unsigned long long mine = 0ull;
+  if (l1_bounds) {
+    // one view: the bounds sit next to the ids; four independent 16-byte loads in flight per step
+    const float nanv = __builtin_nanf("");
+    for (int b = 0; b < nb; b += 4) {
+      float4 bb[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int j = lo + ((b + u) << 6) + lane;
+        bb[u] = (j < hi) ? l1_bounds[j] : make_float4(nanv, nanv, nanv, nanv);
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        if (b + u < nb) {
+          const unsigned long long m = __ballot(rect_overlap(bb[u], x0, x1, y0, y1));
+          mine = (lane == ((b + u) & 63)) ? m : mine;
+          if (((b + u) & 63) == 63) masks[b + u - 63 + lane] = mine;
+          running += __popcll(m);
+        }
+      }
+    }
+    if ((nb & 63) != 0 && lane < (nb & 63)) masks[(nb & ~63) + lane] = mine;
+    if (lane == 0) tile_offsets[tile] = running;
+    return;
+  }
+  for (int base = lo, b = 0; base < hi; base += 64, ++b) {
     const int j = base + lane;
     int id = -1;
     bool keep = false;
@@ -301,10 +412,12 @@ __global__ __launch_bounds__(kBinThreads) void bin_level2_kernel(const float4* _
       keep = rect_overlap(l1_bounds ? l1_bounds[j] : vb[id], x0, x1, y0, y1);
     }
     const unsigned long long m = __ballot(keep);
-    if (FILL && keep) cand[running + lanes_below(m)] = id;
+    mine = (lane == (b & 63)) ? m : mine;
+    if ((b & 63) == 63) masks[b - 63 + lane] = mine;       // 64 ballots at a time, one coalesced store
     running += __popcll(m);
   }
-  if (!FILL && lane == 0) tile_offsets[tile] = running;
+  if ((nb & 63) != 0 && lane < (nb & 63)) masks[(nb & ~63) + lane] = mine;
+  if (lane == 0) tile_offsets[tile] = running;
 }
 
 inline BinGeom make_geom(int N, int K, int W, int H, int ts) {
@@ -327,9 +440,12 @@ MLPSP_API size_t mlpsp_bin_scratch_bytes(int num_primitives, int num_views, int 
   size_t bytes = align256((size_t)(num_views + 1) * 16 * sizeof(float)) +
                  align256((size_t)num_views * num_primitives * sizeof(float4)) +
                  align256((S * g.NC + 1) * sizeof(int32_t)) + 256;
-  // room for every primitive to touch 8 super-tiles per view, plus slack for tiny scenes
-  const size_t entry = sizeof(int32_t) + (num_views == 1 ? sizeof(float4) : 0);
-  bytes += align256(((size_t)8 * num_views * num_primitives + 65536) * entry) + 512;
+  bytes += align256(S * g.NC * (kChunk / 64) * sizeof(unsigned long long));
+  bytes += 1024 + align256((S + 1) * 64 * sizeof(unsigned long long));
+  // room for every primitive to touch 8 super-tiles per view, plus slack for tiny scenes; per entry the id,
+  // the bounds (one view) and the 64 survivor bits of the super-tile's tiles
+  const size_t entry = sizeof(int32_t) + (num_views == 1 ? sizeof(float4) : 0) + 8;
+  bytes += align256(((size_t)8 * num_views * num_primitives + 65536) * entry) + 1024;
   return bytes;
 }
 
@@ -363,17 +479,17 @@ int enqueue_bin_count(const float* positions_dev, const float* log_scales_dev, i
   }
   MLPSP_LAUNCH_CHECK();
   hipLaunchKernelGGL((bin_level1_kernel<false>), dim3(g.NC, ceil_div(S, kBinThreads / 64)), dim3(kBinThreads), 0, s, b.bounds, g,
-                     tile_view_ids_dev, b.l1_counts, b.l1_list, b.l1_bounds, b.l1_capacity);
+                     tile_view_ids_dev, b.l1_counts, b.l1_list, b.l1_bounds, b.l1_capacity, b.l1_masks);
   MLPSP_LAUNCH_CHECK();
   hipLaunchKernelGGL(exclusive_scan_kernel, dim3(1), dim3(1024), 0, s, b.l1_counts, S * g.NC, b.totals,
                      (long long*)nullptr);
   MLPSP_LAUNCH_CHECK();
   hipLaunchKernelGGL((bin_level1_kernel<true>), dim3(g.NC, ceil_div(S, kBinThreads / 64)), dim3(kBinThreads), 0, s, b.bounds, g,
-                     tile_view_ids_dev, b.l1_counts, b.l1_list, b.l1_bounds, b.l1_capacity);
+                     tile_view_ids_dev, b.l1_counts, b.l1_list, b.l1_bounds, b.l1_capacity, b.l1_masks);
   MLPSP_LAUNCH_CHECK();
   hipLaunchKernelGGL((bin_level2_kernel<false>), dim3(ceil_div((int)T, kBinThreads / 64)), dim3(kBinThreads), 0, s,
                      b.bounds, g, tile_view_ids_dev, b.l1_counts, b.l1_list, b.l1_bounds, b.l1_capacity, tile_offsets_dev,
-                     (int32_t*)nullptr);
+                     (int32_t*)nullptr, b.l2_masks, b.l2_mask_stride);
   MLPSP_LAUNCH_CHECK();
   hipLaunchKernelGGL(exclusive_scan_kernel, dim3(1), dim3(1024), 0, s, tile_offsets_dev, (int)T, b.totals + 1,
                      b.totals + 2);
@@ -478,7 +594,7 @@ MLPSP_API int mlpsp_bin_legacy_async(const float* positions_dev, const float* lo
   MLPSP_LAUNCH_CHECK();
   hipLaunchKernelGGL((bin_level2_kernel<true>), dim3(ceil_div((int)T, kBinThreads / 64)), dim3(kBinThreads), 0, s,
                      b.bounds, g, tile_view_ids_dev, b.l1_counts, b.l1_list, b.l1_bounds, b.l1_capacity, tile_offsets_dev,
-                     candidates_dev, (const long long*)(b.totals + 3));
+                     candidates_dev, b.l2_masks, b.l2_mask_stride, (const long long*)(b.totals + 3));
   MLPSP_LAUNCH_CHECK();
   return MLPSP_OK;
 }
@@ -494,7 +610,7 @@ MLPSP_API int mlpsp_bin_legacy_fill(int num_primitives, int num_views, const int
   const BinScratch b = carve(const_cast<void*>(scratch_dev), scratch_bytes, num_primitives, num_views, g.nsx * g.nsy, g.NC);
   hipLaunchKernelGGL((bin_level2_kernel<true>), dim3(ceil_div((int)T, kBinThreads / 64)), dim3(kBinThreads), 0,
                      (hipStream_t)stream, b.bounds, g, tile_view_ids_dev, b.l1_counts, b.l1_list, b.l1_bounds, b.l1_capacity,
-                     const_cast<int32_t*>(tile_offsets_dev), candidates_dev);
+                     const_cast<int32_t*>(tile_offsets_dev), candidates_dev, b.l2_masks, b.l2_mask_stride);
   MLPSP_LAUNCH_CHECK();
   return MLPSP_OK;
 }
