@@ -275,6 +275,11 @@ __global__ __launch_bounds__(1024) void exclusive_scan_kernel(int32_t* __restric
     long long incl[kScanSlabs];
 #pragma unroll
     for (int u = 0; u < kScanSlabs; ++u) {
+      incl[u] = 0;
+      if (pass0 + u * 4096 >= n) {            // slab beyond the data (workgroup-uniform): nothing to scan
+        if (lane == 63) s_wave[u][wave] = 0;
+        continue;
+      }
       mx = max(max(mx, max(v[u].x, v[u].y)), max(v[u].z, v[u].w));
       long long x = (long long)v[u].x + v[u].y + v[u].z + v[u].w;
 #pragma unroll
@@ -289,6 +294,7 @@ __global__ __launch_bounds__(1024) void exclusive_scan_kernel(int32_t* __restric
     long long base = carry;
 #pragma unroll
     for (int u = 0; u < kScanSlabs; ++u) {
+      if (pass0 + u * 4096 >= n) continue;
       long long before = 0, slab = 0;
 #pragma unroll
       for (int w = 0; w < 16; ++w) {
