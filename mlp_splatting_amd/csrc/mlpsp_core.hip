@@ -126,34 +126,38 @@ __global__ __launch_bounds__(kSortThreads) void sort_tiles_kernel(
   const float ox = rays_o[pc * 3 + 0], oy = rays_o[pc * 3 + 1], oz = rays_o[pc * 3 + 2];
   const float dx = rays_d[pc * 3 + 0], dy = rays_d[pc * 3 + 1], dz = rays_d[pc * 3 + 2];
 
+  // The first round's candidate id and geometry record are requested before the pyramid phase (two dependent
+  // gathers whose latency then overlaps the corner-ray loads and the barriers below); every round requests the
+  // next round's in the same way.
+  int p_next = (tid < n) ? cand[start + tid] : 0;
+  PrimRecord P_next = prims[p_next];
+
   // ---- the tile's ray pyramid (only when culling is requested)
   const bool culling = cull_r2 > 0.f;
   if (culling) {
     const int tx = tile % g.ntx, ty = tile / g.ntx;
     const int x0 = tx * g.TW, y0 = ty * g.TH;
     const int x1 = min(x0 + g.TW, g.W) - 1, y1 = min(y0 + g.TH, g.H) - 1;
-    if (tid == 0) {
-      const int corner[4] = {y0 * g.W + x0, y0 * g.W + x1, y1 * g.W + x1, y1 * g.W + x0};
-      float d[4][3];
-      for (int k = 0; k < 4; ++k)
-        for (int e = 0; e < 3; ++e) d[k][e] = rays_d[corner[k] * 3 + e];
-      s_pyr.ox = rays_o[corner[0] * 3 + 0];
-      s_pyr.oy = rays_o[corner[0] * 3 + 1];
-      s_pyr.oz = rays_o[corner[0] * 3 + 2];
-      for (int j = 0; j < 4; ++j) {
-        const float* a = d[j];
-        const float* b = d[(j + 1) & 3];
-        float nx = a[1] * b[2] - a[2] * b[1], ny = a[2] * b[0] - a[0] * b[2], nz = a[0] * b[1] - a[1] * b[0];
-        // orient towards the tile-centre ray; a face the centre ray (nearly) lies in is not used
-        const float side = nx * dx + ny * dy + nz * dz;
-        const float len = sqrtf(nx * nx + ny * ny + nz * nz);
-        const float sgn = side < 0.f ? -1.f : 1.f;
-        s_pyr.n[j][0] = sgn * nx;
-        s_pyr.n[j][1] = sgn * ny;
-        s_pyr.n[j][2] = sgn * nz;
-        s_face_ok[j] = (len > 0.f && fabsf(side) > 1e-4f * len) ? 1 : 0;
+    if (tid < 4) {      // lane j builds face j from corner rays j and j+1
+      const int cx[4] = {x0, x1, x1, x0}, cy[4] = {y0, y0, y1, y1};
+      const int ca = cy[tid] * g.W + cx[tid], cb = cy[(tid + 1) & 3] * g.W + cx[(tid + 1) & 3];
+      const float a0 = rays_d[ca * 3], a1 = rays_d[ca * 3 + 1], a2 = rays_d[ca * 3 + 2];
+      const float b0 = rays_d[cb * 3], b1 = rays_d[cb * 3 + 1], b2 = rays_d[cb * 3 + 2];
+      if (tid == 0) {
+        s_pyr.ox = rays_o[ca * 3 + 0];
+        s_pyr.oy = rays_o[ca * 3 + 1];
+        s_pyr.oz = rays_o[ca * 3 + 2];
+        s_origin_ok = 1;
       }
-      s_origin_ok = 1;
+      const float nx = a1 * b2 - a2 * b1, ny = a2 * b0 - a0 * b2, nz = a0 * b1 - a1 * b0;
+      // orient towards the tile-centre ray; a face the centre ray (nearly) lies in is not used
+      const float side = nx * dx + ny * dy + nz * dz;
+      const float len = sqrtf(nx * nx + ny * ny + nz * nz);
+      const float sgn = side < 0.f ? -1.f : 1.f;
+      s_pyr.n[tid][0] = sgn * nx;
+      s_pyr.n[tid][1] = sgn * ny;
+      s_pyr.n[tid][2] = sgn * nz;
+      s_face_ok[tid] = (len > 0.f && fabsf(side) > 1e-4f * len) ? 1 : 0;
     }
     __syncthreads();
     // every ray of the tile must start at the common origin and lie inside every face used
@@ -189,9 +193,13 @@ __global__ __launch_bounds__(kSortThreads) void sort_tiles_kernel(
     bool keep = false, outside = false;
     int p = 0;
     float key = 0.f;
+    const PrimRecord P = P_next;
+    p = p_next;
+    if (i + kSortThreads < n) {
+      p_next = cand[start + i + kSortThreads];
+      P_next = prims[p_next];
+    }
     if (i < n) {
-      p = cand[start + i];
-      const PrimRecord P = prims[p];
       if (faces) {
         const float ex = P.cx - s_pyr.ox, ey = P.cy - s_pyr.oy, ez = P.cz - s_pyr.oz;
 #pragma unroll
