@@ -183,6 +183,37 @@ int mlpsp_records_emit(const float* rays_o_dev, const float* rays_d_dev, const v
                        int32_t* masks_dev, float* raw_dev, float* gates_dev, float* out_rgb_dev, float* out_alpha_dev,
                        int32_t* overflow_dev, mlpsp_stream_t stream);
 
+/* Training-records forward with the MLP on the matrix cores = render_training_wmma_kernel
+ * (scannet/cuda/training_wmma.cuh:62-253; wrapper render_tiles_training_records_wmma :267-357).  8x8 tiles,
+ * 72->32->32->4 MLP with six frequencies; packed_dev = mlpsp_pack_mfma_weights of the six weight tensors in
+ * the precision of use_bf16.  order_dev is the tile list sorted by mlpsp_sort_tiles (t* key): the reference
+ * sorts inside its kernel, here the sorted list is shared with the scalar record forward.  Geometry, record
+ * order, x6, decay and gates are the f32 expressions of mlpsp_records_count/emit; R, G, B, sigma, alpha follow
+ * the reduced-precision MLP.  Same two steps and outputs as mlpsp_records_count/emit.  status_dev (int32, NOT
+ * cleared here: the caller clears it once per frame) collects 1 = non-finite operand, activation or output
+ * (the reference repeats the whole frame with the scalar f32 record forward), 2 = a live pixel reached
+ * max_hits (hit capacity, refused), 4 = the emit step met a pixel whose hit count differs from its offsets
+ * interval (nothing is written outside the interval). */
+int mlpsp_records_mfma_count(const float* rays_o_dev, const float* rays_d_dev, const void* prim_records_dev,
+                             const int32_t* order_dev, const int32_t* tile_offsets_dev, const float* freq_dev,
+                             const float* att_dev, const void* packed_dev, int num_primitives, int width, int height,
+                             float threshold, int max_hits, int use_bf16, int32_t* counts_dev, int32_t* status_dev,
+                             mlpsp_stream_t stream);
+int mlpsp_records_mfma_emit(const float* rays_o_dev, const float* rays_d_dev, const void* prim_records_dev,
+                            const int32_t* order_dev, const int32_t* tile_offsets_dev, const float* freq_dev,
+                            const float* att_dev, const void* packed_dev, int num_primitives, int width, int height,
+                            float threshold, int max_hits, int use_bf16, float gating_beta, float gating_temp,
+                            const int64_t* record_offsets_dev, int64_t total_records, int32_t* ids_dev, float* x6_dev,
+                            int32_t* masks_dev, float* raw_dev, float* gates_dev, float* out_rgb_dev,
+                            float* out_alpha_dev, int32_t* status_dev, mlpsp_stream_t stream);
+
+/* flag_dev[0] = 1 if any element of the num_arrays (<= 16) f32 device arrays is NaN or infinite, else 0 =
+ * training_wmma_finite_kernel (scannet/cuda/training_wmma.cuh:24-60): one fused read-only scan in front of the
+ * reduced-precision record forward, which refuses non-finite inputs.  arrays_dev and lengths are HOST arrays of
+ * device pointers and element counts; empty arrays are skipped. */
+int mlpsp_all_finite(const float* const* arrays_dev, const int64_t* lengths, int num_arrays, int32_t* flag_dev,
+                     mlpsp_stream_t stream);
+
 /* Workspace of the feature renders below.  The render kernel hands the feature kernel one "hit record"
  * per (64-pixel wavefront of a tile, primitive that hits one of its pixels); how many there will be is
  * only known after the frame (early termination), so records come from a pool of pool_records records.

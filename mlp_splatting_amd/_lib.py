@@ -54,6 +54,9 @@ SIGNATURES = {
     "mlpsp_render_tilecenter_stats_f32": (_i, [_vp] * 7 + [_i] + [_vp] * 6 + [_i, _i, _i, _i, _i, _i, _f] + [_vp] * 9),
     "mlpsp_records_count": (_i, [_vp] * 7 + [_i] + [_vp] * 6 + [_i, _i, _i, _i, _i, _i, _f, _i, _vp, _vp, _vp]),
     "mlpsp_records_emit": (_i, [_vp] * 7 + [_i] + [_vp] * 6 + [_i, _i, _i, _i, _i, _i, _f, _i, _f, _f] + [_vp] * 10),
+    "mlpsp_records_mfma_count": (_i, [_vp] * 8 + [_i, _i, _i, _f, _i, _i, _vp, _vp, _vp]),
+    "mlpsp_records_mfma_emit": (_i, [_vp] * 8 + [_i, _i, _i, _f, _i, _i, _f, _f, _vp, _i64] + [_vp] * 9),
+    "mlpsp_all_finite": (_i, [_vp, _vp, _i, _vp, _vp]),
     "mlpsp_feat_workspace_bytes": (_sz, [_i64, _i, _i, _i, _i, _i, _i, _i64]),
     "mlpsp_render_tilecenter_mfma_feat": (_i, [_vp] * 5 + [_i64, _vp, _vp, _vp, _i, _i, _vp, _i, _i, _f, _f, _i, _i, _f,
                                                _vp, _sz, _vp, _vp, _vp, _vp, _vp, _vp]),

@@ -1,0 +1,299 @@
+// Matrix-core (v_mfma_f32_32x32x16, bf16 or fp16 operands, f32 accumulation) evaluation of the per-primitive
+// 72->32->32->4 MLP for one wavefront = 64 pixels = two column blocks of 32, shared by the forward render
+// (mlpsp_render_mfma.hip) and the training-records forward (mlpsp_records_mfma.hip).
+//
+// The GEMMs are computed TRANSPOSED: D[hidden][pixel] = W[hidden][k] * X[k][pixel], i.e. the weights are the
+// A operand and the pixels are the B/N dimension.  With the 32x32x16 register layout
+//     A: lane l holds row  l%32, k = 8*(l/32) + 0..7        B: lane l holds column l%32, same k
+//     D: lane l holds column l%32, rows 8*(r/4) + 4*(l/32) + r%4 for r = 0..15
+// a lane's D registers of one layer ARE a valid B operand of the next layer (same pixel column, 8 k-slots
+// per K-step) provided the next layer's weight columns are stored in that register order.  Weights are
+// therefore repacked (pack kernel in mlpsp_render_mfma.hip) into A-fragment order with the k-permutation
+// folded in, and the chain layer1 -> ReLU -> layer2 -> ReLU -> layer3 needs no LDS, no barrier and no
+// cross-lane traffic.  Staging a primitive's weights is 9 coalesced 1 KiB loads straight into VGPRs.
+//
+// Layer-1 k-slots: lane group g = l/32 owns frequencies 3g..3g+2 of every input component, so both groups
+// evaluate 18 (sin, cos) pairs per pixel block and each pair lands in one 32-bit operand word.  sin/cos use
+// the native v_sin_f32/v_cos_f32 (argument in revolutions); their error (~1e-6) is far below the operand
+// rounding applied next.  The 9 words of the ray direction do not depend on the primitive: the caller
+// computes them once per pixel (encode_direction_words) and parks them in LDS in operand form.
+#pragma once
+#include "../../include/mlpsp.h"
+#include "mlpsp_device.hpp"
+
+namespace mlpsp {
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+
+// packed per-primitive block (bytes)
+constexpr int kOffW1 = 0;       // 5 K-steps x 64 lanes x 16 B
+constexpr int kOffW2 = 5120;    // 2 K-steps x 64 lanes x 16 B
+constexpr int kOffW3 = 7168;    // 2 K-steps x 2 lane groups x 4 rows x 16 B
+constexpr int kOffB1 = 7424;    // 2 lane groups x 16 f32 in D-register order
+constexpr int kOffB2 = 7552;
+constexpr int kOffB3 = 7680;    // 4 f32
+constexpr int kOffFlag = 7696;  // int32: 1 if any rounded weight or bias is non-finite
+constexpr int kPackStride = MLPSP_MFMA_PACK_BYTES;
+static_assert(kPackStride >= kOffFlag + 4 && kPackStride % 128 == 0, "pack stride");
+
+template <typename T> struct Ops;
+template <> struct Ops<__bf16> {
+  using vec8 = bf16x8;
+  static __device__ __forceinline__ unsigned pack2(float a, float b) {
+    bf16x2 v = {(__bf16)a, (__bf16)b};
+    return __builtin_bit_cast(unsigned, v);
+  }
+  static __device__ __forceinline__ f32x16 mfma(u32x4 a, u32x4 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ float round_trip(float a) { return (float)(__bf16)a; }
+  static constexpr float kMax = 3.38953139e38f;
+  // bf16 has the exponent range of f32: a hidden pre-activation is out of range only if it is (within one
+  // rounding step of) +-inf.  Rounded to +inf it survives the ReLU and turns the next layer's sums into
+  // +-inf or NaN, down to the outputs, whose finiteness every hit checks; rounded to -inf the ReLU removes
+  // it, as it does in exact arithmetic.  The per-layer range check is therefore not needed for this type.
+  static constexpr bool kCheckHidden = false;
+};
+template <> struct Ops<_Float16> {
+  using vec8 = f16x8;
+  static __device__ __forceinline__ unsigned pack2(float a, float b) {
+    f16x2 v = {(_Float16)a, (_Float16)b};
+    return __builtin_bit_cast(unsigned, v);
+  }
+  static __device__ __forceinline__ f32x16 mfma(u32x4 a, u32x4 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ float round_trip(float a) { return (float)(_Float16)a; }
+  static constexpr float kMax = 65504.0f;
+  static constexpr bool kCheckHidden = true;   // a finite f32 pre-activation above 65504 must be reported
+};
+
+// row of the 32x32 accumulator tile held by D register r of lane group g (fixed by the instruction)
+__host__ __device__ constexpr int d_row(int r, int g) { return 8 * (r / 4) + 4 * g + (r % 4); }
+// Hidden unit assigned to that row.  Which unit sits in which row is free as long as the pack kernel uses
+// one assignment for a layer's output rows, its bias and the next layer's weight columns.  This one makes
+// the ReLU masks of the training records cheap: a lane's packed operand word (s, d) holds registers
+// r = 8s + 2d (low half) and r + 1 (high half), i.e. units 4s + d + 8g and 16 + 4s + d + 8g, so "half is
+// non-zero" shifted left by 4s + d lands on the unit's bit of the 32-bit mask (relu_mask_bits below).
+__host__ __device__ constexpr int hidden_unit(int r, int g) { return 16 * (r & 1) + (r >> 1) + 8 * g; }
+// ... and the unit held by accumulator row m (the A operand row a lane m%32 loads weights for)
+__host__ __device__ constexpr int hidden_unit_of_row(int m) { return hidden_unit(4 * (m >> 3) + (m & 3), (m >> 2) & 1); }
+
+// True if some pre-activation is +-inf or exceeds the operand type's range.  A NaN cannot appear here
+// on its own: the operands are finite (weights are checked when packed, phases when encoded), so a
+// non-finite accumulator is an overflow, which shows as +-inf -- and the max chain sees infinities.
+// ReLU of two packed 16-bit floats in one instruction: as signed 16-bit integers every negative float
+// (and -0) is below zero and every non-negative one keeps its bits, for bf16 and fp16 alike; rounding
+// commutes with ReLU, so rounding first gives the same operand.
+__device__ __forceinline__ unsigned relu_packed(unsigned x) {
+  unsigned y;
+  asm("v_pk_max_i16 %0, %1, 0" : "=v"(y) : "v"(x));
+  return y;
+}
+__device__ __forceinline__ float max3_abs(float a, float b, float c) {
+  float y;
+  asm("v_max3_f32 %0, |%1|, |%2|, |%3|" : "=v"(y) : "v"(a), "v"(b), "v"(c));
+  return y;
+}
+// The first read of the accumulator tile is a plain C++ operation, not inline assembly: the compiler
+// inserts the wait states a matrix-core result needs before its first reader only for instructions it
+// can see, and everything below depends on that first read.
+template <typename T>
+__device__ __forceinline__ bool out_of_range_in(const f32x16& v) {
+  float m = __builtin_fabsf(v[0]);
+  m = max3_abs(m, v[1], v[2]);
+#pragma unroll
+  for (int r = 3; r < 15; r += 2) m = max3_abs(m, v[r], v[r + 1]);
+  m = max3_abs(m, v[15], v[15]);
+  return !(m <= Ops<T>::kMax);
+}
+
+
+// Operand words of the ray direction for both column blocks, [block][.][lane]; one wavefront per workgroup
+// writes and reads its own copy, so no barrier is needed.
+struct DirWords {
+  u32x4 q[2][2][64];
+  unsigned w8[2][64];
+};
+
+// kf[j] = freq * att / (2 pi) of frequency 3g + j: the phase scale, in revolutions per unit input, of the
+// three frequencies this lane's group evaluates.
+__device__ __forceinline__ void phase_scales(const float* __restrict__ freq, const float* __restrict__ att, int g,
+                                             float kf[3]) {
+  constexpr float kInvTwoPi = 0.159154943f;
+#pragma unroll
+  for (int j = 0; j < 3; ++j) kf[j] = (freq[3 * g + j] * att[3 * g + j]) * kInvTwoPi;
+}
+
+template <typename T>
+__device__ __forceinline__ void encode_direction_words(float rdx, float rdy, float rdz, const float kf[3], int l,
+                                                       DirWords& s) {
+  const int g = l >> 5;
+  // the pixel this lane shares an MFMA column with: lane l and lane l^32 both hold column l%32
+  const float prdx = __shfl_xor(rdx, 32), prdy = __shfl_xor(rdy, 32), prdz = __shfl_xor(rdz, 32);
+#pragma unroll
+  for (int b = 0; b < 2; ++b) {
+    const bool own = (b == g);
+    const float xd[3] = {own ? rdx : prdx, own ? rdy : prdy, own ? rdz : prdz};
+    unsigned wd[9];
+#pragma unroll
+    for (int t = 0; t < 9; ++t) {
+      const float rev = xd[t / 3] * kf[t % 3];
+      wd[t] = Ops<T>::pack2(__builtin_amdgcn_sinf(rev), __builtin_amdgcn_cosf(rev));
+    }
+    s.q[b][0][l] = u32x4{wd[0], wd[1], wd[2], wd[3]};
+    s.q[b][1][l] = u32x4{wd[4], wd[5], wd[6], wd[7]};
+    s.w8[b][l] = wd[8];
+  }
+}
+
+// Bits 4s+d and 16+4s+d of a lane's partial ReLU mask from the rectified operand word (s, d): a half that is
+// not zero is an active unit (the rounded activation the next layer really multiplies).
+__device__ __forceinline__ unsigned relu_mask_bits(unsigned rectified, int shift) {
+  typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
+  const u16x2 one = {1, 1};
+  const u16x2 nz = __builtin_elementwise_min(__builtin_bit_cast(u16x2, rectified), one);
+  return __builtin_bit_cast(unsigned, nz) << shift;
+}
+
+// The MLP of primitive block `blk` for the pixels of `mask` (ballot of the lanes that hit).  dx, dy, dz: this
+// lane's own hit offset (inputs 3..5; lanes that did not hit pass anything finite).  o[k] = output k of THIS
+// lane's pixel, output bias included.
+// CHECK: report pre-activations outside the operand type's range.  MASKS: also return the pixel's two
+// 32-bit ReLU masks (bit u = hidden unit u active) in mk.  Returns true if a stored weight was flagged
+// non-finite when packed or (CHECK) a pre-activation of a hit pixel is out of range.
+template <typename T, bool CHECK, bool MASKS>
+__device__ __forceinline__ bool mlp_wave_mfma16(const unsigned char* __restrict__ blk, unsigned long long mask, int l,
+                                                float dx, float dy, float dz, const float kf[3], const DirWords& dir,
+                                                float o[4], unsigned mk[2]) {
+  const int g = l >> 5;
+  bool bad = false;
+  // ---- stage the primitive's weights: MFMA A fragments, straight from global memory
+  u32x4 a1[5], a2[2], a3[2];
+#pragma unroll
+  for (int s = 0; s < 5; ++s) a1[s] = *reinterpret_cast<const u32x4*>(blk + kOffW1 + s * 1024 + l * 16);
+#pragma unroll
+  for (int s = 0; s < 2; ++s) a2[s] = *reinterpret_cast<const u32x4*>(blk + kOffW2 + s * 1024 + l * 16);
+#pragma unroll
+  for (int s = 0; s < 2; ++s) {
+    // every lane loads one of the four stored rows (no divergent branch, no wait in the middle of the
+    // staging); rows 4..31 of the operand are zero
+    const u32x4 row = *reinterpret_cast<const u32x4*>(blk + kOffW3 + ((s * 2 + g) * 4 + (l & 3)) * 16);
+    const bool stored = (l & 31) < 4;
+    a3[s] = u32x4{stored ? row[0] : 0u, stored ? row[1] : 0u, stored ? row[2] : 0u, stored ? row[3] : 0u};
+  }
+  const f32x4 b3v = *reinterpret_cast<const f32x4*>(blk + kOffB3);
+  const int wflag = *reinterpret_cast<const int32_t*>(blk + kOffFlag);
+  bad |= (wflag != 0);
+
+  // ---- inputs of the column partner
+  const float pdx = __shfl_xor(dx, 32), pdy = __shfl_xor(dy, 32), pdz = __shfl_xor(dz, 32);
+  float o_blk[2][4];
+  unsigned m_blk[2][2] = {{0u, 0u}, {0u, 0u}};
+#pragma unroll
+  for (int b = 0; b < 2; ++b) {
+    const unsigned half_mask = (unsigned)(mask >> (32 * b));
+    if (half_mask != 0u) {   // wave-uniform: skip a 32-pixel block nobody hits
+      const bool own = (b == g);
+      const float xin[3] = {own ? dx : pdx, own ? dy : pdy, own ? dz : pdz};
+      const bool col_active = (half_mask >> (l & 31)) & 1u;
+      // biases are the C operand of each layer's first MFMA; an MFMA overwrites its C registers,
+      // so each column block fetches its own copy (L1-resident) instead of copying 32 registers
+      f32x16 d1, d2;
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const f32x4 v1 = *reinterpret_cast<const f32x4*>(blk + kOffB1 + g * 64 + q * 16);
+        const f32x4 v2 = *reinterpret_cast<const f32x4*>(blk + kOffB2 + g * 64 + q * 16);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          d1[4 * q + e] = v1[e];
+          d2[4 * q + e] = v2[e];
+        }
+      }
+      // layer 1: 18 (sin, cos) words per lane, 5 K-steps; words 0..8 come from LDS.  (The lane index is
+      // made opaque so that the loads stay here and are not hoisted out of the primitive loop into
+      // registers.)
+      int ll = l;
+      asm volatile("" : "+v"(ll));
+      const u32x4 dq0 = dir.q[b][0][ll], dq1 = dir.q[b][1][ll];
+      const unsigned d8 = dir.w8[b][ll];
+#pragma unroll
+      for (int s = 0; s < 5; ++s) {
+        u32x4 bw;
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+          const int t = 4 * s + d;
+          if (t < 4) {
+            bw[d] = dq0[d];
+          } else if (t < 8) {
+            bw[d] = dq1[d];
+          } else if (t == 8) {
+            bw[d] = d8;
+          } else if (t < 18) {
+            const float rev = xin[t / 3 - 3] * kf[t % 3];
+            bw[d] = Ops<T>::pack2(__builtin_amdgcn_sinf(rev), __builtin_amdgcn_cosf(rev));
+          } else {
+            bw[d] = 0u;
+          }
+        }
+        d1 = Ops<T>::mfma(a1[s], bw, d1);
+      }
+      if constexpr (CHECK) bad |= col_active && out_of_range_in<T>(d1);
+      // layer 2: the D registers, rectified and rounded, are the next B operand
+#pragma unroll
+      for (int s = 0; s < 2; ++s) {
+        u32x4 bw;
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+          bw[d] = relu_packed(Ops<T>::pack2(d1[8 * s + 2 * d], d1[8 * s + 2 * d + 1]));
+          if constexpr (MASKS) m_blk[b][0] |= relu_mask_bits(bw[d], 4 * s + d);
+        }
+        d2 = Ops<T>::mfma(a2[s], bw, d2);
+      }
+      if constexpr (CHECK) bad |= col_active && out_of_range_in<T>(d2);
+      // layer 3: rows 0..3 of a 32-row product; row k lands in register k of lane group 0
+      f32x16 d3 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int s = 0; s < 2; ++s) {
+        u32x4 bw;
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+          bw[d] = relu_packed(Ops<T>::pack2(d2[8 * s + 2 * d], d2[8 * s + 2 * d + 1]));
+          if constexpr (MASKS) m_blk[b][1] |= relu_mask_bits(bw[d], 4 * s + d);
+        }
+        d3 = Ops<T>::mfma(a3[s], bw, d3);
+      }
+#pragma unroll
+      for (int k = 0; k < 4; ++k) o_blk[b][k] = d3[k];
+    } else {
+#pragma unroll
+      for (int k = 0; k < 4; ++k) o_blk[b][k] = 0.f;
+    }
+  }
+  // pixel l < 32 reads block 0 from its own lane; pixel l >= 32 reads block 1 from lane l-32
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const float from_partner = __shfl_xor(o_blk[1][k], 32);
+    o[k] = (g ? from_partner : o_blk[0][k]) + b3v[k];
+  }
+  if constexpr (MASKS) {
+    // lane group g holds the units 8g..8g+7 and 16+8g..16+8g+7 of its column: shift into place, merge the
+    // two groups, and take the block this lane's pixel belongs to (block g)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const unsigned mine0 = m_blk[0][j] << (8 * g), mine1 = m_blk[1][j] << (8 * g);
+      const unsigned full0 = mine0 | (unsigned)__shfl_xor((int)mine0, 32);
+      const unsigned full1 = mine1 | (unsigned)__shfl_xor((int)mine1, 32);
+      mk[j] = g ? full1 : full0;
+    }
+  }
+  return bad;
+}
+
+}  // namespace mlpsp

@@ -4,26 +4,14 @@
 // activations and compositing stay f32; encoded inputs, weights and hidden activations are rounded
 // to bf16 (or fp16) and multiplied with v_mfma_f32_32x32x16 with f32 accumulation.
 //
-// Shape of the work.  One wavefront = one 8x8 tile = 64 pixels = two MFMA column blocks of 32.
-// The GEMMs are computed TRANSPOSED: D[hidden][pixel] = W[hidden][k] * X[k][pixel], i.e. the weights
-// are the A operand and the pixels are the B/N dimension.  With the 32x32x16 register layout
-//     A: lane l holds row  l%32, k = 8*(l/32) + 0..7        B: lane l holds column l%32, same k
-//     D: lane l holds column l%32, rows 8*(r/4) + 4*(l/32) + r%4 for r = 0..15
-// a lane's D registers of one layer ARE a valid B operand of the next layer (same pixel column, 8
-// k-slots per K-step) provided the next layer's weight columns are stored in that register order.
-// Weights are therefore repacked once per scene (pack kernel below) into MFMA A-fragment order with
-// the k-permutation folded in, and the chain layer1 -> ReLU -> layer2 -> ReLU -> layer3 needs no LDS,
-// no barrier and no cross-lane traffic at all.  Staging a primitive's weights is 9 coalesced 1 KiB
-// loads straight into VGPRs.
-//
-// Layer-1 k-slots: lane group g = l/32 owns frequencies 3g..3g+2 of every input component, so both
-// groups evaluate 18 (sin, cos) pairs per pixel block and each pair lands in one 32-bit operand word.
-// sin/cos use the native v_sin_f32/v_cos_f32 (argument in revolutions); their error (~1e-6) is far
-// below the bf16 rounding applied next.  (Measured alternatives that did not pay on gfx950: a 4096-entry
-// LDS sin/cos table -- same kernel time, 2x the image error; persistent wavefronts with a tile work
-// queue -- 6 % slower than one wavefront per tile.)
+// One wavefront = one 8x8 tile = 64 pixels; the MLP of a hit runs as mlp_wave_mfma16 (mlpsp_mfma16.hpp:
+// transposed GEMMs, weights as the A operand in a layout packed once per scene by the kernel below, no LDS
+// or cross-lane traffic between the layers).  (Measured alternatives that did not pay on gfx950: a
+// 4096-entry LDS sin/cos table -- same kernel time, 2x the image error; persistent wavefronts with a tile
+// work queue -- 6 % slower than one wavefront per tile.)
 #include "mlpsp_device.hpp"
 #include "mlpsp_hitrec.hpp"
+#include "mlpsp_mfma16.hpp"
 #include "mlpsp_host.hpp"
 
 // 32-channel accumulator tiles per wavefront of the feature GEMM (2 and 4 measure the same: the kernel moves
@@ -33,60 +21,6 @@
 #endif
 
 namespace mlpsp {
-
-typedef float f32x16 __attribute__((ext_vector_type(16)));
-typedef float f32x4 __attribute__((ext_vector_type(4)));
-typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
-typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
-typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
-
-// packed per-primitive block (bytes)
-constexpr int kOffW1 = 0;       // 5 K-steps x 64 lanes x 16 B
-constexpr int kOffW2 = 5120;    // 2 K-steps x 64 lanes x 16 B
-constexpr int kOffW3 = 7168;    // 2 K-steps x 2 lane groups x 4 rows x 16 B
-constexpr int kOffB1 = 7424;    // 2 lane groups x 16 f32 in D-register order
-constexpr int kOffB2 = 7552;
-constexpr int kOffB3 = 7680;    // 4 f32
-constexpr int kOffFlag = 7696;  // int32: 1 if any rounded weight or bias is non-finite
-constexpr int kPackStride = MLPSP_MFMA_PACK_BYTES;
-static_assert(kPackStride >= kOffFlag + 4 && kPackStride % 128 == 0, "pack stride");
-
-template <typename T> struct Ops;
-template <> struct Ops<__bf16> {
-  using vec8 = bf16x8;
-  static __device__ __forceinline__ unsigned pack2(float a, float b) {
-    bf16x2 v = {(__bf16)a, (__bf16)b};
-    return __builtin_bit_cast(unsigned, v);
-  }
-  static __device__ __forceinline__ f32x16 mfma(u32x4 a, u32x4 b, f32x16 c) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
-  }
-  static __device__ __forceinline__ float round_trip(float a) { return (float)(__bf16)a; }
-  static constexpr float kMax = 3.38953139e38f;
-  // bf16 has the exponent range of f32: a hidden pre-activation is out of range only if it is (within one
-  // rounding step of) +-inf.  Rounded to +inf it survives the ReLU and turns the next layer's sums into
-  // +-inf or NaN, down to the outputs, whose finiteness every hit checks; rounded to -inf the ReLU removes
-  // it, as it does in exact arithmetic.  The per-layer range check is therefore not needed for this type.
-  static constexpr bool kCheckHidden = false;
-};
-template <> struct Ops<_Float16> {
-  using vec8 = f16x8;
-  static __device__ __forceinline__ unsigned pack2(float a, float b) {
-    f16x2 v = {(_Float16)a, (_Float16)b};
-    return __builtin_bit_cast(unsigned, v);
-  }
-  static __device__ __forceinline__ f32x16 mfma(u32x4 a, u32x4 b, f32x16 c) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
-  }
-  static __device__ __forceinline__ float round_trip(float a) { return (float)(_Float16)a; }
-  static constexpr float kMax = 65504.0f;
-  static constexpr bool kCheckHidden = true;   // a finite f32 pre-activation above 65504 must be reported
-};
-
-// hidden-unit index held by D register r of lane group g
-__host__ __device__ constexpr int d_row(int r, int g) { return 8 * (r / 4) + 4 * g + (r % 4); }
 
 // ---------------------------------------------------------------------------------------------
 // pack: f32 [N,32,72] [N,32] [N,32,32] [N,32] [N,4,32] [N,4]  ->  N blocks of kPackStride bytes
@@ -100,8 +34,9 @@ __global__ __launch_bounds__(64) void pack_mfma_weights_kernel(const float* __re
   if (p >= N) return;
   const int l = threadIdx.x, m = l & 31, g = l >> 5;
   unsigned char* blk = out + (size_t)p * kPackStride;
-  const float* w1 = W1 + (size_t)p * 32 * 72 + m * 72;
-  const float* w2 = W2 + (size_t)p * 32 * 32 + m * 32;
+  // accumulator row m holds hidden unit hidden_unit_of_row(m), for both hidden layers
+  const float* w1 = W1 + (size_t)p * 32 * 72 + hidden_unit_of_row(m) * 72;
+  const float* w2 = W2 + (size_t)p * 32 * 32 + hidden_unit_of_row(m) * 32;
   bool bad = false;
   auto pk = [&](float a, float b) {
     bad |= !(__builtin_fabsf(Ops<T>::round_trip(a)) <= Ops<T>::kMax) || !(__builtin_fabsf(Ops<T>::round_trip(b)) <= Ops<T>::kMax);
@@ -123,19 +58,19 @@ __global__ __launch_bounds__(64) void pack_mfma_weights_kernel(const float* __re
   }
   for (int s = 0; s < 2; ++s) {
     u32x4 v;
-    for (int d = 0; d < 4; ++d) v[d] = pk(w2[d_row(8 * s + 2 * d, g)], w2[d_row(8 * s + 2 * d + 1, g)]);
+    for (int d = 0; d < 4; ++d) v[d] = pk(w2[hidden_unit(8 * s + 2 * d, g)], w2[hidden_unit(8 * s + 2 * d + 1, g)]);
     *reinterpret_cast<u32x4*>(blk + kOffW2 + s * 1024 + l * 16) = v;
   }
   if (l < 16) {
     const int row = l & 3, gg = (l >> 2) & 1, s = l >> 3;
     const float* w3 = W3 + (size_t)p * 4 * 32 + row * 32;
     u32x4 v;
-    for (int d = 0; d < 4; ++d) v[d] = pk(w3[d_row(8 * s + 2 * d, gg)], w3[d_row(8 * s + 2 * d + 1, gg)]);
+    for (int d = 0; d < 4; ++d) v[d] = pk(w3[hidden_unit(8 * s + 2 * d, gg)], w3[hidden_unit(8 * s + 2 * d + 1, gg)]);
     *reinterpret_cast<u32x4*>(blk + kOffW3 + ((s * 2 + gg) * 4 + row) * 16) = v;
   }
   if (l < 32) {
     const int r = l & 15, gg = l >> 4;
-    const float v1 = b1[(size_t)p * 32 + d_row(r, gg)], v2 = b2[(size_t)p * 32 + d_row(r, gg)];
+    const float v1 = b1[(size_t)p * 32 + hidden_unit(r, gg)], v2 = b2[(size_t)p * 32 + hidden_unit(r, gg)];
     bad |= !(__builtin_fabsf(v1) <= 3.4028235e38f) || !(__builtin_fabsf(v2) <= 3.4028235e38f);
     reinterpret_cast<float*>(blk + kOffB1)[gg * 16 + r] = v1;
     reinterpret_cast<float*>(blk + kOffB2)[gg * 16 + r] = v2;
@@ -152,35 +87,6 @@ __global__ __launch_bounds__(64) void pack_mfma_weights_kernel(const float* __re
 // ---------------------------------------------------------------------------------------------
 // render
 // ---------------------------------------------------------------------------------------------
-
-// True if some pre-activation is +-inf or exceeds the operand type's range.  A NaN cannot appear here
-// on its own: the operands are finite (weights are checked when packed, phases when encoded), so a
-// non-finite accumulator is an overflow, which shows as +-inf -- and the max chain sees infinities.
-// ReLU of two packed 16-bit floats in one instruction: as signed 16-bit integers every negative float
-// (and -0) is below zero and every non-negative one keeps its bits, for bf16 and fp16 alike; rounding
-// commutes with ReLU, so rounding first gives the same operand.
-__device__ __forceinline__ unsigned relu_packed(unsigned x) {
-  unsigned y;
-  asm("v_pk_max_i16 %0, %1, 0" : "=v"(y) : "v"(x));
-  return y;
-}
-__device__ __forceinline__ float max3_abs(float a, float b, float c) {
-  float y;
-  asm("v_max3_f32 %0, |%1|, |%2|, |%3|" : "=v"(y) : "v"(a), "v"(b), "v"(c));
-  return y;
-}
-// The first read of the accumulator tile is a plain C++ operation, not inline assembly: the compiler
-// inserts the wait states a matrix-core result needs before its first reader only for instructions it
-// can see, and everything below depends on that first read.
-template <typename T>
-__device__ __forceinline__ bool out_of_range_in(const f32x16& v) {
-  float m = __builtin_fabsf(v[0]);
-  m = max3_abs(m, v[1], v[2]);
-#pragma unroll
-  for (int r = 3; r < 15; r += 2) m = max3_abs(m, v[r], v[r + 1]);
-  m = max3_abs(m, v[15], v[15]);
-  return !(m <= Ops<T>::kMax);
-}
 
 // f32 activations with the native exp2/log2/rcp instructions (relative error ~1e-6, far below the
 // operand rounding of this path).  Same formulas as np_tile_kernels.cu:75-83, 2092-2103.
@@ -278,13 +184,9 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 4))) void
   // row-major order, so neighbouring tiles -- which share most primitives -- run together on one L2.
   const int tile = (blockIdx.x % kNumXcd) * per_xcd + blockIdx.x / kNumXcd;
   if (tile >= num_tiles) return;
-  const int l = threadIdx.x, g = l >> 5;
-  // per-lane phase scales, freq_f * att_f / (2 pi) revolutions per unit input: lane group g evaluates
-  // frequencies 3g, 3g+1, 3g+2
-  constexpr float kInvTwoPi = 0.159154943f;
-  const float kf0 = (freq[3 * g + 0] * att[3 * g + 0]) * kInvTwoPi;
-  const float kf1 = (freq[3 * g + 1] * att[3 * g + 1]) * kInvTwoPi;
-  const float kf2 = (freq[3 * g + 2] * att[3 * g + 2]) * kInvTwoPi;
+  const int l = threadIdx.x;
+  float kf[3];
+  phase_scales(freq, att, l >> 5, kf);
   unsigned n_proc = 0, n_proc_hit = 0, n_hits = 0;
   bool bad = false;
   const int tx = tile % ntx, ty = tile / ntx;
@@ -295,29 +197,11 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 4))) void
               roz = valid ? rays_o[pix * 3 + 2] : 0.f;
   const float rdx = valid ? rays_d[pix * 3 + 0] : 0.f, rdy = valid ? rays_d[pix * 3 + 1] : 0.f,
               rdz = valid ? rays_d[pix * 3 + 2] : 0.f;
-  // the pixel this lane shares an MFMA column with: lane l and lane l^32 both hold column l%32
-  const float prdx = __shfl_xor(rdx, 32), prdy = __shfl_xor(rdy, 32), prdz = __shfl_xor(rdz, 32);
-
   // The encoding of the ray direction (input components 0..2, operand words 0..8 of both column blocks) does
   // not depend on the primitive: it is computed once per pixel and parked in LDS in operand form -- 18 more
   // live registers would cost the fourth wavefront per SIMD.  One wavefront per workgroup: no barrier.
-  __shared__ u32x4 s_dirq[2][2][64];
-  __shared__ unsigned s_dir8[2][64];
-#pragma unroll
-  for (int b = 0; b < 2; ++b) {
-    const bool own = (b == g);
-    const float xd[3] = {own ? rdx : prdx, own ? rdy : prdy, own ? rdz : prdz};
-    unsigned wd[9];
-#pragma unroll
-    for (int t = 0; t < 9; ++t) {
-      const float kf = (t % 3 == 0) ? kf0 : ((t % 3 == 1) ? kf1 : kf2);
-      const float rev = xd[t / 3] * kf;
-      wd[t] = Ops<T>::pack2(__builtin_amdgcn_sinf(rev), __builtin_amdgcn_cosf(rev));
-    }
-    s_dirq[b][0][l] = u32x4{wd[0], wd[1], wd[2], wd[3]};
-    s_dirq[b][1][l] = u32x4{wd[4], wd[5], wd[6], wd[7]};
-    s_dir8[b][l] = wd[8];
-  }
+  __shared__ DirWords s_dir;
+  encode_direction_words<T>(rdx, rdy, rdz, kf, l, s_dir);
 
   const int start = offsets[tile], end = offsets[tile + 1];
   PixelAcc acc = {0.f, 0.f, 0.f, 1.f, 0.f, 0.f};
@@ -343,112 +227,9 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 4))) void
       ++n_proc_hit;
       n_hits += __popcll(mask);
       const unsigned char* __restrict__ blk = packed + (size_t)p * kPackStride;
-      // ---- stage the primitive's weights: MFMA A fragments, straight from global memory
-      u32x4 a1[5], a2[2], a3[2];
-#pragma unroll
-      for (int s = 0; s < 5; ++s) a1[s] = *reinterpret_cast<const u32x4*>(blk + kOffW1 + s * 1024 + l * 16);
-#pragma unroll
-      for (int s = 0; s < 2; ++s) a2[s] = *reinterpret_cast<const u32x4*>(blk + kOffW2 + s * 1024 + l * 16);
-#pragma unroll
-      for (int s = 0; s < 2; ++s) {
-        // every lane loads one of the four stored rows (no divergent branch, no wait in the middle of the
-        // staging); rows 4..31 of the operand are zero
-        const u32x4 row = *reinterpret_cast<const u32x4*>(blk + kOffW3 + ((s * 2 + g) * 4 + (l & 3)) * 16);
-        const bool stored = (l & 31) < 4;
-        a3[s] = u32x4{stored ? row[0] : 0u, stored ? row[1] : 0u, stored ? row[2] : 0u, stored ? row[3] : 0u};
-      }
-      const f32x4 b3v = *reinterpret_cast<const f32x4*>(blk + kOffB3);
-      const int wflag = *reinterpret_cast<const int32_t*>(blk + kOffFlag);
-      bad |= (wflag != 0);
       bad |= hit && !(__builtin_fabsf((h.dx + h.dy) + h.dz) <= 3.4028235e38f);
-
-      // ---- inputs of the column partner
-      const float pdx = __shfl_xor(h.dx, 32), pdy = __shfl_xor(h.dy, 32), pdz = __shfl_xor(h.dz, 32);
-      float o_blk[2][4];
-#pragma unroll
-      for (int b = 0; b < 2; ++b) {
-        const unsigned half_mask = (unsigned)(mask >> (32 * b));
-        if (half_mask != 0u) {   // wave-uniform: skip a 32-pixel block nobody hits
-          const bool own = (b == g);
-          const float xin[3] = {own ? h.dx : pdx, own ? h.dy : pdy, own ? h.dz : pdz};
-          const bool col_active = (half_mask >> (l & 31)) & 1u;
-          // biases are the C operand of each layer's first MFMA; an MFMA overwrites its C registers,
-          // so each column block fetches its own copy (L1-resident) instead of copying 32 registers
-          f32x16 d1, d2;
-#pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            const f32x4 v1 = *reinterpret_cast<const f32x4*>(blk + kOffB1 + g * 64 + q * 16);
-            const f32x4 v2 = *reinterpret_cast<const f32x4*>(blk + kOffB2 + g * 64 + q * 16);
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-              d1[4 * q + e] = v1[e];
-              d2[4 * q + e] = v2[e];
-            }
-          }
-          // layer 1: 18 (sin, cos) words per lane, 5 K-steps; words 0..8 come from LDS.  (The lane index is
-          // made opaque so that the loads stay here and are not hoisted out of the primitive loop into
-          // registers.)
-          int ll = l;
-          asm volatile("" : "+v"(ll));
-          const u32x4 dq0 = s_dirq[b][0][ll], dq1 = s_dirq[b][1][ll];
-          const unsigned d8 = s_dir8[b][ll];
-#pragma unroll
-          for (int s = 0; s < 5; ++s) {
-            u32x4 bw;
-#pragma unroll
-            for (int d = 0; d < 4; ++d) {
-              const int t = 4 * s + d;
-              if (t < 4) {
-                bw[d] = dq0[d];
-              } else if (t < 8) {
-                bw[d] = dq1[d];
-              } else if (t == 8) {
-                bw[d] = d8;
-              } else if (t < 18) {
-                const float kf = (t % 3 == 0) ? kf0 : ((t % 3 == 1) ? kf1 : kf2);
-                const float rev = xin[t / 3 - 3] * kf;
-                bw[d] = Ops<T>::pack2(__builtin_amdgcn_sinf(rev), __builtin_amdgcn_cosf(rev));
-              } else {
-                bw[d] = 0u;
-              }
-            }
-            d1 = Ops<T>::mfma(a1[s], bw, d1);
-          }
-          if constexpr (Ops<T>::kCheckHidden) bad |= col_active && out_of_range_in<T>(d1);
-          // layer 2: the D registers, rectified and rounded, are the next B operand
-#pragma unroll
-          for (int s = 0; s < 2; ++s) {
-            u32x4 bw;
-#pragma unroll
-            for (int d = 0; d < 4; ++d)
-              bw[d] = relu_packed(Ops<T>::pack2(d1[8 * s + 2 * d], d1[8 * s + 2 * d + 1]));
-            d2 = Ops<T>::mfma(a2[s], bw, d2);
-          }
-          if constexpr (Ops<T>::kCheckHidden) bad |= col_active && out_of_range_in<T>(d2);
-          // layer 3: rows 0..3 of a 32-row product; row k lands in register k of lane group 0
-          f32x16 d3 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-          for (int s = 0; s < 2; ++s) {
-            u32x4 bw;
-#pragma unroll
-            for (int d = 0; d < 4; ++d)
-              bw[d] = relu_packed(Ops<T>::pack2(d2[8 * s + 2 * d], d2[8 * s + 2 * d + 1]));
-            d3 = Ops<T>::mfma(a3[s], bw, d3);
-          }
-#pragma unroll
-          for (int k = 0; k < 4; ++k) o_blk[b][k] = d3[k];
-        } else {
-#pragma unroll
-          for (int k = 0; k < 4; ++k) o_blk[b][k] = 0.f;
-        }
-      }
-      // pixel l < 32 reads block 0 from its own lane; pixel l >= 32 reads block 1 from lane l-32
       float o[4];
-#pragma unroll
-      for (int k = 0; k < 4; ++k) {
-        const float from_partner = __shfl_xor(o_blk[1][k], 32);
-        o[k] = (g ? from_partner : o_blk[0][k]) + b3v[k];
-      }
+      bad |= mlp_wave_mfma16<T, Ops<T>::kCheckHidden, false>(blk, mask, l, h.dx, h.dy, h.dz, kf, s_dir, o, nullptr);
       float w = 0.f;
       if (hit) {
         bad |= !(__builtin_fabsf(o[0]) <= 3.4028235e38f) || !(__builtin_fabsf(o[1]) <= 3.4028235e38f) ||

@@ -1,4 +1,4 @@
-"""Scene module with the Python-facing API of the reference's ``scannet/cumodel.py``, forward only.
+"""Scene module with the Python-facing API of the reference's ``scannet/cumodel.py``.
 
 Same module-level names (``_tile_ext``, ``_tile_ext_key``, ``_tile_ext_build_config``, the two
 encodings, ``_encode_x6``, ``_mlp_forward_indexed``) and the same class
@@ -8,8 +8,9 @@ harness, a test that monkeypatches ``_tile_ext`` -- runs against this one.  What
 the API: culling is the sparse HIP binning instead of a dense [tiles x primitives] tensor
 expression, and the extension object is ``tile_ext.TileExt`` on ``libmlpsp_hip.so``.
 
-Training (autograd backward, record emission) is outside this build: ``forward`` returns tensors
-without a graph.
+``forward`` renders without a graph under ``torch.no_grad()``; in grad mode with parameters that require
+grad it goes through ``_TileRenderAutogradFn`` (RGB) or, with a feature target, through the record-based
+training step of ``csr_training``.  The dense feature-image backward of the reference is not provided.
 """
 from __future__ import annotations
 

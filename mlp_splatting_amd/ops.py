@@ -246,6 +246,55 @@ def training_records(rays_o, rays_d, records, order, tile_offsets, freq, att, W1
     return rgb, alpha, ids, x6, raw, masks, gates, offsets
 
 
+def all_finite_flag(tensors):
+    """int32 device flag [1]: 1 if any element of the float32 tensors (at most 16, one device) is NaN or infinite.
+    One fused scan; reading the flag is the caller's (single) synchronisation."""
+    tensors = [t for t in tensors if t.numel()]
+    dev = tensors[0].device if tensors else torch.device("cuda", torch.cuda.current_device())
+    flag = torch.empty(1, dtype=torch.int32, device=dev)
+    for t in tensors:
+        if not (t.is_cuda and t.dtype == torch.float32 and t.is_contiguous() and t.device == dev):
+            raise RuntimeError("all_finite_flag expects contiguous float32 CUDA tensors on one device")
+    pointers = (C.c_void_p * max(len(tensors), 1))(*[t.data_ptr() for t in tensors])
+    lengths = (C.c_int64 * max(len(tensors), 1))(*[t.numel() for t in tensors])
+    _check(_lib.load().mlpsp_all_finite(pointers, lengths, len(tensors), _ptr(flag), _stream(dev)), "mlpsp_all_finite")
+    return flag
+
+
+def training_records_mfma(rays_o, rays_d, records, order, tile_offsets, freq, att, packed, n, W, H, threshold, beta,
+                          temp, max_hits, bf16):
+    """Matrix-core training-records forward -> (status bits, (rgb, alpha, ids, x6, raw, masks, gates, offsets) or
+    None).  Bits: 1 numeric, 2 hit capacity, 4 count/emit disagreement (training_wmma.cuh:21-22); the policy --
+    retry in f32, raise -- is the caller's.  A non-zero status after the count step skips the emit step."""
+    dev = rays_o.device
+    lib = _lib.load()
+    B = W * H
+    counts = torch.zeros(B, dtype=torch.int32, device=dev)
+    status = torch.zeros(1, dtype=torch.int32, device=dev)
+    head = (_ptr(rays_o), _ptr(rays_d), _ptr(records), _ptr(order), _ptr(tile_offsets), _ptr(freq), _ptr(att),
+            _ptr(packed), int(n), W, H, float(threshold), int(max_hits), 1 if bf16 else 0)
+    _check(lib.mlpsp_records_mfma_count(*head, _ptr(counts), _ptr(status), _stream(dev)), "mlpsp_records_mfma_count")
+    offsets = torch.zeros(B + 1, dtype=torch.int64, device=dev)
+    torch.cumsum(counts, 0, out=offsets[1:])
+    total, bits = torch.cat([offsets[-1:], status.to(torch.int64)]).tolist()
+    if bits:
+        return int(bits), None
+    if not 0 <= total <= B * int(max_hits):
+        raise RuntimeError("Training WMMA count total is outside the bounded allocation contract")
+    ids = torch.empty(total, dtype=torch.int32, device=dev)
+    x6 = torch.empty(total, 6, dtype=torch.float32, device=dev)
+    masks = torch.empty(total, 2, dtype=torch.int32, device=dev)
+    raw = torch.empty(total, 8, dtype=torch.float32, device=dev)
+    gates = torch.empty(total, 4, dtype=torch.float32, device=dev)
+    rgb = torch.zeros(B, 3, dtype=torch.float32, device=dev)
+    alpha = torch.zeros(B, 1, dtype=torch.float32, device=dev)
+    # launched for an empty record set too: the emit step then checks that every pixel's count is zero
+    _check(lib.mlpsp_records_mfma_emit(*head, float(beta), float(temp), _ptr(offsets), int(total), _ptr(ids), _ptr(x6),
+                                       _ptr(masks), _ptr(raw), _ptr(gates), _ptr(rgb), _ptr(alpha), _ptr(status),
+                                       _stream(dev)), "mlpsp_records_mfma_emit")
+    return int(status.item()), (rgb, alpha, ids, x6, raw, masks, gates, offsets)
+
+
 def _feat_shape(feat_attr):
     """(slots, channels) with the reference's checks (np_tile_kernels.cu:6158-6169)."""
     if not (feat_attr.is_cuda and feat_attr.dtype == torch.float32 and feat_attr.dim() in (2, 3)):

@@ -3,8 +3,9 @@ error texts as the reference's pybind11 module (scannet/cuda/np_tile_kernels.cu:
 forward entry points), implemented on the C ABI of ``libmlpsp_hip.so``.
 
 ``TileExt()`` is what ``cumodel._ensure_tile_ext_static()`` returns and what a test installs with
-``monkeypatch.setattr(cumodel, "_tile_ext", ...)``.  Entry points that belong to the reference's
-training/backward side are not provided; calling one raises ``NotImplementedError`` naming it.
+``monkeypatch.setattr(cumodel, "_tile_ext", ...)``.  The entry points of the reference's fused backward
+kernels that are not provided raise ``NotImplementedError`` naming them; the record pipeline (records forward in
+f32 or on the matrix cores, reverse compositing, grouped gradients) is.
 """
 from __future__ import annotations
 
@@ -23,9 +24,9 @@ _BACKWARD_ONLY = (
     "render_tiles_backward_emit_per_pixel", "render_tiles_backward_emit_tilecenter",
     "render_tiles_backward_featattr_per_pixel", "render_tiles_backward_featattr_tilecenter",
     "render_tiles_backward_tilecenter_full_with_feat",
-    "render_tiles_mlp_records", "render_tiles_training_records_wmma",
+    "render_tiles_mlp_records",
     "render_tiles_backward_tilecenter_traversal",
-    "render_tiles_backward_tilecenter_backprop_noatomic", "training_wmma_safety_stats",
+    "render_tiles_backward_tilecenter_backprop_noatomic",
 )
 
 
@@ -48,6 +49,7 @@ class TileExt:
         self._lock = threading.Lock()
         self._mfma_calls = 0
         self._mfma_fallbacks = 0
+        self._training_mfma_stats = [0, 0, 0, 0, 0]
         self._pack_key = None
         self._pack = None
         self._feat_pack_key = None
@@ -61,7 +63,7 @@ class TileExt:
     def __getattr__(self, name):
         if name in _BACKWARD_ONLY:
             def _missing(*_a, **_k):
-                raise NotImplementedError(f"{name} belongs to the training/backward path, which this build does not provide")
+                raise NotImplementedError(f"{name} is one of the reference's fused backward entry points, which this build does not provide")
             return _missing
         raise AttributeError(name)
 
@@ -351,6 +353,80 @@ class TileExt:
                                           self.max_tile_prims, cull_threshold=float(threshold))
             return list(ops.training_records(x[0], x[1], rec, order, x[6], x[7], x[8], *x[9:15], width, height, tile,
                                              tile, float(threshold), float(beta), float(temp), self.max_hits, name))
+
+    def training_wmma_safety_stats(self):
+        """[calls, frame_fallbacks, fp32_nonfinite_failures, count_emit_failures, capacity_failures] of
+        :meth:`render_tiles_training_records_wmma` since this object was made (training_wmma.cuh:7-19: calls
+        are accepted count-pass launches; rejected arguments and candidate lists are not counted)."""
+        with self._lock:
+            return list(self._training_mfma_stats)
+
+    def _count_training_mfma(self, index):
+        with self._lock:
+            self._training_mfma_stats[index] += 1
+
+    def render_tiles_training_records_wmma(self, x, width, height, tile, threshold, beta, temp, precision):
+        """The records of :meth:`render_tiles_training_records` with the MLP on the matrix cores in ``precision``
+        ("float16" or "bfloat16") and everything else in the same f32 expressions (wrapper and policy of
+        training_wmma.cuh:267-357): non-finite inputs are refused, a numeric overflow of the reduced-precision
+        pass discards it and repeats the whole frame with the scalar f32 record forward, hit capacity and a
+        count/emit disagreement raise."""
+        import math
+        _chk(len(x) == 17, "Training WMMA requires 15 scene inputs and two RGB/T adjoint placeholders")
+        _chk(int(tile) == 8, "Training WMMA requires tile8")
+        _chk(precision in ("float16", "bfloat16"), "Training WMMA precision must be float16 or bfloat16")
+        width, height = int(width), int(height)
+        _chk(0 < width <= 2147483647 and 0 < height <= 2147483647 and width <= 2147483647 // height,
+             "Training WMMA image dimensions exceed int32 pixel indexing")
+        thr32 = torch.tensor(float(threshold), dtype=torch.float32).item()
+        _chk(math.isfinite(threshold) and 0.0 < thr32 < 1.0,
+             "Training WMMA threshold must remain in (0,1) after FP32 conversion")
+        for v in (beta, temp):
+            _chk(math.isfinite(v) and math.isfinite(torch.tensor(float(v), dtype=torch.float32).item()),
+                 "Training WMMA gating parameters must be finite FP32 values")
+        for i, t in enumerate(x):
+            _chk(t.is_cuda and t.is_contiguous() and t.device == x[0].device,
+                 "Training WMMA inputs must be contiguous CUDA tensors on one device")
+            _chk(t.dtype == (torch.int32 if i in (5, 6) else torch.float32),
+                 "Training WMMA requires FP32 inputs and int32 tile lists")
+        pixels, n = width * height, x[2].shape[0] if x[2].dim() == 2 else -1
+        _chk(tuple(x[0].shape) == (pixels, 3) and x[1].shape == x[0].shape)
+        _chk(x[2].dim() == 2 and x[2].shape[1] == 3 and x[3].shape == x[2].shape and tuple(x[4].shape) == (n, 4))
+        _chk(x[7].dim() == 1 and x[7].numel() == 6 and x[8].shape == x[7].shape)
+        _chk(tuple(x[9].shape) == (n, 32, 72) and tuple(x[10].shape) == (n, 32) and tuple(x[11].shape) == (n, 32, 32))
+        _chk(x[12].shape == x[10].shape and tuple(x[13].shape) == (n, 4, 32) and tuple(x[14].shape) == (n, 4))
+        _chk(x[15].shape == x[0].shape and x[16].dim() == 1 and x[16].numel() == pixels)
+        name = "render_tiles_training_records_wmma"
+        with torch.cuda.device(x[0].device):
+            self._validate(x[5], x[6], ops.num_tiles(width, height, 8, 8), self.max_tile_prims, n, name)
+            nonfinite = ops.all_finite_flag([t for i, t in enumerate(x) if i not in (5, 6)])
+            _chk(int(nonfinite.item()) == 0, "Training WMMA input is nonfinite; refusing unsafe forward/fallback")
+            self._count_training_mfma(0)
+            bf16 = precision == "bfloat16"
+            rec = self._records(x[2], x[3], x[4])
+            order = x[5]
+            if x[5].numel() > 0:
+                order, _ = ops.sort_tiles(x[0], x[1], rec, x[5], x[6], width, height, 8, 8, _lib.KEY_TSTAR,
+                                          self.max_tile_prims, cull_threshold=float(threshold))
+            packed = self._packed_weights(list(x[9:15]), bf16)
+            bits, records = ops.training_records_mfma(x[0], x[1], rec, order, x[6], x[7], x[8], packed, n, width, height,
+                                                      float(threshold), float(beta), float(temp), self.max_hits, bf16)
+            if bits & 2:
+                self._count_training_mfma(4)
+                raise RuntimeError(f"Training WMMA hit capacity {self.max_hits} exceeded; refusing truncated records")
+            if bits & 4:
+                self._count_training_mfma(3)
+                raise RuntimeError("Training WMMA count/emit mismatch; bounded partial records were discarded")
+            if bits & 1:
+                self._count_training_mfma(1)
+                warnings.warn("Training WMMA numeric overflow: discarding both mixed passes and rerunning the whole "
+                              "FP32 record forward")
+                del records
+                records = self.render_tiles_training_records(x, width, height, 8, threshold, beta, temp)
+                if int(ops.all_finite_flag([t for t in records if t.is_floating_point()]).item()):
+                    self._count_training_mfma(2)
+                    raise RuntimeError("Training WMMA scalar FP32 fallback records are nonfinite")
+            return list(records)
 
     def primitive_records_reverse(self, ids, offsets, x6, raw, logs, quats, grgb, gt):
         """[d4, grad_positions, grad_log_scales, grad_quats] from saved forward records
