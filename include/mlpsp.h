@@ -321,9 +321,21 @@ int mlpsp_grouped_vjp(const float* x6_dev, const float* grad4_dev, const int32_t
 
 /* Sum of every primitive's segments = _reduce_partials (scannet/primitive_gemm.py:169-183): out_dev
  * [num_primitives, 3524] = sum over g in [group_offsets[p], group_offsets[p+1]) of partial_dev[g];
- * nonfinite_dev[0] is cleared and then set to 1 if any sum is NaN or infinite. */
-int mlpsp_reduce_partials(const float* partial_dev, const int64_t* group_offsets_dev, int num_primitives,
-                          float* out_dev, int32_t* nonfinite_dev, mlpsp_stream_t stream);
+ * nonfinite_dev[0] is cleared and then set to 1 if any sum is NaN or infinite.  The sums are formed by chunks of
+ * 32 consecutive segments and then per primitive (a fixed tree, so the result does not depend on scheduling),
+ * which needs scratch rows behind the partial sums: partial_dev holds mlpsp_segment_reduce_rows(num_groups) rows
+ * of 3524 floats, of which mlpsp_grouped_vjp fills the first num_groups.  group_primitives_dev as there. */
+int64_t mlpsp_segment_reduce_rows(int64_t num_groups);
+int mlpsp_reduce_partials(const float* partial_dev, const int64_t* group_primitives_dev,
+                          const int64_t* group_offsets_dev, int64_t num_groups, int num_primitives, float* out_dev,
+                          int32_t* nonfinite_dev, mlpsp_stream_t stream);
+/* The same sums written straight into the six gradient tensors [N,32,72] [N,32] [N,32,32] [N,32] [N,4,32] [N,4]
+ * (the reference splits and copies the packed rows afterwards, scannet/primitive_gemm.py:279); all 16-byte
+ * aligned. */
+int mlpsp_reduce_partials_split(const float* partial_dev, const int64_t* group_primitives_dev,
+                                const int64_t* group_offsets_dev, int64_t num_groups, int num_primitives,
+                                float* gW1_dev, float* gb1_dev, float* gW2_dev, float* gb2_dev, float* gW3_dev,
+                                float* gb3_dev, int32_t* nonfinite_dev, mlpsp_stream_t stream);
 
 /* Reverse compositing over saved forward records = primitive_records_reverse_kernel
  * (scannet/cuda/primitive_records.cuh:3-46; argument checks of its wrapper :48-74 are the caller's).
@@ -377,7 +389,8 @@ int mlpsp_stream_feature_l1(const int32_t* ids_dev, const int64_t* pixel_offsets
  * (scannet/record_feature_loss.py:114-185).  Records in primitive-major order: record_indices [R] (int64) maps a
  * row of the CSR (csr_offsets [N+1]) to its record, record_pixels [R] (int32) gives a record's pixel; segments as
  * for mlpsp_grouped_vjp.  mixed != 0 rounds both factors of every product to fp16 (f32 accumulation).
- * partial_dev [num_groups, slots, channels] is scratch, out_dev [N, slots, channels] the result. */
+ * partial_dev [mlpsp_segment_reduce_rows(num_groups), slots, channels] is scratch (per-segment sums, then the
+ * chunk sums of the per-primitive reduction), out_dev [N, slots, channels] the result. */
 int mlpsp_feature_attribute_gradients(const int8_t* signs_dev, const int64_t* record_indices_dev,
                                       const int32_t* record_pixels_dev, const float* raw_dev, const float* gates_dev,
                                       const int64_t* csr_offsets_dev, const int64_t* group_primitives_dev,

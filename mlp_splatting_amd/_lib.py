@@ -64,7 +64,9 @@ SIGNATURES = {
     "mlpsp_probe_issue": (_i, [_i, _i, _vp, _vp]),
     "mlpsp_grouped_vjp": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _f, _i, _vp,
                                _vp]),
-    "mlpsp_reduce_partials": (_i, [_vp, _vp, _i, _vp, _vp, _vp]),
+    "mlpsp_segment_reduce_rows": (_i64, [_i64]),
+    "mlpsp_reduce_partials": (_i, [_vp, _vp, _vp, _i64, _i, _vp, _vp, _vp]),
+    "mlpsp_reduce_partials_split": (_i, [_vp, _vp, _vp, _i64, _i] + [_vp] * 8),
     "mlpsp_stream_feature_l1": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp]),
     "mlpsp_feature_attribute_gradients": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i, _i, _i, _i, _i, _i,
                                                _i, _i, _i, _vp, _vp, _vp]),

@@ -6,6 +6,7 @@
 // of this loss (:5).
 #include "mlpsp_device.hpp"
 #include "mlpsp_host.hpp"
+#include "mlpsp_segment_reduce.hpp"
 
 namespace mlpsp {
 
@@ -190,18 +191,6 @@ __global__ __launch_bounds__(64) void feature_vjp_kernel(const int8_t* __restric
       if (c0 + k < C) partial[(group * SLOTS + s) * C + c0 + k] = accum[s][k] / norm;
 }
 
-// out[p][k] = sum over the primitive's segments (_feature_reduce, :152-161)
-__global__ __launch_bounds__(256) void feature_reduce_kernel(const float* __restrict__ partial,
-                                                             const long long* __restrict__ group_offsets,
-                                                             float* __restrict__ out, long long params) {
-  const long long p = blockIdx.x;
-  const long long k = (long long)blockIdx.y * 256 + threadIdx.x;
-  if (k >= params) return;
-  float acc = 0.f;
-  for (long long g = group_offsets[p]; g < group_offsets[p + 1]; ++g) acc += partial[g * params + k];
-  out[p * params + k] = acc;
-}
-
 }  // namespace mlpsp
 
 using namespace mlpsp;
@@ -274,13 +263,13 @@ MLPSP_API int mlpsp_feature_attribute_gradients(const int8_t* signs_dev, const i
 #undef MLPSP_FV_LAUNCH
     MLPSP_LAUNCH_CHECK();
   }
+  // out[p] = sum over the primitive's segments (_feature_reduce, :152-161)
   if (num_primitives > 0) {
-    if (!group_offsets_dev || !out_dev) return MLPSP_E_ARGUMENT;
-    const long long params = (long long)slots * channels;
-    const dim3 grid((unsigned)num_primitives, (unsigned)((params + 255) / 256)), block(256);
-    hipLaunchKernelGGL(feature_reduce_kernel, grid, block, 0, s, partial_dev, (const long long*)group_offsets_dev,
-                       out_dev, params);
-    MLPSP_LAUNCH_CHECK();
+    ReduceDest dest{};
+    dest.packed = out_dev;
+    const int rc = segment_reduce<false>(partial_dev, group_primitives_dev, group_offsets_dev, num_groups, num_primitives,
+                                         (int64_t)slots * channels, dest, nullptr, s);
+    if (rc != MLPSP_OK) return rc;
   }
   return MLPSP_OK;
 }

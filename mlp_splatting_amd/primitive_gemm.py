@@ -123,18 +123,23 @@ def resolve_groups(csr, segment_size=512, groups=None):
 _PRECISION_CODE = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
 
 
-def _launch_grouped_vjp(csr, freq, attenuation, weights, groups, dtype, block_size, scale):
+def _launch_grouped_vjp(csr, freq, attenuation, weights, groups, dtype, block_size, scale, split=False):
     """(result [n,3524] f32, nonfinite flag [1] int32): per-segment partial gradients, then their sum per
     primitive (scannet/primitive_gemm.py:214-230).  ``block_size`` only chose the Triton tile height; the
-    HIP kernel always walks a segment in blocks of 32 records."""
+    HIP kernel always walks a segment in blocks of 32 records.  ``split``: the result is the list of the six
+    gradient tensors, written in place by the summing kernel instead of being cut out of packed rows."""
     from . import _lib
     lib = _lib.load()
     group_primitives, group_starts, group_offsets = groups
     device = weights[0].device
     n = len(weights[0])
     num_groups = int(group_primitives.numel())
-    partial = torch.empty((max(num_groups, 1), sum(PACKED_GRADIENT_SIZES)), dtype=torch.float32, device=device)
-    result = torch.empty((n, sum(PACKED_GRADIENT_SIZES)), dtype=torch.float32, device=device)
+    partial = torch.empty((max(int(lib.mlpsp_segment_reduce_rows(num_groups)), 1), sum(PACKED_GRADIENT_SIZES)),
+                          dtype=torch.float32, device=device)       # per-segment sums + the reduction's chunk sums
+    if split:
+        result = [torch.empty_like(w) for w in weights]
+    else:
+        result = torch.empty((n, sum(PACKED_GRADIENT_SIZES)), dtype=torch.float32, device=device)
     flag = torch.zeros(1, dtype=torch.int32, device=device)
     stream = torch.cuda.current_stream(device).cuda_stream
     masks = csr.relu_masks
@@ -146,8 +151,12 @@ def _launch_grouped_vjp(csr, freq, attenuation, weights, groups, dtype, block_si
                                    stream)
         if rc != 0:
             raise RuntimeError(f"mlpsp_grouped_vjp: {_lib.strerror(rc)}")
-        rc = lib.mlpsp_reduce_partials(partial.data_ptr(), group_offsets.data_ptr(), n, result.data_ptr(),
-                                       flag.data_ptr(), stream)
+        if split:
+            rc = lib.mlpsp_reduce_partials_split(partial.data_ptr(), group_primitives.data_ptr(), group_offsets.data_ptr(),
+                                                 num_groups, n, *[r.data_ptr() for r in result], flag.data_ptr(), stream)
+        else:
+            rc = lib.mlpsp_reduce_partials(partial.data_ptr(), group_primitives.data_ptr(), group_offsets.data_ptr(),
+                                           num_groups, n, result.data_ptr(), flag.data_ptr(), stream)
         if rc != 0:
             raise RuntimeError(f"mlpsp_reduce_partials: {_lib.strerror(rc)}")
     return result, flag
@@ -189,7 +198,7 @@ def grouped_weight_gradients(csr, freq, attenuation, weights, *, dtype=torch.flo
         raise ValueError("loss_scale must be finite and strictly positive")
 
     def launch(operand_dtype, operand_scale):
-        return _launch_grouped_vjp(csr, freq, attenuation, weights, groups, operand_dtype, block_size, operand_scale)
+        return _launch_grouped_vjp(csr, freq, attenuation, weights, groups, operand_dtype, block_size, operand_scale,
+                                   split=True)
 
-    flat = _checked_grouped_vjp(launch, dtype, scale)
-    return [part.reshape(w.shape).contiguous() for part, w in zip(flat.split(list(PACKED_GRADIENT_SIZES), dim=1), weights)]
+    return _checked_grouped_vjp(launch, dtype, scale)

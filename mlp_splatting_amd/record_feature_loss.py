@@ -65,7 +65,8 @@ def feature_weight_gradients(records, csr, signs, attributes, width, height, *, 
     device = ids.device
     pixels = torch.repeat_interleave(torch.arange(width * height, device=device, dtype=torch.int32),
                                      pixel_offsets.diff(), output_size=len(ids))
-    partial = torch.empty((max(len(primitives), 1), slots, channels), device=device, dtype=torch.float32)
+    rows = int(_lib.load().mlpsp_segment_reduce_rows(len(primitives)))      # per-segment sums + the reduction's chunk sums
+    partial = torch.empty((max(rows, 1), slots, channels), device=device, dtype=torch.float32)
     result = torch.empty_like(attributes)
     with torch.cuda.device(device):
         rc = _lib.load().mlpsp_feature_attribute_gradients(

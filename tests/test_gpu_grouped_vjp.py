@@ -186,3 +186,44 @@ def test_c_abi_rejects_bad_arguments(device):
     assert ok(groups=-1) != 0
     assert ok(groups=0) == 0
     torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("counts", [
+    [0, 1, 31, 32, 33, 0, 64, 100, 1, 0],          # runs that start/end on, before and after chunk boundaries
+    [32, 32, 32],                                  # every primitive is exactly one chunk
+    [5] * 40,                                      # several whole primitives per chunk, some straddling
+    [0, 0, 700, 0, 3],                             # one primitive over 22 chunks
+    [0, 0, 0],                                     # no segment at all
+    [1],
+])
+def test_segment_sums_per_primitive(device, counts):
+    """mlpsp_reduce_partials / _split: chunked two-pass sums against a float64 index_add, and the non-finite flag."""
+    from mlp_splatting_amd import _lib
+    lib = _lib.load()
+    n, total = len(counts), sum(counts)
+    counts_t = torch.tensor(counts, dtype=torch.int64, device=device)
+    owners = torch.repeat_interleave(torch.arange(n, device=device), counts_t)
+    offsets = torch.cat((counts_t.new_zeros(1), counts_t.cumsum(0)))
+    rows = int(lib.mlpsp_segment_reduce_rows(total))
+    assert rows == total + 2 * ((total + 31) // 32)
+    torch.manual_seed(len(counts) + total)
+    partial = torch.full((max(rows, 1), 3524), float("nan"), device=device)       # the scratch rows start as garbage
+    partial[:total] = torch.randn(total, 3524, device=device)
+    expected = torch.zeros(n, 3524, dtype=torch.float64, device=device).index_add_(0, owners, partial[:total].double())
+    stream = torch.cuda.current_stream(device).cuda_stream
+    packed = torch.full((n, 3524), float("nan"), device=device)
+    flag = torch.ones(1, dtype=torch.int32, device=device)
+    assert lib.mlpsp_reduce_partials(partial.data_ptr(), owners.data_ptr(), offsets.data_ptr(), total, n, packed.data_ptr(),
+                                     flag.data_ptr(), stream) == 0
+    assert int(flag) == 0
+    torch.testing.assert_close(packed.double(), expected, atol=2e-5, rtol=1e-5)
+    parts = [torch.full((n, *shape), float("nan"), device=device) for shape in SHAPES]
+    assert lib.mlpsp_reduce_partials_split(partial.data_ptr(), owners.data_ptr(), offsets.data_ptr(), total, n,
+                                           *[t.data_ptr() for t in parts], flag.data_ptr(), stream) == 0
+    assert int(flag) == 0
+    assert torch.equal(torch.cat([t.reshape(n, -1) for t in parts], dim=1), packed)
+    if total:
+        partial[total // 2, 1234] = float("inf")
+        assert lib.mlpsp_reduce_partials(partial.data_ptr(), owners.data_ptr(), offsets.data_ptr(), total, n,
+                                         packed.data_ptr(), flag.data_ptr(), stream) == 0
+        assert int(flag) == 1
