@@ -187,6 +187,13 @@ def _add_background(rgb, alpha, bg):
     return rgb + (1.0 - alpha).clamp(0.0, 1.0) * bg.view(1, 3)
 
 
+def _uncached(ext):
+    """``ext.uncached()`` where the extension object has derived-tensor caches (``tile_ext.TileExt``), else nothing."""
+    import contextlib
+    manager = getattr(ext, "uncached", None)
+    return manager() if callable(manager) else contextlib.nullcontext()
+
+
 class _TileRenderAutogradFn(torch.autograd.Function):
     """RGB render with gradients for geometry and MLP weights (scannet/cumodel.py:219-378).  The forward is the
     ordinary f32 render; the backward re-traverses the frame (``render_tiles_backward_tilecenter_full``)."""
@@ -198,12 +205,14 @@ class _TileRenderAutogradFn(torch.autograd.Function):
         args = (rays_o, rays_d, positions, log_scales, quats, culled_prim_indices, tile_offsets, freq, att,
                 W1, b1, W2, b2, W3, b3)
         dims = (int(Wimg), int(Himg), int(TW), int(TH), float(threshold))
-        if mode == 0:
-            rgb, alpha = ext.render_tiles_forward(*args, *dims)
-        elif mode == 1:
-            rgb, alpha = ext.render_tiles_forward_tilecenter(*args, *dims)
-        else:
-            raise ValueError("Unsupported tile mode for backward")
+        # a training step: nothing derived from the parameters may be reused from, or kept for, another call
+        with _uncached(ext):
+            if mode == 0:
+                rgb, alpha = ext.render_tiles_forward(*args, *dims)
+            elif mode == 1:
+                rgb, alpha = ext.render_tiles_forward_tilecenter(*args, *dims)
+            else:
+                raise ValueError("Unsupported tile mode for backward")
         rgb = _add_background(rgb, alpha, bg_color)
         ctx.save_for_backward(*args)
         ctx.dims, ctx.mode, ctx.bg_color = dims, int(mode), bg_color
@@ -544,10 +553,21 @@ class NeuralPrimitiveSceneTileCUDA(nn.Module):
                 rgb, alpha, feat = ext.render_tiles_forward_per_pixel_with_feat(*base, *feat_args, *dims)
             return _add_background(rgb, alpha, bg), feat
 
+    def invalidate_render_caches(self):
+        """Drop everything derived from the parameters (unit quaternions, geometry records, matrix-core operand
+        copies).  Called by every grad-mode forward: the caches are keyed on the parameters' identity and in-place
+        version, which a fused optimizer step (``Adam(fused=True)``) does not advance.  Call it yourself after
+        changing parameters in any other way that leaves ``tensor._version`` unchanged."""
+        self.__dict__.pop("_mlpsp_cache", None)
+        ext = _tile_ext
+        if ext is not None and callable(getattr(ext, "invalidate_caches", None)):
+            ext.invalidate_caches()
+
     def _forward_csr_training(self, ray_o, ray_d, score_threshold, bg_color, view_matrix, proj_matrix,
                               culled_prim_indices, tile_offsets, return_feature, feature_target, device):
         """(rgb, streamed feature L1 loss) through the record-based training function
         (scannet/cumodel.py:1098-1108)."""
+        self.invalidate_render_caches()
         W, H = self.image_size
         ts = int(self.tile_size)
         use_tilecenter = self._resolve_tile_order_mode() == "tilecenter"
@@ -571,6 +591,7 @@ class NeuralPrimitiveSceneTileCUDA(nn.Module):
                                 culled_prim_indices, tile_offsets, return_feature, device):
         """RGB with autograd (scannet/cumodel.py:1110-1131): tile lists and encodings are constants, positions,
         log-scales, normalised quaternions and MLP weights carry gradients."""
+        self.invalidate_render_caches()
         W, H = self.image_size
         ts = int(self.tile_size)
         with torch.no_grad():

@@ -9,6 +9,7 @@ f32 or on the matrix cores, reverse compositing, grouped gradients) is.
 """
 from __future__ import annotations
 
+import contextlib
 import threading
 import warnings
 
@@ -50,6 +51,7 @@ class TileExt:
         self._mfma_calls = 0
         self._mfma_fallbacks = 0
         self._training_mfma_stats = [0, 0, 0, 0, 0]
+        self._uncached = threading.local()
         self._pack_key = None
         self._pack = None
         self._feat_pack_key = None
@@ -59,6 +61,37 @@ class TileExt:
         self._queue_capacity = 0          # candidate-buffer estimate of render_frame_queued (0: not seeded yet)
         self._queue_scratch_scale = 1
         self._feat_pack = None
+
+    # ------------------------------------------------------------------------------------------
+    # derived-tensor caches (geometry records, matrix-core operand copies)
+    # ------------------------------------------------------------------------------------------
+    def invalidate_caches(self):
+        """Forget every derived tensor.  The caches are keyed on the identity, shape and in-place version of
+        their source tensors -- enough while a scene is only rendered, but a fused optimizer step
+        (``torch.optim.Adam(..., fused=True)``) rewrites parameters WITHOUT advancing their version counter.
+        Every training entry point therefore works uncached and leaves the caches empty; call this after
+        changing parameters by any other means that does not advance the version."""
+        with self._lock:
+            self._pack_key = self._pack = None
+            self._feat_pack_key = self._feat_pack = None
+            self._rec_key = self._rec = None
+            self._binned = None
+
+    @contextlib.contextmanager
+    def uncached(self):
+        """Inside: derived tensors are rebuilt from their sources on every use and not kept (training steps:
+        the parameters change between calls in ways a version counter does not always show)."""
+        self.invalidate_caches()
+        depth = getattr(self._uncached, "depth", 0)
+        self._uncached.depth = depth + 1
+        try:
+            yield self
+        finally:
+            self._uncached.depth = depth
+            self.invalidate_caches()
+
+    def _caching(self):
+        return getattr(self._uncached, "depth", 0) == 0
 
     def __getattr__(self, name):
         if name in _BACKWARD_ONLY:
@@ -344,7 +377,7 @@ class TileExt:
         _chk(tuple(x[10].shape) == (n, h) and tuple(x[11].shape) == (n, h, h) and x[12].shape == x[10].shape)
         _chk(tuple(x[13].shape) == (n, 4, h) and tuple(x[14].shape) == (n, 4))
         _chk(x[15].shape == x[0].shape and x[16].dim() == 1 and x[16].numel() == pixels)
-        with torch.cuda.device(x[0].device):
+        with torch.cuda.device(x[0].device), self.uncached():
             self._validate(x[5], x[6], ops.num_tiles(width, height, tile, tile), self.max_tile_prims, n, name)
             rec = self._records(x[2], x[3], x[4])
             order = x[5]
@@ -397,7 +430,7 @@ class TileExt:
         _chk(x[12].shape == x[10].shape and tuple(x[13].shape) == (n, 4, 32) and tuple(x[14].shape) == (n, 4))
         _chk(x[15].shape == x[0].shape and x[16].dim() == 1 and x[16].numel() == pixels)
         name = "render_tiles_training_records_wmma"
-        with torch.cuda.device(x[0].device):
+        with torch.cuda.device(x[0].device), self.uncached():
             self._validate(x[5], x[6], ops.num_tiles(width, height, 8, 8), self.max_tile_prims, n, name)
             nonfinite = ops.all_finite_flag([t for i, t in enumerate(x) if i not in (5, 6)])
             _chk(int(nonfinite.item()) == 0, "Training WMMA input is nonfinite; refusing unsafe forward/fallback")
@@ -531,6 +564,8 @@ class TileExt:
 
     def _records(self, positions, log_scales, quats):
         """Per-primitive geometry records, rebuilt only when one of the three tensors changed."""
+        if not self._caching():
+            return ops.prepare_primitives(positions, log_scales, quats)
         try:
             key = tuple((t.data_ptr(), t._version, tuple(t.shape), str(t.device)) for t in (positions, log_scales, quats))
         except RuntimeError:                      # inference tensors have no version counter: no caching
@@ -544,6 +579,8 @@ class TileExt:
     def _packed_weights(self, ws, bf16):
         """Matrix-core operand copy of the six weight tensors, rebuilt only when one of them changed
         (identity, shape or in-place version) -- the scene's weights are constant during inference."""
+        if not self._caching():
+            return ops.pack_mfma_weights(*ws, bf16=bf16)
         key = (bool(bf16),) + tuple((w.data_ptr(), w._version, tuple(w.shape), str(w.device)) for w in ws)
         with self._lock:
             if self._pack_key != key:
@@ -553,6 +590,8 @@ class TileExt:
 
     def _packed_feat(self, feat_attr):
         """fp16 operand copy of the feature attributes, cached like the weights -> (packed, nonfinite)."""
+        if not self._caching():
+            return ops.pack_mfma_feat(feat_attr)
         key = (feat_attr.data_ptr(), feat_attr._version, tuple(feat_attr.shape), str(feat_attr.device))
         with self._lock:
             if self._feat_pack_key != key:

@@ -118,3 +118,43 @@ def test_a_few_optimiser_steps_reduce_an_image_loss(device, oracle_mod):
         opt.step()
         losses.append(float(loss.detach()))
     assert all(np.isfinite(losses)) and losses[-1] < 0.7 * losses[0], losses
+
+
+@pytest.mark.parametrize("precision", ["f32", "bf16"])
+def test_fused_optimiser_steps_are_seen_by_the_next_render(device, oracle_mod, precision):
+    """Adam(fused=True) rewrites parameters without advancing ``tensor._version``, the key of the derived-tensor
+    caches (geometry records, unit quaternions, matrix-core operand copies): the grad-mode forward must leave no
+    cache behind, so that the render after the step uses the new parameters, as a scene built from them does."""
+    fr = Frame("cfg1_5k_160x120", n=400, hidden=32, width=48, height=32)
+    scene = _scene_from(fr, device).train()
+    scene.render_precision = precision
+    args = (to_dev(fr.rays_o, device), to_dev(fr.rays_d, device))
+    kw = dict(score_threshold=fr.thr, view_matrix=to_dev(fr.view, device), proj_matrix=to_dev(fr.proj, device))
+    with torch.no_grad():
+        before = scene(*args, **kw)              # fills the caches
+    target = (before * 0.5 + 0.2).clamp(0, 1)
+    opt = torch.optim.Adam([{"params": [scene.W1, scene.b1, scene.W2, scene.b2, scene.W3, scene.b3], "lr": 2e-2},
+                            {"params": [scene.positions, scene.log_scales, scene.quats], "lr": 5e-3}], fused=True)
+    versions = [p._version for p in scene.parameters()]
+    for _ in range(2):
+        opt.zero_grad(set_to_none=True)
+        (scene(*args, **kw) - target).abs().mean().backward()
+        opt.step()
+    with torch.no_grad():
+        after = scene(*args, **kw)
+        fresh = _scene_from(fr, device)
+        fresh.render_precision = precision
+        fresh.load_state_dict(scene.state_dict())
+        from mlp_splatting_amd.tile_ext import TileExt
+        fresh_ext = TileExt()
+        rd = torch.nn.functional.normalize(args[1], dim=-1).contiguous()
+        cand, off = fresh._tile_lists(args[0], rd, fr.thr, kw["view_matrix"], kw["proj_matrix"], None, None, device)
+        base = fresh._base_args(args[0], args[1], cand, off, device)
+        if precision == "f32":
+            expected = fresh_ext.render_tiles_forward_tilecenter(*base, fr.W, fr.H, 8, 8, fr.thr)[0]
+        else:
+            expected = fresh_ext.render_tiles_rgb_wmma(list(base), fr.W, fr.H, fr.thr, True)[0]
+    assert float((after - before).abs().max()) > 1e-3             # the steps did change the image
+    assert torch.equal(after, expected)
+    if [p._version for p in scene.parameters()] != versions:
+        pytest.skip("this torch build advances the version in fused steps; the caches would have seen them anyway")
