@@ -78,12 +78,14 @@ __global__ __launch_bounds__(128) void stream_l1_kernel(const int32_t* __restric
 // What a record contributes does not depend on the channel except through the signs it samples: its four
 // bilinear taps (offset of the target pixel's sign row, weight) and its slot factors T alpha gate_s.  Per batch
 // of 64 records these are computed once, lane = record, and parked in LDS; then lane = 4 consecutive channels and
-// every record costs four 4-byte sign loads and the multiply-adds.
+// every record costs four 4-byte sign loads, the tap sums, and a share of a small matrix product (below).
 struct RecordTaps {
-  int off[4];      // (iy * WF + ix) * C of the tap's target pixel, or -1 outside the target
-  float weight[4];
-  float a[8];      // slot factors (SLOTS of them), rounded to fp16 in mixed mode
+  int off[4];      // (iy * WF + ix) * C of the tap's target pixel (0 outside the target)
+  float weight[4]; // bilinear weight (0 outside the target)
 };
+
+typedef _Float16 fh4 __attribute__((ext_vector_type(4)));
+typedef float ff4 __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ void record_taps(int pix, int W, int H, int WF, int HF, int C, RecordTaps& t) {
   const int xx = pix % W, yy = pix / W;
@@ -97,10 +99,12 @@ __device__ __forceinline__ void record_taps(int pix, int W, int H, int WF, int H
       const int ix = tx + dx, iy = ty + dy;
       const float srcx = fmaxf(((float)ix + .5f) * bx - .5f, 0.f);
       const float srcy = fmaxf(((float)iy + .5f) * by - .5f, 0.f);
-      t.weight[dy * 2 + dx] = fmaxf(0.f, 1.f - __builtin_fabsf(srcx - (float)xx)) *
-                              fmaxf(0.f, 1.f - __builtin_fabsf(srcy - (float)yy));
+      const float weight = fmaxf(0.f, 1.f - __builtin_fabsf(srcx - (float)xx)) *
+                           fmaxf(0.f, 1.f - __builtin_fabsf(srcy - (float)yy));
       const bool inside = ix >= 0 && ix < WF && iy >= 0 && iy < HF;
-      t.off[dy * 2 + dx] = inside ? (iy * WF + ix) * C : -1;
+      // a tap outside the target reads row 0 with weight 0: the loads of the channel loop need no branch
+      t.weight[dy * 2 + dx] = inside ? weight : 0.f;
+      t.off[dy * 2 + dx] = inside ? (iy * WF + ix) * C : 0;
     }
   }
 }
@@ -109,7 +113,14 @@ __device__ __forceinline__ void record_taps(int pix, int W, int H, int WF, int H
 // accum[slot][channel] += (T alpha gate_slot)[record] * adjoint[record's pixel, channel], the adjoint being the
 // bilinear transpose of the signs (_resample_adjoint, :92-111: taps added in the order (0,0), (0,1), (1,0),
 // (1,1)).  MIXED rounds both factors to fp16 first, as the reference's mixed GEMM does; accumulation is f32.
-template <int SLOTS, bool MIXED>
+//
+// The sum over records is a [slots x records] x [records x channels] product, and it runs on the matrix cores
+// as 4x4 blocks: v_mfma_f32_4x4x4_f16 (mixed; four records per instruction) or v_mfma_f32_4x4x1_f32 (one record,
+// an exact f32 fma) treats every group of four lanes as one block, takes from lane l row l%4 of A (a slot's
+// factors) and column l%4 of B (the adjoints of ONE of the lane's four channels) and returns to the lane that
+// column of the 4x4 result, one slot per register.  One instruction per channel of the lane replaces sixteen
+// multiply-adds per record.  Five slots take a second product whose only non-zero row is the fifth slot.
+template <int SLOTS, bool MIXED, bool VEC>
 __global__ __launch_bounds__(64) void feature_vjp_kernel(const int8_t* __restrict__ signs,
                                                          const long long* __restrict__ order,
                                                          const int32_t* __restrict__ record_pixels,
@@ -119,76 +130,135 @@ __global__ __launch_bounds__(64) void feature_vjp_kernel(const int8_t* __restric
                                                          const long long* __restrict__ group_start,
                                                          float* __restrict__ partial, int W, int H, int WF, int HF, int C,
                                                          int segment) {
-  __shared__ RecordTaps s_rec[64];
+  constexpr int ROWS = SLOTS == 5 ? 8 : 4;                   // slot rows kept in LDS (two products for five slots)
+  __shared__ __attribute__((aligned(16))) RecordTaps s_rec[64];
+  __shared__ __attribute__((aligned(16))) float s_a[ROWS][64];          // f32 factors, [slot][record]
+  __shared__ __attribute__((aligned(8))) _Float16 s_ah[ROWS][64];       // the same rounded to fp16 (mixed)
   const long long group = blockIdx.x;
-  const int lane = threadIdx.x;
+  const int lane = threadIdx.x, m = lane & 3;
   const int c0 = blockIdx.y * 256 + lane * 4;
   const long long p = group_prim[group];
   const long long begin = group_start[group];
   const long long seg_end = begin + segment, list_end = offsets[p + 1];
   const long long end = seg_end < list_end ? seg_end : list_end;
-  const bool vec = (C % 4 == 0) && (c0 + 3 < C);     // the lane's four channels are one aligned 4-byte load
-  float accum[SLOTS][4];
+  // VEC (C % 4 == 0): a lane's four channels are one aligned 4-byte load.  Channels past C are clamped to valid
+  // addresses and their sums never stored.
+  constexpr bool vec = VEC;
+  int cc[4];
 #pragma unroll
-  for (int s = 0; s < SLOTS; ++s)
+  for (int k = 0; k < 4; ++k) cc[k] = c0 + k < C ? c0 + k : C - 1;
+  const int cv = c0 + 3 < C ? c0 : 0;
+  ff4 acc[4], acc5[4];                                // [channel of the lane][slot]; acc5[.][0] = fifth slot
 #pragma unroll
-    for (int k = 0; k < 4; ++k) accum[s][k] = 0.f;
+  for (int k = 0; k < 4; ++k) acc[k] = acc5[k] = ff4{0.f, 0.f, 0.f, 0.f};
   for (long long base = begin; base < end; base += 64) {
     const long long row = base + lane;
-    if (row < end) {
-      const long long r = order[row];
+    {
       RecordTaps t;
-      record_taps(record_pixels[r], W, H, WF, HF, C, t);
-      const float w = raw[r * 8 + 4] * raw[r * 8 + 5];
+      float a[ROWS];
 #pragma unroll
-      for (int s = 0; s < SLOTS; ++s) {
-        float g = 1.f;
-        if constexpr (SLOTS == 4) g = gates[r * 4 + s];
-        if constexpr (SLOTS == 5) g = (s == 0) ? 1.f : gates[r * 4 + s - 1];
-        float a = w * g;
-        if constexpr (MIXED) a = (float)(_Float16)a;
-        t.a[s] = a;
+      for (int q = 0; q < 4; ++q) {
+        t.off[q] = 0;
+        t.weight[q] = 0.f;
+      }
+#pragma unroll
+      for (int i = 0; i < ROWS; ++i) a[i] = 0.f;
+      if (row < end) {                                  // rows past the end stay empty records: the loop below
+        const long long r = order[row];                 // then needs no tail case
+        record_taps(record_pixels[r], W, H, WF, HF, C, t);
+        const float w = raw[r * 8 + 4] * raw[r * 8 + 5];
+#pragma unroll
+        for (int sl = 0; sl < SLOTS; ++sl) {
+          float g = 1.f;
+          if constexpr (SLOTS == 4) g = gates[r * 4 + sl];
+          if constexpr (SLOTS == 5) g = (sl == 0) ? 1.f : gates[r * 4 + sl - 1];
+          a[sl] = w * g;
+        }
       }
       s_rec[lane] = t;
+#pragma unroll
+      for (int i = 0; i < ROWS; ++i) {
+        if constexpr (MIXED) s_ah[i][lane] = (_Float16)a[i];
+        else s_a[i][lane] = a[i];
+      }
     }
     __syncthreads();
     const int count = (int)((end - base) < 64 ? (end - base) : 64);
-    for (int rr = 0; rr < count; ++rr) {
-      const RecordTaps& t = s_rec[rr];
-      float b[4] = {0.f, 0.f, 0.f, 0.f};
+    // the sign words of the NEXT four records are requested before the current four are used: with four
+    // wavefronts per SIMD the load latency is otherwise paid once per step
+    int ahead[16] = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+    if constexpr (vec) {
 #pragma unroll
-      for (int tap = 0; tap < 4; ++tap) {
-        const int off = t.off[tap];
-        const float wt = t.weight[tap];
-        float sv[4] = {0.f, 0.f, 0.f, 0.f};
-        if (off >= 0) {
-          if (vec) {
-            const int packed = *reinterpret_cast<const int*>(signs + (long long)off + c0);
+      for (int q = 0; q < 4; ++q)
+#pragma unroll
+        for (int tap = 0; tap < 4; ++tap)
+          ahead[4 * q + tap] = *reinterpret_cast<const int*>(signs + (long long)s_rec[q].off[tap] + cv);
+    }
+    for (int rr = 0; rr < count; rr += 4) {
+      // adjoints of four records for the lane's four channels
+      float bq[4][4];
+      int now[16];
+#pragma unroll
+      for (int i = 0; i < 16; ++i) now[i] = ahead[i];
+      if (vec && rr + 4 < count) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+#pragma unroll
+          for (int tap = 0; tap < 4; ++tap)
+            ahead[4 * q + tap] = *reinterpret_cast<const int*>(signs + (long long)s_rec[rr + 4 + q].off[tap] + cv);
+      }
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const RecordTaps& t = s_rec[rr + q];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) bq[q][k] = 0.f;
+#pragma unroll
+        for (int tap = 0; tap < 4; ++tap) {
+          const float wt = t.weight[tap];
+          float sv[4];
+          if constexpr (vec) {
+            const int packed = now[4 * q + tap];
 #pragma unroll
             for (int k = 0; k < 4; ++k) sv[k] = (float)(int8_t)(packed >> (8 * k));
           } else {
 #pragma unroll
-            for (int k = 0; k < 4; ++k) sv[k] = (c0 + k < C) ? (float)signs[(long long)off + c0 + k] : 0.f;
+            for (int k = 0; k < 4; ++k) sv[k] = (float)signs[(long long)t.off[tap] + cc[k]];
+          }
+#pragma unroll
+          for (int k = 0; k < 4; ++k) bq[q][k] = fmaf(wt, sv[k], bq[q][k]);
+        }
+      }
+      if constexpr (MIXED) {
+        const fh4 a_op = *reinterpret_cast<const fh4*>(&s_ah[m][rr]);            // rows past the last slot are zero
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          const fh4 b_op = {(_Float16)bq[0][k], (_Float16)bq[1][k], (_Float16)bq[2][k], (_Float16)bq[3][k]};
+          acc[k] = __builtin_amdgcn_mfma_f32_4x4x4f16(a_op, b_op, acc[k], 0, 0, 0);
+          if constexpr (SLOTS == 5) {
+            const fh4 a5 = *reinterpret_cast<const fh4*>(&s_ah[4 + m][rr]);       // rows 5..7 are zero
+            acc5[k] = __builtin_amdgcn_mfma_f32_4x4x4f16(a5, b_op, acc5[k], 0, 0, 0);
           }
         }
+      } else {
 #pragma unroll
-        for (int k = 0; k < 4; ++k) b[k] += wt * sv[k];
-      }
+        for (int q = 0; q < 4; ++q) {
+          const float a_op = s_a[m][rr + q];
 #pragma unroll
-      for (int k = 0; k < 4; ++k) {
-        if constexpr (MIXED) b[k] = (float)(_Float16)b[k];
-#pragma unroll
-        for (int s = 0; s < SLOTS; ++s) accum[s][k] += t.a[s] * b[k];
+          for (int k = 0; k < 4; ++k) {
+            acc[k] = __builtin_amdgcn_mfma_f32_4x4x1f32(a_op, bq[q][k], acc[k], 0, 0, 0);
+            if constexpr (SLOTS == 5) acc5[k] = __builtin_amdgcn_mfma_f32_4x4x1f32(s_a[4 + m][rr + q], bq[q][k], acc5[k], 0, 0, 0);
+          }
+        }
       }
     }
     __syncthreads();
   }
   const float norm = (float)((long long)WF * HF * C);
 #pragma unroll
-  for (int s = 0; s < SLOTS; ++s)
+  for (int sl = 0; sl < SLOTS; ++sl)
 #pragma unroll
     for (int k = 0; k < 4; ++k)
-      if (c0 + k < C) partial[(group * SLOTS + s) * C + c0 + k] = accum[s][k] / norm;
+      if (c0 + k < C) partial[(group * SLOTS + sl) * C + c0 + k] = (sl < 4 ? acc[k][sl] : acc5[k][0]) / norm;
 }
 
 }  // namespace mlpsp
@@ -245,20 +315,26 @@ MLPSP_API int mlpsp_feature_attribute_gradients(const int8_t* signs_dev, const i
         !group_primitives_dev || !group_starts_dev || !partial_dev)
       return MLPSP_E_ARGUMENT;
     const dim3 grid((unsigned)num_groups, (unsigned)((channels + 255) / 256)), block(64);
-#define MLPSP_FV_LAUNCH(SL, MX)                                                                                    \
-  hipLaunchKernelGGL((feature_vjp_kernel<SL, MX>), grid, block, 0, s, signs_dev,                                   \
+#define MLPSP_FV_LAUNCH(SL, MX, VC)                                                                                \
+  hipLaunchKernelGGL((feature_vjp_kernel<SL, MX, VC>), grid, block, 0, s, signs_dev,                               \
                      (const long long*)record_indices_dev, record_pixels_dev, raw_dev, gates_dev,                  \
                      (const long long*)csr_offsets_dev, (const long long*)group_primitives_dev,                    \
                      (const long long*)group_starts_dev, partial_dev, width, height, target_width, target_height,  \
                      channels, segment)
-#define MLPSP_FV_SLOTS(MX)                         \
-  do {                                             \
-    if (slots == 1) MLPSP_FV_LAUNCH(1, MX);        \
-    else if (slots == 4) MLPSP_FV_LAUNCH(4, MX);   \
-    else MLPSP_FV_LAUNCH(5, MX);                   \
+#define MLPSP_FV_SLOTS(MX, VC)                         \
+  do {                                                 \
+    if (slots == 1) MLPSP_FV_LAUNCH(1, MX, VC);        \
+    else if (slots == 4) MLPSP_FV_LAUNCH(4, MX, VC);   \
+    else MLPSP_FV_LAUNCH(5, MX, VC);                   \
   } while (0)
-    if (mixed) MLPSP_FV_SLOTS(true);
-    else MLPSP_FV_SLOTS(false);
+    const bool aligned4 = (channels % 4 == 0) && (reinterpret_cast<uintptr_t>(signs_dev) % 4 == 0);
+    if (mixed) {
+      if (aligned4) MLPSP_FV_SLOTS(true, true);
+      else MLPSP_FV_SLOTS(true, false);
+    } else {
+      if (aligned4) MLPSP_FV_SLOTS(false, true);
+      else MLPSP_FV_SLOTS(false, false);
+    }
 #undef MLPSP_FV_SLOTS
 #undef MLPSP_FV_LAUNCH
     MLPSP_LAUNCH_CHECK();
