@@ -19,12 +19,13 @@ if ROOT not in sys.path:
 PEAK = {"f32": 157.3, "bf16": 2500.0}          # MI355X dense peaks, TFLOP/s
 HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the render kernel, from hardware counters: two profiled runs of
-#   rocprofv3 --pmc FETCH_SIZE -- python3 bench.py --steps 16 --warmup 8 --no-cpu-baseline --copy-calibration
+#   rocprofv3 --pmc FETCH_SIZE -- python3 bench.py --steps 16 --warmup 8 --no-cpu-baseline --wake-seconds 0 --copy-calibration
 #   rocprofv3 --pmc WRITE_SIZE -- (same)
 # averaged over the run's 56 launches, each counter scaled by what it reads for the 1 GiB device copies of
 # --copy-calibration (FETCH_SIZE reads 524,307 KiB for 1,048,576 KiB copied: factor 2.0; WRITE_SIZE reads
-# 1,048,576 KiB: factor 1.0).  Render kernel: 50,777 KiB x 2.0 fetched + 16,813 KiB written.
-MEASURED_TRAFFIC_BYTES = {("cfg3_200k_1200x680", "bf16"): int((121920.7 * 2.0 + 54889.0) * 1024)}
+# 1,048,576 KiB: factor 1.0).  Render kernel: 51,118 KiB x 2.0 fetched + 16,832 KiB written = 121.9 MB
+# (profiles/render_tilecenter_mfma_cfg3_200k_1200x680.txt).
+MEASURED_TRAFFIC_BYTES = {("cfg3_200k_1200x680", "bf16"): int((51117.9 * 2.0 + 16831.6) * 1024)}
 
 
 def train_steps(args, scene, frames, proj, thr, W, H, sc, dev):
