@@ -75,7 +75,7 @@ class TileExt:
             self._pack_key = self._pack = None
             self._feat_pack_key = self._feat_pack = None
             self._rec_key = self._rec = None
-            self._binned = None
+        # (the note about freshly binned tile lists is keyed on the list tensors themselves, not on parameters)
 
     @contextlib.contextmanager
     def uncached(self):
