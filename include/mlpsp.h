@@ -167,19 +167,23 @@ int mlpsp_render_tilecenter_stats_f32(const float* rays_o_dev, const float* rays
  * Step 1 (count): counts_dev [B] int32.  The caller scans them into record_offsets_dev [B+1] int64
  * (exclusive) and allocates R = record_offsets[B] records.  Step 2 (emit) writes them.
  * overflow_dev (int32, zeroed by the count step): 1 if a live pixel reached max_hits -- the reference
- * raises "hit capacity" then (:4601-4609); nothing is truncated silently. */
+ * raises "hit capacity" then (:4601-4609); nothing is truncated silently.
+ * render_order: 0 = the record kernels' rounding of layer 2 (bias added after a sum started at zero,
+ * np_tile_kernels.cu:349-353); 1 = the render kernels' (sum started at the bias): image, alpha and every record
+ * field are then those of mlpsp_render_tilecenter_f32 bit for bit, so a differentiable render can use the
+ * records forward AS its forward.  1 needs the 72->32->32->4 shape with 16-byte aligned weights. */
 int mlpsp_records_count(const float* rays_o_dev, const float* rays_d_dev, const void* prim_records_dev,
                         const int32_t* order_dev, const int32_t* tile_offsets_dev, const float* freq_dev,
                         const float* att_dev, int num_frequencies, const float* W1, const float* b1, const float* W2,
                         const float* b2, const float* W3, const float* b3, int num_primitives, int hidden, int width,
-                        int height, int tile_w, int tile_h, float threshold, int max_hits, int32_t* counts_dev,
-                        int32_t* overflow_dev, mlpsp_stream_t stream);
+                        int height, int tile_w, int tile_h, float threshold, int max_hits, int render_order,
+                        int32_t* counts_dev, int32_t* overflow_dev, mlpsp_stream_t stream);
 int mlpsp_records_emit(const float* rays_o_dev, const float* rays_d_dev, const void* prim_records_dev,
                        const int32_t* order_dev, const int32_t* tile_offsets_dev, const float* freq_dev,
                        const float* att_dev, int num_frequencies, const float* W1, const float* b1, const float* W2,
                        const float* b2, const float* W3, const float* b3, int num_primitives, int hidden, int width,
-                       int height, int tile_w, int tile_h, float threshold, int max_hits, float gating_beta,
-                       float gating_temp, const int64_t* record_offsets_dev, int32_t* ids_dev, float* x6_dev,
+                       int height, int tile_w, int tile_h, float threshold, int max_hits, int render_order,
+                       float gating_beta, float gating_temp, const int64_t* record_offsets_dev, int32_t* ids_dev, float* x6_dev,
                        int32_t* masks_dev, float* raw_dev, float* gates_dev, float* out_rgb_dev, float* out_alpha_dev,
                        int32_t* overflow_dev, mlpsp_stream_t stream);
 

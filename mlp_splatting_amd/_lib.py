@@ -52,8 +52,8 @@ SIGNATURES = {
     "mlpsp_mfma_feat_pack_bytes": (_sz, [_i, _i, _i]),
     "mlpsp_pack_mfma_feat": (_i, [_vp, _i, _i, _i, _vp, _vp, _vp]),
     "mlpsp_render_tilecenter_stats_f32": (_i, [_vp] * 7 + [_i] + [_vp] * 6 + [_i, _i, _i, _i, _i, _i, _f] + [_vp] * 9),
-    "mlpsp_records_count": (_i, [_vp] * 7 + [_i] + [_vp] * 6 + [_i, _i, _i, _i, _i, _i, _f, _i, _vp, _vp, _vp]),
-    "mlpsp_records_emit": (_i, [_vp] * 7 + [_i] + [_vp] * 6 + [_i, _i, _i, _i, _i, _i, _f, _i, _f, _f] + [_vp] * 10),
+    "mlpsp_records_count": (_i, [_vp] * 7 + [_i] + [_vp] * 6 + [_i, _i, _i, _i, _i, _i, _f, _i, _i, _vp, _vp, _vp]),
+    "mlpsp_records_emit": (_i, [_vp] * 7 + [_i] + [_vp] * 6 + [_i, _i, _i, _i, _i, _i, _f, _i, _i, _f, _f] + [_vp] * 10),
     "mlpsp_records_mfma_count": (_i, [_vp] * 8 + [_i, _i, _i, _f, _i, _i, _vp, _vp, _vp]),
     "mlpsp_records_mfma_emit": (_i, [_vp] * 8 + [_i, _i, _i, _f, _i, _i, _f, _f, _vp, _i64] + [_vp] * 9),
     "mlpsp_all_finite": (_i, [_vp, _vp, _i, _vp, _vp]),

@@ -84,9 +84,9 @@ __device__ __forceinline__ void encode_direction(float rdx, float rdy, float rdz
 
 // All 64 lanes must be active.  x6 is the lane's own pixel's input (components 0..2 enter through dir,
 // which encode_direction() made from them); out is the lane's own pixel's output.
-// REC selects the record kernels' layer-2 rounding (bias added after a chain started at zero) and fills
+// REC selects the record kernels' layer-2 rounding (bias added after a chain started at zero); MASKS fills
 // masks[0..1] with the ReLU masks of the lane's pixel.
-template <bool REC = false>
+template <bool REC = false, bool MASKS = REC>
 __device__ __forceinline__ void mlp_wave_mfma32(const float x6[6], const float* __restrict__ freq,
                                                 const float* __restrict__ att, const float* __restrict__ W1,
                                                 const float* __restrict__ b1, const float* __restrict__ W2,
@@ -165,11 +165,11 @@ __device__ __forceinline__ void mlp_wave_mfma32(const float x6[6], const float* 
       acc[k] = fmaf(w3[k * H + 2 * i], even, acc[k]);
       acc[k] = fmaf(w3[k * H + 2 * i + 1], odd, acc[k]);
     }
-    if constexpr (REC) m2 |= (even > 0.f ? (1u << (2 * i)) : 0u) | (odd > 0.f ? (2u << (2 * i)) : 0u);
+    if constexpr (MASKS) m2 |= (even > 0.f ? (1u << (2 * i)) : 0u) | (odd > 0.f ? (2u << (2 * i)) : 0u);
   }
 #pragma unroll
   for (int k = 0; k < 4; ++k) out[k] = acc[k];
-  if constexpr (REC) {
+  if constexpr (MASKS) {
     uint32_t lo = 0u, hi = 0u;   // bits 2i + g of blocks 0 and 1, as held by this lane
 #pragma unroll
     for (int i = 0; i < 16; ++i) {

@@ -24,7 +24,10 @@ struct RecordOut {
 };
 
 // MF: the MLP of a hit runs on the matrix cores for the whole wavefront (mlp_wave_mfma32, same bits).
-template <int HT, int FT, bool EMIT, bool MF = false>
+// RORD (with MF only): layer 2 in the rounding order of the RENDER kernels instead of the record kernels', so
+// that image and records are those of mlpsp_render_tilecenter_f32 bit for bit -- the differentiable render
+// then needs no separate forward pass.
+template <int HT, int FT, bool EMIT, bool MF = false, bool RORD = false>
 __global__ __launch_bounds__(64) void records_kernel(
     const float* __restrict__ rays_o, const float* __restrict__ rays_d, const PrimRecord* __restrict__ prims,
     const int32_t* __restrict__ order, const int32_t* __restrict__ offsets, const float* __restrict__ freq,
@@ -65,7 +68,7 @@ __global__ __launch_bounds__(64) void records_kernel(
       const float x6[6] = {rdx, rdy, rdz, hit ? h.dx : 0.f, hit ? h.dy : 0.f, hit ? h.dz : 0.f};
       float o[4];
       uint32_t mk[2];
-      if constexpr (MF) mlp_wave_mfma32<true>(x6, freq, att, W1, b1, W2, b2, W3, b3, p, dir, o, mk);
+      if constexpr (MF) mlp_wave_mfma32<!RORD, true>(x6, freq, att, W1, b1, W2, b2, W3, b3, p, dir, o, mk);
       if (hit) {
         if constexpr (!MF) mlp_eval<HT, FT, true>(x6, freq, att, F, H, mlp, p, o, mk);
         const float R = sigmoid(o[0]), G = sigmoid(o[1]), Bc = sigmoid(o[2]);
@@ -126,14 +129,15 @@ namespace {
 int records_launch(bool emit, const float* rays_o, const float* rays_d, const void* prims, const int32_t* order,
                    const int32_t* offsets, const float* freq, const float* att, int F, const float* W1, const float* b1,
                    const float* W2, const float* b2, const float* W3, const float* b3, int N, int hidden, int width,
-                   int height, int tile_w, int tile_h, float thr, int max_hits, float beta, float temp, int32_t* counts,
-                   int32_t* overflow, RecordOut out, hipStream_t s) {
+                   int height, int tile_w, int tile_h, float thr, int max_hits, int render_order, float beta, float temp,
+                   int32_t* counts, int32_t* overflow, RecordOut out, hipStream_t s) {
   const int64_t T = checked_num_tiles(width, height, tile_w, tile_h);
   if (T <= 0) return MLPSP_E_ARGUMENT;
   const int64_t tile_px = (int64_t)tile_w * tile_h;
   if (tile_px <= 0 || tile_px > 256) return MLPSP_E_ARGUMENT;
   if (F <= 0 || F > 16 || hidden <= 0 || hidden > 32 || N < 0 || max_hits <= 0) return MLPSP_E_ARGUMENT;
   if (!rays_o || !rays_d || !offsets || !overflow) return MLPSP_E_ARGUMENT;
+  if (render_order && !use_mfma32(hidden, F, W1, b1, W2, b2)) return MLPSP_E_ARGUMENT;
   const int wpt = (int)((tile_px + 63) / 64);
   const int64_t items = T * wpt;
   if (items > 2147483647LL - 8) return MLPSP_E_ARGUMENT;
@@ -146,7 +150,8 @@ int records_launch(bool emit, const float* rays_o, const float* rays_d, const vo
                      thr, max_hits, beta, temp, counts, overflow, out)
 #define MLPSP_REC_SHAPES(EM)                                          \
   do {                                                                \
-    if (use_mfma32(hidden, F, W1, b1, W2, b2)) MLPSP_REC_LAUNCH(32, 6, EM, true); \
+    if (render_order) MLPSP_REC_LAUNCH(32, 6, EM, true, true);          \
+    else if (use_mfma32(hidden, F, W1, b1, W2, b2)) MLPSP_REC_LAUNCH(32, 6, EM, true); \
     else if (hidden == 32 && F == 6) MLPSP_REC_LAUNCH(32, 6, EM);     \
     else if (hidden == 16 && F == 6) MLPSP_REC_LAUNCH(16, 6, EM);     \
     else MLPSP_REC_LAUNCH(0, 0, EM);                                  \
@@ -165,14 +170,14 @@ MLPSP_API int mlpsp_records_count(const float* rays_o_dev, const float* rays_d_d
                                   const float* att_dev, int num_frequencies, const float* W1, const float* b1,
                                   const float* W2, const float* b2, const float* W3, const float* b3,
                                   int num_primitives, int hidden, int width, int height, int tile_w, int tile_h,
-                                  float threshold, int max_hits, int32_t* counts_dev, int32_t* overflow_dev,
-                                  mlpsp_stream_t stream) {
+                                  float threshold, int max_hits, int render_order, int32_t* counts_dev,
+                                  int32_t* overflow_dev, mlpsp_stream_t stream) {
   if (!counts_dev || !overflow_dev) return MLPSP_E_ARGUMENT;
   hipStream_t s = (hipStream_t)stream;
   MLPSP_HIP_TRY(hipMemsetAsync(overflow_dev, 0, sizeof(int32_t), s));
   return records_launch(false, rays_o_dev, rays_d_dev, prim_records_dev, order_dev, tile_offsets_dev, freq_dev, att_dev,
                         num_frequencies, W1, b1, W2, b2, W3, b3, num_primitives, hidden, width, height, tile_w, tile_h,
-                        threshold, max_hits, 0.f, 0.f, counts_dev, overflow_dev, RecordOut{}, s);
+                        threshold, max_hits, render_order, 0.f, 0.f, counts_dev, overflow_dev, RecordOut{}, s);
 }
 
 MLPSP_API int mlpsp_records_emit(const float* rays_o_dev, const float* rays_d_dev, const void* prim_records_dev,
@@ -180,7 +185,7 @@ MLPSP_API int mlpsp_records_emit(const float* rays_o_dev, const float* rays_d_de
                                  const float* att_dev, int num_frequencies, const float* W1, const float* b1,
                                  const float* W2, const float* b2, const float* W3, const float* b3,
                                  int num_primitives, int hidden, int width, int height, int tile_w, int tile_h,
-                                 float threshold, int max_hits, float gating_beta, float gating_temp,
+                                 float threshold, int max_hits, int render_order, float gating_beta, float gating_temp,
                                  const int64_t* record_offsets_dev, int32_t* ids_dev, float* x6_dev,
                                  int32_t* masks_dev, float* raw_dev, float* gates_dev, float* out_rgb_dev,
                                  float* out_alpha_dev, int32_t* overflow_dev, mlpsp_stream_t stream) {
@@ -190,5 +195,6 @@ MLPSP_API int mlpsp_records_emit(const float* rays_o_dev, const float* rays_d_de
                 out_alpha_dev};
   return records_launch(true, rays_o_dev, rays_d_dev, prim_records_dev, order_dev, tile_offsets_dev, freq_dev, att_dev,
                         num_frequencies, W1, b1, W2, b2, W3, b3, num_primitives, hidden, width, height, tile_w, tile_h,
-                        threshold, max_hits, gating_beta, gating_temp, nullptr, overflow_dev, out, (hipStream_t)stream);
+                        threshold, max_hits, render_order, gating_beta, gating_temp, nullptr, overflow_dev, out,
+                        (hipStream_t)stream);
 }

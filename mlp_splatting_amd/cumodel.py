@@ -206,21 +206,33 @@ class _TileRenderAutogradFn(torch.autograd.Function):
                 W1, b1, W2, b2, W3, b3)
         dims = (int(Wimg), int(Himg), int(TW), int(TH), float(threshold))
         # a training step: nothing derived from the parameters may be reused from, or kept for, another call
+        records = None
         with _uncached(ext):
             if mode == 0:
                 rgb, alpha = ext.render_tiles_forward(*args, *dims)
             elif mode == 1:
-                rgb, alpha = ext.render_tiles_forward_tilecenter(*args, *dims)
+                matches = getattr(ext, "records_forward_matches_render", None)
+                if (dims[2] == dims[3] and callable(matches) and matches(freq, W1, b1, W2, b2, dims[2])
+                        and os.environ.get("MLPSP_AUTOGRAD_KEEP_RECORDS", "1") != "0"):
+                    # the records forward in the render kernels' rounding IS this forward (same bits), and its
+                    # records serve the backward: one traversal of the frame less per step
+                    placeholders = [torch.zeros_like(rays_o), torch.zeros(rays_o.shape[0], device=rays_o.device)]
+                    records = ext.render_tiles_training_records(list(args) + placeholders, dims[0], dims[1], dims[2],
+                                                                dims[4], 1.5, 2.0, render_order=True)
+                    rgb, alpha = records[0], records[1]
+                else:
+                    rgb, alpha = ext.render_tiles_forward_tilecenter(*args, *dims)
             else:
                 raise ValueError("Unsupported tile mode for backward")
         rgb = _add_background(rgb, alpha, bg_color)
-        ctx.save_for_backward(*args)
+        ctx.save_for_backward(*args, *(records[2:] if records is not None else ()))
+        ctx.has_records = records is not None
         ctx.dims, ctx.mode, ctx.bg_color = dims, int(mode), bg_color
         return rgb
 
     @staticmethod
     def backward(ctx, grad_out_rgb):
-        args = ctx.saved_tensors
+        args, kept = ctx.saved_tensors[:15], ctx.saved_tensors[15:]
         grad_out_rgb = grad_out_rgb.contiguous()
         if ctx.bg_color is None:
             grad_t_end = torch.zeros(args[0].shape[0], device=grad_out_rgb.device, dtype=grad_out_rgb.dtype)
@@ -233,8 +245,12 @@ class _TileRenderAutogradFn(torch.autograd.Function):
             raise NotImplementedError("the backward of the per-pixel order render is not built; train with the "
                                       "tile-centre order (MLPSP_TILE_ORDER_MODE=tilecenter, the default)")
         ext = NeuralPrimitiveSceneTileCUDA._ensure_tile_ext_static()
-        gW1, gb1, gW2, gb2, gW3, gb3, gp, gs, gq = ext.render_tiles_backward_tilecenter_full(
-            *args, grad_out_rgb, grad_t_end, *ctx.dims)
+        if ctx.has_records:
+            gW1, gb1, gW2, gb2, gW3, gb3, gp, gs, gq = ext.backward_from_records(
+                [None, None, *kept], args[2], args[3], args[4], args[7], args[8], *args[9:15], grad_out_rgb, grad_t_end)
+        else:
+            gW1, gb1, gW2, gb2, gW3, gb3, gp, gs, gq = ext.render_tiles_backward_tilecenter_full(
+                *args, grad_out_rgb, grad_t_end, *ctx.dims)
         return (None, None, gp, gs, gq, None, None, None, None, gW1, gb1, gW2, gb2, gW3, gb3,
                 None, None, None, None, None, None, None)
 

@@ -209,9 +209,10 @@ def render_tilecenter_stats_f32(rays_o, rays_d, records, order, tile_offsets, fr
 
 
 def training_records(rays_o, rays_d, records, order, tile_offsets, freq, att, W1, b1, W2, b2, W3, b3, W, H, TW, TH,
-                     threshold, beta, temp, max_hits, path_name="render_tiles_training_records"):
+                     threshold, beta, temp, max_hits, path_name="render_tiles_training_records", render_order=False):
     """Training-records forward -> (rgb, alpha, ids, x6, raw, masks, gates, offsets int64 [B+1]);
-    raises the reference's hit-capacity error (np_tile_kernels.cu:4601-4609)."""
+    raises the reference's hit-capacity error (np_tile_kernels.cu:4601-4609).  ``render_order``: layer 2 rounded as
+    the render kernels round it, which makes image and records those of the f32 render bit for bit."""
     dev = rays_o.device
     lib = _lib.load()
     B = W * H
@@ -220,7 +221,7 @@ def training_records(rays_o, rays_d, records, order, tile_offsets, freq, att, W1
     overflow = torch.empty(1, dtype=torch.int32, device=dev)
     head = (_ptr(rays_o), _ptr(rays_d), _ptr(records), _ptr(order), _ptr(tile_offsets), _ptr(freq), _ptr(att), F,
             _ptr(W1), _ptr(b1), _ptr(W2), _ptr(b2), _ptr(W3), _ptr(b3), n, hidden, W, H, TW, TH, float(threshold),
-            int(max_hits))
+            int(max_hits), 1 if render_order else 0)
 
     def refuse():
         raise RuntimeError(f"{path_name}: tile-center backward hit capacity {int(max_hits)} reached before "

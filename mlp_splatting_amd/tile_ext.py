@@ -355,10 +355,12 @@ class TileExt:
     # ------------------------------------------------------------------------------------------
     # training-records forward (np_tile_kernels.cu:6897-6998, forward_only = true)
     # ------------------------------------------------------------------------------------------
-    def render_tiles_training_records(self, x, width, height, tile, threshold, beta, temp):
+    def render_tiles_training_records(self, x, width, height, tile, threshold, beta, temp, *, render_order=False):
         """[rgb, alpha, ids, x6, raw, masks, gates, offsets]: one record per hit and pixel, in each
         pixel's compositing order.  ``x`` = the 15 scene tensors + two adjoint placeholders that the
-        forward-only mode never reads (scannet/csr_training.py:37-39)."""
+        forward-only mode never reads (scannet/csr_training.py:37-39).  ``render_order`` (not in the reference):
+        image and records in the rounding of ``render_tiles_forward_tilecenter`` instead of the record kernels'
+        own; see :meth:`records_forward_matches_render`."""
         name = "render_tiles_mlp_records"
         _chk(len(x) == 17, "Expected 15 scene inputs and RGB/T adjoints")
         width, height, tile = int(width), int(height), int(tile)
@@ -385,7 +387,17 @@ class TileExt:
                 order, _ = ops.sort_tiles(x[0], x[1], rec, x[5], x[6], width, height, tile, tile, _lib.KEY_TSTAR,
                                           self.max_tile_prims, cull_threshold=float(threshold))
             return list(ops.training_records(x[0], x[1], rec, order, x[6], x[7], x[8], *x[9:15], width, height, tile,
-                                             tile, float(threshold), float(beta), float(temp), self.max_hits, name))
+                                             tile, float(threshold), float(beta), float(temp), self.max_hits, name,
+                                             render_order=bool(render_order)))
+
+    @staticmethod
+    def records_forward_matches_render(freq, W1, b1, W2, b2, tile):
+        """True if ``render_tiles_training_records(..., render_order=True)`` is available for this frame: 8x8 tiles
+        and the 72->32->32->4 MLP with six frequencies in 16-byte aligned f32 tensors.  Its rgb/alpha are then the
+        bits of ``render_tiles_forward_tilecenter``, and a differentiable render can keep the records of its
+        forward pass for the backward instead of traversing the frame again."""
+        return (int(tile) == 8 and freq.numel() == 6 and tuple(W1.shape[1:]) == (32, 72) and tuple(W2.shape[1:]) == (32, 32)
+                and all(t.dtype == torch.float32 and t.is_contiguous() and t.data_ptr() % 16 == 0 for t in (W1, b1, W2, b2)))
 
     def training_wmma_safety_stats(self):
         """[calls, frame_fallbacks, fp32_nonfinite_failures, count_emit_failures, capacity_failures] of
@@ -515,8 +527,18 @@ class TileExt:
         _chk(int(TW) == int(TH), "square tiles only")
         x = [rays_o, rays_d, positions, log_scales, quats, cand, offsets, freq, att, W1, b1, W2, b2, W3, b3,
              grad_rgb.contiguous(), grad_t.contiguous()]
-        rgb, alpha, ids, x6, raw, masks, gates, pixel_offsets = self.render_tiles_training_records(
-            x, Wimg, Himg, TW, thr, 1.5, 2.0)
+        records = self.render_tiles_training_records(x, Wimg, Himg, TW, thr, 1.5, 2.0)
+        return self.backward_from_records(records, positions, log_scales, quats, freq, att, W1, b1, W2, b2, W3, b3,
+                                          x[15], x[16])
+
+    def backward_from_records(self, records, positions, log_scales, quats, freq, att, W1, b1, W2, b2, W3, b3,
+                              grad_rgb, grad_t):
+        """The nine gradients of :meth:`render_tiles_backward_tilecenter_full` from records that a forward pass
+        already holds (no counterpart in the reference, whose fused backward traverses the frame again)."""
+        from .primitive_csr import group_records, reference_weight_gradients
+        from . import primitive_gemm
+        rgb, alpha, ids, x6, raw, masks, gates, pixel_offsets = records
+        x = {15: grad_rgb.contiguous(), 16: grad_t.contiguous()}
         # reverse walk without atomics; the geometry sums are formed from the primitive-major order that the
         # weight gradients need anyway
         with torch.cuda.device(ids.device):

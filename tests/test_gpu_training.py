@@ -158,3 +158,56 @@ def test_fused_optimiser_steps_are_seen_by_the_next_render(device, oracle_mod, p
     assert torch.equal(after, expected)
     if [p._version for p in scene.parameters()] != versions:
         pytest.skip("this torch build advances the version in fused steps; the caches would have seen them anyway")
+
+
+def test_records_forward_in_render_order_is_the_render(device, oracle_mod):
+    """render_tiles_training_records(render_order=True): image and alpha are the bits of the f32 tile-centre render
+    (itself bit-exact against the oracle), the record topology is that of the ordinary records forward."""
+    from mlp_splatting_amd.tile_ext import TileExt
+    fr = Frame("cfg1_5k_160x120", n=1500, hidden=32, width=80, height=48)
+    cand, off = fr.oracle_lists(oracle_mod)
+    base = [to_dev(a, device) for a in fr.base_numpy(cand, off)]
+    x = base + [torch.zeros_like(base[0]), torch.zeros(fr.W * fr.H, device=device)]
+    ext = TileExt()
+    assert ext.records_forward_matches_render(base[7], base[9], base[10], base[11], base[12], 8)
+    rgb, alpha = ext.render_tiles_forward_tilecenter(*base, fr.W, fr.H, 8, 8, fr.thr)
+    kept = ext.render_tiles_training_records(x, fr.W, fr.H, 8, fr.thr, 1.5, 2.0, render_order=True)
+    plain = ext.render_tiles_training_records(x, fr.W, fr.H, 8, fr.thr, 1.5, 2.0)
+    assert kept[2].numel() > 5000
+    assert torch.equal(kept[0], rgb) and torch.equal(kept[1], alpha)
+    same_lists = torch.equal(kept[7], plain[7])
+    assert float((kept[7].diff() == plain[7].diff()).float().mean()) > 0.999
+    if same_lists:
+        for index in (2, 3, 6):
+            assert torch.equal(kept[index], plain[index])
+        torch.testing.assert_close(kept[4], plain[4], atol=2e-6, rtol=2e-6)
+    # other shapes are refused rather than silently rendered in the other rounding
+    fr16 = Frame("cfg1_5k_160x120", n=200, hidden=16, width=32, height=24)
+    cand16, off16 = fr16.oracle_lists(oracle_mod)
+    base16 = [to_dev(a, device) for a in fr16.base_numpy(cand16, off16)]
+    assert not ext.records_forward_matches_render(base16[7], base16[9], base16[10], base16[11], base16[12], 8)
+    x16 = base16 + [torch.zeros_like(base16[0]), torch.zeros(fr16.W * fr16.H, device=device)]
+    with pytest.raises(RuntimeError):
+        ext.render_tiles_training_records(x16, fr16.W, fr16.H, 8, fr16.thr, 1.5, 2.0, render_order=True)
+
+
+def test_gradients_with_and_without_kept_records_agree(device, oracle_mod, monkeypatch):
+    """The autograd forward that keeps its records against the one that renders first and re-traverses the frame
+    in the backward: same image bits, gradients equal to the rounding of the two record forwards."""
+    fr = Frame("cfg1_5k_160x120", n=600, hidden=32, width=32, height=24)
+    args = (to_dev(fr.rays_o, device), to_dev(fr.rays_d, device))
+    kw = dict(score_threshold=fr.thr, view_matrix=to_dev(fr.view, device), proj_matrix=to_dev(fr.proj, device))
+    torch.manual_seed(4)
+    weight = torch.randn(fr.W * fr.H, 3, device=device)
+    results = {}
+    for keep in ("1", "0"):
+        monkeypatch.setenv("MLPSP_AUTOGRAD_KEEP_RECORDS", keep)
+        scene = _scene_from(fr, device).train()
+        rgb = scene(*args, **kw)
+        (rgb * weight).sum().backward()
+        results[keep] = (rgb.detach(), {k: getattr(scene, k).grad.clone() for k in PARAMS})
+    assert torch.equal(results["1"][0], results["0"][0])
+    for k in PARAMS:
+        a, b = results["1"][1][k], results["0"][1][k]
+        assert float(b.abs().max()) > 0
+        assert float((a - b).abs().max()) <= 1e-4 * float(b.abs().max()), k
