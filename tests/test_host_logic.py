@@ -172,3 +172,47 @@ def test_mosaic_frame_quadrants_project_into_their_own_quadrant():
         clip = P @ (views[q] @ np.append(pt, 1.0))
         assert abs((clip[0] / clip[3] + 1) * W - px) < 1e-3 and abs((clip[1] / clip[3] + 1) * H - py) < 1e-3
         assert tv[(py // 8) * (2 * W // 8) + px // 8] == q
+
+
+def test_training_paths_leave_no_derived_tensor_behind():
+    """TileExt.uncached(): caches are emptied on entry and exit, nothing is kept inside, and nesting holds."""
+    from mlp_splatting_amd.tile_ext import TileExt
+    ext = TileExt()
+
+    def fill():
+        ext._pack_key, ext._pack = ("k",), object()
+        ext._rec_key, ext._rec = ("k",), object()
+        ext._feat_pack_key, ext._feat_pack = ("k",), object()
+
+    def empty():
+        return all(v is None for v in (ext._pack_key, ext._pack, ext._rec_key, ext._rec, ext._feat_pack_key, ext._feat_pack))
+
+    fill()
+    assert ext._caching() and not empty()
+    with ext.uncached():
+        assert empty() and not ext._caching()
+        fill()                                   # whatever a call inside might have stored ...
+        with ext.uncached():
+            assert empty() and not ext._caching()
+        assert not ext._caching()
+        fill()
+    assert empty() and ext._caching()            # ... is gone afterwards
+    fill()
+    with pytest.raises(ValueError):
+        with ext.uncached():
+            raise ValueError("a failing training call")
+    assert empty() and ext._caching()
+    ext._binned = ("lists", 7)
+    ext.invalidate_caches()
+    assert ext._binned == ("lists", 7)           # keyed on the list tensors, not on parameters
+
+
+def test_scene_invalidation_reaches_the_extension(monkeypatch):
+    from mlp_splatting_amd.tile_ext import TileExt
+    ext = TileExt()
+    monkeypatch.setattr(cumodel, "_tile_ext", ext)
+    scene = NeuralPrimitiveSceneTileCUDA(num_primitives=4, hidden_dim=32)
+    scene.__dict__["_mlpsp_cache"] = {"unit_quats": (("key",), object())}
+    ext._rec_key, ext._rec = ("k",), object()
+    scene.invalidate_render_caches()
+    assert "_mlpsp_cache" not in scene.__dict__ and ext._rec_key is None and ext._rec is None
