@@ -9,6 +9,13 @@
 #include "mlpsp_mlp.hpp"
 #include "mlpsp_mlp_mfma32.hpp"
 #include "mlpsp_render_f32.hpp"
+#include "mlpsp_record_stage.hpp"
+
+// records of a pixel staged in LDS before they are written (mlpsp_record_stage.hpp); 8x8 tiles on the matrix-core
+// path only -- the scalar shapes keep the direct stores
+#ifndef MLPSP_STAGE_K
+#define MLPSP_STAGE_K 2
+#endif
 
 namespace mlpsp {
 
@@ -22,6 +29,9 @@ struct RecordOut {
   float* rgb;                 // [B,3]
   float* alpha;               // [B,1]
 };
+
+template <bool STAGED> struct F32StageFor { using type = RecordStage<MLPSP_STAGE_K>; };
+template <> struct F32StageFor<false> { struct type {}; };
 
 // MF: the MLP of a hit runs on the matrix cores for the whole wavefront (mlp_wave_mfma32, same bits).
 // RORD (with MF only): layer 2 in the rounding order of the RENDER kernels instead of the record kernels', so
@@ -51,6 +61,12 @@ __global__ __launch_bounds__(64) void records_kernel(
   const int start = offsets[tile], end = offsets[tile + 1];
   long long rec_base = 0;
   if constexpr (EMIT) rec_base = valid ? out.offsets[pix] : 0;
+  // MF kernels run one wavefront per workgroup, which is what the staging needs
+  constexpr bool STAGED = EMIT && MF;
+  __shared__ typename F32StageFor<STAGED>::type s_stage;
+  const RecordArrays arrays{out.ids, out.x6, out.masks, out.raw, out.gates};
+  int pending = 0, flushed = 0;
+  if constexpr (STAGED) stage_begin(s_stage, (int)threadIdx.x, rdx, rdy, rdz);
 
   float trans = 1.f, cr = 0.f, cg = 0.f, cb = 0.f;
   int used = 0;
@@ -76,25 +92,31 @@ __global__ __launch_bounds__(64) void records_kernel(
         const float sigma = sigma_raw * h.decay;
         const float alpha = 1.f - det_exp(-sigma);
         if constexpr (EMIT) {
-          const long long r = rec_base + used;
-          out.ids[r] = p;
-#pragma unroll
-          for (int c = 0; c < 6; ++c) out.x6[r * 6 + c] = x6[c];
-          out.masks[r * 2] = (int32_t)mk[0];
-          out.masks[r * 2 + 1] = (int32_t)mk[1];
-          float* __restrict__ raw = out.raw + r * 8;
-          raw[0] = R;
-          raw[1] = G;
-          raw[2] = Bc;
-          raw[3] = sigma_raw;
-          raw[4] = trans;
-          raw[5] = alpha;
-          raw[6] = h.decay;
-          raw[7] = o[3];
           float gt[4];
           tetra_gates(h.qlx, h.qly, h.qlz, P.lgx, P.lgy, P.lgz, beta, temp, gt);
+          if constexpr (STAGED) {
+            const float rawv[8] = {R, G, Bc, sigma_raw, trans, alpha, h.decay, o[3]};
+            stage_put(s_stage, (int)threadIdx.x, pending, p, x6[3], x6[4], x6[5], mk[0], mk[1], rawv, gt);
+            ++pending;
+          } else {
+            const long long r = rec_base + used;
+            out.ids[r] = p;
 #pragma unroll
-          for (int k = 0; k < 4; ++k) out.gates[r * 4 + k] = gt[k];
+            for (int c = 0; c < 6; ++c) out.x6[r * 6 + c] = x6[c];
+            out.masks[r * 2] = (int32_t)mk[0];
+            out.masks[r * 2 + 1] = (int32_t)mk[1];
+            float* __restrict__ raw = out.raw + r * 8;
+            raw[0] = R;
+            raw[1] = G;
+            raw[2] = Bc;
+            raw[3] = sigma_raw;
+            raw[4] = trans;
+            raw[5] = alpha;
+            raw[6] = h.decay;
+            raw[7] = o[3];
+#pragma unroll
+            for (int k = 0; k < 4; ++k) out.gates[r * 4 + k] = gt[k];
+          }
           const float weight = trans * alpha;
           cr = fmaf(weight, R, cr);
           cg = fmaf(weight, G, cg);
@@ -104,9 +126,19 @@ __global__ __launch_bounds__(64) void records_kernel(
         ++used;
       }
     }
+    if constexpr (STAGED) {
+      if (__ballot(pending == MLPSP_STAGE_K) != 0ull) {
+        stage_flush(s_stage, (int)threadIdx.x, rec_base + flushed, pending, arrays);
+        flushed += pending;
+        pending = 0;
+      }
+    }
     const bool live = valid && (trans >= kTransmittanceFloor);
     over |= live && (used >= max_hits);      // np_tile_kernels.cu:3166-3168: refused, never truncated silently
     if (__ballot(live) == 0ull) break;
+  }
+  if constexpr (STAGED) {
+    if (__ballot(pending > 0) != 0ull) stage_flush(s_stage, (int)threadIdx.x, rec_base + flushed, pending, arrays);
   }
   if (__ballot(over) != 0ull && threadIdx.x == 0) atomicExch(overflow, 1);
   if (valid) {

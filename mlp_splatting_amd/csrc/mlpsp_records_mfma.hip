@@ -21,6 +21,12 @@
 #include "mlpsp_device.hpp"
 #include "mlpsp_host.hpp"
 #include "mlpsp_mfma16.hpp"
+#include "mlpsp_record_stage.hpp"
+
+// records of a pixel staged in LDS before they are written (mlpsp_record_stage.hpp)
+#ifndef MLPSP_STAGE_K
+#define MLPSP_STAGE_K 2
+#endif
 
 namespace mlpsp {
 
@@ -39,6 +45,9 @@ struct MixedRecordOut {
 };
 
 __device__ __forceinline__ bool not_finite(float v) { return !(__builtin_fabsf(v) <= 3.4028235e38f); }
+
+template <bool EMIT> struct StageFor { using type = RecordStage<MLPSP_STAGE_K>; };
+template <> struct StageFor<false> { struct type {}; };
 
 // One read-only pass over up to 16 f32 arrays; flag[0] |= 1 if any element is NaN or infinite
 // (training_wmma.cuh:24-60: one fused scan and one read-back instead of a reduction per tensor).
@@ -92,9 +101,12 @@ __device__ __forceinline__ void records_mfma_body(
   encode_direction_words<T>(rdx, rdy, rdz, kf, l, s_dir);
 
   long long rec_base = 0;
-  int expected = 0;
+  int expected = 0, pending = 0, flushed = 0;
   bool mismatch = false;
+  __shared__ typename StageFor<EMIT>::type s_stage;
+  const RecordArrays arrays{out.ids, out.x6, out.masks, out.raw, out.gates};
   if constexpr (EMIT) {
+    stage_begin(s_stage, l, rdx, rdy, rdz);
     if (valid) {
       rec_base = out.offsets[pix];
       const long long rec_end = out.offsets[pix + 1];
@@ -131,31 +143,12 @@ __device__ __forceinline__ void records_mfma_body(
         bad |= not_finite((o[0] + o[1]) + (o[2] + o[3])) || not_finite((R + G) + (Bc + sigma_raw)) || not_finite(alpha);
         if constexpr (EMIT) {
           if (used < expected) {
-            const long long r = rec_base + used;
-            out.ids[r] = p;
-            float* __restrict__ xr = out.x6 + r * 6;
-            xr[0] = rdx;
-            xr[1] = rdy;
-            xr[2] = rdz;
-            xr[3] = dx;
-            xr[4] = dy;
-            xr[5] = dz;
-            out.masks[r * 2] = (int32_t)mk[0];
-            out.masks[r * 2 + 1] = (int32_t)mk[1];
-            float* __restrict__ raw = out.raw + r * 8;
-            raw[0] = R;
-            raw[1] = G;
-            raw[2] = Bc;
-            raw[3] = sigma_raw;
-            raw[4] = trans;
-            raw[5] = alpha;
-            raw[6] = h.decay;
-            raw[7] = o[3];
+            const float rawv[8] = {R, G, Bc, sigma_raw, trans, alpha, h.decay, o[3]};
             float gt[4];
             tetra_gates(h.qlx, h.qly, h.qlz, P.lgx, P.lgy, P.lgz, beta, temp, gt);
             bad |= not_finite((gt[0] + gt[1]) + (gt[2] + gt[3]));
-#pragma unroll
-            for (int k = 0; k < 4; ++k) out.gates[r * 4 + k] = gt[k];
+            stage_put(s_stage, l, pending, p, dx, dy, dz, mk[0], mk[1], rawv, gt);
+            ++pending;
           } else {
             mismatch = true;
           }
@@ -169,11 +162,20 @@ __device__ __forceinline__ void records_mfma_body(
         bad |= not_finite(trans);
       }
     }
+    if constexpr (EMIT) {
+      // a pixel's interval holds `expected` records and `flushed + pending` never exceeds it
+      if (__ballot(pending == MLPSP_STAGE_K) != 0ull) {
+        stage_flush(s_stage, l, rec_base + flushed, pending, arrays);
+        flushed += pending;
+        pending = 0;
+      }
+    }
     const bool live = valid && (trans >= kTransmittanceFloor);
     over |= live && (used >= max_hits);      // refused, never truncated silently (training_wmma.cuh:243-244)
     if (__ballot(live) == 0ull) break;
   }
   if constexpr (EMIT) {
+    if (__ballot(pending > 0) != 0ull) stage_flush(s_stage, l, rec_base + flushed, pending, arrays);
     mismatch |= valid && (used != expected);
     bad |= not_finite((cr + cg) + cb);
   }
@@ -205,7 +207,9 @@ __device__ __forceinline__ void records_mfma_body(
       temp, counts, status, out
 
 // The count pass fits 128 registers without spilling: four wavefronts per SIMD (measured 1.19 -> 1.12 ms at
-// 200k primitives).  The emit pass needs 146; capped at 128 it spills 20 and measured slower (3.6 -> 3.8 ms).
+// 200k primitives).  The emit pass does not (capped at 128 it spills and measured slower), and its staging area
+// limits it to two wavefronts per SIMD; staged stores still win: 3.6 -> 3.0 ms, HBM writes 7.0 -> 4.2 GB and
+// re-fetched weights 2.9 -> 1.0 GB per launch (K = 4 measures the same as K = 2 and holds more LDS).
 template <typename T>
 __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 4))) void records_mfma_count_kernel(MLPSP_RECM_PARAMS) {
   records_mfma_body<T, false>(MLPSP_RECM_ARGS);
