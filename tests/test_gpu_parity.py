@@ -394,11 +394,14 @@ def test_statistics_forward_against_oracle(device, oracle_mod, tile, hidden):
     assert np.array_equal(st2[2].cpu().numpy(), want["hits"])
 
 
-@pytest.mark.parametrize("tile,hidden,n", [(8, 32, 1500), (16, 16, 2500), (8, 8, 900)])
-def test_training_records_are_bit_exact(device, oracle_mod, tile, hidden, n):
-    # np_tile_kernels.cu:2925-3206 (record modes 1/3): counts, order, every record field, rgb, alpha
+@pytest.mark.parametrize("tile,hidden,n,size", [(8, 32, 1500, (72, 48)), (16, 16, 2500, (72, 48)), (8, 8, 900, (72, 48)),
+                                                (16, 32, 2000, (72, 48)), (8, 32, 1500, (69, 43)), (16, 32, 1200, (37, 50))])
+def test_training_records_are_bit_exact(device, oracle_mod, tile, hidden, n, size):
+    # np_tile_kernels.cu:2925-3206 (record modes 1/3): counts, order, every record field, rgb, alpha; 8x8 and 16x16
+    # tiles, scalar and matrix-core MLP (the latter stages its records in LDS before writing them), image sizes that
+    # are and are not multiples of the tile
     from mlp_splatting_amd.tile_ext import TileExt
-    fr = Frame("cfg1_5k_160x120", n=n, hidden=hidden, width=72, height=48, tile=tile)
+    fr = Frame("cfg1_5k_160x120", n=n, hidden=hidden, width=size[0], height=size[1], tile=tile)
     cand, off = fr.oracle_lists(oracle_mod)
     want = oracle_mod.records(*fr.base_numpy(cand, off), *fr.dims, max_hits=512, beta=1.3, temp=2.2)
     x = [_t(a, device) for a in fr.base_numpy(cand, off)]
@@ -406,7 +409,7 @@ def test_training_records_are_bit_exact(device, oracle_mod, tile, hidden, n):
     ext = TileExt()
     rgb, alpha, ids, x6, raw, masks, gates, offsets = ext.render_tiles_training_records(x, fr.W, fr.H, tile, fr.thr, 1.3, 2.2)
     assert offsets.dtype == torch.int64 and np.array_equal(offsets.cpu().numpy(), want["offsets"])
-    assert want["offsets"][-1] > 5000 and np.array_equal(ids.cpu().numpy(), want["ids"])
+    assert want["offsets"][-1] > 3000 and np.array_equal(ids.cpu().numpy(), want["ids"])
     assert np.array_equal(masks.cpu().numpy(), want["masks"])
     for got, key in ((rgb, "rgb"), (alpha, "alpha"), (x6, "x6"), (raw, "raw"), (gates, "gates")):
         _assert_bits(got, want[key], key)
