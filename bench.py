@@ -204,9 +204,9 @@ def main() -> int:
         render(i)
         torch.cuda.synchronize()
         lat.append((time.perf_counter() - t1) * 1e3)
-    lat = np.sort(np.asarray(lat))
-    latency = {"mean_ms": round(float(lat.mean()), 4), "median_ms": round(float(np.median(lat)), 4),
-               "p95_ms": round(float(lat[min(len(lat) - 1, int(0.95 * len(lat)))]), 4), "frames": int(len(lat))}
+    from mlp_splatting_amd.harness import timing_stats
+    latency = {k: (round(v, 4) if isinstance(v, float) else v) for k, v in timing_stats(lat).items()}
+    latency["frames"] = latency.pop("samples")
 
     # ---- the render kernel alone: HIP events on the stream it is launched on, and its work counters
     freq, att = scene._frequency_tables(dev)

@@ -282,3 +282,31 @@ def test_queued_frames_equal_step_by_step_frames(device, oracle_mod, monkeypatch
     cumodel._tile_ext.max_tile_prims = longest - 1
     with pytest.raises(RuntimeError, match=f"capacity {longest - 1} exceeded \\(maximum observed tile length {longest}\\)"):
         _call(scene, fr, device)
+
+
+def test_harness_renders_times_and_scores_a_view(device, oracle_mod):
+    """mlp_splatting_amd.harness: the timed view of tools/benchmark_inference.py:121-149, its statistics, PSNR and
+    the RGB parity of the feature render, on a frame whose image the oracle pins."""
+    from mlp_splatting_amd import harness
+    fr = Frame("cfg1_5k_160x120", n=800, width=40, height=24, feature_dim=64)
+    scene = _scene_from(fr, device, feature=True).eval()
+    frame = (to_dev(fr.rays_o, device), to_dev(fr.rays_d, device), to_dev(fr.view, device), to_dev(fr.proj, device),
+             fr.W, fr.H, fr.thr)
+    rgb, wall_ms, device_ms, shape = harness.render_view(scene, *frame)
+    assert tuple(rgb.shape) == (fr.H, fr.W, 3) and shape is None and wall_ms > 0 and 0 < device_ms <= wall_ms * 1.5
+    cand, off = fr.oracle_lists(oracle_mod)
+    sc = fr.scene
+    # the oracle is fed the module's own normalised directions, quaternions and frequency tables, as above
+    q = torch.nn.functional.normalize(to_dev(sc.quats, device), dim=-1).cpu().numpy()
+    rd = torch.nn.functional.normalize(to_dev(fr.rays_d, device), dim=-1).cpu().numpy()
+    freq, att = (t.cpu().numpy() for t in scene._frequency_tables(device))
+    want = oracle_mod.render_tilecenter(fr.rays_o, rd, sc.positions, sc.log_scales, q, cand, off, freq, att, *sc.mlp(),
+                                        *fr.dims)["rgb"].reshape(fr.H, fr.W, 3).clip(0.0, 1.0)
+    assert np.array_equal(rgb.cpu().numpy(), want)
+    _, _, _, shape = harness.render_view(scene, *frame, return_feature=True)
+    assert shape == [fr.W * fr.H, 64]
+    assert harness.rgb_parity_with_features(scene, *frame) == 0.0
+    q = harness.quality([rgb, rgb], [torch.from_numpy(want).to(device), (rgb + 0.1)])
+    assert q["per_view_psnr_db"][0] == float("inf") and abs(q["per_view_psnr_db"][1] - 20.0) < 1e-4
+    st = harness.timing_stats([harness.render_view(scene, *frame)[1] for _ in range(5)])
+    assert st["samples"] == 5 and st["mean_ms"] > 0 and st["std_ms"] >= 0

@@ -216,3 +216,23 @@ def test_scene_invalidation_reaches_the_extension(monkeypatch):
     ext._rec_key, ext._rec = ("k",), object()
     scene.invalidate_render_caches()
     assert "_mlpsp_cache" not in scene.__dict__ and ext._rec_key is None and ext._rec is None
+
+
+def test_harness_statistics_closed_forms():
+    from mlp_splatting_amd.harness import quality, timing_stats
+    st = timing_stats([1.0, 2.0, 3.0, 4.0, 10.0])
+    assert st["samples"] == 5 and st["mean_ms"] == 4.0 and st["median_ms"] == 3.0
+    assert math.isclose(st["std_ms"], math.sqrt(50.0 / 4.0)) and math.isclose(st["coefficient_of_variation"], st["std_ms"] / 4.0)
+    assert math.isclose(st["p95_ms"], 8.8) and st["fps_from_mean"] == 250.0 and math.isclose(st["fps_from_median"], 1000.0 / 3.0)
+    assert timing_stats([2.5])["std_ms"] == 0.0
+    with pytest.raises(ValueError):
+        timing_stats([])
+    # a uniform error of 0.1 is 20 dB, of 0.01 is 40 dB; pooled: mse = (0.01 + 0.0001) / 2
+    a, b = torch.zeros(4, 5, 3), torch.zeros(2, 2, 3)
+    q = quality([a + 0.1, b + 0.01, b], [a, b, b])
+    assert math.isclose(q["per_view_psnr_db"][0], 20.0, abs_tol=1e-5) and math.isclose(q["per_view_psnr_db"][1], 40.0, abs_tol=1e-4)
+    assert q["per_view_psnr_db"][2] == float("inf") and q["median_psnr_db"] == q["per_view_psnr_db"][1]
+    pooled = (60 * 0.01 + 12 * 0.0001) / (60 + 12 + 12)
+    assert math.isclose(q["global_psnr_db"], -10.0 * math.log10(pooled), abs_tol=1e-5)
+    with pytest.raises(ValueError):
+        quality([a], [])
