@@ -131,6 +131,11 @@ def main() -> int:
     feature_dim = int(syn.CONFIGS[args.workload]["feature_dim"])
     sc, cfg = syn.scene_for_config(args.workload, with_features=False)
     W, H, f, thr = cfg["width"], cfg["height"], cfg["focal"], cfg["threshold"]
+    if precision == "bf16" and sc.hidden != 32:
+        if args.precision == "bf16":
+            print(f"--precision bf16 needs the 72->32->32->4 MLP; {args.workload} has hidden width {sc.hidden}", file=sys.stderr)
+            return 2
+        precision = "f32"        # the matrix-core render exists for the released MLP width only (as the reference's)
     mosaic = args.workload.startswith("cfg4")
 
     def t(a):
