@@ -284,7 +284,7 @@ def main() -> int:
     stream = torch.cuda.current_stream(dev).cuda_stream
     sink = torch.zeros(1, device=dev)
     probe_ms = []
-    for mode in range(4):
+    for mode in range(5):
         lib.mlpsp_probe_issue(mode, 500, sink.data_ptr(), stream)
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
@@ -296,7 +296,9 @@ def main() -> int:
     issue_probe = {"mfma_ms": round(probe_ms[0], 4), "valu_ms": round(probe_ms[1], 4), "mixed_ms": round(probe_ms[2], 4),
                    "mixed_if_serial_ms": round(serial, 4), "mixed_if_overlapped_ms": round(ideal, 4),
                    "overlap": round((serial - probe_ms[2]) / max(serial - ideal, 1e-9), 3),
-                   "sin_issue_vs_fma": round((probe_ms[3] / 2.0) / (probe_ms[1] / 8.0), 2)}
+                   "sin_issue_vs_fma": round((probe_ms[3] / 2.0) / (probe_ms[1] / 8.0), 2),
+                   "same_wavefront_ms": round(probe_ms[4], 4),
+                   "same_wavefront_vs_serial": round(probe_ms[4] / (probe_ms[0] + probe_ms[1]), 3)}
     flops_per_hit = 2 * (72 * sc.hidden + sc.hidden * sc.hidden + 4 * sc.hidden)
     achieved_tflops = flops_per_hit * hits / (kernel_ms * 1e-3) / 1e12
     # sort kernel: 8 compulsory bytes per candidate (4 id in, 4 id out) + the 64-byte record of every primitive

@@ -411,10 +411,13 @@ int64_t mlpsp_probe_mfma_bf16(int iterations, float* sink_dev, mlpsp_stream_t st
 
 /* Measurement aid, no counterpart in the reference: 256 workgroups of 8 wavefronts (two per SIMD) run
  * `iterations` rounds of  mode 0: one 32x32x16 bf16 MFMA,  mode 1: eight independent f32 FMAs,
- * mode 2: the MFMA in one wavefront of every SIMD and the FMAs in the other,  mode 3: two v_sin_f32.
- * Timed on the stream, modes 0-2 show whether the matrix pipe and the vector ALU of a SIMD overlap (they
- * do not: mode 2 takes about half the sum of modes 0 and 1, not half their maximum), mode 3 the issue rate
- * of transcendentals.  Returns 0 or an MLPSP_E_* code.  sink_dev: one float, left untouched in practice. */
+ * mode 2: the MFMA in one wavefront of every SIMD and the FMAs in the other,  mode 3: two v_sin_f32,
+ * mode 4: the MFMA and the eight FMAs, independent of each other, in every wavefront.
+ * Timed on the stream, modes 0-2 show whether the matrix pipe and the vector ALU of a SIMD overlap across
+ * wavefronts (they do not: mode 2 takes about half the sum of modes 0 and 1, not half their maximum), mode 4
+ * how much of an MFMA the following vector instructions of the SAME wavefront hide (about 12 of its 32
+ * cycles: mode 4 takes ~0.72 of modes 0 + 1), mode 3 the issue rate of transcendentals.
+ * Returns 0 or an MLPSP_E_* code.  sink_dev: one float, left untouched in practice. */
 int mlpsp_probe_issue(int mode, int iterations, float* sink_dev, mlpsp_stream_t stream);
 
 #ifdef __cplusplus

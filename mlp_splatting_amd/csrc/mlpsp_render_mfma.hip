@@ -458,7 +458,10 @@ __global__ __launch_bounds__(256) void probe_mfma_bf16_kernel(int iterations, fl
 // f32 FMAs per iteration (32 cycles of the vector ALU); mode 2: on every SIMD one wavefront does the
 // former and one the latter; mode 3: all issue 2 v_sin_f32 per iteration.  If the two pipes overlapped,
 // mode 2 would take as long as the slower of modes 0 and 1 run with one wavefront per SIMD, i.e. half of
-// their two-wavefront times; it takes about the sum.
+// their two-wavefront times; it takes about the sum.  mode 4: every wavefront issues the MFMA and then the 8
+// FMAs, independent of each other: ~0.72 of modes 0 + 1 -- vector instructions that FOLLOW an MFMA in the
+// same wavefront do start before it has finished (about 12 of its 32 cycles), which the render kernel's
+// instruction order already uses (operand preparation for the next MFMA sits behind the current one).
 __global__ __launch_bounds__(512) void probe_issue_kernel(int mode, int iterations, float* __restrict__ sink) {
   const int wave = threadIdx.x >> 6;
   const bool do_mfma = mode == 0 || (mode == 2 && wave < 4);
@@ -480,6 +483,13 @@ __global__ __launch_bounds__(512) void probe_issue_kernel(int mode, int iteratio
     for (int it = 0; it < iterations; ++it) {
       v[0] = __builtin_amdgcn_sinf(v[0]);
       v[1] = __builtin_amdgcn_sinf(v[1]);
+    }
+  }
+  if (mode == 4) {      // both in every wavefront, independent of each other
+    for (int it = 0; it < iterations; ++it) {
+      acc = Ops<__bf16>::mfma(a, b, acc);
+#pragma unroll
+      for (int k = 0; k < 8; ++k) v[k] = fmaf(v[k], m, c);
     }
   }
   float r = acc[0];
@@ -643,7 +653,7 @@ MLPSP_API int64_t mlpsp_probe_mfma_bf16(int iterations, float* sink_dev, mlpsp_s
 }
 
 MLPSP_API int mlpsp_probe_issue(int mode, int iterations, float* sink_dev, mlpsp_stream_t stream) {
-  if (mode < 0 || mode > 3 || iterations <= 0 || !sink_dev) return MLPSP_E_ARGUMENT;
+  if (mode < 0 || mode > 4 || iterations <= 0 || !sink_dev) return MLPSP_E_ARGUMENT;
   hipLaunchKernelGGL(probe_issue_kernel, dim3(256), dim3(512), 0, (hipStream_t)stream, mode, iterations, sink_dev);
   MLPSP_LAUNCH_CHECK();
   return MLPSP_OK;
