@@ -403,6 +403,22 @@ int mlpsp_feature_attribute_gradients(const int8_t* signs_dev, const int64_t* re
                                       int target_height, int channels, int slots, int segment, int mixed,
                                       float* partial_dev, float* out_dev, mlpsp_stream_t stream);
 
+/* Adjoint of the dense feature image with respect to the attributes = render_tiles_backward_featattr_tilecenter
+ * (scannet/cuda/np_tile_kernels.cu:3531-3760, wrapper :6537-6620; called from _TileRenderWithFeatAutogradFn.backward,
+ * scannet/cumodel.py:466-477): out[p, slot, c] = sum over the primitive's records of T * alpha * gate_slot *
+ * grad_feat[record's pixel, c] (one slot: no gate; five slots: slot 0 has no gate).  The reference traverses the
+ * frame again and adds with atomics; here the records saved by the records forward are used, in the layout of
+ * mlpsp_feature_attribute_gradients (record_indices, record_pixels, csr_offsets, segments), and summed in a fixed
+ * order.  grad_feat_dev [pixels, channels] f32; gates_dev may be NULL for one slot.
+ * partial_dev [mlpsp_segment_reduce_rows(num_groups), slots, channels] is scratch, out_dev [N, slots, channels]. */
+int mlpsp_feature_dense_attribute_gradients(const float* grad_feat_dev, const int64_t* record_indices_dev,
+                                            const int32_t* record_pixels_dev, const float* raw_dev,
+                                            const float* gates_dev, const int64_t* csr_offsets_dev,
+                                            const int64_t* group_primitives_dev, const int64_t* group_starts_dev,
+                                            const int64_t* group_offsets_dev, int64_t num_groups, int num_primitives,
+                                            int channels, int slots, int segment, float* partial_dev, float* out_dev,
+                                            mlpsp_stream_t stream);
+
 /* Measurement aid, no counterpart in the reference: launches a kernel that does nothing but
  * v_mfma_f32_32x32x16_bf16 on register operands (2,048 workgroups x 4 wavefronts x iterations x 8
  * instructions) and returns the FLOPs it issues (-1 on error); time it on the stream to see what the

@@ -70,6 +70,8 @@ SIGNATURES = {
     "mlpsp_stream_feature_l1": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp]),
     "mlpsp_feature_attribute_gradients": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i, _i, _i, _i, _i, _i,
                                                _i, _i, _i, _vp, _vp, _vp]),
+    "mlpsp_feature_dense_attribute_gradients": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i, _i, _i, _i,
+                                                     _vp, _vp, _vp]),
     "mlpsp_records_reverse_adjoints": (_i, [_vp, _vp, _vp, _vp, _vp, _i64, _vp, _vp, _vp]),
     "mlpsp_geometry_gradients": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i, _i, _vp, _vp, _vp, _vp,
                                       _vp]),

@@ -261,6 +261,109 @@ __global__ __launch_bounds__(64) void feature_vjp_kernel(const int8_t* __restric
       if (c0 + k < C) partial[(group * SLOTS + sl) * C + c0 + k] = (sl < 4 ? acc[k][sl] : acc5[k][0]) / norm;
 }
 
+// Dense adjoint of the feature image (render_tiles_backward_featattr_tilecenter, np_tile_kernels.cu:3531-3760):
+// accum[slot][channel] += (T alpha gate_slot)[record] * grad_feat[record's pixel, channel] -- the adjoint of
+// the feature image reaches the attributes only, geometry, alpha and gates are constants of it.  The reference
+// walks the frame again and adds with atomics in launch order; here the saved records of a primitive are summed
+// per segment in record order (f32 fma on the 4x4 matrix-core blocks, as feature_vjp_kernel's exact mode) and the
+// segments by the fixed tree of the segmented reduction, so the result does not depend on scheduling.
+// One wavefront = one segment x 256 channels; VEC (C % 4 == 0 and a 16-byte aligned image): one load per record.
+template <int SLOTS, bool VEC>
+__global__ __launch_bounds__(64) void feature_dense_vjp_kernel(const float* __restrict__ grad_feat,
+                                                               const long long* __restrict__ order,
+                                                               const int32_t* __restrict__ record_pixels,
+                                                               const float* __restrict__ raw,
+                                                               const float* __restrict__ gates,
+                                                               const long long* __restrict__ offsets,
+                                                               const long long* __restrict__ group_prim,
+                                                               const long long* __restrict__ group_start,
+                                                               float* __restrict__ partial, int C, int segment) {
+  constexpr int ROWS = SLOTS == 5 ? 8 : 4;
+  __shared__ long long s_row[64];                                       // pixel * C of the staged records
+  __shared__ __attribute__((aligned(16))) float s_a[ROWS][64];          // factors, [slot][record]
+  const long long group = blockIdx.x;
+  const int lane = threadIdx.x, m = lane & 3;
+  const int c0 = blockIdx.y * 256 + lane * 4;
+  const long long p = group_prim[group];
+  const long long begin = group_start[group];
+  const long long seg_end = begin + segment, list_end = offsets[p + 1];
+  const long long end = seg_end < list_end ? seg_end : list_end;
+  int cc[4];
+#pragma unroll
+  for (int k = 0; k < 4; ++k) cc[k] = c0 + k < C ? c0 + k : C - 1;
+  const int cv = c0 + 3 < C ? c0 : 0;
+  ff4 acc[4], acc5[4];                                // [channel of the lane][slot]; acc5[.][0] = fifth slot
+#pragma unroll
+  for (int k = 0; k < 4; ++k) acc[k] = acc5[k] = ff4{0.f, 0.f, 0.f, 0.f};
+  auto fetch = [&](int rec, float (&v)[4]) {
+    const float* __restrict__ src = grad_feat + s_row[rec];
+    if constexpr (VEC) {
+      const float4 q = *reinterpret_cast<const float4*>(src + cv);
+      v[0] = q.x, v[1] = q.y, v[2] = q.z, v[3] = q.w;
+    } else {
+#pragma unroll
+      for (int k = 0; k < 4; ++k) v[k] = src[cc[k]];
+    }
+  };
+  for (long long base = begin; base < end; base += 64) {
+    const long long row = base + lane;
+    {
+      float a[ROWS];
+#pragma unroll
+      for (int i = 0; i < ROWS; ++i) a[i] = 0.f;
+      long long pixel_row = 0;
+      if (row < end) {
+        const long long r = order[row];
+        pixel_row = (long long)record_pixels[r] * C;
+        const float w = raw[r * 8 + 4] * raw[r * 8 + 5];
+#pragma unroll
+        for (int sl = 0; sl < SLOTS; ++sl) {
+          float g = 1.f;
+          if constexpr (SLOTS == 4) g = gates[r * 4 + sl];
+          if constexpr (SLOTS == 5) g = (sl == 0) ? 1.f : gates[r * 4 + sl - 1];
+          a[sl] = w * g;
+        }
+      }
+      s_row[lane] = pixel_row;
+#pragma unroll
+      for (int i = 0; i < ROWS; ++i) s_a[i][lane] = a[i];
+    }
+    __syncthreads();
+    const int count = (int)((end - base) < 64 ? (end - base) : 64);
+    // the adjoint rows of the NEXT four records are requested before the current four are used
+    float ahead[4][4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) fetch(q, ahead[q]);
+    for (int rr = 0; rr < count; rr += 4) {
+      float now[4][4];
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+#pragma unroll
+        for (int k = 0; k < 4; ++k) now[q][k] = (rr + q < count) ? ahead[q][k] : 0.f;   // an empty record adds +0
+      if (rr + 4 < count) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) fetch(rr + 4 + q, ahead[q]);
+      }
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const float a_op = s_a[m][rr + q];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          acc[k] = __builtin_amdgcn_mfma_f32_4x4x1f32(a_op, now[q][k], acc[k], 0, 0, 0);
+          if constexpr (SLOTS == 5)
+            acc5[k] = __builtin_amdgcn_mfma_f32_4x4x1f32(s_a[4 + m][rr + q], now[q][k], acc5[k], 0, 0, 0);
+        }
+      }
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int sl = 0; sl < SLOTS; ++sl)
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+      if (c0 + k < C) partial[(group * SLOTS + sl) * C + c0 + k] = sl < 4 ? acc[k][sl] : acc5[k][0];
+}
+
 }  // namespace mlpsp
 
 using namespace mlpsp;
@@ -340,6 +443,51 @@ MLPSP_API int mlpsp_feature_attribute_gradients(const int8_t* signs_dev, const i
     MLPSP_LAUNCH_CHECK();
   }
   // out[p] = sum over the primitive's segments (_feature_reduce, :152-161)
+  if (num_primitives > 0) {
+    ReduceDest dest{};
+    dest.packed = out_dev;
+    const int rc = segment_reduce<false>(partial_dev, group_primitives_dev, group_offsets_dev, num_groups, num_primitives,
+                                         (int64_t)slots * channels, dest, nullptr, s);
+    if (rc != MLPSP_OK) return rc;
+  }
+  return MLPSP_OK;
+}
+
+MLPSP_API int mlpsp_feature_dense_attribute_gradients(const float* grad_feat_dev, const int64_t* record_indices_dev,
+                                                      const int32_t* record_pixels_dev, const float* raw_dev,
+                                                      const float* gates_dev, const int64_t* csr_offsets_dev,
+                                                      const int64_t* group_primitives_dev,
+                                                      const int64_t* group_starts_dev, const int64_t* group_offsets_dev,
+                                                      int64_t num_groups, int num_primitives, int channels, int slots,
+                                                      int segment, float* partial_dev, float* out_dev,
+                                                      mlpsp_stream_t stream) {
+  if (channels <= 0 || segment <= 0 || num_groups < 0 || num_groups > 2147483647LL || num_primitives < 0)
+    return MLPSP_E_ARGUMENT;
+  if (slots != 1 && slots != 4 && slots != 5) return MLPSP_E_ARGUMENT;
+  if (slots != 1 && num_groups > 0 && !gates_dev) return MLPSP_E_ARGUMENT;
+  hipStream_t s = (hipStream_t)stream;
+  if (num_groups > 0) {
+    if (!grad_feat_dev || !record_indices_dev || !record_pixels_dev || !raw_dev || !csr_offsets_dev ||
+        !group_primitives_dev || !group_starts_dev || !partial_dev)
+      return MLPSP_E_ARGUMENT;
+    const dim3 grid((unsigned)num_groups, (unsigned)((channels + 255) / 256)), block(64);
+#define MLPSP_FD_LAUNCH(SL, VC)                                                                                    \
+  hipLaunchKernelGGL((feature_dense_vjp_kernel<SL, VC>), grid, block, 0, s, grad_feat_dev,                         \
+                     (const long long*)record_indices_dev, record_pixels_dev, raw_dev, gates_dev,                  \
+                     (const long long*)csr_offsets_dev, (const long long*)group_primitives_dev,                    \
+                     (const long long*)group_starts_dev, partial_dev, channels, segment)
+#define MLPSP_FD_SLOTS(VC)                         \
+  do {                                             \
+    if (slots == 1) MLPSP_FD_LAUNCH(1, VC);        \
+    else if (slots == 4) MLPSP_FD_LAUNCH(4, VC);   \
+    else MLPSP_FD_LAUNCH(5, VC);                   \
+  } while (0)
+    if ((channels % 4 == 0) && (reinterpret_cast<uintptr_t>(grad_feat_dev) % 16 == 0)) MLPSP_FD_SLOTS(true);
+    else MLPSP_FD_SLOTS(false);
+#undef MLPSP_FD_SLOTS
+#undef MLPSP_FD_LAUNCH
+    MLPSP_LAUNCH_CHECK();
+  }
   if (num_primitives > 0) {
     ReduceDest dest{};
     dest.packed = out_dev;

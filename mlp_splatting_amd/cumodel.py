@@ -243,7 +243,7 @@ class _TileRenderAutogradFn(torch.autograd.Function):
             grad_t_end = (grad_out_rgb * bg.view(1, 3)).sum(dim=-1)
         if ctx.mode != 1:
             raise NotImplementedError("the backward of the per-pixel order render is not built; train with the "
-                                      "tile-centre order (MLPSP_TILE_ORDER_MODE=tilecenter, the default)")
+                                      "tile-centre order (MLPSP_TILE_ORDER=tilecenter, the default)")
         ext = NeuralPrimitiveSceneTileCUDA._ensure_tile_ext_static()
         if ctx.has_records:
             gW1, gb1, gW2, gb2, gW3, gb3, gp, gs, gq = ext.backward_from_records(
@@ -253,6 +253,67 @@ class _TileRenderAutogradFn(torch.autograd.Function):
                 *args, grad_out_rgb, grad_t_end, *ctx.dims)
         return (None, None, gp, gs, gq, None, None, None, None, gW1, gb1, gW2, gb2, gW3, gb3,
                 None, None, None, None, None, None, None)
+
+
+class _TileRenderWithFeatAutogradFn(torch.autograd.Function):
+    """(rgb, feature image) in tile-centre order with gradients (scannet/cumodel.py:381-489): the RGB adjoint reaches
+    geometry and MLP weights as in :class:`_TileRenderAutogradFn`, the feature adjoint reaches ``feat_attr`` only.
+    An output without an adjoint contributes nothing (``set_materialize_grads(False)``), so its parameters get
+    ``None`` and an optimizer leaves them and their moments alone.  The backward runs the records forward once and
+    serves both adjoints from it."""
+
+    @staticmethod
+    def forward(ctx, rays_o, rays_d, positions, log_scales, quats, culled_prim_indices, tile_offsets, freq, att,
+                W1, b1, W2, b2, W3, b3, feat_attr, gating_beta, gating_temp, Wimg, Himg, TW, TH, threshold, bg_color):
+        ext = NeuralPrimitiveSceneTileCUDA._ensure_tile_ext_static()
+        args = (rays_o, rays_d, positions, log_scales, quats, culled_prim_indices, tile_offsets, freq, att,
+                W1, b1, W2, b2, W3, b3)
+        dims = (int(Wimg), int(Himg), int(TW), int(TH), float(threshold))
+        with _uncached(ext):
+            rgb, alpha, feat = ext.render_tiles_forward_tilecenter_with_feat(*args, feat_attr, float(gating_beta),
+                                                                             float(gating_temp), *dims)
+        rgb = _add_background(rgb, alpha, bg_color)
+        ctx.save_for_backward(*args, feat_attr)
+        ctx.dims, ctx.bg_color, ctx.gating = dims, bg_color, (float(gating_beta), float(gating_temp))
+        ctx.set_materialize_grads(False)
+        return rgb, feat
+
+    @staticmethod
+    def backward(ctx, grad_out_rgb, grad_out_feat):
+        args, feat_attr = ctx.saved_tensors[:15], ctx.saved_tensors[15]
+        ext = NeuralPrimitiveSceneTileCUDA._ensure_tile_ext_static()
+        W, H, TW, TH, thr = ctx.dims
+        grads = [None] * 9
+        grad_attr = None
+        if grad_out_rgb is None and grad_out_feat is None:
+            return (None,) * 24
+        if grad_out_feat is not None:
+            grad_out_feat = grad_out_feat.contiguous()
+        if grad_out_rgb is None:
+            with _uncached(ext):
+                grad_attr = ext.render_tiles_backward_featattr_tilecenter(*args, feat_attr, grad_out_feat, *ctx.gating,
+                                                                          W, H, TW, TH, thr)
+        else:
+            grad_out_rgb = grad_out_rgb.contiguous()
+            if ctx.bg_color is None:
+                grad_t_end = torch.zeros(args[0].shape[0], device=grad_out_rgb.device, dtype=grad_out_rgb.dtype)
+            else:
+                bg = ctx.bg_color.to(device=grad_out_rgb.device, dtype=grad_out_rgb.dtype)
+                if bg.numel() == 1:
+                    bg = bg.repeat(3)
+                grad_t_end = (grad_out_rgb * bg.view(1, 3)).sum(dim=-1)
+            with _uncached(ext):
+                if grad_out_feat is None:
+                    grads = ext.render_tiles_backward_tilecenter_full(*args, grad_out_rgb, grad_t_end, W, H, TW, TH, thr)
+                else:
+                    x = [*args, grad_out_rgb, grad_t_end]
+                    records = ext.render_tiles_training_records(x, W, H, TW, thr, *ctx.gating)
+                    *grads, grad_attr = ext.backward_from_records(
+                        records, args[2], args[3], args[4], args[7], args[8], *args[9:15], grad_out_rgb, grad_t_end,
+                        feat_attr=feat_attr, grad_feat=grad_out_feat)
+        gW1, gb1, gW2, gb2, gW3, gb3, gp, gs, gq = grads
+        return (None, None, gp, gs, gq, None, None, None, None, gW1, gb1, gW2, gb2, gW3, gb3, grad_attr,
+                None, None, None, None, None, None, None, None)
 
 
 class NeuralPrimitiveSceneTileCUDA(nn.Module):
@@ -514,9 +575,12 @@ class NeuralPrimitiveSceneTileCUDA(nn.Module):
         if feature_target is not None:
             return self._forward_csr_training(ray_o, ray_d, score_threshold, bg_color, view_matrix, proj_matrix,
                                               culled_prim_indices, tile_offsets, return_feature, feature_target, device)
-        if (torch.is_grad_enabled() and feature_target is None and not (return_feature and self.feat_attr is not None)
-                and any(t.requires_grad for t in (self.positions, self.log_scales, self.quats, self.W1, self.b1,
-                                                  self.W2, self.b2, self.W3, self.b3))):
+        trainable = (self.positions, self.log_scales, self.quats, self.W1, self.b1, self.W2, self.b2, self.W3, self.b3)
+        if torch.is_grad_enabled() and return_feature and self.feat_attr is not None:
+            if any(t.requires_grad for t in (*trainable, self.feat_attr)):
+                return self._forward_differentiable_with_feat(ray_o, ray_d, score_threshold, bg_color, view_matrix,
+                                                              proj_matrix, culled_prim_indices, tile_offsets, device)
+        elif torch.is_grad_enabled() and any(t.requires_grad for t in trainable):
             return self._forward_differentiable(ray_o, ray_d, score_threshold, bg_color, view_matrix, proj_matrix,
                                                 culled_prim_indices, tile_offsets, return_feature, device)
         with torch.no_grad():
@@ -625,6 +689,29 @@ class NeuralPrimitiveSceneTileCUDA(nn.Module):
         if return_feature and self.feat_attr is None:
             raise RuntimeError("return_feature=True requested but feat_attr is not initialized.")
         return rgb
+
+    def _forward_differentiable_with_feat(self, ray_o, ray_d, score_threshold, bg_color, view_matrix, proj_matrix,
+                                          culled_prim_indices, tile_offsets, device):
+        """(rgb, feature image) with autograd (scannet/cumodel.py:1128-1143); tile-centre order only: the dense
+        feature backward of the per-pixel order (``_TileRenderWithFeatPerPixelAutogradFn``, :492-600) is not built."""
+        if self._resolve_tile_order_mode() != "tilecenter":
+            raise NotImplementedError("the backward of the per-pixel order render is not built; train with the "
+                                      "tile-centre order (MLPSP_TILE_ORDER=tilecenter, the default)")
+        self.invalidate_render_caches()
+        W, H = self.image_size
+        ts = int(self.tile_size)
+        with torch.no_grad():
+            unit_dirs = F.normalize(ray_d, dim=-1).contiguous()
+            culled_prim_indices, tile_offsets = self._tile_lists(
+                ray_o, ray_d, score_threshold, view_matrix, proj_matrix, culled_prim_indices, tile_offsets, device)
+            freq, att = self._frequency_tables(device)
+        return _TileRenderWithFeatAutogradFn.apply(
+            ray_o.contiguous(), unit_dirs, self.positions.contiguous(), self.log_scales.contiguous(),
+            F.normalize(self.quats, dim=-1).contiguous(), culled_prim_indices, tile_offsets.to(torch.int32), freq, att,
+            self.W1.contiguous(), self.b1.contiguous(), self.W2.contiguous(), self.b2.contiguous(),
+            self.W3.contiguous(), self.b3.contiguous(), self.feat_attr.contiguous(), float(self.feature_gating_beta),
+            float(self.feature_gating_temp), int(W), int(H), ts, ts, float(score_threshold),
+            self._background(bg_color, ray_o))
 
     def _forward_queued(self, ext, ray_o, unit_dirs, score_threshold, view_matrix, proj_matrix, bg_color, device):
         """The RGB frame with binning, sort and render queued back to back and one read-back at the end

@@ -77,3 +77,39 @@ def feature_weight_gradients(records, csr, signs, attributes, width, height, *, 
     if rc != 0:
         raise RuntimeError(f"mlpsp_feature_attribute_gradients: {_lib.strerror(rc)}")
     return result
+
+
+@torch.no_grad()
+def dense_feature_attribute_gradients(records, csr, grad_feature, attributes, *, segment_size=512, groups=None):
+    """Adjoint of the dense feature image with respect to ``attributes`` (shaped like them), from saved records:
+    what ``render_tiles_backward_featattr_tilecenter`` returns to ``_TileRenderWithFeatAutogradFn.backward``
+    (scannet/cumodel.py:466-477; kernel scannet/cuda/np_tile_kernels.cu:3531-3760).  ``grad_feature`` [pixels, C]
+    f32; geometry, alpha and the gates are constants of the feature image, as in the reference."""
+    from .primitive_gemm import resolve_groups
+    _, _, ids, x6, raw, masks, gates, pixel_offsets = records
+    device = ids.device
+    num_pixels = pixel_offsets.numel() - 1
+    slots = 1 if attributes.ndim == 2 else attributes.shape[1]
+    channels = attributes.shape[-1]
+    if slots not in (1, 4, 5):
+        raise RuntimeError("feat_attr must be [N,C] or [N,S,C] with slots in {4,5}")
+    if (grad_feature.dtype != torch.float32 or not grad_feature.is_contiguous()
+            or tuple(grad_feature.shape) != (num_pixels, channels)):
+        raise ValueError("the feature adjoint must be contiguous float32 [pixels, channels]")
+    if attributes.dtype != torch.float32:
+        raise ValueError("feature attributes must be float32")
+    primitives, starts, group_offsets = resolve_groups(csr, segment_size, groups)
+    pixels = torch.repeat_interleave(torch.arange(num_pixels, device=device, dtype=torch.int32), pixel_offsets.diff(),
+                                     output_size=len(ids))
+    rows = int(_lib.load().mlpsp_segment_reduce_rows(len(primitives)))
+    partial = torch.empty((max(rows, 1), slots, channels), device=device, dtype=torch.float32)
+    result = torch.empty(attributes.shape, device=device, dtype=torch.float32)
+    with torch.cuda.device(device):
+        rc = _lib.load().mlpsp_feature_dense_attribute_gradients(
+            _ptr(grad_feature), _ptr(csr.record_indices), _ptr(pixels), _ptr(raw), _ptr(gates), _ptr(csr.offsets),
+            _ptr(primitives), _ptr(starts), _ptr(group_offsets), int(len(primitives)), int(len(attributes)),
+            int(channels), int(slots), int(segment_size), _ptr(partial), _ptr(result),
+            torch.cuda.current_stream(device).cuda_stream)
+    if rc != 0:
+        raise RuntimeError(f"mlpsp_feature_dense_attribute_gradients: {_lib.strerror(rc)}")
+    return result

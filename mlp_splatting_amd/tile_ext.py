@@ -23,7 +23,7 @@ MAX_H_TILECENTER = 32          # MLPSP_MAX_H (np_tile_kernels.cu:36-38)
 _BACKWARD_ONLY = (
     "render_tiles_backward_count_per_pixel", "render_tiles_backward_count_tilecenter",
     "render_tiles_backward_emit_per_pixel", "render_tiles_backward_emit_tilecenter",
-    "render_tiles_backward_featattr_per_pixel", "render_tiles_backward_featattr_tilecenter",
+    "render_tiles_backward_featattr_per_pixel",
     "render_tiles_backward_tilecenter_full_with_feat",
     "render_tiles_mlp_records",
     "render_tiles_backward_tilecenter_traversal",
@@ -364,7 +364,7 @@ class TileExt:
         name = "render_tiles_mlp_records"
         _chk(len(x) == 17, "Expected 15 scene inputs and RGB/T adjoints")
         width, height, tile = int(width), int(height), int(tile)
-        _chk(width > 0 and height > 0 and tile in (8, 16))
+        _chk(width > 0 and height > 0 and tile in (8, 16), "the records forward supports 8x8 and 16x16 tiles")
         for i, t in enumerate(x):
             _chk(t.is_cuda and t.is_contiguous(), "Inputs must be contiguous CUDA tensors")
             _chk(t.device == x[0].device, "Inputs must share a device")
@@ -531,10 +531,48 @@ class TileExt:
         return self.backward_from_records(records, positions, log_scales, quats, freq, att, W1, b1, W2, b2, W3, b3,
                                           x[15], x[16])
 
+    def render_tiles_backward_featattr_tilecenter(self, rays_o, rays_d, positions, log_scales, quats, cand, offsets,
+                                                  freq, att, W1, b1, W2, b2, W3, b3, feat_attr, grad_out_feat, beta,
+                                                  temp, Wimg, Himg, TW, TH, thr):
+        """grad_feat_attr (shaped like ``feat_attr``) of the tile-centre-order feature image for its adjoint
+        ``grad_out_feat`` [B,C] (np_tile_kernels.cu:3531-3760, wrapper :6537-6620): every hit adds
+        T * alpha * gate_slot * grad_out_feat[pixel] to its primitive's slot rows; geometry, MLP and gates get no
+        gradient from the feature image.  The reference traverses the frame with atomics; here the hits come from
+        the records forward and are summed per primitive in a fixed order."""
+        _chk(int(TW) == int(TH), "square tiles only")
+        _chk(feat_attr.is_cuda and feat_attr.dtype == torch.float32 and feat_attr.is_contiguous())
+        _chk(feat_attr.dim() in (2, 3) and feat_attr.shape[0] == positions.shape[0])
+        _chk(feat_attr.dim() == 2 or feat_attr.shape[1] in (4, 5), "feat_attr must be [N,C] or [N,S,C] with slots in {4,5}")
+        pixels = int(Wimg) * int(Himg)
+        _chk(grad_out_feat.is_cuda and grad_out_feat.dtype == torch.float32
+             and tuple(grad_out_feat.shape) == (pixels, feat_attr.shape[-1]), "grad_out_feat must be [B, C]")
+        placeholders = [torch.zeros_like(rays_o), torch.zeros(pixels, device=rays_o.device)]
+        x = [rays_o, rays_d, positions, log_scales, quats, cand, offsets, freq, att, W1, b1, W2, b2, W3, b3, *placeholders]
+        records = self.render_tiles_training_records(x, Wimg, Himg, TW, thr, float(beta), float(temp))
+        return self.feature_gradients_from_records(records, feat_attr, grad_out_feat.contiguous())
+
+    @staticmethod
+    def feature_gradients_from_records(records, feat_attr, grad_out_feat, csr=None, groups=None):
+        """:meth:`render_tiles_backward_featattr_tilecenter` from records that the caller already holds; ``csr`` and
+        ``groups`` when it has grouped them by primitive as well."""
+        from .primitive_csr import group_records
+        from . import primitive_gemm
+        from .record_feature_loss import dense_feature_attribute_gradients
+        ids, x6 = records[2], records[3]
+        with torch.cuda.device(ids.device):
+            if csr is None:
+                csr = group_records(ids, x6, torch.empty((ids.numel(), 0), device=ids.device), feat_attr.shape[0])
+                groups = None
+            if groups is None:
+                groups = primitive_gemm.prepare_groups(csr)
+            return dense_feature_attribute_gradients(records, csr, grad_out_feat, feat_attr, groups=groups)
+
     def backward_from_records(self, records, positions, log_scales, quats, freq, att, W1, b1, W2, b2, W3, b3,
-                              grad_rgb, grad_t):
+                              grad_rgb, grad_t, feat_attr=None, grad_feat=None):
         """The nine gradients of :meth:`render_tiles_backward_tilecenter_full` from records that a forward pass
-        already holds (no counterpart in the reference, whose fused backward traverses the frame again)."""
+        already holds (no counterpart in the reference, whose fused backward traverses the frame again).  With
+        ``feat_attr`` and ``grad_feat`` the gradient of :meth:`render_tiles_backward_featattr_tilecenter` is appended,
+        from the same grouping of the records."""
         from .primitive_csr import group_records, reference_weight_gradients
         from . import primitive_gemm
         rgb, alpha, ids, x6, raw, masks, gates, pixel_offsets = records
@@ -552,6 +590,8 @@ class TileExt:
             grads = primitive_gemm.grouped_weight_gradients(csr, freq, att, weights, dtype=torch.float32, groups=groups)
         else:   # other MLP shapes: the dense chain per primitive (small scenes and tests only)
             grads = reference_weight_gradients(csr, freq, att, weights)
+        if feat_attr is not None and grad_feat is not None:
+            return [*grads, gp, gs, gq, self.feature_gradients_from_records(records, feat_attr, grad_feat, csr, groups)]
         return [*grads, gp, gs, gq]
 
     # ------------------------------------------------------------------------------------------

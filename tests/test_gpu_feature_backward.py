@@ -1,0 +1,148 @@
+"""Backward of the dense feature image (render_tiles_backward_featattr_tilecenter and the scene module's
+differentiable (rgb, feature) render) against autograd through a float64 framebuffer built from the records, which
+is itself tied to the exact render kernel's feature image (bit-identical to the oracle, tests/test_gpu_parity.py).
+f32 sums in a fixed order: atol 2e-6, rtol 2e-5 as for the streamed loss's f32 gradients."""
+import numpy as np
+import pytest
+import torch
+
+from conftest import to_dev
+from helpers import Frame
+from test_gpu_feature_loss import _frame_records, _framebuffer64
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("slots", [1, 4, 5])
+@pytest.mark.parametrize("size,channels", [((24, 16), 150), ((33, 19), 64), ((9, 7), 3), ((40, 24), 512)])
+def test_dense_feature_adjoint_reaches_the_attributes_as_defined(device, oracle_mod, slots, size, channels):
+    width, height = size
+    fr, ext, base, records = _frame_records(device, oracle_mod, width, height)
+    n = fr.scene.n
+    torch.manual_seed(90 + slots)
+    attr = torch.randn((n, channels) if slots == 1 else (n, slots, channels), device=device) * 0.2
+    adjoint = torch.randn(width * height, channels, device=device)
+    assert records[2].numel() > 0
+    _, _, dense = ext.render_tiles_forward_tilecenter_with_feat(*base, attr, 1.5, 2.0, width, height, 8, 8, fr.thr)
+    leaf = attr.detach().cpu().double().requires_grad_(True)
+    image64 = _framebuffer64(records, leaf, width, height)
+    torch.testing.assert_close(image64.float(), dense.cpu(), atol=3e-6, rtol=3e-6)
+    (image64 * adjoint.cpu().double()).sum().backward()
+    got = ext.render_tiles_backward_featattr_tilecenter(*base, attr, adjoint, 1.5, 2.0, width, height, 8, 8, fr.thr)
+    assert got.shape == attr.shape and got.dtype == torch.float32
+    scale = float(leaf.grad.abs().max())
+    torch.testing.assert_close(got.cpu().double(), leaf.grad, atol=2e-6 * max(scale, 1.0), rtol=2e-5)
+    untouched = torch.bincount(records[2].long().cpu(), minlength=n) == 0
+    assert untouched.any() and not got.cpu()[untouched].any()
+    # the same sums from records the caller holds, with small segments (many partial rows per primitive)
+    from mlp_splatting_amd.primitive_csr import group_records
+    from mlp_splatting_amd.record_feature_loss import dense_feature_attribute_gradients
+    csr = group_records(records[2], records[3], torch.zeros((records[2].numel(), 4), device=device), n, records[5])
+    small = dense_feature_attribute_gradients(records, csr, adjoint, attr, segment_size=32)
+    torch.testing.assert_close(small.cpu().double(), leaf.grad, atol=2e-6 * max(scale, 1.0), rtol=2e-5)
+
+
+def test_dense_feature_adjoint_ignores_non_finite_rows_of_pixels_without_records(device, oracle_mod):
+    """A pixel nothing hits contributes nothing, whatever its adjoint row holds (the kernel pads a segment's last
+    step with empty records that point at row 0)."""
+    for eye in ((0.3, 0.2, -2.0), (0.3, 0.2, -3.5), (1.5, 0.2, -3.0), (0.0, 2.5, -3.0), (-2.0, -1.0, -3.0)):
+        fr, ext, base, records = _frame_records(device, oracle_mod, 24, 16, n=40, seed_eye=eye)
+        counts = records[7].diff()
+        if int(counts[0]) == 0 and records[2].numel() > 0:       # row 0 is the one the padding points at
+            break
+    else:
+        raise AssertionError("no frame with an empty first pixel among the candidates")
+    empty = (counts == 0).nonzero().flatten()
+    attr = torch.randn(fr.scene.n, 4, 8, device=device)
+    adjoint = torch.randn(24 * 16, 8, device=device)
+    want = ext.render_tiles_backward_featattr_tilecenter(*base, attr, adjoint, 1.5, 2.0, 24, 16, 8, 8, fr.thr)
+    adjoint[empty] = float("nan")
+    got = ext.render_tiles_backward_featattr_tilecenter(*base, attr, adjoint, 1.5, 2.0, 24, 16, 8, 8, fr.thr)
+    assert torch.equal(got, want) and bool(torch.isfinite(got).all())
+
+
+def test_dense_feature_adjoint_argument_checks(device, oracle_mod):
+    fr, ext, base, records = _frame_records(device, oracle_mod, 16, 8, n=100)
+    attr = torch.zeros(fr.scene.n, 4, 6, device=device)
+    good = torch.zeros(16 * 8, 6, device=device)
+    with pytest.raises(RuntimeError, match="slots in"):
+        ext.render_tiles_backward_featattr_tilecenter(*base, torch.zeros(fr.scene.n, 3, 6, device=device), good, 1.5, 2.0,
+                                                      16, 8, 8, 8, fr.thr)
+    with pytest.raises(RuntimeError, match=r"\[B, C\]"):
+        ext.render_tiles_backward_featattr_tilecenter(*base, attr, torch.zeros(16 * 8, 5, device=device), 1.5, 2.0, 16, 8,
+                                                      8, 8, fr.thr)
+    with pytest.raises(RuntimeError):
+        ext.render_tiles_backward_featattr_tilecenter(*base, attr, good.double(), 1.5, 2.0, 16, 8, 8, 8, fr.thr)
+
+
+def _scene(device, n=400, width=32, height=24, channels=12, slots=4):
+    from mlp_splatting_amd import synthetic as syn
+    from mlp_splatting_amd.cumodel import NeuralPrimitiveSceneTileCUDA
+    fr = Frame("cfg1_5k_160x120", n=n, hidden=32, width=width, height=height, eye=(0.3, 0.2, -2.0), target=(0.0, 0.0, 0.0))
+    scene = NeuralPrimitiveSceneTileCUDA(num_primitives=n, hidden_dim=32, pe_frequencies=6, feature_dim_low=channels,
+                                         feature_slots=slots).to(device)
+    sc = fr.scene
+    with torch.no_grad():
+        for name, value in (("positions", sc.positions), ("log_scales", sc.log_scales), ("quats", sc.quats),
+                            ("W1", sc.W1), ("b1", sc.b1), ("W2", sc.W2), ("b2", sc.b2), ("W3", sc.W3), ("b3", sc.b3)):
+            getattr(scene, name).copy_(to_dev(value, device))
+        scene.feat_attr.normal_(0.0, 0.3)
+    scene.set_image_size(width, height)
+    view = torch.from_numpy(fr.view)
+    proj = torch.from_numpy(fr.proj)
+    rays = (to_dev(fr.rays_o, device), to_dev(fr.rays_d, device))
+    return fr, scene, rays, view, proj
+
+
+def test_scene_renders_rgb_and_features_with_gradients(device):
+    """forward(return_feature=True) under autograd: the feature adjoint reaches feat_attr only, the RGB adjoint
+    everything else; each agrees with the function that serves it alone, and an unused output leaves its
+    parameters without a gradient (scannet/cumodel.py:427-431)."""
+    fr, scene, (ro, rd), view, proj = _scene(device)
+    thr = fr.thr
+    names = ("positions", "log_scales", "quats", "W1", "b1", "W2", "b2", "W3", "b3")
+    rgb, feat = scene(ro, rd, score_threshold=thr, view_matrix=view, proj_matrix=proj, return_feature=True)
+    assert rgb.requires_grad and feat.requires_grad and feat.shape == (ro.shape[0], scene.feat_attr.shape[-1])
+    with torch.no_grad():
+        rgb0, feat0 = scene(ro, rd, score_threshold=thr, view_matrix=view, proj_matrix=proj, return_feature=True)
+    assert torch.equal(rgb, rgb0) and torch.equal(feat, feat0)
+    torch.manual_seed(3)
+    g_rgb, g_feat = torch.randn_like(rgb), torch.randn_like(feat)
+    # both adjoints at once
+    scene.zero_grad(set_to_none=True)
+    ((rgb * g_rgb).sum() + (feat * g_feat).sum()).backward()
+    both = {k: getattr(scene, k).grad.clone() for k in names}
+    both_attr = scene.feat_attr.grad.clone()
+    assert all(bool(torch.isfinite(v).all()) for v in both.values()) and float(both_attr.abs().max()) > 0
+    # the feature adjoint alone: attributes only
+    scene.zero_grad(set_to_none=True)
+    rgb, feat = scene(ro, rd, score_threshold=thr, view_matrix=view, proj_matrix=proj, return_feature=True)
+    (feat * g_feat).sum().backward()
+    assert all(getattr(scene, k).grad is None for k in names)
+    torch.testing.assert_close(scene.feat_attr.grad, both_attr, atol=1e-6, rtol=1e-5)
+    # the RGB adjoint alone: the RGB-only render's gradients, and none for the attributes
+    scene.zero_grad(set_to_none=True)
+    rgb, feat = scene(ro, rd, score_threshold=thr, view_matrix=view, proj_matrix=proj, return_feature=True)
+    (rgb * g_rgb).sum().backward()
+    assert scene.feat_attr.grad is None
+    only_rgb = {k: getattr(scene, k).grad.clone() for k in names}
+    scene.zero_grad(set_to_none=True)
+    plain = scene(ro, rd, score_threshold=thr, view_matrix=view, proj_matrix=proj)
+    (plain * g_rgb).sum().backward()
+    for k in names:
+        want = getattr(scene, k).grad
+        scale = max(float(want.abs().max()), 1e-6)
+        torch.testing.assert_close(only_rgb[k], want, atol=2e-4 * scale, rtol=2e-3, msg=lambda m, k=k: f"{k}: {m}")
+        torch.testing.assert_close(both[k], want, atol=2e-4 * scale, rtol=2e-3, msg=lambda m, k=k: f"{k} (both): {m}")
+    # the attribute gradient against the float64 definition
+    from mlp_splatting_amd.cumodel import NeuralPrimitiveSceneTileCUDA
+    ext = NeuralPrimitiveSceneTileCUDA._ensure_tile_ext_static()
+    cand, off = scene._tile_lists(ro, rd, thr, view, proj, None, None, device)
+    base = scene._base_args(ro, rd, cand, off, device)
+    x = list(base) + [torch.zeros_like(ro), torch.zeros(ro.shape[0], device=device)]
+    records = ext.render_tiles_training_records(x, *scene.image_size, 8, thr, float(scene.feature_gating_beta),
+                                                float(scene.feature_gating_temp))
+    leaf = scene.feat_attr.detach().cpu().double().requires_grad_(True)
+    (_framebuffer64(records, leaf, *scene.image_size) * g_feat.cpu().double()).sum().backward()
+    torch.testing.assert_close(both_attr.cpu().double(), leaf.grad, atol=2e-6 * max(float(leaf.grad.abs().max()), 1.0),
+                               rtol=2e-5)
