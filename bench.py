@@ -54,6 +54,13 @@ def train_steps(args, scene, frames, proj, thr, W, H, sc, dev):
         if feature_target is None:
             rgb = scene(ro, rd, score_threshold=thr, view_matrix=views[0], proj_matrix=proj)
             loss = (rgb - target).abs().mean()
+        elif args.dense_feature_loss:
+            # the reference's "legacy" training backend: dense feature image under autograd, resampled by torch
+            rgb, feat = scene(ro, rd, score_threshold=thr, view_matrix=views[0], proj_matrix=proj, return_feature=True)
+            low = torch.nn.functional.interpolate(feat.view(H, W, feature_dim).permute(2, 0, 1).unsqueeze(0),
+                                                  size=(H // 4, W // 4), mode="bilinear", align_corners=False)
+            feature_loss = (low.squeeze(0).permute(1, 2, 0) - feature_target.float()).abs().mean()
+            loss = (rgb - target).abs().mean() + 0.5 * feature_loss
         else:
             rgb, feature_loss = scene(ro, rd, score_threshold=thr, view_matrix=views[0], proj_matrix=proj,
                                       return_feature=True, feature_target=feature_target)
@@ -84,8 +91,11 @@ def train_steps(args, scene, frames, proj, thr, W, H, sc, dev):
         "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": args.workload, "primitives": sc.n, "width": W, "height": H, "tile": 8, "threshold": thr,
                    "poses": len(frames), "loss": ("L1 against a fixed random image" if not feature_dim else
+                            "L1 image loss + L1 of the dense feature image, resampled by torch, against a "
+                            "quarter-resolution target" if args.dense_feature_loss else
                             "L1 image loss + streamed feature L1 against a quarter-resolution fp16 target"),
-                   "feature_channels": feature_dim, "mlp_gradient_precision": ("f32" if not feature_dim else
+                   "feature_channels": feature_dim,
+                   "mlp_gradient_precision": ("f32" if not feature_dim or args.dense_feature_loss else
                                                                                os.environ.get("MLPSP_CSR_MLP_PRECISION", "float16")),
                    "optimizer": "Adam (fused), all parameter tensors",
                    "entry": "NeuralPrimitiveSceneTileCUDA.forward + backward"},
@@ -102,6 +112,9 @@ def main() -> int:
     ap.add_argument("--precision", choices=["f32", "bf16"], default=None,
                     help="MLP arithmetic of the render kernel (default: bf16 matrix cores when built, else f32)")
     ap.add_argument("--poses", type=int, default=32)
+    ap.add_argument("--dense-feature-loss", action="store_true",
+                    help="with --train on a feature workload: the dense feature image under autograd (the reference's "
+                         "legacy training backend) instead of the record-based streamed loss")
     ap.add_argument("--train", action="store_true",
                     help="time full training steps instead (f32 render with autograd, L1 image loss, backward through "
                          "the record pipeline, Adam on all nine parameter tensors); prints its own JSON line")
