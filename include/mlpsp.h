@@ -262,6 +262,30 @@ int mlpsp_render_per_pixel_f32(const float* rays_o_dev, const float* rays_d_dev,
                                int tile_w, int tile_h, float threshold, void* workspace_dev, size_t workspace_bytes,
                                float* out_rgb_dev, float* out_alpha_dev, float* out_feat_dev, mlpsp_stream_t stream);
 
+/* Training records in per-pixel order: the traversal of render_tiles_backward_count_per_pixel and
+ * render_tiles_backward_emit_per_pixel (scannet/cuda/np_tile_kernels.cu:1211-1836, wrappers :6290-6400; called from
+ * _TileRenderAutogradFn.backward mode 0, scannet/cumodel.py:297-331) with the record schema of mlpsp_records_emit:
+ * every pixel's hits (at most 256; a 257th returns MLPSP_E_PIXEL_OVERFLOW) in the order of its own t, blended until
+ * the transmittance falls below 1e-3.  count leaves the number of blended hits per pixel in counts_dev [W*H];
+ * the caller scans them into record_offsets_dev [W*H+1] (int64) and calls emit, which writes ids [R], x6 [R,6],
+ * masks [R,2], raw [R,8], gates [R,4] and the image (rgb [W*H,3], alpha [W*H]).  The reference's emit kernel also
+ * composes the adjoints; here they come from mlpsp_records_reverse_adjoints over these records.  workspace as for
+ * mlpsp_render_per_pixel_f32; blocking (one 4-byte read-back), like it.  hidden <= 32. */
+int mlpsp_records_per_pixel_count(
+    const float* rays_o_dev, const float* rays_d_dev, const void* prim_records_dev, const int32_t* candidates_dev,
+    const int32_t* tile_offsets_dev, const float* freq_dev, const float* att_dev, int num_frequencies,
+    const float* W1, const float* b1, const float* W2, const float* b2, const float* W3, const float* b3,
+    int num_primitives, int hidden, int width, int height, int tile_w, int tile_h, float threshold,
+    void* workspace_dev, size_t workspace_bytes, int32_t* counts_dev, mlpsp_stream_t stream);
+int mlpsp_records_per_pixel_emit(
+    const float* rays_o_dev, const float* rays_d_dev, const void* prim_records_dev, const int32_t* candidates_dev,
+    const int32_t* tile_offsets_dev, const float* freq_dev, const float* att_dev, int num_frequencies,
+    const float* W1, const float* b1, const float* W2, const float* b2, const float* W3, const float* b3,
+    int num_primitives, int hidden, float gating_beta, float gating_temp, int width, int height, int tile_w,
+    int tile_h, float threshold, void* workspace_dev, size_t workspace_bytes, const int64_t* record_offsets_dev,
+    int64_t total_records, int32_t* ids_dev, float* x6_dev, int32_t* masks_dev, float* raw_dev, float* gates_dev,
+    float* out_rgb_dev, float* out_alpha_dev, mlpsp_stream_t stream);
+
 /* Matrix-core path for the released 72->32->32->4 MLP (F = 6, H = 32), 8x8 tiles; the counterpart of
  * render_tiles_rgb_wmma (scannet/cuda/rgb_wmma.cuh:75-274).
  * mlpsp_pack_mfma_weights: rounds W1, W2, W3 to bf16 (use_bf16 != 0) or fp16 and stores them, with the

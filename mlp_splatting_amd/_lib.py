@@ -46,6 +46,9 @@ SIGNATURES = {
     "mlpsp_per_pixel_workspace_bytes": (_sz, [_i, _i, _i, _i]),
     "mlpsp_render_per_pixel_f32": (_i, [_vp] * 7 + [_i] + [_vp] * 6 + [_i, _i, _vp, _i, _i, _f, _f, _i, _i, _i, _i, _f,
                                                                       _vp, _sz, _vp, _vp, _vp, _vp]),
+    "mlpsp_records_per_pixel_count": (_i, [_vp] * 7 + [_i] + [_vp] * 6 + [_i, _i, _i, _i, _i, _i, _f, _vp, _sz, _vp, _vp]),
+    "mlpsp_records_per_pixel_emit": (_i, [_vp] * 7 + [_i] + [_vp] * 6 + [_i, _i, _f, _f, _i, _i, _i, _i, _f, _vp, _sz, _vp,
+                                                                        _i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "mlpsp_mfma_pack_bytes": (_sz, [_i]),
     "mlpsp_pack_mfma_weights": (_i, [_vp] * 6 + [_i, _i, _vp, _vp]),
     "mlpsp_render_tilecenter_mfma": (_i, [_vp] * 8 + [_i, _i, _i, _i, _f, _vp, _vp, _vp, _vp, _vp]),

@@ -241,11 +241,15 @@ class _TileRenderAutogradFn(torch.autograd.Function):
             if bg.numel() == 1:
                 bg = bg.repeat(3)
             grad_t_end = (grad_out_rgb * bg.view(1, 3)).sum(dim=-1)
-        if ctx.mode != 1:
-            raise NotImplementedError("the backward of the per-pixel order render is not built; train with the "
-                                      "tile-centre order (MLPSP_TILE_ORDER=tilecenter, the default)")
         ext = NeuralPrimitiveSceneTileCUDA._ensure_tile_ext_static()
-        if ctx.has_records:
+        if ctx.mode == 0:
+            # per-pixel order (scannet/cumodel.py:297-364): the records of every pixel in its own depth order, then
+            # the same reverse walk and grouped weight gradients as the tile-centre order
+            with _uncached(ext):
+                records = ext.render_tiles_per_pixel_records(args, *ctx.dims, 1.5, 2.0)
+                gW1, gb1, gW2, gb2, gW3, gb3, gp, gs, gq = ext.backward_from_records(
+                    records, args[2], args[3], args[4], args[7], args[8], *args[9:15], grad_out_rgb, grad_t_end)
+        elif ctx.has_records:
             gW1, gb1, gW2, gb2, gW3, gb3, gp, gs, gq = ext.backward_from_records(
                 [None, None, *kept], args[2], args[3], args[4], args[7], args[8], *args[9:15], grad_out_rgb, grad_t_end)
         else:
@@ -311,6 +315,58 @@ class _TileRenderWithFeatAutogradFn(torch.autograd.Function):
                     *grads, grad_attr = ext.backward_from_records(
                         records, args[2], args[3], args[4], args[7], args[8], *args[9:15], grad_out_rgb, grad_t_end,
                         feat_attr=feat_attr, grad_feat=grad_out_feat)
+        gW1, gb1, gW2, gb2, gW3, gb3, gp, gs, gq = grads
+        return (None, None, gp, gs, gq, None, None, None, None, gW1, gb1, gW2, gb2, gW3, gb3, grad_attr,
+                None, None, None, None, None, None, None, None)
+
+
+class _TileRenderWithFeatPerPixelAutogradFn(torch.autograd.Function):
+    """(rgb, feature image) in per-pixel order under autograd (scannet/cumodel.py:492-600).  The forward is the
+    per-pixel render; the backward takes the records of every pixel in its own depth order and serves both adjoints
+    from them, as :class:`_TileRenderWithFeatAutogradFn` does in tile-centre order."""
+
+    @staticmethod
+    def forward(ctx, rays_o, rays_d, positions, log_scales, quats, culled_prim_indices, tile_offsets, freq, att,
+                W1, b1, W2, b2, W3, b3, feat_attr, gating_beta, gating_temp, Wimg, Himg, TW, TH, threshold, bg_color):
+        ext = NeuralPrimitiveSceneTileCUDA._ensure_tile_ext_static()
+        with _uncached(ext):
+            rgb, alpha, feat = ext.render_tiles_forward_per_pixel_with_feat(
+                rays_o, rays_d, positions, log_scales, quats, culled_prim_indices, tile_offsets, freq, att,
+                W1, b1, W2, b2, W3, b3, feat_attr, float(gating_beta), float(gating_temp), int(Wimg), int(Himg), int(TW),
+                int(TH), float(threshold))
+        ctx.save_for_backward(rays_o, rays_d, positions, log_scales, quats, culled_prim_indices, tile_offsets, freq, att,
+                              W1, b1, W2, b2, W3, b3, feat_attr)
+        ctx.dims = (int(Wimg), int(Himg), int(TW), int(TH), float(threshold))
+        ctx.bg_color, ctx.gating = bg_color, (float(gating_beta), float(gating_temp))
+        ctx.set_materialize_grads(False)
+        return _add_background(rgb, alpha, bg_color), feat
+
+    @staticmethod
+    def backward(ctx, grad_out_rgb, grad_out_feat):
+        args, feat_attr = ctx.saved_tensors[:15], ctx.saved_tensors[15]
+        if grad_out_rgb is None and grad_out_feat is None:
+            return (None,) * 24
+        ext = NeuralPrimitiveSceneTileCUDA._ensure_tile_ext_static()
+        grads, grad_attr = [None] * 9, None
+        with _uncached(ext):
+            records = ext.render_tiles_per_pixel_records(args, *ctx.dims, *ctx.gating)
+            if grad_out_rgb is None:
+                grad_attr = ext.feature_gradients_from_records(records, feat_attr, grad_out_feat.contiguous())
+            else:
+                grad_out_rgb = grad_out_rgb.contiguous()
+                if ctx.bg_color is None:
+                    grad_t_end = torch.zeros(args[0].shape[0], device=grad_out_rgb.device, dtype=grad_out_rgb.dtype)
+                else:
+                    bg = ctx.bg_color.to(device=grad_out_rgb.device, dtype=grad_out_rgb.dtype)
+                    if bg.numel() == 1:
+                        bg = bg.repeat(3)
+                    grad_t_end = (grad_out_rgb * bg.view(1, 3)).sum(dim=-1)
+                out = ext.backward_from_records(
+                    records, args[2], args[3], args[4], args[7], args[8], *args[9:15], grad_out_rgb, grad_t_end,
+                    feat_attr=feat_attr if grad_out_feat is not None else None,
+                    grad_feat=grad_out_feat.contiguous() if grad_out_feat is not None else None)
+                grads = out[:9]
+                grad_attr = out[9] if len(out) > 9 else None
         gW1, gb1, gW2, gb2, gW3, gb3, gp, gs, gq = grads
         return (None, None, gp, gs, gq, None, None, None, None, gW1, gb1, gW2, gb2, gW3, gb3, grad_attr,
                 None, None, None, None, None, None, None, None)
@@ -692,11 +748,9 @@ class NeuralPrimitiveSceneTileCUDA(nn.Module):
 
     def _forward_differentiable_with_feat(self, ray_o, ray_d, score_threshold, bg_color, view_matrix, proj_matrix,
                                           culled_prim_indices, tile_offsets, device):
-        """(rgb, feature image) with autograd (scannet/cumodel.py:1128-1143); tile-centre order only: the dense
-        feature backward of the per-pixel order (``_TileRenderWithFeatPerPixelAutogradFn``, :492-600) is not built."""
-        if self._resolve_tile_order_mode() != "tilecenter":
-            raise NotImplementedError("the backward of the per-pixel order render is not built; train with the "
-                                      "tile-centre order (MLPSP_TILE_ORDER=tilecenter, the default)")
+        """(rgb, feature image) with autograd (scannet/cumodel.py:1128-1160), in either order."""
+        fn = (_TileRenderWithFeatAutogradFn if self._resolve_tile_order_mode() == "tilecenter"
+              else _TileRenderWithFeatPerPixelAutogradFn)
         self.invalidate_render_caches()
         W, H = self.image_size
         ts = int(self.tile_size)
@@ -705,7 +759,7 @@ class NeuralPrimitiveSceneTileCUDA(nn.Module):
             culled_prim_indices, tile_offsets = self._tile_lists(
                 ray_o, ray_d, score_threshold, view_matrix, proj_matrix, culled_prim_indices, tile_offsets, device)
             freq, att = self._frequency_tables(device)
-        return _TileRenderWithFeatAutogradFn.apply(
+        return fn.apply(
             ray_o.contiguous(), unit_dirs, self.positions.contiguous(), self.log_scales.contiguous(),
             F.normalize(self.quats, dim=-1).contiguous(), culled_prim_indices, tile_offsets.to(torch.int32), freq, att,
             self.W1.contiguous(), self.b1.contiguous(), self.W2.contiguous(), self.b2.contiguous(),

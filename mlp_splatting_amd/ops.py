@@ -374,6 +374,47 @@ def render_per_pixel_f32(rays_o, rays_d, records, candidates, tile_offsets, freq
     return rgb, alpha, feat
 
 
+def records_per_pixel(rays_o, rays_d, records, candidates, tile_offsets, freq, att, W1, b1, W2, b2, W3, b3, W, H, TW,
+                      TH, threshold, beta, temp, path_name, counts_only=False):
+    """Training records in per-pixel order -> (rgb, alpha, ids, x6, raw, masks, gates, offsets int64 [B+1]), or the
+    per-pixel counts (int32 [B]) alone; raises the reference's per-pixel overflow error."""
+    dev = rays_o.device
+    lib = _lib.load()
+    B = W * H
+    n, hidden, F = W1.shape[0], W2.shape[1], freq.shape[0]
+    nbytes = lib.mlpsp_per_pixel_workspace_bytes(W, H, TW, TH)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    head = (_ptr(rays_o), _ptr(rays_d), _ptr(records), _ptr(candidates), _ptr(tile_offsets), _ptr(freq), _ptr(att), F,
+            _ptr(W1), _ptr(b1), _ptr(W2), _ptr(b2), _ptr(W3), _ptr(b3), n, hidden)
+
+    def check(code, what):
+        if code & _lib.E_PIXEL_OVERFLOW:
+            raise RuntimeError(f"{path_name}: per-pixel intersection capacity {_lib.PIXEL_HIT_CAPACITY} exceeded; "
+                               "refusing to return a silently truncated result")
+        _check(code, what)
+
+    counts = torch.zeros(B, dtype=torch.int32, device=dev)
+    check(lib.mlpsp_records_per_pixel_count(*head, W, H, TW, TH, float(threshold), _ptr(ws), nbytes, _ptr(counts),
+                                            _stream(dev)), "mlpsp_records_per_pixel_count")
+    if counts_only:
+        return counts
+    offsets = torch.zeros(B + 1, dtype=torch.int64, device=dev)
+    torch.cumsum(counts, 0, out=offsets[1:])
+    total = int(offsets[-1].item())
+    ids = torch.empty(total, dtype=torch.int32, device=dev)
+    x6 = torch.empty(total, 6, dtype=torch.float32, device=dev)
+    masks = torch.empty(total, 2, dtype=torch.int32, device=dev)
+    raw = torch.empty(total, 8, dtype=torch.float32, device=dev)
+    gates = torch.empty(total, 4, dtype=torch.float32, device=dev)
+    rgb = torch.zeros(B, 3, dtype=torch.float32, device=dev)
+    alpha = torch.zeros(B, 1, dtype=torch.float32, device=dev)
+    check(lib.mlpsp_records_per_pixel_emit(*head, float(beta), float(temp), W, H, TW, TH, float(threshold), _ptr(ws),
+                                           nbytes, _ptr(offsets), total, _ptr(ids), _ptr(x6), _ptr(masks), _ptr(raw),
+                                           _ptr(gates), _ptr(rgb), _ptr(alpha), _stream(dev)),
+          "mlpsp_records_per_pixel_emit")
+    return rgb, alpha, ids, x6, raw, masks, gates, offsets
+
+
 def pack_mfma_weights(W1, b1, W2, b2, W3, b3, bf16=True):
     """Weights of the 72->32->32->4 MLP in matrix-core operand order (uint8 [N*7808]); once per scene."""
     n = W1.shape[0]

@@ -21,9 +21,8 @@ MAX_TILE_PRIMS = 1536          # MLPSP_MAX_TILE_PRIMS as built by scannet/cumode
 MAX_H_TILECENTER = 32          # MLPSP_MAX_H (np_tile_kernels.cu:36-38)
 
 _BACKWARD_ONLY = (
-    "render_tiles_backward_count_per_pixel", "render_tiles_backward_count_tilecenter",
+    "render_tiles_backward_count_tilecenter",
     "render_tiles_backward_emit_per_pixel", "render_tiles_backward_emit_tilecenter",
-    "render_tiles_backward_featattr_per_pixel",
     "render_tiles_backward_tilecenter_full_with_feat",
     "render_tiles_mlp_records",
     "render_tiles_backward_tilecenter_traversal",
@@ -273,6 +272,28 @@ class TileExt:
         """Forward-only alias of the per-pixel renderer (np_tile_kernels.cu:4989-5038)."""
         rgb, alpha, _ = self._per_pixel(args, "render_tiles_autograd")
         return rgb, alpha
+
+    def render_tiles_backward_count_per_pixel(self, *args):
+        """counts [B] int32: the hits every pixel blends in its own depth order before its transmittance falls below
+        1e-3 -- the record count of the per-pixel backward (np_tile_kernels.cu:1424-1566, wrapper :6210-6290)."""
+        return self.render_tiles_per_pixel_records(args[:15], *args[15:], 1.5, 2.0, counts_only=True,
+                                                   name="render_tiles_backward_count_per_pixel")
+
+    def render_tiles_per_pixel_records(self, base, Wimg, Himg, TW, TH, thr, beta, temp, *, counts_only=False,
+                                       name="render_tiles_backward_emit_per_pixel"):
+        """[rgb, alpha, ids, x6, raw, masks, gates, offsets] as :meth:`render_tiles_training_records`, every pixel's
+        records in the order of its own t: what the reference's per-pixel backward kernels traverse
+        (np_tile_kernels.cu:1211-1836).  Tile lists are validated without a capacity (:6238), a 257th hit of a pixel
+        raises the per-pixel overflow error."""
+        geo, cand, offsets, freq, att, ws, (W, H, TW, TH, thr) = self._prepare((*base, Wimg, Himg, TW, TH, thr), name, 0,
+                                                                               None, False, MAX_H_TILECENTER)
+        _chk(0 < TW * TH <= 256, "Tile size too large")
+        rays_o, rays_d, positions, log_scales, quats = geo
+        with torch.cuda.device(rays_o.device), self.uncached():
+            rec = self._records(positions, log_scales, quats)
+            out = ops.records_per_pixel(rays_o, rays_d, rec, cand, offsets, freq, att, *ws, W, H, TW, TH, thr, float(beta),
+                                        float(temp), name, counts_only=counts_only)
+        return out if counts_only else list(out)
 
     def render_tiles_forward_per_pixel_with_feat(self, *args):
         """(rgb, alpha, feat); np_tile_kernels.cu:5134-5222."""
@@ -549,6 +570,21 @@ class TileExt:
         placeholders = [torch.zeros_like(rays_o), torch.zeros(pixels, device=rays_o.device)]
         x = [rays_o, rays_d, positions, log_scales, quats, cand, offsets, freq, att, W1, b1, W2, b2, W3, b3, *placeholders]
         records = self.render_tiles_training_records(x, Wimg, Himg, TW, thr, float(beta), float(temp))
+        return self.feature_gradients_from_records(records, feat_attr, grad_out_feat.contiguous())
+
+    def render_tiles_backward_featattr_per_pixel(self, rays_o, rays_d, positions, log_scales, quats, cand, offsets,
+                                                 freq, att, W1, b1, W2, b2, W3, b3, feat_attr, grad_out_feat, beta, temp,
+                                                 Wimg, Himg, TW, TH, thr):
+        """:meth:`render_tiles_backward_featattr_tilecenter` for the per-pixel order (np_tile_kernels.cu:1211-1422,
+        wrapper :6629-6720): the same sums over every pixel's hits in its own depth order."""
+        _chk(feat_attr.is_cuda and feat_attr.dtype == torch.float32 and feat_attr.is_contiguous())
+        _chk(feat_attr.dim() in (2, 3) and feat_attr.shape[0] == positions.shape[0])
+        _chk(feat_attr.dim() == 2 or feat_attr.shape[1] in (4, 5), "feat_attr must be [N,C] or [N,S,C] with slots in {4,5}")
+        _chk(grad_out_feat.is_cuda and grad_out_feat.dtype == torch.float32
+             and tuple(grad_out_feat.shape) == (int(Wimg) * int(Himg), feat_attr.shape[-1]), "grad_out_feat must be [B, C]")
+        base = (rays_o, rays_d, positions, log_scales, quats, cand, offsets, freq, att, W1, b1, W2, b2, W3, b3)
+        records = self.render_tiles_per_pixel_records(base, Wimg, Himg, TW, TH, thr, float(beta), float(temp),
+                                                      name="render_tiles_backward_featattr_per_pixel")
         return self.feature_gradients_from_records(records, feat_attr, grad_out_feat.contiguous())
 
     @staticmethod

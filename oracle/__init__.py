@@ -256,6 +256,33 @@ def records(rays_o, rays_d, pos, log_s, quats, cand, offsets, freq, att, W1, b1,
             "offsets": offs, "overflow": bool(ovf[0])}
 
 
+def records_per_pixel(rays_o, rays_d, pos, log_s, quats, cand, offsets, freq, att, W1, b1, W2, b2, W3, b3,
+                      W, H, TW, TH, thr, *, beta=1.5, temp=2.0, nthreads=0):
+    """Training records in per-pixel order -> the dict of :func:`records` (overflow: a pixel met a 257th hit)."""
+    args, keep = _scene_args(rays_o, rays_d, pos, log_s, quats, cand, offsets, freq, att, W1, b1, W2, b2, W3, b3)
+    B = W * H
+    counts = np.zeros(B, np.int32)
+    tail = (int(W), int(H), int(TW), int(TH), C.c_float(thr), C.c_float(beta), C.c_float(temp))
+    fn = lib().mlpsp_oracle_records_per_pixel
+    fn.restype = C.c_int
+    ovf = fn(*args, *tail, _p(counts, _i), None, None, None, None, None, None, None, None, int(nthreads))
+    offs = np.zeros(B + 1, np.int64)
+    np.cumsum(counts, out=offs[1:])
+    R = int(offs[-1])
+    ids = np.zeros(R, np.int32)
+    x6 = np.zeros((R, 6), np.float32)
+    masks = np.zeros((R, 2), np.int32)
+    raw = np.zeros((R, 8), np.float32)
+    gates = np.zeros((R, 4), np.float32)
+    rgb = np.zeros((B, 3), np.float32)
+    alpha = np.zeros((B, 1), np.float32)
+    fn(*args, *tail, _p(counts, _i), _p(offs, _l), _p(ids, _i), _p(x6, _f), _p(masks, _i), _p(raw, _f), _p(gates, _f),
+       _p(rgb, _f), _p(alpha, _f), int(nthreads))
+    del keep
+    return {"rgb": rgb, "alpha": alpha, "ids": ids, "x6": x6, "raw": raw, "masks": masks, "gates": gates,
+            "offsets": offs, "overflow": bool(ovf)}
+
+
 def render_per_pixel(rays_o, rays_d, pos, log_s, quats, cand, offsets, freq, att, W1, b1, W2, b2, W3, b3,
                      W, H, TW, TH, thr, *, feat_attr=None, beta=1.5, temp=2.0, nthreads=0):
     """Returns dict(rgb, alpha, feat|None, overflow: bool)."""

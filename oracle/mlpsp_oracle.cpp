@@ -1111,6 +1111,87 @@ ORACLE_API int mlpsp_oracle_render_per_pixel(
 }
 
 // ------------------------------------------------------------------------------------------
+// Training records in PER-PIXEL order: what render_tiles_backward_count_per_pixel / _emit_per_pixel traverse
+// (scannet/cuda/np_tile_kernels.cu:1211-1836: gather <= 256 hits in list order, stable sort by the pixel's own t,
+// blend until T < 1e-3), with the record schema of the tile-centre records (:3138-3154) and the record kernels'
+// MLP arithmetic (mlp_eval_rgb_sigma).  Two-phase: ids == nullptr -> counts[B]; else records at
+// rec_offsets[pix] + k and the image.  Returns 1 if some pixel met a 257th hit.
+// ------------------------------------------------------------------------------------------
+ORACLE_API int mlpsp_oracle_records_per_pixel(
+    const float* rays_o, const float* rays_d, const float* pos, const float* logs, const float* quats,
+    const int32_t* cand, const int32_t* offsets, const float* freq, const float* att, int F,
+    const float* W1, const float* b1, const float* W2, const float* b2, const float* W3, const float* b3,
+    int N, int H, int Wimg, int Himg, int TW, int TH, float thr, float beta, float temp,
+    int32_t* counts, const int64_t* rec_offsets, int32_t* ids, float* x6_out, int32_t* masks_out,
+    float* raw_out, float* gates_out, float* out_rgb, float* out_alpha, int nthreads) {
+  Scene S{};
+  S.rays_o = rays_o; S.rays_d = rays_d; S.pos = pos; S.logs = logs; S.quats = quats;
+  S.cand = cand; S.offsets = offsets; S.freq = freq; S.att = att; S.F = F;
+  S.W1 = W1; S.b1 = b1; S.W2 = W2; S.b2 = b2; S.W3 = W3; S.b3 = b3; S.N = N; S.H = H;
+  S.Wimg = Wimg; S.Himg = Himg; S.TW = TW; S.TH = TH; S.thr = thr;
+  const int ntx = (Wimg + TW - 1) / TW;
+  constexpr int MAXI = 256;
+  int overflow = 0;
+  if (nthreads <= 0) nthreads = omp_get_max_threads();
+#pragma omp parallel for schedule(dynamic, 64) num_threads(nthreads) reduction(| : overflow)
+  for (int pix = 0; pix < Wimg * Himg; ++pix) {
+    const int x = pix % Wimg, y = pix / Wimg;
+    const int tile = (y / TH) * ntx + (x / TW);
+    const float* ro = rays_o + (size_t)pix * 3;
+    const float* rd = rays_d + (size_t)pix * 3;
+    struct Rec { Hit h; int p; };
+    std::vector<Rec> recs;
+    for (int k = offsets[tile]; k < offsets[tile + 1]; ++k) {
+      const int p = cand[k];
+      const Prim P = load_prim(pos, logs, quats, p);
+      Hit h;
+      if (hit_rot(ro[0], ro[1], ro[2], rd[0], rd[1], rd[2], P, thr, h)) {
+        if ((int)recs.size() < MAXI) recs.push_back(Rec{h, p});
+        else { overflow |= 1; break; }
+      }
+    }
+    std::stable_sort(recs.begin(), recs.end(), [](const Rec& a, const Rec& b) { return a.h.t < b.h.t; });
+    float trans = 1.f, cr = 0.f, cg = 0.f, cb = 0.f;
+    int used = 0;
+    for (const Rec& rec : recs) {
+      if (trans < 1e-3f) break;
+      const float v6[6] = {rd[0], rd[1], rd[2], rec.h.dx, rec.h.dy, rec.h.dz};
+      float o[4];
+      uint32_t mk[2];
+      mlp_f32_records(v6, freq, att, mlp_of(S, rec.p), o, mk);
+      const float R = o_sigmoid(o[0]), G = o_sigmoid(o[1]), Bc = o_sigmoid(o[2]);
+      const float sigma_raw = o_softplus(o[3]);
+      const float alpha = 1.f - det_exp(-(sigma_raw * rec.h.decay));
+      if (ids) {
+        const int64_t r = rec_offsets[pix] + used;
+        ids[r] = rec.p;
+        for (int c = 0; c < 6; ++c) x6_out[r * 6 + c] = v6[c];
+        masks_out[r * 2] = (int32_t)mk[0];
+        masks_out[r * 2 + 1] = (int32_t)mk[1];
+        float* raw = raw_out + r * 8;
+        raw[0] = R; raw[1] = G; raw[2] = Bc; raw[3] = sigma_raw;
+        raw[4] = trans; raw[5] = alpha; raw[6] = rec.h.decay; raw[7] = o[3];
+        const Prim P = load_prim(pos, logs, quats, rec.p);
+        tetra_gates(rec.h.qlx, rec.h.qly, rec.h.qlz, P.lgx, P.lgy, P.lgz, beta, temp, gates_out + r * 4);
+        const float weight = trans * alpha;
+        cr = fmaf(weight, R, cr);
+        cg = fmaf(weight, G, cg);
+        cb = fmaf(weight, Bc, cb);
+      }
+      trans *= (1.f - alpha);
+      ++used;
+    }
+    if (!ids) {
+      counts[pix] = used;
+    } else {
+      out_rgb[pix * 3] = cr; out_rgb[pix * 3 + 1] = cg; out_rgb[pix * 3 + 2] = cb;
+      out_alpha[pix] = 1.f - trans;
+    }
+  }
+  return overflow;
+}
+
+// ------------------------------------------------------------------------------------------
 // Reverse compositing over saved forward records (scannet/cuda/primitive_records.cuh:3-46): per pixel, last
 // record first, the adjoint d4 of the four pre-activation MLP outputs of every record and the geometry
 // gradients that flow through the Gaussian falloff `decay` (the hit offset x6[3:6] is treated as given):

@@ -146,3 +146,47 @@ def test_scene_renders_rgb_and_features_with_gradients(device):
     (_framebuffer64(records, leaf, *scene.image_size) * g_feat.cpu().double()).sum().backward()
     torch.testing.assert_close(both_attr.cpu().double(), leaf.grad, atol=2e-6 * max(float(leaf.grad.abs().max()), 1.0),
                                rtol=2e-5)
+
+
+def test_per_pixel_order_serves_both_adjoints_from_its_records(device, monkeypatch):
+    """scannet/cumodel.py:492-600: (rgb, feature image) in per-pixel order under autograd.  The forward equals the
+    no-grad render; the attribute gradient is the float64 definition over the per-pixel records; the RGB gradients
+    are those of the RGB-only render in the same order."""
+    monkeypatch.setenv("MLPSP_TILE_ORDER", "per_pixel")
+    fr, scene, (ro, rd), view, proj = _scene(device, n=300, width=24, height=16, channels=6)
+    names = ("positions", "log_scales", "quats", "W1", "b1", "W2", "b2", "W3", "b3")
+    args = dict(score_threshold=fr.thr, view_matrix=view, proj_matrix=proj)
+    rgb, feat = scene(ro, rd, return_feature=True, **args)
+    with torch.no_grad():
+        rgb0, feat0 = scene(ro, rd, return_feature=True, **args)
+    assert rgb.requires_grad and feat.requires_grad and torch.equal(rgb, rgb0) and torch.equal(feat, feat0)
+    torch.manual_seed(4)
+    g_rgb, g_feat = torch.randn_like(rgb), torch.randn_like(feat)
+    ((rgb * g_rgb).sum() + (feat * g_feat).sum()).backward()
+    both = {k: getattr(scene, k).grad.clone() for k in names}
+    attr_grad = scene.feat_attr.grad.clone()
+    scene.zero_grad(set_to_none=True)
+    (scene(ro, rd, **args) * g_rgb).sum().backward()
+    for k in names:
+        torch.testing.assert_close(both[k], getattr(scene, k).grad, atol=1e-6, rtol=1e-5, msg=lambda m, k=k: f"{k}: {m}")
+    scene.zero_grad(set_to_none=True)
+    _, feat = scene(ro, rd, return_feature=True, **args)
+    (feat * g_feat).sum().backward()
+    assert all(getattr(scene, k).grad is None for k in names)
+    torch.testing.assert_close(scene.feat_attr.grad, attr_grad, atol=1e-6, rtol=1e-5)
+    from mlp_splatting_amd.cumodel import NeuralPrimitiveSceneTileCUDA
+    ext = NeuralPrimitiveSceneTileCUDA._ensure_tile_ext_static()
+    cand, off = scene._tile_lists(ro, rd, fr.thr, view, proj, None, None, device)
+    base = scene._base_args(ro, rd, cand, off, device)
+    records = ext.render_tiles_per_pixel_records(base, *scene.image_size, 8, 8, fr.thr, float(scene.feature_gating_beta),
+                                                 float(scene.feature_gating_temp))
+    direct = ext.render_tiles_backward_featattr_per_pixel(*base, scene.feat_attr.detach().contiguous(), g_feat,
+                                                          float(scene.feature_gating_beta),
+                                                          float(scene.feature_gating_temp), *scene.image_size, 8, 8, fr.thr)
+    assert torch.equal(direct, attr_grad)
+    leaf = scene.feat_attr.detach().cpu().double().requires_grad_(True)
+    image64 = _framebuffer64(records, leaf, *scene.image_size)
+    torch.testing.assert_close(image64.float(), feat0.cpu(), atol=3e-6, rtol=3e-6)
+    (image64 * g_feat.cpu().double()).sum().backward()
+    torch.testing.assert_close(attr_grad.cpu().double(), leaf.grad, atol=2e-6 * max(float(leaf.grad.abs().max()), 1.0),
+                               rtol=2e-5)

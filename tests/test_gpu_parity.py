@@ -358,6 +358,44 @@ def test_per_pixel_render_is_bit_exact(device, oracle_mod, with_feat):
     assert np.abs(tc["rgb"] - want["rgb"]).max() > 1e-4
 
 
+@pytest.mark.parametrize("tile,hidden,n,size", [(8, 32, 1200, (56, 40)), (16, 16, 900, (50, 30)), (8, 7, 700, (33, 17)),
+                                                (4, 32, 500, (21, 13))])
+def test_per_pixel_records_are_bit_exact(device, oracle_mod, tile, hidden, n, size):
+    """mlpsp_records_per_pixel_count / _emit against the oracle's records_per_pixel: counts, offsets, every record
+    field and the image, to the bit."""
+    from mlp_splatting_amd.tile_ext import TileExt
+    fr = Frame("cfg1_5k_160x120", n=n, hidden=hidden, width=size[0], height=size[1], tile=tile)
+    cand, off = fr.oracle_lists(oracle_mod)
+    want = oracle_mod.records_per_pixel(*fr.base_numpy(cand, off), *fr.dims, beta=1.3, temp=2.2)
+    assert not want["overflow"] and want["offsets"][-1] > 500
+    ext = TileExt()
+    base = fr.base_torch(cand, off, device)
+    counts = ext.render_tiles_backward_count_per_pixel(*base, fr.W, fr.H, tile, tile, fr.thr)
+    assert counts.dtype == torch.int32
+    np.testing.assert_array_equal(counts.cpu().numpy(), np.diff(want["offsets"]))
+    rgb, alpha, ids, x6, raw, masks, gates, offsets = ext.render_tiles_per_pixel_records(base, fr.W, fr.H, tile, tile,
+                                                                                         fr.thr, 1.3, 2.2)
+    np.testing.assert_array_equal(offsets.cpu().numpy(), want["offsets"])
+    np.testing.assert_array_equal(ids.cpu().numpy(), want["ids"])
+    np.testing.assert_array_equal(masks.cpu().numpy(), want["masks"])
+    for got, key in ((x6, "x6"), (raw, "raw"), (gates, "gates"), (rgb, "rgb"), (alpha, "alpha")):
+        _assert_bits(got, want[key], key)
+    # the order differs from the tile-centre records on a real frame
+    tc = oracle_mod.records(*fr.base_numpy(cand, off), *fr.dims, max_hits=512)
+    assert tile == 4 or not (len(tc["ids"]) == len(want["ids"]) and np.array_equal(tc["ids"], want["ids"]))
+
+
+def test_per_pixel_records_refuse_a_257th_hit(device):
+    from mlp_splatting_amd.tile_ext import TileExt
+    from test_gpu_contract import _renderer_inputs, _base
+    ext = TileExt()
+    d = _renderer_inputs(257, device)
+    with pytest.raises(RuntimeError, match="per-pixel intersection capacity 256 exceeded"):
+        ext.render_tiles_backward_count_per_pixel(*_base(d), 1, 1, 1, 1, 0.005)
+    ok = ext.render_tiles_backward_count_per_pixel(*_base(_renderer_inputs(256, device)), 1, 1, 1, 1, 0.005)
+    assert 0 < int(ok[0]) <= 256
+
+
 @pytest.mark.parametrize("tile,hidden", [(8, 32), (16, 16), (8, 8)])
 def test_statistics_forward_against_oracle(device, oracle_mod, tile, hidden):
     # np_tile_kernels.cu:2139-2519.  Image bit-exact; integer statistics and the maximum exact; the two

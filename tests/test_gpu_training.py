@@ -19,7 +19,7 @@ pytestmark = pytest.mark.gpu
 PARAMS = ("positions", "log_scales", "quats", "W1", "b1", "W2", "b2", "W3", "b3")
 
 
-def _float64_gradients(scene, fr, device, weight_img, bg):
+def _float64_gradients(scene, fr, device, weight_img, bg, per_pixel=False):
     """d/dparams of  sum(weight_img * rgb)  with rgb recomposed from the frame's records in float64."""
     ext = scene._ensure_tile_ext()
     with torch.no_grad():
@@ -31,7 +31,12 @@ def _float64_gradients(scene, fr, device, weight_img, bg):
              torch.nn.functional.normalize(scene.quats.detach(), dim=-1).contiguous(), cand, off.to(torch.int32), freq, att,
              *[getattr(scene, k).detach().contiguous() for k in PARAMS[3:]]]
         x += [torch.zeros_like(x[0]), torch.zeros(fr.W * fr.H, device=device)]
-        rgb, alpha, ids, x6, raw, masks, gates, offsets = ext.render_tiles_training_records(x, fr.W, fr.H, 8, fr.thr, 1.5, 2.0)
+        if per_pixel:
+            rgb, alpha, ids, x6, raw, masks, gates, offsets = ext.render_tiles_per_pixel_records(x[:15], fr.W, fr.H, 8, 8,
+                                                                                                 fr.thr, 1.5, 2.0)
+        else:
+            rgb, alpha, ids, x6, raw, masks, gates, offsets = ext.render_tiles_training_records(x, fr.W, fr.H, 8, fr.thr,
+                                                                                                1.5, 2.0)
     ids, x6, offsets = ids.cpu().long(), x6.cpu().double(), offsets.cpu()
     leaves = {k: getattr(scene, k).detach().cpu().double().requires_grad_(True) for k in PARAMS}
     freq, att = freq.cpu().double(), att.cpu().double()
@@ -84,6 +89,39 @@ def test_scene_gradients_match_float64_autograd_over_the_same_records(device, or
         assert scale > 1e-4, k
         assert float((g - w).abs().max()) <= 2e-3 * scale, (k, float((g - w).abs().max()), scale)
         assert float((g - w).norm() / w.norm()) < 1e-3, k
+
+
+def test_per_pixel_order_gradients_match_float64_autograd_over_its_records(device, oracle_mod, monkeypatch):
+    """MLPSP_TILE_ORDER=per_pixel: the backward of the per-pixel order (scannet/cumodel.py:297-364) through the
+    per-pixel records, against the same float64 restatement over those records; the forward is the per-pixel
+    render."""
+    monkeypatch.setenv("MLPSP_TILE_ORDER", "per_pixel")
+    fr = Frame("cfg1_5k_160x120", n=600, hidden=32, width=32, height=24)
+    scene = _scene_from(fr, device).train()
+    torch.manual_seed(1)
+    weight_img = torch.randn(fr.W * fr.H, 3, device=device)
+    bg = torch.tensor([0.3, 0.1, 0.7], device=device)
+    args = dict(score_threshold=fr.thr, bg_color=bg, view_matrix=to_dev(fr.view, device),
+                proj_matrix=to_dev(fr.proj, device))
+    rgb = scene(to_dev(fr.rays_o, device), to_dev(fr.rays_d, device), **args)
+    with torch.no_grad():
+        plain = scene(to_dev(fr.rays_o, device), to_dev(fr.rays_d, device), **args)
+    assert rgb.requires_grad and torch.equal(rgb, plain)
+    (rgb * weight_img).sum().backward()
+    want, num_records, _ = _float64_gradients(scene, fr, device, weight_img, bg, per_pixel=True)
+    assert num_records > 1500
+    for k in PARAMS:
+        got = getattr(scene, k).grad
+        assert got is not None and got.shape == getattr(scene, k).shape, k
+        g, w = got.cpu().double(), want[k]
+        scale = float(w.abs().max())
+        assert scale > 1e-4, k
+        assert float((g - w).abs().max()) <= 2e-3 * scale, (k, float((g - w).abs().max()), scale)
+        assert float((g - w).norm() / w.norm()) < 1e-3, k
+    monkeypatch.setenv("MLPSP_TILE_ORDER", "tilecenter")
+    scene.zero_grad(set_to_none=True)
+    other = scene(to_dev(fr.rays_o, device), to_dev(fr.rays_d, device), **args)
+    assert float((other.detach() - rgb.detach()).abs().max()) > 1e-5            # the two orders are different images here
 
 
 def test_inference_calls_are_untouched_by_the_training_path(device, oracle_mod):

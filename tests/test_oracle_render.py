@@ -276,6 +276,57 @@ def test_per_pixel_equals_tile_centre_on_one_pixel_tiles(oracle_mod):
     np.testing.assert_array_equal(a["alpha"], b["alpha"])
 
 
+def test_per_pixel_records_are_each_pixels_hits_in_its_own_depth_order(oracle_mod):
+    """Pins records_per_pixel by properties that do not restate it: on 1x1 tiles it IS the tile-centre records
+    forward; on 8x8 tiles every pixel's ids are a prefix of ALL its hits (brute force through the scalar hit
+    function) in ascending own-t order with list-order ties, cut where the transmittance falls below 1e-3; the
+    image recomposes from the raw fields and agrees with the per-pixel render (another MLP rounding: 2e-6)."""
+    from helpers import Frame
+    one = Frame("cfg1_5k_160x120", n=600, hidden=16, width=16, height=12, tile=1)
+    cand, off = one.oracle_lists(oracle_mod)
+    a = oracle_mod.records(*one.base_numpy(cand, off), *one.dims, max_hits=512, beta=1.3, temp=2.2)
+    b = oracle_mod.records_per_pixel(*one.base_numpy(cand, off), *one.dims, beta=1.3, temp=2.2)
+    assert a["offsets"][-1] > 300 and not b["overflow"]
+    for k in ("rgb", "alpha", "ids", "x6", "raw", "masks", "gates", "offsets"):
+        np.testing.assert_array_equal(a[k], b[k], err_msg=k)
+
+    from mlp_splatting_amd import synthetic as syn
+    fr = Frame("cfg1_5k_160x120", n=8, hidden=16, width=24, height=16, eye=(0.3, -0.2, -0.9), target=(0.0, 0.0, 0.0))
+    fr.scene = sc = syn.make_scene(160, 16, 11, -2.4, cluster_frac=1.0)      # dense cluster: some pixels saturate
+    cand, off = fr.oracle_lists(oracle_mod)
+    out = oracle_mod.records_per_pixel(*fr.base_numpy(cand, off), *fr.dims)
+    ren = oracle_mod.render_per_pixel(*fr.base_numpy(cand, off), *fr.dims)
+    np.testing.assert_allclose(out["rgb"], ren["rgb"], atol=2e-6)
+    np.testing.assert_allclose(out["alpha"], ren["alpha"], atol=2e-6)
+    offs, raw, ids = out["offsets"], out["raw"].astype(np.float64), out["ids"]
+    assert offs[-1] > 2000
+    ntx = (fr.W + 7) // 8
+    cut_short = 0
+    for pix in range(fr.W * fr.H):
+        tile = (pix // fr.W // 8) * ntx + (pix % fr.W) // 8
+        lst = cand[off[tile]:off[tile + 1]]
+        hit, t = [], []
+        for p in lst:
+            is_hit, h = oracle_mod.hit(fr.rays_o[pix], fr.rays_d[pix], sc.positions[p], sc.log_scales[p], sc.quats[p], fr.thr)
+            if is_hit:
+                hit.append(int(p))
+                t.append(np.float32(h["t"]))
+        order = np.argsort(np.asarray(t, np.float32), kind="stable")
+        want = np.asarray(hit, np.int64)[order]
+        got = ids[offs[pix]:offs[pix + 1]]
+        assert len(got) <= len(want) and np.array_equal(got, want[:len(got)]), pix
+        if len(got) < len(want):                       # stopped early: only because the pixel is saturated
+            last = raw[offs[pix + 1] - 1]
+            assert last[4] * (1 - last[5]) < 1e-3 and last[4] >= 1e-3
+            cut_short += 1
+    assert cut_short > 0
+    pix_of = np.repeat(np.arange(fr.W * fr.H), np.diff(offs))
+    rgb = np.zeros((fr.W * fr.H, 3))
+    np.add.at(rgb, pix_of, (raw[:, 4] * raw[:, 5])[:, None] * raw[:, :3])
+    np.testing.assert_allclose(rgb, out["rgb"], atol=2e-6)
+    assert np.array_equal(out["x6"][:, :3], fr.rays_d[pix_of])
+
+
 # ---------------------------------------------------------------------------------------------
 # feature channel
 # ---------------------------------------------------------------------------------------------
