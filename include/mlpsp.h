@@ -418,12 +418,15 @@ int mlpsp_stream_feature_l1(const int32_t* ids_dev, const int64_t* pixel_offsets
  * row of the CSR (csr_offsets [N+1]) to its record, record_pixels [R] (int32) gives a record's pixel; segments as
  * for mlpsp_grouped_vjp.  mixed != 0 rounds both factors of every product to fp16 (f32 accumulation).
  * partial_dev [mlpsp_segment_reduce_rows(num_groups), slots, channels] is scratch (per-segment sums, then the
- * chunk sums of the per-primitive reduction), out_dev [N, slots, channels] the result. */
+ * chunk sums of the per-primitive reduction), out_dev [N, slots, channels] the result.  group_order_dev (int64
+ * [num_groups], a permutation, or NULL): the order in which the segments are launched; sorted by the segments' first
+ * pixels, concurrent workgroups read neighbouring sign rows.  The result does not depend on it. */
 int mlpsp_feature_attribute_gradients(const int8_t* signs_dev, const int64_t* record_indices_dev,
                                       const int32_t* record_pixels_dev, const float* raw_dev, const float* gates_dev,
                                       const int64_t* csr_offsets_dev, const int64_t* group_primitives_dev,
                                       const int64_t* group_starts_dev, const int64_t* group_offsets_dev,
-                                      int64_t num_groups, int num_primitives, int width, int height, int target_width,
+                                      const int64_t* group_order_dev, int64_t num_groups, int num_primitives,
+                                      int width, int height, int target_width,
                                       int target_height, int channels, int slots, int segment, int mixed,
                                       float* partial_dev, float* out_dev, mlpsp_stream_t stream);
 
@@ -433,15 +436,17 @@ int mlpsp_feature_attribute_gradients(const int8_t* signs_dev, const int64_t* re
  * grad_feat[record's pixel, c] (one slot: no gate; five slots: slot 0 has no gate).  The reference traverses the
  * frame again and adds with atomics; here the records saved by the records forward are used, in the layout of
  * mlpsp_feature_attribute_gradients (record_indices, record_pixels, csr_offsets, segments), and summed in a fixed
- * order.  grad_feat_dev [pixels, channels] f32; gates_dev may be NULL for one slot.
+ * order.  grad_feat_dev [pixels, channels] f32; gates_dev may be NULL for one slot.  group_order_dev (int64
+ * [num_groups], a permutation, or NULL) is the order in which the segments are launched: sorted by the segments' first
+ * pixels, concurrent workgroups read neighbouring rows of grad_feat; the result does not depend on it.
  * partial_dev [mlpsp_segment_reduce_rows(num_groups), slots, channels] is scratch, out_dev [N, slots, channels]. */
 int mlpsp_feature_dense_attribute_gradients(const float* grad_feat_dev, const int64_t* record_indices_dev,
                                             const int32_t* record_pixels_dev, const float* raw_dev,
                                             const float* gates_dev, const int64_t* csr_offsets_dev,
                                             const int64_t* group_primitives_dev, const int64_t* group_starts_dev,
-                                            const int64_t* group_offsets_dev, int64_t num_groups, int num_primitives,
-                                            int channels, int slots, int segment, float* partial_dev, float* out_dev,
-                                            mlpsp_stream_t stream);
+                                            const int64_t* group_offsets_dev, const int64_t* group_order_dev,
+                                            int64_t num_groups, int num_primitives, int channels, int slots, int segment,
+                                            float* partial_dev, float* out_dev, mlpsp_stream_t stream);
 
 /* Measurement aid, no counterpart in the reference: launches a kernel that does nothing but
  * v_mfma_f32_32x32x16_bf16 on register operands (2,048 workgroups x 4 wavefronts x iterations x 8

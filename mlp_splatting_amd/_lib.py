@@ -71,10 +71,10 @@ SIGNATURES = {
     "mlpsp_reduce_partials": (_i, [_vp, _vp, _vp, _i64, _i, _vp, _vp, _vp]),
     "mlpsp_reduce_partials_split": (_i, [_vp, _vp, _vp, _i64, _i] + [_vp] * 8),
     "mlpsp_stream_feature_l1": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp]),
-    "mlpsp_feature_attribute_gradients": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i, _i, _i, _i, _i, _i,
-                                               _i, _i, _i, _vp, _vp, _vp]),
-    "mlpsp_feature_dense_attribute_gradients": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i, _i, _i, _i,
-                                                     _vp, _vp, _vp]),
+    "mlpsp_feature_attribute_gradients": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i, _i, _i, _i, _i,
+                                               _i, _i, _i, _i, _vp, _vp, _vp]),
+    "mlpsp_feature_dense_attribute_gradients": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i, _i, _i,
+                                                     _i, _vp, _vp, _vp]),
     "mlpsp_records_reverse_adjoints": (_i, [_vp, _vp, _vp, _vp, _vp, _i64, _vp, _vp, _vp]),
     "mlpsp_geometry_gradients": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i, _i, _vp, _vp, _vp, _vp,
                                       _vp]),

@@ -128,13 +128,16 @@ __global__ __launch_bounds__(64) void feature_vjp_kernel(const int8_t* __restric
                                                          const long long* __restrict__ offsets,
                                                          const long long* __restrict__ group_prim,
                                                          const long long* __restrict__ group_start,
+                                                         const long long* __restrict__ group_order,
                                                          float* __restrict__ partial, int W, int H, int WF, int HF, int C,
                                                          int segment) {
   constexpr int ROWS = SLOTS == 5 ? 8 : 4;                   // slot rows kept in LDS (two products for five slots)
   __shared__ __attribute__((aligned(16))) RecordTaps s_rec[64];
   __shared__ __attribute__((aligned(16))) float s_a[ROWS][64];          // f32 factors, [slot][record]
   __shared__ __attribute__((aligned(8))) _Float16 s_ah[ROWS][64];       // the same rounded to fp16 (mixed)
-  const long long group = blockIdx.x;
+  // group_order (optional): the segment that workgroup x takes; in the order of the segments' first pixels,
+  // workgroups that run together read neighbouring sign rows
+  const long long group = group_order ? group_order[blockIdx.x] : (long long)blockIdx.x;
   const int lane = threadIdx.x, m = lane & 3;
   const int c0 = blockIdx.y * 256 + lane * 4;
   const long long p = group_prim[group];
@@ -277,11 +280,14 @@ __global__ __launch_bounds__(64) void feature_dense_vjp_kernel(const float* __re
                                                                const long long* __restrict__ offsets,
                                                                const long long* __restrict__ group_prim,
                                                                const long long* __restrict__ group_start,
+                                                               const long long* __restrict__ group_order,
                                                                float* __restrict__ partial, int C, int segment) {
   constexpr int ROWS = SLOTS == 5 ? 8 : 4;
   __shared__ long long s_row[64];                                       // pixel * C of the staged records
   __shared__ __attribute__((aligned(16))) float s_a[ROWS][64];          // factors, [slot][record]
-  const long long group = blockIdx.x;
+  // group_order (optional): the segment that workgroup x takes.  Launched in the order of the segments' first
+  // pixels, workgroups that run together read neighbouring adjoint rows and share them in L2.
+  const long long group = group_order ? group_order[blockIdx.x] : (long long)blockIdx.x;
   const int lane = threadIdx.x, m = lane & 3;
   const int c0 = blockIdx.y * 256 + lane * 4;
   const long long p = group_prim[group];
@@ -402,8 +408,9 @@ MLPSP_API int mlpsp_feature_attribute_gradients(const int8_t* signs_dev, const i
                                                 const int32_t* record_pixels_dev, const float* raw_dev,
                                                 const float* gates_dev, const int64_t* csr_offsets_dev,
                                                 const int64_t* group_primitives_dev, const int64_t* group_starts_dev,
-                                                const int64_t* group_offsets_dev, int64_t num_groups,
-                                                int num_primitives, int width, int height, int target_width,
+                                                const int64_t* group_offsets_dev, const int64_t* group_order_dev,
+                                                int64_t num_groups, int num_primitives, int width, int height,
+                                                int target_width,
                                                 int target_height, int channels, int slots, int segment, int mixed,
                                                 float* partial_dev, float* out_dev, mlpsp_stream_t stream) {
   if (width <= 0 || height <= 0 || target_width <= 0 || target_height <= 0 || channels <= 0 || segment <= 0)
@@ -422,8 +429,8 @@ MLPSP_API int mlpsp_feature_attribute_gradients(const int8_t* signs_dev, const i
   hipLaunchKernelGGL((feature_vjp_kernel<SL, MX, VC>), grid, block, 0, s, signs_dev,                               \
                      (const long long*)record_indices_dev, record_pixels_dev, raw_dev, gates_dev,                  \
                      (const long long*)csr_offsets_dev, (const long long*)group_primitives_dev,                    \
-                     (const long long*)group_starts_dev, partial_dev, width, height, target_width, target_height,  \
-                     channels, segment)
+                     (const long long*)group_starts_dev, (const long long*)group_order_dev, partial_dev, width,    \
+                     height, target_width, target_height, channels, segment)
 #define MLPSP_FV_SLOTS(MX, VC)                         \
   do {                                                 \
     if (slots == 1) MLPSP_FV_LAUNCH(1, MX, VC);        \
@@ -458,7 +465,8 @@ MLPSP_API int mlpsp_feature_dense_attribute_gradients(const float* grad_feat_dev
                                                       const float* gates_dev, const int64_t* csr_offsets_dev,
                                                       const int64_t* group_primitives_dev,
                                                       const int64_t* group_starts_dev, const int64_t* group_offsets_dev,
-                                                      int64_t num_groups, int num_primitives, int channels, int slots,
+                                                      const int64_t* group_order_dev, int64_t num_groups,
+                                                      int num_primitives, int channels, int slots,
                                                       int segment, float* partial_dev, float* out_dev,
                                                       mlpsp_stream_t stream) {
   if (channels <= 0 || segment <= 0 || num_groups < 0 || num_groups > 2147483647LL || num_primitives < 0)
@@ -475,7 +483,8 @@ MLPSP_API int mlpsp_feature_dense_attribute_gradients(const float* grad_feat_dev
   hipLaunchKernelGGL((feature_dense_vjp_kernel<SL, VC>), grid, block, 0, s, grad_feat_dev,                         \
                      (const long long*)record_indices_dev, record_pixels_dev, raw_dev, gates_dev,                  \
                      (const long long*)csr_offsets_dev, (const long long*)group_primitives_dev,                    \
-                     (const long long*)group_starts_dev, partial_dev, channels, segment)
+                     (const long long*)group_starts_dev, (const long long*)group_order_dev, partial_dev, channels,  \
+                     segment)
 #define MLPSP_FD_SLOTS(VC)                         \
   do {                                             \
     if (slots == 1) MLPSP_FD_LAUNCH(1, VC);        \

@@ -9,6 +9,8 @@ loss (scannet/record_feature_loss.py:1-6).  The kernels are libmlpsp_hip's ``mlp
 """
 from __future__ import annotations
 
+import os
+
 import torch
 
 from . import _lib
@@ -16,6 +18,15 @@ from . import _lib
 
 def _ptr(t):
     return None if t is None else t.data_ptr()
+
+
+def _launch_order(pixels, csr, starts):
+    """Segments sorted by their first pixels (int64 permutation, or None): workgroups that run together then read
+    neighbouring rows of the adjoint (or sign) image and find them in L2.  MLPSP_FEATURE_VJP_ORDER=primitive keeps
+    the primitive-major launch order; the sums do not depend on it."""
+    if len(starts) < 2 or os.environ.get("MLPSP_FEATURE_VJP_ORDER", "pixel") == "primitive":
+        return None
+    return torch.argsort(pixels[csr.record_indices[starts]].to(torch.int64))
 
 
 def streaming_feature_l1(records, attributes, target, width, height, *, debug=False):
@@ -68,10 +79,12 @@ def feature_weight_gradients(records, csr, signs, attributes, width, height, *, 
     rows = int(_lib.load().mlpsp_segment_reduce_rows(len(primitives)))      # per-segment sums + the reduction's chunk sums
     partial = torch.empty((max(rows, 1), slots, channels), device=device, dtype=torch.float32)
     result = torch.empty_like(attributes)
+    order = _launch_order(pixels, csr, starts)
     with torch.cuda.device(device):
         rc = _lib.load().mlpsp_feature_attribute_gradients(
             _ptr(signs), _ptr(csr.record_indices), _ptr(pixels), _ptr(raw), _ptr(gates), _ptr(csr.offsets),
-            _ptr(primitives), _ptr(starts), _ptr(group_offsets), int(len(primitives)), int(len(attributes)), int(width),
+            _ptr(primitives), _ptr(starts), _ptr(group_offsets), _ptr(order), int(len(primitives)), int(len(attributes)),
+            int(width),
             int(height), int(wf), int(hf), int(channels), int(slots), int(segment_size), int(bool(mixed)),
             _ptr(partial), _ptr(result), torch.cuda.current_stream(device).cuda_stream)
     if rc != 0:
@@ -104,10 +117,11 @@ def dense_feature_attribute_gradients(records, csr, grad_feature, attributes, *,
     rows = int(_lib.load().mlpsp_segment_reduce_rows(len(primitives)))
     partial = torch.empty((max(rows, 1), slots, channels), device=device, dtype=torch.float32)
     result = torch.empty(attributes.shape, device=device, dtype=torch.float32)
+    order = _launch_order(pixels, csr, starts)
     with torch.cuda.device(device):
         rc = _lib.load().mlpsp_feature_dense_attribute_gradients(
             _ptr(grad_feature), _ptr(csr.record_indices), _ptr(pixels), _ptr(raw), _ptr(gates), _ptr(csr.offsets),
-            _ptr(primitives), _ptr(starts), _ptr(group_offsets), int(len(primitives)), int(len(attributes)),
+            _ptr(primitives), _ptr(starts), _ptr(group_offsets), _ptr(order), int(len(primitives)), int(len(attributes)),
             int(channels), int(slots), int(segment_size), _ptr(partial), _ptr(result),
             torch.cuda.current_stream(device).cuda_stream)
     if rc != 0:
