@@ -209,7 +209,8 @@ def render_tilecenter_stats_f32(rays_o, rays_d, records, order, tile_offsets, fr
 
 
 def training_records(rays_o, rays_d, records, order, tile_offsets, freq, att, W1, b1, W2, b2, W3, b3, W, H, TW, TH,
-                     threshold, beta, temp, max_hits, path_name="render_tiles_training_records", render_order=False):
+                     threshold, beta, temp, max_hits, path_name="render_tiles_training_records", render_order=False,
+                     counts_only=False):
     """Training-records forward -> (rgb, alpha, ids, x6, raw, masks, gates, offsets int64 [B+1]);
     raises the reference's hit-capacity error (np_tile_kernels.cu:4601-4609).  ``render_order``: layer 2 rounded as
     the render kernels round it, which makes image and records those of the f32 render bit for bit."""
@@ -233,6 +234,8 @@ def training_records(rays_o, rays_d, records, order, tile_offsets, freq, att, W1
     total, over = int(offsets[-1].item()), int(overflow.item())
     if over:
         refuse()
+    if counts_only:
+        return counts
     ids = torch.empty(total, dtype=torch.int32, device=dev)
     x6 = torch.empty(total, 6, dtype=torch.float32, device=dev)
     masks = torch.empty(total, 2, dtype=torch.int32, device=dev)

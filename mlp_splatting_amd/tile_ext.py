@@ -21,9 +21,6 @@ MAX_TILE_PRIMS = 1536          # MLPSP_MAX_TILE_PRIMS as built by scannet/cumode
 MAX_H_TILECENTER = 32          # MLPSP_MAX_H (np_tile_kernels.cu:36-38)
 
 _BACKWARD_ONLY = (
-    "render_tiles_backward_count_tilecenter",
-    "render_tiles_backward_emit_per_pixel", "render_tiles_backward_emit_tilecenter",
-    "render_tiles_backward_tilecenter_full_with_feat",
     "render_tiles_mlp_records",
     "render_tiles_backward_tilecenter_traversal",
     "render_tiles_backward_tilecenter_backprop_noatomic",
@@ -376,16 +373,18 @@ class TileExt:
     # ------------------------------------------------------------------------------------------
     # training-records forward (np_tile_kernels.cu:6897-6998, forward_only = true)
     # ------------------------------------------------------------------------------------------
-    def render_tiles_training_records(self, x, width, height, tile, threshold, beta, temp, *, render_order=False):
+    def render_tiles_training_records(self, x, width, height, tile, threshold, beta, temp, *, render_order=False,
+                                      any_tile=False, counts_only=False, name="render_tiles_mlp_records"):
         """[rgb, alpha, ids, x6, raw, masks, gates, offsets]: one record per hit and pixel, in each
         pixel's compositing order.  ``x`` = the 15 scene tensors + two adjoint placeholders that the
         forward-only mode never reads (scannet/csr_training.py:37-39).  ``render_order`` (not in the reference):
         image and records in the rounding of ``render_tiles_forward_tilecenter`` instead of the record kernels'
         own; see :meth:`records_forward_matches_render`."""
-        name = "render_tiles_mlp_records"
         _chk(len(x) == 17, "Expected 15 scene inputs and RGB/T adjoints")
         width, height, tile = int(width), int(height), int(tile)
-        _chk(width > 0 and height > 0 and tile in (8, 16), "the records forward supports 8x8 and 16x16 tiles")
+        # any_tile: the backward entry points, whose reference kernels take any square tile of up to 256 pixels
+        _chk(width > 0 and height > 0 and (tile in (8, 16) or (any_tile and 0 < tile * tile <= 256)),
+             "the records forward supports 8x8 and 16x16 tiles")
         for i, t in enumerate(x):
             _chk(t.is_cuda and t.is_contiguous(), "Inputs must be contiguous CUDA tensors")
             _chk(t.device == x[0].device, "Inputs must share a device")
@@ -407,9 +406,10 @@ class TileExt:
             if x[5].numel() > 0:
                 order, _ = ops.sort_tiles(x[0], x[1], rec, x[5], x[6], width, height, tile, tile, _lib.KEY_TSTAR,
                                           self.max_tile_prims, cull_threshold=float(threshold))
-            return list(ops.training_records(x[0], x[1], rec, order, x[6], x[7], x[8], *x[9:15], width, height, tile,
-                                             tile, float(threshold), float(beta), float(temp), self.max_hits, name,
-                                             render_order=bool(render_order)))
+            out = ops.training_records(x[0], x[1], rec, order, x[6], x[7], x[8], *x[9:15], width, height, tile, tile,
+                                       float(threshold), float(beta), float(temp), self.max_hits, name,
+                                       render_order=bool(render_order), counts_only=counts_only)
+            return out if counts_only else list(out)
 
     @staticmethod
     def records_forward_matches_render(freq, W1, b1, W2, b2, tile):
@@ -548,9 +548,100 @@ class TileExt:
         _chk(int(TW) == int(TH), "square tiles only")
         x = [rays_o, rays_d, positions, log_scales, quats, cand, offsets, freq, att, W1, b1, W2, b2, W3, b3,
              grad_rgb.contiguous(), grad_t.contiguous()]
-        records = self.render_tiles_training_records(x, Wimg, Himg, TW, thr, 1.5, 2.0)
+        records = self.render_tiles_training_records(x, Wimg, Himg, TW, thr, 1.5, 2.0, any_tile=True,
+                                                     name="render_tiles_backward_tilecenter_full")
         return self.backward_from_records(records, positions, log_scales, quats, freq, att, W1, b1, W2, b2, W3, b3,
                                           x[15], x[16])
+
+    def render_tiles_backward_tilecenter_full_with_feat(self, rays_o, rays_d, positions, log_scales, quats, cand, offsets,
+                                                        freq, att, W1, b1, W2, b2, W3, b3, feat_attr, grad_rgb, grad_t,
+                                                        grad_feat, beta, temp, Wimg, Himg, TW, TH, thr):
+        """The nine gradients of :meth:`render_tiles_backward_tilecenter_full` and grad_feat_attr of
+        :meth:`render_tiles_backward_featattr_tilecenter` from one traversal (np_tile_kernels.cu:7005-7114): here one
+        records forward and one grouping of its records."""
+        _chk(int(TW) == int(TH), "square tiles only")
+        self._check_feature_adjoint(feat_attr, grad_feat, positions, int(Wimg) * int(Himg))
+        x = [rays_o, rays_d, positions, log_scales, quats, cand, offsets, freq, att, W1, b1, W2, b2, W3, b3,
+             grad_rgb.contiguous(), grad_t.contiguous()]
+        records = self.render_tiles_training_records(x, Wimg, Himg, TW, thr, float(beta), float(temp), any_tile=True,
+                                                     name="render_tiles_backward_tilecenter_full_with_feat")
+        return self.backward_from_records(records, positions, log_scales, quats, freq, att, W1, b1, W2, b2, W3, b3,
+                                          x[15], x[16], feat_attr=feat_attr, grad_feat=grad_feat.contiguous())
+
+    @staticmethod
+    def _check_feature_adjoint(feat_attr, grad_out_feat, positions, pixels):
+        _chk(feat_attr.is_cuda and feat_attr.dtype == torch.float32 and feat_attr.is_contiguous())
+        _chk(feat_attr.dim() in (2, 3) and feat_attr.shape[0] == positions.shape[0],
+             "feat_attr first dimension must match primitive count")
+        _chk(feat_attr.dim() == 2 or feat_attr.shape[1] in (4, 5), "3D feat_attr expects slots in {4,5}")
+        _chk(grad_out_feat.is_cuda and grad_out_feat.dtype == torch.float32
+             and tuple(grad_out_feat.shape) == (pixels, feat_attr.shape[-1]), "grad_out_feat must be [B, C]")
+
+    def render_tiles_backward_count_tilecenter(self, rays_o, rays_d, positions, log_scales, quats, cand, offsets, freq,
+                                               att, W1, b1, W2, b2, W3, b3, Wimg, Himg, TW, TH, thr):
+        """counts [B] int32 of the tile-centre-order backward: the hits every pixel blends before its transmittance
+        falls below 1e-3 (np_tile_kernels.cu:6275-6340)."""
+        _chk(int(TW) == int(TH), "square tiles only")
+        pixels = int(Wimg) * int(Himg)
+        x = [rays_o, rays_d, positions, log_scales, quats, cand, offsets, freq, att, W1, b1, W2, b2, W3, b3,
+             torch.zeros_like(rays_o), torch.zeros(pixels, device=rays_o.device)]
+        return self.render_tiles_training_records(x, Wimg, Himg, TW, thr, 1.5, 2.0, any_tile=True, counts_only=True,
+                                                  name="render_tiles_backward_count_tilecenter")
+
+    def _emit(self, records, log_scales, quats, grad_rgb, grad_t, counts, offsets, total):
+        """The emit entry points' outputs from records: (prim_id, x6, grad_rgb, grad_sigma_raw, grad_positions,
+        grad_log_scales, grad_quats) with record k of pixel p at offsets[p] + k for k < counts[p]
+        (np_tile_kernels.cu:1568-1836: out_grad_rgb = T alpha grad_out_rgb[p], out_grad_sigma_raw = the adjoint of
+        softplus(o3))."""
+        _, _, ids, x6, raw, _, _, rec_off = records
+        pixels = rec_off.numel() - 1
+        _chk(counts.dtype == torch.int32 and counts.numel() == pixels, "counts must have size B")
+        _chk(offsets.dtype == torch.int32 and offsets.numel() == pixels, "offsets must have size B")
+        dev = ids.device
+        total = int(total)
+        with torch.cuda.device(dev):
+            d4, gp, gs, gq = ops.records_reverse(ids, rec_off, x6, raw, log_scales, quats, grad_rgb.contiguous(),
+                                                 grad_t.contiguous())
+            pix = torch.repeat_interleave(torch.arange(pixels, device=dev), rec_off.diff(), output_size=ids.numel())
+            k = torch.arange(ids.numel(), device=dev) - rec_off[pix]
+            dest = offsets.long()[pix] + k
+            keep = (k < counts.long()[pix]) & (dest < total)
+            dest = dest[keep]
+            weight = (raw[:, 4] * raw[:, 5])[:, None]
+            sigma_adjoint = d4[:, 3:4] / torch.sigmoid(raw[:, 7:8]).clamp_min(1e-38)
+            out_ids = torch.zeros(total, dtype=torch.int32, device=dev)
+            out_x6 = torch.zeros(total, 6, device=dev)
+            out_rgb = torch.zeros(total, 3, device=dev)
+            out_sigma = torch.zeros(total, 1, device=dev)
+            out_ids[dest] = ids[keep]
+            out_x6[dest] = x6[keep]
+            out_rgb[dest] = (weight * grad_rgb[pix])[keep]
+            out_sigma[dest] = sigma_adjoint[keep]
+        return [out_ids, out_x6, out_rgb, out_sigma, gp, gs, gq]
+
+    def render_tiles_backward_emit_tilecenter(self, rays_o, rays_d, positions, log_scales, quats, cand, offsets, freq,
+                                              att, W1, b1, W2, b2, W3, b3, grad_rgb, grad_t, counts, record_offsets,
+                                              total_records, Wimg, Himg, TW, TH, thr):
+        """(prim_id, x6, grad_rgb, grad_sigma_raw, grad_positions, grad_log_scales) of the tile-centre order
+        (np_tile_kernels.cu:6443-6535)."""
+        _chk(int(TW) == int(TH), "square tiles only")
+        x = [rays_o, rays_d, positions, log_scales, quats, cand, offsets, freq, att, W1, b1, W2, b2, W3, b3,
+             grad_rgb.contiguous(), grad_t.contiguous()]
+        records = self.render_tiles_training_records(x, Wimg, Himg, TW, thr, 1.5, 2.0, any_tile=True,
+                                                     name="render_tiles_backward_emit_tilecenter")
+        return self._emit(records, log_scales, quats, x[15], x[16], counts, record_offsets, total_records)[:6]
+
+    def render_tiles_backward_emit_per_pixel(self, rays_o, rays_d, positions, log_scales, quats, cand, offsets, freq, att,
+                                             W1, b1, W2, b2, W3, b3, grad_rgb, grad_t, counts, record_offsets,
+                                             total_records, Wimg, Himg, TW, TH, thr):
+        """(prim_id, x6, grad_rgb, grad_sigma_raw, grad_positions, grad_log_scales, grad_quats) of the per-pixel order
+        (np_tile_kernels.cu:6344-6400)."""
+        base = (rays_o, rays_d, positions, log_scales, quats, cand, offsets, freq, att, W1, b1, W2, b2, W3, b3)
+        _chk(grad_rgb.is_cuda and grad_rgb.dtype == torch.float32 and tuple(grad_rgb.shape) == (int(Wimg) * int(Himg), 3))
+        _chk(grad_t.is_cuda and grad_t.dtype == torch.float32 and grad_t.numel() == int(Wimg) * int(Himg),
+             "grad_T_end must have size B")
+        records = self.render_tiles_per_pixel_records(base, Wimg, Himg, TW, TH, thr, 1.5, 2.0)
+        return self._emit(records, log_scales, quats, grad_rgb, grad_t, counts, record_offsets, total_records)
 
     def render_tiles_backward_featattr_tilecenter(self, rays_o, rays_d, positions, log_scales, quats, cand, offsets,
                                                   freq, att, W1, b1, W2, b2, W3, b3, feat_attr, grad_out_feat, beta,
@@ -563,13 +654,14 @@ class TileExt:
         _chk(int(TW) == int(TH), "square tiles only")
         _chk(feat_attr.is_cuda and feat_attr.dtype == torch.float32 and feat_attr.is_contiguous())
         _chk(feat_attr.dim() in (2, 3) and feat_attr.shape[0] == positions.shape[0])
-        _chk(feat_attr.dim() == 2 or feat_attr.shape[1] in (4, 5), "feat_attr must be [N,C] or [N,S,C] with slots in {4,5}")
+        _chk(feat_attr.dim() == 2 or feat_attr.shape[1] in (4, 5), "3D feat_attr expects slots in {4,5}")
         pixels = int(Wimg) * int(Himg)
         _chk(grad_out_feat.is_cuda and grad_out_feat.dtype == torch.float32
              and tuple(grad_out_feat.shape) == (pixels, feat_attr.shape[-1]), "grad_out_feat must be [B, C]")
         placeholders = [torch.zeros_like(rays_o), torch.zeros(pixels, device=rays_o.device)]
         x = [rays_o, rays_d, positions, log_scales, quats, cand, offsets, freq, att, W1, b1, W2, b2, W3, b3, *placeholders]
-        records = self.render_tiles_training_records(x, Wimg, Himg, TW, thr, float(beta), float(temp))
+        records = self.render_tiles_training_records(x, Wimg, Himg, TW, thr, float(beta), float(temp), any_tile=True,
+                                                     name="render_tiles_backward_featattr_tilecenter")
         return self.feature_gradients_from_records(records, feat_attr, grad_out_feat.contiguous())
 
     def render_tiles_backward_featattr_per_pixel(self, rays_o, rays_d, positions, log_scales, quats, cand, offsets,
@@ -579,7 +671,7 @@ class TileExt:
         wrapper :6629-6720): the same sums over every pixel's hits in its own depth order."""
         _chk(feat_attr.is_cuda and feat_attr.dtype == torch.float32 and feat_attr.is_contiguous())
         _chk(feat_attr.dim() in (2, 3) and feat_attr.shape[0] == positions.shape[0])
-        _chk(feat_attr.dim() == 2 or feat_attr.shape[1] in (4, 5), "feat_attr must be [N,C] or [N,S,C] with slots in {4,5}")
+        _chk(feat_attr.dim() == 2 or feat_attr.shape[1] in (4, 5), "3D feat_attr expects slots in {4,5}")
         _chk(grad_out_feat.is_cuda and grad_out_feat.dtype == torch.float32
              and tuple(grad_out_feat.shape) == (int(Wimg) * int(Himg), feat_attr.shape[-1]), "grad_out_feat must be [B, C]")
         base = (rays_o, rays_d, positions, log_scales, quats, cand, offsets, freq, att, W1, b1, W2, b2, W3, b3)

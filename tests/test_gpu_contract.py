@@ -32,6 +32,8 @@ def _renderer_inputs(n, device):
         "W2": torch.zeros((n, hidden, hidden), device=device), "b2": torch.zeros((n, hidden), device=device),
         "W3": torch.zeros((n, 4, hidden), device=device), "b3": torch.zeros((n, 4), device=device),
         "feat_attr": torch.zeros((n, 4, 2), device=device),
+        "grad_rgb": torch.ones((1, 3), device=device), "grad_t": torch.zeros(1, device=device),
+        "grad_feat": torch.ones((1, 2), device=device),
     }
 
 
@@ -44,6 +46,12 @@ DIMS = (1, 1, 1, 1, 1.0e-3)
 PLAIN = {"render_tiles_forward", "render_tiles_autograd", "render_tiles_autograd_tilecenter",
          "render_tiles_autograd_tilecenter_presorted", "render_tiles_forward_tilecenter",
          "render_tiles_forward_tilecenter_with_t"}
+BACKWARD_COUNT = {"render_tiles_backward_count_per_pixel", "render_tiles_backward_count_tilecenter"}
+PER_PIXEL_BACKWARD = ["render_tiles_backward_count_per_pixel", "render_tiles_backward_emit_per_pixel",
+                      "render_tiles_backward_featattr_per_pixel"]
+TILECENTER_BACKWARD = ["render_tiles_backward_count_tilecenter", "render_tiles_backward_emit_tilecenter",
+                       "render_tiles_backward_featattr_tilecenter", "render_tiles_backward_tilecenter_full",
+                       "render_tiles_backward_tilecenter_full_with_feat"]
 ALL_FORWARD = sorted(PLAIN | {"render_tiles_forward_per_pixel_with_feat", "render_tiles_forward_tilecenter_with_feat",
                               "render_tiles_forward_tilecenter_stats"})
 
@@ -54,6 +62,20 @@ def _invoke(ext, name, d):
         return getattr(ext, name)(*base, *DIMS)
     if name in ("render_tiles_forward_per_pixel_with_feat", "render_tiles_forward_tilecenter_with_feat"):
         return getattr(ext, name)(*base, d["feat_attr"], 1.0, 1.0, *DIMS)
+    if name in BACKWARD_COUNT:
+        return (getattr(ext, name)(*base, *DIMS),)
+    if name in ("render_tiles_backward_featattr_per_pixel", "render_tiles_backward_featattr_tilecenter"):
+        return (getattr(ext, name)(*base, d["feat_attr"], d["grad_feat"], 1.0, 1.0, *DIMS),)
+    if name in ("render_tiles_backward_emit_per_pixel", "render_tiles_backward_emit_tilecenter"):
+        n = d["positions"].shape[0]
+        counts = torch.full((1,), n, device=d["positions"].device, dtype=torch.int32)
+        record_offsets = torch.zeros(1, device=d["positions"].device, dtype=torch.int32)
+        return getattr(ext, name)(*base, d["grad_rgb"], d["grad_t"], counts, record_offsets, n, *DIMS)
+    if name == "render_tiles_backward_tilecenter_full":
+        return ext.render_tiles_backward_tilecenter_full(*base, d["grad_rgb"], d["grad_t"], *DIMS)
+    if name == "render_tiles_backward_tilecenter_full_with_feat":
+        return ext.render_tiles_backward_tilecenter_full_with_feat(*base, d["feat_attr"], d["grad_rgb"], d["grad_t"],
+                                                                   d["grad_feat"], 1.0, 1.0, *DIMS)
     if name == "render_tiles_forward_tilecenter_stats":
         n = d["positions"].shape[0]
         dev = d["positions"].device
@@ -238,9 +260,60 @@ def test_inputs_are_not_mutated(tile_ext, device):
         assert torch.equal(v, before[k]), k
 
 
+@pytest.mark.parametrize("name", PER_PIXEL_BACKWARD + TILECENTER_BACKWARD)
+def test_backward_entry_points_follow_the_forward_contracts(tile_ext, device, name):
+    """tests/test_cuda_renderer.py:250-371 for the backward entry points: capacity refusals (256 hits per pixel /
+    1,536 candidates per tile), 386 candidates with 256 hits accepted in per-pixel order, invalid ids rejected
+    before anything runs, finite outputs on a valid stack."""
+    per_pixel = name in PER_PIXEL_BACKWARD
+    error = "per-pixel intersection capacity 256 exceeded" if per_pixel else "tile candidate capacity 1536 exceeded"
+    with pytest.raises(RuntimeError, match=error):
+        _invoke(tile_ext, name, _renderer_inputs((256 if per_pixel else 1536) + 1, device))
+    for invalid in (-1, 2):
+        d = _renderer_inputs(2, device)
+        d["candidates"][0] = invalid
+        with pytest.raises(RuntimeError, match="candidate primitive IDs must be in"):
+            _invoke(tile_ext, name, d)
+    torch.cuda.synchronize()
+    d = _renderer_inputs(386 if per_pixel else 300, device)
+    if per_pixel:
+        d["positions"][256:, 0] = 100.0
+    outputs = _invoke(tile_ext, name, d)
+    assert all(torch.isfinite(o).all() for o in outputs)
+    if "featattr" in name:
+        d = _renderer_inputs(1, device)
+        d["feat_attr"] = torch.zeros((1, 8, 2), device=device)
+        with pytest.raises(RuntimeError, match=r"slots in \{4,5\}"):
+            _invoke(tile_ext, name, d)
+
+
+def test_emit_entry_points_return_the_adjoints_of_the_activated_outputs(tile_ext, device):
+    """np_tile_kernels.cu:1568-1836: out_grad_rgb = T alpha grad_out_rgb[pixel]; out_grad_sigma_raw = the adjoint of
+    softplus(o3).  On a stack of identical zero-weight primitives along one ray (R = G = B = 1/2, sigma_raw = ln 2)
+    both have closed forms: alpha = 1 - 2^-decay with decay = 1, T_k = 2^-k, and with grad_out_rgb = 1, grad_t = 0
+    the colour adjoint of record k is T_k alpha and d loss / d sigma_raw_k = -(1 - alpha) * sum_{j>k} T_j alpha 3/2
+    + T_k (1 - alpha) 3/2."""
+    n = 6
+    d = _renderer_inputs(n, device)
+    for name in ("render_tiles_backward_emit_per_pixel", "render_tiles_backward_emit_tilecenter"):
+        out = _invoke(tile_ext, name, d)
+        ids, x6, g_rgb, g_sigma = out[:4]
+        assert len(out) == (7 if "per_pixel" in name else 6)
+        assert ids.cpu().tolist() == list(range(n)) and tuple(x6.shape) == (n, 6)
+        alpha = 0.5
+        trans = torch.tensor([0.5 ** k for k in range(n)], dtype=torch.float64)
+        torch.testing.assert_close(g_rgb.cpu().double(), (trans * alpha)[:, None].expand(n, 3), atol=1e-6, rtol=1e-5)
+        colour = 1.5                                        # sum over channels of grad_out_rgb * (R, G, B)
+        later = torch.stack([(trans[k + 1:] * alpha * colour).sum() for k in range(n)])
+        # d/d sigma_k: alpha_k' = (1 - alpha) decay; the hit's own term T_k colour alpha_k', and every later term
+        # scaled by (1 - alpha_k) loses (1 - alpha) decay / (1 - alpha_k) of itself
+        want = (1 - alpha) * trans * colour - later
+        torch.testing.assert_close(g_sigma.cpu().double().flatten(), want, atol=1e-6, rtol=1e-5)
+
+
 def test_backward_entry_points_that_are_not_built_say_so(tile_ext):
     with pytest.raises(NotImplementedError, match="fused backward entry points"):
-        tile_ext.render_tiles_backward_tilecenter_full_with_feat()
+        tile_ext.render_tiles_backward_tilecenter_traversal()
     assert callable(tile_ext.render_tiles_backward_tilecenter_full) and callable(tile_ext.primitive_records_reverse)
     with pytest.raises(AttributeError):
         tile_ext.no_such_entry_point
