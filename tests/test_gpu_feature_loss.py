@@ -49,15 +49,17 @@ def _resize(dense, width, height, wf, hf):
     return F.interpolate(image, size=(hf, wf), mode="bilinear", align_corners=False).squeeze(0).permute(1, 2, 0)
 
 
-@pytest.mark.parametrize("slots", [1, 4, 5])
-@pytest.mark.parametrize("size", [(9, 7, 7, 5), (8, 8, 8, 8), (33, 19, 23, 11), (9, 7, 1, 1), (15, 1, 8, 1), (1, 13, 1, 7)])
-@pytest.mark.parametrize("half_target", [False, True])
+_SIZES = [(9, 7, 7, 5), (8, 8, 8, 8), (33, 19, 23, 11), (9, 7, 1, 1), (15, 1, 8, 1), (1, 13, 1, 7)]
+# f32 targets for every slot count and size; fp16 targets with four slots on the sizes whose width is 9 or 33
+_CASES = ([(slots, size, False) for slots in (1, 4, 5) for size in _SIZES]
+          + [(4, size, True) for size in _SIZES if size[0] in (9, 33)])
+
+
+@pytest.mark.parametrize("slots,size,half_target", _CASES)
 def test_streamed_l1_and_attribute_gradients_match_the_dense_definition(device, oracle_mod, slots, size, half_target):
     from mlp_splatting_amd import primitive_gemm as gemm
     from mlp_splatting_amd.primitive_csr import group_records
     from mlp_splatting_amd.record_feature_loss import feature_weight_gradients, streaming_feature_l1
-    if half_target and (slots != 4 or size[0] not in (9, 33)):
-        pytest.skip("the fp16 target is covered on two sizes")
     width, height, wf, hf = size
     fr, ext, base, records = _frame_records(device, oracle_mod, width, height)
     n, channels = fr.scene.n, 150
