@@ -10,7 +10,7 @@ expression, and the extension object is ``tile_ext.TileExt`` on ``libmlpsp_hip.s
 
 ``forward`` renders without a graph under ``torch.no_grad()``; in grad mode with parameters that require
 grad it goes through ``_TileRenderAutogradFn`` (RGB) or, with a feature target, through the record-based
-training step of ``csr_training``.  The dense feature-image backward of the reference is not provided.
+training step of ``record_training``.  The dense feature-image backward of the reference is not provided.
 """
 from __future__ import annotations
 
@@ -709,7 +709,7 @@ class NeuralPrimitiveSceneTileCUDA(nn.Module):
         use_tilecenter = self._resolve_tile_order_mode() == "tilecenter"
         if not return_feature or self.feat_attr is None or not use_tilecenter or ts != 8:
             raise ValueError("CSR feature training requires tilecenter8 and direct feature attributes")
-        from .csr_training import render_training_csr
+        from .record_training import Frame, feature_training_step
         with torch.no_grad():
             unit_dirs = F.normalize(ray_d, dim=-1).contiguous()
             culled_prim_indices, tile_offsets = self._tile_lists(
@@ -719,9 +719,10 @@ class NeuralPrimitiveSceneTileCUDA(nn.Module):
                 F.normalize(self.quats, dim=-1).contiguous(), culled_prim_indices, tile_offsets.to(torch.int32), freq, att,
                 self.W1.contiguous(), self.b1.contiguous(), self.W2.contiguous(), self.b2.contiguous(),
                 self.W3.contiguous(), self.b3.contiguous()]
-        return render_training_csr(base, self.feat_attr.contiguous(), feature_target, int(W), int(H),
-                                   float(score_threshold), float(self.feature_gating_beta),
-                                   float(self.feature_gating_temp), self._background(bg_color, ray_o))
+        frame = Frame(int(W), int(H), float(score_threshold), float(self.feature_gating_beta),
+                      float(self.feature_gating_temp))
+        return feature_training_step(base, self.feat_attr.contiguous(), feature_target, frame,
+                                     self._background(bg_color, ray_o))
 
     def _forward_differentiable(self, ray_o, ray_d, score_threshold, bg_color, view_matrix, proj_matrix,
                                 culled_prim_indices, tile_offsets, return_feature, device):

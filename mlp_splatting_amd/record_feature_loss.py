@@ -29,23 +29,31 @@ def _launch_order(pixels, csr, starts):
     return torch.argsort(pixels[csr.record_indices[starts]].to(torch.int64))
 
 
+def _loss_geometry(attributes, target, record_tensors, width, height):
+    """(target height, target width, channels, slots) after the argument checks of the streamed loss
+    (the conditions and texts of scannet/record_feature_loss.py:66-82, which callers and tests match)."""
+    on_one_gpu = all(t.is_cuda and t.device == attributes.device for t in (*record_tensors, attributes, target))
+    slots = attributes.shape[1] if attributes.ndim == 3 else 1
+    shape_ok = target.ndim == 3 and min(target.shape) > 0
+    for ok, text in (
+            (shape_ok, "feature target must have nonempty HWC dimensions"),
+            (attributes.dtype == torch.float32 and attributes.is_contiguous(),
+             "feature master attributes must be contiguous FP32"),
+            (target.dtype in (torch.float16, torch.float32), "feature target must be FP16 or FP32"),
+            (on_one_gpu, "feature tensors and records must share a CUDA device"),
+            (slots in (1, 4, 5) and shape_ok and attributes.shape[-1] == target.shape[-1],
+             "feature shape does not match the 1/4/5-slot renderer"),
+            (shape_ok and target.shape[0] <= height and target.shape[1] <= width,
+             "streamed feature loss supports downsampling only")):
+        if not ok:
+            raise ValueError(text)
+    return target.shape[0], target.shape[1], target.shape[2], slots
+
+
 def streaming_feature_l1(records, attributes, target, width, height, *, debug=False):
     """(loss, signs int8 [hf, wf, C], prediction or None) -- scannet/record_feature_loss.py:66-89."""
-    _, _, ids, x6, raw, masks, gates, offsets = records
-    if target.ndim != 3 or min(target.shape) <= 0:
-        raise ValueError("feature target must have nonempty HWC dimensions")
-    if attributes.dtype != torch.float32 or not attributes.is_contiguous():
-        raise ValueError("feature master attributes must be contiguous FP32")
-    if target.dtype not in (torch.float16, torch.float32):
-        raise ValueError("feature target must be FP16 or FP32")
-    if any(not t.is_cuda or t.device != attributes.device for t in (ids, offsets, raw, gates, attributes, target)):
-        raise ValueError("feature tensors and records must share a CUDA device")
-    hf, wf, channels = target.shape
-    slots = 1 if attributes.ndim == 2 else attributes.shape[1]
-    if slots not in (1, 4, 5) or attributes.shape[-1] != channels:
-        raise ValueError("feature shape does not match the 1/4/5-slot renderer")
-    if hf > height or wf > width:
-        raise ValueError("streamed feature loss supports downsampling only")
+    ids, raw, gates, offsets = records[2], records[4], records[6], records[7]
+    hf, wf, channels, slots = _loss_geometry(attributes, target, (ids, offsets, raw, gates), width, height)
     target = target.contiguous()
     device = target.device
     signs = torch.empty(target.shape, device=device, dtype=torch.int8)

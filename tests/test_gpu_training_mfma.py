@@ -36,45 +36,64 @@ def _delta(ext, before):
     return {k: after[k] - before[k] for k in STATS}
 
 
-def _case(device, n=13, width=9, height=7, *, constant=False, mosaic=False):
-    """A slab of n primitives in front of a near-orthographic camera; every tile lists every primitive."""
-    g = torch.Generator(device="cpu").manual_seed(42157 + n + width + height)
-    rnd = lambda *shape: torch.randn(*shape, generator=g).to(device)
-    uni = lambda lo, hi, *shape: (torch.rand(*shape, generator=g) * (hi - lo) + lo).to(device)
-    d = {}
-    yy, xx = torch.meshgrid(torch.linspace(-.45, .45, height, device=device),
-                            torch.linspace(-.55, .55, width, device=device), indexing="ij")
-    d["rays_o"] = torch.stack((xx.flatten(), yy.flatten(), torch.zeros(width * height, device=device)), -1).contiguous()
-    d["rays_d"] = torch.tensor([.025, -.015, 1.], device=device).repeat(width * height, 1)
+# Mosaic variant: four cameras, one per image quadrant (the quadrant boundary is NOT a tile edge, so origins and
+# directions both change inside a tile).
+_QUADRANT_ORIGIN_SHIFT = ((0., 0., 0.), (.19, 0., -.12), (0., -.17, .09), (-.14, .13, -.08))
+_QUADRANT_DIRECTION = ((0., 0., 1.), (-.09, .04, 1.), (.07, .08, 1.), (.12, -.05, 1.))
+
+
+def _slab_rays(device, width, height, mosaic):
+    """Near-orthographic rays: origins on a width x height grid in the z = 0 plane, one shared direction (or one
+    direction and origin shift per quadrant)."""
+    xs = torch.linspace(-.55, .55, width, device=device)
+    ys = torch.linspace(-.45, .45, height, device=device)
+    origins = torch.zeros(height, width, 3, device=device)
+    origins[..., 0] = xs[None, :]
+    origins[..., 1] = ys[:, None]
+    origins = origins.reshape(-1, 3)
+    directions = torch.tensor([.025, -.015, 1.], device=device).expand(width * height, 3)
     if mosaic:
-        # origins AND directions differ inside a tile, with a view boundary that is not a tile edge
-        ix = torch.arange(width * height, device=device)
-        quadrant = (ix % width >= width // 2).long() + 2 * (ix // width >= height // 2).long()
-        cameras = torch.tensor([[0., 0., 0.], [.19, 0., -.12], [0., -.17, .09], [-.14, .13, -.08]], device=device)
-        directions = torch.tensor([[0., 0., 1.], [-.09, .04, 1.], [.07, .08, 1.], [.12, -.05, 1.]], device=device)
-        d["rays_o"] = (d["rays_o"] + cameras[quadrant]).contiguous()
-        d["rays_d"] = directions[quadrant]
-    d["rays_d"] = F.normalize(d["rays_d"], dim=-1).contiguous()
-    d["positions"] = torch.cat((uni(-.2, .2, n, 2), torch.linspace(.75, 1.75, n, device=device)[:, None]), 1).contiguous()
-    d["log_scales"] = uni(-.45, .15, n, 3)
-    d["quats"] = F.normalize(rnd(n, 4), dim=-1).contiguous() if n else torch.zeros(0, 4, device=device)
-    d["freq"] = 2. ** torch.arange(6, device=device, dtype=torch.float32)
-    d["attenuation"] = torch.exp(-.5 * d["freq"].square() * .0001)
+        col = torch.arange(width, device=device)[None, :].expand(height, width)
+        row = torch.arange(height, device=device)[:, None].expand(height, width)
+        quadrant = ((col >= width // 2).long() + 2 * (row >= height // 2).long()).reshape(-1)
+        origins = origins + torch.tensor(_QUADRANT_ORIGIN_SHIFT, device=device)[quadrant]
+        directions = torch.tensor(_QUADRANT_DIRECTION, device=device)[quadrant]
+    return origins.contiguous(), F.normalize(directions, dim=-1).contiguous()
+
+
+def _case(device, n=13, width=9, height=7, *, constant=False, mosaic=False):
+    """n primitives stacked in depth (z from 0.75 to 1.75) in front of the rays of _slab_rays; every tile lists every
+    primitive in id order.  Small random MLPs with the density logit pinned at -2, far from early termination, so
+    that the reduced-precision forward must reproduce the f32 record topology; ``constant``: zero weights and only
+    output biases, for which every record field is exact in any operand precision."""
+    rng = torch.Generator(device="cpu").manual_seed(42157 + n + width + height)
+
+    def normal(*shape, scale=1.):
+        return (torch.randn(*shape, generator=rng) * scale).to(device)
+
+    def uniform(lo, hi, *shape):
+        return (lo + (hi - lo) * torch.rand(*shape, generator=rng)).to(device)
+
+    pixels = width * height
+    tiles = ((width + 7) // 8) * ((height + 7) // 8)
+    d = dict(zip(("rays_o", "rays_d"), _slab_rays(device, width, height, mosaic)))
+    depth = torch.linspace(.75, 1.75, n, device=device)
+    d["positions"] = torch.cat((uniform(-.2, .2, n, 2), depth[:, None]), dim=1).contiguous()
+    d["log_scales"] = uniform(-.45, .15, n, 3)
+    d["quats"] = F.normalize(normal(n, 4), dim=-1).contiguous() if n else torch.zeros(0, 4, device=device)
+    d["freq"] = torch.tensor([1., 2., 4., 8., 16., 32.], device=device)
+    d["attenuation"] = torch.exp(-.5e-4 * d["freq"] ** 2)
     for name, shape in zip(WEIGHTS, SHAPES):
-        d[name] = rnd(n, *shape) * .035
-    d["b3"][:, 3] = -2.          # far from termination: the record topology must match the f32 path
+        d[name] = torch.zeros(n, *shape, device=device) if constant else normal(n, *shape, scale=.035)
     if constant:
-        for name in WEIGHTS:
-            d[name].zero_()
         d["b3"][:, 0] = torch.linspace(-1., 1., n, device=device)
         d["b3"][:, 1] = -.25
         d["b3"][:, 2] = .5
-        d["b3"][:, 3] = -2.
-    tiles = ((width + 7) // 8) * ((height + 7) // 8)
+    d["b3"][:, 3] = -2.
     d["candidates"] = torch.arange(n, device=device, dtype=torch.int32).repeat(tiles)
-    d["offsets"] = torch.arange(tiles + 1, device=device, dtype=torch.int32) * n
-    d["grad_rgb"] = rnd(width * height, 3) * .1
-    d["grad_t"] = rnd(width * height) * .1
+    d["offsets"] = (n * torch.arange(tiles + 1, device=device)).to(torch.int32)
+    d["grad_rgb"] = normal(pixels, 3, scale=.1)
+    d["grad_t"] = normal(pixels, scale=.1)
     return d
 
 
@@ -91,37 +110,54 @@ def _scalar(ext, d, width, height, threshold=.001):
     return ext.render_tiles_training_records(_args(d), width, height, 8, threshold, 1.5, 2.)
 
 
+RECORD_FIELDS = (       # name, trailing shape, dtype, leading dimension ("B" pixels, "R" records, "B+1")
+    ("rgb", (3,), torch.float32, "B"), ("alpha", (1,), torch.float32, "B"), ("ids", (), torch.int32, "R"),
+    ("x6", (6,), torch.float32, "R"), ("raw", (8,), torch.float32, "R"), ("masks", (2,), torch.int32, "R"),
+    ("gates", (4,), torch.float32, "R"), ("offsets", (), torch.int64, "B+1"))
+
+
 def _schema(records, d, width, height):
-    assert len(records) == 8
-    rgb, alpha, ids, x6, raw, masks, gates, offsets = records
-    count = len(ids)
-    shapes = ((width * height, 3), (width * height, 1), (count,), (count, 6), (count, 8), (count, 2), (count, 4),
-              (width * height + 1,))
-    dtypes = (torch.float32, torch.float32, torch.int32, torch.float32, torch.float32, torch.int32, torch.float32,
-              torch.int64)
-    for value, shape, dtype in zip(records, shapes, dtypes):
-        assert tuple(value.shape) == shape and value.dtype == dtype and value.device == d["positions"].device
-        assert value.is_contiguous() and bool(torch.isfinite(value).all())
-    assert int(offsets[0]) == 0 and int(offsets[-1]) == count and bool((offsets.diff() >= 0).all())
-    assert bool(((ids >= 0) & (ids < len(d["positions"]))).all())
-    if count:
-        assert bool(((raw[:, 4:6] >= 0) & (raw[:, 4:6] <= 1)).all())
-        torch.testing.assert_close(gates.sum(-1), torch.ones(count, device=ids.device), atol=2e-6, rtol=2e-6)
-        pixels = torch.repeat_interleave(torch.arange(width * height, device=ids.device), offsets.diff(), output_size=count)
-        assert torch.equal(x6[:, :3], d["rays_d"][pixels])
+    """Layout and internal consistency of a record list: field shapes and types, a monotone offsets vector that
+    covers the records, valid ids, T and alpha inside [0, 1], gates that sum to one, and x6[:, :3] equal to the
+    ray direction of the record's pixel."""
+    assert len(records) == len(RECORD_FIELDS)
+    pixels = width * height
+    fields = {name: value for (name, *_), value in zip(RECORD_FIELDS, records)}
+    total = fields["ids"].numel()
+    leading = {"B": pixels, "R": total, "B+1": pixels + 1}
+    for (name, trailing, dtype, lead), value in zip(RECORD_FIELDS, records):
+        assert value.dtype == dtype and tuple(value.shape) == (leading[lead], *trailing), name
+        assert value.device == d["positions"].device and value.is_contiguous(), name
+        assert bool(torch.isfinite(value).all()), name
+    per_pixel = fields["offsets"].diff()
+    assert int(fields["offsets"][0]) == 0 and int(fields["offsets"][-1]) == total and int(per_pixel.min()) >= 0
+    if total == 0:
+        return
+    ids, raw = fields["ids"], fields["raw"]
+    assert int(ids.min()) >= 0 and int(ids.max()) < d["positions"].shape[0]
+    transmittance_and_alpha = raw[:, 4:6]
+    assert float(transmittance_and_alpha.min()) >= 0. and float(transmittance_and_alpha.max()) <= 1.
+    torch.testing.assert_close(fields["gates"].sum(-1), torch.ones_like(raw[:, 0]), atol=2e-6, rtol=2e-6)
+    pixel_of_record = torch.repeat_interleave(torch.arange(pixels, device=ids.device), per_pixel, output_size=total)
+    assert torch.equal(fields["x6"][:, :3], d["rays_d"][pixel_of_record])
 
 
 def _parity(actual, expected, precision, exact=False):
-    for index in (2, 3, 6, 7):                        # ids, x6, gates, offsets: the f32 expression path
-        assert torch.equal(actual[index], expected[index]), index
-    assert torch.equal(actual[4][:, 6], expected[4][:, 6])        # decay
+    """Reduced-precision records against the f32 records: topology (ids, offsets) and everything computed by the
+    f32 geometry expressions (x6, gates, decay) bit for bit; image, alpha and the raw MLP outputs within the operand
+    precision's tolerance -- or every field bit for bit when the MLP is constant."""
+    names = [name for name, *_ in RECORD_FIELDS]
+    got, want = dict(zip(names, actual)), dict(zip(names, expected))
+    for name in ("ids", "offsets", "x6", "gates"):
+        assert torch.equal(got[name], want[name]), name
+    assert torch.equal(got["raw"][:, 6], want["raw"][:, 6]), "decay"
     if exact:
-        for index, (a, b) in enumerate(zip(actual, expected)):
-            assert torch.equal(a, b), index
-    else:
-        tol = .003 if precision == "bfloat16" else .0005
-        for index in (0, 1, 4):
-            torch.testing.assert_close(actual[index], expected[index], atol=tol, rtol=tol)
+        for name in names:
+            assert torch.equal(got[name], want[name]), name
+        return
+    tol = {"bfloat16": 3e-3, "float16": 5e-4}[precision]
+    for name in ("rgb", "alpha", "raw"):
+        torch.testing.assert_close(got[name], want[name], atol=tol, rtol=tol)
 
 
 @pytest.mark.parametrize("precision", PRECISIONS)
@@ -439,26 +475,27 @@ def test_saved_records_feed_reverse_and_grouped_vjp(ext, device, precision, cons
 
 @pytest.mark.parametrize("backend,precision", [("wmma_fp16", "float16"), ("wmma_bf16", "bfloat16")])
 def test_environment_selects_the_record_forward(ext, device, monkeypatch, backend, precision):
-    from mlp_splatting_amd import csr_training
+    from mlp_splatting_amd import record_training
+    frame = record_training.Frame(9, 7, .001, 1.5, 2.)
     d = _case(device, 7, 9, 7, mosaic=True)
     monkeypatch.setenv("MLPSP_CSR_FORWARD_BACKEND", backend)
     before = _stats(ext)
-    chosen = csr_training._record_forward(ext, _args(d), 9, 7, .001, 1.5, 2.)
+    chosen = record_training.records_forward(ext, _args(d)[:15], frame)
     assert _delta(ext, before)["calls"] == 1
     direct = _render(ext, d, 9, 7, precision)
     for a, b in zip(chosen, direct):
         assert torch.equal(a, b)
     monkeypatch.setenv("MLPSP_CSR_FORWARD_BACKEND", "tensor_cores")
     with pytest.raises(ValueError, match="MLPSP_CSR_FORWARD_BACKEND"):
-        csr_training._record_forward(ext, _args(d), 9, 7, .001, 1.5, 2.)
+        record_training.records_forward(ext, _args(d)[:15], frame)
 
 
 @pytest.mark.parametrize("precision", PRECISIONS)
 def test_training_step_on_matrix_core_records(ext, device, monkeypatch, precision):
-    """CSRTrainingFunction on the reduced-precision records: the 512-channel attribute gradient equals autograd
+    """The record-based training step on the reduced-precision records: the 512-channel attribute gradient equals autograd
     through a dense framebuffer of those very records, and no MLP-input adjoint exists."""
     from mlp_splatting_amd import cumodel
-    from mlp_splatting_amd.csr_training import CSRTrainingFunction
+    from mlp_splatting_amd.record_training import Frame, feature_training_step
     from test_gpu_feature_loss import _framebuffer64, _resize
     monkeypatch.setattr(cumodel, "_tile_ext", ext, raising=False)
     monkeypatch.setattr(cumodel, "_tile_ext_key", cumodel._tile_ext_build_config(8)[0])
@@ -478,7 +515,7 @@ def test_training_step_on_matrix_core_records(ext, device, monkeypatch, precisio
         noise = (torch.rand(prediction.shape, generator=g) * .05 + .01) * (torch.rand(prediction.shape, generator=g) < .5).double().mul(2).sub(1)
         target = (prediction + noise).float().to(device).contiguous()
     before = _stats(ext)
-    rgb, feature_loss = CSRTrainingFunction.apply(*base, attributes, target, (9, 7, .001, 1.5, 2.), None)
+    rgb, feature_loss = feature_training_step(base, attributes, target, Frame(9, 7, .001, 1.5, 2.), None)
     assert _delta(ext, before)["calls"] == 1
     (rgb.square().mean() + feature_loss).backward()
     for index in (0, 1, 7, 8):
