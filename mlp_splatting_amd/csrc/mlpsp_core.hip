@@ -37,13 +37,14 @@ __global__ __launch_bounds__(256) void prepare_primitives_kernel(const float* __
   dst[1] = make_float4(r.my, r.mz, r.qw, r.qx);
   dst[2] = make_float4(r.qy, r.qz, r.lgx, r.lgy);
   dst[3] = make_float4(r.lgz, r.s2x, r.s2y, r.s2z);
-  // R(q)^T of the unit quaternion, row by row
+  // second half: centre, then R(q)^T of the unit quaternion row by row, row k scaled by exp(-log_s[k])
   const float w = r.qw, x = r.qx, y = r.qy, z = r.qz;
-  dst[4] = make_float4(1.f - 2.f * (y * y + z * z), 2.f * (x * y + w * z), 2.f * (x * z - w * y),
-                       2.f * (x * y - w * z));
-  dst[5] = make_float4(1.f - 2.f * (x * x + z * z), 2.f * (y * z + w * x), 2.f * (x * z + w * y),
-                       2.f * (y * z - w * x));
-  dst[6] = make_float4(1.f - 2.f * (x * x + y * y), 0.f, 0.f, 0.f);
+  const float ix = det_exp(-r.lgx), iy = det_exp(-r.lgy), iz = det_exp(-r.lgz);
+  dst[4] = make_float4(r.cx, r.cy, r.cz, ix * (1.f - 2.f * (y * y + z * z)));
+  dst[5] = make_float4(ix * (2.f * (x * y + w * z)), ix * (2.f * (x * z - w * y)), iy * (2.f * (x * y - w * z)),
+                       iy * (1.f - 2.f * (x * x + z * z)));
+  dst[6] = make_float4(iy * (2.f * (y * z + w * x)), iz * (2.f * (x * z + w * y)), iz * (2.f * (y * z - w * x)),
+                       iz * (1.f - 2.f * (x * x + y * y)));
   dst[7] = make_float4(0.f, 0.f, 0.f, 0.f);
 }
 

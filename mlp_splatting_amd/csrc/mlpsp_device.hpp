@@ -127,17 +127,20 @@ __device__ __forceinline__ Vec3 quat_rotate_conj(float qw, float qx, float qy, f
 }
 
 // One primitive's geometry as the kernels consume it: 128 bytes, written by the prepare kernel.
-// m = exp(-2 log_s) is the diagonal of the precision matrix, s2 = exp(2 log_s) the squared semi-axes (used
-// only by the conservative tile culling of the sort kernel).  rt is the world -> local rotation as a matrix,
-// rt[k] = row k of R(q)^T; only the reduced-precision render path uses it (three dot products per vector
-// instead of the quaternion form, which the exact paths must keep to reproduce the reference's roundings).
+// First 64 bytes, for the exactly rounded paths and the sort: m = exp(-2 log_s) is the diagonal of the precision
+// matrix, s2 = exp(2 log_s) the squared semi-axes (used only by the conservative tile culling of the sort kernel).
+// Second 64 bytes (one cache line, one scalar load), for the reduced-precision render path only: the centre again
+// and rs[k] = exp(-log_s[k]) * row k of R(q)^T, the world -> local rotation with the inverse scales folded in, so
+// that |rs (x - c)|^2 is the Mahalanobis distance (three dot products per vector instead of the quaternion form,
+// which the exact paths must keep to reproduce the reference's roundings).
 struct __attribute__((aligned(128))) PrimRecord {
   float cx, cy, cz, mx;
   float my, mz, qw, qx;
   float qy, qz, lgx, lgy;
   float lgz, s2x, s2y, s2z;
-  float rt[3][3];
-  float pad[7];
+  float fcx, fcy, fcz;
+  float rs[3][3];
+  float pad[4];
 };
 static_assert(sizeof(PrimRecord) == 128, "record size is part of the C ABI");
 

@@ -10,7 +10,8 @@
 // per K-step) provided the next layer's weight columns are stored in that register order.  Weights are
 // therefore repacked (pack kernel in mlpsp_render_mfma.hip) into A-fragment order with the k-permutation
 // folded in, and the chain layer1 -> ReLU -> layer2 -> ReLU -> layer3 needs no LDS, no barrier and no
-// cross-lane traffic.  Staging a primitive's weights is 9 coalesced 1 KiB loads straight into VGPRs.
+// cross-lane traffic.  Staging a primitive's weights is 7 coalesced 1 KiB loads straight into VGPRs (plus three
+// small ones for the layer-2 bias words and the four output rows).
 //
 // Layer-1 k-slots: lane group g = l/32 owns frequencies 3g..3g+2 of every input component, so both groups
 // evaluate 18 (sin, cos) pairs per pixel block and each pair lands in one 32-bit operand word.  sin/cos use
@@ -31,12 +32,15 @@ typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 
-// packed per-primitive block (bytes)
-constexpr int kOffW1 = 0;       // 5 K-steps x 64 lanes x 16 B
+// packed per-primitive block (bytes).  The biases of the two hidden layers travel as operands: b = hi + lo with
+// hi = round(b) and lo = round(b - hi) in the operand type (17 significant bits for bf16, 22 for fp16), multiplied
+// by a constant (1, 1) operand word and summed in f32 by the MFMA itself.  Layer 1 has spare k-slots for that
+// (72 of 80 used); layer 2 gets a third K-step whose A operand is one word per lane.  No bias is loaded as a
+// 16-register C operand any more: such loads cost the vector-memory pipe as much as the weights themselves.
+constexpr int kOffW1 = 0;       // 5 K-steps x 64 lanes x 16 B; word 18 of lane group 0 = (b1 hi, b1 lo)
 constexpr int kOffW2 = 5120;    // 2 K-steps x 64 lanes x 16 B
-constexpr int kOffW3 = 7168;    // 2 K-steps x 2 lane groups x 4 rows x 16 B
-constexpr int kOffB1 = 7424;    // 2 lane groups x 16 f32 in D-register order
-constexpr int kOffB2 = 7552;
+constexpr int kOffB2 = 7168;    // 64 lanes x 4 B: lanes 0..31 (b2 hi, b2 lo) of their row, lanes 32..63 zero
+constexpr int kOffW3 = 7424;    // 2 K-steps x 2 lane groups x 4 rows x 16 B
 constexpr int kOffB3 = 7680;    // 4 f32
 constexpr int kOffFlag = 7696;  // int32: 1 if any rounded weight or bias is non-finite
 constexpr int kPackStride = MLPSP_MFMA_PACK_BYTES;
@@ -53,6 +57,7 @@ template <> struct Ops<__bf16> {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
   }
   static __device__ __forceinline__ float round_trip(float a) { return (float)(__bf16)a; }
+  static constexpr unsigned kOneWord = 0x3f803f80u;   // (1, 1)
   static constexpr float kMax = 3.38953139e38f;
   // bf16 has the exponent range of f32: a hidden pre-activation is out of range only if it is (within one
   // rounding step of) +-inf.  Rounded to +inf it survives the ReLU and turns the next layer's sums into
@@ -70,6 +75,7 @@ template <> struct Ops<_Float16> {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
   }
   static __device__ __forceinline__ float round_trip(float a) { return (float)(_Float16)a; }
+  static constexpr unsigned kOneWord = 0x3c003c00u;   // (1, 1)
   static constexpr float kMax = 65504.0f;
   static constexpr bool kCheckHidden = true;   // a finite f32 pre-activation above 65504 must be reported
 };
@@ -162,12 +168,41 @@ __device__ __forceinline__ unsigned relu_mask_bits(unsigned rectified, int shift
   return __builtin_bit_cast(unsigned, nz) << shift;
 }
 
+// (hi, lo) operand word of a bias: hi + lo reproduces b to twice the operand type's precision.
+template <typename T>
+__device__ __forceinline__ unsigned bias_word(float b) {
+  const float hi = Ops<T>::round_trip(b);
+  return Ops<T>::pack2(hi, b - hi);
+}
+
+// Both halves of the wavefront exchange a value in one instruction: returns {[x lanes 0..31 | x lanes 0..31],
+// [x lanes 32..63 | x lanes 32..63]}, i.e. for column block b the value of pixel 32 b + l % 32 in every lane.
+struct HalfPair {
+  float blk0, blk1;
+};
+// (The two results are copied into scalars before they are reinterpreted: __builtin_bit_cast applied to an
+// element expression of the returned vector reads element 0 whatever the index.)
+__device__ __forceinline__ HalfPair both_halves(float x) {
+  const unsigned u = __float_as_uint(x);
+  const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  const unsigned lo = r[0], hi = r[1];
+  return HalfPair{__uint_as_float(lo), __uint_as_float(hi)};
+}
+// lanes 0..31 of a in the lower half, lanes 0..31 of b in the upper half
+__device__ __forceinline__ float lower_halves(float a, float b) {
+  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(a), __float_as_uint(b), false, false);
+  const unsigned lo = r[0];
+  return __uint_as_float(lo);
+}
+
 // The MLP of primitive block `blk` for the pixels of `mask` (ballot of the lanes that hit).  dx, dy, dz: this
 // lane's own hit offset (inputs 3..5; lanes that did not hit pass anything finite).  o[k] = output k of THIS
 // lane's pixel, output bias included.
 // CHECK: report pre-activations outside the operand type's range.  MASKS: also return the pixel's two
 // 32-bit ReLU masks (bit u = hidden unit u active) in mk.  Returns true if a stored weight was flagged
 // non-finite when packed or (CHECK) a pre-activation of a hit pixel is out of range.
+// Vector-memory instructions per call: 7 (W1, W2) + 1 (b2 words) + 2 (W3); the output bias and the flag are
+// wave-uniform scalar loads.
 template <typename T, bool CHECK, bool MASKS>
 __device__ __forceinline__ bool mlp_wave_mfma16(const unsigned char* __restrict__ blk, unsigned long long mask, int l,
                                                 float dx, float dy, float dz, const float kf[3], const DirWords& dir,
@@ -180,6 +215,7 @@ __device__ __forceinline__ bool mlp_wave_mfma16(const unsigned char* __restrict_
   for (int s = 0; s < 5; ++s) a1[s] = *reinterpret_cast<const u32x4*>(blk + kOffW1 + s * 1024 + l * 16);
 #pragma unroll
   for (int s = 0; s < 2; ++s) a2[s] = *reinterpret_cast<const u32x4*>(blk + kOffW2 + s * 1024 + l * 16);
+  const unsigned a2b_word = *reinterpret_cast<const unsigned*>(blk + kOffB2 + l * 4);
 #pragma unroll
   for (int s = 0; s < 2; ++s) {
     // every lane loads one of the four stored rows (no divergent branch, no wait in the middle of the
@@ -191,38 +227,28 @@ __device__ __forceinline__ bool mlp_wave_mfma16(const unsigned char* __restrict_
   const f32x4 b3v = *reinterpret_cast<const f32x4*>(blk + kOffB3);
   const int wflag = *reinterpret_cast<const int32_t*>(blk + kOffFlag);
   bad |= (wflag != 0);
+  // the constant operand word that multiplies the (hi, lo) bias words: k-slots of lane group 0 only
+  const unsigned one_word = g ? 0u : Ops<T>::kOneWord;
 
-  // ---- inputs of the column partner
-  const float pdx = __shfl_xor(dx, 32), pdy = __shfl_xor(dy, 32), pdz = __shfl_xor(dz, 32);
+  // ---- inputs 3..5 of both column blocks
+  const HalfPair hx = both_halves(dx), hy = both_halves(dy), hz = both_halves(dz);
   float o_blk[2][4];
   unsigned m_blk[2][2] = {{0u, 0u}, {0u, 0u}};
+  const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
   for (int b = 0; b < 2; ++b) {
     const unsigned half_mask = (unsigned)(mask >> (32 * b));
     if (half_mask != 0u) {   // wave-uniform: skip a 32-pixel block nobody hits
-      const bool own = (b == g);
-      const float xin[3] = {own ? dx : pdx, own ? dy : pdy, own ? dz : pdz};
+      const float xin[3] = {b ? hx.blk1 : hx.blk0, b ? hy.blk1 : hy.blk0, b ? hz.blk1 : hz.blk0};
       const bool col_active = (half_mask >> (l & 31)) & 1u;
-      // biases are the C operand of each layer's first MFMA; an MFMA overwrites its C registers,
-      // so each column block fetches its own copy (L1-resident) instead of copying 32 registers
-      f32x16 d1, d2;
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const f32x4 v1 = *reinterpret_cast<const f32x4*>(blk + kOffB1 + g * 64 + q * 16);
-        const f32x4 v2 = *reinterpret_cast<const f32x4*>(blk + kOffB2 + g * 64 + q * 16);
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          d1[4 * q + e] = v1[e];
-          d2[4 * q + e] = v2[e];
-        }
-      }
-      // layer 1: 18 (sin, cos) words per lane, 5 K-steps; words 0..8 come from LDS.  (The lane index is
-      // made opaque so that the loads stay here and are not hoisted out of the primitive loop into
+      // layer 1: 18 (sin, cos) words per lane + the bias word, 5 K-steps; words 0..8 come from LDS.  (The lane
+      // index is made opaque so that the loads stay here and are not hoisted out of the primitive loop into
       // registers.)
       int ll = l;
       asm volatile("" : "+v"(ll));
       const u32x4 dq0 = dir.q[b][0][ll], dq1 = dir.q[b][1][ll];
       const unsigned d8 = dir.w8[b][ll];
+      f32x16 d1 = zero16;
 #pragma unroll
       for (int s = 0; s < 5; ++s) {
         u32x4 bw;
@@ -238,6 +264,8 @@ __device__ __forceinline__ bool mlp_wave_mfma16(const unsigned char* __restrict_
           } else if (t < 18) {
             const float rev = xin[t / 3 - 3] * kf[t % 3];
             bw[d] = Ops<T>::pack2(__builtin_amdgcn_sinf(rev), __builtin_amdgcn_cosf(rev));
+          } else if (t == 18) {
+            bw[d] = one_word;
           } else {
             bw[d] = 0u;
           }
@@ -245,7 +273,12 @@ __device__ __forceinline__ bool mlp_wave_mfma16(const unsigned char* __restrict_
         d1 = Ops<T>::mfma(a1[s], bw, d1);
       }
       if constexpr (CHECK) bad |= col_active && out_of_range_in<T>(d1);
-      // layer 2: the D registers, rectified and rounded, are the next B operand
+      // layer 2: the bias K-step first (its operands are ready), then the D registers of layer 1, rectified and
+      // rounded, as the B operand
+      // (the zero words of the two operands are made here, not kept in registers across the primitive loop)
+      unsigned z0, z1, z2;
+      asm volatile("v_mov_b32 %0, 0\n v_mov_b32 %1, 0\n v_mov_b32 %2, 0" : "=v"(z0), "=v"(z1), "=v"(z2));
+      f32x16 d2 = Ops<T>::mfma(u32x4{a2b_word, z0, z1, z2}, u32x4{one_word, z0, z1, z2}, zero16);
 #pragma unroll
       for (int s = 0; s < 2; ++s) {
         u32x4 bw;
@@ -258,7 +291,7 @@ __device__ __forceinline__ bool mlp_wave_mfma16(const unsigned char* __restrict_
       }
       if constexpr (CHECK) bad |= col_active && out_of_range_in<T>(d2);
       // layer 3: rows 0..3 of a 32-row product; row k lands in register k of lane group 0
-      f32x16 d3 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+      f32x16 d3 = zero16;
 #pragma unroll
       for (int s = 0; s < 2; ++s) {
         u32x4 bw;
@@ -276,12 +309,9 @@ __device__ __forceinline__ bool mlp_wave_mfma16(const unsigned char* __restrict_
       for (int k = 0; k < 4; ++k) o_blk[b][k] = 0.f;
     }
   }
-  // pixel l < 32 reads block 0 from its own lane; pixel l >= 32 reads block 1 from lane l-32
+  // pixel l < 32 reads block 0 from its own lane; pixel l >= 32 reads block 1 from lane l - 32
 #pragma unroll
-  for (int k = 0; k < 4; ++k) {
-    const float from_partner = __shfl_xor(o_blk[1][k], 32);
-    o[k] = (g ? from_partner : o_blk[0][k]) + b3v[k];
-  }
+  for (int k = 0; k < 4; ++k) o[k] = lower_halves(o_blk[0][k], o_blk[1][k]) + b3v[k];
   if constexpr (MASKS) {
     // lane group g holds the units 8g..8g+7 and 16+8g..16+8g+7 of its column: shift into place, merge the
     // two groups, and take the block this lane's pixel belongs to (block g)

@@ -42,6 +42,8 @@ __global__ __launch_bounds__(64) void pack_mfma_weights_kernel(const float* __re
     bad |= !(__builtin_fabsf(Ops<T>::round_trip(a)) <= Ops<T>::kMax) || !(__builtin_fabsf(Ops<T>::round_trip(b)) <= Ops<T>::kMax);
     return Ops<T>::pack2(a, b);
   };
+  const float bias1 = b1[(size_t)p * 32 + hidden_unit_of_row(m)], bias2 = b2[(size_t)p * 32 + hidden_unit_of_row(m)];
+  bad |= !(__builtin_fabsf(Ops<T>::round_trip(bias1)) <= Ops<T>::kMax) || !(__builtin_fabsf(Ops<T>::round_trip(bias2)) <= Ops<T>::kMax);
   for (int s = 0; s < 5; ++s) {
     u32x4 v;
     for (int d = 0; d < 4; ++d) {
@@ -53,6 +55,7 @@ __global__ __launch_bounds__(64) void pack_mfma_weights_kernel(const float* __re
         wc = w1[36 + j];
       }
       v[d] = pk(ws, wc);
+      if (t == 18 && g == 0) v[d] = bias_word<T>(bias1);     // multiplied by the constant (1, 1) operand word
     }
     *reinterpret_cast<u32x4*>(blk + kOffW1 + s * 1024 + l * 16) = v;
   }
@@ -61,19 +64,13 @@ __global__ __launch_bounds__(64) void pack_mfma_weights_kernel(const float* __re
     for (int d = 0; d < 4; ++d) v[d] = pk(w2[hidden_unit(8 * s + 2 * d, g)], w2[hidden_unit(8 * s + 2 * d + 1, g)]);
     *reinterpret_cast<u32x4*>(blk + kOffW2 + s * 1024 + l * 16) = v;
   }
+  reinterpret_cast<unsigned*>(blk + kOffB2)[l] = (g == 0) ? bias_word<T>(bias2) : 0u;
   if (l < 16) {
     const int row = l & 3, gg = (l >> 2) & 1, s = l >> 3;
     const float* w3 = W3 + (size_t)p * 4 * 32 + row * 32;
     u32x4 v;
     for (int d = 0; d < 4; ++d) v[d] = pk(w3[hidden_unit(8 * s + 2 * d, gg)], w3[hidden_unit(8 * s + 2 * d + 1, gg)]);
     *reinterpret_cast<u32x4*>(blk + kOffW3 + ((s * 2 + gg) * 4 + row) * 16) = v;
-  }
-  if (l < 32) {
-    const int r = l & 15, gg = l >> 4;
-    const float v1 = b1[(size_t)p * 32 + hidden_unit(r, gg)], v2 = b2[(size_t)p * 32 + hidden_unit(r, gg)];
-    bad |= !(__builtin_fabsf(v1) <= 3.4028235e38f) || !(__builtin_fabsf(v2) <= 3.4028235e38f);
-    reinterpret_cast<float*>(blk + kOffB1)[gg * 16 + r] = v1;
-    reinterpret_cast<float*>(blk + kOffB2)[gg * 16 + r] = v2;
   }
   if (l < 4) {
     const float v3 = b3[(size_t)p * 4 + l];
@@ -82,6 +79,7 @@ __global__ __launch_bounds__(64) void pack_mfma_weights_kernel(const float* __re
   }
   const unsigned long long any = __ballot(bad);
   if (l == 0) *reinterpret_cast<int32_t*>(blk + kOffFlag) = any ? 1 : 0;
+  if (l < (kPackStride - kOffFlag - 4) / 4) reinterpret_cast<unsigned*>(blk + kOffFlag + 4)[l] = 0u;   // unused tail
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -109,12 +107,14 @@ __device__ __forceinline__ float fast_blend_step(PixelAcc& a, float o0, float o1
   a.trans = a.trans * (1.f - alpha);
   return w;
 }
-// tetrahedral gates (np_tile_kernels.cu:97-124) with the native exp/rcp
-__device__ __forceinline__ void fast_tetra_gates(float qlx, float qly, float qlz, float lgx, float lgy, float lgz,
+// tetrahedral gates (np_tile_kernels.cu:97-124) with the native exp/rcp.  qs = local hit offset divided by the
+// scales (what hit_fast() returns); u = q / (beta s + 1e-6) = qs s / (beta s + 1e-6).
+__device__ __forceinline__ void fast_tetra_gates(float qsx, float qsy, float qsz, float lgx, float lgy, float lgz,
                                                  float beta, float temp, float g[4]) {
-  const float ux = fminf(1.f, fmaxf(-1.f, qlx * __builtin_amdgcn_rcpf(beta * fast_exp(lgx) + 1e-6f)));
-  const float uy = fminf(1.f, fmaxf(-1.f, qly * __builtin_amdgcn_rcpf(beta * fast_exp(lgy) + 1e-6f)));
-  const float uz = fminf(1.f, fmaxf(-1.f, qlz * __builtin_amdgcn_rcpf(beta * fast_exp(lgz) + 1e-6f)));
+  const float sx = fast_exp(lgx), sy = fast_exp(lgy), sz = fast_exp(lgz);
+  const float ux = fminf(1.f, fmaxf(-1.f, (qsx * sx) * __builtin_amdgcn_rcpf(beta * sx + 1e-6f)));
+  const float uy = fminf(1.f, fmaxf(-1.f, (qsy * sy) * __builtin_amdgcn_rcpf(beta * sy + 1e-6f)));
+  const float uz = fminf(1.f, fmaxf(-1.f, (qsz * sz) * __builtin_amdgcn_rcpf(beta * sz + 1e-6f)));
   const float l0 = temp * ((ux + uy) + uz), l1 = temp * ((ux - uy) - uz);
   const float l2 = temp * ((-ux + uy) - uz), l3 = temp * ((-ux - uy) + uz);
   const float lm = fmaxf(fmaxf(l0, l1), fmaxf(l2, l3));
@@ -126,29 +126,59 @@ __device__ __forceinline__ void fast_tetra_gates(float qlx, float qly, float qlz
   g[3] = e3 * inv;
 }
 
+// The second half of a PrimRecord (mlpsp_device.hpp): one 64-byte line per primitive.
+struct FastRec {
+  float cx, cy, cz;
+  float r[9];
+  float pad[4];
+};
+static_assert(sizeof(FastRec) == 64, "second half of PrimRecord");
+
+// The 12 floats of a FastRec as scalar registers, requested with explicit scalar loads so that the request sits
+// exactly where it is written (the compiler otherwise sinks such a load to its first use, which is the next
+// loop iteration: every candidate would then wait for its own record).  fast_arrived() must run before the
+// registers are read; waits the compiler inserts for its own scalar and LDS operations in between only wait
+// longer for having one more operation outstanding.
+typedef float f32x8 __attribute__((ext_vector_type(8)));
+struct FastRegs {
+  f32x4 a;   // cx cy cz r0
+  f32x8 b;   // r1 .. r8
+};
+__device__ __forceinline__ void fast_request(const unsigned char* __restrict__ line, FastRegs& q) {
+  asm volatile("s_load_dwordx4 %0, %2, 0x0\n\ts_load_dwordx8 %1, %2, 0x10" : "=&s"(q.a), "=&s"(q.b) : "s"(line));
+}
+__device__ __forceinline__ FastRec fast_arrived(FastRegs& q) {
+  asm volatile("s_waitcnt lgkmcnt(0)" : "+s"(q.a), "+s"(q.b));
+  FastRec F;
+  F.cx = q.a[0]; F.cy = q.a[1]; F.cz = q.a[2];
+  F.r[0] = q.a[3];
+#pragma unroll
+  for (int k = 0; k < 8; ++k) F.r[1 + k] = q.b[k];
+  return F;
+}
+
 // Ray against rotated ellipsoid for this path: same quantities as hit_rot() (np_tile_kernels.cu:659-711), with
-// the world -> local rotation applied as a matrix, the local hit offset taken as vl - t dl (equal to the
-// rotated world offset up to rounding), and the native reciprocal and exp2.  About a third of the
-// instructions of the exactly-rounded form; the differences are of the order of f32 rounding (about 1e-5
-// relative in decay, through the cancellation in vl - t dl).
+// the world -> local rotation and the inverse scales applied as one matrix, the local hit offset taken as
+// vl - t dl (equal to the rotated world offset up to rounding), and the native reciprocal and exp2.  About a
+// third of the instructions of the exactly-rounded form; the differences are of the order of f32 rounding
+// (about 1e-5 relative in decay, through the cancellation in vl - t dl).  h.ql* are in units of the scales.
 //
 // The hit decision itself is a hard threshold, and a primitive that barely hits still contributes up to a
 // few 1e-3 to a pixel, so a decision that differs from the exact path's would show as isolated pixel
 // errors well above the rounding noise of this path.  unsure = the fast quantities are too close to one of
 // the three decision boundaries (decay within 0.4 % of thr, t or denom near zero) to be trusted; the
 // caller then takes the decision -- only the decision -- from hit_rot().
-__device__ __forceinline__ bool hit_rot_fast(float rox, float roy, float roz, float rdx, float rdy, float rdz,
-                                             const PrimRecord& P, float thr, HitInfo& h, bool& unsure) {
-  const float vx = P.cx - rox, vy = P.cy - roy, vz = P.cz - roz;
-  const float dlx = fmaf(P.rt[0][0], rdx, fmaf(P.rt[0][1], rdy, P.rt[0][2] * rdz));
-  const float dly = fmaf(P.rt[1][0], rdx, fmaf(P.rt[1][1], rdy, P.rt[1][2] * rdz));
-  const float dlz = fmaf(P.rt[2][0], rdx, fmaf(P.rt[2][1], rdy, P.rt[2][2] * rdz));
-  const float vlx = fmaf(P.rt[0][0], vx, fmaf(P.rt[0][1], vy, P.rt[0][2] * vz));
-  const float vly = fmaf(P.rt[1][0], vx, fmaf(P.rt[1][1], vy, P.rt[1][2] * vz));
-  const float vlz = fmaf(P.rt[2][0], vx, fmaf(P.rt[2][1], vy, P.rt[2][2] * vz));
-  const float ax = P.mx * dlx, ay = P.my * dly, az = P.mz * dlz;
-  const float denom = fmaf(ax, dlx, fmaf(ay, dly, az * dlz));
-  const float numer = fmaf(ax, vlx, fmaf(ay, vly, az * vlz));
+__device__ __forceinline__ bool hit_fast(float rox, float roy, float roz, float rdx, float rdy, float rdz,
+                                         const FastRec& F, float thr, HitInfo& h, bool& unsure) {
+  const float vx = F.cx - rox, vy = F.cy - roy, vz = F.cz - roz;
+  const float dlx = fmaf(F.r[0], rdx, fmaf(F.r[1], rdy, F.r[2] * rdz));
+  const float dly = fmaf(F.r[3], rdx, fmaf(F.r[4], rdy, F.r[5] * rdz));
+  const float dlz = fmaf(F.r[6], rdx, fmaf(F.r[7], rdy, F.r[8] * rdz));
+  const float vlx = fmaf(F.r[0], vx, fmaf(F.r[1], vy, F.r[2] * vz));
+  const float vly = fmaf(F.r[3], vx, fmaf(F.r[4], vy, F.r[5] * vz));
+  const float vlz = fmaf(F.r[6], vx, fmaf(F.r[7], vy, F.r[8] * vz));
+  const float denom = fmaf(dlx, dlx, fmaf(dly, dly, dlz * dlz));
+  const float numer = fmaf(dlx, vlx, fmaf(dly, vly, dlz * vlz));
   const float t = numer * __builtin_amdgcn_rcpf(denom);
   h.t = t;
   h.dx = fmaf(-t, rdx, vx);
@@ -157,8 +187,8 @@ __device__ __forceinline__ bool hit_rot_fast(float rox, float roy, float roz, fl
   h.qlx = fmaf(-t, dlx, vlx);
   h.qly = fmaf(-t, dly, vly);
   h.qlz = fmaf(-t, dlz, vlz);
-  const float r2 = fmaf(P.mx * h.qlx, h.qlx, fmaf(P.my * h.qly, h.qly, (P.mz * h.qlz) * h.qlz));
-  h.decay = __builtin_amdgcn_exp2f(fmaxf(r2, 0.f) * -0.72134752f);
+  const float r2 = fmaf(h.qlx, h.qlx, fmaf(h.qly, h.qly, h.qlz * h.qlz));
+  h.decay = __builtin_amdgcn_exp2f(r2 * -0.72134752f);
   unsure = (__builtin_fabsf(h.decay - thr) <= 4e-3f * thr) || !(__builtin_fabsf(t) >= 1e-4f) || !(denom >= 1e-18f);
   return !(denom <= 1e-20f) && !(t <= 0.f) && (h.decay > thr);
 }
@@ -206,56 +236,86 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 4))) void
   const int start = offsets[tile], end = offsets[tile + 1];
   PixelAcc acc = {0.f, 0.f, 0.f, 1.f, 0.f, 0.f};
   HitEmitter em = hit_emitter_begin(hp, 0, start, tile);
+  bool live = valid;
+  const unsigned char* __restrict__ fast_half = reinterpret_cast<const unsigned char*>(prims) + 64;
 
-  for (int i = start; i < end; ++i) {
-    const int p = __builtin_amdgcn_readfirstlane(order[i]);
-    if (p < 0 || p >= N) continue;
-    const PrimRecord P = prims[p];
-    HitInfo h;
-    const bool live = valid && (acc.trans >= kTransmittanceFloor);
-    bool unsure;
-    bool hit = hit_rot_fast(rox, roy, roz, rdx, rdy, rdz, P, thr, h, unsure) && live;
-    if (__ballot(unsure && live) != 0ull) {   // rare (about one wavefront step in twenty)
-      if (unsure && live) {
-        HitInfo exact;
-        hit = hit_rot(rox, roy, roz, rdx, rdy, rdz, P, thr, exact);
+  // The tile's list is read 64 entries at a time, one coalesced load; a lane's entry is broadcast with
+  // v_readlane when its turn comes.  Culled (negative) entries never get a turn.  The geometry line of the next
+  // entry is requested before the current one is tested, so that neither the id nor the record is waited for
+  // in the common case of a run of candidates that hit nothing.
+  bool finished = false;
+  for (int base = start; base < end && !finished; base += 64) {
+    const int id_lane = (base + l < end) ? order[base + l] : -1;
+    unsigned long long todo = __ballot(id_lane >= 0 && id_lane < N);
+    if (todo == 0ull) continue;
+    int p = __builtin_amdgcn_readlane(id_lane, (int)__builtin_ctzll(todo));
+    todo &= todo - 1ull;
+    FastRegs q;
+    fast_request(fast_half + (size_t)p * sizeof(PrimRecord), q);
+    for (;;) {
+      const FastRec R = fast_arrived(q);
+      const bool more = todo != 0ull;
+      int p_next = p;
+      if (more) {
+        p_next = __builtin_amdgcn_readlane(id_lane, (int)__builtin_ctzll(todo));
+        todo &= todo - 1ull;
       }
-    }
-    const unsigned long long mask = __ballot(hit);
-    ++n_proc;
-    if (mask != 0ull) {
-      ++n_proc_hit;
-      n_hits += __popcll(mask);
-      const unsigned char* __restrict__ blk = packed + (size_t)p * kPackStride;
-      bad |= hit && !(__builtin_fabsf((h.dx + h.dy) + h.dz) <= 3.4028235e38f);
-      float o[4];
-      bad |= mlp_wave_mfma16<T, Ops<T>::kCheckHidden, false>(blk, mask, l, h.dx, h.dy, h.dz, kf, s_dir, o, nullptr);
-      float w = 0.f;
-      if (hit) {
-        bad |= !(__builtin_fabsf(o[0]) <= 3.4028235e38f) || !(__builtin_fabsf(o[1]) <= 3.4028235e38f) ||
-               !(__builtin_fabsf(o[2]) <= 3.4028235e38f) || !(__builtin_fabsf(o[3]) <= 3.4028235e38f);
-        w = fast_blend_step(acc, o[0], o[1], o[2], o[3], h.decay);
-      }
-      if constexpr (SP > 0) {
-        float gt[4] = {0.f, 0.f, 0.f, 0.f};
-        if (hit && slots > 1) fast_tetra_gates(h.qlx, h.qly, h.qlz, P.lgx, P.lgy, P.lgz, beta, temp, gt);
-        const int rs = hit_emitter_next(hp, em, l);
-        if (rs >= 0) {
-          unsigned* __restrict__ coef = reinterpret_cast<unsigned*>(hp.records + (size_t)rs * hp.record_bytes);
-          if constexpr (SP == 4) {
-            const unsigned c01 = (slots > 1) ? Ops<_Float16>::pack2(w * gt[0], w * gt[1]) : Ops<_Float16>::pack2(w, 0.f);
-            const unsigned c23 = Ops<_Float16>::pack2(w * gt[2], w * gt[3]);
-            *reinterpret_cast<uint2*>(coef + l * 2) = make_uint2(c01, c23);
-          } else {
-            const u32x4 c = {Ops<_Float16>::pack2(w, w * gt[0]), Ops<_Float16>::pack2(w * gt[1], w * gt[2]),
-                             Ops<_Float16>::pack2(w * gt[3], 0.f), 0u};
-            *reinterpret_cast<u32x4*>(coef + l * 4) = c;
-          }
-          if (l == 0) hp.hit_ids[rs] = p;
+      fast_request(fast_half + (size_t)p_next * sizeof(PrimRecord), q);   // (the last entry asks for its own line again)
+
+      HitInfo h;
+      bool unsure;
+      bool hit = hit_fast(rox, roy, roz, rdx, rdy, rdz, R, thr, h, unsure) && live;
+      if (__ballot(unsure && live) != 0ull) {   // rare (about one wavefront step in twenty)
+        if (unsure && live) {
+          const PrimRecord P = prims[p];
+          HitInfo exact;
+          hit = hit_rot(rox, roy, roz, rdx, rdy, rdz, P, thr, exact);
         }
       }
+      const unsigned long long mask = __ballot(hit);
+      ++n_proc;
+      if (mask != 0ull) {
+        ++n_proc_hit;
+        n_hits += __popcll(mask);
+        const unsigned char* __restrict__ blk = packed + (size_t)p * kPackStride;
+        bad |= hit && !(__builtin_fabsf((h.dx + h.dy) + h.dz) <= 3.4028235e38f);
+        float o[4];
+        bad |= mlp_wave_mfma16<T, Ops<T>::kCheckHidden, false>(blk, mask, l, h.dx, h.dy, h.dz, kf, s_dir, o, nullptr);
+        float w = 0.f;
+        if (hit) {
+          bad |= !(max3_abs(o[0], o[1], o[2]) <= 3.4028235e38f) || !(__builtin_fabsf(o[3]) <= 3.4028235e38f);
+          w = fast_blend_step(acc, o[0], o[1], o[2], o[3], h.decay);
+        }
+        if constexpr (SP > 0) {
+          float gt[4] = {0.f, 0.f, 0.f, 0.f};
+          if (slots > 1) {
+            const PrimRecord& P = prims[p];
+            if (hit) fast_tetra_gates(h.qlx, h.qly, h.qlz, P.lgx, P.lgy, P.lgz, beta, temp, gt);
+          }
+          const int rs = hit_emitter_next(hp, em, l);
+          if (rs >= 0) {
+            unsigned* __restrict__ coef = reinterpret_cast<unsigned*>(hp.records + (size_t)rs * hp.record_bytes);
+            if constexpr (SP == 4) {
+              const unsigned c01 = (slots > 1) ? Ops<_Float16>::pack2(w * gt[0], w * gt[1]) : Ops<_Float16>::pack2(w, 0.f);
+              const unsigned c23 = Ops<_Float16>::pack2(w * gt[2], w * gt[3]);
+              *reinterpret_cast<uint2*>(coef + l * 2) = make_uint2(c01, c23);
+            } else {
+              const u32x4 c = {Ops<_Float16>::pack2(w, w * gt[0]), Ops<_Float16>::pack2(w * gt[1], w * gt[2]),
+                               Ops<_Float16>::pack2(w * gt[3], 0.f), 0u};
+              *reinterpret_cast<u32x4*>(coef + l * 4) = c;
+            }
+            if (l == 0) hp.hit_ids[rs] = p;
+          }
+        }
+        live = valid && (acc.trans >= kTransmittanceFloor);
+        if (__ballot(live) == 0ull) {
+          finished = true;
+          break;
+        }
+      }
+      if (!more) break;
+      p = p_next;
     }
-    if (__ballot(valid && (acc.trans >= kTransmittanceFloor)) == 0ull) break;
   }
 
   if (valid) {
