@@ -263,7 +263,11 @@ __device__ __forceinline__ bool mlp_wave_mfma16(const unsigned char* __restrict_
             bw[d] = d8;
           } else if (t < 18) {
             const float rev = xin[t / 3 - 3] * kf[t % 3];
+#ifdef MLPSP_EXP_NOTRANS
+            bw[d] = Ops<T>::pack2(rev, rev + 0.25f);
+#else
             bw[d] = Ops<T>::pack2(__builtin_amdgcn_sinf(rev), __builtin_amdgcn_cosf(rev));
+#endif
           } else if (t == 18) {
             bw[d] = one_word;
           } else {
@@ -323,6 +327,107 @@ __device__ __forceinline__ bool mlp_wave_mfma16(const unsigned char* __restrict_
       mk[j] = g ? full1 : full0;
     }
   }
+  return bad;
+}
+
+// The same evaluation with the two column blocks advanced together, for a wavefront whose hit mask has pixels in
+// both halves.  A wavefront's MLP is otherwise one dependent chain (K-step after K-step of a layer, the layer's
+// sixteen registers rectified and packed, the next layer, ...), and with four wavefronts per SIMD there is often
+// nothing else to issue while an MFMA or its first reader waits.  Here every MFMA of block 0 is followed by the
+// independent MFMA of block 1, and the operand preparation of one block sits behind the MFMA of the other.
+// No ReLU masks (render only).
+template <typename T, bool CHECK>
+__device__ __forceinline__ bool mlp_pair_mfma16(const unsigned char* __restrict__ blk, unsigned long long mask, int l,
+                                                float dx, float dy, float dz, const float kf[3], const DirWords& dir,
+                                                float o[4]) {
+  const int g = l >> 5;
+  bool bad = false;
+  u32x4 a1[5], a2[2], a3[2];
+#pragma unroll
+  for (int s = 0; s < 5; ++s) a1[s] = *reinterpret_cast<const u32x4*>(blk + kOffW1 + s * 1024 + l * 16);
+#pragma unroll
+  for (int s = 0; s < 2; ++s) a2[s] = *reinterpret_cast<const u32x4*>(blk + kOffW2 + s * 1024 + l * 16);
+  const unsigned a2b_word = *reinterpret_cast<const unsigned*>(blk + kOffB2 + l * 4);
+#pragma unroll
+  for (int s = 0; s < 2; ++s) {
+    const u32x4 row = *reinterpret_cast<const u32x4*>(blk + kOffW3 + ((s * 2 + g) * 4 + (l & 3)) * 16);
+    const bool stored = (l & 31) < 4;
+    a3[s] = u32x4{stored ? row[0] : 0u, stored ? row[1] : 0u, stored ? row[2] : 0u, stored ? row[3] : 0u};
+  }
+  const f32x4 b3v = *reinterpret_cast<const f32x4*>(blk + kOffB3);
+  const int wflag = *reinterpret_cast<const int32_t*>(blk + kOffFlag);
+  bad |= (wflag != 0);
+  const unsigned one_word = g ? 0u : Ops<T>::kOneWord;
+  const HalfPair hx = both_halves(dx), hy = both_halves(dy), hz = both_halves(dz);
+  const float xin[2][3] = {{hx.blk0, hy.blk0, hz.blk0}, {hx.blk1, hy.blk1, hz.blk1}};
+  const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  int ll = l;
+  asm volatile("" : "+v"(ll));
+  f32x16 d1[2] = {zero16, zero16};
+#pragma unroll
+  for (int s = 0; s < 5; ++s) {
+#pragma unroll
+    for (int b = 0; b < 2; ++b) {
+      u32x4 bw;
+      if (s == 0) {
+        bw = dir.q[b][0][ll];
+      } else if (s == 1) {
+        bw = dir.q[b][1][ll];
+      } else {
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+          const int t = 4 * s + d;
+          if (t == 8) {
+            bw[d] = dir.w8[b][ll];
+          } else if (t < 18) {
+            const float rev = xin[b][t / 3 - 3] * kf[t % 3];
+            bw[d] = Ops<T>::pack2(__builtin_amdgcn_sinf(rev), __builtin_amdgcn_cosf(rev));
+          } else if (t == 18) {
+            bw[d] = one_word;
+          } else {
+            bw[d] = 0u;
+          }
+        }
+      }
+      d1[b] = Ops<T>::mfma(a1[s], bw, d1[b]);
+    }
+  }
+  if constexpr (CHECK) {
+    bad |= ((mask >> (l & 31)) & 1ull) && out_of_range_in<T>(d1[0]);
+    bad |= ((mask >> (32 + (l & 31))) & 1ull) && out_of_range_in<T>(d1[1]);
+  }
+  unsigned z0, z1, z2;
+  asm volatile("v_mov_b32 %0, 0\n v_mov_b32 %1, 0\n v_mov_b32 %2, 0" : "=v"(z0), "=v"(z1), "=v"(z2));
+  f32x16 d2[2];
+#pragma unroll
+  for (int b = 0; b < 2; ++b) d2[b] = Ops<T>::mfma(u32x4{a2b_word, z0, z1, z2}, u32x4{one_word, z0, z1, z2}, zero16);
+#pragma unroll
+  for (int s = 0; s < 2; ++s) {
+#pragma unroll
+    for (int b = 0; b < 2; ++b) {
+      u32x4 bw;
+#pragma unroll
+      for (int d = 0; d < 4; ++d) bw[d] = relu_packed(Ops<T>::pack2(d1[b][8 * s + 2 * d], d1[b][8 * s + 2 * d + 1]));
+      d2[b] = Ops<T>::mfma(a2[s], bw, d2[b]);
+    }
+  }
+  if constexpr (CHECK) {
+    bad |= ((mask >> (l & 31)) & 1ull) && out_of_range_in<T>(d2[0]);
+    bad |= ((mask >> (32 + (l & 31))) & 1ull) && out_of_range_in<T>(d2[1]);
+  }
+  f32x16 d3[2] = {zero16, zero16};
+#pragma unroll
+  for (int s = 0; s < 2; ++s) {
+#pragma unroll
+    for (int b = 0; b < 2; ++b) {
+      u32x4 bw;
+#pragma unroll
+      for (int d = 0; d < 4; ++d) bw[d] = relu_packed(Ops<T>::pack2(d2[b][8 * s + 2 * d], d2[b][8 * s + 2 * d + 1]));
+      d3[b] = Ops<T>::mfma(a3[s], bw, d3[b]);
+    }
+  }
+#pragma unroll
+  for (int k = 0; k < 4; ++k) o[k] = lower_halves(d3[0][k], d3[1][k]) + b3v[k];
   return bad;
 }
 
