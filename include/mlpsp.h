@@ -43,6 +43,8 @@ extern "C" {
 #define MLPSP_PIXEL_HIT_CAPACITY 256 /* per-pixel-order hit buffer (np_tile_kernels.cu:760) */
 #define MLPSP_PRIM_RECORD_BYTES 128  /* bytes per primitive of the prepared geometry buffer */
 #define MLPSP_MFMA_PACK_BYTES 7808   /* bytes per primitive of the packed matrix-core weight buffer */
+#define MLPSP_BIN_STATIC_SCRATCH_BYTES 67108864 /* scratch array of mlpsp_bin_legacy_async_noalloc (64 MiB) */
+#define MLPSP_BIN_STATIC_MAX_VIEWS 8           /* most views mlpsp_bin_legacy_async_noalloc accepts */
 
 #define MLPSP_KEY_LIST_ORDER 0 /* consume the list as given (presorted kernel, np_tile_kernels.cu:4242-4478) */
 #define MLPSP_KEY_TSTAR 1      /* Mahalanobis t* of the tile-centre ray (np_tile_kernels.cu:483-518) */
@@ -103,6 +105,22 @@ int mlpsp_bin_legacy_async(const float* positions_dev, const float* log_scales_d
 int mlpsp_bin_legacy_fill(int num_primitives, int num_views, const int32_t* tile_view_ids_dev, int width,
                           int height, int tile, const void* scratch_dev, size_t scratch_bytes,
                           const int32_t* tile_offsets_dev, int32_t* candidates_dev, mlpsp_stream_t stream);
+
+/* mlpsp_bin_legacy_async without a scratch argument and without any allocation.  No counterpart in the reference;
+ * it is for callers that cannot allocate device memory where they call the renderer: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  The scratch is a device array inside the library
+ * (mlpsp_bin_static_scratch_bytes() = MLPSP_BIN_STATIC_SCRATCH_BYTES bytes, held on every GPU the library runs on
+ * until the process ends); inputs whose mlpsp_bin_scratch_bytes() exceed it return MLPSP_E_SCRATCH, more than
+ * MLPSP_BIN_STATIC_MAX_VIEWS views MLPSP_E_ARGUMENT (the matrices travel as kernel arguments).  Same outputs,
+ * guard behaviour and launches as mlpsp_bin_legacy_async; nothing is cleared with a memset (a fill kernel where
+ * needed), so the call may be captured.  All calls on one GPU share the one array: calls that overlap on a GPU
+ * (two streams, two threads) race and must be serialised by the caller. */
+size_t mlpsp_bin_static_scratch_bytes(void);
+int mlpsp_bin_legacy_async_noalloc(const float* positions_dev, const float* log_scales_dev, int num_primitives,
+                                   const float* view_matrices_host, int num_views, const int32_t* tile_view_ids_dev,
+                                   const float* proj_host, int width, int height, int tile, float threshold,
+                                   int32_t* tile_offsets_dev, int32_t* candidates_dev, int64_t cand_capacity,
+                                   int64_t* counts_dev, mlpsp_stream_t stream);
 
 /* Ray-cone culling from the actual rays = ray_cone_candidates (scannet/camera.py:102-146), for
  * cameras that are not a centred pinhole.  Same two steps and blocking behaviour as the legacy

@@ -461,7 +461,8 @@ namespace {
 int enqueue_bin_count(const float* positions_dev, const float* log_scales_dev, int num_primitives,
                       const float* view_matrices_host, int num_views, const int32_t* tile_view_ids_dev,
                       const float* proj_host, int width, int height, int tile, float threshold, const BinGeom& g,
-                      const BinScratch& b, int64_t T, int32_t* tile_offsets_dev, hipStream_t s) {
+                      const BinScratch& b, int64_t T, int32_t* tile_offsets_dev, hipStream_t s,
+                      bool matrices_in_scratch = false) {
   const int S = g.nsx * g.nsy;
   // scalar constants in f32, in the order the reference's tensor expressions evaluate them
   const float rm = sqrtf(-2.0f * logf(threshold));
@@ -476,10 +477,12 @@ int enqueue_bin_count(const float* positions_dev, const float* log_scales_dev, i
     hipLaunchKernelGGL(bin_bounds_kernel<true>, dim3(ceil_div(num_primitives, kBinThreads), 1), dim3(kBinThreads), 0, s,
                        positions_dev, log_scales_dev, (const float*)nullptr, one, g, rm, focal, b.bounds);
   } else {
-    MLPSP_HIP_TRY(hipMemcpyAsync(b.mats, view_matrices_host, (size_t)num_views * 16 * sizeof(float),
-                                 hipMemcpyHostToDevice, s));
-    MLPSP_HIP_TRY(hipMemcpyAsync(b.mats + (size_t)num_views * 16, proj_host, 16 * sizeof(float), hipMemcpyHostToDevice,
-                                 s));
+    if (!matrices_in_scratch) {
+      MLPSP_HIP_TRY(hipMemcpyAsync(b.mats, view_matrices_host, (size_t)num_views * 16 * sizeof(float),
+                                   hipMemcpyHostToDevice, s));
+      MLPSP_HIP_TRY(hipMemcpyAsync(b.mats + (size_t)num_views * 16, proj_host, 16 * sizeof(float),
+                                   hipMemcpyHostToDevice, s));
+    }
     hipLaunchKernelGGL(bin_bounds_kernel<false>, dim3(ceil_div(num_primitives, kBinThreads), num_views),
                        dim3(kBinThreads), 0, s, positions_dev, log_scales_dev, b.mats, one, g, rm, focal, b.bounds);
   }
@@ -617,6 +620,110 @@ MLPSP_API int mlpsp_bin_legacy_fill(int num_primitives, int num_views, const int
   hipLaunchKernelGGL((bin_level2_kernel<true>), dim3(ceil_div((int)T, kBinThreads / 64)), dim3(kBinThreads), 0,
                      (hipStream_t)stream, b.bounds, g, tile_view_ids_dev, b.l1_counts, b.l1_list, b.l1_bounds, b.l1_capacity,
                      const_cast<int32_t*>(tile_offsets_dev), candidates_dev, b.l2_masks, b.l2_mask_stride);
+  MLPSP_LAUNCH_CHECK();
+  return MLPSP_OK;
+}
+
+// ---------------------------------------------------------------------------------------------
+// The asynchronous binning for callers that cannot allocate: its scratch is a file-scope device array.
+// ---------------------------------------------------------------------------------------------
+namespace mlpsp {
+constexpr size_t kStaticBinScratchBytes = MLPSP_BIN_STATIC_SCRATCH_BYTES;
+constexpr int kStaticBinMaxViews = MLPSP_BIN_STATIC_MAX_VIEWS;
+static __device__ __align__(256) unsigned char scratch[kStaticBinScratchBytes];
+
+struct ManyMats {
+  float v[kStaticBinMaxViews][16];
+  float p[16];
+};
+// view and projection matrices travel as kernel arguments and are stored where the binning kernels read them
+__global__ __launch_bounds__(64) void store_matrices_kernel(ManyMats m, int num_views, float* __restrict__ dst) {
+  const int t = threadIdx.x;
+  if (t < 16) {
+    for (int k = 0; k < num_views; ++k) dst[k * 16 + t] = m.v[k][t];
+    dst[num_views * 16 + t] = m.p[t];
+  }
+}
+__global__ __launch_bounds__(256) void fill_i32_kernel(int32_t* __restrict__ dst, long long n, int32_t value) {
+  for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long long)gridDim.x * blockDim.x)
+    dst[i] = value;
+}
+}  // namespace mlpsp
+
+namespace {
+// address of the array on each device, taken once per device with that device current
+constexpr int kMaxDevices = 64;
+void* g_static_scratch[kMaxDevices];
+bool g_static_scratch_known[kMaxDevices];
+
+int static_scratch_of_current_device(void** out) {
+  int dev = -1;
+  MLPSP_HIP_TRY(hipGetDevice(&dev));
+  if (dev < 0 || dev >= kMaxDevices) return MLPSP_E_ARGUMENT;
+  // (two threads racing here both obtain the same address; the flag is written last)
+  if (!g_static_scratch_known[dev]) {
+    void* ptr = nullptr;
+    MLPSP_HIP_TRY(hipGetSymbolAddress(&ptr, HIP_SYMBOL(mlpsp::scratch)));
+    if (!ptr) return MLPSP_E_RUNTIME;
+    g_static_scratch[dev] = ptr;
+    __atomic_store_n(&g_static_scratch_known[dev], true, __ATOMIC_RELEASE);
+  }
+  *out = g_static_scratch[dev];
+  return MLPSP_OK;
+}
+}  // namespace
+
+MLPSP_API size_t mlpsp_bin_static_scratch_bytes(void) { return kStaticBinScratchBytes; }
+
+MLPSP_API int mlpsp_bin_legacy_async_noalloc(const float* positions_dev, const float* log_scales_dev,
+                                             int num_primitives, const float* view_matrices_host, int num_views,
+                                             const int32_t* tile_view_ids_dev, const float* proj_host, int width,
+                                             int height, int tile, float threshold, int32_t* tile_offsets_dev,
+                                             int32_t* candidates_dev, int64_t cand_capacity, int64_t* counts_dev,
+                                             mlpsp_stream_t stream) {
+  const int64_t T = checked_num_tiles(width, height, tile, tile);
+  if (!counts_dev || cand_capacity < 0 || cand_capacity > 2147483647LL || (cand_capacity > 0 && !candidates_dev))
+    return MLPSP_E_ARGUMENT;
+  if (num_views > kStaticBinMaxViews) return MLPSP_E_ARGUMENT;
+  void* scratch_dev = nullptr;
+  const int src = static_scratch_of_current_device(&scratch_dev);
+  if (src != MLPSP_OK) return src;
+  const size_t need = mlpsp_bin_scratch_bytes(num_primitives, num_views, width, height, tile);
+  if (need == 0) return MLPSP_E_ARGUMENT;
+  if (need > kStaticBinScratchBytes) return MLPSP_E_SCRATCH;      // beyond the fixed maximum: use mlpsp_bin_legacy_async
+  const int rc = check_bin_args(T, view_matrices_host, proj_host, scratch_dev, kStaticBinScratchBytes, tile_offsets_dev,
+                                num_primitives, num_views, width, height, tile, threshold);
+  if (rc != MLPSP_OK) return rc;
+  hipStream_t s = (hipStream_t)stream;
+  const BinGeom g = make_geom(num_primitives, num_views, width, height, tile);
+  // the array is carved for exactly the size the ordinary entry point would be given, so that both run the
+  // same launches on the same layout
+  const BinScratch b = carve(scratch_dev, need, num_primitives, num_views, g.nsx * g.nsy, g.NC);
+  if (num_primitives == 0) {
+    hipLaunchKernelGGL(fill_i32_kernel, dim3(64), dim3(256), 0, s, tile_offsets_dev, (long long)(T + 1), 0);
+    MLPSP_LAUNCH_CHECK();
+    hipLaunchKernelGGL(fill_i32_kernel, dim3(1), dim3(256), 0, s, reinterpret_cast<int32_t*>(counts_dev), 8LL, 0);
+    MLPSP_LAUNCH_CHECK();
+    return MLPSP_OK;
+  }
+  if (num_views > 1) {
+    ManyMats m{};
+    for (int k = 0; k < num_views; ++k)
+      for (int e = 0; e < 16; ++e) m.v[k][e] = view_matrices_host[k * 16 + e];
+    for (int e = 0; e < 16; ++e) m.p[e] = proj_host[e];
+    hipLaunchKernelGGL(store_matrices_kernel, dim3(1), dim3(64), 0, s, m, num_views, b.mats);
+    MLPSP_LAUNCH_CHECK();
+  }
+  const int erc = enqueue_bin_count(positions_dev, log_scales_dev, num_primitives, view_matrices_host, num_views,
+                                    tile_view_ids_dev, proj_host, width, height, tile, threshold, g, b, T,
+                                    tile_offsets_dev, s, /*matrices_in_scratch=*/true);
+  if (erc != MLPSP_OK) return erc;
+  hipLaunchKernelGGL(bin_guard_kernel, dim3(64), dim3(256), 0, s, b.totals, b.l1_capacity, (long long)cand_capacity,
+                     tile_offsets_dev, (int)(T + 1), (long long*)counts_dev);
+  MLPSP_LAUNCH_CHECK();
+  hipLaunchKernelGGL((bin_level2_kernel<true>), dim3(ceil_div((int)T, kBinThreads / 64)), dim3(kBinThreads), 0, s,
+                     b.bounds, g, tile_view_ids_dev, b.l1_counts, b.l1_list, b.l1_bounds, b.l1_capacity, tile_offsets_dev,
+                     candidates_dev, b.l2_masks, b.l2_mask_stride, (const long long*)(b.totals + 3));
   MLPSP_LAUNCH_CHECK();
   return MLPSP_OK;
 }
