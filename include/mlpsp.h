@@ -141,10 +141,13 @@ int mlpsp_bin_raycone_fill(int num_primitives, int width, int height, int tile, 
  * cull_threshold: 0 = off.  In (0,1) (the render's score threshold): a candidate that provably hits
  * no ray of its tile at that threshold is written as ~id (negative).  The render entry points skip
  * negative ids, so images are unchanged; ~ recovers the plain sorted list.  Has no counterpart in the
- * reference, whose kernels run the full ray test on every candidate. */
+ * reference, whose kernels run the full ray test on every candidate.
+ * prim_records_dev holds num_primitives records.  Null pointers (sorted_keys_dev aside) return MLPSP_E_ARGUMENT;
+ * a candidate id outside [0, num_primitives) -- a list that was not validated -- is not dereferenced: it sorts
+ * last with the invalid key and is passed on as it is (the render entry points skip such ids). */
 int mlpsp_sort_tiles(const float* rays_o_dev, const float* rays_d_dev, const void* prim_records_dev,
-                     const int32_t* candidates_dev, const int32_t* tile_offsets_dev, int width, int height,
-                     int tile_w, int tile_h, int key_family, int capacity, float cull_threshold,
+                     int num_primitives, const int32_t* candidates_dev, const int32_t* tile_offsets_dev, int width,
+                     int height, int tile_w, int tile_h, int key_family, int capacity, float cull_threshold,
                      int32_t* sorted_ids_dev, float* sorted_keys_dev, mlpsp_stream_t stream);
 
 /* Tile-centre-order forward, scalar f32 (render_tiles_kernel_tilecenter_order,

@@ -41,7 +41,7 @@ SIGNATURES = {
     "mlpsp_bin_raycone_scratch_bytes": (_sz, [_i, _i, _i, _i]),
     "mlpsp_bin_raycone_count": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _f, _vp, _sz, _vp, C.POINTER(_i64), _vp]),
     "mlpsp_bin_raycone_fill": (_i, [_i, _i, _i, _i, _vp, _sz, _vp, _vp, _vp]),
-    "mlpsp_sort_tiles": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _vp, _vp, _vp]),
+    "mlpsp_sort_tiles": (_i, [_vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _vp, _vp, _vp]),
     "mlpsp_render_tilecenter_f32": (_i, [_vp] * 7 + [_i] + [_vp] * 6 + [_i, _i, _i, _i, _i, _i, _f, _vp, _vp, _vp,
                                                                        _vp, _vp]),
     "mlpsp_render_tilecenter_feat_f32": (_i, [_vp] * 7 + [_i] + [_vp] * 6 + [_i, _i, _vp, _i, _i, _f, _f, _i, _i, _i, _i,

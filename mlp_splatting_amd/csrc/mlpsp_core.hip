@@ -110,7 +110,7 @@ struct TilePyramid {
 __global__ __launch_bounds__(kSortThreads) void sort_tiles_kernel(
     const float* __restrict__ rays_o, const float* __restrict__ rays_d, const PrimRecord* __restrict__ prims,
     const int32_t* __restrict__ cand, const int32_t* __restrict__ offsets, TileGeom g, int family, int capacity,
-    float cull_r2, int32_t* __restrict__ sorted_ids, float* __restrict__ sorted_keys) {
+    float cull_r2, int num_prims, int32_t* __restrict__ sorted_ids, float* __restrict__ sorted_keys) {
   __shared__ unsigned long long s_key[kSortMax];
   __shared__ int s_wave_cnt[2][kSortThreads / 64];
   __shared__ TilePyramid s_pyr;
@@ -130,8 +130,10 @@ __global__ __launch_bounds__(kSortThreads) void sort_tiles_kernel(
   // The first round's candidate id and geometry record are requested before the pyramid phase (two dependent
   // gathers whose latency then overlaps the corner-ray loads and the barriers below); every round requests the
   // next round's in the same way.
+  // An id outside [0, num_prims) (lists that were never validated) reads record 0, is never culled and sorts last
+  // with the invalid key; it is passed on unchanged, and the render kernels skip it.
   int p_next = (tid < n) ? cand[start + tid] : 0;
-  PrimRecord P_next = prims[p_next];
+  PrimRecord P_next = prims[((unsigned)p_next < (unsigned)num_prims) ? p_next : 0];
 
   // ---- the tile's ray pyramid (only when culling is requested)
   const bool culling = cull_r2 > 0.f;
@@ -198,10 +200,11 @@ __global__ __launch_bounds__(kSortThreads) void sort_tiles_kernel(
     p = p_next;
     if (i + kSortThreads < n) {
       p_next = cand[start + i + kSortThreads];
-      P_next = prims[p_next];
+      P_next = prims[((unsigned)p_next < (unsigned)num_prims) ? p_next : 0];
     }
+    const bool known = (unsigned)p < (unsigned)num_prims;
     if (i < n) {
-      if (faces) {
+      if (faces && known) {
         const float ex = P.cx - s_pyr.ox, ey = P.cy - s_pyr.oy, ez = P.cz - s_pyr.oz;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
@@ -214,7 +217,8 @@ __global__ __launch_bounds__(kSortThreads) void sort_tiles_kernel(
       }
       keep = !outside;
       if (keep)
-        key = (family == MLPSP_KEY_DEPTH) ? key_depth(ox, oy, oz, dx, dy, dz, P) : key_tstar(ox, oy, oz, dx, dy, dz, P);
+        key = !known ? kInvalidKey
+                     : (family == MLPSP_KEY_DEPTH) ? key_depth(ox, oy, oz, dx, dy, dz, P) : key_tstar(ox, oy, oz, dx, dy, dz, P);
     }
     const unsigned long long m = __ballot(keep);
     if (lane == 0) s_wave_cnt[round][wave] = __popcll(m);
@@ -343,8 +347,8 @@ MLPSP_API int mlpsp_validate_tile_lists(const int32_t* tile_offsets_dev, const i
 }
 
 MLPSP_API int mlpsp_sort_tiles(const float* rays_o_dev, const float* rays_d_dev, const void* prim_records_dev,
-                               const int32_t* candidates_dev, const int32_t* tile_offsets_dev, int width,
-                               int height, int tile_w, int tile_h, int key_family, int capacity,
+                               int num_primitives, const int32_t* candidates_dev, const int32_t* tile_offsets_dev,
+                               int width, int height, int tile_w, int tile_h, int key_family, int capacity,
                                float cull_threshold, int32_t* sorted_ids_dev, float* sorted_keys_dev,
                                mlpsp_stream_t stream) {
   const int64_t T = checked_num_tiles(width, height, tile_w, tile_h);
@@ -352,15 +356,16 @@ MLPSP_API int mlpsp_sort_tiles(const float* rays_o_dev, const float* rays_d_dev,
   if (key_family != MLPSP_KEY_TSTAR && key_family != MLPSP_KEY_DEPTH) return MLPSP_E_ARGUMENT;
   if (capacity < 0 || capacity > MLPSP_TILE_CAPACITY_MAX) return MLPSP_E_ARGUMENT;
   if (capacity == 0) capacity = MLPSP_TILE_CAPACITY_MAX;
-  if (!rays_o_dev || !rays_d_dev || !tile_offsets_dev) return MLPSP_E_ARGUMENT;
-  if (sorted_ids_dev && sorted_ids_dev == candidates_dev) return MLPSP_E_ARGUMENT;   // not an in-place sort
+  if (!rays_o_dev || !rays_d_dev || !tile_offsets_dev || !candidates_dev || !sorted_ids_dev) return MLPSP_E_ARGUMENT;
+  if (num_primitives <= 0 || !prim_records_dev) return MLPSP_E_ARGUMENT;
+  if (sorted_ids_dev == candidates_dev) return MLPSP_E_ARGUMENT;   // not an in-place sort
   TileGeom g{width, height, tile_w, tile_h, ceil_div(width, tile_w), ceil_div(height, tile_h)};
   // squared radius of the threshold ellipsoid in units of the scales, with a 2 % margin on the radius
   float cull_r2 = 0.f;
   if (cull_threshold > 0.f && cull_threshold < 1.f) cull_r2 = -2.0f * logf(cull_threshold) * 1.0404f + 1e-6f;
   hipLaunchKernelGGL(sort_tiles_kernel, dim3((unsigned)T), dim3(kSortThreads), 0, (hipStream_t)stream, rays_o_dev,
                      rays_d_dev, (const PrimRecord*)prim_records_dev, candidates_dev, tile_offsets_dev, g, key_family,
-                     capacity, cull_r2, sorted_ids_dev, sorted_keys_dev);
+                     capacity, cull_r2, num_primitives, sorted_ids_dev, sorted_keys_dev);
   MLPSP_LAUNCH_CHECK();
   return MLPSP_OK;
 }

@@ -162,7 +162,11 @@ def sort_tiles(rays_o, rays_d, records, candidates, tile_offsets, W, H, TW, TH, 
     dev = rays_o.device
     sorted_ids = torch.empty_like(candidates)
     keys = torch.empty(candidates.numel(), dtype=torch.float32, device=dev) if want_keys else None
-    code = _lib.load().mlpsp_sort_tiles(_ptr(rays_o), _ptr(rays_d), _ptr(records), _ptr(candidates), _ptr(tile_offsets),
+    if candidates.numel() == 0:
+        return sorted_ids, keys
+    num_primitives = records.numel() // _lib.PRIM_RECORD_BYTES
+    code = _lib.load().mlpsp_sort_tiles(_ptr(rays_o), _ptr(rays_d), _ptr(records), num_primitives, _ptr(candidates),
+                                        _ptr(tile_offsets),
                                         W, H, TW, TH, int(family), int(capacity), float(cull_threshold),
                                         _ptr(sorted_ids), _ptr(keys), _stream(dev))
     _check(code, "mlpsp_sort_tiles")

@@ -48,15 +48,12 @@ class TileExt:
         self._mfma_fallbacks = 0
         self._training_mfma_stats = [0, 0, 0, 0, 0]
         self._uncached = threading.local()
-        self._pack_key = None
-        self._pack = None
-        self._feat_pack_key = None
-        self._binned = None
-        self._rec_key = None
+        self._pack = None                 # cache entries: (key, value, source tensors) -- see _derived
+        self._feat_pack = None
         self._rec = None
+        self._binned = None
         self._queue_capacity = 0          # candidate-buffer estimate of render_frame_queued (0: not seeded yet)
         self._queue_scratch_scale = 1
-        self._feat_pack = None
 
     # ------------------------------------------------------------------------------------------
     # derived-tensor caches (geometry records, matrix-core operand copies)
@@ -68,9 +65,7 @@ class TileExt:
         Every training entry point therefore works uncached and leaves the caches empty; call this after
         changing parameters by any other means that does not advance the version."""
         with self._lock:
-            self._pack_key = self._pack = None
-            self._feat_pack_key = self._feat_pack = None
-            self._rec_key = self._rec = None
+            self._pack = self._feat_pack = self._rec = None
         # (the note about freshly binned tile lists is keyed on the list tensors themselves, not on parameters)
 
     @contextlib.contextmanager
@@ -119,7 +114,8 @@ class TileExt:
         read-back (np_tile_kernels.cu:4553-4588).  Anything else is validated on the device."""
         key = self._list_key(cand, offsets, num_primitives)
         with self._lock:
-            self._binned = None if key is None else (key, int(longest))
+            # (the note keeps the two tensors: their addresses identify them only while they are allocated)
+            self._binned = None if key is None else (key, int(longest), cand, offsets)
 
     def _validate(self, cand, offsets, n_tiles, capacity, n, name):
         with self._lock:
@@ -752,42 +748,45 @@ class TileExt:
     def rgb_wmma_safety_stats(self):
         return [self._mfma_calls, self._mfma_fallbacks]
 
+    @staticmethod
+    def _source_key(tensors, extra=()):
+        """Cache key of a derived tensor: address, in-place version, shape and device of every source.  None for
+        inference tensors, which carry no version counter (an edit could not be seen: no caching)."""
+        try:
+            return tuple(extra) + tuple((t.data_ptr(), t._version, tuple(t.shape), str(t.device)) for t in tensors)
+        except RuntimeError:
+            return None
+
+    def _derived(self, slot, sources, extra, build):
+        """``build()`` once per state of ``sources``.  The entry keeps the source tensors themselves: while it lives
+        their memory cannot be freed and handed to another scene's tensors of the same shape, whose key would then
+        match (the address is only an identity for memory that is still allocated).  The price is that the last
+        scene's tensors stay allocated until another scene is rendered or :meth:`invalidate_caches` is called."""
+        if not self._caching():
+            return build()
+        key = self._source_key(sources, extra)
+        if key is None:
+            return build()
+        with self._lock:
+            entry = getattr(self, slot)
+            if entry is None or entry[0] != key:
+                entry = (key, build(), tuple(sources))
+                setattr(self, slot, entry)
+            return entry[1]
+
     def _records(self, positions, log_scales, quats):
         """Per-primitive geometry records, rebuilt only when one of the three tensors changed."""
-        if not self._caching():
-            return ops.prepare_primitives(positions, log_scales, quats)
-        try:
-            key = tuple((t.data_ptr(), t._version, tuple(t.shape), str(t.device)) for t in (positions, log_scales, quats))
-        except RuntimeError:                      # inference tensors have no version counter: no caching
-            return ops.prepare_primitives(positions, log_scales, quats)
-        with self._lock:
-            if self._rec_key != key:
-                self._rec = ops.prepare_primitives(positions, log_scales, quats)
-                self._rec_key = key
-            return self._rec
+        return self._derived("_rec", (positions, log_scales, quats), (),
+                             lambda: ops.prepare_primitives(positions, log_scales, quats))
 
     def _packed_weights(self, ws, bf16):
         """Matrix-core operand copy of the six weight tensors, rebuilt only when one of them changed
         (identity, shape or in-place version) -- the scene's weights are constant during inference."""
-        if not self._caching():
-            return ops.pack_mfma_weights(*ws, bf16=bf16)
-        key = (bool(bf16),) + tuple((w.data_ptr(), w._version, tuple(w.shape), str(w.device)) for w in ws)
-        with self._lock:
-            if self._pack_key != key:
-                self._pack = ops.pack_mfma_weights(*ws, bf16=bf16)
-                self._pack_key = key
-            return self._pack
+        return self._derived("_pack", tuple(ws), (bool(bf16),), lambda: ops.pack_mfma_weights(*ws, bf16=bf16))
 
     def _packed_feat(self, feat_attr):
         """fp16 operand copy of the feature attributes, cached like the weights -> (packed, nonfinite)."""
-        if not self._caching():
-            return ops.pack_mfma_feat(feat_attr)
-        key = (feat_attr.data_ptr(), feat_attr._version, tuple(feat_attr.shape), str(feat_attr.device))
-        with self._lock:
-            if self._feat_pack_key != key:
-                self._feat_pack = ops.pack_mfma_feat(feat_attr)
-                self._feat_pack_key = key
-            return self._feat_pack
+        return self._derived("_feat_pack", (feat_attr,), (), lambda: ops.pack_mfma_feat(feat_attr))
 
     def render_tiles_rgb_wmma(self, x, width, height, threshold, bf16):
         """[rgb, alpha] with the 72->32->32->4 MLP on the matrix cores, f32 everywhere else."""

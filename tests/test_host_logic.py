@@ -180,12 +180,10 @@ def test_training_paths_leave_no_derived_tensor_behind():
     ext = TileExt()
 
     def fill():
-        ext._pack_key, ext._pack = ("k",), object()
-        ext._rec_key, ext._rec = ("k",), object()
-        ext._feat_pack_key, ext._feat_pack = ("k",), object()
+        ext._pack = ext._rec = ext._feat_pack = (("k",), object(), ())
 
     def empty():
-        return all(v is None for v in (ext._pack_key, ext._pack, ext._rec_key, ext._rec, ext._feat_pack_key, ext._feat_pack))
+        return all(v is None for v in (ext._pack, ext._rec, ext._feat_pack))
 
     fill()
     assert ext._caching() and not empty()
@@ -202,9 +200,9 @@ def test_training_paths_leave_no_derived_tensor_behind():
         with ext.uncached():
             raise ValueError("a failing training call")
     assert empty() and ext._caching()
-    ext._binned = ("lists", 7)
+    ext._binned = ("lists", 7, None, None)
     ext.invalidate_caches()
-    assert ext._binned == ("lists", 7)           # keyed on the list tensors, not on parameters
+    assert ext._binned == ("lists", 7, None, None)     # keyed on the list tensors, not on parameters
 
 
 def test_scene_invalidation_reaches_the_extension(monkeypatch):
@@ -213,9 +211,45 @@ def test_scene_invalidation_reaches_the_extension(monkeypatch):
     monkeypatch.setattr(cumodel, "_tile_ext", ext)
     scene = NeuralPrimitiveSceneTileCUDA(num_primitives=4, hidden_dim=32)
     scene.__dict__["_mlpsp_cache"] = {"unit_quats": (("key",), object())}
-    ext._rec_key, ext._rec = ("k",), object()
+    ext._rec = (("k",), object(), ())
     scene.invalidate_render_caches()
-    assert "_mlpsp_cache" not in scene.__dict__ and ext._rec_key is None and ext._rec is None
+    assert "_mlpsp_cache" not in scene.__dict__ and ext._rec is None
+
+
+def test_derived_tensor_cache_cannot_be_served_to_recycled_memory():
+    """A cache entry is keyed on the sources' addresses and versions -- an identity only while that memory stays
+    allocated -- so the entry keeps the source tensors: with the first scene's tensor dropped by its owner, a second
+    tensor of the same shape cannot land on its address, and a faked collision of the key alone never happens.
+    Inference tensors (no version counter) are never cached."""
+    from mlp_splatting_amd.tile_ext import TileExt
+    ext = TileExt()
+    built = []
+
+    def build(tag):
+        built.append(tag)
+        return tag
+
+    first = torch.zeros(8)
+    address = first.data_ptr()
+    assert ext._derived("_rec", (first,), (), lambda: build("first")) == "first"
+    assert ext._derived("_rec", (first,), (), lambda: build("again")) == "first"        # served from the cache
+    del first                                               # the owner lets go; the entry still holds the memory
+    assert ext._rec[2][0].data_ptr() == address
+    second = torch.zeros(8)
+    assert second.data_ptr() != address                      # so an equal-shaped newcomer lives elsewhere
+    assert ext._derived("_rec", (second,), (), lambda: build("second")) == "second"
+    second.add_(1)                                           # an in-place edit is seen through the version counter
+    assert ext._derived("_rec", (second,), (), lambda: build("edited")) == "edited"
+    with torch.inference_mode():
+        frozen = torch.zeros(8)
+    assert ext._source_key((frozen,)) is None
+    assert ext._derived("_pack", (frozen,), (True,), lambda: build("a")) == "a"
+    assert ext._derived("_pack", (frozen,), (True,), lambda: build("b")) == "b" and ext._pack is None
+    assert built == ["first", "second", "edited", "a", "b"]
+    # the note about freshly binned lists holds its two tensors for the same reason
+    cand, offsets = torch.zeros(4, dtype=torch.int32), torch.zeros(3, dtype=torch.int32)
+    ext.note_binned_lists(cand, offsets, 2, 10)
+    assert ext._binned[2] is cand and ext._binned[3] is offsets
 
 
 def test_harness_statistics_closed_forms():
