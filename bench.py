@@ -18,14 +18,64 @@ if ROOT not in sys.path:
 
 PEAK = {"f32": 157.3, "bf16": 2500.0}          # MI355X dense peaks, TFLOP/s
 HBM_PEAK_GBS = 8000.0
-# HBM bytes per launch of the render kernel, from hardware counters: two profiled runs of
-#   rocprofv3 --pmc FETCH_SIZE -- python3 bench.py --steps 16 --warmup 8 --no-cpu-baseline --wake-seconds 0 --copy-calibration
-#   rocprofv3 --pmc WRITE_SIZE -- (same)
-# averaged over the run's 56 launches, each counter scaled by what it reads for the 1 GiB device copies of
-# --copy-calibration (FETCH_SIZE reads 524,307 KiB for 1,048,576 KiB copied: factor 2.0; WRITE_SIZE reads
-# 1,048,576 KiB: factor 1.0).  Render kernel: 51,118 KiB x 2.0 fetched + 16,832 KiB written = 121.9 MB
-# (profiles/render_tilecenter_mfma_cfg3_200k_1200x680.txt).
-MEASURED_TRAFFIC_BYTES = {("cfg3_200k_1200x680", "bf16"): int((51117.9 * 2.0 + 16831.6) * 1024)}
+PROFILES = os.path.join(ROOT, "profiles")
+
+
+def measured_traffic(kernel: str, workload: str, ms_per_launch: float):
+    """HBM bytes per launch of `kernel` from the committed hardware-counter profile profiles/<kernel>_<workload>.txt
+    (two rocprofv3 --pmc runs, FETCH_SIZE and WRITE_SIZE, each scaled by what the counter reads for a device copy of
+    known size; the file states the commands).  The profile carries the kernel's average duration when the counters
+    were taken: if this run's duration differs from it by more than 10 %, the kernel is no longer the one that was
+    profiled and no traffic figure is reported.  -> (bytes or None, note)"""
+    import re
+    path = os.path.join(PROFILES, f"{kernel}_{workload}.txt")
+    if not os.path.exists(path):
+        return None, f"no profile {os.path.basename(path)}"
+    text = open(path).read()
+    got = {k: re.search(rf"^bench\.{k}\s*=\s*([0-9.eE+]+)", text, flags=re.M) for k in ("traffic_bytes", "kernel_avg_us")}
+    if not all(got.values()):
+        return None, f"{os.path.basename(path)} holds no bench.traffic_bytes / bench.kernel_avg_us lines"
+    traffic, avg_us = float(got["traffic_bytes"].group(1)), float(got["kernel_avg_us"].group(1))
+    if abs(ms_per_launch * 1e3 - avg_us) > 0.10 * avg_us:
+        return None, (f"profiled kernel took {avg_us:.1f} us, this run {ms_per_launch * 1e3:.1f} us: "
+                      f"{os.path.basename(path)} is stale")
+    return int(traffic), f"profiles/{os.path.basename(path)} (kernel {avg_us:.1f} us when profiled)"
+
+
+def dense_culling_cpu_torch(positions, log_scales, view, proj, W, H, tile, thr):
+    """The reference's culling as it writes it -- a dense [tiles x primitives] overlap matrix turned into a tile-major
+    list (scannet/cumodel.py:994-1070) -- evaluated with CPU torch.  Measurement aid of the cpu_baseline leg only:
+    the renderer itself never bins this way.  -> (seconds, number of tile-primitive pairs)"""
+    import torch
+    t0 = time.perf_counter()
+    with torch.no_grad():
+        n = positions.shape[0]
+        homogeneous = torch.cat([positions, positions.new_ones(n, 1)], dim=1)
+        in_view = homogeneous @ view.T
+        z = in_view[:, 2]
+        visible = z > 1e-3
+        largest_axis = log_scales.exp().amax(dim=1)
+        focal = 0.5 * (proj[0, 0] * W / 2.0 + proj[1, 1] * H / 2.0)
+        reach = largest_axis * torch.sqrt(-2.0 * torch.log(torch.tensor(float(thr)))) / (z + 1e-8) * focal
+        clip = in_view @ proj.T
+        w = clip[:, 3:4]
+        w = w + 1e-6 * (w == 0)
+        ndc = clip[:, :3] / w
+        cx, cy = (ndc[:, 0] + 1) * 0.5 * W, (ndc[:, 1] + 1) * 0.5 * H
+        ntx, nty = (W + tile - 1) // tile, (H + tile - 1) // tile
+        tiles = torch.arange(ntx * nty)
+        left, top = ((tiles % ntx) * tile)[:, None], ((tiles // ntx) * tile)[:, None]
+        touches = ((cx - reach)[None] < left + tile) & ((cx + reach)[None] > left) \
+            & ((cy - reach)[None] < top + tile) & ((cy + reach)[None] > top) & visible[None]
+        pairs = touches.nonzero()
+        order = torch.argsort(pairs[:, 0])
+        pairs = pairs[order]
+        offsets = torch.zeros(ntx * nty + 1, dtype=torch.long)
+        which, how_many = torch.unique_consecutive(pairs[:, 0], return_counts=True)
+        offsets.scatter_add_(0, which + 1, how_many)
+        offsets = offsets.cumsum(0).to(torch.int32)
+        listed = pairs[:, 1].to(torch.int32)
+    return time.perf_counter() - t0, int(listed.numel())
 
 
 def train_steps(args, scene, frames, proj, thr, W, H, sc, dev):
@@ -120,6 +170,9 @@ def main() -> int:
                          "the record pipeline, Adam on all nine parameter tensors); prints its own JSON line")
     ap.add_argument("--wake-seconds", type=float, default=1.0,
                     help="untimed rendering before the warm-up steps, to bring an idle GPU to its sustained clocks")
+    ap.add_argument("--min-seconds", type=float, default=0.5,
+                    help="the timed region is extended, in whole passes of --steps, until it lasts at least this long; "
+                         "the JSON line reports the steps actually timed")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run 4 plain device copies of 1 GiB, the known-size kernel that hardware counter "
@@ -222,11 +275,17 @@ def main() -> int:
         render(i)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for i in range(args.steps):
-        render(i)
+    timed_steps = 0
+    while True:
+        for i in range(args.steps):
+            render(timed_steps + i)
+        timed_steps += args.steps
+        # (checked on the host clock without a synchronisation: the queue is a few frames deep at most)
+        if time.perf_counter() - t0 >= args.min_seconds:
+            break
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
-    fps = args.steps / elapsed
+    fps = timed_steps / elapsed
 
     # per-frame latency distribution, the way tools/benchmark_inference.py:121-149 times a frame: a
     # synchronise on both sides of every call (so nothing overlaps between frames, unlike the loop above)
@@ -257,9 +316,12 @@ def main() -> int:
         rd = torch.nn.functional.normalize(rd_raw, dim=-1).contiguous()
         e = [torch.cuda.Event(enable_timing=True) for _ in range(4)]
         rec = ops.prepare_primitives(scene.positions.detach(), scene.log_scales.detach(), quats)
-        e[0].record()
         cand, off = ops.bin_legacy(scene.positions.detach(), scene.log_scales.detach(), views, proj, W, H, 8, thr,
                                    tile_view_ids=tv)
+        # the binning as a frame queues it: no host synchronisation, candidate buffer sized beforehand
+        e[0].record()
+        ops.bin_legacy_async(scene.positions.detach(), scene.log_scales.detach(), views, proj, W, H, 8, thr,
+                             cand.numel(), tile_view_ids=tv)
         e[1].record()
         order, _ = ops.sort_tiles(ro, rd, rec, cand, off, W, H, 8, 8, cull_threshold=thr)
         counters = torch.zeros(4, dtype=torch.int64, device=dev)
@@ -292,26 +354,38 @@ def main() -> int:
         e1.record()
         torch.cuda.synchronize()
         mfma_probe = round(probe_flops / (e0.elapsed_time(e1) * 1e-3) / 1e12, 1)
-    # do the matrix pipe and the vector ALU of one SIMD overlap?  (mlpsp_probe_issue: modes 0..3)
+    # how matrix-core, vector and transcendental instructions share a SIMD's issue time at the render kernel's
+    # occupancy (four wavefronts per SIMD): core clocks per instruction and SIMD for each mix (mlpsp_probe_issue)
+    import ctypes
     lib = _lib.load()
     stream = torch.cuda.current_stream(dev).cuda_stream
     sink = torch.zeros(1, device=dev)
-    probe_ms = []
-    for mode in range(5):
-        lib.mlpsp_probe_issue(mode, 500, sink.data_ptr(), stream)
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        lib.mlpsp_probe_issue(mode, 20000, sink.data_ptr(), stream)
-        e1.record()
+    probe_out = torch.zeros(4096 * 3, dtype=torch.int64, device=dev)
+    per_batch = {1: ("mfma", 16), 2: ("valu", 128), 3: ("trans", 128), 4: ("mfma", 16)}
+
+    def issue(roles):
+        arr = (ctypes.c_int32 * 4)(*roles)
+        lib.mlpsp_probe_issue(arr, 1500, probe_out.data_ptr(), sink.data_ptr(), stream)
         torch.cuda.synchronize()
-        probe_ms.append(e0.elapsed_time(e1))
-    serial, ideal = 0.5 * (probe_ms[0] + probe_ms[1]), 0.5 * max(probe_ms[0], probe_ms[1])
-    issue_probe = {"mfma_ms": round(probe_ms[0], 4), "valu_ms": round(probe_ms[1], 4), "mixed_ms": round(probe_ms[2], 4),
-                   "mixed_if_serial_ms": round(serial, 4), "mixed_if_overlapped_ms": round(ideal, 4),
-                   "overlap": round((serial - probe_ms[2]) / max(serial - ideal, 1e-9), 3),
-                   "sin_issue_vs_fma": round((probe_ms[3] / 2.0) / (probe_ms[1] / 8.0), 2),
-                   "same_wavefront_ms": round(probe_ms[4], 4),
-                   "same_wavefront_vs_serial": round(probe_ms[4] / (probe_ms[0] + probe_ms[1]), 3)}
+        rec = probe_out.cpu().numpy().reshape(4096, 3)
+        role_of = (rec[:, 2] & 0xffffffff).astype(int)
+        out_clk = {}
+        for role in sorted(set(roles) - {0}):
+            sel = role_of == role
+            clocks_per_batch_simd = rec[sel, 1].mean() / (rec[sel, 0].mean() * roles.count(role))
+            out_clk[role] = clocks_per_batch_simd / per_batch[role][1]
+        return out_clk
+    issue((1, 1, 1, 1))                                         # (clock ramp)
+    alone = {**issue((1, 1, 1, 1)), **issue((2, 2, 2, 2)), **issue((3, 3, 3, 3))}
+    mixed_wave = issue((4, 4, 4, 4))[4]                         # clocks per (MFMA + 8 FMA), every wavefront doing both
+    across = issue((1, 2, 1, 2))                                # two MFMA wavefronts and two FMA wavefronts per SIMD
+    issue_probe = {"waves_per_simd": 4,
+                   "clk_per_mfma_32x32x16": round(alone[1], 2), "clk_per_valu_fma": round(alone[2], 2),
+                   "clk_per_transcendental": round(alone[3], 2),
+                   "same_wave_mfma_plus_8_fma_clk": round(mixed_wave, 2),
+                   "same_wave_if_serial_clk": round(alone[1] + 8 * alone[2], 2),
+                   "across_waves_clk_per_mfma": round(across[1], 2), "across_waves_clk_per_fma": round(across[2], 2),
+                   "across_waves_fma_issued_per_mfma": round(across[1] / across[2], 2)}
     flops_per_hit = 2 * (72 * sc.hidden + sc.hidden * sc.hidden + 4 * sc.hidden)
     achieved_tflops = flops_per_hit * hits / (kernel_ms * 1e-3) / 1e12
     # sort kernel: 8 compulsory bytes per candidate (4 id in, 4 id out) + the 64-byte record of every primitive
@@ -321,12 +395,18 @@ def main() -> int:
     T_tiles = ((W + 7) // 8) * ((H + 7) // 8)
     bin_gbs = (24.0 * sc.n * n_probe + 4.0 * cand_total + 4.0 * (T_tiles + 1) * n_probe) / (bin_ms * 1e-3) / 1e9
 
+    render_kernel = "render_tilecenter_" + ("mfma" if precision == "bf16" else "f32")
+    traffic, traffic_note = measured_traffic(render_kernel, args.workload, kernel_ms / n_probe)
+    sort_traffic, sort_note = measured_traffic("sort_tiles", args.workload, sort_ms / n_probe)
+    # the sort by the accounting of the hot-path scope table: 4 B id in + 40 B gathered geometry + 4 B id out per
+    # candidate (next to the kernel's own compulsory bytes above, in which every 64-byte record counts once)
+    sort_gbs_per_candidate = 48.0 * cand_total / (sort_ms * 1e-3) / 1e9
     out = {
         "metric": ("forward_render_frames_per_sec_1200x680_200k_primitives" if args.workload.startswith("cfg3")
                    else f"forward_render_frames_per_sec_{args.workload}"),
-        "value": round(fps, 3), "unit": "frames/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "wake_seconds": args.wake_seconds,
-        "ms_per_step": round(1000.0 * elapsed / args.steps, 4), "higher_is_better": True, "scaling": "weak",
+        "value": round(fps, 3), "unit": "frames/s", "n_gpus": 1, "steps": timed_steps, "warmup": args.warmup,
+        "wake_seconds": args.wake_seconds, "steps_per_pass": args.steps, "min_seconds": args.min_seconds,
+        "ms_per_step": round(1000.0 * elapsed / timed_steps, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": precision, "data": "synthetic",
         "config": {"workload": args.workload, "primitives": sc.n, "width": W, "height": H, "tile": 8,
                    "threshold": thr, "poses": len(frames), "poses_over_capacity_left_out": skipped_poses,
@@ -337,7 +417,7 @@ def main() -> int:
         "roofline": {"bound": "mfma", "kernel": "render_tilecenter_" + ("mfma" if precision == "bf16" else "f32"),
                      "achieved": round(achieved_tflops, 3), "peak": PEAK[precision], "unit": "TFLOP/s",
                      "frac": round(achieved_tflops / PEAK[precision], 5),
-                     "traffic": MEASURED_TRAFFIC_BYTES.get((args.workload, precision)),
+                     "traffic": traffic, "traffic_source": traffic_note,
                      "ms_per_launch": round(kernel_ms / n_probe, 4), "hits_per_launch": hits // n_probe,
                      "tile_primitives_per_launch": proc // n_probe,
                      "hit_wavefronts_per_launch": hit_waves // n_probe, "flops_per_hit": flops_per_hit,
@@ -345,7 +425,10 @@ def main() -> int:
         "stages": {"bin_ms": round(bin_ms / n_probe, 4), "sort_ms": round(sort_ms / n_probe, 4),
                    "render_ms": round(kernel_ms / n_probe, 4),
                    "sort_hbm": {"bound": "hbm", "achieved": round(sort_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                                "frac": round(sort_gbs / HBM_PEAK_GBS, 5)},
+                                "frac": round(sort_gbs / HBM_PEAK_GBS, 5),
+                                "achieved_at_48B_per_candidate": round(sort_gbs_per_candidate, 1),
+                                "frac_at_48B_per_candidate": round(sort_gbs_per_candidate / HBM_PEAK_GBS, 5),
+                                "traffic": sort_traffic, "traffic_source": sort_note},
                    "bin_hbm": {"bound": "hbm", "achieved": round(bin_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                                "frac": round(bin_gbs / HBM_PEAK_GBS, 5)},
                    "candidates_per_launch": cand_total // n_probe},
@@ -360,31 +443,45 @@ def main() -> int:
         del src, dst
 
     if not args.no_cpu_baseline:
-        # the CPU restatement of the same algorithm, on this host's cores: ONE full frame (pose 0)
+        # the CPU restatement of the same algorithm, on this host's cores: full frames of pose 0, median of the runs
         import oracle
         ro, rd_raw, views, tv = frames[0]
         rd = torch.nn.functional.normalize(rd_raw, dim=-1).cpu().numpy()
         ro_np = ro.cpu().numpy()
-        tc = time.perf_counter()
-        cand, off = oracle.bin_legacy(sc.positions, sc.log_scales, views.cpu().numpy(), proj.cpu().numpy(), W, H, 8, thr,
-                                      tile_view_ids=None if tv is None else tv.cpu().numpy())
         fkw = {}
-        if feature_dim:
+        if feature_dim:            # (the 1.6 GB attribute download is not part of the CPU figure)
             fkw = dict(feat_attr=scene.feat_attr.detach().cpu().numpy(), beta=float(scene.feature_gating_beta),
                        temp=float(scene.feature_gating_temp))
-            tc = time.perf_counter()          # the 1.6 GB attribute download is not part of the CPU figure
-            cand, off = oracle.bin_legacy(sc.positions, sc.log_scales, views.cpu().numpy(), proj.cpu().numpy(), W, H, 8,
-                                          thr)
-        res = oracle.render_tilecenter(ro_np, rd, sc.positions, sc.log_scales, quats.cpu().numpy(), cand, off,
-                                       freq.cpu().numpy(), att.cpu().numpy(), *sc.mlp(), W, H, 8, 8, thr, **fkw)
-        cpu_s = time.perf_counter() - tc
+        views_np, proj_np = views.cpu().numpy(), proj.cpu().numpy()
+        tv_np = None if tv is None else tv.cpu().numpy()
+        runs, budget_s, res = [], 30.0, None
+        while len(runs) < 3 and (not runs or sum(runs) + runs[-1] <= budget_s):
+            tc = time.perf_counter()
+            cand, off = oracle.bin_legacy(sc.positions, sc.log_scales, views_np, proj_np, W, H, 8, thr, tile_view_ids=tv_np)
+            res = oracle.render_tilecenter(ro_np, rd, sc.positions, sc.log_scales, quats.cpu().numpy(), cand, off,
+                                           freq.cpu().numpy(), att.cpu().numpy(), *sc.mlp(), W, H, 8, 8, thr, **fkw)
+            runs.append(time.perf_counter() - tc)
+        cpu_s = float(np.median(runs))
         gpu_rgb = render(0).cpu().numpy()
         out["cpu_baseline"] = {"value": round(1.0 / cpu_s, 4), "unit": "frames/s", "cores": oracle.num_threads(),
-                               "kind": "port", "sample": "1 full frame (pose 0) of the same workload: binning + "
+                               "kind": "port",
+                               "sample": f"median of {len(runs)} full frame(s) (pose 0) of the same workload: binning + "
                                "per-tile sort + f32 render" + (" with the feature channel" if feature_dim else "") +
                                ", OpenMP over tiles",
-                               "ms_per_frame": round(cpu_s * 1e3, 1),
+                               "ms_per_frame": round(cpu_s * 1e3, 1), "runs_ms": [round(r * 1e3, 1) for r in runs],
                                "gpu_vs_cpu_image_max_abs": float(np.abs(gpu_rgb - res["rgb"]).max())}
+        if sc.n * T_tiles <= 300_000_000 and tv is None:
+            # the reference's own culling expression (dense [tiles x primitives] booleans), once, with CPU torch:
+            # the part of its path that is PyTorch and therefore runs on a CPU at all
+            torch.set_num_threads(oracle.num_threads())
+            dense_s, dense_pairs = dense_culling_cpu_torch(torch.from_numpy(sc.positions), torch.from_numpy(sc.log_scales),
+                                                           torch.from_numpy(views_np[0]), torch.from_numpy(proj_np), W, H,
+                                                           8, thr)
+            out["cpu_baseline"]["reference_culling"] = {
+                "kind": "reference culling expression, CPU torch", "ms": round(dense_s * 1e3, 1), "pairs": dense_pairs,
+                "pairs_of_this_build": int(cand.size), "threads": torch.get_num_threads(),
+                "sample": "one evaluation of scannet/cumodel.py:994-1070 restated with torch on the CPU (dense overlap "
+                          "matrix, nonzero, argsort, offsets), pose 0"}
     print(json.dumps(out))
     return 0
 

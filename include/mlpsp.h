@@ -475,16 +475,15 @@ int mlpsp_feature_dense_attribute_gradients(const float* grad_feat_dev, const in
  * chip sustains next to the data-sheet peak.  sink_dev: one float, left untouched in practice. */
 int64_t mlpsp_probe_mfma_bf16(int iterations, float* sink_dev, mlpsp_stream_t stream);
 
-/* Measurement aid, no counterpart in the reference: 256 workgroups of 8 wavefronts (two per SIMD) run
- * `iterations` rounds of  mode 0: one 32x32x16 bf16 MFMA,  mode 1: eight independent f32 FMAs,
- * mode 2: the MFMA in one wavefront of every SIMD and the FMAs in the other,  mode 3: two v_sin_f32,
- * mode 4: the MFMA and the eight FMAs, independent of each other, in every wavefront.
- * Timed on the stream, modes 0-2 show whether the matrix pipe and the vector ALU of a SIMD overlap across
- * wavefronts (they do not: mode 2 takes about half the sum of modes 0 and 1, not half their maximum), mode 4
- * how much of an MFMA the following vector instructions of the SAME wavefront hide (about 12 of its 32
- * cycles: mode 4 takes ~0.72 of modes 0 + 1), mode 3 the issue rate of transcendentals.
+/* Measurement aid, no counterpart in the reference: how matrix-core, vector-ALU and transcendental instructions
+ * share a SIMD's issue time.  256 workgroups of 16 wavefronts, one per CU, four wavefronts per SIMD (the render
+ * kernel's occupancy); the wavefront of rank k on its SIMD (hardware id) runs roles[k] for window_us microseconds of
+ * the constant-rate clock: 0 idle, 1 MFMA (16 v_mfma_f32_32x32x16_bf16 per batch, four independent accumulators),
+ * 2 VALU (128 independent v_fma_f32), 3 transcendental (128 v_sin_f32), 4 mixed (16 x one MFMA followed by eight
+ * independent v_fma_f32).  out_dev: 4096 records of 24 bytes {int64 batches, int64 core clocks, int32 role,
+ * int32 simd}, one per wavefront.  Clocks per batch and SIMD = clocks / (batches x wavefronts of that role per SIMD).
  * Returns 0 or an MLPSP_E_* code.  sink_dev: one float, left untouched in practice. */
-int mlpsp_probe_issue(int mode, int iterations, float* sink_dev, mlpsp_stream_t stream);
+int mlpsp_probe_issue(const int32_t roles[4], int window_us, void* out_dev, float* sink_dev, mlpsp_stream_t stream);
 
 #ifdef __cplusplus
 }

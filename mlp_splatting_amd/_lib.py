@@ -67,7 +67,7 @@ SIGNATURES = {
     "mlpsp_render_tilecenter_mfma_feat": (_i, [_vp] * 5 + [_i64, _vp, _vp, _vp, _i, _i, _vp, _i, _i, _f, _f, _i, _i, _f,
                                                _vp, _sz, _vp, _vp, _vp, _vp, _vp, _vp]),
     "mlpsp_probe_mfma_bf16": (_i64, [_i, _vp, _vp]),
-    "mlpsp_probe_issue": (_i, [_i, _i, _vp, _vp]),
+    "mlpsp_probe_issue": (_i, [C.POINTER(C.c_int32), _i, _vp, _vp, _vp]),
     "mlpsp_grouped_vjp": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _f, _i, _vp,
                                _vp]),
     "mlpsp_segment_reduce_rows": (_i64, [_i64]),

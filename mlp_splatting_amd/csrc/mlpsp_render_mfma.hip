@@ -547,50 +547,87 @@ __global__ __launch_bounds__(256) void probe_mfma_bf16_kernel(int iterations, fl
   if (v == 12345.678f) sink[0] = v;      // keeps the accumulations alive; practically never true
 }
 
-// Measurement aid: do matrix-core and vector-ALU instructions of different wavefronts of one SIMD run
-// concurrently?  Workgroups of 8 wavefronts, one per CU, so every SIMD holds two.  mode 0: all wavefronts
-// issue one 32x32x16 bf16 MFMA per iteration (32 cycles of the matrix pipe); mode 1: all issue 8 independent
-// f32 FMAs per iteration (32 cycles of the vector ALU); mode 2: on every SIMD one wavefront does the
-// former and one the latter; mode 3: all issue 2 v_sin_f32 per iteration.  If the two pipes overlapped,
-// mode 2 would take as long as the slower of modes 0 and 1 run with one wavefront per SIMD, i.e. half of
-// their two-wavefront times; it takes about the sum.  mode 4: every wavefront issues the MFMA and then the 8
-// FMAs, independent of each other: ~0.72 of modes 0 + 1 -- vector instructions that FOLLOW an MFMA in the
-// same wavefront do start before it has finished (about 12 of its 32 cycles), which the render kernel's
-// instruction order already uses (operand preparation for the next MFMA sits behind the current one).
-__global__ __launch_bounds__(512) void probe_issue_kernel(int mode, int iterations, float* __restrict__ sink) {
-  const int wave = threadIdx.x >> 6;
-  const bool do_mfma = mode == 0 || (mode == 2 && wave < 4);
-  const bool do_valu = mode == 1 || (mode == 2 && wave >= 4);
+// Measurement aid: how do matrix-core, vector-ALU and transcendental instructions share a SIMD's issue time, inside
+// one wavefront and across the wavefronts of a SIMD?  One workgroup of 16 wavefronts per CU (100 KB of dynamic LDS
+// keeps a second one away): four wavefronts per SIMD, the render kernel's occupancy.  Every wavefront reads the SIMD
+// it landed on from the hardware id register, takes a rank among that SIMD's wavefronts and with it one of the four
+// roles the caller lists, runs the role's instruction batch over and over for a fixed stretch of the constant-rate
+// clock, and reports how many batches it finished and how many core clocks passed.  Roles (instructions per batch):
+//   0 idle   1 MFMA: 16 v_mfma_f32_32x32x16_bf16 on four independent accumulators   2 VALU: 128 independent v_fma_f32
+//   3 transcendental: 128 v_sin_f32   4 mixed: 16 x (one MFMA, then eight v_fma_f32 that do not depend on it)
+// The instructions are inline assembly so that the batches are exactly these sequences.
+struct ProbeOut {
+  long long batches, clocks;
+  int role, simd;
+};
+#define MLPSP_PROBE_MFMA(acc) asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(acc) : "v"(a), "v"(b))
+#define MLPSP_PROBE_FMA(x) asm volatile("v_fma_f32 %0, %0, %1, %2" : "+v"(x) : "v"(m), "v"(c))
+#define MLPSP_PROBE_SIN(x) asm volatile("v_sin_f32 %0, %0" : "+v"(x))
+#define MLPSP_PROBE_8(OP) OP(v[0]); OP(v[1]); OP(v[2]); OP(v[3]); OP(v[4]); OP(v[5]); OP(v[6]); OP(v[7])
+
+template <int ROLE>
+__device__ __noinline__ long long probe_role(unsigned long long ticks, float* sink) {
   u32x4 a = {0x3f803f80u + threadIdx.x, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u}, b = a;
-  f32x16 acc = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  f32x16 acc0, acc1, acc2, acc3;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) acc0[r] = acc1[r] = acc2[r] = acc3[r] = 0.f;
   float v[8];
 #pragma unroll
   for (int k = 0; k < 8; ++k) v[k] = 1e-3f * (float)(threadIdx.x + k);
   const float m = 1.0001f, c = 1e-3f * (float)threadIdx.x;
-  if (do_mfma) {
-    for (int it = 0; it < iterations; ++it) acc = Ops<__bf16>::mfma(a, b, acc);
-  } else if (do_valu) {
-    for (int it = 0; it < iterations; ++it) {
-#pragma unroll
-      for (int k = 0; k < 8; ++k) v[k] = fmaf(v[k], m, c);
-    }
-  } else if (mode == 3) {
-    for (int it = 0; it < iterations; ++it) {
-      v[0] = __builtin_amdgcn_sinf(v[0]);
-      v[1] = __builtin_amdgcn_sinf(v[1]);
+  long long batches = 0;
+  const unsigned long long t0 = wall_clock64();
+  while (wall_clock64() - t0 < ticks) {
+    for (int rep = 0; rep < 4; ++rep) {
+      if constexpr (ROLE == 0) __builtin_amdgcn_s_sleep(64);
+      if constexpr (ROLE == 1)
+        for (int i = 0; i < 4; ++i) { MLPSP_PROBE_MFMA(acc0); MLPSP_PROBE_MFMA(acc1); MLPSP_PROBE_MFMA(acc2); MLPSP_PROBE_MFMA(acc3); }
+      if constexpr (ROLE == 2)
+        for (int i = 0; i < 16; ++i) { MLPSP_PROBE_8(MLPSP_PROBE_FMA); }
+      if constexpr (ROLE == 3)
+        for (int i = 0; i < 16; ++i) { MLPSP_PROBE_8(MLPSP_PROBE_SIN); }
+      if constexpr (ROLE == 4)
+        for (int i = 0; i < 4; ++i) {
+          MLPSP_PROBE_MFMA(acc0); MLPSP_PROBE_8(MLPSP_PROBE_FMA);
+          MLPSP_PROBE_MFMA(acc1); MLPSP_PROBE_8(MLPSP_PROBE_FMA);
+          MLPSP_PROBE_MFMA(acc2); MLPSP_PROBE_8(MLPSP_PROBE_FMA);
+          MLPSP_PROBE_MFMA(acc3); MLPSP_PROBE_8(MLPSP_PROBE_FMA);
+        }
+      ++batches;
     }
   }
-  if (mode == 4) {      // both in every wavefront, independent of each other
-    for (int it = 0; it < iterations; ++it) {
-      acc = Ops<__bf16>::mfma(a, b, acc);
-#pragma unroll
-      for (int k = 0; k < 8; ++k) v[k] = fmaf(v[k], m, c);
-    }
-  }
-  float r = acc[0];
+  asm volatile("s_nop 15\n s_nop 15\n s_nop 15");      // the accumulators are read below: let the last MFMA finish
+  float r = 0.f;
+  if constexpr (ROLE == 1 || ROLE == 4) r = (acc0[0] + acc1[1]) + (acc2[2] + acc3[3]);
 #pragma unroll
   for (int k = 0; k < 8; ++k) r += v[k];
-  if (r == 12345.678f) sink[0] = r;
+  if (r == 12345.678f) *sink = r;      // keeps the work alive; practically never true
+  return batches;
+}
+
+__global__ __launch_bounds__(1024) void probe_issue_kernel(int r0, int r1, int r2, int r3, unsigned long long ticks,
+                                                           ProbeOut* __restrict__ out, float* __restrict__ sink) {
+  __shared__ int s_rank[4];
+  if (threadIdx.x < 4) s_rank[threadIdx.x] = 0;
+  __syncthreads();
+  const int lane = threadIdx.x & 63;
+  const int simd = (int)(__builtin_amdgcn_s_getreg((1 << 11) | (4 << 6) | 4) & 3u);   // HW_ID bits [5:4]
+  int rank = 0;
+  if (lane == 0) rank = atomicAdd(&s_rank[simd], 1);
+  rank = __builtin_amdgcn_readfirstlane(rank) & 3;
+  __syncthreads();
+  const int role = rank == 0 ? r0 : rank == 1 ? r1 : rank == 2 ? r2 : r3;
+  const long long c0 = clock64();
+  long long batches = 0;
+  switch (role) {
+    case 1: batches = probe_role<1>(ticks, sink); break;
+    case 2: batches = probe_role<2>(ticks, sink); break;
+    case 3: batches = probe_role<3>(ticks, sink); break;
+    case 4: batches = probe_role<4>(ticks, sink); break;
+    default: batches = probe_role<0>(ticks, sink); break;
+  }
+  const long long c1 = clock64();
+  if (lane == 0) out[blockIdx.x * 16 + (threadIdx.x >> 6)] = ProbeOut{batches, c1 - c0, role, simd};
 }
 
 }  // namespace mlpsp
@@ -752,9 +789,20 @@ MLPSP_API int64_t mlpsp_probe_mfma_bf16(int iterations, float* sink_dev, mlpsp_s
   return (int64_t)blocks * 4 * iterations * 8 * (2LL * 32 * 32 * 16);   // FLOPs issued
 }
 
-MLPSP_API int mlpsp_probe_issue(int mode, int iterations, float* sink_dev, mlpsp_stream_t stream) {
-  if (mode < 0 || mode > 4 || iterations <= 0 || !sink_dev) return MLPSP_E_ARGUMENT;
-  hipLaunchKernelGGL(probe_issue_kernel, dim3(256), dim3(512), 0, (hipStream_t)stream, mode, iterations, sink_dev);
+MLPSP_API int mlpsp_probe_issue(const int32_t roles[4], int window_us, void* out_dev, float* sink_dev,
+                                mlpsp_stream_t stream) {
+  if (!roles || window_us <= 0 || window_us > 100000 || !out_dev || !sink_dev) return MLPSP_E_ARGUMENT;
+  for (int k = 0; k < 4; ++k)
+    if (roles[k] < 0 || roles[k] > 4) return MLPSP_E_ARGUMENT;
+  int rate_khz = 0;
+  int dev = 0;
+  MLPSP_HIP_TRY(hipGetDevice(&dev));
+  MLPSP_HIP_TRY(hipDeviceGetAttribute(&rate_khz, hipDeviceAttributeWallClockRate, dev));
+  if (rate_khz <= 0) return MLPSP_E_RUNTIME;
+  const unsigned long long ticks = (unsigned long long)rate_khz * (unsigned long long)window_us / 1000ull;
+  MLPSP_HIP_TRY(hipFuncSetAttribute((const void*)probe_issue_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 100 * 1024));
+  hipLaunchKernelGGL(probe_issue_kernel, dim3(256), dim3(1024), 100 * 1024, (hipStream_t)stream, roles[0], roles[1],
+                     roles[2], roles[3], ticks, (ProbeOut*)out_dev, sink_dev);
   MLPSP_LAUNCH_CHECK();
   return MLPSP_OK;
 }
