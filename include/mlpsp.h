@@ -321,6 +321,13 @@ size_t mlpsp_mfma_pack_bytes(int num_primitives);
 int mlpsp_pack_mfma_weights(const float* W1, const float* b1, const float* W2, const float* b2, const float* W3,
                             const float* b3, int num_primitives, int use_bf16, void* packed_dev,
                             mlpsp_stream_t stream);
+/* The same blocks from tensors STORED as fp16 -- the reference's inference export keeps MLP weights, biases and
+ * feature attributes that way (scannet/checkpoints.py:317-381) and widens them to f32 when it loads them
+ * (:299-314); here they are read as they are, with no f32 copy in between.  Every fp16 value is an f32 value, so
+ * the blocks equal those of mlpsp_pack_mfma_weights on the widened tensors bit for bit. */
+int mlpsp_pack_mfma_weights_half(const void* W1, const void* b1, const void* W2, const void* b2, const void* W3,
+                                 const void* b3, int num_primitives, int use_bf16, void* packed_dev,
+                                 mlpsp_stream_t stream);
 int mlpsp_render_tilecenter_mfma(const float* rays_o_dev, const float* rays_d_dev, const void* prim_records_dev,
                                  const int32_t* order_dev, const int32_t* tile_offsets_dev, const float* freq_dev,
                                  const float* att_dev, const void* packed_dev, int num_primitives, int use_bf16,
@@ -343,6 +350,9 @@ int mlpsp_render_tilecenter_mfma(const float* rays_o_dev, const float* rays_d_de
 size_t mlpsp_mfma_feat_pack_bytes(int num_primitives, int feat_slots, int feat_channels);
 int mlpsp_pack_mfma_feat(const float* feat_attr_dev, int num_primitives, int feat_slots, int feat_channels,
                          void* packed_feat_dev, int32_t* status_dev, mlpsp_stream_t stream);
+/* mlpsp_pack_mfma_feat for attributes stored as fp16 [N,S,C] (the inference export): a pure re-ordering. */
+int mlpsp_pack_mfma_feat_half(const void* feat_attr_dev, int num_primitives, int feat_slots, int feat_channels,
+                              void* packed_feat_dev, int32_t* status_dev, mlpsp_stream_t stream);
 int mlpsp_render_tilecenter_mfma_feat(const float* rays_o_dev, const float* rays_d_dev, const void* prim_records_dev,
                                       const int32_t* order_dev, const int32_t* tile_offsets_dev, int64_t num_pairs,
                                       const float* freq_dev, const float* att_dev, const void* packed_dev,

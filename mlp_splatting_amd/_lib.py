@@ -54,6 +54,8 @@ SIGNATURES = {
                                                                         _i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "mlpsp_mfma_pack_bytes": (_sz, [_i]),
     "mlpsp_pack_mfma_weights": (_i, [_vp] * 6 + [_i, _i, _vp, _vp]),
+    "mlpsp_pack_mfma_weights_half": (_i, [_vp] * 6 + [_i, _i, _vp, _vp]),
+    "mlpsp_pack_mfma_feat_half": (_i, [_vp, _i, _i, _i, _vp, _vp, _vp]),
     "mlpsp_render_tilecenter_mfma": (_i, [_vp] * 8 + [_i, _i, _i, _i, _f, _vp, _vp, _vp, _vp, _vp]),
     "mlpsp_mfma_feat_pack_bytes": (_sz, [_i, _i, _i]),
     "mlpsp_pack_mfma_feat": (_i, [_vp, _i, _i, _i, _vp, _vp, _vp]),

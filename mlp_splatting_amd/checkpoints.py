@@ -190,13 +190,27 @@ def load_checkpoint(path):
     return torch.load(path, map_location="cpu", weights_only=True)
 
 
+def half_stored_tensors(state_dict) -> dict:
+    """The tensors of a checkpoint that an inference export stores as float16 (MLP weights, biases, feature
+    attributes; scannet/checkpoints.py:317-381), under their canonical names and exactly as stored."""
+    state = normalize_scene_state_dict(state_dict)
+    return {name: value for name, value in state.items()
+            if name in HALF_STORAGE_OK and torch.is_tensor(value) and value.dtype == torch.float16}
+
+
 def scene_from_checkpoint(checkpoint, device, *, min_points: int = 10, tile_size: int = 8, feature_gating_beta=None,
-                          feature_gating_temp=None, feature_slots: int | None = None, render_precision: str | None = None):
+                          feature_gating_temp=None, feature_slots: int | None = None, render_precision: str | None = None,
+                          keep_half_storage: bool = False):
     """Build the renderer module for a checkpoint (mapping or path), the way the reference's evaluators do
     (scannet/eval_rgb_psnr.py:156-235): dimensions from the tensors, encoding and gating constants from the
     wrapper's ``metadata``, float16-stored tensors widened, ``load_state_dict(strict=False)`` with the benign
     missing buffers, ``camera_mode`` from the metadata, ``eval()``.  ``feature_slots`` re-expresses 4/5-slot
-    features in the other layout first."""
+    features in the other layout first.
+
+    ``keep_half_storage``: the tensors an inference export stores as float16 stay float16 on the device (half the
+    memory of the scene), and the matrix-core render (``render_precision`` "bf16" / "fp16") packs its operand blocks
+    and its fp16 attribute layout straight from them -- the checkpoint's values reach the kernels without an f32
+    copy in between.  All six MLP tensors must be stored that way; the f32 render paths widen per call."""
     from .cumodel import NeuralPrimitiveSceneTileCUDA
     if not isinstance(checkpoint, Mapping):
         checkpoint = load_checkpoint(checkpoint)
@@ -209,11 +223,17 @@ def scene_from_checkpoint(checkpoint, device, *, min_points: int = 10, tile_size
     kind = str(metadata.get("encoding_kind", "attenuated_phase_v1"))
     if kind not in {"attenuated_phase_v1", "fourier_features_v1"}:
         raise ValueError(f"Unsupported checkpoint encoding_kind={kind!r}")
+    stored_half = half_stored_tensors(state) if keep_half_storage else {}
     state = restore_scene_state_dict(state)
     spec = infer_scene_spec(state)
     if feature_slots is not None and spec.feature_slots in (4, 5) and feature_slots != spec.feature_slots:
         state["feat_attr"] = convert_feature_slots(state["feat_attr"], int(feature_slots))
+        stored_half.pop("feat_attr", None)          # re-expressed in f32: no longer the stored tensor
         spec = infer_scene_spec(state)
+    mlp_names = ("W1", "b1", "W2", "b2", "W3", "b3")
+    if stored_half and not all(k in stored_half for k in mlp_names):
+        for k in mlp_names:                         # a mixture of storage types is widened as a whole
+            stored_half.pop(k, None)
     beta = float(metadata.get("feature_gating_beta", 1.5) if feature_gating_beta is None else feature_gating_beta)
     temp = float(metadata.get("feature_gating_temperature", 2.0) if feature_gating_temp is None else feature_gating_temp)
     scene = NeuralPrimitiveSceneTileCUDA(
@@ -228,6 +248,8 @@ def scene_from_checkpoint(checkpoint, device, *, min_points: int = 10, tile_size
         raise RuntimeError(f"Checkpoint is missing required scene tensors: {missing[:10]} (total={len(missing)})")
     if unexpected:
         print(f"[Warn] Unexpected keys while loading scene: {unexpected[:10]} (total={len(unexpected)})")
+    for name, value in stored_half.items():
+        setattr(scene, name, torch.nn.Parameter(value.to(device).contiguous(), requires_grad=False))
     scene.camera_mode = checkpoint_camera_mode(checkpoint)
     scene.checkpoint_metadata = dict(metadata)
     if render_precision is not None:

@@ -25,24 +25,26 @@ namespace mlpsp {
 // ---------------------------------------------------------------------------------------------
 // pack: f32 [N,32,72] [N,32] [N,32,32] [N,32] [N,4,32] [N,4]  ->  N blocks of kPackStride bytes
 // ---------------------------------------------------------------------------------------------
-template <typename T>
-__global__ __launch_bounds__(64) void pack_mfma_weights_kernel(const float* __restrict__ W1, const float* __restrict__ b1,
-                                                               const float* __restrict__ W2, const float* __restrict__ b2,
-                                                               const float* __restrict__ W3, const float* __restrict__ b3,
+// S: the type the six tensors are stored in (float, or _Float16 for an inference export read without widening it first:
+// every fp16 value is an f32 value, so both sources give the same blocks bit for bit).
+template <typename T, typename S>
+__global__ __launch_bounds__(64) void pack_mfma_weights_kernel(const S* __restrict__ W1, const S* __restrict__ b1,
+                                                               const S* __restrict__ W2, const S* __restrict__ b2,
+                                                               const S* __restrict__ W3, const S* __restrict__ b3,
                                                                int N, unsigned char* __restrict__ out) {
   const int p = blockIdx.x;
   if (p >= N) return;
   const int l = threadIdx.x, m = l & 31, g = l >> 5;
   unsigned char* blk = out + (size_t)p * kPackStride;
   // accumulator row m holds hidden unit hidden_unit_of_row(m), for both hidden layers
-  const float* w1 = W1 + (size_t)p * 32 * 72 + hidden_unit_of_row(m) * 72;
-  const float* w2 = W2 + (size_t)p * 32 * 32 + hidden_unit_of_row(m) * 32;
+  const S* w1 = W1 + (size_t)p * 32 * 72 + hidden_unit_of_row(m) * 72;
+  const S* w2 = W2 + (size_t)p * 32 * 32 + hidden_unit_of_row(m) * 32;
   bool bad = false;
   auto pk = [&](float a, float b) {
     bad |= !(__builtin_fabsf(Ops<T>::round_trip(a)) <= Ops<T>::kMax) || !(__builtin_fabsf(Ops<T>::round_trip(b)) <= Ops<T>::kMax);
     return Ops<T>::pack2(a, b);
   };
-  const float bias1 = b1[(size_t)p * 32 + hidden_unit_of_row(m)], bias2 = b2[(size_t)p * 32 + hidden_unit_of_row(m)];
+  const float bias1 = (float)b1[(size_t)p * 32 + hidden_unit_of_row(m)], bias2 = (float)b2[(size_t)p * 32 + hidden_unit_of_row(m)];
   bad |= !(__builtin_fabsf(Ops<T>::round_trip(bias1)) <= Ops<T>::kMax) || !(__builtin_fabsf(Ops<T>::round_trip(bias2)) <= Ops<T>::kMax);
   for (int s = 0; s < 5; ++s) {
     u32x4 v;
@@ -51,8 +53,8 @@ __global__ __launch_bounds__(64) void pack_mfma_weights_kernel(const float* __re
       float ws = 0.f, wc = 0.f;
       if (t < 18) {
         const int j = (t / 3) * 6 + 3 * g + (t % 3);
-        ws = w1[j];
-        wc = w1[36 + j];
+        ws = (float)w1[j];
+        wc = (float)w1[36 + j];
       }
       v[d] = pk(ws, wc);
       if (t == 18 && g == 0) v[d] = bias_word<T>(bias1);     // multiplied by the constant (1, 1) operand word
@@ -61,19 +63,19 @@ __global__ __launch_bounds__(64) void pack_mfma_weights_kernel(const float* __re
   }
   for (int s = 0; s < 2; ++s) {
     u32x4 v;
-    for (int d = 0; d < 4; ++d) v[d] = pk(w2[hidden_unit(8 * s + 2 * d, g)], w2[hidden_unit(8 * s + 2 * d + 1, g)]);
+    for (int d = 0; d < 4; ++d) v[d] = pk((float)w2[hidden_unit(8 * s + 2 * d, g)], (float)w2[hidden_unit(8 * s + 2 * d + 1, g)]);
     *reinterpret_cast<u32x4*>(blk + kOffW2 + s * 1024 + l * 16) = v;
   }
   reinterpret_cast<unsigned*>(blk + kOffB2)[l] = (g == 0) ? bias_word<T>(bias2) : 0u;
   if (l < 16) {
     const int row = l & 3, gg = (l >> 2) & 1, s = l >> 3;
-    const float* w3 = W3 + (size_t)p * 4 * 32 + row * 32;
+    const S* w3 = W3 + (size_t)p * 4 * 32 + row * 32;
     u32x4 v;
-    for (int d = 0; d < 4; ++d) v[d] = pk(w3[hidden_unit(8 * s + 2 * d, gg)], w3[hidden_unit(8 * s + 2 * d + 1, gg)]);
+    for (int d = 0; d < 4; ++d) v[d] = pk((float)w3[hidden_unit(8 * s + 2 * d, gg)], (float)w3[hidden_unit(8 * s + 2 * d + 1, gg)]);
     *reinterpret_cast<u32x4*>(blk + kOffW3 + ((s * 2 + gg) * 4 + row) * 16) = v;
   }
   if (l < 4) {
-    const float v3 = b3[(size_t)p * 4 + l];
+    const float v3 = (float)b3[(size_t)p * 4 + l];
     bad |= !(__builtin_fabsf(v3) <= 3.4028235e38f);
     reinterpret_cast<float*>(blk + kOffB3)[l] = v3;
   }
@@ -378,8 +380,8 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(MLPSP_EXP_WA
 // these attributes as fp16 too, scannet/cumodel.py:317-381), the SP slot values of one (primitive, channel)
 // contiguous (slot order as the coefficient records above, zero padded).  flag[0] = 1 if a rounded value
 // is not finite.
-template <int SP>
-__global__ __launch_bounds__(256) void pack_feat_kernel(const float* __restrict__ attr, int N, int S, int C,
+template <int SP, typename SRC>
+__global__ __launch_bounds__(256) void pack_feat_kernel(const SRC* __restrict__ attr, int N, int S, int C,
                                                         unsigned* __restrict__ out, int32_t* __restrict__ flag) {
   const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
   if (idx >= (size_t)N * C) return;
@@ -388,7 +390,7 @@ __global__ __launch_bounds__(256) void pack_feat_kernel(const float* __restrict_
   float v[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
   bool bad = false;
   for (int s = 0; s < S; ++s) {
-    v[s] = attr[(p * S + s) * C + c];
+    v[s] = (float)attr[(p * S + s) * C + c];
     bad |= !(__builtin_fabsf(Ops<_Float16>::round_trip(v[s])) <= Ops<_Float16>::kMax);
   }
 #pragma unroll
@@ -638,22 +640,37 @@ MLPSP_API size_t mlpsp_mfma_pack_bytes(int num_primitives) {
   return num_primitives < 0 ? 0 : (size_t)(num_primitives > 0 ? num_primitives : 1) * kPackStride;
 }
 
-MLPSP_API int mlpsp_pack_mfma_weights(const float* W1, const float* b1, const float* W2, const float* b2,
-                                      const float* W3, const float* b3, int num_primitives, int use_bf16,
-                                      void* packed_dev, mlpsp_stream_t stream) {
+namespace {
+template <typename S>
+int pack_weights_from(const S* W1, const S* b1, const S* W2, const S* b2, const S* W3, const S* b3, int num_primitives,
+                      int use_bf16, void* packed_dev, hipStream_t s) {
   if (num_primitives < 0) return MLPSP_E_ARGUMENT;
   if (num_primitives == 0) return MLPSP_OK;
   if (!W1 || !b1 || !W2 || !b2 || !W3 || !b3 || !packed_dev) return MLPSP_E_ARGUMENT;
   if (reinterpret_cast<uintptr_t>(packed_dev) % 128 != 0) return MLPSP_E_ARGUMENT;
-  hipStream_t s = (hipStream_t)stream;
   if (use_bf16)
-    hipLaunchKernelGGL(pack_mfma_weights_kernel<__bf16>, dim3(num_primitives), dim3(64), 0, s, W1, b1, W2, b2, W3, b3,
-                       num_primitives, (unsigned char*)packed_dev);
+    hipLaunchKernelGGL((pack_mfma_weights_kernel<__bf16, S>), dim3(num_primitives), dim3(64), 0, s, W1, b1, W2, b2, W3,
+                       b3, num_primitives, (unsigned char*)packed_dev);
   else
-    hipLaunchKernelGGL(pack_mfma_weights_kernel<_Float16>, dim3(num_primitives), dim3(64), 0, s, W1, b1, W2, b2, W3, b3,
-                       num_primitives, (unsigned char*)packed_dev);
+    hipLaunchKernelGGL((pack_mfma_weights_kernel<_Float16, S>), dim3(num_primitives), dim3(64), 0, s, W1, b1, W2, b2, W3,
+                       b3, num_primitives, (unsigned char*)packed_dev);
   MLPSP_LAUNCH_CHECK();
   return MLPSP_OK;
+}
+}  // namespace
+
+MLPSP_API int mlpsp_pack_mfma_weights(const float* W1, const float* b1, const float* W2, const float* b2,
+                                      const float* W3, const float* b3, int num_primitives, int use_bf16,
+                                      void* packed_dev, mlpsp_stream_t stream) {
+  return pack_weights_from<float>(W1, b1, W2, b2, W3, b3, num_primitives, use_bf16, packed_dev, (hipStream_t)stream);
+}
+
+MLPSP_API int mlpsp_pack_mfma_weights_half(const void* W1, const void* b1, const void* W2, const void* b2,
+                                           const void* W3, const void* b3, int num_primitives, int use_bf16,
+                                           void* packed_dev, mlpsp_stream_t stream) {
+  typedef const _Float16* H;
+  return pack_weights_from<_Float16>((H)W1, (H)b1, (H)W2, (H)b2, (H)W3, (H)b3, num_primitives, use_bf16, packed_dev,
+                                     (hipStream_t)stream);
 }
 
 namespace {
@@ -677,25 +694,41 @@ MLPSP_API size_t mlpsp_mfma_feat_pack_bytes(int num_primitives, int feat_slots, 
   return align256((size_t)(num_primitives > 0 ? num_primitives : 1) * feat_channels * feat_pad(feat_slots) * 2);
 }
 
-MLPSP_API int mlpsp_pack_mfma_feat(const float* feat_attr_dev, int num_primitives, int feat_slots, int feat_channels,
-                                   void* packed_feat_dev, int32_t* status_dev, mlpsp_stream_t stream) {
+namespace {
+template <typename S>
+int pack_feat_from(const S* feat_attr_dev, int num_primitives, int feat_slots, int feat_channels, void* packed_feat_dev,
+                   int32_t* status_dev, hipStream_t s) {
   if (num_primitives < 0 || feat_channels <= 0 || feat_channels > 512 ||
       !(feat_slots == 1 || feat_slots == 4 || feat_slots == 5) || !status_dev)
     return MLPSP_E_ARGUMENT;
-  hipStream_t s = (hipStream_t)stream;
   MLPSP_HIP_TRY(hipMemsetAsync(status_dev, 0, sizeof(int32_t), s));
   if (num_primitives == 0) return MLPSP_OK;
   if (!feat_attr_dev || !packed_feat_dev || reinterpret_cast<uintptr_t>(packed_feat_dev) % 16 != 0) return MLPSP_E_ARGUMENT;
   const size_t total = (size_t)num_primitives * feat_channels;
   const dim3 grid((unsigned)((total + 255) / 256)), block(256);
   unsigned* out = (unsigned*)packed_feat_dev;
-#define MLPSP_PACK_FEAT(SP) \
-  hipLaunchKernelGGL((pack_feat_kernel<SP>), grid, block, 0, s, feat_attr_dev, num_primitives, feat_slots, feat_channels, out, status_dev)
-  if (feat_pad(feat_slots) == 4) MLPSP_PACK_FEAT(4);
-  else MLPSP_PACK_FEAT(8);
-#undef MLPSP_PACK_FEAT
+  if (feat_pad(feat_slots) == 4)
+    hipLaunchKernelGGL((pack_feat_kernel<4, S>), grid, block, 0, s, feat_attr_dev, num_primitives, feat_slots,
+                       feat_channels, out, status_dev);
+  else
+    hipLaunchKernelGGL((pack_feat_kernel<8, S>), grid, block, 0, s, feat_attr_dev, num_primitives, feat_slots,
+                       feat_channels, out, status_dev);
   MLPSP_LAUNCH_CHECK();
   return MLPSP_OK;
+}
+}  // namespace
+
+MLPSP_API int mlpsp_pack_mfma_feat(const float* feat_attr_dev, int num_primitives, int feat_slots, int feat_channels,
+                                   void* packed_feat_dev, int32_t* status_dev, mlpsp_stream_t stream) {
+  return pack_feat_from<float>(feat_attr_dev, num_primitives, feat_slots, feat_channels, packed_feat_dev, status_dev,
+                               (hipStream_t)stream);
+}
+
+MLPSP_API int mlpsp_pack_mfma_feat_half(const void* feat_attr_dev, int num_primitives, int feat_slots,
+                                        int feat_channels, void* packed_feat_dev, int32_t* status_dev,
+                                        mlpsp_stream_t stream) {
+  return pack_feat_from<_Float16>((const _Float16*)feat_attr_dev, num_primitives, feat_slots, feat_channels,
+                                  packed_feat_dev, status_dev, (hipStream_t)stream);
 }
 
 MLPSP_API int mlpsp_render_tilecenter_mfma_feat(const float* rays_o_dev, const float* rays_d_dev,

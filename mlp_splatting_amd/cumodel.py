@@ -678,8 +678,10 @@ class NeuralPrimitiveSceneTileCUDA(nn.Module):
                 if return_feature and self.feat_attr is None:
                     raise RuntimeError("return_feature=True requested but feat_attr is not initialized.")
                 return rgb
-            feat_args = (self.feat_attr.detach().contiguous(), float(self.feature_gating_beta),
-                         float(self.feature_gating_temp))
+            feat_attr = self.feat_attr.detach()
+            if not matrix_cores and feat_attr.dtype != torch.float32:
+                feat_attr = feat_attr.float()          # fp16-stored attributes: only the matrix-core path reads them as they are
+            feat_args = (feat_attr.contiguous(), float(self.feature_gating_beta), float(self.feature_gating_temp))
             if matrix_cores:
                 rgb, alpha, feat = ext.render_tiles_rgb_wmma_with_feat(list(base), *feat_args, int(W), int(H),
                                                                        float(score_threshold), precision == "bf16")
@@ -780,8 +782,9 @@ class NeuralPrimitiveSceneTileCUDA(nn.Module):
         W, H = self.image_size
         freq, att = self._frequency_tables(device)
         ws = [p.detach().contiguous() for p in (self.W1, self.b1, self.W2, self.b2, self.W3, self.b3)]
-        if any(w.dtype != torch.float32 for w in ws):
-            return None                       # stored half-precision weights take the step-by-step path
+        half = all(w.dtype == torch.float16 for w in ws)
+        if any(w.dtype != torch.float32 for w in ws) and not (half and precision != "f32"):
+            return None                       # stored half-precision weights: only the matrix-core frame reads them as they are
         out = ext.render_frame_queued(ray_o.contiguous(), unit_dirs, self.positions.detach().contiguous(),
                                       self.log_scales.detach().contiguous(), self._unit_quats(), freq, att, ws,
                                       _host_matrix(view_matrix).reshape(1, 4, 4), _host_matrix(proj_matrix), int(W),

@@ -303,9 +303,11 @@ def training_records_mfma(rays_o, rays_d, records, order, tile_offsets, freq, at
     return int(status.item()), (rgb, alpha, ids, x6, raw, masks, gates, offsets)
 
 
-def _feat_shape(feat_attr):
-    """(slots, channels) with the reference's checks (np_tile_kernels.cu:6158-6169)."""
-    if not (feat_attr.is_cuda and feat_attr.dtype == torch.float32 and feat_attr.dim() in (2, 3)):
+def _feat_shape(feat_attr, allow_half=False):
+    """(slots, channels) with the reference's checks (np_tile_kernels.cu:6158-6169).  ``allow_half``: attributes
+    stored as fp16 (an inference export) are accepted by the matrix-core path, which reads them as they are."""
+    dtypes = (torch.float32, torch.float16) if allow_half else (torch.float32,)
+    if not (feat_attr.is_cuda and feat_attr.dtype in dtypes and feat_attr.dim() in (2, 3)):
         raise RuntimeError("feat_attr must be a float32 CUDA tensor of 2 or 3 dimensions")
     if feat_attr.dim() == 2:
         slots, ch = 1, feat_attr.shape[1]
@@ -427,10 +429,16 @@ def pack_mfma_weights(W1, b1, W2, b2, W3, b3, bf16=True):
     n = W1.shape[0]
     if tuple(W1.shape[1:]) != (32, 72) or tuple(W2.shape[1:]) != (32, 32) or tuple(W3.shape[1:]) != (4, 32):
         raise RuntimeError("the matrix-core path supports the 72->32->32->4 MLP only")
-    ws = [_f32c(w, "weights") for w in (W1, b1, W2, b2, W3, b3)]
     lib = _lib.load()
     packed = torch.empty(lib.mlpsp_mfma_pack_bytes(n), dtype=torch.uint8, device=W1.device)
-    code = lib.mlpsp_pack_mfma_weights(*[_ptr(w) for w in ws], n, int(bool(bf16)), _ptr(packed), _stream(W1.device))
+    if all(w.is_cuda and w.dtype == torch.float16 for w in (W1, b1, W2, b2, W3, b3)):
+        # stored as fp16 (an inference export): packed straight from that storage, no f32 copy in between
+        ws = [w.contiguous() for w in (W1, b1, W2, b2, W3, b3)]
+        code = lib.mlpsp_pack_mfma_weights_half(*[_ptr(w) for w in ws], n, int(bool(bf16)), _ptr(packed),
+                                                _stream(W1.device))
+    else:
+        ws = [_f32c(w, "weights") for w in (W1, b1, W2, b2, W3, b3)]
+        code = lib.mlpsp_pack_mfma_weights(*[_ptr(w) for w in ws], n, int(bool(bf16)), _ptr(packed), _stream(W1.device))
     _check(code, "mlpsp_pack_mfma_weights")
     return packed
 
@@ -461,13 +469,14 @@ def render_tilecenter_mfma(rays_o, rays_d, records, order, tile_offsets, freq, a
 def pack_mfma_feat(feat_attr):
     """fp16 matrix-core operand copy of the feature attributes -> (packed uint8 tensor, nonfinite flag)."""
     dev = feat_attr.device
-    slots, ch = _feat_shape(feat_attr)
+    slots, ch = _feat_shape(feat_attr, allow_half=True)
     lib = _lib.load()
     n = feat_attr.shape[0]
     packed = torch.empty(lib.mlpsp_mfma_feat_pack_bytes(n, slots, ch), dtype=torch.uint8, device=dev)
     flag = torch.empty(1, dtype=torch.int32, device=dev)
-    _check(lib.mlpsp_pack_mfma_feat(_ptr(feat_attr), n, slots, ch, _ptr(packed), _ptr(flag),
-                                    _stream(dev)), "mlpsp_pack_mfma_feat")
+    entry = lib.mlpsp_pack_mfma_feat_half if feat_attr.dtype == torch.float16 else lib.mlpsp_pack_mfma_feat
+    feat_attr = feat_attr.contiguous()
+    _check(entry(_ptr(feat_attr), n, slots, ch, _ptr(packed), _ptr(flag), _stream(dev)), "mlpsp_pack_mfma_feat")
     return packed, bool(flag.item())
 
 
@@ -480,7 +489,7 @@ def render_tilecenter_mfma_feat(rays_o, rays_d, records, order, tile_offsets, fr
     dev = rays_o.device
     if freq.numel() != 6:
         raise RuntimeError("the matrix-core path supports 6 frequencies only")
-    slots, ch = _feat_shape(feat_attr)
+    slots, ch = _feat_shape(feat_attr, allow_half=True)
     if packed is None:
         packed = pack_mfma_weights(W1, b1, W2, b2, W3, b3, bf16)
     if packed_feat is None:

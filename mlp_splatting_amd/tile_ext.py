@@ -354,8 +354,8 @@ class TileExt:
                 warnings.warn("WMMA operand/activation overflow: rendering this frame with scalar FP32 instead")
                 with self._lock:
                     self._mfma_fallbacks += 1
-                rgb, alpha, _ = ops.render_tilecenter_f32(rays_o, unit_dirs, rec, order, offsets, freq, att, *ws, width,
-                                                          height, 8, 8, threshold)
+                rgb, alpha, _ = ops.render_tilecenter_f32(rays_o, unit_dirs, rec, order, offsets, freq, att,
+                                                          *[w.float() for w in ws], width, height, 8, 8, threshold)
                 _chk(bool(torch.isfinite(rgb).all()) and bool(torch.isfinite(alpha).all()),
                      "Scalar FP32 fallback output is nonfinite")
         return rgb, alpha
@@ -796,10 +796,10 @@ class TileExt:
         """[rgb, alpha, feat]: the matrix-core render with the gated feature channel composited by the
         same weights (feature semantics of np_tile_kernels.cu:6036-6075; the reference's tensor-core
         kernel itself is RGB only)."""
-        _chk(feat_attr.is_cuda and feat_attr.dtype == torch.float32 and feat_attr.dim() in (2, 3),
+        _chk(feat_attr.is_cuda and feat_attr.dtype in (torch.float32, torch.float16) and feat_attr.dim() in (2, 3),
              "feat_attr must be a CUDA float32 tensor with 2 or 3 dimensions")
         _chk(feat_attr.shape[0] == x[2].shape[0], "feat_attr first dimension must match primitive count")
-        ops._feat_shape(feat_attr)
+        ops._feat_shape(feat_attr, allow_half=True)
         return self._rgb_wmma(x, (feat_attr.contiguous(), float(beta), float(temp)), width, height, threshold, bf16,
                               "render_tiles_rgb_wmma_with_feat")
 
@@ -809,9 +809,12 @@ class TileExt:
         _chk(width > 0 and height > 0 and 0.0 < threshold < 1.0)
         _chk(width <= 2147483647 and height <= 2147483647 and width <= 2147483647 // height,
              "WMMA image dimensions exceed int32 pixel indexing")
+        # The six MLP tensors may all be stored as fp16 (an inference export kept as it is on disk: the operand blocks
+        # are then packed straight from that storage); everything else is f32 as in the reference's entry point.
+        half_weights = all(t.dtype == torch.float16 for t in x[9:15])
         for i, t in enumerate(x):
             _chk(t.is_cuda and t.is_contiguous() and t.device == x[0].device)
-            _chk(t.dtype == (torch.int32 if i in (5, 6) else torch.float32))
+            _chk(t.dtype == (torch.int32 if i in (5, 6) else torch.float16 if (half_weights and i >= 9) else torch.float32))
         pixels, n = width * height, x[2].shape[0]
         _chk(tuple(x[0].shape) == (pixels, 3) and x[1].shape == x[0].shape)
         _chk(x[2].dim() == 2 and x[2].shape[1] == 3 and x[3].shape == x[2].shape)
@@ -838,8 +841,9 @@ class TileExt:
                                   "rendering this frame with scalar FP32 instead")
                     with self._lock:
                         self._mfma_fallbacks += 1
-                    return list(ops.render_tilecenter_feat_f32(x[0], x[1], rec, order, x[6], x[7], x[8], *x[9:15],
-                                                               feat[0], feat[1], feat[2], width, height, 8, 8, threshold))
+                    return list(ops.render_tilecenter_feat_f32(x[0], x[1], rec, order, x[6], x[7], x[8],
+                                                               *[w.float() for w in x[9:15]], feat[0].float(), feat[1],
+                                                               feat[2], width, height, 8, 8, threshold))
             if feat is None:
                 rgb, alpha, nonfinite = ops.render_tilecenter_mfma(x[0], x[1], rec, order, x[6], x[7], x[8], *x[9:15],
                                                                    width, height, threshold, bf16=bool(bf16),
@@ -857,11 +861,13 @@ class TileExt:
                 warnings.warn("WMMA operand/activation overflow: rendering this frame with scalar FP32 instead")
                 with self._lock:
                     self._mfma_fallbacks += 1
+                wide = [w.float() for w in x[9:15]]
                 if feat is None:
-                    out = list(ops.render_tilecenter_f32(x[0], x[1], rec, order, x[6], x[7], x[8], *x[9:15], width,
+                    out = list(ops.render_tilecenter_f32(x[0], x[1], rec, order, x[6], x[7], x[8], *wide, width,
                                                          height, 8, 8, threshold))[:2]
                 else:
-                    out = list(ops.render_tilecenter_feat_f32(x[0], x[1], rec, order, x[6], x[7], x[8], *x[9:15],
-                                                              feat[0], feat[1], feat[2], width, height, 8, 8, threshold))
+                    out = list(ops.render_tilecenter_feat_f32(x[0], x[1], rec, order, x[6], x[7], x[8], *wide,
+                                                              feat[0].float(), feat[1], feat[2], width, height, 8, 8,
+                                                              threshold))
                 _chk(all(bool(torch.isfinite(t).all()) for t in out), "Scalar FP32 fallback output is nonfinite")
         return out
