@@ -100,6 +100,7 @@ __global__ __launch_bounds__(256) void validate_tile_lists_kernel(const int32_t*
 // ---------------------------------------------------------------------------------------------
 constexpr int kSortThreads = 256;
 constexpr int kSortMax = MLPSP_TILE_CAPACITY_MAX;
+constexpr int kRankPairsMax = 64 * 1024;   // in-bucket comparisons beyond which the sorting network is used instead
 
 struct TilePyramid {
   float ox, oy, oz;
@@ -116,6 +117,10 @@ __global__ __launch_bounds__(kSortThreads) void sort_tiles_kernel(
   __shared__ TilePyramid s_pyr;
   __shared__ int s_face_ok[4];
   __shared__ int s_origin_ok;
+  __shared__ int s_cnt[kSortThreads], s_off[kSortThreads];
+  __shared__ uint16_t s_perm[kSortMax], s_order[kSortMax];
+  __shared__ uint32_t s_kmin, s_kmax;
+  __shared__ int s_flags, s_pairs;
   const int tile = blockIdx.x;
   const int tid = threadIdx.x;
   const int start = offsets[tile];
@@ -186,10 +191,19 @@ __global__ __launch_bounds__(kSortThreads) void sort_tiles_kernel(
   }
   const int faces = culling ? s_pyr.enabled : 0;
 
-  // ---- keys; survivors are compacted to the front of s_key (the network then sorts only them),
-  //      culled entries are written straight to the end of the tile's output, last one first
+  // ---- keys.  Survivors with an ordinary key are compacted to the front of s_key in list order; survivors
+  //      whose key is the invalid key or larger go to the back of s_key, last slot first (the "late" stream: all
+  //      of them normally carry the invalid key, and a stable sort leaves those in list order after everything
+  //      else); culled entries are written straight to the end of the tile's output, last one first.
   const int wave = tid >> 6, lane = tid & 63;
-  int ns = 0;                                            // survivors so far (block-uniform)
+  const uint32_t invalid_bits = float_to_bits(kInvalidKey);
+  if (tid == 0) {
+    s_kmin = 0xffffffffu;
+    s_kmax = 0u;
+    s_flags = 0;
+    s_pairs = 0;
+  }
+  int nv = 0, nl = 0;                                    // ordinary and late survivors so far (block-uniform)
   int round = 0;
   for (int i0 = 0; i0 < n; i0 += kSortThreads, round ^= 1) {
     const int i = i0 + tid;
@@ -210,8 +224,8 @@ __global__ __launch_bounds__(kSortThreads) void sort_tiles_kernel(
         for (int j = 0; j < 4; ++j) {
           const float nx = s_pyr.n[j][0], ny = s_pyr.n[j][1], nz = s_pyr.n[j][2];
           const float dist = nx * ex + ny * ey + nz * ez;
-          const Vec3 nl = quat_rotate_conj(P.qw, P.qx, P.qy, P.qz, Vec3{nx, ny, nz});
-          const float h2 = P.s2x * (nl.x * nl.x) + P.s2y * (nl.y * nl.y) + P.s2z * (nl.z * nl.z);
+          const Vec3 nl_ = quat_rotate_conj(P.qw, P.qx, P.qy, P.qz, Vec3{nx, ny, nz});
+          const float h2 = P.s2x * (nl_.x * nl_.x) + P.s2y * (nl_.y * nl_.y) + P.s2z * (nl_.z * nl_.z);
           outside |= ((faces >> j) & 1) && (dist < 0.f) && (dist * dist >= cull_r2 * h2);
         }
       }
@@ -220,62 +234,161 @@ __global__ __launch_bounds__(kSortThreads) void sort_tiles_kernel(
         key = !known ? kInvalidKey
                      : (family == MLPSP_KEY_DEPTH) ? key_depth(ox, oy, oz, dx, dy, dz, P) : key_tstar(ox, oy, oz, dx, dy, dz, P);
     }
-    const unsigned long long m = __ballot(keep);
-    if (lane == 0) s_wave_cnt[round][wave] = __popcll(m);
+    const uint32_t kb = float_to_bits(key);
+    const bool late = keep && kb >= invalid_bits;
+    const bool front = keep && !late;
+    const unsigned long long mf = __ballot(front), ml = __ballot(late);
+    if (lane == 0) s_wave_cnt[round][wave] = __popcll(mf) | (__popcll(ml) << 16);
     __syncthreads();                                     // (the two count buffers alternate: one barrier per round)
-    int before = 0, total = 0;
+    int before_f = 0, before_l = 0, total_f = 0, total_l = 0;
 #pragma unroll
     for (int v = 0; v < kSortThreads / 64; ++v) {
       const int c = s_wave_cnt[round][v];
-      before += (v < wave) ? c : 0;
-      total += c;
+      before_f += (v < wave) ? (c & 0xffff) : 0;
+      before_l += (v < wave) ? (c >> 16) : 0;
+      total_f += c & 0xffff;
+      total_l += c >> 16;
     }
-    const int kept_before = ns + before + __popcll(m & ((1ull << lane) - 1ull));
-    if (keep) {
-      s_key[kept_before] = ((unsigned long long)float_to_bits(key) << 32) | (unsigned)i;
+    const unsigned long long below = (1ull << lane) - 1ull;
+    const int f_before = nv + before_f + __popcll(mf & below);
+    const int l_before = nl + before_l + __popcll(ml & below);
+    const unsigned long long entry = ((unsigned long long)kb << 32) | (unsigned)i;
+    if (front) {
+      s_key[f_before] = entry;
+    } else if (late) {
+      s_key[kSortMax - 1 - l_before] = entry;
     } else if (i < n) {
-      const int pos = start + n - 1 - (i - kept_before);
+      const int pos = start + n - 1 - (i - (f_before + l_before));
       sorted_ids[pos] = ~p;
       if (sorted_keys) sorted_keys[pos] = kInvalidKey;
     }
-    ns += total;
+    // range of the ordinary keys (one pair of LDS atomics per wavefront) and whether any late key is not the
+    // invalid key itself
+    if (mf) {
+      uint32_t lo = front ? kb : 0xffffffffu, hi = front ? kb : 0u;
+#pragma unroll
+      for (int d = 32; d > 0; d >>= 1) {
+        lo = min(lo, (uint32_t)__shfl_xor((int)lo, d));
+        hi = max(hi, (uint32_t)__shfl_xor((int)hi, d));
+      }
+      if (lane == 0) {
+        atomicMin(&s_kmin, lo);
+        atomicMax(&s_kmax, hi);
+      }
+    }
+    if (__ballot(late && kb != invalid_bits) && lane == 0) atomicOr(&s_flags, 1);
+    nv += total_f;
+    nl += total_l;
   }
-  int npad = 2;
-  while (npad < ns) npad <<= 1;
-  for (int i = ns + tid; i < npad; i += kSortThreads) s_key[i] = ~0ull;
   __syncthreads();
 
-  // ---- bitonic network.  Thread t of a step handles the pair (lo, lo | j) with lo built from t, so for
-  //      j < 64 the 64 lanes of a wavefront touch only their own 128 consecutive entries: those steps
-  //      need no workgroup barrier, only program order inside the wavefront (LDS operations of one
-  //      wavefront complete in order).  A workgroup barrier separates any step with j >= 64 from its
-  //      neighbours.
-  int prev_j = 64;
-  for (int k = 2; k <= npad; k <<= 1) {
-    for (int j = k >> 1; j > 0; j >>= 1) {
-      if (j >= 64 || prev_j >= 64) __syncthreads();
-      else {
-        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-        __builtin_amdgcn_wave_barrier();
+  // ---- order of the ordinary survivors.  Usual case: a counting pass into 256 buckets that are linear in the
+  //      key bits between the smallest and the largest key (monotone, so bucket order is key order), then every
+  //      entry ranks itself among the entries of its own bucket by its (key, list position) word.  The work of
+  //      that last step is the sum of the squared bucket sizes; when keys pile up in few buckets (or a late key
+  //      is not the invalid key, which the late stream's list order would misplace) the bitonic network below
+  //      sorts instead.
+  const uint32_t kmin = s_kmin;
+  const float bucket_scale = (float)kSortThreads / ((float)(s_kmax - kmin) + 1.f);
+  auto bucket_of = [&](unsigned long long w) {
+    const int b = (int)((float)((uint32_t)(w >> 32) - kmin) * bucket_scale);
+    return b < kSortThreads - 1 ? b : kSortThreads - 1;
+  };
+  bool network = (s_flags & 1) != 0;
+  const bool ranked = !network && nv > 1;
+  if (ranked) {
+    s_cnt[tid] = 0;
+    __syncthreads();
+    for (int i = tid; i < nv; i += kSortThreads) atomicAdd(&s_cnt[bucket_of(s_key[i])], 1);
+    __syncthreads();
+    const int c = s_cnt[tid];
+    int incl = c, pairs = c * c;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const int up = __shfl_up(incl, d);
+      if (lane >= d) incl += up;
+    }
+#pragma unroll
+    for (int d = 32; d > 0; d >>= 1) pairs += __shfl_xor(pairs, d);
+    if (lane == 63) s_wave_cnt[0][wave] = incl;
+    if (lane == 0) atomicAdd(&s_pairs, pairs);
+    __syncthreads();
+    int base = 0;
+#pragma unroll
+    for (int v = 0; v < kSortThreads / 64; ++v) base += (v < wave) ? s_wave_cnt[0][v] : 0;
+    const int excl = base + incl - c;
+    s_off[tid] = excl;
+    s_cnt[tid] = excl;                                   // from here on: the bucket's fill cursor
+    network = s_pairs > kRankPairsMax;
+    __syncthreads();
+    if (!network) {
+      for (int i = tid; i < nv; i += kSortThreads) s_perm[atomicAdd(&s_cnt[bucket_of(s_key[i])], 1)] = (uint16_t)i;
+      __syncthreads();
+      for (int a = tid; a < nv; a += kSortThreads) {
+        const int ia = s_perm[a];
+        const unsigned long long wa = s_key[ia];
+        const int b = bucket_of(wa);
+        const int lo = s_off[b], hi = s_cnt[b];          // the cursor ended at the bucket's end
+        int r = 0;
+        for (int q = lo; q < hi; ++q) r += (s_key[s_perm[q]] < wa) ? 1 : 0;
+        s_order[lo + r] = (uint16_t)ia;
       }
-      prev_j = j;
-      for (int t = tid; t < (npad >> 1); t += kSortThreads) {
-        const int lo = ((t & ~(j - 1)) << 1) | (t & (j - 1));
-        const int hi = lo | j;
-        const unsigned long long a = s_key[lo], b = s_key[hi];
-        const bool ascending = (lo & k) == 0;
-        if ((a > b) == ascending) {
-          s_key[lo] = b;
-          s_key[hi] = a;
+    }
+  }
+  if (network) {
+    // the late entries join the others (through registers: the two regions can overlap)
+    unsigned long long moved[kSortMax / kSortThreads];
+#pragma unroll
+    for (int v = 0; v < kSortMax / kSortThreads; ++v) {
+      const int j = tid + v * kSortThreads;
+      moved[v] = (j < nl) ? s_key[kSortMax - 1 - j] : 0ull;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int v = 0; v < kSortMax / kSortThreads; ++v) {
+      const int j = tid + v * kSortThreads;
+      if (j < nl) s_key[nv + j] = moved[v];
+    }
+    nv += nl;
+    nl = 0;
+    int npad = 2;
+    while (npad < nv) npad <<= 1;
+    for (int i = nv + tid; i < npad; i += kSortThreads) s_key[i] = ~0ull;
+    __syncthreads();
+
+    // Bitonic network.  Thread t of a step handles the pair (lo, lo | j) with lo built from t, so for
+    // j < 64 the 64 lanes of a wavefront touch only their own 128 consecutive entries: those steps
+    // need no workgroup barrier, only program order inside the wavefront (LDS operations of one
+    // wavefront complete in order).  A workgroup barrier separates any step with j >= 64 from its
+    // neighbours.
+    int prev_j = 64;
+    for (int k = 2; k <= npad; k <<= 1) {
+      for (int j = k >> 1; j > 0; j >>= 1) {
+        if (j >= 64 || prev_j >= 64) __syncthreads();
+        else {
+          __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+          __builtin_amdgcn_wave_barrier();
+        }
+        prev_j = j;
+        for (int t = tid; t < (npad >> 1); t += kSortThreads) {
+          const int lo = ((t & ~(j - 1)) << 1) | (t & (j - 1));
+          const int hi = lo | j;
+          const unsigned long long a = s_key[lo], b = s_key[hi];
+          const bool ascending = (lo & k) == 0;
+          if ((a > b) == ascending) {
+            s_key[lo] = b;
+            s_key[hi] = a;
+          }
         }
       }
     }
   }
   __syncthreads();
 
+  const bool through_order = ranked && !network;
   for (int i = tid; i < len; i += kSortThreads) {
-    if (i < ns) {
-      const unsigned long long w = s_key[i];
+    if (i < nv + nl) {
+      const unsigned long long w = (i >= nv) ? s_key[kSortMax - 1 - (i - nv)] : s_key[through_order ? s_order[i] : i];
       sorted_ids[start + i] = cand[start + (int)(w & 0xffffffffu)];
       if (sorted_keys) sorted_keys[start + i] = bits_to_float((uint32_t)(w >> 32));
     } else if (i >= n) {

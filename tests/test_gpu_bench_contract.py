@@ -30,13 +30,18 @@ def test_one_json_line_with_roofline_and_cpu_baseline(device):
     for key in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better", "scaling",
                 "vs_baseline", "dtype", "data", "config", "roofline", "cpu_baseline"):
         assert key in d, key
-    assert d["n_gpus"] == 1 and d["steps"] == 4 and d["warmup"] == 2 and d["higher_is_better"] is True
+    # the timed region is whole passes of --steps until --min-seconds have gone by; "steps" is what was timed
+    assert d["steps_per_pass"] == 4 and d["steps"] >= 4 and d["steps"] % 4 == 0
+    assert d["n_gpus"] == 1 and d["warmup"] == 2 and d["higher_is_better"] is True
     assert d["vs_baseline"] is None and d["data"] == "synthetic" and d["config"]["workload"] == "cfg1_5k_160x120"
     assert d["value"] > 0 and abs(d["ms_per_step"] * d["value"] - 1000.0) < 1.0
     roof = d["roofline"]
     for key in ("bound", "achieved", "peak", "unit", "frac", "traffic"):
         assert key in roof, key
     assert roof["bound"] in ("hbm", "mfma") and roof["peak"] > 0 and abs(roof["frac"] - roof["achieved"] / roof["peak"]) < 1e-4
+    exact = json.loads([l for l in _run("--workload", "cfg1_5k_160x120", "--steps", "4", "--warmup", "1", "--wake-seconds", "0.1",
+                                        "--poses", "4", "--min-seconds", "0").stdout.splitlines() if l.startswith("{")][0])
+    assert exact["steps"] == 4
     cpu = d["cpu_baseline"]
     for key in ("value", "unit", "cores", "kind", "sample"):
         assert key in cpu, key
