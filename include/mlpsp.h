@@ -66,6 +66,11 @@ const char* mlpsp_strerror(int code);
 int mlpsp_prepare_primitives(const float* positions_dev, const float* log_scales_dev, const float* quats_dev,
                              int num_primitives, void* prim_records_dev, mlpsp_stream_t stream);
 
+/* Unit ray directions: unit_dirs[i] = rays_d[i] / max(|rays_d[i]|, 1e-12), bit for bit what
+ * torch.nn.functional.normalize(ray_d, dim=-1) returns on this device (scannet/cumodel.py:1088, 1325, 1498), in one
+ * launch.  rays_d_dev, unit_dirs_dev: num_rays x 3 floats, contiguous; they may be the same buffer. */
+int mlpsp_normalize_rays(const float* rays_d_dev, long long num_rays, float* unit_dirs_dev, mlpsp_stream_t stream);
+
 /* Tile-list validation = validate_tile_candidate_capacity (np_tile_kernels.cu:4485-4589).
  * capacity 0 = no cap (per-pixel and presorted entry points).  status_dev: 2 int32 of device
  * scratch.  BLOCKS: one 8-byte device-to-host copy, then returns the status mask;

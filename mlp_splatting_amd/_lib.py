@@ -28,6 +28,7 @@ SIGNATURES = {
     "mlpsp_version": (_i, []),
     "mlpsp_strerror": (C.c_char_p, [_i]),
     "mlpsp_prepare_primitives": (_i, [_vp, _vp, _vp, _i, _vp, _vp]),
+    "mlpsp_normalize_rays": (_i, [_vp, _i64, _vp, _vp]),
     "mlpsp_validate_tile_lists": (_i, [_vp, _vp, _i, _i, _i, _i, _vp, C.POINTER(C.c_int32), _vp]),
     "mlpsp_bin_scratch_bytes": (_sz, [_i, _i, _i, _i, _i]),
     "mlpsp_bin_legacy_count": (_i, [_vp, _vp, _i, C.POINTER(_f), _i, _vp, C.POINTER(_f), _i, _i, _i, _f, _vp, _sz, _vp,

@@ -79,12 +79,28 @@ __global__ __launch_bounds__(256) void validate_tile_lists_kernel(const int32_t*
   if (invalid) atomicOr(status, 4);
 }
 
+// d / max(|d|, 1e-12) per ray, as torch.nn.functional.normalize(ray_d, dim=-1) rounds it on this device
+// (scannet/cumodel.py:1088): the squares are summed as (x^2 + z^2) + y^2 -- the order of torch's reduction over a
+// last dimension of three -- then an exactly rounded square root and three exactly rounded divisions.  One launch
+// in place of the library's four.
+__global__ __launch_bounds__(256) void normalize_rays_kernel(const float* __restrict__ d, long long n,
+                                                             float* __restrict__ out) {
+  const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const float x = d[i * 3], y = d[i * 3 + 1], z = d[i * 3 + 2];
+  const float den = fmaxf(sqrtf((x * x + z * z) + y * y), 1e-12f);
+  out[i * 3] = x / den;
+  out[i * 3 + 1] = y / den;
+  out[i * 3 + 2] = z / den;
+}
+
 // ---------------------------------------------------------------------------------------------
 // per-tile key + stable sort.  One 256-thread workgroup per tile.  Each candidate becomes the
 // 64-bit word (key bits << 32 | list index): keys are positive floats, whose bit patterns order
 // like their values, and the list index in the low word makes equal keys keep list order, which
-// is what a stable radix sort on the key alone yields.  Bitonic network in LDS on the next power
-// of two, padded with all-ones words.
+// is what a stable radix sort on the key alone yields.  The words are ordered in LDS: normally by a
+// counting pass into 256 key buckets followed by ranking inside each bucket, else (keys piled up in few
+// buckets) by a bitonic network on the next power of two, padded with all-ones words.
 //
 // Optional conservative culling (cull_threshold in (0,1)): a candidate list comes from a bounding
 // circle on screen, and more than half of its entries hit no pixel of the tile -- yet the render
@@ -96,17 +112,11 @@ __global__ __launch_bounds__(256) void validate_tile_lists_kernel(const int32_t*
 // (n.(c-o))^2 >= -2 ln thr * sum_k s_k^2 (R^T n)_k^2, tested with a 2 % margin on the radius, far
 // above f32 rounding.  Such an entry is written as ~id (negative) AFTER the tile's sorted survivors, in
 // reverse list order: the render kernels skip negative ids, so the image is unchanged bit for bit, and only the
-// survivors go through the sorting network.
+// survivors are ordered.
 // ---------------------------------------------------------------------------------------------
 constexpr int kSortThreads = 256;
 constexpr int kSortMax = MLPSP_TILE_CAPACITY_MAX;
 constexpr int kRankPairsMax = 64 * 1024;   // in-bucket comparisons beyond which the sorting network is used instead
-
-struct TilePyramid {
-  float ox, oy, oz;
-  float n[4][3];
-  int enabled;   // bit j: face j usable
-};
 
 __global__ __launch_bounds__(kSortThreads) void sort_tiles_kernel(
     const float* __restrict__ rays_o, const float* __restrict__ rays_d, const PrimRecord* __restrict__ prims,
@@ -114,14 +124,14 @@ __global__ __launch_bounds__(kSortThreads) void sort_tiles_kernel(
     float cull_r2, int num_prims, int32_t* __restrict__ sorted_ids, float* __restrict__ sorted_keys) {
   __shared__ unsigned long long s_key[kSortMax];
   __shared__ int s_wave_cnt[2][kSortThreads / 64];
-  __shared__ TilePyramid s_pyr;
-  __shared__ int s_face_ok[4];
-  __shared__ int s_origin_ok;
+  __shared__ int s_wave_ok[kSortThreads / 64];
   __shared__ int s_cnt[kSortThreads], s_off[kSortThreads];
   __shared__ uint16_t s_perm[kSortMax], s_order[kSortMax];
   __shared__ uint32_t s_kmin, s_kmax;
   __shared__ int s_flags, s_pairs;
-  const int tile = blockIdx.x;
+  // super-blocks of tiles per XCD: the geometry records a tile gathers are mostly those of its neighbours
+  const int tile = superblock_tile(blockIdx.x, g.ntx, g.nty);
+  if (tile < 0) return;
   const int tid = threadIdx.x;
   const int start = offsets[tile];
   const int len = offsets[tile + 1] - start;
@@ -132,70 +142,84 @@ __global__ __launch_bounds__(kSortThreads) void sort_tiles_kernel(
   const float ox = rays_o[pc * 3 + 0], oy = rays_o[pc * 3 + 1], oz = rays_o[pc * 3 + 2];
   const float dx = rays_d[pc * 3 + 0], dy = rays_d[pc * 3 + 1], dz = rays_d[pc * 3 + 2];
 
-  // The first round's candidate id and geometry record are requested before the pyramid phase (two dependent
-  // gathers whose latency then overlaps the corner-ray loads and the barriers below); every round requests the
-  // next round's in the same way.
+  // Every candidate id this thread will handle is requested up front (at most kSortMax / kSortThreads of them),
+  // and the first round's geometry record right behind: their latencies overlap the pyramid phase below, and each
+  // round of the key loop then requests the next round's record.
   // An id outside [0, num_prims) (lists that were never validated) reads record 0, is never culled and sorts last
   // with the invalid key; it is passed on unchanged, and the render kernels skip it.
-  int p_next = (tid < n) ? cand[start + tid] : 0;
-  PrimRecord P_next = prims[((unsigned)p_next < (unsigned)num_prims) ? p_next : 0];
+  constexpr int kRounds = kSortMax / kSortThreads;
+  int my_id[kRounds];
+#pragma unroll
+  for (int r = 0; r < kRounds; ++r) my_id[r] = (tid + r * kSortThreads < n) ? cand[start + tid + r * kSortThreads] : 0;
+  PrimRecord P_next = prims[((unsigned)my_id[0] < (unsigned)num_prims) ? my_id[0] : 0];
 
-  // ---- the tile's ray pyramid (only when culling is requested)
+  // ---- the tile's ray pyramid (only when culling is requested).  Every thread builds the four faces from the
+  //      corner rays for itself (uniform addresses: one broadcast load each), threads then check the tile's rays
+  //      against them, and one barrier combines the verdicts.
   const bool culling = cull_r2 > 0.f;
+  const int wave = tid >> 6, lane = tid & 63;
+  float pox = 0.f, poy = 0.f, poz = 0.f;
+  float pn[4][3] = {};
+  int faces = 0;
   if (culling) {
     const int tx = tile % g.ntx, ty = tile / g.ntx;
     const int x0 = tx * g.TW, y0 = ty * g.TH;
     const int x1 = min(x0 + g.TW, g.W) - 1, y1 = min(y0 + g.TH, g.H) - 1;
-    if (tid < 4) {      // lane j builds face j from corner rays j and j+1
-      const int cx[4] = {x0, x1, x1, x0}, cy[4] = {y0, y0, y1, y1};
-      const int ca = cy[tid] * g.W + cx[tid], cb = cy[(tid + 1) & 3] * g.W + cx[(tid + 1) & 3];
-      const float a0 = rays_d[ca * 3], a1 = rays_d[ca * 3 + 1], a2 = rays_d[ca * 3 + 2];
-      const float b0 = rays_d[cb * 3], b1 = rays_d[cb * 3 + 1], b2 = rays_d[cb * 3 + 2];
-      if (tid == 0) {
-        s_pyr.ox = rays_o[ca * 3 + 0];
-        s_pyr.oy = rays_o[ca * 3 + 1];
-        s_pyr.oz = rays_o[ca * 3 + 2];
-        s_origin_ok = 1;
-      }
-      const float nx = a1 * b2 - a2 * b1, ny = a2 * b0 - a0 * b2, nz = a0 * b1 - a1 * b0;
+    const int corner[4] = {y0 * g.W + x0, y0 * g.W + x1, y1 * g.W + x1, y1 * g.W + x0};
+    float cd[4][3];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int c = 0; c < 3; ++c) cd[j][c] = rays_d[corner[j] * 3 + c];
+    pox = rays_o[corner[0] * 3 + 0];
+    poy = rays_o[corner[0] * 3 + 1];
+    poz = rays_o[corner[0] * 3 + 2];
+    int ok = 0x1f;                                       // bits 0..3: face usable; bit 4: common origin
+    float nlen[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {                        // face j from corner rays j and j+1
+      const float* a = cd[j];
+      const float* b = cd[(j + 1) & 3];
+      const float nx = a[1] * b[2] - a[2] * b[1], ny = a[2] * b[0] - a[0] * b[2], nz = a[0] * b[1] - a[1] * b[0];
       // orient towards the tile-centre ray; a face the centre ray (nearly) lies in is not used
       const float side = nx * dx + ny * dy + nz * dz;
       const float len = sqrtf(nx * nx + ny * ny + nz * nz);
       const float sgn = side < 0.f ? -1.f : 1.f;
-      s_pyr.n[tid][0] = sgn * nx;
-      s_pyr.n[tid][1] = sgn * ny;
-      s_pyr.n[tid][2] = sgn * nz;
-      s_face_ok[tid] = (len > 0.f && fabsf(side) > 1e-4f * len) ? 1 : 0;
+      pn[j][0] = sgn * nx;
+      pn[j][1] = sgn * ny;
+      pn[j][2] = sgn * nz;
+      nlen[j] = sqrtf(pn[j][0] * pn[j][0] + pn[j][1] * pn[j][1] + pn[j][2] * pn[j][2]);
+      if (!(len > 0.f && fabsf(side) > 1e-4f * len)) ok &= ~(1 << j);
     }
-    __syncthreads();
     // every ray of the tile must start at the common origin and lie inside every face used
     for (int k = tid; k < g.TW * g.TH; k += kSortThreads) {
       const int x = x0 + k % g.TW, y = y0 + k / g.TW;
       if (x < g.W && y < g.H) {
         const int pix = y * g.W + x;
-        if (rays_o[pix * 3] != s_pyr.ox || rays_o[pix * 3 + 1] != s_pyr.oy || rays_o[pix * 3 + 2] != s_pyr.oz)
-          s_origin_ok = 0;
+        if (rays_o[pix * 3] != pox || rays_o[pix * 3 + 1] != poy || rays_o[pix * 3 + 2] != poz) ok &= ~0x10;
         const float rx = rays_d[pix * 3], ry = rays_d[pix * 3 + 1], rz = rays_d[pix * 3 + 2];
+#pragma unroll
         for (int j = 0; j < 4; ++j) {
-          const float inside = s_pyr.n[j][0] * rx + s_pyr.n[j][1] * ry + s_pyr.n[j][2] * rz;
-          const float len = sqrtf(s_pyr.n[j][0] * s_pyr.n[j][0] + s_pyr.n[j][1] * s_pyr.n[j][1] +
-                                  s_pyr.n[j][2] * s_pyr.n[j][2]);
-          if (!(inside >= -1e-6f * len)) s_face_ok[j] = 0;
+          const float inside = pn[j][0] * rx + pn[j][1] * ry + pn[j][2] * rz;
+          if (!(inside >= -1e-6f * nlen[j])) ok &= ~(1 << j);
         }
       }
     }
+    int wave_ok = 0;
+#pragma unroll
+    for (int b = 0; b < 5; ++b) wave_ok |= __ballot(!((ok >> b) & 1)) ? 0 : (1 << b);
+    if (lane == 0) s_wave_ok[wave] = wave_ok;
     __syncthreads();
-    if (tid == 0)
-      s_pyr.enabled = s_origin_ok ? (s_face_ok[0] | (s_face_ok[1] << 1) | (s_face_ok[2] << 2) | (s_face_ok[3] << 3)) : 0;
-    __syncthreads();
+    ok = s_wave_ok[0];
+#pragma unroll
+    for (int v = 1; v < kSortThreads / 64; ++v) ok &= s_wave_ok[v];
+    faces = (ok & 0x10) ? (ok & 0xf) : 0;
   }
-  const int faces = culling ? s_pyr.enabled : 0;
 
   // ---- keys.  Survivors with an ordinary key are compacted to the front of s_key in list order; survivors
   //      whose key is the invalid key or larger go to the back of s_key, last slot first (the "late" stream: all
   //      of them normally carry the invalid key, and a stable sort leaves those in list order after everything
   //      else); culled entries are written straight to the end of the tile's output, last one first.
-  const int wave = tid >> 6, lane = tid & 63;
   const uint32_t invalid_bits = float_to_bits(kInvalidKey);
   if (tid == 0) {
     s_kmin = 0xffffffffu;
@@ -204,25 +228,24 @@ __global__ __launch_bounds__(kSortThreads) void sort_tiles_kernel(
     s_pairs = 0;
   }
   int nv = 0, nl = 0;                                    // ordinary and late survivors so far (block-uniform)
-  int round = 0;
-  for (int i0 = 0; i0 < n; i0 += kSortThreads, round ^= 1) {
-    const int i = i0 + tid;
+#pragma unroll
+  for (int r = 0; r < kRounds; ++r) {
+    if (r * kSortThreads >= n) break;
+    const int round = r & 1;
+    const int i = r * kSortThreads + tid;
     bool keep = false, outside = false;
-    int p = 0;
     float key = 0.f;
     const PrimRecord P = P_next;
-    p = p_next;
-    if (i + kSortThreads < n) {
-      p_next = cand[start + i + kSortThreads];
-      P_next = prims[((unsigned)p_next < (unsigned)num_prims) ? p_next : 0];
-    }
+    const int p = my_id[r];
+    if (r + 1 < kRounds && i + kSortThreads < n)
+      P_next = prims[((unsigned)my_id[r + 1] < (unsigned)num_prims) ? my_id[r + 1] : 0];
     const bool known = (unsigned)p < (unsigned)num_prims;
     if (i < n) {
       if (faces && known) {
-        const float ex = P.cx - s_pyr.ox, ey = P.cy - s_pyr.oy, ez = P.cz - s_pyr.oz;
+        const float ex = P.cx - pox, ey = P.cy - poy, ez = P.cz - poz;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-          const float nx = s_pyr.n[j][0], ny = s_pyr.n[j][1], nz = s_pyr.n[j][2];
+          const float nx = pn[j][0], ny = pn[j][1], nz = pn[j][2];
           const float dist = nx * ex + ny * ey + nz * ez;
           const Vec3 nl_ = quat_rotate_conj(P.qw, P.qx, P.qy, P.qz, Vec3{nx, ny, nz});
           const float h2 = P.s2x * (nl_.x * nl_.x) + P.s2y * (nl_.y * nl_.y) + P.s2z * (nl_.z * nl_.z);
@@ -262,9 +285,8 @@ __global__ __launch_bounds__(kSortThreads) void sort_tiles_kernel(
       sorted_ids[pos] = ~p;
       if (sorted_keys) sorted_keys[pos] = kInvalidKey;
     }
-    // range of the ordinary keys (one pair of LDS atomics per wavefront) and whether any late key is not the
-    // invalid key itself
-    if (mf) {
+    // range of the ordinary keys, and whether any late key is not the invalid key itself
+    if (mf) {                                            // (one pair of LDS atomics per wavefront)
       uint32_t lo = front ? kb : 0xffffffffu, hi = front ? kb : 0u;
 #pragma unroll
       for (int d = 32; d > 0; d >>= 1) {
@@ -424,6 +446,18 @@ MLPSP_API const char* mlpsp_strerror(int code) {
   }
 }
 
+MLPSP_API int mlpsp_normalize_rays(const float* rays_d_dev, long long num_rays, float* unit_dirs_dev,
+                                   mlpsp_stream_t stream) {
+  if (num_rays < 0) return MLPSP_E_ARGUMENT;
+  if (num_rays == 0) return MLPSP_OK;
+  if (!rays_d_dev || !unit_dirs_dev) return MLPSP_E_ARGUMENT;
+  if (num_rays > 2147483647LL * 256) return MLPSP_E_ARGUMENT;
+  hipLaunchKernelGGL(normalize_rays_kernel, dim3((unsigned)((num_rays + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
+                     rays_d_dev, num_rays, unit_dirs_dev);
+  MLPSP_LAUNCH_CHECK();
+  return MLPSP_OK;
+}
+
 MLPSP_API int mlpsp_prepare_primitives(const float* positions_dev, const float* log_scales_dev,
                                        const float* quats_dev, int num_primitives, void* prim_records_dev,
                                        mlpsp_stream_t stream) {
@@ -476,7 +510,7 @@ MLPSP_API int mlpsp_sort_tiles(const float* rays_o_dev, const float* rays_d_dev,
   // squared radius of the threshold ellipsoid in units of the scales, with a 2 % margin on the radius
   float cull_r2 = 0.f;
   if (cull_threshold > 0.f && cull_threshold < 1.f) cull_r2 = -2.0f * logf(cull_threshold) * 1.0404f + 1e-6f;
-  hipLaunchKernelGGL(sort_tiles_kernel, dim3((unsigned)T), dim3(kSortThreads), 0, (hipStream_t)stream, rays_o_dev,
+  hipLaunchKernelGGL(sort_tiles_kernel, dim3(superblock_grid(g.ntx, g.nty)), dim3(kSortThreads), 0, (hipStream_t)stream, rays_o_dev,
                      rays_d_dev, (const PrimRecord*)prim_records_dev, candidates_dev, tile_offsets_dev, g, key_family,
                      capacity, cull_r2, num_primitives, sorted_ids_dev, sorted_keys_dev);
   MLPSP_LAUNCH_CHECK();

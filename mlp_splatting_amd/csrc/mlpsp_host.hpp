@@ -37,4 +37,26 @@ inline int64_t checked_num_tiles(int64_t W, int64_t H, int64_t TW, int64_t TH) {
 // [k*per_xcd, (k+1)*per_xcd) of logical work items.
 constexpr int kNumXcd = 8;
 
+// Tile kernels whose neighbouring tiles share most of their primitives use a two-dimensional version of the same
+// idea: the tile grid is cut into super-blocks of kSuperSide x kSuperSide tiles and the super-blocks are dealt to
+// the XCDs in turn, so the (up to) 64 tiles of a super-block run on one L2 while every XCD still gets an equal
+// share of every image region.  Workgroup b belongs to XCD b % 8; it is that XCD's j-th workgroup, j = b / 8, and
+// takes tile j % 64 of the XCD's (j / 64)-th super-block.  Tiles outside the image return -1.
+constexpr int kSuperSide = 8;
+
+inline unsigned superblock_grid(int ntx, int nty) {
+  const int nsb = ((ntx + kSuperSide - 1) / kSuperSide) * ((nty + kSuperSide - 1) / kSuperSide);
+  return (unsigned)(((nsb + kNumXcd - 1) / kNumXcd) * kNumXcd * kSuperSide * kSuperSide);
+}
+
+__device__ __forceinline__ int superblock_tile(unsigned block, int ntx, int nty) {
+  constexpr int SB = kSuperSide;
+  const int nsx = (ntx + SB - 1) / SB, nsy = (nty + SB - 1) / SB;
+  const int xcd = block % kNumXcd, j = block / kNumXcd;
+  const int sb = kNumXcd * (j / (SB * SB)) + xcd, within = j % (SB * SB);
+  if (sb >= nsx * nsy) return -1;
+  const int stx = (sb % nsx) * SB + within % SB, sty = (sb / nsx) * SB + within / SB;
+  return (stx < ntx && sty < nty) ? sty * ntx + stx : -1;
+}
+
 }  // namespace mlpsp

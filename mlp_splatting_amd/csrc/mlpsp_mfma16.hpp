@@ -263,11 +263,7 @@ __device__ __forceinline__ bool mlp_wave_mfma16(const unsigned char* __restrict_
             bw[d] = d8;
           } else if (t < 18) {
             const float rev = xin[t / 3 - 3] * kf[t % 3];
-#ifdef MLPSP_EXP_NOTRANS
-            bw[d] = Ops<T>::pack2(rev, rev + 0.25f);
-#else
             bw[d] = Ops<T>::pack2(__builtin_amdgcn_sinf(rev), __builtin_amdgcn_cosf(rev));
-#endif
           } else if (t == 18) {
             bw[d] = one_word;
           } else {

@@ -205,37 +205,17 @@ __device__ __forceinline__ bool hit_fast(float rox, float roy, float roz, float 
 // Register budget: 128 VGPRs, i.e. four wavefronts per SIMD (a dozen values spill; measured 4.5 % faster
 // than the 146 registers and three wavefronts the compiler picks on its own).
 template <typename T, int SP>
-#ifndef MLPSP_EXP_WAVES
-#define MLPSP_EXP_WAVES 4
-#endif
-__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(MLPSP_EXP_WAVES, MLPSP_EXP_WAVES))) void render_tilecenter_mfma_kernel(
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 4))) void render_tilecenter_mfma_kernel(
     const float* __restrict__ rays_o, const float* __restrict__ rays_d, const PrimRecord* __restrict__ prims,
     const int32_t* __restrict__ order, const int32_t* __restrict__ offsets, const float* __restrict__ freq,
     const float* __restrict__ att, const unsigned char* __restrict__ packed, int N, int W, int H, int ntx,
     int per_xcd, int num_tiles, float thr, float* __restrict__ out_rgb, float* __restrict__ out_alpha,
     int32_t* __restrict__ status, unsigned long long* __restrict__ counters, int slots, float beta, float temp,
     HitPool hp) {
-  // XCD-aware work assignment: XCD k (blockIdx.x % 8) walks tiles [k*per_xcd, (k+1)*per_xcd) in
-  // row-major order, so neighbouring tiles -- which share most primitives -- run together on one L2.
-#ifndef MLPSP_EXP_MAP
-#define MLPSP_EXP_MAP 8
-#endif
-#if MLPSP_EXP_MAP == 0
-  const int tile = (blockIdx.x % kNumXcd) * per_xcd + blockIdx.x / kNumXcd;
-  if (tile >= num_tiles) return;
-#elif MLPSP_EXP_MAP == 1
-  const int tile = blockIdx.x;
-  if (tile >= num_tiles) return;
-#else
-  constexpr int SB = MLPSP_EXP_MAP;            // super-blocks of SB x SB tiles, dealt to the XCDs in turn
-  const int nty = num_tiles / ntx, nsx = (ntx + SB - 1) / SB, nsy = (nty + SB - 1) / SB;
-  const int xcd = blockIdx.x % kNumXcd, j = blockIdx.x / kNumXcd;
-  const int sb = kNumXcd * (j / (SB * SB)) + xcd, within = j % (SB * SB);
-  if (sb >= nsx * nsy) return;
-  const int stx = (sb % nsx) * SB + within % SB, sty = (sb / nsx) * SB + within / SB;
-  if (stx >= ntx || sty >= nty) return;
-  const int tile = sty * ntx + stx;
-#endif
+  // 8x8 super-blocks of tiles dealt to the XCDs in turn: neighbouring tiles, which share most primitives (their
+  // records and weight blocks), run on one L2
+  const int tile = superblock_tile(blockIdx.x, ntx, num_tiles / ntx);
+  if (tile < 0) return;
   const int l = threadIdx.x;
   float kf[3];
   phase_scales(freq, att, l >> 5, kf);
@@ -299,25 +279,13 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(MLPSP_EXP_WA
       if (mask != 0ull) {
         ++n_proc_hit;
         n_hits += __popcll(mask);
-#ifdef MLPSP_EXP_SAMEBLK
-        const unsigned char* __restrict__ blk = packed + (size_t)(p & 7) * kPackStride;
-#else
         const unsigned char* __restrict__ blk = packed + (size_t)p * kPackStride;
-#endif
         bad |= hit && !(__builtin_fabsf((h.dx + h.dy) + h.dz) <= 3.4028235e38f);
         float o[4];
-#ifdef MLPSP_EXP_NOMLP
-        o[0] = h.dx; o[1] = h.dy; o[2] = h.dz; o[3] = h.decay;
-#else
-#ifdef MLPSP_EXP_NOPAIR
-        bad |= mlp_wave_mfma16<T, Ops<T>::kCheckHidden, false>(blk, mask, l, h.dx, h.dy, h.dz, kf, s_dir, o, nullptr);
-#else
         if ((unsigned)mask != 0u && (unsigned)(mask >> 32) != 0u)
           bad |= mlp_pair_mfma16<T, Ops<T>::kCheckHidden>(blk, mask, l, h.dx, h.dy, h.dz, kf, s_dir, o);
         else
           bad |= mlp_wave_mfma16<T, Ops<T>::kCheckHidden, false>(blk, mask, l, h.dx, h.dy, h.dz, kf, s_dir, o, nullptr);
-#endif
-#endif
         float w = 0.f;
         if (hit) {
           bad |= !(max3_abs(o[0], o[1], o[2]) <= 3.4028235e38f) || !(__builtin_fabsf(o[3]) <= 3.4028235e38f);
@@ -763,12 +731,7 @@ MLPSP_API int mlpsp_render_tilecenter_mfma_feat(const float* rays_o_dev, const f
   MLPSP_HIP_TRY(hipMemsetAsync(status_dev, 0, 16 * sizeof(int32_t), s));
   const int per_xcd = (int)((T + kNumXcd - 1) / kNumXcd);
   const int ntx = ceil_div(width, 8);
-#if MLPSP_EXP_MAP >= 2
-  const int nsb = ceil_div(ntx, MLPSP_EXP_MAP) * ceil_div(ceil_div(height, 8), MLPSP_EXP_MAP);
-  const dim3 grid((unsigned)(ceil_div(nsb, kNumXcd) * kNumXcd * MLPSP_EXP_MAP * MLPSP_EXP_MAP));
-#else
-  const dim3 grid((unsigned)(per_xcd * kNumXcd));
-#endif
+  const dim3 grid(superblock_grid(ntx, ceil_div(height, 8)));
   auto* ctr = reinterpret_cast<unsigned long long*>(counters_dev);
   const int sp = feat_slots ? feat_pad(feat_slots) : 0;
 #define MLPSP_MFMA_GO(TT, SP)                                                                                     \

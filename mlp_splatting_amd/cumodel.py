@@ -65,6 +65,16 @@ def _tile_ext_build_config(tile_size=None):
 _host_copies = {}
 
 
+def _unit_directions(ray_d):
+    """``F.normalize(ray_d, dim=-1)`` (scannet/cumodel.py:1088); for float32 rays on the device one libmlpsp_hip
+    launch that returns the same bits."""
+    if ray_d.is_cuda and ray_d.dtype == torch.float32 and ray_d.dim() == 2 and ray_d.shape[1] == 3 \
+            and not ray_d.requires_grad:
+        from . import ops
+        return ops.normalize_rays(ray_d)
+    return F.normalize(ray_d, dim=-1).contiguous()
+
+
 def _host_matrix(t):
     """A float32 host copy of a small device tensor (view / projection matrices), remembered for as long
     as that very tensor object is alive and unmodified: the binning reads its matrices on the host, and a
@@ -603,7 +613,7 @@ class NeuralPrimitiveSceneTileCUDA(nn.Module):
     def _base_args(self, ray_o, ray_d, culled_prim_indices, tile_offsets, device, unit_dirs=None):
         freq, att = self._frequency_tables(device)
         if unit_dirs is None:
-            unit_dirs = F.normalize(ray_d, dim=-1).contiguous()
+            unit_dirs = _unit_directions(ray_d)
         return (ray_o.contiguous(), unit_dirs, self.positions.detach().contiguous(),
                 self.log_scales.detach().contiguous(), self._unit_quats(),
                 culled_prim_indices, tile_offsets.to(torch.int32), freq, att,
@@ -642,7 +652,7 @@ class NeuralPrimitiveSceneTileCUDA(nn.Module):
         with torch.no_grad():
             # queued before the binning, whose pair count is a blocking read-back: the device then has
             # this work to do while the host waits, instead of idling while the host issues it afterwards
-            unit_dirs = F.normalize(ray_d, dim=-1).contiguous()
+            unit_dirs = _unit_directions(ray_d)
             use_tilecenter = self._resolve_tile_order_mode() == "tilecenter"
             ext = self._ensure_tile_ext()
             own_lists = (culled_prim_indices is None and tile_offsets is None and view_matrix is not None
@@ -713,7 +723,7 @@ class NeuralPrimitiveSceneTileCUDA(nn.Module):
             raise ValueError("CSR feature training requires tilecenter8 and direct feature attributes")
         from .record_training import Frame, feature_training_step
         with torch.no_grad():
-            unit_dirs = F.normalize(ray_d, dim=-1).contiguous()
+            unit_dirs = _unit_directions(ray_d)
             culled_prim_indices, tile_offsets = self._tile_lists(
                 ray_o, ray_d, score_threshold, view_matrix, proj_matrix, culled_prim_indices, tile_offsets, device)
             freq, att = self._frequency_tables(device)
@@ -734,7 +744,7 @@ class NeuralPrimitiveSceneTileCUDA(nn.Module):
         W, H = self.image_size
         ts = int(self.tile_size)
         with torch.no_grad():
-            unit_dirs = F.normalize(ray_d, dim=-1).contiguous()
+            unit_dirs = _unit_directions(ray_d)
             culled_prim_indices, tile_offsets = self._tile_lists(
                 ray_o, ray_d, score_threshold, view_matrix, proj_matrix, culled_prim_indices, tile_offsets, device)
             freq, att = self._frequency_tables(device)
@@ -758,7 +768,7 @@ class NeuralPrimitiveSceneTileCUDA(nn.Module):
         W, H = self.image_size
         ts = int(self.tile_size)
         with torch.no_grad():
-            unit_dirs = F.normalize(ray_d, dim=-1).contiguous()
+            unit_dirs = _unit_directions(ray_d)
             culled_prim_indices, tile_offsets = self._tile_lists(
                 ray_o, ray_d, score_threshold, view_matrix, proj_matrix, culled_prim_indices, tile_offsets, device)
             freq, att = self._frequency_tables(device)

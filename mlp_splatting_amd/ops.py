@@ -50,6 +50,17 @@ def prepare_primitives(positions, log_scales, quats):
     return rec
 
 
+def normalize_rays(rays_d):
+    """[B,3] float32 on the device -> unit directions, the bits of ``F.normalize(rays_d, dim=-1)`` in one launch."""
+    rays_d = _f32c(rays_d, "rays_d")
+    if rays_d.dim() != 2 or rays_d.shape[1] != 3:
+        raise ValueError("rays_d must be [B, 3]")
+    out = torch.empty_like(rays_d)
+    code = _lib.load().mlpsp_normalize_rays(_ptr(rays_d), rays_d.shape[0], _ptr(out), _stream(rays_d.device))
+    _check(code, "mlpsp_normalize_rays")
+    return out
+
+
 def validate_tile_lists(candidates, tile_offsets, n_tiles: int, capacity: int, num_primitives: int, path_name: str):
     """Raise the reference's RuntimeError texts (np_tile_kernels.cu:4578-4588) for a bad tile list."""
     for t, nm in ((candidates, "culled_prim_indices"), (tile_offsets, "tile_offsets")):

@@ -96,6 +96,25 @@ def test_raycone_binning_matches_oracle(device, oracle_mod):
         ray_cone_candidates(ro, torch.ones_like(ro), torch.ones(1, 3, device=device), torch.zeros(1, 3, device=device), 8, 8, 8, 0.005)
 
 
+@pytest.mark.parametrize("rays,scale", [(1200 * 680, 1.0), (160 * 120, 1e-4), (999_983, 250.0), (5, 1.0)])
+def test_unit_directions_are_the_bits_of_torch_normalize(device, rays, scale):
+    """The render's ray directions are F.normalize(ray_d, dim=-1) (scannet/cumodel.py:1088); the one-launch kernel
+    must return exactly those bits (its order of summing the squares is the library's), zero and tiny rays included."""
+    from mlp_splatting_amd import ops
+    g = torch.Generator(device="cpu").manual_seed(rays)
+    d = (torch.randn(rays, 3, generator=g) * scale).to(device)
+    d[0] = 0.0                                             # |d| below eps: divided by eps, stays zero
+    if rays > 4:
+        d[1] = torch.tensor([3e-13, -4e-13, 0.0])
+        d[2] = torch.tensor([1e19, 1e19, -1e19])           # squares overflow: inf norm, zero direction
+        d[3] = torch.tensor([1e-23, 2e-23, 2e-23])         # squares underflow
+    want = torch.nn.functional.normalize(d, dim=-1)
+    got = ops.normalize_rays(d)
+    assert torch.equal(got.view(torch.int32), want.view(torch.int32))
+    sliced = torch.randn(64, 6, generator=g).to(device)[:, :3]           # not contiguous: copied first
+    assert torch.equal(ops.normalize_rays(sliced), torch.nn.functional.normalize(sliced, dim=-1))
+
+
 @pytest.mark.parametrize("family", [1, 2])
 def test_sorted_tile_lists_match_oracle_keys_and_order(device, oracle_mod, frame1, family):
     from mlp_splatting_amd import ops
@@ -107,6 +126,52 @@ def test_sorted_tile_lists_match_oracle_keys_and_order(device, oracle_mod, frame
                                fr.W, fr.H, 8, 8, family=family, want_keys=True)
     want_ids, want_keys = oracle_mod.sort_tiles(fr.rays_o, fr.rays_d, sc.positions, sc.log_scales, sc.quats, cand, off,
                                                 fr.W, fr.H, 8, 8, family=family)
+    np.testing.assert_array_equal(ids.cpu().numpy(), want_ids)
+    _assert_bits(keys, want_keys, "sort keys")
+
+
+@pytest.mark.parametrize("case", ["spread", "ties", "behind", "clusters", "beyond_invalid", "two", "capacity"])
+@pytest.mark.parametrize("family", [1, 2])
+def test_sort_is_the_stable_key_order_for_every_key_distribution(device, oracle_mod, case, family):
+    """One 8x8 tile with a hand-made list.  The kernel ranks survivors inside 256 key buckets and falls back to a
+    sorting network when keys pile up in few buckets or a key exceeds the invalid key; each case below steers it
+    down one of those routes, and the result must be the oracle's stable sort by key every time."""
+    from mlp_splatting_amd import ops
+    rng = np.random.default_rng(11)
+    fr = Frame("cfg1_5k_160x120", n=8, width=8, height=8, eye=(0, 0, -2.0), target=(0, 0, 0))
+    n = {"spread": 1500, "ties": 700, "behind": 900, "clusters": 1200, "beyond_invalid": 300, "two": 2, "capacity": 1536}[case]
+    pos = np.zeros((n, 3), np.float32)
+    pos[:, :2] = rng.uniform(-0.05, 0.05, (n, 2))
+    if case in ("spread", "capacity"):
+        pos[:, 2] = rng.uniform(-1.5, 6.0, n)
+    elif case == "ties":
+        pos[:] = (0.01, -0.02, 0.75)                       # every key equal: list order decides
+        pos[n // 2:] = (0.0, 0.0, 1.25)
+    elif case == "behind":
+        pos[:, 2] = np.where(rng.random(n) < 0.5, rng.uniform(-6.0, -2.5, n), rng.uniform(-1.0, 3.0, n))
+    elif case == "clusters":
+        pos[:, 2] = rng.choice([-0.5, 0.8, 0.8000001, 3.0], n) + rng.normal(0, 1e-6, n)
+    elif case == "beyond_invalid":
+        pos[:, 2] = rng.uniform(-1.0, 3.0, n)
+        pos[::5, 2] = rng.uniform(2e30, 9e31, pos[::5].shape[0])     # in front, but farther than the invalid key
+        pos[1::7, 2] = -5.0                                          # behind: the invalid key itself
+    else:
+        pos[:, 2] = (1.0, 0.5)
+    pos = pos.astype(np.float32)
+    log_s = rng.uniform(-3.0, -2.0, (n, 3)).astype(np.float32)
+    quat = rng.normal(size=(n, 4)).astype(np.float32)
+    quat /= np.linalg.norm(quat, axis=1, keepdims=True)
+    cand = rng.permutation(n).astype(np.int32) if case != "capacity" else np.arange(n, dtype=np.int32)
+    cand = np.sort(cand)
+    off = np.array([0, n], np.int32)
+    rec = ops.prepare_primitives(_t(pos, device), _t(log_s, device), _t(quat, device))
+    ids, keys = ops.sort_tiles(_t(fr.rays_o, device), _t(fr.rays_d, device), rec, _t(cand, device), _t(off, device),
+                               8, 8, 8, 8, family=family, want_keys=True)
+    want_ids, want_keys = oracle_mod.sort_tiles(fr.rays_o, fr.rays_d, pos, log_s, quat, cand, off, 8, 8, 8, 8, family=family)
+    if case == "beyond_invalid":
+        assert (want_keys > 1e30).any() and (want_keys == np.float32(1e30)).any()
+    if case == "behind":
+        assert 0.2 < (want_keys == np.float32(1e30)).mean() < 0.8
     np.testing.assert_array_equal(ids.cpu().numpy(), want_ids)
     _assert_bits(keys, want_keys, "sort keys")
 
