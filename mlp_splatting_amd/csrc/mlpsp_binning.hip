@@ -249,10 +249,20 @@ __global__ __launch_bounds__(kBinThreads) void bin_level1_kernel(const float4* _
 // elements: thread t owns elements 4t..4t+3 of every slab, so all loads and stores are coalesced 16-byte
 // accesses and the 8 loads of a pass are independent (one memory latency per pass, and one pass covers
 // 32768 elements).  Thread sums are scanned with wavefront shuffles, wavefront totals through LDS.
+//
+// Optional guard (asynchronous binning, scan of the tile counts): if the level-1 lists overflowed their scratch
+// (all_totals[0] > l1_capacity) or the sum does not fit the caller's candidate buffer, every offset is written as
+// 0 instead and the guard word all_totals[3] is raised, so that the fill, sort and render kernels queued behind
+// find nothing to read or write; counts_out receives (pairs, longest list, level-1 entries, guard).
+struct ScanGuard {
+  long long* all_totals;     // null: no guard
+  long long* counts_out;
+  long long l1_capacity, cand_capacity;
+};
 constexpr int kScanSlabs = 8;
 __global__ __launch_bounds__(1024) void exclusive_scan_kernel(int32_t* __restrict__ data, int n,
                                                               long long* __restrict__ total,
-                                                              long long* __restrict__ largest) {
+                                                              long long* __restrict__ largest, ScanGuard guard) {
   __shared__ long long s_wave[kScanSlabs][16];
   __shared__ int s_wmax[16];
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
@@ -323,12 +333,22 @@ __global__ __launch_bounds__(1024) void exclusive_scan_kernel(int32_t* __restric
   for (int d = 1; d < 64; d <<= 1) mx = max(mx, __shfl_xor(mx, d));
   if (lane == 0) s_wmax[wave] = mx;
   __syncthreads();
+  const bool bad = guard.all_totals && (guard.all_totals[0] > guard.l1_capacity || carry > guard.cand_capacity);
+  if (bad)                                         // (the scan's own stores are behind the barriers above)
+    for (int i = t; i < n; i += 1024) data[i] = 0;
   if (t == 0) {
     int all_max = 0;
     for (int w = 0; w < 16; ++w) all_max = max(all_max, s_wmax[w]);
-    data[n] = (int32_t)carry;
+    data[n] = bad ? 0 : (int32_t)carry;
     *total = carry;
     if (largest) *largest = all_max;
+    if (guard.all_totals) {
+      guard.all_totals[3] = bad ? 1 : 0;
+      guard.counts_out[0] = carry;
+      guard.counts_out[1] = all_max;
+      guard.counts_out[2] = guard.all_totals[0];
+      guard.counts_out[3] = bad ? 1 : 0;
+    }
   }
 }
 
@@ -462,7 +482,7 @@ int enqueue_bin_count(const float* positions_dev, const float* log_scales_dev, i
                       const float* view_matrices_host, int num_views, const int32_t* tile_view_ids_dev,
                       const float* proj_host, int width, int height, int tile, float threshold, const BinGeom& g,
                       const BinScratch& b, int64_t T, int32_t* tile_offsets_dev, hipStream_t s,
-                      bool matrices_in_scratch = false) {
+                      bool matrices_in_scratch = false, ScanGuard guard = ScanGuard{nullptr, nullptr, 0, 0}) {
   const int S = g.nsx * g.nsy;
   // scalar constants in f32, in the order the reference's tensor expressions evaluate them
   const float rm = sqrtf(-2.0f * logf(threshold));
@@ -491,7 +511,7 @@ int enqueue_bin_count(const float* positions_dev, const float* log_scales_dev, i
                      tile_view_ids_dev, b.l1_counts, b.l1_list, b.l1_bounds, b.l1_capacity, b.l1_masks);
   MLPSP_LAUNCH_CHECK();
   hipLaunchKernelGGL(exclusive_scan_kernel, dim3(1), dim3(1024), 0, s, b.l1_counts, S * g.NC, b.totals,
-                     (long long*)nullptr);
+                     (long long*)nullptr, ScanGuard{nullptr, nullptr, 0, 0});
   MLPSP_LAUNCH_CHECK();
   hipLaunchKernelGGL((bin_level1_kernel<true>), dim3(g.NC, ceil_div(S, kBinThreads / 64)), dim3(kBinThreads), 0, s, b.bounds, g,
                      tile_view_ids_dev, b.l1_counts, b.l1_list, b.l1_bounds, b.l1_capacity, b.l1_masks);
@@ -501,7 +521,7 @@ int enqueue_bin_count(const float* positions_dev, const float* log_scales_dev, i
                      (int32_t*)nullptr, b.l2_masks, b.l2_mask_stride);
   MLPSP_LAUNCH_CHECK();
   hipLaunchKernelGGL(exclusive_scan_kernel, dim3(1), dim3(1024), 0, s, tile_offsets_dev, (int)T, b.totals + 1,
-                     b.totals + 2);
+                     b.totals + 2, guard);
   MLPSP_LAUNCH_CHECK();
   return MLPSP_OK;
 }
@@ -519,26 +539,6 @@ int check_bin_args(int64_t T, const float* view_matrices_host, const float* proj
   return MLPSP_OK;
 }
 }  // namespace
-
-namespace mlpsp {
-// After the counting pass of the asynchronous binning: if the level-1 lists overflowed their scratch or the
-// pairs do not fit the caller's candidate buffer, empty every tile list (offsets := 0) and raise the guard
-// word, so that the fill, sort and render kernels queued behind find nothing to read or write.
-__global__ __launch_bounds__(256) void bin_guard_kernel(long long* __restrict__ totals, long long l1_capacity,
-                                                        long long cand_capacity, int32_t* __restrict__ tile_offsets,
-                                                        int num_offsets, long long* __restrict__ counts_out) {
-  const bool bad = totals[0] > l1_capacity || totals[1] > cand_capacity;
-  if (bad)
-    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < num_offsets; i += gridDim.x * blockDim.x) tile_offsets[i] = 0;
-  if (blockIdx.x == 0 && threadIdx.x == 0) {
-    totals[3] = bad ? 1 : 0;
-    counts_out[0] = totals[1];
-    counts_out[1] = totals[2];
-    counts_out[2] = totals[0];
-    counts_out[3] = bad ? 1 : 0;
-  }
-}
-}  // namespace mlpsp
 
 MLPSP_API int mlpsp_bin_legacy_count(const float* positions_dev, const float* log_scales_dev, int num_primitives,
                                      const float* view_matrices_host, int num_views,
@@ -596,11 +596,9 @@ MLPSP_API int mlpsp_bin_legacy_async(const float* positions_dev, const float* lo
   }
   const int erc = enqueue_bin_count(positions_dev, log_scales_dev, num_primitives, view_matrices_host, num_views,
                                     tile_view_ids_dev, proj_host, width, height, tile, threshold, g, b, T,
-                                    tile_offsets_dev, s);
+                                    tile_offsets_dev, s, false,
+                                    ScanGuard{b.totals, (long long*)counts_dev, b.l1_capacity, (long long)cand_capacity});
   if (erc != MLPSP_OK) return erc;
-  hipLaunchKernelGGL(bin_guard_kernel, dim3(64), dim3(256), 0, s, b.totals, b.l1_capacity, (long long)cand_capacity,
-                     tile_offsets_dev, (int)(T + 1), (long long*)counts_dev);
-  MLPSP_LAUNCH_CHECK();
   hipLaunchKernelGGL((bin_level2_kernel<true>), dim3(ceil_div((int)T, kBinThreads / 64)), dim3(kBinThreads), 0, s,
                      b.bounds, g, tile_view_ids_dev, b.l1_counts, b.l1_list, b.l1_bounds, b.l1_capacity, tile_offsets_dev,
                      candidates_dev, b.l2_masks, b.l2_mask_stride, (const long long*)(b.totals + 3));
@@ -716,11 +714,9 @@ MLPSP_API int mlpsp_bin_legacy_async_noalloc(const float* positions_dev, const f
   }
   const int erc = enqueue_bin_count(positions_dev, log_scales_dev, num_primitives, view_matrices_host, num_views,
                                     tile_view_ids_dev, proj_host, width, height, tile, threshold, g, b, T,
-                                    tile_offsets_dev, s, /*matrices_in_scratch=*/true);
+                                    tile_offsets_dev, s, /*matrices_in_scratch=*/true,
+                                    ScanGuard{b.totals, (long long*)counts_dev, b.l1_capacity, (long long)cand_capacity});
   if (erc != MLPSP_OK) return erc;
-  hipLaunchKernelGGL(bin_guard_kernel, dim3(64), dim3(256), 0, s, b.totals, b.l1_capacity, (long long)cand_capacity,
-                     tile_offsets_dev, (int)(T + 1), (long long*)counts_dev);
-  MLPSP_LAUNCH_CHECK();
   hipLaunchKernelGGL((bin_level2_kernel<true>), dim3(ceil_div((int)T, kBinThreads / 64)), dim3(kBinThreads), 0, s,
                      b.bounds, g, tile_view_ids_dev, b.l1_counts, b.l1_list, b.l1_bounds, b.l1_capacity, tile_offsets_dev,
                      candidates_dev, b.l2_masks, b.l2_mask_stride, (const long long*)(b.totals + 3));

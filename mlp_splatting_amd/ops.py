@@ -133,11 +133,12 @@ def bin_legacy(positions, log_scales, view_matrices, proj_matrix, W: int, H: int
 
 
 def bin_legacy_async(positions, log_scales, view_matrices, proj_matrix, W: int, H: int, tile: int, threshold: float,
-                     cand_capacity: int, tile_view_ids=None, scratch_scale: int = 1):
+                     cand_capacity: int, tile_view_ids=None, scratch_scale: int = 1, counts=None):
     """:func:`bin_legacy` without any host synchronisation -> (candidates [cand_capacity], tile_offsets [T+1],
     counts int64 [4] on the device = pairs, longest tile list, level-1 entries, guard).  If guard is set the
     lists are empty: read ``counts`` at the next synchronisation, enlarge ``cand_capacity`` (pairs) or
-    ``scratch_scale`` (level-1 entries) and repeat."""
+    ``scratch_scale`` (level-1 entries) and repeat.  ``counts``: an int64 [4] device tensor to write them to (e.g. a
+    view of a buffer that is read back in one copy together with other results)."""
     positions, log_scales = _f32c(positions, "positions"), _f32c(log_scales, "log_scales")
     dev = positions.device
     vm = view_matrices.detach().to("cpu", torch.float32).reshape(-1, 4, 4).contiguous()
@@ -156,7 +157,10 @@ def bin_legacy_async(positions, log_scales, view_matrices, proj_matrix, W: int, 
         offsets = torch.empty(T + 1, dtype=torch.int32, device=dev)
         cand = torch.empty(int(cand_capacity), dtype=torch.int32, device=dev)
     scratch = torch.empty(nbytes, dtype=torch.uint8, device=dev)
-    counts = torch.empty(4, dtype=torch.int64, device=dev)
+    if counts is None:
+        counts = torch.empty(4, dtype=torch.int64, device=dev)
+    elif not (counts.is_cuda and counts.dtype == torch.int64 and counts.numel() == 4 and counts.is_contiguous()):
+        raise ValueError("counts must be a contiguous int64 [4] tensor on the device")
     code = lib.mlpsp_bin_legacy_async(_ptr(positions), _ptr(log_scales), n, C.cast(vm.data_ptr(), fp), K, _ptr(tv),
                                       C.cast(pm.data_ptr(), fp), W, H, tile, float(threshold), _ptr(scratch), nbytes,
                                       _ptr(offsets), _ptr(cand), int(cand_capacity), _ptr(counts), _stream(dev))
@@ -455,10 +459,11 @@ def pack_mfma_weights(W1, b1, W2, b2, W3, b3, bf16=True):
 
 
 def render_tilecenter_mfma(rays_o, rays_d, records, order, tile_offsets, freq, att, W1, b1, W2, b2, W3, b3, W, H,
-                           threshold, bf16=True, counters=None, packed=None, check=True):
+                           threshold, bf16=True, counters=None, packed=None, check=True, status=None):
     """Matrix-core tile-centre forward (8x8 tiles) -> (rgb, alpha, nonfinite).
 
-    ``nonfinite`` is a bool when ``check`` (one 4-byte readback) or the int32 device flag otherwise.
+    ``nonfinite`` is a bool when ``check`` (one 4-byte readback) or the int32 device flag otherwise.  ``status``: an
+    int32 [16] device tensor for the flag words (word 0 = non-finite), allocated here when omitted.
     """
     dev = rays_o.device
     if freq.numel() != 6:
@@ -468,7 +473,9 @@ def render_tilecenter_mfma(rays_o, rays_d, records, order, tile_offsets, freq, a
     B = W * H
     rgb = torch.empty(B, 3, dtype=torch.float32, device=dev)
     alpha = torch.empty(B, 1, dtype=torch.float32, device=dev)
-    flag = torch.empty(16, dtype=torch.int32, device=dev)
+    flag = status if status is not None else torch.empty(16, dtype=torch.int32, device=dev)
+    if not (flag.is_cuda and flag.dtype == torch.int32 and flag.numel() == 16 and flag.is_contiguous()):
+        raise ValueError("status must be a contiguous int32 [16] tensor on the device")
     code = _lib.load().mlpsp_render_tilecenter_mfma(
         _ptr(rays_o), _ptr(rays_d), _ptr(records), _ptr(order), _ptr(tile_offsets), _ptr(freq), _ptr(att), _ptr(packed),
         W1.shape[0], int(bool(bf16)), W, H, float(threshold), _ptr(rgb), _ptr(alpha), _ptr(flag), _ptr(counters),

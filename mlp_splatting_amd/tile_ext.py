@@ -318,16 +318,22 @@ class TileExt:
         n = positions.shape[0]
         with torch.cuda.device(rays_o.device):
             rec = self._records(positions, log_scales, unit_quats)
+            # counts of the binning (4 x int64) and flag words of the render (16 x int32) share one buffer: the
+            # frame's single read-back is one 96-byte copy
+            tail = torch.empty(96, dtype=torch.uint8, device=rays_o.device)
+            counts, status = tail[:32].view(torch.int64), tail[32:].view(torch.int32)
             cand, offsets, counts = ops.bin_legacy_async(positions, log_scales, view_matrices, proj_matrix, width,
-                                                         height, 8, threshold, cap, scratch_scale=scale)
+                                                         height, 8, threshold, cap, scratch_scale=scale, counts=counts)
             order, _ = ops.sort_tiles(rays_o, unit_dirs, rec, cand, offsets, width, height, 8, 8, _lib.KEY_TSTAR,
                                       self.max_tile_prims, cull_threshold=threshold)
             if precision != "f32":
                 packed = self._packed_weights(list(ws), precision == "bf16")
-                rgb, alpha, flag = ops.render_tilecenter_mfma(rays_o, unit_dirs, rec, order, offsets, freq, att, *ws,
-                                                              width, height, threshold, bf16=(precision == "bf16"),
-                                                              packed=packed, check=False)
-                pairs, longest, l1_entries, guard, nonfinite = torch.cat([counts, flag[:1].to(torch.int64)]).tolist()
+                rgb, alpha, _ = ops.render_tilecenter_mfma(rays_o, unit_dirs, rec, order, offsets, freq, att, *ws,
+                                                           width, height, threshold, bf16=(precision == "bf16"),
+                                                           packed=packed, check=False, status=status)
+                host = tail.cpu().numpy()
+                pairs, longest, l1_entries, guard = (int(v) for v in host[:32].view("int64"))
+                nonfinite = int(host[32:36].view("int32")[0])
             else:
                 rgb, alpha, _ = ops.render_tilecenter_f32(rays_o, unit_dirs, rec, order, offsets, freq, att, *ws, width,
                                                           height, 8, 8, threshold)
