@@ -14,10 +14,10 @@
 #include "mlpsp_mfma16.hpp"
 #include "mlpsp_host.hpp"
 
-// 32-channel accumulator tiles per wavefront of the feature GEMM (2 and 4 measure the same: the kernel moves
-// ~4 GB per frame through L2 and the fabric and is bound there, not by occupancy)
+// 32-channel accumulator tiles per wavefront of the feature GEMM: a block of four wavefronts covers 128 x this many
+// channels of a tile (2: three blocks per CU instead of two, a few percent faster than 4 on 512 channels)
 #ifndef MLPSP_GEMM_NCB
-#define MLPSP_GEMM_NCB 4
+#define MLPSP_GEMM_NCB 2
 #endif
 
 namespace mlpsp {
@@ -368,29 +368,52 @@ __global__ __launch_bounds__(256) void pack_feat_kernel(const SRC* __restrict__ 
 
 // out_feat[pixel, c] = sum over the tile's hit records e and slots s of coef[e, pixel, s] * attr[id_e, c, s]:
 // per tile a [64 pixels] x [K = SP * hits] x [C] product on v_mfma_f32_32x32x16.  One 256-thread block per
-// tile; wavefront v owns channels [128 v, 128 v + 128) as 2 pixel blocks x 4 channel blocks of f32
-// accumulators (NCB = 4).  The records' pool slots and primitive ids are staged in LDS once per block, and
-// the operands of one K-step are loaded while the previous one multiplies.  Pixels are the M operand and channels the N operand, so that an accumulator register
-// holds 32 consecutive channels of one pixel across lanes: every store is a full 128-byte line.
-// K-slot j of lane group g is (record 16/SP * step + g * 8/SP + j / SP, slot j % SP): both operands are
-// plain 8- or 16-byte loads, coalesced over 32 pixels / 32 channels.
+// (tile, slice of 128 NCB channels); wavefront v owns channels [128 v, 128 v + 128) of the slice as 2 pixel blocks
+// x 4 channel blocks of f32 accumulators (NCB = 4).  Pixels are the M operand and channels the N operand, so
+// that an accumulator register holds 32 consecutive channels of one pixel across lanes: every store is a full
+// 128-byte line.
+//
+// The product is bound by the latency of its operand loads, not by the matrix cores (13 K-steps per tile on
+// average, each needing 4 KB of attributes per record from L2), so the operands go through LDS in chunks of
+// kGemmChunk records: all 256 threads request the chunk's attribute rows (the block's channel slice, up to 4 KB per
+// record for 4 slots) and its coefficient records (contiguous in the pool: a pool chunk is kHitChunk records) at
+// once -- ten or more 16-byte loads in flight per thread instead of one K-step's -- then write them to LDS, and
+// after a barrier the wavefronts multiply out of LDS (8-byte or 16-byte reads, lanes on consecutive addresses).
+// Two or three blocks share a CU, so one block's loads overlap another's multiplications and stores.  (Holding the
+// next chunk's loads in registers across the multiplication measured slower: the registers cost a block per CU.)
+// K-slot j of lane group g is (record 16/SP * step + g * 8/SP + j / SP, slot j % SP).
+template <int SP>
+struct GemmChunk {
+  static constexpr int kRecords = 64 / SP;      // 16 records of 4 slots, 8 records of 8: K = 64 per chunk
+};
+
 template <int SP, int NCB>
 __global__ __launch_bounds__(256) void feat_gemm_kernel(const unsigned* __restrict__ attr, HitPool hp,
                                                         const int32_t* __restrict__ offsets, int C, int W, int H,
                                                         int ntx, int per_xcd, int num_tiles,
                                                         float* __restrict__ out_feat) {
-  const int tile = (blockIdx.x % kNumXcd) * per_xcd + blockIdx.x / kNumXcd;
-  if (tile >= num_tiles) return;
+  // super-blocks of 8x8 tiles per XCD, as in the render: the 64 tiles that run together on an XCD are neighbours,
+  // and a primitive's attribute row is fetched into that L2 once for all of them
+  const int tile = superblock_tile(blockIdx.x, ntx, num_tiles / ntx);
+  if (tile < 0) return;
   const int wave = threadIdx.x >> 6, l = threadIdx.x & 63, g = l >> 5, m = l & 31;
-  const int c0 = ((int)blockIdx.y * 4 + wave) * (32 * NCB);
-  const bool active = c0 < C;              // a wavefront without channels still helps staging and meets the barriers
-  const int ncb = active ? min(NCB, (C - c0 + 31) / 32) : 0;
   constexpr int EPL = 8 / SP;         // records per lane group and K-step
   constexpr int STEP = 2 * EPL;       // records per K-step (one MFMA per accumulator tile)
   constexpr int DW = SP / 2;          // dwords per (record, pixel) and per (primitive, channel)
-  constexpr int kStage = 1024;        // records whose pool slot and primitive id are staged in LDS at a time
-  __shared__ int s_slot[kStage];
+  constexpr int R = GemmChunk<SP>::kRecords;
+  constexpr int kSlice = 128 * NCB;   // channels per block
+  constexpr int kRowDw = kSlice * DW; // dwords of one record's attribute row slice in LDS
+  constexpr int kCoefDw = 64 * DW;    // dwords of one coefficient record
+  constexpr int kStage = 512;         // records whose pool slot and primitive id are staged in LDS at a time
+  static_assert(kHitChunk % R == 0, "a chunk of the product lies inside one chunk of the record pool");
+  __shared__ __attribute__((aligned(16))) unsigned s_b[R * kRowDw];
+  __shared__ __attribute__((aligned(16))) unsigned s_a[R * kCoefDw];
+  __shared__ int s_slot[kStage / R];  // pool slot of the first record of each staged chunk
   __shared__ int s_prim[kStage];
+  const int slice0 = (int)blockIdx.y * kSlice;           // first channel of the block
+  const int c0 = slice0 + wave * (32 * NCB);
+  const bool active = c0 < C;              // a wavefront without channels still helps staging and meets the barriers
+  const int ncb = active ? min(NCB, (C - c0 + 31) / 32) : 0;
   const int hits = hp.item_hits[tile];
   const int table_base = (offsets[tile] >> 4) + tile;
   f32x16 acc[2][NCB];
@@ -400,82 +423,104 @@ __global__ __launch_bounds__(256) void feat_gemm_kernel(const unsigned* __restri
     for (int cb = 0; cb < NCB; ++cb)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[pb][cb][r] = 0.f;
-  int ch[NCB];
-#pragma unroll
-  for (int cb = 0; cb < NCB; ++cb) ch[cb] = min(c0 + 32 * cb + m, C - 1);
 
-  // operands of the K-step that starts at staged record e (zero where the list has ended)
-  auto load = [&](int e, int n, u32x4 (&apix)[2], u32x4 (&bch)[NCB]) {
+  // dwords of an attribute row that belong to this block's slice and exist: [0, row_dw)
+  const int row_dw = min(kSlice, C - slice0) * DW;
+  const bool wide = ((C * DW) & 3) == 0;                // rows start on 16-byte boundaries
+  constexpr int kBLoads = R * kRowDw / 4 / 256;          // 16-byte pieces of the chunk's rows per thread
+  constexpr int kALoads = R * kCoefDw / 4 / 256;         // ... of its coefficient records
+  static_assert(kBLoads * 256 * 4 == R * kRowDw && kALoads * 256 * 4 == R * kCoefDw, "whole pieces per thread");
+
+  for (int base = 0; base < hits; base += kStage) {
+    const int n = min(kStage, hits - base);
+    // record -> primitive id (and chunk -> pool slot) once per block, so that the chunk loop below has a single
+    // level of global loads to wait for
+    for (int k = threadIdx.x; k < n; k += 256) {
+      const int rs = hit_slot(hp, table_base, base + k);
+      if ((k & (R - 1)) == 0) s_slot[k / R] = rs;
+      s_prim[k] = hp.hit_ids[rs];
+    }
+    __syncthreads();
+    // requests chunk e0 of the staged records into registers (records past the end of the list as zeros)
+    auto request = [&](int e0, u32x4 (&vb)[kBLoads], u32x4 (&va)[kALoads]) {
+      const int nrec = min(R, n - e0);
 #pragma unroll
-    for (int pb = 0; pb < 2; ++pb) apix[pb] = u32x4{0u, 0u, 0u, 0u};
+      for (int i = 0; i < kBLoads; ++i) {
+        const int piece = threadIdx.x + 256 * i;           // 16-byte piece of the chunk's row slices
+        const int rec = piece / (kRowDw / 4), dw = (piece % (kRowDw / 4)) * 4;
+        vb[i] = u32x4{0u, 0u, 0u, 0u};
+        if (rec < nrec && dw < row_dw) {
+          const unsigned* __restrict__ src = attr + ((size_t)s_prim[e0 + rec] * C + slice0) * DW + dw;
+          if (wide && dw + 3 < row_dw) {
+            vb[i] = *reinterpret_cast<const u32x4*>(src);
+          } else {
 #pragma unroll
-    for (int cb = 0; cb < NCB; ++cb) bch[cb] = u32x4{0u, 0u, 0u, 0u};
+            for (int j = 0; j < 4; ++j)
+              if (dw + j < row_dw) vb[i][j] = src[j];
+          }
+        }
+      }
+      const unsigned* __restrict__ coef =
+          reinterpret_cast<const unsigned*>(hp.records + (size_t)s_slot[e0 / R] * hp.record_bytes);
 #pragma unroll
-    for (int u = 0; u < EPL; ++u) {
-      const int ent = e + g * EPL + u;
-      if (ent < n) {
-        const int rs = s_slot[ent];
-        const size_t prim = (size_t)s_prim[ent];
-        const unsigned* __restrict__ crow = reinterpret_cast<const unsigned*>(hp.records + (size_t)rs * hp.record_bytes) + m * DW;
-        const unsigned* __restrict__ arow = attr + prim * C * DW;
-        if constexpr (SP == 4) {
+      for (int i = 0; i < kALoads; ++i) {
+        const int piece = threadIdx.x + 256 * i;
+        va[i] = (piece / (kCoefDw / 4) < nrec) ? *reinterpret_cast<const u32x4*>(coef + piece * 4) : u32x4{0u, 0u, 0u, 0u};
+      }
+    };
+    for (int e0 = 0; e0 < n; e0 += R) {
+      const int nrec = min(R, n - e0);
+      u32x4 vb[kBLoads], va[kALoads];
+      request(e0, vb, va);
+      // ---- into LDS
 #pragma unroll
-          for (int pb = 0; pb < 2; ++pb) {
-            const uint2 v = *reinterpret_cast<const uint2*>(crow + pb * 32 * DW);
-            apix[pb][2 * u] = v.x;
-            apix[pb][2 * u + 1] = v.y;
+      for (int i = 0; i < kBLoads; ++i) *reinterpret_cast<u32x4*>(&s_b[(threadIdx.x + 256 * i) * 4]) = vb[i];
+#pragma unroll
+      for (int i = 0; i < kALoads; ++i) *reinterpret_cast<u32x4*>(&s_a[(threadIdx.x + 256 * i) * 4]) = va[i];
+      __syncthreads();
+      // ---- multiply
+      if (active) {
+#pragma unroll
+        for (int ks = 0; ks < R / STEP; ++ks) {
+          if (ks * STEP >= nrec) break;
+          u32x4 apix[2], bch[NCB];
+#pragma unroll
+          for (int u = 0; u < EPL; ++u) {
+            const int rec = ks * STEP + g * EPL + u;
+#pragma unroll
+            for (int pb = 0; pb < 2; ++pb) {
+              const unsigned* pa = &s_a[rec * kCoefDw + (pb * 32 + m) * DW];
+              if constexpr (SP == 4) {
+                const uint2 v = *reinterpret_cast<const uint2*>(pa);
+                apix[pb][2 * u] = v.x;
+                apix[pb][2 * u + 1] = v.y;
+              } else {
+                apix[pb] = *reinterpret_cast<const u32x4*>(pa);
+              }
+            }
+#pragma unroll
+            for (int cb = 0; cb < NCB; ++cb) {
+              const unsigned* pbch = &s_b[rec * kRowDw + (wave * (32 * NCB) + 32 * cb + m) * DW];
+              if constexpr (SP == 4) {
+                const uint2 v = *reinterpret_cast<const uint2*>(pbch);
+                bch[cb][2 * u] = v.x;
+                bch[cb][2 * u + 1] = v.y;
+              } else {
+                bch[cb] = *reinterpret_cast<const u32x4*>(pbch);
+              }
+            }
           }
 #pragma unroll
           for (int cb = 0; cb < NCB; ++cb) {
             if (cb < ncb) {
-              const uint2 v = *reinterpret_cast<const uint2*>(arow + (size_t)ch[cb] * DW);
-              bch[cb][2 * u] = v.x;
-              bch[cb][2 * u + 1] = v.y;
+#pragma unroll
+              for (int pb = 0; pb < 2; ++pb) acc[pb][cb] = Ops<_Float16>::mfma(apix[pb], bch[cb], acc[pb][cb]);
             }
           }
-        } else {
-#pragma unroll
-          for (int pb = 0; pb < 2; ++pb) apix[pb] = *reinterpret_cast<const u32x4*>(crow + pb * 32 * DW);
-#pragma unroll
-          for (int cb = 0; cb < NCB; ++cb)
-            if (cb < ncb) bch[cb] = *reinterpret_cast<const u32x4*>(arow + (size_t)ch[cb] * DW);
         }
       }
+      __syncthreads();
     }
-  };
-  auto multiply = [&](const u32x4 (&apix)[2], const u32x4 (&bch)[NCB]) {
-#pragma unroll
-    for (int cb = 0; cb < NCB; ++cb) {
-      if (cb < ncb) {
-#pragma unroll
-        for (int pb = 0; pb < 2; ++pb) acc[pb][cb] = Ops<_Float16>::mfma(apix[pb], bch[cb], acc[pb][cb]);
-      }
-    }
-  };
-
-  for (int base = 0; base < hits; base += kStage) {
-    const int n = min(kStage, hits - base);
-    // record -> (pool slot, primitive id) once per block, so that the K loop below has a single level of
-    // global loads to wait for
-    for (int k = threadIdx.x; k < n; k += 256) {
-      const int rs = hit_slot(hp, table_base, base + k);
-      s_slot[k] = rs;
-      s_prim[k] = hp.hit_ids[rs];
-    }
-    __syncthreads();
-    if (active) {
-      // two operand sets: the loads of one K-step are in flight while the other multiplies
-      u32x4 apA[2], bcA[NCB], apB[2], bcB[NCB];
-      load(0, n, apA, bcA);
-      for (int e = 0; e < n; e += 2 * STEP) {
-        if (e + STEP < n) load(e + STEP, n, apB, bcB);
-        multiply(apA, bcA);
-        if (e + STEP >= n) break;
-        if (e + 2 * STEP < n) load(e + 2 * STEP, n, apA, bcA);
-        multiply(apB, bcB);
-      }
-    }
-    __syncthreads();
   }
   if (!active) return;
 
@@ -750,7 +795,7 @@ MLPSP_API int mlpsp_render_tilecenter_mfma_feat(const float* rays_o_dev, const f
 #undef MLPSP_MFMA_GO
   MLPSP_LAUNCH_CHECK();
   if (sp != 0) {
-    const dim3 ggrid((unsigned)(per_xcd * kNumXcd), (unsigned)ceil_div(feat_channels, 128 * kGemmNcb)), gblock(256);
+    const dim3 ggrid(superblock_grid(ntx, ceil_div(height, 8)), (unsigned)ceil_div(feat_channels, 128 * kGemmNcb)), gblock(256);
 #define MLPSP_FEAT_GEMM(SP)                                                                                       \
   hipLaunchKernelGGL((feat_gemm_kernel<SP, kGemmNcb>), ggrid, gblock, 0, s, (const unsigned*)packed_feat_dev, hp, \
                      tile_offsets_dev, feat_channels, width, height, ntx, per_xcd, (int)T, out_feat_dev)

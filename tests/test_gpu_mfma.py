@@ -125,7 +125,7 @@ def test_scene_module_precision_switch(device, oracle_mod):
         _call(scene, fr, device)
 
 
-@pytest.mark.parametrize("slots,channels", [(4, 200), (5, 512), (1, 36)])
+@pytest.mark.parametrize("slots,channels", [(4, 200), (5, 512), (1, 36), (4, 37), (4, 509), (5, 3)])
 @pytest.mark.parametrize("bf16", [True, False])
 def test_matrix_core_feature_render_against_oracle(device, oracle_mod, bf16, slots, channels):
     # the feature image shares the weights w of the RGB image, so it inherits the same tolerance scaled
