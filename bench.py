@@ -490,6 +490,11 @@ def main() -> int:
                 "pairs_of_this_build": int(cand.size), "threads": torch.get_num_threads(),
                 "sample": "one evaluation of scannet/cumodel.py:994-1070 restated with torch on the CPU (dense overlap "
                           "matrix, nonzero, argsort, offsets), pose 0"}
+        else:
+            out["cpu_baseline"]["reference_culling"] = {
+                "kind": "reference culling expression, CPU torch", "ms": None,
+                "skipped": (f"tiles x primitives = {sc.n * T_tiles:.3g}: the dense overlap matrix is timed only up to 3e8 "
+                            "elements and for one view (run --workload cfg1_5k_160x120 or cfg2_50k_640x480)")}
     print(json.dumps(out))
     return 0
 
