@@ -204,19 +204,15 @@ __device__ __forceinline__ bool hit_fast(float rox, float roy, float roz, float 
 // (feat_gemm_kernel below).
 // Register budget: 128 VGPRs, i.e. four wavefronts per SIMD (a dozen values spill; measured 4.5 % faster
 // than the 146 registers and three wavefronts the compiler picks on its own).
+// One tile, rendered by the calling wavefront (lane l = pixel l of the tile); s_dir: LDS of this wavefront alone.
 template <typename T, int SP>
-__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 4))) void render_tilecenter_mfma_kernel(
-    const float* __restrict__ rays_o, const float* __restrict__ rays_d, const PrimRecord* __restrict__ prims,
-    const int32_t* __restrict__ order, const int32_t* __restrict__ offsets, const float* __restrict__ freq,
-    const float* __restrict__ att, const unsigned char* __restrict__ packed, int N, int W, int H, int ntx,
-    int per_xcd, int num_tiles, float thr, float* __restrict__ out_rgb, float* __restrict__ out_alpha,
+__device__ __forceinline__ void render_tile_mfma(
+    const int tile, const int l, DirWords& s_dir, const float* __restrict__ rays_o, const float* __restrict__ rays_d,
+    const PrimRecord* __restrict__ prims, const int32_t* __restrict__ order, const int32_t* __restrict__ offsets,
+    const float* __restrict__ freq, const float* __restrict__ att, const unsigned char* __restrict__ packed, int N,
+    int W, int H, int ntx, float thr, float* __restrict__ out_rgb, float* __restrict__ out_alpha,
     int32_t* __restrict__ status, unsigned long long* __restrict__ counters, int slots, float beta, float temp,
-    HitPool hp) {
-  // 8x8 super-blocks of tiles dealt to the XCDs in turn: neighbouring tiles, which share most primitives (their
-  // records and weight blocks), run on one L2
-  const int tile = superblock_tile(blockIdx.x, ntx, num_tiles / ntx);
-  if (tile < 0) return;
-  const int l = threadIdx.x;
+    const HitPool& hp) {
   float kf[3];
   phase_scales(freq, att, l >> 5, kf);
   unsigned n_proc = 0, n_proc_hit = 0, n_hits = 0;
@@ -231,8 +227,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 4))) void
               rdz = valid ? rays_d[pix * 3 + 2] : 0.f;
   // The encoding of the ray direction (input components 0..2, operand words 0..8 of both column blocks) does
   // not depend on the primitive: it is computed once per pixel and parked in LDS in operand form -- 18 more
-  // live registers would cost the fourth wavefront per SIMD.  One wavefront per workgroup: no barrier.
-  __shared__ DirWords s_dir;
+  // live registers would cost the fourth wavefront per SIMD.  Written and read by this wavefront only: no barrier.
   encode_direction_words<T>(rdx, rdy, rdz, kf, l, s_dir);
 
   const int start = offsets[tile], end = offsets[tile + 1];
@@ -338,6 +333,23 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 4))) void
     atomicAdd(counters + 2, (unsigned long long)n_proc_hit);
     atomicAdd(counters + 3, (unsigned long long)n_hits);
   }
+}
+
+template <typename T, int SP>
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 4))) void render_tilecenter_mfma_kernel(
+    const float* __restrict__ rays_o, const float* __restrict__ rays_d, const PrimRecord* __restrict__ prims,
+    const int32_t* __restrict__ order, const int32_t* __restrict__ offsets, const float* __restrict__ freq,
+    const float* __restrict__ att, const unsigned char* __restrict__ packed, int N, int W, int H, int ntx,
+    int per_xcd, int num_tiles, float thr, float* __restrict__ out_rgb, float* __restrict__ out_alpha,
+    int32_t* __restrict__ status, unsigned long long* __restrict__ counters, int slots, float beta, float temp,
+    HitPool hp) {
+  // 8x8 super-blocks of tiles dealt to the XCDs in turn: neighbouring tiles, which share most primitives (their
+  // records and weight blocks), run on one L2
+  const int tile = superblock_tile(blockIdx.x, ntx, num_tiles / ntx);
+  if (tile < 0) return;
+  __shared__ DirWords s_dir;
+  render_tile_mfma<T, SP>(tile, (int)threadIdx.x, s_dir, rays_o, rays_d, prims, order, offsets, freq, att, packed, N, W,
+                          H, ntx, thr, out_rgb, out_alpha, status, counters, slots, beta, temp, hp);
 }
 
 // ---------------------------------------------------------------------------------------------
