@@ -169,13 +169,20 @@ __device__ __forceinline__ void sort_one_tile(SortLds<kSortMax>& lds,
     const bool known = (unsigned)p < (unsigned)num_prims;
     if (i < n) {
       if (faces && known) {
+        // (fused multiply-adds here: the test is conservative by a 2 % margin, its roundings are free)
         const float ex = P.cx - pox, ey = P.cy - poy, ez = P.cz - poz;
+        const float qw = P.qw, qx = -P.qx, qy = -P.qy, qz = -P.qz;       // conjugate: world -> local
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           const float nx = pn[j][0], ny = pn[j][1], nz = pn[j][2];
-          const float dist = nx * ex + ny * ey + nz * ez;
-          const Vec3 nl_ = quat_rotate_conj(P.qw, P.qx, P.qy, P.qz, Vec3{nx, ny, nz});
-          const float h2 = P.s2x * (nl_.x * nl_.x) + P.s2y * (nl_.y * nl_.y) + P.s2z * (nl_.z * nl_.z);
+          const float dist = fmaf(nx, ex, fmaf(ny, ey, nz * ez));
+          // R^T n = n + qw t + q x t with t = 2 q x n
+          const float tx = 2.f * fmaf(qy, nz, -(qz * ny)), ty = 2.f * fmaf(qz, nx, -(qx * nz)),
+                      tz = 2.f * fmaf(qx, ny, -(qy * nx));
+          const float lx = fmaf(qw, tx, nx) + fmaf(qy, tz, -(qz * ty));
+          const float ly = fmaf(qw, ty, ny) + fmaf(qz, tx, -(qx * tz));
+          const float lz = fmaf(qw, tz, nz) + fmaf(qx, ty, -(qy * tx));
+          const float h2 = fmaf(P.s2x, lx * lx, fmaf(P.s2y, ly * ly, P.s2z * (lz * lz)));
           outside |= ((faces >> j) & 1) && (dist < 0.f) && (dist * dist >= cull_r2 * h2);
         }
       }
