@@ -78,7 +78,8 @@ __device__ __forceinline__ void sort_one_tile(SortLds<kSortMax>& lds,
   int my_id[kRounds];
 #pragma unroll
   for (int r = 0; r < kRounds; ++r) my_id[r] = (tid + r * kSortThreads < n) ? cand[start + tid + r * kSortThreads] : 0;
-  PrimRecord P_next = prims[((unsigned)my_id[0] < (unsigned)num_prims) ? my_id[0] : 0];
+  PrimRecord P_buf[2];                                   // this round's record and the next round's
+  P_buf[0] = prims[((unsigned)my_id[0] < (unsigned)num_prims) ? my_id[0] : 0];
 
   // ---- the tile's ray pyramid (only when culling is requested).  Every thread builds the four faces from the
   //      corner rays for itself (uniform addresses: one broadcast load each), threads then check the tile's rays
@@ -155,6 +156,8 @@ __device__ __forceinline__ void sort_one_tile(SortLds<kSortMax>& lds,
     s_pairs = 0;
   }
   int nv = 0, nl = 0;                                    // ordinary and late survivors so far (block-uniform)
+  uint32_t key_lo = 0xffffffffu, key_hi = 0u;
+  bool odd_late = false;
 #pragma unroll
   for (int r = 0; r < kRounds; ++r) {
     if (r * kSortThreads >= n) break;
@@ -162,10 +165,10 @@ __device__ __forceinline__ void sort_one_tile(SortLds<kSortMax>& lds,
     const int i = r * kSortThreads + tid;
     bool keep = false, outside = false;
     float key = 0.f;
-    const PrimRecord P = P_next;
+    const PrimRecord& P = P_buf[r & 1];
     const int p = my_id[r];
     if (r + 1 < kRounds && i + kSortThreads < n)
-      P_next = prims[((unsigned)my_id[r + 1] < (unsigned)num_prims) ? my_id[r + 1] : 0];
+      P_buf[(r + 1) & 1] = prims[((unsigned)my_id[r + 1] < (unsigned)num_prims) ? my_id[r + 1] : 0];
     const bool known = (unsigned)p < (unsigned)num_prims;
     if (i < n) {
       if (faces && known) {
@@ -219,22 +222,25 @@ __device__ __forceinline__ void sort_one_tile(SortLds<kSortMax>& lds,
       sorted_ids[pos] = ~p;
       if (sorted_keys) sorted_keys[pos] = kInvalidKey;
     }
-    // range of the ordinary keys, and whether any late key is not the invalid key itself
-    if (mf) {                                            // (one pair of LDS atomics per wavefront)
-      uint32_t lo = front ? kb : 0xffffffffu, hi = front ? kb : 0u;
-#pragma unroll
-      for (int d = 32; d > 0; d >>= 1) {
-        lo = min(lo, (uint32_t)__shfl_xor((int)lo, d));
-        hi = max(hi, (uint32_t)__shfl_xor((int)hi, d));
-      }
-      if (lane == 0) {
-        atomicMin(&s_kmin, lo);
-        atomicMax(&s_kmax, hi);
-      }
-    }
-    if (__ballot(late && kb != invalid_bits) && lane == 0) atomicOr(&s_flags, 1);
+    // range of the ordinary keys (per lane here, combined after the loop), and whether any late key is not the
+    // invalid key itself
+    key_lo = front ? min(key_lo, kb) : key_lo;
+    key_hi = front ? max(key_hi, kb) : key_hi;
+    odd_late |= late && kb != invalid_bits;
     nv += total_f;
     nl += total_l;
+  }
+  {
+#pragma unroll
+    for (int d = 32; d > 0; d >>= 1) {
+      key_lo = min(key_lo, (uint32_t)__shfl_xor((int)key_lo, d));
+      key_hi = max(key_hi, (uint32_t)__shfl_xor((int)key_hi, d));
+    }
+    if (lane == 0) {                                     // one pair of LDS atomics per wavefront
+      atomicMin(&s_kmin, key_lo);
+      atomicMax(&s_kmax, key_hi);
+    }
+    if (__ballot(odd_late) && lane == 0) atomicOr(&s_flags, 1);
   }
   __syncthreads();
 

@@ -132,6 +132,26 @@ def bin_legacy(positions, log_scales, view_matrices, proj_matrix, W: int, H: int
     return cand, offsets
 
 
+def _host_f32(t):
+    """A contiguous float32 host tensor of `t` (itself when it already is one)."""
+    if t.device.type == "cpu" and t.dtype == torch.float32 and t.is_contiguous() and not t.requires_grad:
+        return t
+    return t.detach().to("cpu", torch.float32).contiguous()
+
+
+_scratch_bytes = {}
+
+
+def _bin_scratch_bytes(n, K, W, H, tile):
+    key = (n, K, W, H, tile)
+    got = _scratch_bytes.get(key)
+    if got is None:
+        if len(_scratch_bytes) > 64:
+            _scratch_bytes.clear()
+        got = _scratch_bytes[key] = _lib.load().mlpsp_bin_scratch_bytes(n, K, W, H, tile)
+    return got
+
+
 def bin_legacy_async(positions, log_scales, view_matrices, proj_matrix, W: int, H: int, tile: int, threshold: float,
                      cand_capacity: int, tile_view_ids=None, scratch_scale: int = 1, counts=None):
     """:func:`bin_legacy` without any host synchronisation -> (candidates [cand_capacity], tile_offsets [T+1],
@@ -141,8 +161,7 @@ def bin_legacy_async(positions, log_scales, view_matrices, proj_matrix, W: int, 
     view of a buffer that is read back in one copy together with other results)."""
     positions, log_scales = _f32c(positions, "positions"), _f32c(log_scales, "log_scales")
     dev = positions.device
-    vm = view_matrices.detach().to("cpu", torch.float32).reshape(-1, 4, 4).contiguous()
-    pm = proj_matrix.detach().to("cpu", torch.float32).reshape(4, 4).contiguous()
+    vm, pm = _host_f32(view_matrices).reshape(-1, 4, 4), _host_f32(proj_matrix).reshape(4, 4)
     K, n = vm.shape[0], positions.shape[0]
     T = num_tiles(W, H, tile, tile)
     tv = None
@@ -152,7 +171,7 @@ def bin_legacy_async(positions, log_scales, view_matrices, proj_matrix, W: int, 
             raise ValueError(f"tile_view_ids length mismatch: got {tv.numel()}, expected {T}")
     lib = _lib.load()
     fp = C.POINTER(C.c_float)
-    nbytes = lib.mlpsp_bin_scratch_bytes(n, K, W, H, tile) * int(scratch_scale)
+    nbytes = _bin_scratch_bytes(n, K, W, H, tile) * int(scratch_scale)
     with torch.inference_mode(False):
         offsets = torch.empty(T + 1, dtype=torch.int32, device=dev)
         cand = torch.empty(int(cand_capacity), dtype=torch.int32, device=dev)
