@@ -107,6 +107,16 @@ int mlpsp_bin_legacy_async(const float* positions_dev, const float* log_scales_d
                            void* scratch_dev, size_t scratch_bytes, int32_t* tile_offsets_dev,
                            int32_t* candidates_dev, int64_t cand_capacity, int64_t* counts_dev,
                            mlpsp_stream_t stream);
+
+/* mlpsp_bin_legacy_async for ONE view whose two matrices are device tensors (4x4 row-major float each), as the
+ * reference's evaluators hold them (scannet/eval_rgb_psnr.py:465-466): nothing is copied to the host, so a frame
+ * that starts with this call starts without a synchronisation.  Same lists and counts, bit for bit (the focal
+ * length is formed on the device with the host's expression). */
+int mlpsp_bin_legacy_async_device_matrices(const float* positions_dev, const float* log_scales_dev,
+                                           int num_primitives, const float* view_matrix_dev, const float* proj_dev,
+                                           int width, int height, int tile, float threshold, void* scratch_dev,
+                                           size_t scratch_bytes, int32_t* tile_offsets_dev, int32_t* candidates_dev,
+                                           int64_t cand_capacity, int64_t* counts_dev, mlpsp_stream_t stream);
 int mlpsp_bin_legacy_fill(int num_primitives, int num_views, const int32_t* tile_view_ids_dev, int width,
                           int height, int tile, const void* scratch_dev, size_t scratch_bytes,
                           const int32_t* tile_offsets_dev, int32_t* candidates_dev, mlpsp_stream_t stream);

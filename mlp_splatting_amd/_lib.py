@@ -33,6 +33,8 @@ SIGNATURES = {
     "mlpsp_bin_scratch_bytes": (_sz, [_i, _i, _i, _i, _i]),
     "mlpsp_bin_legacy_count": (_i, [_vp, _vp, _i, C.POINTER(_f), _i, _vp, C.POINTER(_f), _i, _i, _i, _f, _vp, _sz, _vp,
                                     C.POINTER(_i64), _vp]),
+    "mlpsp_bin_legacy_async_device_matrices": (_i, [_vp, _vp, _i, _vp, _vp, _i, _i, _i, _f, _vp, _sz, _vp, _vp, _i64, _vp,
+                                                     _vp]),
     "mlpsp_bin_legacy_async": (_i, [_vp, _vp, _i, C.POINTER(_f), _i, _vp, C.POINTER(_f), _i, _i, _i, _f, _vp, _sz, _vp, _vp,
                                     _i64, _vp, _vp]),
     "mlpsp_bin_legacy_fill": (_i, [_i, _i, _vp, _i, _i, _i, _vp, _sz, _vp, _vp, _vp]),

@@ -81,16 +81,22 @@ struct BinMats {
   float v[16], p[16];
 };
 
-template <bool ARGS>
+// MODE 0: K view matrices then the projection at `mats` (device).  MODE 1: one view, both matrices in `one`.
+// MODE 2: one view, the view matrix at `mats` and the projection at `proj_dev` (device tensors of the caller: no
+// host copy of them exists, so the focal length is formed here, with the host's expression).
+template <int MODE>
 __global__ __launch_bounds__(kBinThreads) void bin_bounds_kernel(const float* __restrict__ pos,
                                                                  const float* __restrict__ logs,
-                                                                 const float* __restrict__ mats, BinMats one, BinGeom g,
-                                                                 float rm, float focal, float4* __restrict__ bounds) {
+                                                                 const float* __restrict__ mats,
+                                                                 const float* __restrict__ proj_dev, BinMats one,
+                                                                 BinGeom g, float rm, float focal,
+                                                                 float4* __restrict__ bounds) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   const int k = blockIdx.y;
   if (i >= g.N) return;
-  const float* V = ARGS ? one.v : mats + k * 16;
-  const float* Pm = ARGS ? one.p : mats + g.K * 16;
+  const float* V = MODE == 1 ? one.v : mats + k * 16;
+  const float* Pm = MODE == 1 ? one.p : MODE == 2 ? proj_dev : mats + g.K * 16;
+  if (MODE == 2) focal = ((Pm[0] * (float)g.W) / 2.0f + (Pm[5] * (float)g.H) / 2.0f) * 0.5f;
   const float x = pos[i * 3 + 0], y = pos[i * 3 + 1], z = pos[i * 3 + 2];
   float pv[4], clip[4];
 #pragma unroll
@@ -476,37 +482,10 @@ MLPSP_API size_t mlpsp_bin_scratch_bytes(int num_primitives, int num_views, int 
 }
 
 namespace {
-// Enqueues bounds -> level 1 (count, scan, fill) -> level 2 count -> scan.  Leaves the exclusive tile offsets in
-// tile_offsets_dev and (level-1 entries, pairs, longest tile list) in b.totals[0..2]; no host synchronisation.
-int enqueue_bin_count(const float* positions_dev, const float* log_scales_dev, int num_primitives,
-                      const float* view_matrices_host, int num_views, const int32_t* tile_view_ids_dev,
-                      const float* proj_host, int width, int height, int tile, float threshold, const BinGeom& g,
-                      const BinScratch& b, int64_t T, int32_t* tile_offsets_dev, hipStream_t s,
-                      bool matrices_in_scratch = false, ScanGuard guard = ScanGuard{nullptr, nullptr, 0, 0}) {
+// level 1 (count, scan, fill) -> level 2 count -> scan, behind the bounds kernel
+int enqueue_bin_levels(const BinGeom& g, const BinScratch& b, int64_t T, const int32_t* tile_view_ids_dev,
+                       int32_t* tile_offsets_dev, hipStream_t s, ScanGuard guard) {
   const int S = g.nsx * g.nsy;
-  // scalar constants in f32, in the order the reference's tensor expressions evaluate them
-  const float rm = sqrtf(-2.0f * logf(threshold));
-  const float fx = (proj_host[0] * (float)width) / 2.0f, fy = (proj_host[5] * (float)height) / 2.0f;
-  const float focal = (fx + fy) * 0.5f;
-  BinMats one{};
-  if (num_views == 1) {
-    for (int e = 0; e < 16; ++e) {
-      one.v[e] = view_matrices_host[e];
-      one.p[e] = proj_host[e];
-    }
-    hipLaunchKernelGGL(bin_bounds_kernel<true>, dim3(ceil_div(num_primitives, kBinThreads), 1), dim3(kBinThreads), 0, s,
-                       positions_dev, log_scales_dev, (const float*)nullptr, one, g, rm, focal, b.bounds);
-  } else {
-    if (!matrices_in_scratch) {
-      MLPSP_HIP_TRY(hipMemcpyAsync(b.mats, view_matrices_host, (size_t)num_views * 16 * sizeof(float),
-                                   hipMemcpyHostToDevice, s));
-      MLPSP_HIP_TRY(hipMemcpyAsync(b.mats + (size_t)num_views * 16, proj_host, 16 * sizeof(float),
-                                   hipMemcpyHostToDevice, s));
-    }
-    hipLaunchKernelGGL(bin_bounds_kernel<false>, dim3(ceil_div(num_primitives, kBinThreads), num_views),
-                       dim3(kBinThreads), 0, s, positions_dev, log_scales_dev, b.mats, one, g, rm, focal, b.bounds);
-  }
-  MLPSP_LAUNCH_CHECK();
   hipLaunchKernelGGL((bin_level1_kernel<false>), dim3(g.NC, ceil_div(S, kBinThreads / 64)), dim3(kBinThreads), 0, s, b.bounds, g,
                      tile_view_ids_dev, b.l1_counts, b.l1_list, b.l1_bounds, b.l1_capacity, b.l1_masks);
   MLPSP_LAUNCH_CHECK();
@@ -524,6 +503,49 @@ int enqueue_bin_count(const float* positions_dev, const float* log_scales_dev, i
                      b.totals + 2, guard);
   MLPSP_LAUNCH_CHECK();
   return MLPSP_OK;
+}
+
+// Enqueues bounds -> level 1 (count, scan, fill) -> level 2 count -> scan.  Leaves the exclusive tile offsets in
+// tile_offsets_dev and (level-1 entries, pairs, longest tile list) in b.totals[0..2]; no host synchronisation.
+int enqueue_bin_count(const float* positions_dev, const float* log_scales_dev, int num_primitives,
+                      const float* view_matrices_host, int num_views, const int32_t* tile_view_ids_dev,
+                      const float* proj_host, int width, int height, int tile, float threshold, const BinGeom& g,
+                      const BinScratch& b, int64_t T, int32_t* tile_offsets_dev, hipStream_t s,
+                      bool matrices_in_scratch = false, ScanGuard guard = ScanGuard{nullptr, nullptr, 0, 0},
+                      const float* view_dev = nullptr, const float* proj_dev = nullptr) {
+  const int S = g.nsx * g.nsy;
+  // scalar constants in f32, in the order the reference's tensor expressions evaluate them
+  const float rm = sqrtf(-2.0f * logf(threshold));
+  BinMats one{};
+  if (view_dev) {             // one view, matrices on the device
+    hipLaunchKernelGGL(bin_bounds_kernel<2>, dim3(ceil_div(num_primitives, kBinThreads), 1), dim3(kBinThreads), 0, s,
+                       positions_dev, log_scales_dev, view_dev, proj_dev, one, g, rm, 0.f, b.bounds);
+    MLPSP_LAUNCH_CHECK();
+    return enqueue_bin_levels(g, b, T, tile_view_ids_dev, tile_offsets_dev, s, guard);
+  }
+  const float fx = (proj_host[0] * (float)width) / 2.0f, fy = (proj_host[5] * (float)height) / 2.0f;
+  const float focal = (fx + fy) * 0.5f;
+  if (num_views == 1) {
+    for (int e = 0; e < 16; ++e) {
+      one.v[e] = view_matrices_host[e];
+      one.p[e] = proj_host[e];
+    }
+    hipLaunchKernelGGL(bin_bounds_kernel<1>, dim3(ceil_div(num_primitives, kBinThreads), 1), dim3(kBinThreads), 0, s,
+                       positions_dev, log_scales_dev, (const float*)nullptr, (const float*)nullptr, one, g, rm, focal,
+                       b.bounds);
+  } else {
+    if (!matrices_in_scratch) {
+      MLPSP_HIP_TRY(hipMemcpyAsync(b.mats, view_matrices_host, (size_t)num_views * 16 * sizeof(float),
+                                   hipMemcpyHostToDevice, s));
+      MLPSP_HIP_TRY(hipMemcpyAsync(b.mats + (size_t)num_views * 16, proj_host, 16 * sizeof(float),
+                                   hipMemcpyHostToDevice, s));
+    }
+    hipLaunchKernelGGL(bin_bounds_kernel<0>, dim3(ceil_div(num_primitives, kBinThreads), num_views),
+                       dim3(kBinThreads), 0, s, positions_dev, log_scales_dev, b.mats, (const float*)nullptr, one, g, rm,
+                       focal, b.bounds);
+  }
+  MLPSP_LAUNCH_CHECK();
+  return enqueue_bin_levels(g, b, T, tile_view_ids_dev, tile_offsets_dev, s, guard);
 }
 
 int check_bin_args(int64_t T, const float* view_matrices_host, const float* proj_host, void* scratch_dev,
@@ -574,19 +596,21 @@ MLPSP_API int mlpsp_bin_legacy_count(const float* positions_dev, const float* lo
   return MLPSP_OK;
 }
 
-MLPSP_API int mlpsp_bin_legacy_async(const float* positions_dev, const float* log_scales_dev, int num_primitives,
-                                     const float* view_matrices_host, int num_views,
-                                     const int32_t* tile_view_ids_dev, const float* proj_host, int width, int height,
-                                     int tile, float threshold, void* scratch_dev, size_t scratch_bytes,
-                                     int32_t* tile_offsets_dev, int32_t* candidates_dev, int64_t cand_capacity,
-                                     int64_t* counts_dev, mlpsp_stream_t stream) {
+namespace {
+int bin_legacy_async_impl(const float* positions_dev, const float* log_scales_dev, int num_primitives,
+                          const float* view_matrices_host, int num_views, const int32_t* tile_view_ids_dev,
+                          const float* proj_host, const float* view_dev, const float* proj_dev, int width, int height,
+                          int tile, float threshold, void* scratch_dev, size_t scratch_bytes, int32_t* tile_offsets_dev,
+                          int32_t* candidates_dev, int64_t cand_capacity, int64_t* counts_dev, hipStream_t s) {
   const int64_t T = checked_num_tiles(width, height, tile, tile);
   if (!counts_dev || cand_capacity < 0 || cand_capacity > 2147483647LL || (cand_capacity > 0 && !candidates_dev))
     return MLPSP_E_ARGUMENT;
-  const int rc = check_bin_args(T, view_matrices_host, proj_host, scratch_dev, scratch_bytes, tile_offsets_dev,
-                                num_primitives, num_views, width, height, tile, threshold);
+  // (with device matrices the host pointers stand in for themselves in the argument check: they are not read)
+  const float* vh = view_dev ? view_dev : view_matrices_host;
+  const float* ph = proj_dev ? proj_dev : proj_host;
+  const int rc = check_bin_args(T, vh, ph, scratch_dev, scratch_bytes, tile_offsets_dev, num_primitives, num_views, width,
+                                height, tile, threshold);
   if (rc != MLPSP_OK) return rc;
-  hipStream_t s = (hipStream_t)stream;
   const BinGeom g = make_geom(num_primitives, num_views, width, height, tile);
   const BinScratch b = carve(scratch_dev, scratch_bytes, num_primitives, num_views, g.nsx * g.nsy, g.NC);
   if (num_primitives == 0) {
@@ -597,13 +621,40 @@ MLPSP_API int mlpsp_bin_legacy_async(const float* positions_dev, const float* lo
   const int erc = enqueue_bin_count(positions_dev, log_scales_dev, num_primitives, view_matrices_host, num_views,
                                     tile_view_ids_dev, proj_host, width, height, tile, threshold, g, b, T,
                                     tile_offsets_dev, s, false,
-                                    ScanGuard{b.totals, (long long*)counts_dev, b.l1_capacity, (long long)cand_capacity});
+                                    ScanGuard{b.totals, (long long*)counts_dev, b.l1_capacity, (long long)cand_capacity},
+                                    view_dev, proj_dev);
   if (erc != MLPSP_OK) return erc;
   hipLaunchKernelGGL((bin_level2_kernel<true>), dim3(ceil_div((int)T, kBinThreads / 64)), dim3(kBinThreads), 0, s,
                      b.bounds, g, tile_view_ids_dev, b.l1_counts, b.l1_list, b.l1_bounds, b.l1_capacity, tile_offsets_dev,
                      candidates_dev, b.l2_masks, b.l2_mask_stride, (const long long*)(b.totals + 3));
   MLPSP_LAUNCH_CHECK();
   return MLPSP_OK;
+}
+}  // namespace
+
+MLPSP_API int mlpsp_bin_legacy_async(const float* positions_dev, const float* log_scales_dev, int num_primitives,
+                                     const float* view_matrices_host, int num_views,
+                                     const int32_t* tile_view_ids_dev, const float* proj_host, int width, int height,
+                                     int tile, float threshold, void* scratch_dev, size_t scratch_bytes,
+                                     int32_t* tile_offsets_dev, int32_t* candidates_dev, int64_t cand_capacity,
+                                     int64_t* counts_dev, mlpsp_stream_t stream) {
+  return bin_legacy_async_impl(positions_dev, log_scales_dev, num_primitives, view_matrices_host, num_views,
+                               tile_view_ids_dev, proj_host, nullptr, nullptr, width, height, tile, threshold, scratch_dev,
+                               scratch_bytes, tile_offsets_dev, candidates_dev, cand_capacity, counts_dev,
+                               (hipStream_t)stream);
+}
+
+MLPSP_API int mlpsp_bin_legacy_async_device_matrices(const float* positions_dev, const float* log_scales_dev,
+                                                     int num_primitives, const float* view_matrix_dev,
+                                                     const float* proj_dev, int width, int height, int tile,
+                                                     float threshold, void* scratch_dev, size_t scratch_bytes,
+                                                     int32_t* tile_offsets_dev, int32_t* candidates_dev,
+                                                     int64_t cand_capacity, int64_t* counts_dev,
+                                                     mlpsp_stream_t stream) {
+  if (!view_matrix_dev || !proj_dev) return MLPSP_E_ARGUMENT;
+  return bin_legacy_async_impl(positions_dev, log_scales_dev, num_primitives, nullptr, 1, nullptr, nullptr, view_matrix_dev,
+                               proj_dev, width, height, tile, threshold, scratch_dev, scratch_bytes, tile_offsets_dev,
+                               candidates_dev, cand_capacity, counts_dev, (hipStream_t)stream);
 }
 
 MLPSP_API int mlpsp_bin_legacy_fill(int num_primitives, int num_views, const int32_t* tile_view_ids_dev, int width,

@@ -75,6 +75,14 @@ def _unit_directions(ray_d):
     return F.normalize(ray_d, dim=-1).contiguous()
 
 
+def _frame_matrix(t):
+    """The matrix as the queued frame takes it: a float32 device tensor stays where it is (the binning reads it
+    there; no copy to the host, no synchronisation), anything else becomes a host copy."""
+    if torch.is_tensor(t) and t.is_cuda and t.dtype == torch.float32 and t.numel() == 16:
+        return t.detach().contiguous()
+    return _host_matrix(t)
+
+
 def _host_matrix(t):
     """A float32 host copy of a small device tensor (view / projection matrices), remembered for as long
     as that very tensor object is alive and unmodified: the binning reads its matrices on the host, and a
@@ -797,7 +805,7 @@ class NeuralPrimitiveSceneTileCUDA(nn.Module):
             return None                       # stored half-precision weights: only the matrix-core frame reads them as they are
         out = ext.render_frame_queued(ray_o.contiguous(), unit_dirs, self.positions.detach().contiguous(),
                                       self.log_scales.detach().contiguous(), self._unit_quats(), freq, att, ws,
-                                      _host_matrix(view_matrix).reshape(1, 4, 4), _host_matrix(proj_matrix), int(W),
+                                      _frame_matrix(view_matrix).reshape(1, 4, 4), _frame_matrix(proj_matrix), int(W),
                                       int(H), float(score_threshold), precision)
         if out is None:
             return None

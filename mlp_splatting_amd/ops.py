@@ -161,8 +161,15 @@ def bin_legacy_async(positions, log_scales, view_matrices, proj_matrix, W: int, 
     view of a buffer that is read back in one copy together with other results)."""
     positions, log_scales = _f32c(positions, "positions"), _f32c(log_scales, "log_scales")
     dev = positions.device
-    vm, pm = _host_f32(view_matrices).reshape(-1, 4, 4), _host_f32(proj_matrix).reshape(4, 4)
-    K, n = vm.shape[0], positions.shape[0]
+    on_device = (tile_view_ids is None and all(m.is_cuda and m.dtype == torch.float32 and m.numel() == 16 and
+                                               m.is_contiguous() for m in (view_matrices, proj_matrix)))
+    if on_device:               # one view, both matrices already on the device: nothing is brought to the host
+        vm, pm = view_matrices, proj_matrix
+        K = 1
+    else:
+        vm, pm = _host_f32(view_matrices).reshape(-1, 4, 4), _host_f32(proj_matrix).reshape(4, 4)
+        K = vm.shape[0]
+    n = positions.shape[0]
     T = num_tiles(W, H, tile, tile)
     tv = None
     if tile_view_ids is not None:
@@ -180,9 +187,14 @@ def bin_legacy_async(positions, log_scales, view_matrices, proj_matrix, W: int, 
         counts = torch.empty(4, dtype=torch.int64, device=dev)
     elif not (counts.is_cuda and counts.dtype == torch.int64 and counts.numel() == 4 and counts.is_contiguous()):
         raise ValueError("counts must be a contiguous int64 [4] tensor on the device")
-    code = lib.mlpsp_bin_legacy_async(_ptr(positions), _ptr(log_scales), n, C.cast(vm.data_ptr(), fp), K, _ptr(tv),
-                                      C.cast(pm.data_ptr(), fp), W, H, tile, float(threshold), _ptr(scratch), nbytes,
-                                      _ptr(offsets), _ptr(cand), int(cand_capacity), _ptr(counts), _stream(dev))
+    if on_device:
+        code = lib.mlpsp_bin_legacy_async_device_matrices(_ptr(positions), _ptr(log_scales), n, _ptr(vm), _ptr(pm), W, H,
+                                                          tile, float(threshold), _ptr(scratch), nbytes, _ptr(offsets),
+                                                          _ptr(cand), int(cand_capacity), _ptr(counts), _stream(dev))
+    else:
+        code = lib.mlpsp_bin_legacy_async(_ptr(positions), _ptr(log_scales), n, C.cast(vm.data_ptr(), fp), K, _ptr(tv),
+                                          C.cast(pm.data_ptr(), fp), W, H, tile, float(threshold), _ptr(scratch), nbytes,
+                                          _ptr(offsets), _ptr(cand), int(cand_capacity), _ptr(counts), _stream(dev))
     _check(code, "mlpsp_bin_legacy_async")
     return cand, offsets, counts
 

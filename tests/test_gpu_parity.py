@@ -546,3 +546,24 @@ def test_training_records_hit_capacity_is_an_error(device, oracle_mod):
     x[5], x[6] = torch.zeros(0, dtype=torch.int32, device=device), torch.zeros_like(x[6])
     out = TileExt().render_tiles_training_records(x, fr.W, fr.H, 8, fr.thr, 1.5, 2.0)
     assert out[2].numel() == 0 and int(out[7][-1]) == 0 and float(out[0].abs().max()) == 0.0
+
+
+def test_async_binning_with_device_matrices_equals_host_matrices(device, oracle_mod):
+    """The asynchronous binning takes one view's matrices from the host or straight from device tensors (what the
+    reference's evaluators hold); lists and counts are the same bits, and equal the oracle's."""
+    from mlp_splatting_amd import ops
+    fr = Frame("cfg1_5k_160x120", n=3000, width=104, height=72, eye=(0.4, 0.1, -0.7))
+    sc = fr.scene
+    pos, logs = _t(sc.positions, device), _t(sc.log_scales, device)
+    view_host, proj_host = torch.from_numpy(fr.view), torch.from_numpy(fr.proj)
+    want_cand, want_off = fr.oracle_lists(oracle_mod)
+    results = []
+    for view, proj in ((view_host[None], proj_host), (view_host.to(device), proj_host.to(device))):
+        cand, off, counts = ops.bin_legacy_async(pos, logs, view, proj, fr.W, fr.H, 8, fr.thr, want_cand.size + 100)
+        pairs, longest, _, guard = counts.tolist()
+        assert guard == 0 and pairs == want_cand.size
+        results.append((cand[:pairs].cpu().numpy(), off.cpu().numpy(), longest))
+    for cand, off, longest in results:
+        np.testing.assert_array_equal(off, want_off)
+        np.testing.assert_array_equal(cand, want_cand)
+        assert longest == int(np.diff(want_off).max())
