@@ -487,7 +487,8 @@ class NeuralPrimitiveSceneTileCUDA(nn.Module):
             raise RuntimeError("NeuralPrimitiveSceneTileCUDA must be moved to a CUDA device before rendering.")
         if device.index is None:
             device = torch.device("cuda", torch.cuda.current_device())
-        torch.cuda.set_device(device.index)
+        elif torch.cuda.current_device() != device.index:
+            torch.cuda.set_device(device.index)
         return device
 
     def _resolve_tile_order_mode(self) -> str:
@@ -521,7 +522,7 @@ class NeuralPrimitiveSceneTileCUDA(nn.Module):
         scene is constant while rendering, and every small torch op skipped is a kernel launch less per
         frame.  The value is built outside inference mode so that it carries a version counter itself."""
         try:
-            key = tuple((t.data_ptr(), t._version, tuple(t.shape), str(t.device)) for t in sources) + tuple(extra)
+            key = tuple((t.data_ptr(), t._version, t.shape, t.device) for t in sources) + tuple(extra)
         except RuntimeError:                      # inference tensors have no version counter: do not cache
             return build()
         cache = self.__dict__.setdefault("_mlpsp_cache", {})
@@ -537,7 +538,7 @@ class NeuralPrimitiveSceneTileCUDA(nn.Module):
         sources = [self.encoder.freq_bands]
         if hasattr(self.encoder, "runtime_frequency_weights"):
             sources.append(self.encoder.runtime_frequency_weights)
-        extra = (str(device), float(getattr(self.encoder, "sigma2", 0.0)))
+        extra = (device, float(getattr(self.encoder, "sigma2", 0.0)))
         return self._cached("frequency_tables", sources, extra, lambda: self._build_frequency_tables(device))
 
     def _build_frequency_tables(self, device):

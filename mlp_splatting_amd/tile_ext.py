@@ -36,6 +36,14 @@ def _is_f32_2d(t, cols):
     return t.is_cuda and t.dtype == torch.float32 and t.dim() == 2 and t.shape[1] == cols
 
 
+
+def _on_device(device):
+    """``torch.cuda.device(device)``, or nothing when that device is current already (saves two device switches)."""
+    if device.index is None or torch.cuda.current_device() == device.index:
+        return contextlib.nullcontext()
+    return torch.cuda.device(device)
+
+
 class TileExt:
     """Forward entry points of the tile renderer on one MI355X."""
 
@@ -316,7 +324,7 @@ class TileExt:
         if cap <= 0:
             return None
         n = positions.shape[0]
-        with torch.cuda.device(rays_o.device):
+        with _on_device(rays_o.device):
             rec = self._records(positions, log_scales, unit_quats)
             # counts of the binning (4 x int64) and flag words of the render (16 x int32) share one buffer: the
             # frame's single read-back is one 96-byte copy
