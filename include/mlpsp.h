@@ -257,7 +257,7 @@ int mlpsp_all_finite(const float* const* arrays_dev, const int64_t* lengths, int
 /* Workspace of the feature renders below.  The render kernel hands the feature kernel one "hit record"
  * per (64-pixel wavefront of a tile, primitive that hits one of its pixels); how many there will be is
  * only known after the frame (early termination), so records come from a pool of pool_records records.
- * pool_records < 0 asks for the worst case (one per candidate and wavefront + 15 per wavefront), which can
+ * pool_records < 0 asks for the worst case (one per candidate and wavefront + 63 per wavefront), which can
  * never run out; a smaller pool that runs out sets the call's overflow status and the caller repeats the
  * frame with a larger one.  fp16_records: 0 for mlpsp_render_tilecenter_feat_f32, 1 for
  * mlpsp_render_tilecenter_mfma_feat (tile_w = tile_h = 8).  0 on bad arguments. */

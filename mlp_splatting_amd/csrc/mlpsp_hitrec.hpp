@@ -22,6 +22,7 @@
 namespace mlpsp {
 
 constexpr int kHitChunk = 16;
+constexpr int kHitGrab = 4;      // chunks a wavefront draws from the pool per atomic
 
 struct HitPool {
   int32_t* counters;
@@ -92,22 +93,27 @@ __device__ __forceinline__ HitEmitter hit_emitter_begin(const HitPool& hp, int w
 }
 
 // Slot (record index in the pool) for the item's next record, or -1 on overflow.  Call with the whole
-// wavefront active; the result is wave-uniform.
+// wavefront active; the result is wave-uniform.  The pool is drawn kHitGrab chunks at a time (one atomic per 64
+// records: the wavefront waits for its result, and every vector-memory wait behind it waits with it), the chunk
+// table still has one entry per chunk.
 __device__ __forceinline__ int hit_emitter_next(const HitPool& hp, HitEmitter& em, int lane) {
   if (em.chunk < 0) return -1;
-  if ((em.count & (kHitChunk - 1)) == 0) {
+  constexpr int kGroup = kHitChunk * kHitGrab;
+  if ((em.count & (kGroup - 1)) == 0) {
     int c = 0;
-    if (lane == 0) c = atomicAdd(hp.counters, 1);
+    if (lane == 0) c = atomicAdd(hp.counters, kHitGrab);
     c = __builtin_amdgcn_readfirstlane(c);
-    if (c >= hp.pool_chunks) {
+    if (c + kHitGrab > hp.pool_chunks) {
       if (lane == 0) atomicExch(hp.counters + 1, 1);
       em.chunk = -1;
       return -1;
     }
-    if (lane == 0) hp.chunk_table[em.table_base + (em.count >> 4)] = c;
-    em.chunk = c;
+    em.chunk = c;                       // first chunk of the group
   }
-  const int slot = em.chunk * kHitChunk + (em.count & (kHitChunk - 1));
+  const int within = em.count & (kGroup - 1);
+  if ((within & (kHitChunk - 1)) == 0 && lane == 0)
+    hp.chunk_table[em.table_base + (em.count >> 4)] = em.chunk + (within >> 4);
+  const int slot = em.chunk * kHitChunk + within;
   ++em.count;
   return slot;
 }

@@ -130,7 +130,8 @@ MLPSP_API size_t mlpsp_feat_workspace_bytes(int64_t num_pairs, int width, int he
     return 0;
   const int wpt = (int)((tile_px + 63) / 64);
   const int rec = fp16_records ? 64 * 2 * (feat_slots == 5 ? 8 : 4) : 64 * 4 * (feat_slots > 1 ? 5 : 1);
-  const int64_t worst = num_pairs * wpt + (int64_t)(kHitChunk - 1) * T * wpt;
+  // every wavefront draws records 64 at a time: its last draw can stay 63 short of full
+  const int64_t worst = num_pairs * wpt + (int64_t)(kHitChunk * kHitGrab - 1) * T * wpt + kHitChunk * kHitGrab;
   if (pool_records < 0 || pool_records > worst) pool_records = worst;
   return hitpool_bytes(num_pairs, T, wpt, pool_records, rec);
 }
