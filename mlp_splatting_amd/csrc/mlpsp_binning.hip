@@ -29,7 +29,9 @@ struct BinScratch {
   int32_t* l1_counts; // [S*NC + 1] counts, then exclusive offsets after the scan
   long long* totals;  // [0] level-1 entries, [1] tile-list entries, [2] longest tile list, [3] guard status
   int32_t* l1_list;   // [l1_capacity]
-  float4* l1_bounds;  // [l1_capacity] bounds of the listed primitives, one view only (else null)
+  float4* l1_bounds;  // [l1_capacity] bounds of the listed primitives under the super-tile's view (garbage for a
+                      // super-tile whose tiles use several views: super_view says which)
+  int32_t* super_view;    // [S] the one view all tiles of the super-tile use, or -1
   long long l1_capacity;
   // survivor masks of the counting passes (one ballot per 64 tested entries), so that the fill passes neither
   // re-read the bounds nor repeat the tests:
@@ -52,19 +54,21 @@ inline BinScratch carve(void* base, size_t bytes, int N, int K, int S, int NC) {
   off += align256(((size_t)S * NC + 1) * sizeof(int32_t));
   b.totals = reinterpret_cast<long long*>(p + off);
   off += 256;
-  // one view: the level-1 lists carry the bounds next to the ids (20 bytes per entry), so that level 2
-  // streams them instead of gathering 16 bytes per lane from all over the bounds array
+  // the level-1 lists carry the bounds next to the ids (20 bytes per entry), so that level 2 streams them
+  // instead of gathering 16 bytes per lane from all over the bounds array
   b.l1_masks = reinterpret_cast<unsigned long long*>(p + off);
   off += align256((size_t)S * NC * (kChunk / 64) * sizeof(unsigned long long));
-  // per level-1 entry: 4 bytes id (+ 16 bytes bounds with one view) + 64 mask bits for the 64 tiles = 8 bytes
-  const size_t entry = sizeof(int32_t) + (K == 1 ? sizeof(float4) : 0) + 8;
+  b.super_view = reinterpret_cast<int32_t*>(p + off);
+  off += align256((size_t)S * sizeof(int32_t));
+  // per level-1 entry: 4 bytes id + 16 bytes bounds + 64 mask bits for the 64 tiles = 8 bytes
+  const size_t entry = sizeof(int32_t) + sizeof(float4) + 8;
   const size_t fixed = off + 1024 + align256((size_t)(S + 1) * 64 * sizeof(unsigned long long));
   b.l1_capacity = bytes > fixed ? (long long)((bytes - fixed) / entry) : 0;
   b.l1_capacity &= ~63LL;
   b.l1_list = reinterpret_cast<int32_t*>(p + off);
   off += align256((size_t)b.l1_capacity * sizeof(int32_t));
-  b.l1_bounds = (K == 1) ? reinterpret_cast<float4*>(p + off) : nullptr;
-  if (K == 1) off += align256((size_t)b.l1_capacity * sizeof(float4));
+  b.l1_bounds = reinterpret_cast<float4*>(p + off);
+  off += align256((size_t)b.l1_capacity * sizeof(float4));
   b.l2_mask_stride = b.l1_capacity / 64 + S + 1;
   b.l2_masks = reinterpret_cast<unsigned long long*>(p + off);
   return b;
@@ -157,7 +161,8 @@ __global__ __launch_bounds__(kBinThreads) void bin_level1_kernel(const float4* _
                                                                  int32_t* __restrict__ l1_counts,
                                                                  int32_t* __restrict__ l1_list,
                                                                  float4* __restrict__ l1_bounds, long long l1_capacity,
-                                                                 unsigned long long* __restrict__ l1_masks) {
+                                                                 unsigned long long* __restrict__ l1_masks,
+                                                                 int32_t* __restrict__ super_view) {
   const int c = blockIdx.x, s = blockIdx.y * (kBinThreads / 64) + (threadIdx.x >> 6);
   const int lane = threadIdx.x & 63;
   if (s >= g.nsx * g.nsy) return;
@@ -183,6 +188,10 @@ __global__ __launch_bounds__(kBinThreads) void bin_level1_kernel(const float4* _
     }
     if (found <= 4) nviews = -found;       // negative: use the explicit list
   }
+  // one view for the whole super-tile (always so with one camera): the fast paths below, here and in level 2
+  const bool single = g.K == 1 || nviews == -1;
+  const float4* __restrict__ sb = bounds + (size_t)(g.K == 1 ? 0 : v0) * g.N;
+  if (!FILL && c == 0 && lane == 0) super_view[s] = single ? (g.K == 1 ? 0 : v0) : -1;
   long long running = FILL ? l1_counts[s * g.NC + c] : 0;
   const int first = c * kChunk;
   unsigned long long* __restrict__ masks = l1_masks + ((size_t)s * g.NC + c) * (kChunk / 64);
@@ -199,7 +208,7 @@ __global__ __launch_bounds__(kBinThreads) void bin_level1_kernel(const float4* _
         const long long dst = running + lanes_below(m);
         if (dst < l1_capacity) {
           l1_list[dst] = i;
-          if (l1_bounds) l1_bounds[dst] = bounds[i];
+          if (single) l1_bounds[dst] = sb[i];
         }
       }
       running += __popcll(m);
@@ -207,7 +216,7 @@ __global__ __launch_bounds__(kBinThreads) void bin_level1_kernel(const float4* _
     return;
   }
   unsigned long long mine = 0ull;
-  if (g.K == 1) {
+  if (single) {
     // one view: eight independent 16-byte loads in flight per step (NaN bounds fail every comparison)
     const float nanv = __builtin_nanf("");
     for (int r0 = 0; r0 < kChunk / 64; r0 += 8) {
@@ -215,7 +224,7 @@ __global__ __launch_bounds__(kBinThreads) void bin_level1_kernel(const float4* _
 #pragma unroll
       for (int u = 0; u < 8; ++u) {
         const int i = first + (r0 + u) * 64 + lane;
-        bb[u] = (i < g.N) ? bounds[i] : make_float4(nanv, nanv, nanv, nanv);
+        bb[u] = (i < g.N) ? sb[i] : make_float4(nanv, nanv, nanv, nanv);
       }
 #pragma unroll
       for (int u = 0; u < 8; ++u) {
@@ -370,6 +379,7 @@ __global__ __launch_bounds__(kBinThreads) void bin_level2_kernel(const float4* _
                                                                  int32_t* __restrict__ cand,
                                                                  unsigned long long* __restrict__ l2_masks,
                                                                  long long l2_mask_stride,
+                                                                 const int32_t* __restrict__ super_view,
                                                                  const long long* __restrict__ skip_flag = nullptr) {
   const int tile = blockIdx.x * (kBinThreads / 64) + (threadIdx.x >> 6);
   const int lane = threadIdx.x & 63;
@@ -411,8 +421,8 @@ __global__ __launch_bounds__(kBinThreads) void bin_level2_kernel(const float4* _
     return;
   }
   unsigned long long mine = 0ull;
-  if (l1_bounds) {
-    // one view: the bounds sit next to the ids; four independent 16-byte loads in flight per step
+  if (super_view[s] == view) {
+    // one view for the super-tile: its bounds sit next to the ids; four independent 16-byte loads in flight per step
     const float nanv = __builtin_nanf("");
     for (int b = 0; b < nb; b += 4) {
       float4 bb[4];
@@ -441,7 +451,7 @@ __global__ __launch_bounds__(kBinThreads) void bin_level2_kernel(const float4* _
     bool keep = false;
     if (j < hi) {
       id = l1_list[j];
-      keep = rect_overlap(l1_bounds ? l1_bounds[j] : vb[id], x0, x1, y0, y1);
+      keep = rect_overlap(vb[id], x0, x1, y0, y1);
     }
     const unsigned long long m = __ballot(keep);
     mine = (lane == (b & 63)) ? m : mine;
@@ -472,11 +482,11 @@ MLPSP_API size_t mlpsp_bin_scratch_bytes(int num_primitives, int num_views, int 
   size_t bytes = align256((size_t)(num_views + 1) * 16 * sizeof(float)) +
                  align256((size_t)num_views * num_primitives * sizeof(float4)) +
                  align256((S * g.NC + 1) * sizeof(int32_t)) + 256;
-  bytes += align256(S * g.NC * (kChunk / 64) * sizeof(unsigned long long));
+  bytes += align256(S * g.NC * (kChunk / 64) * sizeof(unsigned long long)) + align256(S * sizeof(int32_t));
   bytes += 1024 + align256((S + 1) * 64 * sizeof(unsigned long long));
   // room for every primitive to touch 8 super-tiles per view, plus slack for tiny scenes; per entry the id,
-  // the bounds (one view) and the 64 survivor bits of the super-tile's tiles
-  const size_t entry = sizeof(int32_t) + (num_views == 1 ? sizeof(float4) : 0) + 8;
+  // the bounds and the 64 survivor bits of the super-tile's tiles
+  const size_t entry = sizeof(int32_t) + sizeof(float4) + 8;
   bytes += align256(((size_t)8 * num_views * num_primitives + 65536) * entry) + 1024;
   return bytes;
 }
@@ -487,17 +497,17 @@ int enqueue_bin_levels(const BinGeom& g, const BinScratch& b, int64_t T, const i
                        int32_t* tile_offsets_dev, hipStream_t s, ScanGuard guard) {
   const int S = g.nsx * g.nsy;
   hipLaunchKernelGGL((bin_level1_kernel<false>), dim3(g.NC, ceil_div(S, kBinThreads / 64)), dim3(kBinThreads), 0, s, b.bounds, g,
-                     tile_view_ids_dev, b.l1_counts, b.l1_list, b.l1_bounds, b.l1_capacity, b.l1_masks);
+                     tile_view_ids_dev, b.l1_counts, b.l1_list, b.l1_bounds, b.l1_capacity, b.l1_masks, b.super_view);
   MLPSP_LAUNCH_CHECK();
   hipLaunchKernelGGL(exclusive_scan_kernel, dim3(1), dim3(1024), 0, s, b.l1_counts, S * g.NC, b.totals,
                      (long long*)nullptr, ScanGuard{nullptr, nullptr, 0, 0});
   MLPSP_LAUNCH_CHECK();
   hipLaunchKernelGGL((bin_level1_kernel<true>), dim3(g.NC, ceil_div(S, kBinThreads / 64)), dim3(kBinThreads), 0, s, b.bounds, g,
-                     tile_view_ids_dev, b.l1_counts, b.l1_list, b.l1_bounds, b.l1_capacity, b.l1_masks);
+                     tile_view_ids_dev, b.l1_counts, b.l1_list, b.l1_bounds, b.l1_capacity, b.l1_masks, b.super_view);
   MLPSP_LAUNCH_CHECK();
   hipLaunchKernelGGL((bin_level2_kernel<false>), dim3(ceil_div((int)T, kBinThreads / 64)), dim3(kBinThreads), 0, s,
                      b.bounds, g, tile_view_ids_dev, b.l1_counts, b.l1_list, b.l1_bounds, b.l1_capacity, tile_offsets_dev,
-                     (int32_t*)nullptr, b.l2_masks, b.l2_mask_stride);
+                     (int32_t*)nullptr, b.l2_masks, b.l2_mask_stride, b.super_view);
   MLPSP_LAUNCH_CHECK();
   hipLaunchKernelGGL(exclusive_scan_kernel, dim3(1), dim3(1024), 0, s, tile_offsets_dev, (int)T, b.totals + 1,
                      b.totals + 2, guard);
@@ -626,7 +636,7 @@ int bin_legacy_async_impl(const float* positions_dev, const float* log_scales_de
   if (erc != MLPSP_OK) return erc;
   hipLaunchKernelGGL((bin_level2_kernel<true>), dim3(ceil_div((int)T, kBinThreads / 64)), dim3(kBinThreads), 0, s,
                      b.bounds, g, tile_view_ids_dev, b.l1_counts, b.l1_list, b.l1_bounds, b.l1_capacity, tile_offsets_dev,
-                     candidates_dev, b.l2_masks, b.l2_mask_stride, (const long long*)(b.totals + 3));
+                     candidates_dev, b.l2_masks, b.l2_mask_stride, b.super_view, (const long long*)(b.totals + 3));
   MLPSP_LAUNCH_CHECK();
   return MLPSP_OK;
 }
@@ -668,7 +678,7 @@ MLPSP_API int mlpsp_bin_legacy_fill(int num_primitives, int num_views, const int
   const BinScratch b = carve(const_cast<void*>(scratch_dev), scratch_bytes, num_primitives, num_views, g.nsx * g.nsy, g.NC);
   hipLaunchKernelGGL((bin_level2_kernel<true>), dim3(ceil_div((int)T, kBinThreads / 64)), dim3(kBinThreads), 0,
                      (hipStream_t)stream, b.bounds, g, tile_view_ids_dev, b.l1_counts, b.l1_list, b.l1_bounds, b.l1_capacity,
-                     const_cast<int32_t*>(tile_offsets_dev), candidates_dev, b.l2_masks, b.l2_mask_stride);
+                     const_cast<int32_t*>(tile_offsets_dev), candidates_dev, b.l2_masks, b.l2_mask_stride, b.super_view);
   MLPSP_LAUNCH_CHECK();
   return MLPSP_OK;
 }
@@ -770,7 +780,7 @@ MLPSP_API int mlpsp_bin_legacy_async_noalloc(const float* positions_dev, const f
   if (erc != MLPSP_OK) return erc;
   hipLaunchKernelGGL((bin_level2_kernel<true>), dim3(ceil_div((int)T, kBinThreads / 64)), dim3(kBinThreads), 0, s,
                      b.bounds, g, tile_view_ids_dev, b.l1_counts, b.l1_list, b.l1_bounds, b.l1_capacity, tile_offsets_dev,
-                     candidates_dev, b.l2_masks, b.l2_mask_stride, (const long long*)(b.totals + 3));
+                     candidates_dev, b.l2_masks, b.l2_mask_stride, b.super_view, (const long long*)(b.totals + 3));
   MLPSP_LAUNCH_CHECK();
   return MLPSP_OK;
 }
