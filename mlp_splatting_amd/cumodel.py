@@ -659,9 +659,6 @@ class NeuralPrimitiveSceneTileCUDA(nn.Module):
             return self._forward_differentiable(ray_o, ray_d, score_threshold, bg_color, view_matrix, proj_matrix,
                                                 culled_prim_indices, tile_offsets, return_feature, device)
         with torch.no_grad():
-            # queued before the binning, whose pair count is a blocking read-back: the device then has
-            # this work to do while the host waits, instead of idling while the host issues it afterwards
-            unit_dirs = _unit_directions(ray_d)
             use_tilecenter = self._resolve_tile_order_mode() == "tilecenter"
             ext = self._ensure_tile_ext()
             own_lists = (culled_prim_indices is None and tile_offsets is None and view_matrix is not None
@@ -669,10 +666,13 @@ class NeuralPrimitiveSceneTileCUDA(nn.Module):
                          and getattr(self, "camera_mode", "legacy-centered") != "colmap-native")
             if (own_lists and use_tilecenter and ts == 8 and not return_feature and feature_target is None
                     and getattr(self, "queued_frames", True) and hasattr(ext, "render_frame_queued")):
-                done = self._forward_queued(ext, ray_o, unit_dirs, score_threshold, view_matrix, proj_matrix, bg_color,
+                done = self._forward_queued(ext, ray_o, ray_d, score_threshold, view_matrix, proj_matrix, bg_color,
                                             device)
                 if done is not None:
                     return done
+            # queued before the binning, whose pair count is a blocking read-back: the device then has
+            # this work to do while the host waits, instead of idling while the host issues it afterwards
+            unit_dirs = _unit_directions(ray_d)
             culled_prim_indices, tile_offsets = self._tile_lists(
                 ray_o, ray_d, score_threshold, view_matrix, proj_matrix, culled_prim_indices, tile_offsets, device)
             if own_lists and hasattr(ext, "note_frame_pairs"):
@@ -789,25 +789,34 @@ class NeuralPrimitiveSceneTileCUDA(nn.Module):
             float(self.feature_gating_temp), int(W), int(H), ts, ts, float(score_threshold),
             self._background(bg_color, ray_o))
 
-    def _forward_queued(self, ext, ray_o, unit_dirs, score_threshold, view_matrix, proj_matrix, bg_color, device):
+    def _forward_queued(self, ext, ray_o, ray_d, score_threshold, view_matrix, proj_matrix, bg_color, device):
         """The RGB frame with binning, sort and render queued back to back and one read-back at the end
         (``TileExt.render_frame_queued``); None when that path does not apply or has to be repeated the
-        synchronous way.  Same images and errors as the step-by-step path."""
+        synchronous way.  Same images and errors as the step-by-step path.  The binning goes first: it needs only
+        the primitives and the camera, and the device is busy with it while the host prepares the rest of the
+        frame (unit ray directions, tables, weights)."""
         precision = str(getattr(self, "render_precision", "f32")).lower()
         if precision not in {"f32", "bf16", "fp16"}:
             raise ValueError(f"Unsupported render_precision {precision!r}; use 'f32', 'bf16' or 'fp16'.")
         if precision != "f32" and not (int(self.hidden_dim) == 32 and int(self.pe_frequencies) == 6):
             precision = "f32"
-        W, H = self.image_size
-        freq, att = self._frequency_tables(device)
         ws = [p.detach().contiguous() for p in (self.W1, self.b1, self.W2, self.b2, self.W3, self.b3)]
         half = all(w.dtype == torch.float16 for w in ws)
         if any(w.dtype != torch.float32 for w in ws) and not (half and precision != "f32"):
             return None                       # stored half-precision weights: only the matrix-core frame reads them as they are
-        out = ext.render_frame_queued(ray_o.contiguous(), unit_dirs, self.positions.detach().contiguous(),
-                                      self.log_scales.detach().contiguous(), self._unit_quats(), freq, att, ws,
-                                      _frame_matrix(view_matrix).reshape(1, 4, 4), _frame_matrix(proj_matrix), int(W),
-                                      int(H), float(score_threshold), precision)
+        W, H = self.image_size
+        positions, log_scales = self.positions.detach().contiguous(), self.log_scales.detach().contiguous()
+        views, proj = _frame_matrix(view_matrix).reshape(1, 4, 4), _frame_matrix(proj_matrix)
+        binned = None
+        if hasattr(ext, "frame_binning_queued"):
+            binned = ext.frame_binning_queued(positions, log_scales, views, proj, int(W), int(H), float(score_threshold))
+            if binned is None:
+                return None
+        unit_dirs = _unit_directions(ray_d)
+        freq, att = self._frequency_tables(device)
+        out = ext.render_frame_queued(ray_o.contiguous(), unit_dirs, positions, log_scales, self._unit_quats(), freq, att,
+                                      ws, views, proj, int(W), int(H), float(score_threshold), precision,
+                                      **({"binned": binned} if binned is not None else {}))
         if out is None:
             return None
         return _add_background(out[0], out[1], self._background(bg_color, ray_o))

@@ -308,30 +308,47 @@ class TileExt:
     # ------------------------------------------------------------------------------------------
     # a whole frame queued without a host synchronisation in its middle (no counterpart in the reference)
     # ------------------------------------------------------------------------------------------
+    def frame_binning_queued(self, positions, log_scales, view_matrices, proj_matrix, width, height, threshold):
+        """First half of :meth:`render_frame_queued`: the frame's binning, queued.  It needs nothing but the
+        primitives and the camera, so a caller queues it before it prepares anything else for the frame (ray
+        directions, weights): the device works through the binning while the host does that.  Returns what
+        :meth:`render_frame_queued` takes as ``binned``, or None when no candidate-buffer estimate exists yet."""
+        with self._lock:
+            cap, scale = self._queue_capacity, self._queue_scratch_scale
+        if cap <= 0:
+            return None
+        with _on_device(positions.device):
+            # counts of the binning (4 x int64) and flag words of the render (16 x int32) share one buffer: the
+            # frame's single read-back is one 96-byte copy
+            tail = torch.empty(96, dtype=torch.uint8, device=positions.device)
+            cand, offsets, counts = ops.bin_legacy_async(positions, log_scales, view_matrices, proj_matrix, int(width),
+                                                         int(height), 8, float(threshold), cap, scratch_scale=scale,
+                                                         counts=tail[:32].view(torch.int64))
+        return cand, offsets, counts, tail, cap, scale
+
     def render_frame_queued(self, rays_o, unit_dirs, positions, log_scales, unit_quats, freq, att, ws, view_matrices,
-                            proj_matrix, width, height, threshold, precision):
+                            proj_matrix, width, height, threshold, precision, binned=None):
         """(rgb, alpha) of one 8x8-tile, tile-centre-order RGB frame: binning, sort and render are queued
         back to back and ONE read-back at the end brings the pair count, the longest tile list and the
         non-finite flag.  The candidate buffer is sized from the previous frame's count; if this frame
         needs more (or the level-1 scratch overflows) every list was left empty on the device: the
         estimate is enlarged and None is returned, and the caller renders the frame the synchronous way.
+        ``binned``: the result of :meth:`frame_binning_queued` for the same primitives and camera, when the caller
+        has queued the binning already.
         Errors are those of the entry points it stands for (capacity text of np_tile_kernels.cu:4578-4588,
         fallback policy of rgb_wmma.cuh:260-272)."""
         name = "render_tiles_rgb_wmma" if precision != "f32" else "render_tiles_forward_tilecenter"
         width, height, threshold = int(width), int(height), float(threshold)
-        with self._lock:
-            cap, scale = self._queue_capacity, self._queue_scratch_scale
-        if cap <= 0:
-            return None
+        if binned is None:
+            binned = self.frame_binning_queued(positions, log_scales, view_matrices, proj_matrix, width, height,
+                                               threshold)
+            if binned is None:
+                return None
+        cand, offsets, counts, tail, cap, scale = binned
+        status = tail[32:].view(torch.int32)
         n = positions.shape[0]
         with _on_device(rays_o.device):
             rec = self._records(positions, log_scales, unit_quats)
-            # counts of the binning (4 x int64) and flag words of the render (16 x int32) share one buffer: the
-            # frame's single read-back is one 96-byte copy
-            tail = torch.empty(96, dtype=torch.uint8, device=rays_o.device)
-            counts, status = tail[:32].view(torch.int64), tail[32:].view(torch.int32)
-            cand, offsets, counts = ops.bin_legacy_async(positions, log_scales, view_matrices, proj_matrix, width,
-                                                         height, 8, threshold, cap, scratch_scale=scale, counts=counts)
             order, _ = ops.sort_tiles(rays_o, unit_dirs, rec, cand, offsets, width, height, 8, 8, _lib.KEY_TSTAR,
                                       self.max_tile_prims, cull_threshold=threshold)
             if precision != "f32":
