@@ -650,14 +650,16 @@ class NeuralPrimitiveSceneTileCUDA(nn.Module):
         if feature_target is not None:
             return self._forward_csr_training(ray_o, ray_d, score_threshold, bg_color, view_matrix, proj_matrix,
                                               culled_prim_indices, tile_offsets, return_feature, feature_target, device)
-        trainable = (self.positions, self.log_scales, self.quats, self.W1, self.b1, self.W2, self.b2, self.W3, self.b3)
-        if torch.is_grad_enabled() and return_feature and self.feat_attr is not None:
-            if any(t.requires_grad for t in (*trainable, self.feat_attr)):
-                return self._forward_differentiable_with_feat(ray_o, ray_d, score_threshold, bg_color, view_matrix,
-                                                              proj_matrix, culled_prim_indices, tile_offsets, device)
-        elif torch.is_grad_enabled() and any(t.requires_grad for t in trainable):
-            return self._forward_differentiable(ray_o, ray_d, score_threshold, bg_color, view_matrix, proj_matrix,
-                                                culled_prim_indices, tile_offsets, return_feature, device)
+        if torch.is_grad_enabled():
+            trainable = (self.positions, self.log_scales, self.quats, self.W1, self.b1, self.W2, self.b2, self.W3,
+                         self.b3)
+            if return_feature and self.feat_attr is not None:
+                if any(t.requires_grad for t in (*trainable, self.feat_attr)):
+                    return self._forward_differentiable_with_feat(ray_o, ray_d, score_threshold, bg_color, view_matrix,
+                                                                  proj_matrix, culled_prim_indices, tile_offsets, device)
+            elif any(t.requires_grad for t in trainable):
+                return self._forward_differentiable(ray_o, ray_d, score_threshold, bg_color, view_matrix, proj_matrix,
+                                                    culled_prim_indices, tile_offsets, return_feature, device)
         with torch.no_grad():
             use_tilecenter = self._resolve_tile_order_mode() == "tilecenter"
             ext = self._ensure_tile_ext()
@@ -800,10 +802,11 @@ class NeuralPrimitiveSceneTileCUDA(nn.Module):
             raise ValueError(f"Unsupported render_precision {precision!r}; use 'f32', 'bf16' or 'fp16'.")
         if precision != "f32" and not (int(self.hidden_dim) == 32 and int(self.pe_frequencies) == 6):
             precision = "f32"
-        ws = [p.detach().contiguous() for p in (self.W1, self.b1, self.W2, self.b2, self.W3, self.b3)]
-        half = all(w.dtype == torch.float16 for w in ws)
-        if any(w.dtype != torch.float32 for w in ws) and not (half and precision != "f32"):
-            return None                       # stored half-precision weights: only the matrix-core frame reads them as they are
+        params = (self.W1, self.b1, self.W2, self.b2, self.W3, self.b3)
+        if any(w.dtype != torch.float32 for w in params):
+            half = all(w.dtype == torch.float16 for w in params)
+            if not (half and precision != "f32"):
+                return None                   # stored half-precision weights: only the matrix-core frame reads them as they are
         W, H = self.image_size
         positions, log_scales = self.positions.detach().contiguous(), self.log_scales.detach().contiguous()
         views, proj = _frame_matrix(view_matrix).reshape(1, 4, 4), _frame_matrix(proj_matrix)
@@ -812,6 +815,7 @@ class NeuralPrimitiveSceneTileCUDA(nn.Module):
             binned = ext.frame_binning_queued(positions, log_scales, views, proj, int(W), int(H), float(score_threshold))
             if binned is None:
                 return None
+        ws = [p.detach().contiguous() for p in params]
         unit_dirs = _unit_directions(ray_d)
         freq, att = self._frequency_tables(device)
         out = ext.render_frame_queued(ray_o.contiguous(), unit_dirs, positions, log_scales, self._unit_quats(), freq, att,

@@ -26,7 +26,9 @@ def _ptr(t):
 
 
 def _stream(device):
-    return C.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+    """The raw handle of torch's current stream on ``device`` (the launches of a call go there)."""
+    index = device.index if device.index is not None else torch.cuda.current_device()
+    return C.c_void_p(torch._C._cuda_getCurrentRawStream(index))
 
 
 def _f32c(t, name):
