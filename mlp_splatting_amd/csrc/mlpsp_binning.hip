@@ -16,6 +16,7 @@
 #include "mlpsp_host.hpp"
 
 #include <math.h>
+#include <stdlib.h>
 
 namespace mlpsp {
 
@@ -89,15 +90,10 @@ struct BinMats {
 // MODE 2: one view, the view matrix at `mats` and the projection at `proj_dev` (device tensors of the caller: no
 // host copy of them exists, so the focal length is formed here, with the host's expression).
 template <int MODE>
-__global__ __launch_bounds__(kBinThreads) void bin_bounds_kernel(const float* __restrict__ pos,
-                                                                 const float* __restrict__ logs,
-                                                                 const float* __restrict__ mats,
-                                                                 const float* __restrict__ proj_dev, BinMats one,
-                                                                 BinGeom g, float rm, float focal,
-                                                                 float4* __restrict__ bounds) {
-  const int i = blockIdx.x * blockDim.x + threadIdx.x;
-  const int k = blockIdx.y;
-  if (i >= g.N) return;
+__device__ __forceinline__ float4 primitive_bounds(const float* __restrict__ pos, const float* __restrict__ logs,
+                                                   const float* __restrict__ mats, const float* __restrict__ proj_dev,
+                                                   const BinMats& one, const BinGeom& g, float rm, float focal, int i,
+                                                   int k) {
   const float* V = MODE == 1 ? one.v : mats + k * 16;
   const float* Pm = MODE == 1 ? one.p : MODE == 2 ? proj_dev : mats + g.K * 16;
   if (MODE == 2) focal = ((Pm[0] * (float)g.W) / 2.0f + (Pm[5] * (float)g.H) / 2.0f) * 0.5f;
@@ -118,7 +114,20 @@ __global__ __launch_bounds__(kBinThreads) void bin_bounds_kernel(const float* __
   const float sy = (((clip[1] / w) + 1.f) * 0.5f) * (float)g.H;
   const float nan = __builtin_nanf("");
   const bool front = depth > 0.001f;
-  bounds[(size_t)k * g.N + i] = front ? make_float4(sx - pr, sx + pr, sy - pr, sy + pr) : make_float4(nan, nan, nan, nan);
+  return front ? make_float4(sx - pr, sx + pr, sy - pr, sy + pr) : make_float4(nan, nan, nan, nan);
+}
+
+template <int MODE>
+__global__ __launch_bounds__(kBinThreads) void bin_bounds_kernel(const float* __restrict__ pos,
+                                                                 const float* __restrict__ logs,
+                                                                 const float* __restrict__ mats,
+                                                                 const float* __restrict__ proj_dev, BinMats one,
+                                                                 BinGeom g, float rm, float focal,
+                                                                 float4* __restrict__ bounds) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  const int k = blockIdx.y;
+  if (i >= g.N) return;
+  bounds[(size_t)k * g.N + i] = primitive_bounds<MODE>(pos, logs, mats, proj_dev, one, g, rm, focal, i, k);
 }
 
 // strict inequalities of scannet/cumodel.py:1043-1044 on an axis-aligned pixel rectangle
@@ -146,6 +155,27 @@ __device__ __forceinline__ unsigned long long lane_value(unsigned long long v, i
   const unsigned lo = __builtin_amdgcn_readlane((unsigned)v, which);
   const unsigned hi = __builtin_amdgcn_readlane((unsigned)(v >> 32), which);
   return ((unsigned long long)hi << 32) | lo;
+}
+
+// position of the n-th (from 0) set bit of m; n < popcount(m)
+__device__ __forceinline__ int nth_set_bit(unsigned long long m, int n) {
+  unsigned x = (unsigned)m;
+  int pos = 0, c = __popc(x);
+  if (n >= c) {
+    n -= c;
+    pos = 32;
+    x = (unsigned)(m >> 32);
+  }
+#pragma unroll
+  for (int width = 16; width >= 1; width >>= 1) {
+    c = __popc(x & ((1u << width) - 1u));
+    if (n >= c) {
+      n -= c;
+      pos += width;
+      x >>= width;
+    }
+  }
+  return pos;
 }
 
 __device__ __forceinline__ unsigned lanes_below(unsigned long long mask) {
@@ -197,21 +227,41 @@ __global__ __launch_bounds__(kBinThreads) void bin_level1_kernel(const float4* _
   unsigned long long* __restrict__ masks = l1_masks + ((size_t)s * g.NC + c) * (kChunk / 64);
   static_assert(kChunk / 64 <= 64, "one ballot per lane");
   if constexpr (FILL) {
-    // the counting pass left one ballot per 64 primitives: no bounds are read again except the survivors'.
-    // Lane r fetches ballot r (one coalesced load instead of a chain of dependent ones).
+    // The counting pass left one ballot per 64 primitives: no bounds are read again except the survivors'.  Lane r
+    // fetches ballot r (one coalesced load), the ballots' bit counts are scanned, and then lane k writes the k-th
+    // survivor: it finds the ballot that holds it (a search over the scanned counts) and the bit inside.  All
+    // survivors' bounds are gathered at once -- one memory latency per 64 survivors; walking the ballots one after
+    // the other instead costs one per ballot that is not empty.
     const unsigned long long mine = lane < kChunk / 64 ? masks[lane] : 0ull;
-    for (int r = 0; r < kChunk / 64; ++r) {
-      const unsigned long long m = lane_value(mine, r);
-      if (m == 0ull) continue;
-      if ((m >> lane) & 1ull) {
-        const int i = first + r * 64 + lane;
-        const long long dst = running + lanes_below(m);
+    const int own = __popcll(mine);
+    int incl = own;
+#pragma unroll
+    for (int d = 1; d < kChunk / 64; d <<= 1) {
+      const int up = __shfl_up(incl, d);
+      if (lane >= d) incl += up;
+    }
+    const int before = incl - own;                     // survivors in the ballots ahead of this lane's
+    const int total = __shfl(incl, kChunk / 64 - 1);
+    static_assert(kChunk / 64 == 32, "the search below halves 32 ballots");
+    for (int k0 = 0; k0 < total; k0 += 64) {
+      const int k = k0 + lane;
+      int r = 0;                                       // the last ballot whose `before` is <= k holds survivor k
+#pragma unroll
+      for (int step = 16; step >= 1; step >>= 1) {
+        const int ahead = __shfl(before, r + step);
+        if (ahead <= k) r += step;
+      }
+      const int nth = k - __shfl(before, r);
+      const unsigned long long m = ((unsigned long long)(unsigned)__shfl((int)(mine >> 32), r) << 32) |
+                                   (unsigned)__shfl((int)mine, r);
+      if (k < total) {
+        const int i = first + r * 64 + nth_set_bit(m, nth);
+        const long long dst = running + k;
         if (dst < l1_capacity) {
           l1_list[dst] = i;
           if (single) l1_bounds[dst] = sb[i];
         }
       }
-      running += __popcll(m);
     }
     return;
   }
@@ -257,6 +307,119 @@ __global__ __launch_bounds__(kBinThreads) void bin_level1_kernel(const float4* _
   }
   if (lane < kChunk / 64) masks[lane] = mine;
   if (lane == 0) l1_counts[s * g.NC + c] = (int32_t)running;
+}
+
+// The counting pass of level 1 for one view and a screen of at most kScatterMaxSuper super-tiles: by primitive
+// instead of by (chunk, super-tile), and with the bounds computed on the way (every primitive is visited exactly
+// once, so this is also the bounds kernel).  The walk above tests every primitive against every super-tile (N x S
+// rectangle tests); here one workgroup per chunk lets each primitive find the few super-tiles it overlaps and set
+// its bit in that super-tile's row of an LDS bitmap [S][kChunk bits].  The rows are the very ballots the walk
+// produces: they are stored where the walk stores them, counted, and the walk's fill pass writes the lists from
+// them (it writes consecutive list positions from consecutive lanes; a fill by primitive scatters 20-byte stores and
+// measured slower).  Dynamic LDS: scatter_lds_bytes(S) -- the bitmap and the list of wide primitives.
+constexpr int kScatterThreads = 1024;
+constexpr int kScatterMaxSuper = 400;
+constexpr int kWordsPerRow = kChunk / 64;
+__host__ __device__ constexpr size_t scatter_lds_bytes(int S) {
+  return (size_t)S * kWordsPerRow * sizeof(unsigned long long) + kChunk * sizeof(uint2);
+}
+
+// super-tile columns (rows) a [lo, hi] pixel interval overlaps under rect_overlap's strict inequalities: [a, b],
+// empty when a > b.  n: super-tiles along the axis, nt: tiles along it.  Column k spans [x0(k), x1(k)) pixels and
+// passes when lo < x1(k) and hi > x0(k); x0 and x1 grow with k, so a is the first k with lo < x1(k) and b the last
+// with hi > x0(k).  Both are estimated from a division, moved by one where the comparison itself says so, and
+// checked against their definition; the walk over all columns is the fallback that the check never asks for in
+// practice but that makes the result exact whatever the rounding of the estimate.
+__device__ __forceinline__ void super_range(float lo, float hi, int n, int nt, int ts, int& a, int& b) {
+  a = 0;
+  b = -1;
+  if (lo != lo || hi != hi) return;      // behind the near plane: NaN bounds overlap nothing
+  const float inv = 1.f / (float)(kSuper * ts);
+  auto x0 = [&](int k) { return (float)(k * kSuper * ts); };
+  auto x1 = [&](int k) { return (float)(min((k + 1) * kSuper, nt) * ts); };
+  int ea = (int)fmaxf(fminf(floorf(lo * inv), (float)n), 0.f);
+  if (ea > 0 && lo < x1(ea - 1)) --ea;
+  else if (ea < n && !(lo < x1(ea))) ++ea;
+  int eb = (int)fmaxf(fminf(floorf(hi * inv), (float)(n - 1)), -1.f);
+  if (eb < n - 1 && hi > x0(eb + 1)) ++eb;
+  else if (eb >= 0 && !(hi > x0(eb))) --eb;
+  const bool a_ok = (ea == n || lo < x1(ea)) && (ea == 0 || !(lo < x1(ea - 1)));
+  const bool b_ok = (eb == -1 || hi > x0(eb)) && (eb == n - 1 || !(hi > x0(eb + 1)));
+  if (!(a_ok && b_ok)) {
+    ea = n;
+    eb = -1;
+    for (int k = 0; k < n; ++k) {
+      if ((lo < x1(k)) && (hi > x0(k))) {
+        ea = min(ea, k);
+        eb = k;
+      }
+    }
+  }
+  a = ea;
+  b = eb;
+}
+
+template <int MODE>
+__global__ __launch_bounds__(kScatterThreads) void bin_level1_scatter_kernel(
+    const float* __restrict__ pos, const float* __restrict__ logs, const float* __restrict__ mats,
+    const float* __restrict__ proj_dev, BinMats one, BinGeom g, float rm, float focal, float4* __restrict__ bounds,
+    int32_t* __restrict__ l1_counts, int32_t* __restrict__ super_view, unsigned long long* __restrict__ l1_masks) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char s_raw[];
+  const int S = g.nsx * g.nsy;
+  unsigned long long* __restrict__ bits = reinterpret_cast<unsigned long long*>(s_raw);      // [S][kWordsPerRow]
+  uint2* __restrict__ wide = reinterpret_cast<uint2*>(bits + (size_t)S * kWordsPerRow);       // [kChunk]: p, and xa xb ya yb one byte each
+  __shared__ int s_nwide;
+  const int c = blockIdx.x, t = threadIdx.x, lane = t & 63, wave = t >> 6;
+  for (int w = t; w < S * kWordsPerRow; w += kScatterThreads) bits[w] = 0ull;
+  if (t == 0) s_nwide = 0;
+  __syncthreads();
+  // A primitive that overlaps more than kNarrow super-tiles is not walked by its own thread (the workgroup would wait
+  // for the few threads that hold such primitives): it goes on a list, and a whole wavefront walks its super-tiles.
+  constexpr int kNarrow = 4;
+  constexpr int kPer = kChunk / kScatterThreads;     // primitives per thread
+#pragma unroll
+  for (int u = 0; u < kPer; ++u) {
+    const int p = t + u * kScatterThreads, i = c * kChunk + p;
+    if (i < g.N) {
+      const float4 bb = primitive_bounds<MODE>(pos, logs, mats, proj_dev, one, g, rm, focal, i, 0);
+      bounds[i] = bb;
+      int xa, xb, ya, yb;
+      super_range(bb.x, bb.y, g.nsx, g.ntx, g.ts, xa, xb);
+      super_range(bb.z, bb.w, g.nsy, g.nty, g.ts, ya, yb);
+      if (xa > xb) yb = ya - 1;      // (no column: no row either)
+      if ((xb - xa + 1) * (yb - ya + 1) > kNarrow) {
+        wide[atomicAdd(&s_nwide, 1)] = make_uint2((unsigned)p, (unsigned)xa | ((unsigned)xb << 8) |
+                                                                   ((unsigned)ya << 16) | ((unsigned)yb << 24));
+        yb = ya - 1;                        // not walked by this thread
+      }
+      for (int sy = ya; sy <= yb; ++sy)
+        for (int sx = xa; sx <= xb; ++sx)
+          atomicOr(&bits[(size_t)(sy * g.nsx + sx) * kWordsPerRow + (p >> 6)], 1ull << (p & 63));
+    }
+  }
+  __syncthreads();
+  const int nwide = s_nwide;
+  for (int e = wave; e < nwide; e += kScatterThreads / 64) {
+    const uint2 we = wide[e];
+    const int p = (int)we.x, wxa = we.y & 255, wxb = (we.y >> 8) & 255, wya = (we.y >> 16) & 255, wyb = we.y >> 24;
+    const int nx = wxb - wxa + 1, cells = nx * (wyb - wya + 1);
+    for (int k = lane; k < cells; k += 64)
+      atomicOr(&bits[(size_t)((wya + k / nx) * g.nsx + wxa + k % nx) * kWordsPerRow + (p >> 6)], 1ull << (p & 63));
+  }
+  __syncthreads();
+  // 32 lanes per row: lane w of the group holds word w of the row
+  static_assert(kWordsPerRow == 32, "a row is handled by half a wavefront");
+  const int w = t & 31;
+  for (int row = t >> 5; row < S; row += kScatterThreads / 32) {
+    const unsigned long long word = bits[(size_t)row * kWordsPerRow + w];
+    l1_masks[((size_t)row * g.NC + c) * kWordsPerRow + w] = word;
+    int n = __popcll(word);
+#pragma unroll
+    for (int d = 16; d >= 1; d >>= 1) n += __shfl_xor(n, d);
+    if (w == 0) l1_counts[row * g.NC + c] = n;
+  }
+  if (c == 0)
+    for (int k = t; k < S; k += kScatterThreads) super_view[k] = 0;
 }
 
 // In-place exclusive scan of data[0..n) by one workgroup; data[n] and *total receive the sum, *largest
@@ -492,18 +655,87 @@ MLPSP_API size_t mlpsp_bin_scratch_bytes(int num_primitives, int num_views, int 
 }
 
 namespace {
-// level 1 (count, scan, fill) -> level 2 count -> scan, behind the bounds kernel
-int enqueue_bin_levels(const BinGeom& g, const BinScratch& b, int64_t T, const int32_t* tile_view_ids_dev,
-                       int32_t* tile_offsets_dev, hipStream_t s, ScanGuard guard) {
+// MLPSP_BIN_LEVEL1_WALK=1 keeps the counting pass of level 1 on the (chunk, super-tile) walk where the by-primitive
+// kernel would apply (for comparing the two; read once)
+bool level1_walk_forced() {
+  static const bool forced = [] {
+    const char* v = getenv("MLPSP_BIN_LEVEL1_WALK");
+    return v && v[0] == '1';
+  }();
+  return forced;
+}
+
+// the by-primitive counting kernel uses more dynamic LDS than a kernel may without saying so: said once per device
+int allow_scatter_lds() {
+  constexpr int kMaxDevices = 64;
+  static bool done[kMaxDevices];
+  int dev = -1;
+  MLPSP_HIP_TRY(hipGetDevice(&dev));
+  if (dev < 0 || dev >= kMaxDevices) return MLPSP_E_ARGUMENT;
+  if (!__atomic_load_n(&done[dev], __ATOMIC_ACQUIRE)) {
+    const int bytes = (int)scatter_lds_bytes(kScatterMaxSuper);
+    MLPSP_HIP_TRY(hipFuncSetAttribute((const void*)bin_level1_scatter_kernel<1>,
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, bytes));
+    MLPSP_HIP_TRY(hipFuncSetAttribute((const void*)bin_level1_scatter_kernel<2>,
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, bytes));
+    __atomic_store_n(&done[dev], true, __ATOMIC_RELEASE);
+  }
+  return MLPSP_OK;
+}
+
+// what the bounds of a frame are computed from (bin_bounds_kernel's arguments)
+struct BoundsSource {
+  const float* positions;
+  const float* log_scales;
+  int mode;                 // bin_bounds_kernel's MODE
+  const float* mats;        // mode 0: K views then the projection; mode 2: the view matrix
+  const float* proj_dev;    // mode 2
+  BinMats one;              // mode 1
+  float rm, focal;
+};
+
+// bounds -> level 1 (count, scan, fill) -> level 2 count -> scan
+int enqueue_bin_levels(const BoundsSource& src, const BinGeom& g, const BinScratch& b, int64_t T,
+                       const int32_t* tile_view_ids_dev, int32_t* tile_offsets_dev, hipStream_t s, ScanGuard guard) {
   const int S = g.nsx * g.nsy;
-  hipLaunchKernelGGL((bin_level1_kernel<false>), dim3(g.NC, ceil_div(S, kBinThreads / 64)), dim3(kBinThreads), 0, s, b.bounds, g,
-                     tile_view_ids_dev, b.l1_counts, b.l1_list, b.l1_bounds, b.l1_capacity, b.l1_masks, b.super_view);
+  // one view on a screen of few super-tiles: bounds and level-1 counts in one launch, by primitive
+  const bool scatter = g.K == 1 && src.mode != 0 && S <= kScatterMaxSuper && g.nsx < 256 && g.nsy < 256 &&
+                       !level1_walk_forced();
+  if (scatter) {
+    const int rc = allow_scatter_lds();
+    if (rc != MLPSP_OK) return rc;
+    const size_t lds = scatter_lds_bytes(S);
+    if (src.mode == 1)
+      hipLaunchKernelGGL(bin_level1_scatter_kernel<1>, dim3(g.NC), dim3(kScatterThreads), lds, s, src.positions,
+                         src.log_scales, src.mats, src.proj_dev, src.one, g, src.rm, src.focal, b.bounds, b.l1_counts,
+                         b.super_view, b.l1_masks);
+    else
+      hipLaunchKernelGGL(bin_level1_scatter_kernel<2>, dim3(g.NC), dim3(kScatterThreads), lds, s, src.positions,
+                         src.log_scales, src.mats, src.proj_dev, src.one, g, src.rm, src.focal, b.bounds, b.l1_counts,
+                         b.super_view, b.l1_masks);
+  } else {
+    const dim3 grid(ceil_div(g.N, kBinThreads), src.mode == 0 ? g.K : 1), block(kBinThreads);
+    if (src.mode == 0)
+      hipLaunchKernelGGL(bin_bounds_kernel<0>, grid, block, 0, s, src.positions, src.log_scales, src.mats, src.proj_dev,
+                         src.one, g, src.rm, src.focal, b.bounds);
+    else if (src.mode == 1)
+      hipLaunchKernelGGL(bin_bounds_kernel<1>, grid, block, 0, s, src.positions, src.log_scales, src.mats, src.proj_dev,
+                         src.one, g, src.rm, src.focal, b.bounds);
+    else
+      hipLaunchKernelGGL(bin_bounds_kernel<2>, grid, block, 0, s, src.positions, src.log_scales, src.mats, src.proj_dev,
+                         src.one, g, src.rm, src.focal, b.bounds);
+    MLPSP_LAUNCH_CHECK();
+    hipLaunchKernelGGL((bin_level1_kernel<false>), dim3(g.NC, ceil_div(S, kBinThreads / 64)), dim3(kBinThreads), 0, s,
+                       b.bounds, g, tile_view_ids_dev, b.l1_counts, b.l1_list, b.l1_bounds, b.l1_capacity, b.l1_masks,
+                       b.super_view);
+  }
   MLPSP_LAUNCH_CHECK();
   hipLaunchKernelGGL(exclusive_scan_kernel, dim3(1), dim3(1024), 0, s, b.l1_counts, S * g.NC, b.totals,
                      (long long*)nullptr, ScanGuard{nullptr, nullptr, 0, 0});
   MLPSP_LAUNCH_CHECK();
-  hipLaunchKernelGGL((bin_level1_kernel<true>), dim3(g.NC, ceil_div(S, kBinThreads / 64)), dim3(kBinThreads), 0, s, b.bounds, g,
-                     tile_view_ids_dev, b.l1_counts, b.l1_list, b.l1_bounds, b.l1_capacity, b.l1_masks, b.super_view);
+  hipLaunchKernelGGL((bin_level1_kernel<true>), dim3(g.NC, ceil_div(S, kBinThreads / 64)), dim3(kBinThreads), 0, s,
+                     b.bounds, g, tile_view_ids_dev, b.l1_counts, b.l1_list, b.l1_bounds, b.l1_capacity, b.l1_masks,
+                     b.super_view);
   MLPSP_LAUNCH_CHECK();
   hipLaunchKernelGGL((bin_level2_kernel<false>), dim3(ceil_div((int)T, kBinThreads / 64)), dim3(kBinThreads), 0, s,
                      b.bounds, g, tile_view_ids_dev, b.l1_counts, b.l1_list, b.l1_bounds, b.l1_capacity, tile_offsets_dev,
@@ -523,39 +755,36 @@ int enqueue_bin_count(const float* positions_dev, const float* log_scales_dev, i
                       const BinScratch& b, int64_t T, int32_t* tile_offsets_dev, hipStream_t s,
                       bool matrices_in_scratch = false, ScanGuard guard = ScanGuard{nullptr, nullptr, 0, 0},
                       const float* view_dev = nullptr, const float* proj_dev = nullptr) {
-  const int S = g.nsx * g.nsy;
+  BoundsSource src{};
+  src.positions = positions_dev;
+  src.log_scales = log_scales_dev;
   // scalar constants in f32, in the order the reference's tensor expressions evaluate them
-  const float rm = sqrtf(-2.0f * logf(threshold));
-  BinMats one{};
-  if (view_dev) {             // one view, matrices on the device
-    hipLaunchKernelGGL(bin_bounds_kernel<2>, dim3(ceil_div(num_primitives, kBinThreads), 1), dim3(kBinThreads), 0, s,
-                       positions_dev, log_scales_dev, view_dev, proj_dev, one, g, rm, 0.f, b.bounds);
-    MLPSP_LAUNCH_CHECK();
-    return enqueue_bin_levels(g, b, T, tile_view_ids_dev, tile_offsets_dev, s, guard);
+  src.rm = sqrtf(-2.0f * logf(threshold));
+  if (view_dev) {             // one view, matrices on the device (the kernel forms the focal length)
+    src.mode = 2;
+    src.mats = view_dev;
+    src.proj_dev = proj_dev;
+    return enqueue_bin_levels(src, g, b, T, tile_view_ids_dev, tile_offsets_dev, s, guard);
   }
   const float fx = (proj_host[0] * (float)width) / 2.0f, fy = (proj_host[5] * (float)height) / 2.0f;
-  const float focal = (fx + fy) * 0.5f;
+  src.focal = (fx + fy) * 0.5f;
   if (num_views == 1) {
+    src.mode = 1;
     for (int e = 0; e < 16; ++e) {
-      one.v[e] = view_matrices_host[e];
-      one.p[e] = proj_host[e];
+      src.one.v[e] = view_matrices_host[e];
+      src.one.p[e] = proj_host[e];
     }
-    hipLaunchKernelGGL(bin_bounds_kernel<1>, dim3(ceil_div(num_primitives, kBinThreads), 1), dim3(kBinThreads), 0, s,
-                       positions_dev, log_scales_dev, (const float*)nullptr, (const float*)nullptr, one, g, rm, focal,
-                       b.bounds);
   } else {
+    src.mode = 0;
+    src.mats = b.mats;
     if (!matrices_in_scratch) {
       MLPSP_HIP_TRY(hipMemcpyAsync(b.mats, view_matrices_host, (size_t)num_views * 16 * sizeof(float),
                                    hipMemcpyHostToDevice, s));
       MLPSP_HIP_TRY(hipMemcpyAsync(b.mats + (size_t)num_views * 16, proj_host, 16 * sizeof(float),
                                    hipMemcpyHostToDevice, s));
     }
-    hipLaunchKernelGGL(bin_bounds_kernel<0>, dim3(ceil_div(num_primitives, kBinThreads), num_views),
-                       dim3(kBinThreads), 0, s, positions_dev, log_scales_dev, b.mats, (const float*)nullptr, one, g, rm,
-                       focal, b.bounds);
   }
-  MLPSP_LAUNCH_CHECK();
-  return enqueue_bin_levels(g, b, T, tile_view_ids_dev, tile_offsets_dev, s, guard);
+  return enqueue_bin_levels(src, g, b, T, tile_view_ids_dev, tile_offsets_dev, s, guard);
 }
 
 int check_bin_args(int64_t T, const float* view_matrices_host, const float* proj_host, void* scratch_dev,
