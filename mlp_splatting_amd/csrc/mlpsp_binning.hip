@@ -6,7 +6,9 @@
 //   level 1: the frame is cut into super-tiles of 8x8 tiles.  Wavefront (chunk c, super-tile s)
 //            tests 2048 consecutive primitives against the super-tile rectangle (a superset of the
 //            union of its tiles' tests), counts, and after a scan writes the survivors in ascending
-//            id order -> one ascending candidate list per super-tile.
+//            id order -> one ascending candidate list per super-tile.  With one view and a screen of
+//            few super-tiles the counting goes the other way round: every primitive finds the
+//            super-tiles it overlaps (bin_level1_scatter_kernel, which also computes the bounds).
 //   level 2: one wavefront per tile walks its super-tile's list 64 ids at a time, applies the exact
 //            per-tile test, counts with a ballot, and after a scan writes the tile's candidates at
 //            ballot-prefix positions -> tile-major lists, ascending id inside a tile, which is the
