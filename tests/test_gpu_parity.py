@@ -57,6 +57,24 @@ def test_binning_ragged_frames_and_tile_sizes(device, oracle_mod, width, height,
     np.testing.assert_array_equal(cand.cpu().numpy(), want[0])
 
 
+@pytest.mark.parametrize("n,grow", [(4500, 2.5), (2049, 4.0), (1, 3.0), (63, 0.0)])
+def test_binning_with_primitives_that_span_many_super_tiles(device, oracle_mod, n, grow):
+    """Level 1 by primitive hands every primitive that overlaps more than four super-tiles to a whole wavefront: here
+    (log-scales raised by `grow`) most or all primitives of a 2048-chunk are such, on a 20-super-tile screen, and the
+    chunk boundaries fall at 2048 + 1 and inside a single wavefront."""
+    from mlp_splatting_amd import ops
+    fr = Frame("cfg1_5k_160x120", n=n, width=320, height=200, eye=(0.2, 0.1, -1.0), target=(0, 0, 0.2))
+    sc = fr.scene
+    logs = (sc.log_scales + np.float32(grow)).astype(np.float32)
+    want = oracle_mod.bin_legacy(sc.positions, logs, fr.view[None], fr.proj, fr.W, fr.H, 8, fr.thr)
+    cand, off = ops.bin_legacy(_t(sc.positions, device), _t(logs, device), torch.from_numpy(fr.view)[None],
+                               torch.from_numpy(fr.proj), fr.W, fr.H, 8, fr.thr)
+    if grow >= 2.5 and n > 1000:
+        assert want[0].size > 100 * n          # (a primitive lands in hundreds of tiles: the case is what it says)
+    np.testing.assert_array_equal(off.cpu().numpy(), want[1])
+    np.testing.assert_array_equal(cand.cpu().numpy(), want[0])
+
+
 def test_tile_view_binning_matches_oracle(device, oracle_mod):
     from mlp_splatting_amd import ops, synthetic as syn
     fr = Frame("cfg1_5k_160x120", n=4000, width=96, height=64)
