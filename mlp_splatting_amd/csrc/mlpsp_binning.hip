@@ -311,7 +311,7 @@ __global__ __launch_bounds__(kBinThreads) void bin_level1_kernel(const float4* _
   if (lane == 0) l1_counts[s * g.NC + c] = (int32_t)running;
 }
 
-// The counting pass of level 1 for one view and a screen of at most kScatterMaxSuper super-tiles: by primitive
+// The counting pass of level 1 for one view, in bands of at most kScatterMaxSuper super-tiles: by primitive
 // instead of by (chunk, super-tile), and with the bounds computed on the way (every primitive is visited exactly
 // once, so this is also the bounds kernel).  The walk above tests every primitive against every super-tile (N x S
 // rectangle tests); here one workgroup per chunk lets each primitive find the few super-tiles it overlaps and set
@@ -361,15 +361,19 @@ __device__ __forceinline__ void super_range(float lo, float hi, int n, int nt, i
   b = eb;
 }
 
+// grid = (NC, bands): workgroup (c, band) handles chunk c and the super-tile rows [band * band_rows, + band_rows), so
+// that the bitmap of any screen fits LDS (every band computes the chunk's bounds; band 0 stores them).
 template <int MODE>
 __global__ __launch_bounds__(kScatterThreads) void bin_level1_scatter_kernel(
     const float* __restrict__ pos, const float* __restrict__ logs, const float* __restrict__ mats,
-    const float* __restrict__ proj_dev, BinMats one, BinGeom g, float rm, float focal, float4* __restrict__ bounds,
-    int32_t* __restrict__ l1_counts, int32_t* __restrict__ super_view, unsigned long long* __restrict__ l1_masks) {
+    const float* __restrict__ proj_dev, BinMats one, BinGeom g, float rm, float focal, int band_rows,
+    float4* __restrict__ bounds, int32_t* __restrict__ l1_counts, int32_t* __restrict__ super_view,
+    unsigned long long* __restrict__ l1_masks) {
   extern __shared__ __attribute__((aligned(16))) unsigned char s_raw[];
-  const int S = g.nsx * g.nsy;
+  const int row0 = blockIdx.y * band_rows, rows = min(band_rows, g.nsy - row0);
+  const int S = g.nsx * rows;                          // super-tiles of this band; the first is row0 * nsx
   unsigned long long* __restrict__ bits = reinterpret_cast<unsigned long long*>(s_raw);      // [S][kWordsPerRow]
-  uint2* __restrict__ wide = reinterpret_cast<uint2*>(bits + (size_t)S * kWordsPerRow);       // [kChunk]: p, and xa xb ya yb one byte each
+  uint2* __restrict__ wide = reinterpret_cast<uint2*>(bits + (size_t)g.nsx * band_rows * kWordsPerRow);   // [kChunk]: p, and xa xb ya yb (ya, yb from row0) one byte each
   __shared__ int s_nwide;
   const int c = blockIdx.x, t = threadIdx.x, lane = t & 63, wave = t >> 6;
   for (int w = t; w < S * kWordsPerRow; w += kScatterThreads) bits[w] = 0ull;
@@ -384,11 +388,13 @@ __global__ __launch_bounds__(kScatterThreads) void bin_level1_scatter_kernel(
     const int p = t + u * kScatterThreads, i = c * kChunk + p;
     if (i < g.N) {
       const float4 bb = primitive_bounds<MODE>(pos, logs, mats, proj_dev, one, g, rm, focal, i, 0);
-      bounds[i] = bb;
+      if (blockIdx.y == 0) bounds[i] = bb;
       int xa, xb, ya, yb;
       super_range(bb.x, bb.y, g.nsx, g.ntx, g.ts, xa, xb);
       super_range(bb.z, bb.w, g.nsy, g.nty, g.ts, ya, yb);
-      if (xa > xb) yb = ya - 1;      // (no column: no row either)
+      ya = max(ya, row0) - row0;           // rows of this band only, counted from its first row
+      yb = min(yb, row0 + rows - 1) - row0;
+      if (xa > xb) yb = ya - 1;            // (no column: no row either)
       if ((xb - xa + 1) * (yb - ya + 1) > kNarrow) {
         wide[atomicAdd(&s_nwide, 1)] = make_uint2((unsigned)p, (unsigned)xa | ((unsigned)xb << 8) |
                                                                    ((unsigned)ya << 16) | ((unsigned)yb << 24));
@@ -411,17 +417,17 @@ __global__ __launch_bounds__(kScatterThreads) void bin_level1_scatter_kernel(
   __syncthreads();
   // 32 lanes per row: lane w of the group holds word w of the row
   static_assert(kWordsPerRow == 32, "a row is handled by half a wavefront");
-  const int w = t & 31;
+  const int w = t & 31, first = row0 * g.nsx;
   for (int row = t >> 5; row < S; row += kScatterThreads / 32) {
     const unsigned long long word = bits[(size_t)row * kWordsPerRow + w];
-    l1_masks[((size_t)row * g.NC + c) * kWordsPerRow + w] = word;
+    l1_masks[((size_t)(first + row) * g.NC + c) * kWordsPerRow + w] = word;
     int n = __popcll(word);
 #pragma unroll
     for (int d = 16; d >= 1; d >>= 1) n += __shfl_xor(n, d);
-    if (w == 0) l1_counts[row * g.NC + c] = n;
+    if (w == 0) l1_counts[(first + row) * g.NC + c] = n;
   }
   if (c == 0)
-    for (int k = t; k < S; k += kScatterThreads) super_view[k] = 0;
+    for (int k = t; k < S; k += kScatterThreads) super_view[first + k] = 0;
 }
 
 // In-place exclusive scan of data[0..n) by one workgroup; data[n] and *total receive the sum, *largest
@@ -700,21 +706,22 @@ struct BoundsSource {
 int enqueue_bin_levels(const BoundsSource& src, const BinGeom& g, const BinScratch& b, int64_t T,
                        const int32_t* tile_view_ids_dev, int32_t* tile_offsets_dev, hipStream_t s, ScanGuard guard) {
   const int S = g.nsx * g.nsy;
-  // one view on a screen of few super-tiles: bounds and level-1 counts in one launch, by primitive
-  const bool scatter = g.K == 1 && src.mode != 0 && S <= kScatterMaxSuper && g.nsx < 256 && g.nsy < 256 &&
-                       !level1_walk_forced();
+  // one view: bounds and level-1 counts in one launch, by primitive (super-tile rows in bands that fit LDS)
+  const bool scatter = g.K == 1 && src.mode != 0 && g.nsx <= kScatterMaxSuper && g.nsx < 256 && !level1_walk_forced();
   if (scatter) {
     const int rc = allow_scatter_lds();
     if (rc != MLPSP_OK) return rc;
-    const size_t lds = scatter_lds_bytes(S);
+    const int band_rows = min(min(g.nsy, kScatterMaxSuper / g.nsx), 255);
+    const size_t lds = scatter_lds_bytes(g.nsx * band_rows);
+    const dim3 grid(g.NC, ceil_div(g.nsy, band_rows));
     if (src.mode == 1)
-      hipLaunchKernelGGL(bin_level1_scatter_kernel<1>, dim3(g.NC), dim3(kScatterThreads), lds, s, src.positions,
-                         src.log_scales, src.mats, src.proj_dev, src.one, g, src.rm, src.focal, b.bounds, b.l1_counts,
-                         b.super_view, b.l1_masks);
+      hipLaunchKernelGGL(bin_level1_scatter_kernel<1>, grid, dim3(kScatterThreads), lds, s, src.positions,
+                         src.log_scales, src.mats, src.proj_dev, src.one, g, src.rm, src.focal, band_rows, b.bounds,
+                         b.l1_counts, b.super_view, b.l1_masks);
     else
-      hipLaunchKernelGGL(bin_level1_scatter_kernel<2>, dim3(g.NC), dim3(kScatterThreads), lds, s, src.positions,
-                         src.log_scales, src.mats, src.proj_dev, src.one, g, src.rm, src.focal, b.bounds, b.l1_counts,
-                         b.super_view, b.l1_masks);
+      hipLaunchKernelGGL(bin_level1_scatter_kernel<2>, grid, dim3(kScatterThreads), lds, s, src.positions,
+                         src.log_scales, src.mats, src.proj_dev, src.one, g, src.rm, src.focal, band_rows, b.bounds,
+                         b.l1_counts, b.super_view, b.l1_masks);
   } else {
     const dim3 grid(ceil_div(g.N, kBinThreads), src.mode == 0 ? g.K : 1), block(kBinThreads);
     if (src.mode == 0)

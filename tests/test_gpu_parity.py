@@ -43,9 +43,10 @@ def test_binning_matches_oracle_bit_exactly(device, oracle_mod, frame1):
     assert cand.dtype == torch.int32 and off.dtype == torch.int32
 
 
-# (the last frame has 504 super-tiles: more than the by-primitive counting pass of level 1 takes, so it runs the
-# walk over (chunk, super-tile) pairs that multi-view frames run too)
-@pytest.mark.parametrize("width,height,tile", [(100, 76, 8), (100, 76, 16), (33, 17, 8), (3000, 2600, 16)])
+# (the last two frames have 504 and 510 super-tiles: more than one LDS bitmap of the by-primitive counting pass of
+# level 1 holds, so it runs in two bands of super-tile rows)
+@pytest.mark.parametrize("width,height,tile", [(100, 76, 8), (100, 76, 16), (33, 17, 8), (3000, 2600, 16),
+                                               (1920, 1080, 8)])
 def test_binning_ragged_frames_and_tile_sizes(device, oracle_mod, width, height, tile):
     from mlp_splatting_amd import ops
     fr = Frame("cfg1_5k_160x120", n=3000, width=width, height=height, tile=tile, eye=(1.0, 0.8, -1.2), target=(0, 0, 0))
