@@ -322,8 +322,10 @@ __global__ __launch_bounds__(kBinThreads) void bin_level1_kernel(const float4* _
 constexpr int kScatterThreads = 1024;
 constexpr int kScatterMaxSuper = 400;
 constexpr int kWordsPerRow = kChunk / 64;
+constexpr int kScatterWide = 2 * kChunk;     // entries of the list of wide (primitive, view) pairs
+constexpr int kScatterMaxViews = 32;
 __host__ __device__ constexpr size_t scatter_lds_bytes(int S) {
-  return (size_t)S * kWordsPerRow * sizeof(unsigned long long) + kChunk * sizeof(uint2);
+  return (size_t)S * (kWordsPerRow * sizeof(unsigned long long) + sizeof(unsigned)) + kScatterWide * sizeof(uint2);
 }
 
 // super-tile columns (rows) a [lo, hi] pixel interval overlaps under rect_overlap's strict inequalities: [a, b],
@@ -363,56 +365,95 @@ __device__ __forceinline__ void super_range(float lo, float hi, int n, int nt, i
 
 // grid = (NC, bands): workgroup (c, band) handles chunk c and the super-tile rows [band * band_rows, + band_rows), so
 // that the bitmap of any screen fits LDS (every band computes the chunk's bounds; band 0 stores them).
+// MODE 1, 2: one view, bounds computed here (bin_bounds_kernel's modes).  MODE 0: several views (at most 32) with
+// tile_view_ids; the bounds of all views come from bin_bounds_kernel, the workgroup first collects which views the
+// tiles of each of its super-tiles use, and a primitive sets its bit in a super-tile when its rectangle under one of
+// THOSE views overlaps it (the walk tests the same views, or all of them when a super-tile uses more than four: the
+// lists are a superset either way, and level 2 applies each tile's own view).
 template <int MODE>
 __global__ __launch_bounds__(kScatterThreads) void bin_level1_scatter_kernel(
     const float* __restrict__ pos, const float* __restrict__ logs, const float* __restrict__ mats,
     const float* __restrict__ proj_dev, BinMats one, BinGeom g, float rm, float focal, int band_rows,
-    float4* __restrict__ bounds, int32_t* __restrict__ l1_counts, int32_t* __restrict__ super_view,
-    unsigned long long* __restrict__ l1_masks) {
+    const int32_t* __restrict__ tile_view_ids, float4* __restrict__ bounds, int32_t* __restrict__ l1_counts,
+    int32_t* __restrict__ super_view, unsigned long long* __restrict__ l1_masks) {
   extern __shared__ __attribute__((aligned(16))) unsigned char s_raw[];
   const int row0 = blockIdx.y * band_rows, rows = min(band_rows, g.nsy - row0);
   const int S = g.nsx * rows;                          // super-tiles of this band; the first is row0 * nsx
+  const int smax = g.nsx * band_rows;
   unsigned long long* __restrict__ bits = reinterpret_cast<unsigned long long*>(s_raw);      // [S][kWordsPerRow]
-  uint2* __restrict__ wide = reinterpret_cast<uint2*>(bits + (size_t)g.nsx * band_rows * kWordsPerRow);   // [kChunk]: p, and xa xb ya yb (ya, yb from row0) one byte each
+  // wide primitives: (p | view << 16, xa xb ya yb one byte each, ya and yb counted from row0)
+  uint2* __restrict__ wide = reinterpret_cast<uint2*>(bits + (size_t)smax * kWordsPerRow);
+  unsigned* __restrict__ views = reinterpret_cast<unsigned*>(wide + kScatterWide);            // [S] (MODE 0)
   __shared__ int s_nwide;
   const int c = blockIdx.x, t = threadIdx.x, lane = t & 63, wave = t >> 6;
   for (int w = t; w < S * kWordsPerRow; w += kScatterThreads) bits[w] = 0ull;
+  if (MODE == 0)
+    for (int k = t; k < S; k += kScatterThreads) views[k] = 0u;
   if (t == 0) s_nwide = 0;
   __syncthreads();
+  if (MODE == 0) {
+    // one item = one row of 8 tiles of a super-tile
+    for (int item = t; item < S * kSuper; item += kScatterThreads) {
+      const int sl = item / kSuper, ty = (row0 + sl / g.nsx) * kSuper + item % kSuper, tx0 = (sl % g.nsx) * kSuper;
+      unsigned m = 0u;
+      if (ty < g.nty) {
+#pragma unroll
+        for (int j = 0; j < kSuper; ++j) {
+          const int v = (tx0 + j < g.ntx) ? tile_view_ids[ty * g.ntx + tx0 + j] : -1;
+          m |= ((unsigned)v < (unsigned)g.K) ? (1u << v) : 0u;
+        }
+      }
+      if (m) atomicOr(&views[sl], m);
+    }
+    __syncthreads();
+  }
   // A primitive that overlaps more than kNarrow super-tiles is not walked by its own thread (the workgroup would wait
   // for the few threads that hold such primitives): it goes on a list, and a whole wavefront walks its super-tiles.
   constexpr int kNarrow = 4;
   constexpr int kPer = kChunk / kScatterThreads;     // primitives per thread
+  auto mark = [&](int cell, int p, int view) {
+    if (MODE != 0 || ((views[cell] >> view) & 1u))
+      atomicOr(&bits[(size_t)cell * kWordsPerRow + (p >> 6)], 1ull << (p & 63));
+  };
 #pragma unroll
   for (int u = 0; u < kPer; ++u) {
     const int p = t + u * kScatterThreads, i = c * kChunk + p;
     if (i < g.N) {
-      const float4 bb = primitive_bounds<MODE>(pos, logs, mats, proj_dev, one, g, rm, focal, i, 0);
-      if (blockIdx.y == 0) bounds[i] = bb;
-      int xa, xb, ya, yb;
-      super_range(bb.x, bb.y, g.nsx, g.ntx, g.ts, xa, xb);
-      super_range(bb.z, bb.w, g.nsy, g.nty, g.ts, ya, yb);
-      ya = max(ya, row0) - row0;           // rows of this band only, counted from its first row
-      yb = min(yb, row0 + rows - 1) - row0;
-      if (xa > xb) yb = ya - 1;            // (no column: no row either)
-      if ((xb - xa + 1) * (yb - ya + 1) > kNarrow) {
-        wide[atomicAdd(&s_nwide, 1)] = make_uint2((unsigned)p, (unsigned)xa | ((unsigned)xb << 8) |
-                                                                   ((unsigned)ya << 16) | ((unsigned)yb << 24));
-        yb = ya - 1;                        // not walked by this thread
+      for (int view = 0; view < (MODE == 0 ? g.K : 1); ++view) {
+        float4 bb;
+        if (MODE == 0) {
+          bb = bounds[(size_t)view * g.N + i];
+        } else {
+          bb = primitive_bounds<MODE>(pos, logs, mats, proj_dev, one, g, rm, focal, i, 0);
+          if (blockIdx.y == 0) bounds[i] = bb;
+        }
+        int xa, xb, ya, yb;
+        super_range(bb.x, bb.y, g.nsx, g.ntx, g.ts, xa, xb);
+        super_range(bb.z, bb.w, g.nsy, g.nty, g.ts, ya, yb);
+        ya = max(ya, row0) - row0;           // rows of this band only, counted from its first row
+        yb = min(yb, row0 + rows - 1) - row0;
+        if (xa > xb) yb = ya - 1;            // (no column: no row either)
+        if ((xb - xa + 1) * (yb - ya + 1) > kNarrow) {
+          const int slot = atomicAdd(&s_nwide, 1);
+          if (slot < kScatterWide) {         // (a full list: the thread walks the primitive after all)
+            wide[slot] = make_uint2((unsigned)p | ((unsigned)view << 16), (unsigned)xa | ((unsigned)xb << 8) |
+                                                                              ((unsigned)ya << 16) | ((unsigned)yb << 24));
+            yb = ya - 1;
+          }
+        }
+        for (int sy = ya; sy <= yb; ++sy)
+          for (int sx = xa; sx <= xb; ++sx) mark(sy * g.nsx + sx, p, view);
       }
-      for (int sy = ya; sy <= yb; ++sy)
-        for (int sx = xa; sx <= xb; ++sx)
-          atomicOr(&bits[(size_t)(sy * g.nsx + sx) * kWordsPerRow + (p >> 6)], 1ull << (p & 63));
     }
   }
   __syncthreads();
-  const int nwide = s_nwide;
+  const int nwide = min(s_nwide, kScatterWide);
   for (int e = wave; e < nwide; e += kScatterThreads / 64) {
     const uint2 we = wide[e];
-    const int p = (int)we.x, wxa = we.y & 255, wxb = (we.y >> 8) & 255, wya = (we.y >> 16) & 255, wyb = we.y >> 24;
+    const int p = (int)(we.x & 0xffffu), view = (int)(we.x >> 16);
+    const int wxa = we.y & 255, wxb = (we.y >> 8) & 255, wya = (we.y >> 16) & 255, wyb = we.y >> 24;
     const int nx = wxb - wxa + 1, cells = nx * (wyb - wya + 1);
-    for (int k = lane; k < cells; k += 64)
-      atomicOr(&bits[(size_t)((wya + k / nx) * g.nsx + wxa + k % nx) * kWordsPerRow + (p >> 6)], 1ull << (p & 63));
+    for (int k = lane; k < cells; k += 64) mark((wya + k / nx) * g.nsx + wxa + k % nx, p, view);
   }
   __syncthreads();
   // 32 lanes per row: lane w of the group holds word w of the row
@@ -426,8 +467,12 @@ __global__ __launch_bounds__(kScatterThreads) void bin_level1_scatter_kernel(
     for (int d = 16; d >= 1; d >>= 1) n += __shfl_xor(n, d);
     if (w == 0) l1_counts[(first + row) * g.NC + c] = n;
   }
-  if (c == 0)
-    for (int k = t; k < S; k += kScatterThreads) super_view[first + k] = 0;
+  if (c == 0) {
+    for (int k = t; k < S; k += kScatterThreads) {
+      const unsigned m = MODE == 0 ? views[k] : 1u;
+      super_view[first + k] = (__popc(m) == 1) ? (int)__builtin_ctz(m) : -1;
+    }
+  }
 }
 
 // In-place exclusive scan of data[0..n) by one workgroup; data[n] and *total receive the sum, *largest
@@ -682,6 +727,8 @@ int allow_scatter_lds() {
   if (dev < 0 || dev >= kMaxDevices) return MLPSP_E_ARGUMENT;
   if (!__atomic_load_n(&done[dev], __ATOMIC_ACQUIRE)) {
     const int bytes = (int)scatter_lds_bytes(kScatterMaxSuper);
+    MLPSP_HIP_TRY(hipFuncSetAttribute((const void*)bin_level1_scatter_kernel<0>,
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, bytes));
     MLPSP_HIP_TRY(hipFuncSetAttribute((const void*)bin_level1_scatter_kernel<1>,
                                       hipFuncAttributeMaxDynamicSharedMemorySize, bytes));
     MLPSP_HIP_TRY(hipFuncSetAttribute((const void*)bin_level1_scatter_kernel<2>,
@@ -706,23 +753,12 @@ struct BoundsSource {
 int enqueue_bin_levels(const BoundsSource& src, const BinGeom& g, const BinScratch& b, int64_t T,
                        const int32_t* tile_view_ids_dev, int32_t* tile_offsets_dev, hipStream_t s, ScanGuard guard) {
   const int S = g.nsx * g.nsy;
-  // one view: bounds and level-1 counts in one launch, by primitive (super-tile rows in bands that fit LDS)
-  const bool scatter = g.K == 1 && src.mode != 0 && g.nsx <= kScatterMaxSuper && g.nsx < 256 && !level1_walk_forced();
-  if (scatter) {
-    const int rc = allow_scatter_lds();
-    if (rc != MLPSP_OK) return rc;
-    const int band_rows = min(min(g.nsy, kScatterMaxSuper / g.nsx), 255);
-    const size_t lds = scatter_lds_bytes(g.nsx * band_rows);
-    const dim3 grid(g.NC, ceil_div(g.nsy, band_rows));
-    if (src.mode == 1)
-      hipLaunchKernelGGL(bin_level1_scatter_kernel<1>, grid, dim3(kScatterThreads), lds, s, src.positions,
-                         src.log_scales, src.mats, src.proj_dev, src.one, g, src.rm, src.focal, band_rows, b.bounds,
-                         b.l1_counts, b.super_view, b.l1_masks);
-    else
-      hipLaunchKernelGGL(bin_level1_scatter_kernel<2>, grid, dim3(kScatterThreads), lds, s, src.positions,
-                         src.log_scales, src.mats, src.proj_dev, src.one, g, src.rm, src.focal, band_rows, b.bounds,
-                         b.l1_counts, b.super_view, b.l1_masks);
-  } else {
+  // level-1 counts by primitive (super-tile rows in bands that fit LDS): with one view the same launch computes the
+  // bounds, with several (and tile_view_ids) it reads them
+  const bool one_view = g.K == 1 && src.mode != 0;
+  const bool many_views = src.mode == 0 && g.K > 1 && g.K <= kScatterMaxViews && tile_view_ids_dev != nullptr;
+  const bool scatter = (one_view || many_views) && g.nsx <= kScatterMaxSuper && g.nsx < 256 && !level1_walk_forced();
+  if (!scatter || many_views) {
     const dim3 grid(ceil_div(g.N, kBinThreads), src.mode == 0 ? g.K : 1), block(kBinThreads);
     if (src.mode == 0)
       hipLaunchKernelGGL(bin_bounds_kernel<0>, grid, block, 0, s, src.positions, src.log_scales, src.mats, src.proj_dev,
@@ -734,6 +770,22 @@ int enqueue_bin_levels(const BoundsSource& src, const BinGeom& g, const BinScrat
       hipLaunchKernelGGL(bin_bounds_kernel<2>, grid, block, 0, s, src.positions, src.log_scales, src.mats, src.proj_dev,
                          src.one, g, src.rm, src.focal, b.bounds);
     MLPSP_LAUNCH_CHECK();
+  }
+  if (scatter) {
+    const int rc = allow_scatter_lds();
+    if (rc != MLPSP_OK) return rc;
+    const int band_rows = min(min(g.nsy, kScatterMaxSuper / g.nsx), 255);
+    const size_t lds = scatter_lds_bytes(g.nsx * band_rows);
+    const dim3 grid(g.NC, ceil_div(g.nsy, band_rows));
+#define MLPSP_SCATTER(M)                                                                                             \
+  hipLaunchKernelGGL(bin_level1_scatter_kernel<M>, grid, dim3(kScatterThreads), lds, s, src.positions, src.log_scales, \
+                     src.mats, src.proj_dev, src.one, g, src.rm, src.focal, band_rows, tile_view_ids_dev, b.bounds,    \
+                     b.l1_counts, b.super_view, b.l1_masks)
+    if (src.mode == 0) MLPSP_SCATTER(0);
+    else if (src.mode == 1) MLPSP_SCATTER(1);
+    else MLPSP_SCATTER(2);
+#undef MLPSP_SCATTER
+  } else {
     hipLaunchKernelGGL((bin_level1_kernel<false>), dim3(g.NC, ceil_div(S, kBinThreads / 64)), dim3(kBinThreads), 0, s,
                        b.bounds, g, tile_view_ids_dev, b.l1_counts, b.l1_list, b.l1_bounds, b.l1_capacity, b.l1_masks,
                        b.super_view);
