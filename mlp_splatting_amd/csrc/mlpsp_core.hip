@@ -103,6 +103,12 @@ __global__ __launch_bounds__(kSortThreads) void sort_tiles_kernel(
     float cull_r2, int num_prims, int32_t* __restrict__ sorted_ids, float* __restrict__ sorted_keys) {
   const int tile = superblock_tile(blockIdx.x, g.ntx, g.nty);
   if (tile < 0) return;
+  const int start = offsets[tile], len = offsets[tile + 1] - start;
+  if (len <= 64 && len <= capacity) {       // a short list: the first wavefront alone, in registers
+    if (len > 0 && threadIdx.x < 64)
+      sort_small_tile(rays_o, rays_d, prims, cand, g, family, cull_r2, num_prims, sorted_ids, sorted_keys, tile, start, len);
+    return;
+  }
   __shared__ SortLds<MLPSP_TILE_CAPACITY_MAX> lds;
   sort_one_tile<MLPSP_TILE_CAPACITY_MAX>(lds, rays_o, rays_d, prims, cand, offsets, g, family, capacity, cull_r2, num_prims,
                                          sorted_ids, sorted_keys, tile);

@@ -40,6 +40,120 @@ struct SortLds {
   int flags, pairs;
 };
 
+// A tile whose list has at most 64 entries, sorted by ONE wavefront (lane = entry) in registers: no LDS, no barrier.
+// Same output as sort_one_tile() -- the kept entries ordered by their (key bits, list position) words, which also
+// puts keys at or above the invalid key last and in list order among equals; culled entries as ~id at the end of
+// the tile's output, last one first -- at a fifth of its instructions: for short lists sort_one_tile()'s cost is
+// what four wavefronts spend per tile whatever its length (the pyramid built four times, the passes of the bucket
+// ranking, a dozen barriers).  The pyramid and the per-candidate test are those of sort_one_tile(), statement for
+// statement.  Requires len <= 64 and len <= capacity; called by a whole wavefront.
+__device__ __forceinline__ void sort_small_tile(
+    const float* __restrict__ rays_o, const float* __restrict__ rays_d, const PrimRecord* __restrict__ prims,
+    const int32_t* __restrict__ cand, const TileGeom& g, int family, float cull_r2, int num_prims,
+    int32_t* __restrict__ sorted_ids, float* __restrict__ sorted_keys, int tile, int start, int n) {
+  const int lane = threadIdx.x & 63;
+  const int pc = centre_pixel(g, tile);
+  const float ox = rays_o[pc * 3 + 0], oy = rays_o[pc * 3 + 1], oz = rays_o[pc * 3 + 2];
+  const float dx = rays_d[pc * 3 + 0], dy = rays_d[pc * 3 + 1], dz = rays_d[pc * 3 + 2];
+  const int p = (lane < n) ? cand[start + lane] : 0;
+  const bool known = (unsigned)p < (unsigned)num_prims;
+  const PrimRecord P = prims[known ? p : 0];
+
+  float pox = 0.f, poy = 0.f, poz = 0.f;
+  float pn[4][3] = {};
+  int faces = 0;
+  if (cull_r2 > 0.f) {
+    const int tx = tile % g.ntx, ty = tile / g.ntx;
+    const int x0 = tx * g.TW, y0 = ty * g.TH;
+    const int x1 = min(x0 + g.TW, g.W) - 1, y1 = min(y0 + g.TH, g.H) - 1;
+    const int corner[4] = {y0 * g.W + x0, y0 * g.W + x1, y1 * g.W + x1, y1 * g.W + x0};
+    float cd[4][3];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int c = 0; c < 3; ++c) cd[j][c] = rays_d[corner[j] * 3 + c];
+    pox = rays_o[corner[0] * 3 + 0];
+    poy = rays_o[corner[0] * 3 + 1];
+    poz = rays_o[corner[0] * 3 + 2];
+    int ok = 0x1f;                                       // bits 0..3: face usable; bit 4: common origin
+    float nlen[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {                        // face j from corner rays j and j+1
+      const float* a = cd[j];
+      const float* b = cd[(j + 1) & 3];
+      const float nx = a[1] * b[2] - a[2] * b[1], ny = a[2] * b[0] - a[0] * b[2], nz = a[0] * b[1] - a[1] * b[0];
+      const float side = nx * dx + ny * dy + nz * dz;
+      const float len = sqrtf(nx * nx + ny * ny + nz * nz);
+      const float sgn = side < 0.f ? -1.f : 1.f;
+      pn[j][0] = sgn * nx;
+      pn[j][1] = sgn * ny;
+      pn[j][2] = sgn * nz;
+      nlen[j] = sqrtf(pn[j][0] * pn[j][0] + pn[j][1] * pn[j][1] + pn[j][2] * pn[j][2]);
+      if (!(len > 0.f && fabsf(side) > 1e-4f * len)) ok &= ~(1 << j);
+    }
+    for (int k = lane; k < g.TW * g.TH; k += 64) {
+      const int x = x0 + k % g.TW, y = y0 + k / g.TW;
+      if (x < g.W && y < g.H) {
+        const int pix = y * g.W + x;
+        if (rays_o[pix * 3] != pox || rays_o[pix * 3 + 1] != poy || rays_o[pix * 3 + 2] != poz) ok &= ~0x10;
+        const float rx = rays_d[pix * 3], ry = rays_d[pix * 3 + 1], rz = rays_d[pix * 3 + 2];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const float inside = pn[j][0] * rx + pn[j][1] * ry + pn[j][2] * rz;
+          if (!(inside >= -1e-6f * nlen[j])) ok &= ~(1 << j);
+        }
+      }
+    }
+    int all_ok = 0;
+#pragma unroll
+    for (int b = 0; b < 5; ++b) all_ok |= __ballot(!((ok >> b) & 1)) ? 0 : (1 << b);
+    faces = (all_ok & 0x10) ? (all_ok & 0xf) : 0;
+  }
+
+  bool keep = false;
+  float key = 0.f;
+  if (lane < n) {
+    bool outside = false;
+    if (faces && known) {
+      const float ex = P.cx - pox, ey = P.cy - poy, ez = P.cz - poz;
+      const float qw = P.qw, qx = -P.qx, qy = -P.qy, qz = -P.qz;       // conjugate: world -> local
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float nx = pn[j][0], ny = pn[j][1], nz = pn[j][2];
+        const float dist = fmaf(nx, ex, fmaf(ny, ey, nz * ez));
+        const float tx = 2.f * fmaf(qy, nz, -(qz * ny)), ty = 2.f * fmaf(qz, nx, -(qx * nz)),
+                    tz = 2.f * fmaf(qx, ny, -(qy * nx));
+        const float lx = fmaf(qw, tx, nx) + fmaf(qy, tz, -(qz * ty));
+        const float ly = fmaf(qw, ty, ny) + fmaf(qz, tx, -(qx * tz));
+        const float lz = fmaf(qw, tz, nz) + fmaf(qx, ty, -(qy * tx));
+        const float h2 = fmaf(P.s2x, lx * lx, fmaf(P.s2y, ly * ly, P.s2z * (lz * lz)));
+        outside |= ((faces >> j) & 1) && (dist < 0.f) && (dist * dist >= cull_r2 * h2);
+      }
+    }
+    keep = !outside;
+    if (keep)
+      key = !known ? kInvalidKey
+                   : (family == MLPSP_KEY_DEPTH) ? key_depth(ox, oy, oz, dx, dy, dz, P) : key_tstar(ox, oy, oz, dx, dy, dz, P);
+  }
+  const uint32_t kb = float_to_bits(key);
+  const unsigned long long kept = __ballot(keep);
+  int rank = 0;                                          // kept words below this lane's
+  for (unsigned long long m = kept; m != 0ull; m &= m - 1ull) {
+    const int j = (int)__builtin_ctzll(m);
+    const uint32_t kj = (uint32_t)__builtin_amdgcn_readlane((int)kb, j);
+    rank += (kj < kb || (kj == kb && j < lane)) ? 1 : 0;
+  }
+  if (keep) {
+    sorted_ids[start + rank] = p;
+    if (sorted_keys) sorted_keys[start + rank] = key;
+  } else if (lane < n) {
+    const unsigned long long culled_before = ~kept & ((1ull << lane) - 1ull);
+    const int pos = start + n - 1 - __popcll(culled_before);
+    sorted_ids[pos] = ~p;
+    if (sorted_keys) sorted_keys[pos] = kInvalidKey;
+  }
+}
+
 // Sorts one tile with the calling 256-thread workgroup (every thread must call it; `tile` is uniform).  kSortMax
 // bounds `capacity`.  A workgroup that sorts several tiles in a row, or uses `lds` for something else afterwards,
 // puts a barrier in between.
