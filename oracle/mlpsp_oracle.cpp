@@ -605,7 +605,7 @@ ORACLE_API int64_t mlpsp_oracle_bin_legacy(const float* pos, const float* logs, 
       for (int ty = y0; ty <= y1; ++ty)
         for (int tx = x0; tx <= x1; ++tx) {
           const int t = ty * ntx + tx;
-          if (tile_view_ids && tile_view_ids[t] != k) continue;
+          if ((tile_view_ids ? tile_view_ids[t] : 0) != k) continue;   // (without ids every tile uses view 0)
           if (!overlaps(b, tx, ty, ts)) continue;
           if (cand) cand[cursor[t]++] = i; else cursor[t + 1]++;
         }

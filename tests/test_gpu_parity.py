@@ -76,6 +76,23 @@ def test_binning_with_primitives_that_span_many_super_tiles(device, oracle_mod, 
     np.testing.assert_array_equal(cand.cpu().numpy(), want[0])
 
 
+def test_binning_with_several_views_and_no_view_per_tile(device, oracle_mod):
+    """Several view matrices without tile_view_ids: every tile is binned against view 0 (level 1 then runs the walk
+    over (chunk, super-tile) pairs with all the views, a superset that level 2 cuts down)."""
+    from mlp_splatting_amd import ops, synthetic as syn
+    fr = Frame("cfg1_5k_160x120", n=5000, width=200, height=136)
+    sc = fr.scene
+    views = np.stack([fr.view, syn.view_matrix(syn.look_at((1.0, 0.3, -0.8), (0, 0, 0)))]).astype(np.float32)
+    want = oracle_mod.bin_legacy(sc.positions, sc.log_scales, views, fr.proj, fr.W, fr.H, 8, fr.thr)
+    cand, off = ops.bin_legacy(_t(sc.positions, device), _t(sc.log_scales, device), torch.from_numpy(views),
+                               torch.from_numpy(fr.proj), fr.W, fr.H, 8, fr.thr)
+    assert want[0].size > 1000
+    np.testing.assert_array_equal(off.cpu().numpy(), want[1])
+    np.testing.assert_array_equal(cand.cpu().numpy(), want[0])
+    one = oracle_mod.bin_legacy(sc.positions, sc.log_scales, views[:1], fr.proj, fr.W, fr.H, 8, fr.thr)
+    np.testing.assert_array_equal(one[0], want[0])
+
+
 def test_tile_view_binning_matches_oracle(device, oracle_mod):
     from mlp_splatting_amd import ops, synthetic as syn
     fr = Frame("cfg1_5k_160x120", n=4000, width=96, height=64)

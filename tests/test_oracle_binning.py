@@ -31,6 +31,21 @@ def test_sparse_binning_equals_dense_brute_force(oracle_mod, eye, target, tile):
     np.testing.assert_array_equal(cand, c2)          # tile-major, ascending id inside a tile
 
 
+def test_several_views_without_view_ids_bin_against_view_zero(oracle_mod):
+    """K view matrices and no per-tile view ids: every tile uses view 0, in the sparse form as in the dense one."""
+    from mlp_splatting_amd import synthetic as syn
+    fr = Frame("cfg1_5k_160x120", n=1500, width=100, height=76)
+    sc = fr.scene
+    views = np.stack([fr.view, syn.view_matrix(syn.look_at((1.0, 0.3, -0.8), (0, 0, 0)))]).astype(np.float32)
+    cand, off = oracle_mod.bin_legacy(sc.positions, sc.log_scales, views, fr.proj, fr.W, fr.H, 8, fr.thr)
+    c2, o2 = _lists_from_mask(oracle_mod.bin_legacy_dense(sc.positions, sc.log_scales, views, fr.proj, fr.W, fr.H, 8, fr.thr))
+    one = oracle_mod.bin_legacy(sc.positions, sc.log_scales, views[:1], fr.proj, fr.W, fr.H, 8, fr.thr)
+    assert cand.size > 1000
+    np.testing.assert_array_equal(off, o2)
+    np.testing.assert_array_equal(cand, c2)
+    np.testing.assert_array_equal(cand, one[0])
+
+
 def _torch_dense_rule(pos, log_s, view, proj, W, H, ts, thr):
     """The reference's culling as tensor expressions (scannet/cumodel.py:996-1046), written here with
     torch on the CPU as an independent check of the oracle's scalar restatement."""
