@@ -168,16 +168,21 @@ def test_sorted_tile_lists_match_oracle_keys_and_order(device, oracle_mod, frame
     _assert_bits(keys, want_keys, "sort keys")
 
 
-@pytest.mark.parametrize("case", ["spread", "ties", "behind", "clusters", "beyond_invalid", "two", "capacity"])
+@pytest.mark.parametrize("case", ["spread", "ties", "behind", "clusters", "beyond_invalid", "two", "capacity",
+                                  "ties:64", "behind:64", "beyond_invalid:63", "spread:65", "clusters:1"])
 @pytest.mark.parametrize("family", [1, 2])
 def test_sort_is_the_stable_key_order_for_every_key_distribution(device, oracle_mod, case, family):
     """One 8x8 tile with a hand-made list.  The kernel ranks survivors inside 256 key buckets and falls back to a
     sorting network when keys pile up in few buckets or a key exceeds the invalid key; each case below steers it
-    down one of those routes, and the result must be the oracle's stable sort by key every time."""
+    down one of those routes, and the result must be the oracle's stable sort by key every time.  A list of at most
+    64 entries is sorted by one wavefront in registers: the cases with a length after the colon go that way (65:
+    the first length that does not)."""
     from mlp_splatting_amd import ops
     rng = np.random.default_rng(11)
     fr = Frame("cfg1_5k_160x120", n=8, width=8, height=8, eye=(0, 0, -2.0), target=(0, 0, 0))
+    case, _, short = case.partition(":")
     n = {"spread": 1500, "ties": 700, "behind": 900, "clusters": 1200, "beyond_invalid": 300, "two": 2, "capacity": 1536}[case]
+    n = int(short) if short else n
     pos = np.zeros((n, 3), np.float32)
     pos[:, :2] = rng.uniform(-0.05, 0.05, (n, 2))
     if case in ("spread", "capacity"):
