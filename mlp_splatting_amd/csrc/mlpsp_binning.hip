@@ -1,8 +1,8 @@
 // libmlpsp_hip: projection of primitive supports and tile binning (the "legacy" screen-space rule).
 //
 // The reference evaluates a dense [tiles x primitives] boolean matrix (scannet/cumodel.py:1028-1070).
-// Here the same predicate is evaluated sparsely and deterministically, without atomics and without
-// a sort, in two levels:
+// Here the same predicate is evaluated sparsely and deterministically, without atomics on global
+// memory and without a sort, in two levels:
 //   level 1: the frame is cut into super-tiles of 8x8 tiles.  Wavefront (chunk c, super-tile s)
 //            tests 2048 consecutive primitives against the super-tile rectangle (a superset of the
 //            union of its tiles' tests), counts, and after a scan writes the survivors in ascending
