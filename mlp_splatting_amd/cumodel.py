@@ -578,6 +578,7 @@ class NeuralPrimitiveSceneTileCUDA(nn.Module):
         if tile_size <= 0:
             raise ValueError("tile_size must be a positive integer.")
         num_tiles = ops.num_tiles(W, H, tile_size, tile_size)
+        given = tile_view_ids
         tile_view_ids = tile_view_ids.to(device=device, dtype=torch.long).reshape(-1)
         if tile_view_ids.numel() != num_tiles:
             raise ValueError(f"tile_view_ids length mismatch: got {tile_view_ids.numel()}, expected {num_tiles}")
@@ -585,10 +586,33 @@ class NeuralPrimitiveSceneTileCUDA(nn.Module):
             raise ValueError("view_matrices must have shape (K,4,4)")
         if int(view_matrices.shape[0]) <= 0:
             raise ValueError("view_matrices must contain at least one view")
-        lo, hi = torch.stack(torch.aminmax(tile_view_ids)).tolist()          # one read-back for both bounds
+        # one read-back for both bounds, and -- with the int32 copy the binning takes -- only once per state of the
+        # caller's tensor (a mosaic's layout is the same frame after frame; the check is a reduction and a
+        # synchronisation)
+        lo, hi, ids32 = self._tile_view_check(given, tile_view_ids)
         if lo < 0 or hi >= int(view_matrices.shape[0]):
             raise ValueError("tile_view_ids contains out-of-range view indices")
-        return self._legacy_culling(view_matrices, proj_matrix, score_threshold, tile_size, tile_view_ids)
+        return self._legacy_culling(view_matrices, proj_matrix, score_threshold, tile_size, ids32)
+
+    def _tile_view_check(self, given, ids):
+        """(smallest id, largest id, int32 copy) of a caller's tile_view_ids, remembered for the last few tensors seen
+        (a renderer cycles through a handful of mosaic layouts).  An entry keeps the caller's tensor itself: while it
+        lives its memory cannot be handed to another tensor, whose address, shape and version would match."""
+        try:
+            key = (given.data_ptr(), given._version, tuple(given.shape), given.dtype, str(given.device))
+        except RuntimeError:                      # inference tensors have no version counter: do not remember
+            key = None
+        memo = self.__dict__.setdefault("_mlpsp_tile_views", {})
+        hit = memo.get(key) if key is not None else None
+        if hit is None:
+            with torch.inference_mode(False), torch.no_grad():
+                lo, hi = torch.stack(torch.aminmax(ids)).tolist()
+                hit = (lo, hi, ids.to(torch.int32).contiguous(), given)
+            if key is not None:
+                if len(memo) >= 16:
+                    memo.pop(next(iter(memo)))
+                memo[key] = hit
+        return hit[:3]
 
     def _tile_lists(self, ray_o, ray_d, score_threshold, view_matrix, proj_matrix, culled_prim_indices, tile_offsets,
                     device, allow_native=True):
@@ -718,6 +742,7 @@ class NeuralPrimitiveSceneTileCUDA(nn.Module):
         version, which a fused optimizer step (``Adam(fused=True)``) does not advance.  Call it yourself after
         changing parameters in any other way that leaves ``tensor._version`` unchanged."""
         self.__dict__.pop("_mlpsp_cache", None)
+        self.__dict__.pop("_mlpsp_tile_views", None)
         ext = _tile_ext
         if ext is not None and callable(getattr(ext, "invalidate_caches", None)):
             ext.invalidate_caches()
