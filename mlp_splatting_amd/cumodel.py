@@ -690,10 +690,12 @@ class NeuralPrimitiveSceneTileCUDA(nn.Module):
             own_lists = (culled_prim_indices is None and tile_offsets is None and view_matrix is not None
                          and proj_matrix is not None
                          and getattr(self, "camera_mode", "legacy-centered") != "colmap-native")
-            if (own_lists and use_tilecenter and ts == 8 and not return_feature and feature_target is None
-                    and getattr(self, "queued_frames", True) and hasattr(ext, "render_frame_queued")):
+            with_feat = return_feature and self.feat_attr is not None
+            if (own_lists and use_tilecenter and ts == 8 and (with_feat or not return_feature)
+                    and feature_target is None and getattr(self, "queued_frames", True)
+                    and hasattr(ext, "render_frame_queued")):
                 done = self._forward_queued(ext, ray_o, ray_d, score_threshold, view_matrix, proj_matrix, bg_color,
-                                            device)
+                                            device, with_feat)
                 if done is not None:
                     return done
             # queued before the binning, whose pair count is a blocking read-back: the device then has
@@ -816,7 +818,8 @@ class NeuralPrimitiveSceneTileCUDA(nn.Module):
             float(self.feature_gating_temp), int(W), int(H), ts, ts, float(score_threshold),
             self._background(bg_color, ray_o))
 
-    def _forward_queued(self, ext, ray_o, ray_d, score_threshold, view_matrix, proj_matrix, bg_color, device):
+    def _forward_queued(self, ext, ray_o, ray_d, score_threshold, view_matrix, proj_matrix, bg_color, device,
+                        with_feat=False):
         """The RGB frame with binning, sort and render queued back to back and one read-back at the end
         (``TileExt.render_frame_queued``); None when that path does not apply or has to be repeated the
         synchronous way.  Same images and errors as the step-by-step path.  The binning goes first: it needs only
@@ -827,6 +830,8 @@ class NeuralPrimitiveSceneTileCUDA(nn.Module):
             raise ValueError(f"Unsupported render_precision {precision!r}; use 'f32', 'bf16' or 'fp16'.")
         if precision != "f32" and not (int(self.hidden_dim) == 32 and int(self.pe_frequencies) == 6):
             precision = "f32"
+        if with_feat and precision == "f32":
+            return None                       # the exact feature frame goes step by step
         params = (self.W1, self.b1, self.W2, self.b2, self.W3, self.b3)
         if any(w.dtype != torch.float32 for w in params):
             half = all(w.dtype == torch.float16 for w in params)
@@ -843,12 +848,16 @@ class NeuralPrimitiveSceneTileCUDA(nn.Module):
         ws = [p.detach().contiguous() for p in params]
         unit_dirs = _unit_directions(ray_d)
         freq, att = self._frequency_tables(device)
+        more = {"binned": binned} if binned is not None else {}
+        if with_feat:
+            more["feat"] = (self.feat_attr.detach().contiguous(), float(self.feature_gating_beta),
+                            float(self.feature_gating_temp))
         out = ext.render_frame_queued(ray_o.contiguous(), unit_dirs, positions, log_scales, self._unit_quats(), freq, att,
-                                      ws, views, proj, int(W), int(H), float(score_threshold), precision,
-                                      **({"binned": binned} if binned is not None else {}))
+                                      ws, views, proj, int(W), int(H), float(score_threshold), precision, **more)
         if out is None:
             return None
-        return _add_background(out[0], out[1], self._background(bg_color, ray_o))
+        rgb = _add_background(out[0], out[1], self._background(bg_color, ray_o))
+        return (rgb, out[2]) if with_feat else rgb
 
     def render_feature_map(self, ray_o, ray_d, score_threshold: float = 1e-3, view_matrix=None, proj_matrix=None,
                            culled_prim_indices=None, tile_offsets=None):

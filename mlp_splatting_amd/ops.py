@@ -533,10 +533,12 @@ def pack_mfma_feat(feat_attr):
 
 def render_tilecenter_mfma_feat(rays_o, rays_d, records, order, tile_offsets, freq, att, W1, b1, W2, b2, W3, b3,
                                 feat_attr, beta, temp, W, H, threshold, bf16=True, packed=None, packed_feat=None,
-                                check=True):
+                                check=True, status=None):
     """Matrix-core tile-centre forward with the gated feature channel -> (rgb, alpha, feat, nonfinite).
     ``packed_feat`` is the result of :func:`pack_mfma_feat` for ``feat_attr`` (built here when omitted;
-    non-finite rounded attributes raise)."""
+    non-finite rounded attributes raise).  ``status`` (an int32 [16] device tensor): ONE attempt with the first
+    record-pool size and no read-back -- word 0 = non-finite, word 1 = the pool ran out (the feature image is then
+    incomplete and the caller repeats the call without ``status``); returns (rgb, alpha, feat, status)."""
     dev = rays_o.device
     if freq.numel() != 6:
         raise RuntimeError("the matrix-core path supports 6 frequencies only")
@@ -553,7 +555,10 @@ def render_tilecenter_mfma_feat(rays_o, rays_d, records, order, tile_offsets, fr
     rgb = torch.empty(B, 3, dtype=torch.float32, device=dev)
     alpha = torch.empty(B, 1, dtype=torch.float32, device=dev)
     feat = torch.empty(B, ch, dtype=torch.float32, device=dev)
-    flag = torch.empty(16, dtype=torch.int32, device=dev)
+    if status is not None and not (status.is_cuda and status.dtype == torch.int32 and status.numel() == 16
+                                   and status.is_contiguous()):
+        raise ValueError("status must be a contiguous int32 [16] tensor on the device")
+    flag = status if status is not None else torch.empty(16, dtype=torch.int32, device=dev)
     for pool in _feat_pool_sizes(pairs):
         ws_bytes = lib.mlpsp_feat_workspace_bytes(pairs, W, H, 8, 8, slots, 1, pool)
         workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
@@ -563,6 +568,8 @@ def render_tilecenter_mfma_feat(rays_o, rays_d, records, order, tile_offsets, fr
             float(threshold), _ptr(workspace), ws_bytes, _ptr(rgb), _ptr(alpha), _ptr(feat), _ptr(flag), None,
             _stream(dev))
         _check(code, "mlpsp_render_tilecenter_mfma_feat")
+        if status is not None:
+            return rgb, alpha, feat, status
         if pool < 0:
             break
         host_flag = flag[:2].tolist()               # one read-back: [non-finite, pool ran out]

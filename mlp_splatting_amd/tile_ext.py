@@ -327,18 +327,26 @@ class TileExt:
         return cand, offsets, counts, tail, cap, scale
 
     def render_frame_queued(self, rays_o, unit_dirs, positions, log_scales, unit_quats, freq, att, ws, view_matrices,
-                            proj_matrix, width, height, threshold, precision, binned=None):
+                            proj_matrix, width, height, threshold, precision, binned=None, feat=None):
         """(rgb, alpha) of one 8x8-tile, tile-centre-order RGB frame: binning, sort and render are queued
         back to back and ONE read-back at the end brings the pair count, the longest tile list and the
         non-finite flag.  The candidate buffer is sized from the previous frame's count; if this frame
         needs more (or the level-1 scratch overflows) every list was left empty on the device: the
         estimate is enlarged and None is returned, and the caller renders the frame the synchronous way.
         ``binned``: the result of :meth:`frame_binning_queued` for the same primitives and camera, when the caller
-        has queued the binning already.
+        has queued the binning already.  ``feat`` = (feat_attr, beta, temp) adds the gated feature image (matrix-core
+        precisions only): (rgb, alpha, feat); None is also returned when the record pool of the first size ran out
+        or the attributes do not fit fp16 (the step-by-step path then decides what to do).
         Errors are those of the entry points it stands for (capacity text of np_tile_kernels.cu:4578-4588,
         fallback policy of rgb_wmma.cuh:260-272)."""
         name = "render_tiles_rgb_wmma" if precision != "f32" else "render_tiles_forward_tilecenter"
         width, height, threshold = int(width), int(height), float(threshold)
+        if feat is not None and precision == "f32":
+            return None                                   # (the exact feature path is not queued)
+        if feat is not None:
+            _chk(feat[0].is_cuda and feat[0].dtype in (torch.float32, torch.float16) and feat[0].dim() in (2, 3),
+                 "feat_attr must be a CUDA float32 tensor with 2 or 3 dimensions")
+            _chk(feat[0].shape[0] == positions.shape[0], "feat_attr first dimension must match primitive count")
         if binned is None:
             binned = self.frame_binning_queued(positions, log_scales, view_matrices, proj_matrix, width, height,
                                                threshold)
@@ -351,14 +359,24 @@ class TileExt:
             rec = self._records(positions, log_scales, unit_quats)
             order, _ = ops.sort_tiles(rays_o, unit_dirs, rec, cand, offsets, width, height, 8, 8, _lib.KEY_TSTAR,
                                       self.max_tile_prims, cull_threshold=threshold)
+            fmap, pool_ran_out = None, 0
             if precision != "f32":
                 packed = self._packed_weights(list(ws), precision == "bf16")
-                rgb, alpha, _ = ops.render_tilecenter_mfma(rays_o, unit_dirs, rec, order, offsets, freq, att, *ws,
-                                                           width, height, threshold, bf16=(precision == "bf16"),
-                                                           packed=packed, check=False, status=status)
+                if feat is None:
+                    rgb, alpha, _ = ops.render_tilecenter_mfma(rays_o, unit_dirs, rec, order, offsets, freq, att, *ws,
+                                                               width, height, threshold, bf16=(precision == "bf16"),
+                                                               packed=packed, check=False, status=status)
+                else:
+                    packed_feat, bad_attr = self._packed_feat(feat[0])
+                    if bad_attr:
+                        return None
+                    rgb, alpha, fmap, _ = ops.render_tilecenter_mfma_feat(
+                        rays_o, unit_dirs, rec, order, offsets, freq, att, *ws, feat[0], feat[1], feat[2], width, height,
+                        threshold, bf16=(precision == "bf16"), packed=packed, packed_feat=packed_feat, status=status)
                 host = tail.cpu().numpy()
                 pairs, longest, l1_entries, guard = (int(v) for v in host[:32].view("int64"))
                 nonfinite = int(host[32:36].view("int32")[0])
+                pool_ran_out = int(host[36:40].view("int32")[0]) if feat is not None else 0
             else:
                 rgb, alpha, _ = ops.render_tilecenter_f32(rays_o, unit_dirs, rec, order, offsets, freq, att, *ws, width,
                                                           height, 8, 8, threshold)
@@ -373,8 +391,11 @@ class TileExt:
                     return None
                 if pairs > 0.9 * cap:                       # stay ahead of a slowly growing scene
                     self._queue_capacity = int(pairs * 1.3) + 65536
-                if precision != "f32":
+                redo = feat is not None and bool(nonfinite or pool_ran_out)
+                if precision != "f32" and not redo:
                     self._mfma_calls += 1
+            if redo:
+                return None                               # rare: the step-by-step path repeats the frame
             if longest > self.max_tile_prims:
                 raise RuntimeError(f"{name}: tile candidate capacity {self.max_tile_prims} exceeded (maximum observed "
                                    f"tile length {longest}); refusing to truncate or use an inconsistent "
@@ -389,7 +410,7 @@ class TileExt:
                                                           *[w.float() for w in ws], width, height, 8, 8, threshold)
                 _chk(bool(torch.isfinite(rgb).all()) and bool(torch.isfinite(alpha).all()),
                      "Scalar FP32 fallback output is nonfinite")
-        return rgb, alpha
+        return (rgb, alpha) if feat is None else (rgb, alpha, fmap)
 
     def note_frame_pairs(self, pairs: int):
         """Seed the candidate-buffer estimate of :meth:`render_frame_queued` from a synchronous frame."""

@@ -238,6 +238,36 @@ def test_statistics_collection_through_the_scene_module(device, oracle_mod):
     assert int(scene.stat_hits.sum()) == 0 and float(scene.stat_sum_werr.sum()) == 0.0
 
 
+def test_queued_feature_frames_equal_step_by_step_frames(device, oracle_mod, monkeypatch):
+    # the matrix-core frame with its feature image, queued without a mid-frame read-back, is the same frame
+    from mlp_splatting_amd import cumodel
+    from mlp_splatting_amd.tile_ext import TileExt
+    fr = Frame("cfg1_5k_160x120", n=1500, hidden=32, width=64, height=48, feature_dim=48)
+    monkeypatch.setattr(cumodel, "_tile_ext", TileExt())
+    scene = _scene_from(fr, device, feature=True)
+    scene.render_precision = "bf16"
+    scene.queued_frames = False
+    ref_rgb, ref_feat = _call(scene, fr, device, return_feature=True)
+    scene.queued_frames = True
+    ext = cumodel._tile_ext
+    assert ext._queue_capacity > 0                       # seeded by the step-by-step frame
+    calls = []
+    real = ext.render_frame_queued
+    monkeypatch.setattr(ext, "render_frame_queued", lambda *a, **k: (calls.append(k.get("feat") is not None), real(*a, **k))[1])
+    rgb, feat = _call(scene, fr, device, return_feature=True)
+    assert calls == [True] and torch.equal(rgb, ref_rgb) and torch.equal(feat, ref_feat)
+    assert float(feat.abs().max()) > 1e-2
+    # a candidate-buffer estimate that is too small: repeated step by step, same images
+    ext._queue_capacity = 16
+    rgb, feat = _call(scene, fr, device, return_feature=True)
+    assert torch.equal(rgb, ref_rgb) and torch.equal(feat, ref_feat) and ext._queue_capacity > 1000
+    # the exact path is not queued
+    scene.render_precision = "f32"
+    calls.clear()
+    exact = _call(scene, fr, device, return_feature=True)
+    assert calls == [] and float((exact[1] - ref_feat).abs().max()) < 5e-2
+
+
 def test_queued_frames_equal_step_by_step_frames(device, oracle_mod, monkeypatch):
     # the frame queued without a mid-frame read-back (TileExt.render_frame_queued) is the same frame
     from mlp_splatting_amd import cumodel
