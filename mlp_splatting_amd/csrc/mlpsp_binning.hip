@@ -497,6 +497,8 @@ __global__ __launch_bounds__(1024) void exclusive_scan_kernel(int32_t* __restric
   __shared__ long long s_wave[kScanSlabs][16];
   __shared__ int s_wmax[16];
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+  // (requested up front: by the end of the scan it has long arrived)
+  const long long l1_entries = guard.all_totals ? guard.all_totals[0] : 0;
   long long carry = 0;
   int mx = 0;
   for (int pass0 = 0; pass0 < n; pass0 += kScanSlabs * 4096) {
@@ -564,7 +566,7 @@ __global__ __launch_bounds__(1024) void exclusive_scan_kernel(int32_t* __restric
   for (int d = 1; d < 64; d <<= 1) mx = max(mx, __shfl_xor(mx, d));
   if (lane == 0) s_wmax[wave] = mx;
   __syncthreads();
-  const bool bad = guard.all_totals && (guard.all_totals[0] > guard.l1_capacity || carry > guard.cand_capacity);
+  const bool bad = guard.all_totals && (l1_entries > guard.l1_capacity || carry > guard.cand_capacity);
   if (bad)                                         // (the scan's own stores are behind the barriers above)
     for (int i = t; i < n; i += 1024) data[i] = 0;
   if (t == 0) {
@@ -577,7 +579,7 @@ __global__ __launch_bounds__(1024) void exclusive_scan_kernel(int32_t* __restric
       guard.all_totals[3] = bad ? 1 : 0;
       guard.counts_out[0] = carry;
       guard.counts_out[1] = all_max;
-      guard.counts_out[2] = guard.all_totals[0];
+      guard.counts_out[2] = l1_entries;
       guard.counts_out[3] = bad ? 1 : 0;
     }
   }
