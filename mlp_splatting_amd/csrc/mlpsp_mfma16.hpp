@@ -27,6 +27,9 @@ namespace mlpsp {
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+typedef short i16x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
@@ -56,6 +59,9 @@ template <> struct Ops<__bf16> {
   static __device__ __forceinline__ f32x16 mfma(u32x4 a, u32x4 b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
   }
+  static __device__ __forceinline__ f32x4 mfma4(u32x2 a, u32x2 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(__builtin_bit_cast(i16x4, a), __builtin_bit_cast(i16x4, b), c, 0, 0, 0);
+  }
   static __device__ __forceinline__ float round_trip(float a) { return (float)(__bf16)a; }
   static constexpr unsigned kOneWord = 0x3f803f80u;   // (1, 1)
   static constexpr float kMax = 3.38953139e38f;
@@ -73,6 +79,9 @@ template <> struct Ops<_Float16> {
   }
   static __device__ __forceinline__ f32x16 mfma(u32x4 a, u32x4 b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ f32x4 mfma4(u32x2 a, u32x2 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(f16x4, a), __builtin_bit_cast(f16x4, b), c, 0, 0, 0);
   }
   static __device__ __forceinline__ float round_trip(float a) { return (float)(_Float16)a; }
   static constexpr unsigned kOneWord = 0x3c003c00u;   // (1, 1)
@@ -97,10 +106,16 @@ __host__ __device__ constexpr int hidden_unit_of_row(int m) { return hidden_unit
 // ReLU of two packed 16-bit floats in one instruction: as signed 16-bit integers every negative float
 // (and -0) is below zero and every non-negative one keeps its bits, for bf16 and fp16 alike; rounding
 // commutes with ReLU, so rounding first gives the same operand.
+// The instruction itself is left to the compiler, not written as inline assembly: the output layer's 4x4x4 products
+// may write another register group than the one they accumulate from, and the compiler keeps the next writer of
+// the old group one wait state away from such a product only if it can see that the writer is a vector
+// instruction.  The empty statement only hides where x comes from; otherwise the conversion that produced x is
+// split into two conversions and a byte permute to fit the integer maximum.
 __device__ __forceinline__ unsigned relu_packed(unsigned x) {
-  unsigned y;
-  asm("v_pk_max_i16 %0, %1, 0" : "=v"(y) : "v"(x));
-  return y;
+  typedef short i16x2 __attribute__((ext_vector_type(2)));
+  asm("" : "+v"(x));
+  const i16x2 zero = {0, 0};
+  return __builtin_bit_cast(unsigned, __builtin_elementwise_max(__builtin_bit_cast(i16x2, x), zero));
 }
 __device__ __forceinline__ float max3_abs(float a, float b, float c) {
   float y;
@@ -110,13 +125,14 @@ __device__ __forceinline__ float max3_abs(float a, float b, float c) {
 // The first read of the accumulator tile is a plain C++ operation, not inline assembly: the compiler
 // inserts the wait states a matrix-core result needs before its first reader only for instructions it
 // can see, and everything below depends on that first read.
+// (The running maximum is updated in place: an inline-assembly instruction that writes a register of its own
+// could be given one that a 4x4x4 product issued just before still reads as its addend.)
 template <typename T>
 __device__ __forceinline__ bool out_of_range_in(const f32x16& v) {
   float m = __builtin_fabsf(v[0]);
-  m = max3_abs(m, v[1], v[2]);
 #pragma unroll
-  for (int r = 3; r < 15; r += 2) m = max3_abs(m, v[r], v[r + 1]);
-  m = max3_abs(m, v[15], v[15]);
+  for (int r = 1; r < 15; r += 2) asm("v_max3_f32 %0, |%0|, |%1|, |%2|" : "+v"(m) : "v"(v[r]), "v"(v[r + 1]));
+  asm("v_max3_f32 %0, |%0|, |%1|, |%1|" : "+v"(m) : "v"(v[15]));
   return !(m <= Ops<T>::kMax);
 }
 
@@ -188,11 +204,24 @@ __device__ __forceinline__ HalfPair both_halves(float x) {
   const unsigned lo = r[0], hi = r[1];
   return HalfPair{__uint_as_float(lo), __uint_as_float(hi)};
 }
-// lanes 0..31 of a in the lower half, lanes 0..31 of b in the upper half
-__device__ __forceinline__ float lower_halves(float a, float b) {
+
+// [a lanes 0..31 + a lanes 32..63 | b lanes 0..31 + b lanes 32..63]
+__device__ __forceinline__ float sum_of_halves(float a, float b) {
   const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(a), __float_as_uint(b), false, false);
-  const unsigned lo = r[0];
-  return __uint_as_float(lo);
+  const unsigned lo = r[0], hi = r[1];
+  return __uint_as_float(lo) + __uint_as_float(hi);
+}
+
+// The output layer has four rows: as a 32x32x16 product 28 of its 32 accumulator rows would be zero.  It runs on
+// v_mfma_f32_4x4x4 (sixteen independent 4x4x4 products, one per group of four lanes, 8 clocks) instead: in the
+// group of lane l, lane l supplies A row l % 4 = output row l % 4 and B column l % 4 = its own pixel column, four
+// k-slots each, and receives the four sums of its own column.  The k-slots a lane can supply are the hidden units
+// its accumulator registers hold, so lanes l and l ^ 32 each get one half of the column's sums (added by
+// sum_of_halves); a packed row of eight weights (16 bytes, registers 8s .. 8s+7 of lane group g) is two such steps.
+template <typename T>
+__device__ __forceinline__ f32x4 layer3_small(u32x4 a, u32x4 b, f32x4 c) {
+  c = Ops<T>::mfma4(u32x2{a[0], a[1]}, u32x2{b[0], b[1]}, c);
+  return Ops<T>::mfma4(u32x2{a[2], a[3]}, u32x2{b[2], b[3]}, c);
 }
 
 // The MLP of primitive block `blk` for the pixels of `mask` (ballot of the lanes that hit).  dx, dy, dz: this
@@ -209,21 +238,27 @@ __device__ __forceinline__ bool mlp_wave_mfma16(const unsigned char* __restrict_
                                                 float o[4], unsigned mk[2]) {
   const int g = l >> 5;
   bool bad = false;
+  // Addresses of the weight loads: wave-uniform base in scalar registers + zero-extended 32-bit lane offset +
+  // immediate, the form the global loads take as they are, so that no address is computed per lane and hit.  The
+  // compiler picks that form only if it sees the zero extension next to the load; the lane index is therefore made
+  // opaque here, once per call (otherwise the extended offsets are hoisted out of the primitive loop as 64-bit
+  // registers and added to the base per lane).  Everything beyond the first 4 KiB of the block is addressed from a
+  // second scalar base: the immediates end at 4095.
+  int ll = l;
+  unsigned row16 = (unsigned)(g * 4 + (l & 3)) * 16u, upper = 4096u;
+  asm volatile("" : "+v"(ll), "+v"(row16), "+s"(upper));
+  const unsigned lane16 = (unsigned)ll * 16u, lane4 = (unsigned)ll * 4u;
+  const unsigned char* hi = blk + upper;
   // ---- stage the primitive's weights: MFMA A fragments, straight from global memory
   u32x4 a1[5], a2[2], a3[2];
 #pragma unroll
-  for (int s = 0; s < 5; ++s) a1[s] = *reinterpret_cast<const u32x4*>(blk + kOffW1 + s * 1024 + l * 16);
+  for (int s = 0; s < 5; ++s) a1[s] = *reinterpret_cast<const u32x4*>((s < 4 ? blk : hi - 4096) + kOffW1 + s * 1024 + lane16);
 #pragma unroll
-  for (int s = 0; s < 2; ++s) a2[s] = *reinterpret_cast<const u32x4*>(blk + kOffW2 + s * 1024 + l * 16);
-  const unsigned a2b_word = *reinterpret_cast<const unsigned*>(blk + kOffB2 + l * 4);
+  for (int s = 0; s < 2; ++s) a2[s] = *reinterpret_cast<const u32x4*>(hi + (kOffW2 - 4096) + s * 1024 + lane16);
+  const unsigned a2b_word = *reinterpret_cast<const unsigned*>(hi + (kOffB2 - 4096) + lane4);
 #pragma unroll
-  for (int s = 0; s < 2; ++s) {
-    // every lane loads one of the four stored rows (no divergent branch, no wait in the middle of the
-    // staging); rows 4..31 of the operand are zero
-    const u32x4 row = *reinterpret_cast<const u32x4*>(blk + kOffW3 + ((s * 2 + g) * 4 + (l & 3)) * 16);
-    const bool stored = (l & 31) < 4;
-    a3[s] = u32x4{stored ? row[0] : 0u, stored ? row[1] : 0u, stored ? row[2] : 0u, stored ? row[3] : 0u};
-  }
+  // output layer: lane l supplies output row l % 4 for the hidden units its lane group holds (layer3_small)
+  for (int s = 0; s < 2; ++s) a3[s] = *reinterpret_cast<const u32x4*>(hi + (kOffW3 - 4096) + s * 128 + row16);
   const f32x4 b3v = *reinterpret_cast<const f32x4*>(blk + kOffB3);
   const int wflag = *reinterpret_cast<const int32_t*>(blk + kOffFlag);
   bad |= (wflag != 0);
@@ -244,8 +279,6 @@ __device__ __forceinline__ bool mlp_wave_mfma16(const unsigned char* __restrict_
       // layer 1: 18 (sin, cos) words per lane + the bias word, 5 K-steps; words 0..8 come from LDS.  (The lane
       // index is made opaque so that the loads stay here and are not hoisted out of the primitive loop into
       // registers.)
-      int ll = l;
-      asm volatile("" : "+v"(ll));
       const u32x4 dq0 = dir.q[b][0][ll], dq1 = dir.q[b][1][ll];
       const unsigned d8 = dir.w8[b][ll];
       f32x16 d1 = zero16;
@@ -290,8 +323,8 @@ __device__ __forceinline__ bool mlp_wave_mfma16(const unsigned char* __restrict_
         d2 = Ops<T>::mfma(a2[s], bw, d2);
       }
       if constexpr (CHECK) bad |= col_active && out_of_range_in<T>(d2);
-      // layer 3: rows 0..3 of a 32-row product; row k lands in register k of lane group 0
-      f32x16 d3 = zero16;
+      // output layer: this lane's half of the four sums of its column (layer3_small)
+      f32x4 d3 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int s = 0; s < 2; ++s) {
         u32x4 bw;
@@ -300,7 +333,7 @@ __device__ __forceinline__ bool mlp_wave_mfma16(const unsigned char* __restrict_
           bw[d] = relu_packed(Ops<T>::pack2(d2[8 * s + 2 * d], d2[8 * s + 2 * d + 1]));
           if constexpr (MASKS) m_blk[b][1] |= relu_mask_bits(bw[d], 4 * s + d);
         }
-        d3 = Ops<T>::mfma(a3[s], bw, d3);
+        d3 = layer3_small<T>(a3[s], bw, d3);
       }
 #pragma unroll
       for (int k = 0; k < 4; ++k) o_blk[b][k] = d3[k];
@@ -309,9 +342,9 @@ __device__ __forceinline__ bool mlp_wave_mfma16(const unsigned char* __restrict_
       for (int k = 0; k < 4; ++k) o_blk[b][k] = 0.f;
     }
   }
-  // pixel l < 32 reads block 0 from its own lane; pixel l >= 32 reads block 1 from lane l - 32
+  // pixel l < 32 belongs to block 0, pixel l >= 32 to block 1: both lane groups' halves of its sums
 #pragma unroll
-  for (int k = 0; k < 4; ++k) o[k] = lower_halves(o_blk[0][k], o_blk[1][k]) + b3v[k];
+  for (int k = 0; k < 4; ++k) o[k] = sum_of_halves(o_blk[0][k], o_blk[1][k]) + b3v[k];
   if constexpr (MASKS) {
     // lane group g holds the units 8g..8g+7 and 16+8g..16+8g+7 of its column: shift into place, merge the
     // two groups, and take the block this lane's pixel belongs to (block g)
@@ -338,18 +371,25 @@ __device__ __forceinline__ bool mlp_pair_mfma16(const unsigned char* __restrict_
                                                 float o[4]) {
   const int g = l >> 5;
   bool bad = false;
+  // Addresses of the weight loads: wave-uniform base in scalar registers + zero-extended 32-bit lane offset +
+  // immediate, the form the global loads take as they are, so that no address is computed per lane and hit.  The
+  // compiler picks that form only if it sees the zero extension next to the load; the lane index is therefore made
+  // opaque here, once per call (otherwise the extended offsets are hoisted out of the primitive loop as 64-bit
+  // registers and added to the base per lane).  Everything beyond the first 4 KiB of the block is addressed from a
+  // second scalar base: the immediates end at 4095.
+  int ll = l;
+  unsigned row16 = (unsigned)(g * 4 + (l & 3)) * 16u, upper = 4096u;
+  asm volatile("" : "+v"(ll), "+v"(row16), "+s"(upper));
+  const unsigned lane16 = (unsigned)ll * 16u, lane4 = (unsigned)ll * 4u;
+  const unsigned char* hi = blk + upper;
   u32x4 a1[5], a2[2], a3[2];
 #pragma unroll
-  for (int s = 0; s < 5; ++s) a1[s] = *reinterpret_cast<const u32x4*>(blk + kOffW1 + s * 1024 + l * 16);
+  for (int s = 0; s < 5; ++s) a1[s] = *reinterpret_cast<const u32x4*>((s < 4 ? blk : hi - 4096) + kOffW1 + s * 1024 + lane16);
 #pragma unroll
-  for (int s = 0; s < 2; ++s) a2[s] = *reinterpret_cast<const u32x4*>(blk + kOffW2 + s * 1024 + l * 16);
-  const unsigned a2b_word = *reinterpret_cast<const unsigned*>(blk + kOffB2 + l * 4);
+  for (int s = 0; s < 2; ++s) a2[s] = *reinterpret_cast<const u32x4*>(hi + (kOffW2 - 4096) + s * 1024 + lane16);
+  const unsigned a2b_word = *reinterpret_cast<const unsigned*>(hi + (kOffB2 - 4096) + lane4);
 #pragma unroll
-  for (int s = 0; s < 2; ++s) {
-    const u32x4 row = *reinterpret_cast<const u32x4*>(blk + kOffW3 + ((s * 2 + g) * 4 + (l & 3)) * 16);
-    const bool stored = (l & 31) < 4;
-    a3[s] = u32x4{stored ? row[0] : 0u, stored ? row[1] : 0u, stored ? row[2] : 0u, stored ? row[3] : 0u};
-  }
+  for (int s = 0; s < 2; ++s) a3[s] = *reinterpret_cast<const u32x4*>(hi + (kOffW3 - 4096) + s * 128 + row16);
   const f32x4 b3v = *reinterpret_cast<const f32x4*>(blk + kOffB3);
   const int wflag = *reinterpret_cast<const int32_t*>(blk + kOffFlag);
   bad |= (wflag != 0);
@@ -357,8 +397,6 @@ __device__ __forceinline__ bool mlp_pair_mfma16(const unsigned char* __restrict_
   const HalfPair hx = both_halves(dx), hy = both_halves(dy), hz = both_halves(dz);
   const float xin[2][3] = {{hx.blk0, hy.blk0, hz.blk0}, {hx.blk1, hy.blk1, hz.blk1}};
   const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-  int ll = l;
-  asm volatile("" : "+v"(ll));
   f32x16 d1[2] = {zero16, zero16};
   // The wavefront asks for issue priority while it walks its MFMA chains (the other wavefronts of the SIMD are
   // mostly in vector work, which also issues beside an MFMA): 0.7 % off the kernel, measured against priority 0
@@ -415,7 +453,7 @@ __device__ __forceinline__ bool mlp_pair_mfma16(const unsigned char* __restrict_
     bad |= ((mask >> (l & 31)) & 1ull) && out_of_range_in<T>(d2[0]);
     bad |= ((mask >> (32 + (l & 31))) & 1ull) && out_of_range_in<T>(d2[1]);
   }
-  f32x16 d3[2] = {zero16, zero16};
+  f32x4 d3[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
 #pragma unroll
   for (int s = 0; s < 2; ++s) {
 #pragma unroll
@@ -423,12 +461,12 @@ __device__ __forceinline__ bool mlp_pair_mfma16(const unsigned char* __restrict_
       u32x4 bw;
 #pragma unroll
       for (int d = 0; d < 4; ++d) bw[d] = relu_packed(Ops<T>::pack2(d2[b][8 * s + 2 * d], d2[b][8 * s + 2 * d + 1]));
-      d3[b] = Ops<T>::mfma(a3[s], bw, d3[b]);
+      d3[b] = layer3_small<T>(a3[s], bw, d3[b]);
     }
   }
   __builtin_amdgcn_s_setprio(0);
 #pragma unroll
-  for (int k = 0; k < 4; ++k) o[k] = lower_halves(d3[0][k], d3[1][k]) + b3v[k];
+  for (int k = 0; k < 4; ++k) o[k] = sum_of_halves(d3[0][k], d3[1][k]) + b3v[k];
   return bad;
 }
 
