@@ -436,9 +436,9 @@ __device__ __forceinline__ bool mlp_pair_mfma16(const unsigned char* __restrict_
   }
   unsigned z0, z1, z2;
   asm volatile("v_mov_b32 %0, 0\n v_mov_b32 %1, 0\n v_mov_b32 %2, 0" : "=v"(z0), "=v"(z1), "=v"(z2));
-  f32x16 d2[2];
-#pragma unroll
-  for (int b = 0; b < 2; ++b) d2[b] = Ops<T>::mfma(u32x4{a2b_word, z0, z1, z2}, u32x4{one_word, z0, z1, z2}, zero16);
+  // the bias tile of layer 2 (every column the same) is computed once and is the addend of both blocks' first K-step
+  const f32x16 bias2 = Ops<T>::mfma(u32x4{a2b_word, z0, z1, z2}, u32x4{one_word, z0, z1, z2}, zero16);
+  f32x16 d2[2] = {bias2, bias2};
 #pragma unroll
   for (int s = 0; s < 2; ++s) {
 #pragma unroll
