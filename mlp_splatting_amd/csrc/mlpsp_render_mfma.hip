@@ -170,30 +170,47 @@ __device__ __forceinline__ FastRec fast_arrived(FastRegs& q) {
 // errors well above the rounding noise of this path.  unsure = the fast quantities are too close to one of
 // the three decision boundaries (decay within 0.4 % of thr, t or denom near zero) to be trusted; the
 // caller then takes the decision -- only the decision -- from hit_rot().
-__device__ __forceinline__ bool hit_fast(float rox, float roy, float roz, float rdx, float rdy, float rdz,
-                                         const FastRec& F, float thr, HitInfo& h, bool& unsure) {
-  const float vx = F.cx - rox, vy = F.cy - roy, vz = F.cz - roz;
-  const float dlx = fmaf(F.r[0], rdx, fmaf(F.r[1], rdy, F.r[2] * rdz));
-  const float dly = fmaf(F.r[3], rdx, fmaf(F.r[4], rdy, F.r[5] * rdz));
-  const float dlz = fmaf(F.r[6], rdx, fmaf(F.r[7], rdy, F.r[8] * rdz));
-  const float vlx = fmaf(F.r[0], vx, fmaf(F.r[1], vy, F.r[2] * vz));
-  const float vly = fmaf(F.r[3], vx, fmaf(F.r[4], vy, F.r[5] * vz));
-  const float vlz = fmaf(F.r[6], vx, fmaf(F.r[7], vy, F.r[8] * vz));
+// What hit_fast() needs of (primitive, ray origin) alone: the offset centre - origin and its image under r.
+struct OriginTerms {
+  float vx, vy, vz, vlx, vly, vlz;
+};
+__device__ __forceinline__ OriginTerms origin_terms(float ox, float oy, float oz, float cx, float cy, float cz,
+                                                    const float r[9]) {
+  OriginTerms o;
+  o.vx = cx - ox;
+  o.vy = cy - oy;
+  o.vz = cz - oz;
+  o.vlx = fmaf(r[0], o.vx, fmaf(r[1], o.vy, r[2] * o.vz));
+  o.vly = fmaf(r[3], o.vx, fmaf(r[4], o.vy, r[5] * o.vz));
+  o.vlz = fmaf(r[6], o.vx, fmaf(r[7], o.vy, r[8] * o.vz));
+  return o;
+}
+__device__ __forceinline__ bool hit_fast(const OriginTerms& o, float rdx, float rdy, float rdz, const float r[9],
+                                         float thr, HitInfo& h, bool& unsure) {
+  const float dlx = fmaf(r[0], rdx, fmaf(r[1], rdy, r[2] * rdz));
+  const float dly = fmaf(r[3], rdx, fmaf(r[4], rdy, r[5] * rdz));
+  const float dlz = fmaf(r[6], rdx, fmaf(r[7], rdy, r[8] * rdz));
   const float denom = fmaf(dlx, dlx, fmaf(dly, dly, dlz * dlz));
-  const float numer = fmaf(dlx, vlx, fmaf(dly, vly, dlz * vlz));
+  const float numer = fmaf(dlx, o.vlx, fmaf(dly, o.vly, dlz * o.vlz));
   const float t = numer * __builtin_amdgcn_rcpf(denom);
   h.t = t;
-  h.dx = fmaf(-t, rdx, vx);
-  h.dy = fmaf(-t, rdy, vy);
-  h.dz = fmaf(-t, rdz, vz);
-  h.qlx = fmaf(-t, dlx, vlx);
-  h.qly = fmaf(-t, dly, vly);
-  h.qlz = fmaf(-t, dlz, vlz);
+  h.dx = fmaf(-t, rdx, o.vx);
+  h.dy = fmaf(-t, rdy, o.vy);
+  h.dz = fmaf(-t, rdz, o.vz);
+  h.qlx = fmaf(-t, dlx, o.vlx);
+  h.qly = fmaf(-t, dly, o.vly);
+  h.qlz = fmaf(-t, dlz, o.vlz);
   const float r2 = fmaf(h.qlx, h.qlx, fmaf(h.qly, h.qly, h.qlz * h.qlz));
   h.decay = __builtin_amdgcn_exp2f(r2 * -0.72134752f);
   unsure = (__builtin_fabsf(h.decay - thr) <= 4e-3f * thr) || !(__builtin_fabsf(t) >= 1e-4f) || !(denom >= 1e-18f);
   return !(denom <= 1e-20f) && !(t <= 0.f) && (h.decay > thr);
 }
+
+// LDS of one wavefront: the OriginTerms of the 64 list entries it is walking, entry j at 32 j bytes (one address
+// register for the two reads of a step).
+struct OriginLds {
+  float e[64][8];
+};
 
 // SP = 0: RGB only.  SP = 4 or 8: the kernel also emits, per tile, the compact list of primitives that
 // hit at least one pixel (hit records, mlpsp_hitrec.hpp) and per (such primitive, pixel) the SP compositing
@@ -207,8 +224,8 @@ __device__ __forceinline__ bool hit_fast(float rox, float roy, float roz, float 
 // One tile, rendered by the calling wavefront (lane l = pixel l of the tile); s_dir: LDS of this wavefront alone.
 template <typename T, int SP>
 __device__ __forceinline__ void render_tile_mfma(
-    const int tile, const int l, DirWords& s_dir, const float* __restrict__ rays_o, const float* __restrict__ rays_d,
-    const PrimRecord* __restrict__ prims, const int32_t* __restrict__ order, const int32_t* __restrict__ offsets,
+    const int tile, const int l, DirWords& s_dir, OriginLds& s_org, const float* __restrict__ rays_o,
+    const float* __restrict__ rays_d, const PrimRecord* __restrict__ prims, const int32_t* __restrict__ order, const int32_t* __restrict__ offsets,
     const float* __restrict__ freq, const float* __restrict__ att, const unsigned char* __restrict__ packed, int N,
     int W, int H, int ntx, float thr, float* __restrict__ out_rgb, float* __restrict__ out_alpha,
     int32_t* __restrict__ status, unsigned long long* __restrict__ counters, int slots, float beta, float temp,
@@ -230,6 +247,17 @@ __device__ __forceinline__ void render_tile_mfma(
   // live registers would cost the fourth wavefront per SIMD.  Written and read by this wavefront only: no barrier.
   encode_direction_words<T>(rdx, rdy, rdz, kf, l, s_dir);
 
+  // A tile whose rays start from one point (a pinhole camera: every tile) needs centre - origin and its rotated,
+  // scaled image once per list entry, not once per pixel: lane j works them out for entry j of the 64 the wavefront
+  // is about to walk and parks them in LDS; a step then reads them with two broadcast reads instead of twelve
+  // vector instructions.  Same expressions on the same operands as the per-pixel form, so the same bits.
+  const unsigned long long in_image = __ballot(valid);
+  const int lane0 = in_image ? (int)__builtin_ctzll(in_image) : 0;
+  const float ox = __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(rox), lane0)),
+              oy = __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(roy), lane0)),
+              oz = __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(roz), lane0));
+  const bool one_origin = __ballot(valid && !(rox == ox && roy == oy && roz == oz)) == 0ull;
+
   const int start = offsets[tile], end = offsets[tile + 1];
   PixelAcc acc = {0.f, 0.f, 0.f, 1.f, 0.f, 0.f};
   HitEmitter em = hit_emitter_begin(hp, 0, start, tile);
@@ -245,23 +273,43 @@ __device__ __forceinline__ void render_tile_mfma(
     const int id_lane = (base + l < end) ? order[base + l] : -1;
     unsigned long long todo = __ballot(id_lane >= 0 && id_lane < N);
     if (todo == 0ull) continue;
-    int p = __builtin_amdgcn_readlane(id_lane, (int)__builtin_ctzll(todo));
+    if (one_origin && id_lane >= 0 && id_lane < N) {
+      const FastRec& F = *reinterpret_cast<const FastRec*>(fast_half + (size_t)id_lane * sizeof(PrimRecord));
+      const OriginTerms o = origin_terms(ox, oy, oz, F.cx, F.cy, F.cz, F.r);
+      *reinterpret_cast<f32x4*>(&s_org.e[l][0]) = f32x4{o.vx, o.vy, o.vz, o.vlx};
+      *reinterpret_cast<float2*>(&s_org.e[l][4]) = make_float2(o.vly, o.vlz);
+    }
+    int j = (int)__builtin_ctzll(todo);
+    int p = __builtin_amdgcn_readlane(id_lane, j);
     todo &= todo - 1ull;
     FastRegs q;
     fast_request(fast_half + (size_t)p * sizeof(PrimRecord), q);
     for (;;) {
+      // Between fast_arrived() and the next fast_request() every use of R: the request reloads the same scalar
+      // registers, and a value of R that had to outlive it would be copied out of them at the loop's edge, i.e.
+      // while they are being loaded.
       const FastRec R = fast_arrived(q);
+      OriginTerms ot;
+      if (one_origin) {
+        const f32x4 a = *reinterpret_cast<const f32x4*>(&s_org.e[j][0]);
+        const float2 b = *reinterpret_cast<const float2*>(&s_org.e[j][4]);
+        ot = OriginTerms{a[0], a[1], a[2], a[3], b.x, b.y};
+      } else {
+        ot = origin_terms(rox, roy, roz, R.cx, R.cy, R.cz, R.r);
+      }
+      HitInfo h;
+      bool unsure;
+      bool hit = hit_fast(ot, rdx, rdy, rdz, R.r, thr, h, unsure) && live;
+      asm volatile("" : "+v"(h.t), "+v"(h.qlx), "+v"(h.qly), "+v"(h.qlz), "+v"(h.decay));   // R is used up here
+
       const bool more = todo != 0ull;
-      int p_next = p;
+      int p_next = p, j_next = j;
       if (more) {
-        p_next = __builtin_amdgcn_readlane(id_lane, (int)__builtin_ctzll(todo));
+        j_next = (int)__builtin_ctzll(todo);
+        p_next = __builtin_amdgcn_readlane(id_lane, j_next);
         todo &= todo - 1ull;
       }
       fast_request(fast_half + (size_t)p_next * sizeof(PrimRecord), q);   // (the last entry asks for its own line again)
-
-      HitInfo h;
-      bool unsure;
-      bool hit = hit_fast(rox, roy, roz, rdx, rdy, rdz, R, thr, h, unsure) && live;
       if (__ballot(unsure && live) != 0ull) {   // rare (about one wavefront step in twenty)
         if (unsure && live) {
           const PrimRecord P = prims[p];
@@ -315,6 +363,7 @@ __device__ __forceinline__ void render_tile_mfma(
       }
       if (!more) break;
       p = p_next;
+      j = j_next;
     }
   }
 
@@ -348,7 +397,8 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 4))) void
   const int tile = superblock_tile(blockIdx.x, ntx, num_tiles / ntx);
   if (tile < 0) return;
   __shared__ DirWords s_dir;
-  render_tile_mfma<T, SP>(tile, (int)threadIdx.x, s_dir, rays_o, rays_d, prims, order, offsets, freq, att, packed, N, W,
+  __shared__ __attribute__((aligned(16))) OriginLds s_org;
+  render_tile_mfma<T, SP>(tile, (int)threadIdx.x, s_dir, s_org, rays_o, rays_d, prims, order, offsets, freq, att, packed, N, W,
                           H, ntx, thr, out_rgb, out_alpha, status, counters, slots, beta, temp, hp);
 }
 
