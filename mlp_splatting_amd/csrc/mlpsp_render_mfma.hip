@@ -168,12 +168,24 @@ __device__ __forceinline__ FastRec fast_arrived(FastRegs& q) {
 // The hit decision itself is a hard threshold, and a primitive that barely hits still contributes up to a
 // few 1e-3 to a pixel, so a decision that differs from the exact path's would show as isolated pixel
 // errors well above the rounding noise of this path.  unsure = the fast quantities are too close to one of
-// the three decision boundaries (decay within 0.4 % of thr, t or denom near zero) to be trusted; the
+// the three decision boundaries (decay within `band` of thr, t or denom near zero) to be trusted; the
 // caller then takes the decision -- only the decision -- from hit_rot().
+//
+// How wide the band has to be: with u = 2^-24, vl and dl carry about 4 u |vl| and 4 u |dl| of rounding (entries of
+// r rounded, three-term sums), t = numer / denom about 24 u |vl| / |dl|, so ql = vl - t dl is off by up to
+// 32 u |vl| and r2 = |ql|^2 by 64 u |ql| |vl|, i.e. ln decay by 32 u |ql| |vl|, and the exactly rounded form,
+// which rotates the same long vector, by as much again: 64 u |ql| |vl| = 3.8e-6 |ql| |vl| relative in decay, with
+// |ql| = sqrt(-2 ln thr) at the threshold (3.3 for thr = 5e-3: 1.3e-5 |vl|) and |vl| = distance origin -> centre
+// in units of the scales (a hundred is typical, far small primitives reach thousands).  band_for() is that
+// bound plus a floor for the native exp2; reach = 4e-6 sqrt(-2 ln thr).
 // What hit_fast() needs of (primitive, ray origin) alone: the offset centre - origin and its image under r.
 struct OriginTerms {
   float vx, vy, vz, vlx, vly, vlz;
 };
+__device__ __forceinline__ float band_for(const OriginTerms& o, float thr, float reach) {
+  const float len = __builtin_sqrtf(fmaf(o.vlx, o.vlx, fmaf(o.vly, o.vly, o.vlz * o.vlz)));
+  return thr * fmaf(reach, len, 3e-5f);
+}
 __device__ __forceinline__ OriginTerms origin_terms(float ox, float oy, float oz, float cx, float cy, float cz,
                                                     const float r[9]) {
   OriginTerms o;
@@ -186,7 +198,7 @@ __device__ __forceinline__ OriginTerms origin_terms(float ox, float oy, float oz
   return o;
 }
 __device__ __forceinline__ bool hit_fast(const OriginTerms& o, float rdx, float rdy, float rdz, const float r[9],
-                                         float thr, HitInfo& h, bool& unsure) {
+                                         float thr, float band, HitInfo& h, bool& unsure) {
   const float dlx = fmaf(r[0], rdx, fmaf(r[1], rdy, r[2] * rdz));
   const float dly = fmaf(r[3], rdx, fmaf(r[4], rdy, r[5] * rdz));
   const float dlz = fmaf(r[6], rdx, fmaf(r[7], rdy, r[8] * rdz));
@@ -202,12 +214,12 @@ __device__ __forceinline__ bool hit_fast(const OriginTerms& o, float rdx, float 
   h.qlz = fmaf(-t, dlz, o.vlz);
   const float r2 = fmaf(h.qlx, h.qlx, fmaf(h.qly, h.qly, h.qlz * h.qlz));
   h.decay = __builtin_amdgcn_exp2f(r2 * -0.72134752f);
-  unsure = (__builtin_fabsf(h.decay - thr) <= 4e-3f * thr) || !(__builtin_fabsf(t) >= 1e-4f) || !(denom >= 1e-18f);
+  unsure = (__builtin_fabsf(h.decay - thr) <= band) || !(__builtin_fabsf(t) >= 1e-4f) || !(denom >= 1e-18f);
   return !(denom <= 1e-20f) && !(t <= 0.f) && (h.decay > thr);
 }
 
-// LDS of one wavefront: the OriginTerms of the 64 list entries it is walking, entry j at 32 j bytes (one address
-// register for the two reads of a step).
+// LDS of one wavefront: the OriginTerms of the 64 list entries it is walking and the width of their decision
+// band, entry j at 32 j bytes (one address register for the two reads of a step).
 struct OriginLds {
   float e[64][8];
 };
@@ -256,6 +268,7 @@ __device__ __forceinline__ void render_tile_mfma(
   const float ox = __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(rox), lane0)),
               oy = __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(roy), lane0)),
               oz = __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(roz), lane0));
+  const float reach = 4e-6f * __builtin_sqrtf(fmaxf(-2.f * __logf(thr), 0.f));   // see band_for()
   const bool one_origin = __ballot(valid && !(rox == ox && roy == oy && roz == oz)) == 0ull;
 
   const int start = offsets[tile], end = offsets[tile + 1];
@@ -277,7 +290,7 @@ __device__ __forceinline__ void render_tile_mfma(
       const FastRec& F = *reinterpret_cast<const FastRec*>(fast_half + (size_t)id_lane * sizeof(PrimRecord));
       const OriginTerms o = origin_terms(ox, oy, oz, F.cx, F.cy, F.cz, F.r);
       *reinterpret_cast<f32x4*>(&s_org.e[l][0]) = f32x4{o.vx, o.vy, o.vz, o.vlx};
-      *reinterpret_cast<float2*>(&s_org.e[l][4]) = make_float2(o.vly, o.vlz);
+      *reinterpret_cast<f32x4*>(&s_org.e[l][4]) = f32x4{o.vly, o.vlz, band_for(o, thr, reach), 0.f};
     }
     int j = (int)__builtin_ctzll(todo);
     int p = __builtin_amdgcn_readlane(id_lane, j);
@@ -290,16 +303,19 @@ __device__ __forceinline__ void render_tile_mfma(
       // while they are being loaded.
       const FastRec R = fast_arrived(q);
       OriginTerms ot;
+      float band;
       if (one_origin) {
         const f32x4 a = *reinterpret_cast<const f32x4*>(&s_org.e[j][0]);
-        const float2 b = *reinterpret_cast<const float2*>(&s_org.e[j][4]);
-        ot = OriginTerms{a[0], a[1], a[2], a[3], b.x, b.y};
+        const f32x4 b = *reinterpret_cast<const f32x4*>(&s_org.e[j][4]);
+        ot = OriginTerms{a[0], a[1], a[2], a[3], b[0], b[1]};
+        band = b[2];
       } else {
         ot = origin_terms(rox, roy, roz, R.cx, R.cy, R.cz, R.r);
+        band = band_for(ot, thr, reach);
       }
       HitInfo h;
       bool unsure;
-      bool hit = hit_fast(ot, rdx, rdy, rdz, R.r, thr, h, unsure) && live;
+      bool hit = hit_fast(ot, rdx, rdy, rdz, R.r, thr, band, h, unsure) && live;
       asm volatile("" : "+v"(h.t), "+v"(h.qlx), "+v"(h.qly), "+v"(h.qlz), "+v"(h.decay));   // R is used up here
 
       const bool more = todo != 0ull;
@@ -310,7 +326,7 @@ __device__ __forceinline__ void render_tile_mfma(
         todo &= todo - 1ull;
       }
       fast_request(fast_half + (size_t)p_next * sizeof(PrimRecord), q);   // (the last entry asks for its own line again)
-      if (__ballot(unsure && live) != 0ull) {   // rare (about one wavefront step in twenty)
+      if (__ballot(unsure && live) != 0ull) {   // rare
         if (unsure && live) {
           const PrimRecord P = prims[p];
           HitInfo exact;
