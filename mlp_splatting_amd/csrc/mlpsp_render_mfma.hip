@@ -110,13 +110,17 @@ __device__ __forceinline__ float fast_blend_step(PixelAcc& a, float o0, float o1
   return w;
 }
 // tetrahedral gates (np_tile_kernels.cu:97-124) with the native exp/rcp.  qs = local hit offset divided by the
-// scales (what hit_fast() returns); u = q / (beta s + 1e-6) = qs s / (beta s + 1e-6).
-__device__ __forceinline__ void fast_tetra_gates(float qsx, float qsy, float qsz, float lgx, float lgy, float lgz,
-                                                 float beta, float temp, float g[4]) {
-  const float sx = fast_exp(lgx), sy = fast_exp(lgy), sz = fast_exp(lgz);
-  const float ux = fminf(1.f, fmaxf(-1.f, (qsx * sx) * __builtin_amdgcn_rcpf(beta * sx + 1e-6f)));
-  const float uy = fminf(1.f, fmaxf(-1.f, (qsy * sy) * __builtin_amdgcn_rcpf(beta * sy + 1e-6f)));
-  const float uz = fminf(1.f, fmaxf(-1.f, (qsz * sz) * __builtin_amdgcn_rcpf(beta * sz + 1e-6f)));
+// scales (what hit_fast() returns); u = q / (beta s + 1e-6) = qs k with k = s / (beta s + 1e-6), which depends on
+// the primitive alone (gate_factor).
+__device__ __forceinline__ float gate_factor(float lg, float beta) {
+  const float s = fast_exp(lg);
+  return s * __builtin_amdgcn_rcpf(beta * s + 1e-6f);
+}
+__device__ __forceinline__ void fast_tetra_gates(float qsx, float qsy, float qsz, float kx, float ky, float kz,
+                                                 float temp, float g[4]) {
+  const float ux = fminf(1.f, fmaxf(-1.f, qsx * kx));
+  const float uy = fminf(1.f, fmaxf(-1.f, qsy * ky));
+  const float uz = fminf(1.f, fmaxf(-1.f, qsz * kz));
   const float l0 = temp * ((ux + uy) + uz), l1 = temp * ((ux - uy) - uz);
   const float l2 = temp * ((-ux + uy) - uz), l3 = temp * ((-ux - uy) + uz);
   const float lm = fmaxf(fmaxf(l0, l1), fmaxf(l2, l3));
@@ -219,9 +223,12 @@ __device__ __forceinline__ bool hit_fast(const OriginTerms& o, float rdx, float 
 }
 
 // LDS of one wavefront: the OriginTerms of the 64 list entries it is walking and the width of their decision
-// band, entry j at 32 j bytes (one address register for the two reads of a step).
+// band (one address register for the two reads of a step); with a gated feature channel also the entries' three
+// gate factors, which a hit would otherwise have to fetch from the primitive's record -- a load that nothing but
+// the gates waits for, at the end of the step.
+template <int SP>
 struct OriginLds {
-  float e[64][8];
+  float e[64][SP > 0 ? 12 : 8];
 };
 
 // SP = 0: RGB only.  SP = 4 or 8: the kernel also emits, per tile, the compact list of primitives that
@@ -236,7 +243,7 @@ struct OriginLds {
 // One tile, rendered by the calling wavefront (lane l = pixel l of the tile); s_dir: LDS of this wavefront alone.
 template <typename T, int SP>
 __device__ __forceinline__ void render_tile_mfma(
-    const int tile, const int l, DirWords& s_dir, OriginLds& s_org, const float* __restrict__ rays_o,
+    const int tile, const int l, DirWords& s_dir, OriginLds<SP>& s_org, const float* __restrict__ rays_o,
     const float* __restrict__ rays_d, const PrimRecord* __restrict__ prims, const int32_t* __restrict__ order, const int32_t* __restrict__ offsets,
     const float* __restrict__ freq, const float* __restrict__ att, const unsigned char* __restrict__ packed, int N,
     int W, int H, int ntx, float thr, float* __restrict__ out_rgb, float* __restrict__ out_alpha,
@@ -291,6 +298,13 @@ __device__ __forceinline__ void render_tile_mfma(
       const OriginTerms o = origin_terms(ox, oy, oz, F.cx, F.cy, F.cz, F.r);
       *reinterpret_cast<f32x4*>(&s_org.e[l][0]) = f32x4{o.vx, o.vy, o.vz, o.vlx};
       *reinterpret_cast<f32x4*>(&s_org.e[l][4]) = f32x4{o.vly, o.vlz, band_for(o, thr, reach), 0.f};
+    }
+    if constexpr (SP > 0) {
+      if (slots > 1 && id_lane >= 0 && id_lane < N) {
+        const PrimRecord& P = prims[id_lane];
+        *reinterpret_cast<f32x4*>(&s_org.e[l][8]) =
+            f32x4{gate_factor(P.lgx, beta), gate_factor(P.lgy, beta), gate_factor(P.lgz, beta), 0.f};
+      }
     }
     int j = (int)__builtin_ctzll(todo);
     int p = __builtin_amdgcn_readlane(id_lane, j);
@@ -353,8 +367,8 @@ __device__ __forceinline__ void render_tile_mfma(
         if constexpr (SP > 0) {
           float gt[4] = {0.f, 0.f, 0.f, 0.f};
           if (slots > 1) {
-            const PrimRecord& P = prims[p];
-            if (hit) fast_tetra_gates(h.qlx, h.qly, h.qlz, P.lgx, P.lgy, P.lgz, beta, temp, gt);
+            const f32x4 k = *reinterpret_cast<const f32x4*>(&s_org.e[j][8]);
+            if (hit) fast_tetra_gates(h.qlx, h.qly, h.qlz, k[0], k[1], k[2], temp, gt);
           }
           const int rs = hit_emitter_next(hp, em, l);
           if (rs >= 0) {
@@ -413,7 +427,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 4))) void
   const int tile = superblock_tile(blockIdx.x, ntx, num_tiles / ntx);
   if (tile < 0) return;
   __shared__ DirWords s_dir;
-  __shared__ __attribute__((aligned(16))) OriginLds s_org;
+  __shared__ __attribute__((aligned(16))) OriginLds<SP> s_org;
   render_tile_mfma<T, SP>(tile, (int)threadIdx.x, s_dir, s_org, rays_o, rays_d, prims, order, offsets, freq, att, packed, N, W,
                           H, ntx, thr, out_rgb, out_alpha, status, counters, slots, beta, temp, hp);
 }
