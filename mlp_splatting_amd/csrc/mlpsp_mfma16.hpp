@@ -10,8 +10,9 @@
 // per K-step) provided the next layer's weight columns are stored in that register order.  Weights are
 // therefore repacked (pack kernel in mlpsp_render_mfma.hip) into A-fragment order with the k-permutation
 // folded in, and the chain layer1 -> ReLU -> layer2 -> ReLU -> layer3 needs no LDS, no barrier and no
-// cross-lane traffic.  Staging a primitive's weights is 7 coalesced 1 KiB loads straight into VGPRs (plus three
-// small ones for the layer-2 bias words and the four output rows).
+// cross-lane traffic until the very end (the four-row output layer runs on 4x4x4 products whose two halves are
+// joined by one half-wave swap per output, layer3_small).  Staging a primitive's weights is 7 coalesced 1 KiB loads
+// straight into VGPRs (plus three small ones for the layer-2 bias words and the four output rows).
 //
 // Layer-1 k-slots: lane group g = l/32 owns frequencies 3g..3g+2 of every input component, so both groups
 // evaluate 18 (sin, cos) pairs per pixel block and each pair lands in one 32-bit operand word.  sin/cos use

@@ -166,8 +166,8 @@ __device__ __forceinline__ FastRec fast_arrived(FastRegs& q) {
 // Ray against rotated ellipsoid for this path: same quantities as hit_rot() (np_tile_kernels.cu:659-711), with
 // the world -> local rotation and the inverse scales applied as one matrix, the local hit offset taken as
 // vl - t dl (equal to the rotated world offset up to rounding), and the native reciprocal and exp2.  About a
-// third of the instructions of the exactly-rounded form; the differences are of the order of f32 rounding
-// (about 1e-5 relative in decay, through the cancellation in vl - t dl).  h.ql* are in units of the scales.
+// third of the instructions of the exactly-rounded form; the differences are of the order of f32 rounding of
+// the long vector vl (how large: below).  h.ql* are in units of the scales.
 //
 // The hit decision itself is a hard threshold, and a primitive that barely hits still contributes up to a
 // few 1e-3 to a pixel, so a decision that differs from the exact path's would show as isolated pixel
