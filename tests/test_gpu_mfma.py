@@ -49,6 +49,38 @@ def test_matrix_core_render_against_oracle(device, oracle_mod, bf16, width, heig
     assert c[1] >= c[2] > 0
 
 
+@pytest.mark.parametrize("bf16", [True, False])
+def test_rays_from_separate_origins_take_the_per_pixel_form_with_the_same_bits(device, oracle_mod, bf16):
+    # A tile whose rays share an origin reads centre - origin and its rotated image per list entry; any other tile
+    # computes them per pixel.  One pixel per tile moved to another origin sends every tile down the per-pixel form:
+    # all the other pixels must come out bit-identical, and the moved ones must still match the oracle.
+    fr = Frame("cfg1_5k_160x120", hidden=32, width=88, height=60)          # ragged on both edges
+    cand, off = fr.oracle_lists(oracle_mod)
+    shared = _mfma(fr, device, cand, off, bf16)
+    ys, xs = np.meshgrid(np.arange(fr.H), np.arange(fr.W), indexing="ij")
+    moved = ((ys % 8 == 4) & (xs % 8 == 5)).ravel()
+    pinhole_o = fr.rays_o.copy()
+    fr.rays_o = pinhole_o.copy()
+    fr.rays_o[moved] += np.float32([0.02, -0.015, 0.01])
+    counters = torch.zeros(4, dtype=torch.int64, device=device)
+    mixed = _mfma(fr, device, cand, off, bf16, counters)
+    assert not shared[2] and not mixed[2]
+    keep = torch.from_numpy(~moved).to(device)
+    assert torch.equal(mixed[0][keep], shared[0][keep]) and torch.equal(mixed[1][keep], shared[1][keep])
+    assert not torch.equal(mixed[0][~keep], shared[0][~keep])
+    emu = oracle_mod.render_tilecenter(*fr.base_numpy(cand, off), *fr.dims, precision=1 if bf16 else 2)
+    assert np.abs(mixed[0].cpu().numpy() - emu["rgb"]).max() <= TOL[bf16]
+    assert np.abs(mixed[1].cpu().numpy() - emu["alpha"]).max() <= TOL[bf16]
+    c = counters.cpu().numpy()
+    assert abs(int(c[3]) - int(emu["stats"][3])) <= 0.002 * emu["stats"][3]
+    # every origin different: no pixel shares anything with its neighbours
+    rng = np.random.default_rng(3)
+    fr.rays_o = pinhole_o + rng.uniform(-0.01, 0.01, pinhole_o.shape).astype(np.float32)
+    loose = _mfma(fr, device, cand, off, bf16)
+    emu = oracle_mod.render_tilecenter(*fr.base_numpy(cand, off), *fr.dims, precision=1 if bf16 else 2)
+    assert not loose[2] and np.abs(loose[0].cpu().numpy() - emu["rgb"]).max() <= TOL[bf16]
+
+
 def test_matrix_core_matches_rounded_closed_form(device):
     # zero weights: colour = sigmoid(b3), independent of the operand rounding -> must equal the f32 kernel
     from mlp_splatting_amd.tile_ext import TileExt
@@ -153,6 +185,27 @@ def test_matrix_core_feature_render_against_oracle(device, oracle_mod, bf16, slo
     print(f"bf16={bf16} slots={slots} C={channels}: max|feat err|={err:.2e} of max|feat|={scale:.2e}")
     assert scale > 1e-2 and 0 < err <= TOL[bf16] * max(1.0, scale)
     assert np.abs(rgb.cpu().numpy() - want["rgb"]).max() <= TOL[bf16]
+
+
+def test_matrix_core_feature_render_with_separate_origins(device, oracle_mod):
+    from mlp_splatting_amd import ops
+    fr = Frame("cfg1_5k_160x120", n=1200, hidden=32, width=56, height=40, feature_dim=72, feature_slots=4)
+    rng = np.random.default_rng(5)
+    fr.rays_o = fr.rays_o + rng.uniform(-0.01, 0.01, fr.rays_o.shape).astype(np.float32)
+    sc = fr.scene
+    cand, off = fr.oracle_lists(oracle_mod)
+    want = oracle_mod.render_tilecenter(*fr.base_numpy(cand, off), *fr.dims, feat_attr=sc.feat_attr, beta=1.3, temp=2.2)
+    t = lambda a: to_dev(a, device)
+    rec = ops.prepare_primitives(t(sc.positions), t(sc.log_scales), t(sc.quats))
+    ro, rd, c, o = t(fr.rays_o), t(fr.rays_d), t(cand), t(off)
+    order, _ = ops.sort_tiles(ro, rd, rec, c, o, fr.W, fr.H, 8, 8, cull_threshold=fr.thr)
+    rgb, alpha, feat, nonfinite = ops.render_tilecenter_mfma_feat(ro, rd, rec, order, o, t(sc.freq), t(sc.att),
+                                                                  *[t(w) for w in sc.mlp()], t(sc.feat_attr), 1.3, 2.2,
+                                                                  fr.W, fr.H, fr.thr, bf16=True)
+    assert not nonfinite
+    scale = float(np.abs(want["feat"]).max())
+    assert scale > 1e-2 and np.abs(feat.cpu().numpy() - want["feat"]).max() <= TOL[True] * max(1.0, scale)
+    assert np.abs(rgb.cpu().numpy() - want["rgb"]).max() <= TOL[True]
 
 
 def test_scene_module_feature_precision_switch(device, oracle_mod):
