@@ -81,6 +81,50 @@ def test_rays_from_separate_origins_take_the_per_pixel_form_with_the_same_bits(d
     assert not loose[2] and np.abs(loose[0].cpu().numpy() - emu["rgb"]).max() <= TOL[bf16]
 
 
+@pytest.mark.parametrize("threshold,log_scale,depth,zoom", [(5e-3, -3.0, 1.0, 0.9), (5e-3, -5.5, 20.0, 40.0),
+                                                            (0.2, -4.5, 6.0, 10.0), (1e-4, -4.0, 2.0, 2.0)])
+def test_hit_sets_equal_the_exact_path_for_near_and_far_primitives(device, oracle_mod, threshold, log_scale, depth,
+                                                                   zoom):
+    # The reduced path decides hits with fast arithmetic and re-tests, exactly, only what lies within a band around
+    # the threshold whose width follows the distance to the primitive (in units of its scales).  With zero weights
+    # and a faint density no pixel ever saturates, so the hit counters depend on the hit decisions alone and must
+    # equal the exact kernel's to the last hit -- for primitives a few dozen scales away (the first case) and ten
+    # thousand (the second: a long lens on small far primitives) alike.
+    from mlp_splatting_amd import ops, synthetic as syn
+    W, H, n = 320, 240, 6000
+    sc = syn.make_scene(n, 32, seed=11, log_scale_mean=log_scale)
+    rng = np.random.default_rng(12)
+    f = zoom * W
+    z = rng.random(n, dtype=np.float32) * np.float32(3.0 * depth) + np.float32(depth)
+    sc.positions[:, 2] = z
+    sc.positions[:, 0] = (rng.random(n, dtype=np.float32) - np.float32(0.5)) * z * np.float32(W / f)
+    sc.positions[:, 1] = (rng.random(n, dtype=np.float32) - np.float32(0.5)) * z * np.float32(H / f)
+    for w in (sc.W1, sc.b1, sc.W2, sc.b2, sc.W3):
+        w[...] = 0
+    sc.b3[:, :3] = 0.3
+    sc.b3[:, 3] = -12.0                                                   # softplus ~ 6e-6: transmittance stays ~1
+    c2w = syn.look_at((0.0, 0.0, 0.0), (0.0, 0.0, 1.0))
+    ro, rd = syn.pinhole_rays(W, H, f, c2w)
+    rd = syn.normalize_rays(rd)
+    view, proj = syn.view_matrix(c2w), syn.projection_matrix(f, W, H)
+    cand, off = oracle_mod.bin_legacy(sc.positions, sc.log_scales, view[None], proj, W, H, 8, threshold)
+    assert len(cand) > 20000
+    t = lambda a: to_dev(a, device)
+    rec = ops.prepare_primitives(t(sc.positions), t(sc.log_scales), t(sc.quats))
+    ro_t, rd_t, c, o = t(ro), t(rd), t(cand), t(off)
+    order, _ = ops.sort_tiles(ro_t, rd_t, rec, c, o, W, H, 8, 8, cull_threshold=threshold)
+    ws = [t(w) for w in sc.mlp()]
+    exact_counters = torch.zeros(4, dtype=torch.int64, device=device)
+    ops.render_tilecenter_f32(ro_t, rd_t, rec, order, o, t(sc.freq), t(sc.att), *ws, W, H, 8, 8, threshold,
+                              counters=exact_counters)
+    for bf16 in (True, False):
+        counters = torch.zeros(4, dtype=torch.int64, device=device)
+        _, alpha, bad = ops.render_tilecenter_mfma(ro_t, rd_t, rec, order, o, t(sc.freq), t(sc.att), *ws, W, H, threshold,
+                                                   bf16=bf16, counters=counters)
+        assert not bad and float(alpha.max()) < 0.05
+        assert int(counters[3]) == int(exact_counters[3]) > 10000
+
+
 def test_matrix_core_matches_rounded_closed_form(device):
     # zero weights: colour = sigmoid(b3), independent of the operand rounding -> must equal the f32 kernel
     from mlp_splatting_amd.tile_ext import TileExt
