@@ -155,12 +155,15 @@ def _bin_scratch_bytes(n, K, W, H, tile):
 
 
 def bin_legacy_async(positions, log_scales, view_matrices, proj_matrix, W: int, H: int, tile: int, threshold: float,
-                     cand_capacity: int, tile_view_ids=None, scratch_scale: int = 1, counts=None):
+                     cand_capacity: int, tile_view_ids=None, scratch_scale: int = 1, counts=None, reuse=None):
     """:func:`bin_legacy` without any host synchronisation -> (candidates [cand_capacity], tile_offsets [T+1],
     counts int64 [4] on the device = pairs, longest tile list, level-1 entries, guard).  If guard is set the
     lists are empty: read ``counts`` at the next synchronisation, enlarge ``cand_capacity`` (pairs) or
     ``scratch_scale`` (level-1 entries) and repeat.  ``counts``: an int64 [4] device tensor to write them to (e.g. a
-    view of a buffer that is read back in one copy together with other results)."""
+    view of a buffer that is read back in one copy together with other results).  ``reuse``: a dict the caller keeps
+    between calls whose launches follow each other on one stream; the candidate, offset and scratch buffers are
+    then allocated once and handed out again while their sizes stay the same (four allocations less between the
+    end of one frame and the first launch of the next)."""
     positions, log_scales = _f32c(positions, "positions"), _f32c(log_scales, "log_scales")
     dev = positions.device
     on_device = (tile_view_ids is None and all(m.is_cuda and m.dtype == torch.float32 and m.numel() == 16 and
@@ -181,10 +184,16 @@ def bin_legacy_async(positions, log_scales, view_matrices, proj_matrix, W: int, 
     lib = _lib.load()
     fp = C.POINTER(C.c_float)
     nbytes = _bin_scratch_bytes(n, K, W, H, tile) * int(scratch_scale)
-    with torch.inference_mode(False):
-        offsets = torch.empty(T + 1, dtype=torch.int32, device=dev)
-        cand = torch.empty(int(cand_capacity), dtype=torch.int32, device=dev)
-    scratch = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    held = reuse.get("bin") if reuse is not None else None
+    if held is not None and held[0] == (T, int(cand_capacity), nbytes, dev):
+        offsets, cand, scratch = held[1]
+    else:
+        with torch.inference_mode(False):
+            offsets = torch.empty(T + 1, dtype=torch.int32, device=dev)
+            cand = torch.empty(int(cand_capacity), dtype=torch.int32, device=dev)
+        scratch = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+        if reuse is not None:
+            reuse["bin"] = ((T, int(cand_capacity), nbytes, dev), (offsets, cand, scratch))
     if counts is None:
         counts = torch.empty(4, dtype=torch.int64, device=dev)
     elif not (counts.is_cuda and counts.dtype == torch.int64 and counts.numel() == 4 and counts.is_contiguous()):

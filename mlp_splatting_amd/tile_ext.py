@@ -53,6 +53,7 @@ class TileExt:
         self.max_hits = int(max_hits)          # MLPSP_TILECENTER_MAX_HITS (np_tile_kernels.cu:48-50, 67-69)
         self._lock = threading.Lock()
         self._mfma_calls = 0
+        self._queued_buffers = {}
         self._mfma_fallbacks = 0
         self._training_mfma_stats = [0, 0, 0, 0, 0]
         self._uncached = threading.local()
@@ -319,12 +320,30 @@ class TileExt:
             return None
         with _on_device(positions.device):
             # counts of the binning (4 x int64) and flag words of the render (16 x int32) share one buffer: the
-            # frame's single read-back is one 96-byte copy
-            tail = torch.empty(96, dtype=torch.uint8, device=positions.device)
+            # frame's single read-back is one 96-byte copy.  The buffers a queued frame keeps to itself (this one,
+            # lists, offsets, scratch) are handed out again to the next frame of the same thread on the same stream:
+            # that frame starts after this one's read-back, and its first launch is four allocations nearer.
+            held = self._frame_buffers(positions.device)
+            if "tail" not in held:
+                fresh = torch.empty(96, dtype=torch.uint8, device=positions.device)
+                held["tail"] = (fresh, fresh[:32].view(torch.int64))
+            tail, counts_view = held["tail"]
             cand, offsets, counts = ops.bin_legacy_async(positions, log_scales, view_matrices, proj_matrix, int(width),
                                                          int(height), 8, float(threshold), cap, scratch_scale=scale,
-                                                         counts=tail[:32].view(torch.int64))
+                                                         counts=counts_view, reuse=held)
         return cand, offsets, counts, tail, cap, scale
+
+    def _frame_buffers(self, device):
+        """The reusable buffers of queued frames, per (thread, device, stream)."""
+        index = device.index if device.index is not None else torch.cuda.current_device()
+        key = (threading.get_ident(), index, torch._C._cuda_getCurrentRawStream(index))
+        held = self._queued_buffers.get(key)
+        if held is None:
+            with self._lock:
+                if len(self._queued_buffers) > 16:
+                    self._queued_buffers.clear()
+                held = self._queued_buffers.setdefault(key, {})
+        return held
 
     def render_frame_queued(self, rays_o, unit_dirs, positions, log_scales, unit_quats, freq, att, ws, view_matrices,
                             proj_matrix, width, height, threshold, precision, binned=None, feat=None):
