@@ -286,8 +286,8 @@ __device__ __forceinline__ void render_tile_mfma(
 
   // The tile's list is read 64 entries at a time, one coalesced load; a lane's entry is broadcast with
   // v_readlane when its turn comes.  Culled (negative) entries never get a turn.  The geometry line of the next
-  // entry is requested before the current one is tested, so that neither the id nor the record is waited for
-  // in the common case of a run of candidates that hit nothing.
+  // entry is requested as soon as the current one has been tested -- ahead of its MLP, if it hit -- so that neither
+  // the id nor the record is waited for long in a run of candidates that hit nothing.
   bool finished = false;
   for (int base = start; base < end && !finished; base += 64) {
     const int id_lane = (base + l < end) ? order[base + l] : -1;
