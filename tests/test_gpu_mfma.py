@@ -252,6 +252,36 @@ def test_matrix_core_feature_render_with_separate_origins(device, oracle_mod):
     assert np.abs(rgb.cpu().numpy() - want["rgb"]).max() <= TOL[True]
 
 
+@pytest.mark.parametrize("bf16", [True, False])
+@pytest.mark.parametrize("slots", [0, 4, 5])
+def test_repeated_launches_give_the_same_bits(device, oracle_mod, bf16, slots):
+    # Every value the kernel reads is either loaded and waited for or computed: nothing depends on timing.  (The walk
+    # keeps a scalar load in flight across a whole step; a register of it read too early shows as run-to-run noise.)
+    from mlp_splatting_amd import ops
+    fr = Frame("cfg2_50k_640x480", n=20000, hidden=32, width=320, height=240, feature_dim=40 if slots else 0,
+               feature_slots=max(slots, 4))
+    sc = fr.scene
+    cand, off = fr.oracle_lists(oracle_mod)
+    t = lambda a: to_dev(a, device)
+    rec = ops.prepare_primitives(t(sc.positions), t(sc.log_scales), t(sc.quats))
+    ro, rd, c, o = t(fr.rays_o), t(fr.rays_d), t(cand), t(off)
+    order, _ = ops.sort_tiles(ro, rd, rec, c, o, fr.W, fr.H, 8, 8, cull_threshold=fr.thr)
+    ws = [t(w) for w in sc.mlp()]
+    fa = t(sc.feat_attr) if slots else None
+
+    def once():
+        if not slots:
+            return ops.render_tilecenter_mfma(ro, rd, rec, order, o, t(sc.freq), t(sc.att), *ws, fr.W, fr.H, fr.thr,
+                                              bf16=bf16)[:2]
+        return ops.render_tilecenter_mfma_feat(ro, rd, rec, order, o, t(sc.freq), t(sc.att), *ws, fa, 1.3, 2.2, fr.W,
+                                               fr.H, fr.thr, bf16=bf16)[:3]
+    first = once()
+    assert float(first[1].mean()) > 0.2
+    for _ in range(4):
+        again = once()
+        assert all(torch.equal(a, b) for a, b in zip(first, again))
+
+
 def test_scene_module_feature_precision_switch(device, oracle_mod):
     from test_gpu_scene import _call, _scene_from
     fr = Frame("cfg1_5k_160x120", n=800, width=40, height=24, hidden=32, feature_dim=64)
