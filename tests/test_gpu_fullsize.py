@@ -209,3 +209,28 @@ def test_cfg4_mosaic_lists_and_image_match_the_oracle(device, oracle_mod):
     ops.validate_tile_lists(cand, off, ops.num_tiles(W, H, 8, 8), 1536, b.sc.n, "mosaic")
     with pytest.raises(RuntimeError, match=f"capacity {int(counts.max()) - 1} exceeded"):
         ops.validate_tile_lists(cand, off, ops.num_tiles(W, H, 8, 8), int(counts.max()) - 1, b.sc.n, "mosaic")
+
+
+@pytest.mark.parametrize("pose", [0, 7, 19])
+def test_cfg3_matrix_core_hit_sets_equal_the_exact_kernel(cfg3, device, pose):
+    # With zero weights and a density that keeps every pixel transparent, no ray is ever cut short, so the work
+    # counters depend on the hit decisions alone: the reduced-precision kernel (fast test + exact re-test inside a
+    # band whose width follows the distance to the primitive) must count exactly the hits of the f32 kernel, all
+    # tens of millions of them.
+    from mlp_splatting_amd import ops
+    b = cfg3
+    fr = b.single_view(pose)
+    ids, _ = ops.sort_tiles(fr["ro_t"], fr["rd_t"], b.rec, fr["cand"], fr["off"], b.W, b.H, 8, 8, cull_threshold=b.thr)
+    ws = [torch.zeros_like(w) for w in b.ws]
+    ws[5] = ws[5].clone()
+    ws[5][:, :3] = 0.3
+    ws[5][:, 3] = -12.0
+    exact = torch.zeros(4, dtype=torch.int64, device=device)
+    ops.render_tilecenter_f32(fr["ro_t"], fr["rd_t"], b.rec, ids, fr["off"], b.freq, b.att, *ws, b.W, b.H, 8, 8, b.thr,
+                              counters=exact)
+    for bf16 in (True, False):
+        fast = torch.zeros(4, dtype=torch.int64, device=device)
+        _, alpha, bad = ops.render_tilecenter_mfma(fr["ro_t"], fr["rd_t"], b.rec, ids, fr["off"], b.freq, b.att, *ws,
+                                                   b.W, b.H, b.thr, bf16=bf16, counters=fast)
+        assert not bad and float(alpha.max()) < 0.05
+        assert int(fast[3]) == int(exact[3]) > 30_000_000
