@@ -12,7 +12,7 @@
 // folded in, and the chain layer1 -> ReLU -> layer2 -> ReLU -> layer3 needs no LDS, no barrier and no
 // cross-lane traffic until the very end (the four-row output layer runs on 4x4x4 products whose two halves are
 // joined by one half-wave swap per output, layer3_small).  Staging a primitive's weights is 7 coalesced 1 KiB loads
-// straight into VGPRs (plus three small ones for the layer-2 bias words and the four output rows).
+// straight into VGPRs (plus two small ones for the four output rows).
 //
 // Layer-1 k-slots: lane group g = l/32 owns frequencies 3g..3g+2 of every input component, so both groups
 // evaluate 18 (sin, cos) pairs per pixel block and each pair lands in one 32-bit operand word.  sin/cos use
@@ -39,11 +39,13 @@ typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 // packed per-primitive block (bytes).  The biases of the two hidden layers travel as operands: b = hi + lo with
 // hi = round(b) and lo = round(b - hi) in the operand type (17 significant bits for bf16, 22 for fp16), multiplied
 // by a constant (1, 1) operand word and summed in f32 by the MFMA itself.  Layer 1 has spare k-slots for that
-// (72 of 80 used); layer 2 gets a third K-step whose A operand is one word per lane.  No bias is loaded as a
-// 16-register C operand any more: such loads cost the vector-memory pipe as much as the weights themselves.
-constexpr int kOffW1 = 0;       // 5 K-steps x 64 lanes x 16 B; word 18 of lane group 0 = (b1 hi, b1 lo)
+// (72 of 80 used), and for the bias of layer 2 as well: its word sits in the last of them, where layer 1 multiplies
+// it by zero, and layer 2 gets a third K-step that multiplies the same A operand (the last K-step of W1) by an
+// operand that is (1, 1) in that slot and zero elsewhere.  No bias is loaded as a 16-register C operand any more
+// (such loads cost the vector-memory pipe as much as the weights themselves), nor as a word of its own.
+constexpr int kOffW1 = 0;       // 5 K-steps x 64 lanes x 16 B; words 18, 19 of lane group 0 = (b1 hi, b1 lo), (b2 hi, b2 lo)
 constexpr int kOffW2 = 5120;    // 2 K-steps x 64 lanes x 16 B
-constexpr int kOffB2 = 7168;    // 64 lanes x 4 B: lanes 0..31 (b2 hi, b2 lo) of their row, lanes 32..63 zero
+constexpr int kOffB2 = 7168;    // 256 B, zero (reserved)
 constexpr int kOffW3 = 7424;    // 2 K-steps x 2 lane groups x 4 rows x 16 B
 constexpr int kOffB3 = 7680;    // 4 f32
 constexpr int kOffFlag = 7696;  // int32: 1 if any rounded weight or bias is non-finite
@@ -201,7 +203,11 @@ struct HalfPair {
 // element expression of the returned vector reads element 0 whatever the index.)
 __device__ __forceinline__ HalfPair both_halves(float x) {
   const unsigned u = __float_as_uint(x);
-  const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  // (the swap rewrites both of its operands: given the same value twice the compiler copies it twice; given a
+  // second name for it, once)
+  unsigned twin = u;
+  asm("" : "+v"(twin));
+  const auto r = __builtin_amdgcn_permlane32_swap(u, twin, false, false);
   const unsigned lo = r[0], hi = r[1];
   return HalfPair{__uint_as_float(lo), __uint_as_float(hi)};
 }
@@ -248,7 +254,7 @@ __device__ __forceinline__ bool mlp_wave_mfma16(const unsigned char* __restrict_
   int ll = l;
   unsigned row16 = (unsigned)(g * 4 + (l & 3)) * 16u, upper = 4096u;
   asm volatile("" : "+v"(ll), "+v"(row16), "+s"(upper));
-  const unsigned lane16 = (unsigned)ll * 16u, lane4 = (unsigned)ll * 4u;
+  const unsigned lane16 = (unsigned)ll * 16u;
   const unsigned char* hi = blk + upper;
   // ---- stage the primitive's weights: MFMA A fragments, straight from global memory
   u32x4 a1[5], a2[2], a3[2];
@@ -256,7 +262,6 @@ __device__ __forceinline__ bool mlp_wave_mfma16(const unsigned char* __restrict_
   for (int s = 0; s < 5; ++s) a1[s] = *reinterpret_cast<const u32x4*>((s < 4 ? blk : hi - 4096) + kOffW1 + s * 1024 + lane16);
 #pragma unroll
   for (int s = 0; s < 2; ++s) a2[s] = *reinterpret_cast<const u32x4*>(hi + (kOffW2 - 4096) + s * 1024 + lane16);
-  const unsigned a2b_word = *reinterpret_cast<const unsigned*>(hi + (kOffB2 - 4096) + lane4);
 #pragma unroll
   // output layer: lane l supplies output row l % 4 for the hidden units its lane group holds (layer3_small)
   for (int s = 0; s < 2; ++s) a3[s] = *reinterpret_cast<const u32x4*>(hi + (kOffW3 - 4096) + s * 128 + row16);
@@ -312,7 +317,7 @@ __device__ __forceinline__ bool mlp_wave_mfma16(const unsigned char* __restrict_
       // (the zero words of the two operands are made here, not kept in registers across the primitive loop)
       unsigned z0, z1, z2;
       asm volatile("v_mov_b32 %0, 0\n v_mov_b32 %1, 0\n v_mov_b32 %2, 0" : "=v"(z0), "=v"(z1), "=v"(z2));
-      f32x16 d2 = Ops<T>::mfma(u32x4{a2b_word, z0, z1, z2}, u32x4{one_word, z0, z1, z2}, zero16);
+      f32x16 d2 = Ops<T>::mfma(a1[4], u32x4{z0, z1, z2, one_word}, zero16);
 #pragma unroll
       for (int s = 0; s < 2; ++s) {
         u32x4 bw;
@@ -381,14 +386,13 @@ __device__ __forceinline__ bool mlp_pair_mfma16(const unsigned char* __restrict_
   int ll = l;
   unsigned row16 = (unsigned)(g * 4 + (l & 3)) * 16u, upper = 4096u;
   asm volatile("" : "+v"(ll), "+v"(row16), "+s"(upper));
-  const unsigned lane16 = (unsigned)ll * 16u, lane4 = (unsigned)ll * 4u;
+  const unsigned lane16 = (unsigned)ll * 16u;
   const unsigned char* hi = blk + upper;
   u32x4 a1[5], a2[2], a3[2];
 #pragma unroll
   for (int s = 0; s < 5; ++s) a1[s] = *reinterpret_cast<const u32x4*>((s < 4 ? blk : hi - 4096) + kOffW1 + s * 1024 + lane16);
 #pragma unroll
   for (int s = 0; s < 2; ++s) a2[s] = *reinterpret_cast<const u32x4*>(hi + (kOffW2 - 4096) + s * 1024 + lane16);
-  const unsigned a2b_word = *reinterpret_cast<const unsigned*>(hi + (kOffB2 - 4096) + lane4);
 #pragma unroll
   for (int s = 0; s < 2; ++s) a3[s] = *reinterpret_cast<const u32x4*>(hi + (kOffW3 - 4096) + s * 128 + row16);
   const f32x4 b3v = *reinterpret_cast<const f32x4*>(blk + kOffB3);
@@ -438,7 +442,7 @@ __device__ __forceinline__ bool mlp_pair_mfma16(const unsigned char* __restrict_
   unsigned z0, z1, z2;
   asm volatile("v_mov_b32 %0, 0\n v_mov_b32 %1, 0\n v_mov_b32 %2, 0" : "=v"(z0), "=v"(z1), "=v"(z2));
   // the bias tile of layer 2 (every column the same) is computed once and is the addend of both blocks' first K-step
-  const f32x16 bias2 = Ops<T>::mfma(u32x4{a2b_word, z0, z1, z2}, u32x4{one_word, z0, z1, z2}, zero16);
+  const f32x16 bias2 = Ops<T>::mfma(a1[4], u32x4{z0, z1, z2, one_word}, zero16);
   f32x16 d2[2] = {bias2, bias2};
 #pragma unroll
   for (int s = 0; s < 2; ++s) {

@@ -58,6 +58,7 @@ __global__ __launch_bounds__(64) void pack_mfma_weights_kernel(const S* __restri
       }
       v[d] = pk(ws, wc);
       if (t == 18 && g == 0) v[d] = bias_word<T>(bias1);     // multiplied by the constant (1, 1) operand word
+      if (t == 19 && g == 0) v[d] = bias_word<T>(bias2);     // by zero in layer 1, by (1, 1) in layer 2's bias step
     }
     *reinterpret_cast<u32x4*>(blk + kOffW1 + s * 1024 + l * 16) = v;
   }
@@ -66,7 +67,7 @@ __global__ __launch_bounds__(64) void pack_mfma_weights_kernel(const S* __restri
     for (int d = 0; d < 4; ++d) v[d] = pk((float)w2[hidden_unit(8 * s + 2 * d, g)], (float)w2[hidden_unit(8 * s + 2 * d + 1, g)]);
     *reinterpret_cast<u32x4*>(blk + kOffW2 + s * 1024 + l * 16) = v;
   }
-  reinterpret_cast<unsigned*>(blk + kOffB2)[l] = (g == 0) ? bias_word<T>(bias2) : 0u;
+  reinterpret_cast<unsigned*>(blk + kOffB2)[l] = 0u;         // reserved
   if (l < 16) {
     const int row = l & 3, gg = (l >> 2) & 1, s = l >> 3;
     const S* w3 = W3 + (size_t)p * 4 * 32 + row * 32;
@@ -187,7 +188,7 @@ struct OriginTerms {
   float vx, vy, vz, vlx, vly, vlz;
 };
 __device__ __forceinline__ float band_for(const OriginTerms& o, float thr, float reach) {
-  const float len = __builtin_sqrtf(fmaf(o.vlx, o.vlx, fmaf(o.vly, o.vly, o.vlz * o.vlz)));
+  const float len = __builtin_amdgcn_sqrtf(fmaf(o.vlx, o.vlx, fmaf(o.vly, o.vly, o.vlz * o.vlz)));   // (one ulp is plenty)
   return thr * fmaf(reach, len, 3e-5f);
 }
 __device__ __forceinline__ OriginTerms origin_terms(float ox, float oy, float oz, float cx, float cy, float cz,
