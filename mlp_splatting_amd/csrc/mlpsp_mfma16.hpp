@@ -314,9 +314,9 @@ __device__ __forceinline__ bool mlp_wave_mfma16(const unsigned char* __restrict_
       if constexpr (CHECK) bad |= col_active && out_of_range_in<T>(d1);
       // layer 2: the bias K-step first (its operands are ready), then the D registers of layer 1, rectified and
       // rounded, as the B operand
-      // (the zero words of the two operands are made here, not kept in registers across the primitive loop)
-      unsigned z0, z1, z2;
-      asm volatile("v_mov_b32 %0, 0\n v_mov_b32 %1, 0\n v_mov_b32 %2, 0" : "=v"(z0), "=v"(z1), "=v"(z2));
+      // (its B operand is constant, three zero words and the (1, 1) word: the compiler keeps it in four registers
+      // across the primitive loop, which there is room for)
+      const unsigned z0 = 0u, z1 = 0u, z2 = 0u;
       f32x16 d2 = Ops<T>::mfma(a1[4], u32x4{z0, z1, z2, one_word}, zero16);
 #pragma unroll
       for (int s = 0; s < 2; ++s) {
@@ -439,8 +439,7 @@ __device__ __forceinline__ bool mlp_pair_mfma16(const unsigned char* __restrict_
     bad |= ((mask >> (l & 31)) & 1ull) && out_of_range_in<T>(d1[0]);
     bad |= ((mask >> (32 + (l & 31))) & 1ull) && out_of_range_in<T>(d1[1]);
   }
-  unsigned z0, z1, z2;
-  asm volatile("v_mov_b32 %0, 0\n v_mov_b32 %1, 0\n v_mov_b32 %2, 0" : "=v"(z0), "=v"(z1), "=v"(z2));
+  const unsigned z0 = 0u, z1 = 0u, z2 = 0u;
   // the bias tile of layer 2 (every column the same) is computed once and is the addend of both blocks' first K-step
   const f32x16 bias2 = Ops<T>::mfma(a1[4], u32x4{z0, z1, z2, one_word}, zero16);
   f32x16 d2[2] = {bias2, bias2};
