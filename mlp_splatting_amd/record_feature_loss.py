@@ -69,32 +69,46 @@ def streaming_feature_l1(records, attributes, target, width, height, *, debug=Fa
     return partial.sum(), signs, pred
 
 
+class _SegmentPlan:
+    """What both attribute-gradient kernels need beside their adjoint: the segments of the primitive-major record
+    grouping, the pixel of every record, the buffer of per-segment sums and the launch order."""
+
+    def __init__(self, records, csr, num_pixels, attributes, segment_size, groups):
+        from .primitive_gemm import resolve_groups
+        ids, pixel_offsets = records[2], records[7]
+        dev = ids.device
+        self.primitives, self.starts, self.group_offsets = resolve_groups(csr, segment_size, groups)
+        # record -> pixel: pixel p owns records [pixel_offsets[p], pixel_offsets[p + 1])
+        self.pixels = torch.repeat_interleave(torch.arange(num_pixels, device=dev, dtype=torch.int32),
+                                              pixel_offsets.diff(), output_size=len(ids))
+        self.slots = attributes.shape[1] if attributes.ndim == 3 else 1
+        self.channels = attributes.shape[-1]
+        # per-segment sums followed by the chunk sums of the reduction over a primitive's segments
+        rows = int(_lib.load().mlpsp_segment_reduce_rows(len(self.primitives)))
+        self.partial = torch.empty((max(rows, 1), self.slots, self.channels), device=dev, dtype=torch.float32)
+        self.order = _launch_order(self.pixels, csr, self.starts)
+        self.device = dev
+
+
 def feature_weight_gradients(records, csr, signs, attributes, width, height, *, mixed=True, segment_size=512,
                              groups=None):
-    """d loss / d attributes, shaped like ``attributes`` -- scannet/record_feature_loss.py:164-185."""
-    from .primitive_gemm import resolve_groups
-    _, _, ids, x6, raw, masks, gates, pixel_offsets = records
-    hf, wf, channels = signs.shape
+    """d loss / d attributes, shaped like ``attributes``, from the residual signs the streamed loss kept
+    (API, checks and error texts of scannet/record_feature_loss.py:164-185)."""
     if signs.dtype != torch.int8 or not signs.is_contiguous():
         raise ValueError("feature loss signs must be contiguous int8")
-    slots = 1 if attributes.ndim == 2 else attributes.shape[1]
-    if hf > height or wf > width:
+    low_h, low_w, channels = signs.shape
+    if low_h > height or low_w > width:
         raise ValueError("streamed feature loss supports downsampling only")
-    primitives, starts, group_offsets = resolve_groups(csr, segment_size, groups)
-    device = ids.device
-    pixels = torch.repeat_interleave(torch.arange(width * height, device=device, dtype=torch.int32),
-                                     pixel_offsets.diff(), output_size=len(ids))
-    rows = int(_lib.load().mlpsp_segment_reduce_rows(len(primitives)))      # per-segment sums + the reduction's chunk sums
-    partial = torch.empty((max(rows, 1), slots, channels), device=device, dtype=torch.float32)
+    plan = _SegmentPlan(records, csr, width * height, attributes, segment_size, groups)
+    raw, gates = records[4], records[6]
     result = torch.empty_like(attributes)
-    order = _launch_order(pixels, csr, starts)
-    with torch.cuda.device(device):
+    with torch.cuda.device(plan.device):
         rc = _lib.load().mlpsp_feature_attribute_gradients(
-            _ptr(signs), _ptr(csr.record_indices), _ptr(pixels), _ptr(raw), _ptr(gates), _ptr(csr.offsets),
-            _ptr(primitives), _ptr(starts), _ptr(group_offsets), _ptr(order), int(len(primitives)), int(len(attributes)),
-            int(width),
-            int(height), int(wf), int(hf), int(channels), int(slots), int(segment_size), int(bool(mixed)),
-            _ptr(partial), _ptr(result), torch.cuda.current_stream(device).cuda_stream)
+            _ptr(signs), _ptr(csr.record_indices), _ptr(plan.pixels), _ptr(raw), _ptr(gates), _ptr(csr.offsets),
+            _ptr(plan.primitives), _ptr(plan.starts), _ptr(plan.group_offsets), _ptr(plan.order),
+            int(len(plan.primitives)), int(len(attributes)), int(width), int(height), int(low_w), int(low_h),
+            int(channels), int(plan.slots), int(segment_size), int(bool(mixed)), _ptr(plan.partial), _ptr(result),
+            torch.cuda.current_stream(plan.device).cuda_stream)
     if rc != 0:
         raise RuntimeError(f"mlpsp_feature_attribute_gradients: {_lib.strerror(rc)}")
     return result
@@ -106,32 +120,24 @@ def dense_feature_attribute_gradients(records, csr, grad_feature, attributes, *,
     what ``render_tiles_backward_featattr_tilecenter`` returns to ``_TileRenderWithFeatAutogradFn.backward``
     (scannet/cumodel.py:466-477; kernel scannet/cuda/np_tile_kernels.cu:3531-3760).  ``grad_feature`` [pixels, C]
     f32; geometry, alpha and the gates are constants of the feature image, as in the reference."""
-    from .primitive_gemm import resolve_groups
-    _, _, ids, x6, raw, masks, gates, pixel_offsets = records
-    device = ids.device
-    num_pixels = pixel_offsets.numel() - 1
+    num_pixels = records[7].numel() - 1
     slots = 1 if attributes.ndim == 2 else attributes.shape[1]
-    channels = attributes.shape[-1]
     if slots not in (1, 4, 5):
         raise RuntimeError("feat_attr must be [N,C] or [N,S,C] with slots in {4,5}")
     if (grad_feature.dtype != torch.float32 or not grad_feature.is_contiguous()
-            or tuple(grad_feature.shape) != (num_pixels, channels)):
+            or tuple(grad_feature.shape) != (num_pixels, attributes.shape[-1])):
         raise ValueError("the feature adjoint must be contiguous float32 [pixels, channels]")
     if attributes.dtype != torch.float32:
         raise ValueError("feature attributes must be float32")
-    primitives, starts, group_offsets = resolve_groups(csr, segment_size, groups)
-    pixels = torch.repeat_interleave(torch.arange(num_pixels, device=device, dtype=torch.int32), pixel_offsets.diff(),
-                                     output_size=len(ids))
-    rows = int(_lib.load().mlpsp_segment_reduce_rows(len(primitives)))
-    partial = torch.empty((max(rows, 1), slots, channels), device=device, dtype=torch.float32)
-    result = torch.empty(attributes.shape, device=device, dtype=torch.float32)
-    order = _launch_order(pixels, csr, starts)
-    with torch.cuda.device(device):
+    plan = _SegmentPlan(records, csr, num_pixels, attributes, segment_size, groups)
+    raw, gates = records[4], records[6]
+    result = torch.empty(attributes.shape, device=plan.device, dtype=torch.float32)
+    with torch.cuda.device(plan.device):
         rc = _lib.load().mlpsp_feature_dense_attribute_gradients(
-            _ptr(grad_feature), _ptr(csr.record_indices), _ptr(pixels), _ptr(raw), _ptr(gates), _ptr(csr.offsets),
-            _ptr(primitives), _ptr(starts), _ptr(group_offsets), _ptr(order), int(len(primitives)), int(len(attributes)),
-            int(channels), int(slots), int(segment_size), _ptr(partial), _ptr(result),
-            torch.cuda.current_stream(device).cuda_stream)
+            _ptr(grad_feature), _ptr(csr.record_indices), _ptr(plan.pixels), _ptr(raw), _ptr(gates), _ptr(csr.offsets),
+            _ptr(plan.primitives), _ptr(plan.starts), _ptr(plan.group_offsets), _ptr(plan.order),
+            int(len(plan.primitives)), int(len(attributes)), int(plan.channels), int(slots), int(segment_size),
+            _ptr(plan.partial), _ptr(result), torch.cuda.current_stream(plan.device).cuda_stream)
     if rc != 0:
         raise RuntimeError(f"mlpsp_feature_dense_attribute_gradients: {_lib.strerror(rc)}")
     return result
