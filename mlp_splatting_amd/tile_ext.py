@@ -10,6 +10,8 @@ f32 or on the matrix cores, reverse compositing, grouped gradients) is.
 from __future__ import annotations
 
 import contextlib
+import os
+import sys
 import threading
 import warnings
 
@@ -57,7 +59,7 @@ class TileExt:
         self._mfma_fallbacks = 0
         self._training_mfma_stats = [0, 0, 0, 0, 0]
         self._uncached = threading.local()
-        self._pack = None                 # cache entries: (key, value, source tensors) -- see _derived
+        self._pack = None                 # cache slots: lists of (key, value, source tensors) -- see _derived
         self._feat_pack = None
         self._rec = None
         self._binned = None
@@ -828,21 +830,50 @@ class TileExt:
         except RuntimeError:
             return None
 
+    @staticmethod
+    def _held_only_here(sources):
+        """True when the cache entry's own references are all that keeps the sources' memory allocated (their
+        owner -- a scene module -- is gone): nobody else holds these tensor objects, and nobody holds another tensor
+        on their storages (a tensor handed in is usually a fresh ``detach()`` of a parameter: then the tensor object
+        is the entry's alone and the parameter shows in the storage's holder count)."""
+        count = getattr(torch._C, "_storage_Use_Count", None)
+        if count is None:
+            return False
+        try:
+            mine = {}
+            for t in sources:
+                # the entry's tuple (once per occurrence), this loop variable and getrefcount's own argument
+                if sys.getrefcount(t) > sum(1 for u in sources if u is t) + 2:
+                    return False
+                mine.setdefault(t.untyped_storage()._cdata, set()).add(id(t))
+            # (+1: the wrapper untyped_storage() makes for the question itself)
+            return all(count(c) <= len(tensors) + 1 for c, tensors in mine.items())
+        except Exception:
+            return False
+
     def _derived(self, slot, sources, extra, build):
-        """``build()`` once per state of ``sources``.  The entry keeps the source tensors themselves: while it lives
-        their memory cannot be freed and handed to another scene's tensors of the same shape, whose key would then
-        match (the address is only an identity for memory that is still allocated).  The price is that the last
-        scene's tensors stay allocated until another scene is rendered or :meth:`invalidate_caches` is called."""
+        """``build()`` once per state of ``sources``; a slot keeps the derived tensors of the last
+        ``MLPSP_CACHE_SCENES`` (default 2) source states, most recent first, so that two scenes rendered in turn
+        do not rebuild each other's copies.  An entry keeps the source tensors themselves: while it lives their
+        memory cannot be freed and handed to another scene's tensors of the same shape, whose key would then match
+        (the address is only an identity for memory that is still allocated).  Entries whose sources nothing else
+        holds any more are dropped on the next call; :meth:`invalidate_caches` drops everything."""
         if not self._caching():
             return build()
         key = self._source_key(sources, extra)
         if key is None:
             return build()
         with self._lock:
-            entry = getattr(self, slot)
-            if entry is None or entry[0] != key:
-                entry = (key, build(), tuple(sources))
-                setattr(self, slot, entry)
+            entries = getattr(self, slot) or []
+            for i, entry in enumerate(entries):
+                if entry[0] == key:
+                    if i:
+                        entries.insert(0, entries.pop(i))
+                    return entry[1]
+            depth = max(1, int(os.environ.get("MLPSP_CACHE_SCENES", "2")))
+            entries = [e for e in entries if not self._held_only_here(e[2])][:depth - 1]
+            entry = (key, build(), tuple(sources))
+            setattr(self, slot, [entry] + entries)
             return entry[1]
 
     def _records(self, positions, log_scales, quats):

@@ -211,7 +211,7 @@ def test_scene_invalidation_reaches_the_extension(monkeypatch):
     monkeypatch.setattr(cumodel, "_tile_ext", ext)
     scene = NeuralPrimitiveSceneTileCUDA(num_primitives=4, hidden_dim=32)
     scene.__dict__["_mlpsp_cache"] = {"unit_quats": (("key",), object())}
-    ext._rec = (("k",), object(), ())
+    ext._rec = [(("k",), object(), ())]
     scene.invalidate_render_caches()
     assert "_mlpsp_cache" not in scene.__dict__ and ext._rec is None
 
@@ -234,7 +234,7 @@ def test_derived_tensor_cache_cannot_be_served_to_recycled_memory():
     assert ext._derived("_rec", (first,), (), lambda: build("first")) == "first"
     assert ext._derived("_rec", (first,), (), lambda: build("again")) == "first"        # served from the cache
     del first                                               # the owner lets go; the entry still holds the memory
-    assert ext._rec[2][0].data_ptr() == address
+    assert ext._rec[0][2][0].data_ptr() == address
     second = torch.zeros(8)
     assert second.data_ptr() != address                      # so an equal-shaped newcomer lives elsewhere
     assert ext._derived("_rec", (second,), (), lambda: build("second")) == "second"
@@ -246,10 +246,31 @@ def test_derived_tensor_cache_cannot_be_served_to_recycled_memory():
     assert ext._derived("_pack", (frozen,), (True,), lambda: build("a")) == "a"
     assert ext._derived("_pack", (frozen,), (True,), lambda: build("b")) == "b" and ext._pack is None
     assert built == ["first", "second", "edited", "a", "b"]
+    # the entry of the tensor nobody else holds any more went when the next one was built
+    assert all(e[1] != "first" for e in ext._rec)
     # the note about freshly binned lists holds its two tensors for the same reason
     cand, offsets = torch.zeros(4, dtype=torch.int32), torch.zeros(3, dtype=torch.int32)
     ext.note_binned_lists(cand, offsets, 2, 10)
     assert ext._binned[2] is cand and ext._binned[3] is offsets
+
+
+def test_derived_tensor_cache_keeps_two_scenes_and_drops_the_least_recent(monkeypatch):
+    from mlp_splatting_amd.tile_ext import TileExt
+    ext = TileExt()
+    built = []
+
+    def derived(t, tag):
+        return ext._derived("_pack", (t,), (True,), lambda: built.append(tag) or tag)
+
+    a, b, c = torch.zeros(8), torch.zeros(8), torch.zeros(8)
+    assert [derived(a, "a"), derived(b, "b"), derived(a, "a2"), derived(b, "b2")] == ["a", "b", "a", "b"]
+    assert built == ["a", "b"]                               # two scenes rendered in turn rebuild nothing
+    assert derived(c, "c") == "c" and [e[1] for e in ext._pack] == ["c", "b"]      # the least recent one goes
+    assert derived(a, "a3") == "a3" and [e[1] for e in ext._pack] == ["a3", "c"]
+    monkeypatch.setenv("MLPSP_CACHE_SCENES", "1")
+    assert derived(b, "b3") == "b3" and [e[1] for e in ext._pack] == ["b3"]
+    ext.invalidate_caches()
+    assert ext._pack is None
 
 
 def test_harness_statistics_closed_forms():
