@@ -52,7 +52,10 @@ extern "C" {
 
 typedef void* mlpsp_stream_t;
 
-/* Library version (major*10000 + minor*100 + patch). */
+/* Library version (major*10000 + minor*100 + patch).  MLPSP_VERSION is the version this header describes: a caller
+ * built against it must find mlpsp_version() == MLPSP_VERSION (argument lists and the PrimRecord layout are not
+ * compatible across versions). */
+#define MLPSP_VERSION 300
 int mlpsp_version(void);
 
 /* Message for one MLPSP_E_* bit, worded as the reference's TORCH_CHECK for that condition

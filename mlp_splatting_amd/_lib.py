@@ -20,6 +20,7 @@ TILE_CAPACITY_MAX = 2048
 PIXEL_HIT_CAPACITY = 256
 PRIM_RECORD_BYTES = 128
 MFMA_PACK_BYTES = 7808
+VERSION = 300      # MLPSP_VERSION of include/mlpsp.h: the interface this binding was written against
 
 _vp, _i, _f, _i64, _sz = C.c_void_p, C.c_int, C.c_float, C.c_int64, C.c_size_t
 
@@ -116,6 +117,9 @@ def load():
             raise RuntimeError(f"libmlpsp_hip.so does not export {name}; rebuild the library") from exc
         fn.restype = restype
         fn.argtypes = argtypes
+    if lib.mlpsp_version() != VERSION:
+        raise RuntimeError(f"libmlpsp_hip.so is version {lib.mlpsp_version()}, this binding expects {VERSION}: "
+                           f"rebuild the library (`make -C {CSRC_DIR}`)")
     _lib = lib
     return lib
 

@@ -1012,7 +1012,7 @@ int static_scratch_of_current_device(void** out) {
   MLPSP_HIP_TRY(hipGetDevice(&dev));
   if (dev < 0 || dev >= kMaxDevices) return MLPSP_E_ARGUMENT;
   // (two threads racing here both obtain the same address; the flag is written last)
-  if (!g_static_scratch_known[dev]) {
+  if (!__atomic_load_n(&g_static_scratch_known[dev], __ATOMIC_ACQUIRE)) {
     void* ptr = nullptr;
     MLPSP_HIP_TRY(hipGetSymbolAddress(&ptr, HIP_SYMBOL(mlpsp::scratch)));
     if (!ptr) return MLPSP_E_RUNTIME;

@@ -118,7 +118,7 @@ __global__ __launch_bounds__(kSortThreads) void sort_tiles_kernel(
 
 using namespace mlpsp;
 
-MLPSP_API int mlpsp_version(void) { return 100; }
+MLPSP_API int mlpsp_version(void) { return MLPSP_VERSION; }
 
 MLPSP_API const char* mlpsp_strerror(int code) {
   switch (code) {

@@ -339,8 +339,10 @@ __device__ __forceinline__ void render_tile_mfma(
         j_next = (int)__builtin_ctzll(todo);
         p_next = __builtin_amdgcn_readlane(id_lane, j_next);
         todo &= todo - 1ull;
+        // (only when an entry follows: a request nobody waits for would still be landing in these registers after
+        // the loop, when the compiler has long given them to something else)
+        fast_request(fast_half + (size_t)p_next * sizeof(PrimRecord), q);
       }
-      fast_request(fast_half + (size_t)p_next * sizeof(PrimRecord), q);   // (the last entry asks for its own line again)
       if (__ballot(unsure && live) != 0ull) {   // rare
         if (unsure && live) {
           const PrimRecord P = prims[p];

@@ -28,9 +28,13 @@ namespace mlpsp {
 constexpr int kSortThreads = 256;
 constexpr int kRankPairsMax = 64 * 1024;   // in-bucket comparisons beyond which the sorting network is used instead
 
-// The workgroup's LDS for one tile's sort (27 KB at 2048 entries, 20 KB at 1536).
+// The workgroup's LDS for one tile's sort (27 KB at 2048 entries, 14 KB at 1024).
 template <int kSortMax>
 struct SortLds {
+  // a power of two: the sorting network pads a list to the next power of two inside key[]; a multiple of the
+  // workgroup: every thread handles kSortMax / kSortThreads entries; perm[] and order[] hold 16-bit positions
+  static_assert((kSortMax & (kSortMax - 1)) == 0 && kSortMax % kSortThreads == 0 && kSortMax <= 65536,
+                "capacity of the in-LDS tile sort");
   unsigned long long key[kSortMax];
   int wave_cnt[2][kSortThreads / 64];
   int wave_ok[kSortThreads / 64];

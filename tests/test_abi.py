@@ -50,6 +50,7 @@ def test_status_constants_agree_with_the_header():
     assert int(consts["TILE_CAPACITY_MAX"]) == _lib.TILE_CAPACITY_MAX
     assert int(consts["PIXEL_HIT_CAPACITY"]) == _lib.PIXEL_HIT_CAPACITY == 256
     assert int(consts["PRIM_RECORD_BYTES"]) == _lib.PRIM_RECORD_BYTES
+    assert int(consts["VERSION"]) == _lib.VERSION == _lib.load().mlpsp_version()
 
 
 def test_error_messages_carry_the_reference_wording():
@@ -63,7 +64,7 @@ def test_error_messages_carry_the_reference_wording():
 def test_size_queries_need_no_gpu():
     from mlp_splatting_amd import _lib
     lib = _lib.load()
-    assert lib.mlpsp_version() >= 100
+    assert lib.mlpsp_version() == _lib.VERSION
     assert lib.mlpsp_per_pixel_workspace_bytes(160, 120, 8, 8) == 300 * 64 * 256 * 8 + 256
     assert lib.mlpsp_per_pixel_workspace_bytes(0, 120, 8, 8) == 0
     assert lib.mlpsp_bin_scratch_bytes(5000, 1, 160, 120, 8) > 5000 * 16
