@@ -153,6 +153,230 @@ def train_steps(args, scene, frames, proj, thr, W, H, sc, dev):
     return 0
 
 
+class Workload:
+    """One of synthetic.CONFIGS on the device: the scene module, its camera frames and the call that renders one."""
+
+    def __init__(self, name, precision, poses, dev):
+        import numpy as np
+        import torch
+
+        from mlp_splatting_amd import ops, synthetic as syn
+        from mlp_splatting_amd.cumodel import NeuralPrimitiveSceneTileCUDA
+
+        self.name, self.dev = name, dev
+        self.feature_dim = int(syn.CONFIGS[name]["feature_dim"])
+        self.sc, self.cfg = syn.scene_for_config(name, with_features=False)
+        sc, cfg = self.sc, self.cfg
+        self.W, self.H, self.f, self.thr = cfg["width"], cfg["height"], cfg["focal"], cfg["threshold"]
+        self.precision = precision if sc.hidden == 32 else "f32"   # the matrix-core render exists for the released width
+        self.mosaic = name.startswith("cfg4")
+
+        def t(a):
+            return torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+
+        scene = NeuralPrimitiveSceneTileCUDA(num_primitives=sc.n, hidden_dim=sc.hidden, feature_dim_low=self.feature_dim)
+        scene.load_state_dict({"positions": torch.from_numpy(sc.positions), "log_scales": torch.from_numpy(sc.log_scales),
+                               "quats": torch.from_numpy(sc.quats), "W1": torch.from_numpy(sc.W1),
+                               "b1": torch.from_numpy(sc.b1), "W2": torch.from_numpy(sc.W2), "b2": torch.from_numpy(sc.b2),
+                               "W3": torch.from_numpy(sc.W3), "b3": torch.from_numpy(sc.b3)}, strict=False)
+        scene = scene.to(dev).eval()
+        if self.feature_dim:
+            # feat_attr [N,4,C] ~ N(0, 0.05), drawn on the device (1.6 GB at 200k x 4 x 512)
+            gen = torch.Generator(device=dev)
+            gen.manual_seed(0)
+            with torch.no_grad():
+                scene.feat_attr.copy_(torch.randn(scene.feat_attr.shape, device=dev, generator=gen) * 0.05)
+        scene.set_image_size(self.W, self.H)
+        scene.render_precision = self.precision
+        self.scene = scene
+        self.proj = t(syn.projection_matrix(self.f, self.W, self.H))
+        cams = syn.random_poses(poses, 0)
+        frames, self.skipped_poses = [], 0
+        if self.mosaic:
+            # four views of (W/2) x (H/2) per call; tile t renders view tile_view_ids[t]
+            for g0 in range(0, len(cams) - 3, 4):
+                ro, rd, tv, views = syn.mosaic_frame(self.W // 2, self.H // 2, self.f, cams[g0:g0 + 4])
+                frames.append((t(ro), t(rd), t(views), t(tv)))
+        else:
+            for c2w in cams:
+                ro, rd = syn.pinhole_rays(self.W, self.H, self.f, c2w)
+                frames.append((t(ro), t(rd), t(syn.view_matrix(c2w))[None], None))
+            # A pose whose fullest tile exceeds the 1,536-candidate capacity is an error of the path, not a frame
+            # (the reference raises, and so does this build); the headline scene was constructed so that all 32 poses
+            # fit, the literally specified smaller scenes were not.  Such poses are left out and counted.
+            fitting = []
+            with torch.no_grad():
+                for frame in frames:
+                    longest = ops.bin_legacy(scene.positions.detach(), scene.log_scales.detach(), frame[2].cpu(),
+                                             self.proj.cpu(), self.W, self.H, int(scene.tile_size), self.thr, None,
+                                             with_longest=True)[2]
+                    if int(longest) <= scene._ensure_tile_ext().max_tile_prims:
+                        fitting.append(frame)
+            self.skipped_poses = len(frames) - len(fitting)
+            frames = fitting
+        self.frames = frames
+
+    def render(self, i):
+        import torch
+        ro, rd, views, tv = self.frames[i % len(self.frames)]
+        scene = self.scene
+        with torch.inference_mode():
+            if tv is not None:
+                cand, off = scene.build_tilecenter_culling_from_tile_views(tv, views, self.proj, self.thr)
+                return scene(ro, rd, score_threshold=self.thr, culled_prim_indices=cand, tile_offsets=off)
+            out = scene(ro, rd, score_threshold=self.thr, view_matrix=views[0], proj_matrix=self.proj,
+                        return_feature=bool(self.feature_dim))
+            return out[0] if self.feature_dim else out
+
+    def timed(self, steps, warmup, wake_seconds, min_seconds):
+        """-> (frames/s, seconds, frames timed).  Untimed first: `wake_seconds` of the same frames (a box whose GPU
+        has idled while the scene was built on the host takes a few hundred milliseconds of work to reach its
+        sustained clocks: the first process on a fresh box timed 1.5 ms per frame in this loop and 1.1 ms in the
+        latency loop right after it; a second process 1.1 ms in both), then `warmup` frames.  The timed region is
+        whole passes of `steps` frames until `min_seconds` have gone by."""
+        import torch
+        wake_until = time.perf_counter() + wake_seconds
+        i = 0
+        while time.perf_counter() < wake_until:
+            self.render(i)
+            i += 1
+        for i in range(warmup):
+            self.render(i)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        timed_steps = 0
+        while True:
+            for i in range(steps):
+                self.render(timed_steps + i)
+            timed_steps += steps
+            # (checked on the host clock without a synchronisation: the queue is a few frames deep at most)
+            if time.perf_counter() - t0 >= min_seconds:
+                break
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - t0
+        return timed_steps / elapsed, elapsed, timed_steps
+
+    def probe_stages(self, n_probe=8):
+        """The stages of a frame one by one, with HIP events on the launch stream around each as a frame queues it
+        (no work counters and no read-back inside a bracket), and the render launch once more, untimed, for its
+        work counters.  Means over the first `n_probe` frames -> dict."""
+        import torch
+
+        from mlp_splatting_amd import ops
+        scene, dev, W, H, thr, precision = self.scene, self.dev, self.W, self.H, self.thr, self.precision
+        freq, att = scene._frequency_tables(dev)
+        quats = torch.nn.functional.normalize(scene.quats.detach(), dim=-1).contiguous()
+        weights = [p.detach().contiguous() for p in (scene.W1, scene.b1, scene.W2, scene.b2, scene.W3, scene.b3)]
+        packed = ops.pack_mfma_weights(*weights, bf16=True) if precision == "bf16" else None
+        feat = scene.feat_attr.detach() if self.feature_dim and precision == "bf16" else None
+        packed_feat = ops.pack_mfma_feat(feat)[0] if feat is not None else None
+        n_probe = min(len(self.frames), n_probe)
+        acc = {}
+        # two passes over the same poses: the first only warms the allocator (a first-time tensor size inside
+        # the event brackets would be timed as kernel time), the second is measured
+        for i in list(range(n_probe)) * 2:
+            if i == 0:
+                acc = dict(bin_ms=0.0, sort_ms=0.0, render_ms=0.0, product_ms=0.0, hits=0, proc=0, hit_waves=0, cand=0)
+            ro, rd_raw, views, tv = self.frames[i]
+            rd = torch.nn.functional.normalize(rd_raw, dim=-1).contiguous()
+            e = [torch.cuda.Event(enable_timing=True) for _ in range(5)]
+            rec = ops.prepare_primitives(scene.positions.detach(), scene.log_scales.detach(), quats)
+            cand, off = ops.bin_legacy(scene.positions.detach(), scene.log_scales.detach(), views, self.proj, W, H, 8, thr,
+                                       tile_view_ids=tv)
+            # the binning as a frame queues it: no host synchronisation, candidate buffer sized beforehand
+            e[0].record()
+            ops.bin_legacy_async(scene.positions.detach(), scene.log_scales.detach(), views, self.proj, W, H, 8, thr,
+                                 cand.numel(), tile_view_ids=tv)
+            e[1].record()
+            order, _ = ops.sort_tiles(ro, rd, rec, cand, off, W, H, 8, 8, cull_threshold=thr)
+            e[2].record()
+            counters = torch.zeros(4, dtype=torch.int64, device=dev)
+            if feat is not None:
+                # render with coefficient records, then the feature product, as two calls
+                marks = {2: e[3], 3: e[4]}
+                ops.render_tilecenter_mfma_feat(ro, rd, rec, order, off, freq, att, *weights, feat,
+                                                float(scene.feature_gating_beta), float(scene.feature_gating_temp), W, H,
+                                                thr, bf16=True, packed=packed, packed_feat=packed_feat, check=False,
+                                                stages=lambda k: marks[k].record() if k in marks else None)
+            elif precision == "bf16":
+                ops.render_tilecenter_mfma(ro, rd, rec, order, off, freq, att, *weights, W, H, thr, bf16=True,
+                                           packed=packed, check=False)
+                e[3].record()
+            else:
+                ops.render_tilecenter_f32(ro, rd, rec, order, off, freq, att, *weights, W, H, 8, 8, thr)
+                e[3].record()
+            torch.cuda.synchronize()
+            # the same render launch once more, untimed, for its work counters (their atomics are not part of a frame)
+            if precision == "bf16":
+                ops.render_tilecenter_mfma(ro, rd, rec, order, off, freq, att, *weights, W, H, thr, bf16=True,
+                                           counters=counters, packed=packed)
+            else:
+                ops.render_tilecenter_f32(ro, rd, rec, order, off, freq, att, *weights, W, H, 8, 8, thr, counters=counters)
+            torch.cuda.synchronize()
+            acc["bin_ms"] += e[0].elapsed_time(e[1])
+            acc["sort_ms"] += e[1].elapsed_time(e[2])
+            acc["render_ms"] += e[2].elapsed_time(e[3])
+            if feat is not None:
+                acc["product_ms"] += e[3].elapsed_time(e[4])
+            c = counters.cpu().numpy()
+            acc["hits"] += int(c[3])
+            acc["proc"] += int(c[1])
+            acc["hit_waves"] += int(c[2])
+            acc["cand"] += int(cand.numel())
+        out = {k: v / n_probe for k, v in acc.items()}
+        out["n_probe"] = n_probe
+        return out
+
+
+def other_workload(name, args, dev):
+    """A short leg of another configuration of the same scene family, outside the headline's timed region: one
+    untimed pose cycle, then whole cycles for at least 0.25 s, and the per-launch figures of its dominant kernels
+    (the reference's benchmark also reports RGB and RGB + feature in one run, tools/benchmark_inference.py:264-313)."""
+    import gc
+
+    import torch
+    wl = Workload(name, "bf16", args.poses, dev)
+    if not wl.frames:
+        return {"skipped": "every pose exceeds the tile candidate capacity"}
+    cycle = len(wl.frames)
+    fps, elapsed, steps = wl.timed(cycle, cycle, 0.0, 0.25)
+    st = wl.probe_stages(min(4, cycle))
+    flops_per_hit = 2 * (72 * 32 + 32 * 32 + 4 * 32)
+    render_s = st["render_ms"] * 1e-3
+    tflops = flops_per_hit * st["hits"] / render_s / 1e12
+    kernel = "render_tilecenter_mfma"
+    traffic, note = measured_traffic(kernel, name, st["render_ms"])
+    out = {"fps": round(fps, 2), "ms_per_step": round(1e3 * elapsed / steps, 4), "steps": steps, "dtype": wl.precision,
+           "views_per_call": 4 if wl.mosaic else 1, "feature_channels": wl.feature_dim, "poses": cycle,
+           "stages": {k: round(st[k], 4) for k in ("bin_ms", "sort_ms", "render_ms") + (("product_ms",) if wl.feature_dim else ())},
+           "hits_per_launch": int(st["hits"]), "hit_wavefronts_per_launch": int(st["hit_waves"])}
+    if wl.mosaic:
+        # 17 of a tile's 64 pixels hit per step here: the launch is bound by the weight blocks it streams, one
+        # 7,808-byte block per (tile, primitive) that hits, plus 40 bytes per pixel
+        bytes_alg = 7808.0 * st["hit_waves"] + 40.0 * wl.W * wl.H
+        gbs = bytes_alg / render_s / 1e9
+        out["roofline"] = {"kernel": kernel, "bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                           "frac": round(gbs / HBM_PEAK_GBS, 5), "traffic": traffic, "traffic_source": note,
+                           "ms_per_launch": round(st["render_ms"], 4), "mfma_tflops": round(tflops, 1),
+                           "mfma_frac": round(tflops / PEAK["bf16"], 5)}
+    else:
+        out["roofline"] = {"kernel": kernel, "bound": "mfma", "achieved": round(tflops, 1), "peak": PEAK["bf16"],
+                           "unit": "TFLOP/s", "frac": round(tflops / PEAK["bf16"], 5), "traffic": traffic,
+                           "traffic_source": note, "ms_per_launch": round(st["render_ms"], 4)}
+    if wl.feature_dim:
+        # feature product: the f32 image written once + the fp16 coefficient records (64 pixels x 8 bytes per hit step)
+        bytes_alg = 4.0 * wl.W * wl.H * wl.feature_dim + 512.0 * st["hit_waves"]
+        gbs = bytes_alg / (st["product_ms"] * 1e-3) / 1e9
+        ptraffic, pnote = measured_traffic("feat_gemm", name, st["product_ms"])
+        out["feature_product"] = {"kernel": "feat_gemm", "bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS,
+                                  "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 5), "traffic": ptraffic,
+                                  "traffic_source": pnote, "ms_per_launch": round(st["product_ms"], 4)}
+    del wl
+    gc.collect()
+    torch.cuda.empty_cache()
+    return out
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -174,6 +398,9 @@ def main() -> int:
                     help="the timed region is extended, in whole passes of --steps, until it lasts at least this long; "
                          "the JSON line reports the steps actually timed")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-other-workloads", action="store_true",
+                    help="skip the short legs of the feature (cfg5) and mosaic (cfg4) configurations that the default "
+                         "run of the headline workload appends under other_workloads")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run 4 plain device copies of 1 GiB, the known-size kernel that hardware counter "
                          "readings of a profiled run are scaled by")
@@ -186,106 +413,30 @@ def main() -> int:
     import numpy as np
     import torch
 
-    from mlp_splatting_amd import _lib, ops, synthetic as syn
-    from mlp_splatting_amd.cumodel import NeuralPrimitiveSceneTileCUDA
+    from mlp_splatting_amd import _lib, ops
 
     _lib.load()
     dev = torch.device("cuda", int(os.environ.get("LOCAL_RANK", "0")))
     torch.cuda.set_device(dev)
     precision = args.precision or ("bf16" if hasattr(ops, "render_tilecenter_mfma") else "f32")
 
-    feature_dim = int(syn.CONFIGS[args.workload]["feature_dim"])
-    sc, cfg = syn.scene_for_config(args.workload, with_features=False)
-    W, H, f, thr = cfg["width"], cfg["height"], cfg["focal"], cfg["threshold"]
-    if precision == "bf16" and sc.hidden != 32:
+    wl = Workload(args.workload, precision, args.poses, dev)
+    if precision == "bf16" and wl.precision != "bf16":
         if args.precision == "bf16":
-            print(f"--precision bf16 needs the 72->32->32->4 MLP; {args.workload} has hidden width {sc.hidden}", file=sys.stderr)
+            print(f"--precision bf16 needs the 72->32->32->4 MLP; {args.workload} has hidden width {wl.sc.hidden}", file=sys.stderr)
             return 2
-        precision = "f32"        # the matrix-core render exists for the released MLP width only (as the reference's)
-    mosaic = args.workload.startswith("cfg4")
-
-    def t(a):
-        return torch.from_numpy(np.ascontiguousarray(a)).to(dev)
-
-    scene = NeuralPrimitiveSceneTileCUDA(num_primitives=sc.n, hidden_dim=sc.hidden, feature_dim_low=feature_dim)
-    scene.load_state_dict({"positions": torch.from_numpy(sc.positions), "log_scales": torch.from_numpy(sc.log_scales),
-                           "quats": torch.from_numpy(sc.quats), "W1": torch.from_numpy(sc.W1),
-                           "b1": torch.from_numpy(sc.b1), "W2": torch.from_numpy(sc.W2), "b2": torch.from_numpy(sc.b2),
-                           "W3": torch.from_numpy(sc.W3), "b3": torch.from_numpy(sc.b3)}, strict=False)
-    scene = scene.to(dev).eval()
-    if feature_dim:
-        # feat_attr [N,4,C] ~ N(0, 0.05), drawn on the device (1.6 GB at 200k x 4 x 512)
-        gen = torch.Generator(device=dev)
-        gen.manual_seed(0)
-        with torch.no_grad():
-            scene.feat_attr.copy_(torch.randn(scene.feat_attr.shape, device=dev, generator=gen) * 0.05)
-    scene.set_image_size(W, H)
-    scene.render_precision = precision
-    proj = t(syn.projection_matrix(f, W, H))
-    poses = syn.random_poses(args.poses, 0)
-    frames, skipped_poses = [], 0
-    if mosaic:
-        # four views of (W/2) x (H/2) per call; tile t renders view tile_view_ids[t]
-        for g0 in range(0, len(poses) - 3, 4):
-            ro, rd, tv, views = syn.mosaic_frame(W // 2, H // 2, f, poses[g0:g0 + 4])
-            frames.append((t(ro), t(rd), t(views), t(tv)))
-    else:
-        for c2w in poses:
-            ro, rd = syn.pinhole_rays(W, H, f, c2w)
-            frames.append((t(ro), t(rd), t(syn.view_matrix(c2w))[None], None))
-        # A pose whose fullest tile exceeds the 1,536-candidate capacity is an error of the path, not a frame
-        # (the reference raises, and so does this build); the headline scene was constructed so that all 32 poses
-        # fit, the literally specified smaller scenes were not.  Such poses are left out and counted.
-        fitting = []
-        with torch.no_grad():
-            for frame in frames:
-                longest = ops.bin_legacy(scene.positions.detach(), scene.log_scales.detach(), frame[2].cpu(), proj.cpu(), W, H,
-                                         int(scene.tile_size), thr, None, with_longest=True)[2]
-                if int(longest) <= scene._ensure_tile_ext().max_tile_prims:
-                    fitting.append(frame)
-        skipped_poses = len(frames) - len(fitting)
-        if not fitting:
-            print(f"{args.workload}: every pose exceeds the tile candidate capacity", file=sys.stderr)
-            return 2
-        frames = fitting
+        precision = "f32"
+    sc, cfg, scene, frames, proj = wl.sc, wl.cfg, wl.scene, wl.frames, wl.proj
+    W, H, thr, feature_dim, mosaic, skipped_poses = wl.W, wl.H, wl.thr, wl.feature_dim, wl.mosaic, wl.skipped_poses
+    if not frames:
+        print(f"{args.workload}: every pose exceeds the tile candidate capacity", file=sys.stderr)
+        return 2
 
     if args.train:
         return train_steps(args, scene, frames, proj, thr, W, H, sc, dev)
 
-    def render(i):
-        ro, rd, views, tv = frames[i % len(frames)]
-        with torch.inference_mode():
-            if tv is not None:
-                cand, off = scene.build_tilecenter_culling_from_tile_views(tv, views, proj, thr)
-                return scene(ro, rd, score_threshold=thr, culled_prim_indices=cand, tile_offsets=off)
-            out = scene(ro, rd, score_threshold=thr, view_matrix=views[0], proj_matrix=proj,
-                        return_feature=bool(feature_dim))
-            return out[0] if feature_dim else out
-
-    # Untimed, before the W warm-up steps: keep the device busy with the same frames for a second.  A box whose
-    # GPU has idled while the scene was built on the host takes a few hundred milliseconds of work to reach its
-    # sustained clocks (measured: the first process on a fresh box timed 1.5 ms per frame in this loop and
-    # 1.1 ms in the latency loop right after it; a second process 1.1 ms in both).
-    wake_until = time.perf_counter() + args.wake_seconds
-    i = 0
-    while time.perf_counter() < wake_until:
-        render(i)
-        i += 1
-    for i in range(args.warmup):
-        render(i)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    timed_steps = 0
-    while True:
-        for i in range(args.steps):
-            render(timed_steps + i)
-        timed_steps += args.steps
-        # (checked on the host clock without a synchronisation: the queue is a few frames deep at most)
-        if time.perf_counter() - t0 >= args.min_seconds:
-            break
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
-    fps = timed_steps / elapsed
+    render = wl.render
+    fps, elapsed, timed_steps = wl.timed(args.steps, args.warmup, args.wake_seconds, args.min_seconds)
 
     # per-frame latency distribution, the way tools/benchmark_inference.py:121-149 times a frame: a
     # synchronise on both sides of every call (so nothing overlaps between frames, unlike the loop above)
@@ -300,55 +451,13 @@ def main() -> int:
     latency = {k: (round(v, 4) if isinstance(v, float) else v) for k, v in timing_stats(lat).items()}
     latency["frames"] = latency.pop("samples")
 
-    # ---- the render kernel alone: HIP events on the stream it is launched on, and its work counters
+    # ---- the stages of a frame alone: HIP events on the stream they are launched on, and the render's work counters
+    st = wl.probe_stages(8)
+    n_probe = st["n_probe"]
+    kernel_ms, sort_ms, bin_ms = st["render_ms"] * n_probe, st["sort_ms"] * n_probe, st["bin_ms"] * n_probe
+    hits, proc, hit_waves, cand_total = (int(st[k] * n_probe) for k in ("hits", "proc", "hit_waves", "cand"))
     freq, att = scene._frequency_tables(dev)
     quats = torch.nn.functional.normalize(scene.quats.detach(), dim=-1).contiguous()
-    weights = [p.detach().contiguous() for p in (scene.W1, scene.b1, scene.W2, scene.b2, scene.W3, scene.b3)]
-    kernel_ms, hits, proc, cand_total, sort_ms, bin_ms, hit_waves = 0.0, 0, 0, 0, 0.0, 0.0, 0
-    packed = ops.pack_mfma_weights(*weights, bf16=True) if precision == "bf16" else None
-    n_probe = min(len(frames), 8)
-    # two passes over the same poses: the first only warms the allocator (a first-time tensor size inside
-    # the event brackets would be timed as kernel time), the second is measured
-    for i in list(range(n_probe)) * 2:
-        if i == 0:
-            kernel_ms, hits, proc, cand_total, sort_ms, bin_ms, hit_waves = 0.0, 0, 0, 0, 0.0, 0.0, 0
-        ro, rd_raw, views, tv = frames[i]
-        rd = torch.nn.functional.normalize(rd_raw, dim=-1).contiguous()
-        e = [torch.cuda.Event(enable_timing=True) for _ in range(4)]
-        rec = ops.prepare_primitives(scene.positions.detach(), scene.log_scales.detach(), quats)
-        cand, off = ops.bin_legacy(scene.positions.detach(), scene.log_scales.detach(), views, proj, W, H, 8, thr,
-                                   tile_view_ids=tv)
-        # the binning as a frame queues it: no host synchronisation, candidate buffer sized beforehand
-        e[0].record()
-        ops.bin_legacy_async(scene.positions.detach(), scene.log_scales.detach(), views, proj, W, H, 8, thr,
-                             cand.numel(), tile_view_ids=tv)
-        e[1].record()
-        order, _ = ops.sort_tiles(ro, rd, rec, cand, off, W, H, 8, 8, cull_threshold=thr)
-        e[2].record()
-        # timed as a frame launches it: no work counters (their atomics are not part of a frame) and no flag read-back
-        if precision == "bf16":
-            ops.render_tilecenter_mfma(ro, rd, rec, order, off, freq, att, *weights, W, H, thr, bf16=True,
-                                       packed=packed, check=False)
-        else:
-            ops.render_tilecenter_f32(ro, rd, rec, order, off, freq, att, *weights, W, H, 8, 8, thr)
-        e[3].record()
-        torch.cuda.synchronize()
-        # the same launch once more, untimed, for its work counters
-        counters = torch.zeros(4, dtype=torch.int64, device=dev)
-        if precision == "bf16":
-            ops.render_tilecenter_mfma(ro, rd, rec, order, off, freq, att, *weights, W, H, thr, bf16=True,
-                                       counters=counters, packed=packed)
-        else:
-            ops.render_tilecenter_f32(ro, rd, rec, order, off, freq, att, *weights, W, H, 8, 8, thr, counters=counters)
-        torch.cuda.synchronize()
-        bin_ms += e[0].elapsed_time(e[1])
-        sort_ms += e[1].elapsed_time(e[2])
-        kernel_ms += e[2].elapsed_time(e[3])
-        c = counters.cpu().numpy()
-        hits += int(c[3])
-        proc += int(c[1])
-        hit_waves += int(c[2])
-        cand_total += int(cand.numel())
     # what the matrix cores sustain on this box with nothing else in the way
     mfma_probe = None
     if precision == "bf16":
@@ -495,6 +604,14 @@ def main() -> int:
                 "kind": "reference culling expression, CPU torch", "ms": None,
                 "skipped": (f"tiles x primitives = {sc.n * T_tiles:.3g}: the dense overlap matrix is timed only up to 3e8 "
                             "elements and for one view (run --workload cfg1_5k_160x120 or cfg2_50k_640x480)")}
+    # ---- short legs of the feature and the mosaic configuration (the headline fields above are not touched)
+    if args.workload.startswith("cfg3") and precision == "bf16" and not args.no_other_workloads:
+        del wl, scene, frames, render
+        import gc
+        gc.collect()
+        torch.cuda.empty_cache()
+        out["other_workloads"] = {name: other_workload(name, args, dev)
+                                  for name in ("cfg5_200k_feat512", "cfg4_200k_mosaic4")}
     print(json.dumps(out))
     return 0
 

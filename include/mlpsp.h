@@ -43,6 +43,7 @@ extern "C" {
 #define MLPSP_PIXEL_HIT_CAPACITY 256 /* per-pixel-order hit buffer (np_tile_kernels.cu:760) */
 #define MLPSP_PRIM_RECORD_BYTES 128  /* bytes per primitive of the prepared geometry buffer */
 #define MLPSP_MFMA_PACK_BYTES 7808   /* bytes per primitive of the packed matrix-core weight buffer */
+#define MLPSP_SORT_RECORD_BYTES 64   /* bytes per primitive (+ one header slot) of the sort's per-frame records */
 #define MLPSP_BIN_STATIC_SCRATCH_BYTES 67108864 /* scratch array of mlpsp_bin_legacy_async_noalloc (64 MiB) */
 #define MLPSP_BIN_STATIC_MAX_VIEWS 8           /* most views mlpsp_bin_legacy_async_noalloc accepts */
 
@@ -162,11 +163,18 @@ int mlpsp_bin_raycone_fill(int num_primitives, int width, int height, int tile, 
  * reference, whose kernels run the full ray test on every candidate.
  * prim_records_dev holds num_primitives records.  Null pointers (sorted_keys_dev aside) return MLPSP_E_ARGUMENT;
  * a candidate id outside [0, num_primitives) -- a list that was not validated -- is not dereferenced: it sorts
- * last with the invalid key and is passed on as it is (the render entry points skip such ids). */
+ * last with the invalid key and is passed on as it is (the render entry points skip such ids).
+ * frame_records_dev: NULL, or mlpsp_sort_frame_records_bytes(num_primitives) bytes of scratch, 64-byte aligned.
+ * With it, one more launch first writes a 64-byte record per primitive for the origin of ray 0 -- the rotated
+ * offset centre - origin of the key (np_tile_kernels.cu:483-500), which depends on the primitive alone when the
+ * rays share an origin -- and every tile whose centre ray starts at that origin takes its keys from those records
+ * (one quaternion rotation per candidate instead of two; same expressions, same key bits); other tiles, and every
+ * tile without the scratch, evaluate the key in full.  Sorted ids and keys do not depend on it. */
+size_t mlpsp_sort_frame_records_bytes(int num_primitives);
 int mlpsp_sort_tiles(const float* rays_o_dev, const float* rays_d_dev, const void* prim_records_dev,
                      int num_primitives, const int32_t* candidates_dev, const int32_t* tile_offsets_dev, int width,
                      int height, int tile_w, int tile_h, int key_family, int capacity, float cull_threshold,
-                     int32_t* sorted_ids_dev, float* sorted_keys_dev, mlpsp_stream_t stream);
+                     void* frame_records_dev, int32_t* sorted_ids_dev, float* sorted_keys_dev, mlpsp_stream_t stream);
 
 /* Tile-centre-order forward, scalar f32 (render_tiles_kernel_tilecenter_order,
  * np_tile_kernels.cu:1837-2137; with out_t_dev != NULL also the expected depth of :5432-5719).
@@ -364,7 +372,10 @@ int mlpsp_render_tilecenter_mfma(const float* rays_o_dev, const float* rays_d_de
  * num_pairs = length of order_dev = tile_offsets[num_tiles].  feat_slots = 0 renders RGB only and
  * ignores the feature and workspace arguments.  Workspace: mlpsp_feat_workspace_bytes(.., fp16_records = 1, ..);
  * status_dev[1] = 1 if its record pool ran out.  MLPSP_E_SCRATCH if the workspace is too small or not
- * 256-byte aligned. */
+ * 256-byte aligned.
+ * stage: 0 = the whole frame; 1 = the render launch alone (RGB, alpha and the coefficient records in the workspace);
+ * 2 = the feature product alone, over the records a stage-1 call with the same arguments left in the same workspace
+ * (for timing the two launches apart; 1 and 2 need feat_slots != 0). */
 size_t mlpsp_mfma_feat_pack_bytes(int num_primitives, int feat_slots, int feat_channels);
 int mlpsp_pack_mfma_feat(const float* feat_attr_dev, int num_primitives, int feat_slots, int feat_channels,
                          void* packed_feat_dev, int32_t* status_dev, mlpsp_stream_t stream);
@@ -378,7 +389,7 @@ int mlpsp_render_tilecenter_mfma_feat(const float* rays_o_dev, const float* rays
                                       int feat_channels, float gating_beta, float gating_temp, int width, int height,
                                       float threshold, void* workspace_dev, size_t workspace_bytes,
                                       float* out_rgb_dev, float* out_alpha_dev, float* out_feat_dev,
-                                      int32_t* status_dev, int64_t* counters_dev, mlpsp_stream_t stream);
+                                      int32_t* status_dev, int64_t* counters_dev, int stage, mlpsp_stream_t stream);
 
 /* Weight and bias gradients of the per-primitive 72->32->32->4 MLP over a primitive-major CSR of hit records
  * = the Triton kernel _grouped_vjp (scannet/primitive_gemm.py:101-166, launched at :214-230).  Segment g covers

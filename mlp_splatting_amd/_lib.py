@@ -45,7 +45,8 @@ SIGNATURES = {
     "mlpsp_bin_raycone_scratch_bytes": (_sz, [_i, _i, _i, _i]),
     "mlpsp_bin_raycone_count": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _f, _vp, _sz, _vp, C.POINTER(_i64), _vp]),
     "mlpsp_bin_raycone_fill": (_i, [_i, _i, _i, _i, _vp, _sz, _vp, _vp, _vp]),
-    "mlpsp_sort_tiles": (_i, [_vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _vp, _vp, _vp]),
+    "mlpsp_sort_frame_records_bytes": (_sz, [_i]),
+    "mlpsp_sort_tiles": (_i, [_vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _vp, _vp, _vp, _vp]),
     "mlpsp_render_tilecenter_f32": (_i, [_vp] * 7 + [_i] + [_vp] * 6 + [_i, _i, _i, _i, _i, _i, _f, _vp, _vp, _vp,
                                                                        _vp, _vp]),
     "mlpsp_render_tilecenter_feat_f32": (_i, [_vp] * 7 + [_i] + [_vp] * 6 + [_i, _i, _vp, _i, _i, _f, _f, _i, _i, _i, _i,
@@ -71,7 +72,7 @@ SIGNATURES = {
     "mlpsp_all_finite": (_i, [_vp, _vp, _i, _vp, _vp]),
     "mlpsp_feat_workspace_bytes": (_sz, [_i64, _i, _i, _i, _i, _i, _i, _i64]),
     "mlpsp_render_tilecenter_mfma_feat": (_i, [_vp] * 5 + [_i64, _vp, _vp, _vp, _i, _i, _vp, _i, _i, _f, _f, _i, _i, _f,
-                                               _vp, _sz, _vp, _vp, _vp, _vp, _vp, _vp]),
+                                               _vp, _sz, _vp, _vp, _vp, _vp, _vp, _i, _vp]),
     "mlpsp_probe_mfma_bf16": (_i64, [_i, _vp, _vp]),
     "mlpsp_probe_issue": (_i, [C.POINTER(C.c_int32), _i, _vp, _vp, _vp]),
     "mlpsp_grouped_vjp": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _f, _i, _vp,

@@ -99,19 +99,21 @@ __global__ __launch_bounds__(256) void normalize_rays_kernel(const float* __rest
 // tile gathers are mostly those of its neighbours.
 __global__ __launch_bounds__(kSortThreads) void sort_tiles_kernel(
     const float* __restrict__ rays_o, const float* __restrict__ rays_d, const PrimRecord* __restrict__ prims,
-    const int32_t* __restrict__ cand, const int32_t* __restrict__ offsets, TileGeom g, int family, int capacity,
-    float cull_r2, int num_prims, int32_t* __restrict__ sorted_ids, float* __restrict__ sorted_keys) {
+    const SortRec* __restrict__ frame, const int32_t* __restrict__ cand, const int32_t* __restrict__ offsets, TileGeom g,
+    int family, int capacity, float cull_r2, int num_prims, int32_t* __restrict__ sorted_ids,
+    float* __restrict__ sorted_keys) {
   const int tile = superblock_tile(blockIdx.x, g.ntx, g.nty);
   if (tile < 0) return;
   const int start = offsets[tile], len = offsets[tile + 1] - start;
   if (len <= 64 && len <= capacity) {       // a short list: the first wavefront alone, in registers
     if (len > 0 && threadIdx.x < 64)
-      sort_small_tile(rays_o, rays_d, prims, cand, g, family, cull_r2, num_prims, sorted_ids, sorted_keys, tile, start, len);
+      sort_small_tile(rays_o, rays_d, prims, frame, cand, g, family, cull_r2, num_prims, sorted_ids, sorted_keys, tile, start,
+                      len);
     return;
   }
   __shared__ SortLds<MLPSP_TILE_CAPACITY_MAX> lds;
-  sort_one_tile<MLPSP_TILE_CAPACITY_MAX>(lds, rays_o, rays_d, prims, cand, offsets, g, family, capacity, cull_r2, num_prims,
-                                         sorted_ids, sorted_keys, tile);
+  sort_one_tile<MLPSP_TILE_CAPACITY_MAX>(lds, rays_o, rays_d, prims, frame, cand, offsets, g, family, capacity, cull_r2,
+                                         num_prims, sorted_ids, sorted_keys, tile);
 }
 
 }  // namespace mlpsp
@@ -187,11 +189,15 @@ MLPSP_API int mlpsp_validate_tile_lists(const int32_t* tile_offsets_dev, const i
   return mask;
 }
 
+MLPSP_API size_t mlpsp_sort_frame_records_bytes(int num_primitives) {
+  return num_primitives < 0 ? 0 : ((size_t)num_primitives + 1) * sizeof(SortRec);
+}
+
 MLPSP_API int mlpsp_sort_tiles(const float* rays_o_dev, const float* rays_d_dev, const void* prim_records_dev,
                                int num_primitives, const int32_t* candidates_dev, const int32_t* tile_offsets_dev,
                                int width, int height, int tile_w, int tile_h, int key_family, int capacity,
-                               float cull_threshold, int32_t* sorted_ids_dev, float* sorted_keys_dev,
-                               mlpsp_stream_t stream) {
+                               float cull_threshold, void* frame_records_dev, int32_t* sorted_ids_dev,
+                               float* sorted_keys_dev, mlpsp_stream_t stream) {
   const int64_t T = checked_num_tiles(width, height, tile_w, tile_h);
   if (T <= 0 || T > 2147483647LL) return MLPSP_E_ARGUMENT;
   if (key_family != MLPSP_KEY_TSTAR && key_family != MLPSP_KEY_DEPTH) return MLPSP_E_ARGUMENT;
@@ -200,13 +206,20 @@ MLPSP_API int mlpsp_sort_tiles(const float* rays_o_dev, const float* rays_d_dev,
   if (!rays_o_dev || !rays_d_dev || !tile_offsets_dev || !candidates_dev || !sorted_ids_dev) return MLPSP_E_ARGUMENT;
   if (num_primitives <= 0 || !prim_records_dev) return MLPSP_E_ARGUMENT;
   if (sorted_ids_dev == candidates_dev) return MLPSP_E_ARGUMENT;   // not an in-place sort
+  if (reinterpret_cast<uintptr_t>(frame_records_dev) % 64 != 0) return MLPSP_E_ARGUMENT;
   TileGeom g{width, height, tile_w, tile_h, ceil_div(width, tile_w), ceil_div(height, tile_h)};
   // squared radius of the threshold ellipsoid in units of the scales, with a 2 % margin on the radius
   float cull_r2 = 0.f;
   if (cull_threshold > 0.f && cull_threshold < 1.f) cull_r2 = -2.0f * logf(cull_threshold) * 1.0404f + 1e-6f;
+  // per-frame records for the origin of ray 0: every tile whose centre ray starts there takes its keys from them
+  if (frame_records_dev) {
+    hipLaunchKernelGGL(frame_sort_records_kernel, dim3(ceil_div(num_primitives, 256)), dim3(256), 0, (hipStream_t)stream,
+                       rays_o_dev, (const PrimRecord*)prim_records_dev, num_primitives, (SortRec*)frame_records_dev);
+    MLPSP_LAUNCH_CHECK();
+  }
   hipLaunchKernelGGL(sort_tiles_kernel, dim3(superblock_grid(g.ntx, g.nty)), dim3(kSortThreads), 0, (hipStream_t)stream, rays_o_dev,
-                     rays_d_dev, (const PrimRecord*)prim_records_dev, candidates_dev, tile_offsets_dev, g, key_family,
-                     capacity, cull_r2, num_primitives, sorted_ids_dev, sorted_keys_dev);
+                     rays_d_dev, (const PrimRecord*)prim_records_dev, (const SortRec*)frame_records_dev, candidates_dev,
+                     tile_offsets_dev, g, key_family, capacity, cull_r2, num_primitives, sorted_ids_dev, sorted_keys_dev);
   MLPSP_LAUNCH_CHECK();
   return MLPSP_OK;
 }

@@ -848,8 +848,9 @@ MLPSP_API int mlpsp_render_tilecenter_mfma_feat(const float* rays_o_dev, const f
                                                 float gating_temp, int width, int height, float threshold,
                                                 void* workspace_dev, size_t workspace_bytes, float* out_rgb_dev,
                                                 float* out_alpha_dev, float* out_feat_dev, int32_t* status_dev,
-                                                int64_t* counters_dev, mlpsp_stream_t stream) {
+                                                int64_t* counters_dev, int stage, mlpsp_stream_t stream) {
   const int64_t T = checked_num_tiles(width, height, 8, 8);
+  if (stage < 0 || stage > 2 || (stage != 0 && feat_slots == 0)) return MLPSP_E_ARGUMENT;
   if (T <= 0 || T > 2147483647LL - 8 || num_primitives < 0 || num_pairs < 0 || num_pairs > 2147483647LL)
     return MLPSP_E_ARGUMENT;
   if (!rays_o_dev || !rays_d_dev || !tile_offsets_dev || !freq_dev || !att_dev || !out_rgb_dev || !out_alpha_dev ||
@@ -866,9 +867,9 @@ MLPSP_API int mlpsp_render_tilecenter_mfma_feat(const float* rays_o_dev, const f
         workspace_bytes < hitpool_min_bytes(num_pairs, T, 1))
       return MLPSP_E_SCRATCH;
     hp = hitpool_carve(workspace_dev, workspace_bytes, num_pairs, T, 1, 64 * 2 * feat_pad(feat_slots));
-    MLPSP_HIP_TRY(hipMemsetAsync(hp.counters, 0, 64 * sizeof(int32_t), s));
+    if (stage != 2) MLPSP_HIP_TRY(hipMemsetAsync(hp.counters, 0, 64 * sizeof(int32_t), s));
   }
-  MLPSP_HIP_TRY(hipMemsetAsync(status_dev, 0, 16 * sizeof(int32_t), s));
+  if (stage != 2) MLPSP_HIP_TRY(hipMemsetAsync(status_dev, 0, 16 * sizeof(int32_t), s));
   const int per_xcd = (int)((T + kNumXcd - 1) / kNumXcd);
   const int ntx = ceil_div(width, 8);
   const dim3 grid(superblock_grid(ntx, ceil_div(height, 8)));
@@ -884,12 +885,14 @@ MLPSP_API int mlpsp_render_tilecenter_mfma_feat(const float* rays_o_dev, const f
     else if (sp == 4) MLPSP_MFMA_GO(TT, 4); \
     else MLPSP_MFMA_GO(TT, 8);            \
   } while (0)
-  if (use_bf16) MLPSP_MFMA_SP(__bf16);
-  else MLPSP_MFMA_SP(_Float16);
+  if (stage != 2) {
+    if (use_bf16) MLPSP_MFMA_SP(__bf16);
+    else MLPSP_MFMA_SP(_Float16);
+    MLPSP_LAUNCH_CHECK();
+  }
 #undef MLPSP_MFMA_SP
 #undef MLPSP_MFMA_GO
-  MLPSP_LAUNCH_CHECK();
-  if (sp != 0) {
+  if (sp != 0 && stage != 1) {
     const dim3 ggrid(superblock_grid(ntx, ceil_div(height, 8)), (unsigned)ceil_div(feat_channels, 128 * kGemmNcb)), gblock(256);
 #define MLPSP_FEAT_GEMM(SP)                                                                                       \
   hipLaunchKernelGGL((feat_gemm_kernel<SP, kGemmNcb>), ggrid, gblock, 0, s, (const unsigned*)packed_feat_dev, hp, \
@@ -914,7 +917,7 @@ MLPSP_API int mlpsp_render_tilecenter_mfma(const float* rays_o_dev, const float*
   return mlpsp_render_tilecenter_mfma_feat(rays_o_dev, rays_d_dev, prim_records_dev, order_dev, tile_offsets_dev, 0,
                                            freq_dev, att_dev, packed_dev, num_primitives, use_bf16, nullptr, 0, 0, 0.f,
                                            0.f, width, height, threshold, nullptr, 0, out_rgb_dev, out_alpha_dev,
-                                           nullptr, status_dev, counters_dev, stream);
+                                           nullptr, status_dev, counters_dev, 0, stream);
 }
 
 MLPSP_API int64_t mlpsp_probe_mfma_bf16(int iterations, float* sink_dev, mlpsp_stream_t stream) {

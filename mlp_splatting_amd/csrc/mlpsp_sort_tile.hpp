@@ -37,107 +37,277 @@ struct SortLds {
                 "capacity of the in-LDS tile sort");
   unsigned long long key[kSortMax];
   int wave_cnt[2][kSortThreads / 64];
-  int wave_ok[kSortThreads / 64];
   int cnt[kSortThreads], off[kSortThreads];
   uint16_t perm[kSortMax], order[kSortMax];
   uint32_t kmin, kmax;
   int flags, pairs;
 };
 
+// Per-frame, per-primitive record of the sort (64 bytes, one cache line per candidate): what the key and the culling
+// test need of a primitive once the ray origin is known.  Whenever the rays of a frame start from one point (a
+// pinhole camera: always) the rotated offset vl = R(q)^T (c - o) of the key (np_tile_kernels.cu:483-500) depends on
+// the primitive alone; frame_sort_records_kernel evaluates it once per primitive with the very expressions of
+// key_tstar(), so the key of a candidate costs one quaternion rotation (the ray direction's) instead of two, with
+// the same bits.  For the culling test the record carries e = c - o and the world-space covariance
+// S = R diag(s^2) R^T, so that the support of the threshold ellipsoid along a face normal n is the quadratic form
+// n^T S n (six multiply-adds against per-tile products of the normal) instead of a rotation of n per face.  S is
+// stored as six bf16 values rounded so that the stored matrix minus the exact one is positive semi-definite
+// (off-diagonal entries to nearest, every diagonal entry raised by its row's rounding errors plus 1e-5 of the
+// trace, then rounded up): the quadratic form never comes out smaller than the exact one, i.e. the test stays
+// conservative, at a few percent of the smallest axis for ordinary shapes.
+struct __attribute__((aligned(64))) SortRec {
+  float qw, qx, qy, qz;
+  float mx, my, mz, vlx;
+  float vly, vlz, ex, ey;
+  float ez;
+  uint32_t s_xx_yy, s_zz_xy, s_xz_yz;      // (first << 16 | second), each the upper half of an f32
+};
+static_assert(sizeof(SortRec) == MLPSP_SORT_RECORD_BYTES, "record size is part of the C ABI");
+// Slot 0 of the record buffer: the origin the records were made for (its bits) and whether they were made at all.
+struct __attribute__((aligned(64))) SortFrameHeader {
+  uint32_t ox, oy, oz;
+  int32_t valid;
+  uint32_t pad[12];
+};
+static_assert(sizeof(SortFrameHeader) == sizeof(SortRec), "the header takes one record slot");
+
+__device__ __forceinline__ uint32_t bf16_nearest(float x) {     // upper 16 bits, round to nearest even
+  const uint32_t u = float_to_bits(x);
+  return (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+}
+__device__ __forceinline__ uint32_t bf16_up(float x) {          // x >= 0: the smallest bf16 at or above x
+  const uint32_t u = float_to_bits(x);
+  return (u >> 16) + ((u & 0xffffu) ? 1u : 0u);
+}
+
+// One thread per primitive; thread 0 of block 0 also writes the header.  origin = rays_o[0..2].
+__global__ __launch_bounds__(256) void frame_sort_records_kernel(const float* __restrict__ rays_o,
+                                                                 const PrimRecord* __restrict__ prims, int N,
+                                                                 SortRec* __restrict__ out) {
+  const int p = blockIdx.x * blockDim.x + threadIdx.x;
+  const float ox = rays_o[0], oy = rays_o[1], oz = rays_o[2];
+  if (p == 0) {
+    SortFrameHeader h = {};
+    h.ox = float_to_bits(ox);
+    h.oy = float_to_bits(oy);
+    h.oz = float_to_bits(oz);
+    h.valid = 1;
+    *reinterpret_cast<SortFrameHeader*>(out) = h;
+  }
+  if (p >= N) return;
+  const float4* src = reinterpret_cast<const float4*>(prims + p);
+  const float4 a = src[0], b = src[1], c = src[2], d = src[3];
+  PrimRecord P;
+  P.cx = a.x; P.cy = a.y; P.cz = a.z; P.mx = a.w;
+  P.my = b.x; P.mz = b.y; P.qw = b.z; P.qx = b.w;
+  P.qy = c.x; P.qz = c.y;
+  P.s2x = d.y; P.s2y = d.z; P.s2z = d.w;
+  // exactly the first statements of key_tstar()
+  const Vec3 v = {P.cx - ox, P.cy - oy, P.cz - oz};
+  const Vec3 vl = quat_rotate_conj(P.qw, P.qx, P.qy, P.qz, v);
+  // covariance in world axes: columns of R(q) are the ellipsoid's axes
+  const float w = P.qw, x = P.qx, y = P.qy, z = P.qz;
+  const float r00 = 1.f - 2.f * (y * y + z * z), r01 = 2.f * (x * y - w * z), r02 = 2.f * (x * z + w * y);
+  const float r10 = 2.f * (x * y + w * z), r11 = 1.f - 2.f * (x * x + z * z), r12 = 2.f * (y * z - w * x);
+  const float r20 = 2.f * (x * z - w * y), r21 = 2.f * (y * z + w * x), r22 = 1.f - 2.f * (x * x + y * y);
+  const float sx = P.s2x, sy = P.s2y, sz = P.s2z;
+  const float cxx = fmaf(sx, r00 * r00, fmaf(sy, r01 * r01, sz * (r02 * r02)));
+  const float cyy = fmaf(sx, r10 * r10, fmaf(sy, r11 * r11, sz * (r12 * r12)));
+  const float czz = fmaf(sx, r20 * r20, fmaf(sy, r21 * r21, sz * (r22 * r22)));
+  const float cxy = fmaf(sx, r00 * r10, fmaf(sy, r01 * r11, sz * (r02 * r12)));
+  const float cxz = fmaf(sx, r00 * r20, fmaf(sy, r01 * r21, sz * (r02 * r22)));
+  const float cyz = fmaf(sx, r10 * r20, fmaf(sy, r11 * r21, sz * (r12 * r22)));
+  const uint32_t hxy = bf16_nearest(cxy), hxz = bf16_nearest(cxz), hyz = bf16_nearest(cyz);
+  const float exy = fabsf(cxy - bits_to_float(hxy << 16)), exz = fabsf(cxz - bits_to_float(hxz << 16)),
+              eyz = fabsf(cyz - bits_to_float(hyz << 16));
+  const float slack = 1e-5f * ((cxx + cyy) + czz);
+  const uint32_t hxx = bf16_up((cxx + slack) + (exy + exz)), hyy = bf16_up((cyy + slack) + (exy + eyz)),
+                 hzz = bf16_up((czz + slack) + (exz + eyz));
+  float4* dst = reinterpret_cast<float4*>(out + 1 + p);
+  dst[0] = make_float4(P.qw, P.qx, P.qy, P.qz);
+  dst[1] = make_float4(P.mx, P.my, P.mz, vl.x);
+  dst[2] = make_float4(vl.y, vl.z, v.x, v.y);
+  dst[3] = make_float4(v.z, bits_to_float((hxx << 16) | (hyy & 0xffffu)), bits_to_float((hzz << 16) | (hxy & 0xffffu)),
+                       bits_to_float((hxz << 16) | (hyz & 0xffffu)));
+}
+
+// key_tstar() with vl taken from the frame record: the remaining statements, unchanged.
+__device__ __forceinline__ float key_tstar_hoisted(float dx, float dy, float dz, const SortRec& R) {
+  const Vec3 vl = {R.vlx, R.vly, R.vlz};
+  const Vec3 dl = quat_rotate_conj(R.qw, R.qx, R.qy, R.qz, Vec3{dx, dy, dz});
+  const float denom = fmaf(dl.x * dl.x, R.mx, fmaf(dl.y * dl.y, R.my, (dl.z * dl.z) * R.mz));
+  const float numer = fmaf(dl.x * vl.x, R.mx, fmaf(dl.y * vl.y, R.my, (dl.z * vl.z) * R.mz));
+  const float t = numer / denom;
+  return (denom > 1e-20f && t > 0.f) ? t : kInvalidKey;
+}
+// key_depth() with c - o taken from the frame record.
+__device__ __forceinline__ float key_depth_hoisted(float dx, float dy, float dz, const SortRec& R) {
+  const float k = fmaf(R.ex, dx, fmaf(R.ey, dy, R.ez * dz));
+  return (k > 0.f) ? k : kInvalidKey;
+}
+
+// The pyramid of a tile's rays: four planes through the common origin, each spanned by two neighbouring corner
+// rays and oriented towards the tile-centre ray.  Everything in it is the same for every lane (it is read out of
+// the lanes that computed it with v_readlane), so the per-candidate tests take it as scalar operands.
+struct TilePyramid {
+  float ox, oy, oz;        // the tile's common origin (corner 0's)
+  float n[4][3];           // inward normals
+  float q[4][6];           // nx^2, ny^2, nz^2, 2 nx ny, 2 nx nz, 2 ny nz of each
+  int faces;               // bit j: face j may be used (0: no culling for this tile)
+};
+__device__ __forceinline__ float lane_value(float v, int lane) {
+  return bits_to_float((uint32_t)__builtin_amdgcn_readlane((int)float_to_bits(v), lane));
+}
+// Called by a whole wavefront: lane l builds face l % 4 (face j from corner rays j and j + 1), then every lane
+// checks rays of the tile (all of them between the 64 lanes) against the four faces and the common origin.  A face
+// the centre ray (nearly) lies in, or that some ray of the tile is outside of, is not used; without a common origin
+// none is.  The roundings here are free: the per-candidate test has a 2 % margin.
+__device__ __forceinline__ TilePyramid tile_pyramid(const float* __restrict__ rays_o, const float* __restrict__ rays_d,
+                                                    const TileGeom& g, int tile, float dx, float dy, float dz) {
+  const int lane = threadIdx.x & 63;
+  const int tx = tile % g.ntx, ty = tile / g.ntx;
+  const int x0 = tx * g.TW, y0 = ty * g.TH;
+  const int x1 = min(x0 + g.TW, g.W) - 1, y1 = min(y0 + g.TH, g.H) - 1;
+  const int j = lane & 3, j1 = (lane + 1) & 3;
+  // corners in the order (x0,y0) (x1,y0) (x1,y1) (x0,y1)
+  const int ca = ((j >> 1) ? y1 : y0) * g.W + ((j == 1 || j == 2) ? x1 : x0);
+  const int cb = ((j1 >> 1) ? y1 : y0) * g.W + ((j1 == 1 || j1 == 2) ? x1 : x0);
+  const float a0 = rays_d[ca * 3], a1 = rays_d[ca * 3 + 1], a2 = rays_d[ca * 3 + 2];
+  const float b0 = rays_d[cb * 3], b1 = rays_d[cb * 3 + 1], b2 = rays_d[cb * 3 + 2];
+  const int c0 = y0 * g.W + x0;
+  TilePyramid py;
+  py.ox = rays_o[c0 * 3];
+  py.oy = rays_o[c0 * 3 + 1];
+  py.oz = rays_o[c0 * 3 + 2];
+  float nx = a1 * b2 - a2 * b1, ny = a2 * b0 - a0 * b2, nz = a0 * b1 - a1 * b0;
+  const float side = nx * dx + ny * dy + nz * dz;
+  const float len = __builtin_amdgcn_sqrtf(nx * nx + ny * ny + nz * nz);
+  const bool usable = len > 0.f && fabsf(side) > 1e-4f * len;
+  const float sgn = side < 0.f ? -1.f : 1.f;
+  nx *= sgn;
+  ny *= sgn;
+  nz *= sgn;
+  const float prod[6] = {nx * nx, ny * ny, nz * nz, 2.f * (nx * ny), 2.f * (nx * nz), 2.f * (ny * nz)};
+  float nlen[4];
+  int ok = 0x10;
+#pragma unroll
+  for (int f = 0; f < 4; ++f) {
+    py.n[f][0] = lane_value(nx, f);
+    py.n[f][1] = lane_value(ny, f);
+    py.n[f][2] = lane_value(nz, f);
+    nlen[f] = lane_value(len, f);
+#pragma unroll
+    for (int k = 0; k < 6; ++k) py.q[f][k] = lane_value(prod[k], f);
+    ok |= ((__ballot(usable) >> f) & 1ull) ? (1 << f) : 0;
+  }
+  for (int k = lane; k < g.TW * g.TH; k += 64) {
+    const int x = x0 + k % g.TW, y = y0 + k / g.TW;
+    if (x < g.W && y < g.H) {
+      const int pix = y * g.W + x;
+      if (rays_o[pix * 3] != py.ox || rays_o[pix * 3 + 1] != py.oy || rays_o[pix * 3 + 2] != py.oz) ok &= ~0x10;
+      const float rx = rays_d[pix * 3], ry = rays_d[pix * 3 + 1], rz = rays_d[pix * 3 + 2];
+#pragma unroll
+      for (int f = 0; f < 4; ++f) {
+        const float inside = py.n[f][0] * rx + py.n[f][1] * ry + py.n[f][2] * rz;
+        if (!(inside >= -1e-6f * nlen[f])) ok &= ~(1 << f);
+      }
+    }
+  }
+  int all_ok = 0;
+#pragma unroll
+  for (int b = 0; b < 5; ++b) all_ok |= __ballot(!((ok >> b) & 1)) ? 0 : (1 << b);
+  py.faces = (all_ok & 0x10) ? (all_ok & 0xf) : 0;
+  return py;
+}
+
+// Can no ray of the tile hit the primitive?  True if its threshold ellipsoid lies wholly beyond one usable face.
+// General form: the face normal is rotated into the primitive's axes (fused multiply-adds: roundings are free here).
+__device__ __forceinline__ bool outside_pyramid(const TilePyramid& py, const PrimRecord& P, float cull_r2) {
+  bool outside = false;
+  const float ex = P.cx - py.ox, ey = P.cy - py.oy, ez = P.cz - py.oz;
+  const float qw = P.qw, qx = -P.qx, qy = -P.qy, qz = -P.qz;       // conjugate: world -> local
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const float nx = py.n[j][0], ny = py.n[j][1], nz = py.n[j][2];
+    const float dist = fmaf(nx, ex, fmaf(ny, ey, nz * ez));
+    // R^T n = n + qw t + q x t with t = 2 q x n
+    const float tx = 2.f * fmaf(qy, nz, -(qz * ny)), ty = 2.f * fmaf(qz, nx, -(qx * nz)), tz = 2.f * fmaf(qx, ny, -(qy * nx));
+    const float lx = fmaf(qw, tx, nx) + fmaf(qy, tz, -(qz * ty));
+    const float ly = fmaf(qw, ty, ny) + fmaf(qz, tx, -(qx * tz));
+    const float lz = fmaf(qw, tz, nz) + fmaf(qx, ty, -(qy * tx));
+    const float h2 = fmaf(P.s2x, lx * lx, fmaf(P.s2y, ly * ly, P.s2z * (lz * lz)));
+    outside |= ((py.faces >> j) & 1) && (dist < 0.f) && (dist * dist >= cull_r2 * h2);
+  }
+  return outside;
+}
+// With a frame record: the support along n is the quadratic form of the (conservatively rounded) covariance.
+__device__ __forceinline__ bool outside_pyramid(const TilePyramid& py, const SortRec& R, float cull_r2) {
+  bool outside = false;
+  const float sxx = bits_to_float(R.s_xx_yy & 0xffff0000u), syy = bits_to_float(R.s_xx_yy << 16);
+  const float szz = bits_to_float(R.s_zz_xy & 0xffff0000u), sxy = bits_to_float(R.s_zz_xy << 16);
+  const float sxz = bits_to_float(R.s_xz_yz & 0xffff0000u), syz = bits_to_float(R.s_xz_yz << 16);
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const float dist = fmaf(py.n[j][0], R.ex, fmaf(py.n[j][1], R.ey, py.n[j][2] * R.ez));
+    const float h2 = fmaf(py.q[j][0], sxx, fmaf(py.q[j][1], syy, fmaf(py.q[j][2], szz,
+                     fmaf(py.q[j][3], sxy, fmaf(py.q[j][4], sxz, py.q[j][5] * syz)))));
+    outside |= ((py.faces >> j) & 1) && (dist < 0.f) && (dist * dist >= cull_r2 * h2);
+  }
+  return outside;
+}
+
+// The two sources of a candidate's geometry as one interface: keep-or-cull, and the key.
+struct FromPrimRecord {
+  typedef PrimRecord Rec;
+  const PrimRecord* __restrict__ base;
+  float ox, oy, oz;                         // origin of the tile-centre ray
+  __device__ __forceinline__ Rec load(int p) const {
+    // (only the first 64 bytes are used below: the compiler requests no more)
+    return base[p];
+  }
+  __device__ __forceinline__ float key(int family, float dx, float dy, float dz, const Rec& P) const {
+    return (family == MLPSP_KEY_DEPTH) ? key_depth(ox, oy, oz, dx, dy, dz, P) : key_tstar(ox, oy, oz, dx, dy, dz, P);
+  }
+};
+struct FromFrameRecord {
+  typedef SortRec Rec;
+  const SortRec* __restrict__ base;         // record of primitive 0
+  __device__ __forceinline__ Rec load(int p) const {
+    return base[p];
+  }
+  __device__ __forceinline__ float key(int family, float dx, float dy, float dz, const Rec& R) const {
+    return (family == MLPSP_KEY_DEPTH) ? key_depth_hoisted(dx, dy, dz, R) : key_tstar_hoisted(dx, dy, dz, R);
+  }
+};
+// Do the frame records (if any) hold for a tile whose centre ray starts at (ox, oy, oz)?
+__device__ __forceinline__ bool frame_records_hold(const SortRec* __restrict__ frame, float ox, float oy, float oz) {
+  if (!frame) return false;
+  const SortFrameHeader& h = *reinterpret_cast<const SortFrameHeader*>(frame);
+  return h.valid == 1 && h.ox == float_to_bits(ox) && h.oy == float_to_bits(oy) && h.oz == float_to_bits(oz);
+}
+
 // A tile whose list has at most 64 entries, sorted by ONE wavefront (lane = entry) in registers: no LDS, no barrier.
 // Same output as sort_one_tile() -- the kept entries ordered by their (key bits, list position) words, which also
 // puts keys at or above the invalid key last and in list order among equals; culled entries as ~id at the end of
 // the tile's output, last one first -- at a fifth of its instructions: for short lists sort_one_tile()'s cost is
-// what four wavefronts spend per tile whatever its length (the pyramid built four times, the passes of the bucket
-// ranking, a dozen barriers).  The pyramid and the per-candidate test are those of sort_one_tile(), statement for
-// statement.  Requires len <= 64 and len <= capacity; called by a whole wavefront.
-__device__ __forceinline__ void sort_small_tile(
-    const float* __restrict__ rays_o, const float* __restrict__ rays_d, const PrimRecord* __restrict__ prims,
-    const int32_t* __restrict__ cand, const TileGeom& g, int family, float cull_r2, int num_prims,
-    int32_t* __restrict__ sorted_ids, float* __restrict__ sorted_keys, int tile, int start, int n) {
+// what four wavefronts spend per tile whatever its length (the passes of the bucket ranking, a dozen barriers).
+// Requires len <= 64 and len <= capacity; called by a whole wavefront.
+template <typename Source>
+__device__ __forceinline__ void sort_small_tile_from(
+    const Source& src, const float* __restrict__ rays_o, const float* __restrict__ rays_d, const TileGeom& g, int tile,
+    float dx, float dy, float dz, const int32_t* __restrict__ cand, int family, float cull_r2, int num_prims,
+    int32_t* __restrict__ sorted_ids, float* __restrict__ sorted_keys, int start, int n) {
   const int lane = threadIdx.x & 63;
-  const int pc = centre_pixel(g, tile);
-  const float ox = rays_o[pc * 3 + 0], oy = rays_o[pc * 3 + 1], oz = rays_o[pc * 3 + 2];
-  const float dx = rays_d[pc * 3 + 0], dy = rays_d[pc * 3 + 1], dz = rays_d[pc * 3 + 2];
   const int p = (lane < n) ? cand[start + lane] : 0;
   const bool known = (unsigned)p < (unsigned)num_prims;
-  const PrimRecord P = prims[known ? p : 0];
-
-  float pox = 0.f, poy = 0.f, poz = 0.f;
-  float pn[4][3] = {};
-  int faces = 0;
-  if (cull_r2 > 0.f) {
-    const int tx = tile % g.ntx, ty = tile / g.ntx;
-    const int x0 = tx * g.TW, y0 = ty * g.TH;
-    const int x1 = min(x0 + g.TW, g.W) - 1, y1 = min(y0 + g.TH, g.H) - 1;
-    const int corner[4] = {y0 * g.W + x0, y0 * g.W + x1, y1 * g.W + x1, y1 * g.W + x0};
-    float cd[4][3];
-#pragma unroll
-    for (int j = 0; j < 4; ++j)
-#pragma unroll
-      for (int c = 0; c < 3; ++c) cd[j][c] = rays_d[corner[j] * 3 + c];
-    pox = rays_o[corner[0] * 3 + 0];
-    poy = rays_o[corner[0] * 3 + 1];
-    poz = rays_o[corner[0] * 3 + 2];
-    int ok = 0x1f;                                       // bits 0..3: face usable; bit 4: common origin
-    float nlen[4];
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {                        // face j from corner rays j and j+1
-      const float* a = cd[j];
-      const float* b = cd[(j + 1) & 3];
-      const float nx = a[1] * b[2] - a[2] * b[1], ny = a[2] * b[0] - a[0] * b[2], nz = a[0] * b[1] - a[1] * b[0];
-      const float side = nx * dx + ny * dy + nz * dz;
-      const float len = sqrtf(nx * nx + ny * ny + nz * nz);
-      const float sgn = side < 0.f ? -1.f : 1.f;
-      pn[j][0] = sgn * nx;
-      pn[j][1] = sgn * ny;
-      pn[j][2] = sgn * nz;
-      nlen[j] = sqrtf(pn[j][0] * pn[j][0] + pn[j][1] * pn[j][1] + pn[j][2] * pn[j][2]);
-      if (!(len > 0.f && fabsf(side) > 1e-4f * len)) ok &= ~(1 << j);
-    }
-    for (int k = lane; k < g.TW * g.TH; k += 64) {
-      const int x = x0 + k % g.TW, y = y0 + k / g.TW;
-      if (x < g.W && y < g.H) {
-        const int pix = y * g.W + x;
-        if (rays_o[pix * 3] != pox || rays_o[pix * 3 + 1] != poy || rays_o[pix * 3 + 2] != poz) ok &= ~0x10;
-        const float rx = rays_d[pix * 3], ry = rays_d[pix * 3 + 1], rz = rays_d[pix * 3 + 2];
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const float inside = pn[j][0] * rx + pn[j][1] * ry + pn[j][2] * rz;
-          if (!(inside >= -1e-6f * nlen[j])) ok &= ~(1 << j);
-        }
-      }
-    }
-    int all_ok = 0;
-#pragma unroll
-    for (int b = 0; b < 5; ++b) all_ok |= __ballot(!((ok >> b) & 1)) ? 0 : (1 << b);
-    faces = (all_ok & 0x10) ? (all_ok & 0xf) : 0;
-  }
-
+  const typename Source::Rec P = src.load(known ? p : 0);
+  TilePyramid py = {};
+  if (cull_r2 > 0.f) py = tile_pyramid(rays_o, rays_d, g, tile, dx, dy, dz);
   bool keep = false;
   float key = 0.f;
   if (lane < n) {
-    bool outside = false;
-    if (faces && known) {
-      const float ex = P.cx - pox, ey = P.cy - poy, ez = P.cz - poz;
-      const float qw = P.qw, qx = -P.qx, qy = -P.qy, qz = -P.qz;       // conjugate: world -> local
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const float nx = pn[j][0], ny = pn[j][1], nz = pn[j][2];
-        const float dist = fmaf(nx, ex, fmaf(ny, ey, nz * ez));
-        const float tx = 2.f * fmaf(qy, nz, -(qz * ny)), ty = 2.f * fmaf(qz, nx, -(qx * nz)),
-                    tz = 2.f * fmaf(qx, ny, -(qy * nx));
-        const float lx = fmaf(qw, tx, nx) + fmaf(qy, tz, -(qz * ty));
-        const float ly = fmaf(qw, ty, ny) + fmaf(qz, tx, -(qx * tz));
-        const float lz = fmaf(qw, tz, nz) + fmaf(qx, ty, -(qy * tx));
-        const float h2 = fmaf(P.s2x, lx * lx, fmaf(P.s2y, ly * ly, P.s2z * (lz * lz)));
-        outside |= ((faces >> j) & 1) && (dist < 0.f) && (dist * dist >= cull_r2 * h2);
-      }
-    }
-    keep = !outside;
-    if (keep)
-      key = !known ? kInvalidKey
-                   : (family == MLPSP_KEY_DEPTH) ? key_depth(ox, oy, oz, dx, dy, dz, P) : key_tstar(ox, oy, oz, dx, dy, dz, P);
+    keep = !(py.faces && known && outside_pyramid(py, P, cull_r2));
+    if (keep) key = !known ? kInvalidKey : src.key(family, dx, dy, dz, P);
   }
   const uint32_t kb = float_to_bits(key);
   const unsigned long long kept = __ballot(keep);
@@ -157,18 +327,31 @@ __device__ __forceinline__ void sort_small_tile(
     if (sorted_keys) sorted_keys[pos] = kInvalidKey;
   }
 }
+__device__ __forceinline__ void sort_small_tile(
+    const float* __restrict__ rays_o, const float* __restrict__ rays_d, const PrimRecord* __restrict__ prims,
+    const SortRec* __restrict__ frame, const int32_t* __restrict__ cand, const TileGeom& g, int family, float cull_r2,
+    int num_prims, int32_t* __restrict__ sorted_ids, float* __restrict__ sorted_keys, int tile, int start, int n) {
+  const int pc = centre_pixel(g, tile);
+  const float ox = rays_o[pc * 3 + 0], oy = rays_o[pc * 3 + 1], oz = rays_o[pc * 3 + 2];
+  const float dx = rays_d[pc * 3 + 0], dy = rays_d[pc * 3 + 1], dz = rays_d[pc * 3 + 2];
+  if (frame_records_hold(frame, ox, oy, oz))
+    sort_small_tile_from(FromFrameRecord{frame + 1}, rays_o, rays_d, g, tile, dx, dy, dz, cand, family, cull_r2,
+                         num_prims, sorted_ids, sorted_keys, start, n);
+  else
+    sort_small_tile_from(FromPrimRecord{prims, ox, oy, oz}, rays_o, rays_d, g, tile, dx, dy, dz, cand, family, cull_r2,
+                         num_prims, sorted_ids, sorted_keys, start, n);
+}
 
 // Sorts one tile with the calling 256-thread workgroup (every thread must call it; `tile` is uniform).  kSortMax
 // bounds `capacity`.  A workgroup that sorts several tiles in a row, or uses `lds` for something else afterwards,
 // puts a barrier in between.
-template <int kSortMax>
-__device__ __forceinline__ void sort_one_tile(SortLds<kSortMax>& lds,
-    const float* __restrict__ rays_o, const float* __restrict__ rays_d, const PrimRecord* __restrict__ prims,
-    const int32_t* __restrict__ cand, const int32_t* __restrict__ offsets, const TileGeom& g, int family, int capacity,
-    float cull_r2, int num_prims, int32_t* __restrict__ sorted_ids, float* __restrict__ sorted_keys, int tile) {
+template <int kSortMax, typename Source>
+__device__ __forceinline__ void sort_one_tile_from(SortLds<kSortMax>& lds, const Source& src,
+    const float* __restrict__ rays_o, const float* __restrict__ rays_d, const TileGeom& g, int tile,
+    float dx, float dy, float dz, const int32_t* __restrict__ cand, int family, float cull_r2, int num_prims,
+    int32_t* __restrict__ sorted_ids, float* __restrict__ sorted_keys, int start, int len, int n) {
   auto& s_key = lds.key;
   auto& s_wave_cnt = lds.wave_cnt;
-  auto& s_wave_ok = lds.wave_ok;
   auto& s_cnt = lds.cnt;
   auto& s_off = lds.off;
   auto& s_perm = lds.perm;
@@ -178,89 +361,25 @@ __device__ __forceinline__ void sort_one_tile(SortLds<kSortMax>& lds,
   auto& s_flags = lds.flags;
   auto& s_pairs = lds.pairs;
   const int tid = threadIdx.x;
-  const int start = offsets[tile];
-  const int len = offsets[tile + 1] - start;
-  if (len <= 0) return;
-  const int n = len < capacity ? len : capacity;
-
-  const int pc = centre_pixel(g, tile);
-  const float ox = rays_o[pc * 3 + 0], oy = rays_o[pc * 3 + 1], oz = rays_o[pc * 3 + 2];
-  const float dx = rays_d[pc * 3 + 0], dy = rays_d[pc * 3 + 1], dz = rays_d[pc * 3 + 2];
+  const int wave = tid >> 6, lane = tid & 63;
 
   // Every candidate id this thread will handle is requested up front (at most kSortMax / kSortThreads of them),
-  // and the first round's geometry record right behind: their latencies overlap the pyramid phase below, and each
-  // round of the key loop then requests the next round's record.
-  // An id outside [0, num_prims) (lists that were never validated) reads record 0, is never culled and sorts last
-  // with the invalid key; it is passed on unchanged, and the render kernels skip it.
+  // and the first round's geometry record right behind; each round of the key loop then requests the next round's
+  // record.  An id outside [0, num_prims) (lists that were never validated) reads record 0, is never culled and
+  // sorts last with the invalid key; it is passed on unchanged, and the render kernels skip it.
   constexpr int kRounds = kSortMax / kSortThreads;
   int my_id[kRounds];
 #pragma unroll
   for (int r = 0; r < kRounds; ++r) my_id[r] = (tid + r * kSortThreads < n) ? cand[start + tid + r * kSortThreads] : 0;
-  PrimRecord P_buf[2];                                   // this round's record and the next round's
-  P_buf[0] = prims[((unsigned)my_id[0] < (unsigned)num_prims) ? my_id[0] : 0];
+  typename Source::Rec P_buf[2];                         // this round's record and the next round's
+  P_buf[0] = src.load(((unsigned)my_id[0] < (unsigned)num_prims) ? my_id[0] : 0);
 
-  // ---- the tile's ray pyramid (only when culling is requested).  Every thread builds the four faces from the
-  //      corner rays for itself (uniform addresses: one broadcast load each), threads then check the tile's rays
-  //      against them, and one barrier combines the verdicts.
-  const bool culling = cull_r2 > 0.f;
-  const int wave = tid >> 6, lane = tid & 63;
-  float pox = 0.f, poy = 0.f, poz = 0.f;
-  float pn[4][3] = {};
-  int faces = 0;
-  if (culling) {
-    const int tx = tile % g.ntx, ty = tile / g.ntx;
-    const int x0 = tx * g.TW, y0 = ty * g.TH;
-    const int x1 = min(x0 + g.TW, g.W) - 1, y1 = min(y0 + g.TH, g.H) - 1;
-    const int corner[4] = {y0 * g.W + x0, y0 * g.W + x1, y1 * g.W + x1, y1 * g.W + x0};
-    float cd[4][3];
-#pragma unroll
-    for (int j = 0; j < 4; ++j)
-#pragma unroll
-      for (int c = 0; c < 3; ++c) cd[j][c] = rays_d[corner[j] * 3 + c];
-    pox = rays_o[corner[0] * 3 + 0];
-    poy = rays_o[corner[0] * 3 + 1];
-    poz = rays_o[corner[0] * 3 + 2];
-    int ok = 0x1f;                                       // bits 0..3: face usable; bit 4: common origin
-    float nlen[4];
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {                        // face j from corner rays j and j+1
-      const float* a = cd[j];
-      const float* b = cd[(j + 1) & 3];
-      const float nx = a[1] * b[2] - a[2] * b[1], ny = a[2] * b[0] - a[0] * b[2], nz = a[0] * b[1] - a[1] * b[0];
-      // orient towards the tile-centre ray; a face the centre ray (nearly) lies in is not used
-      const float side = nx * dx + ny * dy + nz * dz;
-      const float len = sqrtf(nx * nx + ny * ny + nz * nz);
-      const float sgn = side < 0.f ? -1.f : 1.f;
-      pn[j][0] = sgn * nx;
-      pn[j][1] = sgn * ny;
-      pn[j][2] = sgn * nz;
-      nlen[j] = sqrtf(pn[j][0] * pn[j][0] + pn[j][1] * pn[j][1] + pn[j][2] * pn[j][2]);
-      if (!(len > 0.f && fabsf(side) > 1e-4f * len)) ok &= ~(1 << j);
-    }
-    // every ray of the tile must start at the common origin and lie inside every face used
-    for (int k = tid; k < g.TW * g.TH; k += kSortThreads) {
-      const int x = x0 + k % g.TW, y = y0 + k / g.TW;
-      if (x < g.W && y < g.H) {
-        const int pix = y * g.W + x;
-        if (rays_o[pix * 3] != pox || rays_o[pix * 3 + 1] != poy || rays_o[pix * 3 + 2] != poz) ok &= ~0x10;
-        const float rx = rays_d[pix * 3], ry = rays_d[pix * 3 + 1], rz = rays_d[pix * 3 + 2];
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const float inside = pn[j][0] * rx + pn[j][1] * ry + pn[j][2] * rz;
-          if (!(inside >= -1e-6f * nlen[j])) ok &= ~(1 << j);
-        }
-      }
-    }
-    int wave_ok = 0;
-#pragma unroll
-    for (int b = 0; b < 5; ++b) wave_ok |= __ballot(!((ok >> b) & 1)) ? 0 : (1 << b);
-    if (lane == 0) s_wave_ok[wave] = wave_ok;
-    __syncthreads();
-    ok = s_wave_ok[0];
-#pragma unroll
-    for (int v = 1; v < kSortThreads / 64; ++v) ok &= s_wave_ok[v];
-    faces = (ok & 0x10) ? (ok & 0xf) : 0;
-  }
+  // ---- the tile's ray pyramid (only when culling is requested), while those loads are on their way: every
+  //      wavefront builds it for itself -- four faces among its lanes, one ray of the tile per lane -- so no barrier
+  //      is needed for the verdict
+  TilePyramid py = {};
+  if (cull_r2 > 0.f) py = tile_pyramid(rays_o, rays_d, g, tile, dx, dy, dz);
+  const int faces = py.faces;
 
   // ---- keys.  Survivors with an ordinary key are compacted to the front of s_key in list order; survivors
   //      whose key is the invalid key or larger go to the back of s_key, last slot first (the "late" stream: all
@@ -283,34 +402,15 @@ __device__ __forceinline__ void sort_one_tile(SortLds<kSortMax>& lds,
     const int i = r * kSortThreads + tid;
     bool keep = false, outside = false;
     float key = 0.f;
-    const PrimRecord& P = P_buf[r & 1];
+    const typename Source::Rec& P = P_buf[r & 1];
     const int p = my_id[r];
     if (r + 1 < kRounds && i + kSortThreads < n)
-      P_buf[(r + 1) & 1] = prims[((unsigned)my_id[r + 1] < (unsigned)num_prims) ? my_id[r + 1] : 0];
+      P_buf[(r + 1) & 1] = src.load(((unsigned)my_id[r + 1] < (unsigned)num_prims) ? my_id[r + 1] : 0);
     const bool known = (unsigned)p < (unsigned)num_prims;
     if (i < n) {
-      if (faces && known) {
-        // (fused multiply-adds here: the test is conservative by a 2 % margin, its roundings are free)
-        const float ex = P.cx - pox, ey = P.cy - poy, ez = P.cz - poz;
-        const float qw = P.qw, qx = -P.qx, qy = -P.qy, qz = -P.qz;       // conjugate: world -> local
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const float nx = pn[j][0], ny = pn[j][1], nz = pn[j][2];
-          const float dist = fmaf(nx, ex, fmaf(ny, ey, nz * ez));
-          // R^T n = n + qw t + q x t with t = 2 q x n
-          const float tx = 2.f * fmaf(qy, nz, -(qz * ny)), ty = 2.f * fmaf(qz, nx, -(qx * nz)),
-                      tz = 2.f * fmaf(qx, ny, -(qy * nx));
-          const float lx = fmaf(qw, tx, nx) + fmaf(qy, tz, -(qz * ty));
-          const float ly = fmaf(qw, ty, ny) + fmaf(qz, tx, -(qx * tz));
-          const float lz = fmaf(qw, tz, nz) + fmaf(qx, ty, -(qy * tx));
-          const float h2 = fmaf(P.s2x, lx * lx, fmaf(P.s2y, ly * ly, P.s2z * (lz * lz)));
-          outside |= ((faces >> j) & 1) && (dist < 0.f) && (dist * dist >= cull_r2 * h2);
-        }
-      }
+      outside = faces && known && outside_pyramid(py, P, cull_r2);
       keep = !outside;
-      if (keep)
-        key = !known ? kInvalidKey
-                     : (family == MLPSP_KEY_DEPTH) ? key_depth(ox, oy, oz, dx, dy, dz, P) : key_tstar(ox, oy, oz, dx, dy, dz, P);
+      if (keep) key = !known ? kInvalidKey : src.key(family, dx, dy, dz, P);
     }
     const uint32_t kb = float_to_bits(key);
     const bool late = keep && kb >= invalid_bits;
@@ -476,6 +576,27 @@ __device__ __forceinline__ void sort_one_tile(SortLds<kSortMax>& lds,
       if (sorted_keys) sorted_keys[start + i] = kInvalidKey;
     }
   }
+}
+
+template <int kSortMax>
+__device__ __forceinline__ void sort_one_tile(SortLds<kSortMax>& lds,
+    const float* __restrict__ rays_o, const float* __restrict__ rays_d, const PrimRecord* __restrict__ prims,
+    const SortRec* __restrict__ frame, const int32_t* __restrict__ cand, const int32_t* __restrict__ offsets,
+    const TileGeom& g, int family, int capacity, float cull_r2, int num_prims, int32_t* __restrict__ sorted_ids,
+    float* __restrict__ sorted_keys, int tile) {
+  const int start = offsets[tile];
+  const int len = offsets[tile + 1] - start;
+  if (len <= 0) return;
+  const int n = len < capacity ? len : capacity;
+  const int pc = centre_pixel(g, tile);
+  const float ox = rays_o[pc * 3 + 0], oy = rays_o[pc * 3 + 1], oz = rays_o[pc * 3 + 2];
+  const float dx = rays_d[pc * 3 + 0], dy = rays_d[pc * 3 + 1], dz = rays_d[pc * 3 + 2];
+  if (frame_records_hold(frame, ox, oy, oz))
+    sort_one_tile_from<kSortMax>(lds, FromFrameRecord{frame + 1}, rays_o, rays_d, g, tile, dx, dy, dz, cand, family,
+                                 cull_r2, num_prims, sorted_ids, sorted_keys, start, len, n);
+  else
+    sort_one_tile_from<kSortMax>(lds, FromPrimRecord{prims, ox, oy, oz}, rays_o, rays_d, g, tile, dx, dy, dz, cand, family,
+                                 cull_r2, num_prims, sorted_ids, sorted_keys, start, len, n);
 }
 
 }  // namespace mlpsp

@@ -7,6 +7,7 @@ from __future__ import annotations
 
 import ctypes as C
 import math
+import os
 
 import torch
 
@@ -211,21 +212,26 @@ def bin_legacy_async(positions, log_scales, view_matrices, proj_matrix, W: int, 
 
 
 def sort_tiles(rays_o, rays_d, records, candidates, tile_offsets, W, H, TW, TH, family=_lib.KEY_TSTAR,
-               capacity=TILE_CAPACITY_DEFAULT, want_keys=False, cull_threshold=0.0):
+               capacity=TILE_CAPACITY_DEFAULT, want_keys=False, cull_threshold=0.0, frame_records=True):
     """Materialised per-tile depth order: (sorted_ids [P], sorted_keys [P] | None).
 
     With ``cull_threshold`` (the render's score threshold) candidates that provably hit no ray of their
-    tile come back as ``~id``; the render kernels skip them, the image is unchanged."""
+    tile come back as ``~id``; the render kernels skip them, the image is unchanged.  ``frame_records``: let the
+    library write per-frame records for the common ray origin first (keys and order do not depend on it; False keeps
+    the full key evaluation per candidate, for comparing the two)."""
     dev = rays_o.device
     sorted_ids = torch.empty_like(candidates)
     keys = torch.empty(candidates.numel(), dtype=torch.float32, device=dev) if want_keys else None
     if candidates.numel() == 0:
         return sorted_ids, keys
     num_primitives = records.numel() // _lib.PRIM_RECORD_BYTES
-    code = _lib.load().mlpsp_sort_tiles(_ptr(rays_o), _ptr(rays_d), _ptr(records), num_primitives, _ptr(candidates),
-                                        _ptr(tile_offsets),
-                                        W, H, TW, TH, int(family), int(capacity), float(cull_threshold),
-                                        _ptr(sorted_ids), _ptr(keys), _stream(dev))
+    lib = _lib.load()
+    scratch = None
+    if frame_records and os.environ.get("MLPSP_SORT_FRAME_RECORDS", "1") != "0":
+        scratch = torch.empty(lib.mlpsp_sort_frame_records_bytes(num_primitives), dtype=torch.uint8, device=dev)
+    code = lib.mlpsp_sort_tiles(_ptr(rays_o), _ptr(rays_d), _ptr(records), num_primitives, _ptr(candidates),
+                                _ptr(tile_offsets), W, H, TW, TH, int(family), int(capacity), float(cull_threshold),
+                                _ptr(scratch), _ptr(sorted_ids), _ptr(keys), _stream(dev))
     _check(code, "mlpsp_sort_tiles")
     return sorted_ids, keys
 
@@ -542,12 +548,16 @@ def pack_mfma_feat(feat_attr):
 
 def render_tilecenter_mfma_feat(rays_o, rays_d, records, order, tile_offsets, freq, att, W1, b1, W2, b2, W3, b3,
                                 feat_attr, beta, temp, W, H, threshold, bf16=True, packed=None, packed_feat=None,
-                                check=True, status=None):
+                                check=True, status=None, counters=None, stages=None):
     """Matrix-core tile-centre forward with the gated feature channel -> (rgb, alpha, feat, nonfinite).
     ``packed_feat`` is the result of :func:`pack_mfma_feat` for ``feat_attr`` (built here when omitted;
     non-finite rounded attributes raise).  ``status`` (an int32 [16] device tensor): ONE attempt with the first
     record-pool size and no read-back -- word 0 = non-finite, word 1 = the pool ran out (the feature image is then
-    incomplete and the caller repeats the call without ``status``); returns (rgb, alpha, feat, status)."""
+    incomplete and the caller repeats the call without ``status``); returns (rgb, alpha, feat, status).
+    ``counters``: int64 [4] work counters of the render launch, accumulated.  ``stages``: a callable
+    ``stages(which)`` invoked before the render launch (1), before the feature product (2) and after it (3) -- the
+    two launches are then queued by separate calls, with the worst-case record pool, so that a caller can bracket
+    each with events."""
     dev = rays_o.device
     if freq.numel() != 6:
         raise RuntimeError("the matrix-core path supports 6 frequencies only")
@@ -568,15 +578,28 @@ def render_tilecenter_mfma_feat(rays_o, rays_d, records, order, tile_offsets, fr
                                    and status.is_contiguous()):
         raise ValueError("status must be a contiguous int32 [16] tensor on the device")
     flag = status if status is not None else torch.empty(16, dtype=torch.int32, device=dev)
-    for pool in _feat_pool_sizes(pairs):
-        ws_bytes = lib.mlpsp_feat_workspace_bytes(pairs, W, H, 8, 8, slots, 1, pool)
-        workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    def launch(workspace, ws_bytes, stage):
         code = lib.mlpsp_render_tilecenter_mfma_feat(
             _ptr(rays_o), _ptr(rays_d), _ptr(records), _ptr(order), _ptr(tile_offsets), pairs, _ptr(freq), _ptr(att),
             _ptr(packed), W1.shape[0], int(bool(bf16)), _ptr(packed_feat), slots, ch, float(beta), float(temp), W, H,
-            float(threshold), _ptr(workspace), ws_bytes, _ptr(rgb), _ptr(alpha), _ptr(feat), _ptr(flag), None,
-            _stream(dev))
+            float(threshold), _ptr(workspace), ws_bytes, _ptr(rgb), _ptr(alpha), _ptr(feat), _ptr(flag), _ptr(counters),
+            stage, _stream(dev))
         _check(code, "mlpsp_render_tilecenter_mfma_feat")
+        return code
+
+    if stages is not None:
+        ws_bytes = lib.mlpsp_feat_workspace_bytes(pairs, W, H, 8, 8, slots, 1, -1)
+        workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+        stages(1)
+        launch(workspace, ws_bytes, 1)
+        stages(2)
+        launch(workspace, ws_bytes, 2)
+        stages(3)
+        return rgb, alpha, feat, (bool(flag[0].item()) if check else flag)
+    for pool in _feat_pool_sizes(pairs):
+        ws_bytes = lib.mlpsp_feat_workspace_bytes(pairs, W, H, 8, 8, slots, 1, pool)
+        workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+        code = launch(workspace, ws_bytes, 0)
         if status is not None:
             return rgb, alpha, feat, status
         if pool < 0:

@@ -153,15 +153,18 @@ def test_unit_directions_are_the_bits_of_torch_normalize(device, rays, scale):
     assert torch.equal(ops.normalize_rays(sliced), torch.nn.functional.normalize(sliced, dim=-1))
 
 
+@pytest.mark.parametrize("frame_records", [True, False], ids=["frame_records", "full_key"])
 @pytest.mark.parametrize("family", [1, 2])
-def test_sorted_tile_lists_match_oracle_keys_and_order(device, oracle_mod, frame1, family):
+def test_sorted_tile_lists_match_oracle_keys_and_order(device, oracle_mod, frame1, family, frame_records):
+    # frame_records: the rotated offset centre - origin of the key comes from per-frame records (one per primitive,
+    # written for the common ray origin) instead of being evaluated per candidate; the key bits must not depend on it
     from mlp_splatting_amd import ops
     fr = frame1
     sc = fr.scene
     cand, off = fr.lists
     rec = ops.prepare_primitives(_t(sc.positions, device), _t(sc.log_scales, device), _t(sc.quats, device))
     ids, keys = ops.sort_tiles(_t(fr.rays_o, device), _t(fr.rays_d, device), rec, _t(cand, device), _t(off, device),
-                               fr.W, fr.H, 8, 8, family=family, want_keys=True)
+                               fr.W, fr.H, 8, 8, family=family, want_keys=True, frame_records=frame_records)
     want_ids, want_keys = oracle_mod.sort_tiles(fr.rays_o, fr.rays_d, sc.positions, sc.log_scales, sc.quats, cand, off,
                                                 fr.W, fr.H, 8, 8, family=family)
     np.testing.assert_array_equal(ids.cpu().numpy(), want_ids)
@@ -170,8 +173,9 @@ def test_sorted_tile_lists_match_oracle_keys_and_order(device, oracle_mod, frame
 
 @pytest.mark.parametrize("case", ["spread", "ties", "behind", "clusters", "beyond_invalid", "two", "capacity",
                                   "ties:64", "behind:64", "beyond_invalid:63", "spread:65", "clusters:1"])
+@pytest.mark.parametrize("frame_records", [True, False], ids=["frame_records", "full_key"])
 @pytest.mark.parametrize("family", [1, 2])
-def test_sort_is_the_stable_key_order_for_every_key_distribution(device, oracle_mod, case, family):
+def test_sort_is_the_stable_key_order_for_every_key_distribution(device, oracle_mod, case, family, frame_records):
     """One 8x8 tile with a hand-made list.  The kernel ranks survivors inside 256 key buckets and falls back to a
     sorting network when keys pile up in few buckets or a key exceeds the invalid key; each case below steers it
     down one of those routes, and the result must be the oracle's stable sort by key every time.  A list of at most
@@ -209,7 +213,7 @@ def test_sort_is_the_stable_key_order_for_every_key_distribution(device, oracle_
     off = np.array([0, n], np.int32)
     rec = ops.prepare_primitives(_t(pos, device), _t(log_s, device), _t(quat, device))
     ids, keys = ops.sort_tiles(_t(fr.rays_o, device), _t(fr.rays_d, device), rec, _t(cand, device), _t(off, device),
-                               8, 8, 8, 8, family=family, want_keys=True)
+                               8, 8, 8, 8, family=family, want_keys=True, frame_records=frame_records)
     want_ids, want_keys = oracle_mod.sort_tiles(fr.rays_o, fr.rays_d, pos, log_s, quat, cand, off, 8, 8, 8, 8, family=family)
     if case == "beyond_invalid":
         assert (want_keys > 1e30).any() and (want_keys == np.float32(1e30)).any()
@@ -222,7 +226,8 @@ def test_sort_is_the_stable_key_order_for_every_key_distribution(device, oracle_
 @pytest.mark.parametrize("name,n,width,height,tile,eye", [
     ("cfg1_5k_160x120", None, 160, 120, 8, (0.3, -0.2, -0.5)), ("cfg1_5k_160x120", 4000, 100, 76, 16, (1.0, 0.8, -1.2)),
     ("cfg2_50k_640x480", 20000, 200, 136, 8, (-0.7, 0.4, 0.9)), ("cfg1_5k_160x120", 1500, 21, 13, 8, (0.1, 0.1, -0.2))])
-def test_conservative_tile_culling_never_drops_a_hit(device, oracle_mod, name, n, width, height, tile, eye):
+@pytest.mark.parametrize("frame_records", [True, False], ids=["frame_records", "full_key"])
+def test_conservative_tile_culling_never_drops_a_hit(device, oracle_mod, name, n, width, height, tile, eye, frame_records):
     # per tile: the survivors, in front, are the plain sorted list with the culled ids struck out; the
     # culled ones follow as ~id in reverse list (descending id) order; (2) it is a real saving, and (3) no bit
     # of the image changes: the oracle, which tests every candidate, is the witness
@@ -232,8 +237,10 @@ def test_conservative_tile_culling_never_drops_a_hit(device, oracle_mod, name, n
     cand, off = fr.oracle_lists(oracle_mod)
     rec = ops.prepare_primitives(_t(sc.positions, device), _t(sc.log_scales, device), _t(sc.quats, device))
     ro, rd, c, o = _t(fr.rays_o, device), _t(fr.rays_d, device), _t(cand, device), _t(off, device)
-    plain, _ = ops.sort_tiles(ro, rd, rec, c, o, fr.W, fr.H, tile, tile)
-    culled, _ = ops.sort_tiles(ro, rd, rec, c, o, fr.W, fr.H, tile, tile, cull_threshold=fr.thr)
+    # (with frame records the ellipsoid's support along a face normal comes from a stored covariance, rounded up;
+    # without, from the face normal rotated into the primitive's axes: two forms of the same conservative test)
+    plain, _ = ops.sort_tiles(ro, rd, rec, c, o, fr.W, fr.H, tile, tile, frame_records=frame_records)
+    culled, _ = ops.sort_tiles(ro, rd, rec, c, o, fr.W, fr.H, tile, tile, cull_threshold=fr.thr, frame_records=frame_records)
     plain, culled = plain.cpu().numpy(), culled.cpu().numpy()
     for t in range(off.size - 1):
         a, b = plain[off[t]:off[t + 1]], culled[off[t]:off[t + 1]]
@@ -243,6 +250,9 @@ def test_conservative_tile_culling_never_drops_a_hit(device, oracle_mod, name, n
         assert np.array_equal(b[:k], a[~np.isin(a, gone)])
     frac = (culled < 0).mean()
     assert frac > 0.15, frac
+    if frame_records:      # the stored covariance costs next to nothing in culled candidates
+        other, _ = ops.sort_tiles(ro, rd, rec, c, o, fr.W, fr.H, tile, tile, cull_threshold=fr.thr, frame_records=False)
+        assert frac > 0.97 * float((other < 0).float().mean()), (frac, float((other < 0).float().mean()))
     want = oracle_mod.render_tilecenter(*fr.base_numpy(cand, off), *fr.dims)
     rgb, alpha, _ = ops.render_tilecenter_f32(ro, rd, rec, _t(culled, device), o, _t(sc.freq, device), _t(sc.att, device),
                                               *[_t(w, device) for w in sc.mlp()], fr.W, fr.H, tile, tile, fr.thr)
@@ -279,6 +289,61 @@ def test_culling_is_off_for_tiles_with_mixed_origins_or_degenerate_pyramids(devi
     ids1, _ = ops.sort_tiles(_t(fr1.rays_o, device), _t(fr1.rays_d, device), rec1, _t(c1, device), _t(o1, device), 12, 6, 1, 1,
                              cull_threshold=fr1.thr)
     assert int((ids1 < 0).sum()) == 0
+
+
+@pytest.mark.parametrize("family", [1, 2])
+def test_frame_records_serve_only_tiles_that_share_their_origin(device, oracle_mod, family):
+    """The per-frame records are written for the origin of ray 0.  A tile whose centre ray starts elsewhere must
+    evaluate its keys in full: with every seventh pixel's origin moved, both kinds of tile occur, and all keys are
+    still the oracle's bits.  Flat and needle-shaped primitives, far from and near the origin, stay sorted and are
+    culled conservatively with the stored covariance."""
+    from mlp_splatting_amd import ops
+    fr = Frame("cfg1_5k_160x120", n=1500, width=48, height=32)
+    sc = fr.scene
+    cand, off = fr.oracle_lists(oracle_mod)
+    rec = ops.prepare_primitives(_t(sc.positions, device), _t(sc.log_scales, device), _t(sc.quats, device))
+    ro = fr.rays_o.copy()
+    ro[3::7, 1] -= 2e-3
+    ids, keys = ops.sort_tiles(_t(ro, device), _t(fr.rays_d, device), rec, _t(cand, device), _t(off, device), fr.W, fr.H,
+                               8, 8, family=family, want_keys=True, cull_threshold=fr.thr)
+    want_ids, want_keys = oracle_mod.sort_tiles(ro, fr.rays_d, sc.positions, sc.log_scales, sc.quats, cand, off, fr.W,
+                                                fr.H, 8, 8, family=family)
+    centre_moved = [(min(ty * 8 + 4, fr.H - 1) * fr.W + min(tx * 8 + 4, fr.W - 1)) % 7 == 3
+                    for ty in range(fr.H // 8) for tx in range(fr.W // 8)]
+    assert any(centre_moved) and not all(centre_moved)
+    assert int((ids < 0).sum()) == 0                      # mixed origins inside every tile: no pyramid, nothing culled
+    np.testing.assert_array_equal(ids.cpu().numpy(), want_ids)
+    _assert_bits(keys, want_keys, "sort keys with mixed origins")
+
+    # extreme shapes: axis ratios up to e^8, with and without the records
+    rng = np.random.default_rng(5)
+    log_s = sc.log_scales.copy()
+    log_s[::3, 0] -= 6.0
+    log_s[1::3, 1:] -= 5.0
+    log_s[2::9] += 2.0
+    log_s = log_s.astype(np.float32)
+    rec2 = ops.prepare_primitives(_t(sc.positions, device), _t(log_s, device), _t(sc.quats, device))
+    cand2, off2 = oracle_mod.bin_legacy(sc.positions, log_s, fr.view[None], fr.proj, fr.W, fr.H, 8, fr.thr)
+    c2, o2 = _t(cand2, device), _t(off2, device)
+    plain_ids, plain_keys = oracle_mod.sort_tiles(fr.rays_o, fr.rays_d, sc.positions, log_s, sc.quats, cand2, off2, fr.W,
+                                                  fr.H, 8, 8, family=family)
+    want = oracle_mod.render_tilecenter(fr.rays_o, fr.rays_d, sc.positions, log_s, sc.quats, cand2, off2, sc.freq, sc.att,
+                                        *sc.mlp(), *fr.dims)
+    for with_records in (True, False):
+        got, _ = ops.sort_tiles(_t(fr.rays_o, device), _t(fr.rays_d, device), rec2, c2, o2, fr.W, fr.H, 8, 8, family=family,
+                                cull_threshold=fr.thr, frame_records=with_records)
+        got_np = got.cpu().numpy()
+        for t in range(off2.size - 1):
+            b = got_np[off2[t]:off2[t + 1]]
+            gone = ~b[b < 0]
+            a = plain_ids[off2[t]:off2[t + 1]]
+            assert np.array_equal(b[:b.size - gone.size], a[~np.isin(a, gone)])
+        if family == 1:
+            rgb, alpha, _ = ops.render_tilecenter_f32(_t(fr.rays_o, device), _t(fr.rays_d, device), rec2, got, o2,
+                                                      _t(sc.freq, device), _t(sc.att, device),
+                                                      *[_t(w, device) for w in sc.mlp()], fr.W, fr.H, 8, 8, fr.thr)
+            _assert_bits(rgb, want["rgb"], "rgb, extreme shapes, culled")
+            _assert_bits(alpha, want["alpha"], "alpha, extreme shapes, culled")
 
 
 def _render_gpu(fr, device, cand, off, family=1, with_t=False):
