@@ -212,13 +212,14 @@ def bin_legacy_async(positions, log_scales, view_matrices, proj_matrix, W: int, 
 
 
 def sort_tiles(rays_o, rays_d, records, candidates, tile_offsets, W, H, TW, TH, family=_lib.KEY_TSTAR,
-               capacity=TILE_CAPACITY_DEFAULT, want_keys=False, cull_threshold=0.0, frame_records=True):
+               capacity=TILE_CAPACITY_DEFAULT, want_keys=False, cull_threshold=0.0, frame_records=None):
     """Materialised per-tile depth order: (sorted_ids [P], sorted_keys [P] | None).
 
     With ``cull_threshold`` (the render's score threshold) candidates that provably hit no ray of their
     tile come back as ``~id``; the render kernels skip them, the image is unchanged.  ``frame_records``: let the
-    library write per-frame records for the common ray origin first (keys and order do not depend on it; False keeps
-    the full key evaluation per candidate, for comparing the two)."""
+    library write per-frame records for the common ray origin first (one more launch; a fifth fewer vector
+    instructions in the sort itself; keys and order do not depend on it).  None = what ``MLPSP_SORT_FRAME_RECORDS``
+    says, off unless it is 1: on one MI355X the extra launch costs a frame more than the sort kernel gains."""
     dev = rays_o.device
     sorted_ids = torch.empty_like(candidates)
     keys = torch.empty(candidates.numel(), dtype=torch.float32, device=dev) if want_keys else None
@@ -227,7 +228,9 @@ def sort_tiles(rays_o, rays_d, records, candidates, tile_offsets, W, H, TW, TH, 
     num_primitives = records.numel() // _lib.PRIM_RECORD_BYTES
     lib = _lib.load()
     scratch = None
-    if frame_records and os.environ.get("MLPSP_SORT_FRAME_RECORDS", "1") != "0":
+    if frame_records is None:
+        frame_records = os.environ.get("MLPSP_SORT_FRAME_RECORDS", "0") == "1"
+    if frame_records:
         scratch = torch.empty(lib.mlpsp_sort_frame_records_bytes(num_primitives), dtype=torch.uint8, device=dev)
     code = lib.mlpsp_sort_tiles(_ptr(rays_o), _ptr(rays_d), _ptr(records), num_primitives, _ptr(candidates),
                                 _ptr(tile_offsets), W, H, TW, TH, int(family), int(capacity), float(cull_threshold),
