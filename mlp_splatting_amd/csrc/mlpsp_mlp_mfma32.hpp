@@ -1,5 +1,5 @@
-// Wave-level f32 evaluation of one primitive's 72->32->32->4 MLP for the 64 pixels of a wavefront on the
-// matrix cores, bit-identical to the scalar chain of mlp_fixed<32, 6>.
+// Wave-level f32 evaluation of one primitive's 72->32->32->4 (or 72->16->16->4) MLP for the 64 pixels of a
+// wavefront on the matrix cores, bit-identical to the scalar chain of mlp_fixed<32, 6> (mlp_fixed<16, 6>).
 //
 // v_mfma_f32_32x32x2_f32 computes, per output element, fma(a1, b1, fma(a0, b0, c)) with both steps
 // rounded as IEEE f32 fused multiply-adds (no flush of denormals): one instruction is two consecutive links
@@ -15,6 +15,8 @@
 // moved into operand position by one half-wave swap per sin/cos pair; the same swap brings the 32 layer-2
 // outputs of a pixel onto its own lane for the 4-wide output layer, which runs on the vector ALU with
 // scalar weight operands.
+// With 16 hidden units the same tiles are half filled: A rows 16..31 are zero, accumulator registers 8..15 are
+// never read, layer 2 is eight instructions.  The order of every sum is unchanged.
 #pragma once
 #include "mlpsp_device.hpp"
 
@@ -56,6 +58,31 @@ __device__ __forceinline__ void load_interleaved16(const float* __restrict__ src
   }
 }
 
+// 8 consecutive floats at src + 8 g  ->  element i = src[2i + g], i < 8 (the rest of v is left alone).
+__device__ __forceinline__ void load_interleaved8(const float* __restrict__ src, int g, float v[16]) {
+  const mf32x4* __restrict__ s4 = reinterpret_cast<const mf32x4*>(src + 8 * g);
+  float c[8];
+#pragma unroll
+  for (int q = 0; q < 2; ++q) {
+    const mf32x4 t = s4[q];
+    c[4 * q + 0] = t[0];
+    c[4 * q + 1] = t[1];
+    c[4 * q + 2] = t[2];
+    c[4 * q + 3] = t[3];
+  }
+#pragma unroll
+  for (int t = 0; t < 4; ++t) {
+    half_swap(c[2 * t], c[2 * t + 1]);   // c[2t] = (src[2t], src[2t+1]), c[2t+1] = (src[8+2t], src[9+2t])
+    v[t] = c[2 * t];
+    v[4 + t] = c[2 * t + 1];
+  }
+}
+template <int H>
+__device__ __forceinline__ void load_interleaved(const float* __restrict__ src, int g, float v[16]) {
+  if constexpr (H == 32) load_interleaved16(src, g, v);
+  else load_interleaved8(src, g, v);
+}
+
 // max(x, +0): v_max_f32 yields the same bits as x > 0 ? x : 0 for every x (NaN -> 0, -0 -> +0).  Written
 // as a builtin, not as inline assembly: the compiler must see the instruction to keep the wait states
 // between a matrix-core result and its first reader.
@@ -86,38 +113,45 @@ __device__ __forceinline__ void encode_direction(float rdx, float rdy, float rdz
 // which encode_direction() made from them); out is the lane's own pixel's output.
 // REC selects the record kernels' layer-2 rounding (bias added after a chain started at zero); MASKS fills
 // masks[0..1] with the ReLU masks of the lane's pixel.
-template <bool REC = false, bool MASKS = REC>
+template <bool REC = false, bool MASKS = REC, int HID = 32>
 __device__ __forceinline__ void mlp_wave_mfma32(const float x6[6], const float* __restrict__ freq,
                                                 const float* __restrict__ att, const float* __restrict__ W1,
                                                 const float* __restrict__ b1, const float* __restrict__ W2,
                                                 const float* __restrict__ b2, const float* __restrict__ W3,
                                                 const float* __restrict__ b3, int p, const DirOperands& dir,
                                                 float out[4], uint32_t* masks = nullptr) {
-  constexpr int H = 32, IN = 72, HALF = 36;
+  static_assert(HID == 32 || HID == 16, "hidden width of the matrix-core f32 evaluation");
+  constexpr int H = HID, IN = 72, HALF = 36, R = H / 2;   // R: accumulator registers in use (hidden units 2i + g)
   const int lane = threadIdx.x & 63, m = lane & 31, g = lane >> 5;
   const int hid = 8 * (m >> 3) + 2 * (m & 3) + ((m >> 2) & 1);
+  const bool row_used = hid < H;                           // (always, with 32 hidden units)
+  const int row = row_used ? hid : 0;                      // unused rows read row 0 and supply zeros
 
   // A operands: lane (m, g) supplies row hid, k = g of every instruction.
   float a1[HALF];
   {
-    const mf32x4* __restrict__ s4 = reinterpret_cast<const mf32x4*>(W1 + (size_t)p * (H * IN) + hid * IN + HALF * g);
+    const mf32x4* __restrict__ s4 = reinterpret_cast<const mf32x4*>(W1 + (size_t)p * (H * IN) + row * IN + HALF * g);
 #pragma unroll
     for (int q = 0; q < HALF / 4; ++q) {
       const mf32x4 t = s4[q];
-      a1[4 * q + 0] = t[0];
-      a1[4 * q + 1] = t[1];
-      a1[4 * q + 2] = t[2];
-      a1[4 * q + 3] = t[3];
+      a1[4 * q + 0] = row_used ? t[0] : 0.f;
+      a1[4 * q + 1] = row_used ? t[1] : 0.f;
+      a1[4 * q + 2] = row_used ? t[2] : 0.f;
+      a1[4 * q + 3] = row_used ? t[3] : 0.f;
     }
   }
-  float a2[16], bias1[16], bias2[16];
-  load_interleaved16(W2 + (size_t)p * (H * H) + hid * H, g, a2);
-  load_interleaved16(b1 + (size_t)p * H, g, bias1);
-  load_interleaved16(b2 + (size_t)p * H, g, bias2);
+  float a2[16] = {}, bias1[16] = {}, bias2[16] = {};
+  load_interleaved<H>(W2 + (size_t)p * (H * H) + row * H, g, a2);
+  load_interleaved<H>(b1 + (size_t)p * H, g, bias1);
+  load_interleaved<H>(b2 + (size_t)p * H, g, bias2);
+  if constexpr (H != 32) {
+#pragma unroll
+    for (int i = 0; i < R; ++i) a2[i] = row_used ? a2[i] : 0.f;
+  }
 
   mf32x16 d0, d1;
 #pragma unroll
-  for (int i = 0; i < 16; ++i) d0[i] = d1[i] = bias1[i];
+  for (int i = 0; i < 16; ++i) d0[i] = d1[i] = (i < R) ? bias1[i] : 0.f;
 #pragma unroll
   for (int j = 0; j < 18; ++j) {
     d0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a1[j], dir.b0[j], d0, 0, 0, 0);
@@ -137,15 +171,15 @@ __device__ __forceinline__ void mlp_wave_mfma32(const float x6[6], const float* 
 
   mf32x16 e0, e1;
 #pragma unroll
-  for (int i = 0; i < 16; ++i) e0[i] = e1[i] = REC ? 0.f : bias2[i];
+  for (int i = 0; i < 16; ++i) e0[i] = e1[i] = (REC || i >= R) ? 0.f : bias2[i];
 #pragma unroll
-  for (int i = 0; i < 16; ++i) {
+  for (int i = 0; i < R; ++i) {
     e0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a2[i], relu_f32(d0[i]), e0, 0, 0, 0);
     e1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a2[i], relu_f32(d1[i]), e1, 0, 0, 0);
   }
   if constexpr (REC) {
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
+    for (int i = 0; i < R; ++i) {
       e0[i] = bias2[i] + e0[i];
       e1[i] = bias2[i] + e1[i];
     }
@@ -157,7 +191,7 @@ __device__ __forceinline__ void mlp_wave_mfma32(const float x6[6], const float* 
   float acc[4] = {bb3[0], bb3[1], bb3[2], bb3[3]};
   uint32_t m2 = 0u;
 #pragma unroll
-  for (int i = 0; i < 16; ++i) {
+  for (int i = 0; i < R; ++i) {
     float even = relu_f32(e0[i]), odd = relu_f32(e1[i]);
     half_swap(even, odd);
 #pragma unroll
@@ -172,7 +206,7 @@ __device__ __forceinline__ void mlp_wave_mfma32(const float x6[6], const float* 
   if constexpr (MASKS) {
     uint32_t lo = 0u, hi = 0u;   // bits 2i + g of blocks 0 and 1, as held by this lane
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
+    for (int i = 0; i < R; ++i) {
       lo |= d0[i] > 0.f ? (1u << (2 * i + g)) : 0u;
       hi |= d1[i] > 0.f ? (1u << (2 * i + g)) : 0u;
     }

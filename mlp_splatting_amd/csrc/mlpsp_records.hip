@@ -169,7 +169,7 @@ int records_launch(bool emit, const float* rays_o, const float* rays_d, const vo
   if (tile_px <= 0 || tile_px > 256) return MLPSP_E_ARGUMENT;
   if (F <= 0 || F > 16 || hidden <= 0 || hidden > 32 || N < 0 || max_hits <= 0) return MLPSP_E_ARGUMENT;
   if (!rays_o || !rays_d || !offsets || !overflow) return MLPSP_E_ARGUMENT;
-  if (render_order && !use_mfma32(hidden, F, W1, b1, W2, b2)) return MLPSP_E_ARGUMENT;
+  if (render_order && !(hidden == 32 && use_mfma32(hidden, F, W1, b1, W2, b2))) return MLPSP_E_ARGUMENT;
   const int wpt = (int)((tile_px + 63) / 64);
   const int64_t items = T * wpt;
   if (items > 2147483647LL - 8) return MLPSP_E_ARGUMENT;
@@ -183,7 +183,7 @@ int records_launch(bool emit, const float* rays_o, const float* rays_d, const vo
 #define MLPSP_REC_SHAPES(EM)                                          \
   do {                                                                \
     if (render_order) MLPSP_REC_LAUNCH(32, 6, EM, true, true);          \
-    else if (use_mfma32(hidden, F, W1, b1, W2, b2)) MLPSP_REC_LAUNCH(32, 6, EM, true); \
+    else if (hidden == 32 && use_mfma32(hidden, F, W1, b1, W2, b2)) MLPSP_REC_LAUNCH(32, 6, EM, true); \
     else if (hidden == 32 && F == 6) MLPSP_REC_LAUNCH(32, 6, EM);     \
     else if (hidden == 16 && F == 6) MLPSP_REC_LAUNCH(16, 6, EM);     \
     else MLPSP_REC_LAUNCH(0, 0, EM);                                  \

@@ -47,7 +47,10 @@ MLPSP_API int mlpsp_render_tilecenter_f32(const float* rays_o_dev, const float* 
                      (const PrimRecord*)prim_records_dev, order_dev, tile_offsets_dev, freq_dev, att_dev,         \
                      num_frequencies, W1, b1, W2, b2, W3, b3, num_primitives, hidden, g, wpt, per_xcd, (int)items, threshold,           \
                      out_rgb_dev, out_alpha_dev, out_t_dev, ctr, 0.f, 0.f, HitPool{})
-  if (use_mfma32(hidden, num_frequencies, W1, b1, W2, b2)) MLPSP_F32_LAUNCH(32, 6, false, true);
+  if (use_mfma32(hidden, num_frequencies, W1, b1, W2, b2)) {
+    if (hidden == 32) MLPSP_F32_LAUNCH(32, 6, false, true);
+    else MLPSP_F32_LAUNCH(16, 6, false, true);
+  }
   else if (hidden == 32 && num_frequencies == 6) MLPSP_F32_LAUNCH(32, 6);
   else if (hidden == 16 && num_frequencies == 6) MLPSP_F32_LAUNCH(16, 6);
   else MLPSP_F32_LAUNCH(0, 0);
@@ -90,7 +93,10 @@ MLPSP_API int mlpsp_render_tilecenter_stats_f32(const float* rays_o_dev, const f
                      (int)items, threshold, out_rgb_dev, out_alpha_dev, (float*)nullptr,                         \
                      (unsigned long long*)nullptr, 0.f, 0.f, HitPool{}, gt_rgb_dev, stat_sum_w_dev,              \
                      stat_max_w_dev, stat_hits_dev, stat_sum_werr_dev, stat_contrib_dev)
-  if (use_mfma32(hidden, num_frequencies, W1, b1, W2, b2)) MLPSP_STATS_LAUNCH(32, 6, true);
+  if (use_mfma32(hidden, num_frequencies, W1, b1, W2, b2)) {
+    if (hidden == 32) MLPSP_STATS_LAUNCH(32, 6, true);
+    else MLPSP_STATS_LAUNCH(16, 6, true);
+  }
   else if (hidden == 32 && num_frequencies == 6) MLPSP_STATS_LAUNCH(32, 6);
   else if (hidden == 16 && num_frequencies == 6) MLPSP_STATS_LAUNCH(16, 6);
   else MLPSP_STATS_LAUNCH(0, 0);

@@ -30,7 +30,7 @@ __device__ __forceinline__ float wave_max(float v) {
 }
 
 // MF: the 72->32->32->4 MLP runs on the matrix cores for all 64 pixels at once (mlp_wave_mfma32, same bits);
-// requires HT == 32, FT == 6 and 16-byte aligned weight arrays.
+// requires HT == 32 or 16, FT == 6 and 16-byte aligned weight arrays.
 template <int HT, int FT, int EMIT, bool STATS = false, bool MF = false>
 __global__ __launch_bounds__(64) void render_tilecenter_f32_kernel(
     const float* __restrict__ rays_o, const float* __restrict__ rays_d, const PrimRecord* __restrict__ prims,
@@ -100,7 +100,7 @@ __global__ __launch_bounds__(64) void render_tilecenter_f32_kernel(
       // (lanes that did not hit carry no hit point; the matrix-core evaluation runs on all 64 lanes)
       const float x6[6] = {rdx, rdy, rdz, hit ? h.dx : 0.f, hit ? h.dy : 0.f, hit ? h.dz : 0.f};
       float o[4];
-      if constexpr (MF) mlp_wave_mfma32<false>(x6, freq, att, W1, b1, W2, b2, W3, b3, p, dir, o);
+      if constexpr (MF) mlp_wave_mfma32<false, false, HT>(x6, freq, att, W1, b1, W2, b2, W3, b3, p, dir, o);
       if (hit) {
         if constexpr (!MF) mlp_eval<HT, FT>(x6, freq, att, F, H, mlp, p, o);
         const float w = blend_step(acc, o[0], o[1], o[2], o[3], h.decay, h.t);
@@ -158,12 +158,12 @@ __global__ __launch_bounds__(64) void render_tilecenter_f32_kernel(
   }
 }
 
-// Whether the matrix-core f32 evaluation applies: the fixed 72->32->32->4 shape, weight arrays that can be
+// Whether the matrix-core f32 evaluation applies: the 72->32->32->4 or 72->16->16->4 shape, weight arrays that can be
 // read 16 bytes at a time, and no request for the scalar kernel (environment MLPSP_F32_SCALAR=1, which
 // exists for comparison runs).
 inline bool use_mfma32(int hidden, int num_frequencies, const float* W1, const float* b1, const float* W2,
                        const float* b2) {
-  if (hidden != 32 || num_frequencies != 6) return false;
+  if ((hidden != 32 && hidden != 16) || num_frequencies != 6) return false;
   if (((uintptr_t)W1 | (uintptr_t)b1 | (uintptr_t)W2 | (uintptr_t)b2) & 15u) return false;
   const char* e = getenv("MLPSP_F32_SCALAR");
   return !(e && e[0] == '1');

@@ -176,7 +176,7 @@ MLPSP_API int mlpsp_render_tilecenter_feat_f32(
                      out_rgb_dev, out_alpha_dev, (float*)nullptr, (unsigned long long*)nullptr, gating_beta,      \
                      gating_temp, hp)
   const bool gated = feat_slots > 1;
-  if (use_mfma32(hidden, num_frequencies, W1, b1, W2, b2)) {
+  if (hidden == 32 && use_mfma32(hidden, num_frequencies, W1, b1, W2, b2)) {
     if (gated) MLPSP_EMIT_LAUNCH(32, 6, 2, false, true);
     else MLPSP_EMIT_LAUNCH(32, 6, 1, false, true);
   } else if (hidden == 32 && num_frequencies == 6) {

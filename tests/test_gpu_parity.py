@@ -373,8 +373,9 @@ def test_tilecentre_render_is_bit_exact_config1(device, oracle_mod, frame1):
 
 
 def test_scalar_and_matrix_core_f32_evaluations_agree_bit_for_bit(device, oracle_mod, frame1, monkeypatch):
-    """The 72-32-32-4 shape runs on the matrix cores; MLPSP_F32_SCALAR=1 and weight arrays that are not
-    16-byte aligned select the scalar kernel.  All three must produce the oracle's bits."""
+    """The 72-32-32-4 and 72-16-16-4 shapes (this frame: 16 hidden units, half-filled tiles) run on the matrix
+    cores; MLPSP_F32_SCALAR=1 and weight arrays that are not 16-byte aligned select the scalar kernel.  All three
+    must produce the oracle's bits."""
     from mlp_splatting_amd import ops
     fr = frame1
     cand, off = fr.lists
