@@ -169,12 +169,21 @@ int mlpsp_bin_raycone_fill(int num_primitives, int width, int height, int tile, 
  * offset centre - origin of the key (np_tile_kernels.cu:483-500), which depends on the primitive alone when the
  * rays share an origin -- and every tile whose centre ray starts at that origin takes its keys from those records
  * (one quaternion rotation per candidate instead of two; same expressions, same key bits); other tiles, and every
- * tile without the scratch, evaluate the key in full.  Sorted ids and keys do not depend on it. */
+ * tile without the scratch, evaluate the key in full.  Sorted ids and keys do not depend on it.
+ * frame_records_ready != 0: the records are there already -- mlpsp_frame_prologue wrote them, for these rays and
+ * these primitive records, earlier on the same stream -- and no launch is added. */
 size_t mlpsp_sort_frame_records_bytes(int num_primitives);
+/* The per-frame preparations that need nothing but the rays, in ONE launch: the unit directions of
+ * mlpsp_normalize_rays and the sort's frame records (for the origin of ray 0).  No counterpart in the reference,
+ * which normalises with torch (scannet/cumodel.py:1088) and evaluates the whole key per candidate. */
+int mlpsp_frame_prologue(const float* rays_d_dev, long long num_rays, float* unit_dirs_dev, const float* rays_o_dev,
+                         const void* prim_records_dev, int num_primitives, void* frame_records_dev,
+                         mlpsp_stream_t stream);
 int mlpsp_sort_tiles(const float* rays_o_dev, const float* rays_d_dev, const void* prim_records_dev,
                      int num_primitives, const int32_t* candidates_dev, const int32_t* tile_offsets_dev, int width,
                      int height, int tile_w, int tile_h, int key_family, int capacity, float cull_threshold,
-                     void* frame_records_dev, int32_t* sorted_ids_dev, float* sorted_keys_dev, mlpsp_stream_t stream);
+                     void* frame_records_dev, int frame_records_ready, int32_t* sorted_ids_dev,
+                     float* sorted_keys_dev, mlpsp_stream_t stream);
 
 /* Tile-centre-order forward, scalar f32 (render_tiles_kernel_tilecenter_order,
  * np_tile_kernels.cu:1837-2137; with out_t_dev != NULL also the expected depth of :5432-5719).

@@ -46,7 +46,8 @@ SIGNATURES = {
     "mlpsp_bin_raycone_count": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _f, _vp, _sz, _vp, C.POINTER(_i64), _vp]),
     "mlpsp_bin_raycone_fill": (_i, [_i, _i, _i, _i, _vp, _sz, _vp, _vp, _vp]),
     "mlpsp_sort_frame_records_bytes": (_sz, [_i]),
-    "mlpsp_sort_tiles": (_i, [_vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _vp, _vp, _vp, _vp]),
+    "mlpsp_frame_prologue": (_i, [_vp, C.c_longlong, _vp, _vp, _vp, _i, _vp, _vp]),
+    "mlpsp_sort_tiles": (_i, [_vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _vp, _i, _vp, _vp, _vp]),
     "mlpsp_render_tilecenter_f32": (_i, [_vp] * 7 + [_i] + [_vp] * 6 + [_i, _i, _i, _i, _i, _i, _f, _vp, _vp, _vp,
                                                                        _vp, _vp]),
     "mlpsp_render_tilecenter_feat_f32": (_i, [_vp] * 7 + [_i] + [_vp] * 6 + [_i, _i, _vp, _i, _i, _f, _f, _i, _i, _i, _i,

@@ -95,6 +95,26 @@ __global__ __launch_bounds__(256) void normalize_rays_kernel(const float* __rest
   out[i * 3 + 2] = z / den;
 }
 
+// The two per-frame preparations that depend on nothing but the rays, in one launch: blocks [0, ray_blocks) write
+// the unit directions (normalize_rays_kernel's statements), the blocks after them the sort's frame records.
+__global__ __launch_bounds__(256) void frame_prologue_kernel(const float* __restrict__ d, long long n,
+                                                             float* __restrict__ unit, int ray_blocks,
+                                                             const float* __restrict__ rays_o,
+                                                             const PrimRecord* __restrict__ prims, int N,
+                                                             SortRec* __restrict__ frame) {
+  if ((int)blockIdx.x < ray_blocks) {
+    const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const float x = d[i * 3], y = d[i * 3 + 1], z = d[i * 3 + 2];
+    const float den = fmaxf(sqrtf((x * x + z * z) + y * y), 1e-12f);
+    unit[i * 3] = x / den;
+    unit[i * 3 + 1] = y / den;
+    unit[i * 3 + 2] = z / den;
+  } else {
+    write_frame_sort_record(rays_o, prims, N, frame, ((int)blockIdx.x - ray_blocks) * (int)blockDim.x + (int)threadIdx.x);
+  }
+}
+
 // One 256-thread workgroup per tile (mlpsp_sort_tile.hpp); super-blocks of tiles per XCD: the geometry records a
 // tile gathers are mostly those of its neighbours.
 __global__ __launch_bounds__(kSortThreads) void sort_tiles_kernel(
@@ -154,6 +174,23 @@ MLPSP_API int mlpsp_normalize_rays(const float* rays_d_dev, long long num_rays, 
   return MLPSP_OK;
 }
 
+MLPSP_API int mlpsp_frame_prologue(const float* rays_d_dev, long long num_rays, float* unit_dirs_dev,
+                                   const float* rays_o_dev, const void* prim_records_dev, int num_primitives,
+                                   void* frame_records_dev, mlpsp_stream_t stream) {
+  if (num_rays <= 0 || num_rays > 2147483647LL * 128 || num_primitives <= 0) return MLPSP_E_ARGUMENT;
+  if (!rays_d_dev || !unit_dirs_dev || !rays_o_dev || !prim_records_dev || !frame_records_dev) return MLPSP_E_ARGUMENT;
+  if (reinterpret_cast<uintptr_t>(frame_records_dev) % 64 != 0 || reinterpret_cast<uintptr_t>(prim_records_dev) % 128 != 0)
+    return MLPSP_E_ARGUMENT;
+  const long long ray_blocks = (num_rays + 255) / 256;
+  const long long blocks = ray_blocks + ceil_div(num_primitives, 256);
+  if (blocks > 2147483647LL) return MLPSP_E_ARGUMENT;
+  hipLaunchKernelGGL(frame_prologue_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, rays_d_dev, num_rays,
+                     unit_dirs_dev, (int)ray_blocks, rays_o_dev, (const PrimRecord*)prim_records_dev, num_primitives,
+                     (SortRec*)frame_records_dev);
+  MLPSP_LAUNCH_CHECK();
+  return MLPSP_OK;
+}
+
 MLPSP_API int mlpsp_prepare_primitives(const float* positions_dev, const float* log_scales_dev,
                                        const float* quats_dev, int num_primitives, void* prim_records_dev,
                                        mlpsp_stream_t stream) {
@@ -196,8 +233,8 @@ MLPSP_API size_t mlpsp_sort_frame_records_bytes(int num_primitives) {
 MLPSP_API int mlpsp_sort_tiles(const float* rays_o_dev, const float* rays_d_dev, const void* prim_records_dev,
                                int num_primitives, const int32_t* candidates_dev, const int32_t* tile_offsets_dev,
                                int width, int height, int tile_w, int tile_h, int key_family, int capacity,
-                               float cull_threshold, void* frame_records_dev, int32_t* sorted_ids_dev,
-                               float* sorted_keys_dev, mlpsp_stream_t stream) {
+                               float cull_threshold, void* frame_records_dev, int frame_records_ready,
+                               int32_t* sorted_ids_dev, float* sorted_keys_dev, mlpsp_stream_t stream) {
   const int64_t T = checked_num_tiles(width, height, tile_w, tile_h);
   if (T <= 0 || T > 2147483647LL) return MLPSP_E_ARGUMENT;
   if (key_family != MLPSP_KEY_TSTAR && key_family != MLPSP_KEY_DEPTH) return MLPSP_E_ARGUMENT;
@@ -212,7 +249,7 @@ MLPSP_API int mlpsp_sort_tiles(const float* rays_o_dev, const float* rays_d_dev,
   float cull_r2 = 0.f;
   if (cull_threshold > 0.f && cull_threshold < 1.f) cull_r2 = -2.0f * logf(cull_threshold) * 1.0404f + 1e-6f;
   // per-frame records for the origin of ray 0: every tile whose centre ray starts there takes its keys from them
-  if (frame_records_dev) {
+  if (frame_records_dev && !frame_records_ready) {
     hipLaunchKernelGGL(frame_sort_records_kernel, dim3(ceil_div(num_primitives, 256)), dim3(256), 0, (hipStream_t)stream,
                        rays_o_dev, (const PrimRecord*)prim_records_dev, num_primitives, (SortRec*)frame_records_dev);
     MLPSP_LAUNCH_CHECK();

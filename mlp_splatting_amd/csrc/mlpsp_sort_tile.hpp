@@ -80,11 +80,10 @@ __device__ __forceinline__ uint32_t bf16_up(float x) {          // x >= 0: the s
   return (u >> 16) + ((u & 0xffffu) ? 1u : 0u);
 }
 
-// One thread per primitive; thread 0 of block 0 also writes the header.  origin = rays_o[0..2].
-__global__ __launch_bounds__(256) void frame_sort_records_kernel(const float* __restrict__ rays_o,
-                                                                 const PrimRecord* __restrict__ prims, int N,
-                                                                 SortRec* __restrict__ out) {
-  const int p = blockIdx.x * blockDim.x + threadIdx.x;
+// The record of primitive p (thread p = 0 also writes the header).  origin = rays_o[0..2].
+__device__ __forceinline__ void write_frame_sort_record(const float* __restrict__ rays_o,
+                                                        const PrimRecord* __restrict__ prims, int N,
+                                                        SortRec* __restrict__ out, int p) {
   const float ox = rays_o[0], oy = rays_o[1], oz = rays_o[2];
   if (p == 0) {
     SortFrameHeader h = {};
@@ -129,6 +128,12 @@ __global__ __launch_bounds__(256) void frame_sort_records_kernel(const float* __
   dst[2] = make_float4(vl.y, vl.z, v.x, v.y);
   dst[3] = make_float4(v.z, bits_to_float((hxx << 16) | (hyy & 0xffffu)), bits_to_float((hzz << 16) | (hxy & 0xffffu)),
                        bits_to_float((hxz << 16) | (hyz & 0xffffu)));
+}
+// One thread per primitive.
+__global__ __launch_bounds__(256) void frame_sort_records_kernel(const float* __restrict__ rays_o,
+                                                                 const PrimRecord* __restrict__ prims, int N,
+                                                                 SortRec* __restrict__ out) {
+  write_frame_sort_record(rays_o, prims, N, out, blockIdx.x * blockDim.x + threadIdx.x);
 }
 
 // key_tstar() with vl taken from the frame record: the remaining statements, unchanged.

@@ -846,13 +846,21 @@ class NeuralPrimitiveSceneTileCUDA(nn.Module):
             if binned is None:
                 return None
         ws = [p.detach().contiguous() for p in params]
-        unit_dirs = _unit_directions(ray_d)
-        freq, att = self._frequency_tables(device)
         more = {"binned": binned} if binned is not None else {}
+        ray_o = ray_o.contiguous()
+        if (hasattr(ext, "frame_prologue") and ray_d.is_cuda and ray_d.dtype == torch.float32 and ray_d.dim() == 2
+                and ray_d.shape[1] == 3 and not ray_d.requires_grad and ray_o.dtype == torch.float32
+                and ray_o.shape == ray_d.shape and os.environ.get("MLPSP_SORT_FRAME_RECORDS", "0") == "1"):
+            # unit directions and the sort's per-frame records in one launch (opt-in: measured 6 us per frame slower
+            # than the full key evaluation on one MI355X, where the sort is not bound by vector instructions)
+            unit_dirs, more["frame_records"] = ext.frame_prologue(ray_o, ray_d, positions, log_scales, self._unit_quats())
+        else:
+            unit_dirs = _unit_directions(ray_d)
+        freq, att = self._frequency_tables(device)
         if with_feat:
             more["feat"] = (self.feat_attr.detach().contiguous(), float(self.feature_gating_beta),
                             float(self.feature_gating_temp))
-        out = ext.render_frame_queued(ray_o.contiguous(), unit_dirs, positions, log_scales, self._unit_quats(), freq, att,
+        out = ext.render_frame_queued(ray_o, unit_dirs, positions, log_scales, self._unit_quats(), freq, att,
                                       ws, views, proj, int(W), int(H), float(score_threshold), precision, **more)
         if out is None:
             return None

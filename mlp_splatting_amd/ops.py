@@ -64,6 +64,22 @@ def normalize_rays(rays_d):
     return out
 
 
+def frame_prologue(rays_o, rays_d, records):
+    """(unit directions, frame records of the sort) in one launch: what :func:`normalize_rays` returns, and the
+    per-primitive records :func:`sort_tiles` takes as ``frame_records`` (written for the origin of ray 0)."""
+    rays_d, rays_o = _f32c(rays_d, "rays_d"), _f32c(rays_o, "rays_o")
+    if rays_d.dim() != 2 or rays_d.shape[1] != 3 or rays_o.shape != rays_d.shape:
+        raise ValueError("rays_o and rays_d must be [B, 3]")
+    lib = _lib.load()
+    n = records.numel() // _lib.PRIM_RECORD_BYTES
+    unit = torch.empty_like(rays_d)
+    frame = torch.empty(lib.mlpsp_sort_frame_records_bytes(n), dtype=torch.uint8, device=rays_d.device)
+    code = lib.mlpsp_frame_prologue(_ptr(rays_d), rays_d.shape[0], _ptr(unit), _ptr(rays_o), _ptr(records), n, _ptr(frame),
+                                    _stream(rays_d.device))
+    _check(code, "mlpsp_frame_prologue")
+    return unit, frame
+
+
 def validate_tile_lists(candidates, tile_offsets, n_tiles: int, capacity: int, num_primitives: int, path_name: str):
     """Raise the reference's RuntimeError texts (np_tile_kernels.cu:4578-4588) for a bad tile list."""
     for t, nm in ((candidates, "culled_prim_indices"), (tile_offsets, "tile_offsets")):
@@ -216,10 +232,11 @@ def sort_tiles(rays_o, rays_d, records, candidates, tile_offsets, W, H, TW, TH, 
     """Materialised per-tile depth order: (sorted_ids [P], sorted_keys [P] | None).
 
     With ``cull_threshold`` (the render's score threshold) candidates that provably hit no ray of their
-    tile come back as ``~id``; the render kernels skip them, the image is unchanged.  ``frame_records``: let the
-    library write per-frame records for the common ray origin first (one more launch; a fifth fewer vector
-    instructions in the sort itself; keys and order do not depend on it).  None = what ``MLPSP_SORT_FRAME_RECORDS``
-    says, off unless it is 1: on one MI355X the extra launch costs a frame more than the sort kernel gains."""
+    tile come back as ``~id``; the render kernels skip them, the image is unchanged.  ``frame_records``: the records
+    :func:`frame_prologue` wrote for these rays and primitives (a fifth fewer vector instructions in the sort; keys
+    and order do not depend on it), or True to let this call write them first (one more launch, which on one MI355X
+    costs a frame more than the sort kernel gains), or False.  None = what ``MLPSP_SORT_FRAME_RECORDS`` says, off
+    unless it is 1."""
     dev = rays_o.device
     sorted_ids = torch.empty_like(candidates)
     keys = torch.empty(candidates.numel(), dtype=torch.float32, device=dev) if want_keys else None
@@ -227,14 +244,19 @@ def sort_tiles(rays_o, rays_d, records, candidates, tile_offsets, W, H, TW, TH, 
         return sorted_ids, keys
     num_primitives = records.numel() // _lib.PRIM_RECORD_BYTES
     lib = _lib.load()
-    scratch = None
+    scratch, ready = None, 0
     if frame_records is None:
         frame_records = os.environ.get("MLPSP_SORT_FRAME_RECORDS", "0") == "1"
-    if frame_records:
+    if torch.is_tensor(frame_records):
+        if not (frame_records.is_cuda and frame_records.dtype == torch.uint8 and frame_records.is_contiguous()
+                and frame_records.numel() == lib.mlpsp_sort_frame_records_bytes(num_primitives)):
+            raise ValueError("frame_records must be the uint8 buffer frame_prologue() returned for these primitives")
+        scratch, ready = frame_records, 1
+    elif frame_records:
         scratch = torch.empty(lib.mlpsp_sort_frame_records_bytes(num_primitives), dtype=torch.uint8, device=dev)
     code = lib.mlpsp_sort_tiles(_ptr(rays_o), _ptr(rays_d), _ptr(records), num_primitives, _ptr(candidates),
                                 _ptr(tile_offsets), W, H, TW, TH, int(family), int(capacity), float(cull_threshold),
-                                _ptr(scratch), _ptr(sorted_ids), _ptr(keys), _stream(dev))
+                                _ptr(scratch), ready, _ptr(sorted_ids), _ptr(keys), _stream(dev))
     _check(code, "mlpsp_sort_tiles")
     return sorted_ids, keys
 

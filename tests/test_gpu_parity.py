@@ -153,7 +153,7 @@ def test_unit_directions_are_the_bits_of_torch_normalize(device, rays, scale):
     assert torch.equal(ops.normalize_rays(sliced), torch.nn.functional.normalize(sliced, dim=-1))
 
 
-@pytest.mark.parametrize("frame_records", [True, False], ids=["frame_records", "full_key"])
+@pytest.mark.parametrize("frame_records", [True, False, "prologue"], ids=["frame_records", "full_key", "prologue"])
 @pytest.mark.parametrize("family", [1, 2])
 def test_sorted_tile_lists_match_oracle_keys_and_order(device, oracle_mod, frame1, family, frame_records):
     # frame_records: the rotated offset centre - origin of the key comes from per-frame records (one per primitive,
@@ -163,6 +163,10 @@ def test_sorted_tile_lists_match_oracle_keys_and_order(device, oracle_mod, frame
     sc = fr.scene
     cand, off = fr.lists
     rec = ops.prepare_primitives(_t(sc.positions, device), _t(sc.log_scales, device), _t(sc.quats, device))
+    if frame_records == "prologue":
+        # the records written beside the unit directions, in one launch; the directions are normalize_rays' bits
+        unit, frame_records = ops.frame_prologue(_t(fr.rays_o, device), _t(fr.rays_d, device), rec)
+        assert torch.equal(unit.view(torch.int32), ops.normalize_rays(_t(fr.rays_d, device)).view(torch.int32))
     ids, keys = ops.sort_tiles(_t(fr.rays_o, device), _t(fr.rays_d, device), rec, _t(cand, device), _t(off, device),
                                fr.W, fr.H, 8, 8, family=family, want_keys=True, frame_records=frame_records)
     want_ids, want_keys = oracle_mod.sort_tiles(fr.rays_o, fr.rays_d, sc.positions, sc.log_scales, sc.quats, cand, off,
