@@ -131,8 +131,10 @@ int mlpsp_bin_legacy_fill(int num_primitives, int num_views, const int32_t* tile
  * (mlpsp_bin_static_scratch_bytes() = MLPSP_BIN_STATIC_SCRATCH_BYTES bytes, held on every GPU the library runs on
  * until the process ends); inputs whose mlpsp_bin_scratch_bytes() exceed it return MLPSP_E_SCRATCH, more than
  * MLPSP_BIN_STATIC_MAX_VIEWS views MLPSP_E_ARGUMENT (the matrices travel as kernel arguments).  Same outputs,
- * guard behaviour and launches as mlpsp_bin_legacy_async; nothing is cleared with a memset (a fill kernel where
- * needed), so the call may be captured.  All calls on one GPU share the one array: calls that overlap on a GPU
+ * guard behaviour and launches as mlpsp_bin_legacy_async, except that the level-1 lists get all of the array that
+ * the rest leaves free (their overflow -- counts_dev[3] = 1 with counts_dev[2] entries -- is therefore rarer than with
+ * a scratch of mlpsp_bin_scratch_bytes(); if it still happens the input needs mlpsp_bin_legacy_async with a larger
+ * scratch); nothing is cleared with a memset (a fill kernel where needed), so the call may be captured.  All calls on one GPU share the one array: calls that overlap on a GPU
  * (two streams, two threads) race and must be serialised by the caller. */
 size_t mlpsp_bin_static_scratch_bytes(void);
 int mlpsp_bin_legacy_async_noalloc(const float* positions_dev, const float* log_scales_dev, int num_primitives,

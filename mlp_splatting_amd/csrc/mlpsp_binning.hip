@@ -1047,9 +1047,11 @@ MLPSP_API int mlpsp_bin_legacy_async_noalloc(const float* positions_dev, const f
   if (rc != MLPSP_OK) return rc;
   hipStream_t s = (hipStream_t)stream;
   const BinGeom g = make_geom(num_primitives, num_views, width, height, tile);
-  // the array is carved for exactly the size the ordinary entry point would be given, so that both run the
-  // same launches on the same layout
-  const BinScratch b = carve(scratch_dev, need, num_primitives, num_views, g.nsx * g.nsy, g.NC);
+  // The whole array is carved, not just the bytes the ordinary entry point asks for: what is left over goes to the
+  // level-1 lists, whose overflow (guard word raised, lists emptied) a caller that cannot allocate could not answer
+  // with a larger scratch.  Lists do not depend on the capacity they were built in: same outputs as
+  // mlpsp_bin_legacy_async wherever that one does not overflow.
+  const BinScratch b = carve(scratch_dev, kStaticBinScratchBytes, num_primitives, num_views, g.nsx * g.nsy, g.NC);
   if (num_primitives == 0) {
     hipLaunchKernelGGL(fill_i32_kernel, dim3(64), dim3(256), 0, s, tile_offsets_dev, (long long)(T + 1), 0);
     MLPSP_LAUNCH_CHECK();

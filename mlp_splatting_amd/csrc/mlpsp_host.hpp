@@ -49,6 +49,16 @@ inline unsigned superblock_grid(int ntx, int nty) {
   return (unsigned)(((nsb + kNumXcd - 1) / kNumXcd) * kNumXcd * kSuperSide * kSuperSide);
 }
 
+// j-th tile slot of XCD xcd
+__device__ __forceinline__ int superblock_tile_of(int xcd, int j, int ntx, int nty) {
+  constexpr int SB = kSuperSide;
+  const int nsx = (ntx + SB - 1) / SB, nsy = (nty + SB - 1) / SB;
+  const int sb = kNumXcd * (j / (SB * SB)) + xcd, within = j % (SB * SB);
+  if (sb >= nsx * nsy) return -1;
+  const int stx = (sb % nsx) * SB + within % SB, sty = (sb / nsx) * SB + within / SB;
+  return (stx < ntx && sty < nty) ? sty * ntx + stx : -1;
+}
+
 __device__ __forceinline__ int superblock_tile(unsigned block, int ntx, int nty) {
   constexpr int SB = kSuperSide;
   const int nsx = (ntx + SB - 1) / SB, nsy = (nty + SB - 1) / SB;

@@ -156,6 +156,40 @@ __device__ __forceinline__ void phase_scales(const float* __restrict__ freq, con
   for (int j = 0; j < 3; ++j) kf[j] = (freq[3 * g + j] * att[3 * g + j]) * kInvTwoPi;
 }
 
+// sin and cos of the position half of the encoding from a table (forward render, bf16 operands).
+//
+// Every instruction this kernel issues costs its full issue time -- a transcendental twice and a half that of an
+// ordinary vector instruction -- and the 18 (sin, cos) pairs of a hit step were a sixth of it.  A table of
+// kSinCosEntries operand words (sin, cos of entry / kSinCosEntries revolutions, already rounded and packed) in the
+// workgroup's LDS replaces, per pair, two transcendentals and the pack by one mask and one LDS read: the phase
+// x k is formed in units of a quarter table entry by the multiply-add that used to be the multiply,
+//     y = fma(x, k * 4 * kSinCosEntries, 1.5 * 2^23 + 2),
+// whose low mantissa bits ARE the rounded integer (the constant puts y where floats are spaced one apart), so that
+// bits(y) & (4 * kSinCosEntries - 4) is the byte offset of the nearest entry.  The angle is off by at most half an
+// entry, pi / 2048 = 1.5e-3 rad: 0.8 of what rounding sin and cos to bf16 costs anyway (fp16 operands, which round
+// eight times finer, keep the instructions).  Valid while |x k| < 512 revolutions; the caller checks the inputs.
+#ifndef MLPSP_SINCOS_ENTRIES
+#define MLPSP_SINCOS_ENTRIES 2048
+#endif
+constexpr int kSinCosEntries = MLPSP_SINCOS_ENTRIES;
+constexpr float kSinCosMagic = 12582912.0f + 2.0f;
+constexpr float kSinCosRange = 500.0f;          // revolutions (the multiply-add is exact to an entry below 512)
+struct SinCosTable {
+  unsigned w[kSinCosEntries];
+};
+// Filled by the whole workgroup (any size); the caller puts a barrier behind it.
+template <typename T>
+__device__ __forceinline__ void fill_sincos_table(SinCosTable& t) {
+  for (int e = threadIdx.x; e < kSinCosEntries; e += blockDim.x) {
+    const float rev = (float)e * (1.0f / (float)kSinCosEntries);
+    t.w[e] = Ops<T>::pack2(__builtin_amdgcn_sinf(rev), __builtin_amdgcn_cosf(rev));
+  }
+}
+__device__ __forceinline__ unsigned sincos_word(const SinCosTable& t, float x, float k_scaled) {
+  const unsigned off = __float_as_uint(fmaf(x, k_scaled, kSinCosMagic)) & (4u * kSinCosEntries - 4u);
+  return *reinterpret_cast<const unsigned*>(reinterpret_cast<const unsigned char*>(t.w) + off);
+}
+
 template <typename T>
 __device__ __forceinline__ void encode_direction_words(float rdx, float rdy, float rdz, const float kf[3], int l,
                                                        DirWords& s) {
@@ -239,10 +273,12 @@ __device__ __forceinline__ f32x4 layer3_small(u32x4 a, u32x4 b, f32x4 c) {
 // non-finite when packed or (CHECK) a pre-activation of a hit pixel is out of range.
 // Vector-memory instructions per call: 7 (W1, W2) + 1 (b2 words) + 2 (W3); the output bias and the flag are
 // wave-uniform scalar loads.
-template <typename T, bool CHECK, bool MASKS>
+// LUT: the position words come from the workgroup's sin/cos table; kf then holds the phase scales times
+// 4 kSinCosEntries.
+template <typename T, bool CHECK, bool MASKS, bool LUT = false>
 __device__ __forceinline__ bool mlp_wave_mfma16(const unsigned char* __restrict__ blk, unsigned long long mask, int l,
                                                 float dx, float dy, float dz, const float kf[3], const DirWords& dir,
-                                                float o[4], unsigned mk[2]) {
+                                                float o[4], unsigned mk[2], const SinCosTable* table = nullptr) {
   const int g = l >> 5;
   bool bad = false;
   // Addresses of the weight loads: wave-uniform base in scalar registers + zero-extended 32-bit lane offset +
@@ -301,8 +337,12 @@ __device__ __forceinline__ bool mlp_wave_mfma16(const unsigned char* __restrict_
           } else if (t == 8) {
             bw[d] = d8;
           } else if (t < 18) {
-            const float rev = xin[t / 3 - 3] * kf[t % 3];
-            bw[d] = Ops<T>::pack2(__builtin_amdgcn_sinf(rev), __builtin_amdgcn_cosf(rev));
+            if constexpr (LUT) {
+              bw[d] = sincos_word(*table, xin[t / 3 - 3], kf[t % 3]);
+            } else {
+              const float rev = xin[t / 3 - 3] * kf[t % 3];
+              bw[d] = Ops<T>::pack2(__builtin_amdgcn_sinf(rev), __builtin_amdgcn_cosf(rev));
+            }
           } else if (t == 18) {
             bw[d] = one_word;
           } else {
@@ -371,10 +411,10 @@ __device__ __forceinline__ bool mlp_wave_mfma16(const unsigned char* __restrict_
 // nothing else to issue while an MFMA or its first reader waits.  Here every MFMA of block 0 is followed by the
 // independent MFMA of block 1, and the operand preparation of one block sits behind the MFMA of the other.
 // No ReLU masks (render only).
-template <typename T, bool CHECK>
+template <typename T, bool CHECK, bool LUT = false>
 __device__ __forceinline__ bool mlp_pair_mfma16(const unsigned char* __restrict__ blk, unsigned long long mask, int l,
                                                 float dx, float dy, float dz, const float kf[3], const DirWords& dir,
-                                                float o[4]) {
+                                                float o[4], const SinCosTable* table = nullptr) {
   const int g = l >> 5;
   bool bad = false;
   // Addresses of the weight loads: wave-uniform base in scalar registers + zero-extended 32-bit lane offset +
@@ -423,8 +463,12 @@ __device__ __forceinline__ bool mlp_pair_mfma16(const unsigned char* __restrict_
           if (t == 8) {
             bw[d] = dir.w8[b][ll];
           } else if (t < 18) {
-            const float rev = xin[b][t / 3 - 3] * kf[t % 3];
-            bw[d] = Ops<T>::pack2(__builtin_amdgcn_sinf(rev), __builtin_amdgcn_cosf(rev));
+            if constexpr (LUT) {
+              bw[d] = sincos_word(*table, xin[b][t / 3 - 3], kf[t % 3]);
+            } else {
+              const float rev = xin[b][t / 3 - 3] * kf[t % 3];
+              bw[d] = Ops<T>::pack2(__builtin_amdgcn_sinf(rev), __builtin_amdgcn_cosf(rev));
+            }
           } else if (t == 18) {
             bw[d] = one_word;
           } else {

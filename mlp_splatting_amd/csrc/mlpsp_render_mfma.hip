@@ -232,6 +232,12 @@ struct OriginLds {
   float e[64][SP > 0 ? 12 : 8];
 };
 
+// The table only for bf16 operands (see kSinCosEntries).
+template <typename T> struct RenderTable { static constexpr bool kUse = false; unsigned w[1]; };
+#if !defined(MLPSP_RENDER_NO_TABLE)
+template <> struct RenderTable<__bf16> { static constexpr bool kUse = true; SinCosTable t; };
+#endif
+
 // SP = 0: RGB only.  SP = 4 or 8: the kernel also emits, per tile, the compact list of primitives that
 // hit at least one pixel (hit records, mlpsp_hitrec.hpp) and per (such primitive, pixel) the SP compositing
 // coefficients of the gated feature channel, rounded to fp16 (they lie in [0, 1]; fp16 keeps 11
@@ -244,7 +250,8 @@ struct OriginLds {
 // One tile, rendered by the calling wavefront (lane l = pixel l of the tile); s_dir: LDS of this wavefront alone.
 template <typename T, int SP>
 __device__ __forceinline__ void render_tile_mfma(
-    const int tile, const int l, DirWords& s_dir, OriginLds<SP>& s_org, const float* __restrict__ rays_o,
+    const int tile, const int l, DirWords& s_dir, OriginLds<SP>& s_org, const SinCosTable* table,
+    const float* __restrict__ rays_o,
     const float* __restrict__ rays_d, const PrimRecord* __restrict__ prims, const int32_t* __restrict__ order, const int32_t* __restrict__ offsets,
     const float* __restrict__ freq, const float* __restrict__ att, const unsigned char* __restrict__ packed, int N,
     int W, int H, int ntx, float thr, float* __restrict__ out_rgb, float* __restrict__ out_alpha,
@@ -252,6 +259,18 @@ __device__ __forceinline__ void render_tile_mfma(
     const HitPool& hp) {
   float kf[3];
   phase_scales(freq, att, l >> 5, kf);
+  // With the sin/cos table the MLP takes its phase scales in units of a quarter table entry, and the inputs must
+  // stay below kSinCosRange revolutions at the highest frequency (else the frame is flagged and rendered in f32,
+  // like any other operand this path cannot represent).
+  float kfm[3] = {kf[0], kf[1], kf[2]};
+  float input_limit = 3.4028235e38f;
+  if constexpr (RenderTable<T>::kUse) {
+    float kmax = fmaxf(fmaxf(__builtin_fabsf(kf[0]), __builtin_fabsf(kf[1])), __builtin_fabsf(kf[2]));
+    kmax = fmaxf(kmax, __shfl_xor(kmax, 32));
+    input_limit = kSinCosRange / fmaxf(kmax, 1e-30f);
+#pragma unroll
+    for (int j = 0; j < 3; ++j) kfm[j] = kf[j] * (4.0f * (float)kSinCosEntries);
+  }
   unsigned n_proc = 0, n_proc_hit = 0, n_hits = 0;
   bool bad = false;
   const int tx = tile % ntx, ty = tile / ntx;
@@ -356,12 +375,14 @@ __device__ __forceinline__ void render_tile_mfma(
         ++n_proc_hit;
         n_hits += __popcll(mask);
         const unsigned char* __restrict__ blk = packed + (size_t)p * kPackStride;
-        bad |= hit && !(__builtin_fabsf((h.dx + h.dy) + h.dz) <= 3.4028235e38f);
+        bad |= hit && !((__builtin_fabsf(h.dx) + __builtin_fabsf(h.dy)) + __builtin_fabsf(h.dz) <= input_limit);
         float o[4];
         if ((unsigned)mask != 0u && (unsigned)(mask >> 32) != 0u)
-          bad |= mlp_pair_mfma16<T, Ops<T>::kCheckHidden>(blk, mask, l, h.dx, h.dy, h.dz, kf, s_dir, o);
+          bad |= mlp_pair_mfma16<T, Ops<T>::kCheckHidden, RenderTable<T>::kUse>(blk, mask, l, h.dx, h.dy, h.dz, kfm, s_dir, o,
+                                                                               table);
         else
-          bad |= mlp_wave_mfma16<T, Ops<T>::kCheckHidden, false>(blk, mask, l, h.dx, h.dy, h.dz, kf, s_dir, o, nullptr);
+          bad |= mlp_wave_mfma16<T, Ops<T>::kCheckHidden, false, RenderTable<T>::kUse>(blk, mask, l, h.dx, h.dy, h.dz, kfm,
+                                                                                      s_dir, o, nullptr, table);
         float w = 0.f;
         if (hit) {
           bad |= !(max3_abs(o[0], o[1], o[2]) <= 3.4028235e38f) || !(__builtin_fabsf(o[3]) <= 3.4028235e38f);
@@ -417,22 +438,38 @@ __device__ __forceinline__ void render_tile_mfma(
   }
 }
 
+// Four wavefronts = four tiles per workgroup: they share nothing but the sin/cos table, which they fill together
+// (sixteen transcendentals per thread) before each goes its own way.
+#ifndef MLPSP_RENDER_WAVES
+#define MLPSP_RENDER_WAVES 4
+#endif
+constexpr int kRenderWaves = MLPSP_RENDER_WAVES;
 template <typename T, int SP>
-__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 4))) void render_tilecenter_mfma_kernel(
+__global__ __launch_bounds__(64 * kRenderWaves) __attribute__((amdgpu_waves_per_eu(4, 4))) void render_tilecenter_mfma_kernel(
     const float* __restrict__ rays_o, const float* __restrict__ rays_d, const PrimRecord* __restrict__ prims,
     const int32_t* __restrict__ order, const int32_t* __restrict__ offsets, const float* __restrict__ freq,
     const float* __restrict__ att, const unsigned char* __restrict__ packed, int N, int W, int H, int ntx,
     int per_xcd, int num_tiles, float thr, float* __restrict__ out_rgb, float* __restrict__ out_alpha,
     int32_t* __restrict__ status, unsigned long long* __restrict__ counters, int slots, float beta, float temp,
     HitPool hp) {
+  __shared__ DirWords s_dir[kRenderWaves];
+  __shared__ __attribute__((aligned(16))) OriginLds<SP> s_org[kRenderWaves];
+  __shared__ RenderTable<T> s_table;
+  const SinCosTable* table = nullptr;
+  if constexpr (RenderTable<T>::kUse) {
+    fill_sincos_table<T>(s_table.t);
+    __syncthreads();
+    table = &s_table.t;
+  }
   // 8x8 super-blocks of tiles dealt to the XCDs in turn: neighbouring tiles, which share most primitives (their
-  // records and weight blocks), run on one L2
-  const int tile = superblock_tile(blockIdx.x, ntx, num_tiles / ntx);
+  // records and weight blocks), run on one L2.  Workgroup b runs on XCD b % 8 and takes four consecutive slots of it.
+  const int wave = (int)threadIdx.x >> 6;
+  const int tile = superblock_tile_of((int)(blockIdx.x % kNumXcd), (int)(blockIdx.x / kNumXcd) * kRenderWaves + wave, ntx,
+                                      num_tiles / ntx);
   if (tile < 0) return;
-  __shared__ DirWords s_dir;
-  __shared__ __attribute__((aligned(16))) OriginLds<SP> s_org;
-  render_tile_mfma<T, SP>(tile, (int)threadIdx.x, s_dir, s_org, rays_o, rays_d, prims, order, offsets, freq, att, packed, N, W,
-                          H, ntx, thr, out_rgb, out_alpha, status, counters, slots, beta, temp, hp);
+  render_tile_mfma<T, SP>(tile, (int)threadIdx.x & 63, s_dir[wave], s_org[wave], table, rays_o, rays_d, prims, order, offsets,
+                          freq, att, packed, N, W, H, ntx, thr, out_rgb, out_alpha, status, counters, slots, beta, temp,
+                          hp);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -791,7 +828,7 @@ void launch_mfma(dim3 grid, hipStream_t s, const float* rays_o, const float* ray
                  const int32_t* offsets, const float* freq, const float* att, const void* packed, int N, int W, int H,
                  int ntx, int per_xcd, int T, float thr, float* rgb, float* alpha, int32_t* status,
                  unsigned long long* ctr, int slots, float beta, float temp, const HitPool& hp) {
-  hipLaunchKernelGGL((render_tilecenter_mfma_kernel<E, SP>), grid, dim3(64), 0, s, rays_o, rays_d,
+  hipLaunchKernelGGL((render_tilecenter_mfma_kernel<E, SP>), dim3(grid.x / kRenderWaves), dim3(64 * kRenderWaves), 0, s, rays_o, rays_d,
                      (const PrimRecord*)prims, order, offsets, freq, att, (const unsigned char*)packed, N, W, H, ntx,
                      per_xcd, T, thr, rgb, alpha, status, ctr, slots, beta, temp, hp);
 }

@@ -81,6 +81,35 @@ def test_two_calls_in_a_row_the_second_smaller(device):
     assert third == first
 
 
+def test_the_call_allocates_nothing_on_the_device(device):
+    """After one warm-up call (the library takes the array's address once per device), a call changes neither the
+    allocator's books nor the free memory the driver reports."""
+    lib = _lib.load()
+    fp = C.POINTER(C.c_float)
+    for views in (1, 4):
+        n, width, height = 20000, 320, 240
+        positions, log_scales, vm, proj = _frame(n, width, height, 300.0, views, 4)
+        pos, logs = torch.from_numpy(positions).to(device), torch.from_numpy(log_scales).to(device)
+        tiles = ((width + 7) // 8) * ((height + 7) // 8)
+        offsets = torch.empty(tiles + 1, dtype=torch.int32, device=device)
+        cand = torch.empty(4_000_000, dtype=torch.int32, device=device)
+        counts = torch.empty(4, dtype=torch.int64, device=device)
+        tv = _tile_views(width, height, device) if views > 1 else None
+        stream = C.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+        ptr = lambda t: None if t is None else C.c_void_p(t.data_ptr())
+        args = (ptr(pos), ptr(logs), n, C.cast(vm.ctypes.data, fp), views, ptr(tv), C.cast(proj.ctypes.data, fp), width,
+                height, 8, 5e-3, ptr(offsets), ptr(cand), cand.numel(), ptr(counts), stream)
+        assert lib.mlpsp_bin_legacy_async_noalloc(*args) == 0            # warm-up
+        torch.cuda.synchronize(device)
+        before = (torch.cuda.memory_allocated(device), torch.cuda.memory_reserved(device), torch.cuda.mem_get_info(device)[0])
+        for _ in range(3):
+            assert lib.mlpsp_bin_legacy_async_noalloc(*args) == 0
+        torch.cuda.synchronize(device)
+        after = (torch.cuda.memory_allocated(device), torch.cuda.memory_reserved(device), torch.cuda.mem_get_info(device)[0])
+        assert after == before, (before, after)
+        assert int(counts[3]) == 0 and int(counts[0]) > 0
+
+
 def test_four_views_travel_as_kernel_arguments(device):
     case = dict(n=20000, width=320, height=240, focal=300.0, views=4, seed=2, thr=5e-3)
     case["tile_views"] = _tile_views(case["width"], case["height"], device)
