@@ -5,14 +5,18 @@
 // memory and without a sort, in two levels:
 //   level 1: the frame is cut into super-tiles of 8x8 tiles.  Wavefront (chunk c, super-tile s)
 //            tests 2048 consecutive primitives against the super-tile rectangle (a superset of the
-//            union of its tiles' tests), counts, and after a scan writes the survivors in ascending
+//            union of its tiles' tests) and counts; the fill pass writes the survivors in ascending
 //            id order -> one ascending candidate list per super-tile.  With one view and a screen of
 //            few super-tiles the counting goes the other way round: every primitive finds the
 //            super-tiles it overlaps (bin_level1_scatter_kernel, which also computes the bounds).
 //   level 2: one wavefront per tile walks its super-tile's list 64 ids at a time, applies the exact
-//            per-tile test, counts with a ballot, and after a scan writes the tile's candidates at
+//            per-tile test and counts with a ballot; the fill pass writes the tile's candidates at
 //            ballot-prefix positions -> tile-major lists, ascending id inside a tile, which is the
 //            order `nonzero()` on the dense matrix yields.
+// A fill pass needs the exclusive prefix sums of the counts.  Its workgroups form their own from the
+// counts (level 1) or from per-workgroup sums the counting pass leaves (level 2): four launches per
+// frame, count and fill of each level.  Only the two-call interface, whose caller sizes the candidate
+// buffer between the calls, scans the tile counts with a kernel of its own.
 // All kernels are HBM/L2-bound integer and compare work; nothing here wants MFMA.
 #include "mlpsp_device.hpp"
 #include "mlpsp_host.hpp"
@@ -25,12 +29,24 @@ namespace mlpsp {
 constexpr int kSuper = 8;       // tiles per super-tile side
 constexpr int kChunk = 2048;    // primitives per level-1 workgroup
 constexpr int kBinThreads = 256;
+constexpr int kWideThreads = 1024;              // workgroups that work out their own place in a list of lists
+constexpr int kL2Group = kWideThreads / 64;     // tiles per level-2 workgroup
+
+// what the level-2 counting pass leaves per workgroup, so that the fill pass can place its tiles without a scan
+// kernel in between
+struct L2Group {
+  long long sum;      // entries of the group's tile lists
+  int longest;        // its longest tile list
+  int pad;
+};
 
 struct BinScratch {
   float* mats;        // K view matrices (16 floats each) then the projection (16 floats)
   float4* bounds;     // [K][N] (minx, maxx, miny, maxy); all NaN when behind the near plane
-  int32_t* l1_counts; // [S*NC + 1] counts, then exclusive offsets after the scan
+  int32_t* l1_counts; // [S*NC + 1] survivors per (super-tile, chunk)
+  int32_t* l1_super;  // [S + 1] where each super-tile's list starts in l1_list (clamped to l1_capacity)
   long long* totals;  // [0] level-1 entries, [1] tile-list entries, [2] longest tile list, [3] guard status
+  struct L2Group* groups;   // [ceil(T / 16)] entries and longest list of every 16 consecutive tiles
   int32_t* l1_list;   // [l1_capacity]
   float4* l1_bounds;  // [l1_capacity] bounds of the listed primitives under the super-tile's view (garbage for a
                       // super-tile whose tiles use several views: super_view says which)
@@ -63,11 +79,15 @@ inline BinScratch carve(void* base, size_t bytes, int N, int K, int S, int NC) {
   off += align256((size_t)S * NC * (kChunk / 64) * sizeof(unsigned long long));
   b.super_view = reinterpret_cast<int32_t*>(p + off);
   off += align256((size_t)S * sizeof(int32_t));
+  b.l1_super = reinterpret_cast<int32_t*>(p + off);
+  off += align256(((size_t)S + 1) * sizeof(int32_t));
+  b.groups = reinterpret_cast<L2Group*>(p + off);           // a super-tile has at most 64 tiles = 4 groups
+  off += align256(((size_t)S * (64 / kL2Group) + 1) * sizeof(L2Group));
   // per level-1 entry: 4 bytes id + 16 bytes bounds + 64 mask bits for the 64 tiles = 8 bytes
   const size_t entry = sizeof(int32_t) + sizeof(float4) + 8;
   const size_t fixed = off + 1024 + align256((size_t)(S + 1) * 64 * sizeof(unsigned long long));
   b.l1_capacity = bytes > fixed ? (long long)((bytes - fixed) / entry) : 0;
-  b.l1_capacity &= ~63LL;
+  b.l1_capacity = (b.l1_capacity < 2147483584LL ? b.l1_capacity : 2147483584LL) & ~63LL;   // positions are 32-bit
   b.l1_list = reinterpret_cast<int32_t*>(p + off);
   off += align256((size_t)b.l1_capacity * sizeof(int32_t));
   b.l1_bounds = reinterpret_cast<float4*>(p + off);
@@ -184,15 +204,12 @@ __device__ __forceinline__ unsigned lanes_below(unsigned long long mask) {
   return __builtin_amdgcn_mbcnt_hi((unsigned)(mask >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)mask, 0u));
 }
 
-// level 1.  grid = (NC, ceil(S / 4)); wavefront w of a workgroup owns super-tile 4 * blockIdx.y + w and walks the
-// chunk's 2048 primitives 64 at a time (no workgroup barrier: counts and positions come from ballots).
-// FILL = false: l1_counts[s*NC + c] = survivors; FILL = true: write them.
-template <bool FILL>
+// level 1, counting pass by (chunk, super-tile).  grid = (NC, ceil(S / 4)); wavefront w of a workgroup owns super-tile
+// 4 * blockIdx.y + w and walks the chunk's 2048 primitives 64 at a time (no workgroup barrier: counts come from
+// ballots, which are kept for the fill pass): l1_counts[s*NC + c] = survivors.
 __global__ __launch_bounds__(kBinThreads) void bin_level1_kernel(const float4* __restrict__ bounds, BinGeom g,
                                                                  const int32_t* __restrict__ tile_view_ids,
                                                                  int32_t* __restrict__ l1_counts,
-                                                                 int32_t* __restrict__ l1_list,
-                                                                 float4* __restrict__ l1_bounds, long long l1_capacity,
                                                                  unsigned long long* __restrict__ l1_masks,
                                                                  int32_t* __restrict__ super_view) {
   const int c = blockIdx.x, s = blockIdx.y * (kBinThreads / 64) + (threadIdx.x >> 6);
@@ -223,50 +240,11 @@ __global__ __launch_bounds__(kBinThreads) void bin_level1_kernel(const float4* _
   // one view for the whole super-tile (always so with one camera): the fast paths below, here and in level 2
   const bool single = g.K == 1 || nviews == -1;
   const float4* __restrict__ sb = bounds + (size_t)(g.K == 1 ? 0 : v0) * g.N;
-  if (!FILL && c == 0 && lane == 0) super_view[s] = single ? (g.K == 1 ? 0 : v0) : -1;
-  long long running = FILL ? l1_counts[s * g.NC + c] : 0;
+  if (c == 0 && lane == 0) super_view[s] = single ? (g.K == 1 ? 0 : v0) : -1;
+  long long running = 0;
   const int first = c * kChunk;
   unsigned long long* __restrict__ masks = l1_masks + ((size_t)s * g.NC + c) * (kChunk / 64);
   static_assert(kChunk / 64 <= 64, "one ballot per lane");
-  if constexpr (FILL) {
-    // The counting pass left one ballot per 64 primitives: no bounds are read again except the survivors'.  Lane r
-    // fetches ballot r (one coalesced load), the ballots' bit counts are scanned, and then lane k writes the k-th
-    // survivor: it finds the ballot that holds it (a search over the scanned counts) and the bit inside.  All
-    // survivors' bounds are gathered at once -- one memory latency per 64 survivors; walking the ballots one after
-    // the other instead costs one per ballot that is not empty.
-    const unsigned long long mine = lane < kChunk / 64 ? masks[lane] : 0ull;
-    const int own = __popcll(mine);
-    int incl = own;
-#pragma unroll
-    for (int d = 1; d < kChunk / 64; d <<= 1) {
-      const int up = __shfl_up(incl, d);
-      if (lane >= d) incl += up;
-    }
-    const int before = incl - own;                     // survivors in the ballots ahead of this lane's
-    const int total = __shfl(incl, kChunk / 64 - 1);
-    static_assert(kChunk / 64 == 32, "the search below halves 32 ballots");
-    for (int k0 = 0; k0 < total; k0 += 64) {
-      const int k = k0 + lane;
-      int r = 0;                                       // the last ballot whose `before` is <= k holds survivor k
-#pragma unroll
-      for (int step = 16; step >= 1; step >>= 1) {
-        const int ahead = __shfl(before, r + step);
-        if (ahead <= k) r += step;
-      }
-      const int nth = k - __shfl(before, r);
-      const unsigned long long m = ((unsigned long long)(unsigned)__shfl((int)(mine >> 32), r) << 32) |
-                                   (unsigned)__shfl((int)mine, r);
-      if (k < total) {
-        const int i = first + r * 64 + nth_set_bit(m, nth);
-        const long long dst = running + k;
-        if (dst < l1_capacity) {
-          l1_list[dst] = i;
-          if (single) l1_bounds[dst] = sb[i];
-        }
-      }
-    }
-    return;
-  }
   unsigned long long mine = 0ull;
   if (single) {
     // one view: eight independent 16-byte loads in flight per step (NaN bounds fail every comparison)
@@ -475,30 +453,174 @@ __global__ __launch_bounds__(kScatterThreads) void bin_level1_scatter_kernel(
   }
 }
 
+// level 1, fill pass for one (chunk, super-tile) pair by one wavefront; `running` is where the pair's survivors
+// start in the level-1 list.  The counting pass left one ballot per 64 primitives: no bounds are read again except
+// the survivors'.  Lane r fetches ballot r (one coalesced load), the ballots' bit counts are scanned, and then lane
+// k writes the k-th survivor: it finds the ballot that holds it (a search over the scanned counts) and the bit
+// inside.  All survivors' bounds are gathered at once -- one memory latency per 64 survivors; walking the ballots
+// one after the other instead costs one per ballot that is not empty.
+__device__ __forceinline__ unsigned long long level1_ballots(const BinGeom& g, int c, int s,
+                                                             const unsigned long long* __restrict__ l1_masks) {
+  const int lane = threadIdx.x & 63;
+  return lane < kChunk / 64 ? l1_masks[((size_t)s * g.NC + c) * (kChunk / 64) + lane] : 0ull;
+}
+__device__ __forceinline__ void level1_fill_pair(int c, unsigned long long mine, long long running, bool single,
+                                                 const float4* __restrict__ sb, int32_t* __restrict__ l1_list,
+                                                 float4* __restrict__ l1_bounds, long long l1_capacity) {
+  const int lane = threadIdx.x & 63;
+  const int first = c * kChunk;
+  const int own = __popcll(mine);
+  int incl = own;
+#pragma unroll
+  for (int d = 1; d < kChunk / 64; d <<= 1) {
+    const int up = __shfl_up(incl, d);
+    if (lane >= d) incl += up;
+  }
+  const int before = incl - own;                     // survivors in the ballots ahead of this lane's
+  const int total = __shfl(incl, kChunk / 64 - 1);
+  static_assert(kChunk / 64 == 32, "the search below halves 32 ballots");
+  for (int k0 = 0; k0 < total; k0 += 64) {
+    const int k = k0 + lane;
+    int r = 0;                                       // the last ballot whose `before` is <= k holds survivor k
+#pragma unroll
+    for (int step = 16; step >= 1; step >>= 1) {
+      const int ahead = __shfl(before, r + step);
+      if (ahead <= k) r += step;
+    }
+    const int nth = k - __shfl(before, r);
+    const unsigned long long m = ((unsigned long long)(unsigned)__shfl((int)(mine >> 32), r) << 32) |
+                                 (unsigned)__shfl((int)mine, r);
+    if (k < total) {
+      const int i = first + r * 64 + nth_set_bit(m, nth);
+      const long long dst = running + k;
+      if (dst < l1_capacity) {
+        l1_list[dst] = i;
+        if (single) l1_bounds[dst] = sb[i];
+      }
+    }
+  }
+}
+
+__device__ __forceinline__ long long wave_sum(long long x) {
+#pragma unroll
+  for (int d = 32; d >= 1; d >>= 1) x += __shfl_xor(x, d);
+  return x;
+}
+
+// level 1, fill pass.  grid = S workgroups of 1024 threads: workgroup s writes super-tile s's list, chunk after chunk
+// (ascending primitive ids), a wavefront per (chunk, super-tile) pair.  Lists follow each other in super-tile order, so
+// the list starts where the counts of all super-tiles before it add up to: the workgroup adds them up itself (a
+// coalesced read of s * NC counts, all requested before the first is used; a scan kernel between the passes cost a
+// launch in a chain of dependent launches, ~10 us, for the same sums; a row split over several workgroups repeats
+// this read and measured slower), then scans its own row of counts.  l1_super[s] receives the start of list s and
+// l1_super[S] the end of the last one (both clamped to the capacity, like every store to the list), totals[0] the
+// unclamped number of entries.
+__global__ __launch_bounds__(kWideThreads) void bin_level1_fill_kernel(
+    const float4* __restrict__ bounds, BinGeom g, const int32_t* __restrict__ l1_counts,
+    int32_t* __restrict__ l1_list, float4* __restrict__ l1_bounds, long long l1_capacity,
+    const unsigned long long* __restrict__ l1_masks, const int32_t* __restrict__ super_view,
+    int32_t* __restrict__ l1_super, long long* __restrict__ totals) {
+  __shared__ long long s_part[kWideThreads / 64];
+  __shared__ long long s_start[kWideThreads];
+  const int s = blockIdx.x, S = g.nsx * g.nsy;
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+  const long long n_before = (long long)s * g.NC;
+  // the ballots of the wavefront's first pairs do not depend on where the list starts: requested ahead of the sums
+  constexpr int kAhead = 8;
+  unsigned long long ahead[kAhead];
+#pragma unroll
+  for (int j = 0; j < kAhead; ++j) {
+    const int c = wave + j * (kWideThreads / 64);
+    ahead[j] = (c < g.NC) ? level1_ballots(g, c, s, l1_masks) : 0ull;      // (uniform per wavefront)
+  }
+  // eight 16-byte loads in flight per thread and step.  (The array is 256-byte aligned and its size a multiple of
+  // that: the four ints at a multiple of 4 below n_before all lie inside it; those at or beyond n_before are dropped.)
+  long long acc = 0;
+  for (long long i0 = (long long)t * 4; i0 < n_before; i0 += 8 * 4 * kWideThreads) {
+    int4 v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const long long i = i0 + (long long)u * 4 * kWideThreads;
+      // (a load beyond the end reads the array's first ints instead and is dropped below: a load under a condition
+      // would wait for the one before it)
+      v[u] = *reinterpret_cast<const int4*>(l1_counts + ((i < n_before) ? i : 0));
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const long long i = i0 + (long long)u * 4 * kWideThreads;
+      acc += (i < n_before) ? v[u].x : 0;
+      acc += (i + 1 < n_before) ? v[u].y : 0;
+      acc += (i + 2 < n_before) ? v[u].z : 0;
+      acc += (i + 3 < n_before) ? v[u].w : 0;
+    }
+  }
+  acc = wave_sum(acc);
+  if (lane == 0) s_part[wave] = acc;
+  __syncthreads();
+  long long base = 0;
+#pragma unroll
+  for (int w = 0; w < kWideThreads / 64; ++w) base += s_part[w];
+  const int view = super_view[s];
+  const bool single = view >= 0;
+  const float4* __restrict__ sb = bounds + (size_t)(single ? view : 0) * g.N;
+  const int32_t* __restrict__ row = l1_counts + (size_t)s * g.NC;
+  long long carry = base;
+  for (int c0 = 0; c0 < g.NC; c0 += kWideThreads) {
+    const int own = (c0 + t < g.NC) ? row[c0 + t] : 0;
+    long long incl = own;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const long long up = __shfl_up(incl, d);
+      if (lane >= d) incl += up;
+    }
+    __syncthreads();                                  // (s_part and s_start are free again)
+    if (lane == 63) s_part[wave] = incl;
+    __syncthreads();
+    long long before = carry, pass_total = 0;
+#pragma unroll
+    for (int w = 0; w < kWideThreads / 64; ++w) {
+      const long long n = s_part[w];
+      before += (w < wave) ? n : 0;
+      pass_total += n;
+    }
+    s_start[t] = before + incl - own;
+    __syncthreads();
+    const int here = min(g.NC - c0, kWideThreads);
+    if (c0 == 0) {
+#pragma unroll
+      for (int j = 0; j < kAhead; ++j) {
+        const int k = wave + j * (kWideThreads / 64);
+        if (k < here) level1_fill_pair(k, ahead[j], s_start[k], single, sb, l1_list, l1_bounds, l1_capacity);
+      }
+    }
+    for (int k = wave + (c0 == 0 ? kAhead * (kWideThreads / 64) : 0); k < here; k += kWideThreads / 64)
+      level1_fill_pair(c0 + k, level1_ballots(g, c0 + k, s, l1_masks), s_start[k], single, sb, l1_list, l1_bounds,
+                       l1_capacity);
+    carry += pass_total;
+  }
+  if (t == 0) {
+    l1_super[s] = (int32_t)min(base, l1_capacity);
+    if (s == S - 1) {
+      l1_super[S] = (int32_t)min(carry, l1_capacity);
+      totals[0] = carry;
+    }
+  }
+}
+
 // In-place exclusive scan of data[0..n) by one workgroup; data[n] and *total receive the sum, *largest
 // (if not null) the largest element.  data must be 16-byte aligned.  A pass covers 8 slabs of 4096
 // elements: thread t owns elements 4t..4t+3 of every slab, so all loads and stores are coalesced 16-byte
 // accesses and the 8 loads of a pass are independent (one memory latency per pass, and one pass covers
 // 32768 elements).  Thread sums are scanned with wavefront shuffles, wavefront totals through LDS.
-//
-// Optional guard (asynchronous binning, scan of the tile counts): if the level-1 lists overflowed their scratch
-// (all_totals[0] > l1_capacity) or the sum does not fit the caller's candidate buffer, every offset is written as
-// 0 instead and the guard word all_totals[3] is raised, so that the fill, sort and render kernels queued behind
-// find nothing to read or write; counts_out receives (pairs, longest list, level-1 entries, guard).
-struct ScanGuard {
-  long long* all_totals;     // null: no guard
-  long long* counts_out;
-  long long l1_capacity, cand_capacity;
-};
+// (Only the two-call binning, whose caller sizes the candidate buffer from the total, scans with a kernel of its
+// own; the asynchronous entry points place their lists inside the fill passes.)
 constexpr int kScanSlabs = 8;
 __global__ __launch_bounds__(1024) void exclusive_scan_kernel(int32_t* __restrict__ data, int n,
                                                               long long* __restrict__ total,
-                                                              long long* __restrict__ largest, ScanGuard guard) {
+                                                              long long* __restrict__ largest) {
   __shared__ long long s_wave[kScanSlabs][16];
   __shared__ int s_wmax[16];
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
-  // (requested up front: by the end of the scan it has long arrived)
-  const long long l1_entries = guard.all_totals ? guard.all_totals[0] : 0;
   long long carry = 0;
   int mx = 0;
   for (int pass0 = 0; pass0 < n; pass0 += kScanSlabs * 4096) {
@@ -566,80 +688,54 @@ __global__ __launch_bounds__(1024) void exclusive_scan_kernel(int32_t* __restric
   for (int d = 1; d < 64; d <<= 1) mx = max(mx, __shfl_xor(mx, d));
   if (lane == 0) s_wmax[wave] = mx;
   __syncthreads();
-  const bool bad = guard.all_totals && (l1_entries > guard.l1_capacity || carry > guard.cand_capacity);
-  if (bad)                                         // (the scan's own stores are behind the barriers above)
-    for (int i = t; i < n; i += 1024) data[i] = 0;
   if (t == 0) {
     int all_max = 0;
     for (int w = 0; w < 16; ++w) all_max = max(all_max, s_wmax[w]);
-    data[n] = bad ? 0 : (int32_t)carry;
+    data[n] = (int32_t)carry;
     *total = carry;
     if (largest) *largest = all_max;
-    if (guard.all_totals) {
-      guard.all_totals[3] = bad ? 1 : 0;
-      guard.counts_out[0] = carry;
-      guard.counts_out[1] = all_max;
-      guard.counts_out[2] = l1_entries;
-      guard.counts_out[3] = bad ? 1 : 0;
-    }
   }
 }
 
-// level 2.  One wavefront per tile, 4 tiles per workgroup.
-template <bool FILL>
-__global__ __launch_bounds__(kBinThreads) void bin_level2_kernel(const float4* __restrict__ bounds, BinGeom g,
-                                                                 const int32_t* __restrict__ tile_view_ids,
-                                                                 const int32_t* __restrict__ l1_offsets,
-                                                                 const int32_t* __restrict__ l1_list,
-                                                                 const float4* __restrict__ l1_bounds,
-                                                                 long long l1_capacity,
-                                                                 int32_t* __restrict__ tile_offsets,
-                                                                 int32_t* __restrict__ cand,
-                                                                 unsigned long long* __restrict__ l2_masks,
-                                                                 long long l2_mask_stride,
-                                                                 const int32_t* __restrict__ super_view,
-                                                                 const long long* __restrict__ skip_flag = nullptr) {
-  const int tile = blockIdx.x * (kBinThreads / 64) + (threadIdx.x >> 6);
-  const int lane = threadIdx.x & 63;
-  if (tile >= g.ntx * g.nty) return;
-  if (FILL && skip_flag && *skip_flag != 0) return;       // the guard emptied the lists: nothing may be written
+// level 2.  One wavefront per tile.  Ballot b of a tile lives at [tile within its super-tile][lo / 64 + s + b]:
+// super-tile lists are consecutive in the level-1 array, so adding s keeps the slots of neighbouring lists apart.
+struct L2Tile {
+  int lo, hi, nb, s, view;
+  float x0, x1, y0, y1;
+  unsigned long long* masks;
+};
+__device__ __forceinline__ L2Tile level2_tile(const BinGeom& g, int tile, const int32_t* __restrict__ tile_view_ids,
+                                              const int32_t* __restrict__ l1_super, long long l1_capacity,
+                                              unsigned long long* __restrict__ l2_masks, long long l2_mask_stride) {
+  L2Tile t;
   const int tx = tile % g.ntx, ty = tile / g.ntx;
-  const int s = (ty / kSuper) * g.nsx + (tx / kSuper);
-  const int view = tile_view_ids ? tile_view_ids[tile] : 0;
-  const float4* __restrict__ vb = bounds + (size_t)view * g.N;
-  const float x0 = (float)(tx * g.ts), x1 = (float)((tx + 1) * g.ts);
-  const float y0 = (float)(ty * g.ts), y1 = (float)((ty + 1) * g.ts);
+  t.s = (ty / kSuper) * g.nsx + (tx / kSuper);
+  t.view = tile_view_ids ? tile_view_ids[tile] : 0;
+  t.x0 = (float)(tx * g.ts);
+  t.x1 = (float)((tx + 1) * g.ts);
+  t.y0 = (float)(ty * g.ts);
+  t.y1 = (float)((ty + 1) * g.ts);
   // clamped so that an overflowed level-1 list (reported to the host) is never read past its end
-  const int lo = (int)min((long long)l1_offsets[s * g.NC], l1_capacity);
-  const int hi = (int)min((long long)l1_offsets[(s + 1) * g.NC], l1_capacity);
-  int running = FILL ? tile_offsets[tile] : 0;
-  // ballot b of this tile lives at [tile within its super-tile][lo / 64 + s + b]: super-tile lists are
-  // consecutive in the level-1 array, so adding s keeps the slots of neighbouring lists apart
-  unsigned long long* __restrict__ masks =
-      l2_masks + (size_t)((ty % kSuper) * kSuper + (tx % kSuper)) * l2_mask_stride + (lo >> 6) + s;
-  const int nb = (hi - lo + 63) >> 6;
-  if constexpr (FILL) {
-    for (int b0 = 0; b0 < nb; b0 += 64) {       // 64 ballots per coalesced load, lane b holds ballot b0 + b
-      const unsigned long long mine = (b0 + lane < nb) ? masks[b0 + lane] : 0ull;
-      const int nhere = min(64, nb - b0);
-      for (int b = 0; b < nhere; b += 8) {      // eight ballots at a time: their id loads are in flight together
-        unsigned long long m[8];
-        int id[8];
-#pragma unroll
-        for (int u = 0; u < 8; ++u) m[u] = (b + u < nhere) ? lane_value(mine, (b + u) & 63) : 0ull;
-#pragma unroll
-        for (int u = 0; u < 8; ++u) id[u] = ((m[u] >> lane) & 1ull) ? l1_list[lo + ((b0 + b + u) << 6) + lane] : 0;
-#pragma unroll
-        for (int u = 0; u < 8; ++u) {
-          if ((m[u] >> lane) & 1ull) cand[running + lanes_below(m[u])] = id[u];
-          running += __popcll(m[u]);
-        }
-      }
-    }
-    return;
-  }
+  t.lo = (int)min((long long)l1_super[t.s], l1_capacity);
+  t.hi = (int)min((long long)l1_super[t.s + 1], l1_capacity);
+  t.hi = max(t.hi, t.lo);
+  t.nb = (t.hi - t.lo + 63) >> 6;
+  t.masks = l2_masks + (size_t)((ty % kSuper) * kSuper + (tx % kSuper)) * l2_mask_stride + (t.lo >> 6) + t.s;
+  return t;
+}
+
+// counting pass of one tile: tests its super-tile's list, keeps the ballots, returns the number of survivors
+__device__ __forceinline__ int level2_count_tile(const L2Tile& t, const BinGeom& g, const float4* __restrict__ bounds,
+                                                 const int32_t* __restrict__ l1_list,
+                                                 const float4* __restrict__ l1_bounds,
+                                                 const int32_t* __restrict__ super_view) {
+  const int lane = threadIdx.x & 63;
+  const int lo = t.lo, hi = t.hi, nb = t.nb;
+  const float x0 = t.x0, x1 = t.x1, y0 = t.y0, y1 = t.y1;
+  unsigned long long* __restrict__ masks = t.masks;
+  int running = 0;
   unsigned long long mine = 0ull;
-  if (super_view[s] == view) {
+  if (super_view[t.s] == t.view) {
     // one view for the super-tile: its bounds sit next to the ids; four independent 16-byte loads in flight per step
     const float nanv = __builtin_nanf("");
     for (int b = 0; b < nb; b += 4) {
@@ -659,25 +755,179 @@ __global__ __launch_bounds__(kBinThreads) void bin_level2_kernel(const float4* _
         }
       }
     }
-    if ((nb & 63) != 0 && lane < (nb & 63)) masks[(nb & ~63) + lane] = mine;
-    if (lane == 0) tile_offsets[tile] = running;
-    return;
-  }
-  for (int base = lo, b = 0; base < hi; base += 64, ++b) {
-    const int j = base + lane;
-    int id = -1;
-    bool keep = false;
-    if (j < hi) {
-      id = l1_list[j];
-      keep = rect_overlap(vb[id], x0, x1, y0, y1);
+  } else {
+    const float4* __restrict__ vb = bounds + (size_t)t.view * g.N;
+    for (int base = lo, b = 0; base < hi; base += 64, ++b) {
+      const int j = base + lane;
+      bool keep = false;
+      if (j < hi) keep = rect_overlap(vb[l1_list[j]], x0, x1, y0, y1);
+      const unsigned long long m = __ballot(keep);
+      mine = (lane == (b & 63)) ? m : mine;
+      if ((b & 63) == 63) masks[b - 63 + lane] = mine;       // 64 ballots at a time, one coalesced store
+      running += __popcll(m);
     }
-    const unsigned long long m = __ballot(keep);
-    mine = (lane == (b & 63)) ? m : mine;
-    if ((b & 63) == 63) masks[b - 63 + lane] = mine;       // 64 ballots at a time, one coalesced store
-    running += __popcll(m);
   }
   if ((nb & 63) != 0 && lane < (nb & 63)) masks[(nb & ~63) + lane] = mine;
-  if (lane == 0) tile_offsets[tile] = running;
+  return running;
+}
+
+// fill pass of one tile: its survivors' ids, from the ballots, to cand[running...]
+// (first: the tile's first 64 ballots, lane b holding ballot b -- the caller requests them ahead of time)
+__device__ __forceinline__ unsigned long long level2_first_ballots(const L2Tile& t) {
+  const int lane = threadIdx.x & 63;
+  return (lane < t.nb) ? t.masks[lane] : 0ull;
+}
+__device__ __forceinline__ void level2_fill_tile(const L2Tile& t, unsigned long long first,
+                                                 const int32_t* __restrict__ l1_list, int32_t* __restrict__ cand,
+                                                 int running) {
+  const int lane = threadIdx.x & 63;
+  const int lo = t.lo, nb = t.nb;
+  const unsigned long long* __restrict__ masks = t.masks;
+  for (int b0 = 0; b0 < nb; b0 += 64) {         // 64 ballots per coalesced load, lane b holds ballot b0 + b
+    const unsigned long long mine = (b0 == 0) ? first : (b0 + lane < nb) ? masks[b0 + lane] : 0ull;
+    const int nhere = min(64, nb - b0);
+    for (int b = 0; b < nhere; b += 8) {        // eight ballots at a time: their id loads are in flight together
+      unsigned long long m[8];
+      int id[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) m[u] = (b + u < nhere) ? lane_value(mine, (b + u) & 63) : 0ull;
+#pragma unroll
+      for (int u = 0; u < 8; ++u) id[u] = ((m[u] >> lane) & 1ull) ? l1_list[lo + ((b0 + b + u) << 6) + lane] : 0;
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        if ((m[u] >> lane) & 1ull) cand[running + lanes_below(m[u])] = id[u];
+        running += __popcll(m[u]);
+      }
+    }
+  }
+}
+
+// level 2, counting pass: 16 tiles per workgroup.  tile_counts[tile] = survivors, groups[workgroup] = their sum and
+// the longest of the 16 lists.
+__global__ __launch_bounds__(kWideThreads) void bin_level2_count_kernel(
+    const float4* __restrict__ bounds, BinGeom g, const int32_t* __restrict__ tile_view_ids,
+    const int32_t* __restrict__ l1_super, const int32_t* __restrict__ l1_list, const float4* __restrict__ l1_bounds,
+    long long l1_capacity, int32_t* __restrict__ tile_counts, unsigned long long* __restrict__ l2_masks,
+    long long l2_mask_stride, const int32_t* __restrict__ super_view, L2Group* __restrict__ groups) {
+  __shared__ int s_cnt[kL2Group];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int tile = blockIdx.x * kL2Group + wave;
+  int count = 0;
+  if (tile < g.ntx * g.nty) {
+    const L2Tile t = level2_tile(g, tile, tile_view_ids, l1_super, l1_capacity, l2_masks, l2_mask_stride);
+    count = level2_count_tile(t, g, bounds, l1_list, l1_bounds, super_view);
+    if (lane == 0) tile_counts[tile] = count;
+  }
+  if (lane == 0) s_cnt[wave] = count;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    L2Group grp;
+    grp.sum = 0;
+    grp.longest = 0;
+    grp.pad = 0;
+#pragma unroll
+    for (int w = 0; w < kL2Group; ++w) {
+      grp.sum += s_cnt[w];
+      grp.longest = max(grp.longest, s_cnt[w]);
+    }
+    groups[blockIdx.x] = grp;
+  }
+}
+
+// level 2, fill pass: the same 16 tiles per workgroup.
+// OWN_PREFIX = false: tile_offsets holds the exclusive offsets (the caller scanned the counts).
+// OWN_PREFIX = true: tile_offsets holds the counts, and the workgroup places its tiles itself -- it adds up the
+// groups before its own (a few KB that are L2 hits, instead of a scan kernel between the passes), every workgroup
+// also forms the total and applies the guard of the asynchronous entry points: if the level-1 lists overflowed their
+// scratch (totals[0] > l1_capacity) or the total does not fit the caller's candidate buffer, every offset is written
+// as 0, nothing is filled and the guard word totals[3] is raised, so that the sort and render kernels queued behind
+// find nothing to read or write; counts_out receives (pairs, longest list, level-1 entries, guard).  A workgroup
+// reads only its own tiles' counts before it overwrites them with offsets.
+struct FillGuard {
+  long long* totals;
+  long long* counts_out;
+  long long l1_capacity, cand_capacity;
+};
+template <bool OWN_PREFIX>
+__global__ __launch_bounds__(kWideThreads) void bin_level2_fill_kernel(
+    BinGeom g, const int32_t* __restrict__ tile_view_ids, const int32_t* __restrict__ l1_super,
+    const int32_t* __restrict__ l1_list, long long l1_capacity, int32_t* __restrict__ tile_offsets,
+    int32_t* __restrict__ cand, unsigned long long* __restrict__ l2_masks, long long l2_mask_stride,
+    const L2Group* __restrict__ groups, int num_groups, FillGuard guard) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int T = g.ntx * g.nty;
+  const int tile = blockIdx.x * kL2Group + wave;
+  int running = 0;
+  // (what does not depend on the tile's place is requested first: the list bounds, the first ballots)
+  L2Tile tl = {};
+  unsigned long long first = 0ull;
+  if (tile < T) {
+    tl = level2_tile(g, tile, tile_view_ids, l1_super, l1_capacity, l2_masks, l2_mask_stride);
+    first = level2_first_ballots(tl);
+  }
+  if constexpr (OWN_PREFIX) {
+    __shared__ long long s_before[kL2Group], s_total[kL2Group];
+    __shared__ int s_longest[kL2Group], s_cnt[kL2Group];
+    const long long l1_entries = guard.totals[0];      // (requested up front)
+    long long before = 0, total = 0;
+    int longest = 0;
+    for (int k0 = threadIdx.x; k0 < num_groups; k0 += 4 * kWideThreads) {      // four loads in flight
+      L2Group v[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int k = k0 + u * kWideThreads;
+        v[u] = groups[(k < num_groups) ? k : 0];      // (unconditional, so that the four do not wait for each other)
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int k = k0 + u * kWideThreads;
+        total += (k < num_groups) ? v[u].sum : 0;
+        before += (k < (int)blockIdx.x) ? v[u].sum : 0;
+        longest = max(longest, (k < num_groups) ? v[u].longest : 0);
+      }
+    }
+    const int own = (tile < T) ? tile_offsets[tile] : 0;
+    before = wave_sum(before);
+    total = wave_sum(total);
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) longest = max(longest, __shfl_xor(longest, d));
+    if (lane == 0) {
+      s_before[wave] = before;
+      s_total[wave] = total;
+      s_longest[wave] = longest;
+      s_cnt[wave] = own;
+    }
+    __syncthreads();
+    before = 0;
+    total = 0;
+    longest = 0;
+#pragma unroll
+    for (int w = 0; w < kL2Group; ++w) {
+      before += s_before[w] + ((w < wave) ? s_cnt[w] : 0);
+      total += s_total[w];
+      longest = max(longest, s_longest[w]);
+    }
+    const bool bad = l1_entries > guard.l1_capacity || total > guard.cand_capacity;
+    if (lane == 0) {
+      if (tile < T) tile_offsets[tile] = bad ? 0 : (int32_t)before;
+      if (tile == T - 1) tile_offsets[T] = bad ? 0 : (int32_t)total;
+    }
+    if (blockIdx.x == 0 && threadIdx.x == 0) {
+      guard.totals[1] = total;
+      guard.totals[2] = longest;
+      guard.totals[3] = bad ? 1 : 0;
+      guard.counts_out[0] = total;
+      guard.counts_out[1] = longest;
+      guard.counts_out[2] = l1_entries;
+      guard.counts_out[3] = bad ? 1 : 0;
+    }
+    if (bad || tile >= T) return;
+    running = (int)before;
+  } else {
+    if (tile >= T) return;
+    running = tile_offsets[tile];
+  }
+  level2_fill_tile(tl, first, l1_list, cand, running);
 }
 
 inline BinGeom make_geom(int N, int K, int W, int H, int ts) {
@@ -701,6 +951,7 @@ MLPSP_API size_t mlpsp_bin_scratch_bytes(int num_primitives, int num_views, int 
                  align256((size_t)num_views * num_primitives * sizeof(float4)) +
                  align256((S * g.NC + 1) * sizeof(int32_t)) + 256;
   bytes += align256(S * g.NC * (kChunk / 64) * sizeof(unsigned long long)) + align256(S * sizeof(int32_t));
+  bytes += align256((S + 1) * sizeof(int32_t)) + align256((S * (64 / kL2Group) + 1) * sizeof(L2Group));
   bytes += 1024 + align256((S + 1) * 64 * sizeof(unsigned long long));
   // room for every primitive to touch 8 super-tiles per view, plus slack for tiny scenes; per entry the id,
   // the bounds and the 64 survivor bits of the super-tile's tiles
@@ -740,6 +991,8 @@ int allow_scatter_lds() {
   return MLPSP_OK;
 }
 
+inline int level2_groups(int64_t T) { return (int)((T + kL2Group - 1) / kL2Group); }
+
 // what the bounds of a frame are computed from (bin_bounds_kernel's arguments)
 struct BoundsSource {
   const float* positions;
@@ -751,9 +1004,9 @@ struct BoundsSource {
   float rm, focal;
 };
 
-// bounds -> level 1 (count, scan, fill) -> level 2 count -> scan
+// bounds -> level 1 (count, fill) -> level 2 count [-> scan of the tile counts when the caller fills separately]
 int enqueue_bin_levels(const BoundsSource& src, const BinGeom& g, const BinScratch& b, int64_t T,
-                       const int32_t* tile_view_ids_dev, int32_t* tile_offsets_dev, hipStream_t s, ScanGuard guard) {
+                       const int32_t* tile_view_ids_dev, int32_t* tile_offsets_dev, hipStream_t s, bool scan_tiles) {
   const int S = g.nsx * g.nsy;
   // level-1 counts by primitive (super-tile rows in bands that fit LDS): with one view the same launch computes the
   // bounds, with several (and tile_view_ids) it reads them
@@ -788,36 +1041,44 @@ int enqueue_bin_levels(const BoundsSource& src, const BinGeom& g, const BinScrat
     else MLPSP_SCATTER(2);
 #undef MLPSP_SCATTER
   } else {
-    hipLaunchKernelGGL((bin_level1_kernel<false>), dim3(g.NC, ceil_div(S, kBinThreads / 64)), dim3(kBinThreads), 0, s,
-                       b.bounds, g, tile_view_ids_dev, b.l1_counts, b.l1_list, b.l1_bounds, b.l1_capacity, b.l1_masks,
-                       b.super_view);
+    hipLaunchKernelGGL(bin_level1_kernel, dim3(g.NC, ceil_div(S, kBinThreads / 64)), dim3(kBinThreads), 0, s, b.bounds, g,
+                       tile_view_ids_dev, b.l1_counts, b.l1_masks, b.super_view);
   }
   MLPSP_LAUNCH_CHECK();
-  hipLaunchKernelGGL(exclusive_scan_kernel, dim3(1), dim3(1024), 0, s, b.l1_counts, S * g.NC, b.totals,
-                     (long long*)nullptr, ScanGuard{nullptr, nullptr, 0, 0});
+  hipLaunchKernelGGL(bin_level1_fill_kernel, dim3(S), dim3(kWideThreads), 0, s, b.bounds, g, b.l1_counts, b.l1_list,
+                     b.l1_bounds, b.l1_capacity, b.l1_masks, b.super_view, b.l1_super, b.totals);
   MLPSP_LAUNCH_CHECK();
-  hipLaunchKernelGGL((bin_level1_kernel<true>), dim3(g.NC, ceil_div(S, kBinThreads / 64)), dim3(kBinThreads), 0, s,
-                     b.bounds, g, tile_view_ids_dev, b.l1_counts, b.l1_list, b.l1_bounds, b.l1_capacity, b.l1_masks,
-                     b.super_view);
+  hipLaunchKernelGGL(bin_level2_count_kernel, dim3(level2_groups(T)), dim3(kWideThreads), 0, s, b.bounds, g,
+                     tile_view_ids_dev, b.l1_super, b.l1_list, b.l1_bounds, b.l1_capacity, tile_offsets_dev, b.l2_masks,
+                     b.l2_mask_stride, b.super_view, b.groups);
   MLPSP_LAUNCH_CHECK();
-  hipLaunchKernelGGL((bin_level2_kernel<false>), dim3(ceil_div((int)T, kBinThreads / 64)), dim3(kBinThreads), 0, s,
-                     b.bounds, g, tile_view_ids_dev, b.l1_counts, b.l1_list, b.l1_bounds, b.l1_capacity, tile_offsets_dev,
-                     (int32_t*)nullptr, b.l2_masks, b.l2_mask_stride, b.super_view);
-  MLPSP_LAUNCH_CHECK();
-  hipLaunchKernelGGL(exclusive_scan_kernel, dim3(1), dim3(1024), 0, s, tile_offsets_dev, (int)T, b.totals + 1,
-                     b.totals + 2, guard);
-  MLPSP_LAUNCH_CHECK();
+  if (scan_tiles) {
+    hipLaunchKernelGGL(exclusive_scan_kernel, dim3(1), dim3(1024), 0, s, tile_offsets_dev, (int)T, b.totals + 1,
+                       b.totals + 2);
+    MLPSP_LAUNCH_CHECK();
+  }
   return MLPSP_OK;
 }
 
-// Enqueues bounds -> level 1 (count, scan, fill) -> level 2 count -> scan.  Leaves the exclusive tile offsets in
-// tile_offsets_dev and (level-1 entries, pairs, longest tile list) in b.totals[0..2]; no host synchronisation.
+// the fill pass of the asynchronous entry points: places the tiles, applies the guard, writes the lists
+void enqueue_guarded_fill(const BinGeom& g, const BinScratch& b, int64_t T, const int32_t* tile_view_ids_dev,
+                          int32_t* tile_offsets_dev, int32_t* candidates_dev, int64_t cand_capacity, int64_t* counts_dev,
+                          hipStream_t s) {
+  hipLaunchKernelGGL((bin_level2_fill_kernel<true>), dim3(level2_groups(T)), dim3(kWideThreads), 0, s, g,
+                     tile_view_ids_dev, b.l1_super, b.l1_list, b.l1_capacity, tile_offsets_dev, candidates_dev, b.l2_masks,
+                     b.l2_mask_stride, b.groups, level2_groups(T),
+                     FillGuard{b.totals, (long long*)counts_dev, b.l1_capacity, (long long)cand_capacity});
+}
+
+// Enqueues bounds -> level 1 (count, fill) -> level 2 count, no host synchronisation.  With scan_tiles also the
+// scan of the tile counts: exclusive tile offsets in tile_offsets_dev and (level-1 entries, pairs, longest tile
+// list) in b.totals[0..2].  Without, tile_offsets_dev holds the counts for enqueue_guarded_fill().
 int enqueue_bin_count(const float* positions_dev, const float* log_scales_dev, int num_primitives,
                       const float* view_matrices_host, int num_views, const int32_t* tile_view_ids_dev,
                       const float* proj_host, int width, int height, int tile, float threshold, const BinGeom& g,
                       const BinScratch& b, int64_t T, int32_t* tile_offsets_dev, hipStream_t s,
-                      bool matrices_in_scratch = false, ScanGuard guard = ScanGuard{nullptr, nullptr, 0, 0},
-                      const float* view_dev = nullptr, const float* proj_dev = nullptr) {
+                      bool matrices_in_scratch = false, bool scan_tiles = true, const float* view_dev = nullptr,
+                      const float* proj_dev = nullptr) {
   BoundsSource src{};
   src.positions = positions_dev;
   src.log_scales = log_scales_dev;
@@ -827,7 +1088,7 @@ int enqueue_bin_count(const float* positions_dev, const float* log_scales_dev, i
     src.mode = 2;
     src.mats = view_dev;
     src.proj_dev = proj_dev;
-    return enqueue_bin_levels(src, g, b, T, tile_view_ids_dev, tile_offsets_dev, s, guard);
+    return enqueue_bin_levels(src, g, b, T, tile_view_ids_dev, tile_offsets_dev, s, scan_tiles);
   }
   const float fx = (proj_host[0] * (float)width) / 2.0f, fy = (proj_host[5] * (float)height) / 2.0f;
   src.focal = (fx + fy) * 0.5f;
@@ -847,7 +1108,7 @@ int enqueue_bin_count(const float* positions_dev, const float* log_scales_dev, i
                                    hipMemcpyHostToDevice, s));
     }
   }
-  return enqueue_bin_levels(src, g, b, T, tile_view_ids_dev, tile_offsets_dev, s, guard);
+  return enqueue_bin_levels(src, g, b, T, tile_view_ids_dev, tile_offsets_dev, s, scan_tiles);
 }
 
 int check_bin_args(int64_t T, const float* view_matrices_host, const float* proj_host, void* scratch_dev,
@@ -922,13 +1183,9 @@ int bin_legacy_async_impl(const float* positions_dev, const float* log_scales_de
   }
   const int erc = enqueue_bin_count(positions_dev, log_scales_dev, num_primitives, view_matrices_host, num_views,
                                     tile_view_ids_dev, proj_host, width, height, tile, threshold, g, b, T,
-                                    tile_offsets_dev, s, false,
-                                    ScanGuard{b.totals, (long long*)counts_dev, b.l1_capacity, (long long)cand_capacity},
-                                    view_dev, proj_dev);
+                                    tile_offsets_dev, s, false, /*scan_tiles=*/false, view_dev, proj_dev);
   if (erc != MLPSP_OK) return erc;
-  hipLaunchKernelGGL((bin_level2_kernel<true>), dim3(ceil_div((int)T, kBinThreads / 64)), dim3(kBinThreads), 0, s,
-                     b.bounds, g, tile_view_ids_dev, b.l1_counts, b.l1_list, b.l1_bounds, b.l1_capacity, tile_offsets_dev,
-                     candidates_dev, b.l2_masks, b.l2_mask_stride, b.super_view, (const long long*)(b.totals + 3));
+  enqueue_guarded_fill(g, b, T, tile_view_ids_dev, tile_offsets_dev, candidates_dev, cand_capacity, counts_dev, s);
   MLPSP_LAUNCH_CHECK();
   return MLPSP_OK;
 }
@@ -968,9 +1225,10 @@ MLPSP_API int mlpsp_bin_legacy_fill(int num_primitives, int num_views, const int
   if (!candidates_dev) return MLPSP_E_ARGUMENT;
   const BinGeom g = make_geom(num_primitives, num_views, width, height, tile);
   const BinScratch b = carve(const_cast<void*>(scratch_dev), scratch_bytes, num_primitives, num_views, g.nsx * g.nsy, g.NC);
-  hipLaunchKernelGGL((bin_level2_kernel<true>), dim3(ceil_div((int)T, kBinThreads / 64)), dim3(kBinThreads), 0,
-                     (hipStream_t)stream, b.bounds, g, tile_view_ids_dev, b.l1_counts, b.l1_list, b.l1_bounds, b.l1_capacity,
-                     const_cast<int32_t*>(tile_offsets_dev), candidates_dev, b.l2_masks, b.l2_mask_stride, b.super_view);
+  hipLaunchKernelGGL((bin_level2_fill_kernel<false>), dim3(level2_groups(T)), dim3(kWideThreads), 0, (hipStream_t)stream,
+                     g, tile_view_ids_dev, b.l1_super, b.l1_list, b.l1_capacity, const_cast<int32_t*>(tile_offsets_dev),
+                     candidates_dev, b.l2_masks, b.l2_mask_stride, b.groups, level2_groups(T),
+                     FillGuard{nullptr, nullptr, 0, 0});
   MLPSP_LAUNCH_CHECK();
   return MLPSP_OK;
 }
@@ -1069,12 +1327,9 @@ MLPSP_API int mlpsp_bin_legacy_async_noalloc(const float* positions_dev, const f
   }
   const int erc = enqueue_bin_count(positions_dev, log_scales_dev, num_primitives, view_matrices_host, num_views,
                                     tile_view_ids_dev, proj_host, width, height, tile, threshold, g, b, T,
-                                    tile_offsets_dev, s, /*matrices_in_scratch=*/true,
-                                    ScanGuard{b.totals, (long long*)counts_dev, b.l1_capacity, (long long)cand_capacity});
+                                    tile_offsets_dev, s, /*matrices_in_scratch=*/true, /*scan_tiles=*/false);
   if (erc != MLPSP_OK) return erc;
-  hipLaunchKernelGGL((bin_level2_kernel<true>), dim3(ceil_div((int)T, kBinThreads / 64)), dim3(kBinThreads), 0, s,
-                     b.bounds, g, tile_view_ids_dev, b.l1_counts, b.l1_list, b.l1_bounds, b.l1_capacity, tile_offsets_dev,
-                     candidates_dev, b.l2_masks, b.l2_mask_stride, b.super_view, (const long long*)(b.totals + 3));
+  enqueue_guarded_fill(g, b, T, tile_view_ids_dev, tile_offsets_dev, candidates_dev, cand_capacity, counts_dev, s);
   MLPSP_LAUNCH_CHECK();
   return MLPSP_OK;
 }
