@@ -25,8 +25,9 @@ def measured_traffic(kernel: str, workload: str, ms_per_launch: float):
     """HBM bytes per launch of `kernel` from the committed hardware-counter profile profiles/<kernel>_<workload>.txt
     (two rocprofv3 --pmc runs, FETCH_SIZE and WRITE_SIZE, each scaled by what the counter reads for a device copy of
     known size; the file states the commands).  The profile carries the kernel's average duration when the counters
-    were taken: if this run's duration differs from it by more than 10 %, the kernel is no longer the one that was
-    profiled and no traffic figure is reported.  -> (bytes or None, note)"""
+    were taken: if this run's duration differs from it by more than 15 % (boxes of this pool run one build up to 9 %
+    apart), the kernel is no longer the one that was profiled and no traffic figure is reported.
+    -> (bytes or None, note)"""
     import re
     path = os.path.join(PROFILES, f"{kernel}_{workload}.txt")
     if not os.path.exists(path):
@@ -36,7 +37,7 @@ def measured_traffic(kernel: str, workload: str, ms_per_launch: float):
     if not all(got.values()):
         return None, f"{os.path.basename(path)} holds no bench.traffic_bytes / bench.kernel_avg_us lines"
     traffic, avg_us = float(got["traffic_bytes"].group(1)), float(got["kernel_avg_us"].group(1))
-    if abs(ms_per_launch * 1e3 - avg_us) > 0.10 * avg_us:
+    if abs(ms_per_launch * 1e3 - avg_us) > 0.15 * avg_us:
         return None, (f"profiled kernel took {avg_us:.1f} us, this run {ms_per_launch * 1e3:.1f} us: "
                       f"{os.path.basename(path)} is stale")
     return int(traffic), f"profiles/{os.path.basename(path)} (kernel {avg_us:.1f} us when profiled)"

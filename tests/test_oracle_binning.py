@@ -204,3 +204,23 @@ def test_headline_scene_fits_the_tile_capacity_and_the_unshifted_one_does_not(or
     cand, off = oracle_mod.bin_legacy(raw.positions, raw.log_scales, syn.view_matrix(poses[0])[None], P, W, H, 8, thr)
     status = oracle_mod.validate(off, cand, off.size - 1, 1536, 200000)
     assert status[0] == 2 and status[1] > 1536
+
+
+def test_mosaic_scene_fits_the_tile_capacity_and_a_tenth_larger_does_not(oracle_mod):
+    """The clustered 200k scene of the four-view mosaic: log-scale mean -6.0 is the largest in steps of 0.1 whose
+    fullest tile over the eight calls stays within the 1,536 capacity (1,535); at -5.9 the first call overflows."""
+    W, H, f, thr = 2400, 1360, 600.0, 5e-3
+    P = syn.projection_matrix(f, W, H)
+    cams = syn.random_poses(32, 0)
+    fit = syn.make_scene(200000, 1, 0, syn.LOG_SCALE_MEAN_200K_CLUSTERED, cluster_frac=0.3)
+    worst = 0
+    for g0 in range(0, 32, 4):
+        _, _, tv, views = syn.mosaic_frame(W // 2, H // 2, f, cams[g0:g0 + 4])
+        _, off = oracle_mod.bin_legacy(fit.positions, fit.log_scales, views, P, W, H, 8, thr, tile_view_ids=tv)
+        worst = max(worst, int(np.diff(off).max()))
+    assert worst == 1535
+    larger = syn.make_scene(200000, 1, 0, syn.LOG_SCALE_MEAN_200K_CLUSTERED + 0.1, cluster_frac=0.3)
+    _, _, tv, views = syn.mosaic_frame(W // 2, H // 2, f, cams[0:4])
+    cand, off = oracle_mod.bin_legacy(larger.positions, larger.log_scales, views, P, W, H, 8, thr, tile_view_ids=tv)
+    status = oracle_mod.validate(off, cand, off.size - 1, 1536, 200000)
+    assert status[0] == 2 and status[1] == 1672
