@@ -173,6 +173,34 @@ def test_overflow_falls_back_to_f32_for_the_whole_frame(device, oracle_mod):
         ext.render_tiles_rgb_wmma(x, fr.W, fr.H, fr.thr, True)
 
 
+def test_hit_offsets_beyond_the_sincos_table_range_fall_back_to_f32(device, oracle_mod):
+    # the bf16 path takes the position half of the encoding from a table that is exact for up to 500 periods of the
+    # highest frequency (2^5 pi: 31 scene units of |dx| + |dy| + |dz|); a primitive 60 units across that the rays
+    # pass 40 units off its centre is beyond it -> flag -> the frame comes from the f32 kernel, bit for bit.
+    # fp16 operands use the sin/cos instructions and render the same frame themselves.
+    from mlp_splatting_amd.tile_ext import TileExt
+    fr = Frame("cfg1_5k_160x120", n=64, hidden=32, width=32, height=24)
+    sc = fr.scene
+    ahead = fr.rays_d[(fr.H // 2) * fr.W + fr.W // 2]
+    side = np.cross(ahead, [0.0, 1.0, 0.0])
+    sc.positions[0] = fr.rays_o[0] + 10.0 * ahead + 40.0 * side / np.linalg.norm(side)
+    sc.log_scales[0] = np.log(60.0)
+    cand, off = fr.oracle_lists(oracle_mod)
+    assert (cand == 0).sum() == (fr.W // 8) * (fr.H // 8)          # the large primitive is on every tile's list
+    ext = TileExt()
+    x = [to_dev(a, device) for a in fr.base_numpy(cand, off)]
+    calls0, fb0 = ext.rgb_wmma_safety_stats()
+    with pytest.warns(UserWarning, match="scalar FP32 instead"):
+        rgb, alpha = ext.render_tiles_rgb_wmma(x, fr.W, fr.H, fr.thr, True)
+    want = ext.render_tiles_forward_tilecenter(*x, fr.W, fr.H, 8, 8, fr.thr)
+    assert torch.equal(rgb, want[0]) and torch.equal(alpha, want[1])
+    assert float(alpha.max()) > 0.0
+    assert ext.rgb_wmma_safety_stats() == [calls0 + 1, fb0 + 1]
+    rgb_h, alpha_h = ext.render_tiles_rgb_wmma(x, fr.W, fr.H, fr.thr, False)
+    assert ext.rgb_wmma_safety_stats() == [calls0 + 2, fb0 + 1]
+    assert float((rgb_h - want[0]).abs().max()) <= TOL[False]
+
+
 def test_packed_weights_are_cached_until_a_tensor_changes(device, oracle_mod):
     from mlp_splatting_amd.tile_ext import TileExt
     fr = Frame("cfg1_5k_160x120", n=300, hidden=32, width=24, height=16)
