@@ -216,6 +216,8 @@ class Workload:
             self.skipped_poses = len(frames) - len(fitting)
             frames = fitting
         self.frames = frames
+        # the 4x4 view matrix a caller of forward() holds (one tensor per pose, made once)
+        self.view_of = [None if f[3] is not None else f[2][0] for f in frames]
 
     def render(self, i):
         import torch
@@ -225,8 +227,8 @@ class Workload:
             if tv is not None:
                 cand, off = scene.build_tilecenter_culling_from_tile_views(tv, views, self.proj, self.thr)
                 return scene(ro, rd, score_threshold=self.thr, culled_prim_indices=cand, tile_offsets=off)
-            out = scene(ro, rd, score_threshold=self.thr, view_matrix=views[0], proj_matrix=self.proj,
-                        return_feature=bool(self.feature_dim))
+            out = scene(ro, rd, score_threshold=self.thr, view_matrix=self.view_of[i % len(self.frames)],
+                        proj_matrix=self.proj, return_feature=bool(self.feature_dim))
             return out[0] if self.feature_dim else out
 
     def timed(self, steps, warmup, wake_seconds, min_seconds):

@@ -30,18 +30,52 @@ _tile_error = None
 _tile_ext_key = None
 
 
+# The environment is read on every call, as the reference does (a test or a caller may change it between two frames);
+# these reads sit between the end of one frame and the first launch of the next, where the device waits for the
+# host.  CPython keeps the encoded environment in a plain dict behind os.environ: reading that dict costs a tenth of
+# os.environ.get (no key encoding, no default handling in Python code).
+_ENV_DATA = getattr(os.environ, "_data", None)
+_ENV_KEYS = {}
+
+
+def _env(name: str, default: str) -> str:
+    data = _ENV_DATA
+    if type(data) is dict and os.name == "posix":
+        key = _ENV_KEYS.get(name)
+        if key is None:
+            key = _ENV_KEYS[name] = os.fsencode(name)
+        value = data.get(key)
+        return default if value is None else os.fsdecode(value)
+    return os.environ.get(name, default)
+
+
+_BUILD_CONFIGS = {}
+
+
 def _tile_ext_build_config(tile_size=None):
     """(key, name, flags) naming the extension build selected by the environment
     (scannet/cumodel.py:96-130).  The capacities the reference bakes in at compile time are run-time
     arguments of this library, but names, accepted values and errors are kept."""
-    rreg = os.environ.get("MLPSP_NVCC_MAXRREGCOUNT", "").strip()
+    raw = (_env("MLPSP_NVCC_MAXRREGCOUNT", ""), _env("MLPSP_TILE_CANDIDATE_CAPACITY", "1536"),
+           _env("MLPSP_TRAINING_BACKEND", "legacy"), _env("MLPSP_CSR_MAX_HITS", "128"))
+    known = _BUILD_CONFIGS.get(raw)
+    if known is not None:
+        return known[0], known[1], list(known[2])
+    config = _tile_ext_build_config_of(*raw)
+    if len(_BUILD_CONFIGS) < 64:
+        _BUILD_CONFIGS[raw] = (config[0], config[1], tuple(config[2]))
+    return config
+
+
+def _tile_ext_build_config_of(rreg, capacity, backend, csr_hits):
+    rreg = rreg.strip()
     flags = []
     suffix = "default"
-    capacity = int(os.environ.get("MLPSP_TILE_CANDIDATE_CAPACITY", "1536"))
+    capacity = int(capacity)
     if capacity not in {768, 1536}:
         raise ValueError("MLPSP_TILE_CANDIDATE_CAPACITY must be 768 or 1536")
-    if os.environ.get("MLPSP_TRAINING_BACKEND", "legacy") == "csr":
-        hits = int(os.environ.get("MLPSP_CSR_MAX_HITS", "128"))
+    if backend == "csr":
+        hits = int(csr_hits)
         if hits not in {128, 256, 512}:
             raise ValueError("MLPSP_CSR_MAX_HITS must be 128, 256 or 512; overflow is an error")
         flags += ["-DMLPSP_TILECENTER_BLOCK_THREADS=64", "-DMLPSP_BACKWARD_RECOMPUTE_GEOMETRY=1",
@@ -494,7 +528,9 @@ class NeuralPrimitiveSceneTileCUDA(nn.Module):
     def _resolve_tile_order_mode(self) -> str:
         mode = self.tile_order_mode_override
         if mode is None or str(mode).strip() == "":
-            mode = os.environ.get("MLPSP_TILE_ORDER", "tilecenter")
+            mode = _env("MLPSP_TILE_ORDER", "tilecenter")
+        if mode == "tilecenter":
+            return mode
         mode = str(mode).strip().lower()
         mode = {"tile_center": "tilecenter", "tile-center": "tilecenter"}.get(mode, mode)
         if mode not in {"tilecenter", "per_pixel"}:
@@ -687,12 +723,15 @@ class NeuralPrimitiveSceneTileCUDA(nn.Module):
         with torch.no_grad():
             use_tilecenter = self._resolve_tile_order_mode() == "tilecenter"
             ext = self._ensure_tile_ext()
+            # (plain attributes live in the module's __dict__; getattr with a default on a module that lacks the name
+            # walks parameters, buffers and submodules first)
+            plain = self.__dict__
             own_lists = (culled_prim_indices is None and tile_offsets is None and view_matrix is not None
                          and proj_matrix is not None
-                         and getattr(self, "camera_mode", "legacy-centered") != "colmap-native")
+                         and plain.get("camera_mode", "legacy-centered") != "colmap-native")
             with_feat = return_feature and self.feat_attr is not None
             if (own_lists and use_tilecenter and ts == 8 and (with_feat or not return_feature)
-                    and feature_target is None and getattr(self, "queued_frames", True)
+                    and feature_target is None and plain.get("queued_frames", True)
                     and hasattr(ext, "render_frame_queued")):
                 done = self._forward_queued(ext, ray_o, ray_d, score_threshold, view_matrix, proj_matrix, bg_color,
                                             device, with_feat)
@@ -832,13 +871,24 @@ class NeuralPrimitiveSceneTileCUDA(nn.Module):
             precision = "f32"
         if with_feat and precision == "f32":
             return None                       # the exact feature frame goes step by step
-        params = (self.W1, self.b1, self.W2, self.b2, self.W3, self.b3)
-        if any(w.dtype != torch.float32 for w in params):
+        # (up to the binning call below the device waits for the host: parameters are taken from the module's own
+        # table, which a plain attribute read reaches only after a failed instance look-up)
+        registered = self._parameters
+        try:
+            params = (registered["W1"], registered["b1"], registered["W2"], registered["b2"], registered["W3"],
+                      registered["b3"])
+            positions, log_scales = registered["positions"], registered["log_scales"]
+        except KeyError:
+            params = (self.W1, self.b1, self.W2, self.b2, self.W3, self.b3)
+            positions, log_scales = self.positions, self.log_scales
+        f32 = torch.float32
+        if not (params[0].dtype == f32 and params[1].dtype == f32 and params[2].dtype == f32 and params[3].dtype == f32
+                and params[4].dtype == f32 and params[5].dtype == f32):
             half = all(w.dtype == torch.float16 for w in params)
             if not (half and precision != "f32"):
                 return None                   # stored half-precision weights: only the matrix-core frame reads them as they are
         W, H = self.image_size
-        positions, log_scales = self.positions.detach().contiguous(), self.log_scales.detach().contiguous()
+        positions, log_scales = positions.detach().contiguous(), log_scales.detach().contiguous()
         views, proj = _frame_matrix(view_matrix).reshape(1, 4, 4), _frame_matrix(proj_matrix)
         binned = None
         if hasattr(ext, "frame_binning_queued"):
@@ -850,7 +900,7 @@ class NeuralPrimitiveSceneTileCUDA(nn.Module):
         ray_o = ray_o.contiguous()
         if (hasattr(ext, "frame_prologue") and ray_d.is_cuda and ray_d.dtype == torch.float32 and ray_d.dim() == 2
                 and ray_d.shape[1] == 3 and not ray_d.requires_grad and ray_o.dtype == torch.float32
-                and ray_o.shape == ray_d.shape and os.environ.get("MLPSP_SORT_FRAME_RECORDS", "0") == "1"):
+                and ray_o.shape == ray_d.shape and _env("MLPSP_SORT_FRAME_RECORDS", "0") == "1"):
             # unit directions and the sort's per-frame records in one launch (opt-in: measured 6 us per frame slower
             # than the full key evaluation on one MI355X, where the sort is not bound by vector instructions)
             unit_dirs, more["frame_records"] = ext.frame_prologue(ray_o, ray_d, positions, log_scales, self._unit_quats())
