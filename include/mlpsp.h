@@ -56,7 +56,7 @@ typedef void* mlpsp_stream_t;
 /* Library version (major*10000 + minor*100 + patch).  MLPSP_VERSION is the version this header describes: a caller
  * built against it must find mlpsp_version() == MLPSP_VERSION (argument lists and the PrimRecord layout are not
  * compatible across versions). */
-#define MLPSP_VERSION 300
+#define MLPSP_VERSION 301
 int mlpsp_version(void);
 
 /* Message for one MLPSP_E_* bit, worded as the reference's TORCH_CHECK for that condition
@@ -386,7 +386,11 @@ int mlpsp_render_tilecenter_mfma(const float* rays_o_dev, const float* rays_d_de
  * 256-byte aligned.
  * stage: 0 = the whole frame; 1 = the render launch alone (RGB, alpha and the coefficient records in the workspace);
  * 2 = the feature product alone, over the records a stage-1 call with the same arguments left in the same workspace
- * (for timing the two launches apart; 1 and 2 need feat_slots != 0). */
+ * (for timing the two launches apart; 1 and 2 need feat_slots != 0).  MLPSP_STAGE_STATUS_IS_CLEAR may be or-ed in:
+ * the caller vouches that the 16 words at status_dev are zero already (it read them back as zero after the previous
+ * call on this buffer), and the call queues no clear of them -- one launch less between the sort and the render
+ * of a frame. */
+#define MLPSP_STAGE_STATUS_IS_CLEAR 4
 size_t mlpsp_mfma_feat_pack_bytes(int num_primitives, int feat_slots, int feat_channels);
 int mlpsp_pack_mfma_feat(const float* feat_attr_dev, int num_primitives, int feat_slots, int feat_channels,
                          void* packed_feat_dev, int32_t* status_dev, mlpsp_stream_t stream);

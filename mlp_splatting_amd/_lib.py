@@ -20,7 +20,8 @@ TILE_CAPACITY_MAX = 2048
 PIXEL_HIT_CAPACITY = 256
 PRIM_RECORD_BYTES = 128
 MFMA_PACK_BYTES = 7808
-VERSION = 300      # MLPSP_VERSION of include/mlpsp.h: the interface this binding was written against
+VERSION = 301      # MLPSP_VERSION of include/mlpsp.h: the interface this binding was written against
+STAGE_STATUS_IS_CLEAR = 4
 
 _vp, _i, _f, _i64, _sz = C.c_void_p, C.c_int, C.c_float, C.c_int64, C.c_size_t
 

@@ -887,7 +887,10 @@ MLPSP_API int mlpsp_render_tilecenter_mfma_feat(const float* rays_o_dev, const f
                                                 float* out_alpha_dev, float* out_feat_dev, int32_t* status_dev,
                                                 int64_t* counters_dev, int stage, mlpsp_stream_t stream) {
   const int64_t T = checked_num_tiles(width, height, 8, 8);
-  if (stage < 0 || stage > 2 || (stage != 0 && feat_slots == 0)) return MLPSP_E_ARGUMENT;
+  if (stage < 0 || (stage & ~(3 | MLPSP_STAGE_STATUS_IS_CLEAR)) != 0) return MLPSP_E_ARGUMENT;
+  const bool status_is_clear = (stage & MLPSP_STAGE_STATUS_IS_CLEAR) != 0;
+  stage &= 3;
+  if (stage > 2 || (stage != 0 && feat_slots == 0)) return MLPSP_E_ARGUMENT;
   if (T <= 0 || T > 2147483647LL - 8 || num_primitives < 0 || num_pairs < 0 || num_pairs > 2147483647LL)
     return MLPSP_E_ARGUMENT;
   if (!rays_o_dev || !rays_d_dev || !tile_offsets_dev || !freq_dev || !att_dev || !out_rgb_dev || !out_alpha_dev ||
@@ -906,7 +909,7 @@ MLPSP_API int mlpsp_render_tilecenter_mfma_feat(const float* rays_o_dev, const f
     hp = hitpool_carve(workspace_dev, workspace_bytes, num_pairs, T, 1, 64 * 2 * feat_pad(feat_slots));
     if (stage != 2) MLPSP_HIP_TRY(hipMemsetAsync(hp.counters, 0, 64 * sizeof(int32_t), s));
   }
-  if (stage != 2) MLPSP_HIP_TRY(hipMemsetAsync(status_dev, 0, 16 * sizeof(int32_t), s));
+  if (stage != 2 && !status_is_clear) MLPSP_HIP_TRY(hipMemsetAsync(status_dev, 0, 16 * sizeof(int32_t), s));
   const int per_xcd = (int)((T + kNumXcd - 1) / kNumXcd);
   const int ntx = ceil_div(width, 8);
   const dim3 grid(superblock_grid(ntx, ceil_div(height, 8)));

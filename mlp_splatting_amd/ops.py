@@ -532,11 +532,14 @@ def pack_mfma_weights(W1, b1, W2, b2, W3, b3, bf16=True):
 
 
 def render_tilecenter_mfma(rays_o, rays_d, records, order, tile_offsets, freq, att, W1, b1, W2, b2, W3, b3, W, H,
-                           threshold, bf16=True, counters=None, packed=None, check=True, status=None):
+                           threshold, bf16=True, counters=None, packed=None, check=True, status=None,
+                           status_is_clear=False):
     """Matrix-core tile-centre forward (8x8 tiles) -> (rgb, alpha, nonfinite).
 
     ``nonfinite`` is a bool when ``check`` (one 4-byte readback) or the int32 device flag otherwise.  ``status``: an
     int32 [16] device tensor for the flag words (word 0 = non-finite), allocated here when omitted.
+    ``status_is_clear``: the caller read all 16 words of ``status`` back as zero after the previous call that used
+    it, so no clear is queued in front of the kernel.
     """
     dev = rays_o.device
     if freq.numel() != 6:
@@ -549,10 +552,17 @@ def render_tilecenter_mfma(rays_o, rays_d, records, order, tile_offsets, freq, a
     flag = status if status is not None else torch.empty(16, dtype=torch.int32, device=dev)
     if not (flag.is_cuda and flag.dtype == torch.int32 and flag.numel() == 16 and flag.is_contiguous()):
         raise ValueError("status must be a contiguous int32 [16] tensor on the device")
-    code = _lib.load().mlpsp_render_tilecenter_mfma(
-        _ptr(rays_o), _ptr(rays_d), _ptr(records), _ptr(order), _ptr(tile_offsets), _ptr(freq), _ptr(att), _ptr(packed),
-        W1.shape[0], int(bool(bf16)), W, H, float(threshold), _ptr(rgb), _ptr(alpha), _ptr(flag), _ptr(counters),
-        _stream(dev))
+    if status_is_clear and status is not None:
+        # (the RGB entry point is the feature entry point without features; only that one takes the stage word)
+        code = _lib.load().mlpsp_render_tilecenter_mfma_feat(
+            _ptr(rays_o), _ptr(rays_d), _ptr(records), _ptr(order), _ptr(tile_offsets), 0, _ptr(freq), _ptr(att),
+            _ptr(packed), W1.shape[0], int(bool(bf16)), None, 0, 0, 0.0, 0.0, W, H, float(threshold), None, 0, _ptr(rgb),
+            _ptr(alpha), None, _ptr(flag), _ptr(counters), _lib.STAGE_STATUS_IS_CLEAR, _stream(dev))
+    else:
+        code = _lib.load().mlpsp_render_tilecenter_mfma(
+            _ptr(rays_o), _ptr(rays_d), _ptr(records), _ptr(order), _ptr(tile_offsets), _ptr(freq), _ptr(att),
+            _ptr(packed), W1.shape[0], int(bool(bf16)), W, H, float(threshold), _ptr(rgb), _ptr(alpha), _ptr(flag),
+            _ptr(counters), _stream(dev))
     _check(code, "mlpsp_render_tilecenter_mfma")
     return rgb, alpha, (bool(flag[0].item()) if check else flag)
 
@@ -573,7 +583,7 @@ def pack_mfma_feat(feat_attr):
 
 def render_tilecenter_mfma_feat(rays_o, rays_d, records, order, tile_offsets, freq, att, W1, b1, W2, b2, W3, b3,
                                 feat_attr, beta, temp, W, H, threshold, bf16=True, packed=None, packed_feat=None,
-                                check=True, status=None, counters=None, stages=None):
+                                check=True, status=None, counters=None, stages=None, status_is_clear=False):
     """Matrix-core tile-centre forward with the gated feature channel -> (rgb, alpha, feat, nonfinite).
     ``packed_feat`` is the result of :func:`pack_mfma_feat` for ``feat_attr`` (built here when omitted;
     non-finite rounded attributes raise).  ``status`` (an int32 [16] device tensor): ONE attempt with the first
@@ -582,7 +592,7 @@ def render_tilecenter_mfma_feat(rays_o, rays_d, records, order, tile_offsets, fr
     ``counters``: int64 [4] work counters of the render launch, accumulated.  ``stages``: a callable
     ``stages(which)`` invoked before the render launch (1), before the feature product (2) and after it (3) -- the
     two launches are then queued by separate calls, with the worst-case record pool, so that a caller can bracket
-    each with events."""
+    each with events.  ``status_is_clear``: as in :func:`render_tilecenter_mfma` (with ``status`` only)."""
     dev = rays_o.device
     if freq.numel() != 6:
         raise RuntimeError("the matrix-core path supports 6 frequencies only")
@@ -603,12 +613,13 @@ def render_tilecenter_mfma_feat(rays_o, rays_d, records, order, tile_offsets, fr
                                    and status.is_contiguous()):
         raise ValueError("status must be a contiguous int32 [16] tensor on the device")
     flag = status if status is not None else torch.empty(16, dtype=torch.int32, device=dev)
+    clear_bit = _lib.STAGE_STATUS_IS_CLEAR if (status_is_clear and status is not None and stages is None) else 0
     def launch(workspace, ws_bytes, stage):
         code = lib.mlpsp_render_tilecenter_mfma_feat(
             _ptr(rays_o), _ptr(rays_d), _ptr(records), _ptr(order), _ptr(tile_offsets), pairs, _ptr(freq), _ptr(att),
             _ptr(packed), W1.shape[0], int(bool(bf16)), _ptr(packed_feat), slots, ch, float(beta), float(temp), W, H,
             float(threshold), _ptr(workspace), ws_bytes, _ptr(rgb), _ptr(alpha), _ptr(feat), _ptr(flag), _ptr(counters),
-            stage, _stream(dev))
+            stage | clear_bit, _stream(dev))
         _check(code, "mlpsp_render_tilecenter_mfma_feat")
         return code
 

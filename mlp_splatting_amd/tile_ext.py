@@ -39,6 +39,9 @@ def _is_f32_2d(t, cols):
 
 
 
+_SIXTEEN_ZERO_WORDS = bytes(64)
+
+
 def _on_device(device):
     """``torch.cuda.device(device)``, or nothing when that device is current already (saves two device switches)."""
     if device.index is None or torch.cuda.current_device() == device.index:
@@ -329,11 +332,12 @@ class TileExt:
             if "tail" not in held:
                 fresh = torch.empty(96, dtype=torch.uint8, device=positions.device)
                 held["tail"] = (fresh, fresh[:32].view(torch.int64))
+                held["flags_clear"] = False
             tail, counts_view = held["tail"]
             cand, offsets, counts = ops.bin_legacy_async(positions, log_scales, view_matrices, proj_matrix, int(width),
                                                          int(height), 8, float(threshold), cap, scratch_scale=scale,
                                                          counts=counts_view, reuse=held)
-        return cand, offsets, counts, tail, cap, scale
+        return cand, offsets, counts, tail, cap, scale, held
 
     def _frame_buffers(self, device):
         """The reusable buffers of queued frames, per (thread, device, stream)."""
@@ -382,8 +386,13 @@ class TileExt:
                                                threshold)
             if binned is None:
                 return None
-        cand, offsets, counts, tail, cap, scale = binned
+        cand, offsets, counts, tail, cap, scale, held = binned
         status = tail[32:].view(torch.int32)
+        # The flag words live in a buffer that this thread's frames use one after the other, and every frame ends by
+        # reading them back: if the last frame read sixteen zeros they are still zero, and the render's own clear (a
+        # launch between the sort and the render) is left out.  The mark is taken down while a frame is under way.
+        flags_clear = held.get("flags_clear", False) and held.get("tail", (None,))[0] is tail
+        held["flags_clear"] = False
         n = positions.shape[0]
         with _on_device(rays_o.device):
             rec = self._records(positions, log_scales, unit_quats)
@@ -395,15 +404,18 @@ class TileExt:
                 if feat is None:
                     rgb, alpha, _ = ops.render_tilecenter_mfma(rays_o, unit_dirs, rec, order, offsets, freq, att, *ws,
                                                                width, height, threshold, bf16=(precision == "bf16"),
-                                                               packed=packed, check=False, status=status)
+                                                               packed=packed, check=False, status=status,
+                                                               status_is_clear=flags_clear)
                 else:
                     packed_feat, bad_attr = self._packed_feat(feat[0])
                     if bad_attr:
                         return None
                     rgb, alpha, fmap, _ = ops.render_tilecenter_mfma_feat(
                         rays_o, unit_dirs, rec, order, offsets, freq, att, *ws, feat[0], feat[1], feat[2], width, height,
-                        threshold, bf16=(precision == "bf16"), packed=packed, packed_feat=packed_feat, status=status)
+                        threshold, bf16=(precision == "bf16"), packed=packed, packed_feat=packed_feat, status=status,
+                        status_is_clear=flags_clear)
                 host = tail.cpu().numpy()
+                held["flags_clear"] = host[32:].tobytes() == _SIXTEEN_ZERO_WORDS
                 pairs, longest, l1_entries, guard = (int(v) for v in host[:32].view("int64"))
                 nonfinite = int(host[32:36].view("int32")[0])
                 pool_ran_out = int(host[36:40].view("int32")[0]) if feat is not None else 0

@@ -314,6 +314,40 @@ def test_queued_frames_equal_step_by_step_frames(device, oracle_mod, monkeypatch
         _call(scene, fr, device)
 
 
+def test_a_flag_raised_by_one_queued_frame_does_not_reach_the_next(device, oracle_mod, monkeypatch):
+    # Queued frames of a thread share their flag words and skip the clear while the last read-back showed zeros.
+    # A frame that raises the non-finite flag (fp16 cannot hold 1e5) is rendered by the f32 kernel; the frame after
+    # it, with the weight back in range, must come from the matrix cores again, unflagged.
+    import warnings
+    from mlp_splatting_amd import cumodel
+    from mlp_splatting_amd.tile_ext import TileExt
+    fr = Frame("cfg1_5k_160x120", n=1500, hidden=32, width=64, height=48)
+    monkeypatch.setattr(cumodel, "_tile_ext", TileExt())
+    scene = _scene_from(fr, device)
+    scene.render_precision = "fp16"
+    ext = cumodel._tile_ext
+    _call(scene, fr, device)                             # seeds the candidate-buffer estimate
+    clean = _call(scene, fr, device)
+    again = _call(scene, fr, device)                     # (this one ran without the clear)
+    held = ext._frame_buffers(device)
+    assert torch.equal(again, clean) and held["flags_clear"] is True
+    cand, _ = fr.oracle_lists(oracle_mod)
+    with torch.no_grad():
+        kept = scene.W2[int(cand[0]), 3, 5].item()
+        scene.W2[int(cand[0]), 3, 5] = 1.0e5
+    calls0, fb0 = ext.rgb_wmma_safety_stats()
+    with pytest.warns(UserWarning, match="scalar FP32 instead"):
+        flagged = _call(scene, fr, device)
+    assert held["flags_clear"] is False and ext.rgb_wmma_safety_stats() == [calls0 + 1, fb0 + 1]
+    with torch.no_grad():
+        scene.W2[int(cand[0]), 3, 5] = kept
+    with warnings.catch_warnings():
+        warnings.simplefilter("error")
+        after = _call(scene, fr, device)
+    assert torch.equal(after, clean) and not torch.equal(flagged, clean)
+    assert ext.rgb_wmma_safety_stats() == [calls0 + 2, fb0 + 1] and held["flags_clear"] is True
+
+
 def test_harness_renders_times_and_scores_a_view(device, oracle_mod):
     """mlp_splatting_amd.harness: the timed view of tools/benchmark_inference.py:121-149, its statistics, PSNR and
     the RGB parity of the feature render, on a frame whose image the oracle pins."""
