@@ -279,10 +279,12 @@ class Workload:
         # the event brackets would be timed as kernel time), the second is measured
         for i in list(range(n_probe)) * 2:
             if i == 0:
-                acc = dict(bin_ms=0.0, sort_ms=0.0, render_ms=0.0, product_ms=0.0, hits=0, proc=0, hit_waves=0, cand=0)
+                acc = dict(bin_ms=0.0, prologue_ms=0.0, sort_ms=0.0, render_ms=0.0, product_ms=0.0, hits=0, proc=0,
+                           hit_waves=0, cand=0)
             ro, rd_raw, views, tv = self.frames[i]
             rd = torch.nn.functional.normalize(rd_raw, dim=-1).contiguous()
-            e = [torch.cuda.Event(enable_timing=True) for _ in range(5)]
+            e = [torch.cuda.Event(enable_timing=True) for _ in range(6)]
+            flags = torch.zeros(16, dtype=torch.int32, device=dev)     # (a queued frame finds its flag words clear)
             rec = ops.prepare_primitives(scene.positions.detach(), scene.log_scales.detach(), quats)
             cand, off = ops.bin_legacy(scene.positions.detach(), scene.log_scales.detach(), views, self.proj, W, H, 8, thr,
                                        tile_view_ids=tv)
@@ -291,23 +293,29 @@ class Workload:
             ops.bin_legacy_async(scene.positions.detach(), scene.log_scales.detach(), views, self.proj, W, H, 8, thr,
                                  cand.numel(), tile_view_ids=tv)
             e[1].record()
-            order, _ = ops.sort_tiles(ro, rd, rec, cand, off, W, H, 8, 8, cull_threshold=thr)
+            pyramids = None
+            if tv is None:
+                # unit directions and the tiles' ray pyramids in one launch, as a frame of the scene module queues them
+                # (lists handed in by a caller, the mosaic's, are rendered with torch's unit directions)
+                rd, pyramids, _ = ops.frame_prologue(ro, rd_raw, W, H)
             e[2].record()
+            order, _ = ops.sort_tiles(ro, rd, rec, cand, off, W, H, 8, 8, cull_threshold=thr, tile_pyramids=pyramids)
+            e[3].record()
             counters = torch.zeros(4, dtype=torch.int64, device=dev)
             if feat is not None:
                 # render with coefficient records, then the feature product, as two calls
-                marks = {2: e[3], 3: e[4]}
+                marks = {2: e[4], 3: e[5]}
                 ops.render_tilecenter_mfma_feat(ro, rd, rec, order, off, freq, att, *weights, feat,
                                                 float(scene.feature_gating_beta), float(scene.feature_gating_temp), W, H,
                                                 thr, bf16=True, packed=packed, packed_feat=packed_feat, check=False,
                                                 stages=lambda k: marks[k].record() if k in marks else None)
             elif precision == "bf16":
                 ops.render_tilecenter_mfma(ro, rd, rec, order, off, freq, att, *weights, W, H, thr, bf16=True,
-                                           packed=packed, check=False)
-                e[3].record()
+                                           packed=packed, check=False, status=flags, status_is_clear=tv is None)
+                e[4].record()
             else:
                 ops.render_tilecenter_f32(ro, rd, rec, order, off, freq, att, *weights, W, H, 8, 8, thr)
-                e[3].record()
+                e[4].record()
             torch.cuda.synchronize()
             # the same render launch once more, untimed, for its work counters (their atomics are not part of a frame)
             if precision == "bf16":
@@ -317,10 +325,11 @@ class Workload:
                 ops.render_tilecenter_f32(ro, rd, rec, order, off, freq, att, *weights, W, H, 8, 8, thr, counters=counters)
             torch.cuda.synchronize()
             acc["bin_ms"] += e[0].elapsed_time(e[1])
-            acc["sort_ms"] += e[1].elapsed_time(e[2])
-            acc["render_ms"] += e[2].elapsed_time(e[3])
+            acc["prologue_ms"] += e[1].elapsed_time(e[2])
+            acc["sort_ms"] += e[2].elapsed_time(e[3])
+            acc["render_ms"] += e[3].elapsed_time(e[4])
             if feat is not None:
-                acc["product_ms"] += e[3].elapsed_time(e[4])
+                acc["product_ms"] += e[4].elapsed_time(e[5])
             c = counters.cpu().numpy()
             acc["hits"] += int(c[3])
             acc["proc"] += int(c[1])
@@ -351,7 +360,8 @@ def other_workload(name, args, dev):
     traffic, note = measured_traffic(kernel, name, st["render_ms"])
     out = {"fps": round(fps, 2), "ms_per_step": round(1e3 * elapsed / steps, 4), "steps": steps, "dtype": wl.precision,
            "views_per_call": 4 if wl.mosaic else 1, "feature_channels": wl.feature_dim, "poses": cycle,
-           "stages": {k: round(st[k], 4) for k in ("bin_ms", "sort_ms", "render_ms") + (("product_ms",) if wl.feature_dim else ())},
+           "stages": {k: round(st[k], 4) for k in ("bin_ms", "prologue_ms", "sort_ms", "render_ms") +
+                      (("product_ms",) if wl.feature_dim else ())},
            "hits_per_launch": int(st["hits"]), "hit_wavefronts_per_launch": int(st["hit_waves"])}
     if wl.mosaic:
         # 17 of a tile's 64 pixels hit per step here: the launch is bound by the weight blocks it streams, one
@@ -542,8 +552,8 @@ def main() -> int:
                      "tile_primitives_per_launch": proc // n_probe,
                      "hit_wavefronts_per_launch": hit_waves // n_probe, "flops_per_hit": flops_per_hit,
                      "measured_mfma_peak": mfma_probe, "issue_probe": issue_probe},
-        "stages": {"bin_ms": round(bin_ms / n_probe, 4), "sort_ms": round(sort_ms / n_probe, 4),
-                   "render_ms": round(kernel_ms / n_probe, 4),
+        "stages": {"bin_ms": round(bin_ms / n_probe, 4), "prologue_ms": round(st["prologue_ms"], 4),
+                   "sort_ms": round(sort_ms / n_probe, 4), "render_ms": round(kernel_ms / n_probe, 4),
                    "sort_hbm": {"bound": "hbm", "achieved": round(sort_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                                 "frac": round(sort_gbs / HBM_PEAK_GBS, 5),
                                 "achieved_at_48B_per_candidate": round(sort_gbs_per_candidate, 1),

@@ -44,6 +44,7 @@ extern "C" {
 #define MLPSP_PRIM_RECORD_BYTES 128  /* bytes per primitive of the prepared geometry buffer */
 #define MLPSP_MFMA_PACK_BYTES 7808   /* bytes per primitive of the packed matrix-core weight buffer */
 #define MLPSP_SORT_RECORD_BYTES 64   /* bytes per primitive (+ one header slot) of the sort's per-frame records */
+#define MLPSP_TILE_PYRAMID_BYTES 160 /* bytes per tile of the sort's ray-pyramid records */
 #define MLPSP_BIN_STATIC_SCRATCH_BYTES 67108864 /* scratch array of mlpsp_bin_legacy_async_noalloc (64 MiB) */
 #define MLPSP_BIN_STATIC_MAX_VIEWS 8           /* most views mlpsp_bin_legacy_async_noalloc accepts */
 
@@ -56,7 +57,7 @@ typedef void* mlpsp_stream_t;
 /* Library version (major*10000 + minor*100 + patch).  MLPSP_VERSION is the version this header describes: a caller
  * built against it must find mlpsp_version() == MLPSP_VERSION (argument lists and the PrimRecord layout are not
  * compatible across versions). */
-#define MLPSP_VERSION 301
+#define MLPSP_VERSION 302
 int mlpsp_version(void);
 
 /* Message for one MLPSP_E_* bit, worded as the reference's TORCH_CHECK for that condition
@@ -173,19 +174,28 @@ int mlpsp_bin_raycone_fill(int num_primitives, int width, int height, int tile, 
  * (one quaternion rotation per candidate instead of two; same expressions, same key bits); other tiles, and every
  * tile without the scratch, evaluate the key in full.  Sorted ids and keys do not depend on it.
  * frame_records_ready != 0: the records are there already -- mlpsp_frame_prologue wrote them, for these rays and
- * these primitive records, earlier on the same stream -- and no launch is added. */
+ * these primitive records, earlier on the same stream -- and no launch is added.
+ * tile_pyramids_dev: NULL, or the mlpsp_tile_pyramids_bytes() bytes that mlpsp_frame_prologue wrote for these rays
+ * and this tile size earlier on the same stream (32-byte aligned): the four side planes of every tile's rays, which
+ * the culling tests candidates against.  Without them every wavefront of a tile builds the planes from the tile's
+ * 64 rays itself.  Keys and order do not depend on it; the two builds of the planes differ in their last bits, so a
+ * candidate on the very edge of the culling's margin may be struck by one and not the other (the images are the
+ * same: nothing that hits is ever struck). */
 size_t mlpsp_sort_frame_records_bytes(int num_primitives);
-/* The per-frame preparations that need nothing but the rays, in ONE launch: the unit directions of
- * mlpsp_normalize_rays and the sort's frame records (for the origin of ray 0).  No counterpart in the reference,
- * which normalises with torch (scannet/cumodel.py:1088) and evaluates the whole key per candidate. */
-int mlpsp_frame_prologue(const float* rays_d_dev, long long num_rays, float* unit_dirs_dev, const float* rays_o_dev,
-                         const void* prim_records_dev, int num_primitives, void* frame_records_dev,
-                         mlpsp_stream_t stream);
+size_t mlpsp_tile_pyramids_bytes(int width, int height, int tile_w, int tile_h);
+/* The per-frame preparations that need nothing but the rays (and the scene), in ONE launch: the unit directions of
+ * mlpsp_normalize_rays for the width * height rays at rays_d_dev; with tile_pyramids_dev != NULL the sort's ray
+ * pyramid of every tile (formed from the directions as given; needs rays_o_dev); with frame_records_dev != NULL the sort's frame records for the origin of ray 0 (needs rays_o_dev and
+ * the primitive records).  No counterpart in the reference, which normalises with torch (scannet/cumodel.py:1088)
+ * and runs the full ray test on every candidate. */
+int mlpsp_frame_prologue(const float* rays_d_dev, float* unit_dirs_dev, const float* rays_o_dev, int width, int height,
+                         int tile_w, int tile_h, void* tile_pyramids_dev, const void* prim_records_dev,
+                         int num_primitives, void* frame_records_dev, mlpsp_stream_t stream);
 int mlpsp_sort_tiles(const float* rays_o_dev, const float* rays_d_dev, const void* prim_records_dev,
                      int num_primitives, const int32_t* candidates_dev, const int32_t* tile_offsets_dev, int width,
                      int height, int tile_w, int tile_h, int key_family, int capacity, float cull_threshold,
-                     void* frame_records_dev, int frame_records_ready, int32_t* sorted_ids_dev,
-                     float* sorted_keys_dev, mlpsp_stream_t stream);
+                     void* frame_records_dev, int frame_records_ready, const void* tile_pyramids_dev,
+                     int32_t* sorted_ids_dev, float* sorted_keys_dev, mlpsp_stream_t stream);
 
 /* Tile-centre-order forward, scalar f32 (render_tiles_kernel_tilecenter_order,
  * np_tile_kernels.cu:1837-2137; with out_t_dev != NULL also the expected depth of :5432-5719).

@@ -20,7 +20,7 @@ TILE_CAPACITY_MAX = 2048
 PIXEL_HIT_CAPACITY = 256
 PRIM_RECORD_BYTES = 128
 MFMA_PACK_BYTES = 7808
-VERSION = 301      # MLPSP_VERSION of include/mlpsp.h: the interface this binding was written against
+VERSION = 302      # MLPSP_VERSION of include/mlpsp.h: the interface this binding was written against
 STAGE_STATUS_IS_CLEAR = 4
 
 _vp, _i, _f, _i64, _sz = C.c_void_p, C.c_int, C.c_float, C.c_int64, C.c_size_t
@@ -47,8 +47,9 @@ SIGNATURES = {
     "mlpsp_bin_raycone_count": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _f, _vp, _sz, _vp, C.POINTER(_i64), _vp]),
     "mlpsp_bin_raycone_fill": (_i, [_i, _i, _i, _i, _vp, _sz, _vp, _vp, _vp]),
     "mlpsp_sort_frame_records_bytes": (_sz, [_i]),
-    "mlpsp_frame_prologue": (_i, [_vp, C.c_longlong, _vp, _vp, _vp, _i, _vp, _vp]),
-    "mlpsp_sort_tiles": (_i, [_vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _vp, _i, _vp, _vp, _vp]),
+    "mlpsp_tile_pyramids_bytes": (_sz, [_i, _i, _i, _i]),
+    "mlpsp_frame_prologue": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _vp, _vp, _i, _vp, _vp]),
+    "mlpsp_sort_tiles": (_i, [_vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _vp, _i, _vp, _vp, _vp, _vp]),
     "mlpsp_render_tilecenter_f32": (_i, [_vp] * 7 + [_i] + [_vp] * 6 + [_i, _i, _i, _i, _i, _i, _f, _vp, _vp, _vp,
                                                                        _vp, _vp]),
     "mlpsp_render_tilecenter_feat_f32": (_i, [_vp] * 7 + [_i] + [_vp] * 6 + [_i, _i, _vp, _i, _i, _f, _f, _i, _i, _i, _i,

@@ -235,6 +235,16 @@ __device__ __forceinline__ float blend_step(PixelAcc& a, float o0, float o1, flo
 struct TileGeom {
   int W, H, TW, TH, ntx, nty;
 };
+
+// torch.nn.functional.normalize(d, dim=-1) of one direction, bit for bit (scannet/cumodel.py:1088): the squares are
+// summed as (x^2 + z^2) + y^2 -- the order of torch's reduction over a last dimension of three -- then an exactly
+// rounded square root and three exactly rounded divisions.
+__device__ __forceinline__ void unit_direction(float x, float y, float z, float& ux, float& uy, float& uz) {
+  const float den = fmaxf(sqrtf((x * x + z * z) + y * y), 1e-12f);
+  ux = x / den;
+  uy = y / den;
+  uz = z / den;
+}
 __device__ __forceinline__ int centre_pixel(const TileGeom& g, int tile) {
   const int tx = tile % g.ntx, ty = tile / g.ntx;
   const int cx = min(tx * g.TW + (g.TW >> 1), g.W - 1);

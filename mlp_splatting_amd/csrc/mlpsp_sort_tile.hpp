@@ -163,11 +163,46 @@ struct TilePyramid {
 __device__ __forceinline__ float lane_value(float v, int lane) {
   return bits_to_float((uint32_t)__builtin_amdgcn_readlane((int)float_to_bits(v), lane));
 }
+// How tile_pyramid() reads the direction of a pixel's ray: unit vectors as stored, or directions as the caller
+// holds them, normalised on the way (the frame prologue runs beside the kernel that writes the unit vectors).  The
+// pyramid only needs directions of about unit length, so that its tolerances mean what they say: a reciprocal square
+// root and three products, not the exactly rounded square root and divisions of the unit vectors the renderer uses
+// (four of those per lane were three quarters of the prologue's pyramid work).  The planes then differ from those
+// built from the stored unit vectors in their last bits; the culling has a 2 % margin either way.
+// (a ray's three floats as one 12-byte load: the rays of a tile lie 12 bytes apart over several image rows, and what
+// these reads cost is the number of load instructions)
+struct __attribute__((packed, aligned(4))) Float3 {
+  float x, y, z;
+};
+__device__ __forceinline__ Float3 load3(const float* __restrict__ base, int pix) {
+  return *reinterpret_cast<const Float3*>(base + (size_t)pix * 3);
+}
+struct UnitDirs {
+  const float* __restrict__ d;
+  __device__ __forceinline__ void get(int pix, float& x, float& y, float& z) const {
+    const Float3 v = load3(d, pix);
+    x = v.x;
+    y = v.y;
+    z = v.z;
+  }
+};
+struct RawDirs {
+  const float* __restrict__ d;
+  __device__ __forceinline__ void get(int pix, float& x, float& y, float& z) const {
+    const Float3 v = load3(d, pix);
+    const float r = __builtin_amdgcn_rsqf(fmaxf((v.x * v.x + v.z * v.z) + v.y * v.y, 1e-24f));
+    x = v.x * r;
+    y = v.y * r;
+    z = v.z * r;
+  }
+};
+
 // Called by a whole wavefront: lane l builds face l % 4 (face j from corner rays j and j + 1), then every lane
 // checks rays of the tile (all of them between the 64 lanes) against the four faces and the common origin.  A face
 // the centre ray (nearly) lies in, or that some ray of the tile is outside of, is not used; without a common origin
 // none is.  The roundings here are free: the per-candidate test has a 2 % margin.
-__device__ __forceinline__ TilePyramid tile_pyramid(const float* __restrict__ rays_o, const float* __restrict__ rays_d,
+template <typename Dirs>
+__device__ __forceinline__ TilePyramid tile_pyramid(const float* __restrict__ rays_o, const Dirs dirs,
                                                     const TileGeom& g, int tile, float dx, float dy, float dz) {
   const int lane = threadIdx.x & 63;
   const int tx = tile % g.ntx, ty = tile / g.ntx;
@@ -177,13 +212,15 @@ __device__ __forceinline__ TilePyramid tile_pyramid(const float* __restrict__ ra
   // corners in the order (x0,y0) (x1,y0) (x1,y1) (x0,y1)
   const int ca = ((j >> 1) ? y1 : y0) * g.W + ((j == 1 || j == 2) ? x1 : x0);
   const int cb = ((j1 >> 1) ? y1 : y0) * g.W + ((j1 == 1 || j1 == 2) ? x1 : x0);
-  const float a0 = rays_d[ca * 3], a1 = rays_d[ca * 3 + 1], a2 = rays_d[ca * 3 + 2];
-  const float b0 = rays_d[cb * 3], b1 = rays_d[cb * 3 + 1], b2 = rays_d[cb * 3 + 2];
+  float a0, a1, a2, b0, b1, b2;
+  dirs.get(ca, a0, a1, a2);
+  dirs.get(cb, b0, b1, b2);
   const int c0 = y0 * g.W + x0;
   TilePyramid py;
-  py.ox = rays_o[c0 * 3];
-  py.oy = rays_o[c0 * 3 + 1];
-  py.oz = rays_o[c0 * 3 + 2];
+  const Float3 origin = load3(rays_o, c0);
+  py.ox = origin.x;
+  py.oy = origin.y;
+  py.oz = origin.z;
   float nx = a1 * b2 - a2 * b1, ny = a2 * b0 - a0 * b2, nz = a0 * b1 - a1 * b0;
   const float side = nx * dx + ny * dy + nz * dz;
   const float len = __builtin_amdgcn_sqrtf(nx * nx + ny * ny + nz * nz);
@@ -209,8 +246,10 @@ __device__ __forceinline__ TilePyramid tile_pyramid(const float* __restrict__ ra
     const int x = x0 + k % g.TW, y = y0 + k / g.TW;
     if (x < g.W && y < g.H) {
       const int pix = y * g.W + x;
-      if (rays_o[pix * 3] != py.ox || rays_o[pix * 3 + 1] != py.oy || rays_o[pix * 3 + 2] != py.oz) ok &= ~0x10;
-      const float rx = rays_d[pix * 3], ry = rays_d[pix * 3 + 1], rz = rays_d[pix * 3 + 2];
+      const Float3 o = load3(rays_o, pix);
+      if (o.x != py.ox || o.y != py.oy || o.z != py.oz) ok &= ~0x10;
+      float rx, ry, rz;
+      dirs.get(pix, rx, ry, rz);
 #pragma unroll
       for (int f = 0; f < 4; ++f) {
         const float inside = py.n[f][0] * rx + py.n[f][1] * ry + py.n[f][2] * rz;
@@ -222,6 +261,65 @@ __device__ __forceinline__ TilePyramid tile_pyramid(const float* __restrict__ ra
 #pragma unroll
   for (int b = 0; b < 5; ++b) all_ok |= __ballot(!((ok >> b) & 1)) ? 0 : (1 << b);
   py.faces = (all_ok & 0x10) ? (all_ok & 0xf) : 0;
+  return py;
+}
+
+// The pyramid of a tile as the frame prologue leaves it for the sort: the four normals, the origin, the usable
+// faces, the products of the normals' components (forty words).  Built once per tile there; a sort that is not handed such records builds the pyramid in each of a tile's
+// wavefronts, whose strided reads of the tile's 64 rays (12-byte stride over eight image rows, by all four
+// wavefronts) measured 18 us of the 134 us launch at 12,750 tiles.
+struct alignas(32) TilePyramidRec {
+  float n[4][3];
+  float ox, oy, oz;
+  int faces;
+  float q[4][6];
+};
+static_assert(sizeof(TilePyramidRec) == MLPSP_TILE_PYRAMID_BYTES && MLPSP_TILE_PYRAMID_BYTES == 40 * 4,
+              "forty words per tile");
+// One wavefront per tile; `raw` are the directions before normalisation.
+__device__ __forceinline__ void write_tile_pyramid(const float* __restrict__ rays_o, const float* __restrict__ raw,
+                                                   const TileGeom& g, int tile, TilePyramidRec* __restrict__ out) {
+  const int pc = centre_pixel(g, tile);
+  float dx, dy, dz;
+  RawDirs{raw}.get(pc, dx, dy, dz);
+  const TilePyramid py = tile_pyramid(rays_o, RawDirs{raw}, g, tile, dx, dy, dz);
+  if ((threadIdx.x & 63) == 0) {
+    TilePyramidRec r;
+#pragma unroll
+    for (int f = 0; f < 4; ++f) {
+#pragma unroll
+      for (int k = 0; k < 3; ++k) r.n[f][k] = py.n[f][k];
+#pragma unroll
+      for (int k = 0; k < 6; ++k) r.q[f][k] = py.q[f][k];
+    }
+    r.ox = py.ox;
+    r.oy = py.oy;
+    r.oz = py.oz;
+    r.faces = py.faces;
+    out[tile] = r;
+  }
+}
+// A record as a wavefront holds it: lane j has word j (one coalesced load), and the words are taken out of that
+// register with v_readlane, the way tile_pyramid() hands out what its lanes computed.
+__device__ __forceinline__ float pyramid_record_word(const TilePyramidRec* __restrict__ record) {
+  const int lane = threadIdx.x & 63;
+  return reinterpret_cast<const float*>(record)[lane < 40 ? lane : 0];
+}
+__device__ __forceinline__ TilePyramid pyramid_from_word(float word) {
+  TilePyramid py;
+  py.ox = lane_value(word, 12);
+  py.oy = lane_value(word, 13);
+  py.oz = lane_value(word, 14);
+  py.faces = (int)float_to_bits(lane_value(word, 15));
+#pragma unroll
+  for (int f = 0; f < 4; ++f) {
+    const float nx = lane_value(word, f * 3), ny = lane_value(word, f * 3 + 1), nz = lane_value(word, f * 3 + 2);
+    py.n[f][0] = nx;
+    py.n[f][1] = ny;
+    py.n[f][2] = nz;
+#pragma unroll
+    for (int k = 0; k < 6; ++k) py.q[f][k] = lane_value(word, 16 + f * 6 + k);
+  }
   return py;
 }
 
@@ -297,17 +395,21 @@ __device__ __forceinline__ bool frame_records_hold(const SortRec* __restrict__ f
 // the tile's output, last one first -- at a fifth of its instructions: for short lists sort_one_tile()'s cost is
 // what four wavefronts spend per tile whatever its length (the passes of the bucket ranking, a dozen barriers).
 // Requires len <= 64 and len <= capacity; called by a whole wavefront.
-template <typename Source>
+template <bool PYR, typename Source>
 __device__ __forceinline__ void sort_small_tile_from(
-    const Source& src, const float* __restrict__ rays_o, const float* __restrict__ rays_d, const TileGeom& g, int tile,
-    float dx, float dy, float dz, const int32_t* __restrict__ cand, int family, float cull_r2, int num_prims,
-    int32_t* __restrict__ sorted_ids, float* __restrict__ sorted_keys, int start, int n) {
+    const Source& src, const float* __restrict__ rays_o, const float* __restrict__ rays_d,
+    const TilePyramidRec* __restrict__ pyramids, const TileGeom& g, int tile, float dx, float dy, float dz,
+    const int32_t* __restrict__ cand, int family, float cull_r2, int num_prims, int32_t* __restrict__ sorted_ids,
+    float* __restrict__ sorted_keys, int start, int n) {
   const int lane = threadIdx.x & 63;
   const int p = (lane < n) ? cand[start + lane] : 0;
   const bool known = (unsigned)p < (unsigned)num_prims;
   const typename Source::Rec P = src.load(known ? p : 0);
   TilePyramid py = {};
-  if (cull_r2 > 0.f) py = tile_pyramid(rays_o, rays_d, g, tile, dx, dy, dz);
+  if (cull_r2 > 0.f) {
+    if constexpr (PYR) py = pyramid_from_word(pyramid_record_word(pyramids + tile));
+    else py = tile_pyramid(rays_o, UnitDirs{rays_d}, g, tile, dx, dy, dz);
+  }
   bool keep = false;
   float key = 0.f;
   if (lane < n) {
@@ -332,29 +434,32 @@ __device__ __forceinline__ void sort_small_tile_from(
     if (sorted_keys) sorted_keys[pos] = kInvalidKey;
   }
 }
+template <bool PYR>
 __device__ __forceinline__ void sort_small_tile(
     const float* __restrict__ rays_o, const float* __restrict__ rays_d, const PrimRecord* __restrict__ prims,
-    const SortRec* __restrict__ frame, const int32_t* __restrict__ cand, const TileGeom& g, int family, float cull_r2,
-    int num_prims, int32_t* __restrict__ sorted_ids, float* __restrict__ sorted_keys, int tile, int start, int n) {
+    const SortRec* __restrict__ frame, const TilePyramidRec* __restrict__ pyramids, const int32_t* __restrict__ cand,
+    const TileGeom& g, int family, float cull_r2, int num_prims, int32_t* __restrict__ sorted_ids,
+    float* __restrict__ sorted_keys, int tile, int start, int n) {
   const int pc = centre_pixel(g, tile);
   const float ox = rays_o[pc * 3 + 0], oy = rays_o[pc * 3 + 1], oz = rays_o[pc * 3 + 2];
   const float dx = rays_d[pc * 3 + 0], dy = rays_d[pc * 3 + 1], dz = rays_d[pc * 3 + 2];
   if (frame_records_hold(frame, ox, oy, oz))
-    sort_small_tile_from(FromFrameRecord{frame + 1}, rays_o, rays_d, g, tile, dx, dy, dz, cand, family, cull_r2,
-                         num_prims, sorted_ids, sorted_keys, start, n);
+    sort_small_tile_from<PYR>(FromFrameRecord{frame + 1}, rays_o, rays_d, pyramids, g, tile, dx, dy, dz, cand, family,
+                         cull_r2, num_prims, sorted_ids, sorted_keys, start, n);
   else
-    sort_small_tile_from(FromPrimRecord{prims, ox, oy, oz}, rays_o, rays_d, g, tile, dx, dy, dz, cand, family, cull_r2,
-                         num_prims, sorted_ids, sorted_keys, start, n);
+    sort_small_tile_from<PYR>(FromPrimRecord{prims, ox, oy, oz}, rays_o, rays_d, pyramids, g, tile, dx, dy, dz, cand, family,
+                         cull_r2, num_prims, sorted_ids, sorted_keys, start, n);
 }
 
 // Sorts one tile with the calling 256-thread workgroup (every thread must call it; `tile` is uniform).  kSortMax
 // bounds `capacity`.  A workgroup that sorts several tiles in a row, or uses `lds` for something else afterwards,
 // puts a barrier in between.
-template <int kSortMax, typename Source>
+template <int kSortMax, bool PYR, typename Source>
 __device__ __forceinline__ void sort_one_tile_from(SortLds<kSortMax>& lds, const Source& src,
-    const float* __restrict__ rays_o, const float* __restrict__ rays_d, const TileGeom& g, int tile,
-    float dx, float dy, float dz, const int32_t* __restrict__ cand, int family, float cull_r2, int num_prims,
-    int32_t* __restrict__ sorted_ids, float* __restrict__ sorted_keys, int start, int len, int n) {
+    const float* __restrict__ rays_o, const float* __restrict__ rays_d, const TilePyramidRec* __restrict__ pyramids,
+    const TileGeom& g, int tile, float dx, float dy, float dz, const int32_t* __restrict__ cand, int family,
+    float cull_r2, int num_prims, int32_t* __restrict__ sorted_ids, float* __restrict__ sorted_keys, int start, int len,
+    int n) {
   auto& s_key = lds.key;
   auto& s_wave_cnt = lds.wave_cnt;
   auto& s_cnt = lds.cnt;
@@ -382,9 +487,22 @@ __device__ __forceinline__ void sort_one_tile_from(SortLds<kSortMax>& lds, const
   // ---- the tile's ray pyramid (only when culling is requested), while those loads are on their way: every
   //      wavefront builds it for itself -- four faces among its lanes, one ray of the tile per lane -- so no barrier
   //      is needed for the verdict
+  // (PYR is a compile-time choice: with both forms behind one run-time branch, or with the record read as sixteen
+  // scalar words, the compiler keeps the pyramid in vector registers for the candidate loop -- 96 registers instead of
+  // 72 and a wavefront less per SIMD.  A record therefore stays in ONE vector register, a word per lane, and every
+  // round takes the words it needs out of it; the empty statement in the loop keeps those reads there.)
   TilePyramid py = {};
-  if (cull_r2 > 0.f) py = tile_pyramid(rays_o, rays_d, g, tile, dx, dy, dz);
-  const int faces = py.faces;
+  float pyramid_word = 0.f;
+  int faces = 0;
+  if (cull_r2 > 0.f) {
+    if constexpr (PYR) {
+      pyramid_word = pyramid_record_word(pyramids + tile);
+      faces = (int)float_to_bits(lane_value(pyramid_word, 15));
+    } else {
+      py = tile_pyramid(rays_o, UnitDirs{rays_d}, g, tile, dx, dy, dz);
+      faces = py.faces;
+    }
+  }
 
   // ---- keys.  Survivors with an ordinary key are compacted to the front of s_key in list order; survivors
   //      whose key is the invalid key or larger go to the back of s_key, last slot first (the "late" stream: all
@@ -412,6 +530,10 @@ __device__ __forceinline__ void sort_one_tile_from(SortLds<kSortMax>& lds, const
     if (r + 1 < kRounds && i + kSortThreads < n)
       P_buf[(r + 1) & 1] = src.load(((unsigned)my_id[r + 1] < (unsigned)num_prims) ? my_id[r + 1] : 0);
     const bool known = (unsigned)p < (unsigned)num_prims;
+    if constexpr (PYR) {
+      asm volatile("" : "+v"(pyramid_word));
+      py = pyramid_from_word(pyramid_word);
+    }
     if (i < n) {
       outside = faces && known && outside_pyramid(py, P, cull_r2);
       keep = !outside;
@@ -583,12 +705,12 @@ __device__ __forceinline__ void sort_one_tile_from(SortLds<kSortMax>& lds, const
   }
 }
 
-template <int kSortMax>
+template <int kSortMax, bool PYR>
 __device__ __forceinline__ void sort_one_tile(SortLds<kSortMax>& lds,
     const float* __restrict__ rays_o, const float* __restrict__ rays_d, const PrimRecord* __restrict__ prims,
-    const SortRec* __restrict__ frame, const int32_t* __restrict__ cand, const int32_t* __restrict__ offsets,
-    const TileGeom& g, int family, int capacity, float cull_r2, int num_prims, int32_t* __restrict__ sorted_ids,
-    float* __restrict__ sorted_keys, int tile) {
+    const SortRec* __restrict__ frame, const TilePyramidRec* __restrict__ pyramids, const int32_t* __restrict__ cand,
+    const int32_t* __restrict__ offsets, const TileGeom& g, int family, int capacity, float cull_r2, int num_prims,
+    int32_t* __restrict__ sorted_ids, float* __restrict__ sorted_keys, int tile) {
   const int start = offsets[tile];
   const int len = offsets[tile + 1] - start;
   if (len <= 0) return;
@@ -597,11 +719,11 @@ __device__ __forceinline__ void sort_one_tile(SortLds<kSortMax>& lds,
   const float ox = rays_o[pc * 3 + 0], oy = rays_o[pc * 3 + 1], oz = rays_o[pc * 3 + 2];
   const float dx = rays_d[pc * 3 + 0], dy = rays_d[pc * 3 + 1], dz = rays_d[pc * 3 + 2];
   if (frame_records_hold(frame, ox, oy, oz))
-    sort_one_tile_from<kSortMax>(lds, FromFrameRecord{frame + 1}, rays_o, rays_d, g, tile, dx, dy, dz, cand, family,
-                                 cull_r2, num_prims, sorted_ids, sorted_keys, start, len, n);
+    sort_one_tile_from<kSortMax, PYR>(lds, FromFrameRecord{frame + 1}, rays_o, rays_d, pyramids, g, tile, dx, dy, dz, cand,
+                                 family, cull_r2, num_prims, sorted_ids, sorted_keys, start, len, n);
   else
-    sort_one_tile_from<kSortMax>(lds, FromPrimRecord{prims, ox, oy, oz}, rays_o, rays_d, g, tile, dx, dy, dz, cand, family,
-                                 cull_r2, num_prims, sorted_ids, sorted_keys, start, len, n);
+    sort_one_tile_from<kSortMax, PYR>(lds, FromPrimRecord{prims, ox, oy, oz}, rays_o, rays_d, pyramids, g, tile, dx, dy, dz,
+                                 cand, family, cull_r2, num_prims, sorted_ids, sorted_keys, start, len, n);
 }
 
 }  // namespace mlpsp

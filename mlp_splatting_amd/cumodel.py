@@ -900,10 +900,16 @@ class NeuralPrimitiveSceneTileCUDA(nn.Module):
         ray_o = ray_o.contiguous()
         if (hasattr(ext, "frame_prologue") and ray_d.is_cuda and ray_d.dtype == torch.float32 and ray_d.dim() == 2
                 and ray_d.shape[1] == 3 and not ray_d.requires_grad and ray_o.dtype == torch.float32
-                and ray_o.shape == ray_d.shape and _env("MLPSP_SORT_FRAME_RECORDS", "0") == "1"):
-            # unit directions and the sort's per-frame records in one launch (opt-in: measured 6 us per frame slower
-            # than the full key evaluation on one MI355X, where the sort is not bound by vector instructions)
-            unit_dirs, more["frame_records"] = ext.frame_prologue(ray_o, ray_d, positions, log_scales, self._unit_quats())
+                and ray_o.shape == ray_d.shape and ray_o.is_cuda):
+            # unit directions and the tiles' ray pyramids for the sort's culling in one launch; with
+            # MLPSP_SORT_FRAME_RECORDS=1 also the sort's per-frame records (opt-in: measured 6 us per frame slower than
+            # the full key evaluation on one MI355X)
+            geometry = None
+            if _env("MLPSP_SORT_FRAME_RECORDS", "0") == "1":
+                geometry = (positions, log_scales, self._unit_quats())
+            unit_dirs, more["tile_pyramids"], records = ext.frame_prologue(ray_o, ray_d, int(W), int(H), geometry)
+            if records is not None:
+                more["frame_records"] = records
         else:
             unit_dirs = _unit_directions(ray_d)
         freq, att = self._frequency_tables(device)

@@ -64,20 +64,39 @@ def normalize_rays(rays_d):
     return out
 
 
-def frame_prologue(rays_o, rays_d, records):
-    """(unit directions, frame records of the sort) in one launch: what :func:`normalize_rays` returns, and the
-    per-primitive records :func:`sort_tiles` takes as ``frame_records`` (written for the origin of ray 0)."""
+def frame_prologue(rays_o, rays_d, W, H, TW=8, TH=8, records=None):
+    """(unit directions, tile pyramids, frame records | None) of a W x H frame in one launch: what
+    :func:`normalize_rays` returns; the per-tile ray pyramids :func:`sort_tiles` takes as ``tile_pyramids``; and, with
+    the geometry ``records`` of the scene, the per-primitive records it takes as ``frame_records`` (written for the
+    origin of ray 0)."""
     rays_d, rays_o = _f32c(rays_d, "rays_d"), _f32c(rays_o, "rays_o")
-    if rays_d.dim() != 2 or rays_d.shape[1] != 3 or rays_o.shape != rays_d.shape:
-        raise ValueError("rays_o and rays_d must be [B, 3]")
+    if rays_d.dim() != 2 or rays_d.shape[1] != 3 or rays_o.shape != rays_d.shape or rays_d.shape[0] != W * H:
+        raise ValueError("rays_o and rays_d must be [W * H, 3]")
     lib = _lib.load()
-    n = records.numel() // _lib.PRIM_RECORD_BYTES
+    dev = rays_d.device
     unit = torch.empty_like(rays_d)
-    frame = torch.empty(lib.mlpsp_sort_frame_records_bytes(n), dtype=torch.uint8, device=rays_d.device)
-    code = lib.mlpsp_frame_prologue(_ptr(rays_d), rays_d.shape[0], _ptr(unit), _ptr(rays_o), _ptr(records), n, _ptr(frame),
-                                    _stream(rays_d.device))
+    pyramids = torch.empty(_tile_pyramids_bytes(W, H, TW, TH), dtype=torch.uint8, device=dev)
+    n, frame = 0, None
+    if records is not None:
+        n = records.numel() // _lib.PRIM_RECORD_BYTES
+        frame = torch.empty(lib.mlpsp_sort_frame_records_bytes(n), dtype=torch.uint8, device=dev)
+    code = lib.mlpsp_frame_prologue(_ptr(rays_d), _ptr(unit), _ptr(rays_o), W, H, TW, TH, _ptr(pyramids), _ptr(records), n,
+                                    _ptr(frame), _stream(dev))
     _check(code, "mlpsp_frame_prologue")
-    return unit, frame
+    return unit, pyramids, frame
+
+
+_pyramid_bytes = {}
+
+
+def _tile_pyramids_bytes(W, H, TW, TH):
+    key = (W, H, TW, TH)
+    got = _pyramid_bytes.get(key)
+    if got is None:
+        if len(_pyramid_bytes) > 64:
+            _pyramid_bytes.clear()
+        got = _pyramid_bytes[key] = _lib.load().mlpsp_tile_pyramids_bytes(W, H, TW, TH)
+    return got
 
 
 def validate_tile_lists(candidates, tile_offsets, n_tiles: int, capacity: int, num_primitives: int, path_name: str):
@@ -228,7 +247,8 @@ def bin_legacy_async(positions, log_scales, view_matrices, proj_matrix, W: int, 
 
 
 def sort_tiles(rays_o, rays_d, records, candidates, tile_offsets, W, H, TW, TH, family=_lib.KEY_TSTAR,
-               capacity=TILE_CAPACITY_DEFAULT, want_keys=False, cull_threshold=0.0, frame_records=None):
+               capacity=TILE_CAPACITY_DEFAULT, want_keys=False, cull_threshold=0.0, frame_records=None,
+               tile_pyramids=None):
     """Materialised per-tile depth order: (sorted_ids [P], sorted_keys [P] | None).
 
     With ``cull_threshold`` (the render's score threshold) candidates that provably hit no ray of their
@@ -236,7 +256,8 @@ def sort_tiles(rays_o, rays_d, records, candidates, tile_offsets, W, H, TW, TH, 
     :func:`frame_prologue` wrote for these rays and primitives (a fifth fewer vector instructions in the sort; keys
     and order do not depend on it), or True to let this call write them first (one more launch, which on one MI355X
     costs a frame more than the sort kernel gains), or False.  None = what ``MLPSP_SORT_FRAME_RECORDS`` says, off
-    unless it is 1."""
+    unless it is 1.  ``tile_pyramids``: what :func:`frame_prologue` returned for these rays and this tile size (the
+    culling's per-tile planes, which the sort otherwise builds in every wavefront of a tile; same output)."""
     dev = rays_o.device
     sorted_ids = torch.empty_like(candidates)
     keys = torch.empty(candidates.numel(), dtype=torch.float32, device=dev) if want_keys else None
@@ -254,9 +275,13 @@ def sort_tiles(rays_o, rays_d, records, candidates, tile_offsets, W, H, TW, TH, 
         scratch, ready = frame_records, 1
     elif frame_records:
         scratch = torch.empty(lib.mlpsp_sort_frame_records_bytes(num_primitives), dtype=torch.uint8, device=dev)
+    if tile_pyramids is not None and not (tile_pyramids.is_cuda and tile_pyramids.dtype == torch.uint8
+                                          and tile_pyramids.is_contiguous()
+                                          and tile_pyramids.numel() == _tile_pyramids_bytes(W, H, TW, TH)):
+        raise ValueError("tile_pyramids must be the uint8 buffer frame_prologue() returned for this frame and tile size")
     code = lib.mlpsp_sort_tiles(_ptr(rays_o), _ptr(rays_d), _ptr(records), num_primitives, _ptr(candidates),
                                 _ptr(tile_offsets), W, H, TW, TH, int(family), int(capacity), float(cull_threshold),
-                                _ptr(scratch), ready, _ptr(sorted_ids), _ptr(keys), _stream(dev))
+                                _ptr(scratch), ready, _ptr(tile_pyramids), _ptr(sorted_ids), _ptr(keys), _stream(dev))
     _check(code, "mlpsp_sort_tiles")
     return sorted_ids, keys
 

@@ -351,16 +351,18 @@ class TileExt:
                 held = self._queued_buffers.setdefault(key, {})
         return held
 
-    def frame_prologue(self, rays_o, rays_d, positions, log_scales, unit_quats):
-        """(unit ray directions, frame records of the sort) for a queued frame, in one launch
-        (:func:`ops.frame_prologue`); the geometry records they are made from are the cached ones.  ``rays_d`` must be
-        a float32 [B, 3] device tensor."""
+    def frame_prologue(self, rays_o, rays_d, width, height, geometry=None):
+        """(unit ray directions, tile pyramids of the sort, frame records of the sort | None) for a queued frame of
+        8x8 tiles, in one launch (:func:`ops.frame_prologue`).  ``geometry`` = (positions, log_scales, unit_quats) asks
+        for the frame records too; the geometry records they are made from are the cached ones.  ``rays_o`` and
+        ``rays_d`` must be float32 [width * height, 3] device tensors."""
         with _on_device(rays_o.device):
-            return ops.frame_prologue(rays_o, rays_d, self._records(positions, log_scales, unit_quats))
+            records = None if geometry is None else self._records(*geometry)
+            return ops.frame_prologue(rays_o, rays_d, int(width), int(height), 8, 8, records)
 
     def render_frame_queued(self, rays_o, unit_dirs, positions, log_scales, unit_quats, freq, att, ws, view_matrices,
                             proj_matrix, width, height, threshold, precision, binned=None, feat=None,
-                            frame_records=None):
+                            frame_records=None, tile_pyramids=None):
         """(rgb, alpha) of one 8x8-tile, tile-centre-order RGB frame: binning, sort and render are queued
         back to back and ONE read-back at the end brings the pair count, the longest tile list and the
         non-finite flag.  The candidate buffer is sized from the previous frame's count; if this frame
@@ -369,8 +371,8 @@ class TileExt:
         ``binned``: the result of :meth:`frame_binning_queued` for the same primitives and camera, when the caller
         has queued the binning already.  ``feat`` = (feat_attr, beta, temp) adds the gated feature image (matrix-core
         precisions only): (rgb, alpha, feat); None is also returned when the record pool of the first size ran out
-        or the attributes do not fit fp16 (the step-by-step path then decides what to do).  ``frame_records``: what
-        :meth:`frame_prologue` returned beside ``unit_dirs`` for these rays and primitives.
+        or the attributes do not fit fp16 (the step-by-step path then decides what to do).  ``tile_pyramids``,
+        ``frame_records``: what :meth:`frame_prologue` returned beside ``unit_dirs`` for these rays and primitives.
         Errors are those of the entry points it stands for (capacity text of np_tile_kernels.cu:4578-4588,
         fallback policy of rgb_wmma.cuh:260-272)."""
         name = "render_tiles_rgb_wmma" if precision != "f32" else "render_tiles_forward_tilecenter"
@@ -397,7 +399,8 @@ class TileExt:
         with _on_device(rays_o.device):
             rec = self._records(positions, log_scales, unit_quats)
             order, _ = ops.sort_tiles(rays_o, unit_dirs, rec, cand, offsets, width, height, 8, 8, _lib.KEY_TSTAR,
-                                      self.max_tile_prims, cull_threshold=threshold, frame_records=frame_records)
+                                      self.max_tile_prims, cull_threshold=threshold, frame_records=frame_records,
+                                      tile_pyramids=tile_pyramids)
             fmap, pool_ran_out = None, 0
             if precision != "f32":
                 packed = self._packed_weights(list(ws), precision == "bf16")

@@ -163,12 +163,15 @@ def test_sorted_tile_lists_match_oracle_keys_and_order(device, oracle_mod, frame
     sc = fr.scene
     cand, off = fr.lists
     rec = ops.prepare_primitives(_t(sc.positions, device), _t(sc.log_scales, device), _t(sc.quats, device))
+    pyramids = None
     if frame_records == "prologue":
         # the records written beside the unit directions, in one launch; the directions are normalize_rays' bits
-        unit, frame_records = ops.frame_prologue(_t(fr.rays_o, device), _t(fr.rays_d, device), rec)
+        unit, pyramids, frame_records = ops.frame_prologue(_t(fr.rays_o, device), _t(fr.rays_d, device), fr.W, fr.H, 8, 8,
+                                                           rec)
         assert torch.equal(unit.view(torch.int32), ops.normalize_rays(_t(fr.rays_d, device)).view(torch.int32))
     ids, keys = ops.sort_tiles(_t(fr.rays_o, device), _t(fr.rays_d, device), rec, _t(cand, device), _t(off, device),
-                               fr.W, fr.H, 8, 8, family=family, want_keys=True, frame_records=frame_records)
+                               fr.W, fr.H, 8, 8, family=family, want_keys=True, frame_records=frame_records,
+                               tile_pyramids=pyramids)
     want_ids, want_keys = oracle_mod.sort_tiles(fr.rays_o, fr.rays_d, sc.positions, sc.log_scales, sc.quats, cand, off,
                                                 fr.W, fr.H, 8, 8, family=family)
     np.testing.assert_array_equal(ids.cpu().numpy(), want_ids)
