@@ -88,7 +88,10 @@ __global__ __launch_bounds__(256) void normalize_rays_kernel(const float* __rest
                                                              float* __restrict__ out) {
   const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= n) return;
-  unit_direction(d[i * 3], d[i * 3 + 1], d[i * 3 + 2], out[i * 3], out[i * 3 + 1], out[i * 3 + 2]);
+  const Float3 v = load3(d, i);
+  float ux, uy, uz;
+  unit_direction(v.x, v.y, v.z, ux, uy, uz);
+  store3(out, i, ux, uy, uz);
 }
 
 // The per-frame preparations that depend on nothing but the rays (and the scene), in one launch: blocks
@@ -106,7 +109,10 @@ __global__ __launch_bounds__(256) void frame_prologue_kernel(const float* __rest
   if (b < ray_blocks) {
     const long long i = (long long)b * blockDim.x + threadIdx.x;
     if (i >= n) return;
-    unit_direction(d[i * 3], d[i * 3 + 1], d[i * 3 + 2], unit[i * 3], unit[i * 3 + 1], unit[i * 3 + 2]);
+    const Float3 v = load3(d, i);
+    float ux, uy, uz;
+    unit_direction(v.x, v.y, v.z, ux, uy, uz);
+    store3(unit, i, ux, uy, uz);
   } else if (b < ray_blocks + tile_blocks) {
     const int tile = (b - ray_blocks) * (int)(blockDim.x >> 6) + (int)(threadIdx.x >> 6);
     if (tile < g.ntx * g.nty) write_tile_pyramid(rays_o, d, g, tile, pyramids);

@@ -277,10 +277,10 @@ __device__ __forceinline__ void render_tile_mfma(
   const int x = tx * 8 + (l & 7), y = ty * 8 + (l >> 3);
   const bool valid = (x < W) && (y < H);
   const int pix = valid ? (y * W + x) : 0;
-  const float rox = valid ? rays_o[pix * 3 + 0] : 0.f, roy = valid ? rays_o[pix * 3 + 1] : 0.f,
-              roz = valid ? rays_o[pix * 3 + 2] : 0.f;
-  const float rdx = valid ? rays_d[pix * 3 + 0] : 0.f, rdy = valid ? rays_d[pix * 3 + 1] : 0.f,
-              rdz = valid ? rays_d[pix * 3 + 2] : 0.f;
+  const Float3 ray_o = valid ? load3(rays_o, pix) : Float3{0.f, 0.f, 0.f};
+  const Float3 ray_d = valid ? load3(rays_d, pix) : Float3{0.f, 0.f, 0.f};
+  const float rox = ray_o.x, roy = ray_o.y, roz = ray_o.z;
+  const float rdx = ray_d.x, rdy = ray_d.y, rdz = ray_d.z;
   // The encoding of the ray direction (input components 0..2, operand words 0..8 of both column blocks) does
   // not depend on the primitive: it is computed once per pixel and parked in LDS in operand form -- 18 more
   // live registers would cost the fourth wavefront per SIMD.  Written and read by this wavefront only: no barrier.
@@ -422,9 +422,7 @@ __device__ __forceinline__ void render_tile_mfma(
   }
 
   if (valid) {
-    out_rgb[pix * 3 + 0] = acc.cr;
-    out_rgb[pix * 3 + 1] = acc.cg;
-    out_rgb[pix * 3 + 2] = acc.cb;
+    store3(out_rgb, pix, acc.cr, acc.cg, acc.cb);
     out_alpha[pix] = 1.f - acc.trans;
   }
   if constexpr (SP > 0) {

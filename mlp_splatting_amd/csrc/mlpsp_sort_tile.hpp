@@ -169,14 +169,6 @@ __device__ __forceinline__ float lane_value(float v, int lane) {
 // root and three products, not the exactly rounded square root and divisions of the unit vectors the renderer uses
 // (four of those per lane were three quarters of the prologue's pyramid work).  The planes then differ from those
 // built from the stored unit vectors in their last bits; the culling has a 2 % margin either way.
-// (a ray's three floats as one 12-byte load: the rays of a tile lie 12 bytes apart over several image rows, and what
-// these reads cost is the number of load instructions)
-struct __attribute__((packed, aligned(4))) Float3 {
-  float x, y, z;
-};
-__device__ __forceinline__ Float3 load3(const float* __restrict__ base, int pix) {
-  return *reinterpret_cast<const Float3*>(base + (size_t)pix * 3);
-}
 struct UnitDirs {
   const float* __restrict__ d;
   __device__ __forceinline__ void get(int pix, float& x, float& y, float& z) const {

@@ -233,7 +233,7 @@ def test_sort_is_the_stable_key_order_for_every_key_distribution(device, oracle_
 @pytest.mark.parametrize("name,n,width,height,tile,eye", [
     ("cfg1_5k_160x120", None, 160, 120, 8, (0.3, -0.2, -0.5)), ("cfg1_5k_160x120", 4000, 100, 76, 16, (1.0, 0.8, -1.2)),
     ("cfg2_50k_640x480", 20000, 200, 136, 8, (-0.7, 0.4, 0.9)), ("cfg1_5k_160x120", 1500, 21, 13, 8, (0.1, 0.1, -0.2))])
-@pytest.mark.parametrize("frame_records", [True, False], ids=["frame_records", "full_key"])
+@pytest.mark.parametrize("frame_records", [True, False, "pyramids"], ids=["frame_records", "full_key", "pyramids"])
 def test_conservative_tile_culling_never_drops_a_hit(device, oracle_mod, name, n, width, height, tile, eye, frame_records):
     # per tile: the survivors, in front, are the plain sorted list with the culled ids struck out; the
     # culled ones follow as ~id in reverse list (descending id) order; (2) it is a real saving, and (3) no bit
@@ -246,8 +246,16 @@ def test_conservative_tile_culling_never_drops_a_hit(device, oracle_mod, name, n
     ro, rd, c, o = _t(fr.rays_o, device), _t(fr.rays_d, device), _t(cand, device), _t(off, device)
     # (with frame records the ellipsoid's support along a face normal comes from a stored covariance, rounded up;
     # without, from the face normal rotated into the primitive's axes: two forms of the same conservative test)
-    plain, _ = ops.sort_tiles(ro, rd, rec, c, o, fr.W, fr.H, tile, tile, frame_records=frame_records)
-    culled, _ = ops.sort_tiles(ro, rd, rec, c, o, fr.W, fr.H, tile, tile, cull_threshold=fr.thr, frame_records=frame_records)
+    pyramids = None
+    if frame_records == "pyramids":
+        # the tiles' ray pyramids built once per tile by the frame prologue (from the same directions, normalised
+        # again on the way with a reciprocal square root: the planes agree with the sort's own to a few ulps)
+        frame_records = False
+        _, pyramids, none = ops.frame_prologue(ro, rd, fr.W, fr.H, tile, tile)
+        assert none is None and pyramids.numel() == (off.size - 1) * 160
+    plain, _ = ops.sort_tiles(ro, rd, rec, c, o, fr.W, fr.H, tile, tile, frame_records=frame_records, tile_pyramids=pyramids)
+    culled, _ = ops.sort_tiles(ro, rd, rec, c, o, fr.W, fr.H, tile, tile, cull_threshold=fr.thr, frame_records=frame_records,
+                               tile_pyramids=pyramids)
     plain, culled = plain.cpu().numpy(), culled.cpu().numpy()
     for t in range(off.size - 1):
         a, b = plain[off[t]:off[t + 1]], culled[off[t]:off[t + 1]]
@@ -257,7 +265,8 @@ def test_conservative_tile_culling_never_drops_a_hit(device, oracle_mod, name, n
         assert np.array_equal(b[:k], a[~np.isin(a, gone)])
     frac = (culled < 0).mean()
     assert frac > 0.15, frac
-    if frame_records:      # the stored covariance costs next to nothing in culled candidates
+    if frame_records or pyramids is not None:      # the stored covariance, or planes that differ in their last bits,
+        # cost next to nothing in culled candidates
         other, _ = ops.sort_tiles(ro, rd, rec, c, o, fr.W, fr.H, tile, tile, cull_threshold=fr.thr, frame_records=False)
         assert frac > 0.97 * float((other < 0).float().mean()), (frac, float((other < 0).float().mean()))
     want = oracle_mod.render_tilecenter(*fr.base_numpy(cand, off), *fr.dims)
@@ -290,6 +299,15 @@ def test_culling_is_off_for_tiles_with_mixed_origins_or_degenerate_pyramids(devi
     c, o = _t(cand, device), _t(off, device)
     ids, _ = ops.sort_tiles(_t(ro, device), _t(fr.rays_d, device), rec, c, o, fr.W, fr.H, 8, 8, cull_threshold=fr.thr)
     assert int((ids < 0).sum()) == 0
+    # ... and so it is when the pyramids come from the frame prologue: those of such tiles are marked unusable
+    _, pyramids, _ = ops.frame_prologue(_t(ro, device), _t(fr.rays_d, device), fr.W, fr.H)
+    faces = pyramids.view(torch.int32).view(-1, 40)[:, 15]
+    assert int(faces.abs().sum()) == 0
+    with_records, _ = ops.sort_tiles(_t(ro, device), _t(fr.rays_d, device), rec, c, o, fr.W, fr.H, 8, 8, cull_threshold=fr.thr,
+                                     tile_pyramids=pyramids)
+    assert torch.equal(with_records, ids)
+    _, usable, _ = ops.frame_prologue(_t(fr.rays_o, device), _t(fr.rays_d, device), fr.W, fr.H)
+    assert int((usable.view(torch.int32).view(-1, 40)[:, 15] == 15).sum()) == (fr.W // 8) * (fr.H // 8)
     fr1 = Frame("cfg1_5k_160x120", n=300, width=12, height=6, tile=1)           # 1x1 tiles: no pyramid
     c1, o1 = fr1.oracle_lists(oracle_mod)
     rec1 = ops.prepare_primitives(_t(fr1.scene.positions, device), _t(fr1.scene.log_scales, device), _t(fr1.scene.quats, device))
