@@ -76,6 +76,32 @@ def test_binning_with_primitives_that_span_many_super_tiles(device, oracle_mod, 
     np.testing.assert_array_equal(cand.cpu().numpy(), want[0])
 
 
+@pytest.mark.parametrize("n", [300000, 2200000])
+def test_binning_with_more_chunks_than_a_workgroup_takes_at_once(device, oracle_mod, n):
+    """The level-1 fill places a super-tile's list itself: a workgroup adds up the counts before it and scans its row
+    of (chunk, super-tile) counts, 1,024 chunks per pass, the ballots of each wavefront's first eight chunks requested
+    ahead.  147 chunks (300 k primitives) go beyond those eight, 1,075 chunks (2.2 M) into a second pass; both entry
+    points, the two-call one and the asynchronous one with its guard, against the oracle."""
+    from mlp_splatting_amd import ops, synthetic as syn
+    rng = np.random.default_rng(3)
+    pos = (rng.random((n, 3), dtype=np.float32) * 4 - 2).astype(np.float32)
+    logs = (rng.standard_normal((n, 3)).astype(np.float32) * np.float32(0.3) - np.float32(5.5)).astype(np.float32)
+    W, H, f, thr = 96, 64, 60.0, 5e-3
+    view = syn.view_matrix(syn.look_at((0.3, -0.2, -2.5), (0.0, 0.0, 0.4)))
+    proj = syn.projection_matrix(f, W, H)
+    want_cand, want_off = oracle_mod.bin_legacy(pos, logs, view[None], proj, W, H, 8, thr)
+    assert want_cand.size > n // 2
+    p, l = _t(pos, device), _t(logs, device)
+    cand, off = ops.bin_legacy(p, l, torch.from_numpy(view)[None], torch.from_numpy(proj), W, H, 8, thr)
+    np.testing.assert_array_equal(off.cpu().numpy(), want_off)
+    np.testing.assert_array_equal(cand.cpu().numpy(), want_cand)
+    cand2, off2, counts = ops.bin_legacy_async(p, l, _t(view, device), _t(proj, device), W, H, 8, thr, want_cand.size + 7)
+    pairs, longest, _, guard = counts.tolist()
+    assert (pairs, longest, guard) == (want_cand.size, int(np.diff(want_off).max()), 0)
+    np.testing.assert_array_equal(off2.cpu().numpy(), want_off)
+    np.testing.assert_array_equal(cand2.cpu().numpy()[:pairs], want_cand)
+
+
 def test_binning_with_several_views_and_no_view_per_tile(device, oracle_mod):
     """Several view matrices without tile_view_ids: every tile is binned against view 0 (level 1 then runs the walk
     over (chunk, super-tile) pairs with all the views, a superset that level 2 cuts down)."""
