@@ -230,6 +230,18 @@ def _mlp_forward_indexed(x_enc, prim_ids, W1, b1, W2, b2, W3, b3):
     return torch.sigmoid(o[:, :3]), F.softplus(o[:, 3:4])
 
 
+_LANES: dict = {}
+
+
+def _render_lanes(device, count):
+    """The streams (default priority) on which ``render_frames`` keeps ``count`` frames in flight on ``device``."""
+    key = (device.index if device.index is not None else torch.cuda.current_device(), count)
+    lanes = _LANES.get(key)
+    if lanes is None:
+        lanes = _LANES[key] = [torch.cuda.Stream(device) for _ in range(count)]
+    return lanes
+
+
 def _add_background(rgb, alpha, bg):
     """rgb + clamp(1 - alpha, 0, 1) * bg (scannet/cumodel.py:252-256)."""
     if bg is None:
@@ -858,12 +870,13 @@ class NeuralPrimitiveSceneTileCUDA(nn.Module):
             self._background(bg_color, ray_o))
 
     def _forward_queued(self, ext, ray_o, ray_d, score_threshold, view_matrix, proj_matrix, bg_color, device,
-                        with_feat=False):
+                        with_feat=False, defer=False):
         """The RGB frame with binning, sort and render queued back to back and one read-back at the end
         (``TileExt.render_frame_queued``); None when that path does not apply or has to be repeated the
         synchronous way.  Same images and errors as the step-by-step path.  The binning goes first: it needs only
         the primitives and the camera, and the device is busy with it while the host prepares the rest of the
-        frame (unit ray directions, tables, weights)."""
+        frame (unit ray directions, tables, weights).  ``defer``: return a callable that finishes the frame (waits for
+        its read-back, returns the images or None) instead of finishing it here."""
         precision = str(getattr(self, "render_precision", "f32")).lower()
         if precision not in {"f32", "bf16", "fp16"}:
             raise ValueError(f"Unsupported render_precision {precision!r}; use 'f32', 'bf16' or 'fp16'.")
@@ -916,12 +929,94 @@ class NeuralPrimitiveSceneTileCUDA(nn.Module):
         if with_feat:
             more["feat"] = (self.feat_attr.detach().contiguous(), float(self.feature_gating_beta),
                             float(self.feature_gating_temp))
+        if defer:
+            more["defer"] = True
         out = ext.render_frame_queued(ray_o, unit_dirs, positions, log_scales, self._unit_quats(), freq, att,
                                       ws, views, proj, int(W), int(H), float(score_threshold), precision, **more)
-        if out is None:
-            return None
-        rgb = _add_background(out[0], out[1], self._background(bg_color, ray_o))
-        return (rgb, out[2]) if with_feat else rgb
+
+        def finish(out=out):
+            if out is not None and not isinstance(out, tuple):
+                out = ext.finish_frame_queued(out)
+            if out is None:
+                return None
+            rgb = _add_background(out[0], out[1], self._background(bg_color, ray_o))
+            return (rgb, out[2]) if with_feat else rgb
+        return finish if defer else finish()
+
+    def render_frames(self, frames, score_threshold=1e-3, bg_color=None, return_feature: bool = False,
+                      frames_in_flight: int = 2):
+        """``[self(ray_o, ray_d, score_threshold, bg_color, view_matrix, proj_matrix, return_feature=...) for (ray_o,
+        ray_d, view_matrix, proj_matrix) in frames]`` without gradients, with up to ``frames_in_flight`` frames queued
+        on the device at once (no counterpart in the reference, whose callers render camera after camera,
+        tools/benchmark_inference.py:264-313).  One frame alone leaves the device idle twice: at its end, where the
+        last tiles of the render run on a chip that has nothing else to do, and between frames, while the host reads
+        the frame's 96 status bytes and issues the next launches.  Here frame k+1 is queued on a second stream before
+        the host waits for frame k, so its binning and sort run beside the end of frame k's render.  Same images as
+        ``forward`` (each frame runs the same launches in the same order on its stream); the inputs must be ready
+        on the current stream when the call is made, and the results are ready on it when the call returns."""
+        frames = list(frames)
+        W, H = self.image_size if self.image_size is not None else (0, 0)
+        plain = self.__dict__
+        with_feat = return_feature and self.feat_attr is not None
+
+        def one(f):
+            with torch.no_grad():
+                return self.forward(f[0], f[1], score_threshold, bg_color, f[2], f[3], return_feature=return_feature)
+        eligible = (frames_in_flight > 1 and len(frames) > 2 and self.image_size is not None
+                    and self._resolve_tile_order_mode() == "tilecenter" and int(self.tile_size) == 8
+                    and (with_feat or not return_feature) and plain.get("queued_frames", True)
+                    and plain.get("camera_mode", "legacy-centered") != "colmap-native"
+                    and str(getattr(self, "render_precision", "f32")).lower() in {"bf16", "fp16"}
+                    and all(f[2] is not None and f[3] is not None and f[0].shape[0] == W * H for f in frames))
+        if not eligible:
+            return [one(f) for f in frames]
+        device = self._activate_cuda_device()
+        ext = self._ensure_tile_ext()
+        if not (hasattr(ext, "render_frame_queued") and hasattr(ext, "finish_frame_queued")):
+            return [one(f) for f in frames]
+        # The first frame on the caller's stream: whatever is derived from the parameters (geometry records, operand
+        # copies of the weights, tables) is built there, before the lanes read it.
+        results = [one(frames[0])]
+        main = torch.cuda.current_stream(device)
+        lanes = _render_lanes(device, min(int(frames_in_flight), 4))
+        ready = torch.cuda.Event()
+        ready.record(main)
+        for lane in lanes:
+            lane.wait_event(ready)
+        waiting = []                       # (lane, frame, finish) in queue order
+
+        def finish_oldest():
+            lane, f, finish = waiting.pop(0)
+            with torch.cuda.stream(lane):
+                out = finish() if finish is not None else None
+                if out is None:
+                    out = one(f)           # rare: the synchronous way, on the frame's own stream
+            results.append(out)
+        try:
+            with torch.no_grad():
+                for i, f in enumerate(frames[1:]):
+                    lane = lanes[i % len(lanes)]
+                    with torch.cuda.stream(lane):
+                        finish = self._forward_queued(ext, f[0], f[1], score_threshold, f[2], f[3], bg_color, device,
+                                                      with_feat, defer=True)
+                    waiting.append((lane, f, finish))
+                    if i == 0:
+                        # (should this frame have built something the first did not, the other lanes see it built)
+                        built = torch.cuda.Event()
+                        built.record(lane)
+                        for other in lanes[1:]:
+                            other.wait_event(built)
+                    if len(waiting) >= len(lanes):
+                        finish_oldest()
+                while waiting:
+                    finish_oldest()
+        finally:
+            for lane in lanes:
+                main.wait_stream(lane)
+        for out in results[1:]:
+            for t in (out if isinstance(out, tuple) else (out,)):
+                t.record_stream(main)
+        return results
 
     def render_feature_map(self, ray_o, ray_d, score_threshold: float = 1e-3, view_matrix=None, proj_matrix=None,
                            culled_prim_indices=None, tile_offsets=None):

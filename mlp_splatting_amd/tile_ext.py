@@ -49,6 +49,18 @@ def _on_device(device):
     return torch.cuda.device(device)
 
 
+class QueuedFrame:
+    """A frame whose launches are queued and whose 96-byte read-back has not been looked at yet
+    (``TileExt.render_frame_queued(defer=True)`` -> ``TileExt.finish_frame_queued``)."""
+    __slots__ = ("name", "precision", "with_feat", "images", "tail", "held", "cap", "scale", "inputs", "lists", "host",
+                 "landed", "counts")
+
+    def __init__(self, name, precision, with_feat, images, tail, held, cap, scale, inputs, lists):
+        self.name, self.precision, self.with_feat, self.images = name, precision, with_feat, images
+        self.tail, self.held, self.cap, self.scale, self.inputs, self.lists = tail, held, cap, scale, inputs, lists
+        self.host = self.landed = self.counts = None
+
+
 class TileExt:
     """Forward entry points of the tile renderer on one MI355X."""
 
@@ -362,7 +374,7 @@ class TileExt:
 
     def render_frame_queued(self, rays_o, unit_dirs, positions, log_scales, unit_quats, freq, att, ws, view_matrices,
                             proj_matrix, width, height, threshold, precision, binned=None, feat=None,
-                            frame_records=None, tile_pyramids=None):
+                            frame_records=None, tile_pyramids=None, defer=False):
         """(rgb, alpha) of one 8x8-tile, tile-centre-order RGB frame: binning, sort and render are queued
         back to back and ONE read-back at the end brings the pair count, the longest tile list and the
         non-finite flag.  The candidate buffer is sized from the previous frame's count; if this frame
@@ -373,6 +385,10 @@ class TileExt:
         precisions only): (rgb, alpha, feat); None is also returned when the record pool of the first size ran out
         or the attributes do not fit fp16 (the step-by-step path then decides what to do).  ``tile_pyramids``,
         ``frame_records``: what :meth:`frame_prologue` returned beside ``unit_dirs`` for these rays and primitives.
+        ``defer``: queue the frame, start its read-back into pinned memory and return a :class:`QueuedFrame` instead of
+        waiting; :meth:`finish_frame_queued` then waits, decides and returns what this method would have.  A caller
+        that has the next camera at hand queues that frame on another stream in between, so the device never waits
+        for the host (matrix-core precisions; an exact frame is finished before it is returned either way).
         Errors are those of the entry points it stands for (capacity text of np_tile_kernels.cu:4578-4588,
         fallback policy of rgb_wmma.cuh:260-272)."""
         name = "render_tiles_rgb_wmma" if precision != "f32" else "render_tiles_forward_tilecenter"
@@ -417,35 +433,66 @@ class TileExt:
                         rays_o, unit_dirs, rec, order, offsets, freq, att, *ws, feat[0], feat[1], feat[2], width, height,
                         threshold, bf16=(precision == "bf16"), packed=packed, packed_feat=packed_feat, status=status,
                         status_is_clear=flags_clear)
-                host = tail.cpu().numpy()
-                held["flags_clear"] = host[32:].tobytes() == _SIXTEEN_ZERO_WORDS
-                pairs, longest, l1_entries, guard = (int(v) for v in host[:32].view("int64"))
-                nonfinite = int(host[32:36].view("int32")[0])
-                pool_ran_out = int(host[36:40].view("int32")[0]) if feat is not None else 0
-            else:
-                rgb, alpha, _ = ops.render_tilecenter_f32(rays_o, unit_dirs, rec, order, offsets, freq, att, *ws, width,
-                                                          height, 8, 8, threshold)
-                pairs, longest, l1_entries, guard = counts.tolist()
-                nonfinite = 0
-            with self._lock:
-                if guard:
-                    if pairs > cap:
-                        self._queue_capacity = int(pairs * 1.3) + 65536
-                    else:
-                        self._queue_scratch_scale = scale * 4
-                    return None
-                if pairs > 0.9 * cap:                       # stay ahead of a slowly growing scene
+                frame = QueuedFrame(name, precision, feat is not None, (rgb, alpha, fmap), tail, held, cap, scale,
+                                    (rays_o, unit_dirs, positions, log_scales, unit_quats, freq, att, ws),
+                                    (rec, order, offsets, width, height, threshold))
+                if defer:
+                    pinned = held.get("pinned")
+                    if pinned is None:
+                        pinned = held["pinned"] = torch.empty(96, dtype=torch.uint8, pin_memory=True)
+                    pinned.copy_(tail, non_blocking=True)
+                    frame.landed = torch.cuda.Event()
+                    frame.landed.record()
+                    frame.host = pinned.numpy()
+                    return frame
+                frame.host = tail.cpu().numpy()
+                return self.finish_frame_queued(frame)
+            rgb, alpha, _ = ops.render_tilecenter_f32(rays_o, unit_dirs, rec, order, offsets, freq, att, *ws, width,
+                                                      height, 8, 8, threshold)
+            frame = QueuedFrame(name, precision, False, (rgb, alpha, None), tail, held, cap, scale, (), ())
+            frame.counts = counts.tolist()
+            return self.finish_frame_queued(frame)
+
+    def finish_frame_queued(self, frame):
+        """Second half of a frame that :meth:`render_frame_queued` returned as a :class:`QueuedFrame`: waits for its
+        read-back and returns (rgb, alpha[, feat]), None (the caller renders the frame the synchronous way) or raises,
+        as :meth:`render_frame_queued` documents.  Call it with the frame's stream current: a fallback render is
+        queued there."""
+        name, precision, held, cap, scale = frame.name, frame.precision, frame.held, frame.cap, frame.scale
+        rgb, alpha, fmap = frame.images
+        if frame.counts is None:
+            if frame.landed is not None:
+                frame.landed.synchronize()
+            host = frame.host
+            held["flags_clear"] = host[32:].tobytes() == _SIXTEEN_ZERO_WORDS
+            pairs, longest, l1_entries, guard = (int(v) for v in host[:32].view("int64"))
+            nonfinite = int(host[32:36].view("int32")[0])
+            pool_ran_out = int(host[36:40].view("int32")[0]) if frame.with_feat else 0
+        else:
+            pairs, longest, l1_entries, guard = frame.counts
+            nonfinite = pool_ran_out = 0
+        with self._lock:
+            if guard:
+                if pairs > cap:
                     self._queue_capacity = int(pairs * 1.3) + 65536
-                redo = feat is not None and bool(nonfinite or pool_ran_out)
-                if precision != "f32" and not redo:
-                    self._mfma_calls += 1
-            if redo:
-                return None                               # rare: the step-by-step path repeats the frame
-            if longest > self.max_tile_prims:
-                raise RuntimeError(f"{name}: tile candidate capacity {self.max_tile_prims} exceeded (maximum observed "
-                                   f"tile length {longest}); refusing to truncate or use an inconsistent "
-                                   "forward/backward order")
-            if nonfinite:
+                else:
+                    self._queue_scratch_scale = scale * 4
+                return None
+            if pairs > 0.9 * cap:                       # stay ahead of a slowly growing scene
+                self._queue_capacity = int(pairs * 1.3) + 65536
+            redo = frame.with_feat and bool(nonfinite or pool_ran_out)
+            if precision != "f32" and not redo:
+                self._mfma_calls += 1
+        if redo:
+            return None                               # rare: the step-by-step path repeats the frame
+        if longest > self.max_tile_prims:
+            raise RuntimeError(f"{name}: tile candidate capacity {self.max_tile_prims} exceeded (maximum observed "
+                               f"tile length {longest}); refusing to truncate or use an inconsistent "
+                               "forward/backward order")
+        if nonfinite:
+            rays_o, unit_dirs, positions, log_scales, unit_quats, freq, att, ws = frame.inputs
+            rec, order, offsets, width, height, threshold = frame.lists
+            with _on_device(rays_o.device):
                 for t in (rays_o, unit_dirs, positions, log_scales, unit_quats, freq, att, *ws):
                     _chk(bool(torch.isfinite(t).all()), "WMMA input is nonfinite; refusing fallback")
                 warnings.warn("WMMA operand/activation overflow: rendering this frame with scalar FP32 instead")
@@ -455,7 +502,7 @@ class TileExt:
                                                           *[w.float() for w in ws], width, height, 8, 8, threshold)
                 _chk(bool(torch.isfinite(rgb).all()) and bool(torch.isfinite(alpha).all()),
                      "Scalar FP32 fallback output is nonfinite")
-        return (rgb, alpha) if feat is None else (rgb, alpha, fmap)
+        return (rgb, alpha) if not frame.with_feat else (rgb, alpha, fmap)
 
     def note_frame_pairs(self, pairs: int):
         """Seed the candidate-buffer estimate of :meth:`render_frame_queued` from a synchronous frame."""

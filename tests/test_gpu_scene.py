@@ -348,6 +348,103 @@ def test_a_flag_raised_by_one_queued_frame_does_not_reach_the_next(device, oracl
     assert ext.rgb_wmma_safety_stats() == [calls0 + 2, fb0 + 1] and held["flags_clear"] is True
 
 
+def _camera_frames(fr, device, count):
+    """`count` pinhole cameras around the frame's scene: (rays_o, rays_d, view matrix, projection) on the device."""
+    from mlp_splatting_amd import synthetic as syn
+    frames = []
+    for k in range(count):
+        a = 0.35 * k
+        c2w = syn.look_at((0.3 + 0.4 * np.sin(a), -0.2 + 0.1 * k, -0.5 - 0.3 * np.cos(a)), (0.0, 0.0, 0.4))
+        ro, rd = syn.pinhole_rays(fr.W, fr.H, fr.f, c2w)
+        frames.append((to_dev(ro, device), to_dev(rd, device), to_dev(syn.view_matrix(c2w), device),
+                       to_dev(fr.proj, device)))
+    return frames
+
+
+def _same_images(got, want):
+    assert len(got) == len(want)
+    for g, w in zip(got, want):
+        g, w = (g if isinstance(g, tuple) else (g,)), (w if isinstance(w, tuple) else (w,))
+        assert len(g) == len(w) and all(torch.equal(a, b) for a, b in zip(g, w))
+
+
+@pytest.mark.parametrize("precision,feature_dim", [("bf16", 0), ("fp16", 0), ("bf16", 48)])
+def test_frames_in_flight_equal_frames_rendered_one_by_one(device, oracle_mod, monkeypatch, precision, feature_dim):
+    # render_frames keeps two (or three) frames queued on streams of its own; every frame is the frame forward() renders
+    from mlp_splatting_amd import cumodel
+    from mlp_splatting_amd.tile_ext import TileExt
+    fr = Frame("cfg1_5k_160x120", n=1500, hidden=32, width=64, height=48, feature_dim=feature_dim)
+    monkeypatch.setattr(cumodel, "_tile_ext", TileExt())
+    scene = _scene_from(fr, device, feature=bool(feature_dim))
+    scene.render_precision = precision
+    frames = _camera_frames(fr, device, 7)
+    kw = dict(score_threshold=fr.thr, return_feature=bool(feature_dim))
+    with torch.inference_mode():
+        want = [scene(f[0], f[1], view_matrix=f[2], proj_matrix=f[3], **kw) for f in frames]
+    assert not torch.equal(want[0][0] if feature_dim else want[0], want[3][0] if feature_dim else want[3])
+    ext = cumodel._tile_ext
+    deferred = []
+    real = ext.render_frame_queued
+    monkeypatch.setattr(ext, "render_frame_queued", lambda *a, **k: (deferred.append(k.get("defer", False)), real(*a, **k))[1])
+    for in_flight in (2, 3):
+        deferred.clear()
+        _same_images(scene.render_frames(frames, fr.thr, return_feature=bool(feature_dim),
+                                         frames_in_flight=in_flight), want)
+        assert deferred == [False] + [True] * 6           # the first frame on the caller's stream, the rest in flight
+    # one frame at a time, and lists too short to overlap anything: plain calls
+    deferred.clear()
+    _same_images(scene.render_frames(frames[:4], fr.thr, return_feature=bool(feature_dim), frames_in_flight=1), want[:4])
+    _same_images(scene.render_frames(frames[:2], fr.thr, return_feature=bool(feature_dim)), want[:2])
+    assert deferred == [False] * 6
+    # a frame in flight whose candidate buffer turns out too small is repeated the synchronous way on its stream
+    calls = []
+    real_bin = ext.frame_binning_queued
+
+    def small_third(*a, **k):
+        calls.append(1)
+        if len(calls) == 3:
+            ext._queue_capacity = 16
+        return real_bin(*a, **k)
+    monkeypatch.setattr(ext, "frame_binning_queued", small_third)
+    _same_images(scene.render_frames(frames, fr.thr, return_feature=bool(feature_dim)), want)
+    assert ext._queue_capacity > 1000
+    monkeypatch.setattr(ext, "frame_binning_queued", real_bin)
+    # forward() afterwards, on the caller's stream, is undisturbed
+    with torch.inference_mode():
+        _same_images([scene(frames[5][0], frames[5][1], view_matrix=frames[5][2], proj_matrix=frames[5][3], **kw)], want[5:6])
+
+
+def test_frames_in_flight_take_the_f32_fallback_on_their_own_stream(device, oracle_mod, monkeypatch):
+    # fp16 cannot hold 1e5: every frame raises the non-finite flag and is rendered again by the f32 kernel, in flight
+    # as in forward(); with the weight back in range the frames come from the matrix cores again
+    import warnings
+    from mlp_splatting_amd import cumodel
+    from mlp_splatting_amd.tile_ext import TileExt
+    fr = Frame("cfg1_5k_160x120", n=1500, hidden=32, width=64, height=48)
+    monkeypatch.setattr(cumodel, "_tile_ext", TileExt())
+    scene = _scene_from(fr, device)
+    scene.render_precision = "fp16"
+    frames = _camera_frames(fr, device, 5)
+    clean = scene.render_frames(frames, fr.thr)
+    with torch.no_grad():
+        kept = scene.W2[:, 3, 5].clone()
+        scene.W2[:, 3, 5] = 1.0e5
+    ext = cumodel._tile_ext
+    calls0, fb0 = ext.rgb_wmma_safety_stats()
+    with pytest.warns(UserWarning, match="scalar FP32 instead"):
+        with torch.inference_mode():
+            want = [scene(f[0], f[1], score_threshold=fr.thr, view_matrix=f[2], proj_matrix=f[3]) for f in frames]
+        flagged = scene.render_frames(frames, fr.thr)
+    _same_images(flagged, want)
+    assert ext.rgb_wmma_safety_stats() == [calls0 + 10, fb0 + 10]
+    with torch.no_grad():
+        scene.W2[:, 3, 5] = kept
+    with warnings.catch_warnings():
+        warnings.simplefilter("error")
+        _same_images(scene.render_frames(frames, fr.thr), clean)
+    assert not torch.equal(flagged[1], clean[1])
+
+
 def test_harness_renders_times_and_scores_a_view(device, oracle_mod):
     """mlp_splatting_amd.harness: the timed view of tools/benchmark_inference.py:121-149, its statistics, PSNR and
     the RGB parity of the feature render, on a frame whose image the oracle pins."""
