@@ -259,6 +259,35 @@ class Workload:
         elapsed = time.perf_counter() - t0
         return timed_steps / elapsed, elapsed, timed_steps
 
+    def timed_in_flight(self, in_flight, frames_per_call, min_seconds):
+        """Frames per second through ``render_frames``: the same frames, `frames_per_call` cameras handed over per
+        call and `in_flight` of them queued on the device at once (the images are those of ``render``; the tests
+        compare them).  One untimed call, then whole calls for at least `min_seconds`.  None for a workload whose
+        lists are handed in by the caller (the mosaic)."""
+        import torch
+        if self.mosaic:
+            return None
+        n = len(self.frames)
+        feature = bool(self.feature_dim)
+
+        def call(first):
+            batch = [(self.frames[i % n][0], self.frames[i % n][1], self.view_of[i % n], self.proj)
+                     for i in range(first, first + frames_per_call)]
+            with torch.inference_mode():
+                self.scene.render_frames(batch, self.thr, return_feature=feature, frames_in_flight=in_flight)
+        call(0)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        done = 0
+        while time.perf_counter() - t0 < min_seconds:
+            call(done)
+            done += frames_per_call
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - t0
+        return {"value": round(done / elapsed, 1), "unit": "frames/s", "ms_per_frame": round(elapsed / done * 1e3, 4),
+                "frames_in_flight": in_flight, "frames_per_call": frames_per_call, "frames": done,
+                "entry": "NeuralPrimitiveSceneTileCUDA.render_frames"}
+
     def probe_stages(self, n_probe=8):
         """The stages of a frame one by one, with HIP events on the launch stream around each as a frame queues it
         (no work counters and no read-back inside a bracket), and the render launch once more, untimed, for its
@@ -363,6 +392,8 @@ def other_workload(name, args, dev):
            "stages": {k: round(st[k], 4) for k in ("bin_ms", "prologue_ms", "sort_ms", "render_ms") +
                       (("product_ms",) if wl.feature_dim else ())},
            "hits_per_launch": int(st["hits"]), "hit_wavefronts_per_launch": int(st["hit_waves"])}
+    if not wl.mosaic:
+        out["two_frames_in_flight"] = wl.timed_in_flight(2, 8 if wl.feature_dim else cycle, 0.25)
     if wl.mosaic:
         # 17 of a tile's 64 pixels hit per step here: the launch is bound by the weight blocks it streams, one
         # 7,808-byte block per (tile, primitive) that hits, plus 40 bytes per pixel
@@ -464,6 +495,10 @@ def main() -> int:
     latency = {k: (round(v, 4) if isinstance(v, float) else v) for k, v in timing_stats(lat).items()}
     latency["frames"] = latency.pop("samples")
 
+    # ---- the same frames with two in flight (frame k+1 queued on a second stream before the host waits for frame k):
+    # reported beside the headline, which stays the frame-after-frame call of the reference's interface
+    in_flight = wl.timed_in_flight(2, len(frames), args.min_seconds) if precision == "bf16" else None
+
     # ---- the stages of a frame alone: HIP events on the stream they are launched on, and the render's work counters
     st = wl.probe_stages(8)
     n_probe = st["n_probe"]
@@ -543,7 +578,7 @@ def main() -> int:
                    "log_scale_mean": cfg["log_scale_mean"],
                    "mlp": f"72-{sc.hidden}-{sc.hidden}-4", "feature_channels": feature_dim,
                    "views_per_call": 4 if mosaic else 1, "entry": "NeuralPrimitiveSceneTileCUDA.forward"},
-        "mpix_per_sec": round(fps * W * H / 1e6, 2), "latency": latency,
+        "mpix_per_sec": round(fps * W * H / 1e6, 2), "latency": latency, "two_frames_in_flight": in_flight,
         "roofline": {"bound": "mfma", "kernel": "render_tilecenter_" + ("mfma" if precision == "bf16" else "f32"),
                      "achieved": round(achieved_tflops, 3), "peak": PEAK[precision], "unit": "TFLOP/s",
                      "frac": round(achieved_tflops / PEAK[precision], 5),

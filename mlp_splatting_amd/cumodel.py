@@ -962,7 +962,7 @@ class NeuralPrimitiveSceneTileCUDA(nn.Module):
         def one(f):
             with torch.no_grad():
                 return self.forward(f[0], f[1], score_threshold, bg_color, f[2], f[3], return_feature=return_feature)
-        eligible = (frames_in_flight > 1 and len(frames) > 2 and self.image_size is not None
+        eligible = (frames_in_flight > 1 and len(frames) > 1 and self.image_size is not None
                     and self._resolve_tile_order_mode() == "tilecenter" and int(self.tile_size) == 8
                     and (with_feat or not return_feature) and plain.get("queued_frames", True)
                     and plain.get("camera_mode", "legacy-centered") != "colmap-native"
@@ -974,16 +974,13 @@ class NeuralPrimitiveSceneTileCUDA(nn.Module):
         ext = self._ensure_tile_ext()
         if not (hasattr(ext, "render_frame_queued") and hasattr(ext, "finish_frame_queued")):
             return [one(f) for f in frames]
-        # The first frame on the caller's stream: whatever is derived from the parameters (geometry records, operand
-        # copies of the weights, tables) is built there, before the lanes read it.
-        results = [one(frames[0])]
         main = torch.cuda.current_stream(device)
         lanes = _render_lanes(device, min(int(frames_in_flight), 4))
         ready = torch.cuda.Event()
         ready.record(main)
         for lane in lanes:
             lane.wait_event(ready)
-        waiting = []                       # (lane, frame, finish) in queue order
+        results, waiting = [], []          # waiting: (lane, frame, finish) in queue order
 
         def finish_oldest():
             lane, f, finish = waiting.pop(0)
@@ -994,14 +991,17 @@ class NeuralPrimitiveSceneTileCUDA(nn.Module):
             results.append(out)
         try:
             with torch.no_grad():
-                for i, f in enumerate(frames[1:]):
+                for i, f in enumerate(frames):
                     lane = lanes[i % len(lanes)]
                     with torch.cuda.stream(lane):
                         finish = self._forward_queued(ext, f[0], f[1], score_threshold, f[2], f[3], bg_color, device,
                                                       with_feat, defer=True)
                     waiting.append((lane, f, finish))
                     if i == 0:
-                        # (should this frame have built something the first did not, the other lanes see it built)
+                        # Whatever is derived from the parameters (geometry records, operand copies of the weights,
+                        # tables) is built by the first frame, on its lane: the other lanes start after it.
+                        if finish is None:
+                            finish_oldest()
                         built = torch.cuda.Event()
                         built.record(lane)
                         for other in lanes[1:]:
@@ -1013,7 +1013,7 @@ class NeuralPrimitiveSceneTileCUDA(nn.Module):
         finally:
             for lane in lanes:
                 main.wait_stream(lane)
-        for out in results[1:]:
+        for out in results:
             for t in (out if isinstance(out, tuple) else (out,)):
                 t.record_stream(main)
         return results

@@ -390,12 +390,13 @@ def test_frames_in_flight_equal_frames_rendered_one_by_one(device, oracle_mod, m
         deferred.clear()
         _same_images(scene.render_frames(frames, fr.thr, return_feature=bool(feature_dim),
                                          frames_in_flight=in_flight), want)
-        assert deferred == [False] + [True] * 6           # the first frame on the caller's stream, the rest in flight
-    # one frame at a time, and lists too short to overlap anything: plain calls
+        assert deferred == [True] * 7
+    # one frame at a time, or a single frame: plain calls
     deferred.clear()
     _same_images(scene.render_frames(frames[:4], fr.thr, return_feature=bool(feature_dim), frames_in_flight=1), want[:4])
+    _same_images(scene.render_frames(frames[:1], fr.thr, return_feature=bool(feature_dim)), want[:1])
     _same_images(scene.render_frames(frames[:2], fr.thr, return_feature=bool(feature_dim)), want[:2])
-    assert deferred == [False] * 6
+    assert deferred == [False] * 5 + [True] * 2
     # a frame in flight whose candidate buffer turns out too small is repeated the synchronous way on its stream
     calls = []
     real_bin = ext.frame_binning_queued
