@@ -37,18 +37,16 @@ __device__ __forceinline__ void half_swap(uint32_t& a, uint32_t& b) {
   b = r[1];
 }
 
-// 16 consecutive floats at src + 16 g  ->  element i = src[2i + g]  (g = lane / 32): eight swaps pair the
-// even entries of the two half-waves.
-__device__ __forceinline__ void load_interleaved16(const float* __restrict__ src, int g, float v[16]) {
-  const mf32x4* __restrict__ s4 = reinterpret_cast<const mf32x4*>(src + 16 * g);
+// 16 consecutive floats at src + 16 g, as loaded (c[q] = floats 4q .. 4q+3)  ->  element i = src[2i + g]
+// (g = lane / 32): eight swaps pair the even entries of the two half-waves.
+__device__ __forceinline__ void interleave16(const mf32x4 c4[4], float v[16]) {
   float c[16];
 #pragma unroll
   for (int q = 0; q < 4; ++q) {
-    const mf32x4 t = s4[q];
-    c[4 * q + 0] = t[0];
-    c[4 * q + 1] = t[1];
-    c[4 * q + 2] = t[2];
-    c[4 * q + 3] = t[3];
+    c[4 * q + 0] = c4[q][0];
+    c[4 * q + 1] = c4[q][1];
+    c[4 * q + 2] = c4[q][2];
+    c[4 * q + 3] = c4[q][3];
   }
 #pragma unroll
   for (int t = 0; t < 8; ++t) {
@@ -58,17 +56,15 @@ __device__ __forceinline__ void load_interleaved16(const float* __restrict__ src
   }
 }
 
-// 8 consecutive floats at src + 8 g  ->  element i = src[2i + g], i < 8 (the rest of v is left alone).
-__device__ __forceinline__ void load_interleaved8(const float* __restrict__ src, int g, float v[16]) {
-  const mf32x4* __restrict__ s4 = reinterpret_cast<const mf32x4*>(src + 8 * g);
+// 8 consecutive floats at src + 8 g, as loaded  ->  element i = src[2i + g], i < 8 (the rest of v is left alone).
+__device__ __forceinline__ void interleave8(const mf32x4 c4[2], float v[16]) {
   float c[8];
 #pragma unroll
   for (int q = 0; q < 2; ++q) {
-    const mf32x4 t = s4[q];
-    c[4 * q + 0] = t[0];
-    c[4 * q + 1] = t[1];
-    c[4 * q + 2] = t[2];
-    c[4 * q + 3] = t[3];
+    c[4 * q + 0] = c4[q][0];
+    c[4 * q + 1] = c4[q][1];
+    c[4 * q + 2] = c4[q][2];
+    c[4 * q + 3] = c4[q][3];
   }
 #pragma unroll
   for (int t = 0; t < 4; ++t) {
@@ -78,9 +74,52 @@ __device__ __forceinline__ void load_interleaved8(const float* __restrict__ src,
   }
 }
 template <int H>
-__device__ __forceinline__ void load_interleaved(const float* __restrict__ src, int g, float v[16]) {
-  if constexpr (H == 32) load_interleaved16(src, g, v);
-  else load_interleaved8(src, g, v);
+__device__ __forceinline__ void interleave(const mf32x4 c4[H / 8], float v[16]) {
+  if constexpr (H == 32) interleave16(c4, v);
+  else interleave8(c4, v);
+}
+
+// What one lane loads of a primitive's layers 1 and 2, as the loads deliver it: row `hid` of W1 (its half g) and
+// the first bias vector (its half g); the same row of W2 and the second bias vector.  Requesting is separate from
+// using, and layer 1 from layer 2: a caller can have the next primitive's layer-1 operands under way while it
+// evaluates this one, and layer 2's arrive behind layer 1's instructions anyway.
+template <int H>
+struct MlpLayer1 {
+  mf32x4 a1[9], b1[H / 8];
+};
+template <int H>
+struct MlpLayer2 {
+  mf32x4 a2[H / 8], b2[H / 8];
+};
+// Hidden unit whose weight row lane (m, g) supplies.
+__device__ __forceinline__ int mfma32_hidden_row(int m) { return 8 * (m >> 3) + 2 * (m & 3) + ((m >> 2) & 1); }
+template <int H>
+__device__ __forceinline__ void request_layer1(const float* __restrict__ W1, const float* __restrict__ b1, int p,
+                                               MlpLayer1<H>& o) {
+  constexpr int IN = 72, HALF = 36;
+  const int lane = threadIdx.x & 63, m = lane & 31, g = lane >> 5;
+  const int hid = mfma32_hidden_row(m);
+  const int row = hid < H ? hid : 0;                       // unused rows read row 0 and supply zeros
+  const mf32x4* __restrict__ s1 = reinterpret_cast<const mf32x4*>(W1 + (size_t)p * (H * IN) + row * IN + HALF * g);
+#pragma unroll
+  for (int q = 0; q < 9; ++q) o.a1[q] = s1[q];
+  const mf32x4* __restrict__ sb1 = reinterpret_cast<const mf32x4*>(b1 + (size_t)p * H + (H / 2) * g);
+#pragma unroll
+  for (int q = 0; q < H / 8; ++q) o.b1[q] = sb1[q];
+}
+template <int H>
+__device__ __forceinline__ void request_layer2(const float* __restrict__ W2, const float* __restrict__ b2, int p,
+                                               MlpLayer2<H>& o) {
+  const int lane = threadIdx.x & 63, m = lane & 31, g = lane >> 5;
+  const int hid = mfma32_hidden_row(m);
+  const int row = hid < H ? hid : 0;
+  const mf32x4* __restrict__ s2 = reinterpret_cast<const mf32x4*>(W2 + (size_t)p * (H * H) + row * H + (H / 2) * g);
+  const mf32x4* __restrict__ sb2 = reinterpret_cast<const mf32x4*>(b2 + (size_t)p * H + (H / 2) * g);
+#pragma unroll
+  for (int q = 0; q < H / 8; ++q) {
+    o.a2[q] = s2[q];
+    o.b2[q] = sb2[q];
+  }
 }
 
 // max(x, +0): v_max_f32 yields the same bits as x > 0 ? x : 0 for every x (NaN -> 0, -0 -> +0).  Written
@@ -110,40 +149,33 @@ __device__ __forceinline__ void encode_direction(float rdx, float rdy, float rdz
 }
 
 // All 64 lanes must be active.  x6 is the lane's own pixel's input (components 0..2 enter through dir,
-// which encode_direction() made from them); out is the lane's own pixel's output.
+// which encode_direction() made from them); out is the lane's own pixel's output.  `w1`, `w2` = the primitive's
+// operands as request_layer1() and request_layer2() loaded them.
 // REC selects the record kernels' layer-2 rounding (bias added after a chain started at zero); MASKS fills
 // masks[0..1] with the ReLU masks of the lane's pixel.
 template <bool REC = false, bool MASKS = REC, int HID = 32>
-__device__ __forceinline__ void mlp_wave_mfma32(const float x6[6], const float* __restrict__ freq,
-                                                const float* __restrict__ att, const float* __restrict__ W1,
-                                                const float* __restrict__ b1, const float* __restrict__ W2,
-                                                const float* __restrict__ b2, const float* __restrict__ W3,
-                                                const float* __restrict__ b3, int p, const DirOperands& dir,
-                                                float out[4], uint32_t* masks = nullptr) {
+__device__ __forceinline__ void mlp_wave_mfma32_with(const MlpLayer1<HID>& w1, const MlpLayer2<HID>& w2, const float x6[6],
+                                                     const float* __restrict__ freq, const float* __restrict__ att,
+                                                     const float* __restrict__ W3, const float* __restrict__ b3, int p,
+                                                     const DirOperands& dir, float out[4], uint32_t* masks = nullptr) {
   static_assert(HID == 32 || HID == 16, "hidden width of the matrix-core f32 evaluation");
-  constexpr int H = HID, IN = 72, HALF = 36, R = H / 2;   // R: accumulator registers in use (hidden units 2i + g)
+  constexpr int H = HID, R = H / 2;   // R: accumulator registers in use (hidden units 2i + g)
   const int lane = threadIdx.x & 63, m = lane & 31, g = lane >> 5;
-  const int hid = 8 * (m >> 3) + 2 * (m & 3) + ((m >> 2) & 1);
-  const bool row_used = hid < H;                           // (always, with 32 hidden units)
-  const int row = row_used ? hid : 0;                      // unused rows read row 0 and supply zeros
+  const bool row_used = mfma32_hidden_row(m) < H;          // (always, with 32 hidden units)
 
   // A operands: lane (m, g) supplies row hid, k = g of every instruction.
-  float a1[HALF];
-  {
-    const mf32x4* __restrict__ s4 = reinterpret_cast<const mf32x4*>(W1 + (size_t)p * (H * IN) + row * IN + HALF * g);
+  float a1[36];
 #pragma unroll
-    for (int q = 0; q < HALF / 4; ++q) {
-      const mf32x4 t = s4[q];
-      a1[4 * q + 0] = row_used ? t[0] : 0.f;
-      a1[4 * q + 1] = row_used ? t[1] : 0.f;
-      a1[4 * q + 2] = row_used ? t[2] : 0.f;
-      a1[4 * q + 3] = row_used ? t[3] : 0.f;
-    }
+  for (int q = 0; q < 9; ++q) {
+    a1[4 * q + 0] = row_used ? w1.a1[q][0] : 0.f;
+    a1[4 * q + 1] = row_used ? w1.a1[q][1] : 0.f;
+    a1[4 * q + 2] = row_used ? w1.a1[q][2] : 0.f;
+    a1[4 * q + 3] = row_used ? w1.a1[q][3] : 0.f;
   }
   float a2[16] = {}, bias1[16] = {}, bias2[16] = {};
-  load_interleaved<H>(W2 + (size_t)p * (H * H) + row * H, g, a2);
-  load_interleaved<H>(b1 + (size_t)p * H, g, bias1);
-  load_interleaved<H>(b2 + (size_t)p * H, g, bias2);
+  interleave<H>(w2.a2, a2);
+  interleave<H>(w1.b1, bias1);
+  interleave<H>(w2.b2, bias2);
   if constexpr (H != 32) {
 #pragma unroll
     for (int i = 0; i < R; ++i) a2[i] = row_used ? a2[i] : 0.f;
@@ -214,6 +246,106 @@ __device__ __forceinline__ void mlp_wave_mfma32(const float x6[6], const float* 
     masks[0] = lo | hi;
     masks[1] = m2;
   }
+}
+
+// One column block: the 32 pixels of HALF a wavefront's usual share, every pixel on two lanes (n, g = 0 / 1) that
+// hold the same pixel state.  Half the matrix instructions of mlp_wave_mfma32_with() per wavefront -- what a launch
+// too small to fill the chip wants, whose time is the time of one wavefront's chain.  Lane (n, g) supplies k = g of
+// every B operand itself (the sine for g = 0, the cosine for g = 1: no swap), the layer-2 results of a pixel are
+// split over its two lanes as before and one swap per pair brings both to both.  dir[j]: the direction half of the
+// encoding in that form (encode_direction_half).  Same chain, same bits.
+__device__ __forceinline__ void encode_direction_half(float rdx, float rdy, float rdz, const float* __restrict__ freq,
+                                                      const float* __restrict__ att, float dir[18]) {
+  const int g = (threadIdx.x & 63) >> 5;
+  const float x3[3] = {rdx, rdy, rdz};
+#pragma unroll
+  for (int c = 0; c < 3; ++c) {
+#pragma unroll
+    for (int f = 0; f < 6; ++f) {
+      float s, co;
+      det_sincos((x3[c] * freq[f]) * att[f], s, co);
+      dir[c * 6 + f] = g ? co : s;
+    }
+  }
+}
+template <int HID>
+__device__ __forceinline__ void mlp_half_mfma32_with(const MlpLayer1<HID>& w1, const MlpLayer2<HID>& w2,
+                                                     const float x6[6], const float* __restrict__ freq,
+                                                     const float* __restrict__ att, const float* __restrict__ W3,
+                                                     const float* __restrict__ b3, int p, const float dir[18],
+                                                     float out[4]) {
+  static_assert(HID == 32 || HID == 16, "hidden width of the matrix-core f32 evaluation");
+  constexpr int H = HID, R = H / 2;
+  const int lane = threadIdx.x & 63, m = lane & 31, g = lane >> 5;
+  const bool row_used = mfma32_hidden_row(m) < H;
+  float a1[36];
+#pragma unroll
+  for (int q = 0; q < 9; ++q) {
+    a1[4 * q + 0] = row_used ? w1.a1[q][0] : 0.f;
+    a1[4 * q + 1] = row_used ? w1.a1[q][1] : 0.f;
+    a1[4 * q + 2] = row_used ? w1.a1[q][2] : 0.f;
+    a1[4 * q + 3] = row_used ? w1.a1[q][3] : 0.f;
+  }
+  float a2[16] = {}, bias1[16] = {}, bias2[16] = {};
+  interleave<H>(w2.a2, a2);
+  interleave<H>(w1.b1, bias1);
+  interleave<H>(w2.b2, bias2);
+  if constexpr (H != 32) {
+#pragma unroll
+    for (int i = 0; i < R; ++i) a2[i] = row_used ? a2[i] : 0.f;
+  }
+  mf32x16 d;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) d[i] = (i < R) ? bias1[i] : 0.f;
+#pragma unroll
+  for (int j = 0; j < 18; ++j) d = __builtin_amdgcn_mfma_f32_32x32x2f32(a1[j], dir[j], d, 0, 0, 0);
+#pragma unroll
+  for (int c = 3; c < 6; ++c) {
+#pragma unroll
+    for (int f = 0; f < 6; ++f) {
+      float s, co;
+      det_sincos((x6[c] * freq[f]) * att[f], s, co);
+      d = __builtin_amdgcn_mfma_f32_32x32x2f32(a1[c * 6 + f], g ? co : s, d, 0, 0, 0);
+    }
+  }
+  mf32x16 e;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) e[i] = (i >= R) ? 0.f : bias2[i];
+#pragma unroll
+  for (int i = 0; i < R; ++i) e = __builtin_amdgcn_mfma_f32_32x32x2f32(a2[i], relu_f32(d[i]), e, 0, 0, 0);
+
+  const float* __restrict__ w3 = W3 + (size_t)p * (4 * H);
+  const float* __restrict__ bb3 = b3 + (size_t)p * 4;
+  float acc[4] = {bb3[0], bb3[1], bb3[2], bb3[3]};
+#pragma unroll
+  for (int i = 0; i < R; ++i) {
+    // register i of lane (n, g) is hidden unit 2i + g of pixel n: after the swap `even` holds the g = 0 lane's
+    // value and `odd` the g = 1 lane's, on both lanes
+    float even = relu_f32(e[i]), odd = even;
+    half_swap(even, odd);
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      acc[k] = fmaf(w3[k * H + 2 * i], even, acc[k]);
+      acc[k] = fmaf(w3[k * H + 2 * i + 1], odd, acc[k]);
+    }
+  }
+#pragma unroll
+  for (int k = 0; k < 4; ++k) out[k] = acc[k];
+}
+
+// The same with the operands requested here.
+template <bool REC = false, bool MASKS = REC, int HID = 32>
+__device__ __forceinline__ void mlp_wave_mfma32(const float x6[6], const float* __restrict__ freq,
+                                                const float* __restrict__ att, const float* __restrict__ W1,
+                                                const float* __restrict__ b1, const float* __restrict__ W2,
+                                                const float* __restrict__ b2, const float* __restrict__ W3,
+                                                const float* __restrict__ b3, int p, const DirOperands& dir,
+                                                float out[4], uint32_t* masks = nullptr) {
+  MlpLayer1<HID> w1;
+  MlpLayer2<HID> w2;
+  request_layer1<HID>(W1, b1, p, w1);
+  request_layer2<HID>(W2, b2, p, w2);
+  mlp_wave_mfma32_with<REC, MASKS, HID>(w1, w2, x6, freq, att, W3, b3, p, dir, out, masks);
 }
 
 }  // namespace mlpsp

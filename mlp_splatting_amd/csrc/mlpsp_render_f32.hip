@@ -47,13 +47,27 @@ MLPSP_API int mlpsp_render_tilecenter_f32(const float* rays_o_dev, const float* 
                      (const PrimRecord*)prim_records_dev, order_dev, tile_offsets_dev, freq_dev, att_dev,         \
                      num_frequencies, W1, b1, W2, b2, W3, b3, num_primitives, hidden, g, wpt, per_xcd, (int)items, threshold,           \
                      out_rgb_dev, out_alpha_dev, out_t_dev, ctr, 0.f, 0.f, HitPool{})
+#define MLPSP_F32_AHEAD_LAUNCH(HT, HALF, UNITS)                                                                   \
+  hipLaunchKernelGGL((render_tilecenter_f32_ahead_kernel<HT, HALF>), dim3((unsigned)(ceil_div_units(UNITS) * kNumXcd)), block, 0, s, \
+                     rays_o_dev, rays_d_dev, (const PrimRecord*)prim_records_dev, order_dev, tile_offsets_dev,    \
+                     freq_dev, att_dev, W1, b1, W2, b2, W3, b3, num_primitives, g, wpt, ceil_div_units(UNITS),    \
+                     (int)(UNITS), threshold, out_rgb_dev, out_alpha_dev, out_t_dev, ctr)
+  const auto ceil_div_units = [](int64_t units) { return (int)((units + kNumXcd - 1) / kNumXcd); };
   if (use_mfma32(hidden, num_frequencies, W1, b1, W2, b2)) {
-    if (hidden == 32) MLPSP_F32_LAUNCH(32, 6, false, true);
+    const int mode = ahead_mode(items, num_primitives, ctr != nullptr);
+    if (mode == 2) {
+      if (hidden == 32) MLPSP_F32_AHEAD_LAUNCH(32, true, 2 * items);
+      else MLPSP_F32_AHEAD_LAUNCH(16, true, 2 * items);
+    } else if (mode == 1) {
+      if (hidden == 32) MLPSP_F32_AHEAD_LAUNCH(32, false, items);
+      else MLPSP_F32_AHEAD_LAUNCH(16, false, items);
+    } else if (hidden == 32) MLPSP_F32_LAUNCH(32, 6, false, true);
     else MLPSP_F32_LAUNCH(16, 6, false, true);
   }
   else if (hidden == 32 && num_frequencies == 6) MLPSP_F32_LAUNCH(32, 6);
   else if (hidden == 16 && num_frequencies == 6) MLPSP_F32_LAUNCH(16, 6);
   else MLPSP_F32_LAUNCH(0, 0);
+#undef MLPSP_F32_AHEAD_LAUNCH
 #undef MLPSP_F32_LAUNCH
   MLPSP_LAUNCH_CHECK();
   return MLPSP_OK;

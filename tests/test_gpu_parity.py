@@ -452,6 +452,41 @@ def test_scalar_and_matrix_core_f32_evaluations_agree_bit_for_bit(device, oracle
     _assert_bits(alpha2, want["alpha"], "alpha (unaligned weights)")
 
 
+@pytest.mark.parametrize("hidden,tile,width,height", [(16, 8, 160, 120), (32, 8, 90, 70), (32, 16, 100, 76)])
+def test_small_launches_take_kernels_that_look_ahead_with_the_same_bits(device, oracle_mod, monkeypatch, hidden, tile,
+                                                                       width, height):
+    """A launch of at most 512 items runs two wavefronts per item, each on 32 of its pixels; up to 1,024 items one
+    wavefront per item with the next entry requested ahead; with work counters never the split form.
+    MLPSP_F32_AHEAD=0/1/2 picks one by hand: the oracle's bits from all three, on lists that carry culled (negative)
+    ids behind the survivors, with edge tiles that are cut by the image border, and the oracle's work counters from
+    the two forms that keep them."""
+    from mlp_splatting_amd import ops
+    fr = Frame("cfg1_5k_160x120", n=3000, hidden=hidden, width=width, height=height, tile=tile, eye=(0.5, -0.3, -0.9))
+    sc = fr.scene
+    cand, off = fr.oracle_lists(oracle_mod)
+    want = oracle_mod.render_tilecenter(*fr.base_numpy(cand, off), *fr.dims)
+    rec = ops.prepare_primitives(_t(sc.positions, device), _t(sc.log_scales, device), _t(sc.quats, device))
+    ro, rd, c, o = _t(fr.rays_o, device), _t(fr.rays_d, device), _t(cand, device), _t(off, device)
+    order, _ = ops.sort_tiles(ro, rd, rec, c, o, fr.W, fr.H, tile, tile, cull_threshold=fr.thr)
+    assert 0.1 < float((order < 0).float().mean()) < 0.9
+    args = (ro, rd, rec, order, o, _t(sc.freq, device), _t(sc.att, device), *[_t(w, device) for w in sc.mlp()], fr.W, fr.H,
+            tile, tile, fr.thr)
+    for mode in ("0", "1", "2", None):
+        if mode is None:
+            monkeypatch.delenv("MLPSP_F32_AHEAD")
+        else:
+            monkeypatch.setenv("MLPSP_F32_AHEAD", mode)
+        rgb, alpha, _ = ops.render_tilecenter_f32(*args)
+        _assert_bits(rgb, want["rgb"], f"rgb (MLPSP_F32_AHEAD={mode})")
+        _assert_bits(alpha, want["alpha"], f"alpha (MLPSP_F32_AHEAD={mode})")
+        counters = torch.zeros(4, dtype=torch.int64, device=device)
+        rgb, alpha, _ = ops.render_tilecenter_f32(*args, counters=counters)
+        _assert_bits(rgb, want["rgb"], f"rgb with counters (MLPSP_F32_AHEAD={mode})")
+        if tile == 8:      # steps with a hit and hits (the culled entries the oracle also walks through never hit)
+            np.testing.assert_array_equal(counters.cpu().numpy()[2:], want["stats"][2:])
+    assert want["alpha"].mean() > 0.3
+
+
 def test_non_finite_activations_take_the_same_path_in_both_f32_evaluations(device, oracle_mod, monkeypatch):
     """Huge and non-finite weights of a few primitives (inf - inf, NaN through a ReLU, overflow to inf) must
     give the oracle's image -- NaN positions included -- from the matrix-core and the scalar kernel."""
