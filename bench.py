@@ -317,10 +317,18 @@ class Workload:
             rec = ops.prepare_primitives(scene.positions.detach(), scene.log_scales.detach(), quats)
             cand, off = ops.bin_legacy(scene.positions.detach(), scene.log_scales.detach(), views, self.proj, W, H, 8, thr,
                                        tile_view_ids=tv)
+            n_cand = int(cand.numel())
             # the binning as a frame queues it: no host synchronisation, candidate buffer sized beforehand
+            # (an RGB frame on the matrix cores takes its lists in per-tile segments: level 2 in one launch)
+            segments = tv is None and feat is None and precision == "bf16"
+            ends = None
             e[0].record()
-            ops.bin_legacy_async(scene.positions.detach(), scene.log_scales.detach(), views, self.proj, W, H, 8, thr,
-                                 cand.numel(), tile_view_ids=tv)
+            if segments:
+                cand, off, ends, _ = ops.bin_segments_async(scene.positions.detach(), scene.log_scales.detach(), views[0],
+                                                            self.proj, W, H, 8, thr)
+            else:
+                ops.bin_legacy_async(scene.positions.detach(), scene.log_scales.detach(), views, self.proj, W, H, 8, thr,
+                                     cand.numel(), tile_view_ids=tv)
             e[1].record()
             pyramids = None
             if tv is None:
@@ -328,7 +336,8 @@ class Workload:
                 # (lists handed in by a caller, the mosaic's, are rendered with torch's unit directions)
                 rd, pyramids, _ = ops.frame_prologue(ro, rd_raw, W, H)
             e[2].record()
-            order, _ = ops.sort_tiles(ro, rd, rec, cand, off, W, H, 8, 8, cull_threshold=thr, tile_pyramids=pyramids)
+            order, _ = ops.sort_tiles(ro, rd, rec, cand, off, W, H, 8, 8, cull_threshold=thr, tile_pyramids=pyramids,
+                                      tile_ends=ends)
             e[3].record()
             counters = torch.zeros(4, dtype=torch.int64, device=dev)
             if feat is not None:
@@ -340,7 +349,8 @@ class Workload:
                                                 stages=lambda k: marks[k].record() if k in marks else None)
             elif precision == "bf16":
                 ops.render_tilecenter_mfma(ro, rd, rec, order, off, freq, att, *weights, W, H, thr, bf16=True,
-                                           packed=packed, check=False, status=flags, status_is_clear=tv is None)
+                                           packed=packed, check=False, status=flags, status_is_clear=tv is None,
+                                           tile_ends=ends)
                 e[4].record()
             else:
                 ops.render_tilecenter_f32(ro, rd, rec, order, off, freq, att, *weights, W, H, 8, 8, thr)
@@ -349,7 +359,7 @@ class Workload:
             # the same render launch once more, untimed, for its work counters (their atomics are not part of a frame)
             if precision == "bf16":
                 ops.render_tilecenter_mfma(ro, rd, rec, order, off, freq, att, *weights, W, H, thr, bf16=True,
-                                           counters=counters, packed=packed)
+                                           counters=counters, packed=packed, tile_ends=ends)
             else:
                 ops.render_tilecenter_f32(ro, rd, rec, order, off, freq, att, *weights, W, H, 8, 8, thr, counters=counters)
             torch.cuda.synchronize()
@@ -363,7 +373,7 @@ class Workload:
             acc["hits"] += int(c[3])
             acc["proc"] += int(c[1])
             acc["hit_waves"] += int(c[2])
-            acc["cand"] += int(cand.numel())
+            acc["cand"] += n_cand
         out = {k: v / n_probe for k, v in acc.items()}
         out["n_probe"] = n_probe
         return out
@@ -392,7 +402,7 @@ def other_workload(name, args, dev):
            "stages": {k: round(st[k], 4) for k in ("bin_ms", "prologue_ms", "sort_ms", "render_ms") +
                       (("product_ms",) if wl.feature_dim else ())},
            "hits_per_launch": int(st["hits"]), "hit_wavefronts_per_launch": int(st["hit_waves"])}
-    if not wl.mosaic:
+    if not wl.mosaic and not args.no_frames_in_flight:
         out["two_frames_in_flight"] = wl.timed_in_flight(2, 8 if wl.feature_dim else cycle, 0.25)
     if wl.mosaic:
         # 17 of a tile's 64 pixels hit per step here: the launch is bound by the weight blocks it streams, one
@@ -445,6 +455,9 @@ def main() -> int:
     ap.add_argument("--no-other-workloads", action="store_true",
                     help="skip the short legs of the feature (cfg5) and mosaic (cfg4) configurations that the default "
                          "run of the headline workload appends under other_workloads")
+    ap.add_argument("--no-frames-in-flight", action="store_true",
+                    help="skip the leg that renders the same frames with two in flight (render_frames): under a kernel "
+                         "trace its overlapping launches would blur the per-kernel durations")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run 4 plain device copies of 1 GiB, the known-size kernel that hardware counter "
                          "readings of a profiled run are scaled by")
@@ -497,7 +510,9 @@ def main() -> int:
 
     # ---- the same frames with two in flight (frame k+1 queued on a second stream before the host waits for frame k):
     # reported beside the headline, which stays the frame-after-frame call of the reference's interface
-    in_flight = wl.timed_in_flight(2, len(frames), args.min_seconds) if precision == "bf16" else None
+    in_flight = None
+    if precision == "bf16" and not args.no_frames_in_flight:
+        in_flight = wl.timed_in_flight(2, len(frames), args.min_seconds)
 
     # ---- the stages of a frame alone: HIP events on the stream they are launched on, and the render's work counters
     st = wl.probe_stages(8)

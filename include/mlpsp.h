@@ -57,7 +57,7 @@ typedef void* mlpsp_stream_t;
 /* Library version (major*10000 + minor*100 + patch).  MLPSP_VERSION is the version this header describes: a caller
  * built against it must find mlpsp_version() == MLPSP_VERSION (argument lists and the PrimRecord layout are not
  * compatible across versions). */
-#define MLPSP_VERSION 302
+#define MLPSP_VERSION 303
 int mlpsp_version(void);
 
 /* Message for one MLPSP_E_* bit, worded as the reference's TORCH_CHECK for that condition
@@ -122,6 +122,25 @@ int mlpsp_bin_legacy_async_device_matrices(const float* positions_dev, const flo
                                            int width, int height, int tile, float threshold, void* scratch_dev,
                                            size_t scratch_bytes, int32_t* tile_offsets_dev, int32_t* candidates_dev,
                                            int64_t cand_capacity, int64_t* counts_dev, mlpsp_stream_t stream);
+/* The lists of mlpsp_bin_legacy_async_device_matrices in SEGMENTS, for a frame that is queued whole: tile t owns
+ * candidates_dev[t * segment_stride .. (t + 1) * segment_stride) and its list -- the same ids in the same ascending
+ * order -- is the first tile_ends_dev[t] - t * segment_stride entries of it; tile_offsets_dev[t] = t * segment_stride
+ * (T + 1 entries), tile_ends_dev holds T entries, candidates_dev T * segment_stride.  The render path accepts at most
+ * its tile capacity (1,536 by default) entries per tile anyway, so with segment_stride = that capacity nothing is
+ * lost, and the binning needs neither a count of the candidates before it writes them nor a
+ * buffer sized by an estimate: level 2 tests and writes in one launch (three launches in all instead of four, and
+ * no candidate-capacity guard).  A tile with more than segment_stride candidates keeps the first segment_stride and
+ * raises counts_dev[1] to its full length (counts_dev[1] is 0 when every tile fits): the caller reports the
+ * capacity error of np_tile_kernels.cu:4578-4588 from it.  counts_dev = {0, that maximum, level-1 scratch entries,
+ * guard}; guard = 1 (level-1 scratch too small) leaves every list empty, as in mlpsp_bin_legacy_async.
+ * mlpsp_sort_tiles and mlpsp_render_tilecenter_mfma_feat take such lists through their tile_ends_dev argument.
+ * No counterpart in the reference (its culling is synchronous PyTorch, scannet/cumodel.py:994-1070). */
+int mlpsp_bin_segments_async_device_matrices(const float* positions_dev, const float* log_scales_dev,
+                                             int num_primitives, const float* view_matrix_dev, const float* proj_dev,
+                                             int width, int height, int tile, float threshold, void* scratch_dev,
+                                             size_t scratch_bytes, int segment_stride, int32_t* tile_offsets_dev,
+                                             int32_t* tile_ends_dev, int32_t* candidates_dev, int64_t* counts_dev,
+                                             mlpsp_stream_t stream);
 int mlpsp_bin_legacy_fill(int num_primitives, int num_views, const int32_t* tile_view_ids_dev, int width,
                           int height, int tile, const void* scratch_dev, size_t scratch_bytes,
                           const int32_t* tile_offsets_dev, int32_t* candidates_dev, mlpsp_stream_t stream);
@@ -180,7 +199,9 @@ int mlpsp_bin_raycone_fill(int num_primitives, int width, int height, int tile, 
  * the culling tests candidates against.  Without them every wavefront of a tile builds the planes from the tile's
  * 64 rays itself.  Keys and order do not depend on it; the two builds of the planes differ in their last bits, so a
  * candidate on the very edge of the culling's margin may be struck by one and not the other (the images are the
- * same: nothing that hits is ever struck). */
+ * same: nothing that hits is ever struck).
+ * tile_ends_dev: NULL (tile t's list ends where tile t + 1's begins: tile_offsets_dev[t + 1]) or T ends of lists
+ * that lie in segments (mlpsp_bin_segments_async_device_matrices); the sorted lists are written to the same places. */
 size_t mlpsp_sort_frame_records_bytes(int num_primitives);
 size_t mlpsp_tile_pyramids_bytes(int width, int height, int tile_w, int tile_h);
 /* The per-frame preparations that need nothing but the rays (and the scene), in ONE launch: the unit directions of
@@ -195,7 +216,8 @@ int mlpsp_sort_tiles(const float* rays_o_dev, const float* rays_d_dev, const voi
                      int num_primitives, const int32_t* candidates_dev, const int32_t* tile_offsets_dev, int width,
                      int height, int tile_w, int tile_h, int key_family, int capacity, float cull_threshold,
                      void* frame_records_dev, int frame_records_ready, const void* tile_pyramids_dev,
-                     int32_t* sorted_ids_dev, float* sorted_keys_dev, mlpsp_stream_t stream);
+                     const int32_t* tile_ends_dev, int32_t* sorted_ids_dev, float* sorted_keys_dev,
+                     mlpsp_stream_t stream);
 
 /* Tile-centre-order forward, scalar f32 (render_tiles_kernel_tilecenter_order,
  * np_tile_kernels.cu:1837-2137; with out_t_dev != NULL also the expected depth of :5432-5719).
@@ -399,7 +421,9 @@ int mlpsp_render_tilecenter_mfma(const float* rays_o_dev, const float* rays_d_de
  * (for timing the two launches apart; 1 and 2 need feat_slots != 0).  MLPSP_STAGE_STATUS_IS_CLEAR may be or-ed in:
  * the caller vouches that the 16 words at status_dev are zero already (it read them back as zero after the previous
  * call on this buffer), and the call queues no clear of them -- one launch less between the sort and the render
- * of a frame. */
+ * of a frame.
+ * tile_ends_dev: NULL, or the ends of lists that lie in segments (see mlpsp_sort_tiles); num_pairs is then the
+ * number of entries of order_dev, gaps included. */
 #define MLPSP_STAGE_STATUS_IS_CLEAR 4
 size_t mlpsp_mfma_feat_pack_bytes(int num_primitives, int feat_slots, int feat_channels);
 int mlpsp_pack_mfma_feat(const float* feat_attr_dev, int num_primitives, int feat_slots, int feat_channels,
@@ -414,7 +438,8 @@ int mlpsp_render_tilecenter_mfma_feat(const float* rays_o_dev, const float* rays
                                       int feat_channels, float gating_beta, float gating_temp, int width, int height,
                                       float threshold, void* workspace_dev, size_t workspace_bytes,
                                       float* out_rgb_dev, float* out_alpha_dev, float* out_feat_dev,
-                                      int32_t* status_dev, int64_t* counters_dev, int stage, mlpsp_stream_t stream);
+                                      int32_t* status_dev, int64_t* counters_dev, int stage,
+                                      const int32_t* tile_ends_dev, mlpsp_stream_t stream);
 
 /* Weight and bias gradients of the per-primitive 72->32->32->4 MLP over a primitive-major CSR of hit records
  * = the Triton kernel _grouped_vjp (scannet/primitive_gemm.py:101-166, launched at :214-230).  Segment g covers

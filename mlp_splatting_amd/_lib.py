@@ -20,7 +20,7 @@ TILE_CAPACITY_MAX = 2048
 PIXEL_HIT_CAPACITY = 256
 PRIM_RECORD_BYTES = 128
 MFMA_PACK_BYTES = 7808
-VERSION = 302      # MLPSP_VERSION of include/mlpsp.h: the interface this binding was written against
+VERSION = 303      # MLPSP_VERSION of include/mlpsp.h: the interface this binding was written against
 STAGE_STATUS_IS_CLEAR = 4
 
 _vp, _i, _f, _i64, _sz = C.c_void_p, C.c_int, C.c_float, C.c_int64, C.c_size_t
@@ -37,6 +37,8 @@ SIGNATURES = {
                                     C.POINTER(_i64), _vp]),
     "mlpsp_bin_legacy_async_device_matrices": (_i, [_vp, _vp, _i, _vp, _vp, _i, _i, _i, _f, _vp, _sz, _vp, _vp, _i64, _vp,
                                                      _vp]),
+    "mlpsp_bin_segments_async_device_matrices": (_i, [_vp, _vp, _i, _vp, _vp, _i, _i, _i, _f, _vp, _sz, _i, _vp, _vp, _vp,
+                                                       _vp, _vp]),
     "mlpsp_bin_legacy_async": (_i, [_vp, _vp, _i, C.POINTER(_f), _i, _vp, C.POINTER(_f), _i, _i, _i, _f, _vp, _sz, _vp, _vp,
                                     _i64, _vp, _vp]),
     "mlpsp_bin_legacy_fill": (_i, [_i, _i, _vp, _i, _i, _i, _vp, _sz, _vp, _vp, _vp]),
@@ -49,7 +51,7 @@ SIGNATURES = {
     "mlpsp_sort_frame_records_bytes": (_sz, [_i]),
     "mlpsp_tile_pyramids_bytes": (_sz, [_i, _i, _i, _i]),
     "mlpsp_frame_prologue": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _vp, _vp, _i, _vp, _vp]),
-    "mlpsp_sort_tiles": (_i, [_vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _vp, _i, _vp, _vp, _vp, _vp]),
+    "mlpsp_sort_tiles": (_i, [_vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _vp, _i, _vp, _vp, _vp, _vp, _vp]),
     "mlpsp_render_tilecenter_f32": (_i, [_vp] * 7 + [_i] + [_vp] * 6 + [_i, _i, _i, _i, _i, _i, _f, _vp, _vp, _vp,
                                                                        _vp, _vp]),
     "mlpsp_render_tilecenter_feat_f32": (_i, [_vp] * 7 + [_i] + [_vp] * 6 + [_i, _i, _vp, _i, _i, _f, _f, _i, _i, _i, _i,
@@ -75,7 +77,7 @@ SIGNATURES = {
     "mlpsp_all_finite": (_i, [_vp, _vp, _i, _vp, _vp]),
     "mlpsp_feat_workspace_bytes": (_sz, [_i64, _i, _i, _i, _i, _i, _i, _i64]),
     "mlpsp_render_tilecenter_mfma_feat": (_i, [_vp] * 5 + [_i64, _vp, _vp, _vp, _i, _i, _vp, _i, _i, _f, _f, _i, _i, _f,
-                                               _vp, _sz, _vp, _vp, _vp, _vp, _vp, _i, _vp]),
+                                               _vp, _sz, _vp, _vp, _vp, _vp, _vp, _i, _vp, _vp]),
     "mlpsp_probe_mfma_bf16": (_i64, [_i, _vp, _vp]),
     "mlpsp_probe_issue": (_i, [C.POINTER(C.c_int32), _i, _vp, _vp, _vp]),
     "mlpsp_grouped_vjp": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _f, _i, _vp,

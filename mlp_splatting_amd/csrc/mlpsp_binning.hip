@@ -519,7 +519,7 @@ __global__ __launch_bounds__(kWideThreads) void bin_level1_fill_kernel(
     const float4* __restrict__ bounds, BinGeom g, const int32_t* __restrict__ l1_counts,
     int32_t* __restrict__ l1_list, float4* __restrict__ l1_bounds, long long l1_capacity,
     const unsigned long long* __restrict__ l1_masks, const int32_t* __restrict__ super_view,
-    int32_t* __restrict__ l1_super, long long* __restrict__ totals) {
+    int32_t* __restrict__ l1_super, long long* __restrict__ totals, long long* __restrict__ clear_word) {
   __shared__ long long s_part[kWideThreads / 64];
   __shared__ long long s_start[kWideThreads];
   const int s = blockIdx.x, S = g.nsx * g.nsy;
@@ -603,6 +603,7 @@ __global__ __launch_bounds__(kWideThreads) void bin_level1_fill_kernel(
     if (s == S - 1) {
       l1_super[S] = (int32_t)min(carry, l1_capacity);
       totals[0] = carry;
+      if (clear_word) *clear_word = 0;      // (the segment form of level 2, the next launch, takes maxima into it)
     }
   }
 }
@@ -930,6 +931,99 @@ __global__ __launch_bounds__(kWideThreads) void bin_level2_fill_kernel(
   level2_fill_tile(tl, first, l1_list, cand, running);
 }
 
+// level 2 in one pass, into segments: tile t owns cand[t * stride .. (t + 1) * stride) and its list is the first
+// ends[t] - t * stride entries of it.  No counting pass and no placing: a wavefront tests its tile's super-tile list 64
+// entries at a time and appends the survivors where its own count stands.  What the lists of a frame lose in
+// compactness they never needed: the sort and the render read a tile's list from its start to its end.  `stride` is
+// the tile capacity of the render path; a tile with more survivors keeps the first `stride` and reports its length
+// into *longest (a maximum; cleared by the level-1 fill launch), which the caller turns into the capacity error.
+// tile_offsets[t] = t * stride (T + 1 of them).  If the level-1 lists overflowed their scratch every list is left
+// empty and the guard word is raised, as in bin_level2_fill_kernel<true>; counts_out = (0, longest if over the
+// capacity, level-1 entries, guard).
+__device__ __forceinline__ int level2_segment_tile(const L2Tile& t, const BinGeom& g, const float4* __restrict__ bounds,
+                                                   const int32_t* __restrict__ l1_list,
+                                                   const float4* __restrict__ l1_bounds,
+                                                   const int32_t* __restrict__ super_view, int32_t* __restrict__ seg,
+                                                   int stride) {
+  const int lane = threadIdx.x & 63;
+  const int lo = t.lo, hi = t.hi, nb = t.nb;
+  const float x0 = t.x0, x1 = t.x1, y0 = t.y0, y1 = t.y1;
+  int running = 0;
+  if (super_view[t.s] == t.view) {
+    const float nanv = __builtin_nanf("");
+    for (int b = 0; b < nb; b += 4) {
+      float4 bb[4];
+      int id[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int j = lo + ((b + u) << 6) + lane;
+        bb[u] = (j < hi) ? l1_bounds[j] : make_float4(nanv, nanv, nanv, nanv);
+        id[u] = (j < hi) ? l1_list[j] : 0;
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        if (b + u < nb) {
+          const bool keep = rect_overlap(bb[u], x0, x1, y0, y1);
+          const unsigned long long m = __ballot(keep);
+          const int at = running + lanes_below(m);
+          if (keep && at < stride) seg[at] = id[u];
+          running += __popcll(m);
+        }
+      }
+    }
+  } else {
+    const float4* __restrict__ vb = bounds + (size_t)t.view * g.N;
+    for (int base = lo; base < hi; base += 64) {
+      const int j = base + lane;
+      bool keep = false;
+      int id = 0;
+      if (j < hi) {
+        id = l1_list[j];
+        keep = rect_overlap(vb[id], x0, x1, y0, y1);
+      }
+      const unsigned long long m = __ballot(keep);
+      const int at = running + lanes_below(m);
+      if (keep && at < stride) seg[at] = id;
+      running += __popcll(m);
+    }
+  }
+  return running;
+}
+
+__global__ __launch_bounds__(kWideThreads) void bin_level2_segments_kernel(
+    const float4* __restrict__ bounds, BinGeom g, const int32_t* __restrict__ tile_view_ids,
+    const int32_t* __restrict__ l1_super, const int32_t* __restrict__ l1_list, const float4* __restrict__ l1_bounds,
+    long long l1_capacity, unsigned long long* __restrict__ l2_masks, long long l2_mask_stride,
+    const int32_t* __restrict__ super_view, const long long* __restrict__ totals, int stride,
+    int32_t* __restrict__ tile_offsets, int32_t* __restrict__ tile_ends, int32_t* __restrict__ cand,
+    long long* __restrict__ counts_out) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int T = g.ntx * g.nty;
+  const int tile = blockIdx.x * kL2Group + wave;
+  const long long l1_entries = totals[0];
+  const bool bad = l1_entries > l1_capacity;
+  if (blockIdx.x == 0 && threadIdx.x == 0) {
+    counts_out[0] = 0;
+    counts_out[2] = l1_entries;
+    counts_out[3] = bad ? 1 : 0;
+  }
+  if (tile >= T) return;
+  const int start = tile * stride;
+  if (lane == 0) {
+    tile_offsets[tile] = start;
+    if (tile == T - 1) tile_offsets[T] = T * stride;
+  }
+  int count = 0;
+  if (!bad) {
+    const L2Tile t = level2_tile(g, tile, tile_view_ids, l1_super, l1_capacity, l2_masks, l2_mask_stride);
+    count = level2_segment_tile(t, g, bounds, l1_list, l1_bounds, super_view, cand + start, stride);
+  }
+  if (lane == 0) {
+    tile_ends[tile] = start + min(count, stride);
+    if (count > stride) atomicMax(reinterpret_cast<unsigned long long*>(counts_out + 1), (unsigned long long)count);
+  }
+}
+
 inline BinGeom make_geom(int N, int K, int W, int H, int ts) {
   BinGeom g;
   g.W = W; g.H = H; g.ts = ts;
@@ -1005,8 +1099,11 @@ struct BoundsSource {
 };
 
 // bounds -> level 1 (count, fill) -> level 2 count [-> scan of the tile counts when the caller fills separately]
+// count_tiles = false stops after level 1 (the segment form of level 2 follows, which counts and fills in one pass
+// and takes its maxima into *clear_word, cleared here).
 int enqueue_bin_levels(const BoundsSource& src, const BinGeom& g, const BinScratch& b, int64_t T,
-                       const int32_t* tile_view_ids_dev, int32_t* tile_offsets_dev, hipStream_t s, bool scan_tiles) {
+                       const int32_t* tile_view_ids_dev, int32_t* tile_offsets_dev, hipStream_t s, bool scan_tiles,
+                       bool count_tiles = true, long long* clear_word = nullptr) {
   const int S = g.nsx * g.nsy;
   // level-1 counts by primitive (super-tile rows in bands that fit LDS): with one view the same launch computes the
   // bounds, with several (and tile_view_ids) it reads them
@@ -1046,8 +1143,9 @@ int enqueue_bin_levels(const BoundsSource& src, const BinGeom& g, const BinScrat
   }
   MLPSP_LAUNCH_CHECK();
   hipLaunchKernelGGL(bin_level1_fill_kernel, dim3(S), dim3(kWideThreads), 0, s, b.bounds, g, b.l1_counts, b.l1_list,
-                     b.l1_bounds, b.l1_capacity, b.l1_masks, b.super_view, b.l1_super, b.totals);
+                     b.l1_bounds, b.l1_capacity, b.l1_masks, b.super_view, b.l1_super, b.totals, clear_word);
   MLPSP_LAUNCH_CHECK();
+  if (!count_tiles) return MLPSP_OK;
   hipLaunchKernelGGL(bin_level2_count_kernel, dim3(level2_groups(T)), dim3(kWideThreads), 0, s, b.bounds, g,
                      tile_view_ids_dev, b.l1_super, b.l1_list, b.l1_bounds, b.l1_capacity, tile_offsets_dev, b.l2_masks,
                      b.l2_mask_stride, b.super_view, b.groups);
@@ -1078,7 +1176,7 @@ int enqueue_bin_count(const float* positions_dev, const float* log_scales_dev, i
                       const float* proj_host, int width, int height, int tile, float threshold, const BinGeom& g,
                       const BinScratch& b, int64_t T, int32_t* tile_offsets_dev, hipStream_t s,
                       bool matrices_in_scratch = false, bool scan_tiles = true, const float* view_dev = nullptr,
-                      const float* proj_dev = nullptr) {
+                      const float* proj_dev = nullptr, bool count_tiles = true, long long* clear_word = nullptr) {
   BoundsSource src{};
   src.positions = positions_dev;
   src.log_scales = log_scales_dev;
@@ -1088,7 +1186,7 @@ int enqueue_bin_count(const float* positions_dev, const float* log_scales_dev, i
     src.mode = 2;
     src.mats = view_dev;
     src.proj_dev = proj_dev;
-    return enqueue_bin_levels(src, g, b, T, tile_view_ids_dev, tile_offsets_dev, s, scan_tiles);
+    return enqueue_bin_levels(src, g, b, T, tile_view_ids_dev, tile_offsets_dev, s, scan_tiles, count_tiles, clear_word);
   }
   const float fx = (proj_host[0] * (float)width) / 2.0f, fy = (proj_host[5] * (float)height) / 2.0f;
   src.focal = (fx + fy) * 0.5f;
@@ -1108,7 +1206,7 @@ int enqueue_bin_count(const float* positions_dev, const float* log_scales_dev, i
                                    hipMemcpyHostToDevice, s));
     }
   }
-  return enqueue_bin_levels(src, g, b, T, tile_view_ids_dev, tile_offsets_dev, s, scan_tiles);
+  return enqueue_bin_levels(src, g, b, T, tile_view_ids_dev, tile_offsets_dev, s, scan_tiles, count_tiles, clear_word);
 }
 
 int check_bin_args(int64_t T, const float* view_matrices_host, const float* proj_host, void* scratch_dev,
@@ -1214,6 +1312,42 @@ MLPSP_API int mlpsp_bin_legacy_async_device_matrices(const float* positions_dev,
   return bin_legacy_async_impl(positions_dev, log_scales_dev, num_primitives, nullptr, 1, nullptr, nullptr, view_matrix_dev,
                                proj_dev, width, height, tile, threshold, scratch_dev, scratch_bytes, tile_offsets_dev,
                                candidates_dev, cand_capacity, counts_dev, (hipStream_t)stream);
+}
+
+MLPSP_API int mlpsp_bin_segments_async_device_matrices(const float* positions_dev, const float* log_scales_dev,
+                                                       int num_primitives, const float* view_matrix_dev,
+                                                       const float* proj_dev, int width, int height, int tile,
+                                                       float threshold, void* scratch_dev, size_t scratch_bytes,
+                                                       int segment_stride, int32_t* tile_offsets_dev,
+                                                       int32_t* tile_ends_dev, int32_t* candidates_dev,
+                                                       int64_t* counts_dev, mlpsp_stream_t stream) {
+  const int64_t T = checked_num_tiles(width, height, tile, tile);
+  if (!view_matrix_dev || !proj_dev || !counts_dev || !tile_ends_dev || !candidates_dev || segment_stride <= 0)
+    return MLPSP_E_ARGUMENT;
+  const int rc = check_bin_args(T, view_matrix_dev, proj_dev, scratch_dev, scratch_bytes, tile_offsets_dev,
+                                num_primitives, 1, width, height, tile, threshold);
+  if (rc != MLPSP_OK) return rc;
+  if (T > 2147483647LL / segment_stride) return MLPSP_E_ARGUMENT;
+  hipStream_t s = (hipStream_t)stream;
+  const BinGeom g = make_geom(num_primitives, 1, width, height, tile);
+  const BinScratch b = carve(scratch_dev, scratch_bytes, num_primitives, 1, g.nsx * g.nsy, g.NC);
+  if (num_primitives == 0) {        // every list empty: [0, 0)
+    MLPSP_HIP_TRY(hipMemsetAsync(tile_offsets_dev, 0, (size_t)(T + 1) * sizeof(int32_t), s));
+    MLPSP_HIP_TRY(hipMemsetAsync(tile_ends_dev, 0, (size_t)T * sizeof(int32_t), s));
+    MLPSP_HIP_TRY(hipMemsetAsync(counts_dev, 0, 4 * sizeof(int64_t), s));
+    return MLPSP_OK;
+  }
+  const int erc = enqueue_bin_count(positions_dev, log_scales_dev, num_primitives, nullptr, 1, nullptr, nullptr, width,
+                                    height, tile, threshold, g, b, T, tile_offsets_dev, s, false, /*scan_tiles=*/false,
+                                    view_matrix_dev, proj_dev, /*count_tiles=*/false,
+                                    reinterpret_cast<long long*>(counts_dev) + 1);
+  if (erc != MLPSP_OK) return erc;
+  hipLaunchKernelGGL(bin_level2_segments_kernel, dim3(level2_groups(T)), dim3(kWideThreads), 0, s, b.bounds, g,
+                     (const int32_t*)nullptr, b.l1_super, b.l1_list, b.l1_bounds, b.l1_capacity, b.l2_masks,
+                     b.l2_mask_stride, b.super_view, b.totals, segment_stride, tile_offsets_dev, tile_ends_dev,
+                     candidates_dev, reinterpret_cast<long long*>(counts_dev));
+  MLPSP_LAUNCH_CHECK();
+  return MLPSP_OK;
 }
 
 MLPSP_API int mlpsp_bin_legacy_fill(int num_primitives, int num_views, const int32_t* tile_view_ids_dev, int width,

@@ -125,15 +125,16 @@ __global__ __launch_bounds__(256) void frame_prologue_kernel(const float* __rest
 // One 256-thread workgroup per tile (mlpsp_sort_tile.hpp); super-blocks of tiles per XCD: the geometry records a
 // tile gathers are mostly those of its neighbours.
 // PYR: the tiles' ray pyramids come from records (the frame prologue's) instead of being built here.
+// Tile t's list is cand[offsets[t] .. ends[t]) (ends = offsets + 1 for lists that follow one another without gaps).
 template <bool PYR>
 __global__ __launch_bounds__(kSortThreads) void sort_tiles_kernel(
     const float* __restrict__ rays_o, const float* __restrict__ rays_d, const PrimRecord* __restrict__ prims,
     const SortRec* __restrict__ frame, const TilePyramidRec* __restrict__ pyramids, const int32_t* __restrict__ cand,
-    const int32_t* __restrict__ offsets, TileGeom g, int family, int capacity, float cull_r2, int num_prims,
-    int32_t* __restrict__ sorted_ids, float* __restrict__ sorted_keys) {
+    const int32_t* __restrict__ offsets, const int32_t* __restrict__ ends, TileGeom g, int family, int capacity,
+    float cull_r2, int num_prims, int32_t* __restrict__ sorted_ids, float* __restrict__ sorted_keys) {
   const int tile = superblock_tile(blockIdx.x, g.ntx, g.nty);
   if (tile < 0) return;
-  const int start = offsets[tile], len = offsets[tile + 1] - start;
+  const int start = offsets[tile], len = ends[tile] - start;
   if (len <= 64 && len <= capacity) {       // a short list: the first wavefront alone, in registers
     if (len > 0 && threadIdx.x < 64)
       sort_small_tile<PYR>(rays_o, rays_d, prims, frame, pyramids, cand, g, family, cull_r2, num_prims, sorted_ids, sorted_keys,
@@ -141,7 +142,7 @@ __global__ __launch_bounds__(kSortThreads) void sort_tiles_kernel(
     return;
   }
   __shared__ SortLds<MLPSP_TILE_CAPACITY_MAX> lds;
-  sort_one_tile<MLPSP_TILE_CAPACITY_MAX, PYR>(lds, rays_o, rays_d, prims, frame, pyramids, cand, offsets, g, family, capacity,
+  sort_one_tile<MLPSP_TILE_CAPACITY_MAX, PYR>(lds, rays_o, rays_d, prims, frame, pyramids, cand, offsets, ends, g, family, capacity,
                                          cull_r2, num_prims, sorted_ids, sorted_keys, tile);
 }
 
@@ -256,8 +257,8 @@ MLPSP_API int mlpsp_sort_tiles(const float* rays_o_dev, const float* rays_d_dev,
                                int num_primitives, const int32_t* candidates_dev, const int32_t* tile_offsets_dev,
                                int width, int height, int tile_w, int tile_h, int key_family, int capacity,
                                float cull_threshold, void* frame_records_dev, int frame_records_ready,
-                               const void* tile_pyramids_dev, int32_t* sorted_ids_dev, float* sorted_keys_dev,
-                               mlpsp_stream_t stream) {
+                               const void* tile_pyramids_dev, const int32_t* tile_ends_dev, int32_t* sorted_ids_dev,
+                               float* sorted_keys_dev, mlpsp_stream_t stream) {
   const int64_t T = checked_num_tiles(width, height, tile_w, tile_h);
   if (T <= 0 || T > 2147483647LL) return MLPSP_E_ARGUMENT;
   if (key_family != MLPSP_KEY_TSTAR && key_family != MLPSP_KEY_DEPTH) return MLPSP_E_ARGUMENT;
@@ -269,6 +270,7 @@ MLPSP_API int mlpsp_sort_tiles(const float* rays_o_dev, const float* rays_d_dev,
   if (reinterpret_cast<uintptr_t>(frame_records_dev) % 64 != 0) return MLPSP_E_ARGUMENT;
   if (reinterpret_cast<uintptr_t>(tile_pyramids_dev) % 32 != 0) return MLPSP_E_ARGUMENT;
   TileGeom g{width, height, tile_w, tile_h, ceil_div(width, tile_w), ceil_div(height, tile_h)};
+  const int32_t* ends = tile_ends_dev ? tile_ends_dev : tile_offsets_dev + 1;
   // squared radius of the threshold ellipsoid in units of the scales, with a 2 % margin on the radius
   float cull_r2 = 0.f;
   if (cull_threshold > 0.f && cull_threshold < 1.f) cull_r2 = -2.0f * logf(cull_threshold) * 1.0404f + 1e-6f;
@@ -282,12 +284,14 @@ MLPSP_API int mlpsp_sort_tiles(const float* rays_o_dev, const float* rays_d_dev,
     hipLaunchKernelGGL(sort_tiles_kernel<true>, dim3(superblock_grid(g.ntx, g.nty)), dim3(kSortThreads), 0,
                        (hipStream_t)stream, rays_o_dev, rays_d_dev, (const PrimRecord*)prim_records_dev,
                        (const SortRec*)frame_records_dev, (const TilePyramidRec*)tile_pyramids_dev, candidates_dev,
-                       tile_offsets_dev, g, key_family, capacity, cull_r2, num_primitives, sorted_ids_dev, sorted_keys_dev);
+                       tile_offsets_dev, ends, g, key_family, capacity, cull_r2, num_primitives, sorted_ids_dev,
+                       sorted_keys_dev);
   else
     hipLaunchKernelGGL(sort_tiles_kernel<false>, dim3(superblock_grid(g.ntx, g.nty)), dim3(kSortThreads), 0,
                        (hipStream_t)stream, rays_o_dev, rays_d_dev, (const PrimRecord*)prim_records_dev,
                        (const SortRec*)frame_records_dev, (const TilePyramidRec*)nullptr, candidates_dev,
-                       tile_offsets_dev, g, key_family, capacity, cull_r2, num_primitives, sorted_ids_dev, sorted_keys_dev);
+                       tile_offsets_dev, ends, g, key_family, capacity, cull_r2, num_primitives, sorted_ids_dev,
+                       sorted_keys_dev);
   MLPSP_LAUNCH_CHECK();
   return MLPSP_OK;
 }

@@ -253,6 +253,7 @@ __device__ __forceinline__ void render_tile_mfma(
     const int tile, const int l, DirWords& s_dir, OriginLds<SP>& s_org, const SinCosTable* table,
     const float* __restrict__ rays_o,
     const float* __restrict__ rays_d, const PrimRecord* __restrict__ prims, const int32_t* __restrict__ order, const int32_t* __restrict__ offsets,
+    const int32_t* __restrict__ ends,
     const float* __restrict__ freq, const float* __restrict__ att, const unsigned char* __restrict__ packed, int N,
     int W, int H, int ntx, float thr, float* __restrict__ out_rgb, float* __restrict__ out_alpha,
     int32_t* __restrict__ status, unsigned long long* __restrict__ counters, int slots, float beta, float temp,
@@ -298,7 +299,7 @@ __device__ __forceinline__ void render_tile_mfma(
   const float reach = 4e-6f * __builtin_sqrtf(fmaxf(-2.f * __logf(thr), 0.f));   // see band_for()
   const bool one_origin = __ballot(valid && !(rox == ox && roy == oy && roz == oz)) == 0ull;
 
-  const int start = offsets[tile], end = offsets[tile + 1];
+  const int start = offsets[tile], end = ends[tile];
   PixelAcc acc = {0.f, 0.f, 0.f, 1.f, 0.f, 0.f};
   HitEmitter em = hit_emitter_begin(hp, 0, start, tile);
   bool live = valid;
@@ -445,7 +446,8 @@ constexpr int kRenderWaves = MLPSP_RENDER_WAVES;
 template <typename T, int SP>
 __global__ __launch_bounds__(64 * kRenderWaves) __attribute__((amdgpu_waves_per_eu(4, 4))) void render_tilecenter_mfma_kernel(
     const float* __restrict__ rays_o, const float* __restrict__ rays_d, const PrimRecord* __restrict__ prims,
-    const int32_t* __restrict__ order, const int32_t* __restrict__ offsets, const float* __restrict__ freq,
+    const int32_t* __restrict__ order, const int32_t* __restrict__ offsets, const int32_t* __restrict__ ends,
+    const float* __restrict__ freq,
     const float* __restrict__ att, const unsigned char* __restrict__ packed, int N, int W, int H, int ntx,
     int per_xcd, int num_tiles, float thr, float* __restrict__ out_rgb, float* __restrict__ out_alpha,
     int32_t* __restrict__ status, unsigned long long* __restrict__ counters, int slots, float beta, float temp,
@@ -466,7 +468,7 @@ __global__ __launch_bounds__(64 * kRenderWaves) __attribute__((amdgpu_waves_per_
                                       num_tiles / ntx);
   if (tile < 0) return;
   render_tile_mfma<T, SP>(tile, (int)threadIdx.x & 63, s_dir[wave], s_org[wave], table, rays_o, rays_d, prims, order, offsets,
-                          freq, att, packed, N, W, H, ntx, thr, out_rgb, out_alpha, status, counters, slots, beta, temp,
+                          ends, freq, att, packed, N, W, H, ntx, thr, out_rgb, out_alpha, status, counters, slots, beta, temp,
                           hp);
 }
 
@@ -823,11 +825,11 @@ inline int feat_pad(int slots) { return slots == 5 ? 8 : 4; }
 
 template <typename E, int SP>
 void launch_mfma(dim3 grid, hipStream_t s, const float* rays_o, const float* rays_d, const void* prims, const int32_t* order,
-                 const int32_t* offsets, const float* freq, const float* att, const void* packed, int N, int W, int H,
+                 const int32_t* offsets, const int32_t* ends, const float* freq, const float* att, const void* packed, int N, int W, int H,
                  int ntx, int per_xcd, int T, float thr, float* rgb, float* alpha, int32_t* status,
                  unsigned long long* ctr, int slots, float beta, float temp, const HitPool& hp) {
   hipLaunchKernelGGL((render_tilecenter_mfma_kernel<E, SP>), dim3(grid.x / kRenderWaves), dim3(64 * kRenderWaves), 0, s, rays_o, rays_d,
-                     (const PrimRecord*)prims, order, offsets, freq, att, (const unsigned char*)packed, N, W, H, ntx,
+                     (const PrimRecord*)prims, order, offsets, ends, freq, att, (const unsigned char*)packed, N, W, H, ntx,
                      per_xcd, T, thr, rgb, alpha, status, ctr, slots, beta, temp, hp);
 }
 }  // namespace
@@ -883,7 +885,8 @@ MLPSP_API int mlpsp_render_tilecenter_mfma_feat(const float* rays_o_dev, const f
                                                 float gating_temp, int width, int height, float threshold,
                                                 void* workspace_dev, size_t workspace_bytes, float* out_rgb_dev,
                                                 float* out_alpha_dev, float* out_feat_dev, int32_t* status_dev,
-                                                int64_t* counters_dev, int stage, mlpsp_stream_t stream) {
+                                                int64_t* counters_dev, int stage, const int32_t* tile_ends_dev,
+                                                mlpsp_stream_t stream) {
   const int64_t T = checked_num_tiles(width, height, 8, 8);
   if (stage < 0 || (stage & ~(3 | MLPSP_STAGE_STATUS_IS_CLEAR)) != 0) return MLPSP_E_ARGUMENT;
   const bool status_is_clear = (stage & MLPSP_STAGE_STATUS_IS_CLEAR) != 0;
@@ -910,11 +913,12 @@ MLPSP_API int mlpsp_render_tilecenter_mfma_feat(const float* rays_o_dev, const f
   if (stage != 2 && !status_is_clear) MLPSP_HIP_TRY(hipMemsetAsync(status_dev, 0, 16 * sizeof(int32_t), s));
   const int per_xcd = (int)((T + kNumXcd - 1) / kNumXcd);
   const int ntx = ceil_div(width, 8);
+  const int32_t* ends = tile_ends_dev ? tile_ends_dev : tile_offsets_dev + 1;
   const dim3 grid(superblock_grid(ntx, ceil_div(height, 8)));
   auto* ctr = reinterpret_cast<unsigned long long*>(counters_dev);
   const int sp = feat_slots ? feat_pad(feat_slots) : 0;
 #define MLPSP_MFMA_GO(TT, SP)                                                                                     \
-  launch_mfma<TT, SP>(grid, s, rays_o_dev, rays_d_dev, prim_records_dev, order_dev, tile_offsets_dev, freq_dev,   \
+  launch_mfma<TT, SP>(grid, s, rays_o_dev, rays_d_dev, prim_records_dev, order_dev, tile_offsets_dev, ends, freq_dev,   \
                       att_dev, packed_dev, num_primitives, width, height, ntx, per_xcd, (int)T, threshold,        \
                       out_rgb_dev, out_alpha_dev, status_dev, ctr, feat_slots, gating_beta, gating_temp, hp)
 #define MLPSP_MFMA_SP(TT)                 \
@@ -955,7 +959,7 @@ MLPSP_API int mlpsp_render_tilecenter_mfma(const float* rays_o_dev, const float*
   return mlpsp_render_tilecenter_mfma_feat(rays_o_dev, rays_d_dev, prim_records_dev, order_dev, tile_offsets_dev, 0,
                                            freq_dev, att_dev, packed_dev, num_primitives, use_bf16, nullptr, 0, 0, 0.f,
                                            0.f, width, height, threshold, nullptr, 0, out_rgb_dev, out_alpha_dev,
-                                           nullptr, status_dev, counters_dev, 0, stream);
+                                           nullptr, status_dev, counters_dev, 0, nullptr, stream);
 }
 
 MLPSP_API int64_t mlpsp_probe_mfma_bf16(int iterations, float* sink_dev, mlpsp_stream_t stream) {

@@ -701,10 +701,10 @@ template <int kSortMax, bool PYR>
 __device__ __forceinline__ void sort_one_tile(SortLds<kSortMax>& lds,
     const float* __restrict__ rays_o, const float* __restrict__ rays_d, const PrimRecord* __restrict__ prims,
     const SortRec* __restrict__ frame, const TilePyramidRec* __restrict__ pyramids, const int32_t* __restrict__ cand,
-    const int32_t* __restrict__ offsets, const TileGeom& g, int family, int capacity, float cull_r2, int num_prims,
-    int32_t* __restrict__ sorted_ids, float* __restrict__ sorted_keys, int tile) {
+    const int32_t* __restrict__ offsets, const int32_t* __restrict__ ends, const TileGeom& g, int family, int capacity,
+    float cull_r2, int num_prims, int32_t* __restrict__ sorted_ids, float* __restrict__ sorted_keys, int tile) {
   const int start = offsets[tile];
-  const int len = offsets[tile + 1] - start;
+  const int len = ends[tile] - start;
   if (len <= 0) return;
   const int n = len < capacity ? len : capacity;
   const int pc = centre_pixel(g, tile);

@@ -905,7 +905,10 @@ class NeuralPrimitiveSceneTileCUDA(nn.Module):
         views, proj = _frame_matrix(view_matrix).reshape(1, 4, 4), _frame_matrix(proj_matrix)
         binned = None
         if hasattr(ext, "frame_binning_queued"):
-            binned = ext.frame_binning_queued(positions, log_scales, views, proj, int(W), int(H), float(score_threshold))
+            # (an RGB frame on the matrix cores takes its lists in per-tile segments: one binning launch less)
+            segments = not with_feat and precision != "f32" and _env("MLPSP_FRAME_SEGMENTS", "1") != "0"
+            binned = ext.frame_binning_queued(positions, log_scales, views, proj, int(W), int(H), float(score_threshold),
+                                              **({"segments": True} if segments else {}))
             if binned is None:
                 return None
         ws = [p.detach().contiguous() for p in params]

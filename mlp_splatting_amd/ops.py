@@ -246,9 +246,66 @@ def bin_legacy_async(positions, log_scales, view_matrices, proj_matrix, W: int, 
     return cand, offsets, counts
 
 
+def bin_segments_async(positions, log_scales, view_matrix, proj_matrix, W: int, H: int, tile: int, threshold: float,
+                       stride: int = TILE_CAPACITY_DEFAULT, scratch_scale: int = 1, counts=None, reuse=None):
+    """The lists of :func:`bin_legacy_async` for one view (both matrices float32 device tensors of 16 elements) in
+    segments of ``stride`` entries per tile, without any host synchronisation and without a count of the candidates
+    before they are written -> (candidates [T * stride], tile_offsets [T + 1] = t * stride, tile_ends [T], counts
+    int64 [4] on the device = 0, the longest list if one exceeds ``stride`` (else 0), level-1 entries, guard).  Tile
+    t's list -- the same ids in the same order -- is ``candidates[tile_offsets[t]:tile_ends[t]]``; a list longer
+    than ``stride`` keeps its first ``stride`` entries.  :func:`sort_tiles` and :func:`render_tilecenter_mfma` take
+    such lists with ``tile_ends``.  ``counts``, ``reuse``: as in :func:`bin_legacy_async`."""
+    positions, log_scales = _f32c(positions, "positions"), _f32c(log_scales, "log_scales")
+    dev = positions.device
+    for m in (view_matrix, proj_matrix):
+        if not (m.is_cuda and m.dtype == torch.float32 and m.numel() == 16 and m.is_contiguous()):
+            raise ValueError("view_matrix and proj_matrix must be contiguous float32 device tensors of 16 elements")
+    n = positions.shape[0]
+    T = num_tiles(W, H, tile, tile)
+    stride = int(stride)
+    if stride <= 0 or T * stride > 2**31 - 1:
+        raise ValueError(f"segment stride {stride} does not fit {T} tiles")
+    lib = _lib.load()
+    nbytes = _bin_scratch_bytes(n, 1, W, H, tile) * int(scratch_scale)
+    held = reuse.get("segments") if reuse is not None else None
+    if held is not None and held[0] == (T, stride, nbytes, dev):
+        offsets, ends, cand, scratch = held[1]
+    else:
+        with torch.inference_mode(False):
+            offsets = torch.empty(T + 1, dtype=torch.int32, device=dev)
+            ends = torch.empty(T, dtype=torch.int32, device=dev)
+            cand = torch.empty(T * stride, dtype=torch.int32, device=dev)
+        scratch = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+        if reuse is not None:
+            reuse["segments"] = ((T, stride, nbytes, dev), (offsets, ends, cand, scratch))
+    if counts is None:
+        counts = torch.empty(4, dtype=torch.int64, device=dev)
+    elif not (counts.is_cuda and counts.dtype == torch.int64 and counts.numel() == 4 and counts.is_contiguous()):
+        raise ValueError("counts must be a contiguous int64 [4] tensor on the device")
+    code = lib.mlpsp_bin_segments_async_device_matrices(_ptr(positions), _ptr(log_scales), n, _ptr(view_matrix),
+                                                        _ptr(proj_matrix), W, H, tile, float(threshold), _ptr(scratch),
+                                                        nbytes, stride, _ptr(offsets), _ptr(ends), _ptr(cand),
+                                                        _ptr(counts), _stream(dev))
+    _check(code, "mlpsp_bin_segments_async_device_matrices")
+    return cand, offsets, ends, counts
+
+
+def compact_segments(order, tile_offsets, tile_ends):
+    """(lists, offsets [T + 1]) of segment lists written one after the other (torch; for the rare caller that needs
+    the reference's layout of lists that came in segments)."""
+    starts = tile_offsets[:-1].long()
+    lengths = tile_ends.long() - starts
+    offsets = torch.zeros(starts.numel() + 1, dtype=torch.int64, device=order.device)
+    offsets[1:] = torch.cumsum(lengths, 0)
+    total = int(offsets[-1].item())
+    tile_of = torch.repeat_interleave(torch.arange(starts.numel(), device=order.device), lengths, output_size=total)
+    within = torch.arange(total, device=order.device) - offsets[:-1][tile_of]
+    return order[starts[tile_of] + within].contiguous(), offsets.to(torch.int32)
+
+
 def sort_tiles(rays_o, rays_d, records, candidates, tile_offsets, W, H, TW, TH, family=_lib.KEY_TSTAR,
                capacity=TILE_CAPACITY_DEFAULT, want_keys=False, cull_threshold=0.0, frame_records=None,
-               tile_pyramids=None):
+               tile_pyramids=None, tile_ends=None):
     """Materialised per-tile depth order: (sorted_ids [P], sorted_keys [P] | None).
 
     With ``cull_threshold`` (the render's score threshold) candidates that provably hit no ray of their
@@ -257,8 +314,13 @@ def sort_tiles(rays_o, rays_d, records, candidates, tile_offsets, W, H, TW, TH, 
     and order do not depend on it), or True to let this call write them first (one more launch, which on one MI355X
     costs a frame more than the sort kernel gains), or False.  None = what ``MLPSP_SORT_FRAME_RECORDS`` says, off
     unless it is 1.  ``tile_pyramids``: what :func:`frame_prologue` returned for these rays and this tile size (the
-    culling's per-tile planes, which the sort otherwise builds in every wavefront of a tile; same output)."""
+    culling's per-tile planes, which the sort otherwise builds in every wavefront of a tile; same output).
+    ``tile_ends``: the int32 [T] ends of lists that lie in segments (:func:`bin_segments_async`); the sorted lists
+    come back in the same places, what lies between them is not written."""
     dev = rays_o.device
+    if tile_ends is not None and not (tile_ends.is_cuda and tile_ends.dtype == torch.int32 and tile_ends.is_contiguous()
+                                      and tile_ends.numel() == tile_offsets.numel() - 1):
+        raise ValueError("tile_ends must be a contiguous int32 device tensor with one entry per tile")
     sorted_ids = torch.empty_like(candidates)
     keys = torch.empty(candidates.numel(), dtype=torch.float32, device=dev) if want_keys else None
     if candidates.numel() == 0:
@@ -281,7 +343,8 @@ def sort_tiles(rays_o, rays_d, records, candidates, tile_offsets, W, H, TW, TH, 
         raise ValueError("tile_pyramids must be the uint8 buffer frame_prologue() returned for this frame and tile size")
     code = lib.mlpsp_sort_tiles(_ptr(rays_o), _ptr(rays_d), _ptr(records), num_primitives, _ptr(candidates),
                                 _ptr(tile_offsets), W, H, TW, TH, int(family), int(capacity), float(cull_threshold),
-                                _ptr(scratch), ready, _ptr(tile_pyramids), _ptr(sorted_ids), _ptr(keys), _stream(dev))
+                                _ptr(scratch), ready, _ptr(tile_pyramids), _ptr(tile_ends), _ptr(sorted_ids), _ptr(keys),
+                                _stream(dev))
     _check(code, "mlpsp_sort_tiles")
     return sorted_ids, keys
 
@@ -558,13 +621,13 @@ def pack_mfma_weights(W1, b1, W2, b2, W3, b3, bf16=True):
 
 def render_tilecenter_mfma(rays_o, rays_d, records, order, tile_offsets, freq, att, W1, b1, W2, b2, W3, b3, W, H,
                            threshold, bf16=True, counters=None, packed=None, check=True, status=None,
-                           status_is_clear=False):
+                           status_is_clear=False, tile_ends=None):
     """Matrix-core tile-centre forward (8x8 tiles) -> (rgb, alpha, nonfinite).
 
     ``nonfinite`` is a bool when ``check`` (one 4-byte readback) or the int32 device flag otherwise.  ``status``: an
     int32 [16] device tensor for the flag words (word 0 = non-finite), allocated here when omitted.
     ``status_is_clear``: the caller read all 16 words of ``status`` back as zero after the previous call that used
-    it, so no clear is queued in front of the kernel.
+    it, so no clear is queued in front of the kernel.  ``tile_ends``: as in :func:`sort_tiles`.
     """
     dev = rays_o.device
     if freq.numel() != 6:
@@ -577,12 +640,14 @@ def render_tilecenter_mfma(rays_o, rays_d, records, order, tile_offsets, freq, a
     flag = status if status is not None else torch.empty(16, dtype=torch.int32, device=dev)
     if not (flag.is_cuda and flag.dtype == torch.int32 and flag.numel() == 16 and flag.is_contiguous()):
         raise ValueError("status must be a contiguous int32 [16] tensor on the device")
-    if status_is_clear and status is not None:
-        # (the RGB entry point is the feature entry point without features; only that one takes the stage word)
+    if (status_is_clear and status is not None) or tile_ends is not None:
+        # (the RGB entry point is the feature entry point without features; only that one takes the stage word and
+        # the ends of lists in segments)
+        stage = _lib.STAGE_STATUS_IS_CLEAR if (status_is_clear and status is not None) else 0
         code = _lib.load().mlpsp_render_tilecenter_mfma_feat(
             _ptr(rays_o), _ptr(rays_d), _ptr(records), _ptr(order), _ptr(tile_offsets), 0, _ptr(freq), _ptr(att),
             _ptr(packed), W1.shape[0], int(bool(bf16)), None, 0, 0, 0.0, 0.0, W, H, float(threshold), None, 0, _ptr(rgb),
-            _ptr(alpha), None, _ptr(flag), _ptr(counters), _lib.STAGE_STATUS_IS_CLEAR, _stream(dev))
+            _ptr(alpha), None, _ptr(flag), _ptr(counters), stage, _ptr(tile_ends), _stream(dev))
     else:
         code = _lib.load().mlpsp_render_tilecenter_mfma(
             _ptr(rays_o), _ptr(rays_d), _ptr(records), _ptr(order), _ptr(tile_offsets), _ptr(freq), _ptr(att),
@@ -644,7 +709,7 @@ def render_tilecenter_mfma_feat(rays_o, rays_d, records, order, tile_offsets, fr
             _ptr(rays_o), _ptr(rays_d), _ptr(records), _ptr(order), _ptr(tile_offsets), pairs, _ptr(freq), _ptr(att),
             _ptr(packed), W1.shape[0], int(bool(bf16)), _ptr(packed_feat), slots, ch, float(beta), float(temp), W, H,
             float(threshold), _ptr(workspace), ws_bytes, _ptr(rgb), _ptr(alpha), _ptr(feat), _ptr(flag), _ptr(counters),
-            stage | clear_bit, _stream(dev))
+            stage | clear_bit, None, _stream(dev))
         _check(code, "mlpsp_render_tilecenter_mfma_feat")
         return code
 

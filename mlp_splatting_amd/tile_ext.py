@@ -326,14 +326,20 @@ class TileExt:
     # ------------------------------------------------------------------------------------------
     # a whole frame queued without a host synchronisation in its middle (no counterpart in the reference)
     # ------------------------------------------------------------------------------------------
-    def frame_binning_queued(self, positions, log_scales, view_matrices, proj_matrix, width, height, threshold):
+    def frame_binning_queued(self, positions, log_scales, view_matrices, proj_matrix, width, height, threshold,
+                             segments=False):
         """First half of :meth:`render_frame_queued`: the frame's binning, queued.  It needs nothing but the
         primitives and the camera, so a caller queues it before it prepares anything else for the frame (ray
         directions, weights): the device works through the binning while the host does that.  Returns what
-        :meth:`render_frame_queued` takes as ``binned``, or None when no candidate-buffer estimate exists yet."""
+        :meth:`render_frame_queued` takes as ``binned``, or None when no candidate-buffer estimate exists yet.
+        ``segments``: every tile's list in a segment of ``max_tile_prims`` entries of its own
+        (:func:`ops.bin_segments_async`: one launch less, no estimate needed), when the camera's matrices are on the
+        device; for frames whose render takes such lists (RGB on the matrix cores)."""
         with self._lock:
             cap, scale = self._queue_capacity, self._queue_scratch_scale
-        if cap <= 0:
+        segments = (segments and all(m.is_cuda and m.dtype == torch.float32 and m.numel() == 16 and m.is_contiguous()
+                                     for m in (view_matrices, proj_matrix)))
+        if cap <= 0 and not segments:
             return None
         with _on_device(positions.device):
             # counts of the binning (4 x int64) and flag words of the render (16 x int32) share one buffer: the
@@ -346,10 +352,15 @@ class TileExt:
                 held["tail"] = (fresh, fresh[:32].view(torch.int64))
                 held["flags_clear"] = False
             tail, counts_view = held["tail"]
+            if segments:
+                cand, offsets, ends, counts = ops.bin_segments_async(
+                    positions, log_scales, view_matrices, proj_matrix, int(width), int(height), 8, float(threshold),
+                    stride=self.max_tile_prims, scratch_scale=scale, counts=counts_view, reuse=held)
+                return cand, offsets, counts, tail, cap, scale, held, ends
             cand, offsets, counts = ops.bin_legacy_async(positions, log_scales, view_matrices, proj_matrix, int(width),
                                                          int(height), 8, float(threshold), cap, scratch_scale=scale,
                                                          counts=counts_view, reuse=held)
-        return cand, offsets, counts, tail, cap, scale, held
+        return cand, offsets, counts, tail, cap, scale, held, None
 
     def _frame_buffers(self, device):
         """The reusable buffers of queued frames, per (thread, device, stream)."""
@@ -404,7 +415,9 @@ class TileExt:
                                                threshold)
             if binned is None:
                 return None
-        cand, offsets, counts, tail, cap, scale, held = binned
+        cand, offsets, counts, tail, cap, scale, held, ends = binned
+        if ends is not None and (feat is not None or precision == "f32"):
+            raise ValueError("lists in segments are for RGB frames on the matrix cores")
         status = tail[32:].view(torch.int32)
         # The flag words live in a buffer that this thread's frames use one after the other, and every frame ends by
         # reading them back: if the last frame read sixteen zeros they are still zero, and the render's own clear (a
@@ -416,7 +429,7 @@ class TileExt:
             rec = self._records(positions, log_scales, unit_quats)
             order, _ = ops.sort_tiles(rays_o, unit_dirs, rec, cand, offsets, width, height, 8, 8, _lib.KEY_TSTAR,
                                       self.max_tile_prims, cull_threshold=threshold, frame_records=frame_records,
-                                      tile_pyramids=tile_pyramids)
+                                      tile_pyramids=tile_pyramids, tile_ends=ends)
             fmap, pool_ran_out = None, 0
             if precision != "f32":
                 packed = self._packed_weights(list(ws), precision == "bf16")
@@ -424,7 +437,7 @@ class TileExt:
                     rgb, alpha, _ = ops.render_tilecenter_mfma(rays_o, unit_dirs, rec, order, offsets, freq, att, *ws,
                                                                width, height, threshold, bf16=(precision == "bf16"),
                                                                packed=packed, check=False, status=status,
-                                                               status_is_clear=flags_clear)
+                                                               status_is_clear=flags_clear, tile_ends=ends)
                 else:
                     packed_feat, bad_attr = self._packed_feat(feat[0])
                     if bad_attr:
@@ -435,7 +448,7 @@ class TileExt:
                         status_is_clear=flags_clear)
                 frame = QueuedFrame(name, precision, feat is not None, (rgb, alpha, fmap), tail, held, cap, scale,
                                     (rays_o, unit_dirs, positions, log_scales, unit_quats, freq, att, ws),
-                                    (rec, order, offsets, width, height, threshold))
+                                    (rec, order, offsets, width, height, threshold, ends))
                 if defer:
                     pinned = held.get("pinned")
                     if pinned is None:
@@ -491,8 +504,10 @@ class TileExt:
                                "forward/backward order")
         if nonfinite:
             rays_o, unit_dirs, positions, log_scales, unit_quats, freq, att, ws = frame.inputs
-            rec, order, offsets, width, height, threshold = frame.lists
+            rec, order, offsets, width, height, threshold, ends = frame.lists
             with _on_device(rays_o.device):
+                if ends is not None:      # (the f32 kernel reads lists that follow one another)
+                    order, offsets = ops.compact_segments(order, offsets, ends)
                 for t in (rays_o, unit_dirs, positions, log_scales, unit_quats, freq, att, *ws):
                     _chk(bool(torch.isfinite(t).all()), "WMMA input is nonfinite; refusing fallback")
                 warnings.warn("WMMA operand/activation overflow: rendering this frame with scalar FP32 instead")

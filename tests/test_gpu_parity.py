@@ -102,6 +102,71 @@ def test_binning_with_more_chunks_than_a_workgroup_takes_at_once(device, oracle_
     np.testing.assert_array_equal(cand2.cpu().numpy()[:pairs], want_cand)
 
 
+@pytest.mark.parametrize("n,width,height", [(5000, 160, 120), (300000, 96, 64), (1500, 21, 13)])
+def test_lists_in_segments_are_the_oracles_lists(device, oracle_mod, n, width, height):
+    """mlpsp_bin_segments_async_device_matrices: every tile's list in a segment of its own, written by a level 2 that
+    tests and writes in one launch.  The same ids in the same order as the oracle's lists; a stride below the longest
+    list keeps the first `stride` entries and reports the full length; the sort and the matrix-core render read such
+    lists through their ends and give what they give for the lists written one after the other."""
+    from mlp_splatting_amd import ops, synthetic as syn
+    if n == 300000:
+        rng = np.random.default_rng(3)
+        pos = (rng.random((n, 3), dtype=np.float32) * 4 - 2).astype(np.float32)
+        logs = (rng.standard_normal((n, 3)).astype(np.float32) * np.float32(0.3) - np.float32(5.5)).astype(np.float32)
+        view = syn.view_matrix(syn.look_at((0.3, -0.2, -2.5), (0.0, 0.0, 0.4)))
+        proj, thr = syn.projection_matrix(60.0, width, height), 5e-3
+        fr = None
+    else:
+        fr = Frame("cfg1_5k_160x120", n=n, hidden=32, width=width, height=height)
+        pos, logs, view, proj, thr = fr.scene.positions, fr.scene.log_scales, fr.view, fr.proj, fr.thr
+    want_cand, want_off = oracle_mod.bin_legacy(pos, logs, view[None], proj, width, height, 8, thr)
+    lengths = np.diff(want_off)
+    T, longest = lengths.size, int(lengths.max())
+    p, l, v, pr = _t(pos, device), _t(logs, device), _t(view, device), _t(proj, device)
+    for stride in (longest, longest + 37, max(longest // 2, 1)):
+        cand, off, ends, counts = ops.bin_segments_async(p, l, v, pr, width, height, 8, thr, stride=stride)
+        off_h, ends_h, cand_h = off.cpu().numpy(), ends.cpu().numpy(), cand.cpu().numpy()
+        np.testing.assert_array_equal(off_h, np.arange(T + 1) * stride)
+        np.testing.assert_array_equal(ends_h - off_h[:-1], np.minimum(lengths, stride))
+        for t in range(T):
+            np.testing.assert_array_equal(cand_h[off_h[t]:ends_h[t]], want_cand[want_off[t]:want_off[t] + min(lengths[t], stride)])
+        pairs, over, l1_entries, guard = counts.tolist()
+        assert (pairs, over, guard) == (0, longest if longest > stride else 0, 0) and l1_entries > 0
+    if fr is None:
+        return
+    # sort and render through the ends
+    sc = fr.scene
+    stride = longest + 5
+    cand, off, ends, _ = ops.bin_segments_async(p, l, v, pr, width, height, 8, thr, stride=stride)
+    rec = ops.prepare_primitives(p, l, _t(sc.quats, device))
+    ro, rd = _t(fr.rays_o, device), _t(fr.rays_d, device)
+    c, o = _t(want_cand, device), _t(want_off, device)
+    plain, plain_keys = ops.sort_tiles(ro, rd, rec, c, o, width, height, 8, 8, cull_threshold=thr, want_keys=True)
+    seg, seg_keys = ops.sort_tiles(ro, rd, rec, cand, off, width, height, 8, 8, cull_threshold=thr, want_keys=True, tile_ends=ends)
+    plain, seg, plain_keys, seg_keys = plain.cpu().numpy(), seg.cpu().numpy(), plain_keys.cpu().numpy(), seg_keys.cpu().numpy()
+    for t in range(T):
+        np.testing.assert_array_equal(seg[t * stride:t * stride + lengths[t]], plain[want_off[t]:want_off[t + 1]])
+        assert np.array_equal(bits(seg_keys[t * stride:t * stride + lengths[t]]), bits(plain_keys[want_off[t]:want_off[t + 1]]))
+    args = (_t(sc.freq, device), _t(sc.att, device), *[_t(w, device) for w in sc.mlp()], width, height, thr)
+    for bf16 in (True, False):
+        a = ops.render_tilecenter_mfma(ro, rd, rec, _t(plain, device), o, *args, bf16=bf16)
+        b = ops.render_tilecenter_mfma(ro, rd, rec, _t(seg, device), off, *args, bf16=bf16, tile_ends=ends)
+        assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1]) and a[2] == b[2]
+        assert float(a[1].mean()) > 0.2
+    comp, comp_off = ops.compact_segments(_t(seg, device), off, ends)
+    np.testing.assert_array_equal(comp.cpu().numpy(), plain)
+    np.testing.assert_array_equal(comp_off.cpu().numpy(), want_off)
+
+
+def test_lists_in_segments_without_primitives(device):
+    from mlp_splatting_amd import ops
+    none = torch.empty(0, 3, dtype=torch.float32, device=device)
+    eye = torch.eye(4, dtype=torch.float32, device=device)
+    cand, off, ends, counts = ops.bin_segments_async(none, none, eye, eye.clone(), 40, 24, 8, 1e-3, stride=16)
+    assert cand.numel() == 15 * 16 and counts.tolist() == [0, 0, 0, 0]
+    assert not off.any() and not ends.any()
+
+
 def test_binning_with_several_views_and_no_view_per_tile(device, oracle_mod):
     """Several view matrices without tile_view_ids: every tile is binned against view 0 (level 1 then runs the walk
     over (chunk, super-tile) pairs with all the views, a superset that level 2 cuts down)."""

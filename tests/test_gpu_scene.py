@@ -273,6 +273,7 @@ def test_queued_frames_equal_step_by_step_frames(device, oracle_mod, monkeypatch
     from mlp_splatting_amd import cumodel
     from mlp_splatting_amd.tile_ext import TileExt
     fr = Frame("cfg1_5k_160x120", n=1500, hidden=32, width=64, height=48)
+    monkeypatch.setenv("MLPSP_FRAME_SEGMENTS", "0")
     for precision in ("f32", "bf16"):
         monkeypatch.setattr(cumodel, "_tile_ext", TileExt())
         scene = _scene_from(fr, device)
@@ -289,7 +290,8 @@ def test_queued_frames_equal_step_by_step_frames(device, oracle_mod, monkeypatch
         monkeypatch.setattr(ext, "render_frame_queued", lambda *a, **k: (calls.append(1), real(*a, **k))[1])
         assert torch.equal(_call(scene, fr, device), ref) and calls == [1]
         # an estimate that is too small: the lists were left empty on the device, the frame is repeated
-        # step by step and the estimate grows
+        # step by step and the estimate grows (lists in segments, which RGB frames on the matrix cores take, need
+        # no estimate: switched off for this test)
         ext._queue_capacity = 16
         assert torch.equal(_call(scene, fr, device), ref) and ext._queue_capacity > 1000
         assert torch.equal(_call(scene, fr, device), ref)
@@ -312,6 +314,39 @@ def test_queued_frames_equal_step_by_step_frames(device, oracle_mod, monkeypatch
     cumodel._tile_ext.max_tile_prims = longest - 1
     with pytest.raises(RuntimeError, match=f"capacity {longest - 1} exceeded \\(maximum observed tile length {longest}\\)"):
         _call(scene, fr, device)
+
+
+def test_queued_rgb_frames_take_their_lists_in_segments(device, oracle_mod, monkeypatch):
+    # An RGB frame on the matrix cores is queued with every tile's list in a segment of its own: no candidate-buffer
+    # estimate, so the very first frame is queued too; the same image as the step-by-step frame; a tile beyond the
+    # capacity raises the reference's error with the length observed; MLPSP_FRAME_SEGMENTS=0 takes the other lists.
+    from mlp_splatting_amd import cumodel, ops
+    from mlp_splatting_amd.tile_ext import TileExt
+    fr = Frame("cfg1_5k_160x120", n=1500, hidden=32, width=64, height=48)
+    monkeypatch.setattr(cumodel, "_tile_ext", TileExt())
+    scene = _scene_from(fr, device)
+    scene.render_precision = "bf16"
+    scene.queued_frames = False
+    ref = _call(scene, fr, device)
+    scene.queued_frames = True
+    ext = cumodel._tile_ext
+    ext._queue_capacity = 0
+    used = []
+    real = ops.bin_segments_async
+    monkeypatch.setattr(ops, "bin_segments_async", lambda *a, **k: (used.append(k.get("stride")), real(*a, **k))[1])
+    assert torch.equal(_call(scene, fr, device), ref) and used == [ext.max_tile_prims] and ext._queue_capacity == 0
+    assert torch.equal(_call(scene, fr, device), ref) and len(used) == 2
+    monkeypatch.setenv("MLPSP_FRAME_SEGMENTS", "0")
+    assert torch.equal(_call(scene, fr, device), ref) and len(used) == 2
+    monkeypatch.delenv("MLPSP_FRAME_SEGMENTS")
+    cand, off = fr.oracle_lists(oracle_mod)
+    longest = int(np.diff(off).max())
+    ext.max_tile_prims = longest - 1
+    with pytest.raises(RuntimeError, match=f"capacity {longest - 1} exceeded \\(maximum observed tile length {longest}\\)"):
+        _call(scene, fr, device)
+    assert used[-1] == longest - 1
+    ext.max_tile_prims = longest
+    assert torch.equal(_call(scene, fr, device), ref)
 
 
 def test_a_flag_raised_by_one_queued_frame_does_not_reach_the_next(device, oracle_mod, monkeypatch):
@@ -398,6 +433,9 @@ def test_frames_in_flight_equal_frames_rendered_one_by_one(device, oracle_mod, m
     _same_images(scene.render_frames(frames[:2], fr.thr, return_feature=bool(feature_dim)), want[:2])
     assert deferred == [False] * 5 + [True] * 2
     # a frame in flight whose candidate buffer turns out too small is repeated the synchronous way on its stream
+    # (with lists in segments, which RGB frames take, there is no such buffer: switched off from here on)
+    monkeypatch.setenv("MLPSP_FRAME_SEGMENTS", "0")
+    _same_images(scene.render_frames(frames[:3], fr.thr, return_feature=bool(feature_dim)), want[:3])
     calls = []
     real_bin = ext.frame_binning_queued
 
