@@ -291,3 +291,23 @@ def test_harness_statistics_closed_forms():
     assert math.isclose(q["global_psnr_db"], -10.0 * math.log10(pooled), abs_tol=1e-5)
     with pytest.raises(ValueError):
         quality([a], [])
+
+
+def test_compact_segments_writes_segment_lists_one_after_the_other():
+    """ops.compact_segments (plain torch): lists that lie in per-tile segments, with gaps and an empty tile, come out
+    as the reference's layout -- ids in tile order and T + 1 offsets."""
+    import torch
+    from mlp_splatting_amd import ops
+    stride = 5
+    lists = [[7, 9], [], [1, 2, 3, 4, 5], [11]]
+    order = torch.full((len(lists) * stride,), -99, dtype=torch.int32)
+    ends = torch.empty(len(lists), dtype=torch.int32)
+    for t, ids in enumerate(lists):
+        order[t * stride:t * stride + len(ids)] = torch.tensor(ids, dtype=torch.int32)
+        ends[t] = t * stride + len(ids)
+    offsets = torch.arange(len(lists) + 1, dtype=torch.int32) * stride
+    flat, off = ops.compact_segments(order, offsets, ends)
+    assert flat.tolist() == [7, 9, 1, 2, 3, 4, 5, 11] and off.tolist() == [0, 2, 2, 7, 8]
+    assert flat.dtype == torch.int32 and off.dtype == torch.int32
+    none, off0 = ops.compact_segments(order, offsets, offsets[:-1].clone())
+    assert none.numel() == 0 and off0.tolist() == [0, 0, 0, 0, 0]
