@@ -223,7 +223,11 @@ int mlpsp_sort_tiles(const float* rays_o_dev, const float* rays_d_dev, const voi
  * np_tile_kernels.cu:1837-2137; with out_t_dev != NULL also the expected depth of :5432-5719).
  * order_dev: the tile lists in processing order (mlpsp_sort_tiles output, or the candidates
  * themselves for MLPSP_KEY_LIST_ORDER).  counters_dev: NULL or 4 int64 {unused, tile-primitives
- * processed, tile-primitives with a hit, hits}, accumulated (zero them first). */
+ * processed, tile-primitives with a hit, hits}, accumulated (zero them first).
+ * Launches too small to fill the chip (at most 1,024 wavefronts; the 72-32-32-4 and 72-16-16-4 shapes) take a kernel
+ * that requests the next list entry's operands ahead, and at most 512 without counters one that puts two wavefronts
+ * on every 64 pixels; same bits.  MLPSP_F32_AHEAD=0/1/2 in the environment picks the form by hand, MLPSP_F32_SCALAR=1
+ * the kernel without matrix instructions. */
 int mlpsp_render_tilecenter_f32(const float* rays_o_dev, const float* rays_d_dev, const void* prim_records_dev,
                                 const int32_t* order_dev, const int32_t* tile_offsets_dev, const float* freq_dev,
                                 const float* att_dev, int num_frequencies, const float* W1, const float* b1,
