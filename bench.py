@@ -337,7 +337,7 @@ class Workload:
                 rd, pyramids, _ = ops.frame_prologue(ro, rd_raw, W, H)
             e[2].record()
             order, _ = ops.sort_tiles(ro, rd, rec, cand, off, W, H, 8, 8, cull_threshold=thr, tile_pyramids=pyramids,
-                                      tile_ends=ends)
+                                      tile_ends=ends, ids_ascend=tv is None)     # (as a queued frame sorts its own lists)
             e[3].record()
             counters = torch.zeros(4, dtype=torch.int64, device=dev)
             if feat is not None:

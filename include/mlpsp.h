@@ -201,7 +201,10 @@ int mlpsp_bin_raycone_fill(int num_primitives, int width, int height, int tile, 
  * candidate on the very edge of the culling's margin may be struck by one and not the other (the images are the
  * same: nothing that hits is ever struck).
  * tile_ends_dev: NULL (tile t's list ends where tile t + 1's begins: tile_offsets_dev[t + 1]) or T ends of lists
- * that lie in segments (mlpsp_bin_segments_async_device_matrices); the sorted lists are written to the same places. */
+ * that lie in segments (mlpsp_bin_segments_async_device_matrices); the sorted lists are written to the same places.
+ * ids_ascend != 0: the caller vouches that the ids of every list ascend, as the mlpsp_bin_* entry points write them
+ * (ties in list order are then ties in id order and the kernel sorts (key, id) words, which spares it a gather of the
+ * ids at the end; used with tile_pyramids_dev, ignored without).  Lists in any other order must pass 0. */
 size_t mlpsp_sort_frame_records_bytes(int num_primitives);
 size_t mlpsp_tile_pyramids_bytes(int width, int height, int tile_w, int tile_h);
 /* The per-frame preparations that need nothing but the rays (and the scene), in ONE launch: the unit directions of
@@ -216,7 +219,7 @@ int mlpsp_sort_tiles(const float* rays_o_dev, const float* rays_d_dev, const voi
                      int num_primitives, const int32_t* candidates_dev, const int32_t* tile_offsets_dev, int width,
                      int height, int tile_w, int tile_h, int key_family, int capacity, float cull_threshold,
                      void* frame_records_dev, int frame_records_ready, const void* tile_pyramids_dev,
-                     const int32_t* tile_ends_dev, int32_t* sorted_ids_dev, float* sorted_keys_dev,
+                     const int32_t* tile_ends_dev, int ids_ascend, int32_t* sorted_ids_dev, float* sorted_keys_dev,
                      mlpsp_stream_t stream);
 
 /* Tile-centre-order forward, scalar f32 (render_tiles_kernel_tilecenter_order,

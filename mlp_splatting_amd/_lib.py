@@ -51,7 +51,8 @@ SIGNATURES = {
     "mlpsp_sort_frame_records_bytes": (_sz, [_i]),
     "mlpsp_tile_pyramids_bytes": (_sz, [_i, _i, _i, _i]),
     "mlpsp_frame_prologue": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _vp, _vp, _i, _vp, _vp]),
-    "mlpsp_sort_tiles": (_i, [_vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _vp, _i, _vp, _vp, _vp, _vp, _vp]),
+    "mlpsp_sort_tiles": (_i, [_vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _vp, _i, _vp, _vp, _i, _vp, _vp,
+                              _vp]),
     "mlpsp_render_tilecenter_f32": (_i, [_vp] * 7 + [_i] + [_vp] * 6 + [_i, _i, _i, _i, _i, _i, _f, _vp, _vp, _vp,
                                                                        _vp, _vp]),
     "mlpsp_render_tilecenter_feat_f32": (_i, [_vp] * 7 + [_i] + [_vp] * 6 + [_i, _i, _vp, _i, _i, _f, _f, _i, _i, _i, _i,

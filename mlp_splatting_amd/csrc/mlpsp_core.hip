@@ -126,7 +126,8 @@ __global__ __launch_bounds__(256) void frame_prologue_kernel(const float* __rest
 // tile gathers are mostly those of its neighbours.
 // PYR: the tiles' ray pyramids come from records (the frame prologue's) instead of being built here.
 // Tile t's list is cand[offsets[t] .. ends[t]) (ends = offsets + 1 for lists that follow one another without gaps).
-template <bool PYR>
+// ASC: the ids of every list ascend (sort_one_tile_from).
+template <bool PYR, bool ASC = false>
 __global__ __launch_bounds__(kSortThreads) void sort_tiles_kernel(
     const float* __restrict__ rays_o, const float* __restrict__ rays_d, const PrimRecord* __restrict__ prims,
     const SortRec* __restrict__ frame, const TilePyramidRec* __restrict__ pyramids, const int32_t* __restrict__ cand,
@@ -142,7 +143,7 @@ __global__ __launch_bounds__(kSortThreads) void sort_tiles_kernel(
     return;
   }
   __shared__ SortLds<MLPSP_TILE_CAPACITY_MAX> lds;
-  sort_one_tile<MLPSP_TILE_CAPACITY_MAX, PYR>(lds, rays_o, rays_d, prims, frame, pyramids, cand, offsets, ends, g, family, capacity,
+  sort_one_tile<MLPSP_TILE_CAPACITY_MAX, PYR, ASC>(lds, rays_o, rays_d, prims, frame, pyramids, cand, offsets, ends, g, family, capacity,
                                          cull_r2, num_prims, sorted_ids, sorted_keys, tile);
 }
 
@@ -257,8 +258,8 @@ MLPSP_API int mlpsp_sort_tiles(const float* rays_o_dev, const float* rays_d_dev,
                                int num_primitives, const int32_t* candidates_dev, const int32_t* tile_offsets_dev,
                                int width, int height, int tile_w, int tile_h, int key_family, int capacity,
                                float cull_threshold, void* frame_records_dev, int frame_records_ready,
-                               const void* tile_pyramids_dev, const int32_t* tile_ends_dev, int32_t* sorted_ids_dev,
-                               float* sorted_keys_dev, mlpsp_stream_t stream) {
+                               const void* tile_pyramids_dev, const int32_t* tile_ends_dev, int ids_ascend,
+                               int32_t* sorted_ids_dev, float* sorted_keys_dev, mlpsp_stream_t stream) {
   const int64_t T = checked_num_tiles(width, height, tile_w, tile_h);
   if (T <= 0 || T > 2147483647LL) return MLPSP_E_ARGUMENT;
   if (key_family != MLPSP_KEY_TSTAR && key_family != MLPSP_KEY_DEPTH) return MLPSP_E_ARGUMENT;
@@ -280,7 +281,13 @@ MLPSP_API int mlpsp_sort_tiles(const float* rays_o_dev, const float* rays_d_dev,
                        rays_o_dev, (const PrimRecord*)prim_records_dev, num_primitives, (SortRec*)frame_records_dev);
     MLPSP_LAUNCH_CHECK();
   }
-  if (tile_pyramids_dev)
+  if (tile_pyramids_dev && ids_ascend)
+    hipLaunchKernelGGL((sort_tiles_kernel<true, true>), dim3(superblock_grid(g.ntx, g.nty)), dim3(kSortThreads), 0,
+                       (hipStream_t)stream, rays_o_dev, rays_d_dev, (const PrimRecord*)prim_records_dev,
+                       (const SortRec*)frame_records_dev, (const TilePyramidRec*)tile_pyramids_dev, candidates_dev,
+                       tile_offsets_dev, ends, g, key_family, capacity, cull_r2, num_primitives, sorted_ids_dev,
+                       sorted_keys_dev);
+  else if (tile_pyramids_dev)
     hipLaunchKernelGGL(sort_tiles_kernel<true>, dim3(superblock_grid(g.ntx, g.nty)), dim3(kSortThreads), 0,
                        (hipStream_t)stream, rays_o_dev, rays_d_dev, (const PrimRecord*)prim_records_dev,
                        (const SortRec*)frame_records_dev, (const TilePyramidRec*)tile_pyramids_dev, candidates_dev,

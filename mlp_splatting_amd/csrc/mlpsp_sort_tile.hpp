@@ -446,7 +446,10 @@ __device__ __forceinline__ void sort_small_tile(
 // Sorts one tile with the calling 256-thread workgroup (every thread must call it; `tile` is uniform).  kSortMax
 // bounds `capacity`.  A workgroup that sorts several tiles in a row, or uses `lds` for something else afterwards,
 // puts a barrier in between.
-template <int kSortMax, bool PYR, typename Source>
+// ASC: the caller vouches that the list's ids ascend (the own binning writes them so).  Then (key, id) orders like
+// (key, list position), the word that is sorted carries the id itself, and the output needs no second look at the
+// list.
+template <int kSortMax, bool PYR, bool ASC, typename Source>
 __device__ __forceinline__ void sort_one_tile_from(SortLds<kSortMax>& lds, const Source& src,
     const float* __restrict__ rays_o, const float* __restrict__ rays_d, const TilePyramidRec* __restrict__ pyramids,
     const TileGeom& g, int tile, float dx, float dy, float dz, const int32_t* __restrict__ cand, int family,
@@ -549,7 +552,7 @@ __device__ __forceinline__ void sort_one_tile_from(SortLds<kSortMax>& lds, const
     const unsigned long long below = (1ull << lane) - 1ull;
     const int f_before = nv + before_f + __popcll(mf & below);
     const int l_before = nl + before_l + __popcll(ml & below);
-    const unsigned long long entry = ((unsigned long long)kb << 32) | (unsigned)i;
+    const unsigned long long entry = ((unsigned long long)kb << 32) | (unsigned)(ASC ? p : i);
     if (front) {
       s_key[f_before] = entry;
     } else if (late) {
@@ -688,7 +691,7 @@ __device__ __forceinline__ void sort_one_tile_from(SortLds<kSortMax>& lds, const
   for (int i = tid; i < len; i += kSortThreads) {
     if (i < nv + nl) {
       const unsigned long long w = (i >= nv) ? s_key[kSortMax - 1 - (i - nv)] : s_key[through_order ? s_order[i] : i];
-      sorted_ids[start + i] = cand[start + (int)(w & 0xffffffffu)];
+      sorted_ids[start + i] = ASC ? (int)(w & 0xffffffffu) : cand[start + (int)(w & 0xffffffffu)];
       if (sorted_keys) sorted_keys[start + i] = bits_to_float((uint32_t)(w >> 32));
     } else if (i >= n) {
       sorted_ids[start + i] = cand[start + i];     // beyond the sort capacity: list order, never culled
@@ -697,7 +700,7 @@ __device__ __forceinline__ void sort_one_tile_from(SortLds<kSortMax>& lds, const
   }
 }
 
-template <int kSortMax, bool PYR>
+template <int kSortMax, bool PYR, bool ASC = false>
 __device__ __forceinline__ void sort_one_tile(SortLds<kSortMax>& lds,
     const float* __restrict__ rays_o, const float* __restrict__ rays_d, const PrimRecord* __restrict__ prims,
     const SortRec* __restrict__ frame, const TilePyramidRec* __restrict__ pyramids, const int32_t* __restrict__ cand,
@@ -711,10 +714,10 @@ __device__ __forceinline__ void sort_one_tile(SortLds<kSortMax>& lds,
   const float ox = rays_o[pc * 3 + 0], oy = rays_o[pc * 3 + 1], oz = rays_o[pc * 3 + 2];
   const float dx = rays_d[pc * 3 + 0], dy = rays_d[pc * 3 + 1], dz = rays_d[pc * 3 + 2];
   if (frame_records_hold(frame, ox, oy, oz))
-    sort_one_tile_from<kSortMax, PYR>(lds, FromFrameRecord{frame + 1}, rays_o, rays_d, pyramids, g, tile, dx, dy, dz, cand,
+    sort_one_tile_from<kSortMax, PYR, ASC>(lds, FromFrameRecord{frame + 1}, rays_o, rays_d, pyramids, g, tile, dx, dy, dz, cand,
                                  family, cull_r2, num_prims, sorted_ids, sorted_keys, start, len, n);
   else
-    sort_one_tile_from<kSortMax, PYR>(lds, FromPrimRecord{prims, ox, oy, oz}, rays_o, rays_d, pyramids, g, tile, dx, dy, dz,
+    sort_one_tile_from<kSortMax, PYR, ASC>(lds, FromPrimRecord{prims, ox, oy, oz}, rays_o, rays_d, pyramids, g, tile, dx, dy, dz,
                                  cand, family, cull_r2, num_prims, sorted_ids, sorted_keys, start, len, n);
 }
 

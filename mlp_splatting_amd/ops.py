@@ -305,7 +305,7 @@ def compact_segments(order, tile_offsets, tile_ends):
 
 def sort_tiles(rays_o, rays_d, records, candidates, tile_offsets, W, H, TW, TH, family=_lib.KEY_TSTAR,
                capacity=TILE_CAPACITY_DEFAULT, want_keys=False, cull_threshold=0.0, frame_records=None,
-               tile_pyramids=None, tile_ends=None):
+               tile_pyramids=None, tile_ends=None, ids_ascend=False):
     """Materialised per-tile depth order: (sorted_ids [P], sorted_keys [P] | None).
 
     With ``cull_threshold`` (the render's score threshold) candidates that provably hit no ray of their
@@ -316,7 +316,9 @@ def sort_tiles(rays_o, rays_d, records, candidates, tile_offsets, W, H, TW, TH, 
     unless it is 1.  ``tile_pyramids``: what :func:`frame_prologue` returned for these rays and this tile size (the
     culling's per-tile planes, which the sort otherwise builds in every wavefront of a tile; same output).
     ``tile_ends``: the int32 [T] ends of lists that lie in segments (:func:`bin_segments_async`); the sorted lists
-    come back in the same places, what lies between them is not written."""
+    come back in the same places, what lies between them is not written.  ``ids_ascend``: the caller vouches that
+    the ids of every list ascend, as the binning entry points write them (same output, no gather of the ids at the
+    end; lists in any other order must leave it False)."""
     dev = rays_o.device
     if tile_ends is not None and not (tile_ends.is_cuda and tile_ends.dtype == torch.int32 and tile_ends.is_contiguous()
                                       and tile_ends.numel() == tile_offsets.numel() - 1):
@@ -343,8 +345,8 @@ def sort_tiles(rays_o, rays_d, records, candidates, tile_offsets, W, H, TW, TH, 
         raise ValueError("tile_pyramids must be the uint8 buffer frame_prologue() returned for this frame and tile size")
     code = lib.mlpsp_sort_tiles(_ptr(rays_o), _ptr(rays_d), _ptr(records), num_primitives, _ptr(candidates),
                                 _ptr(tile_offsets), W, H, TW, TH, int(family), int(capacity), float(cull_threshold),
-                                _ptr(scratch), ready, _ptr(tile_pyramids), _ptr(tile_ends), _ptr(sorted_ids), _ptr(keys),
-                                _stream(dev))
+                                _ptr(scratch), ready, _ptr(tile_pyramids), _ptr(tile_ends), int(bool(ids_ascend)),
+                                _ptr(sorted_ids), _ptr(keys), _stream(dev))
     _check(code, "mlpsp_sort_tiles")
     return sorted_ids, keys
 

@@ -429,7 +429,7 @@ class TileExt:
             rec = self._records(positions, log_scales, unit_quats)
             order, _ = ops.sort_tiles(rays_o, unit_dirs, rec, cand, offsets, width, height, 8, 8, _lib.KEY_TSTAR,
                                       self.max_tile_prims, cull_threshold=threshold, frame_records=frame_records,
-                                      tile_pyramids=tile_pyramids, tile_ends=ends)
+                                      tile_pyramids=tile_pyramids, tile_ends=ends, ids_ascend=True)
             fmap, pool_ran_out = None, 0
             if precision != "f32":
                 packed = self._packed_weights(list(ws), precision == "bf16")

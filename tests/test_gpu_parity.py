@@ -143,6 +143,18 @@ def test_lists_in_segments_are_the_oracles_lists(device, oracle_mod, n, width, h
     c, o = _t(want_cand, device), _t(want_off, device)
     plain, plain_keys = ops.sort_tiles(ro, rd, rec, c, o, width, height, 8, 8, cull_threshold=thr, want_keys=True)
     seg, seg_keys = ops.sort_tiles(ro, rd, rec, cand, off, width, height, 8, 8, cull_threshold=thr, want_keys=True, tile_ends=ends)
+    # lists whose ids ascend (these do) may be sorted as (key, id) words, with the tiles' pyramids from the prologue:
+    # the same order, and the same lists with or without the vouching
+    _, pyramids, _ = ops.frame_prologue(ro, rd, width, height, 8, 8)
+    for c_, o_, e_ in ((c, o, None), (cand, off, ends)):
+        a = ops.sort_tiles(ro, rd, rec, c_, o_, width, height, 8, 8, cull_threshold=thr, want_keys=True, tile_pyramids=pyramids,
+                           tile_ends=e_)
+        b = ops.sort_tiles(ro, rd, rec, c_, o_, width, height, 8, 8, cull_threshold=thr, want_keys=True, tile_pyramids=pyramids,
+                           tile_ends=e_, ids_ascend=True)
+        ends_h = (o_[1:] if e_ is None else e_).cpu().numpy()
+        for t in range(T):
+            lo, hi = int(o_[t]), int(ends_h[t])
+            assert torch.equal(a[0][lo:hi], b[0][lo:hi]) and torch.equal(a[1][lo:hi], b[1][lo:hi])
     plain, seg, plain_keys, seg_keys = plain.cpu().numpy(), seg.cpu().numpy(), plain_keys.cpu().numpy(), seg_keys.cpu().numpy()
     for t in range(T):
         np.testing.assert_array_equal(seg[t * stride:t * stride + lengths[t]], plain[want_off[t]:want_off[t + 1]])
