@@ -584,27 +584,36 @@ __device__ __forceinline__ void sort_one_tile_from(SortLds<kSortMax>& lds, const
   }
   __syncthreads();
 
-  // ---- order of the ordinary survivors.  Usual case: a counting pass into 256 buckets that are linear in the
+  // ---- order of the ordinary survivors.  Usual case: a counting pass into 512 buckets that are linear in the
   //      key bits between the smallest and the largest key (monotone, so bucket order is key order), then every
   //      entry ranks itself among the entries of its own bucket by its (key, list position) word.  The work of
   //      that last step is the sum of the squared bucket sizes; when keys pile up in few buckets (or a late key
   //      is not the invalid key, which the late stream's list order would misplace) the bitonic network below
   //      sorts instead.
+  // (two buckets per thread: their counts, offsets and cursors are 16-bit halves of one word -- a list holds at
+  // most kSortMax <= 65,535 entries, so a half never carries into its neighbour)
+  constexpr int kBuckets = 2 * kSortThreads;
   const uint32_t kmin = s_kmin;
-  const float bucket_scale = (float)kSortThreads / ((float)(s_kmax - kmin) + 1.f);
+  const float bucket_scale = (float)kBuckets / ((float)(s_kmax - kmin) + 1.f);
   auto bucket_of = [&](unsigned long long w) {
     const int b = (int)((float)((uint32_t)(w >> 32) - kmin) * bucket_scale);
-    return b < kSortThreads - 1 ? b : kSortThreads - 1;
+    return b < kBuckets - 1 ? b : kBuckets - 1;
   };
+  auto half_of = [](int word, int b) { return (word >> ((b & 1) << 4)) & 0xffff; };
+  auto one_in = [](int b) { return 1 << ((b & 1) << 4); };
   bool network = (s_flags & 1) != 0;
   const bool ranked = !network && nv > 1;
   if (ranked) {
     s_cnt[tid] = 0;
     __syncthreads();
-    for (int i = tid; i < nv; i += kSortThreads) atomicAdd(&s_cnt[bucket_of(s_key[i])], 1);
+    for (int i = tid; i < nv; i += kSortThreads) {
+      const int b = bucket_of(s_key[i]);
+      atomicAdd(&s_cnt[b >> 1], one_in(b));
+    }
     __syncthreads();
-    const int c = s_cnt[tid];
-    int incl = c, pairs = c * c;
+    const int c0 = s_cnt[tid] & 0xffff, c1 = (s_cnt[tid] >> 16) & 0xffff;
+    const int c = c0 + c1;
+    int incl = c, pairs = c0 * c0 + c1 * c1;
 #pragma unroll
     for (int d = 1; d < 64; d <<= 1) {
       const int up = __shfl_up(incl, d);
@@ -619,18 +628,21 @@ __device__ __forceinline__ void sort_one_tile_from(SortLds<kSortMax>& lds, const
 #pragma unroll
     for (int v = 0; v < kSortThreads / 64; ++v) base += (v < wave) ? s_wave_cnt[0][v] : 0;
     const int excl = base + incl - c;
-    s_off[tid] = excl;
-    s_cnt[tid] = excl;                                   // from here on: the bucket's fill cursor
+    s_off[tid] = excl | ((excl + c0) << 16);
+    s_cnt[tid] = excl | ((excl + c0) << 16);             // from here on: the buckets' fill cursors
     network = s_pairs > kRankPairsMax;
     __syncthreads();
     if (!network) {
-      for (int i = tid; i < nv; i += kSortThreads) s_perm[atomicAdd(&s_cnt[bucket_of(s_key[i])], 1)] = (uint16_t)i;
+      for (int i = tid; i < nv; i += kSortThreads) {
+        const int b = bucket_of(s_key[i]);
+        s_perm[half_of(atomicAdd(&s_cnt[b >> 1], one_in(b)), b)] = (uint16_t)i;
+      }
       __syncthreads();
       for (int a = tid; a < nv; a += kSortThreads) {
         const int ia = s_perm[a];
         const unsigned long long wa = s_key[ia];
         const int b = bucket_of(wa);
-        const int lo = s_off[b], hi = s_cnt[b];          // the cursor ended at the bucket's end
+        const int lo = half_of(s_off[b >> 1], b), hi = half_of(s_cnt[b >> 1], b);   // the cursor ended at the bucket's end
         int r = 0;
         for (int q = lo; q < hi; ++q) r += (s_key[s_perm[q]] < wa) ? 1 : 0;
         s_order[lo + r] = (uint16_t)ia;
