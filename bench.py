@@ -319,8 +319,8 @@ class Workload:
                                        tile_view_ids=tv)
             n_cand = int(cand.numel())
             # the binning as a frame queues it: no host synchronisation, candidate buffer sized beforehand
-            # (an RGB frame on the matrix cores takes its lists in per-tile segments: level 2 in one launch)
-            segments = tv is None and feat is None and precision == "bf16"
+            # (a frame on the matrix cores takes its lists in per-tile segments: level 2 in one launch)
+            segments = tv is None and precision == "bf16"
             ends = None
             e[0].record()
             if segments:
@@ -347,7 +347,8 @@ class Workload:
                 ops.render_tilecenter_mfma_feat(ro, rd, rec, order, off, freq, att, *weights, feat,
                                                 float(scene.feature_gating_beta), float(scene.feature_gating_temp), W, H,
                                                 thr, bf16=True, packed=packed, packed_feat=packed_feat, check=False,
-                                                stages=lambda k: marks[k].record() if k in marks else None)
+                                                stages=lambda k: marks[k].record() if k in marks else None,
+                                                tile_ends=ends)
             elif precision == "bf16":
                 ops.render_tilecenter_mfma(ro, rd, rec, order, off, freq, att, *weights, W, H, thr, bf16=True,
                                            packed=packed, check=False, status=flags, status_is_clear=tv is None,

@@ -905,8 +905,8 @@ class NeuralPrimitiveSceneTileCUDA(nn.Module):
         views, proj = _frame_matrix(view_matrix).reshape(1, 4, 4), _frame_matrix(proj_matrix)
         binned = None
         if hasattr(ext, "frame_binning_queued"):
-            # (an RGB frame on the matrix cores takes its lists in per-tile segments: one binning launch less)
-            segments = not with_feat and precision != "f32" and _env("MLPSP_FRAME_SEGMENTS", "1") != "0"
+            # (a frame on the matrix cores takes its lists in per-tile segments: one binning launch less)
+            segments = precision != "f32" and _env("MLPSP_FRAME_SEGMENTS", "1") != "0"
             binned = ext.frame_binning_queued(positions, log_scales, views, proj, int(W), int(H), float(score_threshold),
                                               **({"segments": True} if segments else {}))
             if binned is None:

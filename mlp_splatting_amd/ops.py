@@ -675,7 +675,8 @@ def pack_mfma_feat(feat_attr):
 
 def render_tilecenter_mfma_feat(rays_o, rays_d, records, order, tile_offsets, freq, att, W1, b1, W2, b2, W3, b3,
                                 feat_attr, beta, temp, W, H, threshold, bf16=True, packed=None, packed_feat=None,
-                                check=True, status=None, counters=None, stages=None, status_is_clear=False):
+                                check=True, status=None, counters=None, stages=None, status_is_clear=False,
+                                tile_ends=None):
     """Matrix-core tile-centre forward with the gated feature channel -> (rgb, alpha, feat, nonfinite).
     ``packed_feat`` is the result of :func:`pack_mfma_feat` for ``feat_attr`` (built here when omitted;
     non-finite rounded attributes raise).  ``status`` (an int32 [16] device tensor): ONE attempt with the first
@@ -684,7 +685,8 @@ def render_tilecenter_mfma_feat(rays_o, rays_d, records, order, tile_offsets, fr
     ``counters``: int64 [4] work counters of the render launch, accumulated.  ``stages``: a callable
     ``stages(which)`` invoked before the render launch (1), before the feature product (2) and after it (3) -- the
     two launches are then queued by separate calls, with the worst-case record pool, so that a caller can bracket
-    each with events.  ``status_is_clear``: as in :func:`render_tilecenter_mfma` (with ``status`` only)."""
+    each with events.  ``status_is_clear``: as in :func:`render_tilecenter_mfma` (with ``status`` only).
+    ``tile_ends``: as in :func:`sort_tiles` (the record pool is then sized by the segments' total length)."""
     dev = rays_o.device
     if freq.numel() != 6:
         raise RuntimeError("the matrix-core path supports 6 frequencies only")
@@ -711,7 +713,7 @@ def render_tilecenter_mfma_feat(rays_o, rays_d, records, order, tile_offsets, fr
             _ptr(rays_o), _ptr(rays_d), _ptr(records), _ptr(order), _ptr(tile_offsets), pairs, _ptr(freq), _ptr(att),
             _ptr(packed), W1.shape[0], int(bool(bf16)), _ptr(packed_feat), slots, ch, float(beta), float(temp), W, H,
             float(threshold), _ptr(workspace), ws_bytes, _ptr(rgb), _ptr(alpha), _ptr(feat), _ptr(flag), _ptr(counters),
-            stage | clear_bit, None, _stream(dev))
+            stage | clear_bit, _ptr(tile_ends), _stream(dev))
         _check(code, "mlpsp_render_tilecenter_mfma_feat")
         return code
 

@@ -334,7 +334,7 @@ class TileExt:
         :meth:`render_frame_queued` takes as ``binned``, or None when no candidate-buffer estimate exists yet.
         ``segments``: every tile's list in a segment of ``max_tile_prims`` entries of its own
         (:func:`ops.bin_segments_async`: one launch less, no estimate needed), when the camera's matrices are on the
-        device; for frames whose render takes such lists (RGB on the matrix cores)."""
+        device; for frames whose render takes such lists (the matrix cores')."""
         with self._lock:
             cap, scale = self._queue_capacity, self._queue_scratch_scale
         segments = (segments and all(m.is_cuda and m.dtype == torch.float32 and m.numel() == 16 and m.is_contiguous()
@@ -416,8 +416,8 @@ class TileExt:
             if binned is None:
                 return None
         cand, offsets, counts, tail, cap, scale, held, ends = binned
-        if ends is not None and (feat is not None or precision == "f32"):
-            raise ValueError("lists in segments are for RGB frames on the matrix cores")
+        if ends is not None and precision == "f32":
+            raise ValueError("lists in segments are for frames on the matrix cores")
         status = tail[32:].view(torch.int32)
         # The flag words live in a buffer that this thread's frames use one after the other, and every frame ends by
         # reading them back: if the last frame read sixteen zeros they are still zero, and the render's own clear (a
@@ -445,7 +445,7 @@ class TileExt:
                     rgb, alpha, fmap, _ = ops.render_tilecenter_mfma_feat(
                         rays_o, unit_dirs, rec, order, offsets, freq, att, *ws, feat[0], feat[1], feat[2], width, height,
                         threshold, bf16=(precision == "bf16"), packed=packed, packed_feat=packed_feat, status=status,
-                        status_is_clear=flags_clear)
+                        status_is_clear=flags_clear, tile_ends=ends)
                 frame = QueuedFrame(name, precision, feat is not None, (rgb, alpha, fmap), tail, held, cap, scale,
                                     (rays_o, unit_dirs, positions, log_scales, unit_quats, freq, att, ws),
                                     (rec, order, offsets, width, height, threshold, ends))

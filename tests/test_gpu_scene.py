@@ -257,7 +257,9 @@ def test_queued_feature_frames_equal_step_by_step_frames(device, oracle_mod, mon
     rgb, feat = _call(scene, fr, device, return_feature=True)
     assert calls == [True] and torch.equal(rgb, ref_rgb) and torch.equal(feat, ref_feat)
     assert float(feat.abs().max()) > 1e-2
-    # a candidate-buffer estimate that is too small: repeated step by step, same images
+    # a candidate-buffer estimate that is too small: repeated step by step, same images (lists one after the other:
+    # lists in segments, the default, need no estimate)
+    monkeypatch.setenv("MLPSP_FRAME_SEGMENTS", "0")
     ext._queue_capacity = 16
     rgb, feat = _call(scene, fr, device, return_feature=True)
     assert torch.equal(rgb, ref_rgb) and torch.equal(feat, ref_feat) and ext._queue_capacity > 1000
