@@ -337,8 +337,10 @@ class TileExt:
         device; for frames whose render takes such lists (the matrix cores')."""
         with self._lock:
             cap, scale = self._queue_capacity, self._queue_scratch_scale
+        # (not for screens whose segments would take more than 2 GiB per array: those keep the lists one after the other)
         segments = (segments and all(m.is_cuda and m.dtype == torch.float32 and m.numel() == 16 and m.is_contiguous()
-                                     for m in (view_matrices, proj_matrix)))
+                                     for m in (view_matrices, proj_matrix))
+                    and ops.num_tiles(int(width), int(height), 8, 8) * self.max_tile_prims <= 1 << 29)
         if cap <= 0 and not segments:
             return None
         with _on_device(positions.device):
