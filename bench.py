@@ -514,7 +514,8 @@ def main() -> int:
     # reported beside the headline, which stays the frame-after-frame call of the reference's interface
     in_flight = None
     if precision == "bf16" and not args.no_frames_in_flight:
-        in_flight = wl.timed_in_flight(2, len(frames), args.min_seconds)
+        # (a feature frame's result holds a 1.67 GB image: eight cameras per call there)
+        in_flight = wl.timed_in_flight(2, 8 if feature_dim else len(frames), args.min_seconds)
 
     # ---- the stages of a frame alone: HIP events on the stream they are launched on, and the render's work counters
     st = wl.probe_stages(8)
