@@ -170,6 +170,29 @@ def test_lists_in_segments_are_the_oracles_lists(device, oracle_mod, n, width, h
     np.testing.assert_array_equal(comp_off.cpu().numpy(), want_off)
 
 
+def test_level1_overflow_empties_the_lists_in_segments_too(device):
+    """Primitives so large that each overlaps every super-tile overflow the level-1 lists of a scratch of the ordinary
+    size (room for eight super-tiles per primitive): guard = 1, the number of level-1 entries is reported, every list
+    is empty -- from the segment entry as from the asynchronous entry with a candidate buffer --, and four times the
+    scratch holds them."""
+    from mlp_splatting_amd import ops, synthetic as syn
+    n, width, height, thr = 12000, 640, 480, 1e-3
+    rng = np.random.default_rng(5)
+    pos = (rng.random((n, 3), dtype=np.float32) - 0.5).astype(np.float32)
+    logs = np.full((n, 3), -0.5, np.float32)
+    view = syn.view_matrix(syn.look_at((0.0, 0.0, -3.0), (0.0, 0.0, 0.0)))
+    proj = syn.projection_matrix(500.0, width, height)
+    p, l, v, pr = _t(pos, device), _t(logs, device), _t(view, device), _t(proj, device)
+    cand, off, ends, counts = ops.bin_segments_async(p, l, v, pr, width, height, 8, thr, stride=64)
+    pairs, over, l1_entries, guard = counts.tolist()
+    assert guard == 1 and l1_entries > 8 * n + 65536 and torch.equal(ends, off[:-1])
+    _, off2, counts2 = ops.bin_legacy_async(p, l, v, pr, width, height, 8, thr, 1 << 20)
+    assert counts2.tolist()[2:] == [l1_entries, 1] and not off2.any()
+    _, off4, ends4, counts4 = ops.bin_segments_async(p, l, v, pr, width, height, 8, thr, stride=64, scratch_scale=16)
+    pairs, over, l1_entries4, guard = counts4.tolist()
+    assert guard == 0 and l1_entries4 == l1_entries and over > 64 and bool((ends4 - off4[:-1] == 64).all())
+
+
 def test_lists_in_segments_without_primitives(device):
     from mlp_splatting_amd import ops
     none = torch.empty(0, 3, dtype=torch.float32, device=device)
