@@ -656,20 +656,40 @@ __global__ __launch_bounds__(256) void feat_gemm_kernel(const unsigned* __restri
   }
   if (!active) return;
 
+  // The image is written through LDS: an accumulator register holds 32 consecutive channels of two pixels, i.e.
+  // a store of it is two 128-byte lines, and the vector memory path takes as long for such an instruction as for
+  // one that carries 16 bytes per lane.  Half a tile at a time every wavefront parks its accumulators in its own
+  // quarter of the attribute chunk's LDS as [pixel][channel] (its 32 NCB channels of 32 pixels: 8 KB for NCB = 2)
+  // and reads them back 16 bytes per lane, so that a store carries the wavefront's run of channels for 64 / (8 NCB)
+  // pixels.  No workgroup barrier: a wavefront's LDS operations complete in order, and the chunk loop left every
+  // wavefront behind its last barrier.
+  constexpr int CW = 32 * NCB;             // channels of a wavefront
+  constexpr int kLanesPerPixel = CW / 4, kPixelsPerStore = 64 / kLanesPerPixel;
+  static_assert(sizeof(s_b) >= 4 * 32 * CW * sizeof(float), "four wavefronts' half tiles fit the attribute chunk");
+  static_assert(kLanesPerPixel <= 64 && 64 % kLanesPerPixel == 0, "whole pixels per store");
+  float* const s_t = reinterpret_cast<float*>(s_b) + wave * (32 * CW);
   const int tx = tile % ntx, ty = tile / ntx;
+  const bool rows16 = (C & 3) == 0;        // a pixel's channels start on a 16-byte boundary
+  const int cl = (l % kLanesPerPixel) * 4; // this lane's first channel within the wavefront's run
 #pragma unroll
   for (int pb = 0; pb < 2; ++pb) {
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int q = 32 * pb + d_row(r, g);
-      const int x = tx * 8 + (q & 7), y = ty * 8 + (q >> 3);
-      if (x < W && y < H) {
-        float* __restrict__ dst = out_feat + (size_t)(y * W + x) * C;
+    for (int cb = 0; cb < NCB; ++cb)
 #pragma unroll
-        for (int cb = 0; cb < NCB; ++cb) {
-          const int c = c0 + 32 * cb + m;
-          if (cb < ncb && c < C) dst[c] = acc[pb][cb][r];
-        }
+      for (int r = 0; r < 16; ++r) s_t[d_row(r, g) * CW + 32 * cb + m] = acc[pb][cb][r];
+#pragma unroll
+    for (int j = 0; j < 32 / kPixelsPerStore; ++j) {
+      const int ql = j * kPixelsPerStore + l / kLanesPerPixel, q = 32 * pb + ql;
+      const int x = tx * 8 + (q & 7), y = ty * 8 + (q >> 3);
+      const f32x4 v = *reinterpret_cast<const f32x4*>(&s_t[ql * CW + cl]);
+      if (x >= W || y >= H) continue;
+      float* __restrict__ dst = out_feat + (size_t)(y * W + x) * C + c0 + cl;
+      if (rows16 && c0 + cl + 3 < C) {
+        *reinterpret_cast<f32x4*>(dst) = v;
+      } else {
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+          if (c0 + cl + k < C) dst[k] = v[k];
       }
     }
   }
