@@ -528,7 +528,8 @@ class NeuralPrimitiveSceneTileCUDA(nn.Module):
         self.image_size = (int(W), int(H))
 
     def _activate_cuda_device(self) -> torch.device:
-        device = self.positions.device
+        positions = self._parameters.get("positions")
+        device = (positions if positions is not None else self.positions).device
         if device.type != "cuda":
             raise RuntimeError("NeuralPrimitiveSceneTileCUDA must be moved to a CUDA device before rendering.")
         if device.index is None:
@@ -583,10 +584,23 @@ class NeuralPrimitiveSceneTileCUDA(nn.Module):
 
     def _frequency_tables(self, device):
         """freq and att as the kernels take them (scannet/cumodel.py:1078-1086)."""
-        sources = [self.encoder.freq_bands]
-        if hasattr(self.encoder, "runtime_frequency_weights"):
-            sources.append(self.encoder.runtime_frequency_weights)
-        extra = (device, float(getattr(self.encoder, "sigma2", 0.0)))
+        # (once per frame, while the device may be waiting for the host: the encoder and its buffers are taken from
+        # the modules' own tables, which a plain attribute read reaches only after a failed instance look-up)
+        encoder = self._modules.get("encoder")
+        if encoder is None:
+            encoder = self.encoder
+        buffers = encoder._buffers
+        bands = buffers.get("freq_bands")
+        sources = [bands if bands is not None else encoder.freq_bands]
+        weights = buffers.get("runtime_frequency_weights")
+        if weights is None and hasattr(encoder, "runtime_frequency_weights"):
+            weights = encoder.runtime_frequency_weights
+        if weights is not None:
+            sources.append(weights)
+        sigma2 = encoder.__dict__.get("sigma2")
+        if sigma2 is None:
+            sigma2 = getattr(encoder, "sigma2", 0.0) if hasattr(type(encoder), "sigma2") else 0.0
+        extra = (device, float(sigma2))
         return self._cached("frequency_tables", sources, extra, lambda: self._build_frequency_tables(device))
 
     def _build_frequency_tables(self, device):
@@ -688,8 +702,10 @@ class NeuralPrimitiveSceneTileCUDA(nn.Module):
                                     score_threshold, tile_size)
 
     def _unit_quats(self):
-        return self._cached("unit_quats", [self.quats], (),
-                            lambda: F.normalize(self.quats.detach(), dim=-1).contiguous())
+        quats = self._parameters.get("quats")
+        if quats is None:
+            quats = self.quats
+        return self._cached("unit_quats", [quats], (), lambda: F.normalize(quats.detach(), dim=-1).contiguous())
 
     def _base_args(self, ray_o, ray_d, culled_prim_indices, tile_offsets, device, unit_dirs=None):
         freq, att = self._frequency_tables(device)
