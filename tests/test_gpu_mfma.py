@@ -259,6 +259,29 @@ def test_matrix_core_feature_render_against_oracle(device, oracle_mod, bf16, slo
     assert np.abs(rgb.cpu().numpy() - want["rgb"]).max() <= TOL[bf16]
 
 
+@pytest.mark.parametrize("channels", [260, 37])
+def test_matrix_core_feature_image_on_a_ragged_frame(device, oracle_mod, channels):
+    # image sides that are no multiples of the tile side; 260 channels: the second slice of 256 holds a single
+    # 16-byte piece per pixel; 37: a pixel's channels do not start on a 16-byte boundary.  The product writes the image
+    # 16 bytes per lane and has to leave out the pixels beyond the image and the channels beyond the last.
+    from mlp_splatting_amd import ops
+    fr = Frame("cfg1_5k_160x120", n=1200, hidden=32, width=52, height=44, feature_dim=channels, feature_slots=4)
+    sc = fr.scene
+    cand, off = fr.oracle_lists(oracle_mod)
+    want = oracle_mod.render_tilecenter(*fr.base_numpy(cand, off), *fr.dims, feat_attr=sc.feat_attr, beta=1.3, temp=2.2)
+    t = lambda a: to_dev(a, device)
+    rec = ops.prepare_primitives(t(sc.positions), t(sc.log_scales), t(sc.quats))
+    ro, rd, c, o = t(fr.rays_o), t(fr.rays_d), t(cand), t(off)
+    order, _ = ops.sort_tiles(ro, rd, rec, c, o, fr.W, fr.H, 8, 8, cull_threshold=fr.thr)
+    ws = [t(w) for w in sc.mlp()]
+    rgb, alpha, feat, nonfinite = ops.render_tilecenter_mfma_feat(ro, rd, rec, order, o, t(sc.freq), t(sc.att), *ws,
+                                                                  t(sc.feat_attr), 1.3, 2.2, fr.W, fr.H, fr.thr, bf16=True)
+    assert not nonfinite and feat.shape == (fr.W * fr.H, channels)
+    scale = float(np.abs(want["feat"]).max())
+    err = float(np.abs(feat.cpu().numpy() - want["feat"]).max())
+    assert scale > 1e-2 and 0 < err <= TOL[True] * max(1.0, scale)
+
+
 def test_matrix_core_feature_render_with_separate_origins(device, oracle_mod):
     from mlp_splatting_amd import ops
     fr = Frame("cfg1_5k_160x120", n=1200, hidden=32, width=56, height=40, feature_dim=72, feature_slots=4)
