@@ -333,7 +333,10 @@ __device__ __forceinline__ bool outside_pyramid(const TilePyramid& py, const Pri
   // squared semi-axes as reciprocals of the precision diagonal (one unit in the last place, far inside the margin;
   // 1/0 = inf never culls): the record's own s2 words lie in its fourth 16-byte piece, which nothing else here
   // needs -- a candidate is then three requests instead of four
-  const float s2x = __builtin_amdgcn_rcpf(P.mx), s2y = __builtin_amdgcn_rcpf(P.my), s2z = __builtin_amdgcn_rcpf(P.mz);
+  // (with the squared cull radius folded in: beyond a face means dist < 0 and dist^2 > r^2 h^2, i.e.
+  // dist |dist| < -(r^2 h^2): one product and one comparison per face)
+  const float s2x = cull_r2 * __builtin_amdgcn_rcpf(P.mx), s2y = cull_r2 * __builtin_amdgcn_rcpf(P.my),
+              s2z = cull_r2 * __builtin_amdgcn_rcpf(P.mz);
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
     const float nx = py.n[j][0], ny = py.n[j][1], nz = py.n[j][2];
@@ -342,7 +345,7 @@ __device__ __forceinline__ bool outside_pyramid(const TilePyramid& py, const Pri
     const float ly = fmaf(r01, nx, fmaf(r11, ny, r21 * nz));
     const float lz = fmaf(r02, nx, fmaf(r12, ny, r22 * nz));
     const float h2 = fmaf(s2x * lx, lx, fmaf(s2y * ly, ly, (s2z * lz) * lz));
-    outside |= ((py.faces >> j) & 1) && (dist < 0.f) && (dist * dist >= cull_r2 * h2);
+    outside |= ((py.faces >> j) & 1) && (dist * __builtin_fabsf(dist) < -h2);
   }
   return outside;
 }
@@ -477,7 +480,7 @@ __device__ __forceinline__ void sort_one_tile_from(SortLds<kSortMax>& lds, const
   auto& s_flags = lds.flags;
   auto& s_pairs = lds.pairs;
   const int tid = threadIdx.x;
-  const int wave = tid >> 6, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;   // (the wavefront's index as a scalar)
 
   // Every candidate id this thread will handle is requested up front (at most kSortMax / kSortThreads of them),
   // and the first round's geometry record right behind; each round of the key loop then requests the next round's
@@ -522,7 +525,9 @@ __device__ __forceinline__ void sort_one_tile_from(SortLds<kSortMax>& lds, const
     s_flags = 0;
     s_pairs = 0;
   }
-  int nv = 0, nl = 0;                                    // ordinary and late survivors so far (block-uniform)
+  // ordinary survivors so far in the low half, late ones in the high half (block-uniform; a list holds at most
+  // kSortMax <= 65,535 entries, so the halves never carry into each other): one sum serves both streams
+  int survivors = 0;
   uint32_t key_lo = 0xffffffffu, key_hi = 0u;
   bool odd_late = false;
 #pragma unroll
@@ -546,21 +551,21 @@ __device__ __forceinline__ void sort_one_tile_from(SortLds<kSortMax>& lds, const
     const uint32_t kb = float_to_bits(key);
     const bool late = keep && kb >= invalid_bits;
     const bool front = keep && !late;
-    const unsigned long long mf = __ballot(front), ml = __ballot(late);
+    // (the builtin on the predicates themselves: __ballot() takes an int, and the predicate's way through a
+    // register and back is two vector instructions per vote)
+    const unsigned long long mf = __builtin_amdgcn_ballot_w64(front), ml = __builtin_amdgcn_ballot_w64(late);
     if (lane == 0) s_wave_cnt[round][wave] = __popcll(mf) | (__popcll(ml) << 16);
     __syncthreads();                                     // (the two count buffers alternate: one barrier per round)
-    int before_f = 0, before_l = 0, total_f = 0, total_l = 0;
+    int before = survivors, total = 0;
 #pragma unroll
     for (int v = 0; v < kSortThreads / 64; ++v) {
-      const int c = s_wave_cnt[round][v];
-      before_f += (v < wave) ? (c & 0xffff) : 0;
-      before_l += (v < wave) ? (c >> 16) : 0;
-      total_f += c & 0xffff;
-      total_l += c >> 16;
+      const int c = __builtin_amdgcn_readfirstlane(s_wave_cnt[round][v]);     // (the same word in every lane)
+      before += (v < wave) ? c : 0;
+      total += c;
     }
     const unsigned long long below = (1ull << lane) - 1ull;
-    const int f_before = nv + before_f + __popcll(mf & below);
-    const int l_before = nl + before_l + __popcll(ml & below);
+    const int f_before = (before & 0xffff) + __popcll(mf & below);
+    const int l_before = (before >> 16) + __popcll(ml & below);
     const unsigned long long entry = ((unsigned long long)kb << 32) | (unsigned)(ASC ? p : i);
     if (front) {
       s_key[f_before] = entry;
@@ -576,9 +581,9 @@ __device__ __forceinline__ void sort_one_tile_from(SortLds<kSortMax>& lds, const
     key_lo = front ? min(key_lo, kb) : key_lo;
     key_hi = front ? max(key_hi, kb) : key_hi;
     odd_late |= late && kb != invalid_bits;
-    nv += total_f;
-    nl += total_l;
+    survivors += total;
   }
+  int nv = survivors & 0xffff, nl = survivors >> 16;
   {
 #pragma unroll
     for (int d = 32; d > 0; d >>= 1) {
