@@ -305,7 +305,8 @@ def test_sorted_tile_lists_match_oracle_keys_and_order(device, oracle_mod, frame
 
 
 @pytest.mark.parametrize("case", ["spread", "ties", "behind", "clusters", "beyond_invalid", "two", "capacity",
-                                  "ties:64", "behind:64", "beyond_invalid:63", "spread:65", "clusters:1"])
+                                  "ties:64", "behind:64", "beyond_invalid:63", "spread:65", "clusters:1",
+                                  "spread:2000", "clusters:1800", "behind:2048"])
 @pytest.mark.parametrize("frame_records", [True, False], ids=["frame_records", "full_key"])
 @pytest.mark.parametrize("family", [1, 2])
 def test_sort_is_the_stable_key_order_for_every_key_distribution(device, oracle_mod, case, family, frame_records):
@@ -313,7 +314,8 @@ def test_sort_is_the_stable_key_order_for_every_key_distribution(device, oracle_
     sorting network when keys pile up in few buckets or a key exceeds the invalid key; each case below steers it
     down one of those routes, and the result must be the oracle's stable sort by key every time.  A list of at most
     64 entries is sorted by one wavefront in registers: the cases with a length after the colon go that way (65:
-    the first length that does not)."""
+    the first length that does not).  Lists longer than the default capacity of 1536 are sorted with the capacity
+    of the interface, 2048: a workgroup's memory is laid out for the one or the other."""
     from mlp_splatting_amd import ops
     rng = np.random.default_rng(11)
     fr = Frame("cfg1_5k_160x120", n=8, width=8, height=8, eye=(0, 0, -2.0), target=(0, 0, 0))
@@ -345,9 +347,11 @@ def test_sort_is_the_stable_key_order_for_every_key_distribution(device, oracle_
     cand = np.sort(cand)
     off = np.array([0, n], np.int32)
     rec = ops.prepare_primitives(_t(pos, device), _t(log_s, device), _t(quat, device))
+    more = {"capacity": 2048} if n > 1536 else {}
     ids, keys = ops.sort_tiles(_t(fr.rays_o, device), _t(fr.rays_d, device), rec, _t(cand, device), _t(off, device),
-                               8, 8, 8, 8, family=family, want_keys=True, frame_records=frame_records)
-    want_ids, want_keys = oracle_mod.sort_tiles(fr.rays_o, fr.rays_d, pos, log_s, quat, cand, off, 8, 8, 8, 8, family=family)
+                               8, 8, 8, 8, family=family, want_keys=True, frame_records=frame_records, **more)
+    want_ids, want_keys = oracle_mod.sort_tiles(fr.rays_o, fr.rays_d, pos, log_s, quat, cand, off, 8, 8, 8, 8, family=family,
+                                                **more)
     if case == "beyond_invalid":
         assert (want_keys > 1e30).any() and (want_keys == np.float32(1e30)).any()
     if case == "behind":
