@@ -911,11 +911,8 @@ class NeuralPrimitiveSceneTileCUDA(nn.Module):
             params = (self.W1, self.b1, self.W2, self.b2, self.W3, self.b3)
             positions, log_scales = self.positions, self.log_scales
         f32 = torch.float32
-        if not (params[0].dtype == f32 and params[1].dtype == f32 and params[2].dtype == f32 and params[3].dtype == f32
-                and params[4].dtype == f32 and params[5].dtype == f32):
-            half = all(w.dtype == torch.float16 for w in params)
-            if not (half and precision != "f32"):
-                return None                   # stored half-precision weights: only the matrix-core frame reads them as they are
+        if params[0].dtype != f32 and not (precision != "f32" and params[0].dtype == torch.float16):
+            return None                       # stored half-precision weights: only the matrix-core frame reads them as they are
         W, H = self.image_size
         positions, log_scales = positions.detach().contiguous(), log_scales.detach().contiguous()
         views, proj = _frame_matrix(view_matrix).reshape(1, 4, 4), _frame_matrix(proj_matrix)
@@ -926,6 +923,13 @@ class NeuralPrimitiveSceneTileCUDA(nn.Module):
             binned = ext.frame_binning_queued(positions, log_scales, views, proj, int(W), int(H), float(score_threshold),
                                               **({"segments": True} if segments else {}))
             if binned is None:
+                return None
+        # (the other weight tensors are looked at now that the device has the binning to work on; a mixed set goes the
+        # step-by-step way, whose own binning then repeats what was queued here)
+        if not (params[1].dtype == f32 and params[2].dtype == f32 and params[3].dtype == f32 and params[4].dtype == f32
+                and params[5].dtype == f32 and params[0].dtype == f32):
+            half = all(w.dtype == torch.float16 for w in params)
+            if not (half and precision != "f32"):
                 return None
         ws = [p.detach().contiguous() for p in params]
         more = {"binned": binned} if binned is not None else {}
