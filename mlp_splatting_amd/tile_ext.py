@@ -11,6 +11,7 @@ from __future__ import annotations
 
 import contextlib
 import os
+import struct
 import sys
 import threading
 import warnings
@@ -39,7 +40,8 @@ def _is_f32_2d(t, cols):
 
 
 
-_SIXTEEN_ZERO_WORDS = bytes(64)
+_SIXTEEN_ZERO_WORDS = (0,) * 16
+_TAIL_WORDS = struct.Struct("<4q16i")      # the 96 bytes a queued frame reads back
 
 
 def _on_device(device):
@@ -478,11 +480,12 @@ class TileExt:
         if frame.counts is None:
             if frame.landed is not None:
                 frame.landed.synchronize()
-            host = frame.host
-            held["flags_clear"] = host[32:].tobytes() == _SIXTEEN_ZERO_WORDS
-            pairs, longest, l1_entries, guard = (int(v) for v in host[:32].view("int64"))
-            nonfinite = int(host[32:36].view("int32")[0])
-            pool_ran_out = int(host[36:40].view("int32")[0]) if frame.with_feat else 0
+            # (four int64 counts of the binning, sixteen int32 flag words of the render: one unpacking)
+            words = _TAIL_WORDS.unpack_from(frame.host)
+            pairs, longest, l1_entries, guard = words[:4]
+            held["flags_clear"] = words[4:] == _SIXTEEN_ZERO_WORDS
+            nonfinite = words[4]
+            pool_ran_out = words[5] if frame.with_feat else 0
         else:
             pairs, longest, l1_entries, guard = frame.counts
             nonfinite = pool_ran_out = 0
