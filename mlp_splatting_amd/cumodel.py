@@ -914,7 +914,11 @@ class NeuralPrimitiveSceneTileCUDA(nn.Module):
         if params[0].dtype != f32 and not (precision != "f32" and params[0].dtype == torch.float16):
             return None                       # stored half-precision weights: only the matrix-core frame reads them as they are
         W, H = self.image_size
-        positions, log_scales = positions.detach().contiguous(), log_scales.detach().contiguous()
+        # (the kernels take addresses: no detached aliases are made on the way to the first launch)
+        if not positions.is_contiguous():
+            positions = positions.contiguous()
+        if not log_scales.is_contiguous():
+            log_scales = log_scales.contiguous()
         views, proj = _frame_matrix(view_matrix).reshape(1, 4, 4), _frame_matrix(proj_matrix)
         binned = None
         if hasattr(ext, "frame_binning_queued"):

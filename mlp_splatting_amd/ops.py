@@ -23,13 +23,15 @@ def _check(code: int, what: str) -> None:
 
 
 def _ptr(t):
-    return None if t is None else C.c_void_p(t.data_ptr())
+    """The device (or host) address of a tensor as the bound functions take it: every pointer argument is declared
+    ``c_void_p`` in ``_lib.SIGNATURES``, which converts an int or None itself."""
+    return None if t is None else t.data_ptr()
 
 
 def _stream(device):
     """The raw handle of torch's current stream on ``device`` (the launches of a call go there)."""
     index = device.index if device.index is not None else torch.cuda.current_device()
-    return C.c_void_p(torch._C._cuda_getCurrentRawStream(index))
+    return torch._C._cuda_getCurrentRawStream(index)
 
 
 def _f32c(t, name):
